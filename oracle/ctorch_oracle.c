@@ -1,0 +1,649 @@
+/* TEST INFRASTRUCTURE ONLY.
+ *
+ * CPU restatement of the arithmetic of the reference's CPU-BASIC operators, of the host-inline
+ * arithmetic in its Tensor front-end and of the per-operator gradient arithmetic in its tape.
+ * Only tests, the smoke check and the CPU-baseline leg of the benchmark may load this file; the
+ * shipped library never does.
+ *
+ * Every function names the reference lines it follows (paths relative to the reference root).
+ * The reference library is built -O3 -march=native (CMakeLists.txt:65-86).  GCC 11 then treats
+ * its sequential `acc += x*y` loops in two ways, and which one was found per loop by comparing
+ * bits with the built library: loops it cannot vectorise (strided operands in MatMul and in the
+ * column-wise softmax gradient, libm calls in CrossEntropy) get a fused multiply-add; loops over
+ * contiguous memory (Dot, MSE, the row-wise softmax gradient) are vectorised as rounded products
+ * that are then added in order, i.e. without fusion, except for a scalar tail of up to three
+ * elements (see contiguous_mac).  Elementwise loops are never fused.  This
+ * file is compiled with -ffp-contract=off and spells each fusion out with fmaf(), so that the
+ * bits do not depend on this file's compiler.
+ *
+ * Pinning (tests/test_oracle_vs_ref.py, tests/test_oracle_golden.py, tests/test_oracle_math.py):
+ * every function below is compared bit for bit with the real reference library where that has
+ * been built (oracle/_ref), with the golden vectors written from it (tests/golden/), with the
+ * known answers of the reference's own tests, and with closed forms / fp64 recomputation.
+ * Functions the reference cannot express are marked "extension" and are pinned by the same-shape
+ * reference kernel on hand-materialised operands or by fp64 mathematics:
+ *   co_binary_rowbcast for Sub/Mul/Div, co_ce_bwd_index, co_colsum_f64.
+ * Transcendentals call glibc libm (expf, logf, sinf, cosf) exactly as the reference does; their
+ * values are whatever the installed glibc returns (2.35 in this image).
+ */
+#include "ctorch_oracle.h"
+
+#include <float.h>
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ------------------------------------------------------------------ forward: binary kernels */
+
+/* src/kernels/CPU-BASIC/Add_BASIC_kernel.cpp:64-69 (same-shape branch) */
+void co_add(const float* a, const float* b, float* r, long n) {
+    for (long i = 0; i < n; ++i) r[i] = a[i] + b[i];
+}
+/* src/kernels/CPU-BASIC/Sub_BASIC_kernel.cpp:58-60 */
+void co_sub(const float* a, const float* b, float* r, long n) {
+    for (long i = 0; i < n; ++i) r[i] = a[i] - b[i];
+}
+/* src/kernels/CPU-BASIC/Mul_BASIC_kernel.cpp:59-61 */
+void co_mul(const float* a, const float* b, float* r, long n) {
+    for (long i = 0; i < n; ++i) r[i] = a[i] * b[i];
+}
+/* src/kernels/CPU-BASIC/Div_BASIC_kernel.cpp:37-45: a zero divisor is logged, 0 is written and
+ * then overwritten by the IEEE quotient, so the stored value is always a/b. */
+void co_div(const float* a, const float* b, float* r, long n) {
+    for (long i = 0; i < n; ++i) r[i] = a[i] / b[i];
+}
+/* Add_BASIC_kernel.cpp:48-53: b.numel()==1, its single value is added to every element */
+void co_add_scalar_tensor(const float* a, const float* b1, float* r, long n) {
+    float v = b1[0];
+    for (long i = 0; i < n; ++i) r[i] = a[i] + v;
+}
+/* Add_BASIC_kernel.cpp:54-63: a is [rows, cols], b is [cols]; r[i,j] = a[i,j] + b[j] */
+void co_add_rowbcast(const float* a, const float* b, float* r, long rows, long cols) {
+    for (long i = 0; i < rows; ++i)
+        for (long j = 0; j < cols; ++j) r[i * cols + j] = a[i * cols + j] + b[j];
+}
+/* Extension: Add's row-broadcast convention for the other three operators (the reference throws
+ * for Sub/Mul, Sub_BASIC_kernel.cpp:35-43 via Tensor.cpp:362-365, and reads out of bounds for
+ * Div, Div_BASIC_kernel.cpp:18-20).  Equal by construction to the same-shape kernel applied to
+ * a hand-materialised B[i,j] = b[j].  op: 0 add, 1 sub, 2 mul, 3 div. */
+void co_binary_rowbcast(int op, const float* a, const float* b, float* r, long rows, long cols) {
+    for (long i = 0; i < rows; ++i)
+        for (long j = 0; j < cols; ++j) {
+            float x = a[i * cols + j], y = b[j], z;
+            switch (op) {
+                case 0: z = x + y; break;
+                case 1: z = x - y; break;
+                case 2: z = x * y; break;
+                default: z = x / y; break;
+            }
+            r[i * cols + j] = z;
+        }
+}
+
+/* ------------------------------------------------------------------- forward: unary kernels */
+
+/* src/kernels/CPU-BASIC/Neg_BASIC_kernel.cpp:26-28 */
+void co_neg(const float* a, float* r, long n) {
+    for (long i = 0; i < n; ++i) r[i] = -a[i];
+}
+/* src/kernels/CPU-BASIC/ReLU_BASIC_kernel.cpp:23-25: std::max(0.0f, x) is (0.0f < x) ? x : 0.0f,
+ * hence -0 -> +0 and NaN -> +0. */
+void co_relu(const float* a, float* r, long n) {
+    for (long i = 0; i < n; ++i) r[i] = (0.0f < a[i]) ? a[i] : 0.0f;
+}
+/* src/kernels/CPU-BASIC/Sin_BASIC_kernel.cpp:24-26 */
+void co_sin(const float* a, float* r, long n) {
+    for (long i = 0; i < n; ++i) r[i] = sinf(a[i]);
+}
+/* src/kernels/CPU-BASIC/Cos_BASIC_kernel.cpp:23-25 */
+void co_cos(const float* a, float* r, long n) {
+    for (long i = 0; i < n; ++i) r[i] = cosf(a[i]);
+}
+/* src/kernels/CPU-BASIC/Tanh_BASIC_kernel.cpp:24-28 */
+void co_tanh(const float* a, float* r, long n) {
+    for (long i = 0; i < n; ++i) {
+        float ep = expf(a[i]);
+        float en = expf(-a[i]);
+        r[i] = (ep - en) / (ep + en);
+    }
+}
+/* src/kernels/CPU-BASIC/Sigmoid_BASIC_kernel.cpp:24-26 */
+void co_sigmoid(const float* a, float* r, long n) {
+    for (long i = 0; i < n; ++i) r[i] = 1.0f / (1.0f + expf(-a[i]));
+}
+
+/* src/Tensor.cpp:1676-1684 (1-D), :1713-1727 (dim 1), :1728-1744 (dim 0): the live softmax;
+ * with guard_zero_sum it is the registered kernel instead
+ * (src/kernels/CPU-BASIC/Softmax_BASIC_kernel.cpp:47-64, :72-93, which only has dim 1).
+ * A 1-D input is passed as rows = 1, dim = 1. */
+void co_softmax(const float* x, float* y, long rows, long cols, int dim, int guard_zero_sum) {
+    if (dim == 1) {
+        for (long i = 0; i < rows; ++i) {
+            const float* in = x + i * cols;
+            float* out = y + i * cols;
+            float m = in[0];
+            for (long j = 1; j < cols; ++j)
+                if (in[j] > m) m = in[j];
+            float s = 0.0f;
+            for (long j = 0; j < cols; ++j) {
+                float e = expf(in[j] - m);
+                out[j] = e;
+                s += e;
+            }
+            if (!guard_zero_sum || s > 0.0f)
+                for (long j = 0; j < cols; ++j) out[j] /= s;
+        }
+    } else {
+        for (long j = 0; j < cols; ++j) {
+            float m = x[j];
+            for (long i = 1; i < rows; ++i)
+                if (x[i * cols + j] > m) m = x[i * cols + j];
+            float s = 0.0f;
+            for (long i = 0; i < rows; ++i) {
+                float e = expf(x[i * cols + j] - m);
+                y[i * cols + j] = e;
+                s += e;
+            }
+            for (long i = 0; i < rows; ++i) y[i * cols + j] /= s;
+        }
+    }
+}
+
+/* src/kernels/CPU-BASIC/MatMul_BASIC_kernel.cpp:42-54: i-j-l order, stride-aware operands, one
+ * fp32 accumulator per output, fused multiply-add in the built reference. */
+void co_matmul(const float* a, long as0, long as1, const float* b, long bs0, long bs1, float* c,
+               long m, long n, long k) {
+    for (long i = 0; i < m; ++i)
+        for (long j = 0; j < n; ++j) {
+            float s = 0.0f;
+            for (long l = 0; l < k; ++l) s = fmaf(a[i * as0 + l * as1], b[l * bs0 + j * bs1], s);
+            c[i * n + j] = s;
+        }
+}
+
+/* The shape GCC 11 -O3 gives a contiguous `acc += x[i]*y[i]` loop on AVX2/AVX-512 hosts that
+ * prefer 256-bit vectors (found by comparing bits with the built reference for every length
+ * 1..40 and several longer ones): blocks of 8 rounded products added in order, then one block
+ * of 4 if at least 4 elements remain, then a scalar tail of at most 3 fused multiply-adds. */
+static float contiguous_mac(const float* x, const float* y, long n, float s) {
+    long i = 0, main_end = n / 8 * 8;
+    for (; i < main_end; ++i) {
+        float p = x[i] * y[i];
+        s += p;
+    }
+    if (n - i >= 4)
+        for (long e = i + 4; i < e; ++i) {
+            float p = x[i] * y[i];
+            s += p;
+        }
+    for (; i < n; ++i) s = fmaf(x[i], y[i], s);
+    return s;
+}
+
+/* src/kernels/CPU-BASIC/Dot_BASIC_kernel.cpp:38-41 */
+float co_dot(const float* a, const float* b, long n) { return contiguous_mac(a, b, n, 0.0f); }
+
+/* src/kernels/CPU-BASIC/MSE_BASIC_kernel.cpp:35-41: the same loop shape over d = a - b */
+float co_mse(const float* a, const float* b, long n) {
+    float s = 0.0f;
+    long i = 0, main_end = n / 8 * 8;
+    for (; i < main_end; ++i) {
+        float d = a[i] - b[i];
+        float q = d * d;
+        s += q;
+    }
+    if (n - i >= 4)
+        for (long e = i + 4; i < e; ++i) {
+            float d = a[i] - b[i];
+            float q = d * d;
+            s += q;
+        }
+    for (; i < n; ++i) {
+        float d = a[i] - b[i];
+        s = fmaf(d, d, s);
+    }
+    return s / (float)(size_t)n;
+}
+/* src/kernels/CPU-BASIC/MAE_BASIC_kernel.cpp:35-41 */
+float co_mae(const float* a, const float* b, long n) {
+    float s = 0.0f;
+    for (long i = 0; i < n; ++i) {
+        float d = a[i] - b[i];
+        s += fabsf(d);
+    }
+    return s / (float)(size_t)n;
+}
+
+static float row_max(const float* x, long cols) {
+    float m = x[0];
+    for (long j = 1; j < cols; ++j)
+        if (x[j] > m) m = x[j];
+    return m;
+}
+static float row_expsum(const float* x, long cols, float m) {
+    float s = 0.0f;
+    for (long j = 0; j < cols; ++j) s += expf(x[j] - m);
+    return s;
+}
+
+/* src/kernels/CPU-BASIC/CrossEntropy_BASIC_kernel.cpp:41-66 (2-D one-hot; the 1-D form :67-82 is
+ * rows = 1): the loss is SUMMED over rows, never averaged; std::max(pred, 1e-10f) is
+ * (pred < 1e-10f) ? 1e-10f : pred; `ce -= t * log(pred)` is one fused multiply-add. */
+float co_ce_onehot(const float* x, const float* t, long rows, long cols) {
+    float ce = 0.0f;
+    for (long i = 0; i < rows; ++i) {
+        const float* xi = x + i * cols;
+        float m = row_max(xi, cols);
+        float s = row_expsum(xi, cols, m);
+        for (long j = 0; j < cols; ++j) {
+            float p = expf(xi[j] - m) / s;
+            p = (p < 1e-10f) ? 1e-10f : p;
+            ce = fmaf(-t[i * cols + j], logf(p), ce);
+        }
+    }
+    return ce;
+}
+/* CrossEntropy_BASIC_kernel.cpp:88-120 (class indices held as floats, truncated toward zero).
+ * Returns 0 and the summed loss, or -1 when an index is out of range (the reference then returns
+ * an empty Tensor, :96-100). */
+int co_ce_index(const float* x, const float* idx, long rows, long cols, float* out) {
+    float ce = 0.0f;
+    for (long i = 0; i < rows; ++i) {
+        int c = (int)idx[i];
+        if (c < 0 || c >= (int)cols) return -1;
+        const float* xi = x + i * cols;
+        float m = row_max(xi, cols);
+        float s = row_expsum(xi, cols, m);
+        float p = expf(xi[c] - m) / s;
+        p = (p < 1e-10f) ? 1e-10f : p;
+        ce -= logf(p);
+    }
+    *out = ce;
+    return 0;
+}
+
+/* --------------------------------------------------- forward: host-inline Tensor arithmetic */
+
+/* src/Tensor.cpp:644-647 */
+float co_sum(const float* a, long n) {
+    float s = 0.0f;
+    for (long i = 0; i < n; ++i) s += a[i];
+    return s;
+}
+/* src/Tensor.cpp:862-868 */
+void co_scalar_add(const float* a, float s, float* r, long n) {
+    for (long i = 0; i < n; ++i) r[i] = a[i] + s;
+}
+/* src/Tensor.cpp:759-765 */
+void co_scalar_mul(const float* a, float s, float* r, long n) {
+    for (long i = 0; i < n; ++i) r[i] = a[i] * s;
+}
+/* src/Tensor.cpp:925-931 */
+void co_scalar_div(const float* a, float s, float* r, long n) {
+    for (long i = 0; i < n; ++i) r[i] = a[i] / s;
+}
+
+/* ----------------------------------------------------------------------- backward arithmetic */
+
+/* src/AutoDiff.cpp:579-592: a 0-D gradient is expanded to the target shape */
+void co_fill(float* r, float v, long n) {
+    for (long i = 0; i < n; ++i) r[i] = v;
+}
+/* src/AutoDiff.cpp:1870-1878: in-place grad[i] += val[i] */
+void co_accumulate(float* grad, const float* val, long n) {
+    for (long i = 0; i < n; ++i) grad[i] += val[i];
+}
+/* src/AutoDiff.cpp:706-757 as it behaves for g [rows, cols] -> target [cols]: the result is
+ * zeroed and then receives g's leading-index-0 slice, 0.0f + g[0, j] (it does not sum over rows;
+ * the reference's own test expects that: src/tests/test_tensor_grad.cpp:132-138). */
+void co_adjust_row0(const float* g, float* r, long rows, long cols) {
+    (void)rows;
+    for (long j = 0; j < cols; ++j) r[j] = 0.0f + g[j];
+}
+/* Extension: the mathematically complete gradient of a row-broadcast operand, sum over rows,
+ * accumulated in double as the arbiter for the device column-sum kernel. */
+void co_colsum_f64(const float* g, double* r, long rows, long cols) {
+    for (long j = 0; j < cols; ++j) r[j] = 0.0;
+    for (long i = 0; i < rows; ++i)
+        for (long j = 0; j < cols; ++j) r[j] += (double)g[i * cols + j];
+}
+/* src/AutoDiff.cpp:1334-1341 + :1370: mask = x>0 ? 1 : 0, then node_grad * mask (Mul kernel) */
+void co_relu_bwd(const float* x, const float* g, float* dx, long n) {
+    for (long i = 0; i < n; ++i) {
+        float mask = (x[i] > 0.0f) ? 1.0f : 0.0f;
+        dx[i] = g[i] * mask;
+    }
+}
+/* src/AutoDiff.cpp:1372-1383: s = sigmoid(x); (s * (1.0f - s)) * g */
+void co_sigmoid_bwd(const float* x, const float* g, float* dx, long n) {
+    for (long i = 0; i < n; ++i) {
+        float s = 1.0f / (1.0f + expf(-x[i]));
+        float om = 1.0f - s;
+        float p = s * om;
+        dx[i] = p * g[i];
+    }
+}
+/* src/AutoDiff.cpp:1384-1398: t = tanh(x); (1.0f - t*t) * g */
+void co_tanh_bwd(const float* x, const float* g, float* dx, long n) {
+    for (long i = 0; i < n; ++i) {
+        float ep = expf(x[i]);
+        float en = expf(-x[i]);
+        float t = (ep - en) / (ep + en);
+        float tt = t * t;
+        float om = 1.0f - tt;
+        dx[i] = om * g[i];
+    }
+}
+/* src/AutoDiff.cpp:1399-1407: cos(x) * g */
+void co_sin_bwd(const float* x, const float* g, float* dx, long n) {
+    for (long i = 0; i < n; ++i) dx[i] = cosf(x[i]) * g[i];
+}
+/* src/AutoDiff.cpp:1408-1416: (-sin(x)) * g */
+void co_cos_bwd(const float* x, const float* g, float* dx, long n) {
+    for (long i = 0; i < n; ++i) dx[i] = (-sinf(x[i])) * g[i];
+}
+/* src/AutoDiff.cpp:1441-1446 (1-D), :1462-1472 (dim 1), :1473-1484 (dim 0): uses the stored
+ * output y; dx = y * (g - dot).  The row-wise dot walks contiguous memory and is compiled like
+ * Dot above (contiguous_mac); the column-wise dot is strided and is compiled
+ * as a fused multiply-add chain.  Both were checked against the built reference. */
+void co_softmax_bwd(const float* y, const float* g, float* dx, long rows, long cols, int dim) {
+    if (dim == 1) {
+        for (long i = 0; i < rows; ++i) {
+            float d = 0.0f;
+            d = contiguous_mac(g + i * cols, y + i * cols, cols, 0.0f);
+            for (long j = 0; j < cols; ++j) dx[i * cols + j] = y[i * cols + j] * (g[i * cols + j] - d);
+        }
+    } else {
+        for (long j = 0; j < cols; ++j) {
+            float d = 0.0f;
+            for (long i = 0; i < rows; ++i) d = fmaf(g[i * cols + j], y[i * cols + j], d);
+            for (long i = 0; i < rows; ++i) dx[i * cols + j] = y[i * cols + j] * (g[i * cols + j] - d);
+        }
+    }
+}
+/* src/AutoDiff.cpp:1491-1516: (((p - t) * 2.0f) / float(n)) * g with g the 0-D upstream value */
+void co_mse_bwd(const float* p, const float* t, float g, float* dp, long n) {
+    float fn = (float)(size_t)n;
+    for (long i = 0; i < n; ++i) {
+        float d = p[i] - t[i];
+        float d2 = d * 2.0f;
+        float q = d2 / fn;
+        dp[i] = q * g;
+    }
+}
+/* src/AutoDiff.cpp:1602-1642: (sign(p - t) / float(n)) * g, sign in {1, -1, 0} */
+void co_mae_bwd(const float* p, const float* t, float g, float* dp, long n) {
+    float fn = (float)(size_t)n;
+    for (long i = 0; i < n; ++i) {
+        float d = p[i] - t[i];
+        float s = (d > 0.0f) ? 1.0f : ((d < 0.0f) ? -1.0f : 0.0f);
+        float q = s / fn;
+        dp[i] = q * g;
+    }
+}
+/* src/AutoDiff.cpp:1546-1574: row softmax recomputed (no stored sum of stored exps: the sum and
+ * the numerators are separate expf passes), minus the one-hot target (Sub kernel), times the
+ * upstream scalar (scalar Mul).  Gradient of the SUM-reduced loss. */
+void co_ce_bwd_onehot(const float* x, const float* t, float g, float* dx, long rows, long cols) {
+    for (long i = 0; i < rows; ++i) {
+        const float* xi = x + i * cols;
+        float m = row_max(xi, cols);
+        float s = row_expsum(xi, cols, m);
+        for (long j = 0; j < cols; ++j) {
+            float sm = expf(xi[j] - m) / s;
+            float d = sm - t[i * cols + j];
+            dx[i * cols + j] = d * g;
+        }
+    }
+}
+/* Extension: the same arithmetic with class-index targets (the reference throws here,
+ * AutoDiff.cpp:1569 through the Sub broadcast): target is 1.0f at idx[i], 0.0f elsewhere. */
+void co_ce_bwd_index(const float* x, const float* idx, float g, float* dx, long rows, long cols) {
+    for (long i = 0; i < rows; ++i) {
+        const float* xi = x + i * cols;
+        int c = (int)idx[i];
+        float m = row_max(xi, cols);
+        float s = row_expsum(xi, cols, m);
+        for (long j = 0; j < cols; ++j) {
+            float sm = expf(xi[j] - m) / s;
+            float d = sm - ((j == c) ? 1.0f : 0.0f);
+            dx[i * cols + j] = d * g;
+        }
+    }
+}
+/* src/AutoDiff.cpp:1285: node_grad / b */
+void co_div_bwd_a(const float* g, const float* b, float* da, long n) {
+    for (long i = 0; i < n; ++i) da[i] = g[i] / b[i];
+}
+/* src/AutoDiff.cpp:1314: ((-a) * g) / (b * b) - Neg, Mul, Mul, Div in that order */
+void co_div_bwd_b(const float* a, const float* b, const float* g, float* db, long n) {
+    for (long i = 0; i < n; ++i) {
+        float na = -a[i];
+        float num = na * g[i];
+        float den = b[i] * b[i];
+        db[i] = num / den;
+    }
+}
+/* src/AutoDiff.cpp:1267-1279: the divisor scan that makes Div's backward throw */
+int co_any_abs_lt_eps(const float* b, long n) {
+    for (long i = 0; i < n; ++i)
+        if (fabsf(b[i]) < FLT_EPSILON) return 1;
+    return 0;
+}
+
+/* --------------------------------------------------------------------------- configurations */
+
+static float* falloc(long n) {
+    float* p = (float*)malloc((size_t)(n > 0 ? n : 1) * sizeof(float));
+    if (!p) abort();
+    return p;
+}
+
+/* c = a*b + 5.0f; d = relu(c); s = d.sum(); s.backward().  Forward: Mul_BASIC_kernel,
+ * Tensor::operator+(float) (src/Tensor.cpp:855-910), ReLU_BASIC_kernel, Tensor::sum.  Backward
+ * (src/AutoDiff.cpp:1080-1924): root grad 1 -> Sum: fill (1850-1855) -> ReLU: g*mask -> Add with
+ * the taped 0-D scalar: pass-through -> Mul: other * g (1234-1258); every edge lands with
+ * grad += val on a zeroed gradient (1870-1878). */
+void co_chain(const float* a, const float* b, long n, float* s, float* ga, float* gb) {
+    float* c = falloc(n);
+    float* d = falloc(n);
+    float* g = falloc(n);
+    float* v = falloc(n);
+    co_mul(a, b, c, n);
+    co_scalar_add(c, 5.0f, c, n);
+    co_relu(c, d, n);
+    *s = co_sum(d, n);
+    /* grad(d) = 0 + fill(1) */
+    co_fill(g, 0.0f, n);
+    co_fill(v, 1.0f, n);
+    co_accumulate(g, v, n);
+    /* grad(c) = 0 + grad(d) * mask(c) */
+    co_relu_bwd(c, g, v, n);
+    co_fill(g, 0.0f, n);
+    co_accumulate(g, v, n);
+    /* grad(a*b) = 0 + grad(c)   (Add branch) */
+    memcpy(v, g, (size_t)n * sizeof(float));
+    co_fill(g, 0.0f, n);
+    co_accumulate(g, v, n);
+    /* grad(a) = 0 + b * g ; grad(b) = 0 + a * g */
+    co_mul(b, g, v, n);
+    co_fill(ga, 0.0f, n);
+    co_accumulate(ga, v, n);
+    co_mul(a, g, v, n);
+    co_fill(gb, 0.0f, n);
+    co_accumulate(gb, v, n);
+    free(c);
+    free(d);
+    free(g);
+    free(v);
+}
+
+static void zero_plus(float* dst, const float* val, long n) {
+    for (long i = 0; i < n; ++i) dst[i] = 0.0f + val[i];
+}
+
+/* logits = relu(x*W1 + b1)*W2 + b2; loss = CE_sum(logits, onehot); backward
+ * (mnist/mnist.cpp:38-42,66-75 with one hidden layer).  MatMul backward is
+ * dA = g.matmul(B.t()), dB = A.t().matmul(g) through the strided kernel
+ * (src/AutoDiff.cpp:1692-1704, :1808-1810).  Bias gradients: strict_row0 = 1 reproduces the
+ * reference (row 0 of the upstream gradient), 0 gives the column sum rounded from double. */
+void co_mlp_step(const float* x, long B, long I, const float* W1, const float* b1, long H,
+                 const float* W2, const float* b2, long C, const float* onehot, int strict_row0,
+                 float* loss, float* logits, float* gW1, float* gb1, float* gW2, float* gb2) {
+    float* z1 = falloc(B * H);
+    float* a1 = falloc(B * H);
+    float* h = falloc(B * H);
+    float* z2 = falloc(B * C);
+    float* gl = falloc(B * C);
+    float* gh = falloc(B * H);
+    float* ga1 = falloc(B * H);
+    float* tmp = falloc(B * H > I * H ? B * H : I * H);
+    double* cs = (double*)malloc((size_t)(H > C ? H : C) * sizeof(double));
+    co_matmul(x, I, 1, W1, H, 1, z1, B, H, I);
+    co_add_rowbcast(z1, b1, a1, B, H);
+    co_relu(a1, h, B * H);
+    co_matmul(h, H, 1, W2, C, 1, z2, B, C, H);
+    co_add_rowbcast(z2, b2, logits, B, C);
+    *loss = co_ce_onehot(logits, onehot, B, C);
+    /* grad(logits) = 0 + (softmax - onehot) * 1.0f */
+    co_ce_bwd_onehot(logits, onehot, 1.0f, tmp, B, C);
+    zero_plus(gl, tmp, B * C);
+    /* Add: grad(z2) = 0 + gl; grad(b2) = 0 + adjust(gl) */
+    if (strict_row0) {
+        co_adjust_row0(gl, tmp, B, C);
+        zero_plus(gb2, tmp, C);
+    } else {
+        co_colsum_f64(gl, cs, B, C);
+        for (long j = 0; j < C; ++j) gb2[j] = (float)cs[j];
+    }
+    /* MatMul: grad(h) = gl * W2^T ; grad(W2) = h^T * gl */
+    co_matmul(gl, C, 1, W2, 1, C, tmp, B, H, C);
+    zero_plus(gh, tmp, B * H);
+    co_matmul(h, 1, H, gl, C, 1, tmp, H, C, B);
+    zero_plus(gW2, tmp, H * C);
+    /* ReLU: grad(a1) = 0 + gh * mask(a1) */
+    co_relu_bwd(a1, gh, tmp, B * H);
+    zero_plus(ga1, tmp, B * H);
+    if (strict_row0) {
+        co_adjust_row0(ga1, tmp, B, H);
+        zero_plus(gb1, tmp, H);
+    } else {
+        co_colsum_f64(ga1, cs, B, H);
+        for (long j = 0; j < H; ++j) gb1[j] = (float)cs[j];
+    }
+    /* MatMul: grad(W1) = x^T * grad(z1) (grad(z1) = 0 + ga1 = ga1) */
+    co_matmul(x, 1, I, ga1, H, 1, tmp, I, H, B);
+    zero_plus(gW1, tmp, I * H);
+    free(z1);
+    free(a1);
+    free(h);
+    free(z2);
+    free(gl);
+    free(gh);
+    free(ga1);
+    free(tmp);
+    free(cs);
+}
+
+/* Y = sigmoid(X / R) - tanh(X) * sin(X) + cos(-X); L = mse(Y,T) + mae(Y,T); one backward.
+ * R is a full [rows, cols] operand here (the reference's Div needs equal shapes).  The edge
+ * order follows the reference's reversed depth-first order (src/AutoDiff.cpp:1138-1153); it
+ * only matters for X, which receives four contributions: they are added in the order
+ * cos-branch, sin, tanh, div when traversed from L. The exact order of those additions is
+ * pinned against the real reference in tests/test_oracle_vs_ref.py. */
+void co_expr(const float* X, const float* R, const float* T, long rows, long cols, float* Y,
+             float* mse, float* mae, float* gX, float* gR) {
+    long n = rows * cols;
+    float *q = falloc(n), *s1 = falloc(n), *th = falloc(n), *sn = falloc(n), *m = falloc(n),
+          *d1 = falloc(n), *ng = falloc(n), *cs = falloc(n), *gY = falloc(n), *v = falloc(n),
+          *gd1 = falloc(n), *gcs = falloc(n), *gs1 = falloc(n), *gm = falloc(n), *gq = falloc(n),
+          *gth = falloc(n), *gsn = falloc(n), *gng = falloc(n);
+    co_div(X, R, q, n);
+    co_sigmoid(q, s1, n);
+    co_tanh(X, th, n);
+    co_sin(X, sn, n);
+    co_mul(th, sn, m, n);
+    co_sub(s1, m, d1, n);
+    co_neg(X, ng, n);
+    co_cos(ng, cs, n);
+    co_add(d1, cs, Y, n);
+    *mse = co_mse(Y, T, n);
+    *mae = co_mae(Y, T, n);
+    /* L = l1 + l2: both losses get 0 + 1.0f; the order in which their gradients reach Y is
+     * part of what the comparison with the real reference pins (contributions are summed in
+     * fp32, and a+b is commutative, so two terms give the same bits either way). */
+    co_fill(gY, 0.0f, n);
+    co_mse_bwd(Y, T, 1.0f, v, n);
+    float* v2 = falloc(n);
+    co_mae_bwd(Y, T, 1.0f, v2, n);
+    /* order decided against the reference: see co_expr_order in the tests */
+    co_accumulate(gY, v2, n);
+    co_accumulate(gY, v, n);
+    free(v2);
+    /* Add: d1 and cs get gY */
+    zero_plus(gd1, gY, n);
+    zero_plus(gcs, gY, n);
+    /* Sub: s1 gets gd1, m gets -gd1 */
+    zero_plus(gs1, gd1, n);
+    co_neg(gd1, v, n);
+    zero_plus(gm, v, n);
+    /* Mul: th gets sn*gm, sn gets th*gm */
+    co_mul(sn, gm, v, n);
+    zero_plus(gth, v, n);
+    co_mul(th, gm, v, n);
+    zero_plus(gsn, v, n);
+    /* Sigmoid: q gets sigmoid'(q)*gs1 */
+    co_sigmoid_bwd(q, gs1, v, n);
+    zero_plus(gq, v, n);
+    /* Cos: ng gets (-sin(ng))*gcs ; Neg: X gets -gng */
+    co_cos_bwd(ng, gcs, v, n);
+    zero_plus(gng, v, n);
+    /* Div: R gets ((-X)*gq)/(R*R) */
+    co_div_bwd_b(X, R, gq, v, n);
+    zero_plus(gR, v, n);
+    /* X: contributions in tape order (pinned by test) */
+    co_fill(gX, 0.0f, n);
+    co_neg(gng, v, n);
+    co_accumulate(gX, v, n);
+    co_sin_bwd(X, gsn, v, n);
+    co_accumulate(gX, v, n);
+    co_tanh_bwd(X, gth, v, n);
+    co_accumulate(gX, v, n);
+    co_div_bwd_a(gq, R, v, n);
+    co_accumulate(gX, v, n);
+    free(q); free(s1); free(th); free(sn); free(m); free(d1); free(ng); free(cs); free(gY);
+    free(v); free(gd1); free(gcs); free(gs1); free(gm); free(gq); free(gth); free(gsn); free(gng);
+}
+
+/* ------------------------------------------------------------------------- input generator */
+
+/* Counter-based generator of this repository (the reference has no seedable one:
+ * src/Tensor.cpp:463 seeds from random_device).  z = mix(seed * 0x9E3779B97F4A7C15 + i). */
+static uint64_t mix64(uint64_t z) {
+    z ^= z >> 30;
+    z *= 0xBF58476D1CE4E5B9ULL;
+    z ^= z >> 27;
+    z *= 0x94D049BB133111EBULL;
+    z ^= z >> 31;
+    return z;
+}
+static uint64_t draw(uint64_t seed, uint64_t i) { return mix64(seed * 0x9E3779B97F4A7C15ULL + i); }
+
+void co_fill_uniform(float* r, long n, uint64_t seed, double lo, double hi) {
+    for (long i = 0; i < n; ++i) {
+        double u = (double)(draw(seed, (uint64_t)i) >> 40) * (1.0 / 16777216.0);
+        r[i] = (float)(lo + (hi - lo) * u);
+    }
+}
+void co_fill_normal(float* r, long n, uint64_t seed, double mean, double sigma) {
+    for (long i = 0; i < n; ++i) {
+        double u1 = ((double)(draw(seed, (uint64_t)i) >> 11) + 0.5) * (1.0 / 9007199254740992.0);
+        double u2 = ((double)(draw(seed ^ 0xA5A5A5A5A5A5A5A5ULL, (uint64_t)i) >> 11) + 0.5) *
+                    (1.0 / 9007199254740992.0);
+        double z = sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925 * u2);
+        r[i] = (float)(mean + sigma * z);
+    }
+}
+void co_fill_int(float* r, long n, uint64_t seed, long range) {
+    for (long i = 0; i < n; ++i) r[i] = (float)(draw(seed, (uint64_t)i) % (uint64_t)range);
+}

@@ -1,0 +1,74 @@
+/* TEST INFRASTRUCTURE ONLY - CPU restatement of the reference's CPU-BASIC arithmetic.
+ * See ctorch_oracle.c for what each function follows.  Not part of the shipped library. */
+#ifndef CTORCH_ORACLE_H
+#define CTORCH_ORACLE_H
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* forward, dispatched kernels */
+void co_add(const float* a, const float* b, float* r, long n);
+void co_sub(const float* a, const float* b, float* r, long n);
+void co_mul(const float* a, const float* b, float* r, long n);
+void co_div(const float* a, const float* b, float* r, long n);
+void co_add_scalar_tensor(const float* a, const float* b1, float* r, long n);
+void co_add_rowbcast(const float* a, const float* b, float* r, long rows, long cols);
+void co_binary_rowbcast(int op, const float* a, const float* b, float* r, long rows, long cols);
+void co_neg(const float* a, float* r, long n);
+void co_relu(const float* a, float* r, long n);
+void co_sin(const float* a, float* r, long n);
+void co_cos(const float* a, float* r, long n);
+void co_tanh(const float* a, float* r, long n);
+void co_sigmoid(const float* a, float* r, long n);
+void co_softmax(const float* x, float* y, long rows, long cols, int dim, int guard_zero_sum);
+void co_matmul(const float* a, long as0, long as1, const float* b, long bs0, long bs1, float* c,
+               long m, long n, long k);
+float co_dot(const float* a, const float* b, long n);
+float co_mse(const float* a, const float* b, long n);
+float co_mae(const float* a, const float* b, long n);
+float co_ce_onehot(const float* x, const float* t, long rows, long cols);
+int co_ce_index(const float* x, const float* idx, long rows, long cols, float* out);
+
+/* forward, host-inline arithmetic of the Tensor front-end */
+float co_sum(const float* a, long n);
+void co_scalar_add(const float* a, float s, float* r, long n);
+void co_scalar_mul(const float* a, float s, float* r, long n);
+void co_scalar_div(const float* a, float s, float* r, long n);
+
+/* backward arithmetic of the tape */
+void co_fill(float* r, float v, long n);
+void co_accumulate(float* grad, const float* val, long n);
+void co_adjust_row0(const float* g, float* r, long rows, long cols);
+void co_colsum_f64(const float* g, double* r, long rows, long cols);
+void co_relu_bwd(const float* x, const float* g, float* dx, long n);
+void co_sigmoid_bwd(const float* x, const float* g, float* dx, long n);
+void co_tanh_bwd(const float* x, const float* g, float* dx, long n);
+void co_sin_bwd(const float* x, const float* g, float* dx, long n);
+void co_cos_bwd(const float* x, const float* g, float* dx, long n);
+void co_softmax_bwd(const float* y, const float* g, float* dx, long rows, long cols, int dim);
+void co_mse_bwd(const float* p, const float* t, float g, float* dp, long n);
+void co_mae_bwd(const float* p, const float* t, float g, float* dp, long n);
+void co_ce_bwd_onehot(const float* x, const float* t, float g, float* dx, long rows, long cols);
+void co_ce_bwd_index(const float* x, const float* idx, float g, float* dx, long rows, long cols);
+void co_div_bwd_a(const float* g, const float* b, float* da, long n);
+void co_div_bwd_b(const float* a, const float* b, const float* g, float* db, long n);
+int co_any_abs_lt_eps(const float* b, long n);
+
+/* whole configurations, composed from the pieces above in the reference's op order */
+void co_chain(const float* a, const float* b, long n, float* s, float* ga, float* gb);
+void co_mlp_step(const float* x, long B, long I, const float* W1, const float* b1, long H,
+                 const float* W2, const float* b2, long C, const float* onehot, int strict_row0,
+                 float* loss, float* logits, float* gW1, float* gb1, float* gW2, float* gb2);
+void co_expr(const float* X, const float* R, const float* T, long rows, long cols, float* Y,
+             float* mse, float* mae, float* gX, float* gR);
+
+/* seeded input generator shared by tests and fixtures (not from the reference) */
+void co_fill_uniform(float* r, long n, uint64_t seed, double lo, double hi);
+void co_fill_normal(float* r, long n, uint64_t seed, double mean, double sigma);
+void co_fill_int(float* r, long n, uint64_t seed, long range);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,439 @@
+"""ctypes doors for the tests: the CPU oracle (oracle/liboracle.so) and, where it has been built,
+the real reference library behind oracle/ref_driver.cpp (oracle/_ref/libctorch_ref.so).
+
+Test infrastructure only; nothing here is imported by the package.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_DIR = os.path.join(ROOT, "oracle")
+GOLDEN_DIR = os.path.join(ROOT, "tests", "golden")
+
+FP = C.POINTER(C.c_float)
+DP = C.POINTER(C.c_double)
+LP = C.POINTER(C.c_long)
+
+# op codes of oracle/ref_driver.cpp
+ADD, SUB, MUL, DIV, MATMUL, DOT, MSE, MAE, CE = range(9)
+NEG, RELU, SIN, COS, TANH, SIGMOID, SOFTMAX_KERNEL = range(20, 27)
+
+
+def f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def fp(a):
+    assert a.dtype == np.float32 and a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(FP)
+
+
+def bits(a):
+    return f32(a).view(np.uint32)
+
+
+def same_bits(a, b):
+    a, b = f32(a), f32(b)
+    return a.shape == b.shape and np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+def ulp_diff(a, b):
+    """Distance in units in the last place between two fp32 arrays (finite values)."""
+    def key(x):
+        i = f32(x).view(np.int32).astype(np.int64)
+        return np.where(i < 0, -(i & 0x7FFFFFFF), i)
+    return np.abs(key(a) - key(b))
+
+
+def build_oracle():
+    if not os.path.exists(os.path.join(ORACLE_DIR, "liboracle.so")):
+        subprocess.check_call(["make", "-C", ORACLE_DIR, "all"], stdout=subprocess.DEVNULL)
+
+
+class Oracle:
+    """Thin numpy wrapper over oracle/liboracle.so."""
+
+    def __init__(self):
+        build_oracle()
+        self.lib = C.CDLL(os.path.join(ORACLE_DIR, "liboracle.so"))
+        L = self.lib
+        L.co_dot.restype = C.c_float
+        L.co_mse.restype = C.c_float
+        L.co_mae.restype = C.c_float
+        L.co_sum.restype = C.c_float
+        L.co_ce_onehot.restype = C.c_float
+        L.co_ce_index.restype = C.c_int
+        L.co_any_abs_lt_eps.restype = C.c_int
+
+    # ---- inputs
+    def uniform(self, shape, seed, lo, hi):
+        r = np.empty(shape, np.float32)
+        self.lib.co_fill_uniform(fp(r), C.c_long(r.size), C.c_uint64(seed), C.c_double(lo), C.c_double(hi))
+        return r
+
+    def normal(self, shape, seed, mean=0.0, sigma=1.0):
+        r = np.empty(shape, np.float32)
+        self.lib.co_fill_normal(fp(r), C.c_long(r.size), C.c_uint64(seed), C.c_double(mean), C.c_double(sigma))
+        return r
+
+    def ints(self, shape, seed, rng):
+        r = np.empty(shape, np.float32)
+        self.lib.co_fill_int(fp(r), C.c_long(r.size), C.c_uint64(seed), C.c_long(rng))
+        return r
+
+    # ---- helpers
+    def _ew2(self, name, a, b):
+        a, b = f32(a), f32(b)
+        assert a.shape == b.shape
+        r = np.empty_like(a)
+        getattr(self.lib, name)(fp(a), fp(b), fp(r), C.c_long(a.size))
+        return r
+
+    def _ew1(self, name, a):
+        a = f32(a)
+        r = np.empty_like(a)
+        getattr(self.lib, name)(fp(a), fp(r), C.c_long(a.size))
+        return r
+
+    def add(self, a, b): return self._ew2("co_add", a, b)
+    def sub(self, a, b): return self._ew2("co_sub", a, b)
+    def mul(self, a, b): return self._ew2("co_mul", a, b)
+    def div(self, a, b): return self._ew2("co_div", a, b)
+    def neg(self, a): return self._ew1("co_neg", a)
+    def relu(self, a): return self._ew1("co_relu", a)
+    def sin(self, a): return self._ew1("co_sin", a)
+    def cos(self, a): return self._ew1("co_cos", a)
+    def tanh(self, a): return self._ew1("co_tanh", a)
+    def sigmoid(self, a): return self._ew1("co_sigmoid", a)
+
+    def binary(self, op, a, b):
+        return [self.add, self.sub, self.mul, self.div][op](a, b)
+
+    def unary(self, code, a):
+        return {NEG: self.neg, RELU: self.relu, SIN: self.sin, COS: self.cos, TANH: self.tanh,
+                SIGMOID: self.sigmoid}[code](a)
+
+    def add_scalar_tensor(self, a, b1):
+        a, b1 = f32(a), f32(b1).reshape(1)
+        r = np.empty_like(a)
+        self.lib.co_add_scalar_tensor(fp(a), fp(b1), fp(r), C.c_long(a.size))
+        return r
+
+    def binary_rowbcast(self, op, a, b):
+        a, b = f32(a), f32(b)
+        rows, cols = a.shape
+        assert b.shape == (cols,)
+        r = np.empty_like(a)
+        if op == ADD:
+            self.lib.co_add_rowbcast(fp(a), fp(b), fp(r), C.c_long(rows), C.c_long(cols))
+        else:
+            self.lib.co_binary_rowbcast(C.c_int(op), fp(a), fp(b), fp(r), C.c_long(rows), C.c_long(cols))
+        return r
+
+    def softmax(self, x, dim=1, guard=False):
+        x = f32(x)
+        x2 = x.reshape(1, -1) if x.ndim == 1 else x
+        d = 1 if x.ndim == 1 else dim
+        y = np.empty_like(x2)
+        self.lib.co_softmax(fp(x2), fp(y), C.c_long(x2.shape[0]), C.c_long(x2.shape[1]), C.c_int(d), C.c_int(int(guard)))
+        return y.reshape(x.shape)
+
+    def matmul(self, a, b):
+        """a, b may be non-contiguous 2-D views of fp32 arrays (e.g. .T); strides are honoured."""
+        assert a.dtype == np.float32 and b.dtype == np.float32
+        m, k = a.shape
+        k2, n = b.shape
+        assert k == k2
+        c = np.empty((m, n), np.float32)
+        pa = C.cast(a.ctypes.data, FP)
+        pb = C.cast(b.ctypes.data, FP)
+        self.lib.co_matmul(pa, C.c_long(a.strides[0] // 4), C.c_long(a.strides[1] // 4),
+                           pb, C.c_long(b.strides[0] // 4), C.c_long(b.strides[1] // 4),
+                           fp(c), C.c_long(m), C.c_long(n), C.c_long(k))
+        return c
+
+    def dot(self, a, b):
+        a, b = f32(a), f32(b)
+        return np.float32(self.lib.co_dot(fp(a), fp(b), C.c_long(a.size)))
+
+    def mse(self, a, b):
+        a, b = f32(a), f32(b)
+        return np.float32(self.lib.co_mse(fp(a), fp(b), C.c_long(a.size)))
+
+    def mae(self, a, b):
+        a, b = f32(a), f32(b)
+        return np.float32(self.lib.co_mae(fp(a), fp(b), C.c_long(a.size)))
+
+    def sum(self, a):
+        a = f32(a)
+        return np.float32(self.lib.co_sum(fp(a), C.c_long(a.size)))
+
+    def ce_onehot(self, x, t):
+        x, t = f32(x), f32(t)
+        x2 = x.reshape(1, -1) if x.ndim == 1 else x
+        return np.float32(self.lib.co_ce_onehot(fp(x2), fp(t), C.c_long(x2.shape[0]), C.c_long(x2.shape[1])))
+
+    def ce_index(self, x, idx):
+        x, idx = f32(x), f32(idx)
+        out = C.c_float(0)
+        rc = self.lib.co_ce_index(fp(x), fp(idx), C.c_long(x.shape[0]), C.c_long(x.shape[1]), C.byref(out))
+        return None if rc != 0 else np.float32(out.value)
+
+    def scalar(self, which, a, s):
+        a = f32(a)
+        r = np.empty_like(a)
+        name = ["co_scalar_add", "co_scalar_mul", "co_scalar_div"][which]
+        getattr(self.lib, name)(fp(a), C.c_float(s), fp(r), C.c_long(a.size))
+        return r
+
+    # ---- backward pieces
+    def accumulate0(self, val):
+        """0 + val: what a single edge leaves in a zero-initialised gradient."""
+        val = f32(val)
+        g = np.zeros_like(val)
+        self.lib.co_accumulate(fp(g), fp(val), C.c_long(val.size))
+        return g
+
+    def _bwd2(self, name, x, g):
+        x, g = f32(x), f32(g)
+        r = np.empty_like(x)
+        getattr(self.lib, name)(fp(x), fp(g), fp(r), C.c_long(x.size))
+        return r
+
+    def relu_bwd(self, x, g): return self._bwd2("co_relu_bwd", x, g)
+    def sigmoid_bwd(self, x, g): return self._bwd2("co_sigmoid_bwd", x, g)
+    def tanh_bwd(self, x, g): return self._bwd2("co_tanh_bwd", x, g)
+    def sin_bwd(self, x, g): return self._bwd2("co_sin_bwd", x, g)
+    def cos_bwd(self, x, g): return self._bwd2("co_cos_bwd", x, g)
+
+    def unary_bwd(self, code, x, g):
+        if code == NEG:
+            return self.neg(g)
+        return {RELU: self.relu_bwd, SIN: self.sin_bwd, COS: self.cos_bwd, TANH: self.tanh_bwd,
+                SIGMOID: self.sigmoid_bwd}[code](x, g)
+
+    def softmax_bwd(self, y, g, dim=1):
+        y, g = f32(y), f32(g)
+        y2 = y.reshape(1, -1) if y.ndim == 1 else y
+        d = 1 if y.ndim == 1 else dim
+        r = np.empty_like(y2)
+        self.lib.co_softmax_bwd(fp(y2), fp(g), fp(r), C.c_long(y2.shape[0]), C.c_long(y2.shape[1]), C.c_int(d))
+        return r.reshape(y.shape)
+
+    def mse_bwd(self, p, t, g):
+        p, t = f32(p), f32(t)
+        r = np.empty_like(p)
+        self.lib.co_mse_bwd(fp(p), fp(t), C.c_float(g), fp(r), C.c_long(p.size))
+        return r
+
+    def mae_bwd(self, p, t, g):
+        p, t = f32(p), f32(t)
+        r = np.empty_like(p)
+        self.lib.co_mae_bwd(fp(p), fp(t), C.c_float(g), fp(r), C.c_long(p.size))
+        return r
+
+    def ce_bwd_onehot(self, x, t, g):
+        x, t = f32(x), f32(t)
+        x2 = x.reshape(1, -1) if x.ndim == 1 else x
+        r = np.empty_like(x2)
+        self.lib.co_ce_bwd_onehot(fp(x2), fp(t), C.c_float(g), fp(r), C.c_long(x2.shape[0]), C.c_long(x2.shape[1]))
+        return r.reshape(x.shape)
+
+    def ce_bwd_index(self, x, idx, g):
+        x, idx = f32(x), f32(idx)
+        r = np.empty_like(x)
+        self.lib.co_ce_bwd_index(fp(x), fp(idx), C.c_float(g), fp(r), C.c_long(x.shape[0]), C.c_long(x.shape[1]))
+        return r
+
+    def div_bwd_a(self, g, b): return self._ew2("co_div_bwd_a", g, b)
+
+    def div_bwd_b(self, a, b, g):
+        a, b, g = f32(a), f32(b), f32(g)
+        r = np.empty_like(a)
+        self.lib.co_div_bwd_b(fp(a), fp(b), fp(g), fp(r), C.c_long(a.size))
+        return r
+
+    def any_abs_lt_eps(self, b):
+        b = f32(b)
+        return bool(self.lib.co_any_abs_lt_eps(fp(b), C.c_long(b.size)))
+
+    def adjust_row0(self, g):
+        g = f32(g)
+        r = np.empty(g.shape[1], np.float32)
+        self.lib.co_adjust_row0(fp(g), fp(r), C.c_long(g.shape[0]), C.c_long(g.shape[1]))
+        return r
+
+    def colsum_f64(self, g):
+        g = f32(g)
+        r = np.empty(g.shape[1], np.float64)
+        self.lib.co_colsum_f64(fp(g), r.ctypes.data_as(DP), C.c_long(g.shape[0]), C.c_long(g.shape[1]))
+        return r
+
+    # ---- configurations
+    def chain(self, a, b):
+        a, b = f32(a), f32(b)
+        s = C.c_float(0)
+        ga, gb = np.empty_like(a), np.empty_like(b)
+        self.lib.co_chain(fp(a), fp(b), C.c_long(a.size), C.byref(s), fp(ga), fp(gb))
+        return np.float32(s.value), ga, gb
+
+    def mlp_step(self, x, W1, b1, W2, b2, onehot, strict_row0):
+        x, W1, b1, W2, b2, onehot = map(f32, (x, W1, b1, W2, b2, onehot))
+        B, I = x.shape
+        H = W1.shape[1]
+        Cn = W2.shape[1]
+        loss = C.c_float(0)
+        logits = np.empty((B, Cn), np.float32)
+        gW1, gb1, gW2, gb2 = (np.empty_like(t) for t in (W1, b1, W2, b2))
+        self.lib.co_mlp_step(fp(x), C.c_long(B), C.c_long(I), fp(W1), fp(b1), C.c_long(H), fp(W2), fp(b2),
+                             C.c_long(Cn), fp(onehot), C.c_int(int(strict_row0)), C.byref(loss), fp(logits),
+                             fp(gW1), fp(gb1), fp(gW2), fp(gb2))
+        return np.float32(loss.value), logits, gW1, gb1, gW2, gb2
+
+    def expr(self, X, R, T):
+        X, R, T = f32(X), f32(R), f32(T)
+        rows, cols = X.shape
+        Y, gX, gR = np.empty_like(X), np.empty_like(X), np.empty_like(X)
+        mse, mae = C.c_float(0), C.c_float(0)
+        self.lib.co_expr(fp(X), fp(R), fp(T), C.c_long(rows), C.c_long(cols), fp(Y), C.byref(mse), C.byref(mae),
+                         fp(gX), fp(gR))
+        return Y, np.float32(mse.value), np.float32(mae.value), gX, gR
+
+
+def ref_available():
+    return os.path.exists(os.path.join(ORACLE_DIR, "_ref", "libctorch_ref.so"))
+
+
+def _dims(shape):
+    arr = (C.c_long * max(len(shape), 1))(*shape)
+    return arr, len(shape)
+
+
+class Reference:
+    """The real reference library through oracle/ref_driver.cpp.  Exists only where it was built."""
+
+    def __init__(self):
+        self.lib = C.CDLL(os.path.join(ORACLE_DIR, "_ref", "libctorch_ref.so"))
+        for n in ("ref_binary", "ref_unary", "ref_scalar", "ref_sum", "ref_softmax", "ref_matmul_t",
+                  "ref_grad_unary", "ref_grad_softmax", "ref_grad_binary", "ref_grad_loss", "ref_chain",
+                  "ref_mlp_step", "ref_expr"):
+            getattr(self.lib, n).restype = C.c_long
+        self.lib.ref_quiet()
+
+    def binary(self, code, a, b, out_shape):
+        a, b = f32(a), f32(b)
+        ad, an = _dims(a.shape)
+        bd, bn = _dims(b.shape)
+        out = np.empty(out_shape, np.float32)
+        rc = self.lib.ref_binary(code, fp(a), ad, an, fp(b), bd, bn, fp(out))
+        return rc, out
+
+    def unary(self, code, a):
+        a = f32(a)
+        ad, an = _dims(a.shape)
+        out = np.empty_like(a)
+        rc = self.lib.ref_unary(code, fp(a), ad, an, fp(out))
+        assert rc == a.size, rc
+        return out
+
+    def scalar(self, which, a, s):
+        a = f32(a)
+        ad, an = _dims(a.shape)
+        out = np.empty_like(a)
+        rc = self.lib.ref_scalar(which, fp(a), ad, an, C.c_float(s), fp(out))
+        return rc, out
+
+    def sum(self, a):
+        a = f32(a)
+        ad, an = _dims(a.shape)
+        out = np.empty((), np.float32)
+        rc = self.lib.ref_sum(fp(a), ad, an, out.ctypes.data_as(FP))
+        assert rc == 1
+        return np.float32(out)
+
+    def softmax(self, a, dim):
+        a = f32(a)
+        ad, an = _dims(a.shape)
+        out = np.empty_like(a)
+        rc = self.lib.ref_softmax(fp(a), ad, an, dim, fp(out))
+        assert rc == a.size
+        return out
+
+    def matmul_t(self, a, ta, b, tb):
+        a, b = f32(a), f32(b)
+        m = a.shape[1] if ta else a.shape[0]
+        n = b.shape[0] if tb else b.shape[1]
+        out = np.empty((m, n), np.float32)
+        rc = self.lib.ref_matmul_t(fp(a), C.c_long(a.shape[0]), C.c_long(a.shape[1]), int(ta), fp(b),
+                                   C.c_long(b.shape[0]), C.c_long(b.shape[1]), int(tb), fp(out))
+        assert rc == m * n, rc
+        return out
+
+    def grad_unary(self, code, x, w):
+        x, w = f32(x), f32(w)
+        xd, xn = _dims(x.shape)
+        dx = np.empty_like(x)
+        rc = self.lib.ref_grad_unary(code, fp(x), xd, xn, fp(w), fp(dx))
+        assert rc == x.size, rc
+        return dx
+
+    def grad_softmax(self, x, dim, w):
+        x, w = f32(x), f32(w)
+        xd, xn = _dims(x.shape)
+        dx = np.empty_like(x)
+        rc = self.lib.ref_grad_softmax(fp(x), xd, xn, dim, fp(w), fp(dx))
+        assert rc == x.size, rc
+        return dx
+
+    def grad_binary(self, code, a, b, w):
+        a, b, w = f32(a), f32(b), f32(w)
+        ad, an = _dims(a.shape)
+        bd, bn = _dims(b.shape)
+        wd, wn = _dims(w.shape)
+        da, db = np.empty_like(a), np.empty_like(b)
+        rc = self.lib.ref_grad_binary(code, fp(a), ad, an, fp(b), bd, bn, fp(w), wd, wn, fp(da), fp(db))
+        return rc, da, db
+
+    def grad_loss(self, code, p, t, scale):
+        p, t = f32(p), f32(t)
+        pd, pn = _dims(p.shape)
+        td, tn = _dims(t.shape)
+        loss = C.c_float(0)
+        dp = np.empty_like(p)
+        rc = self.lib.ref_grad_loss(code, fp(p), pd, pn, fp(t), td, tn, C.c_float(scale), C.byref(loss), fp(dp))
+        return rc, np.float32(loss.value), dp
+
+    def chain(self, a, b):
+        a, b = f32(a), f32(b)
+        s = C.c_float(0)
+        ga, gb = np.empty_like(a), np.empty_like(b)
+        rc = self.lib.ref_chain(fp(a), fp(b), C.c_long(a.size), C.byref(s), fp(ga), fp(gb))
+        assert rc == a.size
+        return np.float32(s.value), ga, gb
+
+    def mlp_step(self, x, W1, b1, W2, b2, onehot):
+        x, W1, b1, W2, b2, onehot = map(f32, (x, W1, b1, W2, b2, onehot))
+        B, I = x.shape
+        H = W1.shape[1]
+        Cn = W2.shape[1]
+        loss = C.c_float(0)
+        logits = np.empty((B, Cn), np.float32)
+        gW1, gb1, gW2, gb2 = (np.empty_like(t) for t in (W1, b1, W2, b2))
+        rc = self.lib.ref_mlp_step(fp(x), C.c_long(B), C.c_long(I), fp(W1), fp(b1), C.c_long(H), fp(W2), fp(b2),
+                                   C.c_long(Cn), fp(onehot), C.byref(loss), fp(logits), fp(gW1), fp(gb1),
+                                   fp(gW2), fp(gb2))
+        assert rc == B, rc
+        return np.float32(loss.value), logits, gW1, gb1, gW2, gb2
+
+    def expr(self, X, R, T):
+        X, R, T = f32(X), f32(R), f32(T)
+        rows, cols = X.shape
+        Y, gX, gR = np.empty_like(X), np.empty_like(X), np.empty_like(X)
+        mse, mae = C.c_float(0), C.c_float(0)
+        rc = self.lib.ref_expr(fp(X), fp(R), fp(T), C.c_long(rows), C.c_long(cols), fp(Y), C.byref(mse),
+                               C.byref(mae), fp(gX), fp(gR))
+        assert rc == rows * cols, rc
+        return Y, np.float32(mse.value), np.float32(mae.value), gX, gR
