@@ -1,0 +1,49 @@
+// Shared plumbing of the launch layer: error reporting, argument checks, launch geometry and the
+// per-device reduction scratch.
+#ifndef CTORCH_AMD_COMMON_H
+#define CTORCH_AMD_COMMON_H
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/ctorch_amd.h"
+
+namespace ctamd {
+
+// Records the message returned by ctamd_last_error() and passes `code` through.
+int fail(int code, const char* fmt, ...);
+// Maps a hipError_t to 0 / CTAMD_EHIP, recording where it happened.
+int check_hip(hipError_t e, const char* what);
+// Checks the error state after a kernel launch.
+int launched(const char* kernel);
+
+// Scratch for two-stage reductions: kScratchFloats fp32 slots per device, allocated by
+// ctamd_init() and never freed.  Returns nullptr (and records an error) before ctamd_init().
+constexpr size_t kScratchFloats = size_t(1) << 24;   // 64 MiB
+float* scratch();
+// Compute units of the current device (256 on MI355X); 0 before ctamd_init().
+int compute_units();
+
+inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
+
+// Grid for a streaming kernel: enough 256-thread blocks to cover `work_items` (each block
+// iteration handles `per_block` items), capped at `waves_per_cu`-deep occupancy of the chip so
+// that grid-stride loops amortise launch cost on large tensors.
+inline unsigned stream_grid(size_t work_items, size_t per_block, int blocks_per_cu = 8) {
+    size_t need = (work_items + per_block - 1) / per_block;
+    size_t cap = size_t(compute_units() > 0 ? compute_units() : 256) * size_t(blocks_per_cu);
+    if (need < 1) need = 1;
+    return unsigned(need < cap ? need : cap);
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace ctamd
+
+#define CTAMD_REQUIRE(cond, msg)                                                 \
+    do {                                                                         \
+        if (!(cond)) return ::ctamd::fail(CTAMD_EINVAL, "%s: %s", __func__, msg); \
+    } while (0)
+
+#endif

@@ -1,0 +1,178 @@
+// Transcendentals of the device kernels: expf, logf, sinf, cosf evaluated in fp64 and rounded to
+// fp32 once.
+//
+// The reference's CPU kernels call glibc's float routines (Sin_/Cos_/Tanh_/Sigmoid_/Softmax_/
+// CrossEntropy_BASIC_kernel.cpp), and its tanh is (e^x - e^-x)/(e^x + e^-x) in fp32, which
+// amplifies a one-ulp difference in expf into hundreds of ulps near zero.  Matching that formula
+// therefore needs an expf that returns the same float as glibc's for (nearly) every input, not
+// merely an accurate one.  glibc >= 2.27 computes expf/sinf/cosf in double precision with the
+// published algorithms of ARM's optimized-routines (2^(k/32) table + cubic for expf; quadrant
+// reduction + two short polynomials for sinf/cosf).  The functions below follow those published
+// algorithms with the same constants.  Which double operations are fused matters for about one
+// input in 10^9; the fused multiply-adds are spelled out below (CTA_FMA) in the places where
+// glibc's x86-64 FMA build has them, and every file that includes this header is compiled with
+// -ffp-contract=off.  With that, tests/native/devmath_check.c finds zero mismatches against
+// glibc 2.35 over all 2^32 floats for expf and over every |x| < 120 for sinf / cosf on the host,
+// where this header compiles unchanged; fp64 add / mul / fma are IEEE on CDNA, so the device
+// returns the same bits.
+//
+// Everything here is plain C99-compatible so that the same text is compiled by hipcc for the
+// device and by gcc for that host check.
+#ifndef CTORCH_AMD_DEVMATH_H
+#define CTORCH_AMD_DEVMATH_H
+
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#define CTA_FN __device__ __forceinline__ static
+#define CTA_TAB_SPACE __device__ static const
+#define CTA_FMA(a, b, c) __fma_rn((a), (b), (c))
+#else
+#define CTA_FMA(a, b, c) __builtin_fma((a), (b), (c))
+#include <math.h>
+#include <string.h>
+#define CTA_FN static inline
+#define CTA_TAB_SPACE static const
+#endif
+
+CTA_FN uint32_t cta_f2u(float f) {
+#if defined(__HIPCC__)
+    return __float_as_uint(f);
+#else
+    uint32_t u; memcpy(&u, &f, 4); return u;
+#endif
+}
+CTA_FN float cta_u2f(uint32_t u) {
+#if defined(__HIPCC__)
+    return __uint_as_float(u);
+#else
+    float f; memcpy(&f, &u, 4); return f;
+#endif
+}
+CTA_FN uint64_t cta_d2u(double d) {
+#if defined(__HIPCC__)
+    return (uint64_t)__double_as_longlong(d);
+#else
+    uint64_t u; memcpy(&u, &d, 8); return u;
+#endif
+}
+CTA_FN double cta_u2d(uint64_t u) {
+#if defined(__HIPCC__)
+    return __longlong_as_double((long long)u);
+#else
+    double d; memcpy(&d, &u, 8); return d;
+#endif
+}
+
+// tab[i] = bits(2^(i/32)) - (i << 47): adding k << 47 yields bits(2^(k/32)) for any integer k.
+CTA_TAB_SPACE uint64_t cta_exp2_tab[32] = {
+    0x3ff0000000000000ULL, 0x3fefd9b0d3158574ULL, 0x3fefb5586cf9890fULL, 0x3fef9301d0125b51ULL,
+    0x3fef72b83c7d517bULL, 0x3fef54873168b9aaULL, 0x3fef387a6e756238ULL, 0x3fef1e9df51fdee1ULL,
+    0x3fef06fe0a31b715ULL, 0x3feef1a7373aa9cbULL, 0x3feedea64c123422ULL, 0x3feece086061892dULL,
+    0x3feebfdad5362a27ULL, 0x3feeb42b569d4f82ULL, 0x3feeab07dd485429ULL, 0x3feea47eb03a5585ULL,
+    0x3feea09e667f3bcdULL, 0x3fee9f75e8ec5f74ULL, 0x3feea11473eb0187ULL, 0x3feea589994cce13ULL,
+    0x3feeace5422aa0dbULL, 0x3feeb737b0cdc5e5ULL, 0x3feec49182a3f090ULL, 0x3feed503b23e255dULL,
+    0x3feee89f995ad3adULL, 0x3feeff76f2fb5e47ULL, 0x3fef199bdd85529cULL, 0x3fef3720dcef9069ULL,
+    0x3fef5818dcfba487ULL, 0x3fef7c97337b9b5fULL, 0x3fefa4afa2a490daULL, 0x3fefd0765b6e4540ULL};
+
+// `tab` is where the caller keeps the 32 entries (LDS on the device, the array above on the host).
+// Valid for every float: NaN -> NaN, +inf -> +inf, -inf -> 0, overflow -> +inf, underflow ->
+// correctly rounded subnormals and then 0.
+CTA_FN float cta_expf_tab(float x, const uint64_t* tab) {
+    uint32_t ax = cta_f2u(x) & 0x7fffffffu;
+    if (ax >= 0x42b00000u) {                       // |x| >= 88 or NaN
+        if (cta_f2u(x) == 0xff800000u) return 0.0f;
+        if (ax >= 0x7f800000u) return x + x;
+        if (x > 0x1.62e42ep6f) return cta_u2f(0x7f800000u);
+        if (x < -0x1.9fe368p6f) return 0.0f;
+    }
+    double xd = (double)x;
+    const double inv_ln2_n = 0x1.71547652b82fep+0 * 32.0;
+    double kd = CTA_FMA(inv_ln2_n, xd, 0x1.8p+52);   // round to nearest integer in the low bits
+    uint64_t ki = cta_d2u(kd);
+    kd -= 0x1.8p+52;
+    double r = CTA_FMA(inv_ln2_n, xd, -kd);
+    uint64_t t = tab[ki & 31u] + (ki << 47);
+    double s = cta_u2d(t);
+    double p = CTA_FMA(0x1.c6af84b912394p-5 / 32768.0, r, 0x1.ebfce50fac4f3p-3 / 1024.0);
+    double r2 = r * r;
+    double y = CTA_FMA(0x1.62e42ff0c52d6p-1 / 32.0, r, 1.0);
+    y = CTA_FMA(p, r2, y);
+    y = y * s;
+    return (float)y;
+}
+
+// sin / cos: |x| < 0.75 direct, |x| < 120 quadrant reduction with one multiply by pi/2 in double
+// (exact enough: 53-bit pi/2 times |n| < 2^7), beyond that `big` reduces x (any accurate fp64
+// routine; the caller passes the platform's).  sel = 0 sine, 1 cosine.
+CTA_FN double cta_sin_poly(double x, double x2) {
+    double x3 = x * x2;
+    double s1 = CTA_FMA(x2, -0x1.994eb3774cf24p-13, 0x1.1107605230bc4p-7);
+    double x7 = x3 * x2;
+    double s = CTA_FMA(x3, -0x1.555545995a603p-3, x);
+    return CTA_FMA(x7, s1, s);
+}
+CTA_FN double cta_cos_poly(double x2) {
+    double x4 = x2 * x2;
+    double c2 = CTA_FMA(x2, 0x1.99343027bf8c3p-16, -0x1.6c087e89a359dp-10);
+    double c1 = CTA_FMA(x2, -0x1.ffffffd0c621cp-2, 0x1p0);
+    double x6 = x4 * x2;
+    double c = CTA_FMA(x4, 0x1.55553e1068f19p-5, c1);
+    return CTA_FMA(x6, c2, c);
+}
+
+// 32-bit windows of the binary expansion of 2/pi, each shifted 8 bits from the previous one.
+CTA_TAB_SPACE uint32_t cta_inv_pio4[24] = {
+    0x000000a2u, 0x0000a2f9u, 0x00a2f983u, 0xa2f9836eu, 0xf9836e4eu, 0x836e4e44u,
+    0x6e4e4415u, 0x4e441529u, 0x441529fcu, 0x1529fc27u, 0x29fc2757u, 0xfc2757d1u,
+    0x2757d1f5u, 0x57d1f534u, 0xd1f534ddu, 0xf534ddc0u, 0x34ddc0dbu, 0xddc0db62u,
+    0xc0db6295u, 0xdb629599u, 0x6295993cu, 0x95993c43u, 0x993c4390u, 0x3c439041u};
+
+// |x| >= 120: multiply the 24-bit significand by 96 bits of 2/pi chosen by the exponent; the top
+// two bits of the 64-bit product fraction are the quadrant, the rest the reduced argument.
+CTA_FN double cta_reduce_large(uint32_t xi, int* np, const uint32_t* inv_pio4) {
+    const uint32_t* arr = inv_pio4 + ((xi >> 26) & 15);
+    int shift = (int)((xi >> 23) & 7);
+    xi = (xi & 0xffffffu) | 0x800000u;
+    xi <<= shift;
+    uint64_t res0 = (uint64_t)(uint32_t)(xi * arr[0]);
+    uint64_t res1 = (uint64_t)xi * arr[4];
+    uint64_t res2 = (uint64_t)xi * arr[8];
+    res0 = (res2 >> 32) | (res0 << 32);
+    res0 += res1;
+    uint64_t n = (res0 + (1ULL << 61)) >> 62;
+    res0 -= n << 62;
+    double x = (double)(int64_t)res0;
+    *np = (int)n;
+    return x * 0x1.921FB54442D18p-62;
+}
+
+// sinf (want_cos = 0) / cosf (want_cos = 1) for every float.
+CTA_FN float cta_sincosf(float y, int want_cos, const uint32_t* inv_pio4) {
+    uint32_t uy = cta_f2u(y);
+    uint32_t ay = uy & 0x7fffffffu;
+    double x = (double)y;
+    int n;
+    double xr;
+    if (ay < 0x3f400000u) {                        // top 12 bits below those of pi/4: |y| < 0.75
+        if (ay < 0x39800000u) return want_cos ? 1.0f : y;             // |y| < 2^-12
+        double x2 = x * x;
+        return want_cos ? (float)cta_cos_poly(x2) : (float)cta_sin_poly(x, x2);
+    }
+    if (ay < 0x42f00000u) {                        // |y| < 120
+        double r = x * 0x1.45F306DC9C883p+23;      // 2/pi scaled by 2^24
+        n = ((int32_t)r + 0x800000) >> 24;         // nearest quadrant
+        xr = CTA_FMA(-(double)n, 0x1.921FB54442D18p0, x);
+    } else if (ay < 0x7f800000u) {
+        xr = cta_reduce_large(uy, &n, inv_pio4);
+        if (!want_cos) n += (int)(uy >> 31) * 2;   // reduced |y|; sin is odd: sin(t + pi) = -sin(t)
+    } else {
+        return y - y;                              // inf, NaN -> NaN
+    }
+    if (want_cos) n += 1;                          // cos(x) = sin(x + pi/2)
+    double sgn = (n & 2) ? -1.0 : 1.0;
+    if (n & 1) return (float)(sgn * cta_cos_poly(xr * xr));
+    return (float)cta_sin_poly(xr * sgn, xr * xr);
+}
+
+#endif  // CTORCH_AMD_DEVMATH_H

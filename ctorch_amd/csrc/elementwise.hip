@@ -1,0 +1,381 @@
+// Elementwise kernels: binary / broadcast / scalar / unary forward ops and the elementwise
+// gradient arithmetic of the tape.  All of them are HBM-bound streams: one generic grid-stride
+// kernel moves 128-bit vectors (four in flight per thread and operand) and applies a per-element
+// functor; the functors restate the reference's fp32 operation order exactly.  This file must be
+// compiled with -ffp-contract=off: a fused multiply-add would change the bits.
+#include "common.h"
+#include "devmath.h"
+
+namespace ctamd {
+namespace {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 4;
+
+// Lookup tables of devmath.h staged in LDS once per block (random per-lane indices).
+struct Tables {
+    const uint64_t* exp2;
+    const uint32_t* inv_pio4;
+};
+
+template <int N>
+struct Ptrs {
+    const float* p[N > 0 ? N : 1];
+};
+
+// ------------------------------------------------------------------------------- functors
+// Each functor: kIn inputs, kTables whether it needs the LDS tables, and
+// float operator()(const float* x, const Tables&) with x[0..kIn).
+
+struct AddF { static constexpr int kIn = 2; static constexpr bool kTables = false;
+    __device__ float operator()(const float* x, const Tables&) const { return x[0] + x[1]; } };
+struct SubF { static constexpr int kIn = 2; static constexpr bool kTables = false;
+    __device__ float operator()(const float* x, const Tables&) const { return x[0] - x[1]; } };
+struct MulF { static constexpr int kIn = 2; static constexpr bool kTables = false;
+    __device__ float operator()(const float* x, const Tables&) const { return x[0] * x[1]; } };
+struct DivF { static constexpr int kIn = 2; static constexpr bool kTables = false;
+    __device__ float operator()(const float* x, const Tables&) const { return x[0] / x[1]; } };
+
+// a (op) s with s held in the functor (host scalar) - Tensor::operator+(float) etc.
+template <class Op>
+struct ScalarF { static constexpr int kIn = 1; static constexpr bool kTables = false;
+    float s;
+    __device__ float operator()(const float* x, const Tables& t) const { float v[2] = {x[0], s}; return Op()(v, t); } };
+// a (op) *s with s a one-element device tensor
+template <class Op>
+struct DevScalarF { static constexpr int kIn = 1; static constexpr bool kTables = false;
+    const float* s;
+    __device__ float operator()(const float* x, const Tables& t) const { float v[2] = {x[0], *s}; return Op()(v, t); } };
+// *s - b
+struct RSubDevScalarF { static constexpr int kIn = 1; static constexpr bool kTables = false;
+    const float* s;
+    __device__ float operator()(const float* x, const Tables&) const { return *s - x[0]; } };
+
+struct NegF { static constexpr int kIn = 1; static constexpr bool kTables = false;
+    __device__ float operator()(const float* x, const Tables&) const { return -x[0]; } };
+// std::max(0.0f, x): (0 < x) ? x : +0  (NaN and -0 give +0)
+struct ReluF { static constexpr int kIn = 1; static constexpr bool kTables = false;
+    __device__ float operator()(const float* x, const Tables&) const { return (0.0f < x[0]) ? x[0] : 0.0f; } };
+struct SinF { static constexpr int kIn = 1; static constexpr bool kTables = true;
+    __device__ float operator()(const float* x, const Tables& t) const { return cta_sincosf(x[0], 0, t.inv_pio4); } };
+struct CosF { static constexpr int kIn = 1; static constexpr bool kTables = true;
+    __device__ float operator()(const float* x, const Tables& t) const { return cta_sincosf(x[0], 1, t.inv_pio4); } };
+
+__device__ __forceinline__ float tanh_ref(float x, const Tables& t) {
+    float ep = cta_expf_tab(x, t.exp2);
+    float en = cta_expf_tab(-x, t.exp2);
+    return (ep - en) / (ep + en);
+}
+__device__ __forceinline__ float sigmoid_ref(float x, const Tables& t) {
+    return 1.0f / (1.0f + cta_expf_tab(-x, t.exp2));
+}
+struct TanhF { static constexpr int kIn = 1; static constexpr bool kTables = true;
+    __device__ float operator()(const float* x, const Tables& t) const { return tanh_ref(x[0], t); } };
+struct SigmoidF { static constexpr int kIn = 1; static constexpr bool kTables = true;
+    __device__ float operator()(const float* x, const Tables& t) const { return sigmoid_ref(x[0], t); } };
+
+// ---- gradient arithmetic; inputs (x, g) unless noted
+struct ReluBwdF { static constexpr int kIn = 2; static constexpr bool kTables = false;
+    __device__ float operator()(const float* x, const Tables&) const {
+        float mask = (x[0] > 0.0f) ? 1.0f : 0.0f;
+        return x[1] * mask; } };
+struct SigmoidBwdF { static constexpr int kIn = 2; static constexpr bool kTables = true;
+    __device__ float operator()(const float* x, const Tables& t) const {
+        float s = sigmoid_ref(x[0], t);
+        float om = 1.0f - s;
+        float p = s * om;
+        return p * x[1]; } };
+struct TanhBwdF { static constexpr int kIn = 2; static constexpr bool kTables = true;
+    __device__ float operator()(const float* x, const Tables& t) const {
+        float th = tanh_ref(x[0], t);
+        float tt = th * th;
+        float om = 1.0f - tt;
+        return om * x[1]; } };
+struct SinBwdF { static constexpr int kIn = 2; static constexpr bool kTables = true;
+    __device__ float operator()(const float* x, const Tables& t) const {
+        return cta_sincosf(x[0], 1, t.inv_pio4) * x[1]; } };
+struct CosBwdF { static constexpr int kIn = 2; static constexpr bool kTables = true;
+    __device__ float operator()(const float* x, const Tables& t) const {
+        return (-cta_sincosf(x[0], 0, t.inv_pio4)) * x[1]; } };
+// inputs (p, t); fn = float(n); g a 0-D device tensor
+struct MseBwdF { static constexpr int kIn = 2; static constexpr bool kTables = false;
+    float fn; const float* g;
+    __device__ float operator()(const float* x, const Tables&) const {
+        float d = x[0] - x[1];
+        float d2 = d * 2.0f;
+        float q = d2 / fn;
+        return q * *g; } };
+struct MaeBwdF { static constexpr int kIn = 2; static constexpr bool kTables = false;
+    float fn; const float* g;
+    __device__ float operator()(const float* x, const Tables&) const {
+        float d = x[0] - x[1];
+        float s = (d > 0.0f) ? 1.0f : ((d < 0.0f) ? -1.0f : 0.0f);
+        float q = s / fn;
+        return q * *g; } };
+// inputs (a, b, g): ((-a) * g) / (b * b)
+struct DivBwdBF { static constexpr int kIn = 3; static constexpr bool kTables = false;
+    __device__ float operator()(const float* x, const Tables&) const {
+        float na = -x[0];
+        float num = na * x[2];
+        float den = x[1] * x[1];
+        return num / den; } };
+struct FillF { static constexpr int kIn = 0; static constexpr bool kTables = false;
+    float v;
+    __device__ float operator()(const float*, const Tables&) const { return v; } };
+struct FillFromF { static constexpr int kIn = 0; static constexpr bool kTables = false;
+    const float* v;
+    __device__ float operator()(const float*, const Tables&) const { return *v; } };
+
+// -------------------------------------------------------------------------------- kernels
+
+__device__ __forceinline__ void stage_tables(uint64_t* exp2, uint32_t* pio4) {
+    if (threadIdx.x < 32) exp2[threadIdx.x] = cta_exp2_tab[threadIdx.x];
+    if (threadIdx.x >= 32 && threadIdx.x < 56) pio4[threadIdx.x - 32] = cta_inv_pio4[threadIdx.x - 32];
+    __syncthreads();
+}
+
+// VEC = true: all pointers 16-byte aligned, n4 = n / 4 vectors plus a scalar tail handled by
+// block 0.  VEC = false: scalar grid-stride (unaligned views).
+template <class F, bool VEC>
+__global__ __launch_bounds__(kThreads) void map_kernel(Ptrs<F::kIn> in, float* __restrict__ out, size_t n, F f) {
+    __shared__ uint64_t s_exp2[F::kTables ? 32 : 1];
+    __shared__ uint32_t s_pio4[F::kTables ? 24 : 1];
+    if (F::kTables) stage_tables(s_exp2, s_pio4);
+    const Tables tabs{s_exp2, s_pio4};
+    constexpr int NI = F::kIn;
+    const size_t tid = size_t(blockIdx.x) * kThreads + threadIdx.x;
+    const size_t stride = size_t(gridDim.x) * kThreads;
+    if (VEC) {
+        const size_t n4 = n >> 2;
+        for (size_t base = tid; base < n4; base += stride * kUnroll) {
+            v4f v[NI > 0 ? NI : 1][kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                size_t i = base + size_t(u) * stride;
+                if (i < n4) {
+#pragma unroll
+                    for (int k = 0; k < NI; ++k) v[k][u] = reinterpret_cast<const v4f*>(in.p[k])[i];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                size_t i = base + size_t(u) * stride;
+                if (i < n4) {
+                    v4f o;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        float x[NI > 0 ? NI : 1];
+#pragma unroll
+                        for (int k = 0; k < NI; ++k) x[k] = v[k][u][e];
+                        o[e] = f(x, tabs);
+                    }
+                    reinterpret_cast<v4f*>(out)[i] = o;
+                }
+            }
+        }
+        if (blockIdx.x == 0) {
+            size_t i = (n4 << 2) + threadIdx.x;
+            if (i < n) {
+                float x[NI > 0 ? NI : 1];
+#pragma unroll
+                for (int k = 0; k < NI; ++k) x[k] = in.p[k][i];
+                out[i] = f(x, tabs);
+            }
+        }
+    } else {
+        for (size_t i = tid; i < n; i += stride) {
+            float x[NI > 0 ? NI : 1];
+#pragma unroll
+            for (int k = 0; k < NI; ++k) x[k] = in.p[k][i];
+            out[i] = f(x, tabs);
+        }
+    }
+}
+
+template <class F>
+int launch_map(const char* name, Ptrs<F::kIn> in, float* out, size_t n, F f, void* stream) {
+    if (n == 0) return CTAMD_OK;
+    if (!out) return fail(CTAMD_EINVAL, "%s: null output", name);
+    bool vec = aligned16(out);
+    for (int k = 0; k < F::kIn; ++k) {
+        if (!in.p[k]) return fail(CTAMD_EINVAL, "%s: null input %d", name, k);
+        vec = vec && aligned16(in.p[k]);
+    }
+    if (vec) {
+        unsigned grid = stream_grid(n / 4 + 1, size_t(kThreads) * kUnroll);
+        hipLaunchKernelGGL((map_kernel<F, true>), dim3(grid), dim3(kThreads), 0, as_stream(stream), in, out, n, f);
+    } else {
+        unsigned grid = stream_grid(n, size_t(kThreads) * kUnroll);
+        hipLaunchKernelGGL((map_kernel<F, false>), dim3(grid), dim3(kThreads), 0, as_stream(stream), in, out, n, f);
+    }
+    return launched(name);
+}
+
+// r[i,j] = a[i,j] (op) b[j].  VEC: cols % 4 == 0 and aligned pointers - every 128-bit vector of a
+// meets one aligned vector of b (served from cache: b is cols*4 bytes, read rows times).
+template <class Op, bool VEC, class Index>
+__global__ __launch_bounds__(kThreads) void rowbcast_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                            float* __restrict__ r, size_t total, Index cols) {
+    const Tables tabs{nullptr, nullptr};
+    const size_t tid = size_t(blockIdx.x) * kThreads + threadIdx.x;
+    const size_t stride = size_t(gridDim.x) * kThreads;
+    if (VEC) {
+        const size_t n4 = total >> 2;
+        const Index cols4 = cols >> 2;
+        for (size_t base = tid; base < n4; base += stride * kUnroll) {
+            v4f va[kUnroll], vb[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                size_t i = base + size_t(u) * stride;
+                if (i < n4) {
+                    va[u] = reinterpret_cast<const v4f*>(a)[i];
+                    vb[u] = reinterpret_cast<const v4f*>(b)[Index(i) % cols4];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                size_t i = base + size_t(u) * stride;
+                if (i < n4) {
+                    v4f o;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        float x[2] = {va[u][e], vb[u][e]};
+                        o[e] = Op()(x, tabs);
+                    }
+                    reinterpret_cast<v4f*>(r)[i] = o;
+                }
+            }
+        }
+    } else {
+        for (size_t i = tid; i < total; i += stride) {
+            float x[2] = {a[i], b[Index(i) % cols]};
+            r[i] = Op()(x, tabs);
+        }
+    }
+}
+
+template <class Op>
+int launch_rowbcast(const char* name, const float* a, const float* b, float* r, size_t rows, size_t cols,
+                    void* stream) {
+    if (rows == 0 || cols == 0) return CTAMD_OK;
+    if (!a || !b || !r) return fail(CTAMD_EINVAL, "%s: null pointer", name);
+    if (rows > (size_t(1) << 62) / cols) return fail(CTAMD_ERANGE, "%s: rows*cols overflows", name);
+    size_t total = rows * cols;
+    bool vec = (cols % 4 == 0) && aligned16(a) && aligned16(b) && aligned16(r);
+    bool small = total < (size_t(1) << 32);
+    unsigned grid = stream_grid(vec ? total / 4 : total, size_t(kThreads) * kUnroll);
+    hipStream_t s = as_stream(stream);
+    if (vec && small)
+        hipLaunchKernelGGL((rowbcast_kernel<Op, true, uint32_t>), dim3(grid), dim3(kThreads), 0, s, a, b, r, total, uint32_t(cols));
+    else if (vec)
+        hipLaunchKernelGGL((rowbcast_kernel<Op, true, uint64_t>), dim3(grid), dim3(kThreads), 0, s, a, b, r, total, uint64_t(cols));
+    else if (small)
+        hipLaunchKernelGGL((rowbcast_kernel<Op, false, uint32_t>), dim3(grid), dim3(kThreads), 0, s, a, b, r, total, uint32_t(cols));
+    else
+        hipLaunchKernelGGL((rowbcast_kernel<Op, false, uint64_t>), dim3(grid), dim3(kThreads), 0, s, a, b, r, total, uint64_t(cols));
+    return launched(name);
+}
+
+template <class F>
+int binary(const char* name, const float* a, const float* b, float* r, size_t n, void* stream) {
+    Ptrs<2> in{{a, b}};
+    return launch_map<F>(name, in, r, n, F(), stream);
+}
+template <class F>
+int unary(const char* name, const float* a, float* r, size_t n, void* stream) {
+    Ptrs<1> in{{a}};
+    return launch_map<F>(name, in, r, n, F(), stream);
+}
+template <class Op>
+int host_scalar(const char* name, const float* a, float s, float* r, size_t n, void* stream) {
+    Ptrs<1> in{{a}};
+    return launch_map<ScalarF<Op>>(name, in, r, n, ScalarF<Op>{s}, stream);
+}
+template <class Op>
+int dev_scalar(const char* name, const float* a, const float* b1, float* r, size_t n, void* stream) {
+    if (n && !b1) return fail(CTAMD_EINVAL, "%s: null scalar operand", name);
+    Ptrs<1> in{{a}};
+    return launch_map<DevScalarF<Op>>(name, in, r, n, DevScalarF<Op>{b1}, stream);
+}
+
+}  // namespace
+}  // namespace ctamd
+
+using namespace ctamd;
+
+extern "C" {
+
+int ctamd_add_f32(const float* a, const float* b, float* r, size_t n, void* s) { return binary<AddF>(__func__, a, b, r, n, s); }
+int ctamd_sub_f32(const float* a, const float* b, float* r, size_t n, void* s) { return binary<SubF>(__func__, a, b, r, n, s); }
+int ctamd_mul_f32(const float* a, const float* b, float* r, size_t n, void* s) { return binary<MulF>(__func__, a, b, r, n, s); }
+int ctamd_div_f32(const float* a, const float* b, float* r, size_t n, void* s) { return binary<DivF>(__func__, a, b, r, n, s); }
+
+int ctamd_add_rowbcast_f32(const float* a, const float* b, float* r, size_t rows, size_t cols, void* s) {
+    return launch_rowbcast<AddF>(__func__, a, b, r, rows, cols, s);
+}
+int ctamd_sub_rowbcast_f32(const float* a, const float* b, float* r, size_t rows, size_t cols, void* s) {
+    return launch_rowbcast<SubF>(__func__, a, b, r, rows, cols, s);
+}
+int ctamd_mul_rowbcast_f32(const float* a, const float* b, float* r, size_t rows, size_t cols, void* s) {
+    return launch_rowbcast<MulF>(__func__, a, b, r, rows, cols, s);
+}
+int ctamd_div_rowbcast_f32(const float* a, const float* b, float* r, size_t rows, size_t cols, void* s) {
+    return launch_rowbcast<DivF>(__func__, a, b, r, rows, cols, s);
+}
+
+int ctamd_add_bscalar_f32(const float* a, const float* b1, float* r, size_t n, void* s) { return dev_scalar<AddF>(__func__, a, b1, r, n, s); }
+int ctamd_sub_bscalar_f32(const float* a, const float* b1, float* r, size_t n, void* s) { return dev_scalar<SubF>(__func__, a, b1, r, n, s); }
+int ctamd_mul_bscalar_f32(const float* a, const float* b1, float* r, size_t n, void* s) { return dev_scalar<MulF>(__func__, a, b1, r, n, s); }
+int ctamd_div_bscalar_f32(const float* a, const float* b1, float* r, size_t n, void* s) { return dev_scalar<DivF>(__func__, a, b1, r, n, s); }
+int ctamd_rsub_ascalar_f32(const float* a1, const float* b, float* r, size_t n, void* s) {
+    if (n && !a1) return fail(CTAMD_EINVAL, "%s: null scalar operand", __func__);
+    Ptrs<1> in{{b}};
+    return launch_map<RSubDevScalarF>(__func__, in, r, n, RSubDevScalarF{a1}, s);
+}
+
+int ctamd_add_scalar_f32(const float* a, float v, float* r, size_t n, void* s) { return host_scalar<AddF>(__func__, a, v, r, n, s); }
+int ctamd_mul_scalar_f32(const float* a, float v, float* r, size_t n, void* s) { return host_scalar<MulF>(__func__, a, v, r, n, s); }
+int ctamd_div_scalar_f32(const float* a, float v, float* r, size_t n, void* s) { return host_scalar<DivF>(__func__, a, v, r, n, s); }
+
+int ctamd_neg_f32(const float* a, float* r, size_t n, void* s) { return unary<NegF>(__func__, a, r, n, s); }
+int ctamd_relu_f32(const float* a, float* r, size_t n, void* s) { return unary<ReluF>(__func__, a, r, n, s); }
+int ctamd_sin_f32(const float* a, float* r, size_t n, void* s) { return unary<SinF>(__func__, a, r, n, s); }
+int ctamd_cos_f32(const float* a, float* r, size_t n, void* s) { return unary<CosF>(__func__, a, r, n, s); }
+int ctamd_tanh_f32(const float* a, float* r, size_t n, void* s) { return unary<TanhF>(__func__, a, r, n, s); }
+int ctamd_sigmoid_f32(const float* a, float* r, size_t n, void* s) { return unary<SigmoidF>(__func__, a, r, n, s); }
+
+int ctamd_fill_f32(float* r, float v, size_t n, void* s) {
+    Ptrs<0> in{};
+    return launch_map<FillF>(__func__, in, r, n, FillF{v}, s);
+}
+int ctamd_fill_from_f32(float* r, const float* v1, size_t n, void* s) {
+    if (n && !v1) return fail(CTAMD_EINVAL, "%s: null source", __func__);
+    Ptrs<0> in{};
+    return launch_map<FillFromF>(__func__, in, r, n, FillFromF{v1}, s);
+}
+int ctamd_accumulate_f32(float* grad, const float* val, size_t n, void* s) {
+    return binary<AddF>(__func__, grad, val, grad, n, s);
+}
+int ctamd_relu_backward_f32(const float* x, const float* g, float* dx, size_t n, void* s) { return binary<ReluBwdF>(__func__, x, g, dx, n, s); }
+int ctamd_sigmoid_backward_f32(const float* x, const float* g, float* dx, size_t n, void* s) { return binary<SigmoidBwdF>(__func__, x, g, dx, n, s); }
+int ctamd_tanh_backward_f32(const float* x, const float* g, float* dx, size_t n, void* s) { return binary<TanhBwdF>(__func__, x, g, dx, n, s); }
+int ctamd_sin_backward_f32(const float* x, const float* g, float* dx, size_t n, void* s) { return binary<SinBwdF>(__func__, x, g, dx, n, s); }
+int ctamd_cos_backward_f32(const float* x, const float* g, float* dx, size_t n, void* s) { return binary<CosBwdF>(__func__, x, g, dx, n, s); }
+int ctamd_mse_backward_f32(const float* p, const float* t, const float* g1, float* dp, size_t n, void* s) {
+    if (n && !g1) return fail(CTAMD_EINVAL, "%s: null upstream gradient", __func__);
+    Ptrs<2> in{{p, t}};
+    return launch_map<MseBwdF>(__func__, in, dp, n, MseBwdF{float(n), g1}, s);
+}
+int ctamd_mae_backward_f32(const float* p, const float* t, const float* g1, float* dp, size_t n, void* s) {
+    if (n && !g1) return fail(CTAMD_EINVAL, "%s: null upstream gradient", __func__);
+    Ptrs<2> in{{p, t}};
+    return launch_map<MaeBwdF>(__func__, in, dp, n, MaeBwdF{float(n), g1}, s);
+}
+int ctamd_div_backward_b_f32(const float* a, const float* b, const float* g, float* db, size_t n, void* s) {
+    Ptrs<3> in{{a, b, g}};
+    return launch_map<DivBwdBF>(__func__, in, db, n, DivBwdBF(), s);
+}
+
+}  // extern "C"

@@ -1,0 +1,322 @@
+// fp32 MatMul on the CDNA4 matrix cores (v_mfma_f32_32x32x2_f32), fp32 accumulation.
+//
+// C[m,n] = sum_k A[m,k] * B[k,n] for operands given by element strides.  Every operand with a
+// unit stride in one dimension is one of two tile kinds:
+//   K-contiguous  (A row-major, or B given as a transposed view): tile kept in LDS as [rows][BK],
+//                 fragments read with one 128-bit LDS load per 32x32 MFMA tile and 8-wide k chunk;
+//   X-contiguous  (A given as a transposed view, or B row-major): tile kept as [BK][cols],
+//                 fragments read with four 32-bit LDS loads.
+// Within an 8-wide k chunk, lane half h (lane / 32) owns k = 4h .. 4h+3 for both operands - the
+// sum over k is order-free, so the MFMA's (lane / 32) k index is simply re-labelled; that lets
+// the K-contiguous kind fetch four consecutive k with a single load.
+// One 256-thread block (4 waves, 2 x 2) computes a BM x BN tile of C; global -> register ->
+// LDS staging is double buffered so the loads of tile t+1 are in flight while tile t is
+// multiplied, with one barrier per k tile.  Blocks are renumbered so that each XCD (blocks are
+// dealt round-robin to the 8 XCDs) works on a compact band of C and re-uses its operand tiles
+// from its own L2.  Skinny outputs with a long K (the weight gradients of a small layer) are
+// split along K over blockIdx.z; partial products go to the device scratch and are folded in a
+// fixed order, so results stay deterministic.
+#include "common.h"
+
+namespace ctamd {
+namespace {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int kThreads = 256;
+constexpr int kXcds = 8;
+
+template <int BM_, int BN_, int BK_, int WM_, int WN_>
+struct Cfg {
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
+    static constexpr int TM = WM / 32, TN = WN / 32;       // MFMA tiles per wave
+    static constexpr int WAVES_N = BN / WN;
+    static_assert((BM / WM) * (BN / WN) == kThreads / 64, "wave grid must use 4 waves");
+    static_assert(BK % 8 == 0, "k tile is a multiple of the 8-wide chunk");
+    static constexpr int KPAD = BK + 4;                    // K-contiguous row stride (floats)
+    static constexpr int XPAD_M = BM + 8, XPAD_N = BN + 8; // X-contiguous row strides
+};
+
+// LDS footprint of one operand tile (floats)
+template <class C, bool KC, bool IS_A>
+constexpr int tile_floats() {
+    return KC ? (IS_A ? C::BM : C::BN) * C::KPAD : C::BK * (IS_A ? C::XPAD_M : C::XPAD_N);
+}
+
+// Global -> registers for one operand tile.  ROWS x BK (K-contiguous) or BK x ROWS
+// (X-contiguous), as 128-bit pieces dealt to the 256 threads.
+template <int ROWS, int BK, bool KC>
+struct Stage {
+    static constexpr int PIECES = ROWS * BK / 4 / kThreads;
+    static_assert(ROWS * BK / 4 % kThreads == 0, "tile must split evenly over the block");
+    v4f r[PIECES];
+
+    // x0: first row/col of the tile in the X dimension, k0: first k; dimX, K: extents; ld: leading
+    // dimension (elements) of the contiguous direction's rows.  VEC: 16-byte aligned rows.
+    template <bool VEC>
+    __device__ __forceinline__ void load(const float* __restrict__ p, int64_t ld, int x0, int k0, int dimX, int k_end) {
+#pragma unroll
+        for (int q = 0; q < PIECES; ++q) {
+            int idx = threadIdx.x + q * kThreads;
+            int outer, inner;   // outer indexes rows of the contiguous direction
+            if (KC) { outer = idx / (BK / 4); inner = (idx % (BK / 4)) * 4; }
+            else { outer = idx / (ROWS / 4); inner = (idx % (ROWS / 4)) * 4; }
+            int gx = KC ? x0 + outer : x0 + inner;          // position along X
+            int gk = KC ? k0 + inner : k0 + outer;          // position along K
+            const float* src = KC ? p + int64_t(gx) * ld + gk : p + int64_t(gk) * ld + gx;
+            int lim_outer = KC ? dimX : k_end, pos_outer = KC ? gx : gk;
+            int lim_inner = KC ? k_end : dimX, pos_inner = KC ? gk : gx;
+            v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (pos_outer < lim_outer) {
+                if (VEC && pos_inner + 4 <= lim_inner) {
+                    v = *reinterpret_cast<const v4f*>(src);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (pos_inner + e < lim_inner) v[e] = src[e];
+                }
+            }
+            r[q] = v;
+        }
+    }
+    __device__ __forceinline__ void store(float* __restrict__ lds, int stride) const {
+#pragma unroll
+        for (int q = 0; q < PIECES; ++q) {
+            int idx = threadIdx.x + q * kThreads;
+            int outer, inner;
+            if (KC) { outer = idx / (BK / 4); inner = (idx % (BK / 4)) * 4; }
+            else { outer = idx / (ROWS / 4); inner = (idx % (ROWS / 4)) * 4; }
+            *reinterpret_cast<v4f*>(lds + outer * stride + inner) = r[q];
+        }
+    }
+};
+
+// Fragment fetch for one 32-wide MFMA tile and one 8-wide k chunk: f[s] is this lane's operand
+// for k = chunk*8 + 4*(lane/32) + s.
+template <bool KC>
+__device__ __forceinline__ void fetch(const float* __restrict__ lds, int stride, int x, int kbase, float (&f)[4]) {
+    if (KC) {
+        v4f v = *reinterpret_cast<const v4f*>(lds + x * stride + kbase);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) f[s] = v[s];
+    } else {
+#pragma unroll
+        for (int s = 0; s < 4; ++s) f[s] = lds[(kbase + s) * stride + x];
+    }
+}
+
+struct GemmArgs {
+    const float* a; int64_t lda;
+    const float* b; int64_t ldb;
+    float* c; int64_t ldc;          // C, or the partial buffer when split along K
+    int m, n, k;
+    int k_per_split;                // multiple of BK
+    int64_t split_stride;           // elements between partial buffers (0 when not split)
+    int tiles_m, tiles_n;
+};
+
+template <class C, bool A_KC, bool B_KC, bool VEC>
+__global__ __launch_bounds__(kThreads, 2) void gemm_kernel(GemmArgs g) {
+    constexpr int BM = C::BM, BN = C::BN, BK = C::BK, TM = C::TM, TN = C::TN;
+    constexpr int A_STRIDE = A_KC ? C::KPAD : C::XPAD_M;
+    constexpr int B_STRIDE = B_KC ? C::KPAD : C::XPAD_N;
+    constexpr int A_FLOATS = tile_floats<C, A_KC, true>();
+    constexpr int B_FLOATS = tile_floats<C, B_KC, false>();
+    __shared__ __attribute__((aligned(16))) float s_a[2][A_FLOATS];
+    __shared__ __attribute__((aligned(16))) float s_b[2][B_FLOATS];
+
+    // XCD-aware renumbering: hardware block b runs on XCD b % 8; give each XCD a contiguous run of
+    // tiles, and inside the run walk C in column-major bands of 8 tile rows so that co-resident
+    // blocks share A row bands and B column bands in that XCD's L2.
+    const int tiles = g.tiles_m * g.tiles_n;
+    int bid = blockIdx.x;
+    {
+        int per = tiles / kXcds, rem = tiles % kXcds;
+        int xcd = bid % kXcds, local = bid / kXcds;
+        // XCDs with index < rem own per+1 tiles
+        bid = xcd * per + (xcd < rem ? xcd : rem) + local;
+    }
+    constexpr int BAND = 8;
+    int band = bid / (BAND * g.tiles_n);
+    int band_rows = g.tiles_m - band * BAND < BAND ? g.tiles_m - band * BAND : BAND;
+    int in_band = bid - band * BAND * g.tiles_n;
+    const int tile_m = band * BAND + in_band % band_rows;
+    const int tile_n = in_band / band_rows;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const int k_begin = blockIdx.z * g.k_per_split;
+    int k_end = k_begin + g.k_per_split;
+    if (k_end > g.k) k_end = g.k;
+    float* __restrict__ cout = g.c + int64_t(blockIdx.z) * g.split_stride;
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm = (wave / C::WAVES_N) * C::WM, wn = (wave % C::WAVES_N) * C::WN;
+    const int l32 = lane & 31, half = lane >> 5;
+
+    v16f acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    Stage<BM, BK, A_KC> sa;
+    Stage<BN, BK, B_KC> sb;
+    const int ktiles = (k_end - k_begin + BK - 1) / BK;
+    if (ktiles > 0) {
+        sa.template load<VEC>(g.a, g.lda, m0, k_begin, g.m, k_end);
+        sb.template load<VEC>(g.b, g.ldb, n0, k_begin, g.n, k_end);
+        sa.store(s_a[0], A_STRIDE);
+        sb.store(s_b[0], B_STRIDE);
+    }
+    __syncthreads();
+    for (int t = 0; t < ktiles; ++t) {
+        const int cur = t & 1;
+        if (t + 1 < ktiles) {
+            sa.template load<VEC>(g.a, g.lda, m0, k_begin + (t + 1) * BK, g.m, k_end);
+            sb.template load<VEC>(g.b, g.ldb, n0, k_begin + (t + 1) * BK, g.n, k_end);
+        }
+        const float* __restrict__ la = s_a[cur];
+        const float* __restrict__ lb = s_b[cur];
+#pragma unroll
+        for (int ch = 0; ch < BK / 8; ++ch) {
+            float fa[TM][4], fb[TN][4];
+            const int kb = ch * 8 + half * 4;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) fetch<A_KC>(la, A_STRIDE, wm + i * 32 + l32, kb, fa[i]);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) fetch<B_KC>(lb, B_STRIDE, wn + j * 32 + l32, kb, fb[j]);
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
+        }
+        if (t + 1 < ktiles) {
+            sa.store(s_a[cur ^ 1], A_STRIDE);
+            sb.store(s_b[cur ^ 1], B_STRIDE);
+        }
+        __syncthreads();
+    }
+
+    // accumulator register r of lane l holds C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 tile
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int col = n0 + wn + j * 32 + l32;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = m0 + wm + i * 32 + 8 * (r / 4) + 4 * half + (r % 4);
+                if (row < g.m && col < g.n) cout[int64_t(row) * g.ldc + col] = acc[i][j][r];
+            }
+        }
+}
+
+// Folds the K-split partial products: c[i] = sum_z partial[z][i], in order of z.
+__global__ __launch_bounds__(kThreads) void splitk_fold(const float* __restrict__ partial, float* __restrict__ c,
+                                                        size_t mn, int splits) {
+    size_t i = size_t(blockIdx.x) * kThreads + threadIdx.x;
+    if (i >= mn) return;
+    float t = partial[i];
+    for (int z = 1; z < splits; ++z) t += partial[size_t(z) * mn + i];
+    c[i] = t;
+}
+
+// Operands with no unit stride: one thread per output element.  Correct for any strides; only
+// the reference's own transposes of transposes could produce such views.
+__global__ __launch_bounds__(kThreads) void gemm_strided(const float* __restrict__ a, int64_t as0, int64_t as1,
+                                                         const float* __restrict__ b, int64_t bs0, int64_t bs1,
+                                                         float* __restrict__ c, int m, int n, int k) {
+    size_t idx = size_t(blockIdx.x) * kThreads + threadIdx.x;
+    if (idx >= size_t(m) * n) return;
+    int i = int(idx / n), j = int(idx % n);
+    float s = 0.0f;
+    for (int l = 0; l < k; ++l) s = __fmaf_rn(a[i * as0 + l * as1], b[l * bs0 + j * bs1], s);
+    c[idx] = s;
+}
+
+using Tile = Cfg<128, 128, 16, 64, 64>;
+
+template <bool A_KC, bool B_KC>
+int launch_gemm(GemmArgs g, bool vec, int splits, hipStream_t s) {
+    dim3 grid(unsigned(g.tiles_m * g.tiles_n), 1, unsigned(splits));
+    if (vec) hipLaunchKernelGGL((gemm_kernel<Tile, A_KC, B_KC, true>), grid, dim3(kThreads), 0, s, g);
+    else hipLaunchKernelGGL((gemm_kernel<Tile, A_KC, B_KC, false>), grid, dim3(kThreads), 0, s, g);
+    return launched("ctamd_matmul_f32");
+}
+
+}  // namespace
+}  // namespace ctamd
+
+using namespace ctamd;
+
+extern "C" int ctamd_matmul_f32(const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,
+                                float* c, int64_t m, int64_t n, int64_t k, void* stream) {
+    if (m < 0 || n < 0 || k < 0) return fail(CTAMD_EINVAL, "%s: negative extent", __func__);
+    if (m == 0 || n == 0) return CTAMD_OK;
+    if (!c) return fail(CTAMD_EINVAL, "%s: null output", __func__);
+    if (m > 0x7fffffff || n > 0x7fffffff || k > 0x7fffffff || m * n > (int64_t(1) << 40))
+        return fail(CTAMD_ERANGE, "%s: extent too large", __func__);
+    if (k == 0) return ctamd_fill_f32(c, 0.0f, size_t(m) * size_t(n), stream);
+    if (!a || !b) return fail(CTAMD_EINVAL, "%s: null input", __func__);
+    if (as0 < 0 || as1 < 0 || bs0 < 0 || bs1 < 0) return fail(CTAMD_EINVAL, "%s: negative stride", __func__);
+    hipStream_t s = as_stream(stream);
+
+    // a one-row / one-column operand is contiguous in whichever direction has extent > 1
+    const bool a_kc = (as1 == 1) || (k == 1 && as0 != 1), a_xc = (as0 == 1) || (m == 1);
+    const bool b_xc = (bs1 == 1) || (n == 1 && bs0 != 1), b_kc = (bs0 == 1) || (k == 1);
+    if (!(a_kc || a_xc) || !(b_kc || b_xc)) {
+        hipLaunchKernelGGL(gemm_strided, dim3(unsigned((size_t(m) * n + kThreads - 1) / kThreads)), dim3(kThreads), 0, s,
+                           a, as0, as1, b, bs0, bs1, c, int(m), int(n), int(k));
+        return launched(__func__);
+    }
+    const bool A_KC = a_kc, B_KC = !b_xc;
+    GemmArgs g;
+    g.a = a; g.lda = A_KC ? as0 : as1;
+    g.b = b; g.ldb = B_KC ? bs1 : bs0;
+    g.m = int(m); g.n = int(n); g.k = int(k);
+    g.tiles_m = int((m + Tile::BM - 1) / Tile::BM);
+    g.tiles_n = int((n + Tile::BN - 1) / Tile::BN);
+    const bool vec = aligned16(a) && aligned16(b) && (g.lda % 4 == 0) && (g.ldb % 4 == 0);
+
+    // split along K when the output has too few tiles to fill the chip and K is long
+    int splits = 1;
+    const int64_t tiles = int64_t(g.tiles_m) * g.tiles_n;
+    const int cus = compute_units() > 0 ? compute_units() : 256;
+    float* partial = nullptr;
+    if (tiles < cus && k >= 8 * Tile::BK) {
+        int64_t want = (2 * cus + tiles - 1) / tiles;
+        int64_t max_by_k = k / (4 * Tile::BK);
+        int64_t max_by_scratch = int64_t(kScratchFloats) / (m * n);
+        splits = int(want < max_by_k ? want : max_by_k);
+        if (splits > max_by_scratch) splits = int(max_by_scratch);
+        if (splits > 1) {
+            partial = scratch();
+            if (!partial) return CTAMD_EINVAL;
+        } else {
+            splits = 1;
+        }
+    }
+    int kps = int((k + splits - 1) / splits);
+    kps = (kps + Tile::BK - 1) / Tile::BK * Tile::BK;
+    splits = int((k + kps - 1) / kps);
+    g.k_per_split = kps;
+    if (splits > 1) { g.c = partial; g.ldc = n; g.split_stride = m * n; }
+    else { g.c = c; g.ldc = n; g.split_stride = 0; }
+
+    int rc;
+    if (A_KC && B_KC) rc = launch_gemm<true, true>(g, vec, splits, s);
+    else if (A_KC) rc = launch_gemm<true, false>(g, vec, splits, s);
+    else if (B_KC) rc = launch_gemm<false, true>(g, vec, splits, s);
+    else rc = launch_gemm<false, false>(g, vec, splits, s);
+    if (rc || splits == 1) return rc;
+    size_t mn = size_t(m) * size_t(n);
+    hipLaunchKernelGGL(splitk_fold, dim3(unsigned((mn + kThreads - 1) / kThreads)), dim3(kThreads), 0, s, partial, c, mn,
+                       splits);
+    return launched(__func__);
+}

@@ -1,0 +1,124 @@
+// Runtime side of the C ABI: device selection, HBM allocation, explicit transfers, error text.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <mutex>
+
+#include "common.h"
+
+namespace ctamd {
+
+namespace {
+thread_local char g_err[512] = "";
+constexpr int kMaxDevices = 16;
+std::mutex g_mu;
+float* g_scratch[kMaxDevices] = {};
+int g_cus[kMaxDevices] = {};
+}  // namespace
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_hip(hipError_t e, const char* what) {
+    if (e == hipSuccess) return CTAMD_OK;
+    return fail(e == hipErrorOutOfMemory ? CTAMD_ENOMEM : CTAMD_EHIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+int launched(const char* kernel) { return check_hip(hipGetLastError(), kernel); }
+
+static int current_device() {
+    int d = -1;
+    if (hipGetDevice(&d) != hipSuccess) return -1;
+    return d;
+}
+
+float* scratch() {
+    int d = current_device();
+    if (d < 0 || d >= kMaxDevices || g_scratch[d] == nullptr) {
+        fail(CTAMD_EINVAL, "ctamd_init() has not been called for the current device");
+        return nullptr;
+    }
+    return g_scratch[d];
+}
+
+int compute_units() {
+    int d = current_device();
+    return (d < 0 || d >= kMaxDevices) ? 0 : g_cus[d];
+}
+
+}  // namespace ctamd
+
+using namespace ctamd;
+
+extern "C" {
+
+int ctamd_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return n;
+}
+
+int ctamd_init(int device) {
+    int n = ctamd_device_count();
+    if (n <= 0) return fail(CTAMD_ENODEV, "ctamd_init: no HIP device visible");
+    if (device < 0 || device >= n || device >= 16) return fail(CTAMD_EINVAL, "ctamd_init: device %d out of range", device);
+    int rc = check_hip(hipSetDevice(device), "hipSetDevice");
+    if (rc) return rc;
+    std::lock_guard<std::mutex> lock(g_mu);
+    if (g_scratch[device]) return CTAMD_OK;
+    hipDeviceProp_t prop;
+    rc = check_hip(hipGetDeviceProperties(&prop, device), "hipGetDeviceProperties");
+    if (rc) return rc;
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(CTAMD_ENODEV, "ctamd_init: device %d is %s; this library is built for gfx950 only", device,
+                    prop.gcnArchName);
+    g_cus[device] = prop.multiProcessorCount;
+    void* p = nullptr;
+    rc = check_hip(hipMalloc(&p, kScratchFloats * sizeof(float)), "hipMalloc(scratch)");
+    if (rc) return rc;
+    g_scratch[device] = static_cast<float*>(p);
+    return CTAMD_OK;
+}
+
+const char* ctamd_last_error(void) { return g_err; }
+const char* ctamd_version(void) { return "ctorch_amd 0.1 (gfx950)"; }
+
+int ctamd_malloc(void** ptr, size_t bytes) {
+    if (!ptr) return fail(CTAMD_EINVAL, "ctamd_malloc: null result pointer");
+    *ptr = nullptr;
+    if (bytes == 0) return CTAMD_OK;
+    return check_hip(hipMalloc(ptr, bytes), "hipMalloc");
+}
+
+int ctamd_free(void* ptr) {
+    if (!ptr) return CTAMD_OK;
+    return check_hip(hipFree(ptr), "hipFree");
+}
+
+static int copy(void* dst, const void* src, size_t bytes, hipMemcpyKind kind, void* stream, const char* what) {
+    if (bytes == 0) return CTAMD_OK;
+    if (!dst || !src) return fail(CTAMD_EINVAL, "%s: null pointer", what);
+    return check_hip(hipMemcpyAsync(dst, src, bytes, kind, as_stream(stream)), what);
+}
+
+int ctamd_memcpy_h2d(void* dst, const void* src_host, size_t bytes, void* stream) {
+    return copy(dst, src_host, bytes, hipMemcpyHostToDevice, stream, "ctamd_memcpy_h2d");
+}
+int ctamd_memcpy_d2h(void* dst_host, const void* src, size_t bytes, void* stream) {
+    return copy(dst_host, src, bytes, hipMemcpyDeviceToHost, stream, "ctamd_memcpy_d2h");
+}
+int ctamd_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream) {
+    return copy(dst, src, bytes, hipMemcpyDeviceToDevice, stream, "ctamd_memcpy_d2d");
+}
+int ctamd_sync(void* stream) { return check_hip(hipStreamSynchronize(as_stream(stream)), "hipStreamSynchronize"); }
+
+}  // extern "C"

@@ -1,0 +1,188 @@
+/* ctorch_amd - C ABI of the MI355X (gfx950) device backend for CTorch's operator set.
+ *
+ * One entry point per kernel the reference registers in Ctorch_Scheduler
+ * (include/Ctorch_Scheduler.h:30-53) or runs inline in its Tensor front-end / tape
+ * (src/Tensor.cpp, src/AutoDiff.cpp).  Each declaration cites the reference code it replaces
+ * (paths relative to the reference root).
+ *
+ * Conventions
+ *  - Every pointer is DEVICE memory (HBM) unless its name ends in _host.  All data is fp32,
+ *    row-major, contiguous unless strides are passed.  Counts are in elements.
+ *  - Launchers never allocate, free or synchronise: they enqueue on `stream` (a hipStream_t passed
+ *    as void*, NULL = the default stream) and return.  Results are ready after ctamd_sync(stream).
+ *  - Reductions use a per-device scratch buffer that ctamd_init() allocates once; calls that use
+ *    it must not overlap on different streams of one device.
+ *  - Return value: 0 on success, a negative CTAMD_E* code otherwise; ctamd_last_error() gives
+ *    the text.  No C++ exception crosses this boundary.  The C++ shim above maps codes to the
+ *    reference's two error conventions (Ctorch_Error::log / throwException,
+ *    include/Ctorch_Error.h:353-405, :510-515).
+ *  - n == 0 (and rows == 0 or cols == 0) is a successful no-op.
+ */
+#ifndef CTORCH_AMD_H
+#define CTORCH_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CTAMD_OK 0
+#define CTAMD_EINVAL (-1)   /* bad argument: null pointer, negative size, bad op code, shape mismatch */
+#define CTAMD_EHIP (-2)     /* the HIP runtime reported an error (launch, copy, allocation) */
+#define CTAMD_ENOMEM (-3)   /* device allocation failed */
+#define CTAMD_ENODEV (-4)   /* no gfx950 device visible */
+#define CTAMD_ERANGE (-5)   /* a size exceeds what the entry point supports */
+
+/* ------------------------------------------------------------------------------- runtime */
+
+/* Selects device `device`, checks it is a gfx950 part and allocates the reduction scratch.
+ * Idempotent.  Replaces the device gate Ctorch_Scheduler::isDeviceAvailable
+ * (include/Ctorch_Scheduler.h:67-75). */
+int ctamd_init(int device);
+int ctamd_device_count(void);
+const char* ctamd_last_error(void);
+const char* ctamd_version(void);
+
+/* Storage: device allocation and explicit transfers; replaces `new char[]` / memcpy in
+ * Storage (include/Storage.h:77, :175-181). */
+int ctamd_malloc(void** ptr, size_t bytes);
+int ctamd_free(void* ptr);
+int ctamd_memcpy_h2d(void* dst, const void* src_host, size_t bytes, void* stream);
+int ctamd_memcpy_d2h(void* dst_host, const void* src, size_t bytes, void* stream);
+int ctamd_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream);
+int ctamd_sync(void* stream);
+
+/* -------------------------------------------------------- elementwise binary (bit-exact) */
+/* r[i] = a[i] (op) b[i].  Add_BASIC_kernel.cpp:64-69, Sub_BASIC_kernel.cpp:58-60,
+ * Mul_BASIC_kernel.cpp:59-61, Div_BASIC_kernel.cpp:37-45 (IEEE quotient, also for b == 0). */
+int ctamd_add_f32(const float* a, const float* b, float* r, size_t n, void* stream);
+int ctamd_sub_f32(const float* a, const float* b, float* r, size_t n, void* stream);
+int ctamd_mul_f32(const float* a, const float* b, float* r, size_t n, void* stream);
+int ctamd_div_f32(const float* a, const float* b, float* r, size_t n, void* stream);
+
+/* r[i,j] = a[i,j] (op) b[j], a [rows, cols], b [cols].  Add_BASIC_kernel.cpp:27-29, :54-63.
+ * The reference has this form for Add only; Sub/Mul/Div follow the same convention here
+ * (the reference throws for Sub/Mul and reads out of bounds for Div:
+ * Sub_BASIC_kernel.cpp:35-43, Tensor.cpp:362-365, Div_BASIC_kernel.cpp:18-20). */
+int ctamd_add_rowbcast_f32(const float* a, const float* b, float* r, size_t rows, size_t cols, void* stream);
+int ctamd_sub_rowbcast_f32(const float* a, const float* b, float* r, size_t rows, size_t cols, void* stream);
+int ctamd_mul_rowbcast_f32(const float* a, const float* b, float* r, size_t rows, size_t cols, void* stream);
+int ctamd_div_rowbcast_f32(const float* a, const float* b, float* r, size_t rows, size_t cols, void* stream);
+
+/* r[i] = a[i] (op) b[0] with b a one-element DEVICE tensor.  Add_BASIC_kernel.cpp:48-53; for
+ * Sub/Mul the 0-D broadcast branch (Sub_BASIC_kernel.cpp:28-32, Mul_BASIC_kernel.cpp:27-34). */
+int ctamd_add_bscalar_f32(const float* a, const float* b1, float* r, size_t n, void* stream);
+int ctamd_sub_bscalar_f32(const float* a, const float* b1, float* r, size_t n, void* stream);
+int ctamd_mul_bscalar_f32(const float* a, const float* b1, float* r, size_t n, void* stream);
+int ctamd_div_bscalar_f32(const float* a, const float* b1, float* r, size_t n, void* stream);
+/* r[i] = a1[0] - b[i]: a 0-D left operand (Sub_BASIC_kernel.cpp:25-27), used by the tape for
+ * 1 - sigmoid(x) and 1 - tanh(x)^2 (src/AutoDiff.cpp:1379, :1393). */
+int ctamd_rsub_ascalar_f32(const float* a1, const float* b, float* r, size_t n, void* stream);
+
+/* r[i] = a[i] (op) s with s a HOST float.  Tensor::operator+(float) src/Tensor.cpp:855-910,
+ * operator*(float) :751-806, operator/(float) :913-973. */
+int ctamd_add_scalar_f32(const float* a, float s, float* r, size_t n, void* stream);
+int ctamd_mul_scalar_f32(const float* a, float s, float* r, size_t n, void* stream);
+int ctamd_div_scalar_f32(const float* a, float s, float* r, size_t n, void* stream);
+
+/* ---------------------------------------------------------------------- elementwise unary */
+/* Neg_BASIC_kernel.cpp:26-28 (sign-bit flip); ReLU_BASIC_kernel.cpp:23-25 (x > 0 ? x : +0, so
+ * -0 and NaN give +0): bit-exact. */
+int ctamd_neg_f32(const float* a, float* r, size_t n, void* stream);
+int ctamd_relu_f32(const float* a, float* r, size_t n, void* stream);
+/* Sin_BASIC_kernel.cpp:24-26, Cos_BASIC_kernel.cpp:23-25 (glibc sinf / cosf);
+ * Tanh_BASIC_kernel.cpp:24-28 ((e^x - e^-x) / (e^x + e^-x) in fp32);
+ * Sigmoid_BASIC_kernel.cpp:24-26 (1 / (1 + e^-x)).  The device evaluates the same formulas on
+ * exp/sin/cos that return glibc 2.35's floats (see ctorch_amd/csrc/devmath.h). */
+int ctamd_sin_f32(const float* a, float* r, size_t n, void* stream);
+int ctamd_cos_f32(const float* a, float* r, size_t n, void* stream);
+int ctamd_tanh_f32(const float* a, float* r, size_t n, void* stream);
+int ctamd_sigmoid_f32(const float* a, float* r, size_t n, void* stream);
+
+/* ------------------------------------------------------------------------------- reductions */
+/* out[0] = sum of a.  Tensor::sum() src/Tensor.cpp:638-666. */
+int ctamd_sum_f32(const float* a, float* out, size_t n, void* stream);
+/* out[0] = sum a[i]*b[i].  Dot_BASIC_kernel.cpp:38-41. */
+int ctamd_dot_f32(const float* a, const float* b, float* out, size_t n, void* stream);
+/* out[0] = sum (a-b)^2 / n and sum |a-b| / n.  MSE_BASIC_kernel.cpp:35-43, MAE_BASIC_kernel.cpp:35-43. */
+int ctamd_mse_f32(const float* a, const float* b, float* out, size_t n, void* stream);
+int ctamd_mae_f32(const float* a, const float* b, float* out, size_t n, void* stream);
+/* out[j] = sum_i g[i,j], g [rows, cols]: the complete gradient of a row-broadcast operand
+ * (the reference's check_and_adjust_grad_shape, src/AutoDiff.cpp:690-757, returns row 0 instead;
+ * that behaviour is a ctamd_memcpy_d2d of the first row followed by ctamd_accumulate_f32). */
+int ctamd_colsum_f32(const float* g, float* out, size_t rows, size_t cols, void* stream);
+/* flag[0] = 1 if any |b[i]| < FLT_EPSILON else 0: the divisor scan of Div's backward
+ * (src/AutoDiff.cpp:1267-1284). */
+int ctamd_any_abs_lt_eps_f32(const float* b, int32_t* flag, size_t n, void* stream);
+
+/* ---------------------------------------------------------------- softmax and cross entropy */
+/* Row softmax y[i,:] = softmax(x[i,:]) (dim 1 / 1-D with rows = 1) and column softmax (dim 0).
+ * Tensor::softmax src/Tensor.cpp:1713-1727, :1728-1744; Softmax_BASIC_kernel.cpp:72-93.
+ * exp(x - max) is bit-identical to the reference's, the row sum is a tree sum, and the
+ * normalisation is a true division as in the reference. */
+int ctamd_softmax_rows_f32(const float* x, float* y, size_t rows, size_t cols, void* stream);
+int ctamd_softmax_cols_f32(const float* x, float* y, size_t rows, size_t cols, void* stream);
+/* out[0] = SUM over rows of -sum_j t[i,j] * log(max(softmax(x)[i,j], 1e-10)).
+ * CrossEntropy_BASIC_kernel.cpp:41-66 (2-D one-hot or soft targets), :67-82 (1-D: rows = 1). */
+int ctamd_cross_entropy_onehot_f32(const float* x, const float* t, float* out, size_t rows, size_t cols,
+                                   void* stream);
+/* Class-index targets held as floats, truncated toward zero.  CrossEntropy_BASIC_kernel.cpp:88-120.
+ * status[0] is set to 1 when an index is out of range (the reference then returns an empty
+ * Tensor, :96-100) and out[0] is then NaN; status may be NULL. */
+int ctamd_cross_entropy_index_f32(const float* x, const float* idx, float* out, int32_t* status, size_t rows,
+                                  size_t cols, void* stream);
+
+/* -------------------------------------------------------------------------------- matmul */
+/* C[i,j] = sum_l A[i*as0 + l*as1] * B[l*bs0 + j*bs1]; C is [m, n] row-major contiguous; strides
+ * are in elements and may describe a transposed view.  MatMul_BASIC_kernel.cpp:42-54.  The
+ * reference's backward calls the same kernel with t() views: dA = g.matmul(B.t()),
+ * dB = A.t().matmul(g) (src/AutoDiff.cpp:1692-1704, :1808-1810).  fp32 MFMA with fp32
+ * accumulation; every operand layout with a unit stride in one dimension takes the MFMA path,
+ * anything else a generic strided kernel. */
+int ctamd_matmul_f32(const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,
+                     float* c, int64_t m, int64_t n, int64_t k, void* stream);
+
+/* ----------------------------------------------------------------- backward arithmetic */
+/* r[i] = v.  A 0-D gradient expanded to a shape: src/AutoDiff.cpp:579-592; also Tensor::zero()
+ * / ones() src/Tensor.cpp:390-451. */
+int ctamd_fill_f32(float* r, float v, size_t n, void* stream);
+/* r[i] = v1[0] with v1 on the device (the tape's root gradient and loss gradients stay in HBM). */
+int ctamd_fill_from_f32(float* r, const float* v1, size_t n, void* stream);
+/* grad[i] += val[i] in place.  src/AutoDiff.cpp:1870-1878. */
+int ctamd_accumulate_f32(float* grad, const float* val, size_t n, void* stream);
+/* dx = g * (x > 0 ? 1 : 0) as a multiply, so g*0 keeps its sign and NaN/inf propagate.
+ * src/AutoDiff.cpp:1334-1341, :1370. */
+int ctamd_relu_backward_f32(const float* x, const float* g, float* dx, size_t n, void* stream);
+/* s = sigmoid(x); dx = (s * (1 - s)) * g.  src/AutoDiff.cpp:1372-1383. */
+int ctamd_sigmoid_backward_f32(const float* x, const float* g, float* dx, size_t n, void* stream);
+/* t = tanh(x); dx = (1 - t*t) * g.  src/AutoDiff.cpp:1384-1398. */
+int ctamd_tanh_backward_f32(const float* x, const float* g, float* dx, size_t n, void* stream);
+/* dx = cos(x) * g; dx = (-sin(x)) * g.  src/AutoDiff.cpp:1399-1407, :1408-1416. */
+int ctamd_sin_backward_f32(const float* x, const float* g, float* dx, size_t n, void* stream);
+int ctamd_cos_backward_f32(const float* x, const float* g, float* dx, size_t n, void* stream);
+/* dx = y * (g - sum_j g*y) per row (dim 1) or per column (dim 0), y the stored softmax output.
+ * src/AutoDiff.cpp:1462-1472, :1473-1484. */
+int ctamd_softmax_backward_rows_f32(const float* y, const float* g, float* dx, size_t rows, size_t cols,
+                                    void* stream);
+int ctamd_softmax_backward_cols_f32(const float* y, const float* g, float* dx, size_t rows, size_t cols,
+                                    void* stream);
+/* dp = (((p - t) * 2) / n) * g[0]; dp = (sign(p - t) / n) * g[0]; g a 0-D device tensor.
+ * src/AutoDiff.cpp:1491-1516, :1602-1642. */
+int ctamd_mse_backward_f32(const float* p, const float* t, const float* g1, float* dp, size_t n, void* stream);
+int ctamd_mae_backward_f32(const float* p, const float* t, const float* g1, float* dp, size_t n, void* stream);
+/* dx = (softmax(x) - t) * g[0], gradient of the SUM-reduced loss.  src/AutoDiff.cpp:1546-1574.
+ * The index form takes class indices (the reference throws there, :1569) and equals the one-hot
+ * arithmetic with t = onehot(idx). */
+int ctamd_cross_entropy_backward_onehot_f32(const float* x, const float* t, const float* g1, float* dx,
+                                            size_t rows, size_t cols, void* stream);
+int ctamd_cross_entropy_backward_index_f32(const float* x, const float* idx, const float* g1, float* dx,
+                                           size_t rows, size_t cols, void* stream);
+/* db = ((-a) * g) / (b * b).  src/AutoDiff.cpp:1314.  (da = g / b is ctamd_div_f32, :1285.) */
+int ctamd_div_backward_b_f32(const float* a, const float* b, const float* g, float* db, size_t n, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CTORCH_AMD_H */

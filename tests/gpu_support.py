@@ -1,0 +1,191 @@
+"""GPU-side test plumbing: torch provides device memory, every computation goes through the
+C ABI of ctorch_amd/libctorch_amd.so (ctypes), nothing else."""
+import ctypes as C
+
+import numpy as np
+import torch
+
+from ctorch_amd import capi
+
+DEV = "cuda:0"
+_inited = False
+
+
+def lib():
+    global _inited
+    l = capi.load()
+    if not _inited:
+        torch.cuda.init()
+        torch.zeros(1, device=DEV)   # torch's context on device 0 first; the library shares it
+        capi.check(l.ctamd_init(0))
+        _inited = True
+    return l
+
+
+def dev(a):
+    """numpy fp32 array -> device tensor (keeps shape)."""
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(DEV)
+
+
+def host(t):
+    return t.detach().cpu().numpy()
+
+
+def ptr(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(0)
+
+
+def stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def empty_like(t):
+    return torch.empty_like(t)
+
+
+def call(name, *args):
+    capi.check(getattr(lib(), name)(*args))
+
+
+def binary(op, a, b):
+    r = torch.empty_like(a)
+    call("ctamd_%s_f32" % op, ptr(a), ptr(b), ptr(r), a.numel(), stream())
+    return r
+
+
+def rowbcast(op, a, b):
+    r = torch.empty_like(a)
+    call("ctamd_%s_rowbcast_f32" % op, ptr(a), ptr(b), ptr(r), a.shape[0], a.shape[1], stream())
+    return r
+
+
+def bscalar(op, a, b1):
+    r = torch.empty_like(a)
+    call("ctamd_%s_bscalar_f32" % op, ptr(a), ptr(b1), ptr(r), a.numel(), stream())
+    return r
+
+
+def rsub(a1, b):
+    r = torch.empty_like(b)
+    call("ctamd_rsub_ascalar_f32", ptr(a1), ptr(b), ptr(r), b.numel(), stream())
+    return r
+
+
+def scalar(op, a, s):
+    r = torch.empty_like(a)
+    call("ctamd_%s_scalar_f32" % op, ptr(a), C.c_float(s), ptr(r), a.numel(), stream())
+    return r
+
+
+def unary(op, a):
+    r = torch.empty_like(a)
+    call("ctamd_%s_f32" % op, ptr(a), ptr(r), a.numel(), stream())
+    return r
+
+
+def unary_bwd(op, x, g):
+    r = torch.empty_like(x)
+    call("ctamd_%s_backward_f32" % op, ptr(x), ptr(g), ptr(r), x.numel(), stream())
+    return r
+
+
+def reduce1(name, a):
+    out = torch.empty(1, device=DEV)
+    call("ctamd_%s_f32" % name, ptr(a), ptr(out), a.numel(), stream())
+    return out
+
+
+def reduce2(name, a, b):
+    out = torch.empty(1, device=DEV)
+    call("ctamd_%s_f32" % name, ptr(a), ptr(b), ptr(out), a.numel(), stream())
+    return out
+
+
+def colsum(g):
+    out = torch.empty(g.shape[1], device=DEV)
+    call("ctamd_colsum_f32", ptr(g), ptr(out), g.shape[0], g.shape[1], stream())
+    return out
+
+
+def any_tiny(b):
+    flag = torch.full((1,), -7, dtype=torch.int32, device=DEV)
+    call("ctamd_any_abs_lt_eps_f32", ptr(b), ptr(flag), b.numel(), stream())
+    return int(flag.item())
+
+
+def softmax(x, dim=1):
+    y = torch.empty_like(x)
+    rows, cols = (1, x.numel()) if x.dim() == 1 else x.shape
+    name = "ctamd_softmax_rows_f32" if (x.dim() == 1 or dim == 1) else "ctamd_softmax_cols_f32"
+    call(name, ptr(x), ptr(y), rows, cols, stream())
+    return y
+
+
+def softmax_bwd(y, g, dim=1):
+    dx = torch.empty_like(y)
+    rows, cols = (1, y.numel()) if y.dim() == 1 else y.shape
+    name = "ctamd_softmax_backward_rows_f32" if (y.dim() == 1 or dim == 1) else "ctamd_softmax_backward_cols_f32"
+    call(name, ptr(y), ptr(g), ptr(dx), rows, cols, stream())
+    return dx
+
+
+def ce_onehot(x, t):
+    out = torch.empty(1, device=DEV)
+    rows, cols = (1, x.numel()) if x.dim() == 1 else x.shape
+    call("ctamd_cross_entropy_onehot_f32", ptr(x), ptr(t), ptr(out), rows, cols, stream())
+    return out
+
+
+def ce_index(x, idx):
+    out = torch.empty(1, device=DEV)
+    status = torch.full((1,), -7, dtype=torch.int32, device=DEV)
+    call("ctamd_cross_entropy_index_f32", ptr(x), ptr(idx), ptr(out), ptr(status), x.shape[0], x.shape[1], stream())
+    return out, int(status.item())
+
+
+def ce_bwd(x, t, g1, index):
+    dx = torch.empty_like(x)
+    rows, cols = (1, x.numel()) if x.dim() == 1 else x.shape
+    name = "ctamd_cross_entropy_backward_%s_f32" % ("index" if index else "onehot")
+    call(name, ptr(x), ptr(t), ptr(g1), ptr(dx), rows, cols, stream())
+    return dx
+
+
+def loss_bwd(name, p, t, g1):
+    dp = torch.empty_like(p)
+    call("ctamd_%s_backward_f32" % name, ptr(p), ptr(t), ptr(g1), ptr(dp), p.numel(), stream())
+    return dp
+
+
+def div_bwd_b(a, b, g):
+    r = torch.empty_like(a)
+    call("ctamd_div_backward_b_f32", ptr(a), ptr(b), ptr(g), ptr(r), a.numel(), stream())
+    return r
+
+
+def fill(n, v):
+    r = torch.empty(n, device=DEV)
+    call("ctamd_fill_f32", ptr(r), C.c_float(v), n, stream())
+    return r
+
+
+def fill_from(n, v1):
+    r = torch.empty(n, device=DEV)
+    call("ctamd_fill_from_f32", ptr(r), ptr(v1), n, stream())
+    return r
+
+
+def accumulate(grad, val):
+    call("ctamd_accumulate_f32", ptr(grad), ptr(val), grad.numel(), stream())
+    return grad
+
+
+def matmul(a, b):
+    """a, b: 2-D device tensors, possibly transposed views (strides are passed through)."""
+    m, k = a.shape
+    k2, n = b.shape
+    assert k == k2
+    c = torch.empty((m, n), device=DEV)
+    call("ctamd_matmul_f32", ptr(a), a.stride(0), a.stride(1), ptr(b), b.stride(0), b.stride(1), ptr(c), m, n, k,
+         stream())
+    return c

@@ -1,0 +1,55 @@
+/* Host check of ctorch_amd/csrc/devmath.h against the installed glibc: counts the floats for
+ * which the device algorithms (compiled here for the CPU, unchanged) return different bits from
+ * expf / sinf / cosf.  Usage: devmath_check STRIDE  (1 = every one of the 2^32 bit patterns).
+ * Prints one line per function: name, inputs tested, mismatches, worst ulp distance. */
+#include <math.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+
+#include "../../ctorch_amd/csrc/devmath.h"
+
+static int64_t ulpkey(float f) {
+    int32_t i = (int32_t)cta_f2u(f);
+    return i < 0 ? -(int64_t)(i & 0x7fffffff) : i;
+}
+static int differs(float a, float b, int64_t* ulp) {
+    if (a != a && b != b) return 0;
+    if (cta_f2u(a) == cta_f2u(b)) return 0;
+    int64_t d = ulpkey(a) - ulpkey(b);
+    *ulp = d < 0 ? -d : d;
+    return 1;
+}
+
+int main(int argc, char** argv) {
+    uint64_t stride = argc > 1 ? strtoull(argv[1], 0, 10) : 1;
+    if (stride == 0) stride = 1;
+    uint64_t n = 0, bad[3] = {0, 0, 0}, covered[3] = {0, 0, 0};
+    int64_t worst[3] = {0, 0, 0};
+#pragma omp parallel for reduction(+ : n, bad[:3], covered[:3]) reduction(max : worst[:3]) schedule(static)
+    for (uint64_t u = 0; u < (1ULL << 32); u += stride) {
+        float x = cta_u2f((uint32_t)u);
+        int64_t d = 0;
+        ++n;
+        ++covered[0];
+        if (differs(cta_expf_tab(x, cta_exp2_tab), expf(x), &d)) {
+            ++bad[0];
+            if (d > worst[0]) worst[0] = d;
+        }
+        ++covered[1];
+        if (differs(cta_sincosf(x, 0, cta_inv_pio4), sinf(x), &d)) {
+            ++bad[1];
+            if (d > worst[1]) worst[1] = d;
+        }
+        ++covered[2];
+        if (differs(cta_sincosf(x, 1, cta_inv_pio4), cosf(x), &d)) {
+            ++bad[2];
+            if (d > worst[2]) worst[2] = d;
+        }
+    }
+    const char* names[3] = {"expf", "sinf", "cosf"};
+    for (int k = 0; k < 3; ++k)
+        printf("%s tested %llu mismatches %llu worst_ulp %lld\n", names[k], (unsigned long long)covered[k],
+               (unsigned long long)bad[k], (long long)worst[k]);
+    return 0;
+}

@@ -1,0 +1,330 @@
+"""Parity of the HIP path with the CPU oracle, through the C ABI, on the same seeded inputs.
+
+Bars: bit-exact for Add/Sub/Mul/Div/Neg/ReLU, their broadcast and scalar forms and the
+gradient multiplies; <= 2 ulp for Sin/Cos/Tanh/Sigmoid and their gradients (the device routines
+are built to return glibc's floats, so the golden vectors written from the real reference are
+also required to match to <= 2 ulp, and the fraction of exact matches is printed);
+|x - y| <= 1e-5 * sum|terms| for reductions, MatMul, softmax and cross entropy, with fp64 as the
+arbiter."""
+import numpy as np
+import pytest
+import torch
+
+import gpu_support as G
+from support import (ADD, COS, DIV, MUL, NEG, RELU, SIGMOID, SIN, SUB, TANH, same_bits, ulp_diff)
+
+pytestmark = pytest.mark.gpu
+
+F = np.float32
+BIN = [("add", ADD), ("sub", SUB), ("mul", MUL), ("div", DIV)]
+SPECIAL = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 3.4e38, -3.4e38, 1e-38, -1e-38,
+                    88.8, -88.8, 100.0, -100.0, 1.0, -1.0, 0.5, -0.5, 1e-3, -1e-3, 1e-6, 20.0, -20.0,
+                    3.14159274, 1.57079637, 6.28318548, 1e4, -1e4, 1e7, 1e22, 87.3, -87.3, 103.9, 200.0, -200.0,
+                    119.9, 120.0, 120.1, 0.74, 0.75, 0.76, 2.4e-4, 2.5e-4], F)
+
+
+def bits_equal(got, want, what=""):
+    got, want = np.asarray(got, F), np.asarray(want, F)
+    nan_both = np.isnan(got) & np.isnan(want)
+    bad = (got.view(np.uint32) != want.view(np.uint32)) & ~nan_both
+    assert not bad.any(), f"{what}: {bad.sum()} of {bad.size} elements differ, first at {np.argmax(bad)}"
+
+
+def ulp_close(got, want, max_ulp, what=""):
+    got, want = np.asarray(got, F), np.asarray(want, F)
+    assert np.array_equal(np.isnan(got), np.isnan(want)), f"{what}: NaN pattern differs"
+    ok = ~np.isnan(want)
+    d = ulp_diff(got[ok], want[ok])
+    exact = float((d == 0).mean()) if d.size else 1.0
+    print(f"{what}: max ulp {d.max() if d.size else 0}, exact {exact:.6f}")
+    assert d.size == 0 or d.max() <= max_ulp, f"{what}: max ulp {d.max()}"
+
+
+@pytest.mark.parametrize("n", [0, 1, 3, 4, 5, 1023, 4099, (1 << 20) + 3])
+def test_binary_same_shape_bit_exact(oracle, n):
+    print("case binary n", n, flush=True)
+    a = np.concatenate([oracle.normal((n,), 1, 0, 3)])
+    b = np.concatenate([oracle.normal((n,), 2, 0, 3)])
+    if n >= SPECIAL.size:
+        a[:SPECIAL.size] = SPECIAL
+        b[:SPECIAL.size] = SPECIAL[::-1]
+    da, db = G.dev(a), G.dev(b)
+    for name, code in BIN:
+        bits_equal(G.host(G.binary(name, da, db)), oracle.binary(code, a, b), name)
+
+
+def test_binary_unaligned_views_bit_exact(oracle):
+    print("case binary unaligned", flush=True)
+    a = oracle.normal((5003,), 3, 0, 2)
+    b = oracle.normal((5003,), 4, 0, 2)
+    da, db = G.dev(a), G.dev(b)
+    for off in (1, 2, 3):
+        got = G.binary("mul", da[off:], db[off:].clone())   # first operand off the 16-byte grid
+        bits_equal(G.host(got), oracle.mul(a[off:], b[off:]), f"offset {off}")
+
+
+@pytest.mark.parametrize("shape", [(37, 53), (8, 256), (5, 10), (64, 4096), (1, 7), (300, 1)])
+def test_row_broadcast_bit_exact(oracle, shape):
+    print("case rowbcast", shape, flush=True)
+    a = oracle.normal(shape, 5, 0, 2)
+    b = oracle.uniform((shape[1],), 6, 0.5, 2)
+    da, db = G.dev(a), G.dev(b)
+    for name, code in BIN:
+        bits_equal(G.host(G.rowbcast(name, da, db)), oracle.binary_rowbcast(code, a, b), name)
+
+
+def test_scalar_forms_bit_exact(oracle):
+    print("case scalar forms", flush=True)
+    a = np.concatenate([oracle.normal((4099,), 7, 0, 3), SPECIAL])
+    da = G.dev(a)
+    s = F(1.7)
+    ds = G.dev(np.array([s]))
+    full = np.full_like(a, s)
+    for name, code in BIN:
+        bits_equal(G.host(G.bscalar(name, da, ds)), oracle.binary(code, a, full), "bscalar " + name)
+    bits_equal(G.host(G.rsub(ds, da)), oracle.sub(full, a), "rsub")
+    bits_equal(G.host(G.scalar("add", da, 5.0)), oracle.scalar(0, a, 5.0), "scalar add")
+    bits_equal(G.host(G.scalar("mul", da, -2.5)), oracle.scalar(1, a, -2.5), "scalar mul")
+    bits_equal(G.host(G.scalar("div", da, 3.0)), oracle.scalar(2, a, 3.0), "scalar div")
+
+
+def test_neg_relu_fill_accumulate_bit_exact(oracle):
+    print("case neg relu fill accumulate", flush=True)
+    a = np.concatenate([oracle.normal((70001,), 8, 0, 3), SPECIAL])
+    da = G.dev(a)
+    bits_equal(G.host(G.unary("neg", da)), oracle.neg(a), "neg")
+    r = G.host(G.unary("relu", da))
+    want = oracle.relu(a)
+    assert same_bits(r, want), "relu"          # NaN -> +0 here, so plain bit equality
+    assert np.all(G.host(G.fill(1001, 2.5)) == F(2.5))
+    assert np.all(G.host(G.fill_from(1001, G.dev(np.array([-0.75])))) == F(-0.75))
+    g = oracle.normal((70001,), 9)
+    v = oracle.normal((70001,), 10)
+    want = g.copy()
+    oracle.lib.co_accumulate(want.ctypes.data_as(G.C.POINTER(G.C.c_float)),
+                             v.ctypes.data_as(G.C.POINTER(G.C.c_float)), G.C.c_long(g.size))
+    bits_equal(G.host(G.accumulate(G.dev(g), G.dev(v))), want, "accumulate")
+
+
+def test_transcendentals_within_2ulp(oracle):
+    print("case transcendentals", flush=True)
+    x = np.concatenate([oracle.uniform((200000,), 11, -2, 2), oracle.uniform((50000,), 12, -0.02, 0.02),
+                        oracle.uniform((50000,), 13, -90, 90), oracle.uniform((50000,), 14, -1000, 1000),
+                        oracle.normal((50000,), 15, 0, 1e6), SPECIAL])
+    dx = G.dev(x)
+    for name, code in [("sin", SIN), ("cos", COS), ("tanh", TANH), ("sigmoid", SIGMOID)]:
+        ulp_close(G.host(G.unary(name, dx)), oracle.unary(code, x), 2, name)
+
+
+def test_transcendentals_against_golden_reference_vectors(golden):
+    print("case transcendentals golden", flush=True)
+    g = golden("elementwise")
+    for key_in, names in (("x", ["sin", "cos", "tanh", "sigmoid"]), ("t", ["t_sin", "t_cos", "t_tanh", "t_sigmoid"])):
+        dx = G.dev(g[key_in])
+        for nm in names:
+            ulp_close(G.host(G.unary(nm.replace("t_", ""), dx)), g[nm], 2, "golden " + nm)
+    x, y = G.dev(g["x"]), G.dev(g["y"])
+    for name in ("add", "sub", "mul", "div"):
+        bits_equal(G.host(G.binary(name, x, y)), g[name], "golden " + name)
+    bits_equal(G.host(G.unary("neg", x)), g["neg"], "golden neg")
+    assert same_bits(G.host(G.unary("relu", x)), g["relu"])
+
+
+def test_elementwise_gradients(oracle):
+    print("case elementwise gradients", flush=True)
+    x = np.concatenate([oracle.normal((50001,), 16, 0, 2), SPECIAL[:32]])
+    g = np.concatenate([oracle.normal((50001,), 17), SPECIAL[:32][::-1]])
+    dx, dg = G.dev(x), G.dev(g)
+    bits_equal(G.host(G.unary_bwd("relu", dx, dg)), oracle.relu_bwd(x, g), "relu bwd")
+    for name, code in [("sigmoid", SIGMOID), ("tanh", TANH), ("sin", SIN), ("cos", COS)]:
+        ulp_close(G.host(G.unary_bwd(name, dx, dg)), oracle.unary_bwd(code, x, g), 2, name + " bwd")
+    p = oracle.normal((50001,), 18, 0, 2)
+    t = oracle.normal((50001,), 19, 0, 2)
+    t[:100] = p[:100]           # exact ties: sign(0) = 0
+    g1 = G.dev(np.array([0.37]))
+    bits_equal(G.host(G.loss_bwd("mse", G.dev(p), G.dev(t), g1)), oracle.mse_bwd(p, t, F(0.37)), "mse bwd")
+    bits_equal(G.host(G.loss_bwd("mae", G.dev(p), G.dev(t), g1)), oracle.mae_bwd(p, t, F(0.37)), "mae bwd")
+    b = (t + F(4.0) * np.sign(t) + F(0.5)).astype(F)
+    bits_equal(G.host(G.div_bwd_b(G.dev(p), G.dev(b), G.dev(g[:50001]))), oracle.div_bwd_b(p, b, g[:50001]), "div bwd b")
+    assert G.any_tiny(G.dev(b)) == 0
+    b[777] = 1e-8
+    assert G.any_tiny(G.dev(b)) == 1 and oracle.any_abs_lt_eps(b)
+
+
+@pytest.mark.parametrize("n", [0, 1, 5, 1000, 65537, (1 << 22) + 1])
+def test_reductions_normwise(oracle, n):
+    print("case reductions n", n, flush=True)
+    a = oracle.uniform((n,), 21, -1, 1)
+    b = oracle.uniform((n,), 22, -1, 1)
+    da, db = G.dev(a), G.dev(b)
+    a64, b64 = a.astype(np.float64), b.astype(np.float64)
+    cases = [("sum", G.host(G.reduce1("sum", da))[0], a64.sum(), np.abs(a64).sum()),
+             ("dot", G.host(G.reduce2("dot", da, db))[0], a64 @ b64, np.abs(a64 * b64).sum())]
+    if n:
+        cases += [("mse", G.host(G.reduce2("mse", da, db))[0], ((a64 - b64) ** 2).mean(), ((a64 - b64) ** 2).mean()),
+                  ("mae", G.host(G.reduce2("mae", da, db))[0], np.abs(a64 - b64).mean(), np.abs(a64 - b64).mean())]
+    for name, got, want, scale in cases:
+        assert abs(got - want) <= 1e-5 * scale + 1e-30, (name, got, want)
+    if 0 < n <= 70000:   # the oracle's sequential sums agree to the same bound
+        assert abs(G.host(G.reduce2("dot", da, db))[0] - oracle.dot(a, b)) <= 1e-5 * np.abs(a64 * b64).sum()
+        assert abs(G.host(G.reduce2("mse", da, db))[0] - oracle.mse(a, b)) <= 1e-5 * oracle.mse(a, b)
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (2, 3), (37, 53), (8192, 256), (1000, 10), (4096, 4096), (33, 4100), (70000, 3)])
+def test_column_sum(oracle, shape):
+    print("case colsum", shape, flush=True)
+    g = oracle.normal(shape, 23)
+    got = G.host(G.colsum(G.dev(g)))
+    want = g.astype(np.float64).sum(0)
+    assert np.all(np.abs(got - want) <= 1e-5 * np.abs(g).astype(np.float64).sum(0))
+    if shape[0] * shape[1] < 1 << 16:
+        assert np.all(np.abs(got - oracle.colsum_f64(g)) <= 1e-5 * np.abs(g).astype(np.float64).sum(0))
+
+
+SOFTMAX_SHAPES = [(1, 1), (3, 7), (19, 301), (64, 10), (5, 1000), (7, 1024), (4, 2052), (3, 8192), (2, 8200),
+                  (2, 32000), (2, 32768), (2, 33000), (3, 40001)]
+
+
+@pytest.mark.parametrize("shape", SOFTMAX_SHAPES)
+def test_softmax_and_cross_entropy_rows(oracle, shape):
+    print("case softmax/ce", shape, flush=True)
+    rows, cols = shape
+    x = oracle.normal(shape, 24, 0, 2)
+    dx = G.dev(x)
+    y = G.host(G.softmax(dx, 1))
+    want = oracle.softmax(x, 1)
+    # same exp() bits; only the order of the row sum differs (tree here, sequential fp32 in the
+    # reference), which scales a whole row by 1 + O(cols * 2^-24): 1e-5 relative, fp64 as arbiter
+    x64 = x.astype(np.float64)
+    e64 = np.exp(x64 - x64.max(1, keepdims=True))
+    y64 = e64 / e64.sum(1, keepdims=True)
+    assert np.all(np.abs(y - y64) <= 1e-5 * y64 + 1e-45)
+    assert np.all(np.abs(y - want) <= 1e-5 * want + 1e-45)
+    assert np.allclose(y.astype(np.float64).sum(1), 1, atol=1e-5)
+    idx = oracle.ints((rows,), 25, cols)
+    oh = np.zeros(shape, F)
+    oh[np.arange(rows), idx.astype(int)] = 1
+    loss_i, status = G.ce_index(dx, G.dev(idx))
+    assert status == 0
+    loss_o = G.ce_onehot(dx, G.dev(oh))
+    want_loss = oracle.ce_index(x, idx) if rows != cols else oracle.ce_onehot(x, oh)
+    for got in (G.host(loss_i)[0], G.host(loss_o)[0]):
+        assert abs(got - want_loss) <= 1e-5 * abs(want_loss) + 1e-6
+    soft = oracle.softmax(oracle.normal(shape, 26), 1)
+    got = G.host(G.ce_onehot(dx, G.dev(soft)))[0]
+    assert abs(got - oracle.ce_onehot(x, soft)) <= 1e-5 * abs(oracle.ce_onehot(x, soft)) + 1e-6
+    g1 = G.dev(np.array([-1.25]))
+    want_d = oracle.ce_bwd_onehot(x, oh, F(-1.25))
+    for got in (G.host(G.ce_bwd(dx, G.dev(oh), g1, False)), G.host(G.ce_bwd(dx, G.dev(idx), g1, True))):
+        assert np.abs(got - want_d).max() <= 1e-6
+    w = oracle.normal(shape, 27)
+    got = G.host(G.softmax_bwd(G.dev(want), G.dev(w), 1))
+    want_b = oracle.softmax_bwd(want, w, 1)
+    scale = (np.abs(want) * (np.abs(w) + np.abs(w * want).sum(1, keepdims=True))).astype(np.float64)
+    assert np.all(np.abs(got - want_b) <= 1e-5 * scale + 1e-12)
+
+
+def test_cross_entropy_edge_cases(oracle):
+    print("case ce edges", flush=True)
+    x = oracle.normal((19, 31), 28, 0, 2)
+    idx = oracle.ints((19,), 29, 31)
+    bad = idx.copy()
+    bad[3] = 31
+    loss, status = G.ce_index(G.dev(x), G.dev(bad))
+    assert status == 1 and np.isnan(G.host(loss)[0]) and oracle.ce_index(x, bad) is None
+    bad[3] = -1
+    assert G.ce_index(G.dev(x), G.dev(bad))[1] == 1
+    # the 1e-10 clamp
+    hx = x.copy()
+    hx[:, 0] += 60.0
+    oh = np.zeros_like(x)
+    oh[np.arange(19), idx.astype(int)] = 1
+    want = oracle.ce_onehot(hx, oh)
+    assert abs(G.host(G.ce_onehot(G.dev(hx), G.dev(oh)))[0] - want) <= 1e-5 * abs(want)
+    assert abs(G.host(G.ce_index(G.dev(hx), G.dev(idx))[0])[0] - want) <= 1e-5 * abs(want)
+    # 1-D logits (single sample)
+    want = oracle.ce_onehot(x[0], oh[0])
+    assert abs(G.host(G.ce_onehot(G.dev(x[0]), G.dev(oh[0])))[0] - want) <= 1e-5 * abs(want)
+    # rows == 0 gives a zero loss
+    assert G.host(G.ce_onehot(G.dev(np.zeros((0, 5), F)), G.dev(np.zeros((0, 5), F))))[0] == 0
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (3, 7), (37, 53), (301, 19), (1000, 300)])
+def test_softmax_columns(oracle, shape):
+    print("case softmax cols", shape, flush=True)
+    x = oracle.normal(shape, 30, 0, 2)
+    y = G.host(G.softmax(G.dev(x), 0))
+    want = oracle.softmax(x, 0)
+    assert ulp_diff(y, want).max() <= 2
+    w = oracle.normal(shape, 31)
+    got = G.host(G.softmax_bwd(G.dev(want), G.dev(w), 0))
+    bits_equal(got, oracle.softmax_bwd(want, w, 0), "softmax bwd cols")   # same sequential fma chain
+
+
+MM_SHAPES = [(1, 1, 1), (5, 3, 9), (33, 29, 47), (128, 128, 16), (130, 257, 70), (256, 10, 784), (64, 256, 10),
+             (784, 256, 300), (256, 10, 8192), (17, 1, 33), (1, 40, 33), (200, 200, 1), (384, 512, 1024)]
+
+
+@pytest.mark.parametrize("m,n,k", MM_SHAPES)
+def test_matmul_all_layouts_normwise(oracle, m, n, k):
+    print("case matmul", m, n, k, flush=True)
+    A = oracle.normal((m, k), 41)
+    B = oracle.normal((k, n), 42)
+    dA, dB = G.dev(A), G.dev(B)
+    dAt, dBt = G.dev(np.ascontiguousarray(A.T)), G.dev(np.ascontiguousarray(B.T))
+    C64 = A.astype(np.float64) @ B.astype(np.float64)
+    bound = 1e-5 * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64)) + 1e-30
+    small = m * n * k <= 1 << 22
+    want = oracle.matmul(A, B) if small else None
+    for name, a, b in [("nn", dA, dB), ("nt", dA, dBt.t()), ("tn", dAt.t(), dB), ("tt", dAt.t(), dBt.t())]:
+        got = G.host(G.matmul(a, b))
+        assert np.all(np.abs(got - C64) <= bound), name
+        if small:
+            assert np.all(np.abs(got - want) <= 2 * bound), name
+
+
+def test_matmul_exact_on_small_integers_and_unaligned_views(oracle):
+    print("case matmul integers", flush=True)
+    rng = np.random.default_rng(7)
+    A = rng.integers(-8, 9, (150, 203)).astype(F)
+    B = rng.integers(-8, 9, (203, 77)).astype(F)
+    want = (A.astype(np.int64) @ B.astype(np.int64)).astype(F)
+    assert np.array_equal(G.host(G.matmul(G.dev(A), G.dev(B))), want)        # ld 203 / 77: scalar loads
+    # row-sliced views: unit inner stride, leading dimension larger than the extent
+    Abig, Bbig = G.dev(np.pad(A, ((0, 0), (0, 5)))), G.dev(np.pad(B, ((0, 0), (0, 3))))
+    assert np.array_equal(G.host(G.matmul(Abig[:, :203], Bbig[:, :77])), want)
+    # no unit stride at all: generic kernel
+    A2, B2 = G.dev(np.repeat(A, 2, axis=1)), G.dev(np.repeat(B, 2, axis=1))
+    At2 = G.dev(np.repeat(np.ascontiguousarray(A.T), 2, axis=1))
+    assert np.array_equal(G.host(G.matmul(A2[:, ::2], B2[:, ::2])), want)
+    assert np.array_equal(G.host(G.matmul(At2[:, ::2].t(), B2[:, ::2])), want)
+
+
+def test_golden_reference_vectors_reductions_matmul_backward(golden, oracle):
+    print("case golden reductions/matmul/backward", flush=True)
+    g = golden("reduce_softmax_ce")
+    v1, v2 = G.dev(g["v1"]), G.dev(g["v2"])
+    a64, b64 = g["v1"].astype(np.float64), g["v2"].astype(np.float64)
+    assert abs(G.host(G.reduce2("dot", v1, v2))[0] - g["dot"]) <= 1e-5 * np.abs(a64 * b64).sum()
+    assert abs(G.host(G.reduce2("mse", v1, v2))[0] - g["mse"]) <= 1e-5 * g["mse"]
+    assert abs(G.host(G.reduce2("mae", v1, v2))[0] - g["mae"]) <= 1e-5 * g["mae"]
+    assert abs(G.host(G.reduce1("sum", v1))[0] - g["sum"]) <= 1e-5 * np.abs(a64).sum()
+    sx = G.dev(g["sx"])
+    assert np.all(np.abs(G.host(G.softmax(sx, 1)) - g["softmax_d1"]) <= 1e-5 * g["softmax_d1"])
+    assert ulp_diff(G.host(G.softmax(sx, 0)), g["softmax_d0"]).max() <= 2
+    assert abs(G.host(G.ce_index(sx, G.dev(g["idx"]))[0])[0] - g["ce_index"]) <= 1e-5 * g["ce_index"]
+    m = golden("matmul")
+    A, B = m["A"], m["B"]
+    bound = 1e-5 * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64))
+    assert np.all(np.abs(G.host(G.matmul(G.dev(A), G.dev(B))) - m["nn"]) <= 2 * bound)
+    b = golden("backward")
+    x, w = b["x"], b["w"]
+    dx, dw = G.dev(x), G.dev(w)
+    bits_equal(G.host(G.unary_bwd("relu", dx, dw)) + F(0), b["d_relu"], "golden relu bwd")
+    for name in ("sigmoid", "tanh", "sin", "cos"):
+        ulp_close(G.host(G.unary_bwd(name, dx, dw)) + F(0), b["d_" + name], 2, "golden bwd " + name)
+    g1 = G.dev(np.array([0.37]))
+    bits_equal(G.host(G.loss_bwd("mse", dx, G.dev(b["y"]), g1)) + F(0), b["d_mse"], "golden mse bwd")
+    bits_equal(G.host(G.loss_bwd("mae", dx, G.dev(b["y"]), g1)) + F(0), b["d_mae"], "golden mae bwd")
+    bits_equal(G.host(G.binary("div", dw, G.dev(b["yb"]))) + F(0), b["d_div_a"], "golden div bwd a")
+    bits_equal(G.host(G.div_bwd_b(dx, G.dev(b["yb"]), dw)) + F(0), b["d_div_b"], "golden div bwd b")
