@@ -1,0 +1,197 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X hot path through the C ABI (ctorch_amd/libctorch_amd.so).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = one pass of BASELINE.json's configs[1] at its largest size, inputs resident in HBM:
+    C  = A . B            (4096^3 fp32 MatMul, forward)
+    dA = dC . B^T         (backward, dC = ones; B passed as a transposed view)
+    dB = A^T . dC         (backward; A passed as a transposed view)
+    d  = Dot(u, v)        (two fp32 vectors of 2^26 elements)
+`value` is (3 * 2*4096^3 + 2*2^26) flop divided by the step time, in TFLOP/s.  The same JSON line
+carries the roofline of the dominant kernel (the forward GEMM, timed per launch with HIP events on
+the launch stream inside the timed steps), the elementwise leg of the metric (a + b on 256 MiB
+operands, GB/s against 8 TB/s) and the CPU baseline: the reference's own MatMul kernel
+(oracle/_ref, else the oracle port) timed on one host core on a 64-row slab of the same product.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
+M = 4096
+DOT_N = 1 << 26
+EW_N = 1 << 26
+
+# HBM bytes per forward-GEMM launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, scaled
+# by the same counters on a plain copy of known size); see profiles/.  None until measured.
+GEMM_TRAFFIC_BYTES = None
+
+
+def cpu_baseline(seconds_hint=15.0):
+    """Times the reference's MatMul kernel (or the oracle port) on one host core on a slab of
+    `rows` rows of the 4096^3 product and reports TFLOP/s.  Checker code, used here only as the
+    thing the GPU number is reported beside."""
+    import numpy as np
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import support
+    # the reference library logs to stdout when it loads; this process's stdout carries exactly
+    # one JSON line, so point fd 1 at stderr while the baseline runs
+    sys.stdout.flush()
+    saved = os.dup(1)
+    os.dup2(2, 1)
+    try:
+        return _cpu_baseline(np, support)
+    finally:
+        sys.stdout.flush()
+        os.dup2(saved, 1)
+        os.close(saved)
+
+
+def _cpu_baseline(np, support):
+    rng = np.random.default_rng(202)
+    rows = 48
+    A = rng.standard_normal((rows, M), dtype=np.float32)
+    B = rng.standard_normal((M, M), dtype=np.float32)
+    kind = "port"
+    fn = None
+    if support.ref_available():
+        try:
+            ref = support.Reference()
+            fn = lambda: ref.matmul_t(A, 0, B, 0)
+            kind = "reference"
+        except OSError:
+            fn = None
+    if fn is None:
+        o = support.Oracle()
+        fn = lambda: o.matmul(A, B)
+    t0 = time.perf_counter()
+    fn()
+    dt = time.perf_counter() - t0
+    flops = 2.0 * rows * M * M
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": kind,
+            "sample": "rows 0..%d of the 4096^3 product (%d/4096 of the flops), %.1f s on one core; "
+                      "4096^3 extrapolates to %.0f s" % (rows - 1, rows, dt, dt * M / rows)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (every box has one); --gpus %d is not supported"
+              % args.gpus, file=sys.stderr)
+        return 2
+
+    import torch
+    from ctorch_amd import capi
+
+    lib = capi.load()          # raises if the HIP library is missing: there is no fallback
+    torch.cuda.init()
+    dev = "cuda:0"
+    torch.zeros(1, device=dev)
+    capi.check(lib.ctamd_init(0))
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    P = lambda t: C.c_void_p(t.data_ptr())
+
+    g = torch.Generator(device=dev)
+    g.manual_seed(201)
+    A = torch.randn(M, M, device=dev, generator=g)
+    B = torch.randn(M, M, device=dev, generator=g)
+    dC = torch.ones(M, M, device=dev)
+    Cm, dA, dB = (torch.empty(M, M, device=dev) for _ in range(3))
+    u = torch.rand(DOT_N, device=dev, generator=g) * 2 - 1
+    v = torch.rand(DOT_N, device=dev, generator=g) * 2 - 1
+    d = torch.empty(1, device=dev)
+
+    def gemm(a, as0, as1, b, bs0, bs1, c):
+        capi.check(lib.ctamd_matmul_f32(P(a), as0, as1, P(b), bs0, bs1, P(c), M, M, M, stream))
+
+    fwd_events = []
+
+    def step(timed):
+        if timed:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+        gemm(A, M, 1, B, M, 1, Cm)            # C = A . B
+        if timed:
+            e1.record()
+            fwd_events.append((e0, e1))
+        gemm(dC, M, 1, B, 1, M, dA)           # dA = dC . B^T  (B as a [n,k] -> [k,n] view)
+        gemm(A, 1, M, dC, M, 1, dB)           # dB = A^T . dC
+        capi.check(lib.ctamd_dot_f32(P(u), P(v), P(d), DOT_N, stream))
+
+    for _ in range(args.warmup):
+        step(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(True)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    flop_per_step = 3 * 2.0 * M ** 3 + 2.0 * DOT_N
+    value = flop_per_step / (ms_per_step * 1e-3) / 1e12
+    gemm_ms = sum(a.elapsed_time(b) for a, b in fwd_events) / len(fwd_events)
+    achieved = 2.0 * M ** 3 / (gemm_ms * 1e-3) / 1e12
+
+    # sanity of what was timed: C against an fp64 recomputation of a few rows
+    rows = torch.tensor([0, 1337, 4095], device=dev)
+    ref = (A[rows].double() @ B.double())
+    bound = 1e-5 * (A[rows].abs().double() @ B.abs().double())
+    assert bool(((Cm[rows].double() - ref).abs() <= bound).all()), "forward GEMM failed its fp64 check"
+
+    # elementwise leg of the metric: a + b, 256 MiB per operand, four rotating buffer sets
+    sets = [tuple(torch.randn(EW_N, device=dev) for _ in range(2)) + (torch.empty(EW_N, device=dev),)
+            for _ in range(4)]
+    def ew(i):
+        a, b, r = sets[i % 4]
+        capi.check(lib.ctamd_add_f32(P(a), P(b), P(r), EW_N, stream))
+    for i in range(4):
+        ew(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    reps = 40
+    e0.record()
+    for i in range(reps):
+        ew(i)
+    e1.record()
+    torch.cuda.synchronize()
+    ew_s = e0.elapsed_time(e1) * 1e-3 / reps
+    ew_gbs = 12.0 * EW_N / ew_s / 1e9
+    del sets
+
+    out = {
+        "metric": "elementwise HBM GB/s + fp32 MatMul TFLOP/s (% of MI355X roofline), 1 GPU",
+        "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[1]: fp32 MatMul 4096^3 forward + backward (dA = dC.B^T, dB = A^T.dC, "
+                               "dC = ones) + Dot of two 2^26-element vectors; N(0,1) / uniform[-1,1] inputs "
+                               "generated on the device", "M": M, "N": M, "K": M, "dot_n": DOT_N},
+        "roofline": {"bound": "mfma", "kernel": "gemm_kernel<128x128x16, A K-contiguous, B N-contiguous> "
+                                                "(forward C = A.B)",
+                     "achieved": round(achieved, 2), "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / MFMA_FP32_PEAK_TFLOPS, 4), "traffic": GEMM_TRAFFIC_BYTES,
+                     "launch_ms": round(gemm_ms, 4)},
+        "elementwise": {"op": "a + b (ctamd_add_f32), 2^26 elements, 12 B/elem", "achieved": round(ew_gbs, 1),
+                        "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ew_gbs / HBM_PEAK_GBS, 4)},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

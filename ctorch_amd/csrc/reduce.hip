@@ -13,7 +13,7 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / 64;
 constexpr int kUnroll = 4;
-constexpr unsigned kMaxBlocks = 2048;
+constexpr unsigned kMaxBlocks = 2048;   // partials folded by one block: keep that fold short
 
 __device__ __forceinline__ double wave_sum(double v) {
 #pragma unroll
@@ -46,11 +46,12 @@ struct AbsT { static constexpr int kIn = 2;
 struct TinyT { static constexpr int kIn = 1;
     __device__ static float term(float a, float) { return (__builtin_fabsf(a) < 1.1920928955078125e-07f) ? 1.0f : 0.0f; } };
 
+// Block b walks runs of kThreads*kUnroll consecutive vectors (b, b + gridDim, ...); within a run
+// thread t takes vectors t, t+256, t+512, t+768, all loads issued before the first add.  The
+// loads carry the non-temporal hint: every byte is used once.
 template <class T, bool VEC>
 __global__ __launch_bounds__(kThreads) void reduce_stage1(const float* __restrict__ a, const float* __restrict__ b,
                                                           double* __restrict__ partials, size_t n) {
-    const size_t tid = size_t(blockIdx.x) * kThreads + threadIdx.x;
-    const size_t stride = size_t(gridDim.x) * kThreads;
     float acc[kUnroll][4];
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u)
@@ -59,19 +60,20 @@ __global__ __launch_bounds__(kThreads) void reduce_stage1(const float* __restric
     float tail = 0.0f;
     if (VEC) {
         const size_t n4 = n >> 2;
-        for (size_t base = tid; base < n4; base += stride * kUnroll) {
+        constexpr size_t kRun = size_t(kThreads) * kUnroll;
+        for (size_t run = size_t(blockIdx.x) * kRun; run < n4; run += size_t(gridDim.x) * kRun) {
             v4f va[kUnroll], vb[kUnroll];
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u) {
-                size_t i = base + size_t(u) * stride;
+                size_t i = run + size_t(u) * kThreads + threadIdx.x;
                 if (i < n4) {
-                    va[u] = reinterpret_cast<const v4f*>(a)[i];
-                    if (T::kIn == 2) vb[u] = reinterpret_cast<const v4f*>(b)[i];
+                    va[u] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(a) + i);
+                    if (T::kIn == 2) vb[u] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(b) + i);
                 }
             }
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u) {
-                size_t i = base + size_t(u) * stride;
+                size_t i = run + size_t(u) * kThreads + threadIdx.x;
                 if (i < n4) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) acc[u][e] += T::term(va[u][e], T::kIn == 2 ? vb[u][e] : 0.0f);
@@ -83,6 +85,8 @@ __global__ __launch_bounds__(kThreads) void reduce_stage1(const float* __restric
             if (i < n) tail = T::term(a[i], T::kIn == 2 ? b[i] : 0.0f);
         }
     } else {
+        const size_t tid = size_t(blockIdx.x) * kThreads + threadIdx.x;
+        const size_t stride = size_t(gridDim.x) * kThreads;
         for (size_t i = tid; i < n; i += stride) acc[0][0] += T::term(a[i], T::kIn == 2 ? b[i] : 0.0f);
     }
     // pairwise fold of the 16 lanes, in double from here on
@@ -119,8 +123,8 @@ int reduce(const char* name, const float* a, const float* b, float* out, int32_t
     unsigned grid = 0;
     if (n) {
         bool vec = aligned16(a) && (T::kIn == 1 || aligned16(b));
-        grid = stream_grid(vec ? n / 4 + 1 : n, size_t(kThreads) * kUnroll);
-        if (grid > kMaxBlocks) grid = kMaxBlocks;
+        size_t need = ((vec ? n / 4 + 1 : n) + size_t(kThreads) * kUnroll - 1) / (size_t(kThreads) * kUnroll);
+        grid = need < kMaxBlocks ? unsigned(need) : kMaxBlocks;
         if (vec)
             hipLaunchKernelGGL((reduce_stage1<T, true>), dim3(grid), dim3(kThreads), 0, s, a, b, partials, n);
         else
@@ -147,21 +151,29 @@ __global__ __launch_bounds__(kThreads) void colsum_stage1(const float* __restric
     const size_t r0 = size_t(blockIdx.y) * rows_per_block;
     size_t r1 = r0 + rows_per_block;
     if (r1 > rows) r1 = rows;
+    constexpr int U = 8;    // independent row loads in flight per thread
     float acc[2][4] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
     if (col < cols) {
         size_t r = r0 + ty;
-        for (; r + kRowLanes < r1; r += 2 * kRowLanes) {
+        for (; r + size_t(U - 1) * kRowLanes < r1; r += size_t(U) * kRowLanes) {
             if (VEC) {
-                v4f x0 = *reinterpret_cast<const v4f*>(g + r * cols + col);
-                v4f x1 = *reinterpret_cast<const v4f*>(g + (r + kRowLanes) * cols + col);
+                v4f x[U];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) { acc[0][e] += x0[e]; acc[1][e] += x1[e]; }
+                for (int u = 0; u < U; ++u)
+                    x[u] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(g + (r + size_t(u) * kRowLanes) * cols + col));
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[u & 1][e] += x[u][e];
             } else {
-                acc[0][0] += g[r * cols + col];
-                acc[1][0] += g[(r + kRowLanes) * cols + col];
+                float x[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) x[u] = g[(r + size_t(u) * kRowLanes) * cols + col];
+#pragma unroll
+                for (int u = 0; u < U; ++u) acc[u & 1][0] += x[u];
             }
         }
-        if (r < r1) {
+        for (; r < r1; r += kRowLanes) {
             if (VEC) {
                 v4f x0 = *reinterpret_cast<const v4f*>(g + r * cols + col);
 #pragma unroll
@@ -222,7 +234,7 @@ int ctamd_colsum_f32(const float* g, float* out, size_t rows, size_t cols, void*
     // row chunks: fill the chip (about 8 blocks per CU), at least 32 rows per block, and the
     // partial rows must fit the scratch
     size_t want = (size_t(compute_units() > 0 ? compute_units() : 256) * 8 + col_blocks - 1) / col_blocks;
-    size_t chunks = (rows + 31) / 32;
+    size_t chunks = (rows + 63) / 64;
     if (chunks > want) chunks = want;
     if (chunks > kScratchFloats / cols) chunks = kScratchFloats / cols;
     if (chunks > 65535) chunks = 65535;

@@ -1,0 +1,102 @@
+// Tape autograd over device tensors.  Same public surface as the reference's AutoDiff /
+// AutoDiffContext (include/AutoDiff.h:29-67, :144-220): a thread-local current context with an
+// RAII Guard, make_leaf / zero_grad / get_grad / backward / clear_graph, and the two-phase
+// defer_record / commit_record used by the Tensor methods.
+//
+// The gradient arithmetic per operator follows src/AutoDiff.cpp:1216-1862 operation by
+// operation; on kAMD tensors every piece is a kernel of the launch layer (fused where the
+// reference chains several Tensor ops, with the same fp32 operation order inside the kernel), and
+// every edge lands with the in-place accumulate of :1870-1907.
+// Differences, all deliberate:
+//  - nodes hold references (shared storage) to the tensors they describe instead of deep copies
+//    (reference: AutoDiff.cpp:286, :465), so taping costs no HBM traffic;
+//  - the gradient of a row-broadcast operand ([rows, cols] op [cols]) is the column sum by
+//    default; BroadcastGrad::kReferenceRow0 reproduces the reference, which returns row 0 of the
+//    upstream gradient (AutoDiff.cpp:690-757, expected by src/tests/test_tensor_grad.cpp:132-138);
+//  - CrossEntropy's backward accepts class-index targets (the reference throws, :1569);
+//  - backward() does not hold a lock while it runs kernels, so Tensor::backward(grad_output)
+//    cannot self-deadlock (reference: Tensor.cpp:549-550 -> AutoDiff.cpp:1157 + :346).
+#ifndef CTORCH_AMD_HOST_AUTODIFF_H
+#define CTORCH_AMD_HOST_AUTODIFF_H
+#include <memory>
+#include <mutex>
+#include <unordered_map>
+#include <unordered_set>
+#include <vector>
+
+#include "Tensor.h"
+
+class AutoDiff;
+
+class AutoDiffContext {
+   public:
+    static AutoDiff*& current() {
+        thread_local AutoDiff* ctx = nullptr;
+        return ctx;
+    }
+    class Guard {
+        AutoDiff* prev_;
+
+       public:
+        explicit Guard(AutoDiff* ctx) : prev_(current()) { current() = ctx; }
+        ~Guard() { current() = prev_; }
+        Guard(const Guard&) = delete;
+        Guard& operator=(const Guard&) = delete;
+    };
+};
+
+enum class BroadcastGrad { kColumnSum, kReferenceRow0 };
+
+class AutoDiff {
+   public:
+    struct Node {
+        size_t tensor_id = 0;
+        op operation = op::Add;
+        int op_param_i = 0;
+        std::vector<size_t> input_ids;
+        std::unique_ptr<Tensor> tensor;   // shares storage with the user's tensor
+        std::unique_ptr<Tensor> grad;
+        bool requires_grad = false;
+        bool is_leaf = true;
+    };
+
+    AutoDiff() = default;
+    ~AutoDiff() = default;
+
+    void make_leaf(Tensor& t, bool requires_grad);
+    void update_requires_grad(Tensor& t, bool requires_grad);
+    void zero_grad(Tensor& t);
+    Tensor get_grad(const Tensor* t);
+    void defer_record(size_t output_id, op operation, const std::vector<Tensor*>& inputs, int op_param_i = 0);
+    void commit_record(Tensor& output);
+    void set_retain_graph(bool retain) { retain_graph_ = retain; }
+    void backward(Tensor& root);
+    void backward(Tensor& root, Tensor grad_output);
+    void clear_graph();
+    size_t node_count();
+
+    void set_broadcast_grad(BroadcastGrad m) { broadcast_grad_ = m; }
+    BroadcastGrad broadcast_grad() const { return broadcast_grad_; }
+    // Div's backward scans the divisor for |b| < FLT_EPSILON and throws (reference:
+    // AutoDiff.cpp:1267-1284).  On the device that is one more pass over b and a host wait; it can
+    // be switched off.
+    void set_check_div_zero(bool on) { check_div_zero_ = on; }
+
+   private:
+    struct Pending {
+        op operation;
+        std::vector<size_t> input_ids;
+        int op_param_i;
+    };
+    std::mutex records_mutex;
+    std::unordered_map<size_t, std::unique_ptr<Node>> id_to_node;
+    std::unordered_map<size_t, Pending> pending_;
+    bool retain_graph_ = false;
+    BroadcastGrad broadcast_grad_ = BroadcastGrad::kColumnSum;
+    bool check_div_zero_ = true;
+
+    Node* find(size_t id);
+    Tensor adjust_grad_shape(const Tensor& grad, const std::vector<size_t>& target_shape);
+    Tensor input_gradient(Node* node, size_t input_id, size_t input_pos, const Tensor& node_grad);
+};
+#endif

@@ -1,0 +1,133 @@
+// Storage: the bytes behind a Tensor.  Same interface as the reference's include/Storage.h
+// (ctor :77, data<T>() :131-151, clone() :175-181, shallow copies :98-103), with the `device` tag
+// made real: a kAMD storage lives in HBM (allocated through the C ABI's ctamd_malloc, recycled by
+// a size-bucketed pool so that an op's result does not pay a hipMalloc / hipFree), clone() is a
+// device-to-device copy, to(device) is the explicit host <-> device transfer, and data<T>() on a
+// device storage throws instead of handing a host pointer to HBM.
+#ifndef CTORCH_AMD_HOST_STORAGE_H
+#define CTORCH_AMD_HOST_STORAGE_H
+#include <cstring>
+#include <memory>
+#include <type_traits>
+
+#include "Ctools.h"
+#include "Ctorch_Error.h"
+
+namespace ctorch_amd_host {
+// Device memory pool (src/DeviceMemory.cpp).  acquire() returns HBM of at least `bytes` bytes,
+// release() returns it to the pool; trim() frees everything cached.
+void* device_acquire(size_t bytes);
+void device_release(void* p, size_t bytes);
+void device_trim();
+void device_copy_h2d(void* dst, const void* src, size_t bytes);
+void device_copy_d2h(void* dst, const void* src, size_t bytes);
+void device_copy_d2d(void* dst, const void* src, size_t bytes);
+void device_sync();
+}  // namespace ctorch_amd_host
+
+class Storage {
+   private:
+    size_t _size{};
+    DType _dtype;
+    DeviceType _device;
+    std::shared_ptr<char[]> _data;
+
+    template <typename T>
+    void checkDType() const {
+        if ((std::is_same<T, float>::value && _dtype != DType::kFloat) ||
+            (std::is_same<T, double>::value && _dtype != DType::kDouble) ||
+            (std::is_same<T, int32_t>::value && _dtype != DType::kInt) ||
+            (std::is_same<T, int64_t>::value && _dtype != DType::kLong) ||
+            (std::is_same<T, bool>::value && _dtype != DType::kBool)) {
+            Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DATATYPE, "Storage data type mismatch");
+        }
+    }
+    static std::shared_ptr<char[]> allocate(size_t bytes, DeviceType device) {
+        if (bytes == 0) return nullptr;
+        if (device == DeviceType::kAMD) {
+            char* p = static_cast<char*>(ctorch_amd_host::device_acquire(bytes));
+            return std::shared_ptr<char[]>(p, [bytes](char* q) { ctorch_amd_host::device_release(q, bytes); });
+        }
+        return std::shared_ptr<char[]>(new char[bytes], std::default_delete<char[]>());
+    }
+
+   public:
+    Storage(size_t size, DType dtype, DeviceType device = DeviceType::kCPU)
+        : _size(size), _dtype(dtype), _device(device), _data(allocate(size * dtypeSize(dtype), device)) {}
+
+    // copies `size` elements from HOST memory into the new storage (an upload for kAMD)
+    template <typename T>
+    Storage(const T* data, size_t size, DType dtype, DeviceType device = DeviceType::kCPU) : Storage(size, dtype, device) {
+        if (size > 0 && _data.get()) {
+            if (device == DeviceType::kAMD) ctorch_amd_host::device_copy_h2d(_data.get(), data, size * dtypeSize(dtype));
+            else std::memcpy(_data.get(), data, size * dtypeSize(dtype));
+        }
+    }
+
+    Storage(const Storage&) = default;
+    Storage& operator=(const Storage&) = default;
+    Storage(Storage&&) = default;
+    Storage& operator=(Storage&&) = default;
+    Storage() : _size(0), _dtype(DType::kFloat), _device(DeviceType::kCPU) {}
+    ~Storage() = default;
+
+    // host pointer; throws for a device storage (use raw() / to(kCPU))
+    template <typename T>
+    T* data() {
+        if (_size == 0 || !_data) return nullptr;
+        checkDType<T>();
+        requireHost();
+        return reinterpret_cast<T*>(_data.get());
+    }
+    template <typename T>
+    const T* data() const {
+        if (_size == 0 || !_data) return nullptr;
+        checkDType<T>();
+        requireHost();
+        return reinterpret_cast<const T*>(_data.get());
+    }
+    // untyped pointer in the storage's own address space (HBM for kAMD); for the launch layer
+    void* raw() { return _data.get(); }
+    const void* raw() const { return _data.get(); }
+
+    size_t size() const { return _size; }
+    DType dtype() const { return _dtype; }
+    DeviceType device() const { return _device; }
+    size_t nbytes() const { return _size * dtypeSize(_dtype); }
+
+    Storage clone() const {
+        Storage s(_size, _dtype, _device);
+        if (_size > 0 && _data) {
+            if (_device == DeviceType::kAMD) ctorch_amd_host::device_copy_d2d(s._data.get(), _data.get(), nbytes());
+            else std::memcpy(s._data.get(), _data.get(), nbytes());
+        }
+        return s;
+    }
+
+    // explicit transfer: a new storage on `device` holding the same bytes
+    Storage to(DeviceType device) const {
+        if (device == _device) return clone();
+        if (device != DeviceType::kCPU && device != DeviceType::kAMD)
+            Ctorch_Error::throwException(DeviceTypeToErrorPlatform(device), ErrorType::DEVICE_COMPAT, "Storage::to: unsupported device");
+        Storage s(_size, _dtype, device);
+        if (_size > 0 && _data) {
+            if (device == DeviceType::kAMD) ctorch_amd_host::device_copy_h2d(s._data.get(), _data.get(), nbytes());
+            else ctorch_amd_host::device_copy_d2h(s._data.get(), _data.get(), nbytes());
+        }
+        return s;
+    }
+
+    void clear() {
+        _data.reset();
+        _size = 0;
+    }
+    bool empty() const { return _size == 0 || !_data; }
+
+   private:
+    void requireHost() const {
+        if (_device == DeviceType::kAMD)
+            Ctorch_Error::throwException(ErrorPlatform::kAMD, ErrorType::MEMORY,
+                                         "Storage::data<T>(): storage is in device memory; transfer it with to(kCPU)");
+    }
+};
+#endif

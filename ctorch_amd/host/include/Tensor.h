@@ -1,0 +1,140 @@
+// Tensor front-end over the MI355X launch layer.  Mirrors the part of the reference's class Tensor
+// (include/Tensor.h:70-1123, src/Tensor.cpp) that lies on the operator hot path: construction,
+// metadata, the sixteen operator methods that dispatch through Ctorch_Scheduler
+// (src/Tensor.cpp:484,574,590,606,622,681,709,736,811,839,1396,1612,1629,1807,1824,1841), the
+// host-inline ones (sum :638-666, tensor (op) float :751-973, softmax(dim) :1645-1803,
+// transpose / t :246-261, zero / ones :390-451, item :155-165) and backward() / grad().
+//
+// Semantics kept from the reference: a copy is a deep copy with a new id (Tensor.h:320-334), a
+// move keeps the id (:364-377); ids are the tape's keys; results take the first operand's shape;
+// ops throw on dtype / device mismatch (src/Tensor.cpp:726-733).
+// New: DeviceType::kAMD tensors live in HBM; to(device) / cpu() / amd() are the explicit
+// transfers; data<T>() on a device tensor throws; item() copies one element back.
+// Arithmetic exists for kAMD tensors only - kCPU tensors are staging containers (the reference's
+// CPU kernels are not part of this library), and dispatching one reports "no kernel" loudly.
+#ifndef CTORCH_AMD_HOST_TENSOR_H
+#define CTORCH_AMD_HOST_TENSOR_H
+#include <atomic>
+#include <initializer_list>
+#include <numeric>
+#include <vector>
+
+#include "Ctools.h"
+#include "Ctorch_Error.h"
+#include "Storage.h"
+
+struct ShapeTag {};
+
+class Tensor {
+   private:
+    size_t tensor_id_;
+    bool _requires_grad = false;
+    std::vector<size_t> _shape;
+    std::vector<size_t> _strides;
+    size_t _storage_offset = 0;
+    DeviceType _device = DeviceType::kCPU;
+    DType _dtype = DType::kFloat;
+    Storage _storage;
+
+    static std::atomic<size_t> global_tensor_id;
+    void computeStrides();
+    struct AliasTag {};
+    Tensor(AliasTag, const Tensor& other);   // shares storage AND id: the tape's reference to a tensor
+
+   public:
+    Tensor();
+    Tensor(float value);                                         // 0-D tensor on the host
+    Tensor(float value, DeviceType device);                      // 0-D tensor on `device`
+    Tensor(std::initializer_list<float> values);                 // 1-D host tensor
+    Tensor(ShapeTag, const std::vector<size_t>& shape, DType dtype = DType::kFloat,
+           DeviceType device = DeviceType::kCPU, bool zero_init = true);
+    Tensor(const Tensor& other);                                 // deep copy, new id
+    Tensor& operator=(const Tensor& other);
+    Tensor(Tensor&& other) noexcept;                             // keeps the id
+    Tensor& operator=(Tensor&& other) noexcept;
+    ~Tensor() = default;
+
+    static Tensor alias(const Tensor& t) { return Tensor(AliasTag{}, t); }
+    // transposed VIEW of a 2-D tensor: shares storage, no copy (the tape's B^T / A^T operands)
+    static Tensor view_t(const Tensor& t);
+    // a tensor on `device` filled from host memory
+    static Tensor from_host(const float* data, const std::vector<size_t>& shape, DeviceType device);
+
+    // ---- metadata
+    size_t id() const { return tensor_id_; }
+    void requires_grad(bool key);
+    bool requires_grad() const { return _requires_grad; }
+    void set_requires_grad(bool r) { _requires_grad = r; }
+    const std::vector<size_t>& shape() const { return _shape; }
+    const std::vector<size_t>& sizes() const { return _shape; }
+    const std::vector<size_t>& strides() const { return _strides; }
+    size_t dim() const { return _shape.size(); }
+    size_t numel() const;
+    DType dtype() const { return _dtype; }
+    DeviceType device() const { return _device; }
+    bool is_contiguous() const;
+    bool is_cleared() const { return _storage.empty(); }
+    const Storage& storage() const { return _storage; }
+
+    // ---- data access
+    template <typename T>
+    const T* data() const { return _storage.data<T>() + _storage_offset; }   // host tensors only
+    template <typename T>
+    T* data() { return _storage.data<T>() + _storage_offset; }
+    // fp32 pointer in the tensor's own address space (HBM for kAMD), offset applied
+    const float* fptr() const { return static_cast<const float*>(_storage.raw()) + _storage_offset; }
+    float* fptr() { return static_cast<float*>(_storage.raw()) + _storage_offset; }
+    template <typename T>
+    T item() const;
+    std::vector<float> to_vector() const;     // contiguous host copy of the elements (any device)
+
+    // ---- transfers
+    Tensor to(DeviceType device) const;
+    Tensor cpu() const { return to(DeviceType::kCPU); }
+    Tensor amd() const { return to(DeviceType::kAMD); }
+
+    // ---- fills
+    void zero();
+    void ones();
+    void fill(float v);
+
+    // ---- views
+    Tensor transpose(int dim0, int dim1) const;   // deep copy + stride swap, as the reference
+    Tensor t() const;
+    Tensor contiguous() const;
+
+    // ---- operators (dispatched)
+    Tensor operator+(const Tensor& other) const;
+    Tensor operator-(const Tensor& other) const;
+    Tensor operator*(const Tensor& other) const;
+    Tensor operator/(const Tensor& other) const;
+    Tensor operator-() const;
+    Tensor matmul(const Tensor& other) const;
+    Tensor dot(const Tensor& other) const;
+    Tensor relu() const;
+    Tensor sigmoid() const;
+    Tensor tanh() const;
+    Tensor sin() const;
+    Tensor cos() const;
+    Tensor mse_loss(const Tensor& target) const;
+    Tensor mae_loss(const Tensor& target) const;
+    Tensor cross_entropy(const Tensor& target) const;
+    // ---- host-inline in the reference, device kernels here
+    Tensor operator+(float scalar) const;
+    Tensor operator*(float scalar) const;
+    Tensor operator/(float scalar) const;
+    Tensor sum() const;
+    Tensor softmax(int dim = -1) const;
+
+    // ---- autograd
+    void backward() const;
+    void backward(const Tensor& grad_output) const;
+};
+
+void backward(Tensor& root);
+void backward(Tensor& root, Tensor grad_output);
+Tensor grad(const Tensor& t);
+Tensor matMul(const Tensor& a, const Tensor& b);
+
+#include "AutoDiff.h"
+#endif

@@ -1,0 +1,56 @@
+// Kernel ABI of the scheduler: the reference's two function-pointer types
+// (src/kernels/kernels.h:23,31) and, following its naming rule <Op>_<PLATFORM>_kernel
+// (CONTRIBUTING.md:54-55), the AMD column: one shim per registered operator that unpacks the
+// Tensors, allocates the result on the inputs' device and calls the extern "C" launch layer
+// (include/ctorch_amd.h).  Same argument meaning, result shapes and error behaviour as the
+// CPU-BASIC kernels they stand beside.
+#ifndef CTORCH_AMD_HOST_KERNELS_H
+#define CTORCH_AMD_HOST_KERNELS_H
+#include "Tensor.h"
+
+typedef Tensor (*BinaryKernelFunc)(const Tensor& a, const Tensor& b);
+typedef Tensor (*UnaryKernelFunc)(const Tensor& a);
+
+Tensor Add_AMD_kernel(const Tensor& a, const Tensor& b);
+Tensor Sub_AMD_kernel(const Tensor& a, const Tensor& b);
+Tensor Mul_AMD_kernel(const Tensor& a, const Tensor& b);
+Tensor Div_AMD_kernel(const Tensor& a, const Tensor& b);
+Tensor MatMul_AMD_kernel(const Tensor& a, const Tensor& b);
+Tensor Dot_AMD_kernel(const Tensor& a, const Tensor& b);
+Tensor MSE_AMD_kernel(const Tensor& a, const Tensor& b);
+Tensor MAE_AMD_kernel(const Tensor& a, const Tensor& b);
+Tensor CrossEntropy_AMD_kernel(const Tensor& a, const Tensor& b);
+
+Tensor Neg_AMD_kernel(const Tensor& a);
+Tensor ReLU_AMD_kernel(const Tensor& a);
+Tensor Cos_AMD_kernel(const Tensor& a);
+Tensor Sin_AMD_kernel(const Tensor& a);
+Tensor Tanh_AMD_kernel(const Tensor& a);
+Tensor Sigmoid_AMD_kernel(const Tensor& a);
+Tensor Softmax_AMD_kernel(const Tensor& a);
+
+namespace ctorch_amd_host {
+// Device branches of the arithmetic that the reference runs inline on the host (not behind the
+// scheduler): used by the Tensor front-end and the tape.
+Tensor scalar_op(const Tensor& a, float s, op which);                 // a + s, a * s, a / s
+Tensor sum_all(const Tensor& a);
+Tensor softmax_dim(const Tensor& a, int dim);                         // dim already normalised
+Tensor filled(const std::vector<size_t>& shape, float v, DeviceType device);
+Tensor filled_from(const std::vector<size_t>& shape, const Tensor& scalar0d);
+void accumulate(Tensor& grad, const Tensor& val);                     // grad += val
+Tensor column_sum(const Tensor& g);                                   // [rows, cols] -> [cols]
+Tensor first_row(const Tensor& g);                                    // [rows, cols] -> [cols], row 0
+bool any_abs_lt_eps(const Tensor& b);
+Tensor relu_backward(const Tensor& x, const Tensor& g);
+Tensor sigmoid_backward(const Tensor& x, const Tensor& g);
+Tensor tanh_backward(const Tensor& x, const Tensor& g);
+Tensor sin_backward(const Tensor& x, const Tensor& g);
+Tensor cos_backward(const Tensor& x, const Tensor& g);
+Tensor softmax_backward(const Tensor& y, const Tensor& g, int dim);
+Tensor mse_backward(const Tensor& p, const Tensor& t, const Tensor& g0d);
+Tensor mae_backward(const Tensor& p, const Tensor& t, const Tensor& g0d);
+Tensor cross_entropy_backward(const Tensor& x, const Tensor& target, const Tensor& g0d);
+Tensor div_backward_b(const Tensor& a, const Tensor& b, const Tensor& g);
+void init_device();   // ctamd_init(0), once; throws if there is no gfx950 device
+}  // namespace ctorch_amd_host
+#endif

@@ -1,0 +1,263 @@
+// Tape and backward pass.  The per-operator gradient arithmetic follows the reference's
+// AutoDiff::backward (src/AutoDiff.cpp:1216-1862) branch by branch; see AutoDiff.h for the
+// deliberate differences.
+#include "AutoDiff.h"
+
+#include <algorithm>
+
+#include "Ctorch_Scheduler.h"
+#include "kernels.h"
+
+using namespace ctorch_amd_host;
+
+AutoDiff::Node* AutoDiff::find(size_t id) {
+    auto it = id_to_node.find(id);
+    return (it == id_to_node.end() || !it->second) ? nullptr : it->second.get();
+}
+
+size_t AutoDiff::node_count() {
+    std::lock_guard<std::mutex> lock(records_mutex);
+    return id_to_node.size();
+}
+
+// src/AutoDiff.cpp:246-311
+void AutoDiff::make_leaf(Tensor& t, bool requires_grad) {
+    if (t.id() == 0) return;
+    std::lock_guard<std::mutex> lock(records_mutex);
+    Node* n = find(t.id());
+    if (n) {
+        n->requires_grad = n->requires_grad || requires_grad;
+        return;
+    }
+    auto node = std::make_unique<Node>();
+    node->tensor_id = t.id();
+    node->tensor = std::make_unique<Tensor>(Tensor::alias(t));
+    node->requires_grad = requires_grad;
+    node->is_leaf = true;
+    id_to_node[t.id()] = std::move(node);
+}
+
+// src/AutoDiff.cpp:513-546
+void AutoDiff::update_requires_grad(Tensor& t, bool requires_grad) {
+    if (t.id() == 0) return;
+    std::lock_guard<std::mutex> lock(records_mutex);
+    if (Node* n = find(t.id())) n->requires_grad = requires_grad;
+}
+
+// src/AutoDiff.cpp:502-510
+void AutoDiff::zero_grad(Tensor& t) {
+    if (t.id() == 0) return;
+    std::lock_guard<std::mutex> lock(records_mutex);
+    Node* n = find(t.id());
+    if (n && n->grad) n->grad->zero();
+}
+
+// src/AutoDiff.cpp:86-243: a copy of the stored gradient, or zeros of the tensor's shape
+Tensor AutoDiff::get_grad(const Tensor* t) {
+    if (!t || t->id() == 0) return Tensor();
+    std::lock_guard<std::mutex> lock(records_mutex);
+    Node* n = find(t->id());
+    if (n && n->requires_grad && n->grad) return Tensor(*n->grad);
+    return Tensor(ShapeTag{}, t->shape(), t->dtype(), t->device());
+}
+
+// src/AutoDiff.cpp:314-370: inputs not yet on the tape become leaves; the op is parked until the
+// output is known to require a gradient
+void AutoDiff::defer_record(size_t output_id, op operation, const std::vector<Tensor*>& inputs, int op_param_i) {
+    Pending p{operation, {}, op_param_i};
+    for (Tensor* in : inputs) {
+        if (!in || in->id() == 0) continue;
+        make_leaf(*in, in->requires_grad());
+        p.input_ids.push_back(in->id());
+    }
+    std::lock_guard<std::mutex> lock(records_mutex);
+    pending_[output_id] = std::move(p);
+}
+
+// src/AutoDiff.cpp:373-499
+void AutoDiff::commit_record(Tensor& output) {
+    std::lock_guard<std::mutex> lock(records_mutex);
+    auto it = pending_.find(output.id());
+    if (it == pending_.end()) return;
+    auto node = std::make_unique<Node>();
+    node->tensor_id = output.id();
+    node->operation = it->second.operation;
+    node->op_param_i = it->second.op_param_i;
+    node->input_ids = std::move(it->second.input_ids);
+    node->tensor = std::make_unique<Tensor>(Tensor::alias(output));
+    node->requires_grad = true;
+    node->is_leaf = false;
+    pending_.erase(it);
+    id_to_node[output.id()] = std::move(node);
+}
+
+void AutoDiff::clear_graph() {
+    std::lock_guard<std::mutex> lock(records_mutex);
+    id_to_node.clear();
+    pending_.clear();
+}
+
+// src/AutoDiff.cpp:562-1049 for the cases that occur on this path.
+Tensor AutoDiff::adjust_grad_shape(const Tensor& grad, const std::vector<size_t>& target) {
+    if (grad.sizes() == target) return Tensor::alias(grad);
+    if (grad.sizes().empty()) return filled_from(target, grad);                       // :579-627
+    if (grad.dim() == 2 && target.size() == 1 && grad.sizes()[1] == target[0]) {      // :690-757
+        return broadcast_grad_ == BroadcastGrad::kColumnSum ? column_sum(grad) : first_row(grad);
+    }
+    if (target.empty() || (target.size() == 1 && target[0] == 1)) {
+        // gradient of a one-element operand that was broadcast over a whole tensor
+        Tensor flat = Tensor::alias(grad);
+        if (broadcast_grad_ == BroadcastGrad::kColumnSum) {
+            Tensor s = sum_all(flat);
+            return target.empty() ? s : filled_from(target, s);
+        }
+        Tensor first(ShapeTag{}, target, DType::kFloat, grad.device(), false);
+        device_copy_d2d(first.fptr(), grad.fptr(), sizeof(float));
+        return first;
+    }
+    Ctorch_Error::throwException(ErrorPlatform::kAutoDiff, ErrorType::DIMENSION,
+                                 "backward: gradient shape cannot be reduced to the operand's shape");
+}
+
+namespace {
+bool is_row_vector_of(const Tensor& v, const Tensor& m) {
+    return v.dim() == 1 && m.dim() == 2 && v.sizes()[0] == m.sizes()[1];
+}
+}  // namespace
+
+Tensor AutoDiff::input_gradient(Node* node, size_t input_id, size_t /*input_pos*/, const Tensor& g) {
+    Node* in = find(input_id);
+    const Tensor& x = *in->tensor;
+    const bool first = (input_id == node->input_ids[0]);   // the reference tells operands apart by id
+    auto other_node = [&]() -> Node* {
+        if (node->input_ids.size() < 2) return nullptr;
+        return find(first ? node->input_ids[1] : node->input_ids[0]);
+    };
+    switch (node->operation) {
+        case op::Add:                                                   // :1216-1221
+            return adjust_grad_shape(g, x.sizes());
+        case op::Sub: {                                                 // :1222-1233
+            Tensor adj = adjust_grad_shape(g, x.sizes());
+            return first ? adj : Neg_AMD_kernel(adj);
+        }
+        case op::Mul: {                                                 // :1234-1258: other * g
+            Node* o = other_node();
+            if (!o) return Tensor::alias(g);
+            const Tensor& other = *o->tensor;
+            if (is_row_vector_of(other, g)) return Mul_AMD_kernel(g, other);   // row-broadcast operand
+            return Mul_AMD_kernel(other, g);
+        }
+        case op::Div: {                                                 // :1259-1316
+            Node* a_node = find(node->input_ids[0]);
+            Node* b_node = find(node->input_ids[1]);
+            const Tensor& a = *a_node->tensor;
+            const Tensor& b = *b_node->tensor;
+            if (check_div_zero_ && any_abs_lt_eps(b))
+                Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::TENSOR_STATE,
+                                             "division by zero in the gradient of Div");
+            if (first) return Div_AMD_kernel(g, b);                     // g / b
+            if (a.sizes() == b.sizes() && g.sizes() == a.sizes()) return div_backward_b(a, b, g);
+            // broadcast divisor: ((-a) * g) / (b * b) with the same operation order, op by op
+            Tensor na = Neg_AMD_kernel(a);
+            Tensor num = Mul_AMD_kernel(na, g);
+            Tensor den = Mul_AMD_kernel(b, b);
+            return Div_AMD_kernel(num, den);
+        }
+        case op::Neg: return Neg_AMD_kernel(g);                         // :1317-1319
+        case op::ReLU: return relu_backward(x, g);                      // :1320-1371
+        case op::Sigmoid: return sigmoid_backward(x, g);                // :1372-1383
+        case op::Tanh: return tanh_backward(x, g);                      // :1384-1398
+        case op::Sin: return sin_backward(x, g);                        // :1399-1407
+        case op::Cos: return cos_backward(x, g);                        // :1408-1416
+        case op::Softmax: return softmax_backward(*node->tensor, g, node->op_param_i);   // :1417-1490
+        case op::MSE: {                                                 // :1491-1516
+            Node* o = other_node();
+            return mse_backward(x, *o->tensor, g);
+        }
+        case op::MAE: {                                                 // :1602-1642
+            Node* o = other_node();
+            return mae_backward(x, *o->tensor, g);
+        }
+        case op::CE: {                                                  // :1517-1601
+            Node* o = other_node();
+            return cross_entropy_backward(x, *o->tensor, g);
+        }
+        case op::MatMul: {                                              // :1643-1849
+            Node* o = other_node();
+            const Tensor& other = *o->tensor;
+            if (g.dim() != 2)
+                Ctorch_Error::throwException(ErrorPlatform::kAutoDiff, ErrorType::DIMENSION,
+                                             "MatMul gradient must be a 2-D tensor");
+            if (first) return MatMul_AMD_kernel(g, Tensor::view_t(other));      // g . B^T
+            return MatMul_AMD_kernel(Tensor::view_t(other), g);                 // A^T . g
+        }
+        case op::Sum:                                                   // :1850-1855
+            return adjust_grad_shape(g, x.sizes());
+        case op::Dot: {                                                 // extension: g * other
+            Node* o = other_node();
+            Tensor r = Mul_AMD_kernel(Tensor::alias(*o->tensor), g);
+            return r;
+        }
+        default:
+            Ctorch_Error::throwException(ErrorPlatform::kAutoDiff, ErrorType::UNKNOWN,
+                                         "backward: operator has no gradient");
+    }
+}
+
+// src/AutoDiff.cpp:548-553
+void AutoDiff::backward(Tensor& root) {
+    AutoDiffContext::Guard guard(nullptr);
+    Tensor grad_output(1.0f, root.device());
+    backward(root, std::move(grad_output));
+}
+
+// src/AutoDiff.cpp:1080-1924
+void AutoDiff::backward(Tensor& root, Tensor grad_output) {
+    AutoDiffContext::Guard guard(nullptr);   // nothing below is taped
+    if (root.id() == 0)
+        Ctorch_Error::throwException(ErrorPlatform::kAutoDiff, ErrorType::TENSOR_STATE, "backward: invalid root tensor");
+    Node* root_node = find(root.id());
+    if (!root_node) {
+        Ctorch_Error::log(ErrorLevel::ERROR, ErrorPlatform::kAutoDiff, ErrorType::TENSOR_STATE, "backward: root is not on the tape");
+        return;
+    }
+    if (!root_node->requires_grad) return;
+    if (grad_output.device() != root.device()) grad_output = grad_output.to(root.device());
+    root_node->grad = std::make_unique<Tensor>(adjust_grad_shape(grad_output, root.sizes()));
+
+    // reversed depth-first post-order, inputs visited in recorded order (:1058-1077, :1138-1153)
+    std::vector<Node*> order;
+    {
+        std::unordered_set<Node*> visited;
+        std::vector<std::pair<Node*, size_t>> stack;
+        stack.push_back({root_node, 0});
+        visited.insert(root_node);
+        while (!stack.empty()) {
+            Node* n = stack.back().first;
+            size_t& next = stack.back().second;
+            if (next < n->input_ids.size()) {
+                Node* in = find(n->input_ids[next++]);
+                if (in && visited.insert(in).second) stack.push_back({in, 0});
+            } else {
+                order.push_back(n);
+                stack.pop_back();
+            }
+        }
+        std::reverse(order.begin(), order.end());
+    }
+
+    for (Node* node : order) {
+        if (!node->requires_grad || !node->grad || node->is_leaf) continue;
+        const Tensor& node_grad = *node->grad;
+        for (size_t pos = 0; pos < node->input_ids.size(); ++pos) {
+            size_t input_id = node->input_ids[pos];
+            Node* in = find(input_id);
+            if (!in || !in->requires_grad) continue;
+            if (!in->grad)
+                in->grad = std::make_unique<Tensor>(ShapeTag{}, in->tensor->sizes(), in->tensor->dtype(), in->tensor->device());
+            Tensor val = input_gradient(node, input_id, pos, node_grad);
+            Tensor adj = adjust_grad_shape(val, in->tensor->sizes());
+            accumulate(*in->grad, adj);                                  // :1870-1907
+        }
+    }
+}

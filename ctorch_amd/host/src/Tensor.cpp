@@ -1,0 +1,359 @@
+// Tensor front-end: metadata, transfers and the operator methods.  Each operator method keeps the
+// reference's structure (e.g. src/Tensor.cpp:724-747 for operator*): dtype / device checks that
+// throw, dispatch through Ctorch_Scheduler, then the two-phase tape record.
+#include "Tensor.h"
+
+#include <cfloat>
+#include <cmath>
+
+#include "Ctorch_Scheduler.h"
+#include "kernels.h"
+
+using namespace ctorch_amd_host;
+
+std::atomic<size_t> Tensor::global_tensor_id{1};
+
+void Tensor::computeStrides() {
+    _strides.assign(_shape.size(), 1);
+    for (int i = int(_shape.size()) - 2; i >= 0; --i) _strides[i] = _strides[i + 1] * _shape[i + 1];
+}
+
+Tensor::Tensor() : tensor_id_(global_tensor_id++) { computeStrides(); }
+
+Tensor::Tensor(float value) : tensor_id_(global_tensor_id++), _storage(&value, 1, DType::kFloat, DeviceType::kCPU) {
+    computeStrides();
+}
+
+Tensor::Tensor(float value, DeviceType device)
+    : tensor_id_(global_tensor_id++), _device(device), _storage(&value, 1, DType::kFloat, device) {
+    computeStrides();
+}
+
+Tensor::Tensor(std::initializer_list<float> values)
+    : tensor_id_(global_tensor_id++), _shape({values.size()}), _storage(values.begin(), values.size(), DType::kFloat) {
+    computeStrides();
+}
+
+Tensor::Tensor(ShapeTag, const std::vector<size_t>& shape, DType dtype, DeviceType device, bool zero_init)
+    : tensor_id_(global_tensor_id++), _shape(shape), _device(device), _dtype(dtype) {
+    computeStrides();
+    _storage = Storage(numel(), dtype, device);
+    if (zero_init) zero();
+}
+
+Tensor::Tensor(const Tensor& other)
+    : tensor_id_(global_tensor_id++), _requires_grad(other._requires_grad), _shape(other._shape),
+      _strides(other._strides), _storage_offset(other._storage_offset), _device(other._device),
+      _dtype(other._dtype), _storage(other._storage.clone()) {}
+
+Tensor& Tensor::operator=(const Tensor& other) {
+    if (this != &other) {
+        tensor_id_ = global_tensor_id++;
+        _requires_grad = other._requires_grad;
+        _shape = other._shape;
+        _strides = other._strides;
+        _storage_offset = other._storage_offset;
+        _device = other._device;
+        _dtype = other._dtype;
+        _storage = other._storage.clone();
+    }
+    return *this;
+}
+
+Tensor::Tensor(Tensor&& other) noexcept
+    : tensor_id_(other.tensor_id_), _requires_grad(other._requires_grad), _shape(std::move(other._shape)),
+      _strides(std::move(other._strides)), _storage_offset(other._storage_offset), _device(other._device),
+      _dtype(other._dtype), _storage(std::move(other._storage)) {
+    other.tensor_id_ = 0;
+}
+
+Tensor& Tensor::operator=(Tensor&& other) noexcept {
+    if (this != &other) {
+        tensor_id_ = other.tensor_id_;
+        _requires_grad = other._requires_grad;
+        _shape = std::move(other._shape);
+        _strides = std::move(other._strides);
+        _storage_offset = other._storage_offset;
+        _device = other._device;
+        _dtype = other._dtype;
+        _storage = std::move(other._storage);
+        other.tensor_id_ = 0;
+    }
+    return *this;
+}
+
+Tensor::Tensor(AliasTag, const Tensor& other)
+    : tensor_id_(other.tensor_id_), _requires_grad(other._requires_grad), _shape(other._shape),
+      _strides(other._strides), _storage_offset(other._storage_offset), _device(other._device),
+      _dtype(other._dtype), _storage(other._storage) {}
+
+Tensor Tensor::from_host(const float* data, const std::vector<size_t>& shape, DeviceType device) {
+    Tensor t(ShapeTag{}, shape, DType::kFloat, device, false);
+    if (t.numel()) {
+        if (device == DeviceType::kAMD) device_copy_h2d(t.fptr(), data, t.numel() * sizeof(float));
+        else std::memcpy(t.data<float>(), data, t.numel() * sizeof(float));
+    }
+    return t;
+}
+
+size_t Tensor::numel() const {
+    if (_shape.empty()) return 1;
+    return std::accumulate(_shape.begin(), _shape.end(), size_t(1), std::multiplies<size_t>());
+}
+
+bool Tensor::is_contiguous() const {
+    size_t expect = 1;
+    for (int i = int(_shape.size()) - 1; i >= 0; --i) {
+        if (_shape[i] != 1 && _strides[i] != expect) return false;
+        expect *= _shape[i];
+    }
+    return true;
+}
+
+void Tensor::requires_grad(bool key) {
+    _requires_grad = key;
+    if (key && AutoDiffContext::current()) {
+        AutoDiffContext::current()->make_leaf(*this, key);
+        AutoDiffContext::current()->update_requires_grad(*this, key);
+    }
+}
+
+template <>
+float Tensor::item<float>() const {
+    if (numel() != 1 || _storage.empty())
+        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::TENSOR_STATE, "item(): tensor is not a single element");
+    if (_dtype != DType::kFloat)
+        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DATATYPE, "item<float>(): dtype is not float");
+    if (_device == DeviceType::kAMD) {
+        float v;
+        device_copy_d2h(&v, fptr(), sizeof(float));
+        return v;
+    }
+    return *data<float>();
+}
+
+std::vector<float> Tensor::to_vector() const {
+    std::vector<float> out(numel());
+    if (out.empty() || _storage.empty()) return out;
+    if (_dtype != DType::kFloat)
+        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DATATYPE, "to_vector(): dtype is not float");
+    if (is_contiguous()) {
+        if (_device == DeviceType::kAMD) device_copy_d2h(out.data(), fptr(), out.size() * sizeof(float));
+        else std::memcpy(out.data(), data<float>(), out.size() * sizeof(float));
+        return out;
+    }
+    // strided view: bring the whole storage over and gather
+    std::vector<float> all(_storage.size());
+    if (_device == DeviceType::kAMD) device_copy_d2h(all.data(), _storage.raw(), all.size() * sizeof(float));
+    else std::memcpy(all.data(), _storage.raw(), all.size() * sizeof(float));
+    std::vector<size_t> idx(_shape.size(), 0);
+    for (size_t n = 0; n < out.size(); ++n) {
+        size_t off = _storage_offset;
+        for (size_t d = 0; d < idx.size(); ++d) off += idx[d] * _strides[d];
+        out[n] = all[off];
+        for (int d = int(idx.size()) - 1; d >= 0; --d) {
+            if (++idx[d] < _shape[d]) break;
+            idx[d] = 0;
+        }
+    }
+    return out;
+}
+
+Tensor Tensor::to(DeviceType device) const {
+    Tensor r(AliasTag{}, *this);
+    r.tensor_id_ = global_tensor_id++;
+    r._storage = _storage.to(device);
+    r._device = device;
+    return r;
+}
+
+void Tensor::fill(float v) {
+    if (_storage.empty()) return;
+    if (_dtype != DType::kFloat)
+        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DATATYPE, "fill(): only float tensors");
+    if (_device == DeviceType::kAMD) {
+        Tensor f = filled({_storage.size()}, v, DeviceType::kAMD);
+        device_copy_d2d(_storage.raw(), f.fptr(), _storage.nbytes());
+    } else {
+        float* p = _storage.data<float>();
+        for (size_t i = 0; i < _storage.size(); ++i) p[i] = v;
+    }
+}
+void Tensor::zero() {
+    if (_storage.empty()) return;
+    if (_dtype == DType::kFloat) { fill(0.0f); return; }
+    if (_device != DeviceType::kCPU)
+        Ctorch_Error::throwException(ErrorPlatform::kAMD, ErrorType::DATATYPE, "zero(): device tensors are float only");
+    std::memset(_storage.raw(), 0, _storage.nbytes());
+}
+void Tensor::ones() { fill(1.0f); }
+
+Tensor Tensor::transpose(int dim0, int dim1) const {
+    if (dim0 < 0 || dim0 >= int(_shape.size()) || dim1 < 0 || dim1 >= int(_shape.size()))
+        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DIMENSION, "transpose: dimension out of range");
+    Tensor result(*this);
+    std::swap(result._shape[dim0], result._shape[dim1]);
+    std::swap(result._strides[dim0], result._strides[dim1]);
+    return result;
+}
+Tensor Tensor::t() const { return transpose(0, 1); }
+
+Tensor Tensor::view_t(const Tensor& t) {
+    if (t._shape.size() != 2)
+        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DIMENSION, "view_t: tensor is not 2-D");
+    Tensor r(AliasTag{}, t);
+    r.tensor_id_ = global_tensor_id++;
+    std::swap(r._shape[0], r._shape[1]);
+    std::swap(r._strides[0], r._strides[1]);
+    return r;
+}
+
+Tensor Tensor::contiguous() const {
+    if (is_contiguous()) return Tensor(*this);
+    std::vector<float> v = to_vector();
+    Tensor r = from_host(v.data(), _shape, _device);
+    r._requires_grad = _requires_grad;
+    return r;
+}
+
+// ------------------------------------------------------------------------------- operators
+namespace {
+
+void check_pair(const Tensor& a, const Tensor& b) {
+    if (a.dtype() != b.dtype())
+        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DATATYPE, "tensor dtypes differ");
+    if (a.device() != b.device())
+        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DEVICE_COMPAT, "tensors are on different devices");
+}
+
+// defer_record + commit_record, as every operator method of the reference does
+void tape(Tensor& result, op o, std::initializer_list<const Tensor*> inputs, int param = 0) {
+    AutoDiff* ctx = AutoDiffContext::current();
+    if (!ctx) return;
+    std::vector<Tensor*> in;
+    bool rg = false;
+    for (const Tensor* t : inputs) {
+        in.push_back(const_cast<Tensor*>(t));
+        rg = rg || t->requires_grad();
+    }
+    ctx->defer_record(result.id(), o, in, param);
+    result.set_requires_grad(rg);
+    if (rg) ctx->commit_record(result);
+}
+
+Tensor binary(const Tensor& a, const Tensor& b, op o) {
+    check_pair(a, b);
+    Tensor result = Ctorch_Scheduler::getInstance().dispatch(a, b, o);
+    tape(result, o, {&a, &b});
+    return result;
+}
+Tensor unary(const Tensor& a, op o) {
+    Tensor result = Ctorch_Scheduler::getInstance().dispatch(a, o);
+    tape(result, o, {&a});
+    return result;
+}
+
+}  // namespace
+
+Tensor Tensor::operator+(const Tensor& other) const { return binary(*this, other, op::Add); }
+Tensor Tensor::operator-(const Tensor& other) const { return binary(*this, other, op::Sub); }
+Tensor Tensor::operator*(const Tensor& other) const { return binary(*this, other, op::Mul); }
+Tensor Tensor::operator/(const Tensor& other) const { return binary(*this, other, op::Div); }
+Tensor Tensor::matmul(const Tensor& other) const { return binary(*this, other, op::MatMul); }
+Tensor Tensor::mse_loss(const Tensor& target) const { return binary(*this, target, op::MSE); }
+Tensor Tensor::mae_loss(const Tensor& target) const { return binary(*this, target, op::MAE); }
+Tensor Tensor::cross_entropy(const Tensor& target) const { return binary(*this, target, op::CE); }
+// The reference tapes Dot with its first operand only and has no gradient for it
+// (src/Tensor.cpp:593-595, src/AutoDiff.cpp:1856-1862); both operands are taped here and the tape
+// has the closed form (an extension).
+Tensor Tensor::dot(const Tensor& other) const { return binary(*this, other, op::Dot); }
+Tensor Tensor::operator-() const { return unary(*this, op::Neg); }
+Tensor Tensor::relu() const { return unary(*this, op::ReLU); }
+Tensor Tensor::sigmoid() const { return unary(*this, op::Sigmoid); }
+Tensor Tensor::tanh() const { return unary(*this, op::Tanh); }
+Tensor Tensor::sin() const { return unary(*this, op::Sin); }
+Tensor Tensor::cos() const { return unary(*this, op::Cos); }
+
+namespace {
+// tensor (op) float: the reference clones and updates in place on the host, then tapes the op with
+// a temporary 0-D tensor as second input (src/Tensor.cpp:794-796, :898-900, :961-963)
+Tensor with_scalar(const Tensor& a, float s, op o) {
+    Tensor result = scalar_op(a, s, o);
+    if (AutoDiffContext::current()) {
+        Tensor scalar_tensor(s, a.device());
+        tape(result, o, {&a, &scalar_tensor});
+        result.set_requires_grad(a.requires_grad());
+    } else {
+        result.set_requires_grad(a.requires_grad());
+    }
+    return result;
+}
+}  // namespace
+
+Tensor Tensor::operator+(float scalar) const { return with_scalar(*this, scalar, op::Add); }
+Tensor Tensor::operator*(float scalar) const { return with_scalar(*this, scalar, op::Mul); }
+Tensor Tensor::operator/(float scalar) const {
+    if (std::fabs(scalar) < FLT_EPSILON)   // src/Tensor.cpp:919-921
+        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::TENSOR_STATE, "division by a (near) zero scalar");
+    return with_scalar(*this, scalar, op::Div);
+}
+
+Tensor Tensor::sum() const {
+    Tensor result = sum_all(*this);
+    tape(result, op::Sum, {this});
+    return result;
+}
+
+Tensor Tensor::softmax(int dim) const {
+    if (_shape.empty())
+        Ctorch_Error::throwException(ErrorPlatform::kAMD, ErrorType::DIMENSION, "softmax: 0-D tensor");
+    int rank = int(_shape.size());
+    if (dim < 0) dim += rank;
+    if (dim < 0 || dim >= rank)
+        Ctorch_Error::throwException(ErrorPlatform::kAMD, ErrorType::DIMENSION, "softmax: dim out of range");
+    if (rank > 2)
+        Ctorch_Error::throwException(ErrorPlatform::kAMD, ErrorType::DIMENSION, "softmax: only 1-D / 2-D tensors");
+    Tensor result = softmax_dim(*this, dim);
+    tape(result, op::Softmax, {this}, dim);
+    return result;
+}
+
+// --------------------------------------------------------------------------------- autograd
+void Tensor::backward() const {
+    if (!AutoDiffContext::current())
+        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::TENSOR_STATE, "backward needs an autograd context");
+    if (!_requires_grad)
+        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::TENSOR_STATE, "tensor does not require grad");
+    if (is_cleared() || numel() == 0)
+        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::TENSOR_STATE, "tensor has no data");
+    AutoDiffContext::current()->backward(const_cast<Tensor&>(*this));
+}
+void Tensor::backward(const Tensor& grad_output) const {
+    if (!AutoDiffContext::current())
+        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::TENSOR_STATE, "backward needs an autograd context");
+    if (!_requires_grad)
+        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::TENSOR_STATE, "tensor does not require grad");
+    AutoDiffContext::current()->backward(const_cast<Tensor&>(*this), Tensor(grad_output));
+}
+
+void backward(Tensor& root) {
+    if (AutoDiffContext::current()) AutoDiffContext::current()->backward(root);
+}
+void backward(Tensor& root, Tensor grad_output) {
+    if (AutoDiffContext::current()) AutoDiffContext::current()->backward(root, std::move(grad_output));
+}
+Tensor grad(const Tensor& t) {
+    if (AutoDiffContext::current()) return AutoDiffContext::current()->get_grad(&t);
+    return Tensor();
+}
+Tensor matMul(const Tensor& a, const Tensor& b) { return Ctorch_Scheduler::getInstance().dispatch(a, b, op::MatMul); }
+
+bool Ctorch_Scheduler::isDeviceAvailable(DeviceType dev_type) {
+    if (dev_type != DeviceType::kAMD) return false;
+    try {
+        ctorch_amd_host::init_device();
+        return true;
+    } catch (const std::exception&) {
+        return false;
+    }
+}

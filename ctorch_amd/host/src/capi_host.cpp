@@ -1,0 +1,313 @@
+// C doorway into the host front-end for in-process tests: flat fp32 host arrays in, the operator /
+// autograd path through Tensor, Ctorch_Scheduler, the <Op>_AMD_kernel shims and the tape on the
+// MI355X, results copied back.  The entry points have the shape of the ones the tests use for the
+// reference library, so one test body can drive either.  A negative return value means the call
+// threw (-1) or produced an empty tensor (-2).
+#include "Tensor.h"
+#include "AutoDiff.h"
+#include "Ctorch_Error.h"
+#include "Ctorch_Scheduler.h"
+
+#include <cstring>
+#include <vector>
+
+namespace {
+
+std::vector<size_t> shape_of(const long* dims, int nd) {
+    std::vector<size_t> s;
+    for (int i = 0; i < nd; ++i) s.push_back(static_cast<size_t>(dims[i]));
+    return s;
+}
+
+Tensor make(const float* src, const long* dims, int nd) {
+    return Tensor::from_host(src, shape_of(dims, nd), DeviceType::kAMD);
+}
+
+long emit(const Tensor& t, float* dst) {
+    if (t.numel() == 0 || t.is_cleared()) return -2;   // the "empty Tensor()" error return
+    std::vector<float> v = t.to_vector();
+    std::memcpy(dst, v.data(), v.size() * sizeof(float));
+    return static_cast<long>(v.size());
+}
+
+// op codes shared with the Python side (tests/support.py)
+enum Code {
+    kAdd = 0, kSub = 1, kMul = 2, kDiv = 3, kMatMul = 4, kDot = 5, kMSE = 6, kMAE = 7, kCE = 8,
+    kNeg = 20, kReLU = 21, kSin = 22, kCos = 23, kTanh = 24, kSigmoid = 25, kSoftmaxKernel = 26
+};
+
+Tensor run_binary(int code, const Tensor& a, const Tensor& b) {
+    switch (code) {
+        case kAdd: return a + b;
+        case kSub: return a - b;
+        case kMul: return a * b;
+        case kDiv: return a / b;
+        case kMatMul: return a.matmul(b);
+        case kDot: return a.dot(b);
+        case kMSE: return a.mse_loss(b);
+        case kMAE: return a.mae_loss(b);
+        case kCE: return a.cross_entropy(b);
+    }
+    throw std::runtime_error("bad binary code");
+}
+
+Tensor run_unary(int code, const Tensor& a) {
+    switch (code) {
+        case kNeg: return -a;
+        case kReLU: return a.relu();
+        case kSin: return a.sin();
+        case kCos: return a.cos();
+        case kTanh: return a.tanh();
+        case kSigmoid: return a.sigmoid();
+        case kSoftmaxKernel: return Softmax_AMD_kernel(a);
+    }
+    throw std::runtime_error("bad unary code");
+}
+
+}  // namespace
+
+extern "C" {
+
+void cth_quiet() { Ctorch_Error::setPrintLevel(PrintLevel::MINIUM); }
+
+// 0: gradient of a row-broadcast operand = column sum (default); 1: the reference's row-0 slice.
+// Applies to the contexts the entry points below create.
+static int g_row0 = 0;
+void cth_set_reference_row0(int on) { g_row0 = on; }
+static void configure(AutoDiff& ctx) {
+    ctx.set_broadcast_grad(g_row0 ? BroadcastGrad::kReferenceRow0 : BroadcastGrad::kColumnSum);
+}
+
+long cth_binary(int code, const float* a, const long* ad, int an, const float* b, const long* bd,
+                int bn, float* out) {
+    try {
+        Tensor ta = make(a, ad, an), tb = make(b, bd, bn);
+        return emit(run_binary(code, ta, tb), out);
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
+long cth_unary(int code, const float* a, const long* ad, int an, float* out) {
+    try {
+        Tensor ta = make(a, ad, an);
+        return emit(run_unary(code, ta), out);
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
+// tensor (op) host scalar: which = 0 '+', 1 '*', 2 '/'
+long cth_scalar(int which, const float* a, const long* ad, int an, float s, float* out) {
+    try {
+        Tensor ta = make(a, ad, an);
+        Tensor r = which == 0 ? ta + s : which == 1 ? ta * s : ta / s;
+        return emit(r, out);
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
+long cth_sum(const float* a, const long* ad, int an, float* out) {
+    try {
+        return emit(make(a, ad, an).sum(), out);
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
+long cth_softmax(const float* a, const long* ad, int an, int dim, float* out) {
+    try {
+        return emit(make(a, ad, an).softmax(dim), out);
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
+// C = op(A) * op(B) with op = the reference's t() (deep copy + stride swap) when the flag is set.
+// A is stored [am, ak] row-major; ta != 0 multiplies by its transpose, likewise B.
+long cth_matmul_t(const float* a, long ar, long ac, int ta, const float* b, long br, long bc, int tb,
+                  float* out) {
+    try {
+        long ad[2] = {ar, ac}, bd[2] = {br, bc};
+        Tensor A = make(a, ad, 2), B = make(b, bd, 2);
+        Tensor At = ta ? A.t() : A, Bt = tb ? B.t() : B;
+        return emit(At.matmul(Bt), out);
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
+// d/dx of  sum( f(x) * w )  through the reference's tape: the upstream gradient of f is w.
+long cth_grad_unary(int code, const float* x, const long* xd, int xn, const float* w, float* dx) {
+    try {
+        AutoDiff ctx;
+        configure(ctx);
+        AutoDiffContext::Guard guard(&ctx);
+        Tensor tx = make(x, xd, xn), tw = make(w, xd, xn);
+        tx.requires_grad(true);
+        Tensor y = run_unary(code, tx);
+        Tensor z = y * tw;
+        Tensor s = z.sum();
+        backward(s);
+        return emit(grad(tx), dx);
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
+long cth_grad_softmax(const float* x, const long* xd, int xn, int dim, const float* w, float* dx) {
+    try {
+        AutoDiff ctx;
+        configure(ctx);
+        AutoDiffContext::Guard guard(&ctx);
+        Tensor tx = make(x, xd, xn), tw = make(w, xd, xn);
+        tx.requires_grad(true);
+        Tensor y = tx.softmax(dim);
+        Tensor z = y * tw;
+        Tensor s = z.sum();
+        backward(s);
+        return emit(grad(tx), dx);
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
+// d/da, d/db of sum( (a op b) * w ); w has the result's shape (wd, wn).
+long cth_grad_binary(int code, const float* a, const long* ad, int an, const float* b,
+                     const long* bd, int bn, const float* w, const long* wd, int wn, float* da,
+                     float* db) {
+    try {
+        AutoDiff ctx;
+        configure(ctx);
+        AutoDiffContext::Guard guard(&ctx);
+        Tensor ta = make(a, ad, an), tb = make(b, bd, bn), tw = make(w, wd, wn);
+        ta.requires_grad(true);
+        tb.requires_grad(true);
+        Tensor y = run_binary(code, ta, tb);
+        Tensor z = y * tw;
+        Tensor s = z.sum();
+        backward(s);
+        long r1 = emit(grad(ta), da);
+        long r2 = emit(grad(tb), db);
+        return (r1 < 0 || r2 < 0) ? -2 : r1 + r2;
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
+// d/dpred of  loss(pred, target) * scale   (loss in MSE / MAE / CE); the upstream gradient of the
+// loss node is then the 0-D value `scale`.
+long cth_grad_loss(int code, const float* p, const long* pd, int pn, const float* t, const long* td,
+                   int tn, float scale, float* loss_out, float* dp) {
+    try {
+        AutoDiff ctx;
+        configure(ctx);
+        AutoDiffContext::Guard guard(&ctx);
+        Tensor tp = make(p, pd, pn), tt = make(t, td, tn);
+        tp.requires_grad(true);
+        Tensor l = run_binary(code, tp, tt);
+        if (l.numel() == 0) return -2;
+        loss_out[0] = l.item<float>();
+        Tensor root = l * scale;
+        backward(root);
+        return emit(grad(tp), dp);
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
+// Elementwise chain: c = a*b + 5, d = relu(c), s = d.sum(), s.backward().
+long cth_chain(const float* a, const float* b, long n, float* s_out, float* ga, float* gb) {
+    try {
+        AutoDiff ctx;
+        configure(ctx);
+        AutoDiffContext::Guard guard(&ctx);
+        long d1[1] = {n};
+        Tensor ta = make(a, d1, 1), tb = make(b, d1, 1);
+        ta.requires_grad(true);
+        tb.requires_grad(true);
+        Tensor c = ta * tb + 5.0f;
+        Tensor d = c.relu();
+        Tensor s = d.sum();
+        s_out[0] = s.item<float>();
+        s.backward();
+        emit(grad(ta), ga);
+        emit(grad(tb), gb);
+        return n;
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
+// One-hidden-layer MLP step: logits = relu(x*W1 + b1)*W2 + b2, loss = CE_sum(logits, onehot),
+// backward to W1, b1, W2, b2.  `onehot` is [B, C].
+long cth_mlp_step(const float* x, long B, long I, const float* W1, const float* b1, long H,
+                  const float* W2, const float* b2, long C, const float* onehot, float* loss_out,
+                  float* logits_out, float* gW1, float* gb1, float* gW2, float* gb2, int target_is_index) {
+    try {
+        AutoDiff ctx;
+        configure(ctx);
+        AutoDiffContext::Guard guard(&ctx);
+        long xd[2] = {B, I}, w1d[2] = {I, H}, b1d[1] = {H}, w2d[2] = {H, C}, b2d[1] = {C},
+             yd[2] = {B, C}, yi[1] = {B};
+        Tensor tx = make(x, xd, 2), tW1 = make(W1, w1d, 2), tb1 = make(b1, b1d, 1),
+               tW2 = make(W2, w2d, 2), tb2 = make(b2, b2d, 1),
+               ty = target_is_index ? make(onehot, yi, 1) : make(onehot, yd, 2);
+        tW1.requires_grad(true);
+        tb1.requires_grad(true);
+        tW2.requires_grad(true);
+        tb2.requires_grad(true);
+        Tensor h = (tx.matmul(tW1) + tb1).relu();
+        Tensor logits = h.matmul(tW2) + tb2;
+        Tensor loss = logits.cross_entropy(ty);
+        loss_out[0] = loss.item<float>();
+        emit(logits, logits_out);
+        backward(loss);
+        emit(grad(tW1), gW1);
+        emit(grad(tb1), gb1);
+        emit(grad(tW2), gW2);
+        emit(grad(tb2), gb2);
+        return B;
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
+// Broadcast expression with the row vector materialised by hand (the reference's Div needs equal
+// shapes): Y = sigmoid(X / R) - tanh(X) * sin(X) + cos(-X); L = mse(Y,T) + mae(Y,T); one backward.
+long cth_expr(const float* X, const float* R, const float* T, long rows, long cols, float* y_out,
+              float* mse_out, float* mae_out, float* gX, float* gR, int r_is_row_vector) {
+    try {
+        AutoDiff ctx;
+        configure(ctx);
+        AutoDiffContext::Guard guard(&ctx);
+        long d[2] = {rows, cols}, dv[1] = {cols};
+        Tensor tX = make(X, d, 2), tR = r_is_row_vector ? make(R, dv, 1) : make(R, d, 2), tT = make(T, d, 2);
+        tX.requires_grad(true);
+        tR.requires_grad(true);
+        Tensor q = tX / tR;
+        Tensor s1 = q.sigmoid();
+        Tensor th = tX.tanh();
+        Tensor sn = tX.sin();
+        Tensor m = th * sn;
+        Tensor d1 = s1 - m;
+        Tensor ng = -tX;
+        Tensor cs = ng.cos();
+        Tensor Y = d1 + cs;
+        Tensor l1 = Y.mse_loss(tT);
+        Tensor l2 = Y.mae_loss(tT);
+        Tensor L = l1 + l2;
+        emit(Y, y_out);
+        mse_out[0] = l1.item<float>();
+        mae_out[0] = l2.item<float>();
+        backward(L);
+        emit(grad(tX), gX);
+        emit(grad(tR), gR);
+        return rows * cols;
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
+}  // extern "C"

@@ -1,0 +1,307 @@
+// The AMD column of the scheduler: <Op>_AMD_kernel shims with the reference's kernel signatures
+// (src/kernels/kernels.h:23,31).  Each one checks what its CPU-BASIC twin checks, allocates the
+// result in HBM and calls the extern "C" launch layer on the default stream.  Launches are
+// asynchronous; the host only waits where it reads a value (item(), to(kCPU), the CrossEntropy
+// label-range flag).
+#include "kernels.h"
+
+#include "ctorch_amd.h"
+
+namespace ctorch_amd_host {
+namespace {
+
+constexpr ErrorPlatform kP = ErrorPlatform::kAMD;
+
+void run(int rc, const char* what) {
+    if (rc == CTAMD_OK) return;
+    ErrorType t = rc == CTAMD_EINVAL ? ErrorType::DIMENSION : rc == CTAMD_ENOMEM ? ErrorType::MEMORY : ErrorType::KERNEL_LAUNCH;
+    Ctorch_Error::throwException(kP, t, std::string(what) + ": " + ctamd_last_error());
+}
+
+void check_device(const Tensor& a, const char* who) {
+    if (a.device() != DeviceType::kAMD)
+        Ctorch_Error::throwException(DeviceTypeToErrorPlatform(a.device()), ErrorType::DEVICE_COMPAT,
+                                     std::string(who) + ": tensor is not on the AMD device");
+    if (a.dtype() != DType::kFloat)
+        Ctorch_Error::throwException(kP, ErrorType::DATATYPE, std::string(who) + ": only float32 tensors");
+}
+
+Tensor like(const Tensor& a) { return Tensor(ShapeTag{}, a.sizes(), DType::kFloat, DeviceType::kAMD, false); }
+Tensor scalar0d() { return Tensor(ShapeTag{}, {}, DType::kFloat, DeviceType::kAMD, false); }
+
+typedef int (*Bin)(const float*, const float*, float*, size_t, void*);
+typedef int (*BinRow)(const float*, const float*, float*, size_t, size_t, void*);
+typedef int (*Un)(const float*, float*, size_t, void*);
+
+struct BinaryFamily {
+    const char* name;
+    Bin same, bscalar;
+    BinRow rowbcast;
+};
+const BinaryFamily kAdd{"Add_AMD_kernel", ctamd_add_f32, ctamd_add_bscalar_f32, ctamd_add_rowbcast_f32};
+const BinaryFamily kSub{"Sub_AMD_kernel", ctamd_sub_f32, ctamd_sub_bscalar_f32, ctamd_sub_rowbcast_f32};
+const BinaryFamily kMul{"Mul_AMD_kernel", ctamd_mul_f32, ctamd_mul_bscalar_f32, ctamd_mul_rowbcast_f32};
+const BinaryFamily kDiv{"Div_AMD_kernel", ctamd_div_f32, ctamd_div_bscalar_f32, ctamd_div_rowbcast_f32};
+
+bool row_broadcastable(const Tensor& a, const Tensor& b) {
+    return b.sizes().size() == 1 && a.sizes().size() == 2 && b.sizes()[0] == a.sizes()[1];
+}
+
+// Shape rules: same shape; b with one element (Add_BASIC_kernel.cpp:23,48-53; 0-D operands of
+// Sub / Mul: Sub_BASIC_kernel.cpp:25-32); a [rows, cols] with b [cols] (Add_BASIC_kernel.cpp:27-29).
+// A 0-D `a` against a larger `b` follows the reference per op: Sub and Mul broadcast it, Add and
+// Div do not support it.
+Tensor elementwise(const BinaryFamily& f, const Tensor& a, const Tensor& b, bool a_scalar_ok) {
+    check_device(a, f.name);
+    check_device(b, f.name);
+    if (a.sizes() == b.sizes()) {
+        Tensor r = like(a);
+        run(f.same(a.fptr(), b.fptr(), r.fptr(), a.numel(), nullptr), f.name);
+        return r;
+    }
+    if (b.numel() == 1) {
+        Tensor r = like(a);
+        run(f.bscalar(a.fptr(), b.fptr(), r.fptr(), a.numel(), nullptr), f.name);
+        return r;
+    }
+    if (row_broadcastable(a, b)) {
+        Tensor r = like(a);
+        run(f.rowbcast(a.fptr(), b.fptr(), r.fptr(), a.sizes()[0], a.sizes()[1], nullptr), f.name);
+        return r;
+    }
+    if (a_scalar_ok && a.dim() == 0) {
+        Tensor r = like(b);
+        if (&f == &kMul) run(ctamd_mul_bscalar_f32(b.fptr(), a.fptr(), r.fptr(), b.numel(), nullptr), f.name);
+        else run(ctamd_rsub_ascalar_f32(a.fptr(), b.fptr(), r.fptr(), b.numel(), nullptr), f.name);
+        return r;
+    }
+    Ctorch_Error::throwException(kP, ErrorType::DIMENSION, std::string(f.name) + ": shapes differ and cannot be broadcast");
+}
+
+Tensor map(Un fn, const char* name, const Tensor& a) {
+    check_device(a, name);
+    Tensor r = like(a);
+    run(fn(a.fptr(), r.fptr(), a.numel(), nullptr), name);
+    return r;
+}
+
+Tensor reduce2(int (*fn)(const float*, const float*, float*, size_t, void*), const char* name, const Tensor& a,
+               const Tensor& b, bool same_shape) {
+    check_device(a, name);
+    check_device(b, name);
+    if (same_shape ? a.sizes() != b.sizes() : a.numel() != b.numel())
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, std::string(name) + ": operand sizes differ");
+    Tensor r = scalar0d();
+    run(fn(a.fptr(), b.fptr(), r.fptr(), a.numel(), nullptr), name);
+    return r;
+}
+
+void rows_cols(const Tensor& a, size_t& rows, size_t& cols) {
+    if (a.dim() == 1) { rows = 1; cols = a.sizes()[0]; }
+    else { rows = a.sizes()[0]; cols = a.sizes()[1]; }
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------ helpers for Tensor / tape
+Tensor scalar_op(const Tensor& a, float s, op which) {
+    check_device(a, "tensor (op) float");
+    Tensor r = like(a);
+    int rc = which == op::Add ? ctamd_add_scalar_f32(a.fptr(), s, r.fptr(), a.numel(), nullptr)
+           : which == op::Mul ? ctamd_mul_scalar_f32(a.fptr(), s, r.fptr(), a.numel(), nullptr)
+                              : ctamd_div_scalar_f32(a.fptr(), s, r.fptr(), a.numel(), nullptr);
+    run(rc, "tensor (op) float");
+    return r;
+}
+Tensor sum_all(const Tensor& a) {
+    check_device(a, "sum");
+    Tensor r = scalar0d();
+    run(ctamd_sum_f32(a.fptr(), r.fptr(), a.numel(), nullptr), "sum");
+    return r;
+}
+Tensor softmax_dim(const Tensor& a, int dim) {
+    check_device(a, "softmax");
+    Tensor r = like(a);
+    size_t rows, cols;
+    rows_cols(a, rows, cols);
+    if (a.dim() == 1 || dim == 1) run(ctamd_softmax_rows_f32(a.fptr(), r.fptr(), rows, cols, nullptr), "softmax");
+    else run(ctamd_softmax_cols_f32(a.fptr(), r.fptr(), rows, cols, nullptr), "softmax");
+    return r;
+}
+Tensor filled(const std::vector<size_t>& shape, float v, DeviceType device) {
+    Tensor r(ShapeTag{}, shape, DType::kFloat, device, false);
+    if (device == DeviceType::kAMD) run(ctamd_fill_f32(r.fptr(), v, r.numel(), nullptr), "fill");
+    else for (size_t i = 0; i < r.numel(); ++i) r.data<float>()[i] = v;
+    return r;
+}
+Tensor filled_from(const std::vector<size_t>& shape, const Tensor& s) {
+    check_device(s, "fill");
+    Tensor r(ShapeTag{}, shape, DType::kFloat, DeviceType::kAMD, false);
+    run(ctamd_fill_from_f32(r.fptr(), s.fptr(), r.numel(), nullptr), "fill");
+    return r;
+}
+void accumulate(Tensor& grad, const Tensor& val) {
+    check_device(grad, "accumulate");
+    check_device(val, "accumulate");
+    if (grad.numel() != val.numel())
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "accumulate: gradient sizes differ");
+    run(ctamd_accumulate_f32(grad.fptr(), val.fptr(), grad.numel(), nullptr), "accumulate");
+}
+Tensor column_sum(const Tensor& g) {
+    check_device(g, "column_sum");
+    Tensor r(ShapeTag{}, {g.sizes()[1]}, DType::kFloat, DeviceType::kAMD, false);
+    run(ctamd_colsum_f32(g.fptr(), r.fptr(), g.sizes()[0], g.sizes()[1], nullptr), "column_sum");
+    return r;
+}
+Tensor first_row(const Tensor& g) {
+    check_device(g, "first_row");
+    Tensor r(ShapeTag{}, {g.sizes()[1]}, DType::kFloat, DeviceType::kAMD, false);
+    device_copy_d2d(r.fptr(), g.fptr(), g.sizes()[1] * sizeof(float));
+    return r;
+}
+bool any_abs_lt_eps(const Tensor& b) {
+    check_device(b, "any_abs_lt_eps");
+    Tensor flag(ShapeTag{}, {}, DType::kFloat, DeviceType::kAMD, false);   // 4 bytes, read as int32
+    run(ctamd_any_abs_lt_eps_f32(b.fptr(), reinterpret_cast<int32_t*>(flag.fptr()), b.numel(), nullptr), "any_abs_lt_eps");
+    int32_t v = 0;
+    device_copy_d2h(&v, flag.fptr(), sizeof(v));
+    return v != 0;
+}
+
+namespace {
+Tensor grad2(int (*fn)(const float*, const float*, float*, size_t, void*), const char* name, const Tensor& x,
+             const Tensor& g) {
+    check_device(x, name);
+    check_device(g, name);
+    if (x.numel() != g.numel()) Ctorch_Error::throwException(kP, ErrorType::DIMENSION, std::string(name) + ": sizes differ");
+    Tensor r = like(x);
+    run(fn(x.fptr(), g.fptr(), r.fptr(), x.numel(), nullptr), name);
+    return r;
+}
+}  // namespace
+Tensor relu_backward(const Tensor& x, const Tensor& g) { return grad2(ctamd_relu_backward_f32, "relu_backward", x, g); }
+Tensor sigmoid_backward(const Tensor& x, const Tensor& g) { return grad2(ctamd_sigmoid_backward_f32, "sigmoid_backward", x, g); }
+Tensor tanh_backward(const Tensor& x, const Tensor& g) { return grad2(ctamd_tanh_backward_f32, "tanh_backward", x, g); }
+Tensor sin_backward(const Tensor& x, const Tensor& g) { return grad2(ctamd_sin_backward_f32, "sin_backward", x, g); }
+Tensor cos_backward(const Tensor& x, const Tensor& g) { return grad2(ctamd_cos_backward_f32, "cos_backward", x, g); }
+Tensor softmax_backward(const Tensor& y, const Tensor& g, int dim) {
+    check_device(y, "softmax_backward");
+    check_device(g, "softmax_backward");
+    Tensor r = like(y);
+    size_t rows, cols;
+    rows_cols(y, rows, cols);
+    if (y.dim() == 1 || dim == 1) run(ctamd_softmax_backward_rows_f32(y.fptr(), g.fptr(), r.fptr(), rows, cols, nullptr), "softmax_backward");
+    else run(ctamd_softmax_backward_cols_f32(y.fptr(), g.fptr(), r.fptr(), rows, cols, nullptr), "softmax_backward");
+    return r;
+}
+Tensor mse_backward(const Tensor& p, const Tensor& t, const Tensor& g) {
+    check_device(p, "mse_backward");
+    Tensor r = like(p);
+    run(ctamd_mse_backward_f32(p.fptr(), t.fptr(), g.fptr(), r.fptr(), p.numel(), nullptr), "mse_backward");
+    return r;
+}
+Tensor mae_backward(const Tensor& p, const Tensor& t, const Tensor& g) {
+    check_device(p, "mae_backward");
+    Tensor r = like(p);
+    run(ctamd_mae_backward_f32(p.fptr(), t.fptr(), g.fptr(), r.fptr(), p.numel(), nullptr), "mae_backward");
+    return r;
+}
+Tensor cross_entropy_backward(const Tensor& x, const Tensor& target, const Tensor& g) {
+    check_device(x, "cross_entropy_backward");
+    if (x.dim() != 1 && x.dim() != 2)
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "cross_entropy_backward: logits must be 1-D or 2-D");
+    size_t rows, cols;
+    rows_cols(x, rows, cols);
+    Tensor r = like(x);
+    if (x.sizes() == target.sizes())
+        run(ctamd_cross_entropy_backward_onehot_f32(x.fptr(), target.fptr(), g.fptr(), r.fptr(), rows, cols, nullptr), "cross_entropy_backward");
+    else if (target.dim() == 1 && x.dim() == 2 && target.sizes()[0] == rows)
+        run(ctamd_cross_entropy_backward_index_f32(x.fptr(), target.fptr(), g.fptr(), r.fptr(), rows, cols, nullptr), "cross_entropy_backward");
+    else
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "cross_entropy_backward: target shape not understood");
+    return r;
+}
+Tensor div_backward_b(const Tensor& a, const Tensor& b, const Tensor& g) {
+    check_device(a, "div_backward");
+    Tensor r = like(a);
+    run(ctamd_div_backward_b_f32(a.fptr(), b.fptr(), g.fptr(), r.fptr(), a.numel(), nullptr), "div_backward");
+    return r;
+}
+
+}  // namespace ctorch_amd_host
+
+using namespace ctorch_amd_host;
+
+// ----------------------------------------------------------------------- registered kernels
+Tensor Add_AMD_kernel(const Tensor& a, const Tensor& b) { return elementwise(kAdd, a, b, false); }
+Tensor Sub_AMD_kernel(const Tensor& a, const Tensor& b) { return elementwise(kSub, a, b, true); }
+Tensor Mul_AMD_kernel(const Tensor& a, const Tensor& b) { return elementwise(kMul, a, b, true); }
+Tensor Div_AMD_kernel(const Tensor& a, const Tensor& b) { return elementwise(kDiv, a, b, false); }
+
+// MatMul_BASIC_kernel.cpp:25-30: 2-D only, inner extents must agree (both throw); operands may be
+// strided views (t()).
+Tensor MatMul_AMD_kernel(const Tensor& a, const Tensor& b) {
+    check_device(a, "MatMul_AMD_kernel");
+    check_device(b, "MatMul_AMD_kernel");
+    if (a.shape().size() != 2 || b.shape().size() != 2)
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "MatMul_AMD_kernel: only 2-D tensors");
+    if (a.shape()[1] != b.shape()[0])
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "MatMul_AMD_kernel: inner dimensions differ");
+    size_t m = a.shape()[0], k = a.shape()[1], n = b.shape()[1];
+    Tensor r(ShapeTag{}, {m, n}, DType::kFloat, DeviceType::kAMD, false);
+    run(ctamd_matmul_f32(a.fptr(), int64_t(a.strides()[0]), int64_t(a.strides()[1]), b.fptr(), int64_t(b.strides()[0]),
+                         int64_t(b.strides()[1]), r.fptr(), int64_t(m), int64_t(n), int64_t(k), nullptr),
+        "MatMul_AMD_kernel");
+    return r;
+}
+Tensor Dot_AMD_kernel(const Tensor& a, const Tensor& b) { return reduce2(ctamd_dot_f32, "Dot_AMD_kernel", a, b, false); }
+Tensor MSE_AMD_kernel(const Tensor& a, const Tensor& b) { return reduce2(ctamd_mse_f32, "MSE_AMD_kernel", a, b, true); }
+Tensor MAE_AMD_kernel(const Tensor& a, const Tensor& b) { return reduce2(ctamd_mae_f32, "MAE_AMD_kernel", a, b, true); }
+
+// CrossEntropy_BASIC_kernel.cpp: one-hot / soft targets of the logits' shape (:41-82) or class
+// indices [rows] (:88-120); an unsupported shape or an out-of-range index logs an error and
+// returns an empty Tensor (:86, :96-100, :124).  Loss is the SUM over rows.
+Tensor CrossEntropy_AMD_kernel(const Tensor& a, const Tensor& b) {
+    check_device(a, "CrossEntropy_AMD_kernel");
+    check_device(b, "CrossEntropy_AMD_kernel");
+    if (a.sizes() == b.sizes()) {
+        if (a.dim() != 1 && a.dim() != 2) {
+            Ctorch_Error::log(ErrorLevel::ERROR, kP, ErrorType::DIMENSION, "CrossEntropy_AMD_kernel: one-hot targets need 1-D / 2-D logits");
+            return Tensor();
+        }
+        size_t rows, cols;
+        rows_cols(a, rows, cols);
+        Tensor r = scalar0d();
+        run(ctamd_cross_entropy_onehot_f32(a.fptr(), b.fptr(), r.fptr(), rows, cols, nullptr), "CrossEntropy_AMD_kernel");
+        return r;
+    }
+    if (b.dim() == 1 && a.dim() == 2 && b.sizes()[0] == a.sizes()[0]) {
+        Tensor r = scalar0d();
+        Tensor status = scalar0d();   // 4 bytes, used as int32
+        run(ctamd_cross_entropy_index_f32(a.fptr(), b.fptr(), r.fptr(), reinterpret_cast<int32_t*>(status.fptr()),
+                                          a.sizes()[0], a.sizes()[1], nullptr), "CrossEntropy_AMD_kernel");
+        int32_t bad = 0;
+        device_copy_d2h(&bad, status.fptr(), sizeof(bad));
+        if (bad) {
+            Ctorch_Error::log(ErrorLevel::ERROR, kP, ErrorType::TENSOR_STATE, "CrossEntropy_AMD_kernel: class index out of range");
+            return Tensor();
+        }
+        return r;
+    }
+    Ctorch_Error::log(ErrorLevel::ERROR, kP, ErrorType::DIMENSION, "CrossEntropy_AMD_kernel: incompatible shapes");
+    return Tensor();
+}
+
+Tensor Neg_AMD_kernel(const Tensor& a) { return map(ctamd_neg_f32, "Neg_AMD_kernel", a); }
+Tensor ReLU_AMD_kernel(const Tensor& a) { return map(ctamd_relu_f32, "ReLU_AMD_kernel", a); }
+Tensor Cos_AMD_kernel(const Tensor& a) { return map(ctamd_cos_f32, "Cos_AMD_kernel", a); }
+Tensor Sin_AMD_kernel(const Tensor& a) { return map(ctamd_sin_f32, "Sin_AMD_kernel", a); }
+Tensor Tanh_AMD_kernel(const Tensor& a) { return map(ctamd_tanh_f32, "Tanh_AMD_kernel", a); }
+Tensor Sigmoid_AMD_kernel(const Tensor& a) { return map(ctamd_sigmoid_f32, "Sigmoid_AMD_kernel", a); }
+// Softmax_BASIC_kernel.cpp:26-35, :95-98: float only, 1-D or 2-D (last dimension), throws otherwise
+Tensor Softmax_AMD_kernel(const Tensor& a) {
+    check_device(a, "Softmax_AMD_kernel");
+    if (a.dim() != 1 && a.dim() != 2)
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "Softmax_AMD_kernel: only 1-D / 2-D tensors");
+    return softmax_dim(a, int(a.dim()) - 1);
+}

@@ -312,15 +312,32 @@ def _dims(shape):
     return arr, len(shape)
 
 
-class Reference:
-    """The real reference library through oracle/ref_driver.cpp.  Exists only where it was built."""
+class _Lib:
+    """Maps lib.ref_<name> to <prefix><name> of a loaded library."""
 
-    def __init__(self):
-        self.lib = C.CDLL(os.path.join(ORACLE_DIR, "_ref", "libctorch_ref.so"))
-        for n in ("ref_binary", "ref_unary", "ref_scalar", "ref_sum", "ref_softmax", "ref_matmul_t",
-                  "ref_grad_unary", "ref_grad_softmax", "ref_grad_binary", "ref_grad_loss", "ref_chain",
-                  "ref_mlp_step", "ref_expr"):
-            getattr(self.lib, n).restype = C.c_long
+    def __init__(self, cdll, prefix):
+        self._cdll, self._prefix = cdll, prefix
+
+    def __getattr__(self, name):
+        assert name.startswith("ref_")
+        return getattr(self._cdll, self._prefix + name[4:])
+
+
+class Reference:
+    """The real reference library through oracle/ref_driver.cpp.  Exists only where it was built.
+
+    HostLayer (below) drives this repository's C++ front-end on the GPU through entry points of the
+    same shape, so the methods here serve both."""
+
+    ENTRY_POINTS = ("binary", "unary", "scalar", "sum", "softmax", "matmul_t", "grad_unary", "grad_softmax",
+                    "grad_binary", "grad_loss", "chain", "mlp_step", "expr")
+
+    def __init__(self, path=None, prefix="ref_"):
+        cdll = C.CDLL(path or os.path.join(ORACLE_DIR, "_ref", "libctorch_ref.so"))
+        self.cdll = cdll
+        self.lib = _Lib(cdll, prefix)
+        for n in self.ENTRY_POINTS:
+            getattr(cdll, prefix + n).restype = C.c_long
         self.lib.ref_quiet()
 
     def binary(self, code, a, b, out_shape):
@@ -414,8 +431,8 @@ class Reference:
         assert rc == a.size
         return np.float32(s.value), ga, gb
 
-    def mlp_step(self, x, W1, b1, W2, b2, onehot):
-        x, W1, b1, W2, b2, onehot = map(f32, (x, W1, b1, W2, b2, onehot))
+    def mlp_step(self, x, W1, b1, W2, b2, target, *extra):
+        x, W1, b1, W2, b2, target = map(f32, (x, W1, b1, W2, b2, target))
         B, I = x.shape
         H = W1.shape[1]
         Cn = W2.shape[1]
@@ -423,17 +440,38 @@ class Reference:
         logits = np.empty((B, Cn), np.float32)
         gW1, gb1, gW2, gb2 = (np.empty_like(t) for t in (W1, b1, W2, b2))
         rc = self.lib.ref_mlp_step(fp(x), C.c_long(B), C.c_long(I), fp(W1), fp(b1), C.c_long(H), fp(W2), fp(b2),
-                                   C.c_long(Cn), fp(onehot), C.byref(loss), fp(logits), fp(gW1), fp(gb1),
-                                   fp(gW2), fp(gb2))
+                                   C.c_long(Cn), fp(target), C.byref(loss), fp(logits), fp(gW1), fp(gb1),
+                                   fp(gW2), fp(gb2), *extra)
         assert rc == B, rc
         return np.float32(loss.value), logits, gW1, gb1, gW2, gb2
 
-    def expr(self, X, R, T):
+    def expr(self, X, R, T, *extra):
         X, R, T = f32(X), f32(R), f32(T)
         rows, cols = X.shape
-        Y, gX, gR = np.empty_like(X), np.empty_like(X), np.empty_like(X)
+        Y, gX, gR = np.empty_like(X), np.empty_like(X), np.empty_like(R)
         mse, mae = C.c_float(0), C.c_float(0)
         rc = self.lib.ref_expr(fp(X), fp(R), fp(T), C.c_long(rows), C.c_long(cols), fp(Y), C.byref(mse),
-                               C.byref(mae), fp(gX), fp(gR))
+                               C.byref(mae), fp(gX), fp(gR), *extra)
         assert rc == rows * cols, rc
         return Y, np.float32(mse.value), np.float32(mae.value), gX, gR
+
+
+HOST_LIB = os.path.join(ROOT, "ctorch_amd", "host", "libctorch_amd_host.so")
+
+
+class HostLayer(Reference):
+    """This repository's C++ front-end (Tensor / Ctorch_Scheduler / AutoDiff over the HIP launch layer)
+    through ctorch_amd/host/src/capi_host.cpp.  Needs a GPU for every call."""
+
+    def __init__(self):
+        Reference.__init__(self, HOST_LIB, "cth_")
+
+    def set_reference_row0(self, on):
+        self.cdll.cth_set_reference_row0(int(on))
+
+    def mlp_step(self, x, W1, b1, W2, b2, target, target_is_index=False):
+        return Reference.mlp_step(self, x, W1, b1, W2, b2, target, C.c_int(int(target_is_index)))
+
+    def expr(self, X, R, T):
+        """R may be the full [rows, cols] operand or the row vector [cols] (row-broadcast Div)."""
+        return Reference.expr(self, X, R, T, C.c_int(int(np.ndim(R) == 1)))

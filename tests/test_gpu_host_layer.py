@@ -1,0 +1,203 @@
+"""The C++ front-end (Tensor / Storage / Ctorch_Scheduler / AutoDiff over the HIP launch layer),
+driven in-process through ctorch_amd/host/src/capi_host.cpp, against the CPU oracle and the golden
+vectors written from the real reference.  The test bodies read like tests/test_oracle_vs_ref.py:
+the entry points have the same shape as the ones used for the reference library."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from support import (ADD, CE, COS, DIV, DOT, MAE, MATMUL, MSE, MUL, NEG, RELU, ROOT, SIGMOID, SIN, SOFTMAX_KERNEL,
+                     SUB, TANH, HostLayer, same_bits, ulp_diff)
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+UNARY = [(NEG, "neg", 0), (RELU, "relu", 0), (SIN, "sin", 2), (COS, "cos", 2), (TANH, "tanh", 2), (SIGMOID, "sigmoid", 2)]
+
+
+@pytest.fixture(scope="module")
+def host():
+    return HostLayer()
+
+
+def close(got, want, max_ulp, what=""):
+    got, want = np.asarray(got, F), np.asarray(want, F)
+    assert got.shape == want.shape, what
+    if max_ulp == 0:
+        nan_both = np.isnan(got) & np.isnan(want)
+        assert not ((got.view(np.uint32) != want.view(np.uint32)) & ~nan_both).any(), what
+    else:
+        assert np.array_equal(np.isnan(got), np.isnan(want)), what
+        ok = ~np.isnan(want)
+        assert ulp_diff(got[ok], want[ok]).max() <= max_ulp, what
+
+
+def test_forward_operators(oracle, host):
+    print("case host forward", flush=True)
+    x = oracle.normal((37, 53), 10, 0, 3)
+    y = oracle.normal((37, 53), 20, 0, 3)
+    for code in (ADD, SUB, MUL, DIV):
+        rc, out = host.binary(code, x, y, x.shape)
+        assert rc == x.size
+        close(out, oracle.binary(code, x, y), 0, code)
+    for code, name, ulp in UNARY:
+        close(host.unary(code, x), oracle.unary(code, x), ulp, name)
+    for which, s in [(0, 5.0), (1, -2.5), (2, 3.0)]:
+        close(host.scalar(which, x, s)[1], oracle.scalar(which, x, s), 0, which)
+    b = oracle.uniform((53,), 30, 0.5, 2)
+    for code in (ADD, SUB, MUL, DIV):      # row broadcast: Add as the reference, the rest by the same convention
+        rc, out = host.binary(code, x, b, x.shape)
+        assert rc == x.size
+        close(out, oracle.binary_rowbcast(code, x, b), 0, ("rowbcast", code))
+    rc, out = host.binary(ADD, x, b[:1], x.shape)
+    close(out, oracle.add_scalar_tensor(x, b[:1]), 0, "b with one element")
+    # error behaviour kept from the reference
+    assert host.binary(ADD, b, x, x.shape)[0] == -1            # 1-D on the left: Add throws
+    assert host.binary(MATMUL, x, y, (37, 53))[0] == -1        # inner dimensions differ: throws
+    assert abs(host.sum(x) - x.astype(np.float64).sum()) <= 1e-5 * np.abs(x).sum()
+    for code, fn in [(DOT, oracle.dot), (MSE, oracle.mse), (MAE, oracle.mae)]:
+        rc, out = host.binary(code, x, y, ())
+        assert rc == 1 and abs(out - fn(x, y)) <= 1e-5 * max(abs(fn(x, y)), np.abs(x * y).sum() if code == DOT else 0)
+    for dim in (0, 1):
+        assert np.all(np.abs(host.softmax(x, dim) - oracle.softmax(x, dim)) <= 1e-5 * oracle.softmax(x, dim))
+    assert np.all(np.abs(host.unary(SOFTMAX_KERNEL, x) - oracle.softmax(x, 1)) <= 1e-5 * oracle.softmax(x, 1))
+
+
+def test_cross_entropy_target_forms_and_errors(oracle, host):
+    print("case host cross entropy", flush=True)
+    x = oracle.normal((19, 31), 40, 0, 2)
+    idx = oracle.ints((19,), 41, 31)
+    oh = np.zeros_like(x)
+    oh[np.arange(19), idx.astype(int)] = 1
+    want = oracle.ce_onehot(x, oh)
+    for t in (oh, idx):
+        rc, out = host.binary(CE, x, t, ())
+        assert rc == 1 and abs(out - want) <= 1e-5 * want
+    rc, out = host.binary(CE, x[0], oh[0], ())
+    assert rc == 1 and abs(out - oracle.ce_onehot(x[0], oh[0])) <= 1e-5 * oracle.ce_onehot(x[0], oh[0])
+    bad = idx.copy()
+    bad[3] = 31
+    assert host.binary(CE, x, bad, ())[0] == -2          # empty Tensor, as the reference
+    assert host.binary(CE, x, idx[:5], ())[0] == -2      # incompatible shapes: empty Tensor
+    # backward: one-hot as the reference; class indices are accepted too (the reference throws)
+    wantd = oracle.accumulate0(oracle.ce_bwd_onehot(x, oh, F(0.37)))
+    for t in (oh, idx):
+        rc, loss, dp = host.grad_loss(CE, x, t, 0.37)
+        assert rc == x.size and np.abs(dp - wantd).max() <= 1e-6
+
+
+def test_matmul_layouts_and_gradients(oracle, host):
+    print("case host matmul", flush=True)
+    A = oracle.normal((33, 47), 41)
+    B = oracle.normal((47, 29), 42)
+    At, Bt = np.ascontiguousarray(A.T), np.ascontiguousarray(B.T)
+    bound = 1e-5 * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64))
+    want = oracle.matmul(A, B)
+    for got in (host.matmul_t(A, 0, B, 0), host.matmul_t(A, 0, Bt, 1), host.matmul_t(At, 1, B, 0),
+                host.matmul_t(At, 1, Bt, 1)):
+        assert np.all(np.abs(got - want) <= 2 * bound)
+    W = oracle.normal((33, 29), 43)
+    rc, da, db = host.grad_binary(MATMUL, A, B, W)
+    assert rc == A.size + B.size
+    ba = 1e-5 * (np.abs(W).astype(np.float64) @ np.abs(B.T).astype(np.float64))
+    bb = 1e-5 * (np.abs(A.T).astype(np.float64) @ np.abs(W).astype(np.float64))
+    assert np.all(np.abs(da - oracle.matmul(W, B.T)) <= 2 * ba)
+    assert np.all(np.abs(db - oracle.matmul(A.T, W)) <= 2 * bb)
+
+
+def test_elementwise_gradients_through_the_tape(oracle, host, golden):
+    print("case host gradients", flush=True)
+    g = golden("backward")
+    x, y, w = g["x"], g["y"], g["w"]
+    for code, name, ulp in UNARY:
+        close(host.grad_unary(code, x, w), g["d_" + name], ulp, name)          # vs the real reference
+    for code, name in [(MSE, "mse"), (MAE, "mae")]:
+        rc, loss, dp = host.grad_loss(code, x, y, 0.37)
+        close(dp, g["d_" + name], 0, name)
+    rc, da, db = host.grad_binary(DIV, x, g["yb"], w)
+    close(da, g["d_div_a"], 0, "div a")
+    close(db, g["d_div_b"], 0, "div b")
+    rc, da, db = host.grad_binary(MUL, x, y, w)
+    close(da, g["d_mul_a"], 0, "mul a")
+    close(db, g["d_mul_b"], 0, "mul b")
+    rc, da, db = host.grad_binary(SUB, x, y, w)
+    close(da, g["d_sub_a"], 0, "sub a")
+    close(db, g["d_sub_b"], 0, "sub b")
+    yz = y.copy()
+    yz[3, 4] = 0.0
+    assert host.grad_binary(DIV, x, yz, w)[0] == -1           # zero divisor: backward throws
+    for dim in (0, 1):
+        got = host.grad_softmax(x, dim, w)
+        want = g["d_softmax_d%d" % dim]
+        assert np.abs(got - want).max() <= 1e-5 * np.abs(w).max()
+    # row-broadcast operand: column sum by default, the reference's row 0 on request
+    b = g["b"]
+    rc, da, db = host.grad_binary(ADD, x, b, w)
+    close(da, g["d_addrow_a"], 0, "add a")
+    assert np.all(np.abs(db - w.astype(np.float64).sum(0)) <= 1e-5 * np.abs(w).sum(0))
+    host.set_reference_row0(True)
+    try:
+        rc, da, db = host.grad_binary(ADD, x, b, w)
+        close(db, g["d_addrow_b"], 0, "add b, reference row-0 mode")
+    finally:
+        host.set_reference_row0(False)
+    # the other row-broadcast operators (extensions): gradients against fp64
+    for code, dfa, dfb in [(SUB, lambda: w, lambda: -w), (MUL, lambda: w * b, lambda: w * x),
+                           (DIV, lambda: w / b, lambda: -w * x / (b.astype(np.float64) ** 2))]:
+        rc, da, db = host.grad_binary(code, x, np.abs(b) + F(0.5) if code == DIV else b, w)
+        bb = (np.abs(b) + F(0.5)) if code == DIV else b
+        x64, w64, b64 = x.astype(np.float64), w.astype(np.float64), bb.astype(np.float64)
+        want_a = {SUB: w64, MUL: w64 * b64, DIV: w64 / b64}[code]
+        want_b = {SUB: -w64, MUL: w64 * x64, DIV: -w64 * x64 / b64 ** 2}[code]
+        assert np.abs(da - want_a).max() <= 1e-5 * np.abs(want_a).max(), code
+        assert np.abs(db - want_b.sum(0)).max() <= 1e-5 * np.abs(want_b).sum(0).max(), code
+
+
+def test_configurations_small(oracle, host, golden):
+    print("case host configs", flush=True)
+    g = golden("configs")
+    s, ga, gb = host.chain(g["chain_a"], g["chain_b"])
+    assert abs(s - g["chain_s"]) <= 1e-5 * abs(g["chain_s"])
+    close(ga, g["chain_ga"], 0, "chain ga")          # bit-exact against the real reference
+    close(gb, g["chain_gb"], 0, "chain gb")
+    lab = g["mlp_lab"]
+    oh = np.zeros((lab.size, 10), F)
+    oh[np.arange(lab.size), lab.astype(int)] = 1
+    args = (g["mlp_x"], g["mlp_W1"], g["mlp_b1"], g["mlp_W2"], g["mlp_b2"])
+    names = ["loss", "logits", "gW1", "gb1", "gW2", "gb2"]
+    host.set_reference_row0(True)
+    try:
+        got = host.mlp_step(*args, oh)
+    finally:
+        host.set_reference_row0(False)
+    for n, a, b in zip(names, got, [g["mlp_" + n] for n in names]):   # the reference's own numbers
+        assert np.abs(a - b).max() <= 1e-4 * max(1.0, np.abs(b).max()), n
+    want = oracle.mlp_step(*args, oh, False)                            # column-sum bias gradients
+    for target, is_index in ((oh, False), (lab, True)):
+        got = host.mlp_step(*args, target, is_index)
+        for n, a, b in zip(names, got, want):
+            assert np.abs(a - b).max() <= 1e-4 * max(1.0, np.abs(b).max()), (n, is_index)
+    X, rv, T = g["expr_X"], g["expr_r"], g["expr_T"]
+    R = np.broadcast_to(rv, X.shape).copy()
+    Y, mse, mae, gX, gR = host.expr(X, R, T)                           # materialised operand, as the reference
+    assert ulp_diff(Y, g["expr_Y"]).max() <= 2
+    assert abs(mse - g["expr_mse"]) <= 1e-5 * g["expr_mse"] and abs(mae - g["expr_mae"]) <= 1e-5 * g["expr_mae"]
+    assert np.abs(gX - g["expr_gX"]).max() <= 1e-6 * np.abs(g["expr_gX"]).max() + 1e-9
+    assert np.abs(gR - g["expr_gR"]).max() <= 1e-6 * np.abs(g["expr_gR"]).max() + 1e-9
+    Y2, mse2, mae2, gX2, gr = host.expr(X, rv, T)                      # row vector: broadcast Div + column-sum
+    assert same_bits(Y2, Y) and same_bits(gX2, gX)
+    assert np.abs(gr - g["expr_gR"].astype(np.float64).sum(0)).max() <= 1e-5 * np.abs(g["expr_gR"]).sum(0).max()
+
+
+@pytest.mark.parametrize("prog", ["test_scalar_grad", "test_tensor_grad", "test_activation_loss"])
+def test_reference_style_programs(prog):
+    """C++ programs written like the reference's own test executables (src/tests/test.cpp,
+    test_tensor_grad.cpp, test_activation_loss.cpp), on DeviceType::kAMD; exit code 0 = all
+    checks passed."""
+    print("case host program", prog, flush=True)
+    exe = os.path.join(ROOT, "ctorch_amd", "host", "tests", prog + ".bin")
+    assert os.path.exists(exe), "build it with make -C ctorch_amd/host"
+    p = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=110)
+    print(p.stdout[-3000:])
+    assert p.returncode == 0
