@@ -22,6 +22,10 @@ int launched(const char* kernel);
 // ctamd_init() and never freed.  Returns nullptr (and records an error) before ctamd_init().
 constexpr size_t kScratchFloats = size_t(1) << 24;   // 64 MiB
 float* scratch();
+// Four floats of -inf / of 0 in device memory (set up by ctamd_init): what row kernels read in
+// place of a vector that would lie beyond the end of a row.
+const float* pad_neg_inf();
+const float* pad_zero();
 // Compute units of the current device (256 on MI355X); 0 before ctamd_init().
 int compute_units();
 

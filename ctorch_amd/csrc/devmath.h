@@ -64,6 +64,14 @@ CTA_FN double cta_u2d(uint64_t u) {
 #endif
 }
 
+// a / b for a divisor shared by many elements: with rcp_b = 1.0 / (double)b computed once,
+// (float)((double)a * rcp_b) IS the correctly rounded fp32 quotient.  The exact quotient of two
+// 24-bit significands lies at least 2^-49 (relative) away from every midpoint between adjacent
+// floats and can never sit on one (that would need 2^25 to divide a 24-bit integer), while the
+// double product is within 2^-52 of it; zeros, infinities, NaN and subnormals come out as IEEE
+// division gives them.  tests/native/divcheck.c compares it with `a / b` on billions of pairs.
+CTA_FN float cta_div_rcp(float a, double rcp_b) { return (float)((double)a * rcp_b); }
+
 // tab[i] = bits(2^(i/32)) - (i << 47): adding k << 47 yields bits(2^(k/32)) for any integer k.
 CTA_TAB_SPACE uint64_t cta_exp2_tab[32] = {
     0x3ff0000000000000ULL, 0x3fefd9b0d3158574ULL, 0x3fefb5586cf9890fULL, 0x3fef9301d0125b51ULL,
@@ -77,16 +85,16 @@ CTA_TAB_SPACE uint64_t cta_exp2_tab[32] = {
 
 // `tab` is where the caller keeps the 32 entries (LDS on the device, the array above on the host).
 // Valid for every float: NaN -> NaN, +inf -> +inf, -inf -> 0, overflow -> +inf, underflow ->
-// correctly rounded subnormals and then 0.
+// correctly rounded subnormals and then 0.  Branch-free: |x| is clamped to 128 first (NaN passes
+// through), where the double-precision result is still finite and its conversion to float
+// overflows to +inf / rounds to 0 exactly where glibc's range checks return those values.
+CTA_FN float cta_exp_clamp(float x) {
+    uint32_t ux = cta_f2u(x);
+    float ax = cta_u2f(ux & 0x7fffffffu);
+    return (ax > 128.0f) ? cta_u2f((ux & 0x80000000u) | 0x43000000u) : x;
+}
 CTA_FN float cta_expf_tab(float x, const uint64_t* tab) {
-    uint32_t ax = cta_f2u(x) & 0x7fffffffu;
-    if (ax >= 0x42b00000u) {                       // |x| >= 88 or NaN
-        if (cta_f2u(x) == 0xff800000u) return 0.0f;
-        if (ax >= 0x7f800000u) return x + x;
-        if (x > 0x1.62e42ep6f) return cta_u2f(0x7f800000u);
-        if (x < -0x1.9fe368p6f) return 0.0f;
-    }
-    double xd = (double)x;
+    double xd = (double)cta_exp_clamp(x);
     const double inv_ln2_n = 0x1.71547652b82fep+0 * 32.0;
     double kd = CTA_FMA(inv_ln2_n, xd, 0x1.8p+52);   // round to nearest integer in the low bits
     uint64_t ki = cta_d2u(kd);
@@ -100,6 +108,45 @@ CTA_FN float cta_expf_tab(float x, const uint64_t* tab) {
     y = CTA_FMA(p, r2, y);
     y = y * s;
     return (float)y;
+}
+
+// The same for arguments known to be <= 0 or NaN (x - max(x) in softmax): only the lower clamp.
+CTA_FN float cta_expf_nonpos(float x, const uint64_t* tab) {
+    float xc = (x < -128.0f) ? -128.0f : x;        // NaN stays NaN
+    double xd = (double)xc;
+    const double inv_ln2_n = 0x1.71547652b82fep+0 * 32.0;
+    double kd = CTA_FMA(inv_ln2_n, xd, 0x1.8p+52);
+    uint64_t ki = cta_d2u(kd);
+    kd -= 0x1.8p+52;
+    double r = CTA_FMA(inv_ln2_n, xd, -kd);
+    double s = cta_u2d(tab[ki & 31u] + (ki << 47));
+    double p = CTA_FMA(0x1.c6af84b912394p-5 / 32768.0, r, 0x1.ebfce50fac4f3p-3 / 1024.0);
+    double r2 = r * r;
+    double y = CTA_FMA(0x1.62e42ff0c52d6p-1 / 32.0, r, 1.0);
+    y = CTA_FMA(p, r2, y);
+    return (float)(y * s);
+}
+
+// exp(x) and exp(-x) together (tanh needs both).  The reduction of -x is the mirror image of the
+// reduction of x - round-to-nearest-even is symmetric, so k' = -k and r' = -r exactly - hence
+// only the table entry and the polynomial are evaluated twice.
+CTA_FN void cta_expf_pair(float x, const uint64_t* tab, float* e_pos, float* e_neg) {
+    double xd = (double)cta_exp_clamp(x);
+    const double inv_ln2_n = 0x1.71547652b82fep+0 * 32.0;
+    const double c0 = 0x1.c6af84b912394p-5 / 32768.0, c1 = 0x1.ebfce50fac4f3p-3 / 1024.0,
+                 c2 = 0x1.62e42ff0c52d6p-1 / 32.0;
+    double kd = CTA_FMA(inv_ln2_n, xd, 0x1.8p+52);
+    uint64_t ki = cta_d2u(kd);
+    kd -= 0x1.8p+52;
+    double r = CTA_FMA(inv_ln2_n, xd, -kd);
+    double r2 = r * r;
+    uint64_t nki = 0u - ki;                       // low bits and the shifted-in exponent of -k
+    double s_pos = cta_u2d(tab[ki & 31u] + (ki << 47));
+    double s_neg = cta_u2d(tab[nki & 31u] + (nki << 47));
+    double y_pos = CTA_FMA(CTA_FMA(c0, r, c1), r2, CTA_FMA(c2, r, 1.0)) * s_pos;
+    double y_neg = CTA_FMA(CTA_FMA(-c0, r, c1), r2, CTA_FMA(-c2, r, 1.0)) * s_neg;
+    *e_pos = (float)y_pos;
+    *e_neg = (float)y_neg;
 }
 
 // sin / cos: |x| < 0.75 direct, |x| < 120 quadrant reduction with one multiply by pi/2 in double
@@ -147,32 +194,41 @@ CTA_FN double cta_reduce_large(uint32_t xi, int* np, const uint32_t* inv_pio4) {
     return x * 0x1.921FB54442D18p-62;
 }
 
-// sinf (want_cos = 0) / cosf (want_cos = 1) for every float.
+// sinf (want_cos = 0) / cosf (want_cos = 1) for every float.  One straight-line path serves
+// |y| < 120: for |y| < 0.75 the quadrant is 0 and the reduced argument is y itself, so glibc's
+// separate small-argument branches give the same bits (checked over all floats); beyond 120 the
+// 2/pi table reduction runs instead, and inf / NaN give NaN.  The quadrant's sign is applied to the
+// rounded float (both polynomials are odd / even in a way that commutes with rounding).
+CTA_FN float cta_sincos_finish(float y, uint32_t ay, int want_cos, int n, double xr) {
+    if (want_cos) n += 1;                          // cos(x) = sin(x + pi/2)
+    double x2 = xr * xr;
+    double c = cta_cos_poly(x2);
+    double sn = cta_sin_poly(xr, x2);
+    double res = (n & 1) ? c : sn;                 // both evaluated: lanes of a wave differ anyway
+    float f = cta_u2f(cta_f2u((float)res) ^ ((uint32_t)(n & 2) << 30));
+    if (!want_cos) f = (ay < 0x39800000u) ? y : f;   // |y| < 2^-12: sin(y) = y, keeps the sign of -0
+    return f;
+}
+// Straight-line path, correct for |y| < 120 (cta_sincos_is_rare(y) == 0).
+CTA_FN float cta_sincosf_fast(float y, int want_cos) {
+    uint32_t ay = cta_f2u(y) & 0x7fffffffu;
+    double x = (double)y;
+    double r = x * 0x1.45F306DC9C883p+23;          // 2/pi scaled by 2^24
+    int n = ((int32_t)r + 0x800000) >> 24;         // nearest quadrant
+    double xr = CTA_FMA(-(double)n, 0x1.921FB54442D18p0, x);
+    return cta_sincos_finish(y, ay, want_cos, n, xr);
+}
+CTA_FN int cta_sincos_is_rare(float y) { return (cta_f2u(y) & 0x7fffffffu) >= 0x42f00000u; }
+// Every float (the |y| >= 120, inf and NaN cases included).
 CTA_FN float cta_sincosf(float y, int want_cos, const uint32_t* inv_pio4) {
+    if (!cta_sincos_is_rare(y)) return cta_sincosf_fast(y, want_cos);
     uint32_t uy = cta_f2u(y);
     uint32_t ay = uy & 0x7fffffffu;
-    double x = (double)y;
+    if (ay >= 0x7f800000u) return y - y;           // inf, NaN -> NaN
     int n;
-    double xr;
-    if (ay < 0x3f400000u) {                        // top 12 bits below those of pi/4: |y| < 0.75
-        if (ay < 0x39800000u) return want_cos ? 1.0f : y;             // |y| < 2^-12
-        double x2 = x * x;
-        return want_cos ? (float)cta_cos_poly(x2) : (float)cta_sin_poly(x, x2);
-    }
-    if (ay < 0x42f00000u) {                        // |y| < 120
-        double r = x * 0x1.45F306DC9C883p+23;      // 2/pi scaled by 2^24
-        n = ((int32_t)r + 0x800000) >> 24;         // nearest quadrant
-        xr = CTA_FMA(-(double)n, 0x1.921FB54442D18p0, x);
-    } else if (ay < 0x7f800000u) {
-        xr = cta_reduce_large(uy, &n, inv_pio4);
-        if (!want_cos) n += (int)(uy >> 31) * 2;   // reduced |y|; sin is odd: sin(t + pi) = -sin(t)
-    } else {
-        return y - y;                              // inf, NaN -> NaN
-    }
-    if (want_cos) n += 1;                          // cos(x) = sin(x + pi/2)
-    double sgn = (n & 2) ? -1.0 : 1.0;
-    if (n & 1) return (float)(sgn * cta_cos_poly(xr * xr));
-    return (float)cta_sin_poly(xr * sgn, xr * xr);
+    double xr = cta_reduce_large(uy, &n, inv_pio4);
+    if (!want_cos) n += (int)(uy >> 31) * 2;       // reduced |y|; sin is odd: sin(t + pi) = -sin(t)
+    return cta_sincos_finish(y, ay, want_cos, n, xr);
 }
 
 #endif  // CTORCH_AMD_DEVMATH_H

@@ -53,19 +53,34 @@ struct RSubDevScalarF { static constexpr int kIn = 1; static constexpr bool kTab
     const float* s;
     __device__ float operator()(const float* x, const Tables&) const { return *s - x[0]; } };
 
+// a / s for one divisor shared by all elements: the correctly rounded quotient through the
+// divisor's double-precision reciprocal (devmath.h, cta_div_rcp) - 3 instructions instead of the
+// ~12 of a full fp32 division.
+struct DivByRcpF { static constexpr int kIn = 1; static constexpr bool kTables = false;
+    double rcp;
+    __device__ float operator()(const float* x, const Tables&) const { return cta_div_rcp(x[0], rcp); } };
+
 struct NegF { static constexpr int kIn = 1; static constexpr bool kTables = false;
     __device__ float operator()(const float* x, const Tables&) const { return -x[0]; } };
 // std::max(0.0f, x): (0 < x) ? x : +0  (NaN and -0 give +0)
 struct ReluF { static constexpr int kIn = 1; static constexpr bool kTables = false;
     __device__ float operator()(const float* x, const Tables&) const { return (0.0f < x[0]) ? x[0] : 0.0f; } };
-struct SinF { static constexpr int kIn = 1; static constexpr bool kTables = true;
-    __device__ float operator()(const float* x, const Tables& t) const { return cta_sincosf(x[0], 0, t.inv_pio4); } };
-struct CosF { static constexpr int kIn = 1; static constexpr bool kTables = true;
-    __device__ float operator()(const float* x, const Tables& t) const { return cta_sincosf(x[0], 1, t.inv_pio4); } };
+// Sin / Cos family: `operator()` is the straight-line path for |x| < 120; `rare(x)` tells when an
+// element needs `slow()` (the table-driven reduction for huge arguments, inf, NaN).  The kernel
+// runs the fast path for every element and repairs the rare ones afterwards, so the common case
+// carries no per-element branch.
+struct SinF { static constexpr int kIn = 1; static constexpr bool kTables = true; static constexpr bool kRare = true;
+    __device__ float operator()(const float* x, const Tables&) const { return cta_sincosf_fast(x[0], 0); }
+    __device__ bool rare(const float* x) const { return cta_sincos_is_rare(x[0]); }
+    __device__ float slow(const float* x, const Tables& t) const { return cta_sincosf(x[0], 0, t.inv_pio4); } };
+struct CosF { static constexpr int kIn = 1; static constexpr bool kTables = true; static constexpr bool kRare = true;
+    __device__ float operator()(const float* x, const Tables&) const { return cta_sincosf_fast(x[0], 1); }
+    __device__ bool rare(const float* x) const { return cta_sincos_is_rare(x[0]); }
+    __device__ float slow(const float* x, const Tables& t) const { return cta_sincosf(x[0], 1, t.inv_pio4); } };
 
 __device__ __forceinline__ float tanh_ref(float x, const Tables& t) {
-    float ep = cta_expf_tab(x, t.exp2);
-    float en = cta_expf_tab(-x, t.exp2);
+    float ep, en;
+    cta_expf_pair(x, t.exp2, &ep, &en);
     return (ep - en) / (ep + en);
 }
 __device__ __forceinline__ float sigmoid_ref(float x, const Tables& t) {
@@ -93,26 +108,28 @@ struct TanhBwdF { static constexpr int kIn = 2; static constexpr bool kTables = 
         float tt = th * th;
         float om = 1.0f - tt;
         return om * x[1]; } };
-struct SinBwdF { static constexpr int kIn = 2; static constexpr bool kTables = true;
-    __device__ float operator()(const float* x, const Tables& t) const {
-        return cta_sincosf(x[0], 1, t.inv_pio4) * x[1]; } };
-struct CosBwdF { static constexpr int kIn = 2; static constexpr bool kTables = true;
-    __device__ float operator()(const float* x, const Tables& t) const {
-        return (-cta_sincosf(x[0], 0, t.inv_pio4)) * x[1]; } };
-// inputs (p, t); fn = float(n); g a 0-D device tensor
+struct SinBwdF { static constexpr int kIn = 2; static constexpr bool kTables = true; static constexpr bool kRare = true;
+    __device__ float operator()(const float* x, const Tables&) const { return cta_sincosf_fast(x[0], 1) * x[1]; }
+    __device__ bool rare(const float* x) const { return cta_sincos_is_rare(x[0]); }
+    __device__ float slow(const float* x, const Tables& t) const { return cta_sincosf(x[0], 1, t.inv_pio4) * x[1]; } };
+struct CosBwdF { static constexpr int kIn = 2; static constexpr bool kTables = true; static constexpr bool kRare = true;
+    __device__ float operator()(const float* x, const Tables&) const { return (-cta_sincosf_fast(x[0], 0)) * x[1]; }
+    __device__ bool rare(const float* x) const { return cta_sincos_is_rare(x[0]); }
+    __device__ float slow(const float* x, const Tables& t) const { return (-cta_sincosf(x[0], 0, t.inv_pio4)) * x[1]; } };
+// inputs (p, t); rfn = 1.0 / double(float(n)); g a 0-D device tensor
 struct MseBwdF { static constexpr int kIn = 2; static constexpr bool kTables = false;
-    float fn; const float* g;
+    double rfn; const float* g;
     __device__ float operator()(const float* x, const Tables&) const {
         float d = x[0] - x[1];
         float d2 = d * 2.0f;
-        float q = d2 / fn;
+        float q = cta_div_rcp(d2, rfn);          // d2 / float(n)
         return q * *g; } };
 struct MaeBwdF { static constexpr int kIn = 2; static constexpr bool kTables = false;
-    float fn; const float* g;
+    double rfn; const float* g;
     __device__ float operator()(const float* x, const Tables&) const {
         float d = x[0] - x[1];
         float s = (d > 0.0f) ? 1.0f : ((d < 0.0f) ? -1.0f : 0.0f);
-        float q = s / fn;
+        float q = cta_div_rcp(s, rfn);           // sign / float(n)
         return q * *g; } };
 // inputs (a, b, g): ((-a) * g) / (b * b)
 struct DivBwdBF { static constexpr int kIn = 3; static constexpr bool kTables = false;
@@ -129,6 +146,29 @@ struct FillFromF { static constexpr int kIn = 0; static constexpr bool kTables =
     __device__ float operator()(const float*, const Tables&) const { return *v; } };
 
 // -------------------------------------------------------------------------------- kernels
+
+// A functor may turn itself into a cheaper one once per thread before the element loop
+// (DevScalarF<DivF> reads its divisor and becomes DivByRcpF).
+template <class F>
+__device__ __forceinline__ F bind(const F& f) { return f; }
+__device__ __forceinline__ DivByRcpF bind(const DevScalarF<DivF>& f) { return DivByRcpF{1.0 / double(*f.s)}; }
+
+template <class F, class = void>
+struct HasRare { static constexpr bool value = false; };
+template <class F>
+struct HasRare<F, decltype(void(F::kRare))> { static constexpr bool value = F::kRare; };
+
+// One element: the functor's fast path, repaired through slow() when the functor flags the input.
+template <class F, int NI>
+__device__ __forceinline__ float apply1(const F& f, const float* x, const Tables& tabs) {
+    if constexpr (HasRare<F>::value) {
+        float o = f(x, tabs);
+        if (__builtin_expect(f.rare(x), 0)) o = f.slow(x, tabs);
+        return o;
+    } else {
+        return f(x, tabs);
+    }
+}
 
 __device__ __forceinline__ void stage_tables(uint64_t* exp2, uint32_t* pio4) {
     if (threadIdx.x < 32) exp2[threadIdx.x] = cta_exp2_tab[threadIdx.x];
@@ -155,51 +195,76 @@ __device__ __forceinline__ void st_stream(float* p, size_t i4, v4f v) {
 // operands + result above this many bytes cannot stay cache resident (256 MiB Infinity Cache)
 constexpr size_t kStreamBytes = size_t(64) << 20;
 
+// The work of one thread of a vector block: its kUnroll vectors per operand, all loaded before the
+// first use.  CHECK guards each vector against the end of the tensor (last block only).
+template <class F, bool NT, bool CHECK>
+__device__ __forceinline__ void map_block(const Ptrs<F::kIn>& in, float* __restrict__ out, size_t n4, size_t base,
+                                          const F& f, const Tables& tabs) {
+    constexpr int NI = F::kIn;
+    v4f v[NI > 0 ? NI : 1][kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        size_t i = base + size_t(u) * kThreads;
+        if (!CHECK || i < n4) {
+#pragma unroll
+            for (int k = 0; k < NI; ++k) v[k][u] = ld_stream<NT>(in.p[k], i);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        size_t i = base + size_t(u) * kThreads;
+        if (!CHECK || i < n4) {
+            v4f o;
+            bool rare = false;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float x[NI > 0 ? NI : 1];
+#pragma unroll
+                for (int k = 0; k < NI; ++k) x[k] = v[k][u][e];
+                o[e] = f(x, tabs);
+                if constexpr (HasRare<F>::value) rare = rare || f.rare(x);
+            }
+            if constexpr (HasRare<F>::value) {
+                if (__builtin_expect(rare, 0)) {
+                    for (int e = 0; e < 4; ++e) {
+                        float x[NI > 0 ? NI : 1];
+                        for (int k = 0; k < NI; ++k) x[k] = v[k][u][e];
+                        if (f.rare(x)) o[e] = f.slow(x, tabs);
+                    }
+                }
+            }
+            st_stream<NT>(out, i, o);
+        }
+    }
+}
+
 // VEC = true: all pointers 16-byte aligned.  Block b owns the kThreads*kUnroll consecutive
 // vectors starting at b*kThreads*kUnroll (no loop: the grid covers the tensor), thread t takes
 // vectors t, t+256, t+512, t+768 of that run, all loads issued before the first use.  The last
 // n % 4 elements are handled by block 0.  VEC = false: scalar grid-stride (unaligned views).
 template <class F, bool VEC, bool NT>
-__global__ __launch_bounds__(kThreads) void map_kernel(Ptrs<F::kIn> in, float* __restrict__ out, size_t n, F f) {
+__global__ __launch_bounds__(kThreads) void map_kernel(Ptrs<F::kIn> in, float* __restrict__ out, size_t n, F f_in) {
     __shared__ uint64_t s_exp2[F::kTables ? 32 : 1];
     __shared__ uint32_t s_pio4[F::kTables ? 24 : 1];
     if (F::kTables) stage_tables(s_exp2, s_pio4);
     const Tables tabs{s_exp2, s_pio4};
     constexpr int NI = F::kIn;
+    const auto f = bind(f_in);
+    using B = decltype(bind(f_in));
     if (VEC) {
         const size_t n4 = n >> 2;
-        const size_t base = size_t(blockIdx.x) * (kThreads * kUnroll) + threadIdx.x;
-        v4f v[NI > 0 ? NI : 1][kUnroll];
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            size_t i = base + size_t(u) * kThreads;
-            if (i < n4) {
-#pragma unroll
-                for (int k = 0; k < NI; ++k) v[k][u] = ld_stream<NT>(in.p[k], i);
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            size_t i = base + size_t(u) * kThreads;
-            if (i < n4) {
-                v4f o;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float x[NI > 0 ? NI : 1];
-#pragma unroll
-                    for (int k = 0; k < NI; ++k) x[k] = v[k][u][e];
-                    o[e] = f(x, tabs);
-                }
-                st_stream<NT>(out, i, o);
-            }
-        }
+        const size_t block_base = size_t(blockIdx.x) * (kThreads * kUnroll);
+        if (block_base + size_t(kThreads) * kUnroll <= n4)
+            map_block<B, NT, false>(in, out, n4, block_base + threadIdx.x, f, tabs);   // interior block: no bounds checks
+        else
+            map_block<B, NT, true>(in, out, n4, block_base + threadIdx.x, f, tabs);
         if (blockIdx.x == 0) {
             size_t i = (n4 << 2) + threadIdx.x;
             if (i < n) {
                 float x[NI > 0 ? NI : 1];
 #pragma unroll
                 for (int k = 0; k < NI; ++k) x[k] = in.p[k][i];
-                out[i] = f(x, tabs);
+                out[i] = apply1<B, NI>(f, x, tabs);
             }
         }
     } else {
@@ -209,7 +274,7 @@ __global__ __launch_bounds__(kThreads) void map_kernel(Ptrs<F::kIn> in, float* _
             float x[NI > 0 ? NI : 1];
 #pragma unroll
             for (int k = 0; k < NI; ++k) x[k] = in.p[k][i];
-            out[i] = f(x, tabs);
+            out[i] = apply1<B, NI>(f, x, tabs);
         }
     }
 }
@@ -366,7 +431,10 @@ int ctamd_rsub_ascalar_f32(const float* a1, const float* b, float* r, size_t n, 
 
 int ctamd_add_scalar_f32(const float* a, float v, float* r, size_t n, void* s) { return host_scalar<AddF>(__func__, a, v, r, n, s); }
 int ctamd_mul_scalar_f32(const float* a, float v, float* r, size_t n, void* s) { return host_scalar<MulF>(__func__, a, v, r, n, s); }
-int ctamd_div_scalar_f32(const float* a, float v, float* r, size_t n, void* s) { return host_scalar<DivF>(__func__, a, v, r, n, s); }
+int ctamd_div_scalar_f32(const float* a, float v, float* r, size_t n, void* s) {
+    Ptrs<1> in{{a}};
+    return launch_map<DivByRcpF>(__func__, in, r, n, DivByRcpF{1.0 / double(v)}, s);
+}
 
 int ctamd_neg_f32(const float* a, float* r, size_t n, void* s) { return unary<NegF>(__func__, a, r, n, s); }
 int ctamd_relu_f32(const float* a, float* r, size_t n, void* s) { return unary<ReluF>(__func__, a, r, n, s); }
@@ -395,12 +463,12 @@ int ctamd_cos_backward_f32(const float* x, const float* g, float* dx, size_t n, 
 int ctamd_mse_backward_f32(const float* p, const float* t, const float* g1, float* dp, size_t n, void* s) {
     if (n && !g1) return fail(CTAMD_EINVAL, "%s: null upstream gradient", __func__);
     Ptrs<2> in{{p, t}};
-    return launch_map<MseBwdF>(__func__, in, dp, n, MseBwdF{float(n), g1}, s);
+    return launch_map<MseBwdF>(__func__, in, dp, n, MseBwdF{1.0 / double(float(n)), g1}, s);
 }
 int ctamd_mae_backward_f32(const float* p, const float* t, const float* g1, float* dp, size_t n, void* s) {
     if (n && !g1) return fail(CTAMD_EINVAL, "%s: null upstream gradient", __func__);
     Ptrs<2> in{{p, t}};
-    return launch_map<MaeBwdF>(__func__, in, dp, n, MaeBwdF{float(n), g1}, s);
+    return launch_map<MaeBwdF>(__func__, in, dp, n, MaeBwdF{1.0 / double(float(n)), g1}, s);
 }
 int ctamd_div_backward_b_f32(const float* a, const float* b, const float* g, float* db, size_t n, void* s) {
     Ptrs<3> in{{a, b, g}};

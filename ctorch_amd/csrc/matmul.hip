@@ -9,9 +9,9 @@
 // Within an 8-wide k chunk, lane half h (lane / 32) owns k = 4h .. 4h+3 for both operands - the
 // sum over k is order-free, so the MFMA's (lane / 32) k index is simply re-labelled; that lets
 // the K-contiguous kind fetch four consecutive k with a single load.
-// One 256-thread block (4 waves, 2 x 2) computes a BM x BN tile of C; global -> register ->
-// LDS staging is double buffered so the loads of tile t+1 are in flight while tile t is
-// multiplied, with one barrier per k tile.  Blocks are renumbered so that each XCD (blocks are
+// One block (8 waves for the 256 x 256 tile, 4 for the 128 x 128 one) computes a BM x BN tile of C;
+// global -> register -> LDS staging is double buffered so the loads of tile t+1 are in flight while
+// tile t is multiplied, with one barrier per k tile.  Blocks are renumbered so that each XCD (blocks are
 // dealt round-robin to the 8 XCDs) works on a compact band of C and re-uses its operand tiles
 // from its own L2.  Skinny outputs with a long K (the weight gradients of a small layer) are
 // split along K over blockIdx.z; partial products go to the device scratch and are folded in a
@@ -27,12 +27,16 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 constexpr int kThreads = 256;
 constexpr int kXcds = 8;
 
+constexpr int kMinWavesPerSimd = 2;   // register budget of both tile shapes: 256 VGPRs per lane
+
+
 template <int BM_, int BN_, int BK_, int WM_, int WN_>
 struct Cfg {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
     static constexpr int TM = WM / 32, TN = WN / 32;       // MFMA tiles per wave
     static constexpr int WAVES_N = BN / WN;
-    static_assert((BM / WM) * (BN / WN) == kThreads / 64, "wave grid must use 4 waves");
+    static constexpr int THREADS = (BM / WM) * (BN / WN) * 64;
+    static_assert(THREADS == 256 || THREADS == 512, "4 or 8 waves per block");
     static_assert(BK % 8 == 0, "k tile is a multiple of the 8-wide chunk");
     static constexpr int KPAD = BK + 4;                    // K-contiguous row stride (floats)
     static constexpr int XPAD_M = BM + 8, XPAD_N = BN + 8; // X-contiguous row strides
@@ -46,11 +50,32 @@ constexpr int tile_floats() {
 
 // Global -> registers for one operand tile.  ROWS x BK (K-contiguous) or BK x ROWS
 // (X-contiguous), as 128-bit pieces dealt to the 256 threads.
-template <int ROWS, int BK, bool KC>
+template <int ROWS, int BK, bool KC, int THREADS>
 struct Stage {
-    static constexpr int PIECES = ROWS * BK / 4 / kThreads;
-    static_assert(ROWS * BK / 4 % kThreads == 0, "tile must split evenly over the block");
+    static constexpr int PIECES = ROWS * BK / 4 / THREADS;
+    static_assert(ROWS * BK / 4 % THREADS == 0, "tile must split evenly over the block");
     v4f r[PIECES];
+    const float* src[PIECES];   // interior tiles: where this thread's next pieces come from
+
+    // Interior tiles (whole tile inside the matrix, aligned rows): no bounds logic in the loop, one
+    // pointer per piece advanced by a constant each k tile.
+    __device__ __forceinline__ void init_fast(const float* __restrict__ p, int64_t ld, int x0, int k0) {
+#pragma unroll
+        for (int q = 0; q < PIECES; ++q) {
+            int idx = threadIdx.x + q * THREADS;
+            int outer, inner;
+            if (KC) { outer = idx / (BK / 4); inner = (idx % (BK / 4)) * 4; }
+            else { outer = idx / (ROWS / 4); inner = (idx % (ROWS / 4)) * 4; }
+            src[q] = KC ? p + int64_t(x0 + outer) * ld + (k0 + inner) : p + int64_t(k0 + outer) * ld + (x0 + inner);
+        }
+    }
+    __device__ __forceinline__ void load_fast(int64_t step) {
+#pragma unroll
+        for (int q = 0; q < PIECES; ++q) {
+            r[q] = *reinterpret_cast<const v4f*>(src[q]);
+            src[q] += step;
+        }
+    }
 
     // x0: first row/col of the tile in the X dimension, k0: first k; dimX, K: extents; ld: leading
     // dimension (elements) of the contiguous direction's rows.  VEC: 16-byte aligned rows.
@@ -58,7 +83,7 @@ struct Stage {
     __device__ __forceinline__ void load(const float* __restrict__ p, int64_t ld, int x0, int k0, int dimX, int k_end) {
 #pragma unroll
         for (int q = 0; q < PIECES; ++q) {
-            int idx = threadIdx.x + q * kThreads;
+            int idx = threadIdx.x + q * THREADS;
             int outer, inner;   // outer indexes rows of the contiguous direction
             if (KC) { outer = idx / (BK / 4); inner = (idx % (BK / 4)) * 4; }
             else { outer = idx / (ROWS / 4); inner = (idx % (ROWS / 4)) * 4; }
@@ -83,7 +108,7 @@ struct Stage {
     __device__ __forceinline__ void store(float* __restrict__ lds, int stride) const {
 #pragma unroll
         for (int q = 0; q < PIECES; ++q) {
-            int idx = threadIdx.x + q * kThreads;
+            int idx = threadIdx.x + q * THREADS;
             int outer, inner;
             if (KC) { outer = idx / (BK / 4); inner = (idx % (BK / 4)) * 4; }
             else { outer = idx / (ROWS / 4); inner = (idx % (ROWS / 4)) * 4; }
@@ -117,7 +142,7 @@ struct GemmArgs {
 };
 
 template <class C, bool A_KC, bool B_KC, bool VEC>
-__global__ __launch_bounds__(kThreads, 2) void gemm_kernel(GemmArgs g) {
+__global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(GemmArgs g) {
     constexpr int BM = C::BM, BN = C::BN, BK = C::BK, TM = C::TM, TN = C::TN;
     constexpr int A_STRIDE = A_KC ? C::KPAD : C::XPAD_M;
     constexpr int B_STRIDE = B_KC ? C::KPAD : C::XPAD_N;
@@ -162,40 +187,62 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_kernel(GemmArgs g) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    Stage<BM, BK, A_KC> sa;
-    Stage<BN, BK, B_KC> sb;
+    Stage<BM, BK, A_KC, C::THREADS> sa;
+    Stage<BN, BK, B_KC, C::THREADS> sb;
     const int ktiles = (k_end - k_begin + BK - 1) / BK;
+    // interior: the whole BM x BN tile and every k tile lie inside the operands and rows are
+    // 16-byte aligned - true for all blocks of a 4096^3 product, false only on ragged edges
+    const bool interior = VEC && m0 + BM <= g.m && n0 + BN <= g.n && (k_end - k_begin) % BK == 0;
+    const int64_t a_step = A_KC ? BK : int64_t(BK) * g.lda;
+    const int64_t b_step = B_KC ? BK : int64_t(BK) * g.ldb;
+    if (interior) {
+        sa.init_fast(g.a, g.lda, m0, k_begin);
+        sb.init_fast(g.b, g.ldb, n0, k_begin);
+    }
+    auto stage_tile = [&](int t) {
+        if (interior) {
+            sa.load_fast(a_step);
+            sb.load_fast(b_step);
+        } else {
+            sa.template load<VEC>(g.a, g.lda, m0, k_begin + t * BK, g.m, k_end);
+            sb.template load<VEC>(g.b, g.ldb, n0, k_begin + t * BK, g.n, k_end);
+        }
+    };
     if (ktiles > 0) {
-        sa.template load<VEC>(g.a, g.lda, m0, k_begin, g.m, k_end);
-        sb.template load<VEC>(g.b, g.ldb, n0, k_begin, g.n, k_end);
+        stage_tile(0);
         sa.store(s_a[0], A_STRIDE);
         sb.store(s_b[0], B_STRIDE);
     }
     __syncthreads();
     for (int t = 0; t < ktiles; ++t) {
         const int cur = t & 1;
-        if (t + 1 < ktiles) {
-            sa.template load<VEC>(g.a, g.lda, m0, k_begin + (t + 1) * BK, g.m, k_end);
-            sb.template load<VEC>(g.b, g.ldb, n0, k_begin + (t + 1) * BK, g.n, k_end);
-        }
         const float* __restrict__ la = s_a[cur];
         const float* __restrict__ lb = s_b[cur];
+        // 1. every fragment of this k tile into registers, 2. the next tile's global loads,
+        // 3. all MFMAs back to back.  The scheduling fences keep that order: interleaving a
+        // fragment load and its wait into each group of four MFMAs (what the scheduler does when
+        // left alone, to save registers) left the matrix pipe idle about a fifth of the time.
+        float fa[BK / 8][TM][4], fb[BK / 8][TN][4];
 #pragma unroll
         for (int ch = 0; ch < BK / 8; ++ch) {
-            float fa[TM][4], fb[TN][4];
             const int kb = ch * 8 + half * 4;
 #pragma unroll
-            for (int i = 0; i < TM; ++i) fetch<A_KC>(la, A_STRIDE, wm + i * 32 + l32, kb, fa[i]);
+            for (int i = 0; i < TM; ++i) fetch<A_KC>(la, A_STRIDE, wm + i * 32 + l32, kb, fa[ch][i]);
 #pragma unroll
-            for (int j = 0; j < TN; ++j) fetch<B_KC>(lb, B_STRIDE, wn + j * 32 + l32, kb, fb[j]);
+            for (int j = 0; j < TN; ++j) fetch<B_KC>(lb, B_STRIDE, wn + j * 32 + l32, kb, fb[ch][j]);
+        }
+        if (t + 1 < ktiles) stage_tile(t + 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ch = 0; ch < BK / 8; ++ch)
 #pragma unroll
             for (int s = 0; s < 4; ++s)
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
 #pragma unroll
                     for (int j = 0; j < TN; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
-        }
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[ch][i][s], fb[ch][j][s], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
         if (t + 1 < ktiles) {
             sa.store(s_a[cur ^ 1], A_STRIDE);
             sb.store(s_b[cur ^ 1], B_STRIDE);
@@ -240,14 +287,27 @@ __global__ __launch_bounds__(kThreads) void gemm_strided(const float* __restrict
     c[idx] = s;
 }
 
-using Tile = Cfg<128, 128, 16, 64, 64>;
+// Two tile shapes.  Big: 256 x 256 x 16 with 8 waves (each 128 x 64, 128 accumulator registers, two
+// waves per SIMD) - the fewest LDS and global bytes per flop, 134-137 TFLOP/s at 4096^3 against
+// 122-124 for the small tile; it needs about one tile per CU to fill the chip.  Small:
+// 128 x 128 x 16 with 4 waves (each 64 x 64) for everything else (113 against 109 TFLOP/s at 2048^3).
+using BigTile = Cfg<256, 256, 16, 128, 64>;
+using SmallTile = Cfg<128, 128, 16, 64, 64>;
 
-template <bool A_KC, bool B_KC>
+template <class Tile, bool A_KC, bool B_KC>
 int launch_gemm(GemmArgs g, bool vec, int splits, hipStream_t s) {
     dim3 grid(unsigned(g.tiles_m * g.tiles_n), 1, unsigned(splits));
-    if (vec) hipLaunchKernelGGL((gemm_kernel<Tile, A_KC, B_KC, true>), grid, dim3(kThreads), 0, s, g);
-    else hipLaunchKernelGGL((gemm_kernel<Tile, A_KC, B_KC, false>), grid, dim3(kThreads), 0, s, g);
+    if (vec) hipLaunchKernelGGL((gemm_kernel<Tile, A_KC, B_KC, true>), grid, dim3(Tile::THREADS), 0, s, g);
+    else hipLaunchKernelGGL((gemm_kernel<Tile, A_KC, B_KC, false>), grid, dim3(Tile::THREADS), 0, s, g);
     return launched("ctamd_matmul_f32");
+}
+
+template <class Tile>
+int launch_layout(GemmArgs g, bool a_kc, bool b_kc, bool vec, int splits, hipStream_t s) {
+    if (a_kc && b_kc) return launch_gemm<Tile, true, true>(g, vec, splits, s);
+    if (a_kc) return launch_gemm<Tile, true, false>(g, vec, splits, s);
+    if (b_kc) return launch_gemm<Tile, false, true>(g, vec, splits, s);
+    return launch_gemm<Tile, false, false>(g, vec, splits, s);
 }
 
 }  // namespace
@@ -276,22 +336,27 @@ extern "C" int ctamd_matmul_f32(const float* a, int64_t as0, int64_t as1, const 
         return launched(__func__);
     }
     const bool A_KC = a_kc, B_KC = !b_xc;
+    const int cus = compute_units() > 0 ? compute_units() : 256;
+    const int64_t big_tiles = ((m + BigTile::BM - 1) / BigTile::BM) * ((n + BigTile::BN - 1) / BigTile::BN);
+    const bool big = big_tiles >= cus;
+    const int BM = big ? BigTile::BM : SmallTile::BM, BN = big ? BigTile::BN : SmallTile::BN;
+    constexpr int BK = SmallTile::BK;
+    static_assert(BigTile::BK == SmallTile::BK, "both tile shapes step K alike");
     GemmArgs g;
     g.a = a; g.lda = A_KC ? as0 : as1;
     g.b = b; g.ldb = B_KC ? bs1 : bs0;
     g.m = int(m); g.n = int(n); g.k = int(k);
-    g.tiles_m = int((m + Tile::BM - 1) / Tile::BM);
-    g.tiles_n = int((n + Tile::BN - 1) / Tile::BN);
+    g.tiles_m = int((m + BM - 1) / BM);
+    g.tiles_n = int((n + BN - 1) / BN);
     const bool vec = aligned16(a) && aligned16(b) && (g.lda % 4 == 0) && (g.ldb % 4 == 0);
 
     // split along K when the output has too few tiles to fill the chip and K is long
     int splits = 1;
     const int64_t tiles = int64_t(g.tiles_m) * g.tiles_n;
-    const int cus = compute_units() > 0 ? compute_units() : 256;
     float* partial = nullptr;
-    if (tiles < cus && k >= 8 * Tile::BK) {
+    if (tiles < cus && k >= 8 * BK) {
         int64_t want = (2 * cus + tiles - 1) / tiles;
-        int64_t max_by_k = k / (4 * Tile::BK);
+        int64_t max_by_k = k / (4 * BK);
         int64_t max_by_scratch = int64_t(kScratchFloats) / (m * n);
         splits = int(want < max_by_k ? want : max_by_k);
         if (splits > max_by_scratch) splits = int(max_by_scratch);
@@ -303,17 +368,14 @@ extern "C" int ctamd_matmul_f32(const float* a, int64_t as0, int64_t as1, const 
         }
     }
     int kps = int((k + splits - 1) / splits);
-    kps = (kps + Tile::BK - 1) / Tile::BK * Tile::BK;
+    kps = (kps + BK - 1) / BK * BK;
     splits = int((k + kps - 1) / kps);
     g.k_per_split = kps;
     if (splits > 1) { g.c = partial; g.ldc = n; g.split_stride = m * n; }
     else { g.c = c; g.ldc = n; g.split_stride = 0; }
 
-    int rc;
-    if (A_KC && B_KC) rc = launch_gemm<true, true>(g, vec, splits, s);
-    else if (A_KC) rc = launch_gemm<true, false>(g, vec, splits, s);
-    else if (B_KC) rc = launch_gemm<false, true>(g, vec, splits, s);
-    else rc = launch_gemm<false, false>(g, vec, splits, s);
+    int rc = big ? launch_layout<BigTile>(g, A_KC, B_KC, vec, splits, s)
+                 : launch_layout<SmallTile>(g, A_KC, B_KC, vec, splits, s);
     if (rc || splits == 1) return rc;
     size_t mn = size_t(m) * size_t(n);
     hipLaunchKernelGGL(splitk_fold, dim3(unsigned((mn + kThreads - 1) / kThreads)), dim3(kThreads), 0, s, partial, c, mn,

@@ -137,72 +137,103 @@ int reduce(const char* name, const float* a, const float* b, float* out, int32_t
 }
 
 // ----------------------------------------------------------------------------- column sum
-// Block = 64 column groups x 4 row lanes.  Each block folds a chunk of rows for its columns and
-// writes one partial row; stage 2 adds the partial rows in double.
-constexpr int kColLanes = 64;
-constexpr int kRowLanes = 4;
-
-template <bool VEC>
+// A block owns a strip of 256 * CU vectors of columns (CU = 4: up to 4096 columns, 16 KiB per row;
+// CU = 1 when that would leave the chip short of blocks) and a chunk of rows, and walks its rows in
+// order, two rows in flight per thread.  Each block writes one partial row per strip; stage 2 adds
+// the (at most 256) partial rows in double, four lanes per column with eight loads in flight each -
+// a serial walk over the partial rows by one thread per column cost more than stage 1 itself.
+template <bool VEC, int CU>
 __global__ __launch_bounds__(kThreads) void colsum_stage1(const float* __restrict__ g, float* __restrict__ partials,
                                                           size_t rows, size_t cols, size_t rows_per_block) {
     constexpr int W = VEC ? 4 : 1;
-    const int tx = threadIdx.x % kColLanes, ty = threadIdx.x / kColLanes;
-    const size_t col = (size_t(blockIdx.x) * kColLanes + tx) * W;
+    const size_t strip0 = size_t(blockIdx.x) * (size_t(kThreads) * CU * W);
     const size_t r0 = size_t(blockIdx.y) * rows_per_block;
     size_t r1 = r0 + rows_per_block;
     if (r1 > rows) r1 = rows;
-    constexpr int U = 8;    // independent row loads in flight per thread
-    float acc[2][4] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
-    if (col < cols) {
-        size_t r = r0 + ty;
-        for (; r + size_t(U - 1) * kRowLanes < r1; r += size_t(U) * kRowLanes) {
-            if (VEC) {
-                v4f x[U];
+    float acc[2][CU][4];
 #pragma unroll
-                for (int u = 0; u < U; ++u)
-                    x[u] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(g + (r + size_t(u) * kRowLanes) * cols + col));
+    for (int p = 0; p < 2; ++p)
 #pragma unroll
-                for (int u = 0; u < U; ++u)
+        for (int u = 0; u < CU; ++u)
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) acc[u & 1][e] += x[u][e];
-            } else {
-                float x[U];
+            for (int e = 0; e < 4; ++e) acc[p][u][e] = 0.0f;
+    size_t col[CU];
+    bool live[CU];
 #pragma unroll
-                for (int u = 0; u < U; ++u) x[u] = g[(r + size_t(u) * kRowLanes) * cols + col];
-#pragma unroll
-                for (int u = 0; u < U; ++u) acc[u & 1][0] += x[u];
-            }
-        }
-        for (; r < r1; r += kRowLanes) {
-            if (VEC) {
-                v4f x0 = *reinterpret_cast<const v4f*>(g + r * cols + col);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) acc[0][e] += x0[e];
-            } else {
-                acc[0][0] += g[r * cols + col];
-            }
-        }
+    for (int u = 0; u < CU; ++u) {
+        col[u] = strip0 + (size_t(u) * kThreads + threadIdx.x) * W;
+        live[u] = col[u] < cols;
     }
-    __shared__ float s_acc[kRowLanes][kColLanes][4];
+    size_t r = r0;
+    for (; r + 1 < r1; r += 2) {
+        v4f x[2][CU];
 #pragma unroll
-    for (int e = 0; e < W; ++e) s_acc[ty][tx][e] = acc[0][e] + acc[1][e];
-    __syncthreads();
-    if (ty == 0 && col < cols) {
+        for (int p = 0; p < 2; ++p)
 #pragma unroll
-        for (int e = 0; e < W; ++e) {
-            float t = (s_acc[0][tx][e] + s_acc[1][tx][e]) + (s_acc[2][tx][e] + s_acc[3][tx][e]);
-            partials[size_t(blockIdx.y) * cols + col + e] = t;
-        }
+            for (int u = 0; u < CU; ++u)
+                if (live[u]) {
+                    const float* src = g + (r + p) * cols + col[u];
+                    if (VEC) x[p][u] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(src));
+                    else x[p][u][0] = *src;
+                }
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+#pragma unroll
+            for (int u = 0; u < CU; ++u)
+                if (live[u]) {
+#pragma unroll
+                    for (int e = 0; e < W; ++e) acc[p][u][e] += x[p][u][e];
+                }
     }
+    if (r < r1) {
+#pragma unroll
+        for (int u = 0; u < CU; ++u)
+            if (live[u]) {
+                const float* src = g + r * cols + col[u];
+                if (VEC) {
+                    v4f x0 = *reinterpret_cast<const v4f*>(src);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[0][u][e] += x0[e];
+                } else {
+                    acc[0][u][0] += *src;
+                }
+            }
+    }
+#pragma unroll
+    for (int u = 0; u < CU; ++u)
+        if (live[u]) {
+#pragma unroll
+            for (int e = 0; e < W; ++e) partials[size_t(blockIdx.y) * cols + col[u] + e] = acc[0][u][e] + acc[1][u][e];
+        }
 }
 
+constexpr int kFoldLanes = 4;   // lanes per column in stage 2
 __global__ __launch_bounds__(kThreads) void colsum_stage2(const float* __restrict__ partials, float* __restrict__ out,
                                                           size_t cols, unsigned chunks) {
-    size_t c = size_t(blockIdx.x) * kThreads + threadIdx.x;
-    if (c >= cols) return;
-    double t = 0.0;
-    for (unsigned k = 0; k < chunks; ++k) t += double(partials[size_t(k) * cols + c]);
-    out[c] = float(t);
+    constexpr int TX = kThreads / kFoldLanes;
+    const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+    const size_t c = size_t(blockIdx.x) * TX + tx;
+    double acc = 0.0;
+    if (c < cols) {
+        unsigned k = ty;
+        for (; k + 7 * kFoldLanes < chunks; k += 8 * kFoldLanes) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = partials[size_t(k + u * kFoldLanes) * cols + c];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc += double(v[u]);
+        }
+        for (; k < chunks; k += kFoldLanes) acc += double(partials[size_t(k) * cols + c]);
+    }
+    __shared__ double s_acc[kFoldLanes][TX];
+    s_acc[ty][tx] = acc;
+    __syncthreads();
+    if (ty == 0 && c < cols) {
+        double t = 0.0;
+#pragma unroll
+        for (int y = 0; y < kFoldLanes; ++y) t += s_acc[y][tx];
+        out[c] = float(t);
+    }
 }
 
 }  // namespace
@@ -230,27 +261,34 @@ int ctamd_colsum_f32(const float* g, float* out, size_t rows, size_t cols, void*
     if (!partials) return CTAMD_EINVAL;
     if (cols > kScratchFloats) return fail(CTAMD_ERANGE, "%s: more than %zu columns", __func__, kScratchFloats);
     bool vec = (cols % 4 == 0) && aligned16(g);
-    size_t col_blocks = (cols + size_t(kColLanes) * (vec ? 4 : 1) - 1) / (size_t(kColLanes) * (vec ? 4 : 1));
-    // row chunks: fill the chip (about 8 blocks per CU), at least 32 rows per block, and the
-    // partial rows must fit the scratch
-    size_t want = (size_t(compute_units() > 0 ? compute_units() : 256) * 8 + col_blocks - 1) / col_blocks;
-    size_t chunks = (rows + 63) / 64;
-    if (chunks > want) chunks = want;
+    const size_t w = vec ? 4 : 1;
+    const size_t cus = size_t(compute_units() > 0 ? compute_units() : 256);
+    // at most 256 row chunks of at least 32 rows; wide strips unless that leaves the chip short of blocks
+    size_t chunks = (rows + 31) / 32;
+    if (chunks > 256) chunks = 256;
     if (chunks > kScratchFloats / cols) chunks = kScratchFloats / cols;
-    if (chunks > 65535) chunks = 65535;
     if (chunks < 1) chunks = 1;
     size_t rows_per_block = (rows + chunks - 1) / chunks;
     chunks = (rows + rows_per_block - 1) / rows_per_block;
+    const size_t wide_strips = (cols + size_t(kThreads) * 4 * w - 1) / (size_t(kThreads) * 4 * w);
+    const bool wide = wide_strips * chunks >= 4 * cus;
+    const size_t strip = size_t(kThreads) * (wide ? 4 : 1) * w;
+    size_t col_blocks = (cols + strip - 1) / strip;
     hipStream_t s = as_stream(stream);
-    dim3 grid((unsigned)col_blocks, (unsigned)chunks);
     if (col_blocks > 0x7fffffffu) return fail(CTAMD_ERANGE, "%s: too many columns", __func__);
-    if (vec)
-        hipLaunchKernelGGL((colsum_stage1<true>), grid, dim3(kThreads), 0, s, g, partials, rows, cols, rows_per_block);
+    dim3 grid((unsigned)col_blocks, (unsigned)chunks);
+    if (vec && wide)
+        hipLaunchKernelGGL((colsum_stage1<true, 4>), grid, dim3(kThreads), 0, s, g, partials, rows, cols, rows_per_block);
+    else if (vec)
+        hipLaunchKernelGGL((colsum_stage1<true, 1>), grid, dim3(kThreads), 0, s, g, partials, rows, cols, rows_per_block);
+    else if (wide)
+        hipLaunchKernelGGL((colsum_stage1<false, 4>), grid, dim3(kThreads), 0, s, g, partials, rows, cols, rows_per_block);
     else
-        hipLaunchKernelGGL((colsum_stage1<false>), grid, dim3(kThreads), 0, s, g, partials, rows, cols, rows_per_block);
+        hipLaunchKernelGGL((colsum_stage1<false, 1>), grid, dim3(kThreads), 0, s, g, partials, rows, cols, rows_per_block);
     int rc = launched(__func__);
     if (rc) return rc;
-    hipLaunchKernelGGL(colsum_stage2, dim3((unsigned)((cols + kThreads - 1) / kThreads)), dim3(kThreads), 0, s, partials,
+    constexpr size_t kFoldCols = kThreads / kFoldLanes;
+    hipLaunchKernelGGL(colsum_stage2, dim3((unsigned)((cols + kFoldCols - 1) / kFoldCols)), dim3(kThreads), 0, s, partials,
                        out, cols, (unsigned)chunks);
     return launched(__func__);
 }

@@ -38,6 +38,15 @@ static int current_device() {
     return d;
 }
 
+const float* pad_neg_inf() {
+    float* s = scratch();
+    return s ? s + kScratchFloats : nullptr;
+}
+const float* pad_zero() {
+    float* s = scratch();
+    return s ? s + kScratchFloats + 4 : nullptr;
+}
+
 float* scratch() {
     int d = current_device();
     if (d < 0 || d >= kMaxDevices || g_scratch[d] == nullptr) {
@@ -83,8 +92,16 @@ int ctamd_init(int device) {
                     prop.gcnArchName);
     g_cus[device] = prop.multiProcessorCount;
     void* p = nullptr;
-    rc = check_hip(hipMalloc(&p, kScratchFloats * sizeof(float)), "hipMalloc(scratch)");
+    rc = check_hip(hipMalloc(&p, (kScratchFloats + 8) * sizeof(float)), "hipMalloc(scratch)");
     if (rc) return rc;
+    const float inf = __builtin_huge_valf();
+    const float pads[8] = {-inf, -inf, -inf, -inf, 0.0f, 0.0f, 0.0f, 0.0f};
+    rc = check_hip(hipMemcpy(static_cast<float*>(p) + kScratchFloats, pads, sizeof(pads), hipMemcpyHostToDevice),
+                   "hipMemcpy(pads)");
+    if (rc) {
+        (void)hipFree(p);
+        return rc;
+    }
     g_scratch[device] = static_cast<float*>(p);
     return CTAMD_OK;
 }

@@ -37,6 +37,12 @@ __device__ __forceinline__ double wave_sum(double v) {
     return v;
 }
 
+// Barrier for exchanges through LDS only.  __syncthreads() also waits for every outstanding global
+// load of the wave (its fence covers global memory), which would make the prefetched next row land
+// before the current row is processed - exactly the latency the prefetch is there to hide.  Here
+// only LDS traffic (lgkmcnt) is drained before the barrier.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // Block-wide reductions whose result every thread receives.  `slot` is LDS of THREADS/64 + 1
 // entries; consecutive calls must use distinct slots or be separated by the caller's barrier -
 // each call ends with the barrier that makes its slot reusable two calls later.
@@ -45,11 +51,11 @@ __device__ __forceinline__ V block_all(V v, V* slot, Fold fold) {
     if (THREADS == 64) return v;
     constexpr int W = THREADS / 64;
     if ((threadIdx.x & 63) == 0) slot[threadIdx.x >> 6] = v;
-    __syncthreads();
+    lds_barrier();
     V t = slot[0];
 #pragma unroll
     for (int w = 1; w < W; ++w) t = fold(t, slot[w]);
-    __syncthreads();
+    lds_barrier();
     return t;
 }
 template <int THREADS>
@@ -72,33 +78,34 @@ __device__ __forceinline__ void stage_exp_table(uint64_t* exp2) {
 
 constexpr float kNegInf = -__builtin_huge_valf();
 
+
 // A row held in registers: ITEMS groups of W floats per thread, group k of thread t covering
 // elements [(t + k*THREADS) * W, +W).
 template <int THREADS, int ITEMS, int W>
 struct Row {
     float v[ITEMS][W];
-    __device__ __forceinline__ void load(const float* __restrict__ p, size_t cols, float pad) {
+    // Branch-free: a group past the end of the row is fetched from a constant pad vector instead
+    // (the select is on the address, not on the data), so the loads form one straight-line burst
+    // whose results nothing touches until the row is processed - the compiler can then count them
+    // exactly when it places its waits, and the next row's loads stay in flight meanwhile.
+    __device__ __forceinline__ void load(const float* __restrict__ p, unsigned cols, const float* __restrict__ pad) {
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) {
-            size_t e = (size_t(threadIdx.x) + size_t(k) * THREADS) * W;
-            if (e < cols) {
-                if (W == 4) {
-                    v4f t = *reinterpret_cast<const v4f*>(p + e);
+            const unsigned e = (threadIdx.x + unsigned(k) * THREADS) * W;
+            const float* src = (e < cols) ? p + e : pad;
+            if (W == 4) {
+                v4f t = *reinterpret_cast<const v4f*>(src);
 #pragma unroll
-                    for (int i = 0; i < W; ++i) v[k][i] = t[i];
-                } else {
-                    v[k][0] = p[e];
-                }
+                for (int i = 0; i < W; ++i) v[k][i] = t[i];
             } else {
-#pragma unroll
-                for (int i = 0; i < W; ++i) v[k][i] = pad;
+                v[k][0] = *src;
             }
         }
     }
-    __device__ __forceinline__ void store(float* __restrict__ p, size_t cols) const {
+    __device__ __forceinline__ void store(float* __restrict__ p, unsigned cols) const {
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) {
-            size_t e = (size_t(threadIdx.x) + size_t(k) * THREADS) * W;
+            const unsigned e = (threadIdx.x + unsigned(k) * THREADS) * W;
             if (e < cols) {
                 if (W == 4) {
                     v4f t;
@@ -116,7 +123,7 @@ struct Row {
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k)
 #pragma unroll
-            for (int i = 0; i < W; ++i) m = (v[k][i] > m) ? v[k][i] : m;
+            for (int i = 0; i < W; ++i) m = __builtin_fmaxf(m, v[k][i]);
         return m;
     }
     // v <- exp(v - m) (padding lanes hold -inf and give exactly 0); returns this thread's sum
@@ -126,13 +133,43 @@ struct Row {
         for (int k = 0; k < ITEMS; ++k)
 #pragma unroll
             for (int i = 0; i < W; ++i) {
-                v[k][i] = cta_expf_tab(v[k][i] - m, exp2);
+                v[k][i] = cta_expf_nonpos(v[k][i] - m, exp2);
                 s += v[k][i];
             }
         return s;
     }
-    __device__ __forceinline__ size_t index(int k, int i) const {
-        return (size_t(threadIdx.x) + size_t(k) * THREADS) * W + i;
+    // sum of exp(v - m) without changing v, with the hardware exp2: the loss only needs this sum
+    // to ~1e-7 relative (the reference's own sequential sum is no closer), so the forward loss
+    // kernels skip the bit-exact exp for it and stay bandwidth-bound
+    __device__ __forceinline__ float sum_exp_fast(float m) const {
+        float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k)
+#pragma unroll
+            for (int i = 0; i < W; ++i) {
+                float e = __builtin_amdgcn_exp2f((v[k][i] - m) * 1.44269504088896340736f);
+                if ((k * W + i) & 1) s1 += e; else s0 += e;
+            }
+        return s0 + s1;
+    }
+    __device__ __forceinline__ unsigned index(int k, int i) const {
+        return (threadIdx.x + unsigned(k) * THREADS) * W + i;
+    }
+    // group k of another row-shaped operand, fetched when it is needed (keeps register pressure low)
+    __device__ __forceinline__ void group(const float* __restrict__ p, unsigned cols, int k, float pad, float (&g)[W]) const {
+        const unsigned e = (threadIdx.x + unsigned(k) * THREADS) * W;
+        if (e < cols) {
+            if (W == 4) {
+                v4f t = *reinterpret_cast<const v4f*>(p + e);
+#pragma unroll
+                for (int i = 0; i < W; ++i) g[i] = t[i];
+            } else {
+                g[0] = p[e];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < W; ++i) g[i] = pad;
+        }
     }
 };
 
@@ -146,49 +183,43 @@ struct Args {
     double* partials;    // per-block loss partials (forward loss modes)
     int32_t* status;     // bad-index flag (kCeIndex), may be null
     size_t rows, cols;
+    // what a row's register copy holds beyond the row's end: four floats of -inf for logits (exp
+    // gives exactly 0) and of 0 for the factors of a dot product, in device memory
+    const float* pad_neg_inf;
+    const float* pad_zero;
 };
 
+// A block walks rows blockIdx.x, blockIdx.x + gridDim.x, ...  For the one-operand modes (softmax,
+// class-index cross entropy forward / backward) the next row's loads are issued before the current
+// row is processed, so HBM latency hides behind the exp / divide work of the row in hand: with
+// 1024-thread blocks only one block fits a CU, and without this the CU would alternate between
+// waiting for memory and computing.
 template <int MODE, int THREADS, int ITEMS, int W>
 __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
     __shared__ uint64_t s_exp2[32];
     __shared__ float s_f[2][THREADS / 64 + 1];
     __shared__ double s_d[THREADS / 64 + 1];
     stage_exp_table(s_exp2);
+    constexpr bool kPipelined = (MODE == kSoftmax || MODE == kCeIndex || MODE == kCeBwdIndex);
     double block_loss = 0.0;
-    for (size_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
-        const float* xr = a.x + row * a.cols;
-        Row<THREADS, ITEMS, W> r;
-        if (MODE == kSoftmaxBwd) {
-            // r = y, q = g: d = sum g*y, dx = y * (g - d)
-            Row<THREADS, ITEMS, W> q;
-            r.load(xr, a.cols, 0.0f);
-            q.load(a.t + row * a.cols, a.cols, 0.0f);
-            float d = 0.0f;
-#pragma unroll
-            for (int k = 0; k < ITEMS; ++k)
-#pragma unroll
-                for (int i = 0; i < W; ++i) d += q.v[k][i] * r.v[k][i];
-            d = block_sum<THREADS>(d, s_f[0]);
-#pragma unroll
-            for (int k = 0; k < ITEMS; ++k)
-#pragma unroll
-                for (int i = 0; i < W; ++i) r.v[k][i] = r.v[k][i] * (q.v[k][i] - d);
-            r.store(a.out + row * a.cols, a.cols);
-            continue;
-        }
-        r.load(xr, a.cols, kNegInf);
-        const float m = block_max<THREADS>(r.max(), s_f[0]);
-        const float s = block_sum<THREADS>(r.exp_shifted(m, s_exp2), s_f[1]);
+
+    // everything that happens to one row once it sits in `r`; `mloc` is this thread's maximum
+    auto process = [&](Row<THREADS, ITEMS, W>& r, size_t row, float mloc) {
+        const float m = block_max<THREADS>(mloc, s_f[0]);
+        constexpr bool kLossOnly = (MODE == kCeOnehot || MODE == kCeIndex);
+        // loss kernels keep x in r and only need the row sum; the others turn r into exp(x - m)
+        const float s = block_sum<THREADS>(kLossOnly ? r.sum_exp_fast(m) : r.exp_shifted(m, s_exp2), s_f[1]);
+        const double rcp_s = 1.0 / double(s);     // e / s below is the exact fp32 quotient (cta_div_rcp)
         if (MODE == kSoftmax) {
 #pragma unroll
             for (int k = 0; k < ITEMS; ++k)
 #pragma unroll
-                for (int i = 0; i < W; ++i) r.v[k][i] = r.v[k][i] / s;
-            r.store(a.out + row * a.cols, a.cols);
+                for (int i = 0; i < W; ++i) r.v[k][i] = cta_div_rcp(r.v[k][i], rcp_s);
+            r.store(a.out + row * a.cols, unsigned(a.cols));
         } else if (MODE == kCeOnehot) {
             // -sum_j t_j * log(max(e_j / s, 1e-10)); terms with t_j == 0 contribute exactly 0
             Row<THREADS, ITEMS, W> q;
-            q.load(a.t + row * a.cols, a.cols, 0.0f);
+            q.load(a.t + row * a.cols, unsigned(a.cols), a.pad_zero);
             double loss = 0.0;
 #pragma unroll
             for (int k = 0; k < ITEMS; ++k)
@@ -196,7 +227,7 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
                 for (int i = 0; i < W; ++i) {
                     float tj = q.v[k][i];
                     if (tj != 0.0f) {
-                        float p = r.v[k][i] / s;
+                        float p = cta_div_rcp(cta_expf_nonpos(r.v[k][i] - m, s_exp2), rcp_s);
                         p = (p < 1e-10f) ? 1e-10f : p;
                         float lg = float(log(double(p)));
                         loss -= double(tj * lg);
@@ -210,13 +241,19 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
                 if (threadIdx.x == 0 && a.status) a.status[0] = 1;
                 block_loss += double(__builtin_nanf(""));
             } else {
-                // the thread that holds column c publishes exp(x_c - m)
-                float ec = 0.0f;
+                // the thread that holds column c publishes exp(x_c - m): pick x_c by selects, then
+                // one exact exp per thread (not one per element)
+                float xc = 0.0f;
+                bool mine = false;
 #pragma unroll
                 for (int k = 0; k < ITEMS; ++k)
 #pragma unroll
-                    for (int i = 0; i < W; ++i)
-                        if (r.index(k, i) == size_t(c)) ec = r.v[k][i];
+                    for (int i = 0; i < W; ++i) {
+                        const bool hit = r.index(k, i) == unsigned(c);
+                        xc = hit ? r.v[k][i] : xc;
+                        mine = mine || hit;
+                    }
+                float ec = mine ? cta_expf_nonpos(xc - m, s_exp2) : 0.0f;
                 ec = block_sum<THREADS>(ec, s_f[0]);
                 float p = ec / s;
                 p = (p < 1e-10f) ? 1e-10f : p;
@@ -225,28 +262,81 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
         } else {   // kCeBwdOnehot / kCeBwdIndex: dx = (e / s - t) * g
             const float g = a.g1[0];
             if (MODE == kCeBwdOnehot) {
-                Row<THREADS, ITEMS, W> q;
-                q.load(a.t + row * a.cols, a.cols, 0.0f);
 #pragma unroll
-                for (int k = 0; k < ITEMS; ++k)
+                for (int k = 0; k < ITEMS; ++k) {
+                    float tq[W];
+                    r.group(a.t + row * a.cols, unsigned(a.cols), k, 0.0f, tq);
 #pragma unroll
                     for (int i = 0; i < W; ++i) {
-                        float sm = r.v[k][i] / s;
-                        float d = sm - q.v[k][i];
+                        float sm = cta_div_rcp(r.v[k][i], rcp_s);
+                        float d = sm - tq[i];
                         r.v[k][i] = d * g;
                     }
+                }
             } else {
                 const int c = int(a.t[row]);
 #pragma unroll
                 for (int k = 0; k < ITEMS; ++k)
 #pragma unroll
                     for (int i = 0; i < W; ++i) {
-                        float sm = r.v[k][i] / s;
-                        float d = sm - ((r.index(k, i) == size_t(c) && c >= 0) ? 1.0f : 0.0f);
+                        float sm = cta_div_rcp(r.v[k][i], rcp_s);
+                        float d = sm - ((r.index(k, i) == unsigned(c)) ? 1.0f : 0.0f);
                         r.v[k][i] = d * g;
                     }
             }
-            r.store(a.out + row * a.cols, a.cols);
+            r.store(a.out + row * a.cols, unsigned(a.cols));
+        }
+    };
+
+    const size_t stride = gridDim.x;
+    size_t row = blockIdx.x;
+    if (MODE == kSoftmaxBwd) {
+        for (; row < a.rows; row += stride) {
+            // r = y, q = g: d = sum g*y, dx = y * (g - d)
+            Row<THREADS, ITEMS, W> r, q;
+            r.load(a.x + row * a.cols, unsigned(a.cols), a.pad_zero);
+            q.load(a.t + row * a.cols, unsigned(a.cols), a.pad_zero);
+            float d = 0.0f;
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k)
+#pragma unroll
+                for (int i = 0; i < W; ++i) d += q.v[k][i] * r.v[k][i];
+            d = block_sum<THREADS>(d, s_f[0]);
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k)
+#pragma unroll
+                for (int i = 0; i < W; ++i) r.v[k][i] = r.v[k][i] * (q.v[k][i] - d);
+            r.store(a.out + row * a.cols, unsigned(a.cols));
+        }
+    } else if (kPipelined) {
+        // Two register copies of a row, alternating.  Per row: take the thread's maximum (the first
+        // touch of the row's data, i.e. the wait for its loads), THEN issue the next row's loads,
+        // then do the exp / divide / store work, during which those loads are in flight.  The
+        // order matters: loads and stores share one in-order counter on this architecture, and a
+        // wait with both kinds outstanding drains everything - issued before the first touch, the
+        // new loads would be waited for at once.
+        Row<THREADS, ITEMS, W> ra, rb;
+        if (row < a.rows) ra.load(a.x + row * a.cols, unsigned(a.cols), a.pad_neg_inf);
+        while (row < a.rows) {
+            float mloc = ra.max();
+            asm volatile("" : "+v"(mloc) : : "memory");   // the loads below may not move above this
+            if (row + stride < a.rows) rb.load(a.x + (row + stride) * a.cols, unsigned(a.cols), a.pad_neg_inf);
+            __builtin_amdgcn_sched_barrier(0);
+            process(ra, row, mloc);
+            row += stride;
+            if (row >= a.rows) break;
+            mloc = rb.max();
+            asm volatile("" : "+v"(mloc) : : "memory");
+            if (row + stride < a.rows) ra.load(a.x + (row + stride) * a.cols, unsigned(a.cols), a.pad_neg_inf);
+            __builtin_amdgcn_sched_barrier(0);
+            process(rb, row, mloc);
+            row += stride;
+        }
+    } else {
+        for (; row < a.rows; row += stride) {
+            Row<THREADS, ITEMS, W> r;
+            r.load(a.x + row * a.cols, unsigned(a.cols), a.pad_neg_inf);
+            process(r, row, r.max());
         }
     }
     if ((MODE == kCeOnehot || MODE == kCeIndex) && threadIdx.x == 0) a.partials[blockIdx.x] = block_loss;
@@ -287,7 +377,7 @@ __global__ __launch_bounds__(1024) void row_stream_kernel(Args a) {
         const float S = block_sum<THREADS>(s, s_f[1]);
         if (MODE == kSoftmax) {
             for (size_t j = threadIdx.x; j < a.cols; j += THREADS)
-                a.out[row * a.cols + j] = cta_expf_tab(xr[j] - M, s_exp2) / S;
+                a.out[row * a.cols + j] = cta_div_rcp(cta_expf_tab(xr[j] - M, s_exp2), 1.0 / double(S));
         } else if (MODE == kCeOnehot) {
             const float* tr = a.t + row * a.cols;
             double loss = 0.0;
@@ -322,6 +412,73 @@ __global__ __launch_bounds__(1024) void row_stream_kernel(Args a) {
         }
     }
     if ((MODE == kCeOnehot || MODE == kCeIndex) && threadIdx.x == 0) a.partials[blockIdx.x] = block_loss;
+}
+
+// Class-index cross entropy, forward, for long rows: a single pass with an online (max, sum) pair
+// per thread.  Nothing of the row is kept, so a 256-thread block per row needs few registers, many
+// blocks share a CU and the kernel runs at memory speed (the register-resident variant, one
+// 1024-thread block per CU, reached 3.9 TB/s on 8192 x 32000).  Each 128-bit vector first raises
+// the running maximum (rescaling the running sum by exp(old - new) when it grows) and then adds its
+// four exp(x - max) terms, all with the hardware exp2: only the row's log-sum is needed, to ~1e-7
+// relative.  The target logit's own term exp(x_c - max) is evaluated with the bit-exact exp.
+constexpr float kLog2e = 1.44269504088896340736f;
+
+template <bool VEC>
+__global__ __launch_bounds__(256) void ce_index_online_kernel(Args a) {
+    constexpr int THREADS = 256;
+    __shared__ uint64_t s_exp2[32];
+    __shared__ float s_f[2][THREADS / 64 + 1];
+    stage_exp_table(s_exp2);
+    double block_loss = 0.0;
+    for (size_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
+        const float* __restrict__ xr = a.x + row * a.cols;
+        float m = kNegInf, s = 0.0f;
+        auto absorb4 = [&](v4f v) {
+            float cm = __builtin_fmaxf(__builtin_fmaxf(v[0], v[1]), __builtin_fmaxf(v[2], v[3]));
+            if (cm > m) {
+                s *= __builtin_amdgcn_exp2f((m - cm) * kLog2e);     // exp2(-inf) = 0 on the first vector
+                m = cm;
+            }
+            const float b = (m == kNegInf) ? 0.0f : m;              // all -inf so far: terms are exp(-inf) = 0, not NaN
+            s += (__builtin_amdgcn_exp2f((v[0] - b) * kLog2e) + __builtin_amdgcn_exp2f((v[1] - b) * kLog2e)) +
+                 (__builtin_amdgcn_exp2f((v[2] - b) * kLog2e) + __builtin_amdgcn_exp2f((v[3] - b) * kLog2e));
+        };
+        if (VEC) {
+            const unsigned n4 = unsigned(a.cols >> 2);
+            constexpr int U = 8;
+            unsigned i = threadIdx.x;
+            for (; i + (U - 1) * THREADS < n4; i += U * THREADS) {
+                v4f v[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(xr) + i + u * THREADS);
+#pragma unroll
+                for (int u = 0; u < U; ++u) absorb4(v[u]);
+            }
+            for (; i < n4; i += THREADS) absorb4(reinterpret_cast<const v4f*>(xr)[i]);
+        } else {
+            for (size_t j = threadIdx.x; j < a.cols; j += THREADS) {
+                float v = xr[j];
+                if (v > m) {
+                    s *= __builtin_amdgcn_exp2f((m - v) * kLog2e);
+                    m = v;
+                }
+                s += __builtin_amdgcn_exp2f((v - ((m == kNegInf) ? 0.0f : m)) * kLog2e);
+            }
+        }
+        const float M = block_max<THREADS>(m, s_f[0]);
+        s = (m == kNegInf) ? 0.0f : s * __builtin_amdgcn_exp2f((m - M) * kLog2e);
+        const float S = block_sum<THREADS>(s, s_f[1]);
+        const int c = int(a.t[row]);
+        if (c < 0 || c >= int(a.cols)) {
+            if (threadIdx.x == 0 && a.status) a.status[0] = 1;
+            block_loss += double(__builtin_nanf(""));
+        } else if (threadIdx.x == 0) {
+            float p = cta_expf_nonpos(xr[c] - M, s_exp2) / S;
+            p = (p < 1e-10f) ? 1e-10f : p;
+            block_loss -= double(float(log(double(p))));
+        }
+    }
+    if (threadIdx.x == 0) a.partials[blockIdx.x] = block_loss;
 }
 
 // out[0] = float(sum of partials), folded in a fixed order.
@@ -370,13 +527,28 @@ int run_rows(const char* name, Args a, float* loss_out, void* stream) {
     if ((MODE == kCeBwdOnehot || MODE == kCeBwdIndex) && !a.g1) return fail(CTAMD_EINVAL, "%s: null upstream gradient", name);
     if (a.rows > (size_t(1) << 62) / a.cols) return fail(CTAMD_ERANGE, "%s: rows*cols overflows", name);
     if (a.cols > size_t(0x7fffffff)) return fail(CTAMD_ERANGE, "%s: more than 2^31-1 columns", name);
-    if (kLoss) {
-        a.partials = reinterpret_cast<double*>(scratch());
-        if (!a.partials) return CTAMD_EINVAL;
-    }
-    unsigned grid = a.rows < kMaxRowBlocks ? unsigned(a.rows) : kMaxRowBlocks;
+    a.pad_neg_inf = pad_neg_inf();
+    a.pad_zero = pad_zero();
+    if (!a.pad_zero) return CTAMD_EINVAL;
+    if (kLoss) a.partials = reinterpret_cast<double*>(scratch());
+    // rows are dealt to a chip-filling number of blocks (each walks several rows, prefetching the next)
+    const size_t groups = (a.cols + 3) / 4;
+    const int threads = groups <= 64 * 8 ? 64 : groups <= 256 * 8 ? 256 : 1024;
+    size_t fill = size_t(compute_units() > 0 ? compute_units() : 256) * size_t(2048 / threads);
+    if (fill > kMaxRowBlocks) fill = kMaxRowBlocks;
+    unsigned grid = a.rows < fill ? unsigned(a.rows) : unsigned(fill);
     bool vec = (a.cols % 4 == 0) && aligned16(a.x) && (MODE == kSoftmax || MODE == kCeIndex || MODE == kCeBwdIndex || aligned16(a.t)) &&
                (kLoss || aligned16(a.out));
+    if (MODE == kCeIndex && a.cols >= 2048) {
+        size_t fill_online = size_t(compute_units() > 0 ? compute_units() : 256) * 8;
+        grid = a.rows < fill_online ? unsigned(a.rows) : unsigned(fill_online);
+        if (vec) hipLaunchKernelGGL((ce_index_online_kernel<true>), dim3(grid), dim3(256), 0, s, a);
+        else hipLaunchKernelGGL((ce_index_online_kernel<false>), dim3(grid), dim3(256), 0, s, a);
+        int rc0 = launched(name);
+        if (rc0) return rc0;
+        hipLaunchKernelGGL(loss_stage2, dim3(1), dim3(256), 0, s, a.partials, grid, loss_out);
+        return launched(name);
+    }
     bool done = vec ? launch_resident<MODE, 4>(a, grid, s) : launch_resident<MODE, 1>(a, grid, s);
     if (!done) hipLaunchKernelGGL((row_stream_kernel<MODE>), dim3(grid), dim3(1024), 0, s, a);
     int rc = launched(name);
@@ -426,11 +598,11 @@ using namespace ctamd;
 extern "C" {
 
 int ctamd_softmax_rows_f32(const float* x, float* y, size_t rows, size_t cols, void* stream) {
-    Args a{x, nullptr, nullptr, y, nullptr, nullptr, rows, cols};
+    Args a{x, nullptr, nullptr, y, nullptr, nullptr, rows, cols, nullptr, nullptr};
     return run_rows<kSoftmax>(__func__, a, nullptr, stream);
 }
 int ctamd_cross_entropy_onehot_f32(const float* x, const float* t, float* out, size_t rows, size_t cols, void* stream) {
-    Args a{x, t, nullptr, nullptr, nullptr, nullptr, rows, cols};
+    Args a{x, t, nullptr, nullptr, nullptr, nullptr, rows, cols, nullptr, nullptr};
     return run_rows<kCeOnehot>(__func__, a, out, stream);
 }
 int ctamd_cross_entropy_index_f32(const float* x, const float* idx, float* out, int32_t* status, size_t rows,
@@ -440,21 +612,21 @@ int ctamd_cross_entropy_index_f32(const float* x, const float* idx, float* out, 
         int rc = launched(__func__);
         if (rc) return rc;
     }
-    Args a{x, idx, nullptr, nullptr, nullptr, status, rows, cols};
+    Args a{x, idx, nullptr, nullptr, nullptr, status, rows, cols, nullptr, nullptr};
     return run_rows<kCeIndex>(__func__, a, out, stream);
 }
 int ctamd_cross_entropy_backward_onehot_f32(const float* x, const float* t, const float* g1, float* dx, size_t rows,
                                             size_t cols, void* stream) {
-    Args a{x, t, g1, dx, nullptr, nullptr, rows, cols};
+    Args a{x, t, g1, dx, nullptr, nullptr, rows, cols, nullptr, nullptr};
     return run_rows<kCeBwdOnehot>(__func__, a, nullptr, stream);
 }
 int ctamd_cross_entropy_backward_index_f32(const float* x, const float* idx, const float* g1, float* dx, size_t rows,
                                            size_t cols, void* stream) {
-    Args a{x, idx, g1, dx, nullptr, nullptr, rows, cols};
+    Args a{x, idx, g1, dx, nullptr, nullptr, rows, cols, nullptr, nullptr};
     return run_rows<kCeBwdIndex>(__func__, a, nullptr, stream);
 }
 int ctamd_softmax_backward_rows_f32(const float* y, const float* g, float* dx, size_t rows, size_t cols, void* stream) {
-    Args a{y, g, nullptr, dx, nullptr, nullptr, rows, cols};
+    Args a{y, g, nullptr, dx, nullptr, nullptr, rows, cols, nullptr, nullptr};
     return run_rows<kSoftmaxBwd>(__func__, a, nullptr, stream);
 }
 

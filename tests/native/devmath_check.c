@@ -1,7 +1,8 @@
 /* Host check of ctorch_amd/csrc/devmath.h against the installed glibc: counts the floats for
  * which the device algorithms (compiled here for the CPU, unchanged) return different bits from
  * expf / sinf / cosf.  Usage: devmath_check STRIDE  (1 = every one of the 2^32 bit patterns).
- * Prints one line per function: name, inputs tested, mismatches, worst ulp distance. */
+ * Prints one line per function: name, inputs tested, mismatches, worst ulp distance
+ * (expf_pair: exp(x) and exp(-x) from the shared reduction, against expf(x) and expf(-x)). */
 #include <math.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -24,9 +25,9 @@ static int differs(float a, float b, int64_t* ulp) {
 int main(int argc, char** argv) {
     uint64_t stride = argc > 1 ? strtoull(argv[1], 0, 10) : 1;
     if (stride == 0) stride = 1;
-    uint64_t n = 0, bad[3] = {0, 0, 0}, covered[3] = {0, 0, 0};
-    int64_t worst[3] = {0, 0, 0};
-#pragma omp parallel for reduction(+ : n, bad[:3], covered[:3]) reduction(max : worst[:3]) schedule(static)
+    uint64_t n = 0, bad[4] = {0, 0, 0, 0}, covered[4] = {0, 0, 0, 0};
+    int64_t worst[4] = {0, 0, 0, 0};
+#pragma omp parallel for reduction(+ : n, bad[:4], covered[:4]) reduction(max : worst[:4]) schedule(static)
     for (uint64_t u = 0; u < (1ULL << 32); u += stride) {
         float x = cta_u2f((uint32_t)u);
         int64_t d = 0;
@@ -35,6 +36,17 @@ int main(int argc, char** argv) {
         if (differs(cta_expf_tab(x, cta_exp2_tab), expf(x), &d)) {
             ++bad[0];
             if (d > worst[0]) worst[0] = d;
+        }
+        if (!(x > 0.0f) && differs(cta_expf_nonpos(x, cta_exp2_tab), expf(x), &d)) {   /* x <= 0 or NaN */
+            ++bad[0];
+            if (d > worst[0]) worst[0] = d;
+        }
+        float ep, en;
+        cta_expf_pair(x, cta_exp2_tab, &ep, &en);
+        ++covered[3];
+        if (differs(ep, expf(x), &d) || differs(en, expf(-x), &d)) {
+            ++bad[3];
+            if (d > worst[3]) worst[3] = d;
         }
         ++covered[1];
         if (differs(cta_sincosf(x, 0, cta_inv_pio4), sinf(x), &d)) {
@@ -47,8 +59,8 @@ int main(int argc, char** argv) {
             if (d > worst[2]) worst[2] = d;
         }
     }
-    const char* names[3] = {"expf", "sinf", "cosf"};
-    for (int k = 0; k < 3; ++k)
+    const char* names[4] = {"expf", "sinf", "cosf", "expf_pair"};
+    for (int k = 0; k < 4; ++k)
         printf("%s tested %llu mismatches %llu worst_ulp %lld\n", names[k], (unsigned long long)covered[k],
                (unsigned long long)bad[k], (long long)worst[k]);
     return 0;

@@ -1,0 +1,36 @@
+/* Host check of cta_div_rcp (ctorch_amd/csrc/devmath.h): division by a shared divisor through its
+ * double-precision reciprocal against IEEE fp32 division, on random operand pairs that include
+ * subnormal numerators and divisors, numerators <= 1 with divisors >= 1 (the softmax case) and the
+ * full exponent range.  Usage: divcheck [PAIRS_PER_THREAD]; prints "tested N bad M". */
+#include <stdio.h>
+#include <stdint.h>
+#include <string.h>
+#include <math.h>
+#include <stdlib.h>
+#include "../../ctorch_amd/csrc/devmath.h"
+static float u2f(uint32_t u){float f;memcpy(&f,&u,4);return f;}
+static uint32_t f2u(float f){uint32_t u;memcpy(&u,&f,4);return u;}
+static uint64_t rng(uint64_t*s){*s^=*s<<13;*s^=*s>>7;*s^=*s<<17;return *s;}
+int main(int argc,char**argv){
+  long per=argc>1?atol(argv[1]):40000000L;
+  uint64_t bad=0,total=0;
+  #pragma omp parallel for reduction(+:bad,total)
+  for(int t=0;t<64;++t){
+    uint64_t s=0x9E3779B97F4A7C15ULL*(t+1);
+    for(long i=0;i<per;++i){
+      uint32_t ua=(uint32_t)rng(&s), ub=(uint32_t)rng(&s);
+      int mode=i%4;
+      if(mode==1){ ua=(ua&0x807fffffu)|((uint32_t)(rng(&s)%40)<<23); }           /* tiny / subnormal numerators */
+      if(mode==2){ ub=(ub&0x807fffffu)|((uint32_t)(127+rng(&s)%32)<<23); ua=(ua&0x807fffffu)|((uint32_t)(rng(&s)%128)<<23);} /* s>=1, e<=1 */
+      if(mode==3){ ub=(ub&0x807fffffu)|((uint32_t)(rng(&s)%3)<<23); }              /* subnormal / tiny divisors */
+      float a=u2f(ua), b=u2f(ub);
+      volatile double rb=1.0/(double)b;
+      float q1=cta_div_rcp(a,rb);
+      float q2=a/b;
+      ++total;
+      if(!((q1!=q1)&&(q2!=q2)) && f2u(q1)!=f2u(q2)){ ++bad; if(bad<5) printf("a=%a b=%a fast=%a ieee=%a\n",a,b,q1,q2);}
+    }
+  }
+  printf("tested %llu bad %llu\n",(unsigned long long)total,(unsigned long long)bad);
+  return 0;
+}

@@ -245,6 +245,15 @@ def test_cross_entropy_edge_cases(oracle):
     # 1-D logits (single sample)
     want = oracle.ce_onehot(x[0], oh[0])
     assert abs(G.host(G.ce_onehot(G.dev(x[0]), G.dev(oh[0])))[0] - want) <= 1e-5 * abs(want)
+    # long rows (single-pass kernel): -inf logits contribute exp(-inf) = 0, also where a whole
+    # thread's share of the row is -inf
+    lx = oracle.normal((3, 4096), 32, 0, 2)
+    lx[:, :2600] = -np.inf
+    lx[1, 5::2] = -np.inf
+    lidx = np.array([3000, 3001, 4095], F)
+    want = oracle.ce_index(lx, lidx)
+    got, status = G.ce_index(G.dev(lx), G.dev(lidx))
+    assert status == 0 and abs(G.host(got)[0] - want) <= 1e-5 * abs(want)
     # rows == 0 gives a zero loss
     assert G.host(G.ce_onehot(G.dev(np.zeros((0, 5), F)), G.dev(np.zeros((0, 5), F))))[0] == 0
 
