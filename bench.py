@@ -12,7 +12,7 @@ One step = one pass of BASELINE.json's configs[1] at its largest size, inputs re
 carries the roofline of the dominant kernel (the forward GEMM, timed per launch with HIP events on
 the launch stream inside the timed steps), the elementwise leg of the metric (a + b on 256 MiB
 operands, GB/s against 8 TB/s) and the CPU baseline: the reference's own MatMul kernel
-(oracle/_ref, else the oracle port) timed on one host core on a 64-row slab of the same product.
+(oracle/_ref, else the oracle port) timed on one host core on a 160-row slab of the same product.
 """
 import argparse
 import ctypes as C
@@ -31,8 +31,9 @@ DOT_N = 1 << 26
 EW_N = 1 << 26
 
 # HBM bytes per forward-GEMM launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, scaled
-# by the same counters on a plain copy of known size); see profiles/.  None until measured.
-GEMM_TRAFFIC_BYTES = None
+# by the same counters on the 768 MiB elementwise add of the same run); see
+# profiles/gemm_f32_4096_hbm_traffic.txt (384 MiB fetched + 64 MiB written; 192 MiB algorithmic).
+GEMM_TRAFFIC_BYTES = 470259787
 
 
 def cpu_baseline(seconds_hint=15.0):
@@ -57,7 +58,7 @@ def cpu_baseline(seconds_hint=15.0):
 
 def _cpu_baseline(np, support):
     rng = np.random.default_rng(202)
-    rows = 48
+    rows = 160
     A = rng.standard_normal((rows, M), dtype=np.float32)
     B = rng.standard_normal((M, M), dtype=np.float32)
     kind = "port"
@@ -179,8 +180,8 @@ def main():
         "config": {"workload": "configs[1]: fp32 MatMul 4096^3 forward + backward (dA = dC.B^T, dB = A^T.dC, "
                                "dC = ones) + Dot of two 2^26-element vectors; N(0,1) / uniform[-1,1] inputs "
                                "generated on the device", "M": M, "N": M, "K": M, "dot_n": DOT_N},
-        "roofline": {"bound": "mfma", "kernel": "gemm_kernel<128x128x16, A K-contiguous, B N-contiguous> "
-                                                "(forward C = A.B)",
+        "roofline": {"bound": "mfma", "kernel": "gemm_kernel<Cfg<256,256,16,128,64>, A K-contiguous, "
+                                                "B N-contiguous> (forward C = A.B)",
                      "achieved": round(achieved, 2), "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / MFMA_FP32_PEAK_TFLOPS, 4), "traffic": GEMM_TRAFFIC_BYTES,
                      "launch_ms": round(gemm_ms, 4)},
