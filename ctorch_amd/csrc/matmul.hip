@@ -55,26 +55,27 @@ struct Stage {
     static constexpr int PIECES = ROWS * BK / 4 / THREADS;
     static_assert(ROWS * BK / 4 % THREADS == 0, "tile must split evenly over the block");
     v4f r[PIECES];
-    const float* src[PIECES];   // interior tiles: where this thread's next pieces come from
+    const char* base;           // interior tiles: block-uniform address of the tile's current k position
+    unsigned off;               // this thread's byte offset of piece 0 from `base`
+    unsigned piece_step;        // block-uniform byte distance between consecutive pieces of a thread
 
-    // Interior tiles (whole tile inside the matrix, aligned rows): no bounds logic in the loop, one
-    // pointer per piece advanced by a constant each k tile.
+    // Interior tiles (whole tile inside the matrix, aligned rows): no bounds logic in the loop.  The
+    // address of piece q is (uniform base + q * uniform step) + one 32-bit per-thread offset, which
+    // the compiler turns into scalar-base + vector-offset loads: one address register per operand
+    // and only scalar arithmetic per k tile.  Needs the tile's byte extent below 2^32.
     __device__ __forceinline__ void init_fast(const float* __restrict__ p, int64_t ld, int x0, int k0) {
-#pragma unroll
-        for (int q = 0; q < PIECES; ++q) {
-            int idx = threadIdx.x + q * THREADS;
-            int outer, inner;
-            if (KC) { outer = idx / (BK / 4); inner = (idx % (BK / 4)) * 4; }
-            else { outer = idx / (ROWS / 4); inner = (idx % (ROWS / 4)) * 4; }
-            src[q] = KC ? p + int64_t(x0 + outer) * ld + (k0 + inner) : p + int64_t(k0 + outer) * ld + (x0 + inner);
-        }
+        constexpr int PER = KC ? (BK / 4) : (ROWS / 4);          // 128-bit pieces per contiguous row
+        const int outer = threadIdx.x / PER, inner = (threadIdx.x % PER) * 4;
+        base = reinterpret_cast<const char*>(KC ? p + int64_t(x0) * ld + k0 : p + int64_t(k0) * ld + x0);
+        off = unsigned((int64_t(outer) * ld + inner) * 4);
+        static_assert(THREADS % PER == 0, "pieces of one thread are whole rows apart");
+        piece_step = unsigned(int64_t(THREADS / PER) * ld * 4);
     }
-    __device__ __forceinline__ void load_fast(int64_t step) {
+    __device__ __forceinline__ void load_fast(int64_t step_bytes) {
 #pragma unroll
-        for (int q = 0; q < PIECES; ++q) {
-            r[q] = *reinterpret_cast<const v4f*>(src[q]);
-            src[q] += step;
-        }
+        for (int q = 0; q < PIECES; ++q)
+            r[q] = *reinterpret_cast<const v4f*>(base + size_t(q) * piece_step + off);
+        base += step_bytes;
     }
 
     // x0: first row/col of the tile in the X dimension, k0: first k; dimX, K: extents; ld: leading
@@ -192,62 +193,141 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
     const int ktiles = (k_end - k_begin + BK - 1) / BK;
     // interior: the whole BM x BN tile and every k tile lie inside the operands and rows are
     // 16-byte aligned - true for all blocks of a 4096^3 product, false only on ragged edges
-    const bool interior = VEC && m0 + BM <= g.m && n0 + BN <= g.n && (k_end - k_begin) % BK == 0;
-    const int64_t a_step = A_KC ? BK : int64_t(BK) * g.lda;
-    const int64_t b_step = B_KC ? BK : int64_t(BK) * g.ldb;
+    const bool interior = VEC && m0 + BM <= g.m && n0 + BN <= g.n && (k_end - k_begin) % BK == 0 &&
+                          g.lda < (int64_t(1) << 21) && g.ldb < (int64_t(1) << 21);   // tile extent < 2^32 bytes
+    const int64_t a_step = (A_KC ? BK : int64_t(BK) * g.lda) * 4;   // bytes per k tile
+    const int64_t b_step = (B_KC ? BK : int64_t(BK) * g.ldb) * 4;
     if (interior) {
         sa.init_fast(g.a, g.lda, m0, k_begin);
         sb.init_fast(g.b, g.ldb, n0, k_begin);
     }
-    auto stage_tile = [&](int t) {
-        if (interior) {
-            sa.load_fast(a_step);
-            sb.load_fast(b_step);
-        } else {
+    // s_waitcnt lgkmcnt(0) as an instruction the compiler's wait-count bookkeeping sees (it cannot
+    // look inside inline asm): vmcnt and expcnt fields at their maxima, lgkmcnt 0.
+    auto lds_wait = [] { __builtin_amdgcn_s_waitcnt(0xC07F); };
+    constexpr int NCH = BK / 8;
+    static_assert(NCH == 2, "the pipeline below alternates two fragment buffers over two chunks");
+    float fa[2][TM][4], fb[2][TN][4];
+    auto fetch_chunk = [&](int buf, int ch, int which) {
+        const float* __restrict__ la = s_a[buf];
+        const float* __restrict__ lb = s_b[buf];
+        const int kb = ch * 8 + half * 4;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fetch<A_KC>(la, A_STRIDE, wm + i * 32 + l32, kb, fa[which][i]);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fetch<B_KC>(lb, B_STRIDE, wn + j * 32 + l32, kb, fb[which][j]);
+    };
+    auto mfmas = [&](int which) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[which][i][s], fb[which][j][s], acc[i][j], 0, 0, 0);
+    };
+    constexpr int kMfmaPerChunk = 4 * TM * TN;
+    constexpr int kStores = Stage<BM, BK, A_KC, C::THREADS>::PIECES + Stage<BN, BK, B_KC, C::THREADS>::PIECES;
+    constexpr int kMaskMfma = 0x008, kMaskVmemRead = 0x020, kMaskDsRead = 0x100, kMaskDsWrite = 0x200;
+
+    // Software pipeline over the two 8-wide k chunks of a k tile, two fragment buffers:
+    //   burst 0: MFMAs of chunk 0 | issued under them: LDS reads of chunk 1, and at the tail the
+    //            staged tile t+1 registers -> LDS;                      then the tile's one barrier
+    //   burst 1: MFMAs of chunk 1 | issued under them: LDS reads of chunk 0 of tile t+1 and the
+    //            global loads of tile t+2
+    // so every fragment is requested most of a burst before its first use and a global load has a
+    // whole k tile to arrive.  A wave issues in order, and an MFMA keeps the matrix pipe busy for
+    // 64 cycles, so one memory instruction slipped in after an MFMA is free; what must not happen
+    // is a wait in front of an MFMA for data requested just before it.  Interior blocks pin the
+    // interleaving with scheduling groups; the two waves of a SIMD run in phase (one barrier per
+    // tile), so housekeeping outside the bursts would idle the pipe for both.
+    if (interior) {
+        sa.load_fast(a_step);
+        sb.load_fast(b_step);
+        sa.store(s_a[0], A_STRIDE);
+        sb.store(s_b[0], B_STRIDE);
+        __syncthreads();
+        // the loop always requests tile t+2; past the end the request repeats the last tile
+        // (in bounds, never stored), which keeps the loop body free of branches
+        if (ktiles > 1) { sa.load_fast(ktiles > 2 ? a_step : 0); sb.load_fast(ktiles > 2 ? b_step : 0); }
+        fetch_chunk(0, 0, 0);
+        for (int t = 0; t + 1 < ktiles; ++t) {
+            const int cur = t & 1;
+            __builtin_amdgcn_sched_barrier(0);
+            lds_wait();
+            fetch_chunk(cur, 1, 1);
+            mfmas(0);
+            sa.store(s_a[cur ^ 1], A_STRIDE);
+            sb.store(s_b[cur ^ 1], B_STRIDE);
+#pragma unroll
+            for (int q = 0; q < 12; ++q) {
+                __builtin_amdgcn_sched_group_barrier(kMaskMfma, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(kMaskDsRead, 1, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(kMaskMfma, kMfmaPerChunk - 12 - kStores, 0);
+#pragma unroll
+            for (int q = 0; q < kStores; ++q) {
+                __builtin_amdgcn_sched_group_barrier(kMaskMfma, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(kMaskDsWrite, 1, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
+            fetch_chunk(cur ^ 1, 0, 0);
+            const bool more = t + 3 < ktiles;
+            sa.load_fast(more ? a_step : 0);
+            sb.load_fast(more ? b_step : 0);
+            mfmas(1);
+#pragma unroll
+            for (int q = 0; q < 12; ++q) {
+                __builtin_amdgcn_sched_group_barrier(kMaskMfma, 1, 1);
+                __builtin_amdgcn_sched_group_barrier(kMaskDsRead, 1, 1);
+            }
+#pragma unroll
+            for (int q = 0; q < kStores; ++q) {
+                __builtin_amdgcn_sched_group_barrier(kMaskMfma, 1, 1);
+                __builtin_amdgcn_sched_group_barrier(kMaskVmemRead, 1, 1);
+            }
+            __builtin_amdgcn_sched_group_barrier(kMaskMfma, kMfmaPerChunk - 12 - kStores, 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    } else {
+        auto stage_tile = [&](int t) {
             sa.template load<VEC>(g.a, g.lda, m0, k_begin + t * BK, g.m, k_end);
             sb.template load<VEC>(g.b, g.ldb, n0, k_begin + t * BK, g.n, k_end);
-        }
-    };
-    if (ktiles > 0) {
+        };
         stage_tile(0);
         sa.store(s_a[0], A_STRIDE);
         sb.store(s_b[0], B_STRIDE);
-    }
-    __syncthreads();
-    for (int t = 0; t < ktiles; ++t) {
-        const int cur = t & 1;
-        const float* __restrict__ la = s_a[cur];
-        const float* __restrict__ lb = s_b[cur];
-        // 1. every fragment of this k tile into registers, 2. the next tile's global loads,
-        // 3. all MFMAs back to back.  The scheduling fences keep that order: interleaving a
-        // fragment load and its wait into each group of four MFMAs (what the scheduler does when
-        // left alone, to save registers) left the matrix pipe idle about a fifth of the time.
-        float fa[BK / 8][TM][4], fb[BK / 8][TN][4];
-#pragma unroll
-        for (int ch = 0; ch < BK / 8; ++ch) {
-            const int kb = ch * 8 + half * 4;
-#pragma unroll
-            for (int i = 0; i < TM; ++i) fetch<A_KC>(la, A_STRIDE, wm + i * 32 + l32, kb, fa[ch][i]);
-#pragma unroll
-            for (int j = 0; j < TN; ++j) fetch<B_KC>(lb, B_STRIDE, wn + j * 32 + l32, kb, fb[ch][j]);
-        }
-        if (t + 1 < ktiles) stage_tile(t + 1);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int ch = 0; ch < BK / 8; ++ch)
-#pragma unroll
-            for (int s = 0; s < 4; ++s)
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[ch][i][s], fb[ch][j][s], acc[i][j], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        if (t + 1 < ktiles) {
+        __syncthreads();
+        if (ktiles > 1) stage_tile(1);
+        fetch_chunk(0, 0, 0);
+        for (int t = 0; t + 1 < ktiles; ++t) {
+            const int cur = t & 1;
+            lds_wait();
+            fetch_chunk(cur, 1, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mfmas(0);
+            __builtin_amdgcn_sched_barrier(0);
             sa.store(s_a[cur ^ 1], A_STRIDE);
             sb.store(s_b[cur ^ 1], B_STRIDE);
+            __syncthreads();
+            fetch_chunk(cur ^ 1, 0, 0);
+            if (t + 2 < ktiles) stage_tile(t + 2);
+            __builtin_amdgcn_sched_barrier(0);
+            mfmas(1);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __syncthreads();
+    }
+    // last k tile: nothing left to stage
+    {
+        const int cur = (ktiles - 1) & 1;
+        lds_wait();
+        fetch_chunk(cur, 1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mfmas(0);
+        __builtin_amdgcn_sched_barrier(0);
+        lds_wait();
+        mfmas(1);
     }
 
     // accumulator register r of lane l holds C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 tile
@@ -340,8 +420,8 @@ extern "C" int ctamd_matmul_f32(const float* a, int64_t as0, int64_t as1, const 
     const int64_t big_tiles = ((m + BigTile::BM - 1) / BigTile::BM) * ((n + BigTile::BN - 1) / BigTile::BN);
     const bool big = big_tiles >= cus;
     const int BM = big ? BigTile::BM : SmallTile::BM, BN = big ? BigTile::BN : SmallTile::BN;
-    constexpr int BK = SmallTile::BK;
-    static_assert(BigTile::BK == SmallTile::BK, "both tile shapes step K alike");
+    const int BK = big ? BigTile::BK : SmallTile::BK;
+    
     GemmArgs g;
     g.a = a; g.lda = A_KC ? as0 : as1;
     g.b = b; g.ldb = B_KC ? bs1 : bs0;
