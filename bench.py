@@ -13,6 +13,13 @@ carries the roofline of the dominant kernel (the forward GEMM, timed per launch 
 the launch stream inside the timed steps), the elementwise leg of the metric (a + b on 256 MiB
 operands, GB/s against 8 TB/s) and the CPU baseline: the reference's own MatMul kernel
 (oracle/_ref, else the oracle port) timed on one host core on a 160-row slab of the same product.
+
+The line also carries `configs`: every BASELINE configuration run as one whole step (forward,
+backward, loss read back) through the C++ front-end (ctorch_amd/host) with inputs resident in HBM:
+milliseconds per step, operator launches, the launch layer's own count of algorithmic bytes and
+flops for exactly the operators that ran, the roofline fraction (time of that work at 8 TB/s /
+157.3 TFLOP/s divided by the measured time), and the reference's CPU path on one host core on a
+bounded sample of the same configuration (--no-configs skips this part).
 """
 import argparse
 import ctypes as C
@@ -82,12 +89,157 @@ def _cpu_baseline(np, support):
                       "4096^3 extrapolates to %.0f s" % (rows - 1, rows, dt, dt * M / rows)}
 
 
+HOST_LIB = os.path.join(ROOT, "ctorch_amd", "host", "libctorch_amd_host.so")
+
+
+def _timed(fn):
+    t0 = time.perf_counter()
+    fn()
+    return (time.perf_counter() - t0) * 1e3
+
+
+def config_report(with_cpu):
+    """One whole step of each BASELINE configuration through the C++ front-end, inputs resident in
+    HBM, next to the reference's CPU path on a bounded sample (one host core)."""
+    import numpy as np
+    if not os.path.exists(HOST_LIB):
+        raise RuntimeError("%s is missing: run `make -C ctorch_amd/host`" % HOST_LIB)
+    host = C.CDLL(HOST_LIB)
+    host.cth_quiet()
+    FP, L, I, D5 = C.POINTER(C.c_float), C.c_long, C.c_int, C.c_double * 5
+    fp = lambda a: a.ctypes.data_as(FP)
+    f32 = lambda a: np.ascontiguousarray(a, dtype=np.float32)
+    rng = np.random.default_rng(7)
+    uni = lambda shape, lo, hi: f32(rng.random(shape, dtype=np.float32) * (hi - lo) + lo)
+    nrm = lambda shape, sd=1.0: f32(rng.standard_normal(shape, dtype=np.float32) * sd)
+
+    ref = None
+    if with_cpu:
+        sys.path.insert(0, os.path.join(ROOT, "tests"))
+        import support
+        if support.ref_available():
+            try:
+                ref = support.Reference()
+            except (OSError, AttributeError):
+                ref = None
+        cpu_kind = "reference" if ref is not None else "port"
+        if ref is None:
+            ref = support.Oracle()
+
+    rows = []
+
+    def add(name, rc, out, cpu_ms=None, cpu_note=None, launch_bound=False):
+        if rc < 0:
+            raise RuntimeError("config step failed: " + name)
+        ms, nbytes, flops, ideal_s, launches = list(out)
+        e = {"name": name, "gpu_ms": round(ms, 4), "launches": int(round(launches)),
+             "algorithmic_GB": round(nbytes / 1e9, 4), "GFLOP": round(flops / 1e9, 3),
+             "GB/s": round(nbytes / ms / 1e6, 1), "TFLOP/s": round(flops / ms / 1e9, 2),
+             "roofline_frac": round(ideal_s * 1e3 / ms, 4)}
+        if launch_bound:
+            e["note"] = "launch-bound: tensors of a few MiB, ~%.1f us per operator launch" % (ms * 1e3 / max(launches, 1))
+        if cpu_ms is not None:
+            e["cpu_ms"] = round(cpu_ms, 1)
+            e["cpu_sample"] = cpu_note
+            e["gpu_over_cpu"] = round(cpu_ms / ms, 1)
+        rows.append(e)
+
+    # config 1: elementwise chain, n = 2^20
+    n = 1 << 20
+    a, b = uni(n, -1, 1), uni(n, -1, 1)
+    out = D5()
+    rc = host.cth_time_chain(fp(a), fp(b), L(n), I(5), I(50), out)
+    cpu = _timed(lambda: ref.chain(a, b)) if with_cpu else None
+    add("config 1: c=a*b+5, relu, sum, backward; n=2^20", rc, out, cpu, "whole step", launch_bound=True)
+
+    # config 2: MatMul forward + backward at 1024, 2048, 4096; Dot 2^26
+    slab_ms = {}
+    for Mm in (1024, 2048, 4096):
+        A, B = nrm((Mm, Mm)), nrm((Mm, Mm))
+        out = D5()
+        rc = host.cth_time_matmul(fp(A), fp(B), L(Mm), I(3), I(10), out)
+        cpu, note = None, None
+        if with_cpu:
+            r = {1024: 64, 2048: 32, 4096: 16}[Mm]
+            t = _timed(lambda: ref.matmul_t(A[:r], 0, B, 0) if cpu_kind == "reference" else ref.matmul(A[:r], B))
+            cpu = t * (Mm / r) * 3
+            note = "forward rows 0..%d (%.2f s), x%d for all rows, x3 for the two backward products" % (r - 1, t / 1e3, Mm // r)
+        add("config 2: MatMul %d^3 forward + backward (dC = ones)" % Mm, rc, out, cpu, note)
+        del A, B
+    u, v = uni(1 << 26, -1, 1), uni(1 << 26, -1, 1)
+    out = D5()
+    rc = host.cth_time_dot(fp(u), fp(v), L(1 << 26), I(3), I(20), out)
+    cpu, note = None, None
+    if with_cpu:
+        m = 1 << 24
+        t = _timed(lambda: ref.binary(5, u[:m], v[:m], ()) if cpu_kind == "reference" else ref.dot(u[:m], v[:m]))
+        cpu, note = t * 4, "first 2^24 elements, x4"
+    add("config 2: Dot, n=2^26", rc, out, cpu, note)
+    del u, v
+
+    # config 3: MLP 784-256-10 train step, batch 256 and 8192
+    W1, b1 = uni((784, 256), -1 / 28.0, 1 / 28.0), uni(256, -1 / 28.0, 1 / 28.0)
+    W2, b2 = uni((256, 10), -1 / 16.0, 1 / 16.0), uni(10, -1 / 16.0, 1 / 16.0)
+    cpu256 = None
+    for Bn in (256, 8192):
+        x = f32(rng.integers(0, 256, (Bn, 784)) / 255.0)
+        lab = f32(rng.integers(0, 10, Bn))
+        out = D5()
+        rc = host.cth_time_mlp(fp(x), L(Bn), L(784), fp(W1), fp(b1), L(256), fp(W2), fp(b2), L(10), fp(lab), I(5),
+                               I(30), out)
+        cpu, note = None, None
+        if with_cpu:
+            if Bn == 256:
+                oh = np.zeros((Bn, 10), np.float32)
+                oh[np.arange(Bn), lab.astype(int)] = 1
+                cpu256 = _timed(lambda: ref.mlp_step(x, W1, b1, W2, b2, oh) if cpu_kind == "reference"
+                                else ref.mlp_step(x, W1, b1, W2, b2, oh, False))
+                cpu, note = cpu256, "whole step (one-hot targets)"
+            else:
+                cpu, note = cpu256 * 32, "batch-256 step x32 (every operator is linear in the batch)"
+        add("config 3: MLP 784-256-10 train step, batch %d" % Bn, rc, out, cpu, note, launch_bound=(Bn == 256))
+
+    # config 4: row softmax + cross entropy, [8192 x 32000]
+    R4, C4 = 8192, 32000
+    logits = nrm((R4, C4), 2.0)
+    lab = f32(rng.integers(0, C4, R4))
+    out = D5()
+    rc = host.cth_time_softmax_ce(fp(logits), fp(lab), L(R4), L(C4), I(2), I(10), out)
+    cpu, note = None, None
+    if with_cpu:
+        r = 512
+        oh = np.zeros((r, C4), np.float32)
+        oh[np.arange(r), lab[:r].astype(int)] = 1
+        sub = np.ascontiguousarray(logits[:r])
+        t = _timed(lambda: ref.grad_loss(8, sub, oh, 1.0) if cpu_kind == "reference" else
+                   (ref.ce_onehot(sub, oh), ref.ce_bwd_onehot(sub, oh, np.float32(1.0))))
+        cpu, note = t * (R4 / r), "rows 0..%d with one-hot targets (%.2f s), x%d" % (r - 1, t / 1e3, R4 // r)
+    add("config 4: CE(sum) over logits [8192 x 32000] (class index) + backward", rc, out, cpu, note)
+    del logits
+
+    # config 5: broadcast expression + MSE + MAE, one backward
+    R5 = 4096
+    X, rv, T = uni((R5, R5), -2, 2), uni(R5, 0.5, 2), nrm((R5, R5))
+    out = D5()
+    rc = host.cth_time_expr(fp(X), fp(rv), fp(T), L(R5), L(R5), I(3), I(10), out)
+    cpu, note = None, None
+    if with_cpu:
+        r = 1024
+        Xs, Ts = np.ascontiguousarray(X[:r]), np.ascontiguousarray(T[:r])
+        Rs = np.ascontiguousarray(np.broadcast_to(rv, (r, R5)))
+        t = _timed(lambda: ref.expr(Xs, Rs, Ts))
+        cpu, note = t * (R5 / r), "rows 0..%d with the row vector materialised (%.2f s), x%d" % (r - 1, t / 1e3, R5 // r)
+    add("config 5: Y=sigmoid(X/r)-tanh(X)*sin(X)+cos(-X), MSE+MAE, backward; X [4096 x 4096]", rc, out, cpu, note)
+    return {"cores": 1, "cpu_kind": cpu_kind if with_cpu else None, "steps": rows}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-configs", action="store_true", help="skip the per-configuration report")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (every box has one); --gpus %d is not supported"
@@ -190,6 +342,17 @@ def main():
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
+    if not args.no_configs:
+        torch.cuda.empty_cache()
+        sys.stdout.flush()
+        saved = os.dup(1)           # the reference library prints to stdout; keep it off the JSON line
+        os.dup2(2, 1)
+        try:
+            out["configs"] = config_report(not args.no_cpu_baseline)
+        finally:
+            sys.stdout.flush()
+            os.dup2(saved, 1)
+            os.close(saved)
     print(json.dumps(out))
     return 0
 

@@ -79,10 +79,23 @@ def load():
         fn.argtypes = args
         fn.restype = C.c_int
     lib.ctamd_device_count.restype = C.c_int
+    lib.ctamd_counters_reset.argtypes = []
+    lib.ctamd_counters_reset.restype = None
+    lib.ctamd_counters_read.argtypes = [C.POINTER(C.c_double)] * 3 + [C.POINTER(C.c_uint64)]
+    lib.ctamd_counters_read.restype = None
     lib.ctamd_last_error.restype = C.c_char_p
     lib.ctamd_version.restype = C.c_char_p
     _lib = lib
     return lib
+
+
+def counters(lib=None):
+    """(algorithmic bytes, flops, seconds at the MI355X peaks, operator launches) since the last
+    ctamd_counters_reset()."""
+    lib = lib or load()
+    b, f, t, n = C.c_double(), C.c_double(), C.c_double(), C.c_uint64()
+    lib.ctamd_counters_read(C.byref(b), C.byref(f), C.byref(t), C.byref(n))
+    return b.value, f.value, t.value, n.value
 
 
 def check(rc):

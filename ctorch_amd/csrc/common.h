@@ -29,6 +29,11 @@ const float* pad_zero();
 // Compute units of the current device (256 on MI355X); 0 before ctamd_init().
 int compute_units();
 
+// Adds one operator launch to the per-process work counters read by ctamd_counters_read():
+// `bytes` and `flops` are the operator's algorithmic traffic and arithmetic (what it must move and
+// compute, not what the kernels happen to do).
+void account(double bytes, double flops);
+
 inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 
 // Grid for a streaming kernel: enough 256-thread blocks to cover `work_items` (each block

@@ -300,6 +300,7 @@ int launch_map(const char* name, Ptrs<F::kIn> in, float* out, size_t n, F f, voi
         unsigned grid = stream_grid(n, size_t(kThreads) * kUnroll);
         hipLaunchKernelGGL((map_kernel<F, false, false>), dim3(grid), dim3(kThreads), 0, as_stream(stream), in, out, n, f);
     }
+    account(double(F::kIn + 1) * 4.0 * double(n), 0.0);
     return launched(name);
 }
 
@@ -369,6 +370,7 @@ int launch_rowbcast(const char* name, const float* a, const float* b, float* r, 
         hipLaunchKernelGGL((rowbcast_kernel<Op, false, uint32_t, false>), dim3(grid), dim3(kThreads), 0, s, a, b, r, total, uint32_t(cols));
     else
         hipLaunchKernelGGL((rowbcast_kernel<Op, false, uint64_t, false>), dim3(grid), dim3(kThreads), 0, s, a, b, r, total, uint64_t(cols));
+    account(8.0 * double(total) + 4.0 * double(cols), 0.0);
     return launched(name);
 }
 

@@ -227,6 +227,10 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
     };
     constexpr int kMfmaPerChunk = 4 * TM * TN;
     constexpr int kStores = Stage<BM, BK, A_KC, C::THREADS>::PIECES + Stage<BN, BK, B_KC, C::THREADS>::PIECES;
+    static_assert(kMfmaPerChunk >= 2 * kStores, "a burst has room for the tile's LDS stores and global loads");
+    // LDS reads of one chunk: at most 4 per MFMA tile of an operand (32-bit reads of the
+    // X-contiguous kind, which the compiler pairs up) - slots for them, one after each leading MFMA
+    constexpr int kReadSlots = (2 * (TM + TN) < kMfmaPerChunk - kStores) ? 2 * (TM + TN) : kMfmaPerChunk - kStores;
     constexpr int kMaskMfma = 0x008, kMaskVmemRead = 0x020, kMaskDsRead = 0x100, kMaskDsWrite = 0x200;
 
     // Software pipeline over the two 8-wide k chunks of a k tile, two fragment buffers:
@@ -259,11 +263,12 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
             sa.store(s_a[cur ^ 1], A_STRIDE);
             sb.store(s_b[cur ^ 1], B_STRIDE);
 #pragma unroll
-            for (int q = 0; q < 12; ++q) {
+            for (int q = 0; q < kReadSlots; ++q) {
                 __builtin_amdgcn_sched_group_barrier(kMaskMfma, 1, 0);
                 __builtin_amdgcn_sched_group_barrier(kMaskDsRead, 1, 0);
             }
-            __builtin_amdgcn_sched_group_barrier(kMaskMfma, kMfmaPerChunk - 12 - kStores, 0);
+            if (kMfmaPerChunk - kReadSlots - kStores > 0)
+                __builtin_amdgcn_sched_group_barrier(kMaskMfma, kMfmaPerChunk - kReadSlots - kStores, 0);
 #pragma unroll
             for (int q = 0; q < kStores; ++q) {
                 __builtin_amdgcn_sched_group_barrier(kMaskMfma, 1, 0);
@@ -278,7 +283,7 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
             sb.load_fast(more ? b_step : 0);
             mfmas(1);
 #pragma unroll
-            for (int q = 0; q < 12; ++q) {
+            for (int q = 0; q < kReadSlots; ++q) {
                 __builtin_amdgcn_sched_group_barrier(kMaskMfma, 1, 1);
                 __builtin_amdgcn_sched_group_barrier(kMaskDsRead, 1, 1);
             }
@@ -287,7 +292,8 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
                 __builtin_amdgcn_sched_group_barrier(kMaskMfma, 1, 1);
                 __builtin_amdgcn_sched_group_barrier(kMaskVmemRead, 1, 1);
             }
-            __builtin_amdgcn_sched_group_barrier(kMaskMfma, kMfmaPerChunk - 12 - kStores, 1);
+            if (kMfmaPerChunk - kReadSlots - kStores > 0)
+                __builtin_amdgcn_sched_group_barrier(kMaskMfma, kMfmaPerChunk - kReadSlots - kStores, 1);
             __builtin_amdgcn_sched_barrier(0);
         }
     } else {
@@ -345,13 +351,30 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
 }
 
 // Folds the K-split partial products: c[i] = sum_z partial[z][i], in order of z.
+template <bool VEC>
 __global__ __launch_bounds__(kThreads) void splitk_fold(const float* __restrict__ partial, float* __restrict__ c,
                                                         size_t mn, int splits) {
     size_t i = size_t(blockIdx.x) * kThreads + threadIdx.x;
-    if (i >= mn) return;
-    float t = partial[i];
-    for (int z = 1; z < splits; ++z) t += partial[size_t(z) * mn + i];
-    c[i] = t;
+    if (VEC) {
+        if (i >= mn / 4) return;
+        const v4f* __restrict__ p = reinterpret_cast<const v4f*>(partial);
+        const size_t stride = mn / 4;
+        v4f t = p[i];
+        int z = 1;
+        for (; z + 3 < splits; z += 4) {       // four loads in flight, added in order of z
+            v4f a = p[size_t(z) * stride + i], b = p[size_t(z + 1) * stride + i];
+            v4f d = p[size_t(z + 2) * stride + i], e = p[size_t(z + 3) * stride + i];
+            t = ((t + a) + b) + d;
+            t = t + e;
+        }
+        for (; z < splits; ++z) t = t + p[size_t(z) * stride + i];
+        reinterpret_cast<v4f*>(c)[i] = t;
+    } else {
+        if (i >= mn) return;
+        float t = partial[i];
+        for (int z = 1; z < splits; ++z) t += partial[size_t(z) * mn + i];
+        c[i] = t;
+    }
 }
 
 // Operands with no unit stride: one thread per output element.  Correct for any strides; only
@@ -367,12 +390,16 @@ __global__ __launch_bounds__(kThreads) void gemm_strided(const float* __restrict
     c[idx] = s;
 }
 
-// Two tile shapes.  Big: 256 x 256 x 16 with 8 waves (each 128 x 64, 128 accumulator registers, two
-// waves per SIMD) - the fewest LDS and global bytes per flop, 134-137 TFLOP/s at 4096^3 against
-// 122-124 for the small tile; it needs about one tile per CU to fill the chip.  Small:
-// 128 x 128 x 16 with 4 waves (each 64 x 64) for everything else (113 against 109 TFLOP/s at 2048^3).
+// Three tile shapes; the host picks the largest one that still gives every CU a tile.
+//   Big   256 x 256 x 16, 8 waves of 128 x 64 (128 accumulator registers, two waves per SIMD): the
+//         fewest LDS and global bytes per flop; 4096^3 in 0.95-0.98 ms (140-145 TFLOP/s).
+//   Small 128 x 128 x 16, 4 waves of 64 x 64: 2048^3 in 0.135 ms (127 TFLOP/s).
+//   Tiny  64 x 64 x 16, 4 waves of 32 x 32, up to 8 blocks per CU: 1024^3 in 27 us (78 TFLOP/s) and
+//         the skinny products of a small layer ([8192 x 784] . [784 x 256] in 32 us); with a K split
+//         when even these tiles are fewer than the CUs ([784 x 8192] . [8192 x 256] in 50 us).
 using BigTile = Cfg<256, 256, 16, 128, 64>;
 using SmallTile = Cfg<128, 128, 16, 64, 64>;
+using TinyTile = Cfg<64, 64, 16, 32, 32>;
 
 template <class Tile, bool A_KC, bool B_KC>
 int launch_gemm(GemmArgs g, bool vec, int splits, hipStream_t s) {
@@ -406,6 +433,7 @@ extern "C" int ctamd_matmul_f32(const float* a, int64_t as0, int64_t as1, const 
     if (!a || !b) return fail(CTAMD_EINVAL, "%s: null input", __func__);
     if (as0 < 0 || as1 < 0 || bs0 < 0 || bs1 < 0) return fail(CTAMD_EINVAL, "%s: negative stride", __func__);
     hipStream_t s = as_stream(stream);
+    account(4.0 * (double(m) * double(k) + double(k) * double(n) + double(m) * double(n)), 2.0 * double(m) * double(n) * double(k));
 
     // a one-row / one-column operand is contiguous in whichever direction has extent > 1
     const bool a_kc = (as1 == 1) || (k == 1 && as0 != 1), a_xc = (as0 == 1) || (m == 1);
@@ -417,11 +445,13 @@ extern "C" int ctamd_matmul_f32(const float* a, int64_t as0, int64_t as1, const 
     }
     const bool A_KC = a_kc, B_KC = !b_xc;
     const int cus = compute_units() > 0 ? compute_units() : 256;
-    const int64_t big_tiles = ((m + BigTile::BM - 1) / BigTile::BM) * ((n + BigTile::BN - 1) / BigTile::BN);
-    const bool big = big_tiles >= cus;
-    const int BM = big ? BigTile::BM : SmallTile::BM, BN = big ? BigTile::BN : SmallTile::BN;
-    const int BK = big ? BigTile::BK : SmallTile::BK;
-    
+    auto tiles_of = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
+    // the largest tile shape that still gives every CU a tile; below that the smallest shape
+    int shape = tiles_of(BigTile::BM, BigTile::BN) >= cus ? 2 : tiles_of(SmallTile::BM, SmallTile::BN) >= cus ? 1 : 0;
+    const int BM = shape == 2 ? BigTile::BM : shape == 1 ? SmallTile::BM : TinyTile::BM;
+    const int BN = shape == 2 ? BigTile::BN : shape == 1 ? SmallTile::BN : TinyTile::BN;
+    constexpr int BK = 16;
+    static_assert(BigTile::BK == BK && SmallTile::BK == BK && TinyTile::BK == BK, "all tile shapes step K alike");
     GemmArgs g;
     g.a = a; g.lda = A_KC ? as0 : as1;
     g.b = b; g.ldb = B_KC ? bs1 : bs0;
@@ -435,8 +465,9 @@ extern "C" int ctamd_matmul_f32(const float* a, int64_t as0, int64_t as1, const 
     const int64_t tiles = int64_t(g.tiles_m) * g.tiles_n;
     float* partial = nullptr;
     if (tiles < cus && k >= 8 * BK) {
-        int64_t want = (2 * cus + tiles - 1) / tiles;
-        int64_t max_by_k = k / (4 * BK);
+        // enough blocks for four per CU (they are co-resident), but at least 8 k tiles per block
+        int64_t want = (4 * cus + tiles - 1) / tiles;
+        int64_t max_by_k = k / (8 * BK);
         int64_t max_by_scratch = int64_t(kScratchFloats) / (m * n);
         splits = int(want < max_by_k ? want : max_by_k);
         if (splits > max_by_scratch) splits = int(max_by_scratch);
@@ -454,11 +485,16 @@ extern "C" int ctamd_matmul_f32(const float* a, int64_t as0, int64_t as1, const 
     if (splits > 1) { g.c = partial; g.ldc = n; g.split_stride = m * n; }
     else { g.c = c; g.ldc = n; g.split_stride = 0; }
 
-    int rc = big ? launch_layout<BigTile>(g, A_KC, B_KC, vec, splits, s)
-                 : launch_layout<SmallTile>(g, A_KC, B_KC, vec, splits, s);
+    int rc = shape == 2 ? launch_layout<BigTile>(g, A_KC, B_KC, vec, splits, s)
+           : shape == 1 ? launch_layout<SmallTile>(g, A_KC, B_KC, vec, splits, s)
+                        : launch_layout<TinyTile>(g, A_KC, B_KC, vec, splits, s);
     if (rc || splits == 1) return rc;
     size_t mn = size_t(m) * size_t(n);
-    hipLaunchKernelGGL(splitk_fold, dim3(unsigned((mn + kThreads - 1) / kThreads)), dim3(kThreads), 0, s, partial, c, mn,
-                       splits);
+    if (mn % 4 == 0 && aligned16(c))
+        hipLaunchKernelGGL(splitk_fold<true>, dim3(unsigned((mn / 4 + kThreads - 1) / kThreads)), dim3(kThreads), 0, s,
+                           partial, c, mn, splits);
+    else
+        hipLaunchKernelGGL(splitk_fold<false>, dim3(unsigned((mn + kThreads - 1) / kThreads)), dim3(kThreads), 0, s,
+                           partial, c, mn, splits);
     return launched(__func__);
 }

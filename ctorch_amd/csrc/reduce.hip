@@ -133,6 +133,7 @@ int reduce(const char* name, const float* a, const float* b, float* out, int32_t
         if (rc) return rc;
     }
     hipLaunchKernelGGL(reduce_stage2, dim3(1), dim3(kThreads), 0, s, partials, grid, out, flag, mode, float(n));
+    account(double(T::kIn) * 4.0 * double(n), T::kIn == 2 ? 2.0 * double(n) : double(n));
     return launched(name);
 }
 
@@ -290,6 +291,7 @@ int ctamd_colsum_f32(const float* g, float* out, size_t rows, size_t cols, void*
     constexpr size_t kFoldCols = kThreads / kFoldLanes;
     hipLaunchKernelGGL(colsum_stage2, dim3((unsigned)((cols + kFoldCols - 1) / kFoldCols)), dim3(kThreads), 0, s, partials,
                        out, cols, (unsigned)chunks);
+    account(4.0 * double(rows) * double(cols), double(rows) * double(cols));
     return launched(__func__);
 }
 

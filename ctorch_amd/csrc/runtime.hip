@@ -15,7 +15,24 @@ constexpr int kMaxDevices = 16;
 std::mutex g_mu;
 float* g_scratch[kMaxDevices] = {};
 int g_cus[kMaxDevices] = {};
+
+// Work counters (per process): what the operators launched since the last reset had to move and
+// compute, and the time that work takes at the published peaks.
+std::mutex g_count_mu;
+double g_bytes = 0.0, g_flops = 0.0, g_ideal_s = 0.0;
+uint64_t g_launches = 0;
+constexpr double kHbmBytesPerS = 8.0e12;        // MI355X HBM3E
+constexpr double kMfmaF32FlopPerS = 157.3e12;   // MI355X dense fp32 matrix
 }  // namespace
+
+void account(double bytes, double flops) {
+    std::lock_guard<std::mutex> lock(g_count_mu);
+    g_bytes += bytes;
+    g_flops += flops;
+    const double tb = bytes / kHbmBytesPerS, tf = flops / kMfmaF32FlopPerS;
+    g_ideal_s += tb > tf ? tb : tf;
+    ++g_launches;
+}
 
 int fail(int code, const char* fmt, ...) {
     va_list ap;
@@ -107,6 +124,19 @@ int ctamd_init(int device) {
 }
 
 const char* ctamd_last_error(void) { return g_err; }
+void ctamd_counters_reset(void) {
+    std::lock_guard<std::mutex> lock(g_count_mu);
+    g_bytes = g_flops = g_ideal_s = 0.0;
+    g_launches = 0;
+}
+void ctamd_counters_read(double* bytes, double* flops, double* roofline_seconds, uint64_t* launches) {
+    std::lock_guard<std::mutex> lock(g_count_mu);
+    if (bytes) *bytes = g_bytes;
+    if (flops) *flops = g_flops;
+    if (roofline_seconds) *roofline_seconds = g_ideal_s;
+    if (launches) *launches = g_launches;
+}
+
 const char* ctamd_version(void) { return "ctorch_amd 0.1 (gfx950)"; }
 
 int ctamd_malloc(void** ptr, size_t bytes) {

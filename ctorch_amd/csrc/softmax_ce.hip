@@ -530,6 +530,15 @@ int run_rows(const char* name, Args a, float* loss_out, void* stream) {
     a.pad_neg_inf = pad_neg_inf();
     a.pad_zero = pad_zero();
     if (!a.pad_zero) return CTAMD_EINVAL;
+    {
+        // algorithmic bytes per element: logits in (+ one-hot target in) (+ result out); a class
+        // index adds 4 bytes per row; one exp per element
+        const double n = double(a.rows) * double(a.cols);
+        const double per = MODE == kSoftmax ? 8.0 : MODE == kCeIndex ? 4.0 : MODE == kCeOnehot ? 8.0
+                         : MODE == kCeBwdIndex ? 8.0 : 12.0;   // kCeBwdOnehot, kSoftmaxBwd: two inputs, one output
+        const bool index = (MODE == kCeIndex || MODE == kCeBwdIndex);
+        account(per * n + (index ? 4.0 * double(a.rows) : 0.0), n);
+    }
     if (kLoss) a.partials = reinterpret_cast<double*>(scratch());
     // rows are dealt to a chip-filling number of blocks (each walks several rows, prefetching the next)
     const size_t groups = (a.cols + 3) / 4;
@@ -635,6 +644,7 @@ int ctamd_softmax_cols_f32(const float* x, float* y, size_t rows, size_t cols, v
     if (!x || !y) return fail(CTAMD_EINVAL, "%s: null pointer", __func__);
     hipLaunchKernelGGL(softmax_cols_kernel, dim3((unsigned)((cols + 255) / 256)), dim3(256), 0, as_stream(stream), x, y,
                        rows, cols);
+    account(8.0 * double(rows) * double(cols), double(rows) * double(cols));
     return launched(__func__);
 }
 int ctamd_softmax_backward_cols_f32(const float* y, const float* g, float* dx, size_t rows, size_t cols, void* stream) {
@@ -642,6 +652,7 @@ int ctamd_softmax_backward_cols_f32(const float* y, const float* g, float* dx, s
     if (!y || !g || !dx) return fail(CTAMD_EINVAL, "%s: null pointer", __func__);
     hipLaunchKernelGGL(softmax_bwd_cols_kernel, dim3((unsigned)((cols + 255) / 256)), dim3(256), 0, as_stream(stream), y,
                        g, dx, rows, cols);
+    account(12.0 * double(rows) * double(cols), 2.0 * double(rows) * double(cols));
     return launched(__func__);
 }
 

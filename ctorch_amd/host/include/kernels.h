@@ -36,8 +36,10 @@ Tensor scalar_op(const Tensor& a, float s, op which);                 // a + s, 
 Tensor sum_all(const Tensor& a);
 Tensor softmax_dim(const Tensor& a, int dim);                         // dim already normalised
 Tensor filled(const std::vector<size_t>& shape, float v, DeviceType device);
+void fill_scalar(Tensor& t, float v);                                  // every element of a device tensor = v
 Tensor filled_from(const std::vector<size_t>& shape, const Tensor& scalar0d);
 void accumulate(Tensor& grad, const Tensor& val);                     // grad += val
+Tensor zero_plus(const Tensor& val, const std::vector<size_t>& shape); // a fresh gradient: 0 + val
 Tensor column_sum(const Tensor& g);                                   // [rows, cols] -> [cols]
 Tensor first_row(const Tensor& g);                                    // [rows, cols] -> [cols], row 0
 bool any_abs_lt_eps(const Tensor& b);

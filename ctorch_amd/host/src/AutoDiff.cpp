@@ -253,11 +253,12 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
             size_t input_id = node->input_ids[pos];
             Node* in = find(input_id);
             if (!in || !in->requires_grad) continue;
-            if (!in->grad)
-                in->grad = std::make_unique<Tensor>(ShapeTag{}, in->tensor->sizes(), in->tensor->dtype(), in->tensor->device());
             Tensor val = input_gradient(node, input_id, pos, node_grad);
             Tensor adj = adjust_grad_shape(val, in->tensor->sizes());
-            accumulate(*in->grad, adj);                                  // :1870-1907
+            // :1870-1907: a zero-filled gradient, then grad += val; the first contribution does
+            // both in one pass
+            if (!in->grad) in->grad = std::make_unique<Tensor>(zero_plus(adj, in->tensor->sizes()));
+            else accumulate(*in->grad, adj);
         }
     }
 }

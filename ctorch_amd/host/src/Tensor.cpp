@@ -24,9 +24,13 @@ Tensor::Tensor(float value) : tensor_id_(global_tensor_id++), _storage(&value, 1
     computeStrides();
 }
 
+// On the device the value is written by a one-element fill launch: a host-to-device copy would
+// drain the stream first (every `tensor + 5.0f` and every backward() makes one of these).
 Tensor::Tensor(float value, DeviceType device)
-    : tensor_id_(global_tensor_id++), _device(device), _storage(&value, 1, DType::kFloat, device) {
+    : tensor_id_(global_tensor_id++), _device(device),
+      _storage(device == DeviceType::kAMD ? Storage(1, DType::kFloat, device) : Storage(&value, 1, DType::kFloat, device)) {
     computeStrides();
+    if (device == DeviceType::kAMD) fill_scalar(*this, value);
 }
 
 Tensor::Tensor(std::initializer_list<float> values)

@@ -8,6 +8,9 @@
 #include "Ctorch_Error.h"
 #include "Ctorch_Scheduler.h"
 
+#include "ctorch_amd.h"
+
+#include <chrono>
 #include <cstring>
 #include <vector>
 
@@ -308,6 +311,142 @@ long cth_expr(const float* X, const float* R, const float* T, long rows, long co
     } catch (const std::exception&) {
         return -1;
     }
+}
+
+// ------------------------------------------------------------------------- timed steps
+// The same graphs as above with every input resident in HBM before the clock starts: `warm`
+// untimed steps, then `reps` timed ones between two device synchronisations.  A step builds its
+// own tape, runs forward and backward through the front-end and reads the loss back (the one
+// host read a training step makes).  out[0] = milliseconds per step, out[1..4] = the launch
+// layer's work counters per step: algorithmic bytes, flops, seconds at the MI355X peaks, operator
+// launches.
+}  // extern "C"
+namespace {
+template <class Step>
+long time_steps(Step step, int warm, int reps, double* out) {
+    try {
+        for (int i = 0; i < warm; ++i) step();
+        ctamd_sync(nullptr);
+        ctamd_counters_reset();
+        auto t0 = std::chrono::steady_clock::now();
+        for (int i = 0; i < reps; ++i) step();
+        ctamd_sync(nullptr);
+        auto t1 = std::chrono::steady_clock::now();
+        double bytes = 0, flops = 0, ideal = 0;
+        uint64_t launches = 0;
+        ctamd_counters_read(&bytes, &flops, &ideal, &launches);
+        out[0] = std::chrono::duration<double, std::milli>(t1 - t0).count() / reps;
+        out[1] = bytes / reps;
+        out[2] = flops / reps;
+        out[3] = ideal / reps;
+        out[4] = double(launches) / reps;
+        return reps;
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+}  // namespace
+extern "C" {
+
+long cth_time_chain(const float* a, const float* b, long n, int warm, int reps, double* out) {
+    long d1[1] = {n};
+    Tensor ta = make(a, d1, 1), tb = make(b, d1, 1);
+    volatile float sink = 0;
+    return time_steps([&] {
+        AutoDiff ctx;
+        configure(ctx);
+        AutoDiffContext::Guard guard(&ctx);
+        ta.requires_grad(true);
+        tb.requires_grad(true);
+        Tensor s = ((ta * tb + 5.0f).relu()).sum();
+        sink = s.item<float>();
+        s.backward();
+        Tensor ga = grad(ta), gb = grad(tb);
+    }, warm, reps, out);
+}
+
+// C = A . B, L = C.sum(), backward: dC = ones, dA = dC . B^T, dB = A^T . dC.
+long cth_time_matmul(const float* A, const float* B, long M, int warm, int reps, double* out) {
+    long d[2] = {M, M};
+    Tensor tA = make(A, d, 2), tB = make(B, d, 2);
+    volatile float sink = 0;
+    return time_steps([&] {
+        AutoDiff ctx;
+        configure(ctx);
+        AutoDiffContext::Guard guard(&ctx);
+        tA.requires_grad(true);
+        tB.requires_grad(true);
+        Tensor L = tA.matmul(tB).sum();
+        sink = L.item<float>();
+        backward(L);
+        Tensor ga = grad(tA), gb = grad(tB);
+    }, warm, reps, out);
+}
+
+long cth_time_dot(const float* a, const float* b, long n, int warm, int reps, double* out) {
+    long d1[1] = {n};
+    Tensor ta = make(a, d1, 1), tb = make(b, d1, 1);
+    volatile float sink = 0;
+    return time_steps([&] { sink = ta.dot(tb).item<float>(); }, warm, reps, out);
+}
+
+long cth_time_mlp(const float* x, long B, long I, const float* W1, const float* b1, long H, const float* W2,
+                  const float* b2, long C, const float* labels, int warm, int reps, double* out) {
+    long xd[2] = {B, I}, w1d[2] = {I, H}, b1d[1] = {H}, w2d[2] = {H, C}, b2d[1] = {C}, yi[1] = {B};
+    Tensor tx = make(x, xd, 2), tW1 = make(W1, w1d, 2), tb1 = make(b1, b1d, 1), tW2 = make(W2, w2d, 2),
+           tb2 = make(b2, b2d, 1), ty = make(labels, yi, 1);
+    volatile float sink = 0;
+    return time_steps([&] {
+        AutoDiff ctx;
+        configure(ctx);
+        AutoDiffContext::Guard guard(&ctx);
+        tW1.requires_grad(true);
+        tb1.requires_grad(true);
+        tW2.requires_grad(true);
+        tb2.requires_grad(true);
+        Tensor h = (tx.matmul(tW1) + tb1).relu();
+        Tensor loss = (h.matmul(tW2) + tb2).cross_entropy(ty);
+        sink = loss.item<float>();
+        backward(loss);
+        Tensor g1 = grad(tW1), g2 = grad(tb1), g3 = grad(tW2), g4 = grad(tb2);
+    }, warm, reps, out);
+}
+
+// loss_sum = CE(logits, class index), backward: dlogits = softmax - onehot.
+long cth_time_softmax_ce(const float* logits, const float* labels, long rows, long cols, int warm, int reps,
+                         double* out) {
+    long d[2] = {rows, cols}, yi[1] = {rows};
+    Tensor tx = make(logits, d, 2), ty = make(labels, yi, 1);
+    volatile float sink = 0;
+    return time_steps([&] {
+        AutoDiff ctx;
+        configure(ctx);
+        AutoDiffContext::Guard guard(&ctx);
+        tx.requires_grad(true);
+        Tensor loss = tx.cross_entropy(ty);
+        sink = loss.item<float>() / float(rows);
+        backward(loss);
+        Tensor g = grad(tx);
+    }, warm, reps, out);
+}
+
+long cth_time_expr(const float* X, const float* R, const float* T, long rows, long cols, int warm, int reps,
+                   double* out) {
+    long d[2] = {rows, cols}, dv[1] = {cols};
+    Tensor tX = make(X, d, 2), tR = make(R, dv, 1), tT = make(T, d, 2);
+    volatile float sink = 0;
+    return time_steps([&] {
+        AutoDiff ctx;
+        configure(ctx);
+        AutoDiffContext::Guard guard(&ctx);
+        tX.requires_grad(true);
+        tR.requires_grad(true);
+        Tensor Y = (tX / tR).sigmoid() - tX.tanh() * tX.sin() + (-tX).cos();
+        Tensor L = Y.mse_loss(tT) + Y.mae_loss(tT);
+        sink = L.item<float>();
+        backward(L);
+        Tensor gX = grad(tX), gR = grad(tR);
+    }, warm, reps, out);
 }
 
 }  // extern "C"

@@ -134,6 +134,10 @@ Tensor filled(const std::vector<size_t>& shape, float v, DeviceType device) {
     else for (size_t i = 0; i < r.numel(); ++i) r.data<float>()[i] = v;
     return r;
 }
+void fill_scalar(Tensor& t, float v) {
+    check_device(t, "fill");
+    run(ctamd_fill_f32(t.fptr(), v, t.numel(), nullptr), "fill");
+}
 Tensor filled_from(const std::vector<size_t>& shape, const Tensor& s) {
     check_device(s, "fill");
     Tensor r(ShapeTag{}, shape, DType::kFloat, DeviceType::kAMD, false);
@@ -146,6 +150,16 @@ void accumulate(Tensor& grad, const Tensor& val) {
     if (grad.numel() != val.numel())
         Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "accumulate: gradient sizes differ");
     run(ctamd_accumulate_f32(grad.fptr(), val.fptr(), grad.numel(), nullptr), "accumulate");
+}
+// grad = 0 + val in one pass: what the reference's "zero-filled gradient, then grad[i] += val[i]"
+// (src/AutoDiff.cpp:1870-1907) leaves after the first contribution, bit for bit (-0 becomes +0).
+Tensor zero_plus(const Tensor& val, const std::vector<size_t>& shape) {
+    check_device(val, "accumulate");
+    Tensor r(ShapeTag{}, shape, DType::kFloat, DeviceType::kAMD, false);
+    if (r.numel() != val.numel())
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "accumulate: gradient sizes differ");
+    run(ctamd_add_scalar_f32(val.fptr(), 0.0f, r.fptr(), r.numel(), nullptr), "accumulate");
+    return r;
 }
 Tensor column_sum(const Tensor& g) {
     check_device(g, "column_sum");

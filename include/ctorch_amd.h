@@ -54,6 +54,15 @@ int ctamd_memcpy_d2h(void* dst_host, const void* src, size_t bytes, void* stream
 int ctamd_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream);
 int ctamd_sync(void* stream);
 
+/* Work counters, a measurement aid with no counterpart in the reference.  Every operator entry
+ * point below adds its algorithmic HBM bytes and flops (what the operator must move and compute:
+ * e.g. 12 bytes per element for r = a + b, 2*m*n*k flops for MatMul), and
+ * max(bytes / 8 TB/s, flops / 157.3 TFLOP/s), the time that work takes at the MI355X peaks, to
+ * per-process totals.  roofline_seconds / measured seconds is the roofline fraction of whatever
+ * sequence of operators ran between a reset and a read.  Any pointer may be NULL. */
+void ctamd_counters_reset(void);
+void ctamd_counters_read(double* bytes, double* flops, double* roofline_seconds, uint64_t* launches);
+
 /* -------------------------------------------------------- elementwise binary (bit-exact) */
 /* r[i] = a[i] (op) b[i].  Add_BASIC_kernel.cpp:64-69, Sub_BASIC_kernel.cpp:58-60,
  * Mul_BASIC_kernel.cpp:59-61, Div_BASIC_kernel.cpp:37-45 (IEEE quotient, also for b == 0). */

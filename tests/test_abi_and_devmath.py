@@ -26,7 +26,8 @@ def test_library_exports_every_declared_entry_point():
     assert len(names) >= 55
     for n in names:
         assert hasattr(lib, n), n
-    untyped = {"ctamd_device_count", "ctamd_last_error", "ctamd_version"}
+    untyped = {"ctamd_device_count", "ctamd_last_error", "ctamd_version", "ctamd_counters_reset",
+               "ctamd_counters_read"}
     assert set(names) - untyped == set(capi.PROTOTYPES), set(names) ^ set(capi.PROTOTYPES)
     assert b"gfx950" in lib.ctamd_version()
 
