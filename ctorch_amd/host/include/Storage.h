@@ -89,6 +89,8 @@ class Storage {
     // untyped pointer in the storage's own address space (HBM for kAMD); for the launch layer
     void* raw() { return _data.get(); }
     const void* raw() const { return _data.get(); }
+    // true while another Storage object (a view, an alias) refers to the same bytes
+    bool shared() const { return _data.use_count() > 1; }
 
     size_t size() const { return _size; }
     DType dtype() const { return _dtype; }

@@ -82,6 +82,7 @@ class Tensor {
     template <typename T>
     T* data() { return _storage.data<T>() + _storage_offset; }
     // fp32 pointer in the tensor's own address space (HBM for kAMD), offset applied
+    bool storage_shared() const { return _storage.shared(); }
     const float* fptr() const { return static_cast<const float*>(_storage.raw()) + _storage_offset; }
     float* fptr() { return static_cast<float*>(_storage.raw()) + _storage_offset; }
     template <typename T>

@@ -39,7 +39,8 @@ Tensor filled(const std::vector<size_t>& shape, float v, DeviceType device);
 void fill_scalar(Tensor& t, float v);                                  // every element of a device tensor = v
 Tensor filled_from(const std::vector<size_t>& shape, const Tensor& scalar0d);
 void accumulate(Tensor& grad, const Tensor& val);                     // grad += val
-Tensor zero_plus(const Tensor& val, const std::vector<size_t>& shape); // a fresh gradient: 0 + val
+Tensor zero_plus(const Tensor& val, const std::vector<size_t>& shape); // a fresh tensor: 0 + val
+Tensor sum_of(const Tensor& a, const Tensor& b);                       // a fresh tensor: a + b, a's shape
 Tensor column_sum(const Tensor& g);                                   // [rows, cols] -> [cols]
 Tensor first_row(const Tensor& g);                                    // [rows, cols] -> [cols], row 0
 bool any_abs_lt_eps(const Tensor& b);

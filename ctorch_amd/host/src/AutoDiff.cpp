@@ -49,7 +49,8 @@ void AutoDiff::zero_grad(Tensor& t) {
     if (t.id() == 0) return;
     std::lock_guard<std::mutex> lock(records_mutex);
     Node* n = find(t.id());
-    if (n && n->grad) n->grad->zero();
+    // a fresh zero tensor: the stored gradient may share its bytes with another node's
+    if (n && n->grad) n->grad = std::make_unique<Tensor>(ShapeTag{}, n->grad->sizes(), n->grad->dtype(), n->grad->device());
 }
 
 // src/AutoDiff.cpp:86-243: a copy of the stored gradient, or zeros of the tensor's shape
@@ -57,7 +58,7 @@ Tensor AutoDiff::get_grad(const Tensor* t) {
     if (!t || t->id() == 0) return Tensor();
     std::lock_guard<std::mutex> lock(records_mutex);
     Node* n = find(t->id());
-    if (n && n->requires_grad && n->grad) return Tensor(*n->grad);
+    if (n && n->requires_grad && n->grad) return zero_plus(*n->grad, n->grad->sizes());   // the copy, and the pending "0 +"
     return Tensor(ShapeTag{}, t->shape(), t->dtype(), t->device());
 }
 
@@ -255,10 +256,20 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
             if (!in || !in->requires_grad) continue;
             Tensor val = input_gradient(node, input_id, pos, node_grad);
             Tensor adj = adjust_grad_shape(val, in->tensor->sizes());
-            // :1870-1907: a zero-filled gradient, then grad += val; the first contribution does
-            // both in one pass
-            if (!in->grad) in->grad = std::make_unique<Tensor>(zero_plus(adj, in->tensor->sizes()));
-            else accumulate(*in->grad, adj);
+            // :1870-1907 is "zero-filled gradient, then grad += val".  Here the first contribution
+            // is kept as it is (no pass over memory; it may share its bytes with another node's
+            // gradient) and the "0 +" is applied when the gradient is read (get_grad): adding +0
+            // only turns -0 into +0, and the sign of a zero in an upstream gradient cannot change
+            // any non-zero value downstream.  Later contributions add in place once the bytes are
+            // this node's own, else into a fresh tensor.
+            if (!in->grad) {
+                if (adj.sizes() == in->tensor->sizes()) in->grad = std::make_unique<Tensor>(Tensor::alias(adj));
+                else in->grad = std::make_unique<Tensor>(zero_plus(adj, in->tensor->sizes()));
+            } else if (in->grad->storage_shared()) {
+                in->grad = std::make_unique<Tensor>(sum_of(*in->grad, adj));
+            } else {
+                accumulate(*in->grad, adj);
+            }
         }
     }
 }

@@ -161,6 +161,15 @@ Tensor zero_plus(const Tensor& val, const std::vector<size_t>& shape) {
     run(ctamd_add_scalar_f32(val.fptr(), 0.0f, r.fptr(), r.numel(), nullptr), "accumulate");
     return r;
 }
+Tensor sum_of(const Tensor& a, const Tensor& b) {
+    check_device(a, "accumulate");
+    check_device(b, "accumulate");
+    if (a.numel() != b.numel())
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "accumulate: gradient sizes differ");
+    Tensor r = like(a);
+    run(ctamd_add_f32(a.fptr(), b.fptr(), r.fptr(), r.numel(), nullptr), "accumulate");
+    return r;
+}
 Tensor column_sum(const Tensor& g) {
     check_device(g, "column_sum");
     Tensor r(ShapeTag{}, {g.sizes()[1]}, DType::kFloat, DeviceType::kAMD, false);
