@@ -545,6 +545,158 @@ void co_mlp_step(const float* x, long B, long I, const float* W1, const float* b
     free(cs);
 }
 
+/* ---- the MNIST demo's path: loader arithmetic, targets, optimiser step, accuracy, train loop.
+ * mnist/mnist.cpp and mnist/mnist_loader.cpp are built by the reference WITHOUT the library's
+ * -O3 -march=native (CMakeLists.txt:56, :65-86 set those on the CTorch target only), so their own
+ * arithmetic is plain IEEE, one rounding per operation: no FMA in the optimiser update. */
+
+/* mnist/mnist_loader.cpp:35-41: pixel / 255.0f */
+void co_u8_to_unit(const unsigned char* src, float* dst, long n) {
+    for (long i = 0; i < n; ++i) dst[i] = (float)src[i] / 255.0f;
+}
+
+/* mnist/mnist.cpp:72-78: out[i, j] = (j == int(label_i)) ? 1 : 0 */
+void co_onehot(const float* labels, float* out, long rows, long classes) {
+    for (long i = 0; i < rows; ++i) {
+        int lab = (int)labels[i];
+        for (long j = 0; j < classes; ++j) out[i * classes + j] = (j == lab) ? 1.0f : 0.0f;
+    }
+}
+
+/* mnist/mnist.cpp:86-92: p[i] -= g[i] * lr, product rounded, then the difference rounded */
+void co_sgd_step(float* p, const float* g, float lr, long n) {
+    for (long i = 0; i < n; ++i) {
+        float step = g[i] * lr;
+        p[i] = p[i] - step;
+    }
+}
+
+/* mnist/mnist.cpp:134-156: per row the first index whose value exceeds every earlier one,
+ * starting from -1.0f at index 0; counted when it equals int(label). */
+long co_count_correct(const float* pred, const float* labels, long rows, long classes) {
+    long correct = 0;
+    for (long i = 0; i < rows; ++i) {
+        int best = 0;
+        float mx = -1.0f;
+        for (long j = 0; j < classes; ++j) {
+            float v = pred[i * classes + j];
+            if (v > mx) {
+                mx = v;
+                best = (int)j;
+            }
+        }
+        if (best == (int)labels[i]) ++correct;
+    }
+    return correct;
+}
+
+/* mnist/mnist.cpp:15-93 (the model and train_step) and :244-265 (the batch loop), `steps`
+ * consecutive batches of `batch` rows, batch index = step % (n_images / batch) (:233, :252):
+ *   logits = relu(relu(x W1 + b1) W2 + b2) W3 + b3; loss = CE_sum(logits, onehot); backward;
+ *   every parameter p -= grad * lr.
+ * Two properties of the reference's tape decide the bits (both reproduced when the flag is set,
+ * both pinned against the built reference in tests/test_oracle_vs_ref.py):
+ *   strict_row0     the gradient of a bias is row 0 of the upstream gradient
+ *                   (src/AutoDiff.cpp:690-757), not the column sum;
+ *   stale_snapshot  a leaf's node holds the deep copy made when the leaf was first seen
+ *                   (src/AutoDiff.cpp:265-278 returns early for a known id) and MatMul's backward
+ *                   reads operands from the nodes (:1692-1704), so the gradients that flow back
+ *                   through W2 and W3 use the weights of the FIRST step, while the forward pass
+ *                   and the weight gradients themselves use live values.
+ * With both flags 0 this is plain SGD with column-sum bias gradients (rounded from double).
+ * Parameters are updated in place; losses[s] is the loss of step s. */
+void co_mnist_train(const float* images, const float* labels, long n_images, long I, long H1, long H2,
+                    long C, float* W1, float* b1, float* W2, float* b2, float* W3, float* b3, long batch,
+                    long steps, float lr, int strict_row0, int stale_snapshot, float* losses) {
+    const long B = batch, nb = n_images / batch;
+    long big = B * I;
+    if (I * H1 > big) big = I * H1;
+    if (H1 * H2 > big) big = H1 * H2;
+    if (B * H1 > big) big = B * H1;
+    float *z = falloc(B * H1), *a1 = falloc(B * H1), *h1 = falloc(B * H1), *a2 = falloc(B * H2),
+          *h2 = falloc(B * H2), *logits = falloc(B * C), *oh = falloc(B * C), *gl = falloc(B * C),
+          *gh2 = falloc(B * H2), *ga2 = falloc(B * H2), *gh1 = falloc(B * H1), *ga1 = falloc(B * H1),
+          *tmp = falloc(big), *gW1 = falloc(I * H1), *gW2 = falloc(H1 * H2), *gW3 = falloc(H2 * C),
+          *gb1 = falloc(H1), *gb2 = falloc(H2), *gb3 = falloc(C), *S2 = falloc(H1 * H2), *S3 = falloc(H2 * C);
+    long widest = H1 > H2 ? H1 : H2;
+    if (C > widest) widest = C;
+    double* cs = (double*)malloc((size_t)widest * sizeof(double));
+    memcpy(S2, W2, (size_t)(H1 * H2) * sizeof(float));
+    memcpy(S3, W3, (size_t)(H2 * C) * sizeof(float));
+    for (long s = 0; s < steps; ++s) {
+        const long b = nb > 0 ? s % nb : 0;
+        const float* x = images + b * B * I;
+        const float* y = labels + b * B;
+        co_matmul(x, I, 1, W1, H1, 1, z, B, H1, I);
+        co_add_rowbcast(z, b1, a1, B, H1);
+        co_relu(a1, h1, B * H1);
+        co_matmul(h1, H1, 1, W2, H2, 1, z, B, H2, H1);
+        co_add_rowbcast(z, b2, a2, B, H2);
+        co_relu(a2, h2, B * H2);
+        co_matmul(h2, H2, 1, W3, C, 1, z, B, C, H2);
+        co_add_rowbcast(z, b3, logits, B, C);
+        co_onehot(y, oh, B, C);
+        losses[s] = co_ce_onehot(logits, oh, B, C);
+        const float* B2 = stale_snapshot ? S2 : W2;
+        const float* B3 = stale_snapshot ? S3 : W3;
+        /* every gradient below is "zero-filled, then += value" (src/AutoDiff.cpp:1870-1907) */
+        co_ce_bwd_onehot(logits, oh, 1.0f, tmp, B, C);
+        zero_plus(gl, tmp, B * C);
+#define CO_BIAS_GRAD(g, out, cols)                                        \
+    if (strict_row0) {                                                     \
+        co_adjust_row0(g, tmp, B, cols);                                   \
+        zero_plus(out, tmp, cols);                                         \
+    } else {                                                               \
+        co_colsum_f64(g, cs, B, cols);                                     \
+        for (long j = 0; j < cols; ++j) out[j] = (float)cs[j];             \
+    }
+        CO_BIAS_GRAD(gl, gb3, C)
+        co_matmul(gl, C, 1, B3, 1, C, tmp, B, H2, C);          /* grad(h2) = gl . W3^T */
+        zero_plus(gh2, tmp, B * H2);
+        co_matmul(h2, 1, H2, gl, C, 1, tmp, H2, C, B);         /* grad(W3) = h2^T . gl */
+        zero_plus(gW3, tmp, H2 * C);
+        co_relu_bwd(a2, gh2, tmp, B * H2);
+        zero_plus(ga2, tmp, B * H2);
+        CO_BIAS_GRAD(ga2, gb2, H2)
+        co_matmul(ga2, H2, 1, B2, 1, H2, tmp, B, H1, H2);      /* grad(h1) = ga2 . W2^T */
+        zero_plus(gh1, tmp, B * H1);
+        co_matmul(h1, 1, H1, ga2, H2, 1, tmp, H1, H2, B);      /* grad(W2) = h1^T . ga2 */
+        zero_plus(gW2, tmp, H1 * H2);
+        co_relu_bwd(a1, gh1, tmp, B * H1);
+        zero_plus(ga1, tmp, B * H1);
+        CO_BIAS_GRAD(ga1, gb1, H1)
+        co_matmul(x, 1, I, ga1, H1, 1, tmp, I, H1, B);         /* grad(W1) = x^T . ga1 */
+        zero_plus(gW1, tmp, I * H1);
+#undef CO_BIAS_GRAD
+        co_sgd_step(W1, gW1, lr, I * H1);
+        co_sgd_step(b1, gb1, lr, H1);
+        co_sgd_step(W2, gW2, lr, H1 * H2);
+        co_sgd_step(b2, gb2, lr, H2);
+        co_sgd_step(W3, gW3, lr, H2 * C);
+        co_sgd_step(b3, gb3, lr, C);
+    }
+    free(z); free(a1); free(h1); free(a2); free(h2); free(logits); free(oh); free(gl); free(gh2);
+    free(ga2); free(gh1); free(ga1); free(tmp); free(gW1); free(gW2); free(gW3); free(gb1); free(gb2);
+    free(gb3); free(S2); free(S3); free(cs);
+}
+
+/* The demo's forward pass for prediction (mnist/mnist.cpp:95-130): logits, then a row softmax. */
+void co_mnist_predict(const float* x, long B, long I, long H1, long H2, long C, const float* W1,
+                      const float* b1, const float* W2, const float* b2, const float* W3, const float* b3,
+                      float* probs) {
+    float *z = falloc(B * (H1 > H2 ? H1 : H2)), *h1 = falloc(B * H1), *h2 = falloc(B * H2), *lg = falloc(B * C);
+    co_matmul(x, I, 1, W1, H1, 1, z, B, H1, I);
+    co_add_rowbcast(z, b1, h1, B, H1);
+    co_relu(h1, h1, B * H1);
+    co_matmul(h1, H1, 1, W2, H2, 1, z, B, H2, H1);
+    co_add_rowbcast(z, b2, h2, B, H2);
+    co_relu(h2, h2, B * H2);
+    co_matmul(h2, H2, 1, W3, C, 1, z, B, C, H2);
+    co_add_rowbcast(z, b3, lg, B, C);
+    co_softmax(lg, probs, B, C, 1, 0);
+    free(z); free(h1); free(h2); free(lg);
+}
+
 /* Y = sigmoid(X / R) - tanh(X) * sin(X) + cos(-X); L = mse(Y,T) + mae(Y,T); one backward.
  * R is a full [rows, cols] operand here (the reference's Div needs equal shapes).  The edge
  * order follows the reference's reversed depth-first order (src/AutoDiff.cpp:1138-1153); it

@@ -63,6 +63,18 @@ void co_mlp_step(const float* x, long B, long I, const float* W1, const float* b
 void co_expr(const float* X, const float* R, const float* T, long rows, long cols, float* Y,
              float* mse, float* mae, float* gX, float* gR);
 
+/* the MNIST demo's path (mnist/mnist.cpp, mnist/mnist_loader.cpp) */
+void co_u8_to_unit(const unsigned char* src, float* dst, long n);
+void co_onehot(const float* labels, float* out, long rows, long classes);
+void co_sgd_step(float* p, const float* g, float lr, long n);
+long co_count_correct(const float* pred, const float* labels, long rows, long classes);
+void co_mnist_train(const float* images, const float* labels, long n_images, long I, long H1, long H2,
+                    long C, float* W1, float* b1, float* W2, float* b2, float* W3, float* b3, long batch,
+                    long steps, float lr, int strict_row0, int stale_snapshot, float* losses);
+void co_mnist_predict(const float* x, long B, long I, long H1, long H2, long C, const float* W1,
+                      const float* b1, const float* W2, const float* b2, const float* W3, const float* b3,
+                      float* probs);
+
 /* seeded input generator shared by tests and fixtures (not from the reference) */
 void co_fill_uniform(float* r, long n, uint64_t seed, double lo, double hi);
 void co_fill_normal(float* r, long n, uint64_t seed, double mean, double sigma);

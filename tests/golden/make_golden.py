@@ -23,6 +23,62 @@ SPECIAL = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 3.4e38, -
                    np.float32)
 
 
+def mnist():
+    """The MNIST demo's path: loader, accuracy, the training loop over the reference library, and
+    the printed results of the demo program's own main() on the synthetic data set."""
+    import contextlib
+    import io
+    import re
+    import tempfile
+    from support import write_mnist_dir
+    o = Oracle()
+    r = Reference()
+    g = {}
+    with tempfile.TemporaryDirectory() as d:
+        tr_i, tr_l, te_i, te_l = write_mnist_dir(d)
+        images, labels = r.mnist_load(d, True)
+        g["loader_first_rows"] = images[:4]
+        g["loader_labels"] = labels[:64]
+        # the demo program's own main(), its stdout captured
+        sys.stdout.flush()
+        saved = os.dup(1)
+        with tempfile.TemporaryFile() as cap:
+            os.dup2(cap.fileno(), 1)
+            try:
+                rc = r.mnist_main_in(d)
+            finally:
+                sys.stdout.flush()
+                os.dup2(saved, 1)
+                os.close(saved)
+            cap.seek(0)
+            text = cap.read().decode("utf-8", "replace")
+        assert rc == 0
+        g["demo_epoch_losses"] = np.array([v for _, v in re.findall(r"Epoch (\d)/5 Loss: ([0-9.]+)", text)])
+        g["demo_accuracies"] = np.array(re.findall(r"准确率: ([0-9.]+)%", text))
+    g["demo_W1_head"] = r.mnist_xavier((784, 128), 784, reseed=42)[0, :32]
+    rng = np.random.default_rng(3)
+    pred = rng.random((300, 10)).astype(np.float32)
+    pred[5] = 0.1
+    pred[6, 3] = pred[6, 7] = 2.0
+    pred[7] = -2.0
+    lab = rng.integers(0, 10, 300).astype(np.float32)
+    lab[5], lab[6], lab[7] = 0, 3, 0
+    g["acc_pred"], g["acc_labels"], g["acc"] = pred, lab, r.mnist_accuracy(pred, lab)
+    for tag, (I, H1, H2, n, batch, steps) in (("s", (20, 12, 8, 48, 16, 9)), ("m", (64, 32, 16, 96, 32, 12))):
+        seed = 600 + I
+        x = o.uniform((n, I), seed, 0, 1)
+        y = o.ints((n,), seed + 1, 10)
+        params = [o.uniform((I, H1), seed + 2, -I ** -0.5, I ** -0.5), np.zeros(H1, np.float32),
+                  o.uniform((H1, H2), seed + 3, -H1 ** -0.5, H1 ** -0.5), np.zeros(H2, np.float32),
+                  o.uniform((H2, 10), seed + 4, -H2 ** -0.5, H2 ** -0.5), np.zeros(10, np.float32)]
+        losses, trained = r.mnist_train(x, y, params, batch, steps, 0.01)
+        g[tag + "_x"], g[tag + "_y"], g[tag + "_losses"] = x, y, losses
+        g[tag + "_cfg"] = np.array([batch, steps], np.int64)
+        for k, (p0, p1) in enumerate(zip(params, trained)):
+            g["%s_p%d" % (tag, k)], g["%s_q%d" % (tag, k)] = p0, p1
+    np.savez_compressed(os.path.join(HERE, "mnist.npz"), **g)
+
+
 def main():
     o = Oracle()   # only for its input generator
     r = Reference()
@@ -177,4 +233,8 @@ def main():
 
 
 if __name__ == "__main__":
-    main()
+    if "mnist" in sys.argv[1:]:
+        mnist()
+    else:
+        main()
+        mnist()

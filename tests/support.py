@@ -302,6 +302,103 @@ class Oracle:
                          fp(gX), fp(gR))
         return Y, np.float32(mse.value), np.float32(mae.value), gX, gR
 
+    # ---- the MNIST demo's path
+    def u8_to_unit(self, src):
+        src = np.ascontiguousarray(src, dtype=np.uint8)
+        r = np.empty(src.shape, np.float32)
+        self.lib.co_u8_to_unit(src.ctypes.data_as(C.POINTER(C.c_ubyte)), fp(r), C.c_long(src.size))
+        return r
+
+    def onehot(self, labels, classes):
+        labels = f32(labels)
+        r = np.empty((labels.size, classes), np.float32)
+        self.lib.co_onehot(fp(labels), fp(r), C.c_long(labels.size), C.c_long(classes))
+        return r
+
+    def sgd_step(self, p, g, lr):
+        p, g = f32(p).copy(), f32(g)
+        self.lib.co_sgd_step(fp(p), fp(g), C.c_float(lr), C.c_long(p.size))
+        return p
+
+    def count_correct(self, pred, labels):
+        pred, labels = f32(pred), f32(labels)
+        self.lib.co_count_correct.restype = C.c_long
+        return int(self.lib.co_count_correct(fp(pred), fp(labels), C.c_long(pred.shape[0]), C.c_long(pred.shape[1])))
+
+    def mnist_train(self, images, labels, params, batch, steps, lr, strict_row0, stale_snapshot):
+        """params = [W1, b1, W2, b2, W3, b3]; returns (losses, updated params)."""
+        images, labels = f32(images), f32(labels)
+        P = [f32(q).copy() for q in params]
+        I, H1 = P[0].shape
+        H2, Cn = P[4].shape
+        losses = np.empty(steps, np.float32)
+        self.lib.co_mnist_train(fp(images), fp(labels), C.c_long(images.shape[0]), C.c_long(I), C.c_long(H1),
+                                C.c_long(H2), C.c_long(Cn), *[fp(q) for q in P], C.c_long(batch), C.c_long(steps),
+                                C.c_float(lr), C.c_int(int(strict_row0)), C.c_int(int(stale_snapshot)), fp(losses))
+        return losses, P
+
+    def mnist_predict(self, x, params):
+        x = f32(x)
+        P = [f32(q) for q in params]
+        I, H1 = P[0].shape
+        H2, Cn = P[4].shape
+        probs = np.empty((x.shape[0], Cn), np.float32)
+        self.lib.co_mnist_predict(fp(x), C.c_long(x.shape[0]), C.c_long(I), C.c_long(H1), C.c_long(H2), C.c_long(Cn),
+                                  *[fp(q) for q in P], fp(probs))
+        return probs
+
+
+def synthetic_digits(n, seed):
+    """[n, 28, 28] uint8 images with a class-dependent bright patch over noise, and labels 0..9
+    (a stand-in for the MNIST image files, which the reference does not ship)."""
+    rng = np.random.default_rng(seed)
+    labels = rng.integers(0, 10, n).astype(np.uint8)
+    img = rng.integers(0, 96, (n, 28, 28)).astype(np.uint8)
+    for i, c in enumerate(labels):
+        r, col = 2 + 5 * (int(c) // 5) * 2, 1 + 5 * (int(c) % 5)
+        img[i, r:r + 8, col:col + 6] = rng.integers(160, 256, (8, 6)).astype(np.uint8)
+    return img, labels
+
+
+def write_mnist_dir(directory, n_train=512, n_test=256):
+    """The four IDX files of the MNIST demo, filled with synthetic_digits (seeds 1 and 2)."""
+    tr_i, tr_l = synthetic_digits(n_train, 1)
+    te_i, te_l = synthetic_digits(n_test, 2)
+    write_idx_images(os.path.join(directory, "train-images-idx3-ubyte"), tr_i)
+    write_idx_labels(os.path.join(directory, "train-labels-idx1-ubyte"), tr_l)
+    write_idx_images(os.path.join(directory, "t10k-images-idx3-ubyte"), te_i)
+    write_idx_labels(os.path.join(directory, "t10k-labels-idx1-ubyte"), te_l)
+    return tr_i, tr_l, te_i, te_l
+
+
+def libc_xavier(shape, fan_in, reseed=None):
+    """The demo's weight initialisation (mnist/mnist.cpp:21-27) from the C library's rand():
+    r = 2.0f * rand() / float(RAND_MAX) - 1.0f, w = r * sqrt(1.0f / fan_in), all in fp32."""
+    libc = C.CDLL("libc.so.6")
+    if reseed is not None:
+        libc.srand(C.c_uint(reseed))
+    n = int(np.prod(shape))
+    raw = np.array([libc.rand() for _ in range(n)], dtype=np.int64)
+    r = (np.float32(2.0) * raw.astype(np.float32)) / np.float32(2147483647) - np.float32(1.0)
+    return (r.astype(np.float32) * np.sqrt(np.float32(1.0) / np.float32(fan_in))).astype(np.float32).reshape(shape)
+
+
+def write_idx_images(path, pixels_u8):
+    """IDX3 file as the MNIST loader reads it (mnist/mnist_loader.cpp:7-44): big-endian magic 2051,
+    count, rows, cols, then one unsigned byte per pixel.  pixels_u8: [n, rows, cols] uint8."""
+    a = np.ascontiguousarray(pixels_u8, dtype=np.uint8)
+    with open(path, "wb") as f:
+        f.write(np.array([2051, a.shape[0], a.shape[1], a.shape[2]], dtype=">i4").tobytes())
+        f.write(a.tobytes())
+
+
+def write_idx_labels(path, labels_u8):
+    """IDX1 file (mnist/mnist_loader.cpp:46-73): big-endian magic 2049, count, one byte per label."""
+    a = np.ascontiguousarray(labels_u8, dtype=np.uint8)
+    with open(path, "wb") as f:
+        f.write(np.array([2049, a.shape[0]], dtype=">i4").tobytes())
+        f.write(a.tobytes())
+
 
 def ref_available():
     return os.path.exists(os.path.join(ORACLE_DIR, "_ref", "libctorch_ref.so"))
@@ -454,6 +551,53 @@ class Reference:
                                C.byref(mae), fp(gX), fp(gR), *extra)
         assert rc == rows * cols, rc
         return Y, np.float32(mse.value), np.float32(mae.value), gX, gR
+
+    # ---- the MNIST demo (oracle/ref_mnist_driver.cpp); reference build only
+    def mnist_load(self, directory, train):
+        dims = (C.c_long * 2)()
+        self.cdll.ref_mnist_load.restype = C.c_long
+        n = self.cdll.ref_mnist_load(directory.encode(), C.c_int(int(train)), None, None, dims)
+        assert n >= 0, n
+        images = np.empty((dims[0], dims[1]), np.float32)
+        labels = np.empty(n, np.float32)
+        self.cdll.ref_mnist_load(directory.encode(), C.c_int(int(train)), fp(images), fp(labels), dims)
+        return images, labels
+
+    def mnist_accuracy(self, pred, labels):
+        pred, labels = f32(pred), f32(labels)
+        self.cdll.ref_mnist_accuracy.restype = C.c_float
+        return np.float32(self.cdll.ref_mnist_accuracy(fp(pred), fp(labels), C.c_long(pred.shape[0])))
+
+    def mnist_get_batch(self, images, labels, batch, idx):
+        images, labels = f32(images), f32(labels)
+        n, px = images.shape
+        bi, bl = np.empty((batch, px), np.float32), np.empty(batch, np.float32)
+        self.cdll.ref_mnist_get_batch.restype = C.c_long
+        got = self.cdll.ref_mnist_get_batch(fp(images), fp(labels), C.c_long(n), C.c_long(px), C.c_long(batch),
+                                            C.c_long(idx), fp(bi), fp(bl))
+        return bi[:got], bl[:got]
+
+    def mnist_xavier(self, shape, fan_in, reseed=None):
+        w = np.empty(shape, np.float32)
+        self.cdll.ref_mnist_xavier(fp(w), C.c_long(w.size), C.c_long(fan_in), C.c_int(reseed is not None),
+                                   C.c_uint(reseed or 0))
+        return w
+
+    def mnist_train(self, images, labels, params, batch, steps, lr):
+        images, labels = f32(images), f32(labels)
+        P = [f32(q).copy() for q in params]
+        I, H1 = P[0].shape
+        H2, Cn = P[4].shape
+        losses = np.empty(steps, np.float32)
+        self.cdll.ref_mnist_train.restype = C.c_long
+        rc = self.cdll.ref_mnist_train(fp(images), fp(labels), C.c_long(images.shape[0]), C.c_long(I), C.c_long(H1),
+                                       C.c_long(H2), C.c_long(Cn), *[fp(q) for q in P], C.c_long(batch),
+                                       C.c_long(steps), C.c_float(lr), fp(losses))
+        assert rc == steps, rc
+        return losses, P
+
+    def mnist_main_in(self, directory):
+        return int(self.cdll.ref_mnist_main_in(directory.encode()))
 
 
 HOST_LIB = os.path.join(ROOT, "ctorch_amd", "host", "libctorch_amd_host.so")

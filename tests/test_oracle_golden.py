@@ -125,3 +125,41 @@ def test_configs(oracle, golden):
     R = np.broadcast_to(rv, X.shape).copy()
     Y, mse, mae, gX, gR = oracle.expr(X, R, T)
     eq(Y, g["expr_Y"]); eq(mse, g["expr_mse"]); eq(mae, g["expr_mae"]); eq(gX, g["expr_gX"]); eq(gR, g["expr_gR"])
+
+
+def test_mnist_path(oracle, golden):
+    """Loader arithmetic, accuracy, the demo's training loop (bit for bit) and the demo program's
+    printed epoch losses / accuracies, all against vectors written from the real reference."""
+    from support import libc_xavier, synthetic_digits
+    g = golden("mnist")
+    F = np.float32
+    tr_i, tr_l = synthetic_digits(512, 1)
+    te_i, te_l = synthetic_digits(256, 2)
+    x = oracle.u8_to_unit(tr_i.reshape(-1, 784))
+    assert same_bits(x[:4], g["loader_first_rows"]) and np.array_equal(tr_l[:64].astype(F), g["loader_labels"])
+    assert F(oracle.count_correct(g["acc_pred"], g["acc_labels"])) / F(300) == g["acc"]
+    for tag in ("s", "m"):
+        batch, steps = (int(v) for v in g[tag + "_cfg"])
+        params = [g["%s_p%d" % (tag, k)] for k in range(6)]
+        losses, trained = oracle.mnist_train(g[tag + "_x"], g[tag + "_y"], params, batch, steps, 0.01, True, True)
+        assert same_bits(losses, g[tag + "_losses"])
+        for k in range(6):
+            assert same_bits(trained[k], g["%s_q%d" % (tag, k)])
+    # the demo program: same initial weights from the C library's rand(), 5 epochs of 4 batches
+    W1 = libc_xavier((784, 128), 784, reseed=42)
+    if not same_bits(W1[0, :32], g["demo_W1_head"]):
+        import pytest
+        pytest.skip("this C library's rand() differs from the one the fixture was written with")
+    params = [W1, np.zeros(128, F), libc_xavier((128, 64), 128), np.zeros(64, F), libc_xavier((64, 10), 64),
+              np.zeros(10, F)]
+    y = tr_l.astype(F)
+    losses, trained = oracle.mnist_train(x, y, params, 128, 20, 0.01, True, True)
+    for e in range(5):
+        acc = F(0)
+        for b in range(4):
+            acc = F(acc + losses[e * 4 + b])
+        assert "%.4f" % F(acc / F(4)) == str(g["demo_epoch_losses"][e])
+    xt = oracle.u8_to_unit(te_i.reshape(-1, 784))
+    train_acc = F(oracle.count_correct(oracle.mnist_predict(x, trained), y)) / F(512)
+    test_acc = F(oracle.count_correct(oracle.mnist_predict(xt, trained), te_l.astype(F))) / F(256)
+    assert ["%.2f" % (train_acc * 100), "%.2f" % (test_acc * 100)] == [str(v) for v in g["demo_accuracies"]]
