@@ -23,6 +23,12 @@ PROTOTYPES = {
     "ctamd_memcpy_d2d": [_P, _P, _Z, _P],
     "ctamd_sync": [_P],
 }
+PROTOTYPES.update({
+    "ctamd_u8_to_unit_f32": [_P, _P, _Z, _P],
+    "ctamd_onehot_f32": [_P, _P, _Z, _Z, _P],
+    "ctamd_sgd_step_f32": [_P, _P, C.c_float, _Z, _P],
+    "ctamd_count_correct_f32": [_P, _P, _P, _Z, _Z, _P],
+})
 for _op in ("add", "sub", "mul", "div"):
     PROTOTYPES["ctamd_%s_f32" % _op] = [_P, _P, _P, _Z, _P]
     PROTOTYPES["ctamd_%s_rowbcast_f32" % _op] = [_P, _P, _P, _Z, _Z, _P]

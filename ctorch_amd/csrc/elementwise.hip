@@ -138,6 +138,13 @@ struct DivBwdBF { static constexpr int kIn = 3; static constexpr bool kTables = 
         float num = na * x[2];
         float den = x[1] * x[1];
         return num / den; } };
+// optimiser update p - g * lr with the product rounded first (mnist/mnist.cpp:86-92; that file is
+// built without FMA contraction by the reference); inputs (p, g)
+struct SgdF { static constexpr int kIn = 2; static constexpr bool kTables = false;
+    float lr;
+    __device__ float operator()(const float* x, const Tables&) const {
+        float step = x[1] * lr;
+        return x[0] - step; } };
 struct FillF { static constexpr int kIn = 0; static constexpr bool kTables = false;
     float v;
     __device__ float operator()(const float*, const Tables&) const { return v; } };
@@ -456,6 +463,10 @@ int ctamd_fill_from_f32(float* r, const float* v1, size_t n, void* s) {
 }
 int ctamd_accumulate_f32(float* grad, const float* val, size_t n, void* s) {
     return binary<AddF>(__func__, grad, val, grad, n, s);
+}
+int ctamd_sgd_step_f32(float* param, const float* grad, float lr, size_t n, void* s) {
+    Ptrs<2> in{{param, grad}};
+    return launch_map<SgdF>(__func__, in, param, n, SgdF{lr}, s);
 }
 int ctamd_relu_backward_f32(const float* x, const float* g, float* dx, size_t n, void* s) { return binary<ReluBwdF>(__func__, x, g, dx, n, s); }
 int ctamd_sigmoid_backward_f32(const float* x, const float* g, float* dx, size_t n, void* s) { return binary<SigmoidBwdF>(__func__, x, g, dx, n, s); }

@@ -46,6 +46,11 @@ class AutoDiffContext {
 };
 
 enum class BroadcastGrad { kColumnSum, kReferenceRow0 };
+// What the tape reads as a leaf's value in backward: the live tensor (default), or - as the
+// reference - the deep copy made when the leaf was first seen and never refreshed
+// (src/AutoDiff.cpp:265-278 returns early for a known id), so that after an in-place optimiser
+// update the gradients flowing back through a weight matrix still use its first-step values.
+enum class LeafValues { kLive, kReferenceFirstSeen };
 
 class AutoDiff {
    public:
@@ -77,6 +82,7 @@ class AutoDiff {
 
     void set_broadcast_grad(BroadcastGrad m) { broadcast_grad_ = m; }
     BroadcastGrad broadcast_grad() const { return broadcast_grad_; }
+    void set_leaf_values(LeafValues m) { leaf_values_ = m; }
     // Div's backward scans the divisor for |b| < FLT_EPSILON and throws (reference:
     // AutoDiff.cpp:1267-1284).  On the device that is one more pass over b and a host wait; it can
     // be switched off.
@@ -93,6 +99,7 @@ class AutoDiff {
     std::unordered_map<size_t, Pending> pending_;
     bool retain_graph_ = false;
     BroadcastGrad broadcast_grad_ = BroadcastGrad::kColumnSum;
+    LeafValues leaf_values_ = LeafValues::kLive;
     bool check_div_zero_ = true;
 
     Node* find(size_t id);

@@ -57,11 +57,15 @@ class Tensor {
     static Tensor alias(const Tensor& t) { return Tensor(AliasTag{}, t); }
     // transposed VIEW of a 2-D tensor: shares storage, no copy (the tape's B^T / A^T operands)
     static Tensor view_t(const Tensor& t);
+    // rows [first, first + count) of a contiguous tensor as a VIEW (shares storage, new id): what
+    // the demo's get_batch copies out (mnist/mnist.cpp:159-182) without the copy
+    static Tensor view_rows(const Tensor& t, size_t first, size_t count);
     // a tensor on `device` filled from host memory
     static Tensor from_host(const float* data, const std::vector<size_t>& shape, DeviceType device);
 
     // ---- metadata
     size_t id() const { return tensor_id_; }
+    void set_id(size_t id) { tensor_id_ = id; }
     void requires_grad(bool key);
     bool requires_grad() const { return _requires_grad; }
     void set_requires_grad(bool r) { _requires_grad = r; }

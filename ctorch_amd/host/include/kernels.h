@@ -44,6 +44,11 @@ Tensor sum_of(const Tensor& a, const Tensor& b);                       // a fres
 Tensor column_sum(const Tensor& g);                                   // [rows, cols] -> [cols]
 Tensor first_row(const Tensor& g);                                    // [rows, cols] -> [cols], row 0
 bool any_abs_lt_eps(const Tensor& b);
+// the MNIST demo's host loops as device launches
+Tensor onehot(const Tensor& labels, size_t classes);                   // mnist/mnist.cpp:72-78
+void sgd_step(Tensor& param, const Tensor& grad, float lr);            // mnist/mnist.cpp:86-92, in place
+size_t count_correct(const Tensor& pred, const Tensor& labels);        // mnist/mnist.cpp:134-156 (reads back)
+Tensor unit_from_bytes(const unsigned char* host_bytes, size_t rows, size_t cols);  // mnist_loader.cpp:33-41
 Tensor relu_backward(const Tensor& x, const Tensor& g);
 Tensor sigmoid_backward(const Tensor& x, const Tensor& g);
 Tensor tanh_backward(const Tensor& x, const Tensor& g);

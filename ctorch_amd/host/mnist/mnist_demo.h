@@ -1,0 +1,69 @@
+// The batch loop of the reference's MNIST demo (main() of mnist/mnist.cpp:220-283) as a function:
+// load the four IDX files from a directory, train, evaluate.  mnist.cpp prints what this returns;
+// tests call it in process.
+#ifndef CTORCH_AMD_HOST_MNIST_DEMO_H
+#define CTORCH_AMD_HOST_MNIST_DEMO_H
+
+#include <chrono>
+#include <string>
+#include <vector>
+
+#include "mnist_loader.h"
+#include "mnist_model.h"
+
+struct MnistDemoOptions {
+    std::string dir = ".";
+    int epochs = 5, batch_size = 128, hidden1 = 128, hidden2 = 64;
+    float learning_rate = 0.01f;
+    unsigned seed = 42;
+    // true: the reference's tape (row-0 bias gradients, leaf values frozen at first sight, tape
+    // never cleared); false: column sums, live leaves, tape cleared after every step
+    bool reference_tape = false;
+};
+
+struct MnistDemoResult {
+    size_t train_images = 0, test_images = 0, pixels = 0;
+    int num_batches = 0;
+    std::vector<float> epoch_loss;       // mean of the batch losses of each epoch, accumulated in fp32
+    float train_accuracy = 0, test_accuracy = 0;
+    double train_seconds = 0;
+};
+
+inline MnistDemoResult run_mnist_demo(const MnistDemoOptions& opt) {
+    MnistDemoResult res;
+    srand(opt.seed);
+    MNISTLoader loader(opt.dir);
+    Tensor train_images, train_labels, test_images, test_labels;
+    loader.load_training_data(train_images, train_labels);
+    loader.load_test_data(test_images, test_labels);
+    res.train_images = train_images.shape()[0];
+    res.test_images = test_images.shape()[0];
+    res.pixels = train_images.shape()[1];
+    NeuralNetwork model(int(res.pixels), opt.hidden1, opt.hidden2, 10, opt.learning_rate);
+    res.num_batches = int(res.train_images) / opt.batch_size;
+
+    AutoDiff autodiff;
+    if (opt.reference_tape) {
+        autodiff.set_broadcast_grad(BroadcastGrad::kReferenceRow0);
+        autodiff.set_leaf_values(LeafValues::kReferenceFirstSeen);
+    }
+    AutoDiffContext::Guard guard(&autodiff);
+    auto t0 = std::chrono::steady_clock::now();
+    for (int epoch = 0; epoch < opt.epochs; ++epoch) {
+        float epoch_loss = 0.0f;
+        for (int batch = 0; batch < res.num_batches; ++batch) {
+            Tensor batch_images, batch_labels;
+            get_batch(train_images, train_labels, opt.batch_size, batch, batch_images, batch_labels);
+            epoch_loss += model.train_step(batch_images, batch_labels);
+            if (!opt.reference_tape) autodiff.clear_graph();
+        }
+        epoch_loss /= static_cast<float>(res.num_batches);
+        res.epoch_loss.push_back(epoch_loss);
+    }
+    res.train_seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    res.test_accuracy = calculate_accuracy(model.predict(test_images), test_labels);
+    res.train_accuracy = calculate_accuracy(model.predict(train_images), train_labels);
+    return res;
+}
+
+#endif

@@ -31,7 +31,12 @@ void AutoDiff::make_leaf(Tensor& t, bool requires_grad) {
     }
     auto node = std::make_unique<Node>();
     node->tensor_id = t.id();
-    node->tensor = std::make_unique<Tensor>(Tensor::alias(t));
+    if (leaf_values_ == LeafValues::kReferenceFirstSeen) {
+        node->tensor = std::make_unique<Tensor>(t);      // deep copy, kept for the tape's lifetime
+        node->tensor->set_id(t.id());
+    } else {
+        node->tensor = std::make_unique<Tensor>(Tensor::alias(t));
+    }
     node->requires_grad = requires_grad;
     node->is_leaf = true;
     id_to_node[t.id()] = std::move(node);

@@ -9,6 +9,7 @@
 #include "Ctorch_Scheduler.h"
 
 #include "ctorch_amd.h"
+#include "mnist_demo.h"
 
 #include <chrono>
 #include <cstring>
@@ -447,6 +448,109 @@ long cth_time_expr(const float* X, const float* R, const float* T, long rows, lo
         backward(L);
         Tensor gX = grad(tX), gR = grad(tR);
     }, warm, reps, out);
+}
+
+// ------------------------------------------------------------------------- MNIST demo path
+// Same shapes as the reference-side doorway (ref_mnist_* of the test infrastructure).
+
+long cth_mnist_load(const char* dir, int which, float* images_out, float* labels_out, long* dims_out) {
+    try {
+        MNISTLoader loader(dir);
+        Tensor images, labels;
+        if (which) loader.load_training_data(images, labels);
+        else loader.load_test_data(images, labels);
+        dims_out[0] = long(images.shape()[0]);
+        dims_out[1] = long(images.shape()[1]);
+        if (images_out) emit(images, images_out);
+        if (labels_out) emit(labels, labels_out);
+        return long(labels.numel());
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
+float cth_mnist_accuracy(const float* pred, const float* labels, long rows) {
+    long pd[2] = {rows, 10}, ld[1] = {rows};
+    Tensor p = make(pred, pd, 2), y = make(labels, ld, 1);
+    return calculate_accuracy(p, y);
+}
+
+// `steps` consecutive batches (batch index = step % (n_images / batch)) inside one autograd
+// context, data set and parameters resident.  reference_tape != 0: leaf values frozen at their
+// first-seen copies and row-0 bias gradients (the reference's behaviour); else live leaves, column
+// sums and a tape cleared after every step.  Parameters are written back; losses_out[s] = loss of
+// step s.  ms_out (may be null) = milliseconds for all the steps.
+long cth_mnist_train(const float* images, const float* labels, long n_images, long I, long H1, long H2, long C,
+                     float* W1, float* b1, float* W2, float* b2, float* W3, float* b3, long batch, long steps,
+                     float lr, int reference_tape, float* losses_out, double* ms_out) {
+    try {
+        long id[2] = {n_images, I}, ld[1] = {n_images};
+        Tensor all_images = make(images, id, 2), all_labels = make(labels, ld, 1);
+        NeuralNetwork model(W1, b1, W2, b2, W3, b3, size_t(I), size_t(H1), size_t(H2), size_t(C), lr);
+        const long num_batches = n_images / batch;
+        AutoDiff autodiff;
+        if (reference_tape) {
+            autodiff.set_broadcast_grad(BroadcastGrad::kReferenceRow0);
+            autodiff.set_leaf_values(LeafValues::kReferenceFirstSeen);
+        }
+        AutoDiffContext::Guard guard(&autodiff);
+        ctamd_sync(nullptr);
+        auto t0 = std::chrono::steady_clock::now();
+        for (long s = 0; s < steps; ++s) {
+            Tensor x, y;
+            get_batch(all_images, all_labels, int(batch), int(s % num_batches), x, y);
+            losses_out[s] = model.train_step(x, y);
+            if (!reference_tape) autodiff.clear_graph();
+        }
+        ctamd_sync(nullptr);
+        if (ms_out) *ms_out = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+        emit(model.W1, W1);
+        emit(model.b1, b1);
+        emit(model.W2, W2);
+        emit(model.b2, b2);
+        emit(model.W3, W3);
+        emit(model.b3, b3);
+        return steps;
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
+// probabilities [B, C] of the demo's predict() for given parameters
+long cth_mnist_predict(const float* x, long B, long I, long H1, long H2, long C, const float* W1, const float* b1,
+                       const float* W2, const float* b2, const float* W3, const float* b3, float* probs_out) {
+    try {
+        long xd[2] = {B, I};
+        Tensor tx = make(x, xd, 2);
+        NeuralNetwork model(W1, b1, W2, b2, W3, b3, size_t(I), size_t(H1), size_t(H2), size_t(C), 0.0f);
+        return emit(model.predict(tx), probs_out);
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
+// The whole demo on the files in `dir`.  epoch_loss_out has room for `epochs` values;
+// acc_out = {train accuracy, test accuracy}; seconds_out = training time.
+long cth_mnist_demo(const char* dir, int epochs, int batch, float lr, int hidden1, int hidden2, int reference_tape,
+                    float* epoch_loss_out, float* acc_out, double* seconds_out) {
+    try {
+        MnistDemoOptions opt;
+        opt.dir = dir;
+        opt.epochs = epochs;
+        opt.batch_size = batch;
+        opt.learning_rate = lr;
+        opt.hidden1 = hidden1;
+        opt.hidden2 = hidden2;
+        opt.reference_tape = reference_tape != 0;
+        MnistDemoResult r = run_mnist_demo(opt);
+        for (size_t e = 0; e < r.epoch_loss.size(); ++e) epoch_loss_out[e] = r.epoch_loss[e];
+        acc_out[0] = r.train_accuracy;
+        acc_out[1] = r.test_accuracy;
+        if (seconds_out) *seconds_out = r.train_seconds;
+        return long(r.num_batches) * epochs;
+    } catch (const std::exception&) {
+        return -1;
+    }
 }
 
 }  // extern "C"

@@ -191,6 +191,44 @@ bool any_abs_lt_eps(const Tensor& b) {
     return v != 0;
 }
 
+Tensor onehot(const Tensor& labels, size_t classes) {
+    check_device(labels, "onehot");
+    Tensor r(ShapeTag{}, {labels.numel(), classes}, DType::kFloat, DeviceType::kAMD, false);
+    run(ctamd_onehot_f32(labels.fptr(), r.fptr(), labels.numel(), classes, nullptr), "onehot");
+    return r;
+}
+void sgd_step(Tensor& param, const Tensor& grad, float lr) {
+    check_device(param, "sgd_step");
+    check_device(grad, "sgd_step");
+    if (param.numel() != grad.numel() || !param.is_contiguous())
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "sgd_step: parameter and gradient differ in size");
+    run(ctamd_sgd_step_f32(param.fptr(), grad.fptr(), lr, param.numel(), nullptr), "sgd_step");
+}
+size_t count_correct(const Tensor& pred, const Tensor& labels) {
+    check_device(pred, "count_correct");
+    check_device(labels, "count_correct");
+    if (pred.dim() != 2 || labels.numel() != pred.sizes()[0])
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "count_correct: predictions must be [rows, classes]");
+    Tensor count(ShapeTag{}, {}, DType::kFloat, DeviceType::kAMD, false);   // 4 bytes, used as int32
+    run(ctamd_count_correct_f32(pred.fptr(), labels.fptr(), reinterpret_cast<int32_t*>(count.fptr()), pred.sizes()[0],
+                                pred.sizes()[1], nullptr), "count_correct");
+    int32_t v = 0;
+    device_copy_d2h(&v, count.fptr(), sizeof(v));
+    return static_cast<size_t>(v);
+}
+Tensor unit_from_bytes(const unsigned char* host_bytes, size_t rows, size_t cols) {
+    const size_t n = rows * cols;
+    Tensor r(ShapeTag{}, {rows, cols}, DType::kFloat, DeviceType::kAMD, false);
+    if (n == 0) return r;
+    void* staging = device_acquire(n);
+    device_copy_h2d(staging, host_bytes, n);
+    int rc = ctamd_u8_to_unit_f32(static_cast<const uint8_t*>(staging), r.fptr(), n, nullptr);
+    if (rc == CTAMD_OK) rc = ctamd_sync(nullptr);      // the staging block goes back to the pool now
+    device_release(staging, n);
+    run(rc, "unit_from_bytes");
+    return r;
+}
+
 namespace {
 Tensor grad2(int (*fn)(const float*, const float*, float*, size_t, void*), const char* name, const Tensor& x,
              const Tensor& g) {

@@ -191,6 +191,21 @@ int ctamd_cross_entropy_backward_index_f32(const float* x, const float* idx, con
 /* db = ((-a) * g) / (b * b).  src/AutoDiff.cpp:1314.  (da = g / b is ctamd_div_f32, :1285.) */
 int ctamd_div_backward_b_f32(const float* a, const float* b, const float* g, float* db, size_t n, void* stream);
 
+/* ------------------------------------------- the MNIST demo's path (mnist/, "next" rows) */
+/* dst[i] = src[i] / 255.0f, the loader's pixel normalisation (mnist/mnist_loader.cpp:35-41);
+ * bit-exact. */
+int ctamd_u8_to_unit_f32(const uint8_t* src, float* dst, size_t n, void* stream);
+/* out[i, j] = (j == (int)labels[i]) ? 1 : 0, the demo's one-hot targets (mnist/mnist.cpp:72-78). */
+int ctamd_onehot_f32(const float* labels, float* out, size_t rows, size_t classes, void* stream);
+/* param[i] -= grad[i] * lr, product and difference rounded separately as in the reference's
+ * binary (mnist/mnist.cpp:86-92; built without -O3/-march, CMakeLists.txt:56,65-86); bit-exact. */
+int ctamd_sgd_step_f32(float* param, const float* grad, float lr, size_t n, void* stream);
+/* count[0] = number of rows whose first maximum (strictly greater, starting from -1.0f at column
+ * 0) is at column (int)labels[row]: calculate_accuracy (mnist/mnist.cpp:134-156) without its
+ * division by the row count. */
+int ctamd_count_correct_f32(const float* pred, const float* labels, int32_t* count, size_t rows, size_t classes,
+                            void* stream);
+
 #ifdef __cplusplus
 }
 #endif

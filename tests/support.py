@@ -555,31 +555,31 @@ class Reference:
     # ---- the MNIST demo (oracle/ref_mnist_driver.cpp); reference build only
     def mnist_load(self, directory, train):
         dims = (C.c_long * 2)()
-        self.cdll.ref_mnist_load.restype = C.c_long
-        n = self.cdll.ref_mnist_load(directory.encode(), C.c_int(int(train)), None, None, dims)
+        self.lib.ref_mnist_load.restype = C.c_long
+        n = self.lib.ref_mnist_load(directory.encode(), C.c_int(int(train)), None, None, dims)
         assert n >= 0, n
         images = np.empty((dims[0], dims[1]), np.float32)
         labels = np.empty(n, np.float32)
-        self.cdll.ref_mnist_load(directory.encode(), C.c_int(int(train)), fp(images), fp(labels), dims)
+        self.lib.ref_mnist_load(directory.encode(), C.c_int(int(train)), fp(images), fp(labels), dims)
         return images, labels
 
     def mnist_accuracy(self, pred, labels):
         pred, labels = f32(pred), f32(labels)
-        self.cdll.ref_mnist_accuracy.restype = C.c_float
-        return np.float32(self.cdll.ref_mnist_accuracy(fp(pred), fp(labels), C.c_long(pred.shape[0])))
+        self.lib.ref_mnist_accuracy.restype = C.c_float
+        return np.float32(self.lib.ref_mnist_accuracy(fp(pred), fp(labels), C.c_long(pred.shape[0])))
 
     def mnist_get_batch(self, images, labels, batch, idx):
         images, labels = f32(images), f32(labels)
         n, px = images.shape
         bi, bl = np.empty((batch, px), np.float32), np.empty(batch, np.float32)
-        self.cdll.ref_mnist_get_batch.restype = C.c_long
-        got = self.cdll.ref_mnist_get_batch(fp(images), fp(labels), C.c_long(n), C.c_long(px), C.c_long(batch),
+        self.lib.ref_mnist_get_batch.restype = C.c_long
+        got = self.lib.ref_mnist_get_batch(fp(images), fp(labels), C.c_long(n), C.c_long(px), C.c_long(batch),
                                             C.c_long(idx), fp(bi), fp(bl))
         return bi[:got], bl[:got]
 
     def mnist_xavier(self, shape, fan_in, reseed=None):
         w = np.empty(shape, np.float32)
-        self.cdll.ref_mnist_xavier(fp(w), C.c_long(w.size), C.c_long(fan_in), C.c_int(reseed is not None),
+        self.lib.ref_mnist_xavier(fp(w), C.c_long(w.size), C.c_long(fan_in), C.c_int(reseed is not None),
                                    C.c_uint(reseed or 0))
         return w
 
@@ -589,15 +589,22 @@ class Reference:
         I, H1 = P[0].shape
         H2, Cn = P[4].shape
         losses = np.empty(steps, np.float32)
-        self.cdll.ref_mnist_train.restype = C.c_long
-        rc = self.cdll.ref_mnist_train(fp(images), fp(labels), C.c_long(images.shape[0]), C.c_long(I), C.c_long(H1),
-                                       C.c_long(H2), C.c_long(Cn), *[fp(q) for q in P], C.c_long(batch),
-                                       C.c_long(steps), C.c_float(lr), fp(losses))
+        self.lib.ref_mnist_train.restype = C.c_long
+        rc = self.lib.ref_mnist_train(fp(images), fp(labels), C.c_long(images.shape[0]), C.c_long(I), C.c_long(H1),
+                                      C.c_long(H2), C.c_long(Cn), *[fp(q) for q in P], C.c_long(batch),
+                                      C.c_long(steps), C.c_float(lr), *self._train_extra(), fp(losses),
+                                      *self._train_tail())
         assert rc == steps, rc
         return losses, P
 
+    def _train_extra(self):
+        return ()
+
+    def _train_tail(self):
+        return ()
+
     def mnist_main_in(self, directory):
-        return int(self.cdll.ref_mnist_main_in(directory.encode()))
+        return int(self.lib.ref_mnist_main_in(directory.encode()))
 
 
 HOST_LIB = os.path.join(ROOT, "ctorch_amd", "host", "libctorch_amd_host.so")
@@ -619,3 +626,42 @@ class HostLayer(Reference):
     def expr(self, X, R, T):
         """R may be the full [rows, cols] operand or the row vector [cols] (row-broadcast Div)."""
         return Reference.expr(self, X, R, T, C.c_int(int(np.ndim(R) == 1)))
+
+    # ---- the MNIST demo's path on the device
+    reference_tape = True     # mnist_train: the reference's tape properties, or live leaves + column sums
+    last_train_ms = 0.0
+
+    def _train_extra(self):
+        return (C.c_int(int(self.reference_tape)),)
+
+    def _train_tail(self):
+        self._ms = C.c_double(0)
+        return (C.byref(self._ms),)
+
+    def mnist_train(self, images, labels, params, batch, steps, lr, reference_tape=True):
+        self.reference_tape = reference_tape
+        out = Reference.mnist_train(self, images, labels, params, batch, steps, lr)
+        self.last_train_ms = self._ms.value
+        return out
+
+    def mnist_predict(self, x, params):
+        x = f32(x)
+        P = [f32(q) for q in params]
+        I, H1 = P[0].shape
+        H2, Cn = P[4].shape
+        probs = np.empty((x.shape[0], Cn), np.float32)
+        self.cdll.cth_mnist_predict.restype = C.c_long
+        rc = self.cdll.cth_mnist_predict(fp(x), C.c_long(x.shape[0]), C.c_long(I), C.c_long(H1), C.c_long(H2),
+                                         C.c_long(Cn), *[fp(q) for q in P], fp(probs))
+        assert rc == probs.size, rc
+        return probs
+
+    def mnist_demo(self, directory, epochs=5, batch=128, lr=0.01, hidden1=128, hidden2=64, reference_tape=False):
+        losses = np.empty(epochs, np.float32)
+        acc = np.empty(2, np.float32)
+        sec = C.c_double(0)
+        self.cdll.cth_mnist_demo.restype = C.c_long
+        rc = self.cdll.cth_mnist_demo(directory.encode(), C.c_int(epochs), C.c_int(batch), C.c_float(lr),
+                                      C.c_int(hidden1), C.c_int(hidden2), C.c_int(int(reference_tape)), fp(losses),
+                                      fp(acc), C.byref(sec))
+        return rc, losses, acc, sec.value
