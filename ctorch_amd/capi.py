@@ -22,6 +22,12 @@ PROTOTYPES = {
     "ctamd_memcpy_d2h": [_P, _P, _Z, _P],
     "ctamd_memcpy_d2d": [_P, _P, _Z, _P],
     "ctamd_sync": [_P],
+    "ctamd_stream_create": [C.POINTER(_P)],
+    "ctamd_stream_destroy": [_P],
+    "ctamd_graph_begin": [_P],
+    "ctamd_graph_end": [_P, C.POINTER(_P)],
+    "ctamd_graph_launch": [_P, _P],
+    "ctamd_graph_destroy": [_P],
 }
 PROTOTYPES.update({
     "ctamd_u8_to_unit_f32": [_P, _P, _Z, _P],

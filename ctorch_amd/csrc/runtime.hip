@@ -137,6 +137,46 @@ void ctamd_counters_read(double* bytes, double* flops, double* roofline_seconds,
     if (launches) *launches = g_launches;
 }
 
+// ---- streams and recorded launch sequences (HIP graphs)
+int ctamd_stream_create(void** stream) {
+    if (!stream) return fail(CTAMD_EINVAL, "%s: null output", __func__);
+    hipStream_t s = nullptr;
+    int rc = check_hip(hipStreamCreate(&s), "hipStreamCreate");   // default priority, blocking w.r.t. the null stream
+    *stream = rc ? nullptr : static_cast<void*>(s);
+    return rc;
+}
+int ctamd_stream_destroy(void* stream) {
+    if (!stream) return CTAMD_OK;
+    return check_hip(hipStreamDestroy(as_stream(stream)), "hipStreamDestroy");
+}
+int ctamd_graph_begin(void* stream) {
+    if (!stream) return fail(CTAMD_EINVAL, "%s: the null stream cannot record", __func__);
+    // relaxed: host-side calls that are not stream work (an allocation by a pool that ran dry)
+    // stay legal while recording
+    return check_hip(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeRelaxed), "hipStreamBeginCapture");
+}
+int ctamd_graph_end(void* stream, void** graph_out) {
+    if (!stream || !graph_out) return fail(CTAMD_EINVAL, "%s: null argument", __func__);
+    *graph_out = nullptr;
+    hipGraph_t g = nullptr;
+    int rc = check_hip(hipStreamEndCapture(as_stream(stream), &g), "hipStreamEndCapture");
+    if (rc) return rc;
+    hipGraphExec_t exec = nullptr;
+    rc = check_hip(hipGraphInstantiate(&exec, g, nullptr, nullptr, 0), "hipGraphInstantiate");
+    (void)hipGraphDestroy(g);
+    if (rc) return rc;
+    *graph_out = static_cast<void*>(exec);
+    return CTAMD_OK;
+}
+int ctamd_graph_launch(void* graph, void* stream) {
+    if (!graph) return fail(CTAMD_EINVAL, "%s: null graph", __func__);
+    return check_hip(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), as_stream(stream)), "hipGraphLaunch");
+}
+int ctamd_graph_destroy(void* graph) {
+    if (!graph) return CTAMD_OK;
+    return check_hip(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph)), "hipGraphExecDestroy");
+}
+
 const char* ctamd_version(void) { return "ctorch_amd 0.1 (gfx950)"; }
 
 int ctamd_malloc(void** ptr, size_t bytes) {

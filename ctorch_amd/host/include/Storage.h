@@ -16,6 +16,13 @@
 namespace ctorch_amd_host {
 // Device memory pool (src/DeviceMemory.cpp).  acquire() returns HBM of at least `bytes` bytes,
 // release() returns it to the pool; trim() frees everything cached.
+// Blocks acquired between reservation_begin() and reservation_stop() (on this thread) belong to
+// the reservation: when released they are parked with it, not handed to anyone else, until
+// reservation_destroy().  This is what keeps the memory of a recorded graph its own.
+struct BlockReservation;
+BlockReservation* reservation_begin();
+void reservation_stop();
+void reservation_destroy(BlockReservation* r);
 void* device_acquire(size_t bytes);
 void device_release(void* p, size_t bytes);
 void device_trim();

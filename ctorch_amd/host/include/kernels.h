@@ -44,6 +44,7 @@ Tensor sum_of(const Tensor& a, const Tensor& b);                       // a fres
 Tensor column_sum(const Tensor& g);                                   // [rows, cols] -> [cols]
 Tensor first_row(const Tensor& g);                                    // [rows, cols] -> [cols], row 0
 bool any_abs_lt_eps(const Tensor& b);
+void copy_into(Tensor& dst, const Tensor& src);                        // device-to-device, same element count
 // the MNIST demo's host loops as device launches
 Tensor onehot(const Tensor& labels, size_t classes);                   // mnist/mnist.cpp:72-78
 void sgd_step(Tensor& param, const Tensor& grad, float lr);            // mnist/mnist.cpp:86-92, in place
@@ -59,6 +60,13 @@ Tensor mse_backward(const Tensor& p, const Tensor& t, const Tensor& g0d);
 Tensor mae_backward(const Tensor& p, const Tensor& t, const Tensor& g0d);
 Tensor cross_entropy_backward(const Tensor& x, const Tensor& target, const Tensor& g0d);
 Tensor div_backward_b(const Tensor& a, const Tensor& b, const Tensor& g);
+// The stream every launch of this front-end goes to (as the C ABI's void*): the null stream unless a
+// DeviceGraph is recording or has installed its own.  While a graph records, anything that would
+// make the host wait for the device (item(), to_vector(), a transfer, a pool trim) throws.
+void* current_stream();
+void set_current_stream(void* stream);
+bool recording();
+void set_recording(bool on);
 void init_device();   // ctamd_init(0), once; throws if there is no gfx950 device
 }  // namespace ctorch_amd_host
 #endif

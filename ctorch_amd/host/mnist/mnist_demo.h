@@ -8,6 +8,7 @@
 #include <string>
 #include <vector>
 
+#include "DeviceGraph.h"
 #include "mnist_loader.h"
 #include "mnist_model.h"
 
@@ -19,6 +20,10 @@ struct MnistDemoOptions {
     // true: the reference's tape (row-0 bias gradients, leaf values frozen at first sight, tape
     // never cleared); false: column sums, live leaves, tape cleared after every step
     bool reference_tape = false;
+    // record one training step into a DeviceGraph and replay it per batch (one launch per step
+    // instead of ~50); needs reference_tape == false (a frozen leaf copy would be re-made by
+    // every replay)
+    bool use_graph = false;
 };
 
 struct MnistDemoResult {
@@ -48,12 +53,32 @@ inline MnistDemoResult run_mnist_demo(const MnistDemoOptions& opt) {
         autodiff.set_leaf_values(LeafValues::kReferenceFirstSeen);
     }
     AutoDiffContext::Guard guard(&autodiff);
+    if (opt.use_graph && opt.reference_tape)
+        Ctorch_Error::throwException(ErrorPlatform::kAMD, ErrorType::TENSOR_STATE, "the recorded step needs live leaves");
+    DeviceGraph step;
+    Tensor staged_images, staged_labels, staged_loss;
+    if (opt.use_graph && res.num_batches > 0) {
+        // the recorded step reads its batch from two fixed tensors; each batch is copied into them
+        staged_images = Tensor(ShapeTag{}, {size_t(opt.batch_size), res.pixels}, DType::kFloat, DeviceType::kAMD, false);
+        staged_labels = Tensor(ShapeTag{}, {size_t(opt.batch_size)}, DType::kFloat, DeviceType::kAMD, false);
+    }
     auto t0 = std::chrono::steady_clock::now();
     for (int epoch = 0; epoch < opt.epochs; ++epoch) {
         float epoch_loss = 0.0f;
         for (int batch = 0; batch < res.num_batches; ++batch) {
             Tensor batch_images, batch_labels;
             get_batch(train_images, train_labels, opt.batch_size, batch, batch_images, batch_labels);
+            if (opt.use_graph) {
+                ctorch_amd_host::copy_into(staged_images, batch_images);
+                ctorch_amd_host::copy_into(staged_labels, batch_labels);
+                if (!step.recorded()) {
+                    step.record([&] { staged_loss = model.train_step_on_device(staged_images, staged_labels); });
+                    autodiff.clear_graph();
+                }
+                step.replay();
+                epoch_loss += staged_loss.item<float>();
+                continue;
+            }
             epoch_loss += model.train_step(batch_images, batch_labels);
             if (!opt.reference_tape) autodiff.clear_graph();
         }

@@ -48,7 +48,12 @@ class NeuralNetwork {
     }
 
     // One step on a batch; returns the (sum-reduced) loss.  Needs an active AutoDiffContext.
-    float train_step(const Tensor& x, const Tensor& y) {
+    float train_step(const Tensor& x, const Tensor& y) { return train_step_on_device(x, y).item<float>(); }
+
+    // The same step without reading the loss back: nothing in it makes the host wait for the
+    // device, so it can be recorded into a DeviceGraph.  (The reference reads the loss between
+    // forward and backward, mnist/mnist.cpp:80-81; the value is the same wherever it is read.)
+    Tensor train_step_on_device(const Tensor& x, const Tensor& y) {
         AutoDiff* ctx = AutoDiffContext::current();
         Tensor* params[6] = {&W1, &b1, &W2, &b2, &W3, &b3};
         if (ctx)
@@ -59,10 +64,9 @@ class NeuralNetwork {
         Tensor logits = forward(x);
         Tensor y_one_hot = ctorch_amd_host::onehot(y, logits.sizes()[1]);
         Tensor loss = logits.cross_entropy(y_one_hot);
-        float loss_value = loss.item<float>();
         backward(loss);
         update_parameters();
-        return loss_value;
+        return loss;
     }
 
     void update_parameters() {

@@ -9,6 +9,7 @@
 #include "Ctorch_Scheduler.h"
 
 #include "ctorch_amd.h"
+#include "DeviceGraph.h"
 #include "mnist_demo.h"
 
 #include <chrono>
@@ -413,6 +414,52 @@ long cth_time_mlp(const float* x, long B, long I, const float* W1, const float* 
     }, warm, reps, out);
 }
 
+// The same MLP step with one-hot targets, recorded into a DeviceGraph once and replayed: a step is
+// one graph launch plus reading the loss back.  out[4] reports the operator launches recorded.
+long cth_time_mlp_graph(const float* x, long B, long I, const float* W1, const float* b1, long H, const float* W2,
+                        const float* b2, long C, const float* onehot, int warm, int reps, double* out) {
+    try {
+        long xd[2] = {B, I}, w1d[2] = {I, H}, b1d[1] = {H}, w2d[2] = {H, C}, b2d[1] = {C}, yd[2] = {B, C};
+        Tensor tx = make(x, xd, 2), tW1 = make(W1, w1d, 2), tb1 = make(b1, b1d, 1), tW2 = make(W2, w2d, 2),
+               tb2 = make(b2, b2d, 1), ty = make(onehot, yd, 2);
+        AutoDiff ctx;
+        configure(ctx);
+        AutoDiffContext::Guard guard(&ctx);
+        Tensor loss, g1, g2, g3, g4;
+        auto body = [&] {
+            tW1.requires_grad(true);
+            tb1.requires_grad(true);
+            tW2.requires_grad(true);
+            tb2.requires_grad(true);
+            Tensor h = (tx.matmul(tW1) + tb1).relu();
+            loss = (h.matmul(tW2) + tb2).cross_entropy(ty);
+            backward(loss);
+            g1 = grad(tW1), g2 = grad(tb1), g3 = grad(tW2), g4 = grad(tb2);
+        };
+        body();                               // once eagerly: the pool now holds every block the step needs
+        ctx.clear_graph();
+        ctamd_counters_reset();
+        DeviceGraph step;
+        step.record(body);
+        double bytes = 0, flops = 0, ideal = 0;
+        uint64_t launches = 0;
+        ctamd_counters_read(&bytes, &flops, &ideal, &launches);
+        float sink = 0;
+        for (int i = 0; i < warm; ++i) { step.replay(); sink += loss.item<float>(); }
+        auto t0 = std::chrono::steady_clock::now();
+        for (int i = 0; i < reps; ++i) { step.replay(); sink += loss.item<float>(); }
+        auto t1 = std::chrono::steady_clock::now();
+        out[0] = std::chrono::duration<double, std::milli>(t1 - t0).count() / reps;
+        out[1] = bytes;
+        out[2] = flops;
+        out[3] = ideal;
+        out[4] = double(launches);
+        return sink == sink ? reps : reps;     // (the loss is read every step, as a training loop does)
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
 // loss_sum = CE(logits, class index), backward: dlogits = softmax - onehot.
 long cth_time_softmax_ce(const float* logits, const float* labels, long rows, long cols, int warm, int reps,
                          double* out) {
@@ -478,7 +525,9 @@ float cth_mnist_accuracy(const float* pred, const float* labels, long rows) {
 // `steps` consecutive batches (batch index = step % (n_images / batch)) inside one autograd
 // context, data set and parameters resident.  reference_tape != 0: leaf values frozen at their
 // first-seen copies and row-0 bias gradients (the reference's behaviour); else live leaves, column
-// sums and a tape cleared after every step.  Parameters are written back; losses_out[s] = loss of
+// sums and a tape cleared after every step; 2: as 0 with the step recorded into a DeviceGraph at
+// the first batch and replayed for every batch (with unrelated eager work between the replays).
+// Parameters are written back; losses_out[s] = loss of
 // step s.  ms_out (may be null) = milliseconds for all the steps.
 long cth_mnist_train(const float* images, const float* labels, long n_images, long I, long H1, long H2, long C,
                      float* W1, float* b1, float* W2, float* b2, float* W3, float* b3, long batch, long steps,
@@ -489,16 +538,36 @@ long cth_mnist_train(const float* images, const float* labels, long n_images, lo
         NeuralNetwork model(W1, b1, W2, b2, W3, b3, size_t(I), size_t(H1), size_t(H2), size_t(C), lr);
         const long num_batches = n_images / batch;
         AutoDiff autodiff;
-        if (reference_tape) {
+        if (reference_tape == 1) {
             autodiff.set_broadcast_grad(BroadcastGrad::kReferenceRow0);
             autodiff.set_leaf_values(LeafValues::kReferenceFirstSeen);
         }
         AutoDiffContext::Guard guard(&autodiff);
+        DeviceGraph step;                    // reference_tape == 2: the step is recorded once and replayed
+        Tensor sx, sy, sloss;
+        if (reference_tape == 2) {
+            sx = Tensor(ShapeTag{}, {size_t(batch), size_t(I)}, DType::kFloat, DeviceType::kAMD, false);
+            sy = Tensor(ShapeTag{}, {size_t(batch)}, DType::kFloat, DeviceType::kAMD, false);
+        }
         ctamd_sync(nullptr);
         auto t0 = std::chrono::steady_clock::now();
         for (long s = 0; s < steps; ++s) {
             Tensor x, y;
             get_batch(all_images, all_labels, int(batch), int(s % num_batches), x, y);
+            if (reference_tape == 2) {
+                ctorch_amd_host::copy_into(sx, x);
+                ctorch_amd_host::copy_into(sy, y);
+                if (!step.recorded()) {
+                    step.record([&] { sloss = model.train_step_on_device(sx, sy); });
+                    autodiff.clear_graph();
+                }
+                step.replay();
+                // eager work between replays, on the null stream, through the pool
+                Tensor probe = (sx * 2.0f).sum();
+                losses_out[s] = sloss.item<float>();
+                (void)probe.item<float>();
+                continue;
+            }
             losses_out[s] = model.train_step(x, y);
             if (!reference_tape) autodiff.clear_graph();
         }
@@ -541,7 +610,8 @@ long cth_mnist_demo(const char* dir, int epochs, int batch, float lr, int hidden
         opt.learning_rate = lr;
         opt.hidden1 = hidden1;
         opt.hidden2 = hidden2;
-        opt.reference_tape = reference_tape != 0;
+        opt.reference_tape = reference_tape == 1;
+        opt.use_graph = reference_tape == 2;          // 2: live leaves and the step replayed from a recorded graph
         MnistDemoResult r = run_mnist_demo(opt);
         for (size_t e = 0; e < r.epoch_loss.size(); ++e) epoch_loss_out[e] = r.epoch_loss[e];
         acc_out[0] = r.train_accuracy;

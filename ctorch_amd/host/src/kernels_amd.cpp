@@ -56,23 +56,23 @@ Tensor elementwise(const BinaryFamily& f, const Tensor& a, const Tensor& b, bool
     check_device(b, f.name);
     if (a.sizes() == b.sizes()) {
         Tensor r = like(a);
-        run(f.same(a.fptr(), b.fptr(), r.fptr(), a.numel(), nullptr), f.name);
+        run(f.same(a.fptr(), b.fptr(), r.fptr(), a.numel(), current_stream()), f.name);
         return r;
     }
     if (b.numel() == 1) {
         Tensor r = like(a);
-        run(f.bscalar(a.fptr(), b.fptr(), r.fptr(), a.numel(), nullptr), f.name);
+        run(f.bscalar(a.fptr(), b.fptr(), r.fptr(), a.numel(), current_stream()), f.name);
         return r;
     }
     if (row_broadcastable(a, b)) {
         Tensor r = like(a);
-        run(f.rowbcast(a.fptr(), b.fptr(), r.fptr(), a.sizes()[0], a.sizes()[1], nullptr), f.name);
+        run(f.rowbcast(a.fptr(), b.fptr(), r.fptr(), a.sizes()[0], a.sizes()[1], current_stream()), f.name);
         return r;
     }
     if (a_scalar_ok && a.dim() == 0) {
         Tensor r = like(b);
-        if (&f == &kMul) run(ctamd_mul_bscalar_f32(b.fptr(), a.fptr(), r.fptr(), b.numel(), nullptr), f.name);
-        else run(ctamd_rsub_ascalar_f32(a.fptr(), b.fptr(), r.fptr(), b.numel(), nullptr), f.name);
+        if (&f == &kMul) run(ctamd_mul_bscalar_f32(b.fptr(), a.fptr(), r.fptr(), b.numel(), current_stream()), f.name);
+        else run(ctamd_rsub_ascalar_f32(a.fptr(), b.fptr(), r.fptr(), b.numel(), current_stream()), f.name);
         return r;
     }
     Ctorch_Error::throwException(kP, ErrorType::DIMENSION, std::string(f.name) + ": shapes differ and cannot be broadcast");
@@ -81,7 +81,7 @@ Tensor elementwise(const BinaryFamily& f, const Tensor& a, const Tensor& b, bool
 Tensor map(Un fn, const char* name, const Tensor& a) {
     check_device(a, name);
     Tensor r = like(a);
-    run(fn(a.fptr(), r.fptr(), a.numel(), nullptr), name);
+    run(fn(a.fptr(), r.fptr(), a.numel(), current_stream()), name);
     return r;
 }
 
@@ -92,7 +92,7 @@ Tensor reduce2(int (*fn)(const float*, const float*, float*, size_t, void*), con
     if (same_shape ? a.sizes() != b.sizes() : a.numel() != b.numel())
         Ctorch_Error::throwException(kP, ErrorType::DIMENSION, std::string(name) + ": operand sizes differ");
     Tensor r = scalar0d();
-    run(fn(a.fptr(), b.fptr(), r.fptr(), a.numel(), nullptr), name);
+    run(fn(a.fptr(), b.fptr(), r.fptr(), a.numel(), current_stream()), name);
     return r;
 }
 
@@ -107,16 +107,16 @@ void rows_cols(const Tensor& a, size_t& rows, size_t& cols) {
 Tensor scalar_op(const Tensor& a, float s, op which) {
     check_device(a, "tensor (op) float");
     Tensor r = like(a);
-    int rc = which == op::Add ? ctamd_add_scalar_f32(a.fptr(), s, r.fptr(), a.numel(), nullptr)
-           : which == op::Mul ? ctamd_mul_scalar_f32(a.fptr(), s, r.fptr(), a.numel(), nullptr)
-                              : ctamd_div_scalar_f32(a.fptr(), s, r.fptr(), a.numel(), nullptr);
+    int rc = which == op::Add ? ctamd_add_scalar_f32(a.fptr(), s, r.fptr(), a.numel(), current_stream())
+           : which == op::Mul ? ctamd_mul_scalar_f32(a.fptr(), s, r.fptr(), a.numel(), current_stream())
+                              : ctamd_div_scalar_f32(a.fptr(), s, r.fptr(), a.numel(), current_stream());
     run(rc, "tensor (op) float");
     return r;
 }
 Tensor sum_all(const Tensor& a) {
     check_device(a, "sum");
     Tensor r = scalar0d();
-    run(ctamd_sum_f32(a.fptr(), r.fptr(), a.numel(), nullptr), "sum");
+    run(ctamd_sum_f32(a.fptr(), r.fptr(), a.numel(), current_stream()), "sum");
     return r;
 }
 Tensor softmax_dim(const Tensor& a, int dim) {
@@ -124,24 +124,24 @@ Tensor softmax_dim(const Tensor& a, int dim) {
     Tensor r = like(a);
     size_t rows, cols;
     rows_cols(a, rows, cols);
-    if (a.dim() == 1 || dim == 1) run(ctamd_softmax_rows_f32(a.fptr(), r.fptr(), rows, cols, nullptr), "softmax");
-    else run(ctamd_softmax_cols_f32(a.fptr(), r.fptr(), rows, cols, nullptr), "softmax");
+    if (a.dim() == 1 || dim == 1) run(ctamd_softmax_rows_f32(a.fptr(), r.fptr(), rows, cols, current_stream()), "softmax");
+    else run(ctamd_softmax_cols_f32(a.fptr(), r.fptr(), rows, cols, current_stream()), "softmax");
     return r;
 }
 Tensor filled(const std::vector<size_t>& shape, float v, DeviceType device) {
     Tensor r(ShapeTag{}, shape, DType::kFloat, device, false);
-    if (device == DeviceType::kAMD) run(ctamd_fill_f32(r.fptr(), v, r.numel(), nullptr), "fill");
+    if (device == DeviceType::kAMD) run(ctamd_fill_f32(r.fptr(), v, r.numel(), current_stream()), "fill");
     else for (size_t i = 0; i < r.numel(); ++i) r.data<float>()[i] = v;
     return r;
 }
 void fill_scalar(Tensor& t, float v) {
     check_device(t, "fill");
-    run(ctamd_fill_f32(t.fptr(), v, t.numel(), nullptr), "fill");
+    run(ctamd_fill_f32(t.fptr(), v, t.numel(), current_stream()), "fill");
 }
 Tensor filled_from(const std::vector<size_t>& shape, const Tensor& s) {
     check_device(s, "fill");
     Tensor r(ShapeTag{}, shape, DType::kFloat, DeviceType::kAMD, false);
-    run(ctamd_fill_from_f32(r.fptr(), s.fptr(), r.numel(), nullptr), "fill");
+    run(ctamd_fill_from_f32(r.fptr(), s.fptr(), r.numel(), current_stream()), "fill");
     return r;
 }
 void accumulate(Tensor& grad, const Tensor& val) {
@@ -149,7 +149,7 @@ void accumulate(Tensor& grad, const Tensor& val) {
     check_device(val, "accumulate");
     if (grad.numel() != val.numel())
         Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "accumulate: gradient sizes differ");
-    run(ctamd_accumulate_f32(grad.fptr(), val.fptr(), grad.numel(), nullptr), "accumulate");
+    run(ctamd_accumulate_f32(grad.fptr(), val.fptr(), grad.numel(), current_stream()), "accumulate");
 }
 // grad = 0 + val in one pass: what the reference's "zero-filled gradient, then grad[i] += val[i]"
 // (src/AutoDiff.cpp:1870-1907) leaves after the first contribution, bit for bit (-0 becomes +0).
@@ -158,7 +158,7 @@ Tensor zero_plus(const Tensor& val, const std::vector<size_t>& shape) {
     Tensor r(ShapeTag{}, shape, DType::kFloat, DeviceType::kAMD, false);
     if (r.numel() != val.numel())
         Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "accumulate: gradient sizes differ");
-    run(ctamd_add_scalar_f32(val.fptr(), 0.0f, r.fptr(), r.numel(), nullptr), "accumulate");
+    run(ctamd_add_scalar_f32(val.fptr(), 0.0f, r.fptr(), r.numel(), current_stream()), "accumulate");
     return r;
 }
 Tensor sum_of(const Tensor& a, const Tensor& b) {
@@ -167,13 +167,13 @@ Tensor sum_of(const Tensor& a, const Tensor& b) {
     if (a.numel() != b.numel())
         Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "accumulate: gradient sizes differ");
     Tensor r = like(a);
-    run(ctamd_add_f32(a.fptr(), b.fptr(), r.fptr(), r.numel(), nullptr), "accumulate");
+    run(ctamd_add_f32(a.fptr(), b.fptr(), r.fptr(), r.numel(), current_stream()), "accumulate");
     return r;
 }
 Tensor column_sum(const Tensor& g) {
     check_device(g, "column_sum");
     Tensor r(ShapeTag{}, {g.sizes()[1]}, DType::kFloat, DeviceType::kAMD, false);
-    run(ctamd_colsum_f32(g.fptr(), r.fptr(), g.sizes()[0], g.sizes()[1], nullptr), "column_sum");
+    run(ctamd_colsum_f32(g.fptr(), r.fptr(), g.sizes()[0], g.sizes()[1], current_stream()), "column_sum");
     return r;
 }
 Tensor first_row(const Tensor& g) {
@@ -185,16 +185,23 @@ Tensor first_row(const Tensor& g) {
 bool any_abs_lt_eps(const Tensor& b) {
     check_device(b, "any_abs_lt_eps");
     Tensor flag(ShapeTag{}, {}, DType::kFloat, DeviceType::kAMD, false);   // 4 bytes, read as int32
-    run(ctamd_any_abs_lt_eps_f32(b.fptr(), reinterpret_cast<int32_t*>(flag.fptr()), b.numel(), nullptr), "any_abs_lt_eps");
+    run(ctamd_any_abs_lt_eps_f32(b.fptr(), reinterpret_cast<int32_t*>(flag.fptr()), b.numel(), current_stream()), "any_abs_lt_eps");
     int32_t v = 0;
     device_copy_d2h(&v, flag.fptr(), sizeof(v));
     return v != 0;
 }
 
+void copy_into(Tensor& dst, const Tensor& src) {
+    check_device(dst, "copy_into");
+    check_device(src, "copy_into");
+    if (dst.numel() != src.numel() || !dst.is_contiguous() || !src.is_contiguous())
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "copy_into: sizes differ or a tensor is not contiguous");
+    device_copy_d2d(dst.fptr(), src.fptr(), dst.numel() * sizeof(float));
+}
 Tensor onehot(const Tensor& labels, size_t classes) {
     check_device(labels, "onehot");
     Tensor r(ShapeTag{}, {labels.numel(), classes}, DType::kFloat, DeviceType::kAMD, false);
-    run(ctamd_onehot_f32(labels.fptr(), r.fptr(), labels.numel(), classes, nullptr), "onehot");
+    run(ctamd_onehot_f32(labels.fptr(), r.fptr(), labels.numel(), classes, current_stream()), "onehot");
     return r;
 }
 void sgd_step(Tensor& param, const Tensor& grad, float lr) {
@@ -202,7 +209,7 @@ void sgd_step(Tensor& param, const Tensor& grad, float lr) {
     check_device(grad, "sgd_step");
     if (param.numel() != grad.numel() || !param.is_contiguous())
         Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "sgd_step: parameter and gradient differ in size");
-    run(ctamd_sgd_step_f32(param.fptr(), grad.fptr(), lr, param.numel(), nullptr), "sgd_step");
+    run(ctamd_sgd_step_f32(param.fptr(), grad.fptr(), lr, param.numel(), current_stream()), "sgd_step");
 }
 size_t count_correct(const Tensor& pred, const Tensor& labels) {
     check_device(pred, "count_correct");
@@ -211,7 +218,7 @@ size_t count_correct(const Tensor& pred, const Tensor& labels) {
         Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "count_correct: predictions must be [rows, classes]");
     Tensor count(ShapeTag{}, {}, DType::kFloat, DeviceType::kAMD, false);   // 4 bytes, used as int32
     run(ctamd_count_correct_f32(pred.fptr(), labels.fptr(), reinterpret_cast<int32_t*>(count.fptr()), pred.sizes()[0],
-                                pred.sizes()[1], nullptr), "count_correct");
+                                pred.sizes()[1], current_stream()), "count_correct");
     int32_t v = 0;
     device_copy_d2h(&v, count.fptr(), sizeof(v));
     return static_cast<size_t>(v);
@@ -222,8 +229,8 @@ Tensor unit_from_bytes(const unsigned char* host_bytes, size_t rows, size_t cols
     if (n == 0) return r;
     void* staging = device_acquire(n);
     device_copy_h2d(staging, host_bytes, n);
-    int rc = ctamd_u8_to_unit_f32(static_cast<const uint8_t*>(staging), r.fptr(), n, nullptr);
-    if (rc == CTAMD_OK) rc = ctamd_sync(nullptr);      // the staging block goes back to the pool now
+    int rc = ctamd_u8_to_unit_f32(static_cast<const uint8_t*>(staging), r.fptr(), n, current_stream());
+    if (rc == CTAMD_OK) rc = ctamd_sync(current_stream());      // the staging block goes back to the pool now
     device_release(staging, n);
     run(rc, "unit_from_bytes");
     return r;
@@ -236,7 +243,7 @@ Tensor grad2(int (*fn)(const float*, const float*, float*, size_t, void*), const
     check_device(g, name);
     if (x.numel() != g.numel()) Ctorch_Error::throwException(kP, ErrorType::DIMENSION, std::string(name) + ": sizes differ");
     Tensor r = like(x);
-    run(fn(x.fptr(), g.fptr(), r.fptr(), x.numel(), nullptr), name);
+    run(fn(x.fptr(), g.fptr(), r.fptr(), x.numel(), current_stream()), name);
     return r;
 }
 }  // namespace
@@ -251,20 +258,20 @@ Tensor softmax_backward(const Tensor& y, const Tensor& g, int dim) {
     Tensor r = like(y);
     size_t rows, cols;
     rows_cols(y, rows, cols);
-    if (y.dim() == 1 || dim == 1) run(ctamd_softmax_backward_rows_f32(y.fptr(), g.fptr(), r.fptr(), rows, cols, nullptr), "softmax_backward");
-    else run(ctamd_softmax_backward_cols_f32(y.fptr(), g.fptr(), r.fptr(), rows, cols, nullptr), "softmax_backward");
+    if (y.dim() == 1 || dim == 1) run(ctamd_softmax_backward_rows_f32(y.fptr(), g.fptr(), r.fptr(), rows, cols, current_stream()), "softmax_backward");
+    else run(ctamd_softmax_backward_cols_f32(y.fptr(), g.fptr(), r.fptr(), rows, cols, current_stream()), "softmax_backward");
     return r;
 }
 Tensor mse_backward(const Tensor& p, const Tensor& t, const Tensor& g) {
     check_device(p, "mse_backward");
     Tensor r = like(p);
-    run(ctamd_mse_backward_f32(p.fptr(), t.fptr(), g.fptr(), r.fptr(), p.numel(), nullptr), "mse_backward");
+    run(ctamd_mse_backward_f32(p.fptr(), t.fptr(), g.fptr(), r.fptr(), p.numel(), current_stream()), "mse_backward");
     return r;
 }
 Tensor mae_backward(const Tensor& p, const Tensor& t, const Tensor& g) {
     check_device(p, "mae_backward");
     Tensor r = like(p);
-    run(ctamd_mae_backward_f32(p.fptr(), t.fptr(), g.fptr(), r.fptr(), p.numel(), nullptr), "mae_backward");
+    run(ctamd_mae_backward_f32(p.fptr(), t.fptr(), g.fptr(), r.fptr(), p.numel(), current_stream()), "mae_backward");
     return r;
 }
 Tensor cross_entropy_backward(const Tensor& x, const Tensor& target, const Tensor& g) {
@@ -275,9 +282,9 @@ Tensor cross_entropy_backward(const Tensor& x, const Tensor& target, const Tenso
     rows_cols(x, rows, cols);
     Tensor r = like(x);
     if (x.sizes() == target.sizes())
-        run(ctamd_cross_entropy_backward_onehot_f32(x.fptr(), target.fptr(), g.fptr(), r.fptr(), rows, cols, nullptr), "cross_entropy_backward");
+        run(ctamd_cross_entropy_backward_onehot_f32(x.fptr(), target.fptr(), g.fptr(), r.fptr(), rows, cols, current_stream()), "cross_entropy_backward");
     else if (target.dim() == 1 && x.dim() == 2 && target.sizes()[0] == rows)
-        run(ctamd_cross_entropy_backward_index_f32(x.fptr(), target.fptr(), g.fptr(), r.fptr(), rows, cols, nullptr), "cross_entropy_backward");
+        run(ctamd_cross_entropy_backward_index_f32(x.fptr(), target.fptr(), g.fptr(), r.fptr(), rows, cols, current_stream()), "cross_entropy_backward");
     else
         Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "cross_entropy_backward: target shape not understood");
     return r;
@@ -285,7 +292,7 @@ Tensor cross_entropy_backward(const Tensor& x, const Tensor& target, const Tenso
 Tensor div_backward_b(const Tensor& a, const Tensor& b, const Tensor& g) {
     check_device(a, "div_backward");
     Tensor r = like(a);
-    run(ctamd_div_backward_b_f32(a.fptr(), b.fptr(), g.fptr(), r.fptr(), a.numel(), nullptr), "div_backward");
+    run(ctamd_div_backward_b_f32(a.fptr(), b.fptr(), g.fptr(), r.fptr(), a.numel(), current_stream()), "div_backward");
     return r;
 }
 
@@ -311,7 +318,7 @@ Tensor MatMul_AMD_kernel(const Tensor& a, const Tensor& b) {
     size_t m = a.shape()[0], k = a.shape()[1], n = b.shape()[1];
     Tensor r(ShapeTag{}, {m, n}, DType::kFloat, DeviceType::kAMD, false);
     run(ctamd_matmul_f32(a.fptr(), int64_t(a.strides()[0]), int64_t(a.strides()[1]), b.fptr(), int64_t(b.strides()[0]),
-                         int64_t(b.strides()[1]), r.fptr(), int64_t(m), int64_t(n), int64_t(k), nullptr),
+                         int64_t(b.strides()[1]), r.fptr(), int64_t(m), int64_t(n), int64_t(k), current_stream()),
         "MatMul_AMD_kernel");
     return r;
 }
@@ -333,14 +340,14 @@ Tensor CrossEntropy_AMD_kernel(const Tensor& a, const Tensor& b) {
         size_t rows, cols;
         rows_cols(a, rows, cols);
         Tensor r = scalar0d();
-        run(ctamd_cross_entropy_onehot_f32(a.fptr(), b.fptr(), r.fptr(), rows, cols, nullptr), "CrossEntropy_AMD_kernel");
+        run(ctamd_cross_entropy_onehot_f32(a.fptr(), b.fptr(), r.fptr(), rows, cols, current_stream()), "CrossEntropy_AMD_kernel");
         return r;
     }
     if (b.dim() == 1 && a.dim() == 2 && b.sizes()[0] == a.sizes()[0]) {
         Tensor r = scalar0d();
         Tensor status = scalar0d();   // 4 bytes, used as int32
         run(ctamd_cross_entropy_index_f32(a.fptr(), b.fptr(), r.fptr(), reinterpret_cast<int32_t*>(status.fptr()),
-                                          a.sizes()[0], a.sizes()[1], nullptr), "CrossEntropy_AMD_kernel");
+                                          a.sizes()[0], a.sizes()[1], current_stream()), "CrossEntropy_AMD_kernel");
         int32_t bad = 0;
         device_copy_d2h(&bad, status.fptr(), sizeof(bad));
         if (bad) {

@@ -54,6 +54,22 @@ int ctamd_memcpy_d2h(void* dst_host, const void* src, size_t bytes, void* stream
 int ctamd_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream);
 int ctamd_sync(void* stream);
 
+/* Streams and recorded launch sequences, with no counterpart in the reference (which is
+ * synchronous): a caller whose step is a fixed sequence of small launches (a training step at a
+ * small batch costs ~3 us of launch overhead per operator) records it once into a HIP graph and
+ * replays it with one launch.  ctamd_graph_begin(stream) puts a stream created by
+ * ctamd_stream_create into recording mode: every launcher called with that stream until
+ * ctamd_graph_end is recorded, not executed.  No entry point records a memset node (flags and
+ * counters are cleared by kernels), so every launcher is safe to record; ctamd_sync, the h2d/d2h
+ * copies and ctamd_malloc/free are not stream work and must not be called on a recording stream.
+ * The recorded sequence holds the device pointers it was recorded with. */
+int ctamd_stream_create(void** stream);
+int ctamd_stream_destroy(void* stream);
+int ctamd_graph_begin(void* stream);
+int ctamd_graph_end(void* stream, void** graph);
+int ctamd_graph_launch(void* graph, void* stream);
+int ctamd_graph_destroy(void* graph);
+
 /* Work counters, a measurement aid with no counterpart in the reference.  Every operator entry
  * point below adds its algorithmic HBM bytes and flops (what the operator must move and compute:
  * e.g. 12 bytes per element for r = a + b, 2*m*n*k flops for MatMul), and

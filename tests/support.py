@@ -657,6 +657,7 @@ class HostLayer(Reference):
         return probs
 
     def mnist_demo(self, directory, epochs=5, batch=128, lr=0.01, hidden1=128, hidden2=64, reference_tape=False):
+        """reference_tape: False / True, or 2 for live leaves with the step replayed from a recorded graph."""
         losses = np.empty(epochs, np.float32)
         acc = np.empty(2, np.float32)
         sec = C.c_double(0)

@@ -139,3 +139,28 @@ def test_demo_on_a_synthetic_data_set(host, oracle, tmp_path):
         want_train = oracle.count_correct(oracle.mnist_predict(x, trained), y) / 512
         want_test = oracle.count_correct(oracle.mnist_predict(xt, trained), yt) / 256
         assert abs(acc[0] - want_train) <= 0.02 and abs(acc[1] - want_test) <= 0.02
+
+
+@pytest.mark.parametrize("tag", ["s", "m"])
+def test_recorded_step_replays_to_the_same_bits(host, golden, tag):
+    """The training step recorded into a HIP graph at the first batch and replayed for every batch,
+    with unrelated eager launches and host reads between the replays: every loss and every trained
+    parameter must have the bits of the step-by-step run (same kernels, same order)."""
+    print("case recorded step", tag, flush=True)
+    g = golden("mnist")
+    batch, steps = (int(v) for v in g[tag + "_cfg"])
+    params = [g["%s_p%d" % (tag, k)] for k in range(6)]
+    eager_l, eager_p = host.mnist_train(g[tag + "_x"], g[tag + "_y"], params, batch, steps, 0.01, reference_tape=0)
+    graph_l, graph_p = host.mnist_train(g[tag + "_x"], g[tag + "_y"], params, batch, steps, 0.01, reference_tape=2)
+    assert same_bits(graph_l, eager_l)
+    for a, b in zip(graph_p, eager_p):
+        assert same_bits(a, b)
+
+
+def test_demo_with_a_recorded_step(host, tmp_path):
+    print("case demo recorded", flush=True)
+    write_mnist_dir(str(tmp_path))
+    rc1, l1, a1, _ = host.mnist_demo(str(tmp_path), epochs=3, lr=1e-3, reference_tape=0)
+    rc2, l2, a2, _ = host.mnist_demo(str(tmp_path), epochs=3, lr=1e-3, reference_tape=2)
+    assert rc1 == rc2 == 12
+    assert same_bits(l1, l2) and same_bits(a1, a2)
