@@ -271,7 +271,9 @@ def test_softmax_columns(oracle, shape):
 
 
 MM_SHAPES = [(1, 1, 1), (5, 3, 9), (33, 29, 47), (128, 128, 16), (130, 257, 70), (256, 10, 784), (64, 256, 10),
-             (784, 256, 300), (256, 10, 8192), (17, 1, 33), (1, 40, 33), (200, 200, 1), (384, 512, 1024)]
+             (784, 256, 300), (256, 10, 8192), (17, 1, 33), (1, 40, 33), (200, 200, 1), (384, 512, 1024),
+             # ragged edges and a K that is no multiple of the k tile, for the 128 x 128 and the 256 x 256 tile shapes
+             (2049, 2050, 33), (4100, 4101, 70)]
 
 
 @pytest.mark.parametrize("m,n,k", MM_SHAPES)
