@@ -30,6 +30,7 @@ PROTOTYPES = {
     "ctamd_graph_destroy": [_P],
 }
 PROTOTYPES.update({
+    "ctamd_div_backward_b_rowbcast_f32": [_P, _P, _P, _P, _Z, _Z, _P],
     "ctamd_u8_to_unit_f32": [_P, _P, _Z, _P],
     "ctamd_onehot_f32": [_P, _P, _Z, _Z, _P],
     "ctamd_sgd_step_f32": [_P, _P, C.c_float, _Z, _P],

@@ -313,20 +313,24 @@ int launch_map(const char* name, Ptrs<F::kIn> in, float* out, size_t n, F f, voi
 
 // r[i,j] = a[i,j] (op) b[j].  VEC: cols % 4 == 0 and aligned pointers - every 128-bit vector of a
 // meets one aligned vector of b (served from cache: b is cols*4 bytes, read rows times).
+// r[i, j] = Op(a[i, j], b[j]) or, for an Op with kIn == 3, Op(a[i, j], b[j], g[i, j]).
 template <class Op, bool VEC, class Index, bool NT>
 __global__ __launch_bounds__(kThreads) void rowbcast_kernel(const float* __restrict__ a, const float* __restrict__ b,
-                                                            float* __restrict__ r, size_t total, Index cols) {
+                                                            const float* __restrict__ g, float* __restrict__ r,
+                                                            size_t total, Index cols) {
     const Tables tabs{nullptr, nullptr};
+    constexpr bool kThird = (Op::kIn == 3);
     if (VEC) {
         const size_t n4 = total >> 2;
         const Index cols4 = cols >> 2;
         const size_t base = size_t(blockIdx.x) * (kThreads * kUnroll) + threadIdx.x;
-        v4f va[kUnroll], vb[kUnroll];
+        v4f va[kUnroll], vb[kUnroll], vg[kUnroll];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             size_t i = base + size_t(u) * kThreads;
             if (i < n4) {
                 va[u] = ld_stream<NT>(a, i);
+                if (kThird) vg[u] = ld_stream<NT>(g, i);
                 vb[u] = reinterpret_cast<const v4f*>(b)[Index(i) % cols4];   // re-used: keep cached
             }
         }
@@ -337,7 +341,7 @@ __global__ __launch_bounds__(kThreads) void rowbcast_kernel(const float* __restr
                 v4f o;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    float x[2] = {va[u][e], vb[u][e]};
+                    float x[3] = {va[u][e], vb[u][e], kThird ? vg[u][e] : 0.0f};
                     o[e] = Op()(x, tabs);
                 }
                 st_stream<NT>(r, i, o);
@@ -347,7 +351,7 @@ __global__ __launch_bounds__(kThreads) void rowbcast_kernel(const float* __restr
         const size_t tid = size_t(blockIdx.x) * kThreads + threadIdx.x;
         const size_t stride = size_t(gridDim.x) * kThreads;
         for (size_t i = tid; i < total; i += stride) {
-            float x[2] = {a[i], b[Index(i) % cols]};
+            float x[3] = {a[i], b[Index(i) % cols], kThird ? g[i] : 0.0f};
             r[i] = Op()(x, tabs);
         }
     }
@@ -355,12 +359,12 @@ __global__ __launch_bounds__(kThreads) void rowbcast_kernel(const float* __restr
 
 template <class Op>
 int launch_rowbcast(const char* name, const float* a, const float* b, float* r, size_t rows, size_t cols,
-                    void* stream) {
+                    void* stream, const float* g = nullptr) {
     if (rows == 0 || cols == 0) return CTAMD_OK;
-    if (!a || !b || !r) return fail(CTAMD_EINVAL, "%s: null pointer", name);
+    if (!a || !b || !r || (Op::kIn == 3 && !g)) return fail(CTAMD_EINVAL, "%s: null pointer", name);
     if (rows > (size_t(1) << 62) / cols) return fail(CTAMD_ERANGE, "%s: rows*cols overflows", name);
     size_t total = rows * cols;
-    bool vec = (cols % 4 == 0) && aligned16(a) && aligned16(b) && aligned16(r);
+    bool vec = (cols % 4 == 0) && aligned16(a) && aligned16(b) && aligned16(r) && (Op::kIn != 3 || aligned16(g));
     bool small = total < (size_t(1) << 32);
     size_t blocks = (total / 4 + size_t(kThreads) * kUnroll - 1) / (size_t(kThreads) * kUnroll);
     if (blocks > 0x7fffffffu) return fail(CTAMD_ERANGE, "%s: more than 2^43 elements", name);
@@ -368,16 +372,16 @@ int launch_rowbcast(const char* name, const float* a, const float* b, float* r, 
     hipStream_t s = as_stream(stream);
     const bool nt = total * sizeof(float) * 2 >= kStreamBytes;
     if (vec && small && nt)
-        hipLaunchKernelGGL((rowbcast_kernel<Op, true, uint32_t, true>), dim3(grid), dim3(kThreads), 0, s, a, b, r, total, uint32_t(cols));
+        hipLaunchKernelGGL((rowbcast_kernel<Op, true, uint32_t, true>), dim3(grid), dim3(kThreads), 0, s, a, b, g, r, total, uint32_t(cols));
     else if (vec && small)
-        hipLaunchKernelGGL((rowbcast_kernel<Op, true, uint32_t, false>), dim3(grid), dim3(kThreads), 0, s, a, b, r, total, uint32_t(cols));
+        hipLaunchKernelGGL((rowbcast_kernel<Op, true, uint32_t, false>), dim3(grid), dim3(kThreads), 0, s, a, b, g, r, total, uint32_t(cols));
     else if (vec)
-        hipLaunchKernelGGL((rowbcast_kernel<Op, true, uint64_t, true>), dim3(grid), dim3(kThreads), 0, s, a, b, r, total, uint64_t(cols));
+        hipLaunchKernelGGL((rowbcast_kernel<Op, true, uint64_t, true>), dim3(grid), dim3(kThreads), 0, s, a, b, g, r, total, uint64_t(cols));
     else if (small)
-        hipLaunchKernelGGL((rowbcast_kernel<Op, false, uint32_t, false>), dim3(grid), dim3(kThreads), 0, s, a, b, r, total, uint32_t(cols));
+        hipLaunchKernelGGL((rowbcast_kernel<Op, false, uint32_t, false>), dim3(grid), dim3(kThreads), 0, s, a, b, g, r, total, uint32_t(cols));
     else
-        hipLaunchKernelGGL((rowbcast_kernel<Op, false, uint64_t, false>), dim3(grid), dim3(kThreads), 0, s, a, b, r, total, uint64_t(cols));
-    account(8.0 * double(total) + 4.0 * double(cols), 0.0);
+        hipLaunchKernelGGL((rowbcast_kernel<Op, false, uint64_t, false>), dim3(grid), dim3(kThreads), 0, s, a, b, g, r, total, uint64_t(cols));
+    account((Op::kIn == 3 ? 12.0 : 8.0) * double(total) + 4.0 * double(cols), 0.0);
     return launched(name);
 }
 
@@ -482,6 +486,10 @@ int ctamd_mae_backward_f32(const float* p, const float* t, const float* g1, floa
     if (n && !g1) return fail(CTAMD_EINVAL, "%s: null upstream gradient", __func__);
     Ptrs<2> in{{p, t}};
     return launch_map<MaeBwdF>(__func__, in, dp, n, MaeBwdF{1.0 / double(float(n)), g1}, s);
+}
+int ctamd_div_backward_b_rowbcast_f32(const float* a, const float* b, const float* g, float* db, size_t rows, size_t cols,
+                                      void* s) {
+    return launch_rowbcast<DivBwdBF>(__func__, a, b, db, rows, cols, s, g);
 }
 int ctamd_div_backward_b_f32(const float* a, const float* b, const float* g, float* db, size_t n, void* s) {
     Ptrs<3> in{{a, b, g}};

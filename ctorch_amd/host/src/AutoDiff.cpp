@@ -163,7 +163,8 @@ Tensor AutoDiff::input_gradient(Node* node, size_t input_id, size_t /*input_pos*
                                              "division by zero in the gradient of Div");
             if (first) return Div_AMD_kernel(g, b);                     // g / b
             if (a.sizes() == b.sizes() && g.sizes() == a.sizes()) return div_backward_b(a, b, g);
-            // broadcast divisor: ((-a) * g) / (b * b) with the same operation order, op by op
+            if (is_row_vector_of(b, a) && g.sizes() == a.sizes()) return div_backward_b(a, b, g);   // same order, one pass
+            // any other broadcast divisor: ((-a) * g) / (b * b) with the same operation order, op by op
             Tensor na = Neg_AMD_kernel(a);
             Tensor num = Mul_AMD_kernel(na, g);
             Tensor den = Mul_AMD_kernel(b, b);

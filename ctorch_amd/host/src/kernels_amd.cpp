@@ -292,7 +292,11 @@ Tensor cross_entropy_backward(const Tensor& x, const Tensor& target, const Tenso
 Tensor div_backward_b(const Tensor& a, const Tensor& b, const Tensor& g) {
     check_device(a, "div_backward");
     Tensor r = like(a);
-    run(ctamd_div_backward_b_f32(a.fptr(), b.fptr(), g.fptr(), r.fptr(), a.numel(), current_stream()), "div_backward");
+    if (b.numel() == a.numel())
+        run(ctamd_div_backward_b_f32(a.fptr(), b.fptr(), g.fptr(), r.fptr(), a.numel(), current_stream()), "div_backward");
+    else   // b is a row vector under a [rows, cols]
+        run(ctamd_div_backward_b_rowbcast_f32(a.fptr(), b.fptr(), g.fptr(), r.fptr(), a.sizes()[0], a.sizes()[1],
+                                              current_stream()), "div_backward");
     return r;
 }
 

@@ -206,6 +206,10 @@ int ctamd_cross_entropy_backward_index_f32(const float* x, const float* idx, con
                                            size_t rows, size_t cols, void* stream);
 /* db = ((-a) * g) / (b * b).  src/AutoDiff.cpp:1314.  (da = g / b is ctamd_div_f32, :1285.) */
 int ctamd_div_backward_b_f32(const float* a, const float* b, const float* g, float* db, size_t n, void* stream);
+/* The same for a row-vector divisor b[cols] under a[rows, cols] (the broadcast Div of this backend):
+ * db_full[i, j] = ((-a[i, j]) * g[i, j]) / (b[j] * b[j]); the caller reduces it to b's shape. */
+int ctamd_div_backward_b_rowbcast_f32(const float* a, const float* b, const float* g, float* db_full, size_t rows,
+                                      size_t cols, void* stream);
 
 /* ------------------------------------------- the MNIST demo's path (mnist/, "next" rows) */
 /* dst[i] = src[i] / 255.0f, the loader's pixel normalisation (mnist/mnist_loader.cpp:35-41);

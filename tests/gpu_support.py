@@ -157,6 +157,12 @@ def loss_bwd(name, p, t, g1):
     return dp
 
 
+def div_bwd_b_rowbcast(a, b, g):
+    r = torch.empty_like(a)
+    call("ctamd_div_backward_b_rowbcast_f32", ptr(a), ptr(b), ptr(g), ptr(r), a.shape[0], a.shape[1], stream())
+    return r
+
+
 def div_bwd_b(a, b, g):
     r = torch.empty_like(a)
     call("ctamd_div_backward_b_f32", ptr(a), ptr(b), ptr(g), ptr(r), a.numel(), stream())

@@ -146,6 +146,14 @@ def test_elementwise_gradients(oracle):
     bits_equal(G.host(G.loss_bwd("mae", G.dev(p), G.dev(t), g1)), oracle.mae_bwd(p, t, F(0.37)), "mae bwd")
     b = (t + F(4.0) * np.sign(t) + F(0.5)).astype(F)
     bits_equal(G.host(G.div_bwd_b(G.dev(p), G.dev(b), G.dev(g[:50001]))), oracle.div_bwd_b(p, b, g[:50001]), "div bwd b")
+    # row-vector divisor: the same arithmetic on the divisor repeated down the rows
+    for rows, cols in ((37, 53), (129, 1024), (5, 4100)):
+        a2 = oracle.normal((rows, cols), 81, 0, 2)
+        g2 = oracle.normal((rows, cols), 82)
+        bv = oracle.uniform((cols,), 83, 0.5, 2)
+        d_a, d_b, d_g = G.dev(a2), G.dev(bv), G.dev(g2)
+        bits_equal(G.host(G.div_bwd_b_rowbcast(d_a, d_b, d_g)),
+                   oracle.div_bwd_b(a2, np.ascontiguousarray(np.broadcast_to(bv, (rows, cols))), g2), "div bwd b rowbcast")
     assert G.any_tiny(G.dev(b)) == 0
     b[777] = 1e-8
     assert G.any_tiny(G.dev(b)) == 1 and oracle.any_abs_lt_eps(b)
