@@ -182,6 +182,7 @@ struct Args {
     float* out;          // y / dx
     double* partials;    // per-block loss partials (forward loss modes)
     int32_t* status;     // bad-index flag (kCeIndex), may be null
+    float* stats;        // kCeIndex: per-row (max, sum of exp(x - max)) for a later backward, may be null
     size_t rows, cols;
     // what a row's register copy holds beyond the row's end: four floats of -inf for logits (exp
     // gives exactly 0) and of 0 for the factors of a dot product, in device memory
@@ -237,6 +238,10 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
             block_loss += loss;
         } else if (MODE == kCeIndex) {
             const int c = int(a.t[row]);
+            if (threadIdx.x == 0 && a.stats) {
+                a.stats[2 * row] = m;
+                a.stats[2 * row + 1] = s;
+            }
             if (c < 0 || c >= int(a.cols)) {
                 if (threadIdx.x == 0 && a.status) a.status[0] = 1;
                 block_loss += double(__builtin_nanf(""));
@@ -392,6 +397,10 @@ __global__ __launch_bounds__(1024) void row_stream_kernel(Args a) {
             block_loss += block_sum<THREADS>(loss, s_d);
         } else if (MODE == kCeIndex) {
             const int c = int(a.t[row]);
+            if (threadIdx.x == 0 && a.stats) {
+                a.stats[2 * row] = M;
+                a.stats[2 * row + 1] = S;
+            }
             if (c < 0 || c >= int(a.cols)) {
                 if (threadIdx.x == 0 && a.status) a.status[0] = 1;
                 block_loss += double(__builtin_nanf(""));
@@ -469,6 +478,10 @@ __global__ __launch_bounds__(256) void ce_index_online_kernel(Args a) {
         s = (m == kNegInf) ? 0.0f : s * __builtin_amdgcn_exp2f((m - M) * kLog2e);
         const float S = block_sum<THREADS>(s, s_f[1]);
         const int c = int(a.t[row]);
+        if (threadIdx.x == 0 && a.stats) {
+            a.stats[2 * row] = M;
+            a.stats[2 * row + 1] = S;
+        }
         if (c < 0 || c >= int(a.cols)) {
             if (threadIdx.x == 0 && a.status) a.status[0] = 1;
             block_loss += double(__builtin_nanf(""));
@@ -479,6 +492,50 @@ __global__ __launch_bounds__(256) void ce_index_online_kernel(Args a) {
         }
     }
     if (threadIdx.x == 0) a.partials[blockIdx.x] = block_loss;
+}
+
+// Class-index cross entropy, backward, from the per-row (max, sum) that the forward pass left
+// behind: dx = (exp(x - max) / sum - onehot) * g needs no reduction any more, so it is a pure
+// streaming kernel - nothing of the row is kept, few registers, 8 blocks of 256 threads per CU,
+// the bit-exact exp and the exact quotient of many rows in flight under each other's loads.
+template <bool VEC>
+__global__ __launch_bounds__(256) void ce_bwd_stats_kernel(Args a) {
+    constexpr int THREADS = 256;
+    __shared__ uint64_t s_exp2[32];
+    stage_exp_table(s_exp2);
+    const float g = a.g1[0];
+    for (size_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
+        const float* __restrict__ xr = a.x + row * a.cols;
+        float* __restrict__ outr = a.out + row * a.cols;
+        const float M = a.stats[2 * row];
+        const double rcp_s = 1.0 / double(a.stats[2 * row + 1]);
+        const unsigned c = unsigned(int(a.t[row]));
+        auto one = [&](float v, unsigned j) {
+            float sm = cta_div_rcp(cta_expf_nonpos(v - M, s_exp2), rcp_s);
+            return (sm - ((j == c) ? 1.0f : 0.0f)) * g;
+        };
+        if (VEC) {
+            const unsigned n4 = unsigned(a.cols >> 2);
+            constexpr int U = 4;
+            auto finish4 = [&](v4f v, unsigned i4) {
+                v4f o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = one(v[e], i4 * 4 + e);
+                __builtin_nontemporal_store(o, reinterpret_cast<v4f*>(outr) + i4);
+            };
+            unsigned i = threadIdx.x;
+            for (; i + (U - 1) * THREADS < n4; i += U * THREADS) {
+                v4f v[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(xr) + i + u * THREADS);
+#pragma unroll
+                for (int u = 0; u < U; ++u) finish4(v[u], i + u * THREADS);
+            }
+            for (; i < n4; i += THREADS) finish4(reinterpret_cast<const v4f*>(xr)[i], i);
+        } else {
+            for (size_t j = threadIdx.x; j < a.cols; j += THREADS) outr[j] = one(xr[j], unsigned(j));
+        }
+    }
 }
 
 // out[0] = float(sum of partials), folded in a fixed order.
@@ -607,35 +664,54 @@ using namespace ctamd;
 extern "C" {
 
 int ctamd_softmax_rows_f32(const float* x, float* y, size_t rows, size_t cols, void* stream) {
-    Args a{x, nullptr, nullptr, y, nullptr, nullptr, rows, cols, nullptr, nullptr};
+    Args a{x, nullptr, nullptr, y, nullptr, nullptr, nullptr, rows, cols, nullptr, nullptr};
     return run_rows<kSoftmax>(__func__, a, nullptr, stream);
 }
 int ctamd_cross_entropy_onehot_f32(const float* x, const float* t, float* out, size_t rows, size_t cols, void* stream) {
-    Args a{x, t, nullptr, nullptr, nullptr, nullptr, rows, cols, nullptr, nullptr};
+    Args a{x, t, nullptr, nullptr, nullptr, nullptr, nullptr, rows, cols, nullptr, nullptr};
     return run_rows<kCeOnehot>(__func__, a, out, stream);
 }
 int ctamd_cross_entropy_index_f32(const float* x, const float* idx, float* out, int32_t* status, size_t rows,
                                   size_t cols, void* stream) {
+    return ctamd_cross_entropy_index_stats_f32(x, idx, out, status, nullptr, rows, cols, stream);
+}
+int ctamd_cross_entropy_backward_index_stats_f32(const float* x, const float* idx, const float* stats, const float* g1,
+                                                 float* dx, size_t rows, size_t cols, void* stream) {
+    if (rows == 0 || cols == 0) return CTAMD_OK;
+    if (!x || !idx || !stats || !g1 || !dx) return fail(CTAMD_EINVAL, "%s: null pointer", __func__);
+    if (rows > (size_t(1) << 62) / cols) return fail(CTAMD_ERANGE, "%s: rows*cols overflows", __func__);
+    if (cols > size_t(0x7fffffff)) return fail(CTAMD_ERANGE, "%s: more than 2^31-1 columns", __func__);
+    Args a{x, idx, g1, dx, nullptr, nullptr, const_cast<float*>(stats), rows, cols, nullptr, nullptr};
+    const size_t fill = size_t(compute_units() > 0 ? compute_units() : 256) * 8;
+    const unsigned grid = rows < fill ? unsigned(rows) : unsigned(fill);
+    const bool vec = (cols % 4 == 0) && aligned16(x) && aligned16(dx);
+    if (vec) hipLaunchKernelGGL((ce_bwd_stats_kernel<true>), dim3(grid), dim3(256), 0, as_stream(stream), a);
+    else hipLaunchKernelGGL((ce_bwd_stats_kernel<false>), dim3(grid), dim3(256), 0, as_stream(stream), a);
+    account(8.0 * double(rows) * double(cols) + 12.0 * double(rows), double(rows) * double(cols));
+    return launched(__func__);
+}
+int ctamd_cross_entropy_index_stats_f32(const float* x, const float* idx, float* out, int32_t* status, float* stats,
+                                        size_t rows, size_t cols, void* stream) {
     if (status) {   // cleared by a kernel, not a memset node, so that callers may capture this call
         hipLaunchKernelGGL(clear_i32, dim3(1), dim3(1), 0, as_stream(stream), status);
         int rc = launched(__func__);
         if (rc) return rc;
     }
-    Args a{x, idx, nullptr, nullptr, nullptr, status, rows, cols, nullptr, nullptr};
+    Args a{x, idx, nullptr, nullptr, nullptr, status, stats, rows, cols, nullptr, nullptr};
     return run_rows<kCeIndex>(__func__, a, out, stream);
 }
 int ctamd_cross_entropy_backward_onehot_f32(const float* x, const float* t, const float* g1, float* dx, size_t rows,
                                             size_t cols, void* stream) {
-    Args a{x, t, g1, dx, nullptr, nullptr, rows, cols, nullptr, nullptr};
+    Args a{x, t, g1, dx, nullptr, nullptr, nullptr, rows, cols, nullptr, nullptr};
     return run_rows<kCeBwdOnehot>(__func__, a, nullptr, stream);
 }
 int ctamd_cross_entropy_backward_index_f32(const float* x, const float* idx, const float* g1, float* dx, size_t rows,
                                            size_t cols, void* stream) {
-    Args a{x, idx, g1, dx, nullptr, nullptr, rows, cols, nullptr, nullptr};
+    Args a{x, idx, g1, dx, nullptr, nullptr, nullptr, rows, cols, nullptr, nullptr};
     return run_rows<kCeBwdIndex>(__func__, a, nullptr, stream);
 }
 int ctamd_softmax_backward_rows_f32(const float* y, const float* g, float* dx, size_t rows, size_t cols, void* stream) {
-    Args a{y, g, nullptr, dx, nullptr, nullptr, rows, cols, nullptr, nullptr};
+    Args a{y, g, nullptr, dx, nullptr, nullptr, nullptr, rows, cols, nullptr, nullptr};
     return run_rows<kSoftmaxBwd>(__func__, a, nullptr, stream);
 }
 

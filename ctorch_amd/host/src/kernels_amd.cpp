@@ -274,6 +274,31 @@ Tensor mae_backward(const Tensor& p, const Tensor& t, const Tensor& g) {
     run(ctamd_mae_backward_f32(p.fptr(), t.fptr(), g.fptr(), r.fptr(), p.numel(), current_stream()), "mae_backward");
     return r;
 }
+namespace {
+// Per-row (max, sum) left by the class-index CrossEntropy forward, for its backward: keyed by the
+// ids of the logits and target tensors (ids are never re-used), a handful of entries, oldest out.
+struct CeStats {
+    size_t logits_id = 0, target_id = 0;
+    Tensor stats;
+};
+constexpr int kCeStatsSlots = 4;
+thread_local CeStats t_ce_stats[kCeStatsSlots];
+thread_local int t_ce_next = 0;
+
+void remember_ce_stats(const Tensor& logits, const Tensor& target, Tensor stats) {
+    CeStats& slot = t_ce_stats[t_ce_next];
+    t_ce_next = (t_ce_next + 1) % kCeStatsSlots;
+    slot.logits_id = logits.id();
+    slot.target_id = target.id();
+    slot.stats = std::move(stats);
+}
+const Tensor* recall_ce_stats(const Tensor& logits, const Tensor& target) {
+    for (const CeStats& c : t_ce_stats)
+        if (c.logits_id == logits.id() && c.target_id == target.id() && c.logits_id != 0) return &c.stats;
+    return nullptr;
+}
+}  // namespace
+
 Tensor cross_entropy_backward(const Tensor& x, const Tensor& target, const Tensor& g) {
     check_device(x, "cross_entropy_backward");
     if (x.dim() != 1 && x.dim() != 2)
@@ -283,8 +308,14 @@ Tensor cross_entropy_backward(const Tensor& x, const Tensor& target, const Tenso
     Tensor r = like(x);
     if (x.sizes() == target.sizes())
         run(ctamd_cross_entropy_backward_onehot_f32(x.fptr(), target.fptr(), g.fptr(), r.fptr(), rows, cols, current_stream()), "cross_entropy_backward");
-    else if (target.dim() == 1 && x.dim() == 2 && target.sizes()[0] == rows)
-        run(ctamd_cross_entropy_backward_index_f32(x.fptr(), target.fptr(), g.fptr(), r.fptr(), rows, cols, current_stream()), "cross_entropy_backward");
+    else if (target.dim() == 1 && x.dim() == 2 && target.sizes()[0] == rows) {
+        // with the forward pass's row statistics at hand the backward pass needs no reductions
+        if (const Tensor* stats = recall_ce_stats(x, target))
+            run(ctamd_cross_entropy_backward_index_stats_f32(x.fptr(), target.fptr(), stats->fptr(), g.fptr(), r.fptr(), rows,
+                                                             cols, current_stream()), "cross_entropy_backward");
+        else
+            run(ctamd_cross_entropy_backward_index_f32(x.fptr(), target.fptr(), g.fptr(), r.fptr(), rows, cols, current_stream()), "cross_entropy_backward");
+    }
     else
         Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "cross_entropy_backward: target shape not understood");
     return r;
@@ -350,8 +381,11 @@ Tensor CrossEntropy_AMD_kernel(const Tensor& a, const Tensor& b) {
     if (b.dim() == 1 && a.dim() == 2 && b.sizes()[0] == a.sizes()[0]) {
         Tensor r = scalar0d();
         Tensor status = scalar0d();   // 4 bytes, used as int32
-        run(ctamd_cross_entropy_index_f32(a.fptr(), b.fptr(), r.fptr(), reinterpret_cast<int32_t*>(status.fptr()),
-                                          a.sizes()[0], a.sizes()[1], current_stream()), "CrossEntropy_AMD_kernel");
+        Tensor stats(ShapeTag{}, {a.sizes()[0], 2}, DType::kFloat, DeviceType::kAMD, false);
+        run(ctamd_cross_entropy_index_stats_f32(a.fptr(), b.fptr(), r.fptr(), reinterpret_cast<int32_t*>(status.fptr()),
+                                                stats.fptr(), a.sizes()[0], a.sizes()[1], current_stream()),
+            "CrossEntropy_AMD_kernel");
+        remember_ce_stats(a, b, std::move(stats));
         int32_t bad = 0;
         device_copy_d2h(&bad, status.fptr(), sizeof(bad));
         if (bad) {

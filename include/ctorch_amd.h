@@ -158,6 +158,15 @@ int ctamd_cross_entropy_onehot_f32(const float* x, const float* t, float* out, s
  * Tensor, :96-100) and out[0] is then NaN; status may be NULL. */
 int ctamd_cross_entropy_index_f32(const float* x, const float* idx, float* out, int32_t* status, size_t rows,
                                   size_t cols, void* stream);
+/* The same, also leaving each row's (max, sum_j exp(x_j - max)) in stats[2*row], stats[2*row+1]
+ * (stats may be NULL), and the backward pass that uses them instead of recomputing the row
+ * reductions: dx = (exp(x - max) / sum - onehot(idx)) * g1[0], one streaming pass.  The sum of a
+ * long row (2048 columns or more) comes from the forward pass's fast exponential, ~1e-7 relative
+ * from the sum of the rounded terms. */
+int ctamd_cross_entropy_index_stats_f32(const float* x, const float* idx, float* out, int32_t* status, float* stats,
+                                        size_t rows, size_t cols, void* stream);
+int ctamd_cross_entropy_backward_index_stats_f32(const float* x, const float* idx, const float* stats, const float* g1,
+                                                 float* dx, size_t rows, size_t cols, void* stream);
 
 /* -------------------------------------------------------------------------------- matmul */
 /* C[i,j] = sum_l A[i*as0 + l*as1] * B[l*bs0 + j*bs1]; C is [m, n] row-major contiguous; strides

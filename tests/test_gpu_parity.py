@@ -232,6 +232,38 @@ def test_softmax_and_cross_entropy_rows(oracle, shape):
     assert np.all(np.abs(got - want_b) <= 1e-5 * scale + 1e-12)
 
 
+@pytest.mark.parametrize("shape", [(64, 10), (19, 301), (4, 2052), (3, 8192), (2, 33000), (3, 40001)])
+def test_cross_entropy_backward_from_forward_statistics(oracle, shape):
+    """The class-index forward pass leaves (max, sum) per row; the backward pass that uses them
+    agrees with the oracle's dlogits and with the backward pass that recomputes them."""
+    print("case ce stats", shape, flush=True)
+    rows, cols = shape
+    x = oracle.normal(shape, 90, 0, 2)
+    idx = oracle.ints((rows,), 91, cols)
+    dx, didx = G.dev(x), G.dev(idx)
+    loss = torch.empty(1, device=G.DEV)
+    status = torch.zeros(1, dtype=torch.int32, device=G.DEV)
+    stats = torch.empty(rows, 2, device=G.DEV)
+    G.call("ctamd_cross_entropy_index_stats_f32", G.ptr(dx), G.ptr(didx), G.ptr(loss), G.ptr(status), G.ptr(stats), rows,
+           cols, G.stream())
+    st = G.host(stats)
+    x64 = x.astype(np.float64)
+    assert int(status.item()) == 0 and np.array_equal(st[:, 0], x.max(1))
+    s64 = np.exp(x64 - x64.max(1, keepdims=True)).sum(1)
+    assert np.all(np.abs(st[:, 1] - s64) <= 1e-5 * s64)
+    want_loss = oracle.ce_index(x, idx)
+    assert abs(G.host(loss)[0] - want_loss) <= 1e-5 * abs(want_loss)
+    g1 = G.dev(np.array([0.75]))
+    out = torch.empty_like(dx)
+    G.call("ctamd_cross_entropy_backward_index_stats_f32", G.ptr(dx), G.ptr(didx), G.ptr(stats), G.ptr(g1), G.ptr(out),
+           rows, cols, G.stream())
+    oh = np.zeros(shape, F)
+    oh[np.arange(rows), idx.astype(int)] = 1
+    want = oracle.ce_bwd_onehot(x, oh, F(0.75))
+    assert np.abs(G.host(out) - want).max() <= 1e-6
+    assert np.abs(G.host(out) - G.host(G.ce_bwd(dx, didx, g1, True))).max() <= 2e-7
+
+
 def test_cross_entropy_edge_cases(oracle):
     print("case ce edges", flush=True)
     x = oracle.normal((19, 31), 28, 0, 2)
