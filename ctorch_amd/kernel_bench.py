@@ -1,0 +1,142 @@
+"""Per-kernel timings of the launch layer through the C ABI on one MI355X.
+
+    python -m ctorch_amd.kernel_bench [--json] [--skip-matmul]
+
+Every operator is launched on operands resident in HBM (torch only provides the memory and the
+stream), timed with events over back-to-back launches after a warm-up, and reported as time,
+achieved rate and fraction of the published peak (8 TB/s HBM, 157.3 TFLOP/s fp32 matrix), with the
+algorithmic bytes per element each operator must move.  Tensors smaller than the 256 MiB memory-side
+cache rotate through four buffer sets so that the cache cannot serve the traffic.  Run it under
+`rocprofv3 --kernel-trace --stats` to get the same kernels' durations from the profiler.
+"""
+import argparse
+import ctypes as C
+import json
+import sys
+
+HBM_PEAK = 8.0e12
+MFMA_F32_PEAK = 157.3e12
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--json", action="store_true", help="one JSON object instead of a table")
+    ap.add_argument("--skip-matmul", action="store_true")
+    args = ap.parse_args()
+
+    import torch
+    from ctorch_amd import capi
+
+    lib = capi.load()
+    torch.cuda.init()
+    torch.zeros(1, device="cuda:0")
+    capi.check(lib.ctamd_init(0))
+    S = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    P = lambda t: C.c_void_p(t.data_ptr())
+    call = lambda name, *a: capi.check(getattr(lib, name)(*a))
+    results = []
+
+    def timeit(fn, reps, warm=3):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps * 1e-3
+
+    def report(name, seconds, nbytes=None, flops=None):
+        e = {"kernel": name, "us": round(seconds * 1e6, 1)}
+        if nbytes is not None:
+            e.update({"GB/s": round(nbytes / seconds / 1e9, 1), "frac_of_hbm_peak": round(nbytes / seconds / HBM_PEAK, 4)})
+        if flops is not None:
+            e.update({"TFLOP/s": round(flops / seconds / 1e12, 2), "frac_of_mfma_peak": round(flops / seconds / MFMA_F32_PEAK, 4)})
+        results.append(e)
+        if not args.json:
+            rate = ("%8.1f GB/s %5.1f%% of 8 TB/s" % (e["GB/s"], 100 * e["frac_of_hbm_peak"]) if nbytes is not None else
+                    "%8.2f TFLOP/s %5.1f%% of 157.3" % (e["TFLOP/s"], 100 * e["frac_of_mfma_peak"]))
+            print("%-44s %9.1f us  %s" % (name, e["us"], rate), flush=True)
+
+    # ---- elementwise, scalar, fill, reductions: 2^26 elements (256 MiB per tensor), four buffer sets
+    n, sets = 1 << 26, 4
+    A = [torch.randn(n, device="cuda") for _ in range(sets)]
+    B = [torch.randn(n, device="cuda").abs_() + 0.5 for _ in range(sets)]
+    R = [torch.empty(n, device="cuda") for _ in range(sets)]
+    out = torch.empty(1, device="cuda")
+    turn = [0]
+
+    def rotating(fn):
+        def f():
+            k = turn[0] % sets
+            turn[0] += 1
+            fn(k)
+        return f
+
+    def ew(name, fn, bytes_per_elem):
+        report("%s, n=2^26 (%d B/elem)" % (name, bytes_per_elem), timeit(rotating(fn), 20), bytes_per_elem * n)
+
+    for op in ("add", "sub", "mul", "div"):
+        ew(op, lambda k, op=op: call("ctamd_%s_f32" % op, P(A[k]), P(B[k]), P(R[k]), n, S), 12)
+    for op in ("neg", "relu", "sin", "cos", "tanh", "sigmoid"):
+        ew(op, lambda k, op=op: call("ctamd_%s_f32" % op, P(A[k]), P(R[k]), n, S), 8)
+    for op in ("relu", "sigmoid", "tanh", "sin", "cos"):
+        ew(op + " backward", lambda k, op=op: call("ctamd_%s_backward_f32" % op, P(A[k]), P(B[k]), P(R[k]), n, S), 12)
+    ew("tensor + scalar", lambda k: call("ctamd_add_scalar_f32", P(A[k]), C.c_float(5.0), P(R[k]), n, S), 8)
+    ew("fill", lambda k: call("ctamd_fill_f32", P(R[k]), C.c_float(5.0), n, S), 4)
+    ew("accumulate", lambda k: call("ctamd_accumulate_f32", P(R[k]), P(A[k]), n, S), 12)
+    ew("sgd step", lambda k: call("ctamd_sgd_step_f32", P(R[k]), P(A[k]), C.c_float(0.01), n, S), 12)
+    ew("row-broadcast div [16384 x 4096]", lambda k: call("ctamd_div_rowbcast_f32", P(A[k]), P(B[0]), P(R[k]), 16384, 4096, S), 8)
+    ew("sum", lambda k: call("ctamd_sum_f32", P(A[k]), P(out), n, S), 4)
+    ew("dot", lambda k: call("ctamd_dot_f32", P(A[k]), P(B[k]), P(out), n, S), 8)
+    ew("mse", lambda k: call("ctamd_mse_f32", P(A[k]), P(B[k]), P(out), n, S), 8)
+    ew("mae", lambda k: call("ctamd_mae_f32", P(A[k]), P(B[k]), P(out), n, S), 8)
+    cs = torch.empty(4096, device="cuda")
+    ew("column sum [16384 x 4096]", lambda k: call("ctamd_colsum_f32", P(A[k]), P(cs), 16384, 4096, S), 4)
+    del A, B, R
+    torch.cuda.empty_cache()
+
+    # ---- row softmax / cross entropy at [8192 x 32000]
+    rows, cols = 8192, 32000
+    m = rows * cols
+    X = torch.randn(rows, cols, device="cuda") * 2
+    Y = torch.empty_like(X)
+    idx = torch.randint(0, cols, (rows,), device="cuda").float()
+    g1 = torch.ones(1, device="cuda")
+    status = torch.zeros(1, dtype=torch.int32, device="cuda")
+    stats = torch.empty(rows, 2, device="cuda")
+
+    def row(name, fn, bytes_per_elem):
+        report("%s [8192 x 32000] (%d B/elem)" % (name, bytes_per_elem), timeit(fn, 10), bytes_per_elem * m)
+
+    row("softmax rows", lambda: call("ctamd_softmax_rows_f32", P(X), P(Y), rows, cols, S), 8)
+    row("cross entropy (class index) forward", lambda: call("ctamd_cross_entropy_index_stats_f32", P(X), P(idx), P(out),
+                                                            P(status), P(stats), rows, cols, S), 4)
+    row("cross entropy (class index) backward", lambda: call("ctamd_cross_entropy_backward_index_f32", P(X), P(idx), P(g1),
+                                                             P(Y), rows, cols, S), 8)
+    row("cross entropy backward from forward statistics", lambda: call("ctamd_cross_entropy_backward_index_stats_f32", P(X),
+                                                                       P(idx), P(stats), P(g1), P(Y), rows, cols, S), 8)
+    row("softmax backward rows", lambda: call("ctamd_softmax_backward_rows_f32", P(Y), P(X), P(Y), rows, cols, S), 12)
+    del X, Y
+    torch.cuda.empty_cache()
+
+    # ---- fp32 MatMul, square, the three operand layouts
+    if not args.skip_matmul:
+        for M in (1024, 2048, 4096, 8192):
+            a, b = torch.randn(M, M, device="cuda"), torch.randn(M, M, device="cuda")
+            c = torch.empty(M, M, device="cuda")
+            for name, (x, y) in (("A.B", (a, b)), ("A.B^T", (a, b.t())), ("A^T.B", (a.t(), b))):
+                fn = lambda x=x, y=y: call("ctamd_matmul_f32", P(x), x.stride(0), x.stride(1), P(y), y.stride(0), y.stride(1),
+                                           P(c), M, M, M, S)
+                report("matmul %s %d^3" % (name, M), timeit(fn, 20 if M < 8192 else 4, warm=8 if M < 8192 else 2),
+                       flops=2.0 * M ** 3)
+            del a, b, c
+    if args.json:
+        print(json.dumps({"device": torch.cuda.get_device_name(0), "results": results}))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
