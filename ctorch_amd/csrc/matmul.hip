@@ -471,6 +471,7 @@ extern "C" int ctamd_matmul_f32(const float* a, int64_t as0, int64_t as1, const 
         int64_t max_by_scratch = int64_t(kScratchFloats) / (m * n);
         splits = int(want < max_by_k ? want : max_by_k);
         if (splits > max_by_scratch) splits = int(max_by_scratch);
+        if (splits < 4) splits = 1;                 // a two- or three-way split does not pay for its fold launch
         if (splits > 1) {
             partial = scratch();
             if (!partial) return CTAMD_EINVAL;

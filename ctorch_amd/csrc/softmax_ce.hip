@@ -602,6 +602,7 @@ int run_rows(const char* name, Args a, float* loss_out, void* stream) {
     const int threads = groups <= 64 * 8 ? 64 : groups <= 256 * 8 ? 256 : 1024;
     size_t fill = size_t(compute_units() > 0 ? compute_units() : 256) * size_t(2048 / threads);
     if (fill > kMaxRowBlocks) fill = kMaxRowBlocks;
+    if (kLoss && fill > 2048) fill = 2048;         // one partial per block: keep the fold of the partials short
     unsigned grid = a.rows < fill ? unsigned(a.rows) : unsigned(fill);
     bool vec = (a.cols % 4 == 0) && aligned16(a.x) && (MODE == kSoftmax || MODE == kCeIndex || MODE == kCeBwdIndex || aligned16(a.t)) &&
                (kLoss || aligned16(a.out));
