@@ -315,6 +315,55 @@ long cth_expr(const float* X, const float* R, const float* T, long rows, long co
     }
 }
 
+// A small straight-line program over tensors, for differential tests of the tape.  Values 0 ..
+// n_in-1 are the inputs (kinds[i] = 0: [rows, cols], 1: row vector [cols]; all require gradients),
+// each op (code, a, b) appends one value: codes 0-3 Add/Sub/Mul/Div of values a and b (same kind,
+// or Add of a full tensor and a row vector), 20-25 the unary operators of value a, 30/31/32
+// value a (+, *, /) the scalar 0.5 + 0.25 * b.  The last value must be a full tensor: it is
+// copied to y_out, L = sum(last * w) goes to l_out, and after backward(L) the gradients of the
+// inputs are written to grads_out one after the other.
+long cth_program(const float* inputs, const int* kinds, int n_in, const int* ops, int n_ops, const float* w,
+                 long rows, long cols, float* y_out, float* l_out, float* grads_out) {
+    try {
+        AutoDiff ctx;
+        configure(ctx);
+        AutoDiffContext::Guard guard(&ctx);
+        long full[2] = {rows, cols}, vec[1] = {cols};
+        std::vector<Tensor> v;
+        v.reserve(size_t(n_in + n_ops));
+        const float* src = inputs;
+        for (int i = 0; i < n_in; ++i) {
+            v.push_back(kinds[i] ? make(src, vec, 1) : make(src, full, 2));
+            src += kinds[i] ? cols : rows * cols;
+        }
+        for (int i = 0; i < n_in; ++i) v[size_t(i)].requires_grad(true);
+        for (int k = 0; k < n_ops; ++k) {
+            const int code = ops[3 * k], a = ops[3 * k + 1], b = ops[3 * k + 2];
+            if (code < 20) v.push_back(run_binary(code, v[size_t(a)], v[size_t(b)]));
+            else if (code < 30) v.push_back(run_unary(code, v[size_t(a)]));
+            else {
+                const float s = 0.5f + 0.25f * float(b);
+                v.push_back(code == 30 ? v[size_t(a)] + s : code == 31 ? v[size_t(a)] * s : v[size_t(a)] / s);
+            }
+        }
+        Tensor tw = make(w, full, 2);
+        Tensor z = v.back() * tw;
+        Tensor L = z.sum();
+        if (emit(v.back(), y_out) < 0) return -2;
+        l_out[0] = L.item<float>();
+        backward(L);
+        float* dst = grads_out;
+        for (int i = 0; i < n_in; ++i) {
+            long got = emit(grad(v[size_t(i)]), dst);
+            if (got < 0) return -2;
+            dst += got;
+        }
+        return long(dst - grads_out);
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
 // ------------------------------------------------------------------------- timed steps
 // The same graphs as above with every input resident in HBM before the clock starts: `warm`
 // untimed steps, then `reps` timed ones between two device synchronisations.  A step builds its

@@ -23,6 +23,34 @@ SPECIAL = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 3.4e38, -
                    np.float32)
 
 
+PROGRAM_SEEDS = range(60)
+
+
+def program_shape(seed):
+    return (6, 8) if seed < 45 else (21, 36)
+
+
+def programs():
+    """Random straight-line programs through the reference's tape (support.random_program): the last
+    value, L and the gradients of every input, as the reference computes them."""
+    from support import program_inputs, random_program
+    o = Oracle()
+    r = Reference()
+    g = {}
+    for seed in PROGRAM_SEEDS:
+        rows, cols = program_shape(seed)
+        kinds, ops = random_program(seed)
+        xs, w = program_inputs(o, seed, kinds, rows, cols)
+        rc, y, L, grads = r.program(xs, kinds, ops, w)
+        assert rc >= 0, seed
+        g["p%d_kinds" % seed] = np.array(kinds, np.int32)
+        g["p%d_ops" % seed] = np.array(ops, np.int32)
+        g["p%d_y" % seed], g["p%d_L" % seed] = y, L
+        for i, t in enumerate(grads):
+            g["p%d_g%d" % (seed, i)] = t
+    np.savez_compressed(os.path.join(HERE, "programs.npz"), **g)
+
+
 def mnist():
     """The MNIST demo's path: loader, accuracy, the training loop over the reference library, and
     the printed results of the demo program's own main() on the synthetic data set."""
@@ -235,6 +263,9 @@ def main():
 if __name__ == "__main__":
     if "mnist" in sys.argv[1:]:
         mnist()
+    elif "programs" in sys.argv[1:]:
+        programs()
     else:
         main()
         mnist()
+        programs()

@@ -383,6 +383,123 @@ def libc_xavier(shape, fan_in, reseed=None):
     return (r.astype(np.float32) * np.sqrt(np.float32(1.0) / np.float32(fan_in))).astype(np.float32).reshape(shape)
 
 
+def random_program(seed, rows=6, cols=8, n_in=4, n_ops=14):
+    """A random straight-line program for the tape tests: (kinds, ops).  Inputs 0..n_in-1 (kind 0 =
+    [rows, cols], 1 = row vector; input 0 is always full, the last input is a positive divisor), ops
+    = (code, a, b) as the program entry points of the two C doorways understand them.  Values are
+    re-used freely, so nodes receive several gradient contributions; some ops use one value twice."""
+    rng = np.random.default_rng(seed)
+    kinds = [0] + [int(rng.integers(0, 4) == 0) for _ in range(n_in - 2)] + [0]
+    vals = list(kinds)                          # kind of every value so far
+    ops = []
+    full = lambda: [i for i, k in enumerate(vals) if k == 0]
+    vecs = lambda: [i for i, k in enumerate(vals) if k == 1]
+    for step in range(n_ops):
+        r = rng.integers(0, 10)
+        if r < 5:                                # binary
+            code = int(rng.integers(0, 4))
+            if code == 3:                        # Div: only by the positive input, same shape
+                a, b = int(rng.choice(full())), n_in - 1
+            elif code == 0 and vecs() and rng.integers(0, 2):
+                a, b = int(rng.choice(full())), int(rng.choice(vecs()))       # full + row vector
+            else:
+                pool = full() if (not vecs() or rng.integers(0, 3)) else vecs()
+                a = int(rng.choice(pool))
+                b = a if rng.integers(0, 6) == 0 else int(rng.choice(pool))  # now and then x (op) x
+            ops.append((code, a, b))
+            vals.append(vals[a])
+        elif r < 8:                              # unary
+            a = int(rng.integers(0, len(vals)))
+            ops.append((int(rng.choice([20, 21, 22, 23, 24, 25])), a, 0))
+            vals.append(vals[a])
+        else:                                    # scalar
+            a = int(rng.integers(0, len(vals)))
+            ops.append((int(rng.choice([30, 31])), a, int(rng.integers(0, 6))))   # no tensor / scalar: the reference's gradient of it reads out of bounds
+            vals.append(vals[a])
+    # fold every value that nothing has consumed into the result, so that no input is dead code and
+    # the last value is a full tensor
+    used = {a for _, a, _ in ops} | {b for c, _, b in ops if c < 20}
+    acc = full()[-1]
+    for i in range(len(vals) - 1, -1, -1):
+        if i in used or i == acc:
+            continue
+        ops.append((0, acc, i) if vals[i] == 1 or vals[acc] == 0 else (0, i, acc))
+        vals.append(0)
+        acc = len(vals) - 1
+    if acc != len(vals) - 1:
+        ops.append((30, acc, 0))
+        vals.append(0)
+    return kinds, ops
+
+
+def program_fp64(inputs, kinds, ops, w, row0=True, same_operand_as_first=True):
+    """The same program by a small fp64 reverse-mode interpreter (an independent statement of the
+    mathematics).  row0: the gradient of a row vector added to a full tensor is row 0 of the upstream
+    gradient, as the reference computes it; False gives the column sum.  same_operand_as_first: in
+    x - x and x / x the reference treats both visits of the operand as the first one (it tells
+    operands apart by tensor id, src/AutoDiff.cpp:1222-1233, :1259-1316), giving 2g and 2g/x where
+    the mathematics gives 0.  Returns (y, L, grads)."""
+    v = [np.asarray(x, np.float64) for x in inputs]
+    for code, a, b in ops:
+        x = v[a]
+        if code < 20:
+            z = v[b]
+            v.append(x + z if code == 0 else x - z if code == 1 else x * z if code == 2 else x / z)
+        elif code < 30:
+            v.append({20: lambda t: -t, 21: lambda t: np.maximum(t, 0), 22: np.sin, 23: np.cos, 24: np.tanh,
+                      25: lambda t: 1 / (1 + np.exp(-t))}[code](x))
+        else:
+            sc = 0.5 + 0.25 * b
+            v.append(x + sc if code == 30 else x * sc)
+    g = [np.zeros_like(t) for t in v]
+    g[-1] = np.asarray(w, np.float64).copy()
+
+    def push(i, val):
+        if g[i].shape != val.shape:
+            val = val[0] if row0 else val.sum(0)
+        g[i] = g[i] + val
+
+    for k in range(len(ops) - 1, -1, -1):
+        code, a, b = ops[k]
+        out = len(inputs) + k
+        go, x = g[out], v[a]
+        if code == 0:
+            push(a, go); push(b, go)
+        elif code == 1:
+            push(a, go); push(b, go if (a == b and same_operand_as_first) else -go)
+        elif code == 2:
+            push(a, go * v[b]); push(b, go * x)
+        elif code == 3:
+            push(a, go / v[b]); push(b, go / v[b] if (a == b and same_operand_as_first) else -x * go / (v[b] * v[b]))
+        elif code == 20:
+            push(a, -go)
+        elif code == 21:
+            push(a, go * (x > 0))
+        elif code == 22:
+            push(a, go * np.cos(x))
+        elif code == 23:
+            push(a, -go * np.sin(x))
+        elif code == 24:
+            push(a, go * (1 - np.tanh(x) ** 2))
+        elif code == 25:
+            sg = 1 / (1 + np.exp(-x))
+            push(a, go * sg * (1 - sg))
+        elif code == 30:
+            push(a, go)
+        else:
+            push(a, go * (0.5 + 0.25 * b))
+    return v[-1], float((v[-1] * np.asarray(w, np.float64)).sum()), g[:len(inputs)]
+
+
+def program_inputs(oracle, seed, kinds, rows, cols):
+    xs = []
+    for i, k in enumerate(kinds):
+        shape = (cols,) if k else (rows, cols)
+        lo, hi = (0.5, 2.0) if i == len(kinds) - 1 else (-1.5, 1.5)
+        xs.append(oracle.uniform(shape, 7000 + 10 * seed + i, lo, hi))
+    return xs, oracle.uniform((rows, cols), 7000 + 10 * seed + 9, -1, 1)
+
+
 def write_idx_images(path, pixels_u8):
     """IDX3 file as the MNIST loader reads it (mnist/mnist_loader.cpp:7-44): big-endian magic 2051,
     count, rows, cols, then one unsigned byte per pixel.  pixels_u8: [n, rows, cols] uint8."""
@@ -551,6 +668,26 @@ class Reference:
                                C.byref(mae), fp(gX), fp(gR), *extra)
         assert rc == rows * cols, rc
         return Y, np.float32(mse.value), np.float32(mae.value), gX, gR
+
+    def program(self, inputs, kinds, ops, w):
+        """Runs a straight-line program (see random_program) through the tape; returns
+        (rc, last value, L, [gradients of the inputs])."""
+        rows, cols = w.shape
+        flat = np.concatenate([f32(x).ravel() for x in inputs])
+        kinds_a = (C.c_int * len(kinds))(*kinds)
+        ops_a = (C.c_int * (3 * len(ops)))(*[v for op in ops for v in op])
+        y = np.empty((rows, cols), np.float32)
+        L = C.c_float(0)
+        grads = np.empty(flat.size, np.float32)
+        fn = self.lib.ref_program
+        fn.restype = C.c_long
+        rc = fn(fp(flat), kinds_a, C.c_int(len(kinds)), ops_a, C.c_int(len(ops)), fp(f32(w)), C.c_long(rows),
+                C.c_long(cols), fp(y), C.byref(L), fp(grads))
+        out, pos = [], 0
+        for x in inputs:
+            out.append(grads[pos:pos + x.size].reshape(x.shape).copy())
+            pos += x.size
+        return rc, y, np.float32(L.value), out
 
     # ---- the MNIST demo (oracle/ref_mnist_driver.cpp); reference build only
     def mnist_load(self, directory, train):

@@ -201,3 +201,34 @@ def test_reference_style_programs(prog):
     p = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=110)
     print(p.stdout[-3000:])
     assert p.returncode == 0
+
+
+def test_tape_programs_against_the_reference_vectors(oracle, host, golden):
+    """Sixty random straight-line programs (values re-used, several gradient contributions per node,
+    x (op) x, row-vector operands) through the device tape: the forward value and every input
+    gradient must have the bits the real reference produced - the operators are bit-exact and the
+    tape adds the contributions in the reference's order; L = sum(...) to the reduction bar."""
+    import importlib.util
+    import os
+    from support import program_inputs, random_program
+    spec = importlib.util.spec_from_file_location("make_golden", os.path.join(os.path.dirname(__file__), "golden",
+                                                                            "make_golden.py"))
+    mg = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mg)
+    g = golden("programs")
+    host.set_reference_row0(True)
+    try:
+        for seed in mg.PROGRAM_SEEDS:
+            print("case program", seed, flush=True)
+            rows, cols = mg.program_shape(seed)
+            kinds, ops = random_program(seed)
+            xs, w = program_inputs(oracle, seed, kinds, rows, cols)
+            rc, y, L, grads = host.program(xs, kinds, ops, w)
+            assert rc >= 0, seed
+            assert same_bits(y, g["p%d_y" % seed]), seed
+            want_L = float(g["p%d_L" % seed])
+            assert abs(float(L) - want_L) <= 1e-5 * float(np.abs(y * w).astype(np.float64).sum()) + 1e-30
+            for i, got in enumerate(grads):
+                assert same_bits(got, g["p%d_g%d" % (seed, i)]), (seed, i)
+    finally:
+        host.set_reference_row0(False)

@@ -163,3 +163,29 @@ def test_mnist_path(oracle, golden):
     train_acc = F(oracle.count_correct(oracle.mnist_predict(x, trained), y)) / F(512)
     test_acc = F(oracle.count_correct(oracle.mnist_predict(xt, trained), te_l.astype(F))) / F(256)
     assert ["%.2f" % (train_acc * 100), "%.2f" % (test_acc * 100)] == [str(v) for v in g["demo_accuracies"]]
+
+
+def test_tape_programs_against_an_fp64_interpreter(golden):
+    """Random straight-line programs through the reference's tape (vectors written from the real
+    reference) against an independent fp64 reverse-mode interpreter that models the two properties
+    of the reference's tape that differ from the mathematics (row-0 gradients of broadcast row
+    vectors; x - x and x / x treated as two 'first' operands)."""
+    import importlib.util
+    import os
+    from support import Oracle, program_fp64, program_inputs, random_program
+    spec = importlib.util.spec_from_file_location("make_golden", os.path.join(os.path.dirname(__file__), "golden",
+                                                                            "make_golden.py"))
+    mg = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mg)
+    g = golden("programs")
+    o = Oracle()
+    for seed in mg.PROGRAM_SEEDS:
+        rows, cols = mg.program_shape(seed)
+        kinds, ops = random_program(seed)
+        assert np.array_equal(g["p%d_kinds" % seed], kinds) and np.array_equal(g["p%d_ops" % seed], np.array(ops))
+        xs, w = program_inputs(o, seed, kinds, rows, cols)
+        y64, L64, g64 = program_fp64(xs, kinds, ops, w)
+        assert np.abs(g["p%d_y" % seed] - y64).max() <= 1e-5 * (1 + np.abs(y64).max())
+        for i, want in enumerate(g64):
+            got = g["p%d_g%d" % (seed, i)]
+            assert np.abs(got - want).max() <= 1e-5 * (1 + np.abs(want).max()), (seed, i)
