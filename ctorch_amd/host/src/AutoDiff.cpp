@@ -3,6 +3,9 @@
 // deliberate differences.
 #include "AutoDiff.h"
 
+#include <cfloat>
+#include <cmath>
+
 #include <algorithm>
 
 #include "Ctorch_Scheduler.h"
@@ -150,6 +153,8 @@ Tensor AutoDiff::input_gradient(Node* node, size_t input_id, size_t /*input_pos*
             Node* o = other_node();
             if (!o) return Tensor::alias(g);
             const Tensor& other = *o->tensor;
+            if (other.device() == DeviceType::kCPU && other.numel() == 1)       // tensor * float: s * g
+                return scalar_op(g, other.item<float>(), op::Mul);
             if (is_row_vector_of(other, g)) return Mul_AMD_kernel(g, other);   // row-broadcast operand
             return Mul_AMD_kernel(other, g);
         }
@@ -158,6 +163,15 @@ Tensor AutoDiff::input_gradient(Node* node, size_t input_id, size_t /*input_pos*
             Node* b_node = find(node->input_ids[1]);
             const Tensor& a = *a_node->tensor;
             const Tensor& b = *b_node->tensor;
+            if (b.device() == DeviceType::kCPU && b.numel() == 1) {             // tensor / float
+                const float sv = b.item<float>();
+                if (check_div_zero_ && std::fabs(sv) < FLT_EPSILON)
+                    Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::TENSOR_STATE,
+                                                 "division by zero in the gradient of Div");
+                if (first) return scalar_op(g, sv, op::Div);                    // g / s
+                Ctorch_Error::throwException(ErrorPlatform::kAutoDiff, ErrorType::TENSOR_STATE,
+                                             "backward: a host scalar operand has no gradient");
+            }
             if (check_div_zero_ && any_abs_lt_eps(b))
                 Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::TENSOR_STATE,
                                              "division by zero in the gradient of Div");
@@ -214,6 +228,14 @@ Tensor AutoDiff::input_gradient(Node* node, size_t input_id, size_t /*input_pos*
 // src/AutoDiff.cpp:548-553
 void AutoDiff::backward(Tensor& root) {
     AutoDiffContext::Guard guard(nullptr);
+    // the seed 1.0 on the device is made once per thread and shared (the tape never writes through
+    // a shared gradient: accumulation goes to a fresh tensor then)
+    thread_local Tensor device_one;
+    if (root.device() == DeviceType::kAMD) {
+        if (device_one.is_cleared()) device_one = Tensor(1.0f, DeviceType::kAMD);
+        backward(root, Tensor::alias(device_one));
+        return;
+    }
     Tensor grad_output(1.0f, root.device());
     backward(root, std::move(grad_output));
 }

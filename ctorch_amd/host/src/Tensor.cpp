@@ -295,7 +295,10 @@ namespace {
 Tensor with_scalar(const Tensor& a, float s, op o) {
     Tensor result = scalar_op(a, s, o);
     if (AutoDiffContext::current()) {
-        Tensor scalar_tensor(s, a.device());
+        // the taped second input stays on the host: its value is only needed by the gradient of
+        // tensor * s and tensor / s, which take it as a launch argument (a device copy of it would
+        // cost an allocation and a fill launch per scalar operator)
+        Tensor scalar_tensor(s);
         tape(result, o, {&a, &scalar_tensor});
         result.set_requires_grad(a.requires_grad());
     } else {
