@@ -198,6 +198,13 @@ def config_report(with_cpu):
             else:
                 cpu, note = cpu256 * 32, "batch-256 step x32 (every operator is linear in the batch)"
         add("config 3: MLP 784-256-10 train step, batch %d" % Bn, rc, out, cpu, note, launch_bound=(Bn == 256))
+        # each layer (matmul + bias row + ReLU) as one fused operator: same values, fewer launches
+        host.cth_set_fused_layers(1)
+        out = D5()
+        rc = host.cth_time_mlp(fp(x), L(Bn), L(784), fp(W1), fp(b1), L(256), fp(W2), fp(b2), L(10), fp(lab), I(5),
+                               I(30), out)
+        host.cth_set_fused_layers(0)
+        add("config 3: MLP 784-256-10 train step, batch %d, fused layers" % Bn, rc, out, cpu, note, launch_bound=(Bn == 256))
         # the same step (one-hot targets) recorded into a HIP graph once and replayed
         oh = np.zeros((Bn, 10), np.float32)
         oh[np.arange(Bn), lab.astype(int)] = 1

@@ -407,6 +407,39 @@ int dev_scalar(const char* name, const float* a, const float* b1, float* r, size
     return launch_map<DevScalarF<Op>>(name, in, r, n, DevScalarF<Op>{b1}, stream);
 }
 
+
+// ---- the optimiser update of several tensors in one launch
+constexpr int kSgdMaxTensors = 32;
+constexpr int kSgdChunk = kThreads * 8;          // elements per block
+struct SgdBatch {
+    float* param[kSgdMaxTensors];
+    const float* grad[kSgdMaxTensors];
+    unsigned count[kSgdMaxTensors];
+    unsigned first_block[kSgdMaxTensors + 1];    // block range of tensor t: [first_block[t], first_block[t+1])
+    int tensors;
+    float lr;
+};
+// param -= (0 + grad) * lr, the three operations rounded one by one.  "0 +" is what reading a
+// gradient from the reference's tape does (a zero-filled buffer that contributions are added to,
+// src/AutoDiff.cpp:1870-1907): it turns a -0 gradient into +0, which matters to the sign of a
+// zero parameter only.
+__global__ __launch_bounds__(kThreads) void sgd_multi_kernel(SgdBatch b) {
+    int t = 0;
+    while (t + 1 < b.tensors && blockIdx.x >= b.first_block[t + 1]) ++t;
+    const unsigned begin = (blockIdx.x - b.first_block[t]) * unsigned(kSgdChunk);
+    float* __restrict__ p = b.param[t];
+    const float* __restrict__ g = b.grad[t];
+    const unsigned n = b.count[t];
+#pragma unroll
+    for (int u = 0; u < kSgdChunk / kThreads; ++u) {
+        unsigned i = begin + unsigned(u) * kThreads + threadIdx.x;
+        if (i < n) {
+            float step = (0.0f + g[i]) * b.lr;
+            p[i] = p[i] - step;
+        }
+    }
+}
+
 }  // namespace
 }  // namespace ctamd
 
@@ -471,6 +504,39 @@ int ctamd_accumulate_f32(float* grad, const float* val, size_t n, void* s) {
 int ctamd_sgd_step_f32(float* param, const float* grad, float lr, size_t n, void* s) {
     Ptrs<2> in{{param, grad}};
     return launch_map<SgdF>(__func__, in, param, n, SgdF{lr}, s);
+}
+int ctamd_sgd_step_multi_f32(float* const* params, const float* const* grads, const size_t* counts, int tensors, float lr,
+                             void* stream) {
+    if (tensors < 0) return fail(CTAMD_EINVAL, "%s: negative tensor count", __func__);
+    if (tensors && (!params || !grads || !counts)) return fail(CTAMD_EINVAL, "%s: null table", __func__);
+    hipStream_t s = as_stream(stream);
+    for (int done = 0; done < tensors;) {
+        SgdBatch b;
+        b.tensors = 0;
+        b.lr = lr;
+        b.first_block[0] = 0;
+        double bytes = 0;
+        while (done < tensors && b.tensors < kSgdMaxTensors) {
+            const size_t n = counts[done];
+            if (n > 0xffffffffu - unsigned(kSgdChunk)) return fail(CTAMD_ERANGE, "%s: tensor too large", __func__);
+            if (n && (!params[done] || !grads[done])) return fail(CTAMD_EINVAL, "%s: null tensor", __func__);
+            if (n) {
+                const int t = b.tensors++;
+                b.param[t] = params[done];
+                b.grad[t] = grads[done];
+                b.count[t] = unsigned(n);
+                b.first_block[t + 1] = b.first_block[t] + unsigned((n + kSgdChunk - 1) / kSgdChunk);
+                bytes += 12.0 * double(n);
+            }
+            ++done;
+        }
+        if (!b.tensors) continue;
+        account(bytes, 0.0);
+        hipLaunchKernelGGL(sgd_multi_kernel, dim3(b.first_block[b.tensors]), dim3(kThreads), 0, s, b);
+        int rc = launched(__func__);
+        if (rc) return rc;
+    }
+    return CTAMD_OK;
 }
 int ctamd_relu_backward_f32(const float* x, const float* g, float* dx, size_t n, void* s) { return binary<ReluBwdF>(__func__, x, g, dx, n, s); }
 int ctamd_sigmoid_backward_f32(const float* x, const float* g, float* dx, size_t n, void* s) { return binary<SigmoidBwdF>(__func__, x, g, dx, n, s); }

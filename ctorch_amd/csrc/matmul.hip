@@ -140,7 +140,18 @@ struct GemmArgs {
     int k_per_split;                // multiple of BK
     int64_t split_stride;           // elements between partial buffers (0 when not split)
     int tiles_m, tiles_n;
+    const float* bias;              // optional row vector [n] added to every row of C (null: none)
+    int relu;                       // then max(0, .) when set; both only when not split along K
 };
+
+// Output epilogue of a product that is not split along K: bias add, then ReLU as `v > 0 ? v : +0`
+// (NaN -> 0, -0 -> +0), each rounded as the separate Add and ReLU kernels round them, so that the
+// fused product equals the three launches bit for bit.
+__device__ __forceinline__ float epilogue(float v, const float* __restrict__ bias, int col, int relu) {
+    if (bias) v = v + bias[col];
+    if (relu) v = v > 0.0f ? v : 0.0f;
+    return v;
+}
 
 template <class C, bool A_KC, bool B_KC, bool VEC>
 __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(GemmArgs g) {
@@ -345,15 +356,17 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int row = m0 + wm + i * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-                if (row < g.m && col < g.n) cout[int64_t(row) * g.ldc + col] = acc[i][j][r];
+                if (row < g.m && col < g.n) cout[int64_t(row) * g.ldc + col] = epilogue(acc[i][j][r], g.bias, col, g.relu);
             }
         }
 }
 
 // Folds the K-split partial products: c[i] = sum_z partial[z][i], in order of z.
+// Then the optional bias add and ReLU of the fused product (n = row length of C).
 template <bool VEC>
 __global__ __launch_bounds__(kThreads) void splitk_fold(const float* __restrict__ partial, float* __restrict__ c,
-                                                        size_t mn, int splits) {
+                                                        size_t mn, int splits, const float* __restrict__ bias, int n,
+                                                        int relu) {
     size_t i = size_t(blockIdx.x) * kThreads + threadIdx.x;
     if (VEC) {
         if (i >= mn / 4) return;
@@ -368,12 +381,16 @@ __global__ __launch_bounds__(kThreads) void splitk_fold(const float* __restrict_
             t = t + e;
         }
         for (; z < splits; ++z) t = t + p[size_t(z) * stride + i];
+        if (bias || relu) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) t[e] = epilogue(t[e], bias, int((i * 4 + e) % size_t(n)), relu);
+        }
         reinterpret_cast<v4f*>(c)[i] = t;
     } else {
         if (i >= mn) return;
         float t = partial[i];
         for (int z = 1; z < splits; ++z) t += partial[size_t(z) * mn + i];
-        c[i] = t;
+        c[i] = epilogue(t, bias, int(i % size_t(n)), relu);
     }
 }
 
@@ -381,13 +398,14 @@ __global__ __launch_bounds__(kThreads) void splitk_fold(const float* __restrict_
 // the reference's own transposes of transposes could produce such views.
 __global__ __launch_bounds__(kThreads) void gemm_strided(const float* __restrict__ a, int64_t as0, int64_t as1,
                                                          const float* __restrict__ b, int64_t bs0, int64_t bs1,
-                                                         float* __restrict__ c, int m, int n, int k) {
+                                                         float* __restrict__ c, int m, int n, int k,
+                                                         const float* __restrict__ bias, int relu) {
     size_t idx = size_t(blockIdx.x) * kThreads + threadIdx.x;
     if (idx >= size_t(m) * n) return;
     int i = int(idx / n), j = int(idx % n);
     float s = 0.0f;
     for (int l = 0; l < k; ++l) s = __fmaf_rn(a[i * as0 + l * as1], b[l * bs0 + j * bs1], s);
-    c[idx] = s;
+    c[idx] = epilogue(s, bias, j, relu);
 }
 
 // Three tile shapes; the host picks the largest one that still gives every CU a tile.
@@ -422,26 +440,36 @@ int launch_layout(GemmArgs g, bool a_kc, bool b_kc, bool vec, int splits, hipStr
 
 using namespace ctamd;
 
-extern "C" int ctamd_matmul_f32(const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,
-                                float* c, int64_t m, int64_t n, int64_t k, void* stream) {
-    if (m < 0 || n < 0 || k < 0) return fail(CTAMD_EINVAL, "%s: negative extent", __func__);
+namespace {
+
+// C = A.B, optionally followed by "+ bias row" and ReLU in the same launch (in the fold launch when
+// the product is split along K).
+int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,
+                const float* bias, int relu, float* c, int64_t m, int64_t n, int64_t k, void* stream) {
+    if (m < 0 || n < 0 || k < 0) return fail(CTAMD_EINVAL, "%s: negative extent", name);
     if (m == 0 || n == 0) return CTAMD_OK;
-    if (!c) return fail(CTAMD_EINVAL, "%s: null output", __func__);
+    if (!c) return fail(CTAMD_EINVAL, "%s: null output", name);
     if (m > 0x7fffffff || n > 0x7fffffff || k > 0x7fffffff || m * n > (int64_t(1) << 40))
-        return fail(CTAMD_ERANGE, "%s: extent too large", __func__);
-    if (k == 0) return ctamd_fill_f32(c, 0.0f, size_t(m) * size_t(n), stream);
-    if (!a || !b) return fail(CTAMD_EINVAL, "%s: null input", __func__);
-    if (as0 < 0 || as1 < 0 || bs0 < 0 || bs1 < 0) return fail(CTAMD_EINVAL, "%s: negative stride", __func__);
+        return fail(CTAMD_ERANGE, "%s: extent too large", name);
+    if (k == 0) {                                   // an empty sum: 0, then the epilogue
+        int rc = ctamd_fill_f32(c, 0.0f, size_t(m) * size_t(n), stream);
+        if (!rc && bias) rc = ctamd_add_rowbcast_f32(c, bias, c, size_t(m), size_t(n), stream);
+        if (!rc && relu) rc = ctamd_relu_f32(c, c, size_t(m) * size_t(n), stream);
+        return rc;
+    }
+    if (!a || !b) return fail(CTAMD_EINVAL, "%s: null input", name);
+    if (as0 < 0 || as1 < 0 || bs0 < 0 || bs1 < 0) return fail(CTAMD_EINVAL, "%s: negative stride", name);
     hipStream_t s = as_stream(stream);
-    account(4.0 * (double(m) * double(k) + double(k) * double(n) + double(m) * double(n)), 2.0 * double(m) * double(n) * double(k));
+    account(4.0 * (double(m) * double(k) + double(k) * double(n) + double(m) * double(n) + (bias ? double(n) : 0.0)),
+            2.0 * double(m) * double(n) * double(k));
 
     // a one-row / one-column operand is contiguous in whichever direction has extent > 1
     const bool a_kc = (as1 == 1) || (k == 1 && as0 != 1), a_xc = (as0 == 1) || (m == 1);
     const bool b_xc = (bs1 == 1) || (n == 1 && bs0 != 1), b_kc = (bs0 == 1) || (k == 1);
     if (!(a_kc || a_xc) || !(b_kc || b_xc)) {
         hipLaunchKernelGGL(gemm_strided, dim3(unsigned((size_t(m) * n + kThreads - 1) / kThreads)), dim3(kThreads), 0, s,
-                           a, as0, as1, b, bs0, bs1, c, int(m), int(n), int(k));
-        return launched(__func__);
+                           a, as0, as1, b, bs0, bs1, c, int(m), int(n), int(k), bias, relu);
+        return launched(name);
     }
     const bool A_KC = a_kc, B_KC = !b_xc;
     const int cus = compute_units() > 0 ? compute_units() : 256;
@@ -483,8 +511,8 @@ extern "C" int ctamd_matmul_f32(const float* a, int64_t as0, int64_t as1, const 
     kps = (kps + BK - 1) / BK * BK;
     splits = int((k + kps - 1) / kps);
     g.k_per_split = kps;
-    if (splits > 1) { g.c = partial; g.ldc = n; g.split_stride = m * n; }
-    else { g.c = c; g.ldc = n; g.split_stride = 0; }
+    if (splits > 1) { g.c = partial; g.ldc = n; g.split_stride = m * n; g.bias = nullptr; g.relu = 0; }
+    else { g.c = c; g.ldc = n; g.split_stride = 0; g.bias = bias; g.relu = relu; }
 
     int rc = shape == 2 ? launch_layout<BigTile>(g, A_KC, B_KC, vec, splits, s)
            : shape == 1 ? launch_layout<SmallTile>(g, A_KC, B_KC, vec, splits, s)
@@ -493,9 +521,22 @@ extern "C" int ctamd_matmul_f32(const float* a, int64_t as0, int64_t as1, const 
     size_t mn = size_t(m) * size_t(n);
     if (mn % 4 == 0 && aligned16(c))
         hipLaunchKernelGGL(splitk_fold<true>, dim3(unsigned((mn / 4 + kThreads - 1) / kThreads)), dim3(kThreads), 0, s,
-                           partial, c, mn, splits);
+                           partial, c, mn, splits, bias, int(n), relu);
     else
         hipLaunchKernelGGL(splitk_fold<false>, dim3(unsigned((mn + kThreads - 1) / kThreads)), dim3(kThreads), 0, s,
-                           partial, c, mn, splits);
-    return launched(__func__);
+                           partial, c, mn, splits, bias, int(n), relu);
+    return launched(name);
+}
+
+}  // namespace
+
+extern "C" int ctamd_matmul_f32(const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,
+                                float* c, int64_t m, int64_t n, int64_t k, void* stream) {
+    return matmul_impl(__func__, a, as0, as1, b, bs0, bs1, nullptr, 0, c, m, n, k, stream);
+}
+
+extern "C" int ctamd_matmul_bias_f32(const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,
+                                     const float* bias, int relu, float* c, int64_t m, int64_t n, int64_t k,
+                                     void* stream) {
+    return matmul_impl(__func__, a, as0, as1, b, bs0, bs1, bias, relu ? 1 : 0, c, m, n, k, stream);
 }

@@ -61,6 +61,7 @@ class AutoDiff {
         std::vector<size_t> input_ids;
         std::unique_ptr<Tensor> tensor;   // shares storage with the user's tensor
         std::unique_ptr<Tensor> grad;
+        std::unique_ptr<Tensor> shared_term;   // backward only: a factor that several inputs' gradients use
         bool requires_grad = false;
         bool is_leaf = true;
     };
@@ -72,6 +73,7 @@ class AutoDiff {
     void update_requires_grad(Tensor& t, bool requires_grad);
     void zero_grad(Tensor& t);
     Tensor get_grad(const Tensor* t);
+    Tensor stored_grad(const Tensor& t);   // extension: the stored bytes, shared; see AutoDiff.cpp
     void defer_record(size_t output_id, op operation, const std::vector<Tensor*>& inputs, int op_param_i = 0);
     void commit_record(Tensor& output);
     void set_retain_graph(bool retain) { retain_graph_ = retain; }

@@ -20,6 +20,7 @@ enum class op {
     LReLU, PReLU,
     MSE, MAE, CE, BCE,
     Sum,
+    Linear,   // not in the reference: matmul + bias row (+ ReLU) as one taped operator, Tensor::linear
 };
 
 enum class ErrorLevel { TRACE = 0, DEBUG = 1, INFO = 2, WARN = 3, ERROR = 4, FATAL = 5 };

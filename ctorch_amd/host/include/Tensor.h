@@ -115,6 +115,11 @@ class Tensor {
     Tensor operator/(const Tensor& other) const;
     Tensor operator-() const;
     Tensor matmul(const Tensor& other) const;
+    // Not in the reference: `(x.matmul(weight) + bias)` and, with relu, `.relu()` of it
+    // (the layer of mnist/mnist.cpp:39-41) as ONE operator: one launch and one tape entry on the
+    // device, with the values and gradients of the three-operator form bit for bit.  On the host it
+    // is the three operators.
+    Tensor linear(const Tensor& weight, const Tensor& bias, bool relu = false) const;
     Tensor dot(const Tensor& other) const;
     Tensor relu() const;
     Tensor sigmoid() const;

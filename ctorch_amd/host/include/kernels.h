@@ -16,6 +16,8 @@ Tensor Sub_AMD_kernel(const Tensor& a, const Tensor& b);
 Tensor Mul_AMD_kernel(const Tensor& a, const Tensor& b);
 Tensor Div_AMD_kernel(const Tensor& a, const Tensor& b);
 Tensor MatMul_AMD_kernel(const Tensor& a, const Tensor& b);
+// x.matmul(w) + bias (row vector), then ReLU when asked, in one launch; equals the separate kernels bit for bit
+Tensor Linear_AMD_kernel(const Tensor& x, const Tensor& w, const Tensor& bias, bool relu);
 Tensor Dot_AMD_kernel(const Tensor& a, const Tensor& b);
 Tensor MSE_AMD_kernel(const Tensor& a, const Tensor& b);
 Tensor MAE_AMD_kernel(const Tensor& a, const Tensor& b);
@@ -48,6 +50,9 @@ void copy_into(Tensor& dst, const Tensor& src);                        // device
 // the MNIST demo's host loops as device launches
 Tensor onehot(const Tensor& labels, size_t classes);                   // mnist/mnist.cpp:72-78
 void sgd_step(Tensor& param, const Tensor& grad, float lr);            // mnist/mnist.cpp:86-92, in place
+// the same update for several parameters in one launch; grads as AutoDiff::stored_grad returns them
+// (an empty gradient leaves its parameter alone), "0 +" applied in the kernel
+void sgd_step_all(const std::vector<Tensor*>& params, const std::vector<Tensor>& grads, float lr);
 size_t count_correct(const Tensor& pred, const Tensor& labels);        // mnist/mnist.cpp:134-156 (reads back)
 Tensor unit_from_bytes(const unsigned char* host_bytes, size_t rows, size_t cols);  // mnist_loader.cpp:33-41
 Tensor relu_backward(const Tensor& x, const Tensor& g);

@@ -24,6 +24,8 @@ struct MnistDemoOptions {
     // instead of ~50); needs reference_tape == false (a frozen leaf copy would be re-made by
     // every replay)
     bool use_graph = false;
+    // each layer as one fused operator (Tensor::linear) and the optimiser update as one launch
+    bool fused_layers = false;
 };
 
 struct MnistDemoResult {
@@ -45,6 +47,7 @@ inline MnistDemoResult run_mnist_demo(const MnistDemoOptions& opt) {
     res.test_images = test_images.shape()[0];
     res.pixels = train_images.shape()[1];
     NeuralNetwork model(int(res.pixels), opt.hidden1, opt.hidden2, 10, opt.learning_rate);
+    model.fused_layers = opt.fused_layers;
     res.num_batches = int(res.train_images) / opt.batch_size;
 
     AutoDiff autodiff;

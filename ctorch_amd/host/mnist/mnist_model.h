@@ -41,7 +41,11 @@ class NeuralNetwork {
         b3 = Tensor::from_host(c3, {C}, DeviceType::kAMD);
     }
 
+    // true: each layer is one fused operator (Tensor::linear); same values and gradients, fewer launches
+    bool fused_layers = false;
+
     Tensor forward(const Tensor& x) {
+        if (fused_layers) return x.linear(W1, b1, true).linear(W2, b2, true).linear(W3, b3, false);
         Tensor h1 = (x.matmul(W1) + b1).relu();
         Tensor h2 = (h1.matmul(W2) + b2).relu();
         return h2.matmul(W3) + b3;
@@ -71,6 +75,14 @@ class NeuralNetwork {
 
     void update_parameters() {
         Tensor* params[6] = {&W1, &b1, &W2, &b2, &W3, &b3};
+        AutoDiff* ctx = AutoDiffContext::current();
+        if (fused_layers && ctx) {                       // one launch for the six tensors
+            std::vector<Tensor*> ps(params, params + 6);
+            std::vector<Tensor> gs;
+            for (Tensor* p : params) gs.push_back(ctx->stored_grad(*p));
+            ctorch_amd_host::sgd_step_all(ps, gs, learning_rate);
+            return;
+        }
         for (Tensor* p : params) {
             Tensor g = grad(*p);
             ctorch_amd_host::sgd_step(*p, g, learning_rate);

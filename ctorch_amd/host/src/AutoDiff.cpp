@@ -57,8 +57,20 @@ void AutoDiff::zero_grad(Tensor& t) {
     if (t.id() == 0) return;
     std::lock_guard<std::mutex> lock(records_mutex);
     Node* n = find(t.id());
-    // a fresh zero tensor: the stored gradient may share its bytes with another node's
-    if (n && n->grad) n->grad = std::make_unique<Tensor>(ShapeTag{}, n->grad->sizes(), n->grad->dtype(), n->grad->device());
+    // no gradient stored reads as zeros (get_grad) and the next contribution becomes the gradient
+    // with its "0 +" pending: the same values as a zero-filled buffer, without the fill
+    if (n) n->grad.reset();
+}
+
+// Not in the reference: the gradient's bytes as the tape holds them (shared, not copied; empty when
+// there is none).  Where get_grad has +0 these bytes may hold -0: the "0 +" of the reference's
+// zero-filled accumulation buffer is left to the reader.
+Tensor AutoDiff::stored_grad(const Tensor& t) {
+    if (t.id() == 0) return Tensor();
+    std::lock_guard<std::mutex> lock(records_mutex);
+    Node* n = find(t.id());
+    if (n && n->requires_grad && n->grad && n->grad->sizes() == t.sizes()) return Tensor::alias(*n->grad);
+    return Tensor();
 }
 
 // src/AutoDiff.cpp:86-243: a copy of the stored gradient, or zeros of the tensor's shape
@@ -134,7 +146,7 @@ bool is_row_vector_of(const Tensor& v, const Tensor& m) {
 }
 }  // namespace
 
-Tensor AutoDiff::input_gradient(Node* node, size_t input_id, size_t /*input_pos*/, const Tensor& g) {
+Tensor AutoDiff::input_gradient(Node* node, size_t input_id, size_t input_pos, const Tensor& g) {
     Node* in = find(input_id);
     const Tensor& x = *in->tensor;
     const bool first = (input_id == node->input_ids[0]);   // the reference tells operands apart by id
@@ -211,6 +223,17 @@ Tensor AutoDiff::input_gradient(Node* node, size_t input_id, size_t /*input_pos*
                                              "MatMul gradient must be a 2-D tensor");
             if (first) return MatMul_AMD_kernel(g, Tensor::view_t(other));      // g . B^T
             return MatMul_AMD_kernel(Tensor::view_t(other), g);                 // A^T . g
+        }
+        case op::Linear: {                                              // the three branches above in one
+            // gradient at the pre-activation: g * [y > 0], which is the reference's g * [z > 0]
+            // (:1320-1371) since y = max(0, z); computed once for the three inputs
+            if (node->op_param_i && !node->shared_term)
+                node->shared_term = std::make_unique<Tensor>(relu_backward(*node->tensor, g));
+            const Tensor& gz = node->op_param_i ? *node->shared_term : g;
+            if (input_pos == 2) return Tensor::alias(gz);               // bias: Add's branch, shaped by the caller
+            const Tensor& other = *find(node->input_ids[input_pos == 0 ? 1 : 0])->tensor;
+            if (input_pos == 0) return MatMul_AMD_kernel(gz, Tensor::view_t(other));   // gz . W^T
+            return MatMul_AMD_kernel(Tensor::view_t(other), gz);                        // x^T . gz
         }
         case op::Sum:                                                   // :1850-1855
             return adjust_grad_shape(g, x.sizes());
@@ -299,5 +322,6 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
                 accumulate(*in->grad, adj);
             }
         }
+        node->shared_term.reset();
     }
 }

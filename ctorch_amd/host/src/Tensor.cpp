@@ -275,6 +275,17 @@ Tensor Tensor::operator-(const Tensor& other) const { return binary(*this, other
 Tensor Tensor::operator*(const Tensor& other) const { return binary(*this, other, op::Mul); }
 Tensor Tensor::operator/(const Tensor& other) const { return binary(*this, other, op::Div); }
 Tensor Tensor::matmul(const Tensor& other) const { return binary(*this, other, op::MatMul); }
+Tensor Tensor::linear(const Tensor& weight, const Tensor& bias, bool relu) const {
+    if (device() != DeviceType::kAMD) {
+        Tensor z = matmul(weight) + bias;
+        return relu ? z.relu() : z;
+    }
+    check_pair(*this, weight);
+    check_pair(*this, bias);
+    Tensor result = Linear_AMD_kernel(*this, weight, bias, relu);
+    tape(result, op::Linear, {this, &weight, &bias}, relu ? 1 : 0);
+    return result;
+}
 Tensor Tensor::mse_loss(const Tensor& target) const { return binary(*this, target, op::MSE); }
 Tensor Tensor::mae_loss(const Tensor& target) const { return binary(*this, target, op::MAE); }
 Tensor Tensor::cross_entropy(const Tensor& target) const { return binary(*this, target, op::CE); }

@@ -78,7 +78,10 @@ void cth_quiet() { Ctorch_Error::setPrintLevel(PrintLevel::MINIUM); }
 // 0: gradient of a row-broadcast operand = column sum (default); 1: the reference's row-0 slice.
 // Applies to the contexts the entry points below create.
 static int g_row0 = 0;
+static int g_fused_layers = 0;
 void cth_set_reference_row0(int on) { g_row0 = on; }
+// the MLP entry points below build each layer with Tensor::linear (one fused operator) when set
+void cth_set_fused_layers(int on) { g_fused_layers = on; }
 static void configure(AutoDiff& ctx) {
     ctx.set_broadcast_grad(g_row0 ? BroadcastGrad::kReferenceRow0 : BroadcastGrad::kColumnSum);
 }
@@ -263,8 +266,8 @@ long cth_mlp_step(const float* x, long B, long I, const float* W1, const float* 
         tb1.requires_grad(true);
         tW2.requires_grad(true);
         tb2.requires_grad(true);
-        Tensor h = (tx.matmul(tW1) + tb1).relu();
-        Tensor logits = h.matmul(tW2) + tb2;
+        Tensor h = g_fused_layers ? tx.linear(tW1, tb1, true) : (tx.matmul(tW1) + tb1).relu();
+        Tensor logits = g_fused_layers ? h.linear(tW2, tb2, false) : h.matmul(tW2) + tb2;
         Tensor loss = logits.cross_entropy(ty);
         loss_out[0] = loss.item<float>();
         emit(logits, logits_out);
@@ -455,8 +458,8 @@ long cth_time_mlp(const float* x, long B, long I, const float* W1, const float* 
         tb1.requires_grad(true);
         tW2.requires_grad(true);
         tb2.requires_grad(true);
-        Tensor h = (tx.matmul(tW1) + tb1).relu();
-        Tensor loss = (h.matmul(tW2) + tb2).cross_entropy(ty);
+        Tensor h = g_fused_layers ? tx.linear(tW1, tb1, true) : (tx.matmul(tW1) + tb1).relu();
+        Tensor loss = (g_fused_layers ? h.linear(tW2, tb2, false) : h.matmul(tW2) + tb2).cross_entropy(ty);
         sink = loss.item<float>();
         backward(loss);
         Tensor g1 = grad(tW1), g2 = grad(tb1), g3 = grad(tW2), g4 = grad(tb2);
@@ -480,8 +483,8 @@ long cth_time_mlp_graph(const float* x, long B, long I, const float* W1, const f
             tb1.requires_grad(true);
             tW2.requires_grad(true);
             tb2.requires_grad(true);
-            Tensor h = (tx.matmul(tW1) + tb1).relu();
-            loss = (h.matmul(tW2) + tb2).cross_entropy(ty);
+            Tensor h = g_fused_layers ? tx.linear(tW1, tb1, true) : (tx.matmul(tW1) + tb1).relu();
+            loss = (g_fused_layers ? h.linear(tW2, tb2, false) : h.matmul(tW2) + tb2).cross_entropy(ty);
             backward(loss);
             g1 = grad(tW1), g2 = grad(tb1), g3 = grad(tW2), g4 = grad(tb2);
         };
@@ -572,19 +575,22 @@ float cth_mnist_accuracy(const float* pred, const float* labels, long rows) {
 }
 
 // `steps` consecutive batches (batch index = step % (n_images / batch)) inside one autograd
-// context, data set and parameters resident.  reference_tape != 0: leaf values frozen at their
+// context, data set and parameters resident.  mode_bits & 3 = reference_tape; reference_tape == 1: leaf values frozen at their
 // first-seen copies and row-0 bias gradients (the reference's behaviour); else live leaves, column
 // sums and a tape cleared after every step; 2: as 0 with the step recorded into a DeviceGraph at
 // the first batch and replayed for every batch (with unrelated eager work between the replays).
-// Parameters are written back; losses_out[s] = loss of
-// step s.  ms_out (may be null) = milliseconds for all the steps.
+// Adding 4 to the mode makes each layer one fused operator and the optimiser update one launch
+// (same values).  Parameters are written back; losses_out[s] = loss of step s.  ms_out (may be null) = milliseconds for all the steps.
 long cth_mnist_train(const float* images, const float* labels, long n_images, long I, long H1, long H2, long C,
                      float* W1, float* b1, float* W2, float* b2, float* W3, float* b3, long batch, long steps,
-                     float lr, int reference_tape, float* losses_out, double* ms_out) {
+                     float lr, int mode_bits, float* losses_out, double* ms_out) {
     try {
+        const int reference_tape = mode_bits & 3;
+        const bool fused = (mode_bits & 4) != 0;
         long id[2] = {n_images, I}, ld[1] = {n_images};
         Tensor all_images = make(images, id, 2), all_labels = make(labels, ld, 1);
         NeuralNetwork model(W1, b1, W2, b2, W3, b3, size_t(I), size_t(H1), size_t(H2), size_t(C), lr);
+        model.fused_layers = fused;
         const long num_batches = n_images / batch;
         AutoDiff autodiff;
         if (reference_tape == 1) {
@@ -649,7 +655,7 @@ long cth_mnist_predict(const float* x, long B, long I, long H1, long H2, long C,
 
 // The whole demo on the files in `dir`.  epoch_loss_out has room for `epochs` values;
 // acc_out = {train accuracy, test accuracy}; seconds_out = training time.
-long cth_mnist_demo(const char* dir, int epochs, int batch, float lr, int hidden1, int hidden2, int reference_tape,
+long cth_mnist_demo(const char* dir, int epochs, int batch, float lr, int hidden1, int hidden2, int mode_bits,
                     float* epoch_loss_out, float* acc_out, double* seconds_out) {
     try {
         MnistDemoOptions opt;
@@ -659,6 +665,8 @@ long cth_mnist_demo(const char* dir, int epochs, int batch, float lr, int hidden
         opt.learning_rate = lr;
         opt.hidden1 = hidden1;
         opt.hidden2 = hidden2;
+        const int reference_tape = mode_bits & 3;
+        opt.fused_layers = (mode_bits & 4) != 0;
         opt.reference_tape = reference_tape == 1;
         opt.use_graph = reference_tape == 2;          // 2: live leaves and the step replayed from a recorded graph
         MnistDemoResult r = run_mnist_demo(opt);

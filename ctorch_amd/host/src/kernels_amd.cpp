@@ -211,6 +211,24 @@ void sgd_step(Tensor& param, const Tensor& grad, float lr) {
         Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "sgd_step: parameter and gradient differ in size");
     run(ctamd_sgd_step_f32(param.fptr(), grad.fptr(), lr, param.numel(), current_stream()), "sgd_step");
 }
+void sgd_step_all(const std::vector<Tensor*>& params, const std::vector<Tensor>& grads, float lr) {
+    if (params.size() != grads.size())
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "sgd_step_all: one gradient per parameter");
+    std::vector<float*> p;
+    std::vector<const float*> g;
+    std::vector<size_t> n;
+    for (size_t i = 0; i < params.size(); ++i) {
+        if (grads[i].is_cleared()) continue;                 // no gradient: p - 0 * lr = p
+        check_device(*params[i], "sgd_step_all");
+        check_device(grads[i], "sgd_step_all");
+        if (params[i]->numel() != grads[i].numel() || !params[i]->is_contiguous() || !grads[i].is_contiguous())
+            Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "sgd_step_all: parameter and gradient differ in size");
+        p.push_back(params[i]->fptr());
+        g.push_back(grads[i].fptr());
+        n.push_back(params[i]->numel());
+    }
+    run(ctamd_sgd_step_multi_f32(p.data(), g.data(), n.data(), int(p.size()), lr, current_stream()), "sgd_step_all");
+}
 size_t count_correct(const Tensor& pred, const Tensor& labels) {
     check_device(pred, "count_correct");
     check_device(labels, "count_correct");
@@ -355,6 +373,25 @@ Tensor MatMul_AMD_kernel(const Tensor& a, const Tensor& b) {
     run(ctamd_matmul_f32(a.fptr(), int64_t(a.strides()[0]), int64_t(a.strides()[1]), b.fptr(), int64_t(b.strides()[0]),
                          int64_t(b.strides()[1]), r.fptr(), int64_t(m), int64_t(n), int64_t(k), current_stream()),
         "MatMul_AMD_kernel");
+    return r;
+}
+Tensor Linear_AMD_kernel(const Tensor& x, const Tensor& w, const Tensor& bias, bool relu) {
+    check_device(x, "Linear_AMD_kernel");
+    check_device(w, "Linear_AMD_kernel");
+    check_device(bias, "Linear_AMD_kernel");
+    if (x.shape().size() != 2 || w.shape().size() != 2)
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "Linear_AMD_kernel: only 2-D tensors");
+    if (x.shape()[1] != w.shape()[0])
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "Linear_AMD_kernel: inner dimensions differ");
+    // the bias must be what operator+ accepts as a row vector (Add_BASIC_kernel.cpp:27-34)
+    if (bias.shape().size() != 1 || bias.shape()[0] != w.shape()[1])
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "Linear_AMD_kernel: bias is not a row vector of the result");
+    size_t m = x.shape()[0], k = x.shape()[1], n = w.shape()[1];
+    Tensor r(ShapeTag{}, {m, n}, DType::kFloat, DeviceType::kAMD, false);
+    run(ctamd_matmul_bias_f32(x.fptr(), int64_t(x.strides()[0]), int64_t(x.strides()[1]), w.fptr(), int64_t(w.strides()[0]),
+                              int64_t(w.strides()[1]), bias.fptr(), relu ? 1 : 0, r.fptr(), int64_t(m), int64_t(n),
+                              int64_t(k), current_stream()),
+        "Linear_AMD_kernel");
     return r;
 }
 Tensor Dot_AMD_kernel(const Tensor& a, const Tensor& b) { return reduce2(ctamd_dot_f32, "Dot_AMD_kernel", a, b, false); }

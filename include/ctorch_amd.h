@@ -178,6 +178,14 @@ int ctamd_cross_entropy_backward_index_stats_f32(const float* x, const float* id
 int ctamd_matmul_f32(const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,
                      float* c, int64_t m, int64_t n, int64_t k, void* stream);
 
+/* One layer of the demo network in one launch: C = A.B, then "+ bias" broadcast over rows (bias
+ * [n], may be NULL), then ReLU when relu != 0 -- the sequence matmul, operator+, relu() of
+ * mnist/mnist.cpp:39-41 (MatMul_BASIC_kernel.cpp:42-54, Add_BASIC_kernel.cpp:54-63,
+ * ReLU_BASIC_kernel.cpp:19-25).  Each step rounds as its own kernel does, so the result equals
+ * ctamd_matmul_f32, ctamd_add_rowbcast_f32, ctamd_relu_f32 in sequence bit for bit. */
+int ctamd_matmul_bias_f32(const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,
+                          const float* bias, int relu, float* c, int64_t m, int64_t n, int64_t k, void* stream);
+
 /* ----------------------------------------------------------------- backward arithmetic */
 /* r[i] = v.  A 0-D gradient expanded to a shape: src/AutoDiff.cpp:579-592; also Tensor::zero()
  * / ones() src/Tensor.cpp:390-451. */
@@ -229,6 +237,13 @@ int ctamd_onehot_f32(const float* labels, float* out, size_t rows, size_t classe
 /* param[i] -= grad[i] * lr, product and difference rounded separately as in the reference's
  * binary (mnist/mnist.cpp:86-92; built without -O3/-march, CMakeLists.txt:56,65-86); bit-exact. */
 int ctamd_sgd_step_f32(float* param, const float* grad, float lr, size_t n, void* stream);
+/* The same update for every parameter of a model in one launch (update_parameters' loop over the
+ * six tensors, mnist/mnist.cpp:86-92): params[t][i] -= (0 + grads[t][i]) * lr for t < tensors,
+ * i < counts[t].  params, grads and counts are HOST arrays of device pointers / element counts,
+ * read before the call returns.  "0 +" stands for reading the gradient out of the reference's tape,
+ * whose buffers start zero-filled (src/AutoDiff.cpp:1870-1907): a -0 gradient counts as +0. */
+int ctamd_sgd_step_multi_f32(float* const* params, const float* const* grads, const size_t* counts, int tensors, float lr,
+                             void* stream);
 /* count[0] = number of rows whose first maximum (strictly greater, starting from -1.0f at column
  * 0) is at column (int)labels[row]: calculate_accuracy (mnist/mnist.cpp:134-156) without its
  * division by the row count. */

@@ -186,6 +186,17 @@ def accumulate(grad, val):
     return grad
 
 
+def matmul_bias(a, b, bias, relu):
+    """The fused layer: a.b (+ bias row) (then ReLU); bias may be None."""
+    m, k = a.shape
+    k2, n = b.shape
+    assert k == k2 and (bias is None or bias.numel() == n)
+    c = torch.empty((m, n), device=DEV)
+    call("ctamd_matmul_bias_f32", ptr(a), a.stride(0), a.stride(1), ptr(b), b.stride(0), b.stride(1),
+         ptr(bias) if bias is not None else None, int(relu), ptr(c), m, n, k, stream())
+    return c
+
+
 def matmul(a, b):
     """a, b: 2-D device tensors, possibly transposed views (strides are passed through)."""
     m, k = a.shape

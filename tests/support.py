@@ -757,6 +757,10 @@ class HostLayer(Reference):
     def set_reference_row0(self, on):
         self.cdll.cth_set_reference_row0(int(on))
 
+    def set_fused_layers(self, on):
+        """mlp_step builds each layer with Tensor::linear (matmul + bias + ReLU as one operator)."""
+        self.cdll.cth_set_fused_layers(int(on))
+
     def mlp_step(self, x, W1, b1, W2, b2, target, target_is_index=False):
         return Reference.mlp_step(self, x, W1, b1, W2, b2, target, C.c_int(int(target_is_index)))
 

@@ -174,6 +174,18 @@ def test_configurations_small(oracle, host, golden):
     for n, a, b in zip(names, got, [g["mlp_" + n] for n in names]):   # the reference's own numbers
         assert np.abs(a - b).max() <= 1e-4 * max(1.0, np.abs(b).max()), n
     want = oracle.mlp_step(*args, oh, False)                            # column-sum bias gradients
+    # each layer as one fused operator: the bits of the three-operator form, in both gradient modes
+    for row0 in (False, True):
+        host.set_reference_row0(row0)
+        try:
+            plain = host.mlp_step(*args, oh)
+            host.set_fused_layers(True)
+            fused = host.mlp_step(*args, oh)
+        finally:
+            host.set_fused_layers(False)
+            host.set_reference_row0(False)
+        for n, a, b in zip(names, fused, plain):
+            assert same_bits(a, b), (n, row0)
     for target, is_index in ((oh, False), (lab, True)):
         got = host.mlp_step(*args, target, is_index)
         for n, a, b in zip(names, got, want):

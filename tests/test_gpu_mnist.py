@@ -157,7 +157,49 @@ def test_recorded_step_replays_to_the_same_bits(host, golden, tag):
         assert same_bits(a, b)
 
 
+def test_sgd_step_of_several_tensors_in_one_launch(oracle):
+    """ctamd_sgd_step_multi_f32 against the single-tensor update on the gradient with its -0 turned
+    into +0 (what reading it from the tape does), for 40 tensors (two launches of at most 32), sizes
+    from 1 to beyond one block's chunk, one of them empty, with -0 gradients on -0 parameters."""
+    print("case sgd multi", flush=True)
+    sizes = [1, 7, 2047, 2048, 2049, 100003, 0, 10, 784 * 128, 64] + [33 + 17 * k for k in range(30)]
+    ps = [oracle.uniform((n,), 500 + k, -1, 1) for k, n in enumerate(sizes)]
+    gs = [oracle.normal((n,), 600 + k, 0, 3) for k, n in enumerate(sizes)]
+    ps[2][:50] = -0.0
+    gs[2][:100:2] = -0.0
+    gs[2][1:100:2] = 0.0
+    d_p = [G.dev(p) for p in ps]
+    d_g = [G.dev(g) for g in gs]
+    ptrs_p = (C.c_void_p * len(sizes))(*[t.data_ptr() if t.numel() else None for t in d_p])
+    ptrs_g = (C.c_void_p * len(sizes))(*[t.data_ptr() if t.numel() else None for t in d_g])
+    counts = (C.c_size_t * len(sizes))(*sizes)
+    G.call("ctamd_sgd_step_multi_f32", ptrs_p, ptrs_g, counts, len(sizes), C.c_float(0.01), G.stream())
+    for k, n in enumerate(sizes):
+        want = oracle.sgd_step(ps[k], gs[k] + F(0), 0.01) if n else ps[k]
+        assert same_bits(G.host(d_p[k]), want), k
+    assert np.signbit(G.host(d_p[2])[:50]).all()               # -0 - (+0 * lr) stays -0; without the "0 +" it would be +0
+
+
+@pytest.mark.parametrize("tag", ["s", "m"])
+def test_fused_layers_and_update_give_the_same_bits(host, golden, tag):
+    """Each layer as one fused operator (matmul + bias + ReLU in one launch, one tape entry) and the
+    optimiser update of the six tensors as one launch: every loss and trained parameter has the
+    bits of the operator-by-operator run, in each tape mode (live leaves, the reference's tape,
+    recorded step)."""
+    print("case fused layers", tag, flush=True)
+    g = golden("mnist")
+    batch, steps = (int(v) for v in g[tag + "_cfg"])
+    params = [g["%s_p%d" % (tag, k)] for k in range(6)]
+    for mode in (0, 1, 2):
+        plain_l, plain_p = host.mnist_train(g[tag + "_x"], g[tag + "_y"], params, batch, steps, 0.01, reference_tape=mode)
+        fused_l, fused_p = host.mnist_train(g[tag + "_x"], g[tag + "_y"], params, batch, steps, 0.01, reference_tape=mode + 4)
+        assert same_bits(fused_l, plain_l), mode
+        for a, b in zip(fused_p, plain_p):
+            assert same_bits(a, b), mode
+
+
 def test_demo_with_a_recorded_step(host, tmp_path):
+
     print("case demo recorded", flush=True)
     write_mnist_dir(str(tmp_path))
     rc1, l1, a1, _ = host.mnist_demo(str(tmp_path), epochs=3, lr=1e-3, reference_tape=0)

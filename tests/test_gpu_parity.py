@@ -348,6 +348,31 @@ def test_matmul_all_layouts_normwise(oracle, m, n, k):
             assert np.all(np.abs(got - want) <= 2 * bound), name
 
 
+@pytest.mark.parametrize("m,n,k", [(256, 128, 784), (128, 10, 64), (70, 33, 129), (8192, 256, 784), (96, 12, 4096),
+                                   (2100, 2050, 40), (5, 7, 0)])
+def test_fused_layer_equals_the_three_launches(oracle, m, n, k):
+    """matmul + bias row + ReLU in one launch against the same three operators launched in sequence,
+    bit for bit, over all tile shapes, the K-split fold ((96, 12, 4096)) and ragged edges; and against
+    the CPU oracle's sequence within the MatMul bound."""
+    print("case fused layer", m, n, k, flush=True)
+    A = oracle.normal((m, k), 61)
+    B = oracle.normal((k, n), 62)
+    bias = oracle.normal((n,), 63)
+    dA, dB, db = G.dev(A), G.dev(B), G.dev(bias)
+    dBt = G.dev(np.ascontiguousarray(B.T))
+    for a, b in ((dA, dB), (dA, dBt.t())):
+        plain = G.matmul(a, b)
+        biased = G.rowbcast("add", plain, db)
+        assert same_bits(G.host(G.matmul_bias(a, b, None, False)), G.host(plain))
+        assert same_bits(G.host(G.matmul_bias(a, b, db, False)), G.host(biased))
+        assert same_bits(G.host(G.matmul_bias(a, b, db, True)), G.host(G.unary("relu", biased)))
+        assert same_bits(G.host(G.matmul_bias(a, b, None, True)), G.host(G.unary("relu", plain)))
+    if m * n * max(k, 1) <= 1 << 22:
+        want = oracle.relu(oracle.binary_rowbcast(ADD, oracle.matmul(A, B), bias)) if k else np.maximum(np.broadcast_to(bias, (m, n)), 0)
+        bound = 2e-5 * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64)) + 1e-6
+        assert np.all(np.abs(G.host(G.matmul_bias(dA, dB, db, True)) - want) <= bound)
+
+
 def test_matmul_exact_on_small_integers_and_unaligned_views(oracle):
     print("case matmul integers", flush=True)
     rng = np.random.default_rng(7)
