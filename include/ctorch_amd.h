@@ -186,6 +186,53 @@ int ctamd_matmul_f32(const float* a, int64_t as0, int64_t as1, const float* b, i
 int ctamd_matmul_bias_f32(const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,
                           const float* bias, int relu, float* c, int64_t m, int64_t n, int64_t k, void* stream);
 
+/* ------------------------------------------------------------------ fused expressions */
+/* A chain of the elementwise operators above evaluated in ONE pass over memory: the front-end
+ * compiles an expression such as Y = sigmoid(X / r) - tanh(X) * sin(X) + cos(-X) (and, separately,
+ * its tape gradients) into a straight-line program over value slots.  Every operator computes
+ * exactly what its one-operator entry point computes, so a program's results equal the
+ * operator-by-operator evaluation bit for bit.  No counterpart in the reference, which runs one
+ * kernel per operator (src/Tensor.cpp dispatch sites); the operator semantics are those of
+ * Add/Sub/Mul/Div/Neg/ReLU/Sigmoid/Tanh/Sin/Cos_BASIC_kernel.cpp, Tensor::operator+,*,/(float)
+ * (src/Tensor.cpp:751-973) and the gradient formulas of src/AutoDiff.cpp:1216-1416. */
+enum {
+    CTAMD_EX_LOAD_FULL = 0, /* slot[dst] = inputs[a][i]            ([rows, cols] tensor)            */
+    CTAMD_EX_LOAD_ROW = 1,  /* slot[dst] = inputs[a][i % cols]     (row vector [cols])              */
+    CTAMD_EX_ADD = 2,       /* slot[dst] = slot[a] + slot[b]; SUB, MUL, DIV alike                   */
+    CTAMD_EX_SUB = 3,
+    CTAMD_EX_MUL = 4,
+    CTAMD_EX_DIV = 5,
+    CTAMD_EX_NEG = 6,       /* slot[dst] = f(slot[a])                                               */
+    CTAMD_EX_RELU = 7,
+    CTAMD_EX_SIGMOID = 8,
+    CTAMD_EX_TANH = 9,
+    CTAMD_EX_SIN = 10,
+    CTAMD_EX_COS = 11,
+    CTAMD_EX_ADDS = 12,     /* slot[dst] = slot[a] + imm; MULS: * imm; DIVS: / imm                  */
+    CTAMD_EX_MULS = 13,
+    CTAMD_EX_DIVS = 14,
+    CTAMD_EX_RSUBS = 15,    /* slot[dst] = imm - slot[a]                                            */
+    CTAMD_EX_RELUMUL = 16,  /* slot[dst] = slot[b] * (slot[a] > 0 ? 1 : 0)    (ReLU's gradient)     */
+    CTAMD_EX_DIVCHK = 17,   /* status[0] |= 1 if |slot[a]| < FLT_EPSILON anywhere                   */
+    CTAMD_EX_STORE = 18,    /* outputs[dst][i] = slot[a]                                            */
+    CTAMD_EX_STORE_ZP = 19  /* outputs[dst][i] = 0 + slot[a]   (a gradient read from the tape)      */
+};
+#define CTAMD_EXPR_MAX_INSNS 96
+#define CTAMD_EXPR_MAX_SLOTS 32
+#define CTAMD_EXPR_MAX_PORTS 8
+typedef struct ctamd_expr_insn {
+    uint8_t op, dst, a, b;
+    float imm;
+} ctamd_expr_insn;
+/* Runs the program for every element of a [rows, cols] value.  prog, inputs and outputs are HOST
+ * arrays (inputs / outputs hold device pointers), read before the call returns.  Full-shape
+ * inputs and all outputs have rows * cols elements, row-vector inputs cols.  A slot must be
+ * written before it is read.  status (one int32 on the device, cleared by the caller) is only
+ * needed by programs with CTAMD_EX_DIVCHK.  An output must not alias an input that the program
+ * reads after the store. */
+int ctamd_expr_run_f32(const ctamd_expr_insn* prog, int n_insn, const float* const* inputs, int n_inputs,
+                       float* const* outputs, int n_outputs, int32_t* status, size_t rows, size_t cols, void* stream);
+
 /* ----------------------------------------------------------------- backward arithmetic */
 /* r[i] = v.  A 0-D gradient expanded to a shape: src/AutoDiff.cpp:579-592; also Tensor::zero()
  * / ones() src/Tensor.cpp:390-451. */

@@ -767,6 +767,62 @@ void co_expr(const float* X, const float* R, const float* T, long rows, long col
     free(v); free(gd1); free(gcs); free(gs1); free(gm); free(gq); free(gth); free(gsn); free(gng);
 }
 
+/* ------------------------------------------------------------- fused expression programs */
+
+/* Extension: the reference evaluates one operator per kernel.  A program is a straight-line list
+ * of (op, dst, a, b) over per-element value slots plus one immediate per instruction; each
+ * opcode is the per-element body of the function named beside it, so running a program equals
+ * calling those functions one after the other on whole tensors.
+ *   0 load full input a        1 load row-vector input a (index i % cols)
+ *   2 co_add  3 co_sub  4 co_mul  5 co_div  6 co_neg  7 co_relu  8 co_sigmoid  9 co_tanh
+ *  10 co_sin  11 co_cos  12 co_scalar_add  13 co_scalar_mul  14 co_scalar_div
+ *  15 imm - x (the "1.0f - s" of co_sigmoid_bwd / co_tanh_bwd)   16 co_relu_bwd (a = x, b = g)
+ *  17 co_any_abs_lt_eps of slot a into status   18 store slot a to output dst
+ *  19 store 0 + slot a (src/AutoDiff.cpp:1870-1907: contributions are added to a zero-filled buffer)
+ * Returns 0, or -1 for a malformed program. */
+int co_expr_run(const int* prog, const float* imm, int n, const float* const* in, int n_in, float* const* out, int n_out,
+                long rows, long cols, int* status) {
+    enum { SLOTS = 32 };
+    for (int pc = 0; pc < n; ++pc) {
+        const int op = prog[4 * pc], d = prog[4 * pc + 1], a = prog[4 * pc + 2], b = prog[4 * pc + 3];
+        if (op < 0 || op > 19 || a < 0 || b < 0 || d < 0) return -1;
+        if (op <= 1 ? (a >= n_in || d >= SLOTS) : (op >= 18 ? (d >= n_out || a >= SLOTS) : (a >= SLOTS || b >= SLOTS || d >= SLOTS)))
+            return -1;
+    }
+    const long total = rows * cols;
+    for (long i = 0; i < total; ++i) {
+        float v[SLOTS];
+        memset(v, 0, sizeof(v));
+        for (int pc = 0; pc < n; ++pc) {
+            const int op = prog[4 * pc], d = prog[4 * pc + 1], a = prog[4 * pc + 2], b = prog[4 * pc + 3];
+            const float s = imm[pc];
+            switch (op) {
+                case 0: v[d] = in[a][i]; break;
+                case 1: v[d] = in[a][i % cols]; break;
+                case 2: v[d] = v[a] + v[b]; break;
+                case 3: v[d] = v[a] - v[b]; break;
+                case 4: v[d] = v[a] * v[b]; break;
+                case 5: v[d] = v[a] / v[b]; break;
+                case 6: v[d] = -v[a]; break;
+                case 7: v[d] = (0.0f < v[a]) ? v[a] : 0.0f; break;
+                case 8: v[d] = 1.0f / (1.0f + expf(-v[a])); break;
+                case 9: { float ep = expf(v[a]), en = expf(-v[a]); v[d] = (ep - en) / (ep + en); break; }
+                case 10: v[d] = sinf(v[a]); break;
+                case 11: v[d] = cosf(v[a]); break;
+                case 12: v[d] = v[a] + s; break;
+                case 13: v[d] = v[a] * s; break;
+                case 14: v[d] = v[a] / s; break;
+                case 15: v[d] = s - v[a]; break;
+                case 16: { float mask = (v[a] > 0.0f) ? 1.0f : 0.0f; v[d] = v[b] * mask; break; }
+                case 17: if (fabsf(v[a]) < FLT_EPSILON && status) *status |= 1; break;
+                case 18: out[d][i] = v[a]; break;
+                case 19: out[d][i] = 0.0f + v[a]; break;
+            }
+        }
+    }
+    return 0;
+}
+
 /* ------------------------------------------------------------------------- input generator */
 
 /* Counter-based generator of this repository (the reference has no seedable one:

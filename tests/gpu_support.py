@@ -206,3 +206,20 @@ def matmul(a, b):
     call("ctamd_matmul_f32", ptr(a), a.stride(0), a.stride(1), ptr(b), b.stride(0), b.stride(1), ptr(c), m, n, k,
          stream())
     return c
+
+
+class ExprInsn(C.Structure):
+    _fields_ = [("op", C.c_uint8), ("dst", C.c_uint8), ("a", C.c_uint8), ("b", C.c_uint8), ("imm", C.c_float)]
+
+
+def expr_run(prog, inputs, n_out, rows, cols, expect=0):
+    """Runs a fused-expression program [(op, dst, a, b, imm)] on device tensors; returns (outputs,
+    status word).  expect: the return code the call must give."""
+    arr = (ExprInsn * max(1, len(prog)))(*[ExprInsn(*q) for q in prog])
+    outs = [torch.zeros((rows, cols), device=DEV) for _ in range(n_out)]
+    status = torch.zeros(1, dtype=torch.int32, device=DEV)
+    pin = (C.c_void_p * max(1, len(inputs)))(*[t.data_ptr() for t in inputs])
+    pout = (C.c_void_p * max(1, n_out))(*[t.data_ptr() for t in outs])
+    rc = lib().ctamd_expr_run_f32(arr, len(prog), pin, len(inputs), pout, n_out, ptr(status), rows, cols, stream())
+    assert rc == expect, (rc, lib().ctamd_last_error().decode())
+    return outs, int(status.cpu()[0])

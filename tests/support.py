@@ -303,6 +303,23 @@ class Oracle:
         return Y, np.float32(mse.value), np.float32(mae.value), gX, gR
 
     # ---- the MNIST demo's path
+    def expr_run(self, prog, inputs, n_out, rows, cols):
+        """prog: [(op, dst, a, b, imm)] of the fused-expression opcodes; inputs: full [rows, cols] or
+        row-vector [cols] arrays; returns (outputs, status)."""
+        prog = list(prog)
+        codes = np.ascontiguousarray([[q[0], q[1], q[2], q[3]] for q in prog], np.int32).reshape(-1, 4)
+        imm = f32([q[4] for q in prog]) if prog else f32([0])
+        ins = [f32(x) for x in inputs]
+        outs = [np.zeros((rows, cols), np.float32) for _ in range(n_out)]
+        pin = (C.c_void_p * max(1, len(ins)))(*[x.ctypes.data for x in ins])
+        pout = (C.c_void_p * max(1, n_out))(*[x.ctypes.data for x in outs])
+        status = C.c_int(0)
+        self.lib.co_expr_run.restype = C.c_int
+        rc = self.lib.co_expr_run(codes.ctypes.data_as(C.c_void_p), fp(imm), C.c_int(len(prog)), pin, C.c_int(len(ins)), pout,
+                                  C.c_int(n_out), C.c_long(rows), C.c_long(cols), C.byref(status))
+        assert rc == 0, rc
+        return outs, status.value
+
     def u8_to_unit(self, src):
         src = np.ascontiguousarray(src, dtype=np.uint8)
         r = np.empty(src.shape, np.float32)
@@ -381,6 +398,41 @@ def libc_xavier(shape, fan_in, reseed=None):
     raw = np.array([libc.rand() for _ in range(n)], dtype=np.int64)
     r = (np.float32(2.0) * raw.astype(np.float32)) / np.float32(2147483647) - np.float32(1.0)
     return (r.astype(np.float32) * np.sqrt(np.float32(1.0) / np.float32(fan_in))).astype(np.float32).reshape(shape)
+
+
+# opcodes of the fused-expression programs (include/ctorch_amd.h, CTAMD_EX_*)
+EX = dict(LOAD_FULL=0, LOAD_ROW=1, ADD=2, SUB=3, MUL=4, DIV=5, NEG=6, RELU=7, SIGMOID=8, TANH=9, SIN=10, COS=11,
+          ADDS=12, MULS=13, DIVS=14, RSUBS=15, RELUMUL=16, DIVCHK=17, STORE=18, STORE_ZP=19)
+
+
+def random_slot_program(seed, n_full=2, n_row=1, n_ops=20, n_out=2, slots=12):
+    """A random well-formed fused-expression program: loads of every input, n_ops operators over
+    slots that have been written (slots are overwritten freely), then n_out stores.  Inputs are
+    ordered full tensors first, then row vectors.  Returns [(op, dst, a, b, imm)]."""
+    rng = np.random.default_rng(seed)
+    prog, written = [], []
+    for k in range(n_full + n_row):
+        prog.append((EX["LOAD_FULL"] if k < n_full else EX["LOAD_ROW"], k, k, 0, 0.0))
+        written.append(k)
+    binary = [EX[n] for n in ("ADD", "SUB", "MUL", "DIV", "RELUMUL")]
+    unary = [EX[n] for n in ("NEG", "RELU", "SIGMOID", "TANH", "SIN", "COS")]
+    scalar = [EX[n] for n in ("ADDS", "MULS", "DIVS", "RSUBS")]
+    for _ in range(n_ops):
+        r = rng.integers(0, 10)
+        dst = int(rng.integers(0, slots))
+        a, b = int(rng.choice(written)), int(rng.choice(written))
+        if r < 4:
+            prog.append((int(rng.choice(binary)), dst, a, b, 0.0))
+        elif r < 8:
+            prog.append((int(rng.choice(unary)), dst, a, 0, 0.0))
+        else:
+            prog.append((int(rng.choice(scalar)), dst, a, 0, float(np.float32(0.5 + 0.25 * rng.integers(0, 8)))))
+        if dst not in written:
+            written.append(dst)
+    prog.append((EX["DIVCHK"], 0, int(rng.choice(written)), 0, 0.0))
+    for k in range(n_out):
+        prog.append((EX["STORE_ZP"] if k % 2 else EX["STORE"], k, int(written[-1 - k % len(written)]), 0, 0.0))
+    return prog
 
 
 def random_program(seed, rows=6, cols=8, n_in=4, n_ops=14):

@@ -189,3 +189,45 @@ def test_tape_programs_against_an_fp64_interpreter(golden):
         for i, want in enumerate(g64):
             got = g["p%d_g%d" % (seed, i)]
             assert np.abs(got - want).max() <= 1e-5 * (1 + np.abs(want).max()), (seed, i)
+
+
+def test_program_interpreter_equals_the_whole_tensor_functions(oracle):
+    """The oracle's per-element program interpreter against its own whole-tensor functions (which
+    the reference build and the golden vectors pin), opcode by opcode and on the config-5 chain."""
+    from support import EX as E
+    rows, cols = 9, 20
+    x = oracle.uniform((rows, cols), 11, -3, 3)
+    y = oracle.uniform((rows, cols), 12, 0.5, 2)
+    r = oracle.uniform((cols,), 13, 0.5, 2)
+    load = [(E["LOAD_FULL"], 0, 0, 0, 0.0), (E["LOAD_FULL"], 1, 1, 0, 0.0), (E["LOAD_ROW"], 2, 2, 0, 0.0)]
+    cases = [("ADD", oracle.add(x, y)), ("SUB", oracle.sub(x, y)), ("MUL", oracle.mul(x, y)), ("DIV", oracle.div(x, y)),
+             ("RELUMUL", oracle.relu_bwd(x, y))]
+    for name, want in cases:
+        (got,), _ = oracle.expr_run(load + [(E[name], 3, 0, 1, 0.0), (E["STORE"], 0, 3, 0, 0.0)], [x, y, r], 1, rows, cols)
+        assert same_bits(got, want), name
+    for name, want in [("NEG", oracle.neg(x)), ("RELU", oracle.relu(x)), ("SIGMOID", oracle.sigmoid(x)),
+                       ("TANH", oracle.tanh(x)), ("SIN", oracle.sin(x)), ("COS", oracle.cos(x))]:
+        (got,), _ = oracle.expr_run(load + [(E[name], 3, 0, 0, 0.0), (E["STORE"], 0, 3, 0, 0.0)], [x, y, r], 1, rows, cols)
+        assert same_bits(got, want), name
+    for name, which in [("ADDS", 0), ("MULS", 1), ("DIVS", 2)]:
+        (got,), _ = oracle.expr_run(load + [(E[name], 3, 0, 0, 0.75), (E["STORE"], 0, 3, 0, 0.0)], [x, y, r], 1, rows, cols)
+        assert same_bits(got, oracle.scalar(which, x, 0.75)), name
+    (got,), _ = oracle.expr_run(load + [(E["RSUBS"], 3, 0, 0, 1.0), (E["STORE"], 0, 3, 0, 0.0)], [x, y, r], 1, rows, cols)
+    assert same_bits(got, (np.float32(1.0) - x).astype(np.float32))
+    (got,), _ = oracle.expr_run(load + [(E["DIV"], 3, 0, 2, 0.0), (E["STORE"], 0, 3, 0, 0.0)], [x, y, r], 1, rows, cols)
+    assert same_bits(got, oracle.binary_rowbcast(DIV, x, r))
+    # -0 + 0 = +0 through STORE_ZP, kept by STORE
+    z = np.full((rows, cols), -0.0, np.float32)
+    (a, b), _ = oracle.expr_run([(E["LOAD_FULL"], 0, 0, 0, 0.0), (E["STORE"], 0, 0, 0, 0.0), (E["STORE_ZP"], 1, 0, 0, 0.0)],
+                                [z], 2, rows, cols)
+    assert np.signbit(a).all() and not np.signbit(b).any()
+    # the config-5 expression against the oracle's own (reference-pinned) statement of it
+    X = oracle.uniform((rows, cols), 501, -2, 2)
+    T = oracle.normal((rows, cols), 503)
+    R = np.broadcast_to(r, X.shape).copy()
+    Y = oracle.expr(X, R, T)[0]
+    prog = [(E["LOAD_FULL"], 0, 0, 0, 0.0), (E["LOAD_ROW"], 1, 1, 0, 0.0), (E["DIV"], 2, 0, 1, 0.0), (E["SIGMOID"], 2, 2, 0, 0.0),
+            (E["TANH"], 3, 0, 0, 0.0), (E["SIN"], 4, 0, 0, 0.0), (E["MUL"], 3, 3, 4, 0.0), (E["SUB"], 2, 2, 3, 0.0),
+            (E["NEG"], 3, 0, 0, 0.0), (E["COS"], 3, 3, 0, 0.0), (E["ADD"], 2, 2, 3, 0.0), (E["STORE"], 0, 2, 0, 0.0)]
+    (got,), _ = oracle.expr_run(prog, [X, r], 1, rows, cols)
+    assert same_bits(got, Y)
