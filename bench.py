@@ -151,6 +151,12 @@ def config_report(with_cpu):
     rc = host.cth_time_chain(fp(a), fp(b), L(n), I(5), I(50), out)
     cpu = _timed(lambda: ref.chain(a, b)) if with_cpu else None
     add("config 1: c=a*b+5, relu, sum, backward; n=2^20", rc, out, cpu, "whole step", launch_bound=True)
+    # the elementwise chain as one fused expression (one launch forward, one backward); same bits
+    host.cth_set_fused_expr(1)
+    out = D5()
+    rc = host.cth_time_chain(fp(a), fp(b), L(n), I(5), I(50), out)
+    host.cth_set_fused_expr(0)
+    add("config 1: c=a*b+5, relu, sum, backward; n=2^20, fused expression", rc, out, cpu, "whole step", launch_bound=True)
 
     # config 2: MatMul forward + backward at 1024, 2048, 4096; Dot 2^26
     slab_ms = {}
@@ -245,6 +251,13 @@ def config_report(with_cpu):
         t = _timed(lambda: ref.expr(Xs, Rs, Ts))
         cpu, note = t * (R5 / r), "rows 0..%d with the row vector materialised (%.2f s), x%d" % (r - 1, t / 1e3, R5 // r)
     add("config 5: Y=sigmoid(X/r)-tanh(X)*sin(X)+cos(-X), MSE+MAE, backward; X [4096 x 4096]", rc, out, cpu, note)
+    # Y as one fused expression: one pass forward, one pass for dX and dr; same Y and dX bits
+    host.cth_set_fused_expr(1)
+    out = D5()
+    rc = host.cth_time_expr(fp(X), fp(rv), fp(T), L(R5), L(R5), I(3), I(10), out)
+    host.cth_set_fused_expr(0)
+    add("config 5: Y=sigmoid(X/r)-tanh(X)*sin(X)+cos(-X), MSE+MAE, backward; X [4096 x 4096], fused expression", rc, out, cpu,
+        note)
     return {"cores": 1, "cpu_kind": cpu_kind if with_cpu else None, "steps": rows}
 
 

@@ -46,31 +46,47 @@ struct ExprArgs {
     DevInsn prog[kMaxInsns];
 };
 
-__device__ __forceinline__ float sincos_any(float x, int want_cos, const Tables& t) {
-    float o = cta_sincosf_fast(x, want_cos);
-    if (__builtin_expect(cta_sincos_is_rare(x), 0)) o = cta_sincosf(x, want_cos, t.inv_pio4);
-    return o;
+// One operator on the four elements of a lane; a, b are the operand values.  The operator is chosen
+// once (a scalar branch) and its four evaluations are independent instruction streams that the
+// compiler interleaves: the long dependent chains of the transcendental functors (fp64 inside
+// sinf / cosf) hide each other's latencies.
+template <class F>
+__device__ __forceinline__ void each(float (&o)[kPerLane], F f) {
+#pragma unroll
+    for (int e = 0; e < kPerLane; ++e) o[e] = f(e);
 }
-
-// One operator on one element; a, b are the operand values.
-__device__ __forceinline__ float apply(const DevInsn& q, float a, float b, const Tables& t) {
+__device__ __forceinline__ void apply(const DevInsn& q, const float (&a)[kPerLane], const float (&b)[kPerLane],
+                                      float (&o)[kPerLane], const Tables& t) {
     switch (q.op) {
-        case CTAMD_EX_ADD: return a + b;
-        case CTAMD_EX_SUB: return a - b;
-        case CTAMD_EX_MUL: return a * b;
-        case CTAMD_EX_DIV: return a / b;
-        case CTAMD_EX_NEG: return -a;
-        case CTAMD_EX_RELU: return (0.0f < a) ? a : 0.0f;
-        case CTAMD_EX_SIGMOID: return sigmoid_ref(a, t);
-        case CTAMD_EX_TANH: return tanh_ref(a, t);
-        case CTAMD_EX_SIN: return sincos_any(a, 0, t);
-        case CTAMD_EX_COS: return sincos_any(a, 1, t);
-        case CTAMD_EX_ADDS: return a + q.imm;
-        case CTAMD_EX_MULS: return a * q.imm;
-        case CTAMD_EX_DIVS: return cta_div_rcp(a, q.rcp);
-        case CTAMD_EX_RSUBS: return q.imm - a;
-        case CTAMD_EX_RELUMUL: return b * ((a > 0.0f) ? 1.0f : 0.0f);
-        default: return a;
+        case CTAMD_EX_ADD: each(o, [&](int e) { return a[e] + b[e]; }); break;
+        case CTAMD_EX_SUB: each(o, [&](int e) { return a[e] - b[e]; }); break;
+        case CTAMD_EX_MUL: each(o, [&](int e) { return a[e] * b[e]; }); break;
+        case CTAMD_EX_DIV: each(o, [&](int e) { return a[e] / b[e]; }); break;
+        case CTAMD_EX_NEG: each(o, [&](int e) { return -a[e]; }); break;
+        case CTAMD_EX_RELU: each(o, [&](int e) { return (0.0f < a[e]) ? a[e] : 0.0f; }); break;
+        case CTAMD_EX_SIGMOID: each(o, [&](int e) { return sigmoid_ref(a[e], t); }); break;
+        case CTAMD_EX_TANH: each(o, [&](int e) { return tanh_ref(a[e], t); }); break;
+        case CTAMD_EX_SIN:
+        case CTAMD_EX_COS: {
+            const int want_cos = (q.op == CTAMD_EX_COS);
+            bool rare = false;
+#pragma unroll
+            for (int e = 0; e < kPerLane; ++e) {
+                o[e] = cta_sincosf_fast(a[e], want_cos);
+                rare = rare || cta_sincos_is_rare(a[e]);
+            }
+            if (__builtin_expect(rare, 0)) {
+                for (int e = 0; e < kPerLane; ++e)
+                    if (cta_sincos_is_rare(a[e])) o[e] = cta_sincosf(a[e], want_cos, t.inv_pio4);
+            }
+            break;
+        }
+        case CTAMD_EX_ADDS: each(o, [&](int e) { return a[e] + q.imm; }); break;
+        case CTAMD_EX_MULS: each(o, [&](int e) { return a[e] * q.imm; }); break;
+        case CTAMD_EX_DIVS: each(o, [&](int e) { return cta_div_rcp(a[e], q.rcp); }); break;
+        case CTAMD_EX_RSUBS: each(o, [&](int e) { return q.imm - a[e]; }); break;
+        case CTAMD_EX_RELUMUL: each(o, [&](int e) { return b[e] * ((a[e] > 0.0f) ? 1.0f : 0.0f); }); break;
+        default: each(o, [&](int e) { return a[e]; }); break;
     }
 }
 
@@ -158,9 +174,15 @@ __global__ __launch_bounds__(kExprThreads) void expr_kernel(ExprArgs g) {
                 if (bad) atomicOr(g.status, 1);
             } else {
                 // lanes past the end compute on whatever their slots hold and store nothing
-#pragma unroll 1
-                for (int e = 0; e < kPerLane; ++e)
-                    d[e * kExprThreads] = apply(q, pa[e * kExprThreads], pb[e * kExprThreads], tabs);
+                float a[kPerLane], b[kPerLane], o[kPerLane];
+#pragma unroll
+                for (int e = 0; e < kPerLane; ++e) {
+                    a[e] = pa[e * kExprThreads];
+                    b[e] = pb[e * kExprThreads];
+                }
+                apply(q, a, b, o, tabs);
+#pragma unroll
+                for (int e = 0; e < kPerLane; ++e) d[e * kExprThreads] = o[e];
             }
         }
     }

@@ -54,6 +54,10 @@ enum class LeafValues { kLive, kReferenceFirstSeen };
 
 class AutoDiff {
    public:
+    // what an operator needs in backward beyond its inputs (the compiled program of op::Fused)
+    struct OpPayload {
+        virtual ~OpPayload() = default;
+    };
     struct Node {
         size_t tensor_id = 0;
         op operation = op::Add;
@@ -62,6 +66,8 @@ class AutoDiff {
         std::unique_ptr<Tensor> tensor;   // shares storage with the user's tensor
         std::unique_ptr<Tensor> grad;
         std::unique_ptr<Tensor> shared_term;   // backward only: a factor that several inputs' gradients use
+        std::vector<Tensor> input_grads;       // backward only: gradients of all inputs, computed together
+        std::shared_ptr<OpPayload> payload;
         bool requires_grad = false;
         bool is_leaf = true;
     };
@@ -74,7 +80,8 @@ class AutoDiff {
     void zero_grad(Tensor& t);
     Tensor get_grad(const Tensor* t);
     Tensor stored_grad(const Tensor& t);   // extension: the stored bytes, shared; see AutoDiff.cpp
-    void defer_record(size_t output_id, op operation, const std::vector<Tensor*>& inputs, int op_param_i = 0);
+    void defer_record(size_t output_id, op operation, const std::vector<Tensor*>& inputs, int op_param_i = 0,
+                      std::shared_ptr<OpPayload> payload = nullptr);
     void commit_record(Tensor& output);
     void set_retain_graph(bool retain) { retain_graph_ = retain; }
     void backward(Tensor& root);
@@ -95,6 +102,7 @@ class AutoDiff {
         op operation;
         std::vector<size_t> input_ids;
         int op_param_i;
+        std::shared_ptr<OpPayload> payload;
     };
     std::mutex records_mutex;
     std::unordered_map<size_t, std::unique_ptr<Node>> id_to_node;

@@ -21,6 +21,7 @@ enum class op {
     MSE, MAE, CE, BCE,
     Sum,
     Linear,   // not in the reference: matmul + bias row (+ ReLU) as one taped operator, Tensor::linear
+    Fused,    // not in the reference: an elementwise expression evaluated in one pass, Expr::eval
 };
 
 enum class ErrorLevel { TRACE = 0, DEBUG = 1, INFO = 2, WARN = 3, ERROR = 4, FATAL = 5 };

@@ -9,6 +9,7 @@
 #include <algorithm>
 
 #include "Ctorch_Scheduler.h"
+#include "Expr.h"
 #include "kernels.h"
 
 using namespace ctorch_amd_host;
@@ -84,8 +85,9 @@ Tensor AutoDiff::get_grad(const Tensor* t) {
 
 // src/AutoDiff.cpp:314-370: inputs not yet on the tape become leaves; the op is parked until the
 // output is known to require a gradient
-void AutoDiff::defer_record(size_t output_id, op operation, const std::vector<Tensor*>& inputs, int op_param_i) {
-    Pending p{operation, {}, op_param_i};
+void AutoDiff::defer_record(size_t output_id, op operation, const std::vector<Tensor*>& inputs, int op_param_i,
+                            std::shared_ptr<OpPayload> payload) {
+    Pending p{operation, {}, op_param_i, std::move(payload)};
     for (Tensor* in : inputs) {
         if (!in || in->id() == 0) continue;
         make_leaf(*in, in->requires_grad());
@@ -104,6 +106,7 @@ void AutoDiff::commit_record(Tensor& output) {
     node->tensor_id = output.id();
     node->operation = it->second.operation;
     node->op_param_i = it->second.op_param_i;
+    node->payload = std::move(it->second.payload);
     node->input_ids = std::move(it->second.input_ids);
     node->tensor = std::make_unique<Tensor>(Tensor::alias(output));
     node->requires_grad = true;
@@ -235,6 +238,24 @@ Tensor AutoDiff::input_gradient(Node* node, size_t input_id, size_t input_pos, c
             if (input_pos == 0) return MatMul_AMD_kernel(gz, Tensor::view_t(other));   // gz . W^T
             return MatMul_AMD_kernel(Tensor::view_t(other), gz);                        // x^T . gz
         }
+        case op::Fused: {                                               // every operator branch above, in one launch
+            if (node->input_grads.empty()) {
+                auto* program = dynamic_cast<FusedPayload*>(node->payload.get());
+                if (!program)
+                    Ctorch_Error::throwException(ErrorPlatform::kAutoDiff, ErrorType::TENSOR_STATE, "backward: fused operator without its program");
+                std::vector<const Tensor*> inputs;
+                std::vector<bool> wanted;
+                for (size_t id : node->input_ids) {
+                    Node* in = find(id);
+                    inputs.push_back(in->tensor.get());
+                    wanted.push_back(in->requires_grad);
+                }
+                node->input_grads = program->backward(inputs, wanted, g, check_div_zero_);
+            }
+            if (input_pos >= node->input_grads.size() || node->input_grads[input_pos].is_cleared())
+                return Tensor(ShapeTag{}, x.sizes(), DType::kFloat, x.device());   // not reached: zeros
+            return Tensor::alias(node->input_grads[input_pos]);
+        }
         case op::Sum:                                                   // :1850-1855
             return adjust_grad_shape(g, x.sizes());
         case op::Dot: {                                                 // extension: g * other
@@ -323,5 +344,6 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
             }
         }
         node->shared_term.reset();
+        node->input_grads.clear();
     }
 }

@@ -5,6 +5,7 @@
 // threw (-1) or produced an empty tensor (-2).
 #include "Tensor.h"
 #include "AutoDiff.h"
+#include "Expr.h"
 #include "Ctorch_Error.h"
 #include "Ctorch_Scheduler.h"
 
@@ -56,6 +57,28 @@ Tensor run_binary(int code, const Tensor& a, const Tensor& b) {
     throw std::runtime_error("bad binary code");
 }
 
+Expr run_binary(int code, const Expr& a, const Expr& b) {
+    switch (code) {
+        case kAdd: return a + b;
+        case kSub: return a - b;
+        case kMul: return a * b;
+        case kDiv: return a / b;
+    }
+    throw std::runtime_error("bad binary code");
+}
+
+Expr run_unary(int code, const Expr& a) {
+    switch (code) {
+        case kNeg: return -a;
+        case kReLU: return a.relu();
+        case kSin: return a.sin();
+        case kCos: return a.cos();
+        case kTanh: return a.tanh();
+        case kSigmoid: return a.sigmoid();
+    }
+    throw std::runtime_error("bad unary code");
+}
+
 Tensor run_unary(int code, const Tensor& a) {
     switch (code) {
         case kNeg: return -a;
@@ -79,6 +102,10 @@ void cth_quiet() { Ctorch_Error::setPrintLevel(PrintLevel::MINIUM); }
 // Applies to the contexts the entry points below create.
 static int g_row0 = 0;
 static int g_fused_layers = 0;
+static int g_fused_expr = 0;
+// the elementwise parts of cth_chain, cth_expr, cth_program and their timed versions are built as
+// one fused expression (Expr::eval: one launch forward, one backward) when set
+void cth_set_fused_expr(int on) { g_fused_expr = on; }
 void cth_set_reference_row0(int on) { g_row0 = on; }
 // the MLP entry points below build each layer with Tensor::linear (one fused operator) when set
 void cth_set_fused_layers(int on) { g_fused_layers = on; }
@@ -235,8 +262,7 @@ long cth_chain(const float* a, const float* b, long n, float* s_out, float* ga, 
         Tensor ta = make(a, d1, 1), tb = make(b, d1, 1);
         ta.requires_grad(true);
         tb.requires_grad(true);
-        Tensor c = ta * tb + 5.0f;
-        Tensor d = c.relu();
+        Tensor d = g_fused_expr ? (Expr(ta) * Expr(tb) + 5.0f).relu().eval() : (ta * tb + 5.0f).relu();
         Tensor s = d.sum();
         s_out[0] = s.item<float>();
         s.backward();
@@ -294,15 +320,21 @@ long cth_expr(const float* X, const float* R, const float* T, long rows, long co
         Tensor tX = make(X, d, 2), tR = r_is_row_vector ? make(R, dv, 1) : make(R, d, 2), tT = make(T, d, 2);
         tX.requires_grad(true);
         tR.requires_grad(true);
-        Tensor q = tX / tR;
-        Tensor s1 = q.sigmoid();
-        Tensor th = tX.tanh();
-        Tensor sn = tX.sin();
-        Tensor m = th * sn;
-        Tensor d1 = s1 - m;
-        Tensor ng = -tX;
-        Tensor cs = ng.cos();
-        Tensor Y = d1 + cs;
+        Tensor Y;
+        if (g_fused_expr) {
+            Expr x(tX), r(tR);
+            Y = (sigmoid(x / r) - tanh(x) * sin(x) + cos(-x)).eval();
+        } else {
+            Tensor q = tX / tR;
+            Tensor s1 = q.sigmoid();
+            Tensor th = tX.tanh();
+            Tensor sn = tX.sin();
+            Tensor m = th * sn;
+            Tensor d1 = s1 - m;
+            Tensor ng = -tX;
+            Tensor cs = ng.cos();
+            Y = d1 + cs;
+        }
         Tensor l1 = Y.mse_loss(tT);
         Tensor l2 = Y.mae_loss(tT);
         Tensor L = l1 + l2;
@@ -340,6 +372,20 @@ long cth_program(const float* inputs, const int* kinds, int n_in, const int* ops
             src += kinds[i] ? cols : rows * cols;
         }
         for (int i = 0; i < n_in; ++i) v[size_t(i)].requires_grad(true);
+        if (g_fused_expr) {                     // the whole program as one expression
+            std::vector<Expr> e(v.begin(), v.end());
+            for (int k = 0; k < n_ops; ++k) {
+                const int code = ops[3 * k], a = ops[3 * k + 1], b = ops[3 * k + 2];
+                if (code < 20) e.push_back(run_binary(code, e[size_t(a)], e[size_t(b)]));
+                else if (code < 30) e.push_back(run_unary(code, e[size_t(a)]));
+                else {
+                    const float s = 0.5f + 0.25f * float(b);
+                    e.push_back(code == 30 ? e[size_t(a)] + s : code == 31 ? e[size_t(a)] * s : e[size_t(a)] / s);
+                }
+            }
+            v.push_back(e.back().eval());
+            n_ops = 0;
+        }
         for (int k = 0; k < n_ops; ++k) {
             const int code = ops[3 * k], a = ops[3 * k + 1], b = ops[3 * k + 2];
             if (code < 20) v.push_back(run_binary(code, v[size_t(a)], v[size_t(b)]));
@@ -412,7 +458,7 @@ long cth_time_chain(const float* a, const float* b, long n, int warm, int reps, 
         AutoDiffContext::Guard guard(&ctx);
         ta.requires_grad(true);
         tb.requires_grad(true);
-        Tensor s = ((ta * tb + 5.0f).relu()).sum();
+        Tensor s = (g_fused_expr ? (Expr(ta) * Expr(tb) + 5.0f).relu().eval() : (ta * tb + 5.0f).relu()).sum();
         sink = s.item<float>();
         s.backward();
         Tensor ga = grad(ta), gb = grad(tb);
@@ -541,7 +587,8 @@ long cth_time_expr(const float* X, const float* R, const float* T, long rows, lo
         AutoDiffContext::Guard guard(&ctx);
         tX.requires_grad(true);
         tR.requires_grad(true);
-        Tensor Y = (tX / tR).sigmoid() - tX.tanh() * tX.sin() + (-tX).cos();
+        Tensor Y = g_fused_expr ? (sigmoid(Expr(tX) / Expr(tR)) - tanh(Expr(tX)) * sin(Expr(tX)) + cos(-Expr(tX))).eval()
+                                : (tX / tR).sigmoid() - tX.tanh() * tX.sin() + (-tX).cos();
         Tensor L = Y.mse_loss(tT) + Y.mae_loss(tT);
         sink = L.item<float>();
         backward(L);

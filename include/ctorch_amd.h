@@ -217,7 +217,7 @@ enum {
     CTAMD_EX_STORE = 18,    /* outputs[dst][i] = slot[a]                                            */
     CTAMD_EX_STORE_ZP = 19  /* outputs[dst][i] = 0 + slot[a]   (a gradient read from the tape)      */
 };
-#define CTAMD_EXPR_MAX_INSNS 96
+#define CTAMD_EXPR_MAX_INSNS 160
 #define CTAMD_EXPR_MAX_SLOTS 32
 #define CTAMD_EXPR_MAX_PORTS 8
 typedef struct ctamd_expr_insn {

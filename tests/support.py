@@ -809,6 +809,11 @@ class HostLayer(Reference):
     def set_reference_row0(self, on):
         self.cdll.cth_set_reference_row0(int(on))
 
+    def set_fused_expr(self, on):
+        """chain, expr, program and their timed versions evaluate their elementwise part as one fused
+        expression (Expr::eval): one launch forward, one backward."""
+        self.cdll.cth_set_fused_expr(int(on))
+
     def set_fused_layers(self, on):
         """mlp_step builds each layer with Tensor::linear (matmul + bias + ReLU as one operator)."""
         self.cdll.cth_set_fused_layers(int(on))
@@ -816,8 +821,16 @@ class HostLayer(Reference):
     def mlp_step(self, x, W1, b1, W2, b2, target, target_is_index=False):
         return Reference.mlp_step(self, x, W1, b1, W2, b2, target, C.c_int(int(target_is_index)))
 
-    def expr(self, X, R, T):
-        """R may be the full [rows, cols] operand or the row vector [cols] (row-broadcast Div)."""
+    def expr(self, X, R, T, expect_failure=False):
+        """R may be the full [rows, cols] operand or the row vector [cols] (row-broadcast Div).
+        expect_failure: the call must report an exception (returns None)."""
+        if expect_failure:
+            try:
+                Reference.expr(self, X, R, T, C.c_int(int(np.ndim(R) == 1)))
+            except AssertionError as e:
+                assert e.args and e.args[0] == -1, e.args
+                return None
+            raise AssertionError("the call succeeded")
         return Reference.expr(self, X, R, T, C.c_int(int(np.ndim(R) == 1)))
 
     # ---- the MNIST demo's path on the device

@@ -99,6 +99,6 @@ def test_malformed_programs_are_refused(oracle):
     for prog in bad:
         rc = -5 if prog[0][1] == 40 else -1
         G.expr_run(prog, [x], 1, 4, 8, expect=rc)
-    G.expr_run([(E["LOAD_FULL"], 0, 0, 0, 0.0)] * 97, [x], 1, 4, 8, expect=-5)   # too long
+    G.expr_run([(E["LOAD_FULL"], 0, 0, 0, 0.0)] * 161, [x], 1, 4, 8, expect=-5)   # too long
     outs, _ = G.expr_run([], [x], 1, 4, 8)                                        # empty: nothing happens
     assert not G.host(outs[0]).any()

@@ -255,3 +255,64 @@ def test_tape_programs_against_the_reference_vectors(oracle, host, golden):
         assert rc >= 0 and np.abs(y - y64).max() <= 1e-5 * (1 + np.abs(y64).max())
         for got, want in zip(grads, g64):
             assert np.abs(got - want).max() <= 2e-5 * (1 + np.abs(want).max()), seed
+
+
+def test_fused_expressions_against_the_reference_vectors(oracle, host, golden):
+    """The same random programs with every chain of elementwise operators built as ONE fused
+    expression (one launch forward, one launch for all gradients): in the reference's gradient mode
+    the result and every gradient must still have the reference's bits; in the default mode the
+    gradients must agree with the mathematics (a row vector used twice is summed over the rows
+    once instead of twice, which rounds differently).  Then the two benchmark chains."""
+    import importlib.util
+    import os
+    from support import program_fp64, program_inputs, random_program
+    spec = importlib.util.spec_from_file_location("make_golden", os.path.join(os.path.dirname(__file__), "golden",
+                                                                            "make_golden.py"))
+    mg = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mg)
+    g = golden("programs")
+    host.set_fused_expr(True)
+    try:
+        host.set_reference_row0(True)
+        for seed in mg.PROGRAM_SEEDS:
+            print("case fused program", seed, flush=True)
+            rows, cols = mg.program_shape(seed)
+            kinds, ops = random_program(seed)
+            xs, w = program_inputs(oracle, seed, kinds, rows, cols)
+            rc, y, L, grads = host.program(xs, kinds, ops, w)
+            assert rc >= 0, seed
+            assert same_bits(y, g["p%d_y" % seed]), seed
+            for i, got in enumerate(grads):
+                assert same_bits(got, g["p%d_g%d" % (seed, i)]), (seed, i)
+        host.set_reference_row0(False)
+        for seed in list(mg.PROGRAM_SEEDS)[::3]:
+            rows, cols = mg.program_shape(seed)
+            kinds, ops = random_program(seed)
+            xs, w = program_inputs(oracle, seed, kinds, rows, cols)
+            rc, y, L, grads = host.program(xs, kinds, ops, w)
+            y64, L64, g64 = program_fp64(xs, kinds, ops, w, row0=False)
+            assert rc >= 0 and np.abs(y - y64).max() <= 1e-5 * (1 + np.abs(y64).max())
+            for got, want in zip(grads, g64):
+                assert np.abs(got - want).max() <= 2e-5 * (1 + np.abs(want).max()), seed
+        # config 1 and config 5, fused, against the operator-by-operator front-end
+        c = golden("configs")
+        s1, ga1, gb1 = host.chain(c["chain_a"], c["chain_b"])
+        X, rv, T = c["expr_X"], c["expr_r"], c["expr_T"]
+        fused5 = host.expr(X, rv, T)
+        host.set_fused_expr(False)
+        s0, ga0, gb0 = host.chain(c["chain_a"], c["chain_b"])
+        assert s1 == s0 and same_bits(ga1, ga0) and same_bits(gb1, gb0)
+        assert same_bits(ga1, c["chain_ga"]) and same_bits(gb1, c["chain_gb"])     # the reference's bits
+        plain5 = host.expr(X, rv, T)
+        assert same_bits(fused5[0], plain5[0]) and fused5[1] == plain5[1] and fused5[2] == plain5[2]
+        assert same_bits(fused5[3], plain5[3])                                       # gX: same order of the four terms
+        assert np.abs(fused5[4] - plain5[4]).max() <= 1e-5 * np.abs(plain5[4]).max()  # gr: one column sum instead of ... one
+        # a zero divisor is refused in backward, as by the tape's own Div gradient
+        host.set_fused_expr(True)
+        rz = rv.copy()
+        rz[3] = 0.0
+        bad = host.expr(X, rz, T, expect_failure=True)
+        assert bad is None
+    finally:
+        host.set_fused_expr(False)
+        host.set_reference_row0(False)
