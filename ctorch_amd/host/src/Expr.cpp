@@ -97,7 +97,23 @@ bool is_load(int op) { return op == CTAMD_EX_LOAD_FULL || op == CTAMD_EX_LOAD_RO
 // Slot assignment: a value's slot is free again after its last use; a result may take the slot of
 // an operand that dies in the same instruction (operands are read before the result is written).
 // False when the program needs more than the launch layer's slots or instructions.
-bool lower(const Code& c, std::vector<ctamd_expr_insn>& out) {
+bool lower(const Code& in, std::vector<ctamd_expr_insn>& out) {
+    // loads first: the kernel issues the loads at the head of a program together
+    Code c;
+    {
+        std::vector<int> renumber(in.code.size(), -1);
+        for (int pass = 0; pass < 2; ++pass)
+            for (size_t i = 0; i < in.code.size(); ++i) {
+                Code::I q = in.code[i];
+                if (is_load(q.op) != (pass == 0)) continue;
+                if (!is_load(q.op)) {
+                    q.a = renumber[size_t(q.a)];
+                    q.b = renumber[size_t(q.b)];
+                }
+                renumber[i] = int(c.code.size());
+                c.code.push_back(q);
+            }
+    }
     const int n = int(c.code.size());
     if (n > CTAMD_EXPR_MAX_INSNS) return false;
     std::vector<int> last(size_t(n), -1);

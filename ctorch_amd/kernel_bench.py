@@ -93,6 +93,27 @@ def main():
     ew("dot", lambda k: call("ctamd_dot_f32", P(A[k]), P(B[k]), P(out), n, S), 8)
     ew("mse", lambda k: call("ctamd_mse_f32", P(A[k]), P(B[k]), P(out), n, S), 8)
     ew("mae", lambda k: call("ctamd_mae_f32", P(A[k]), P(B[k]), P(out), n, S), 8)
+    # fused expressions: a cheap chain (bound by the memory stream) ...
+    class Insn(C.Structure):
+        _fields_ = [("op", C.c_uint8), ("dst", C.c_uint8), ("a", C.c_uint8), ("b", C.c_uint8), ("imm", C.c_float)]
+
+    def program(*insns):
+        return (Insn * len(insns))(*[Insn(*q) for q in insns]), len(insns)
+
+    def run_expr(prog, ins, outs, rows, cols):
+        pin = (C.c_void_p * len(ins))(*[t.data_ptr() for t in ins])
+        pout = (C.c_void_p * len(outs))(*[t.data_ptr() for t in outs])
+        call("ctamd_expr_run_f32", prog[0], prog[1], pin, len(ins), pout, len(outs), None, rows, cols, S)
+
+    LOADF, LOADR, ADD, SUB, MUL, DIV, NEG, RELU, SIGM, TANH, SIN, COS, ADDS, STORE = 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 18
+    chain = program((LOADF, 0, 0, 0, 0.0), (LOADF, 1, 1, 0, 0.0), (MUL, 0, 0, 1, 0.0), (ADDS, 0, 0, 0, 5.0), (RELU, 0, 0, 0, 0.0),
+                    (STORE, 0, 0, 0, 0.0))
+    ew("fused relu(a * b + 5)", lambda k: run_expr(chain, [A[k], B[k]], [R[k]], 16384, 4096), 12)
+    # ... and the config-5 expression sigmoid(X / r) - tanh(X) * sin(X) + cos(-X) (bound by its five transcendentals)
+    c5 = program((LOADF, 0, 0, 0, 0.0), (LOADR, 1, 1, 0, 0.0), (DIV, 2, 0, 1, 0.0), (SIGM, 2, 2, 0, 0.0), (TANH, 3, 0, 0, 0.0),
+                 (SIN, 4, 0, 0, 0.0), (MUL, 3, 3, 4, 0.0), (SUB, 2, 2, 3, 0.0), (NEG, 3, 0, 0, 0.0), (COS, 3, 3, 0, 0.0),
+                 (ADD, 2, 2, 3, 0.0), (STORE, 0, 2, 0, 0.0))
+    ew("fused sigmoid(X/r) - tanh(X)*sin(X) + cos(-X) [16384 x 4096]", lambda k: run_expr(c5, [A[k], B[0]], [R[k]], 16384, 4096), 8)
     cs = torch.empty(4096, device="cuda")
     ew("column sum [16384 x 4096]", lambda k: call("ctamd_colsum_f32", P(A[k]), P(cs), 16384, 4096, S), 4)
     del A, B, R
