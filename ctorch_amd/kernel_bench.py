@@ -1,6 +1,6 @@
 """Per-kernel timings of the launch layer through the C ABI on one MI355X.
 
-    python -m ctorch_amd.kernel_bench [--json] [--skip-matmul]
+    python -m ctorch_amd.kernel_bench [--json] [--skip-matmul] [--only-expr]
 
 Every operator is launched on operands resident in HBM (torch only provides the memory and the
 stream), timed with events over back-to-back launches after a warm-up, and reported as time,
@@ -22,6 +22,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--json", action="store_true", help="one JSON object instead of a table")
     ap.add_argument("--skip-matmul", action="store_true")
+    ap.add_argument("--only-expr", action="store_true", help="only the fused-expression programs (for counter runs)")
     args = ap.parse_args()
 
     import torch
@@ -78,21 +79,23 @@ def main():
     def ew(name, fn, bytes_per_elem):
         report("%s, n=2^26 (%d B/elem)" % (name, bytes_per_elem), timeit(rotating(fn), 20), bytes_per_elem * n)
 
-    for op in ("add", "sub", "mul", "div"):
+    plain = not args.only_expr
+    for op in ("add", "sub", "mul", "div") if plain else ():
         ew(op, lambda k, op=op: call("ctamd_%s_f32" % op, P(A[k]), P(B[k]), P(R[k]), n, S), 12)
-    for op in ("neg", "relu", "sin", "cos", "tanh", "sigmoid"):
+    for op in ("neg", "relu", "sin", "cos", "tanh", "sigmoid") if plain else ():
         ew(op, lambda k, op=op: call("ctamd_%s_f32" % op, P(A[k]), P(R[k]), n, S), 8)
-    for op in ("relu", "sigmoid", "tanh", "sin", "cos"):
+    for op in ("relu", "sigmoid", "tanh", "sin", "cos") if plain else ():
         ew(op + " backward", lambda k, op=op: call("ctamd_%s_backward_f32" % op, P(A[k]), P(B[k]), P(R[k]), n, S), 12)
-    ew("tensor + scalar", lambda k: call("ctamd_add_scalar_f32", P(A[k]), C.c_float(5.0), P(R[k]), n, S), 8)
-    ew("fill", lambda k: call("ctamd_fill_f32", P(R[k]), C.c_float(5.0), n, S), 4)
-    ew("accumulate", lambda k: call("ctamd_accumulate_f32", P(R[k]), P(A[k]), n, S), 12)
-    ew("sgd step", lambda k: call("ctamd_sgd_step_f32", P(R[k]), P(A[k]), C.c_float(0.01), n, S), 12)
-    ew("row-broadcast div [16384 x 4096]", lambda k: call("ctamd_div_rowbcast_f32", P(A[k]), P(B[0]), P(R[k]), 16384, 4096, S), 8)
-    ew("sum", lambda k: call("ctamd_sum_f32", P(A[k]), P(out), n, S), 4)
-    ew("dot", lambda k: call("ctamd_dot_f32", P(A[k]), P(B[k]), P(out), n, S), 8)
-    ew("mse", lambda k: call("ctamd_mse_f32", P(A[k]), P(B[k]), P(out), n, S), 8)
-    ew("mae", lambda k: call("ctamd_mae_f32", P(A[k]), P(B[k]), P(out), n, S), 8)
+    if plain:
+        ew("tensor + scalar", lambda k: call("ctamd_add_scalar_f32", P(A[k]), C.c_float(5.0), P(R[k]), n, S), 8)
+        ew("fill", lambda k: call("ctamd_fill_f32", P(R[k]), C.c_float(5.0), n, S), 4)
+        ew("accumulate", lambda k: call("ctamd_accumulate_f32", P(R[k]), P(A[k]), n, S), 12)
+        ew("sgd step", lambda k: call("ctamd_sgd_step_f32", P(R[k]), P(A[k]), C.c_float(0.01), n, S), 12)
+        ew("row-broadcast div [16384 x 4096]", lambda k: call("ctamd_div_rowbcast_f32", P(A[k]), P(B[0]), P(R[k]), 16384, 4096, S), 8)
+        ew("sum", lambda k: call("ctamd_sum_f32", P(A[k]), P(out), n, S), 4)
+        ew("dot", lambda k: call("ctamd_dot_f32", P(A[k]), P(B[k]), P(out), n, S), 8)
+        ew("mse", lambda k: call("ctamd_mse_f32", P(A[k]), P(B[k]), P(out), n, S), 8)
+        ew("mae", lambda k: call("ctamd_mae_f32", P(A[k]), P(B[k]), P(out), n, S), 8)
     # fused expressions: a cheap chain (bound by the memory stream) ...
     class Insn(C.Structure):
         _fields_ = [("op", C.c_uint8), ("dst", C.c_uint8), ("a", C.c_uint8), ("b", C.c_uint8), ("imm", C.c_float)]
@@ -108,12 +111,18 @@ def main():
     LOADF, LOADR, ADD, SUB, MUL, DIV, NEG, RELU, SIGM, TANH, SIN, COS, ADDS, STORE = 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 18
     chain = program((LOADF, 0, 0, 0, 0.0), (LOADF, 1, 1, 0, 0.0), (MUL, 0, 0, 1, 0.0), (ADDS, 0, 0, 0, 5.0), (RELU, 0, 0, 0, 0.0),
                     (STORE, 0, 0, 0, 0.0))
+    bare = program((LOADF, 0, 0, 0, 0.0), (STORE, 0, 0, 0, 0.0))
+    ew("fused load + store only", lambda k: run_expr(bare, [A[k]], [R[k]], 16384, 4096), 8)
     ew("fused relu(a * b + 5)", lambda k: run_expr(chain, [A[k], B[k]], [R[k]], 16384, 4096), 12)
     # ... and the config-5 expression sigmoid(X / r) - tanh(X) * sin(X) + cos(-X) (bound by its five transcendentals)
     c5 = program((LOADF, 0, 0, 0, 0.0), (LOADR, 1, 1, 0, 0.0), (DIV, 2, 0, 1, 0.0), (SIGM, 2, 2, 0, 0.0), (TANH, 3, 0, 0, 0.0),
                  (SIN, 4, 0, 0, 0.0), (MUL, 3, 3, 4, 0.0), (SUB, 2, 2, 3, 0.0), (NEG, 3, 0, 0, 0.0), (COS, 3, 3, 0, 0.0),
                  (ADD, 2, 2, 3, 0.0), (STORE, 0, 2, 0, 0.0))
     ew("fused sigmoid(X/r) - tanh(X)*sin(X) + cos(-X) [16384 x 4096]", lambda k: run_expr(c5, [A[k], B[0]], [R[k]], 16384, 4096), 8)
+    if args.only_expr:
+        if args.json:
+            print(json.dumps({"device": torch.cuda.get_device_name(0), "results": results}))
+        return 0
     cs = torch.empty(4096, device="cuda")
     ew("column sum [16384 x 4096]", lambda k: call("ctamd_colsum_f32", P(A[k]), P(cs), 16384, 4096, S), 4)
     del A, B, R
