@@ -125,14 +125,14 @@ struct MseBwdF { static constexpr int kIn = 2; static constexpr bool kTables = f
         float d = x[0] - x[1];
         float d2 = d * 2.0f;
         float q = cta_div_rcp(d2, rfn);          // d2 / float(n)
-        return q * *g; } };
+        return 0.0f + q * *g; } };   // "0 +": the tape adds the term to a zero-filled buffer (-0 becomes +0)
 struct MaeBwdF { static constexpr int kIn = 2; static constexpr bool kTables = false;
     double rfn; const float* g;
     __device__ float operator()(const float* x, const Tables&) const {
         float d = x[0] - x[1];
         float s = (d > 0.0f) ? 1.0f : ((d < 0.0f) ? -1.0f : 0.0f);
         float q = cta_div_rcp(s, rfn);           // sign / float(n)
-        return q * *g; } };
+        return 0.0f + q * *g; } };   // "0 +": the tape adds the term to a zero-filled buffer (-0 becomes +0)
 // inputs (a, b, g): ((-a) * g) / (b * b)
 struct DivBwdBF { static constexpr int kIn = 3; static constexpr bool kTables = false;
     __device__ float operator()(const float* x, const Tables&) const {

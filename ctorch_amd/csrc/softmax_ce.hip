@@ -264,7 +264,7 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
                 p = (p < 1e-10f) ? 1e-10f : p;
                 block_loss -= double(float(log(double(p))));
             }
-        } else {   // kCeBwdOnehot / kCeBwdIndex: dx = (e / s - t) * g
+        } else {   // kCeBwdOnehot / kCeBwdIndex: dx = 0 + (e / s - t) * g (the tape adds it to a zero-filled buffer)
             const float g = a.g1[0];
             if (MODE == kCeBwdOnehot) {
 #pragma unroll
@@ -275,7 +275,7 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
                     for (int i = 0; i < W; ++i) {
                         float sm = cta_div_rcp(r.v[k][i], rcp_s);
                         float d = sm - tq[i];
-                        r.v[k][i] = d * g;
+                        r.v[k][i] = 0.0f + d * g;
                     }
                 }
             } else {
@@ -286,7 +286,7 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
                     for (int i = 0; i < W; ++i) {
                         float sm = cta_div_rcp(r.v[k][i], rcp_s);
                         float d = sm - ((r.index(k, i) == unsigned(c)) ? 1.0f : 0.0f);
-                        r.v[k][i] = d * g;
+                        r.v[k][i] = 0.0f + d * g;
                     }
             }
             r.store(a.out + row * a.cols, unsigned(a.cols));
@@ -416,7 +416,7 @@ __global__ __launch_bounds__(1024) void row_stream_kernel(Args a) {
                 float sm = cta_expf_tab(xr[j] - M, s_exp2) / S;
                 float tj = (MODE == kCeBwdOnehot) ? a.t[row * a.cols + j] : ((j == size_t(c) && c >= 0) ? 1.0f : 0.0f);
                 float d = sm - tj;
-                a.out[row * a.cols + j] = d * g;
+                a.out[row * a.cols + j] = 0.0f + d * g;
             }
         }
     }
@@ -517,7 +517,7 @@ __global__ __launch_bounds__(256) void ce_bwd_stats_kernel(Args a) {
         auto one = [&](float v, unsigned j) {
             float sm = FAST ? __builtin_amdgcn_exp2f((v - M) * kLog2e) * rcp_sf
                             : cta_div_rcp(cta_expf_nonpos(v - M, s_exp2), rcp_s);
-            return (sm - ((j == c) ? 1.0f : 0.0f)) * g;
+            return 0.0f + (sm - ((j == c) ? 1.0f : 0.0f)) * g;
         };
         if (VEC) {
             const unsigned n4 = unsigned(a.cols >> 2);

@@ -65,6 +65,7 @@ class AutoDiff {
         std::vector<size_t> input_ids;
         std::unique_ptr<Tensor> tensor;   // shares storage with the user's tensor
         std::unique_ptr<Tensor> grad;
+        bool grad_plus_zero = false;           // grad holds no -0: "0 + grad" (what get_grad returns) is grad itself
         std::unique_ptr<Tensor> shared_term;   // backward only: a factor that several inputs' gradients use
         std::vector<Tensor> input_grads;       // backward only: gradients of all inputs, computed together
         std::shared_ptr<OpPayload> payload;
@@ -111,6 +112,8 @@ class AutoDiff {
     BroadcastGrad broadcast_grad_ = BroadcastGrad::kColumnSum;
     LeafValues leaf_values_ = LeafValues::kLive;
     bool check_div_zero_ = true;
+    bool term_plus_zero_ = false;   // backward: the term just computed holds no -0
+    bool seed_plus_zero_ = false;   // backward: the seed gradient holds no -0
 
     Node* find(size_t id);
     Tensor adjust_grad_shape(const Tensor& grad, const std::vector<size_t>& target_shape);

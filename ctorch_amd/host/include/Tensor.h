@@ -55,6 +55,8 @@ class Tensor {
     ~Tensor() = default;
 
     static Tensor alias(const Tensor& t) { return Tensor(AliasTag{}, t); }
+    // the same bytes as a tensor of its own (new id, not on the tape): read-only sharing
+    static Tensor share(const Tensor& t);
     // transposed VIEW of a 2-D tensor: shares storage, no copy (the tape's B^T / A^T operands)
     static Tensor view_t(const Tensor& t);
     // rows [first, first + count) of a contiguous tensor as a VIEW (shares storage, new id): what

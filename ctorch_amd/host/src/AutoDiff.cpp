@@ -60,7 +60,10 @@ void AutoDiff::zero_grad(Tensor& t) {
     Node* n = find(t.id());
     // no gradient stored reads as zeros (get_grad) and the next contribution becomes the gradient
     // with its "0 +" pending: the same values as a zero-filled buffer, without the fill
-    if (n) n->grad.reset();
+    if (n) {
+        n->grad.reset();
+        n->grad_plus_zero = false;
+    }
 }
 
 // Not in the reference: the gradient's bytes as the tape holds them (shared, not copied; empty when
@@ -79,7 +82,16 @@ Tensor AutoDiff::get_grad(const Tensor* t) {
     if (!t || t->id() == 0) return Tensor();
     std::lock_guard<std::mutex> lock(records_mutex);
     Node* n = find(t->id());
-    if (n && n->requires_grad && n->grad) return zero_plus(*n->grad, n->grad->sizes());   // the copy, and the pending "0 +"
+    if (n && n->requires_grad && n->grad) {
+        // the pending "0 +" (one pass, once); a gradient known to hold no -0 needs none.  The
+        // result shares the tape's bytes instead of copying them: the tape never writes through
+        // shared bytes (a later contribution goes to a fresh tensor), callers must not either.
+        if (!n->grad_plus_zero) {
+            n->grad = std::make_unique<Tensor>(zero_plus(*n->grad, n->grad->sizes()));
+            n->grad_plus_zero = true;
+        }
+        return Tensor::share(*n->grad);
+    }
     return Tensor(ShapeTag{}, t->shape(), t->dtype(), t->device());
 }
 
@@ -126,13 +138,18 @@ Tensor AutoDiff::adjust_grad_shape(const Tensor& grad, const std::vector<size_t>
     if (grad.sizes() == target) return Tensor::alias(grad);
     if (grad.sizes().empty()) return filled_from(target, grad);                       // :579-627
     if (grad.dim() == 2 && target.size() == 1 && grad.sizes()[1] == target[0]) {      // :690-757
-        return broadcast_grad_ == BroadcastGrad::kColumnSum ? column_sum(grad) : first_row(grad);
+        if (broadcast_grad_ == BroadcastGrad::kColumnSum) {
+            term_plus_zero_ = true;                  // a sum that starts from +0 is never -0
+            return column_sum(grad);
+        }
+        return first_row(grad);
     }
     if (target.empty() || (target.size() == 1 && target[0] == 1)) {
         // gradient of a one-element operand that was broadcast over a whole tensor
         Tensor flat = Tensor::alias(grad);
         if (broadcast_grad_ == BroadcastGrad::kColumnSum) {
             Tensor s = sum_all(flat);
+            term_plus_zero_ = true;
             return target.empty() ? s : filled_from(target, s);
         }
         Tensor first(ShapeTag{}, target, DType::kFloat, grad.device(), false);
@@ -153,16 +170,23 @@ Tensor AutoDiff::input_gradient(Node* node, size_t input_id, size_t input_pos, c
     Node* in = find(input_id);
     const Tensor& x = *in->tensor;
     const bool first = (input_id == node->input_ids[0]);   // the reference tells operands apart by id
+    // does the term hold no -0?  (then "0 + term" is the term and reading it needs no pass)
+    term_plus_zero_ = false;
+    const bool upstream_plus_zero = node->grad_plus_zero;
     auto other_node = [&]() -> Node* {
         if (node->input_ids.size() < 2) return nullptr;
         return find(first ? node->input_ids[1] : node->input_ids[0]);
     };
     switch (node->operation) {
         case op::Add:                                                   // :1216-1221
+            term_plus_zero_ = upstream_plus_zero;
             return adjust_grad_shape(g, x.sizes());
         case op::Sub: {                                                 // :1222-1233
+            term_plus_zero_ = upstream_plus_zero;
             Tensor adj = adjust_grad_shape(g, x.sizes());
-            return first ? adj : Neg_AMD_kernel(adj);
+            if (first) return adj;
+            term_plus_zero_ = false;                                    // -(+0) = -0
+            return Neg_AMD_kernel(adj);
         }
         case op::Mul: {                                                 // :1234-1258: other * g
             Node* o = other_node();
@@ -206,16 +230,21 @@ Tensor AutoDiff::input_gradient(Node* node, size_t input_id, size_t input_pos, c
         case op::Sin: return sin_backward(x, g);                        // :1399-1407
         case op::Cos: return cos_backward(x, g);                        // :1408-1416
         case op::Softmax: return softmax_backward(*node->tensor, g, node->op_param_i);   // :1417-1490
+        // the loss, MatMul and fused-expression gradients below come out of their kernels with the
+        // "0 +" applied or as sums that start from +0
         case op::MSE: {                                                 // :1491-1516
             Node* o = other_node();
+            term_plus_zero_ = true;
             return mse_backward(x, *o->tensor, g);
         }
         case op::MAE: {                                                 // :1602-1642
             Node* o = other_node();
+            term_plus_zero_ = true;
             return mae_backward(x, *o->tensor, g);
         }
         case op::CE: {                                                  // :1517-1601
             Node* o = other_node();
+            term_plus_zero_ = true;
             return cross_entropy_backward(x, *o->tensor, g);
         }
         case op::MatMul: {                                              // :1643-1849
@@ -224,6 +253,7 @@ Tensor AutoDiff::input_gradient(Node* node, size_t input_id, size_t input_pos, c
             if (g.dim() != 2)
                 Ctorch_Error::throwException(ErrorPlatform::kAutoDiff, ErrorType::DIMENSION,
                                              "MatMul gradient must be a 2-D tensor");
+            term_plus_zero_ = true;                                             // sums of products from +0
             if (first) return MatMul_AMD_kernel(g, Tensor::view_t(other));      // g . B^T
             return MatMul_AMD_kernel(Tensor::view_t(other), g);                 // A^T . g
         }
@@ -233,7 +263,11 @@ Tensor AutoDiff::input_gradient(Node* node, size_t input_id, size_t input_pos, c
             if (node->op_param_i && !node->shared_term)
                 node->shared_term = std::make_unique<Tensor>(relu_backward(*node->tensor, g));
             const Tensor& gz = node->op_param_i ? *node->shared_term : g;
-            if (input_pos == 2) return Tensor::alias(gz);               // bias: Add's branch, shaped by the caller
+            if (input_pos == 2) {                                       // bias: Add's branch, shaped by the caller
+                term_plus_zero_ = node->op_param_i ? false : upstream_plus_zero;   // g * 0 may be -0
+                return Tensor::alias(gz);
+            }
+            term_plus_zero_ = true;
             const Tensor& other = *find(node->input_ids[input_pos == 0 ? 1 : 0])->tensor;
             if (input_pos == 0) return MatMul_AMD_kernel(gz, Tensor::view_t(other));   // gz . W^T
             return MatMul_AMD_kernel(Tensor::view_t(other), gz);                        // x^T . gz
@@ -254,9 +288,11 @@ Tensor AutoDiff::input_gradient(Node* node, size_t input_id, size_t input_pos, c
             }
             if (input_pos >= node->input_grads.size() || node->input_grads[input_pos].is_cleared())
                 return Tensor(ShapeTag{}, x.sizes(), DType::kFloat, x.device());   // not reached: zeros
+            term_plus_zero_ = true;                                     // the program stores "0 + term"
             return Tensor::alias(node->input_grads[input_pos]);
         }
         case op::Sum:                                                   // :1850-1855
+            term_plus_zero_ = upstream_plus_zero;
             return adjust_grad_shape(g, x.sizes());
         case op::Dot: {                                                 // extension: g * other
             Node* o = other_node();
@@ -277,6 +313,7 @@ void AutoDiff::backward(Tensor& root) {
     thread_local Tensor device_one;
     if (root.device() == DeviceType::kAMD) {
         if (device_one.is_cleared()) device_one = Tensor(1.0f, DeviceType::kAMD);
+        seed_plus_zero_ = true;
         backward(root, Tensor::alias(device_one));
         return;
     }
@@ -297,6 +334,8 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
     if (!root_node->requires_grad) return;
     if (grad_output.device() != root.device()) grad_output = grad_output.to(root.device());
     root_node->grad = std::make_unique<Tensor>(adjust_grad_shape(grad_output, root.sizes()));
+    root_node->grad_plus_zero = seed_plus_zero_;
+    seed_plus_zero_ = false;
 
     // reversed depth-first post-order, inputs visited in recorded order (:1058-1077, :1138-1153)
     std::vector<Node*> order;
@@ -328,6 +367,7 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
             if (!in || !in->requires_grad) continue;
             Tensor val = input_gradient(node, input_id, pos, node_grad);
             Tensor adj = adjust_grad_shape(val, in->tensor->sizes());
+            const bool plus_zero = term_plus_zero_;
             // :1870-1907 is "zero-filled gradient, then grad += val".  Here the first contribution
             // is kept as it is (no pass over memory; it may share its bytes with another node's
             // gradient) and the "0 +" is applied when the gradient is read (get_grad): adding +0
@@ -335,12 +375,19 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
             // any non-zero value downstream.  Later contributions add in place once the bytes are
             // this node's own, else into a fresh tensor.
             if (!in->grad) {
-                if (adj.sizes() == in->tensor->sizes()) in->grad = std::make_unique<Tensor>(Tensor::alias(adj));
-                else in->grad = std::make_unique<Tensor>(zero_plus(adj, in->tensor->sizes()));
+                if (adj.sizes() == in->tensor->sizes()) {
+                    in->grad = std::make_unique<Tensor>(Tensor::alias(adj));
+                    in->grad_plus_zero = plus_zero;
+                } else {
+                    in->grad = std::make_unique<Tensor>(zero_plus(adj, in->tensor->sizes()));
+                    in->grad_plus_zero = true;
+                }
             } else if (in->grad->storage_shared()) {
                 in->grad = std::make_unique<Tensor>(sum_of(*in->grad, adj));
+                in->grad_plus_zero = in->grad_plus_zero && plus_zero;    // no -0 in, no -0 out
             } else {
                 accumulate(*in->grad, adj);
+                in->grad_plus_zero = in->grad_plus_zero && plus_zero;
             }
         }
         node->shared_term.reset();

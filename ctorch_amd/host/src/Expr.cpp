@@ -291,7 +291,8 @@ struct Program : FusedPayload {
         for (int v = 0; v < n; ++v) {
             const Value& q = vals[size_t(v)];
             if (is_load(q.code) && ((mask >> q.a) & 1u) && adj[size_t(v)] >= 0) {
-                c.effect(CTAMD_EX_STORE, adj[size_t(v)], int(out.out_port.size()));
+                // "0 +": what the tape's zero-filled buffer does to a first contribution
+                c.effect(CTAMD_EX_STORE_ZP, adj[size_t(v)], int(out.out_port.size()));
                 out.out_port.push_back(q.a);
             }
         }

@@ -212,6 +212,13 @@ Tensor Tensor::view_t(const Tensor& t) {
     return r;
 }
 
+Tensor Tensor::share(const Tensor& t) {
+    Tensor r(AliasTag{}, t);
+    r.tensor_id_ = global_tensor_id++;
+    r._requires_grad = false;
+    return r;
+}
+
 Tensor Tensor::view_rows(const Tensor& t, size_t first, size_t count) {
     if (t._shape.empty() || !t.is_contiguous() || first + count > t._shape[0])
         Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DIMENSION, "view_rows: rows out of range or tensor not contiguous");

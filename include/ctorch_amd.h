@@ -257,11 +257,13 @@ int ctamd_softmax_backward_rows_f32(const float* y, const float* g, float* dx, s
                                     void* stream);
 int ctamd_softmax_backward_cols_f32(const float* y, const float* g, float* dx, size_t rows, size_t cols,
                                     void* stream);
-/* dp = (((p - t) * 2) / n) * g[0]; dp = (sign(p - t) / n) * g[0]; g a 0-D device tensor.
- * src/AutoDiff.cpp:1491-1516, :1602-1642. */
+/* dp = 0 + (((p - t) * 2) / n) * g[0]; dp = 0 + (sign(p - t) / n) * g[0]; g a 0-D device tensor.
+ * src/AutoDiff.cpp:1491-1516, :1602-1642; the "0 +" is the tape adding the term to its zero-filled
+ * gradient buffer (:1870-1907): a -0 term is stored as +0.  The cross-entropy gradients below
+ * include it as well. */
 int ctamd_mse_backward_f32(const float* p, const float* t, const float* g1, float* dp, size_t n, void* stream);
 int ctamd_mae_backward_f32(const float* p, const float* t, const float* g1, float* dp, size_t n, void* stream);
-/* dx = (softmax(x) - t) * g[0], gradient of the SUM-reduced loss.  src/AutoDiff.cpp:1546-1574.
+/* dx = 0 + (softmax(x) - t) * g[0], gradient of the SUM-reduced loss.  src/AutoDiff.cpp:1546-1574.
  * The index form takes class indices (the reference throws there, :1569) and equals the one-hot
  * arithmetic with t = onehot(idx). */
 int ctamd_cross_entropy_backward_onehot_f32(const float* x, const float* t, const float* g1, float* dx,
