@@ -48,6 +48,14 @@ class Expr {
     // The value as a tensor; taped as one operator when an autograd context is active.
     Tensor eval() const;
 
+    // Size of the device programs compiled last on this thread, for tests and tuning:
+    // {forward instructions, forward slots, backward instructions, backward slots}; zeros when the
+    // last eval() ran operator by operator.
+    struct ProgramStats {
+        int forward_insns = 0, forward_slots = 0, backward_insns = 0, backward_slots = 0;
+    };
+    static ProgramStats last_program_stats();
+
    private:
     explicit Expr(std::shared_ptr<Node> n) : n_(std::move(n)) {}
     static Expr binary(int code, const Expr& a, const Expr& b);

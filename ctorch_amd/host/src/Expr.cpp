@@ -91,6 +91,15 @@ struct Code {
     void effect(int op, int a, int port) { code.push_back({op, a, a, 0.0f, port}); }
 };
 
+thread_local Expr::ProgramStats t_stats;
+
+int slots_of(const std::vector<ctamd_expr_insn>& code) {
+    int most = 0;
+    for (const ctamd_expr_insn& q : code)
+        if (q.op != CTAMD_EX_STORE && q.op != CTAMD_EX_STORE_ZP && q.op != CTAMD_EX_DIVCHK && q.dst + 1 > most) most = q.dst + 1;
+    return most;
+}
+
 bool has_result(int op) { return op != CTAMD_EX_STORE && op != CTAMD_EX_STORE_ZP && op != CTAMD_EX_DIVCHK; }
 bool is_load(int op) { return op == CTAMD_EX_LOAD_FULL || op == CTAMD_EX_LOAD_ROW; }
 
@@ -472,6 +481,8 @@ Expr Expr::tanh() const { return unary(CTAMD_EX_TANH, *this); }
 Expr Expr::sin() const { return unary(CTAMD_EX_SIN, *this); }
 Expr Expr::cos() const { return unary(CTAMD_EX_COS, *this); }
 
+Expr::ProgramStats Expr::last_program_stats() { return t_stats; }
+
 Tensor Expr::eval() const {
     if (n_->code < 0) return Tensor::alias(n_->tensor);                 // a tensor is its own value
     auto program = std::make_shared<Program>();
@@ -518,9 +529,16 @@ Tensor Expr::eval() const {
             program->backward_code.emplace(std::make_pair(mask, true), std::move(b));
         }
     }
+    t_stats = ProgramStats();
     if (!fusable) {
         std::unordered_map<const Node*, Tensor> memo;
         return eval_plain(n_, memo);
+    }
+    t_stats.forward_insns = int(program->forward_code.size());
+    t_stats.forward_slots = slots_of(program->forward_code);
+    for (const auto& kv : program->backward_code) {
+        t_stats.backward_insns = int(kv.second.code.size());
+        t_stats.backward_slots = slots_of(kv.second.code);
     }
 
     std::vector<const Tensor*> inputs;

@@ -106,6 +106,15 @@ static int g_fused_expr = 0;
 // the elementwise parts of cth_chain, cth_expr, cth_program and their timed versions are built as
 // one fused expression (Expr::eval: one launch forward, one backward) when set
 void cth_set_fused_expr(int on) { g_fused_expr = on; }
+// sizes of the programs the last Expr::eval() compiled: out[0..3] = forward instructions, forward
+// slots, backward instructions, backward slots (zeros: evaluated operator by operator)
+void cth_last_expr_stats(int* out) {
+    Expr::ProgramStats s = Expr::last_program_stats();
+    out[0] = s.forward_insns;
+    out[1] = s.forward_slots;
+    out[2] = s.backward_insns;
+    out[3] = s.backward_slots;
+}
 void cth_set_reference_row0(int on) { g_row0 = on; }
 // the MLP entry points below build each layer with Tensor::linear (one fused operator) when set
 void cth_set_fused_layers(int on) { g_fused_layers = on; }
