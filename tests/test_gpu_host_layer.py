@@ -202,7 +202,7 @@ def test_configurations_small(oracle, host, golden):
     assert np.abs(gr - g["expr_gR"].astype(np.float64).sum(0)).max() <= 1e-5 * np.abs(g["expr_gR"]).sum(0).max()
 
 
-@pytest.mark.parametrize("prog", ["test_scalar_grad", "test_tensor_grad", "test_activation_loss"])
+@pytest.mark.parametrize("prog", ["test_scalar_grad", "test_tensor_grad", "test_activation_loss", "test_fused"])
 def test_reference_style_programs(prog):
     """C++ programs written like the reference's own test executables (src/tests/test.cpp,
     test_tensor_grad.cpp, test_activation_loss.cpp), on DeviceType::kAMD; exit code 0 = all
