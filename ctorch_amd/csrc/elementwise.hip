@@ -260,6 +260,73 @@ int dev_scalar(const char* name, const float* a, const float* b1, float* r, size
 }
 
 
+// ---- elementwise comparisons: float in, one byte (0 / 1) per element out
+__device__ __forceinline__ bool compare(int cmp, float a, float b) {
+    switch (cmp) {
+        case CTAMD_CMP_GT: return a > b;
+        case CTAMD_CMP_LT: return a < b;
+        case CTAMD_CMP_EQ: return a == b;
+        case CTAMD_CMP_GE: return a >= b;
+        case CTAMD_CMP_LE: return a <= b;
+        default: return a != b;
+    }
+}
+// VEC: a (and b) 16-byte aligned, out 4-byte aligned: a thread compares 128-bit vectors and stores
+// their four result bytes as one 32-bit word (four vectors per thread, loaded before first use);
+// the last n % 4 elements and unaligned tensors go element by element.  b == nullptr: compare with s.
+template <bool VEC>
+__global__ __launch_bounds__(kThreads) void compare_kernel(const float* __restrict__ a, const float* __restrict__ b, float s,
+                                                           uint8_t* __restrict__ out, size_t n, int cmp) {
+    if (VEC) {
+        const size_t n4 = n >> 2;
+        const size_t base = size_t(blockIdx.x) * (kThreads * kUnroll) + threadIdx.x;
+        v4f va[kUnroll], vb[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            size_t i = base + size_t(u) * kThreads;
+            if (i < n4) {
+                va[u] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(a) + i);
+                if (b) vb[u] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(b) + i);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            size_t i = base + size_t(u) * kThreads;
+            if (i < n4) {
+                uint32_t word = 0;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) word |= uint32_t(compare(cmp, va[u][e], b ? vb[u][e] : s)) << (8 * e);
+                reinterpret_cast<uint32_t*>(out)[i] = word;
+            }
+        }
+        if (blockIdx.x == 0) {
+            size_t i = (n4 << 2) + threadIdx.x;
+            if (i < n) out[i] = uint8_t(compare(cmp, a[i], b ? b[i] : s));
+        }
+    } else {
+        const size_t stride = size_t(gridDim.x) * kThreads;
+        for (size_t i = size_t(blockIdx.x) * kThreads + threadIdx.x; i < n; i += stride)
+            out[i] = uint8_t(compare(cmp, a[i], b ? b[i] : s));
+    }
+}
+
+int launch_compare(const char* name, int cmp, const float* a, const float* b, float s, uint8_t* out, size_t n, void* stream) {
+    if (cmp < CTAMD_CMP_GT || cmp > CTAMD_CMP_NE) return fail(CTAMD_EINVAL, "%s: unknown comparison %d", name, cmp);
+    if (n == 0) return CTAMD_OK;
+    if (!a || !out) return fail(CTAMD_EINVAL, "%s: null pointer", name);
+    const bool vec = aligned16(a) && (!b || aligned16(b)) && (reinterpret_cast<uintptr_t>(out) & 3u) == 0;
+    if (vec) {
+        size_t blocks = (n / 4 + size_t(kThreads) * kUnroll - 1) / (size_t(kThreads) * kUnroll);
+        if (blocks < 1) blocks = 1;
+        if (blocks > 0x7fffffffu) return fail(CTAMD_ERANGE, "%s: more than 2^43 elements", name);
+        hipLaunchKernelGGL(compare_kernel<true>, dim3(unsigned(blocks)), dim3(kThreads), 0, as_stream(stream), a, b, s, out, n, cmp);
+    } else {
+        hipLaunchKernelGGL(compare_kernel<false>, dim3(stream_grid(n, kThreads)), dim3(kThreads), 0, as_stream(stream), a, b, s, out, n, cmp);
+    }
+    account((b ? 9.0 : 5.0) * double(n), 0.0);
+    return launched(name);
+}
+
 // ---- the optimiser update of several tensors in one launch
 constexpr int kSgdMaxTensors = 32;
 constexpr int kSgdChunk = kThreads * 8;          // elements per block
@@ -356,6 +423,13 @@ int ctamd_accumulate_f32(float* grad, const float* val, size_t n, void* s) {
 int ctamd_sgd_step_f32(float* param, const float* grad, float lr, size_t n, void* s) {
     Ptrs<2> in{{param, grad}};
     return launch_map<SgdF>(__func__, in, param, n, SgdF{lr}, s);
+}
+int ctamd_compare_f32(int cmp, const float* a, const float* b, uint8_t* out, size_t n, void* stream) {
+    if (n && !b) return fail(CTAMD_EINVAL, "%s: null pointer", __func__);
+    return launch_compare(__func__, cmp, a, b, 0.0f, out, n, stream);
+}
+int ctamd_compare_scalar_f32(int cmp, const float* a, float s, uint8_t* out, size_t n, void* stream) {
+    return launch_compare(__func__, cmp, a, nullptr, s, out, n, stream);
 }
 int ctamd_sgd_step_multi_f32(float* const* params, const float* const* grads, const size_t* counts, int tensors, float lr,
                              void* stream) {

@@ -89,6 +89,9 @@ class Tensor {
     T* data() { return _storage.data<T>() + _storage_offset; }
     // fp32 pointer in the tensor's own address space (HBM for kAMD), offset applied
     bool storage_shared() const { return _storage.shared(); }
+    // first byte of the elements, any dtype (device or host memory, as device() says)
+    void* raw_ptr() { return static_cast<char*>(_storage.raw()) + _storage_offset * dtypeSize(_dtype); }
+    const void* raw_ptr() const { return static_cast<const char*>(_storage.raw()) + _storage_offset * dtypeSize(_dtype); }
     const float* fptr() const { return static_cast<const float*>(_storage.raw()) + _storage_offset; }
     float* fptr() { return static_cast<float*>(_storage.raw()) + _storage_offset; }
     template <typename T>
@@ -135,6 +138,20 @@ class Tensor {
     Tensor operator+(float scalar) const;
     Tensor operator*(float scalar) const;
     Tensor operator/(float scalar) const;
+    // elementwise comparisons, DType::kBool results (src/Tensor.cpp:985-1309); not taped
+    Tensor operator>(float scalar) const;
+    Tensor operator<(float scalar) const;
+    Tensor operator==(float scalar) const;
+    Tensor operator>=(float scalar) const;
+    Tensor operator<=(float scalar) const;
+    Tensor operator!=(float scalar) const;
+    Tensor operator>(const Tensor& other) const;
+    Tensor operator<(const Tensor& other) const;
+    Tensor operator==(const Tensor& other) const;
+    Tensor operator>=(const Tensor& other) const;
+    Tensor operator<=(const Tensor& other) const;
+    Tensor operator!=(const Tensor& other) const;   // declared by the reference (Tensor.h), defined here
+    std::vector<unsigned char> to_bytes() const;    // a bool tensor's elements on the host (any device)
     Tensor sum() const;
     Tensor softmax(int dim = -1) const;
 

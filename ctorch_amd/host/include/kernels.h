@@ -34,7 +34,9 @@ Tensor Softmax_AMD_kernel(const Tensor& a);
 namespace ctorch_amd_host {
 // Device branches of the arithmetic that the reference runs inline on the host (not behind the
 // scheduler): used by the Tensor front-end and the tape.
-Tensor scalar_op(const Tensor& a, float s, op which);                 // a + s, a * s, a / s
+Tensor scalar_op(const Tensor& a, float s, op which);
+// a (cmp) b or, with b == nullptr, a (cmp) s: a bool tensor; cmp is a CTAMD_CMP_* code
+Tensor compare_op(int cmp, const Tensor& a, const Tensor* b, float s);                 // a + s, a * s, a / s
 Tensor sum_all(const Tensor& a);
 Tensor softmax_dim(const Tensor& a, int dim);                         // dim already normalised
 Tensor filled(const std::vector<size_t>& shape, float v, DeviceType device);

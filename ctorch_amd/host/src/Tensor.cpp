@@ -7,6 +7,7 @@
 #include <cmath>
 
 #include "Ctorch_Scheduler.h"
+#include "ctorch_amd.h"
 #include "kernels.h"
 
 using namespace ctorch_amd_host;
@@ -293,6 +294,37 @@ Tensor Tensor::linear(const Tensor& weight, const Tensor& bias, bool relu) const
     tape(result, op::Linear, {this, &weight, &bias}, relu ? 1 : 0);
     return result;
 }
+namespace {
+Tensor compare_with(int cmp, const Tensor& a, const Tensor* b, float s) {
+    if (a.device() != DeviceType::kAMD)
+        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::PLATFORM_API, "comparison: no kernel for this device");
+    return ctorch_amd_host::compare_op(cmp, a, b, s);
+}
+}  // namespace
+Tensor Tensor::operator>(float s) const { return compare_with(CTAMD_CMP_GT, *this, nullptr, s); }
+Tensor Tensor::operator<(float s) const { return compare_with(CTAMD_CMP_LT, *this, nullptr, s); }
+Tensor Tensor::operator==(float s) const { return compare_with(CTAMD_CMP_EQ, *this, nullptr, s); }
+Tensor Tensor::operator>=(float s) const { return compare_with(CTAMD_CMP_GE, *this, nullptr, s); }
+Tensor Tensor::operator<=(float s) const { return compare_with(CTAMD_CMP_LE, *this, nullptr, s); }
+Tensor Tensor::operator!=(float s) const { return compare_with(CTAMD_CMP_NE, *this, nullptr, s); }
+Tensor Tensor::operator>(const Tensor& o) const { return compare_with(CTAMD_CMP_GT, *this, &o, 0.0f); }
+Tensor Tensor::operator<(const Tensor& o) const { return compare_with(CTAMD_CMP_LT, *this, &o, 0.0f); }
+Tensor Tensor::operator==(const Tensor& o) const { return compare_with(CTAMD_CMP_EQ, *this, &o, 0.0f); }
+Tensor Tensor::operator>=(const Tensor& o) const { return compare_with(CTAMD_CMP_GE, *this, &o, 0.0f); }
+Tensor Tensor::operator<=(const Tensor& o) const { return compare_with(CTAMD_CMP_LE, *this, &o, 0.0f); }
+Tensor Tensor::operator!=(const Tensor& o) const { return compare_with(CTAMD_CMP_NE, *this, &o, 0.0f); }
+
+std::vector<unsigned char> Tensor::to_bytes() const {
+    std::vector<unsigned char> out(numel());
+    if (out.empty() || _storage.empty()) return out;
+    if (_dtype != DType::kBool || !is_contiguous())
+        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DATATYPE, "to_bytes(): a contiguous bool tensor is needed");
+    const unsigned char* src = static_cast<const unsigned char*>(raw_ptr());
+    if (_device == DeviceType::kAMD) device_copy_d2h(out.data(), src, out.size());
+    else std::memcpy(out.data(), src, out.size());
+    return out;
+}
+
 Tensor Tensor::mse_loss(const Tensor& target) const { return binary(*this, target, op::MSE); }
 Tensor Tensor::mae_loss(const Tensor& target) const { return binary(*this, target, op::MAE); }
 Tensor Tensor::cross_entropy(const Tensor& target) const { return binary(*this, target, op::CE); }

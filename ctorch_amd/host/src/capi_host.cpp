@@ -141,6 +141,27 @@ long cth_unary(int code, const float* a, const long* ad, int an, float* out) {
     }
 }
 
+// a (cmp) b, or a (cmp) s when b is null; cmp = 0 '>', 1 '<', 2 '==', 3 '>=', 4 '<=', 5 '!='; one byte per element
+long cth_compare(int cmp, const float* a, const long* ad, int an, const float* b, const long* bd, int bn, float s,
+                 unsigned char* out) {
+    try {
+        Tensor ta = make(a, ad, an);
+        Tensor r;
+        if (b) {
+            Tensor tb = make(b, bd, bn);
+            r = cmp == 0 ? ta > tb : cmp == 1 ? ta < tb : cmp == 2 ? ta == tb : cmp == 3 ? ta >= tb : cmp == 4 ? ta <= tb : ta != tb;
+        } else {
+            r = cmp == 0 ? ta > s : cmp == 1 ? ta < s : cmp == 2 ? ta == s : cmp == 3 ? ta >= s : cmp == 4 ? ta <= s : ta != s;
+        }
+        if (r.dtype() != DType::kBool) return -3;
+        std::vector<unsigned char> v = r.to_bytes();
+        std::memcpy(out, v.data(), v.size());
+        return static_cast<long>(v.size());
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
 // tensor (op) host scalar: which = 0 '+', 1 '*', 2 '/'
 long cth_scalar(int which, const float* a, const long* ad, int an, float s, float* out) {
     try {

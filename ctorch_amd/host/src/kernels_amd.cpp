@@ -113,6 +113,24 @@ Tensor scalar_op(const Tensor& a, float s, op which) {
     run(rc, "tensor (op) float");
     return r;
 }
+Tensor compare_op(int cmp, const Tensor& a, const Tensor* b, float s) {
+    check_device(a, "comparison");
+    if (a.dtype() != DType::kFloat || !a.is_contiguous())
+        Ctorch_Error::throwException(kP, ErrorType::DATATYPE, "comparison: a contiguous float tensor is needed");
+    if (b) {
+        check_device(*b, "comparison");
+        if (a.sizes() != b->sizes())                                    // src/Tensor.cpp:1124-1126
+            Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DIMENSION, "comparison: tensor shapes differ");
+        if (a.dtype() != b->dtype() || !b->is_contiguous())             // :1129-1131
+            Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DATATYPE, "comparison: tensor dtypes differ");
+    }
+    Tensor r(ShapeTag{}, a.sizes(), DType::kBool, DeviceType::kAMD, false);
+    uint8_t* out = static_cast<uint8_t*>(r.raw_ptr());
+    run(b ? ctamd_compare_f32(cmp, a.fptr(), b->fptr(), out, a.numel(), current_stream())
+          : ctamd_compare_scalar_f32(cmp, a.fptr(), s, out, a.numel(), current_stream()),
+        "comparison");
+    return r;
+}
 Tensor sum_all(const Tensor& a) {
     check_device(a, "sum");
     Tensor r = scalar0d();

@@ -186,6 +186,14 @@ int ctamd_matmul_f32(const float* a, int64_t as0, int64_t as1, const float* b, i
 int ctamd_matmul_bias_f32(const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,
                           const float* bias, int relu, float* c, int64_t m, int64_t n, int64_t k, void* stream);
 
+/* -------------------------------------------------------------------------- comparisons */
+/* out[i] = (a[i] cmp b[i]) or (a[i] cmp s) as one byte, 0 or 1 - the reference's bool tensors.
+ * Tensor::operator>,<,==,>=,<=,!=(float) src/Tensor.cpp:985-1116 and (const Tensor&) :1119-1309;
+ * IEEE comparisons (anything against NaN is false, != is true). */
+enum { CTAMD_CMP_GT = 0, CTAMD_CMP_LT = 1, CTAMD_CMP_EQ = 2, CTAMD_CMP_GE = 3, CTAMD_CMP_LE = 4, CTAMD_CMP_NE = 5 };
+int ctamd_compare_f32(int cmp, const float* a, const float* b, uint8_t* out, size_t n, void* stream);
+int ctamd_compare_scalar_f32(int cmp, const float* a, float s, uint8_t* out, size_t n, void* stream);
+
 /* ------------------------------------------------------------------ fused expressions */
 /* A chain of the elementwise operators above evaluated in ONE pass over memory: the front-end
  * compiles an expression such as Y = sigmoid(X / r) - tanh(X) * sin(X) + cos(-X) (and, separately,

@@ -767,6 +767,19 @@ void co_expr(const float* X, const float* R, const float* T, long rows, long col
     free(v); free(gd1); free(gcs); free(gs1); free(gm); free(gq); free(gth); free(gsn); free(gng);
 }
 
+/* ------------------------------------------------------------------------ comparisons */
+
+/* src/Tensor.cpp:985-1116 (tensor against float) and :1119-1309 (tensor against tensor of the same
+ * shape): one bool per element.  cmp: 0 '>', 1 '<', 2 '==', 3 '>=', 4 '<=', 5 '!='.  b == NULL
+ * compares with s.  (operator!=(const Tensor&) is declared in the reference's Tensor.h and never
+ * defined; it is stated here as the negation of ==.) */
+void co_compare(int cmp, const float* a, const float* b, float s, unsigned char* out, long n) {
+    for (long i = 0; i < n; ++i) {
+        const float x = a[i], y = b ? b[i] : s;
+        out[i] = (unsigned char)(cmp == 0 ? x > y : cmp == 1 ? x < y : cmp == 2 ? x == y : cmp == 3 ? x >= y : cmp == 4 ? x <= y : x != y);
+    }
+}
+
 /* ------------------------------------------------------------- fused expression programs */
 
 /* Extension: the reference evaluates one operator per kernel.  A program is a straight-line list

@@ -80,6 +80,8 @@ void co_fill_uniform(float* r, long n, uint64_t seed, double lo, double hi);
 void co_fill_normal(float* r, long n, uint64_t seed, double mean, double sigma);
 void co_fill_int(float* r, long n, uint64_t seed, long range);
 
+void co_compare(int cmp, const float* a, const float* b, float s, unsigned char* out, long n);
+
 /* extension: a straight-line per-element program of the operators above (see the .c file) */
 int co_expr_run(const int* prog, const float* imm, int n, const float* const* in, int n_in, float* const* out, int n_out,
                 long rows, long cols, int* status);

@@ -303,6 +303,14 @@ class Oracle:
         return Y, np.float32(mse.value), np.float32(mae.value), gX, gR
 
     # ---- the MNIST demo's path
+    def compare(self, cmp, a, b=None, s=0.0):
+        """cmp: 0 '>', 1 '<', 2 '==', 3 '>=', 4 '<=', 5 '!='; b an array of a's shape or None (compare with s)."""
+        a = f32(a)
+        out = np.empty(a.shape, np.uint8)
+        self.lib.co_compare(C.c_int(cmp), fp(a), fp(f32(b)) if b is not None else None, C.c_float(s),
+                            out.ctypes.data_as(C.c_void_p), C.c_long(a.size))
+        return out
+
     def expr_run(self, prog, inputs, n_out, rows, cols):
         """prog: [(op, dst, a, b, imm)] of the fused-expression opcodes; inputs: full [rows, cols] or
         row-vector [cols] arrays; returns (outputs, status)."""
@@ -808,6 +816,22 @@ class HostLayer(Reference):
 
     def set_reference_row0(self, on):
         self.cdll.cth_set_reference_row0(int(on))
+
+    def compare(self, cmp, a, b=None, s=0.0):
+        """The Tensor comparison operators on the device; returns the bool tensor as uint8, or the
+        negative return code."""
+        a = f32(a)
+        out = np.empty(a.shape, np.uint8)
+        ad = (C.c_long * a.ndim)(*a.shape)
+        if b is not None:
+            b = f32(b)
+            bd = (C.c_long * b.ndim)(*b.shape)
+            rc = self.cdll.cth_compare(C.c_int(cmp), fp(a), ad, C.c_int(a.ndim), fp(b), bd, C.c_int(b.ndim), C.c_float(0),
+                                       out.ctypes.data_as(C.c_void_p))
+        else:
+            rc = self.cdll.cth_compare(C.c_int(cmp), fp(a), ad, C.c_int(a.ndim), None, None, C.c_int(0), C.c_float(s),
+                                       out.ctypes.data_as(C.c_void_p))
+        return out if rc == a.size else rc
 
     def set_fused_expr(self, on):
         """chain, expr, program and their timed versions evaluate their elementwise part as one fused

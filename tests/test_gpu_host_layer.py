@@ -316,3 +316,16 @@ def test_fused_expressions_against_the_reference_vectors(oracle, host, golden):
     finally:
         host.set_fused_expr(False)
         host.set_reference_row0(False)
+
+
+def test_comparison_operators(oracle, host):
+    """Tensor (cmp) Tensor and Tensor (cmp) float through the front-end: DType::kBool results equal
+    to the oracle's; tensors of different shapes throw (src/Tensor.cpp:1124-1126)."""
+    print("case host compare", flush=True)
+    a = oracle.normal((7, 33), 72, 0, 1)
+    b = oracle.normal((7, 33), 73, 0, 1)
+    b[2] = a[2]
+    for cmp in range(6):
+        assert np.array_equal(host.compare(cmp, a, b), oracle.compare(cmp, a, b)), cmp
+        assert np.array_equal(host.compare(cmp, a, None, 0.1), oracle.compare(cmp, a, None, 0.1)), cmp
+    assert host.compare(0, a, b[:, :32].copy()) == -1

@@ -6,12 +6,14 @@ are built to return glibc's floats, so the golden vectors written from the real 
 also required to match to <= 2 ulp, and the fraction of exact matches is printed);
 |x - y| <= 1e-5 * sum|terms| for reductions, MatMul, softmax and cross entropy, with fp64 as the
 arbiter."""
+import ctypes as C
+
 import numpy as np
 import pytest
 import torch
 
 import gpu_support as G
-from support import (ADD, COS, DIV, MUL, NEG, RELU, SIGMOID, SIN, SUB, TANH, same_bits, ulp_diff)
+from support import (ADD, COS, DIV, MUL, NEG, RELU, SIGMOID, SIN, SUB, TANH, f32, same_bits, ulp_diff)
 
 pytestmark = pytest.mark.gpu
 
@@ -418,3 +420,30 @@ def test_golden_reference_vectors_reductions_matmul_backward(golden, oracle):
     bits_equal(G.host(G.loss_bwd("mae", dx, G.dev(b["y"]), g1)) + F(0), b["d_mae"], "golden mae bwd")
     bits_equal(G.host(G.binary("div", dw, G.dev(b["yb"]))) + F(0), b["d_div_a"], "golden div bwd a")
     bits_equal(G.host(G.div_bwd_b(dx, G.dev(b["yb"]), dw)) + F(0), b["d_div_b"], "golden div bwd b")
+
+
+@pytest.mark.parametrize("n", [1, 3, 1024, 4099, 1 << 20])
+def test_comparisons_bit_exact(oracle, n):
+    """The six comparison operators against a tensor and against a float: one byte per element,
+    identical to the oracle, including equal values, signed zeros, infinities and NaN; aligned and
+    unaligned operands."""
+    print("case compare", n, flush=True)
+    a = oracle.normal((n,), 70, 0, 1)
+    b = oracle.normal((n,), 71, 0, 1)
+    b[::3] = a[::3]                                       # equal elements
+    special = f32([0.0, -0.0, np.inf, -np.inf, np.nan, 1.0, -1.0, np.nan])
+    k = min(n, special.size)
+    a[:k] = special[:k]
+    b[:k] = special[::-1][:k] if n > 1 else special[:1]
+    da, db = G.dev(a), G.dev(b)
+    pad_a, pad_b = G.dev(np.concatenate([[0.0], a])), G.dev(np.concatenate([[0.0], b]))
+    for cmp in range(6):
+        out = torch.empty(n, dtype=torch.uint8, device=G.DEV)
+        G.call("ctamd_compare_f32", cmp, G.ptr(da), G.ptr(db), G.ptr(out), n, G.stream())
+        assert np.array_equal(out.cpu().numpy(), oracle.compare(cmp, a, b)), cmp
+        G.call("ctamd_compare_f32", cmp, G.ptr(pad_a[1:]), G.ptr(pad_b[1:]), G.ptr(out), n, G.stream())   # 4-byte aligned only
+        assert np.array_equal(out.cpu().numpy(), oracle.compare(cmp, a, b)), cmp
+        for s in (0.0, 0.25, float("nan")):
+            G.call("ctamd_compare_scalar_f32", cmp, G.ptr(da), C.c_float(s), G.ptr(out), n, G.stream())
+            assert np.array_equal(out.cpu().numpy(), oracle.compare(cmp, a, None, s)), (cmp, s)
+    assert G.lib().ctamd_compare_f32(9, G.ptr(da), G.ptr(db), G.ptr(out), n, G.stream()) == -1

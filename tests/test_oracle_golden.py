@@ -231,3 +231,14 @@ def test_program_interpreter_equals_the_whole_tensor_functions(oracle):
             (E["NEG"], 3, 0, 0, 0.0), (E["COS"], 3, 3, 0, 0.0), (E["ADD"], 2, 2, 3, 0.0), (E["STORE"], 0, 2, 0, 0.0)]
     (got,), _ = oracle.expr_run(prog, [X, r], 1, rows, cols)
     assert same_bits(got, Y)
+
+
+def test_comparisons_are_the_ieee_predicates(oracle):
+    """co_compare against numpy's IEEE comparisons (the reference's loops are plain C++ comparisons
+    of floats, src/Tensor.cpp:985-1309), including NaN, infinities and signed zeros."""
+    a = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1.0, -1.0, 2.5, np.nan], np.float32)
+    b = np.array([-0.0, 0.0, np.inf, np.inf, 1.0, np.nan, -1.0, 2.0, np.nan], np.float32)
+    fns = [np.greater, np.less, np.equal, np.greater_equal, np.less_equal, np.not_equal]
+    for cmp, fn in enumerate(fns):
+        assert np.array_equal(oracle.compare(cmp, a, b), fn(a, b).astype(np.uint8)), cmp
+        assert np.array_equal(oracle.compare(cmp, a, None, 1.0), fn(a, np.float32(1.0)).astype(np.uint8)), cmp
