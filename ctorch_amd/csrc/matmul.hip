@@ -411,6 +411,9 @@ __global__ __launch_bounds__(kThreads) void gemm_strided(const float* __restrict
 // Three tile shapes; the host picks the largest one that still gives every CU a tile.
 //   Big   256 x 256 x 16, 8 waves of 128 x 64 (128 accumulator registers, two waves per SIMD): the
 //         fewest LDS and global bytes per flop; 4096^3 in 0.95-0.98 ms (140-145 TFLOP/s).
+//   Wide  256 x 128 x 16, 4 waves of 128 x 64, two blocks per CU: 1-5% behind Big per flop, but its
+//         tiles are half as large - 6144^3 (576 Big tiles on 256 CUs: three rounds, the last a
+//         quarter full) in 3.59 ms (129 TFLOP/s) against 4.30 ms with Big tiles.
 //   Small 128 x 128 x 16, 4 waves of 64 x 64: 2048^3 in 0.135 ms (127 TFLOP/s).
 //   Tiny  64 x 64 x 16, 4 waves of 32 x 32, up to 8 blocks per CU: 1024^3 in 27 us (78 TFLOP/s) and
 //         the skinny products of a small layer ([8192 x 784] . [784 x 256] in 32 us); with a K split
@@ -418,6 +421,7 @@ __global__ __launch_bounds__(kThreads) void gemm_strided(const float* __restrict
 using BigTile = Cfg<256, 256, 16, 128, 64>;
 using SmallTile = Cfg<128, 128, 16, 64, 64>;
 using TinyTile = Cfg<64, 64, 16, 32, 32>;
+using WideTile = Cfg<256, 128, 16, 128, 64>;
 
 template <class Tile, bool A_KC, bool B_KC>
 int launch_gemm(GemmArgs g, bool vec, int splits, hipStream_t s) {
@@ -474,12 +478,21 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
     const bool A_KC = a_kc, B_KC = !b_xc;
     const int cus = compute_units() > 0 ? compute_units() : 256;
     auto tiles_of = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
-    // the largest tile shape that still gives every CU a tile; below that the smallest shape
-    int shape = tiles_of(BigTile::BM, BigTile::BN) >= cus ? 2 : tiles_of(SmallTile::BM, SmallTile::BN) >= cus ? 1 : 0;
-    const int BM = shape == 2 ? BigTile::BM : shape == 1 ? SmallTile::BM : TinyTile::BM;
-    const int BN = shape == 2 ? BigTile::BN : shape == 1 ? SmallTile::BN : TinyTile::BN;
+    // Big, Wide or Small by the time the slowest CU needs: rounds of tiles per CU x the tile's share
+    // of a Big tile x what the shape loses per flop (measured at 4096^3); Tiny when even the Small
+    // shape cannot give every CU a tile
+    auto rounds = [&](int64_t tiles) { return double((tiles + cus - 1) / cus); };
+    int shape = 0;
+    if (tiles_of(SmallTile::BM, SmallTile::BN) >= cus) {
+        const double big = rounds(tiles_of(BigTile::BM, BigTile::BN));
+        const double wide = rounds(tiles_of(WideTile::BM, WideTile::BN)) * 0.5 * 1.04;
+        const double small = rounds(tiles_of(SmallTile::BM, SmallTile::BN)) * 0.25 * 1.07;
+        shape = (big <= wide && big <= small) ? 2 : (wide <= small ? 3 : 1);
+    }
+    const int BM = shape == 3 ? WideTile::BM : shape == 2 ? BigTile::BM : shape == 1 ? SmallTile::BM : TinyTile::BM;
+    const int BN = shape == 3 ? WideTile::BN : shape == 2 ? BigTile::BN : shape == 1 ? SmallTile::BN : TinyTile::BN;
     constexpr int BK = 16;
-    static_assert(BigTile::BK == BK && SmallTile::BK == BK && TinyTile::BK == BK, "all tile shapes step K alike");
+    static_assert(BigTile::BK == BK && WideTile::BK == BK && SmallTile::BK == BK && TinyTile::BK == BK, "all tile shapes step K alike");
     GemmArgs g;
     g.a = a; g.lda = A_KC ? as0 : as1;
     g.b = b; g.ldb = B_KC ? bs1 : bs0;
@@ -514,7 +527,8 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
     if (splits > 1) { g.c = partial; g.ldc = n; g.split_stride = m * n; g.bias = nullptr; g.relu = 0; }
     else { g.c = c; g.ldc = n; g.split_stride = 0; g.bias = bias; g.relu = relu; }
 
-    int rc = shape == 2 ? launch_layout<BigTile>(g, A_KC, B_KC, vec, splits, s)
+    int rc = shape == 3 ? launch_layout<WideTile>(g, A_KC, B_KC, vec, splits, s)
+           : shape == 2 ? launch_layout<BigTile>(g, A_KC, B_KC, vec, splits, s)
            : shape == 1 ? launch_layout<SmallTile>(g, A_KC, B_KC, vec, splits, s)
                         : launch_layout<TinyTile>(g, A_KC, B_KC, vec, splits, s);
     if (rc || splits == 1) return rc;

@@ -328,8 +328,9 @@ def test_softmax_columns(oracle, shape):
 
 MM_SHAPES = [(1, 1, 1), (5, 3, 9), (33, 29, 47), (128, 128, 16), (130, 257, 70), (256, 10, 784), (64, 256, 10),
              (784, 256, 300), (256, 10, 8192), (17, 1, 33), (1, 40, 33), (200, 200, 1), (384, 512, 1024),
-             # ragged edges and a K that is no multiple of the k tile, for the 128 x 128 and the 256 x 256 tile shapes
-             (2049, 2050, 33), (4100, 4101, 70)]
+             # ragged edges and a K that is no multiple of the k tile, for the 128 x 128, the 256 x 256 and
+             # the 256 x 128 tile shapes (the launcher picks by rounds of tiles per CU)
+             (2049, 2050, 33), (4100, 4101, 70), (4090, 4093, 40), (4090, 2047, 40)]
 
 
 @pytest.mark.parametrize("m,n,k", MM_SHAPES)
@@ -351,7 +352,7 @@ def test_matmul_all_layouts_normwise(oracle, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(256, 128, 784), (128, 10, 64), (70, 33, 129), (8192, 256, 784), (96, 12, 4096),
-                                   (2100, 2050, 40), (5, 7, 0)])
+                                   (2100, 2050, 40), (4090, 4093, 24), (4090, 2047, 24), (5, 7, 0)])
 def test_fused_layer_equals_the_three_launches(oracle, m, n, k):
     """matmul + bias row + ReLU in one launch against the same three operators launched in sequence,
     bit for bit, over all tile shapes, the K-split fold ((96, 12, 4096)) and ragged edges; and against
