@@ -588,6 +588,49 @@ long cth_time_mlp_graph(const float* x, long B, long I, const float* W1, const f
     }
 }
 
+// The config-5 expression as a fused expression inside a recorded step: X1 is evaluated eagerly
+// (y1, gx1), then the step is recorded on X1, replayed, the staged input is overwritten with X2 and
+// the step replayed again, with eager work in between (y2, gx2 come from the second replay).
+long cth_expr_graph(const float* X1, const float* X2, const float* R, const float* T, long rows, long cols, float* y1,
+                    float* gx1, float* y2, float* gx2) {
+    try {
+        long d[2] = {rows, cols}, dv[1] = {cols};
+        Tensor tX = make(X1, d, 2), tX2 = make(X2, d, 2), tR = make(R, dv, 1), tT = make(T, d, 2);
+        AutoDiff ctx;
+        configure(ctx);
+        AutoDiffContext::Guard guard(&ctx);
+        Tensor Y, gX;
+        auto body = [&] {
+            tX.requires_grad(true);
+            tR.requires_grad(true);
+            Expr x(tX), r(tR);
+            Y = (sigmoid(x / r) - tanh(x) * sin(x) + cos(-x)).eval();
+            Tensor L = Y.mse_loss(tT) + Y.mae_loss(tT);
+            backward(L);
+            gX = grad(tX);
+        };
+        body();                               // eagerly: the reference values for X1, and a warm pool
+        if (emit(Y, y1) < 0 || emit(gX, gx1) < 0) return -2;
+        ctx.clear_graph();
+        DeviceGraph step;
+        step.record(body);
+        ctx.clear_graph();
+        step.replay();
+        Tensor probe = (tT * 2.0f).sum();     // eager work between the replays
+        (void)probe.item<float>();
+        std::vector<float> a(size_t(rows * cols)), b(size_t(rows * cols));
+        if (emit(Y, a.data()) < 0 || emit(gX, b.data()) < 0) return -2;
+        if (std::memcmp(a.data(), y1, a.size() * sizeof(float)) != 0 || std::memcmp(b.data(), gx1, b.size() * sizeof(float)) != 0)
+            return -3;                        // the first replay must reproduce the eager step
+        ctorch_amd_host::copy_into(tX, tX2);
+        step.replay();
+        if (emit(Y, y2) < 0 || emit(gX, gx2) < 0) return -2;
+        return rows * cols;
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
 // loss_sum = CE(logits, class index), backward: dlogits = softmax - onehot.
 long cth_time_softmax_ce(const float* logits, const float* labels, long rows, long cols, int warm, int reps,
                          double* out) {

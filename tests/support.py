@@ -833,6 +833,16 @@ class HostLayer(Reference):
                                        out.ctypes.data_as(C.c_void_p))
         return out if rc == a.size else rc
 
+    def expr_graph(self, X1, X2, r, T):
+        """The fused config-5 expression in a recorded step: eager on X1, recorded, replayed on X1 and
+        (after overwriting the staged input) on X2.  Returns (rc, y1, gx1, y2, gx2)."""
+        X1, X2, r, T = f32(X1), f32(X2), f32(r), f32(T)
+        rows, cols = X1.shape
+        outs = [np.empty_like(X1) for _ in range(4)]
+        self.cdll.cth_expr_graph.restype = C.c_long
+        rc = self.cdll.cth_expr_graph(fp(X1), fp(X2), fp(r), fp(T), C.c_long(rows), C.c_long(cols), *[fp(o) for o in outs])
+        return (rc, *outs)
+
     def set_fused_expr(self, on):
         """chain, expr, program and their timed versions evaluate their elementwise part as one fused
         expression (Expr::eval): one launch forward, one backward."""

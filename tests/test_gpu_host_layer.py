@@ -329,3 +329,26 @@ def test_comparison_operators(oracle, host):
         assert np.array_equal(host.compare(cmp, a, b), oracle.compare(cmp, a, b)), cmp
         assert np.array_equal(host.compare(cmp, a, None, 0.1), oracle.compare(cmp, a, None, 0.1)), cmp
     assert host.compare(0, a, b[:, :32].copy()) == -1
+
+
+def test_fused_expression_in_a_recorded_step(oracle, host):
+    """A fused expression, its losses and its backward recorded into a HIP graph: the first replay
+    reproduces the eager step bit for bit, a replay after the staged input was overwritten equals
+    the eager step on the new input."""
+    print("case fused expr recorded", flush=True)
+    rows, cols = 64, 256
+    X1 = oracle.uniform((rows, cols), 901, -2, 2)
+    X2 = oracle.uniform((rows, cols), 902, -2, 2)
+    r = oracle.uniform((cols,), 903, 0.5, 2)
+    T = oracle.normal((rows, cols), 904)
+    rc, y1, gx1, y2, gx2 = host.expr_graph(X1, X2, r, T)
+    assert rc == rows * cols, rc
+    host.set_fused_expr(True)
+    try:
+        e1 = host.expr(X1, r, T)
+        e2 = host.expr(X2, r, T)
+    finally:
+        host.set_fused_expr(False)
+    assert same_bits(y1, e1[0]) and same_bits(gx1, e1[3])
+    assert same_bits(y2, e2[0]) and same_bits(gx2, e2[3])
+    assert not same_bits(y1, y2)
