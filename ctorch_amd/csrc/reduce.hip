@@ -208,9 +208,15 @@ __global__ __launch_bounds__(kThreads) void colsum_stage1(const float* __restric
         }
 }
 
-constexpr int kFoldLanes = 4;   // lanes per column in stage 2
+constexpr int kFoldLanes = 4;    // lanes per column in stage 2
+constexpr int kSmallLanes = 16;  // lanes per column when a small matrix is summed in one launch
+// out[c] = sum over the `chunks` rows of partials[., c], in double, LANES lanes per column.  Stage 2
+// of the two-stage sum (LANES = 4), and the whole column sum of a small matrix (LANES = 16, a
+// bias gradient of a few hundred rows: one launch instead of two).
+template <int LANES>
 __global__ __launch_bounds__(kThreads) void colsum_stage2(const float* __restrict__ partials, float* __restrict__ out,
                                                           size_t cols, unsigned chunks) {
+    constexpr int kFoldLanes = LANES;
     constexpr int TX = kThreads / kFoldLanes;
     const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
     const size_t c = size_t(blockIdx.x) * TX + tx;
@@ -258,6 +264,14 @@ int ctamd_colsum_f32(const float* g, float* out, size_t rows, size_t cols, void*
     if (rows == 0) return ctamd_fill_f32(out, 0.0f, cols, stream);
     if (!g) return fail(CTAMD_EINVAL, "%s: null input", __func__);
     if (rows > (size_t(1) << 62) / cols) return fail(CTAMD_ERANGE, "%s: rows*cols overflows", __func__);
+    hipStream_t s = as_stream(stream);
+    if (rows <= 1024 && rows * cols <= (size_t(1) << 19)) {       // small: one launch, rows added in order
+        constexpr size_t kCols = kThreads / kSmallLanes;
+        hipLaunchKernelGGL(colsum_stage2<kSmallLanes>, dim3((unsigned)((cols + kCols - 1) / kCols)), dim3(kThreads), 0, s, g, out,
+                           cols, (unsigned)rows);
+        account(4.0 * double(rows) * double(cols), double(rows) * double(cols));
+        return launched(__func__);
+    }
     float* partials = scratch();
     if (!partials) return CTAMD_EINVAL;
     if (cols > kScratchFloats) return fail(CTAMD_ERANGE, "%s: more than %zu columns", __func__, kScratchFloats);
@@ -275,7 +289,6 @@ int ctamd_colsum_f32(const float* g, float* out, size_t rows, size_t cols, void*
     const bool wide = wide_strips * chunks >= 4 * cus;
     const size_t strip = size_t(kThreads) * (wide ? 4 : 1) * w;
     size_t col_blocks = (cols + strip - 1) / strip;
-    hipStream_t s = as_stream(stream);
     if (col_blocks > 0x7fffffffu) return fail(CTAMD_ERANGE, "%s: too many columns", __func__);
     dim3 grid((unsigned)col_blocks, (unsigned)chunks);
     if (vec && wide)
@@ -289,7 +302,7 @@ int ctamd_colsum_f32(const float* g, float* out, size_t rows, size_t cols, void*
     int rc = launched(__func__);
     if (rc) return rc;
     constexpr size_t kFoldCols = kThreads / kFoldLanes;
-    hipLaunchKernelGGL(colsum_stage2, dim3((unsigned)((cols + kFoldCols - 1) / kFoldCols)), dim3(kThreads), 0, s, partials,
+    hipLaunchKernelGGL(colsum_stage2<kFoldLanes>, dim3((unsigned)((cols + kFoldCols - 1) / kFoldCols)), dim3(kThreads), 0, s, partials,
                        out, cols, (unsigned)chunks);
     account(4.0 * double(rows) * double(cols), double(rows) * double(cols));
     return launched(__func__);

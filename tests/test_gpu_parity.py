@@ -194,7 +194,8 @@ def test_reductions_normwise(oracle, n):
         assert abs(G.host(G.reduce2("mse", da, db))[0] - oracle.mse(a, b)) <= 1e-5 * oracle.mse(a, b)
 
 
-@pytest.mark.parametrize("shape", [(1, 1), (2, 3), (37, 53), (8192, 256), (1000, 10), (4096, 4096), (33, 4100), (70000, 3)])
+@pytest.mark.parametrize("shape", [(1, 1), (2, 3), (37, 53), (8192, 256), (1000, 10), (4096, 4096), (33, 4100), (70000, 3), (128, 10),
+                                   (256, 256), (1024, 512), (1025, 16), (1024, 513)])
 def test_column_sum(oracle, shape):
     print("case colsum", shape, flush=True)
     g = oracle.normal(shape, 23)
