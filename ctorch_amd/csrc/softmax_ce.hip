@@ -203,6 +203,7 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
     stage_exp_table(s_exp2);
     constexpr bool kPipelined = (MODE == kSoftmax || MODE == kCeIndex || MODE == kCeBwdIndex);
     double block_loss = 0.0;
+    bool block_bad = false;   // a class index out of range was met (thread 0's copy counts)
 
     // everything that happens to one row once it sits in `r`; `mloc` is this thread's maximum
     auto process = [&](Row<THREADS, ITEMS, W>& r, size_t row, float mloc) {
@@ -243,7 +244,7 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
                 a.stats[2 * row + 1] = s;
             }
             if (c < 0 || c >= int(a.cols)) {
-                if (threadIdx.x == 0 && a.status) a.status[0] = 1;
+                block_bad = true;
                 block_loss += double(__builtin_nanf(""));
             } else {
                 // the thread that holds column c publishes exp(x_c - m): pick x_c by selects, then
@@ -344,7 +345,10 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
             process(r, row, r.max());
         }
     }
-    if ((MODE == kCeOnehot || MODE == kCeIndex) && threadIdx.x == 0) a.partials[blockIdx.x] = block_loss;
+    if ((MODE == kCeOnehot || MODE == kCeIndex) && threadIdx.x == 0) {
+        a.partials[blockIdx.x] = block_loss;
+        if (MODE == kCeIndex && a.status) a.partials[gridDim.x + blockIdx.x] = block_bad ? 1.0 : 0.0;
+    }
 }
 
 // Streaming variant for rows that do not fit a block's registers: pass 1 keeps an online
@@ -358,6 +362,7 @@ __global__ __launch_bounds__(1024) void row_stream_kernel(Args a) {
     __shared__ double s_d[THREADS / 64 + 1];
     stage_exp_table(s_exp2);
     double block_loss = 0.0;
+    bool block_bad = false;   // a class index out of range was met (thread 0's copy counts)
     for (size_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
         const float* xr = a.x + row * a.cols;
         if (MODE == kSoftmaxBwd) {
@@ -402,7 +407,7 @@ __global__ __launch_bounds__(1024) void row_stream_kernel(Args a) {
                 a.stats[2 * row + 1] = S;
             }
             if (c < 0 || c >= int(a.cols)) {
-                if (threadIdx.x == 0 && a.status) a.status[0] = 1;
+                block_bad = true;
                 block_loss += double(__builtin_nanf(""));
             } else {
                 float p = cta_expf_tab(xr[c] - M, s_exp2) / S;
@@ -420,7 +425,10 @@ __global__ __launch_bounds__(1024) void row_stream_kernel(Args a) {
             }
         }
     }
-    if ((MODE == kCeOnehot || MODE == kCeIndex) && threadIdx.x == 0) a.partials[blockIdx.x] = block_loss;
+    if ((MODE == kCeOnehot || MODE == kCeIndex) && threadIdx.x == 0) {
+        a.partials[blockIdx.x] = block_loss;
+        if (MODE == kCeIndex && a.status) a.partials[gridDim.x + blockIdx.x] = block_bad ? 1.0 : 0.0;
+    }
 }
 
 // Class-index cross entropy, forward, for long rows: a single pass with an online (max, sum) pair
@@ -439,6 +447,7 @@ __global__ __launch_bounds__(256) void ce_index_online_kernel(Args a) {
     __shared__ float s_f[2][THREADS / 64 + 1];
     stage_exp_table(s_exp2);
     double block_loss = 0.0;
+    bool block_bad = false;   // a class index out of range was met (thread 0's copy counts)
     for (size_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
         const float* __restrict__ xr = a.x + row * a.cols;
         float m = kNegInf, s = 0.0f;
@@ -483,7 +492,7 @@ __global__ __launch_bounds__(256) void ce_index_online_kernel(Args a) {
             a.stats[2 * row + 1] = S;
         }
         if (c < 0 || c >= int(a.cols)) {
-            if (threadIdx.x == 0 && a.status) a.status[0] = 1;
+            block_bad = true;
             block_loss += double(__builtin_nanf(""));
         } else if (threadIdx.x == 0) {
             float p = cta_expf_nonpos(xr[c] - M, s_exp2) / S;
@@ -491,7 +500,10 @@ __global__ __launch_bounds__(256) void ce_index_online_kernel(Args a) {
             block_loss -= double(float(log(double(p))));
         }
     }
-    if (threadIdx.x == 0) a.partials[blockIdx.x] = block_loss;
+    if (threadIdx.x == 0) {
+        a.partials[blockIdx.x] = block_loss;
+        if (a.status) a.partials[gridDim.x + blockIdx.x] = block_bad ? 1.0 : 0.0;
+    }
 }
 
 // Class-index cross entropy, backward, from the per-row (max, sum) that the forward pass left
@@ -543,17 +555,26 @@ __global__ __launch_bounds__(256) void ce_bwd_stats_kernel(Args a) {
     }
 }
 
-// out[0] = float(sum of partials), folded in a fixed order.
+// out[0] = float(sum of partials), folded in a fixed order; status[0] (when given) = whether any
+// block flagged a bad class index in the second half of the partials (every block writes its flag, so
+// nothing has to be cleared beforehand).
 __global__ __launch_bounds__(256) void loss_stage2(const double* __restrict__ partials, unsigned count,
-                                                   float* __restrict__ out) {
+                                                   float* __restrict__ out, int32_t* __restrict__ status) {
     __shared__ double s_d[256 / 64 + 1];
-    double t = 0.0;
+    double t = 0.0, bad = 0.0;
     for (unsigned i = threadIdx.x; i < count; i += 256) t += partials[i];
+    if (status)
+        for (unsigned i = threadIdx.x; i < count; i += 256) bad += partials[count + i];
     t = block_sum<256>(t, s_d);
-    if (threadIdx.x == 0) out[0] = float(t);
+    if (status) {
+        __syncthreads();
+        bad = block_sum<256>(bad, s_d);
+    }
+    if (threadIdx.x == 0) {
+        out[0] = float(t);
+        if (status) status[0] = bad > 0.0 ? 1 : 0;
+    }
 }
-
-__global__ void clear_i32(int32_t* p) { p[0] = 0; }
 
 constexpr unsigned kMaxRowBlocks = 1u << 16;
 
@@ -618,7 +639,7 @@ int run_rows(const char* name, Args a, float* loss_out, void* stream) {
         else hipLaunchKernelGGL((ce_index_online_kernel<false>), dim3(grid), dim3(256), 0, s, a);
         int rc0 = launched(name);
         if (rc0) return rc0;
-        hipLaunchKernelGGL(loss_stage2, dim3(1), dim3(256), 0, s, a.partials, grid, loss_out);
+        hipLaunchKernelGGL(loss_stage2, dim3(1), dim3(256), 0, s, a.partials, grid, loss_out, MODE == kCeIndex ? a.status : nullptr);
         return launched(name);
     }
     bool done = vec ? launch_resident<MODE, 4>(a, grid, s) : launch_resident<MODE, 1>(a, grid, s);
@@ -626,7 +647,7 @@ int run_rows(const char* name, Args a, float* loss_out, void* stream) {
     int rc = launched(name);
     if (rc) return rc;
     if (kLoss) {
-        hipLaunchKernelGGL(loss_stage2, dim3(1), dim3(256), 0, s, a.partials, grid, loss_out);
+        hipLaunchKernelGGL(loss_stage2, dim3(1), dim3(256), 0, s, a.partials, grid, loss_out, MODE == kCeIndex ? a.status : nullptr);
         rc = launched(name);
     }
     return rc;
@@ -699,11 +720,6 @@ int ctamd_cross_entropy_backward_index_stats_f32(const float* x, const float* id
 }
 int ctamd_cross_entropy_index_stats_f32(const float* x, const float* idx, float* out, int32_t* status, float* stats,
                                         size_t rows, size_t cols, void* stream) {
-    if (status) {   // cleared by a kernel, not a memset node, so that callers may capture this call
-        hipLaunchKernelGGL(clear_i32, dim3(1), dim3(1), 0, as_stream(stream), status);
-        int rc = launched(__func__);
-        if (rc) return rc;
-    }
     Args a{x, idx, nullptr, nullptr, nullptr, status, stats, rows, cols, nullptr, nullptr};
     return run_rows<kCeIndex>(__func__, a, out, stream);
 }
