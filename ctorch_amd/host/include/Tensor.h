@@ -35,6 +35,9 @@ class Tensor {
     DeviceType _device = DeviceType::kCPU;
     DType _dtype = DType::kFloat;
     Storage _storage;
+    // value of a one-element device tensor when the host already holds it (read back together with
+    // something else): item() then needs no transfer.  Dropped by the in-place writers.
+    std::shared_ptr<const float> _known_value;
 
     static std::atomic<size_t> global_tensor_id;
     void computeStrides();
@@ -62,6 +65,10 @@ class Tensor {
     // rows [first, first + count) of a contiguous tensor as a VIEW (shares storage, new id): what
     // the demo's get_batch copies out (mnist/mnist.cpp:159-182) without the copy
     static Tensor view_rows(const Tensor& t, size_t first, size_t count);
+    // element `index` of a contiguous tensor as a 0-D VIEW (shares storage, new id)
+    static Tensor view_element(const Tensor& t, size_t index);
+    void set_known_value(float v) { _known_value = std::make_shared<const float>(v); }
+    void forget_known_value() { _known_value.reset(); }
     // a tensor on `device` filled from host memory
     static Tensor from_host(const float* data, const std::vector<size_t>& shape, DeviceType device);
 

@@ -49,7 +49,7 @@ Tensor::Tensor(ShapeTag, const std::vector<size_t>& shape, DType dtype, DeviceTy
 Tensor::Tensor(const Tensor& other)
     : tensor_id_(global_tensor_id++), _requires_grad(other._requires_grad), _shape(other._shape),
       _strides(other._strides), _storage_offset(other._storage_offset), _device(other._device),
-      _dtype(other._dtype), _storage(other._storage.clone()) {}
+      _dtype(other._dtype), _storage(other._storage.clone()), _known_value(other._known_value) {}
 
 Tensor& Tensor::operator=(const Tensor& other) {
     if (this != &other) {
@@ -61,6 +61,7 @@ Tensor& Tensor::operator=(const Tensor& other) {
         _device = other._device;
         _dtype = other._dtype;
         _storage = other._storage.clone();
+        _known_value = other._known_value;
     }
     return *this;
 }
@@ -68,7 +69,7 @@ Tensor& Tensor::operator=(const Tensor& other) {
 Tensor::Tensor(Tensor&& other) noexcept
     : tensor_id_(other.tensor_id_), _requires_grad(other._requires_grad), _shape(std::move(other._shape)),
       _strides(std::move(other._strides)), _storage_offset(other._storage_offset), _device(other._device),
-      _dtype(other._dtype), _storage(std::move(other._storage)) {
+      _dtype(other._dtype), _storage(std::move(other._storage)), _known_value(std::move(other._known_value)) {
     other.tensor_id_ = 0;
 }
 
@@ -82,6 +83,7 @@ Tensor& Tensor::operator=(Tensor&& other) noexcept {
         _device = other._device;
         _dtype = other._dtype;
         _storage = std::move(other._storage);
+        _known_value = std::move(other._known_value);
         other.tensor_id_ = 0;
     }
     return *this;
@@ -90,7 +92,7 @@ Tensor& Tensor::operator=(Tensor&& other) noexcept {
 Tensor::Tensor(AliasTag, const Tensor& other)
     : tensor_id_(other.tensor_id_), _requires_grad(other._requires_grad), _shape(other._shape),
       _strides(other._strides), _storage_offset(other._storage_offset), _device(other._device),
-      _dtype(other._dtype), _storage(other._storage) {}
+      _dtype(other._dtype), _storage(other._storage), _known_value(other._known_value) {}
 
 Tensor Tensor::from_host(const float* data, const std::vector<size_t>& shape, DeviceType device) {
     Tensor t(ShapeTag{}, shape, DType::kFloat, device, false);
@@ -130,6 +132,7 @@ float Tensor::item<float>() const {
     if (_dtype != DType::kFloat)
         Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DATATYPE, "item<float>(): dtype is not float");
     if (_device == DeviceType::kAMD) {
+        if (_known_value) return *_known_value;
         float v;
         device_copy_d2h(&v, fptr(), sizeof(float));
         return v;
@@ -173,6 +176,7 @@ Tensor Tensor::to(DeviceType device) const {
 }
 
 void Tensor::fill(float v) {
+    _known_value.reset();
     if (_storage.empty()) return;
     if (_dtype != DType::kFloat)
         Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DATATYPE, "fill(): only float tensors");
@@ -228,6 +232,18 @@ Tensor Tensor::view_rows(const Tensor& t, size_t first, size_t count) {
     r._requires_grad = false;
     r._storage_offset = t._storage_offset + first * t._strides[0];
     r._shape[0] = count;
+    return r;
+}
+
+Tensor Tensor::view_element(const Tensor& t, size_t index) {
+    if (!t.is_contiguous() || index >= t.numel())
+        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DIMENSION, "view_element: index out of range or tensor not contiguous");
+    Tensor r(AliasTag{}, t);
+    r.tensor_id_ = global_tensor_id++;
+    r._requires_grad = false;
+    r._storage_offset = t._storage_offset + index;
+    r._shape.clear();
+    r.computeStrides();
     return r;
 }
 

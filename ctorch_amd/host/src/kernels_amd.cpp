@@ -214,6 +214,7 @@ void copy_into(Tensor& dst, const Tensor& src) {
     check_device(src, "copy_into");
     if (dst.numel() != src.numel() || !dst.is_contiguous() || !src.is_contiguous())
         Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "copy_into: sizes differ or a tensor is not contiguous");
+    dst.forget_known_value();
     device_copy_d2d(dst.fptr(), src.fptr(), dst.numel() * sizeof(float));
 }
 Tensor onehot(const Tensor& labels, size_t classes) {
@@ -434,19 +435,23 @@ Tensor CrossEntropy_AMD_kernel(const Tensor& a, const Tensor& b) {
         return r;
     }
     if (b.dim() == 1 && a.dim() == 2 && b.sizes()[0] == a.sizes()[0]) {
-        Tensor r = scalar0d();
-        Tensor status = scalar0d();   // 4 bytes, used as int32
+        // loss and bad-index flag side by side: the host has to wait for the flag anyway (a bad index
+        // returns an empty Tensor), so it fetches the loss in the same transfer and item() is free
+        Tensor pair(ShapeTag{}, {2}, DType::kFloat, DeviceType::kAMD, false);
+        Tensor r = Tensor::view_element(pair, 0);
         Tensor stats(ShapeTag{}, {a.sizes()[0], 2}, DType::kFloat, DeviceType::kAMD, false);
-        run(ctamd_cross_entropy_index_stats_f32(a.fptr(), b.fptr(), r.fptr(), reinterpret_cast<int32_t*>(status.fptr()),
+        run(ctamd_cross_entropy_index_stats_f32(a.fptr(), b.fptr(), r.fptr(), reinterpret_cast<int32_t*>(pair.fptr() + 1),
                                                 stats.fptr(), a.sizes()[0], a.sizes()[1], current_stream()),
             "CrossEntropy_AMD_kernel");
         remember_ce_stats(a, b, std::move(stats));
-        int32_t bad = 0;
-        device_copy_d2h(&bad, status.fptr(), sizeof(bad));
-        if (bad) {
+        if (recording()) return r;              // a recorded step cannot wait: a bad index shows as a NaN loss
+        struct { float loss; int32_t bad; } got = {0.0f, 0};
+        device_copy_d2h(&got, pair.fptr(), sizeof(got));
+        if (got.bad) {
             Ctorch_Error::log(ErrorLevel::ERROR, kP, ErrorType::TENSOR_STATE, "CrossEntropy_AMD_kernel: class index out of range");
             return Tensor();
         }
+        r.set_known_value(got.loss);
         return r;
     }
     Ctorch_Error::log(ErrorLevel::ERROR, kP, ErrorType::DIMENSION, "CrossEntropy_AMD_kernel: incompatible shapes");
