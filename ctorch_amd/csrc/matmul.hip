@@ -505,19 +505,22 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
     int splits = 1;
     const int64_t tiles = int64_t(g.tiles_m) * g.tiles_n;
     float* partial = nullptr;
-    if (tiles < cus && k >= 8 * BK) {
-        // enough blocks for four per CU (they are co-resident), but at least 8 k tiles per block
-        int64_t want = (4 * cus + tiles - 1) / tiles;
-        int64_t max_by_k = k / (8 * BK);
-        int64_t max_by_scratch = int64_t(kScratchFloats) / (m * n);
-        splits = int(want < max_by_k ? want : max_by_k);
-        if (splits > max_by_scratch) splits = int(max_by_scratch);
-        if (splits < 4) splits = 1;                 // a two- or three-way split does not pay for its fold launch
+    if (tiles < cus && k >= 16 * BK) {
+        // enough blocks for four per CU (they are co-resident), with at least 8 k tiles per block - or 4
+        // when K is so short that 8 would leave the product unsplit: a block walks its k tiles one
+        // memory latency after the other (16 tiles of [256 x 256] . [256 x 10]: 15 us unsplit, 8.5 us in
+        // four parts), while many short parts would only lengthen the fold
+        const int64_t want = (4 * cus + tiles - 1) / tiles;
+        const int64_t max_by_scratch = int64_t(kScratchFloats) / (m * n);
+        for (int min_ktiles = 8; min_ktiles >= 4 && splits == 1; min_ktiles /= 2) {
+            const int64_t max_by_k = k / (min_ktiles * BK);
+            int64_t parts = want < max_by_k ? want : max_by_k;
+            if (parts > max_by_scratch) parts = max_by_scratch;
+            if (parts >= 4) splits = int(parts);    // a two- or three-way split does not pay for its fold launch
+        }
         if (splits > 1) {
             partial = scratch();
             if (!partial) return CTAMD_EINVAL;
-        } else {
-            splits = 1;
         }
     }
     int kps = int((k + splits - 1) / splits);
