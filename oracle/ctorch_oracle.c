@@ -23,6 +23,12 @@
  * Functions the reference cannot express are marked "extension" and are pinned by the same-shape
  * reference kernel on hand-materialised operands or by fp64 mathematics:
  *   co_binary_rowbcast for Sub/Mul/Div, co_ce_bwd_index, co_colsum_f64.
+ * co_expr_run (a per-element program of the operators above) is pinned opcode by opcode against
+ * the whole-tensor functions here, which the reference pins, and on the config-5 chain against
+ * co_expr; co_compare against the IEEE predicates the reference's plain C++ comparisons are
+ * (tests/test_oracle_golden.py).  The MNIST functions (co_u8_to_unit ... co_mnist_predict) are
+ * pinned bit for bit against the reference's loader, demo functions and its own main()
+ * (tests/test_oracle_vs_ref_mnist.py, tests/golden/mnist.npz).
  * Transcendentals call glibc libm (expf, logf, sinf, cosf) exactly as the reference does; their
  * values are whatever the installed glibc returns (2.35 in this image).
  */
