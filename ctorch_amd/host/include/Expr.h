@@ -9,7 +9,9 @@
 // Values and gradients are those of the operator-by-operator form bit for bit: every operator is
 // computed by the same per-element code, gradient contributions are formed by the reference's
 // formulas (src/AutoDiff.cpp:1216-1416) and added in the order in which the reference's tape would
-// add them (reversed depth-first post-order from the result, operands in recorded order).
+// add them (reversed depth-first post-order from the result, operands in recorded order).  The
+// tape receives ONE gradient per input from the expression: an input that other taped operators use
+// as well gets the same contributions, but the expression's share arrives as one sum.
 //
 // Operands: tensors of one common shape ("full"), and 1-D row vectors of the last dimension's
 // length as the right operand of + - * / with a full left operand.  Operators between two row

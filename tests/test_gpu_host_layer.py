@@ -352,3 +352,34 @@ def test_fused_expression_in_a_recorded_step(oracle, host):
     assert same_bits(y1, e1[0]) and same_bits(gx1, e1[3])
     assert same_bits(y2, e2[0]) and same_bits(gx2, e2[3])
     assert not same_bits(y1, y2)
+
+
+def test_fused_against_unfused_on_more_programs(oracle, host):
+    """A hundred further random programs (longer, more inputs, shapes with rows that are not a
+    multiple of four elements, so the 32-bit access path runs too, and a tensor large enough for
+    several passes per block): the fused expression against the operator-by-operator tape on the
+    device in the reference's gradient mode - bit for bit for the result and for every full-shape
+    input; a row vector that is also combined with other row vectors outside the expression gets its
+    contributions in another order (the expression hands the tape one sum), so it is held to 1e-5."""
+    from support import program_inputs, random_program
+    shapes = [(5, 7), (6, 8), (33, 20), (40, 36), (9, 130), (520, 1028)]
+    host.set_reference_row0(True)
+    try:
+        for seed in range(1000, 1100):
+            rows, cols = shapes[seed % len(shapes)] if seed % 25 else shapes[-1]
+            kinds, ops = random_program(seed, n_in=3 + seed % 3, n_ops=10 + seed % 15)
+            xs, w = program_inputs(oracle, seed, kinds, rows, cols)
+            host.set_fused_expr(False)
+            rc0, y0, L0, g0 = host.program(xs, kinds, ops, w)
+            host.set_fused_expr(True)
+            rc1, y1, L1, g1 = host.program(xs, kinds, ops, w)
+            assert rc0 >= 0 and rc1 == rc0, seed
+            assert same_bits(y1, y0), seed
+            for i, (a, b) in enumerate(zip(g1, g0)):
+                if kinds[i] == 0:
+                    assert same_bits(a, b), (seed, i)
+                else:
+                    assert np.all(np.abs(a - b) <= 1e-5 * (np.abs(b) + np.abs(b).max())), (seed, i)
+    finally:
+        host.set_fused_expr(False)
+        host.set_reference_row0(False)
