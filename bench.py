@@ -40,7 +40,7 @@ EW_N = 1 << 26
 # HBM bytes per forward-GEMM launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, scaled
 # by the same counters on the 768 MiB elementwise add of the same run); see
 # profiles/gemm_f32_4096_hbm_traffic.txt (384 MiB fetched + 64 MiB written; 192 MiB algorithmic).
-GEMM_TRAFFIC_BYTES = 470189883
+GEMM_TRAFFIC_BYTES = 470203664
 
 
 def cpu_baseline(seconds_hint=15.0):
