@@ -8,9 +8,10 @@ namespace {
 
 constexpr int kThreads = 256;
 typedef float v4f __attribute__((ext_vector_type(4)));
-typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 
-// dst[i] = src[i] / 255.0f.  A thread converts 16 pixels: one 128-bit load, four 128-bit stores.
+// dst[i] = src[i] / 255.0f.  A thread converts four groups of 4 pixels, 256 groups apart: each 32-bit
+// load and each 128-bit store of a wave covers one contiguous run (one thread converting 16
+// neighbouring pixels scatters its four stores over four cache lines: 1.7 TB/s against 5 here).
 // The division goes through the exact double reciprocal (cta_div_rcp): same bits as the IEEE
 // quotient, without the division sequence.
 template <bool VEC>
@@ -18,15 +19,24 @@ __global__ __launch_bounds__(kThreads) void u8_to_unit_kernel(const uint8_t* __r
                                                               size_t n) {
     const double rcp = 1.0 / 255.0;
     if (VEC) {
-        const size_t i16 = size_t(blockIdx.x) * kThreads + threadIdx.x;
-        if (i16 >= n / 16) return;
-        v4u w = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(src) + i16);
+        constexpr int U = 4;
+        const size_t n4 = n / 4;
+        const size_t base = size_t(blockIdx.x) * (kThreads * U) + threadIdx.x;
+        uint32_t w[U];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            v4f o;
+        for (int u = 0; u < U; ++u) {
+            const size_t i = base + size_t(u) * kThreads;
+            if (i < n4) w[u] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(src) + i);
+        }
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = cta_div_rcp(float((w[q] >> (8 * e)) & 0xffu), rcp);
-            __builtin_nontemporal_store(o, reinterpret_cast<v4f*>(dst) + i16 * 4 + q);
+        for (int u = 0; u < U; ++u) {
+            const size_t i = base + size_t(u) * kThreads;
+            if (i < n4) {
+                v4f o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = cta_div_rcp(float((w[u] >> (8 * e)) & 0xffu), rcp);
+                __builtin_nontemporal_store(o, reinterpret_cast<v4f*>(dst) + i);
+            }
         }
     } else {
         const size_t i = size_t(blockIdx.x) * kThreads + threadIdx.x;
@@ -87,9 +97,9 @@ int ctamd_u8_to_unit_f32(const uint8_t* src, float* dst, size_t n, void* stream)
     if (n == 0) return CTAMD_OK;
     if (!src || !dst) return fail(CTAMD_EINVAL, "%s: null pointer", __func__);
     hipStream_t s = as_stream(stream);
-    const bool vec = (n % 16 == 0) && aligned16(src) && aligned16(dst);
-    const size_t items = vec ? n / 16 : n;
-    const size_t blocks = (items + kThreads - 1) / kThreads;
+    const bool vec = (n % 4 == 0) && (reinterpret_cast<uintptr_t>(src) & 3u) == 0 && aligned16(dst);
+    const size_t per_block = vec ? size_t(kThreads) * 16 : size_t(kThreads);
+    const size_t blocks = (n + per_block - 1) / per_block;
     if (blocks > 0x7fffffffu) return fail(CTAMD_ERANGE, "%s: too many elements", __func__);
     if (vec) hipLaunchKernelGGL(u8_to_unit_kernel<true>, dim3(unsigned(blocks)), dim3(kThreads), 0, s, src, dst, n);
     else hipLaunchKernelGGL(u8_to_unit_kernel<false>, dim3(unsigned(blocks)), dim3(kThreads), 0, s, src, dst, n);

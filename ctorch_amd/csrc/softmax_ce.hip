@@ -683,6 +683,216 @@ __global__ __launch_bounds__(256) void softmax_bwd_cols_kernel(const float* __re
     for (size_t i = 0; i < rows; ++i) dx[i * cols + j] = y[i * cols + j] * (g[i * cols + j] - d);
 }
 
+
+// Tall matrices (128 rows or more): the column statistics as chunked reductions over rows, like the
+// column sum - a block owns a strip of 256 * W columns and a chunk of rows and walks its rows in
+// order, two rows in flight; per-chunk partials are folded by a second launch.  Forward: per chunk
+// a running (max, sum of the bit-exact exp(x - max)) pair, rescaled when the maximum moves; the fold
+// brings the chunks to the column maximum; then y = exp(x - max) / sum with the exact quotient (the
+// exponential is recomputed rather than stored: 12 B/elem instead of 16).
+// Backward: column dots of g and y, then dx = y * (g - dot).  The sums are chunked (fp32 inside a
+// chunk, double across chunks) where the reference adds the rows one after the other: the same
+// values to ~1e-7 relative, against 18 ms for a [16384 x 4096] matrix when one thread walks a
+// whole column alone.
+enum ColMode { kColOnline, kColSoftmaxOut, kColDot, kColBwdOut };
+
+template <int MODE, int W>
+__global__ __launch_bounds__(256) void col_walk_kernel(const float* __restrict__ x, const float* __restrict__ x2,
+                                                       const float* __restrict__ p0, const float* __restrict__ p1,
+                                                       float* __restrict__ out, size_t rows, size_t cols,
+                                                       size_t rows_per_block) {
+    __shared__ uint64_t s_exp2[32];
+    if (MODE == kColOnline || MODE == kColSoftmaxOut) stage_exp_table(s_exp2);
+    const size_t col = (size_t(blockIdx.x) * 256 + threadIdx.x) * W;
+    if (col >= cols) return;
+    const size_t r0 = size_t(blockIdx.y) * rows_per_block;
+    size_t r1 = r0 + rows_per_block;
+    if (r1 > rows) r1 = rows;
+    float a0[W], a1[W], q0[W];          // two accumulators (even / odd rows of the chunk); per-column parameter
+    float m0[W], m1[W];                 // kColOnline: the running maxima that a0 / a1 are relative to
+    double rcp[W];
+#pragma unroll
+    for (int e = 0; e < W; ++e) {
+        a0[e] = a1[e] = 0.0f;
+        m0[e] = m1[e] = kNegInf;
+        q0[e] = (MODE == kColSoftmaxOut || MODE == kColBwdOut) ? p0[col + e] : 0.0f;
+        rcp[e] = (MODE == kColSoftmaxOut) ? 1.0 / double(p1[col + e]) : 0.0;
+    }
+    auto load = [&](const float* __restrict__ base, size_t r, float (&v)[W]) {
+        if (W == 4) {
+            v4f t = *reinterpret_cast<const v4f*>(base + r * cols + col);
+#pragma unroll
+            for (int e = 0; e < W; ++e) v[e] = t[e];
+        } else {
+            v[0] = base[r * cols + col];
+        }
+    };
+    auto store = [&](size_t r, const float (&v)[W]) {
+        if (W == 4) {
+            v4f t;
+#pragma unroll
+            for (int e = 0; e < W; ++e) t[e] = v[e];
+            *reinterpret_cast<v4f*>(out + r * cols + col) = t;
+        } else {
+            out[r * cols + col] = v[0];
+        }
+    };
+    auto one_row = [&](size_t r, float (&acc)[W], float (&mx)[W], const float (&v)[W], const float (&w)[W]) {
+        float o[W];
+#pragma unroll
+        for (int e = 0; e < W; ++e) {
+            if (MODE == kColOnline) {
+                // one exponential per element either way, without a branch: of the old maximum's
+                // distance when the maximum moves (the sum is rescaled; exp(-inf) = 0 at the first
+                // row), of the element's distance otherwise (an element of -inf adds nothing)
+                const bool up = v[e] > mx[e];
+                float ex = cta_expf_nonpos(up ? mx[e] - v[e] : v[e] - mx[e], s_exp2);
+                ex = v[e] == kNegInf ? 0.0f : ex;
+                acc[e] = up ? __fmaf_rn(acc[e], ex, 1.0f) : acc[e] + ex;
+                mx[e] = up ? v[e] : mx[e];
+            } else if (MODE == kColSoftmaxOut) o[e] = cta_div_rcp(cta_expf_nonpos(v[e] - q0[e], s_exp2), rcp[e]);
+            else if (MODE == kColDot) acc[e] = __fmaf_rn(w[e], v[e], acc[e]);
+            else o[e] = v[e] * (w[e] - q0[e]);
+        }
+        if (MODE == kColSoftmaxOut || MODE == kColBwdOut) store(r, o);
+    };
+    constexpr bool kTwo = (MODE == kColDot || MODE == kColBwdOut);     // x = y, x2 = g
+    size_t r = r0;
+    for (; r + 3 < r1; r += 4) {            // four rows' loads in flight before the first is used
+        float v0[W], v1[W], v2[W], v3[W], w0[W] = {}, w1[W] = {}, w2[W] = {}, w3[W] = {};
+        load(x, r, v0);
+        load(x, r + 1, v1);
+        load(x, r + 2, v2);
+        load(x, r + 3, v3);
+        if (kTwo) {
+            load(x2, r, w0);
+            load(x2, r + 1, w1);
+            load(x2, r + 2, w2);
+            load(x2, r + 3, w3);
+        }
+        one_row(r, a0, m0, v0, w0);
+        one_row(r + 1, a1, m1, v1, w1);
+        one_row(r + 2, a0, m0, v2, w2);
+        one_row(r + 3, a1, m1, v3, w3);
+    }
+    for (; r < r1; ++r) {
+        float v0[W], w0[W] = {};
+        load(x, r, v0);
+        if (kTwo) load(x2, r, w0);
+        if ((r - r0) & 1) one_row(r, a1, m1, v0, w0);
+        else one_row(r, a0, m0, v0, w0);
+    }
+    if (MODE == kColDot) {
+#pragma unroll
+        for (int e = 0; e < W; ++e) out[size_t(blockIdx.y) * cols + col + e] = a0[e] + a1[e];
+    }
+    if (MODE == kColOnline) {
+        // the chunk's pair: both halves brought to the larger maximum; maxima in the first
+        // gridDim.y partial rows, sums in the next gridDim.y
+#pragma unroll
+        for (int e = 0; e < W; ++e) {
+            const float m = m1[e] > m0[e] ? m1[e] : m0[e];
+            float sum = 0.0f;
+            if (m0[e] != kNegInf) sum += a0[e] * cta_expf_nonpos(m0[e] - m, s_exp2);
+            if (m1[e] != kNegInf) sum += a1[e] * cta_expf_nonpos(m1[e] - m, s_exp2);
+            out[size_t(blockIdx.y) * cols + col + e] = m;
+            out[(size_t(gridDim.y) + blockIdx.y) * cols + col + e] = sum;
+        }
+    }
+}
+
+// The `chunks` partial rows of a column folded in double: their sum (PAIRS = false), or the
+// (max, sum) pairs of the online softmax brought to the column maximum (PAIRS = true: maxima in the
+// first `chunks` rows of partials, sums in the next; out_max[c], out[c]).  A block folds 32 columns;
+// its 8 groups of 32 lanes take every 8th chunk and are added in group order.
+constexpr int kFoldCols = 32, kFoldGroups = 8;
+template <bool PAIRS>
+__global__ __launch_bounds__(256) void col_fold_kernel(const float* __restrict__ partials, float* __restrict__ out_max,
+                                                       float* __restrict__ out, size_t cols, unsigned chunks) {
+    __shared__ uint64_t s_exp2[32];
+    __shared__ float s_m[kFoldGroups][kFoldCols];
+    __shared__ double s_t[kFoldGroups][kFoldCols];
+    if (PAIRS) stage_exp_table(s_exp2);
+    const unsigned lane = threadIdx.x % kFoldCols, group = threadIdx.x / kFoldCols;
+    const size_t c = size_t(blockIdx.x) * kFoldCols + lane;
+    const bool live = c < cols;
+    float m = kNegInf;
+    if (PAIRS) {
+        if (live) {
+#pragma unroll 4
+            for (unsigned k = group; k < chunks; k += kFoldGroups) {
+                const float v = partials[size_t(k) * cols + c];
+                m = v > m ? v : m;
+            }
+        }
+        s_m[group][lane] = m;
+        __syncthreads();
+#pragma unroll
+        for (int g = 0; g < kFoldGroups; ++g) m = s_m[g][lane] > m ? s_m[g][lane] : m;
+    }
+    double t = 0.0;
+    if (live) {
+#pragma unroll 4
+        for (unsigned k = group; k < chunks; k += kFoldGroups) {
+            if (PAIRS) {
+                const float mk = partials[size_t(k) * cols + c];
+                const float sk = partials[(size_t(chunks) + k) * cols + c];
+                if (mk != kNegInf) t += double(sk) * double(cta_expf_nonpos(mk - m, s_exp2));
+            } else {
+                t += double(partials[size_t(k) * cols + c]);
+            }
+        }
+    }
+    s_t[group][lane] = t;
+    __syncthreads();
+    if (group == 0 && live) {
+        double sum = 0.0;
+#pragma unroll
+        for (int g = 0; g < kFoldGroups; ++g) sum += s_t[g][lane];
+        if (PAIRS) out_max[c] = m;
+        out[c] = float(sum);
+    }
+}
+
+struct ColPlan {
+    size_t rows_per_block, chunks;
+    dim3 grid;
+    float* partials;
+    float* v0;      // [cols]
+    float* v1;      // [cols]
+    bool vec;
+};
+// false: the matrix is small (the sequential kernels serve it) or does not fit the scratch layout
+bool plan_cols(size_t rows, size_t cols, bool aligned, ColPlan& p) {
+    if (rows < 128) return false;
+    float* sc = scratch();
+    if (!sc) return false;
+    size_t chunks = (rows + 31) / 32;
+    if (chunks > 256) chunks = 256;
+    if ((2 * chunks + 2) * cols > kScratchFloats) {             // two partial rows per chunk (forward), two vectors
+        if (4 * cols > kScratchFloats) return false;
+        chunks = (kScratchFloats / cols - 2) / 2;
+    }
+    p.rows_per_block = (rows + chunks - 1) / chunks;
+    p.chunks = (rows + p.rows_per_block - 1) / p.rows_per_block;
+    p.vec = aligned && cols % 4 == 0;
+    const size_t per_block = size_t(256) * (p.vec ? 4 : 1);
+    const size_t strips = (cols + per_block - 1) / per_block;
+    if (strips > 0x7fffffffu || p.chunks > 65535) return false;
+    p.grid = dim3(unsigned(strips), unsigned(p.chunks));
+    p.partials = sc;
+    p.v0 = sc + 2 * p.chunks * cols;
+    p.v1 = p.v0 + cols;
+    return true;
+}
+
+template <int MODE>
+void launch_col_walk(const ColPlan& p, const float* x, const float* x2, const float* p0, const float* p1, float* out, size_t rows,
+                     size_t cols, hipStream_t s) {
+    if (p.vec) hipLaunchKernelGGL((col_walk_kernel<MODE, 4>), p.grid, dim3(256), 0, s, x, x2, p0, p1, out, rows, cols, p.rows_per_block);
+    else hipLaunchKernelGGL((col_walk_kernel<MODE, 1>), p.grid, dim3(256), 0, s, x, x2, p0, p1, out, rows, cols, p.rows_per_block);
+}
+
 }  // namespace
 }  // namespace ctamd
 
@@ -741,6 +951,16 @@ int ctamd_softmax_backward_rows_f32(const float* y, const float* g, float* dx, s
 int ctamd_softmax_cols_f32(const float* x, float* y, size_t rows, size_t cols, void* stream) {
     if (rows == 0 || cols == 0) return CTAMD_OK;
     if (!x || !y) return fail(CTAMD_EINVAL, "%s: null pointer", __func__);
+    ColPlan p;
+    if (plan_cols(rows, cols, aligned16(x) && aligned16(y), p)) {
+        hipStream_t s = as_stream(stream);
+        const unsigned fold_blocks = unsigned((cols + kFoldCols - 1) / kFoldCols);
+        launch_col_walk<kColOnline>(p, x, nullptr, nullptr, nullptr, p.partials, rows, cols, s);
+        hipLaunchKernelGGL(col_fold_kernel<true>, dim3(fold_blocks), dim3(256), 0, s, p.partials, p.v0, p.v1, cols, unsigned(p.chunks));
+        launch_col_walk<kColSoftmaxOut>(p, x, nullptr, p.v0, p.v1, y, rows, cols, s);
+        account(8.0 * double(rows) * double(cols), double(rows) * double(cols));
+        return launched(__func__);
+    }
     hipLaunchKernelGGL(softmax_cols_kernel, dim3((unsigned)((cols + 255) / 256)), dim3(256), 0, as_stream(stream), x, y,
                        rows, cols);
     account(8.0 * double(rows) * double(cols), double(rows) * double(cols));
@@ -749,6 +969,16 @@ int ctamd_softmax_cols_f32(const float* x, float* y, size_t rows, size_t cols, v
 int ctamd_softmax_backward_cols_f32(const float* y, const float* g, float* dx, size_t rows, size_t cols, void* stream) {
     if (rows == 0 || cols == 0) return CTAMD_OK;
     if (!y || !g || !dx) return fail(CTAMD_EINVAL, "%s: null pointer", __func__);
+    ColPlan p;
+    if (plan_cols(rows, cols, aligned16(y) && aligned16(g) && aligned16(dx), p)) {
+        hipStream_t s = as_stream(stream);
+        launch_col_walk<kColDot>(p, y, g, nullptr, nullptr, p.partials, rows, cols, s);
+        hipLaunchKernelGGL(col_fold_kernel<false>, dim3(unsigned((cols + kFoldCols - 1) / kFoldCols)), dim3(256), 0, s, p.partials, nullptr, p.v0,
+                           cols, unsigned(p.chunks));
+        launch_col_walk<kColBwdOut>(p, y, g, p.v0, nullptr, dx, rows, cols, s);
+        account(12.0 * double(rows) * double(cols), 2.0 * double(rows) * double(cols));
+        return launched(__func__);
+    }
     hipLaunchKernelGGL(softmax_bwd_cols_kernel, dim3((unsigned)((cols + 255) / 256)), dim3(256), 0, as_stream(stream), y,
                        g, dx, rows, cols);
     account(12.0 * double(rows) * double(cols), 2.0 * double(rows) * double(cols));

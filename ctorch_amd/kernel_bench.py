@@ -123,6 +123,13 @@ def main():
         if args.json:
             print(json.dumps({"device": torch.cuda.get_device_name(0), "results": results}))
         return 0
+    # comparisons (bool out: 9 and 5 B/elem), pixel bytes to floats (5 B/elem), column softmax
+    bout = torch.empty(n, dtype=torch.uint8, device="cuda")
+    ew("a > b (bool tensor)", lambda k: call("ctamd_compare_f32", 0, P(A[k]), P(B[k]), P(bout), n, S), 9)
+    ew("a > 0.25 (bool tensor)", lambda k: call("ctamd_compare_scalar_f32", 0, P(A[k]), C.c_float(0.25), P(bout), n, S), 5)
+    ew("pixel bytes / 255", lambda k: call("ctamd_u8_to_unit_f32", P(bout), P(R[k]), n, S), 5)
+    ew("softmax columns [16384 x 4096]", lambda k: call("ctamd_softmax_cols_f32", P(A[k]), P(R[k]), 16384, 4096, S), 8)
+    ew("softmax backward columns [16384 x 4096]", lambda k: call("ctamd_softmax_backward_cols_f32", P(A[k]), P(B[k]), P(R[k]), 16384, 4096, S), 12)
     cs = torch.empty(4096, device="cuda")
     ew("column sum [16384 x 4096]", lambda k: call("ctamd_colsum_f32", P(A[k]), P(cs), 16384, 4096, S), 4)
     del A, B, R

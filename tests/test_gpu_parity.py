@@ -315,16 +315,62 @@ def test_cross_entropy_edge_cases(oracle):
     assert G.host(G.ce_onehot(G.dev(np.zeros((0, 5), F)), G.dev(np.zeros((0, 5), F))))[0] == 0
 
 
-@pytest.mark.parametrize("shape", [(1, 1), (3, 7), (37, 53), (301, 19), (1000, 300)])
+@pytest.mark.parametrize("shape", [(1, 1), (3, 7), (37, 53), (127, 19), (128, 8), (301, 19), (1000, 300), (4099, 10),
+                                   (700, 1028), (20000, 64)])
 def test_softmax_columns(oracle, shape):
+    """Column (dim 0) softmax and its gradient.  Below 128 rows one thread walks a column in the
+    reference's order: 2 ulp / the same fma chain bit for bit.  Tall matrices use chunked column
+    reductions: the reduction bar (1e-5 relative, fp64 as the arbiter, the oracle to the same bound)."""
     print("case softmax cols", shape, flush=True)
     x = oracle.normal(shape, 30, 0, 2)
     y = G.host(G.softmax(G.dev(x), 0))
     want = oracle.softmax(x, 0)
-    assert ulp_diff(y, want).max() <= 2
     w = oracle.normal(shape, 31)
     got = G.host(G.softmax_bwd(G.dev(want), G.dev(w), 0))
-    bits_equal(got, oracle.softmax_bwd(want, w, 0), "softmax bwd cols")   # same sequential fma chain
+    want_b = oracle.softmax_bwd(want, w, 0)
+    if shape[0] < 128:
+        assert ulp_diff(y, want).max() <= 2
+        bits_equal(got, want_b, "softmax bwd cols")   # same sequential fma chain
+        return
+    x64 = x.astype(np.float64)
+    e64 = np.exp(x64 - x64.max(0, keepdims=True))
+    y64 = e64 / e64.sum(0, keepdims=True)
+    assert np.all(np.abs(y - y64) <= 1e-5 * y64 + 1e-37)
+    assert np.all(np.abs(y - want) <= 1e-5 * want + 1e-37)
+    assert np.all(np.abs(y.astype(np.float64).sum(0) - 1.0) <= 1e-5)
+    w64, s64 = w.astype(np.float64), want.astype(np.float64)
+    d64 = (w64 * s64).sum(0, keepdims=True)
+    scale = np.abs(s64) * (np.abs(w64) + np.abs(w64 * s64).sum(0, keepdims=True))
+    assert np.all(np.abs(got - s64 * (w64 - d64)) <= 1e-5 * scale + 1e-12)
+    assert np.all(np.abs(got - want_b) <= 2e-5 * scale + 1e-12)
+
+
+def test_softmax_columns_tall_edge_cases(oracle):
+    """The running (max, sum) pairs of the tall-matrix column softmax where they are stressed: a
+    maximum that moves at every row, one that never moves, elements of -inf, a spread beyond exp's
+    range, and a column that is -inf everywhere but one row."""
+    print("case softmax cols tall edge cases", flush=True)
+    rows, cols = 777, 12
+    x = oracle.normal((rows, cols), 33, 0, 1)
+    ramp = np.arange(rows, dtype=F)
+    x[:, 0] = ramp * 0.25                       # ascending: every row is a new maximum
+    x[:, 1] = -ramp * 0.25                      # descending: the first row stays the maximum
+    x[::3, 2] = -np.inf                         # holes
+    x[:, 3] = -np.inf
+    x[401, 3] = 2.5                             # one finite element
+    x[:, 4] = np.where(np.arange(rows) % 2 == 0, 300.0, -300.0).astype(F)
+    x[:5, 5] = -np.inf                          # a chunk that begins with -inf
+    x[:, 6] = 88.0 + ramp * 0.01                # exp(x) itself would overflow
+    y = G.host(G.softmax(G.dev(x), 0))
+    x64 = x.astype(np.float64)
+    e64 = np.exp(x64 - x64.max(0, keepdims=True))
+    y64 = e64 / e64.sum(0, keepdims=True)
+    assert np.all(np.isfinite(y))
+    assert np.all(np.abs(y - y64) <= 1e-5 * y64 + 1e-37)
+    assert np.all(y[x == -np.inf] == 0)
+    assert y[401, 3] == 1.0
+    want = oracle.softmax(x, 0)
+    assert np.all(np.abs(y - want) <= 1e-5 * want + 1e-37)
 
 
 MM_SHAPES = [(1, 1, 1), (5, 3, 9), (33, 29, 47), (128, 128, 16), (130, 257, 70), (256, 10, 784), (64, 256, 10),
