@@ -687,7 +687,7 @@ __global__ __launch_bounds__(256) void softmax_bwd_cols_kernel(const float* __re
 // Tall matrices (128 rows or more): the column statistics as chunked reductions over rows, like the
 // column sum - a block owns a strip of 256 * W columns and a chunk of rows and walks its rows in
 // order, two rows in flight; per-chunk partials are folded by a second launch.  Forward: per chunk
-// a running (max, sum of the bit-exact exp(x - max)) pair, rescaled when the maximum moves; the fold
+// a running (max, sum of exp(x - max)) pair, rescaled when the maximum moves; the fold
 // brings the chunks to the column maximum; then y = exp(x - max) / sum with the exact quotient (the
 // exponential is recomputed rather than stored: 12 B/elem instead of 16).
 // Backward: column dots of g and y, then dx = y * (g - dot).  The sums are chunked (fp32 inside a
@@ -702,7 +702,7 @@ __global__ __launch_bounds__(256) void col_walk_kernel(const float* __restrict__
                                                        float* __restrict__ out, size_t rows, size_t cols,
                                                        size_t rows_per_block) {
     __shared__ uint64_t s_exp2[32];
-    if (MODE == kColOnline || MODE == kColSoftmaxOut) stage_exp_table(s_exp2);
+    if (MODE == kColSoftmaxOut) stage_exp_table(s_exp2);
     const size_t col = (size_t(blockIdx.x) * 256 + threadIdx.x) * W;
     if (col >= cols) return;
     const size_t r0 = size_t(blockIdx.y) * rows_per_block;
@@ -745,8 +745,9 @@ __global__ __launch_bounds__(256) void col_walk_kernel(const float* __restrict__
                 // one exponential per element either way, without a branch: of the old maximum's
                 // distance when the maximum moves (the sum is rescaled; exp(-inf) = 0 at the first
                 // row), of the element's distance otherwise (an element of -inf adds nothing)
+                // (the hardware exponential: only the column sum is formed from it, ~1e-7 relative)
                 const bool up = v[e] > mx[e];
-                float ex = cta_expf_nonpos(up ? mx[e] - v[e] : v[e] - mx[e], s_exp2);
+                float ex = __builtin_amdgcn_exp2f((up ? mx[e] - v[e] : v[e] - mx[e]) * kLog2e);
                 ex = v[e] == kNegInf ? 0.0f : ex;
                 acc[e] = up ? __fmaf_rn(acc[e], ex, 1.0f) : acc[e] + ex;
                 mx[e] = up ? v[e] : mx[e];
@@ -758,22 +759,20 @@ __global__ __launch_bounds__(256) void col_walk_kernel(const float* __restrict__
     };
     constexpr bool kTwo = (MODE == kColDot || MODE == kColBwdOut);     // x = y, x2 = g
     size_t r = r0;
-    for (; r + 3 < r1; r += 4) {            // four rows' loads in flight before the first is used
-        float v0[W], v1[W], v2[W], v3[W], w0[W] = {}, w1[W] = {}, w2[W] = {}, w3[W] = {};
-        load(x, r, v0);
-        load(x, r + 1, v1);
-        load(x, r + 2, v2);
-        load(x, r + 3, v3);
+    constexpr int kRows = 4;                // rows whose loads are in flight before the first is used (8: no gain)
+    for (; r + kRows <= r1; r += kRows) {
+        float v[kRows][W], w[kRows][W] = {};
+#pragma unroll
+        for (int i = 0; i < kRows; ++i) load(x, r + i, v[i]);
         if (kTwo) {
-            load(x2, r, w0);
-            load(x2, r + 1, w1);
-            load(x2, r + 2, w2);
-            load(x2, r + 3, w3);
+#pragma unroll
+            for (int i = 0; i < kRows; ++i) load(x2, r + i, w[i]);
         }
-        one_row(r, a0, m0, v0, w0);
-        one_row(r + 1, a1, m1, v1, w1);
-        one_row(r + 2, a0, m0, v2, w2);
-        one_row(r + 3, a1, m1, v3, w3);
+#pragma unroll
+        for (int i = 0; i < kRows; i += 2) {
+            one_row(r + i, a0, m0, v[i], w[i]);
+            one_row(r + i + 1, a1, m1, v[i + 1], w[i + 1]);
+        }
     }
     for (; r < r1; ++r) {
         float v0[W], w0[W] = {};
@@ -793,8 +792,8 @@ __global__ __launch_bounds__(256) void col_walk_kernel(const float* __restrict__
         for (int e = 0; e < W; ++e) {
             const float m = m1[e] > m0[e] ? m1[e] : m0[e];
             float sum = 0.0f;
-            if (m0[e] != kNegInf) sum += a0[e] * cta_expf_nonpos(m0[e] - m, s_exp2);
-            if (m1[e] != kNegInf) sum += a1[e] * cta_expf_nonpos(m1[e] - m, s_exp2);
+            if (m0[e] != kNegInf) sum += a0[e] * __builtin_amdgcn_exp2f((m0[e] - m) * kLog2e);
+            if (m1[e] != kNegInf) sum += a1[e] * __builtin_amdgcn_exp2f((m1[e] - m) * kLog2e);
             out[size_t(blockIdx.y) * cols + col + e] = m;
             out[(size_t(gridDim.y) + blockIdx.y) * cols + col + e] = sum;
         }
