@@ -14,7 +14,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libctorch_amd.so")
-SOURCES = ["runtime.hip", "elementwise.hip", "reduce.hip", "softmax_ce.hip", "matmul.hip", "dataset.hip", "expr.hip"]
+SOURCES = ["runtime.hip", "elementwise.hip", "reduce.hip", "softmax_ce.hip", "matmul.hip", "dataset.hip", "expr.hip", "typed.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function"]
 

@@ -1,0 +1,363 @@
+// The reference's arms for tensors that are not fp32 (double, int32, int64, bool): zero() / ones(),
+// Tensor::to(dtype) from fp32, tensor (+ * /) float, the in-place gradient accumulation, and the
+// double softmax.  All but the softmax are HBM streams of 16-byte vectors; integer arithmetic wraps
+// (computed unsigned) and fp32 -> integer conversion gives the x86 "integer indefinite" value for
+// NaN and out-of-range inputs, which is what the reference's build computes.
+#include <limits.h>
+
+#include "common.h"
+
+namespace ctamd {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 4;
+
+// what a lane moves at once: 16 bytes (bool: four bytes, so that the fp32 source of a conversion
+// is one 16-byte vector as well)
+template <class T>
+struct Vec {
+    static constexpr int kLanes = sizeof(T) == 1 ? 4 : 16 / sizeof(T);
+    typedef T type __attribute__((ext_vector_type(sizeof(T) == 1 ? 4 : 16 / sizeof(T))));
+};
+
+// static_cast<int32_t / int64_t>(float) as cvttss2si computes it: truncation, 0x80..0 otherwise
+__device__ __forceinline__ int32_t to_i32(float x) {
+    return (x >= -2147483648.0f && x < 2147483648.0f) ? int32_t(x) : INT32_MIN;
+}
+__device__ __forceinline__ int64_t to_i64(float x) {
+    return (x >= -9223372036854775808.0f && x < 9223372036854775808.0f) ? int64_t(x) : INT64_MIN;
+}
+inline int32_t host_to_i32(float x) { return (x >= -2147483648.0f && x < 2147483648.0f) ? int32_t(x) : INT32_MIN; }
+inline int64_t host_to_i64(float x) {
+    return (x >= -9223372036854775808.0f && x < 9223372036854775808.0f) ? int64_t(x) : INT64_MIN;
+}
+
+template <class T>
+__device__ __forceinline__ T cast_one(float x);
+template <>
+__device__ __forceinline__ double cast_one<double>(float x) { return double(x); }
+template <>
+__device__ __forceinline__ int32_t cast_one<int32_t>(float x) { return to_i32(x); }
+template <>
+__device__ __forceinline__ int64_t cast_one<int64_t>(float x) { return to_i64(x); }
+template <>
+__device__ __forceinline__ uint8_t cast_one<uint8_t>(float x) { return x != 0.0f ? 1 : 0; }   // NaN is true
+
+enum { kAdd = CTAMD_TS_ADD, kMul = CTAMD_TS_MUL, kDiv = CTAMD_TS_DIV };
+
+template <int OP>
+__device__ __forceinline__ double op_one(double x, double s) { return OP == kAdd ? x + s : OP == kMul ? x * s : x / s; }
+template <int OP>
+__device__ __forceinline__ int32_t op_one(int32_t x, int32_t s) {
+    if (OP == kAdd) return int32_t(uint32_t(x) + uint32_t(s));
+    if (OP == kMul) return int32_t(uint32_t(x) * uint32_t(s));
+    return (s == -1) ? int32_t(0u - uint32_t(x)) : x / s;       // INT_MIN / -1 wraps instead of trapping
+}
+template <int OP>
+__device__ __forceinline__ int64_t op_one(int64_t x, int64_t s) {
+    if (OP == kAdd) return int64_t(uint64_t(x) + uint64_t(s));
+    if (OP == kMul) return int64_t(uint64_t(x) * uint64_t(s));
+    return (s == -1) ? int64_t(uint64_t(0) - uint64_t(x)) : x / s;
+}
+
+// out[i] = f(i-th vector); a thread owns kUnroll vectors one block-width apart, loaded (through
+// `load`) before the first is used; the tail beyond the last whole vector goes element by element
+// to the first threads of the grid.
+template <class T, class LoadF, class ElemF>
+__device__ __forceinline__ void stream_out(T* __restrict__ out, size_t n, LoadF load, ElemF elem) {
+    typedef typename Vec<T>::type V;
+    constexpr int L = Vec<T>::kLanes;
+    const size_t nv = n / L;
+    const size_t per_block = size_t(kThreads) * kUnroll;
+    for (size_t base = size_t(blockIdx.x) * per_block; base < nv; base += size_t(gridDim.x) * per_block) {
+        V r[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const size_t i = base + size_t(u) * kThreads + threadIdx.x;
+            if (i < nv) r[u] = load(i);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const size_t i = base + size_t(u) * kThreads + threadIdx.x;
+            if (i < nv) __builtin_nontemporal_store(r[u], reinterpret_cast<V*>(out) + i);
+        }
+    }
+    const size_t t = size_t(blockIdx.x) * kThreads + threadIdx.x;
+    if (t < n - nv * L) out[nv * L + t] = elem(nv * L + t);
+}
+
+template <class T>
+__global__ __launch_bounds__(kThreads) void fill_typed_kernel(T* __restrict__ out, T v, size_t n) {
+    typedef typename Vec<T>::type V;
+    stream_out<T>(out, n, [&](size_t) { V r; for (int e = 0; e < Vec<T>::kLanes; ++e) r[e] = v; return r; },
+                  [&](size_t) { return v; });
+}
+
+template <class T>
+__global__ __launch_bounds__(kThreads) void cast_kernel(const float* __restrict__ in, T* __restrict__ out, size_t n) {
+    typedef typename Vec<T>::type V;
+    typedef float F __attribute__((ext_vector_type(Vec<T>::kLanes)));
+    stream_out<T>(out, n,
+                  [&](size_t i) {
+                      F x = __builtin_nontemporal_load(reinterpret_cast<const F*>(in) + i);
+                      V r;
+#pragma unroll
+                      for (int e = 0; e < Vec<T>::kLanes; ++e) r[e] = cast_one<T>(x[e]);
+                      return r;
+                  },
+                  [&](size_t i) { return cast_one<T>(in[i]); });
+}
+
+template <class T, int OP>
+__global__ __launch_bounds__(kThreads) void scalar_typed_kernel(const T* __restrict__ in, T* __restrict__ out, T s, size_t n) {
+    typedef typename Vec<T>::type V;
+    stream_out<T>(out, n,
+                  [&](size_t i) {
+                      V x = __builtin_nontemporal_load(reinterpret_cast<const V*>(in) + i);
+                      V r;
+#pragma unroll
+                      for (int e = 0; e < Vec<T>::kLanes; ++e) r[e] = op_one<OP>(T(x[e]), s);
+                      return r;
+                  },
+                  [&](size_t i) { return op_one<OP>(in[i], s); });
+}
+
+template <class T>
+__global__ __launch_bounds__(kThreads) void accumulate_typed_kernel(T* __restrict__ acc, const T* __restrict__ val, size_t n) {
+    typedef typename Vec<T>::type V;
+    stream_out<T>(acc, n,
+                  [&](size_t i) {
+                      V a = __builtin_nontemporal_load(reinterpret_cast<const V*>(acc) + i);
+                      V b = __builtin_nontemporal_load(reinterpret_cast<const V*>(val) + i);
+                      V r;
+#pragma unroll
+                      for (int e = 0; e < Vec<T>::kLanes; ++e) r[e] = op_one<kAdd>(T(a[e]), T(b[e]));
+                      return r;
+                  },
+                  [&](size_t i) { return op_one<kAdd>(acc[i], val[i]); });
+}
+
+template <class T>
+unsigned typed_grid(size_t n) {
+    return stream_grid(n / Vec<T>::kLanes + 1, size_t(kThreads) * kUnroll, 8);
+}
+
+// ------------------------------------------------------------------------------ double softmax
+
+__device__ __forceinline__ double block_reduce(double v, bool is_max, double* s_part) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        double o = __shfl_xor(v, off, 64);
+        v = is_max ? (o > v ? o : v) : v + o;
+    }
+    const int wave = threadIdx.x >> 6;
+    __syncthreads();                    // s_part may still be read from the previous reduction
+    if ((threadIdx.x & 63) == 0) s_part[wave] = v;
+    __syncthreads();
+    double r = s_part[0];
+    for (int w = 1; w < int(blockDim.x >> 6); ++w) r = is_max ? (s_part[w] > r ? s_part[w] : r) : r + s_part[w];
+    return r;
+}
+
+// One block per row (grid-stride over rows): maximum, sum of exp(x - max), y = exp(x - max) / sum.
+// The row is read three times (the second and third time from the caches for rows up to a few
+// MiB) and the exponential computed twice, instead of being stored as the reference does.
+__global__ __launch_bounds__(256) void softmax_rows_f64_kernel(const double* __restrict__ x, double* __restrict__ y, size_t rows,
+                                                               size_t cols) {
+    __shared__ double s_part[4];
+    for (size_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        const double* xr = x + row * cols;
+        double* yr = y + row * cols;
+        double m = -__builtin_huge_val();
+        for (size_t j = threadIdx.x; j < cols; j += blockDim.x) m = xr[j] > m ? xr[j] : m;
+        m = block_reduce(m, true, s_part);
+        double sum = 0.0;
+        for (size_t j = threadIdx.x; j < cols; j += blockDim.x) sum += exp(xr[j] - m);
+        sum = block_reduce(sum, false, s_part);
+        for (size_t j = threadIdx.x; j < cols; j += blockDim.x) yr[j] = exp(xr[j] - m) / sum;
+    }
+}
+
+// A block owns 32 neighbouring columns; its 8 groups of 32 lanes take every 8th row (a group reads
+// 256 contiguous bytes per row) and are combined through LDS in group order: column maximum, sum of
+// exp(x - max), y = exp(x - max) / sum.  (One thread walking a whole column, the reference's
+// order src/Tensor.cpp:1766-1781, took 11.9 ms on [8192 x 8192].)
+constexpr int kColsPerBlock = 32, kRowGroups = 8;
+__global__ __launch_bounds__(256) void softmax_cols_f64_kernel(const double* __restrict__ x, double* __restrict__ y, size_t rows,
+                                                               size_t cols) {
+    __shared__ double s_red[kRowGroups][kColsPerBlock];
+    const unsigned lane = threadIdx.x % kColsPerBlock, group = threadIdx.x / kColsPerBlock;
+    const size_t j = size_t(blockIdx.x) * kColsPerBlock + lane;
+    const bool live = j < cols;
+    double m = -__builtin_huge_val();
+    if (live) {
+#pragma unroll 4
+        for (size_t i = group; i < rows; i += kRowGroups) {
+            const double v = x[i * cols + j];
+            m = v > m ? v : m;
+        }
+    }
+    s_red[group][lane] = m;
+    __syncthreads();
+#pragma unroll
+    for (int g = 0; g < kRowGroups; ++g) m = s_red[g][lane] > m ? s_red[g][lane] : m;
+    __syncthreads();
+    double sum = 0.0;
+    if (live) {
+#pragma unroll 4
+        for (size_t i = group; i < rows; i += kRowGroups) sum += exp(x[i * cols + j] - m);
+    }
+    s_red[group][lane] = sum;
+    __syncthreads();
+    double total = 0.0;
+#pragma unroll
+    for (int g = 0; g < kRowGroups; ++g) total += s_red[g][lane];
+    if (live) {
+#pragma unroll 4
+        for (size_t i = group; i < rows; i += kRowGroups) y[i * cols + j] = exp(x[i * cols + j] - m) / total;
+    }
+}
+
+size_t dtype_bytes(int dtype) {
+    switch (dtype) {
+        case CTAMD_DT_F32: case CTAMD_DT_I32: return 4;
+        case CTAMD_DT_F64: case CTAMD_DT_I64: return 8;
+        case CTAMD_DT_BOOL: return 1;
+    }
+    return 0;
+}
+
+}  // namespace
+}  // namespace ctamd
+
+using namespace ctamd;
+
+extern "C" {
+
+int ctamd_fill_typed(void* out, int dtype, double value, size_t n, void* stream) {
+    const size_t width = dtype_bytes(dtype);
+    if (!width) return fail(CTAMD_EINVAL, "%s: bad dtype %d", __func__, dtype);
+    if (n == 0) return CTAMD_OK;
+    if (!out) return fail(CTAMD_EINVAL, "%s: null pointer", __func__);
+    if (!aligned16(out)) return fail(CTAMD_EINVAL, "%s: the tensor must start on a 16-byte boundary", __func__);
+    hipStream_t s = as_stream(stream);
+    switch (dtype) {
+        case CTAMD_DT_F32:
+            hipLaunchKernelGGL(fill_typed_kernel<float>, dim3(typed_grid<float>(n)), dim3(kThreads), 0, s, static_cast<float*>(out), float(value), n);
+            break;
+        case CTAMD_DT_F64:
+            hipLaunchKernelGGL(fill_typed_kernel<double>, dim3(typed_grid<double>(n)), dim3(kThreads), 0, s, static_cast<double*>(out), value, n);
+            break;
+        case CTAMD_DT_I32:
+            hipLaunchKernelGGL(fill_typed_kernel<int32_t>, dim3(typed_grid<int32_t>(n)), dim3(kThreads), 0, s, static_cast<int32_t*>(out),
+                               int32_t(value), n);
+            break;
+        case CTAMD_DT_I64:
+            hipLaunchKernelGGL(fill_typed_kernel<int64_t>, dim3(typed_grid<int64_t>(n)), dim3(kThreads), 0, s, static_cast<int64_t*>(out),
+                               int64_t(value), n);
+            break;
+        default: {      // whole 32-bit words of four equal bytes, then the last 0..3 bytes
+            const uint8_t b = value != 0.0 ? 1 : 0;
+            const size_t words = n / 4;
+            if (words)
+                hipLaunchKernelGGL(fill_typed_kernel<int32_t>, dim3(typed_grid<int32_t>(words)), dim3(kThreads), 0, s, static_cast<int32_t*>(out),
+                                   int32_t(b * 0x01010101u), words);
+            if (n % 4)
+                hipLaunchKernelGGL(fill_typed_kernel<uint8_t>, dim3(1), dim3(kThreads), 0, s, static_cast<uint8_t*>(out) + words * 4, b, n % 4);
+        }
+    }
+    account(double(n) * double(width), 0.0);
+    return launched(__func__);
+}
+
+int ctamd_cast_from_f32(const float* in, void* out, int dtype, size_t n, void* stream) {
+    const size_t width = dtype_bytes(dtype);
+    if (!width || dtype == CTAMD_DT_F32) return fail(CTAMD_EINVAL, "%s: bad target dtype %d", __func__, dtype);
+    if (n == 0) return CTAMD_OK;
+    if (!in || !out) return fail(CTAMD_EINVAL, "%s: null pointer", __func__);
+    if (!aligned16(out) || !aligned16(in)) return fail(CTAMD_EINVAL, "%s: tensors must start on 16-byte boundaries", __func__);
+    hipStream_t s = as_stream(stream);
+    switch (dtype) {
+        case CTAMD_DT_F64:
+            hipLaunchKernelGGL(cast_kernel<double>, dim3(typed_grid<double>(n)), dim3(kThreads), 0, s, in, static_cast<double*>(out), n);
+            break;
+        case CTAMD_DT_I32:
+            hipLaunchKernelGGL(cast_kernel<int32_t>, dim3(typed_grid<int32_t>(n)), dim3(kThreads), 0, s, in, static_cast<int32_t*>(out), n);
+            break;
+        case CTAMD_DT_I64:
+            hipLaunchKernelGGL(cast_kernel<int64_t>, dim3(typed_grid<int64_t>(n)), dim3(kThreads), 0, s, in, static_cast<int64_t*>(out), n);
+            break;
+        default:
+            hipLaunchKernelGGL(cast_kernel<uint8_t>, dim3(typed_grid<uint8_t>(n)), dim3(kThreads), 0, s, in, static_cast<uint8_t*>(out), n);
+    }
+    account(double(n) * double(4 + width), 0.0);
+    return launched(__func__);
+}
+
+int ctamd_scalar_op_typed(const void* in, void* out, int dtype, int op, float scalar, size_t n, void* stream) {
+    if (dtype != CTAMD_DT_F64 && dtype != CTAMD_DT_I32 && dtype != CTAMD_DT_I64)
+        return fail(CTAMD_EINVAL, "%s: dtype %d has no scalar arithmetic", __func__, dtype);
+    if (op != kAdd && op != kMul && op != kDiv) return fail(CTAMD_EINVAL, "%s: bad op %d", __func__, op);
+    const int64_t si = dtype == CTAMD_DT_I32 ? int64_t(host_to_i32(scalar)) : host_to_i64(scalar);
+    if (op == kDiv && dtype != CTAMD_DT_F64 && si == 0)
+        return fail(CTAMD_EINVAL, "%s: the scalar converts to the integer 0 (the reference's process stops on this division)", __func__);
+    if (n == 0) return CTAMD_OK;
+    if (!in || !out) return fail(CTAMD_EINVAL, "%s: null pointer", __func__);
+    if (!aligned16(out) || !aligned16(in)) return fail(CTAMD_EINVAL, "%s: tensors must start on 16-byte boundaries", __func__);
+    hipStream_t s = as_stream(stream);
+#define CTAMD_TYPED_LAUNCH(T, OP, SV) \
+    hipLaunchKernelGGL((scalar_typed_kernel<T, OP>), dim3(typed_grid<T>(n)), dim3(kThreads), 0, s, static_cast<const T*>(in), static_cast<T*>(out), T(SV), n)
+#define CTAMD_TYPED_OPS(T, SV)                              \
+    do {                                                    \
+        if (op == kAdd) CTAMD_TYPED_LAUNCH(T, kAdd, SV);    \
+        else if (op == kMul) CTAMD_TYPED_LAUNCH(T, kMul, SV); \
+        else CTAMD_TYPED_LAUNCH(T, kDiv, SV);               \
+    } while (0)
+    if (dtype == CTAMD_DT_F64) CTAMD_TYPED_OPS(double, double(scalar));
+    else if (dtype == CTAMD_DT_I32) CTAMD_TYPED_OPS(int32_t, si);
+    else CTAMD_TYPED_OPS(int64_t, si);
+#undef CTAMD_TYPED_OPS
+#undef CTAMD_TYPED_LAUNCH
+    account(double(n) * 2.0 * double(dtype_bytes(dtype)), 0.0);
+    return launched(__func__);
+}
+
+int ctamd_accumulate_typed(void* acc, const void* val, int dtype, size_t n, void* stream) {
+    if (dtype != CTAMD_DT_F64 && dtype != CTAMD_DT_I32 && dtype != CTAMD_DT_I64)
+        return fail(CTAMD_EINVAL, "%s: dtype %d is not accumulated", __func__, dtype);
+    if (n == 0) return CTAMD_OK;
+    if (!acc || !val) return fail(CTAMD_EINVAL, "%s: null pointer", __func__);
+    if (!aligned16(acc) || !aligned16(val)) return fail(CTAMD_EINVAL, "%s: tensors must start on 16-byte boundaries", __func__);
+    hipStream_t s = as_stream(stream);
+    if (dtype == CTAMD_DT_F64)
+        hipLaunchKernelGGL(accumulate_typed_kernel<double>, dim3(typed_grid<double>(n)), dim3(kThreads), 0, s, static_cast<double*>(acc),
+                           static_cast<const double*>(val), n);
+    else if (dtype == CTAMD_DT_I32)
+        hipLaunchKernelGGL(accumulate_typed_kernel<int32_t>, dim3(typed_grid<int32_t>(n)), dim3(kThreads), 0, s, static_cast<int32_t*>(acc),
+                           static_cast<const int32_t*>(val), n);
+    else
+        hipLaunchKernelGGL(accumulate_typed_kernel<int64_t>, dim3(typed_grid<int64_t>(n)), dim3(kThreads), 0, s, static_cast<int64_t*>(acc),
+                           static_cast<const int64_t*>(val), n);
+    account(double(n) * 3.0 * double(dtype_bytes(dtype)), 0.0);
+    return launched(__func__);
+}
+
+int ctamd_softmax_f64(const double* x, double* y, size_t rows, size_t cols, int dim, void* stream) {
+    if (dim != 0 && dim != 1) return fail(CTAMD_EINVAL, "%s: dim must be 0 or 1", __func__);
+    if (rows == 0 || cols == 0) return CTAMD_OK;
+    if (!x || !y) return fail(CTAMD_EINVAL, "%s: null pointer", __func__);
+    hipStream_t s = as_stream(stream);
+    if (dim == 1) {
+        const unsigned blocks = stream_grid(rows, 1, 8);
+        hipLaunchKernelGGL(softmax_rows_f64_kernel, dim3(blocks), dim3(cols <= 64 ? 64 : 256), 0, s, x, y, rows, cols);
+    } else {
+        const size_t blocks = (cols + kColsPerBlock - 1) / kColsPerBlock;
+        if (blocks > 0x7fffffffu) return fail(CTAMD_ERANGE, "%s: too many columns", __func__);
+        hipLaunchKernelGGL(softmax_cols_f64_kernel, dim3(unsigned(blocks)), dim3(256), 0, s, x, y, rows, cols);
+    }
+    account(double(rows) * double(cols) * 16.0, 0.0);
+    return launched(__func__);
+}
+
+}  // extern "C"

@@ -107,6 +107,7 @@ class Tensor {
 
     // ---- transfers
     Tensor to(DeviceType device) const;
+    Tensor to(DType dtype) const;            // from float only, as src/Tensor.cpp:197-243
     Tensor cpu() const { return to(DeviceType::kCPU); }
     Tensor amd() const { return to(DeviceType::kAMD); }
 
@@ -158,7 +159,7 @@ class Tensor {
     Tensor operator>=(const Tensor& other) const;
     Tensor operator<=(const Tensor& other) const;
     Tensor operator!=(const Tensor& other) const;   // declared by the reference (Tensor.h), defined here
-    std::vector<unsigned char> to_bytes() const;    // a bool tensor's elements on the host (any device)
+    std::vector<unsigned char> to_bytes() const;    // the elements' bytes on the host, any dtype (contiguous tensors)
     Tensor sum() const;
     Tensor softmax(int dim = -1) const;
 

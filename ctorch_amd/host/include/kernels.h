@@ -38,6 +38,9 @@ Tensor scalar_op(const Tensor& a, float s, op which);
 // a (cmp) b or, with b == nullptr, a (cmp) s: a bool tensor; cmp is a CTAMD_CMP_* code
 Tensor compare_op(int cmp, const Tensor& a, const Tensor* b, float s);                 // a + s, a * s, a / s
 Tensor sum_all(const Tensor& a);
+// tensors that are not fp32 (the typed arms of src/Tensor.cpp:197-243, :390-448)
+void fill_typed(void* device_ptr, DType dtype, double v, size_t n);    // zero() / ones() of any dtype, device memory
+Tensor cast_from_float(const Tensor& a, DType to);                    // Tensor::to(DType)
 Tensor softmax_dim(const Tensor& a, int dim);                         // dim already normalised
 Tensor filled(const std::vector<size_t>& shape, float v, DeviceType device);
 void fill_scalar(Tensor& t, float v);                                  // every element of a device tensor = v

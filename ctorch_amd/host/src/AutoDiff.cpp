@@ -332,6 +332,10 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
         return;
     }
     if (!root_node->requires_grad) return;
+    // Gradients are float: the seed is (src/AutoDiff.cpp:548-553), and the reference's backward over
+    // a double / int root stops with a DATATYPE exception when that seed meets the typed nodes.
+    if (root.dtype() != DType::kFloat || grad_output.dtype() != DType::kFloat)
+        Ctorch_Error::throwException(ErrorPlatform::kAutoDiff, ErrorType::DATATYPE, "backward: only float tensors have gradients");
     if (grad_output.device() != root.device()) grad_output = grad_output.to(root.device());
     root_node->grad = std::make_unique<Tensor>(adjust_grad_shape(grad_output, root.sizes()));
     root_node->grad_plus_zero = seed_plus_zero_;

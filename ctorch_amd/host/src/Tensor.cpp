@@ -188,14 +188,34 @@ void Tensor::fill(float v) {
         for (size_t i = 0; i < _storage.size(); ++i) p[i] = v;
     }
 }
+// src/Tensor.cpp:390-448: every dtype, the whole storage
 void Tensor::zero() {
     if (_storage.empty()) return;
     if (_dtype == DType::kFloat) { fill(0.0f); return; }
-    if (_device != DeviceType::kCPU)
-        Ctorch_Error::throwException(ErrorPlatform::kAMD, ErrorType::DATATYPE, "zero(): device tensors are float only");
+    if (_device == DeviceType::kAMD) { ctorch_amd_host::fill_typed(_storage.raw(), _dtype, 0.0, _storage.size()); return; }
     std::memset(_storage.raw(), 0, _storage.nbytes());
 }
-void Tensor::ones() { fill(1.0f); }
+void Tensor::ones() {
+    if (_storage.empty()) return;
+    if (_dtype == DType::kFloat) { fill(1.0f); return; }
+    if (_device == DeviceType::kAMD) { ctorch_amd_host::fill_typed(_storage.raw(), _dtype, 1.0, _storage.size()); return; }
+    const size_t n = _storage.size();
+    switch (_dtype) {
+        case DType::kDouble: for (size_t i = 0; i < n; ++i) _storage.data<double>()[i] = 1.0; break;
+        case DType::kInt: for (size_t i = 0; i < n; ++i) _storage.data<int32_t>()[i] = 1; break;
+        case DType::kLong: for (size_t i = 0; i < n; ++i) _storage.data<int64_t>()[i] = 1; break;
+        default: std::memset(_storage.raw(), 1, _storage.nbytes());
+    }
+}
+
+Tensor Tensor::to(DType dtype) const {
+    if (_dtype == dtype) return *this;
+    if (_dtype != DType::kFloat)    // the reference returns an uninitialised tensor here (src/Tensor.cpp:206: only float sources are converted)
+        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DATATYPE, "to(dtype): only float tensors are converted");
+    if (_device != DeviceType::kAMD)
+        Ctorch_Error::throwException(ErrorPlatform::kCPU, ErrorType::DEVICE_COMPAT, "to(dtype): computed on the AMD device only");
+    return ctorch_amd_host::cast_from_float(*this, dtype);
+}
 
 Tensor Tensor::transpose(int dim0, int dim1) const {
     if (dim0 < 0 || dim0 >= int(_shape.size()) || dim1 < 0 || dim1 >= int(_shape.size()))
@@ -333,8 +353,9 @@ Tensor Tensor::operator!=(const Tensor& o) const { return compare_with(CTAMD_CMP
 std::vector<unsigned char> Tensor::to_bytes() const {
     std::vector<unsigned char> out(numel());
     if (out.empty() || _storage.empty()) return out;
-    if (_dtype != DType::kBool || !is_contiguous())
-        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DATATYPE, "to_bytes(): a contiguous bool tensor is needed");
+    if (!is_contiguous())
+        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::TENSOR_STATE, "to_bytes(): a contiguous tensor is needed");
+    out.resize(numel() * dtypeSize(_dtype));
     const unsigned char* src = static_cast<const unsigned char*>(raw_ptr());
     if (_device == DeviceType::kAMD) device_copy_d2h(out.data(), src, out.size());
     else std::memcpy(out.data(), src, out.size());

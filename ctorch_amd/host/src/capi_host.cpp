@@ -162,6 +162,57 @@ long cth_compare(int cmp, const float* a, const long* ad, int an, const float* b
     }
 }
 
+// Tensors that are not fp32: the fp32 input through Tensor::to(dtype) (dtype in the order of enum
+// DType), then through `n_steps` operations in order, step k being whats[k] with scalars[k]:
+// 0 '+ s', 1 '* s', 2 '/ s', 3 zero(), 4 ones(), 5 softmax(dim = (int)s).  The result's bytes are
+// copied to `out`; returns its element count.
+long cth_typed(const float* a, const long* ad, int an, int dtype, const int* whats, const float* scalars, int n_steps,
+               void* out) {
+    try {
+        Tensor t = make(a, ad, an).to(static_cast<DType>(dtype));
+        for (int k = 0; k < n_steps; ++k) {
+            const float s = scalars[k];
+            switch (whats[k]) {
+                case 0: t = t + s; break;
+                case 1: t = t * s; break;
+                case 2: t = t / s; break;
+                case 3: t.zero(); break;
+                case 4: t.ones(); break;
+                case 5: t = t.softmax(static_cast<int>(s)); break;
+                default: return -3;
+            }
+        }
+        std::vector<unsigned char> v = t.to_bytes();
+        std::memcpy(out, v.data(), v.size());
+        return static_cast<long>(t.numel());
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
+// The tape through scalar operators on a tensor that is not fp32: backward() of it throws in the
+// reference (its float seed meets typed nodes: DATATYPE), and must here; returns -1 then.
+long cth_typed_grad(const float* a, const long* ad, int an, int dtype, const int* whats, const float* scalars, int n_steps,
+                    void* grad_out, int* grad_dtype) {
+    try {
+        AutoDiff ctx;
+        configure(ctx);
+        AutoDiffContext::Guard guard(&ctx);
+        Tensor x = make(a, ad, an).to(static_cast<DType>(dtype));
+        x.requires_grad(true);
+        Tensor y = whats[0] == 0 ? x + scalars[0] : whats[0] == 1 ? x * scalars[0] : x / scalars[0];
+        for (int k = 1; k < n_steps; ++k) y = whats[k] == 0 ? y + scalars[k] : whats[k] == 1 ? y * scalars[k] : y / scalars[k];
+        backward(y);
+        Tensor g = grad(x);
+        *grad_dtype = static_cast<int>(g.dtype());
+        std::vector<unsigned char> v = g.to_bytes();
+        std::memcpy(grad_out, v.data(), v.size());
+        return static_cast<long>(g.numel());
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
 // tensor (op) host scalar: which = 0 '+', 1 '*', 2 '/'
 long cth_scalar(int which, const float* a, const long* ad, int an, float s, float* out) {
     try {

@@ -104,7 +104,38 @@ void rows_cols(const Tensor& a, size_t& rows, size_t& cols) {
 }  // namespace
 
 // ------------------------------------------------------------------ helpers for Tensor / tape
+namespace {
+void check_on_device(const Tensor& a, const char* who) {
+    if (a.device() != DeviceType::kAMD)
+        Ctorch_Error::throwException(DeviceTypeToErrorPlatform(a.device()), ErrorType::DEVICE_COMPAT,
+                                     std::string(who) + ": tensor is not on the AMD device");
+    if (!a.is_contiguous())
+        Ctorch_Error::throwException(kP, ErrorType::TENSOR_STATE, std::string(who) + ": a contiguous tensor is needed");
+}
+}  // namespace
+
+void fill_typed(void* device_ptr, DType dtype, double v, size_t n) {
+    run(ctamd_fill_typed(device_ptr, int(dtype), v, n, current_stream()), "zero / ones");
+}
+Tensor cast_from_float(const Tensor& a, DType to) {
+    check_device(a, "to(dtype)");                                       // src/Tensor.cpp:206: conversions start from float only
+    if (!a.is_contiguous())
+        Ctorch_Error::throwException(kP, ErrorType::TENSOR_STATE, "to(dtype): a contiguous tensor is needed");
+    Tensor r(ShapeTag{}, a.sizes(), to, DeviceType::kAMD, false);
+    run(ctamd_cast_from_f32(a.fptr(), r.raw_ptr(), int(to), a.numel(), current_stream()), "to(dtype)");
+    return r;
+}
 Tensor scalar_op(const Tensor& a, float s, op which) {
+    if (a.dtype() != DType::kFloat) {
+        // the typed arms of src/Tensor.cpp:766-786, :870-890, :933-953; anything else is refused as there
+        if (a.dtype() != DType::kDouble && a.dtype() != DType::kInt && a.dtype() != DType::kLong)
+            Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DATATYPE, "tensor (op) float: unsupported dtype");
+        check_on_device(a, "tensor (op) float");
+        Tensor r(ShapeTag{}, a.sizes(), a.dtype(), DeviceType::kAMD, false);
+        const int code = which == op::Add ? CTAMD_TS_ADD : which == op::Mul ? CTAMD_TS_MUL : CTAMD_TS_DIV;
+        run(ctamd_scalar_op_typed(a.raw_ptr(), r.raw_ptr(), int(a.dtype()), code, s, a.numel(), current_stream()), "tensor (op) float");
+        return r;
+    }
     check_device(a, "tensor (op) float");
     Tensor r = like(a);
     int rc = which == op::Add ? ctamd_add_scalar_f32(a.fptr(), s, r.fptr(), a.numel(), current_stream())
@@ -138,6 +169,15 @@ Tensor sum_all(const Tensor& a) {
     return r;
 }
 Tensor softmax_dim(const Tensor& a, int dim) {
+    if (a.dtype() == DType::kDouble) {                                  // src/Tensor.cpp:1686-1696, :1747-1783
+        check_on_device(a, "softmax");
+        Tensor r(ShapeTag{}, a.sizes(), DType::kDouble, DeviceType::kAMD, false);
+        size_t rows = a.dim() == 1 ? 1 : a.sizes()[0], cols = a.dim() == 1 ? a.sizes()[0] : a.sizes()[1];
+        run(ctamd_softmax_f64(static_cast<const double*>(a.raw_ptr()), static_cast<double*>(r.raw_ptr()), rows, cols,
+                              a.dim() == 1 ? 1 : dim, current_stream()),
+            "softmax");
+        return r;
+    }
     check_device(a, "softmax");
     Tensor r = like(a);
     size_t rows, cols;

@@ -132,6 +132,19 @@ def main():
     ew("softmax backward columns [16384 x 4096]", lambda k: call("ctamd_softmax_backward_cols_f32", P(A[k]), P(B[k]), P(R[k]), 16384, 4096, S), 12)
     cs = torch.empty(4096, device="cuda")
     ew("column sum [16384 x 4096]", lambda k: call("ctamd_colsum_f32", P(A[k]), P(cs), 16384, 4096, S), 4)
+    # tensors that are not fp32: conversion, scalar operators, accumulation (2^26 elements), double softmax
+    D64 = [torch.empty(n, dtype=torch.float64, device="cuda").normal_() for _ in range(2)]
+    I32 = [torch.randint(-1000, 1000, (n,), dtype=torch.int32, device="cuda") for _ in range(2)]
+    ew("fp32 -> double", lambda k: call("ctamd_cast_from_f32", P(A[k]), P(D64[0]), 1, n, S), 12)
+    ew("fp32 -> int32", lambda k: call("ctamd_cast_from_f32", P(A[k]), P(I32[0]), 2, n, S), 8)
+    ew("double * 2.5f", lambda k: call("ctamd_scalar_op_typed", P(D64[k % 2]), P(D64[1 - k % 2]), 1, 1, C.c_float(2.5), n, S), 16)
+    ew("int32 / 3.0f", lambda k: call("ctamd_scalar_op_typed", P(I32[k % 2]), P(I32[1 - k % 2]), 2, 2, C.c_float(3.0), n, S), 8)
+    ew("double += double", lambda k: call("ctamd_accumulate_typed", P(D64[0]), P(D64[1]), 1, n, S), 24)
+    ew("ones (double)", lambda k: call("ctamd_fill_typed", P(D64[0]), 1, C.c_double(1.0), n, S), 8)
+    D64[0].normal_()
+    ew("softmax rows, double [8192 x 8192]", lambda k: call("ctamd_softmax_f64", P(D64[0]), P(D64[1]), 8192, 8192, 1, S), 16)
+    ew("softmax columns, double [8192 x 8192]", lambda k: call("ctamd_softmax_f64", P(D64[0]), P(D64[1]), 8192, 8192, 0, S), 16)
+    del D64, I32
     del A, B, R
     torch.cuda.empty_cache()
 

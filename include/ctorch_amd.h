@@ -194,6 +194,33 @@ enum { CTAMD_CMP_GT = 0, CTAMD_CMP_LT = 1, CTAMD_CMP_EQ = 2, CTAMD_CMP_GE = 3, C
 int ctamd_compare_f32(int cmp, const float* a, const float* b, uint8_t* out, size_t n, void* stream);
 int ctamd_compare_scalar_f32(int cmp, const float* a, float s, uint8_t* out, size_t n, void* stream);
 
+/* ------------------------------------------------------- tensors that are not fp32 */
+/* The reference's arms for double, int32, int64 and bool tensors.  dtype codes are the order of
+ * enum DType (include/Ctools.h:163-169).  Tensors start on 16-byte boundaries and are contiguous.
+ * Integer arithmetic wraps; fp32 -> integer conversion truncates and gives the most negative
+ * integer for NaN and for values out of range, as the reference's x86 build does. */
+enum { CTAMD_DT_F32 = 0, CTAMD_DT_F64 = 1, CTAMD_DT_I32 = 2, CTAMD_DT_I64 = 3, CTAMD_DT_BOOL = 4 };
+/* out[i] = value converted to dtype (bool: value != 0): Tensor::zero() / ones()
+ * src/Tensor.cpp:390-448 and the zero tensors of AutoDiff::get_grad src/AutoDiff.cpp:205-245. */
+int ctamd_fill_typed(void* out, int dtype, double value, size_t n, void* stream);
+/* out[i] = static_cast<T>(in[i]) for T = double, int32, int64, bool: Tensor::to(DType)
+ * src/Tensor.cpp:197-243 (which converts from fp32 only). */
+int ctamd_cast_from_f32(const float* in, void* out, int dtype, size_t n, void* stream);
+/* out[i] = in[i] op static_cast<T>(scalar) for T = double, int32, int64: the typed arms of
+ * Tensor::operator+(float) src/Tensor.cpp:870-890, operator*(float) :766-786, operator/(float)
+ * :933-953.  Integer division truncates; CTAMD_EINVAL when the scalar converts to the integer 0
+ * (the reference's process stops with SIGFPE there); the most negative integer divided by -1
+ * wraps to itself (the reference stops there as well). */
+enum { CTAMD_TS_ADD = 0, CTAMD_TS_MUL = 1, CTAMD_TS_DIV = 2 };
+int ctamd_scalar_op_typed(const void* in, void* out, int dtype, int op, float scalar, size_t n, void* stream);
+/* acc[i] += val[i] for double, int32, int64: the typed arms of the gradient accumulation
+ * src/AutoDiff.cpp:1880-1903. */
+int ctamd_accumulate_typed(void* acc, const void* val, int dtype, size_t n, void* stream);
+/* Softmax of a double tensor along dim 1 (rows; a 1-D tensor is one row) or dim 0 (columns):
+ * Tensor::softmax(dim) src/Tensor.cpp:1686-1696, :1747-1783.  exp is the device library's double
+ * exponential, not glibc's: results agree with the reference's to a few units in the last place. */
+int ctamd_softmax_f64(const double* x, double* y, size_t rows, size_t cols, int dim, void* stream);
+
 /* ------------------------------------------------------------------ fused expressions */
 /* A chain of the elementwise operators above evaluated in ONE pass over memory: the front-end
  * compiles an expression such as Y = sigmoid(X / r) - tanh(X) * sin(X) + cos(-X) (and, separately,

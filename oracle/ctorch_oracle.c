@@ -26,7 +26,12 @@
  * co_expr_run (a per-element program of the operators above) is pinned opcode by opcode against
  * the whole-tensor functions here, which the reference pins, and on the config-5 chain against
  * co_expr; co_compare against the IEEE predicates the reference's plain C++ comparisons are
- * (tests/test_oracle_golden.py).  The MNIST functions (co_u8_to_unit ... co_mnist_predict) are
+ * (tests/test_oracle_golden.py).  The functions for tensors that are not fp32 (co_cast_from_f32,
+ * co_scalar_op_typed, co_softmax_f64) are pinned byte for byte against the reference's Tensor::to,
+ * operator+ * / (float), zero / ones and softmax on double, int32, int64 and bool tensors
+ * (tests/golden/typed.npz: edge conversions, wrapping sums and products, truncating scalars);
+ * co_accumulate_typed against IEEE double addition and two's complement wrap.
+ * The MNIST functions (co_u8_to_unit ... co_mnist_predict) are
  * pinned bit for bit against the reference's loader, demo functions and its own main()
  * (tests/test_oracle_vs_ref_mnist.py, tests/golden/mnist.npz).
  * Transcendentals call glibc libm (expf, logf, sinf, cosf) exactly as the reference does; their
@@ -36,6 +41,7 @@
 
 #include <float.h>
 #include <math.h>
+#include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
 
@@ -783,6 +789,106 @@ void co_compare(int cmp, const float* a, const float* b, float s, unsigned char*
     for (long i = 0; i < n; ++i) {
         const float x = a[i], y = b ? b[i] : s;
         out[i] = (unsigned char)(cmp == 0 ? x > y : cmp == 1 ? x < y : cmp == 2 ? x == y : cmp == 3 ? x >= y : cmp == 4 ? x <= y : x != y);
+    }
+}
+
+/* ------------------------------------------------------------- tensors that are not fp32 */
+/* dtype codes are the order of enum DType (include/Ctools.h:163-169): 0 float, 1 double, 2 int32,
+ * 3 int64, 4 bool (one byte). */
+
+/* static_cast<int32_t / int64_t>(float) as the reference's x86-64 build computes it (cvttss2si and
+ * its vector forms): truncation toward zero, and the "integer indefinite" value 0x80...0 for NaN
+ * and for values out of range - which C leaves undefined, so it is spelled out here. */
+static int32_t f32_to_i32(float x) { return (x >= -2147483648.0f && x < 2147483648.0f) ? (int32_t)x : INT32_MIN; }
+static int64_t f32_to_i64(float x) {
+    return (x >= -9223372036854775808.0f && x < 9223372036854775808.0f) ? (int64_t)x : INT64_MIN;
+}
+
+/* Tensor::to(DType) src/Tensor.cpp:197-243 (from fp32 only) */
+int co_cast_from_f32(const float* in, void* out, int dtype, long n) {
+    for (long i = 0; i < n; ++i) {
+        switch (dtype) {
+            case 1: ((double*)out)[i] = (double)in[i]; break;
+            case 2: ((int32_t*)out)[i] = f32_to_i32(in[i]); break;
+            case 3: ((int64_t*)out)[i] = f32_to_i64(in[i]); break;
+            case 4: ((unsigned char*)out)[i] = (unsigned char)(in[i] != 0.0f); break;
+            default: return -1;
+        }
+    }
+    return 0;
+}
+
+/* The typed arms of Tensor::operator+(float) src/Tensor.cpp:870-890, operator*(float) :766-786
+ * and operator/(float) :933-953: the scalar is converted to the tensor's type first (an integer
+ * tensor times 2.7f is times 2).  op: 0 '+', 1 '*', 2 '/'.  Integer sums and products wrap (the
+ * machine's two's complement arithmetic); -1 for an integer division by a scalar that converts
+ * to 0, where the reference's process stops with SIGFPE, as it does for the most negative integer
+ * divided by -1, which is stated here as wrapping to itself. */
+int co_scalar_op_typed(const void* in, void* out, int dtype, int op, float s, long n) {
+    if (op < 0 || op > 2) return -1;
+    if (dtype == 1) {
+        const double d = (double)s;
+        for (long i = 0; i < n; ++i) {
+            const double x = ((const double*)in)[i];
+            ((double*)out)[i] = op == 0 ? x + d : op == 1 ? x * d : x / d;
+        }
+    } else if (dtype == 2) {
+        const int32_t k = f32_to_i32(s);
+        if (op == 2 && k == 0) return -1;
+        for (long i = 0; i < n; ++i) {
+            const int32_t x = ((const int32_t*)in)[i];
+            ((int32_t*)out)[i] = op == 0   ? (int32_t)((uint32_t)x + (uint32_t)k)
+                                 : op == 1 ? (int32_t)((uint32_t)x * (uint32_t)k)
+                                 : k == -1 ? (int32_t)(0u - (uint32_t)x)
+                                           : x / k;
+        }
+    } else if (dtype == 3) {
+        const int64_t k = f32_to_i64(s);
+        if (op == 2 && k == 0) return -1;
+        for (long i = 0; i < n; ++i) {
+            const int64_t x = ((const int64_t*)in)[i];
+            ((int64_t*)out)[i] = op == 0   ? (int64_t)((uint64_t)x + (uint64_t)k)
+                                 : op == 1 ? (int64_t)((uint64_t)x * (uint64_t)k)
+                                 : k == -1 ? (int64_t)((uint64_t)0 - (uint64_t)x)
+                                           : x / k;
+        }
+    } else {
+        return -1;
+    }
+    return 0;
+}
+
+/* grad[i] += val[i], the typed arms of src/AutoDiff.cpp:1880-1903 */
+int co_accumulate_typed(void* acc, const void* val, int dtype, long n) {
+    for (long i = 0; i < n; ++i) {
+        switch (dtype) {
+            case 1: ((double*)acc)[i] += ((const double*)val)[i]; break;
+            case 2: ((int32_t*)acc)[i] = (int32_t)((uint32_t)((int32_t*)acc)[i] + (uint32_t)((const int32_t*)val)[i]); break;
+            case 3: ((int64_t*)acc)[i] = (int64_t)((uint64_t)((int64_t*)acc)[i] + (uint64_t)((const int64_t*)val)[i]); break;
+            default: return -1;
+        }
+    }
+    return 0;
+}
+
+/* Tensor::softmax(dim) for double: src/Tensor.cpp:1686-1696 (1-D: rows = 1, dim = 1), :1749-1764
+ * (dim 1), :1765-1781 (dim 0): first maximum, e = exp(x - max) stored, sequential sum, division. */
+void co_softmax_f64(const double* x, double* y, long rows, long cols, int dim) {
+    const long lines = dim == 1 ? rows : cols, len = dim == 1 ? cols : rows;
+    const long step = dim == 1 ? 1 : cols, line_step = dim == 1 ? cols : 1;
+    for (long l = 0; l < lines; ++l) {
+        const double* in = x + l * line_step;
+        double* out = y + l * line_step;
+        double m = in[0];
+        for (long k = 1; k < len; ++k)
+            if (in[k * step] > m) m = in[k * step];
+        double sum = 0.0;
+        for (long k = 0; k < len; ++k) {
+            const double e = exp(in[k * step] - m);
+            out[k * step] = e;
+            sum += e;
+        }
+        for (long k = 0; k < len; ++k) out[k * step] /= sum;
     }
 }
 

@@ -81,6 +81,10 @@ void co_fill_normal(float* r, long n, uint64_t seed, double mean, double sigma);
 void co_fill_int(float* r, long n, uint64_t seed, long range);
 
 void co_compare(int cmp, const float* a, const float* b, float s, unsigned char* out, long n);
+int co_cast_from_f32(const float* in, void* out, int dtype, long n);
+int co_scalar_op_typed(const void* in, void* out, int dtype, int op, float s, long n);
+int co_accumulate_typed(void* acc, const void* val, int dtype, long n);
+void co_softmax_f64(const double* x, double* y, long rows, long cols, int dim);
 
 /* extension: a straight-line per-element program of the operators above (see the .c file) */
 int co_expr_run(const int* prog, const float* imm, int n, const float* const* in, int n_in, float* const* out, int n_out,

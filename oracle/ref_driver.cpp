@@ -124,6 +124,69 @@ long ref_softmax(const float* a, const long* ad, int an, int dim, float* out) {
     }
 }
 
+// Tensors that are not fp32.  The fp32 input goes through the reference's Tensor::to(dtype)
+// (dtype in the order of enum DType), then through `n_steps` operations in order, step k being
+// whats[k] with scalars[k]: 0 '+ s', 1 '* s', 2 '/ s', 3 zero(), 4 ones(), 5 softmax(dim = (int)s).
+// The result's bytes are copied to `out`; returns its element count.
+long ref_typed(const float* a, const long* ad, int an, int dtype, const int* whats, const float* scalars, int n_steps,
+               void* out) {
+    try {
+        Tensor t = make(a, ad, an).to(static_cast<DType>(dtype));
+        for (int k = 0; k < n_steps; ++k) {
+            const float s = scalars[k];
+            switch (whats[k]) {
+                case 0: t = t + s; break;
+                case 1: t = t * s; break;
+                case 2: t = t / s; break;
+                case 3: t.zero(); break;
+                case 4: t.ones(); break;
+                case 5: t = t.softmax(static_cast<int>(s)); break;
+                default: return -3;
+            }
+        }
+        const size_t n = t.numel();
+        switch (t.dtype()) {
+            case DType::kFloat: std::memcpy(out, t.data<float>(), n * sizeof(float)); break;
+            case DType::kDouble: std::memcpy(out, t.data<double>(), n * sizeof(double)); break;
+            case DType::kInt: std::memcpy(out, t.data<int32_t>(), n * sizeof(int32_t)); break;
+            case DType::kLong: std::memcpy(out, t.data<int64_t>(), n * sizeof(int64_t)); break;
+            case DType::kBool: std::memcpy(out, t.storage().data<bool>(), n * sizeof(bool)); break;   // Tensor::data<bool> is not instantiated
+        }
+        return static_cast<long>(n);
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
+// The tape through scalar operators on a tensor that is not fp32: x = to(dtype) of the input,
+// y = x through the steps (0 '+ s', 1 '* s', 2 '/ s'), backward(y), grad(x).  The gradient's
+// dtype code goes to *grad_dtype and its bytes to grad_out; returns its element count.
+long ref_typed_grad(const float* a, const long* ad, int an, int dtype, const int* whats, const float* scalars, int n_steps,
+                    void* grad_out, int* grad_dtype) {
+    try {
+        AutoDiff ctx;
+        AutoDiffContext::Guard guard(&ctx);
+        Tensor x = make(a, ad, an).to(static_cast<DType>(dtype));
+        x.requires_grad(true);
+        Tensor y = whats[0] == 0 ? x + scalars[0] : whats[0] == 1 ? x * scalars[0] : x / scalars[0];
+        for (int k = 1; k < n_steps; ++k) y = whats[k] == 0 ? y + scalars[k] : whats[k] == 1 ? y * scalars[k] : y / scalars[k];
+        backward(y);
+        Tensor g = grad(x);
+        *grad_dtype = static_cast<int>(g.dtype());
+        const size_t n = g.numel();
+        switch (g.dtype()) {
+            case DType::kFloat: std::memcpy(grad_out, g.data<float>(), n * sizeof(float)); break;
+            case DType::kDouble: std::memcpy(grad_out, g.data<double>(), n * sizeof(double)); break;
+            case DType::kInt: std::memcpy(grad_out, g.data<int32_t>(), n * sizeof(int32_t)); break;
+            case DType::kLong: std::memcpy(grad_out, g.data<int64_t>(), n * sizeof(int64_t)); break;
+            default: return -3;
+        }
+        return static_cast<long>(n);
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
 // C = op(A) * op(B) with op = the reference's t() (deep copy + stride swap) when the flag is set.
 // A is stored [am, ak] row-major; ta != 0 multiplies by its transpose, likewise B.
 long ref_matmul_t(const float* a, long ar, long ac, int ta, const float* b, long br, long bc, int tb,

@@ -107,6 +107,20 @@ def mnist():
     np.savez_compressed(os.path.join(HERE, "mnist.npz"), **g)
 
 
+def typed():
+    """Tensors that are not fp32 (support.typed_cases): the reference's Tensor::to, zero / ones, scalar
+    operators and double softmax; only the outputs are stored, the inputs come from the seeded generator."""
+    from support import typed_cases
+    o = Oracle()
+    r = Reference()
+    g = {}
+    for name, a, dt, steps in typed_cases(o):
+        rc, out = r.typed(a, dt, steps)
+        assert rc == a.size, (name, rc)
+        g[name] = out
+    np.savez_compressed(os.path.join(HERE, "typed.npz"), **g)
+
+
 def main():
     o = Oracle()   # only for its input generator
     r = Reference()
@@ -265,7 +279,10 @@ if __name__ == "__main__":
         mnist()
     elif "programs" in sys.argv[1:]:
         programs()
+    elif "typed" in sys.argv[1:]:
+        typed()
     else:
         main()
         mnist()
         programs()
+        typed()

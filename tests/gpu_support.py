@@ -223,3 +223,38 @@ def expr_run(prog, inputs, n_out, rows, cols, expect=0):
     rc = lib().ctamd_expr_run_f32(arr, len(prog), pin, len(inputs), pout, n_out, ptr(status), rows, cols, stream())
     assert rc == expect, (rc, lib().ctamd_last_error().decode())
     return outs, int(status.cpu()[0])
+
+
+# ----------------------------------------------------------------- tensors that are not fp32
+DT_F32, DT_F64, DT_I32, DT_I64, DT_BOOL = range(5)
+TORCH_DTYPE = {DT_F32: torch.float32, DT_F64: torch.float64, DT_I32: torch.int32, DT_I64: torch.int64, DT_BOOL: torch.uint8}
+
+
+def fill_typed(dtype, value, n):
+    r = torch.empty(n, dtype=TORCH_DTYPE[dtype], device=DEV)
+    call("ctamd_fill_typed", ptr(r), dtype, C.c_double(value), n, stream())
+    return r
+
+
+def cast_from_f32(x, dtype):
+    r = torch.empty(x.shape, dtype=TORCH_DTYPE[dtype], device=DEV)
+    call("ctamd_cast_from_f32", ptr(x), ptr(r), dtype, x.numel(), stream())
+    return r
+
+
+def scalar_op_typed(x, dtype, op, s):
+    r = torch.empty_like(x)
+    call("ctamd_scalar_op_typed", ptr(x), ptr(r), dtype, op, C.c_float(s), x.numel(), stream())
+    return r
+
+
+def accumulate_typed(acc, val, dtype):
+    call("ctamd_accumulate_typed", ptr(acc), ptr(val), dtype, acc.numel(), stream())
+    return acc
+
+
+def softmax_f64(x, dim):
+    r = torch.empty_like(x)
+    rows, cols = (1, x.numel()) if x.dim() == 1 else x.shape
+    call("ctamd_softmax_f64", ptr(x), ptr(r), rows, cols, 1 if x.dim() == 1 else dim, stream())
+    return r

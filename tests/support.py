@@ -22,6 +22,9 @@ ADD, SUB, MUL, DIV, MATMUL, DOT, MSE, MAE, CE = range(9)
 NEG, RELU, SIN, COS, TANH, SIGMOID, SOFTMAX_KERNEL = range(20, 27)
 
 
+NP_DTYPE = {0: np.float32, 1: np.float64, 2: np.int32, 3: np.int64, 4: np.uint8}
+
+
 def f32(a):
     return np.ascontiguousarray(a, dtype=np.float32)
 
@@ -310,6 +313,54 @@ class Oracle:
         self.lib.co_compare(C.c_int(cmp), fp(a), fp(f32(b)) if b is not None else None, C.c_float(s),
                             out.ctypes.data_as(C.c_void_p), C.c_long(a.size))
         return out
+
+    # ---- tensors that are not fp32 (dtype codes: 1 double, 2 int32, 3 int64, 4 bool)
+    def cast_from_f32(self, a, dtype):
+        a = f32(a)
+        out = np.empty(a.shape, NP_DTYPE[dtype])
+        rc = self.lib.co_cast_from_f32(fp(a), out.ctypes.data_as(C.c_void_p), C.c_int(dtype), C.c_long(a.size))
+        assert rc == 0
+        return out
+
+    def scalar_op_typed(self, x, dtype, op, s):
+        """op: 0 '+', 1 '*', 2 '/'; returns None where the reference's process would stop (integer division by 0)."""
+        x = np.ascontiguousarray(x, NP_DTYPE[dtype])
+        out = np.empty_like(x)
+        rc = self.lib.co_scalar_op_typed(x.ctypes.data_as(C.c_void_p), out.ctypes.data_as(C.c_void_p), C.c_int(dtype), C.c_int(op),
+                                         C.c_float(s), C.c_long(x.size))
+        return out if rc == 0 else None
+
+    def accumulate_typed(self, acc, val, dtype):
+        acc = np.array(acc, NP_DTYPE[dtype])
+        val = np.ascontiguousarray(val, NP_DTYPE[dtype])
+        rc = self.lib.co_accumulate_typed(acc.ctypes.data_as(C.c_void_p), val.ctypes.data_as(C.c_void_p), C.c_int(dtype), C.c_long(acc.size))
+        assert rc == 0
+        return acc
+
+    def softmax_f64(self, x, dim):
+        x = np.ascontiguousarray(x, np.float64)
+        out = np.empty_like(x)
+        rows, cols = (1, x.size) if x.ndim == 1 else x.shape
+        self.lib.co_softmax_f64(x.ctypes.data_as(C.c_void_p), out.ctypes.data_as(C.c_void_p), C.c_long(rows), C.c_long(cols),
+                                C.c_int(1 if x.ndim == 1 else dim))
+        return out
+
+    def typed(self, a, dtype, steps):
+        """The fp32 array converted to dtype, then the steps [(what, scalar)] in order: 0 '+', 1 '*', 2 '/',
+        3 zero(), 4 ones(), 5 softmax(dim = scalar).  None where a step has no defined result."""
+        t = self.cast_from_f32(a, dtype)
+        for what, s in steps:
+            if what <= 2:
+                t = self.scalar_op_typed(t, dtype, what, s)
+                if t is None:
+                    return None
+            elif what == 3:
+                t = np.zeros_like(t)
+            elif what == 4:
+                t = np.ones_like(t)
+            else:
+                t = self.softmax_f64(t, int(s))
+        return t
 
     def expr_run(self, prog, inputs, n_out, rows, cols):
         """prog: [(op, dst, a, b, imm)] of the fused-expression opcodes; inputs: full [rows, cols] or
@@ -604,7 +655,7 @@ class Reference:
     same shape, so the methods here serve both."""
 
     ENTRY_POINTS = ("binary", "unary", "scalar", "sum", "softmax", "matmul_t", "grad_unary", "grad_softmax",
-                    "grad_binary", "grad_loss", "chain", "mlp_step", "expr")
+                    "grad_binary", "grad_loss", "chain", "mlp_step", "expr", "typed", "typed_grad")
 
     def __init__(self, path=None, prefix="ref_"):
         cdll = C.CDLL(path or os.path.join(ORACLE_DIR, "_ref", "libctorch_ref.so"))
@@ -636,6 +687,31 @@ class Reference:
         out = np.empty_like(a)
         rc = self.lib.ref_scalar(which, fp(a), ad, an, C.c_float(s), fp(out))
         return rc, out
+
+    def typed(self, a, dtype, steps):
+        """The fp32 array converted by Tensor::to(dtype), then the steps [(what, scalar)] in order (see
+        Oracle.typed); returns (rc, result)."""
+        a = f32(a)
+        ad, an = _dims(a.shape)
+        out = np.empty(a.shape, NP_DTYPE[dtype])
+        whats = (C.c_int * max(1, len(steps)))(*[w for w, _ in steps])
+        scalars = (C.c_float * max(1, len(steps)))(*[s for _, s in steps])
+        rc = self.lib.ref_typed(fp(a), ad, C.c_int(an), C.c_int(dtype), whats, scalars, C.c_int(len(steps)),
+                                out.ctypes.data_as(C.c_void_p))
+        return rc, out
+
+    def typed_grad(self, a, dtype, steps):
+        """backward() through scalar operators ([(what, scalar)], 0 '+', 1 '*', 2 '/') on to(dtype) of a:
+        returns (rc, dtype code of the gradient, its bytes)."""
+        a = f32(a)
+        ad, an = _dims(a.shape)
+        out = np.zeros(a.size * 8, np.uint8)
+        code = C.c_int(-1)
+        whats = (C.c_int * len(steps))(*[w for w, _ in steps])
+        scalars = (C.c_float * len(steps))(*[s for _, s in steps])
+        rc = self.lib.ref_typed_grad(fp(a), ad, C.c_int(an), C.c_int(dtype), whats, scalars, C.c_int(len(steps)),
+                                     out.ctypes.data_as(C.c_void_p), C.byref(code))
+        return rc, code.value, out
 
     def sum(self, a):
         a = f32(a)
@@ -906,3 +982,35 @@ class HostLayer(Reference):
                                       C.c_int(hidden1), C.c_int(hidden2), C.c_int(int(reference_tape)), fp(losses),
                                       fp(acc), C.byref(sec))
         return rc, losses, acc, sec.value
+
+
+# ----------------------------------------------------------------- tensors that are not fp32
+TYPED_EDGE = np.array([0.0, -0.0, 1.5, -1.5, 2.9, -2.9, 3e9, -3e9, 1e19, -1e19, np.nan, np.inf, -np.inf, 2147483520.0,
+                       -2147483648.0, 2147483648.0, 9.2233715e18, 9.223372e18, -9.223372e18, 1e-40, 0.99, -0.99, 16777216.0,
+                       1e10, -1e10, 255.0, 1.0], np.float32)
+
+
+def typed_cases(o):
+    """[(name, fp32 input, dtype, steps)] for Oracle.typed / Reference.typed: conversions of edge values,
+    every scalar operator on every arithmetic dtype (scalars that truncate, wrap and change sign), zero / ones,
+    and the double softmax along both dimensions."""
+    cases = []
+    wide = np.concatenate([TYPED_EDGE, o.normal((997,), 71, 0, 1000), o.normal((300,), 72, 0, 3e9)]).astype(np.float32)
+    for dt in (1, 2, 3, 4):
+        cases.append(("cast_%d" % dt, wide, dt, []))
+        cases.append(("zero_%d" % dt, wide[:37], dt, [(3, 0.0)]))
+        cases.append(("ones_%d" % dt, wide[:37], dt, [(4, 0.0)]))
+    vals = o.normal((1031,), 73, 0, 40000)
+    scalars = [(0, 2.7), (0, -1e10), (0, 3e9), (1, -3.9), (1, 1e6), (1, 0.3), (1, 123456.0), (2, 2.5), (2, -1.0), (2, -7.9), (2, 1e-3),
+               (2, 3e9)]
+    for dt in (1, 2, 3):
+        for k, (what, sc) in enumerate(scalars):
+            if dt != 1 and what == 2 and abs(sc) < 1:
+                continue                               # integer division by 0: the reference's process stops
+            cases.append(("scalar_%d_%d" % (dt, k), vals, dt, [(what, sc)]))
+        cases.append(("chain_%d" % dt, vals, dt, [(1, 3.0), (0, -17.5), (2, 4.0), (1, 65537.0), (1, 65537.0), (0, 1.0)]))
+    for shape, seed in (((37, 19), 74), ((5, 301), 75), ((64,), 76), ((1, 1), 77), ((130, 3), 78)):
+        z = o.normal(shape, seed, 0, 3)
+        for dim in ((0,) if len(shape) == 1 else (0, 1)):
+            cases.append(("softmax_%s_%d" % ("x".join(map(str, shape)), dim), z, 1, [(1, 1.0000001), (0, 0.1), (5, float(dim))]))
+    return cases

@@ -331,6 +331,32 @@ def test_comparison_operators(oracle, host):
     assert host.compare(0, a, b[:, :32].copy()) == -1
 
 
+def test_tensors_that_are_not_fp32(oracle, host, golden):
+    """Tensor::to(dtype), zero / ones, tensor (+ * /) float and the double softmax through the front-end,
+    against the reference's vectors (bytes equal; the softmax to the bound of test_gpu_typed.py);
+    backward() over a typed tensor throws, as it does in the reference."""
+    from support import typed_cases
+    from test_gpu_typed import check_softmax
+    print("case host typed", flush=True)
+    g = golden("typed")
+    for name, a, dt, steps in typed_cases(oracle):
+        rc, got = host.typed(a, dt, steps)
+        assert rc == a.size, (name, rc)
+        if name.startswith("softmax"):
+            x = oracle.typed(a, dt, steps[:-1])
+            check_softmax(got, g[name], x, 0 if x.ndim == 1 else int(steps[-1][1]))
+        else:
+            assert np.array_equal(got.view(np.uint8), g[name].view(np.uint8)), name
+    x = oracle.normal((2, 3), 5, 0, 10)
+    for dt in (1, 2, 3):
+        for steps in ([(0, 5.0)], [(1, 3.0)], [(1, 3.0), (0, 5.0)], [(2, 4.0)]):
+            assert host.typed_grad(x, dt, steps)[0] == -1, (dt, steps)
+    rc, code, raw = host.typed_grad(x, 0, [(1, 3.0), (0, 5.0)])
+    assert rc == 6 and code == 0 and np.array_equal(raw.view(np.float32)[:6], np.full(6, 3.0, np.float32))
+    # an integer division the reference's process would not survive is an exception here
+    assert host.typed(x, 2, [(2, 0.5)])[0] == -1
+
+
 def test_fused_expression_in_a_recorded_step(oracle, host):
     """A fused expression, its losses and its backward recorded into a HIP graph: the first replay
     reproduces the eager step bit for bit, a replay after the staged input was overwritten equals

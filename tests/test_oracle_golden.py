@@ -242,3 +242,38 @@ def test_comparisons_are_the_ieee_predicates(oracle):
     for cmp, fn in enumerate(fns):
         assert np.array_equal(oracle.compare(cmp, a, b), fn(a, b).astype(np.uint8)), cmp
         assert np.array_equal(oracle.compare(cmp, a, None, 1.0), fn(a, np.float32(1.0)).astype(np.uint8)), cmp
+
+
+def test_tensors_that_are_not_fp32(oracle, golden):
+    """Conversion from fp32, zero / ones, the scalar operators and the double softmax of double, int32,
+    int64 and bool tensors against the reference's results, byte for byte (edge values included: NaN and
+    out-of-range conversions, products and sums that wrap, scalars that truncate)."""
+    from support import typed_cases
+    g = golden("typed")
+    cases = typed_cases(oracle)
+    assert len(cases) == len(g.files)
+    for name, a, dt, steps in cases:
+        got = oracle.typed(a, dt, steps)
+        assert got is not None, name
+        want = g[name]
+        assert got.dtype == want.dtype and got.shape == want.shape, name
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), name
+
+
+def test_typed_accumulation_and_refused_division(oracle):
+    """co_accumulate_typed against the closed forms (IEEE double addition, two's complement wrap), and the
+    integer division the reference cannot survive is refused."""
+    rng = np.random.default_rng(5)
+    a = rng.standard_normal(1000)
+    b = rng.standard_normal(1000)
+    assert np.array_equal(oracle.accumulate_typed(a, b, 1), a + b)
+    for dt, t in ((2, np.int32), (3, np.int64)):
+        info = np.iinfo(t)
+        x = rng.integers(info.min, info.max, 1000, dtype=t)
+        y = rng.integers(info.min, info.max, 1000, dtype=t)
+        with np.errstate(over="ignore"):
+            assert np.array_equal(oracle.accumulate_typed(x, y, dt), x + y)
+        assert oracle.scalar_op_typed(x, dt, 2, 0.5) is None
+        assert oracle.scalar_op_typed(x, dt, 2, -0.99) is None
+        lowest = np.array([info.min, info.min + 1, -1, 0, 7], t)
+        assert np.array_equal(oracle.scalar_op_typed(lowest, dt, 2, -1.0), np.array([info.min, info.max, 1, 0, -7], t))

@@ -128,3 +128,20 @@ def test_configurations(oracle, ref):
     R = np.broadcast_to(rv, X.shape).copy()
     for got, want in zip(oracle.expr(X, R, T), ref.expr(X, R, T)):
         eq(got, want)
+
+
+def test_tensors_that_are_not_fp32(oracle, ref):
+    """The typed cases live against the reference (the committed vectors are these results), and the
+    fact the front-end relies on: backward() through a double / int tensor throws in the reference."""
+    from support import typed_cases
+    for name, a, dt, steps in typed_cases(oracle):
+        rc, want = ref.typed(a, dt, steps)
+        assert rc == a.size, name
+        got = oracle.typed(a, dt, steps)
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), name
+    x = oracle.normal((2, 3), 5, 0, 10)
+    for dt in (1, 2, 3):
+        for steps in ([(0, 5.0)], [(1, 3.0)], [(1, 3.0), (0, 5.0)], [(2, 4.0)]):
+            assert ref.typed_grad(x, dt, steps)[0] == -1, (dt, steps)
+    rc, code, raw = ref.typed_grad(x, 0, [(1, 3.0), (0, 5.0)])
+    assert rc == 6 and code == 0 and np.array_equal(raw.view(np.float32)[:6], np.full(6, 3.0, np.float32))
