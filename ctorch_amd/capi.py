@@ -62,6 +62,7 @@ PROTOTYPES.update({
     "ctamd_sgd_step_multi_f32": [_P, _P, _P, C.c_int, C.c_float, _P],
     "ctamd_compare_f32": [C.c_int, _P, _P, _P, _Z, _P],
     "ctamd_compare_scalar_f32": [C.c_int, _P, C.c_float, _P, _Z, _P],
+    "ctamd_cross_entropy_index_fused_f32": [_P, _P, _P, _P, _P, _Z, _Z, _P],
     "ctamd_fill_typed": [_P, C.c_int, C.c_double, _Z, _P],
     "ctamd_cast_from_f32": [_P, _P, C.c_int, _Z, _P],
     "ctamd_scalar_op_typed": [_P, _P, C.c_int, C.c_int, C.c_float, _Z, _P],

@@ -173,7 +173,7 @@ struct Row {
     }
 };
 
-enum Mode { kSoftmax, kCeOnehot, kCeIndex, kCeBwdOnehot, kCeBwdIndex, kSoftmaxBwd };
+enum Mode { kSoftmax, kCeOnehot, kCeIndex, kCeBwdOnehot, kCeBwdIndex, kSoftmaxBwd, kCeIndexBoth };
 
 struct Args {
     const float* x;      // logits / softmax output y (kSoftmaxBwd)
@@ -201,7 +201,7 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
     __shared__ float s_f[2][THREADS / 64 + 1];
     __shared__ double s_d[THREADS / 64 + 1];
     stage_exp_table(s_exp2);
-    constexpr bool kPipelined = (MODE == kSoftmax || MODE == kCeIndex || MODE == kCeBwdIndex);
+    constexpr bool kPipelined = (MODE == kSoftmax || MODE == kCeIndex || MODE == kCeBwdIndex || MODE == kCeIndexBoth);
     double block_loss = 0.0;
     bool block_bad = false;   // a class index out of range was met (thread 0's copy counts)
 
@@ -265,6 +265,36 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
                 p = (p < 1e-10f) ? 1e-10f : p;
                 block_loss -= double(float(log(double(p))));
             }
+        } else if (MODE == kCeIndexBoth) {
+            // loss and gradient from one visit of the row: r holds e = exp(x - m), s is its sum;
+            // the gradient is the one for an upstream gradient of 1 (d * 1.0f is d)
+            // (the class index is read here, not earlier: a wait for it right after the next row's
+            // loads were issued would wait for those as well)
+            const int c = int(a.t[row]);
+            const bool ok = c >= 0 && c < int(a.cols);
+            float ec = 0.0f;
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k)
+#pragma unroll
+                for (int i = 0; i < W; ++i) ec = (ok && r.index(k, i) == unsigned(c)) ? r.v[k][i] : ec;
+            ec = block_sum<THREADS>(ec, s_f[0]);
+            if (!ok) {
+                block_bad = true;
+                block_loss += double(__builtin_nanf(""));
+            } else {
+                float p = ec / s;
+                p = (p < 1e-10f) ? 1e-10f : p;
+                block_loss -= double(float(log(double(p))));
+            }
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k)
+#pragma unroll
+                for (int i = 0; i < W; ++i) {
+                    float sm = cta_div_rcp(r.v[k][i], rcp_s);
+                    float d = sm - ((ok && r.index(k, i) == unsigned(c)) ? 1.0f : 0.0f);
+                    r.v[k][i] = 0.0f + d;
+                }
+            r.store(a.out + row * a.cols, unsigned(a.cols));
         } else {   // kCeBwdOnehot / kCeBwdIndex: dx = 0 + (e / s - t) * g (the tape adds it to a zero-filled buffer)
             const float g = a.g1[0];
             if (MODE == kCeBwdOnehot) {
@@ -345,9 +375,9 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
             process(r, row, r.max());
         }
     }
-    if ((MODE == kCeOnehot || MODE == kCeIndex) && threadIdx.x == 0) {
+    if ((MODE == kCeOnehot || MODE == kCeIndex || MODE == kCeIndexBoth) && threadIdx.x == 0) {
         a.partials[blockIdx.x] = block_loss;
-        if (MODE == kCeIndex && a.status) a.partials[gridDim.x + blockIdx.x] = block_bad ? 1.0 : 0.0;
+        if ((MODE == kCeIndex || MODE == kCeIndexBoth) && a.status) a.partials[gridDim.x + blockIdx.x] = block_bad ? 1.0 : 0.0;
     }
 }
 
@@ -598,7 +628,9 @@ bool launch_resident(const Args& a, unsigned grid, hipStream_t s) {
 
 template <int MODE>
 int run_rows(const char* name, Args a, float* loss_out, void* stream) {
-    constexpr bool kLoss = (MODE == kCeOnehot || MODE == kCeIndex);
+    constexpr bool kLoss = (MODE == kCeOnehot || MODE == kCeIndex || MODE == kCeIndexBoth);
+    constexpr bool kIndexLoss = (MODE == kCeIndex || MODE == kCeIndexBoth);
+    constexpr bool kWrites = !kLoss || MODE == kCeIndexBoth;           // a [rows, cols] result
     if (kLoss && !loss_out) return fail(CTAMD_EINVAL, "%s: null output", name);
     hipStream_t s = as_stream(stream);
     if (a.rows == 0 || a.cols == 0) {
@@ -606,7 +638,7 @@ int run_rows(const char* name, Args a, float* loss_out, void* stream) {
         return CTAMD_OK;
     }
     if (!a.x || (!a.t && MODE != kSoftmax)) return fail(CTAMD_EINVAL, "%s: null input", name);
-    if (!kLoss && !a.out) return fail(CTAMD_EINVAL, "%s: null output", name);
+    if (kWrites && !a.out) return fail(CTAMD_EINVAL, "%s: null output", name);
     if ((MODE == kCeBwdOnehot || MODE == kCeBwdIndex) && !a.g1) return fail(CTAMD_EINVAL, "%s: null upstream gradient", name);
     if (a.rows > (size_t(1) << 62) / a.cols) return fail(CTAMD_ERANGE, "%s: rows*cols overflows", name);
     if (a.cols > size_t(0x7fffffff)) return fail(CTAMD_ERANGE, "%s: more than 2^31-1 columns", name);
@@ -618,8 +650,8 @@ int run_rows(const char* name, Args a, float* loss_out, void* stream) {
         // index adds 4 bytes per row; one exp per element
         const double n = double(a.rows) * double(a.cols);
         const double per = MODE == kSoftmax ? 8.0 : MODE == kCeIndex ? 4.0 : MODE == kCeOnehot ? 8.0
-                         : MODE == kCeBwdIndex ? 8.0 : 12.0;   // kCeBwdOnehot, kSoftmaxBwd: two inputs, one output
-        const bool index = (MODE == kCeIndex || MODE == kCeBwdIndex);
+                         : (MODE == kCeBwdIndex || MODE == kCeIndexBoth) ? 8.0 : 12.0;   // kCeBwdOnehot, kSoftmaxBwd: two inputs, one output
+        const bool index = (MODE == kCeIndex || MODE == kCeBwdIndex || MODE == kCeIndexBoth);
         account(per * n + (index ? 4.0 * double(a.rows) : 0.0), n);
     }
     if (kLoss) a.partials = reinterpret_cast<double*>(scratch());
@@ -630,8 +662,9 @@ int run_rows(const char* name, Args a, float* loss_out, void* stream) {
     if (fill > kMaxRowBlocks) fill = kMaxRowBlocks;
     if (kLoss && fill > 2048) fill = 2048;         // one partial per block: keep the fold of the partials short
     unsigned grid = a.rows < fill ? unsigned(a.rows) : unsigned(fill);
-    bool vec = (a.cols % 4 == 0) && aligned16(a.x) && (MODE == kSoftmax || MODE == kCeIndex || MODE == kCeBwdIndex || aligned16(a.t)) &&
-               (kLoss || aligned16(a.out));
+    bool vec = (a.cols % 4 == 0) && aligned16(a.x) &&
+               (MODE == kSoftmax || MODE == kCeIndex || MODE == kCeBwdIndex || MODE == kCeIndexBoth || aligned16(a.t)) &&
+               (!kWrites || aligned16(a.out));
     if (MODE == kCeIndex && a.cols >= 2048) {
         size_t fill_online = size_t(compute_units() > 0 ? compute_units() : 256) * 8;
         grid = a.rows < fill_online ? unsigned(a.rows) : unsigned(fill_online);
@@ -643,11 +676,17 @@ int run_rows(const char* name, Args a, float* loss_out, void* stream) {
         return launched(name);
     }
     bool done = vec ? launch_resident<MODE, 4>(a, grid, s) : launch_resident<MODE, 1>(a, grid, s);
-    if (!done) hipLaunchKernelGGL((row_stream_kernel<MODE>), dim3(grid), dim3(1024), 0, s, a);
+    if (!done) {
+        if constexpr (MODE == kCeIndexBoth)
+            return fail(CTAMD_ERANGE, "%s: a row does not fit a block's registers (32768 columns, 8192 without 128-bit accesses): "
+                        "use the separate forward and backward entry points", name);
+        else
+            hipLaunchKernelGGL((row_stream_kernel<MODE>), dim3(grid), dim3(1024), 0, s, a);
+    }
     int rc = launched(name);
     if (rc) return rc;
     if (kLoss) {
-        hipLaunchKernelGGL(loss_stage2, dim3(1), dim3(256), 0, s, a.partials, grid, loss_out, MODE == kCeIndex ? a.status : nullptr);
+        hipLaunchKernelGGL(loss_stage2, dim3(1), dim3(256), 0, s, a.partials, grid, loss_out, kIndexLoss ? a.status : nullptr);
         rc = launched(name);
     }
     return rc;
@@ -931,6 +970,11 @@ int ctamd_cross_entropy_index_stats_f32(const float* x, const float* idx, float*
                                         size_t rows, size_t cols, void* stream) {
     Args a{x, idx, nullptr, nullptr, nullptr, status, stats, rows, cols, nullptr, nullptr};
     return run_rows<kCeIndex>(__func__, a, out, stream);
+}
+int ctamd_cross_entropy_index_fused_f32(const float* x, const float* idx, float* out, int32_t* status, float* dx, size_t rows,
+                                        size_t cols, void* stream) {
+    Args a{x, idx, nullptr, dx, nullptr, status, nullptr, rows, cols, nullptr, nullptr};
+    return run_rows<kCeIndexBoth>(__func__, a, out, stream);
 }
 int ctamd_cross_entropy_backward_onehot_f32(const float* x, const float* t, const float* g1, float* dx, size_t rows,
                                             size_t cols, void* stream) {

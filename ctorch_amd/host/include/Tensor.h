@@ -69,6 +69,7 @@ class Tensor {
     static Tensor view_element(const Tensor& t, size_t index);
     void set_known_value(float v) { _known_value = std::make_shared<const float>(v); }
     void forget_known_value() { _known_value.reset(); }
+    const float* known_value() const { return _known_value.get(); }   // null when the host does not know it
     // a tensor on `device` filled from host memory
     static Tensor from_host(const float* data, const std::vector<size_t>& shape, DeviceType device);
 

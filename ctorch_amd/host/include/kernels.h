@@ -38,6 +38,11 @@ Tensor scalar_op(const Tensor& a, float s, op which);
 // a (cmp) b or, with b == nullptr, a (cmp) s: a bool tensor; cmp is a CTAMD_CMP_* code
 Tensor compare_op(int cmp, const Tensor& a, const Tensor* b, float s);                 // a + s, a * s, a / s
 Tensor sum_all(const Tensor& a);
+// Class-index cross entropy under a tape whose logits need a gradient computes loss and gradient in
+// one pass over the logits and keeps the gradient for backward() (default on; off: a forward pass
+// that leaves row statistics, and a streaming backward pass).
+void set_ce_one_pass(bool on);
+bool ce_one_pass();
 // tensors that are not fp32 (the typed arms of src/Tensor.cpp:197-243, :390-448)
 void fill_typed(void* device_ptr, DType dtype, double v, size_t n);    // zero() / ones() of any dtype, device memory
 Tensor cast_from_float(const Tensor& a, DType to);                    // Tensor::to(DType)

@@ -31,7 +31,10 @@ Tensor::Tensor(float value, DeviceType device)
     : tensor_id_(global_tensor_id++), _device(device),
       _storage(device == DeviceType::kAMD ? Storage(1, DType::kFloat, device) : Storage(&value, 1, DType::kFloat, device)) {
     computeStrides();
-    if (device == DeviceType::kAMD) fill_scalar(*this, value);
+    if (device == DeviceType::kAMD) {
+        fill_scalar(*this, value);
+        set_known_value(value);      // the host just chose it
+    }
 }
 
 Tensor::Tensor(std::initializer_list<float> values)

@@ -106,6 +106,9 @@ static int g_fused_expr = 0;
 // the elementwise parts of cth_chain, cth_expr, cth_program and their timed versions are built as
 // one fused expression (Expr::eval: one launch forward, one backward) when set
 void cth_set_fused_expr(int on) { g_fused_expr = on; }
+// class-index cross entropy under a tape: loss and gradient in one pass over the logits (default), or
+// a forward pass that leaves row statistics and a streaming backward pass
+void cth_set_ce_one_pass(int on) { ctorch_amd_host::set_ce_one_pass(on != 0); }
 // sizes of the programs the last Expr::eval() compiled: out[0..3] = forward instructions, forward
 // slots, backward instructions, backward slots (zeros: evaluated operator by operator)
 void cth_last_expr_stats(int* out) {
@@ -325,6 +328,10 @@ long cth_grad_loss(int code, const float* p, const long* pd, int pn, const float
         Tensor l = run_binary(code, tp, tt);
         if (l.numel() == 0) return -2;
         loss_out[0] = l.item<float>();
+        if (scale == 1.0f) {          // the loss itself is the root: its upstream gradient is the seed
+            backward(l);
+            return emit(grad(tp), dp);
+        }
         Tensor root = l * scale;
         backward(root);
         return emit(grad(tp), dp);

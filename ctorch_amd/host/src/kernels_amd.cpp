@@ -5,6 +5,8 @@
 // label-range flag).
 #include "kernels.h"
 
+#include "AutoDiff.h"
+
 #include "ctorch_amd.h"
 
 namespace ctorch_amd_host {
@@ -101,10 +103,7 @@ void rows_cols(const Tensor& a, size_t& rows, size_t& cols) {
     else { rows = a.sizes()[0]; cols = a.sizes()[1]; }
 }
 
-}  // namespace
-
-// ------------------------------------------------------------------ helpers for Tensor / tape
-namespace {
+// a contiguous device tensor of any dtype
 void check_on_device(const Tensor& a, const char* who) {
     if (a.device() != DeviceType::kAMD)
         Ctorch_Error::throwException(DeviceTypeToErrorPlatform(a.device()), ErrorType::DEVICE_COMPAT,
@@ -112,7 +111,14 @@ void check_on_device(const Tensor& a, const char* who) {
     if (!a.is_contiguous())
         Ctorch_Error::throwException(kP, ErrorType::TENSOR_STATE, std::string(who) + ": a contiguous tensor is needed");
 }
+
+bool g_ce_one_pass = true;
+
 }  // namespace
+
+// ------------------------------------------------------------------ helpers for Tensor / tape
+void set_ce_one_pass(bool on) { g_ce_one_pass = on; }
+bool ce_one_pass() { return g_ce_one_pass; }
 
 void fill_typed(void* device_ptr, DType dtype, double v, size_t n) {
     run(ctamd_fill_typed(device_ptr, int(dtype), v, n, current_stream()), "zero / ones");
@@ -352,27 +358,36 @@ Tensor mae_backward(const Tensor& p, const Tensor& t, const Tensor& g) {
     return r;
 }
 namespace {
-// Per-row (max, sum) left by the class-index CrossEntropy forward, for its backward: keyed by the
-// ids of the logits and target tensors (ids are never re-used), a handful of entries, oldest out.
+// What the class-index CrossEntropy forward leaves for its backward: per-row (max, sum), or - when
+// loss and gradient were computed in one pass - the gradient for an upstream gradient of 1.  Keyed
+// by the ids of the logits and target tensors (ids are never re-used), a handful of entries,
+// oldest out; a kept gradient is handed out once and leaves the table with it.
 struct CeStats {
     size_t logits_id = 0, target_id = 0;
     Tensor stats;
+    Tensor grad;
 };
 constexpr int kCeStatsSlots = 4;
 thread_local CeStats t_ce_stats[kCeStatsSlots];
 thread_local int t_ce_next = 0;
-
-void remember_ce_stats(const Tensor& logits, const Tensor& target, Tensor stats) {
+void remember_ce(const Tensor& logits, const Tensor& target, Tensor stats, Tensor grad) {
     CeStats& slot = t_ce_stats[t_ce_next];
     t_ce_next = (t_ce_next + 1) % kCeStatsSlots;
     slot.logits_id = logits.id();
     slot.target_id = target.id();
     slot.stats = std::move(stats);
+    slot.grad = std::move(grad);
 }
-const Tensor* recall_ce_stats(const Tensor& logits, const Tensor& target) {
-    for (const CeStats& c : t_ce_stats)
-        if (c.logits_id == logits.id() && c.target_id == target.id() && c.logits_id != 0) return &c.stats;
+CeStats* recall_ce(const Tensor& logits, const Tensor& target) {
+    for (CeStats& c : t_ce_stats)
+        if (c.logits_id == logits.id() && c.target_id == target.id() && c.logits_id != 0) return &c;
     return nullptr;
+}
+// rows the one-pass kernel keeps in registers: 32768 columns with 128-bit accesses, else 8192
+bool ce_row_fits(const Tensor& logits) {
+    const size_t cols = logits.sizes()[1];
+    const bool vec = cols % 4 == 0 && (reinterpret_cast<uintptr_t>(logits.fptr()) & 15u) == 0;
+    return cols <= (vec ? size_t(32768) : size_t(8192));
 }
 }  // namespace
 
@@ -382,19 +397,29 @@ Tensor cross_entropy_backward(const Tensor& x, const Tensor& target, const Tenso
         Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "cross_entropy_backward: logits must be 1-D or 2-D");
     size_t rows, cols;
     rows_cols(x, rows, cols);
-    Tensor r = like(x);
-    if (x.sizes() == target.sizes())
+    if (x.sizes() == target.sizes()) {
+        Tensor r = like(x);
         run(ctamd_cross_entropy_backward_onehot_f32(x.fptr(), target.fptr(), g.fptr(), r.fptr(), rows, cols, current_stream()), "cross_entropy_backward");
-    else if (target.dim() == 1 && x.dim() == 2 && target.sizes()[0] == rows) {
-        // with the forward pass's row statistics at hand the backward pass needs no reductions
-        if (const Tensor* stats = recall_ce_stats(x, target))
-            run(ctamd_cross_entropy_backward_index_stats_f32(x.fptr(), target.fptr(), stats->fptr(), g.fptr(), r.fptr(), rows,
-                                                             cols, current_stream()), "cross_entropy_backward");
-        else
-            run(ctamd_cross_entropy_backward_index_f32(x.fptr(), target.fptr(), g.fptr(), r.fptr(), rows, cols, current_stream()), "cross_entropy_backward");
+        return r;
     }
-    else
+    if (!(target.dim() == 1 && x.dim() == 2 && target.sizes()[0] == rows))
         Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "cross_entropy_backward: target shape not understood");
+    CeStats* kept = recall_ce(x, target);
+    if (kept && !kept->grad.is_cleared()) {
+        // the forward pass already formed softmax - onehot: for an upstream gradient of 1 (a loss that
+        // is the root of backward()) that is the gradient, d * 1.0f being d.  Handed out once.
+        Tensor d = std::move(kept->grad);
+        kept->grad = Tensor();
+        kept->logits_id = 0;
+        if (g.known_value() && *g.known_value() == 1.0f) return d;
+        kept = nullptr;
+    }
+    Tensor r = like(x);
+    if (kept && !kept->stats.is_cleared())   // with the forward pass's row statistics the backward pass needs no reductions
+        run(ctamd_cross_entropy_backward_index_stats_f32(x.fptr(), target.fptr(), kept->stats.fptr(), g.fptr(), r.fptr(), rows, cols,
+                                                         current_stream()), "cross_entropy_backward");
+    else
+        run(ctamd_cross_entropy_backward_index_f32(x.fptr(), target.fptr(), g.fptr(), r.fptr(), rows, cols, current_stream()), "cross_entropy_backward");
     return r;
 }
 Tensor div_backward_b(const Tensor& a, const Tensor& b, const Tensor& g) {
@@ -479,11 +504,19 @@ Tensor CrossEntropy_AMD_kernel(const Tensor& a, const Tensor& b) {
         // returns an empty Tensor), so it fetches the loss in the same transfer and item() is free
         Tensor pair(ShapeTag{}, {2}, DType::kFloat, DeviceType::kAMD, false);
         Tensor r = Tensor::view_element(pair, 0);
-        Tensor stats(ShapeTag{}, {a.sizes()[0], 2}, DType::kFloat, DeviceType::kAMD, false);
-        run(ctamd_cross_entropy_index_stats_f32(a.fptr(), b.fptr(), r.fptr(), reinterpret_cast<int32_t*>(pair.fptr() + 1),
-                                                stats.fptr(), a.sizes()[0], a.sizes()[1], current_stream()),
-            "CrossEntropy_AMD_kernel");
-        remember_ce_stats(a, b, std::move(stats));
+        if (g_ce_one_pass && AutoDiffContext::current() && a.requires_grad() && ce_row_fits(a)) {
+            Tensor grad = like(a);
+            run(ctamd_cross_entropy_index_fused_f32(a.fptr(), b.fptr(), r.fptr(), reinterpret_cast<int32_t*>(pair.fptr() + 1),
+                                                    grad.fptr(), a.sizes()[0], a.sizes()[1], current_stream()),
+                "CrossEntropy_AMD_kernel");
+            remember_ce(a, b, Tensor(), std::move(grad));
+        } else {
+            Tensor stats(ShapeTag{}, {a.sizes()[0], 2}, DType::kFloat, DeviceType::kAMD, false);
+            run(ctamd_cross_entropy_index_stats_f32(a.fptr(), b.fptr(), r.fptr(), reinterpret_cast<int32_t*>(pair.fptr() + 1),
+                                                    stats.fptr(), a.sizes()[0], a.sizes()[1], current_stream()),
+                "CrossEntropy_AMD_kernel");
+            remember_ce(a, b, std::move(stats), Tensor());
+        }
         if (recording()) return r;              // a recorded step cannot wait: a bad index shows as a NaN loss
         struct { float loss; int32_t bad; } got = {0.0f, 0};
         device_copy_d2h(&got, pair.fptr(), sizeof(got));

@@ -168,6 +168,8 @@ def main():
                                                              P(Y), rows, cols, S), 8)
     row("cross entropy backward from forward statistics", lambda: call("ctamd_cross_entropy_backward_index_stats_f32", P(X),
                                                                        P(idx), P(stats), P(g1), P(Y), rows, cols, S), 8)
+    row("cross entropy loss + gradient in one pass", lambda: call("ctamd_cross_entropy_index_fused_f32", P(X), P(idx), P(out),
+                                                                  P(status), P(Y), rows, cols, S), 8)
     row("softmax backward rows", lambda: call("ctamd_softmax_backward_rows_f32", P(Y), P(X), P(Y), rows, cols, S), 12)
     del X, Y
     torch.cuda.empty_cache()

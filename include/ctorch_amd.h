@@ -167,6 +167,16 @@ int ctamd_cross_entropy_index_stats_f32(const float* x, const float* idx, float*
                                         size_t rows, size_t cols, void* stream);
 int ctamd_cross_entropy_backward_index_stats_f32(const float* x, const float* idx, const float* stats, const float* g1,
                                                  float* dx, size_t rows, size_t cols, void* stream);
+/* Loss and gradient of the logits from ONE visit of each row: out[0] and status[0] as
+ * ctamd_cross_entropy_index_f32, and dx = exp(x - max) / sum - onehot(idx), the gradient of
+ * src/AutoDiff.cpp:1517-1601 for an upstream gradient of 1 (x * 1.0f is x), which is what a loss that
+ * is the root of backward() receives.  The row stays in registers between the two uses: 8 bytes per
+ * element instead of the 12 of a forward pass and a backward pass.  Rows of at most 32768 columns
+ * (8192 when the row length is no multiple of four or a tensor is not 16-byte aligned); CTAMD_ERANGE
+ * beyond, with nothing launched.  The reference computes the two in separate passes (CrossEntropy_BASIC_kernel.cpp:88-120,
+ * then the tape). */
+int ctamd_cross_entropy_index_fused_f32(const float* x, const float* idx, float* out, int32_t* status, float* dx,
+                                        size_t rows, size_t cols, void* stream);
 
 /* -------------------------------------------------------------------------------- matmul */
 /* C[i,j] = sum_l A[i*as0 + l*as1] * B[l*bs0 + j*bs1]; C is [m, n] row-major contiguous; strides

@@ -143,6 +143,15 @@ def ce_index(x, idx):
     return out, int(status.item())
 
 
+def ce_index_fused(x, idx):
+    """loss, status and the gradient for an upstream gradient of 1, one launch over the logits"""
+    out = torch.empty(1, device=DEV)
+    status = torch.full((1,), -7, dtype=torch.int32, device=DEV)
+    dx = torch.empty_like(x)
+    call("ctamd_cross_entropy_index_fused_f32", ptr(x), ptr(idx), ptr(out), ptr(status), ptr(dx), x.shape[0], x.shape[1], stream())
+    return out, int(status.item()), dx
+
+
 def ce_bwd(x, t, g1, index):
     dx = torch.empty_like(x)
     rows, cols = (1, x.numel()) if x.dim() == 1 else x.shape

@@ -893,6 +893,9 @@ class HostLayer(Reference):
     def set_reference_row0(self, on):
         self.cdll.cth_set_reference_row0(int(on))
 
+    def set_ce_one_pass(self, on):
+        self.cdll.cth_set_ce_one_pass(int(on))
+
     def compare(self, cmp, a, b=None, s=0.0):
         """The Tensor comparison operators on the device; returns the bool tensor as uint8, or the
         negative return code."""

@@ -85,6 +85,28 @@ def test_cross_entropy_target_forms_and_errors(oracle, host):
     for t in (oh, idx):
         rc, loss, dp = host.grad_loss(CE, x, t, 0.37)
         assert rc == x.size and np.abs(dp - wantd).max() <= 1e-6
+    # the loss as the root of backward(): with class indices loss and gradient come from one pass over
+    # the logits (the gradient waits in the front-end for backward()), or - switched off - from a
+    # forward pass and a backward pass; a second backward() over the same tape recomputes
+    want1 = oracle.accumulate0(oracle.ce_bwd_onehot(x, oh, F(1.0)))
+    for shape, seed in (((19, 31), 40), ((6, 4096), 44), ((3, 33000), 45)):
+        xs = oracle.normal(shape, seed, 0, 2)
+        ids = oracle.ints((shape[0],), seed + 1, shape[1])
+        ohs = np.zeros_like(xs)
+        ohs[np.arange(shape[0]), ids.astype(int)] = 1
+        wants = oracle.accumulate0(oracle.ce_bwd_onehot(xs, ohs, F(1.0)))
+        got = []
+        for one_pass in (True, False):
+            host.set_ce_one_pass(one_pass)
+            try:
+                rc, loss, dp = host.grad_loss(CE, xs, ids, 1.0)
+            finally:
+                host.set_ce_one_pass(True)
+            assert rc == xs.size and np.abs(dp - wants).max() <= 1e-6, (shape, one_pass)
+            assert abs(loss - oracle.ce_index(xs, ids)) <= 1e-5 * abs(oracle.ce_index(xs, ids))
+            got.append(dp)
+        assert np.abs(got[0] - got[1]).max() <= 5e-7, shape
+    assert want1.shape == x.shape
 
 
 def test_matmul_layouts_and_gradients(oracle, host):

@@ -281,6 +281,45 @@ def test_cross_entropy_backward_from_forward_statistics(oracle, shape):
     assert np.abs(G.host(out) - G.host(G.ce_bwd(dx, didx, g1, True))).max() <= (5e-7 if cols >= 2048 else 2e-7)
 
 
+@pytest.mark.parametrize("shape", [(1, 1), (64, 10), (19, 301), (33, 1000), (4, 2052), (3, 8192), (5, 32768), (2, 8191)])
+def test_cross_entropy_loss_and_gradient_in_one_pass(oracle, shape):
+    """ctamd_cross_entropy_index_fused_f32: the loss of the forward entry point and the gradient the
+    backward entry point gives for an upstream gradient of 1 - bit for bit against the recomputing
+    backward (same exponential, same sums), to the reduction bar against the oracle."""
+    print("case ce fused", shape, flush=True)
+    rows, cols = shape
+    x = oracle.normal(shape, 92, 0, 2)
+    idx = oracle.ints((rows,), 93, cols)
+    dx, didx = G.dev(x), G.dev(idx)
+    loss, status, grad = G.ce_index_fused(dx, didx)
+    want_loss = oracle.ce_index(x, idx)
+    assert status == 0 and abs(G.host(loss)[0] - want_loss) <= 1e-5 * abs(want_loss) + 1e-6
+    oh = np.zeros(shape, F)
+    oh[np.arange(rows), idx.astype(int)] = 1
+    assert np.abs(G.host(grad) - oracle.ce_bwd_onehot(x, oh, F(1.0))).max() <= 1e-6
+    one = G.dev(np.array([1.0]))
+    bits_equal(G.host(grad), G.host(G.ce_bwd(dx, didx, one, True)), "fused gradient vs the backward entry point")
+    assert np.all(np.abs(G.host(grad).astype(np.float64).sum(1)) <= 1e-5)
+    # a bad index: status and a NaN loss as the forward entry point; the row's gradient is its softmax
+    if cols > 1:
+        bad = idx.copy()
+        bad[rows // 2] = cols
+        loss, status, grad_bad = G.ce_index_fused(dx, G.dev(bad))
+        assert status == 1 and np.isnan(G.host(loss)[0])
+        keep = np.arange(rows) != rows // 2
+        bits_equal(G.host(grad_bad)[keep], G.host(grad)[keep], "rows with good indices")
+
+
+def test_cross_entropy_in_one_pass_refuses_rows_beyond_its_registers(oracle):
+    x = torch.zeros(2, 32772, device=G.DEV)
+    idx = torch.zeros(2, device=G.DEV)
+    out = torch.empty(1, device=G.DEV)
+    rc = G.lib().ctamd_cross_entropy_index_fused_f32(G.ptr(x), G.ptr(idx), G.ptr(out), None, G.ptr(torch.empty_like(x)), 2, 32772, G.stream())
+    assert rc == -5
+    rc = G.lib().ctamd_cross_entropy_index_fused_f32(G.ptr(x), G.ptr(idx), G.ptr(out), None, G.ptr(torch.empty_like(x)), 2, 8193, G.stream())
+    assert rc == -5
+
+
 def test_cross_entropy_edge_cases(oracle):
     print("case ce edges", flush=True)
     x = oracle.normal((19, 31), 28, 0, 2)
