@@ -148,7 +148,12 @@ def test_config4_softmax_cross_entropy_8192x32000():
     y = G.softmax(x, 1)
     assert float((y.double().sum(1) - 1).abs().max()) <= 1e-5
     assert float((y[sample].double() - torch.softmax(x[sample].double(), dim=1)).abs().max()) <= 1e-7
-    del d, y
+    # loss and gradient from one pass over the logits: the same loss to the reduction bar, the same
+    # gradient bit for bit (both keep a row in registers and use the exact exponential)
+    loss1, status1, d1pass = G.ce_index_fused(x, idxf)
+    assert status1 == 0 and abs(float(loss1) - want) <= 1e-5 * want
+    assert torch.equal(d1pass, d)
+    del d, y, d1pass
     # linearity of the gradient in the upstream scalar
     half = G.fill(1, 0.5)
     dh = G.ce_bwd(x[:64].contiguous(), idxf[:64].contiguous(), half, True)
