@@ -208,6 +208,68 @@ __global__ __launch_bounds__(kThreads) void colsum_stage1(const float* __restric
         }
 }
 
+// Narrow matrices (a row is at most 128 vectors: the bias gradients of a layer, [8192 x 256] or
+// [8192 x 10]): the strip kernel above would leave most of a block's threads without a column.  Here
+// a block's threads form G = 256 / (vectors per row) row groups; group k walks rows k, k + G, ... of
+// the block's chunk with four rows in flight, so the block reads its chunk as one contiguous run;
+// the groups are added through LDS in group order and the block writes one partial row.
+template <bool VEC>
+__global__ __launch_bounds__(kThreads) void colsum_narrow_stage1(const float* __restrict__ g, float* __restrict__ partials,
+                                                                 size_t rows, size_t cols, unsigned lanes, unsigned groups,
+                                                                 size_t rows_per_block) {
+    constexpr int W = VEC ? 4 : 1;
+    __shared__ float s_part[kThreads][W];
+    const unsigned lane = threadIdx.x % lanes, group = threadIdx.x / lanes;
+    const size_t r0 = size_t(blockIdx.x) * rows_per_block;
+    size_t r1 = r0 + rows_per_block;
+    if (r1 > rows) r1 = rows;
+    float acc[4][W];
+#pragma unroll
+    for (int p = 0; p < 4; ++p)
+#pragma unroll
+        for (int e = 0; e < W; ++e) acc[p][e] = 0.0f;
+    if (group < groups) {
+        const float* col = g + size_t(lane) * W;
+        size_t r = r0 + group;
+        for (; r + 3 * size_t(groups) < r1; r += 4 * size_t(groups)) {
+            float x[4][W];
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const float* src = col + (r + size_t(p) * groups) * cols;
+                if (VEC) {
+                    v4f t = *reinterpret_cast<const v4f*>(src);
+#pragma unroll
+                    for (int e = 0; e < W; ++e) x[p][e] = t[e];
+                } else {
+                    x[p][0] = *src;
+                }
+            }
+#pragma unroll
+            for (int p = 0; p < 4; ++p)
+#pragma unroll
+                for (int e = 0; e < W; ++e) acc[p][e] += x[p][e];
+        }
+        for (; r < r1; r += groups) {
+            const float* src = col + r * cols;
+#pragma unroll
+            for (int e = 0; e < W; ++e) acc[0][e] += src[e];
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < W; ++e) s_part[threadIdx.x][e] = (acc[0][e] + acc[1][e]) + (acc[2][e] + acc[3][e]);
+    __syncthreads();
+    if (group == 0) {
+        float t[W];
+#pragma unroll
+        for (int e = 0; e < W; ++e) t[e] = s_part[lane][e];
+        for (unsigned k = 1; k < groups; ++k)
+#pragma unroll
+            for (int e = 0; e < W; ++e) t[e] += s_part[k * lanes + lane][e];
+#pragma unroll
+        for (int e = 0; e < W; ++e) partials[size_t(blockIdx.x) * cols + size_t(lane) * W + e] = t[e];
+    }
+}
+
 constexpr int kFoldLanes = 4;    // lanes per column in stage 2
 constexpr int kSmallLanes = 16;  // lanes per column when a small matrix is summed in one launch
 // out[c] = sum over the `chunks` rows of partials[., c], in double, LANES lanes per column.  Stage 2
@@ -278,6 +340,29 @@ int ctamd_colsum_f32(const float* g, float* out, size_t rows, size_t cols, void*
     bool vec = (cols % 4 == 0) && aligned16(g);
     const size_t w = vec ? 4 : 1;
     const size_t cus = size_t(compute_units() > 0 ? compute_units() : 256);
+    const size_t lanes = cols / w;                                 // vectors per row
+    if (lanes <= 128) {
+        const size_t groups = kThreads / lanes;
+        size_t rows_per_block = groups * 8;                         // eight rows per thread, four in flight
+        size_t chunks = (rows + rows_per_block - 1) / rows_per_block;
+        if (chunks > 256) {
+            rows_per_block = (rows + 255) / 256;
+            chunks = (rows + rows_per_block - 1) / rows_per_block;
+        }
+        if (vec)
+            hipLaunchKernelGGL((colsum_narrow_stage1<true>), dim3((unsigned)chunks), dim3(kThreads), 0, s, g, partials, rows, cols,
+                               (unsigned)lanes, (unsigned)groups, rows_per_block);
+        else
+            hipLaunchKernelGGL((colsum_narrow_stage1<false>), dim3((unsigned)chunks), dim3(kThreads), 0, s, g, partials, rows, cols,
+                               (unsigned)lanes, (unsigned)groups, rows_per_block);
+        int rc = launched(__func__);
+        if (rc) return rc;
+        constexpr size_t kFoldCols = kThreads / kFoldLanes;
+        hipLaunchKernelGGL(colsum_stage2<kFoldLanes>, dim3((unsigned)((cols + kFoldCols - 1) / kFoldCols)), dim3(kThreads), 0, s,
+                           partials, out, cols, (unsigned)chunks);
+        account(4.0 * double(rows) * double(cols), double(rows) * double(cols));
+        return launched(__func__);
+    }
     // at most 256 row chunks of at least 32 rows; wide strips unless that leaves the chip short of blocks
     size_t chunks = (rows + 31) / 32;
     if (chunks > 256) chunks = 256;

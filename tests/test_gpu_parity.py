@@ -195,7 +195,8 @@ def test_reductions_normwise(oracle, n):
 
 
 @pytest.mark.parametrize("shape", [(1, 1), (2, 3), (37, 53), (8192, 256), (1000, 10), (4096, 4096), (33, 4100), (70000, 3), (128, 10),
-                                   (256, 256), (1024, 512), (1025, 16), (1024, 513)])
+                                   (256, 256), (1024, 512), (1025, 16), (1024, 513), (8192, 10), (100000, 128), (5000, 512), (3001, 129),
+                                   (2049, 1)])
 def test_column_sum(oracle, shape):
     print("case colsum", shape, flush=True)
     g = oracle.normal(shape, 23)
