@@ -138,6 +138,18 @@ struct Row {
             }
         return s;
     }
+    // v <- exp(v - m) with the hardware exp2 (~1e-7 relative near the maximum, where it matters)
+    __device__ __forceinline__ float exp_shifted_fast(float m) {
+        float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k)
+#pragma unroll
+            for (int i = 0; i < W; ++i) {
+                v[k][i] = __builtin_amdgcn_exp2f((v[k][i] - m) * 1.44269504088896340736f);
+                if ((k * W + i) & 1) s1 += v[k][i]; else s0 += v[k][i];
+            }
+        return s0 + s1;
+    }
     // sum of exp(v - m) without changing v, with the hardware exp2: the loss only needs this sum
     // to ~1e-7 relative (the reference's own sequential sum is no closer), so the forward loss
     // kernels skip the bit-exact exp for it and stay bandwidth-bound
@@ -173,7 +185,7 @@ struct Row {
     }
 };
 
-enum Mode { kSoftmax, kCeOnehot, kCeIndex, kCeBwdOnehot, kCeBwdIndex, kSoftmaxBwd, kCeIndexBoth };
+enum Mode { kSoftmax, kCeOnehot, kCeIndex, kCeBwdOnehot, kCeBwdIndex, kSoftmaxBwd, kCeIndexBoth, kCeIndexBothFast };
 
 struct Args {
     const float* x;      // logits / softmax output y (kSoftmaxBwd)
@@ -201,7 +213,8 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
     __shared__ float s_f[2][THREADS / 64 + 1];
     __shared__ double s_d[THREADS / 64 + 1];
     stage_exp_table(s_exp2);
-    constexpr bool kPipelined = (MODE == kSoftmax || MODE == kCeIndex || MODE == kCeBwdIndex || MODE == kCeIndexBoth);
+    constexpr bool kBoth = (MODE == kCeIndexBoth || MODE == kCeIndexBothFast);
+    constexpr bool kPipelined = (MODE == kSoftmax || MODE == kCeIndex || MODE == kCeBwdIndex || kBoth);
     double block_loss = 0.0;
     bool block_bad = false;   // a class index out of range was met (thread 0's copy counts)
 
@@ -210,7 +223,7 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
         const float m = block_max<THREADS>(mloc, s_f[0]);
         constexpr bool kLossOnly = (MODE == kCeOnehot || MODE == kCeIndex);
         // loss kernels keep x in r and only need the row sum; the others turn r into exp(x - m)
-        const float s = block_sum<THREADS>(kLossOnly ? r.sum_exp_fast(m) : r.exp_shifted(m, s_exp2), s_f[1]);
+        const float s = block_sum<THREADS>(kLossOnly ? r.sum_exp_fast(m) : MODE == kCeIndexBothFast ? r.exp_shifted_fast(m) : r.exp_shifted(m, s_exp2), s_f[1]);
         const double rcp_s = 1.0 / double(s);     // e / s below is the exact fp32 quotient (cta_div_rcp)
         if (MODE == kSoftmax) {
 #pragma unroll
@@ -265,19 +278,24 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
                 p = (p < 1e-10f) ? 1e-10f : p;
                 block_loss -= double(float(log(double(p))));
             }
-        } else if (MODE == kCeIndexBoth) {
+        } else if (kBoth) {
             // loss and gradient from one visit of the row: r holds e = exp(x - m), s is its sum;
             // the gradient is the one for an upstream gradient of 1 (d * 1.0f is d)
             // (the class index is read here, not earlier: a wait for it right after the next row's
             // loads were issued would wait for those as well)
             const int c = int(a.t[row]);
             const bool ok = c >= 0 && c < int(a.cols);
+            // which of this thread's elements is column c, as one number (k * W + i, or -1): comparing
+            // it with each element's constant position keeps 32 column indices out of the registers
+            const int q = (ok ? c / W : -1) - int(threadIdx.x);
+            const int slot = (q >= 0 && q % THREADS == 0) ? (q / THREADS) * W + c % W : -1;
             float ec = 0.0f;
 #pragma unroll
             for (int k = 0; k < ITEMS; ++k)
 #pragma unroll
-                for (int i = 0; i < W; ++i) ec = (ok && r.index(k, i) == unsigned(c)) ? r.v[k][i] : ec;
+                for (int i = 0; i < W; ++i) ec = (slot == k * W + i) ? r.v[k][i] : ec;
             ec = block_sum<THREADS>(ec, s_f[0]);
+            const float rcp_sf = 1.0f / s;
             if (!ok) {
                 block_bad = true;
                 block_loss += double(__builtin_nanf(""));
@@ -290,8 +308,8 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
             for (int k = 0; k < ITEMS; ++k)
 #pragma unroll
                 for (int i = 0; i < W; ++i) {
-                    float sm = cta_div_rcp(r.v[k][i], rcp_s);
-                    float d = sm - ((ok && r.index(k, i) == unsigned(c)) ? 1.0f : 0.0f);
+                    float sm = MODE == kCeIndexBothFast ? r.v[k][i] * rcp_sf : cta_div_rcp(r.v[k][i], rcp_s);
+                    float d = sm - ((slot == k * W + i) ? 1.0f : 0.0f);
                     r.v[k][i] = 0.0f + d;
                 }
             r.store(a.out + row * a.cols, unsigned(a.cols));
@@ -375,9 +393,9 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
             process(r, row, r.max());
         }
     }
-    if ((MODE == kCeOnehot || MODE == kCeIndex || MODE == kCeIndexBoth) && threadIdx.x == 0) {
+    if ((MODE == kCeOnehot || MODE == kCeIndex || kBoth) && threadIdx.x == 0) {
         a.partials[blockIdx.x] = block_loss;
-        if ((MODE == kCeIndex || MODE == kCeIndexBoth) && a.status) a.partials[gridDim.x + blockIdx.x] = block_bad ? 1.0 : 0.0;
+        if ((MODE == kCeIndex || kBoth) && a.status) a.partials[gridDim.x + blockIdx.x] = block_bad ? 1.0 : 0.0;
     }
 }
 
@@ -628,9 +646,10 @@ bool launch_resident(const Args& a, unsigned grid, hipStream_t s) {
 
 template <int MODE>
 int run_rows(const char* name, Args a, float* loss_out, void* stream) {
-    constexpr bool kLoss = (MODE == kCeOnehot || MODE == kCeIndex || MODE == kCeIndexBoth);
-    constexpr bool kIndexLoss = (MODE == kCeIndex || MODE == kCeIndexBoth);
-    constexpr bool kWrites = !kLoss || MODE == kCeIndexBoth;           // a [rows, cols] result
+    constexpr bool kBoth = (MODE == kCeIndexBoth || MODE == kCeIndexBothFast);
+    constexpr bool kLoss = (MODE == kCeOnehot || MODE == kCeIndex || kBoth);
+    constexpr bool kIndexLoss = (MODE == kCeIndex || kBoth);
+    constexpr bool kWrites = !kLoss || kBoth;                          // a [rows, cols] result
     if (kLoss && !loss_out) return fail(CTAMD_EINVAL, "%s: null output", name);
     hipStream_t s = as_stream(stream);
     if (a.rows == 0 || a.cols == 0) {
@@ -650,8 +669,8 @@ int run_rows(const char* name, Args a, float* loss_out, void* stream) {
         // index adds 4 bytes per row; one exp per element
         const double n = double(a.rows) * double(a.cols);
         const double per = MODE == kSoftmax ? 8.0 : MODE == kCeIndex ? 4.0 : MODE == kCeOnehot ? 8.0
-                         : (MODE == kCeBwdIndex || MODE == kCeIndexBoth) ? 8.0 : 12.0;   // kCeBwdOnehot, kSoftmaxBwd: two inputs, one output
-        const bool index = (MODE == kCeIndex || MODE == kCeBwdIndex || MODE == kCeIndexBoth);
+                         : (MODE == kCeBwdIndex || kBoth) ? 8.0 : 12.0;   // kCeBwdOnehot, kSoftmaxBwd: two inputs, one output
+        const bool index = (MODE == kCeIndex || MODE == kCeBwdIndex || kBoth);
         account(per * n + (index ? 4.0 * double(a.rows) : 0.0), n);
     }
     if (kLoss) a.partials = reinterpret_cast<double*>(scratch());
@@ -663,7 +682,7 @@ int run_rows(const char* name, Args a, float* loss_out, void* stream) {
     if (kLoss && fill > 2048) fill = 2048;         // one partial per block: keep the fold of the partials short
     unsigned grid = a.rows < fill ? unsigned(a.rows) : unsigned(fill);
     bool vec = (a.cols % 4 == 0) && aligned16(a.x) &&
-               (MODE == kSoftmax || MODE == kCeIndex || MODE == kCeBwdIndex || MODE == kCeIndexBoth || aligned16(a.t)) &&
+               (MODE == kSoftmax || MODE == kCeIndex || MODE == kCeBwdIndex || kBoth || aligned16(a.t)) &&
                (!kWrites || aligned16(a.out));
     if (MODE == kCeIndex && a.cols >= 2048) {
         size_t fill_online = size_t(compute_units() > 0 ? compute_units() : 256) * 8;
@@ -677,7 +696,7 @@ int run_rows(const char* name, Args a, float* loss_out, void* stream) {
     }
     bool done = vec ? launch_resident<MODE, 4>(a, grid, s) : launch_resident<MODE, 1>(a, grid, s);
     if (!done) {
-        if constexpr (MODE == kCeIndexBoth)
+        if constexpr (kBoth)
             return fail(CTAMD_ERANGE, "%s: a row does not fit a block's registers (32768 columns, 8192 without 128-bit accesses): "
                         "use the separate forward and backward entry points", name);
         else
@@ -974,6 +993,9 @@ int ctamd_cross_entropy_index_stats_f32(const float* x, const float* idx, float*
 int ctamd_cross_entropy_index_fused_f32(const float* x, const float* idx, float* out, int32_t* status, float* dx, size_t rows,
                                         size_t cols, void* stream) {
     Args a{x, idx, nullptr, dx, nullptr, status, nullptr, rows, cols, nullptr, nullptr};
+    // long rows use the hardware exponential throughout, as the forward / backward-from-statistics
+    // pair does (<= 2e-7 from the exact form)
+    if (cols >= 2048) return run_rows<kCeIndexBothFast>(__func__, a, out, stream);
     return run_rows<kCeIndexBoth>(__func__, a, out, stream);
 }
 int ctamd_cross_entropy_backward_onehot_f32(const float* x, const float* t, const float* g1, float* dx, size_t rows,

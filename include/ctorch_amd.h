@@ -173,7 +173,10 @@ int ctamd_cross_entropy_backward_index_stats_f32(const float* x, const float* id
  * is the root of backward() receives.  The row stays in registers between the two uses: 8 bytes per
  * element instead of the 12 of a forward pass and a backward pass.  Rows of at most 32768 columns
  * (8192 when the row length is no multiple of four or a tensor is not 16-byte aligned); CTAMD_ERANGE
- * beyond, with nothing launched.  The reference computes the two in separate passes (CrossEntropy_BASIC_kernel.cpp:88-120,
+ * beyond, with nothing launched.  Rows of 2048 columns or more use the hardware exponential and a
+ * multiplication by 1 / sum (<= 2e-7 from the exact form, as ctamd_cross_entropy_backward_index_stats_f32);
+ * shorter rows are bit-equal to ctamd_cross_entropy_backward_index_f32 with g1 = 1.  The reference
+ * computes the two in separate passes (CrossEntropy_BASIC_kernel.cpp:88-120,
  * then the tape). */
 int ctamd_cross_entropy_index_fused_f32(const float* x, const float* idx, float* out, int32_t* status, float* dx,
                                         size_t rows, size_t cols, void* stream);

@@ -149,10 +149,13 @@ def test_config4_softmax_cross_entropy_8192x32000():
     assert float((y.double().sum(1) - 1).abs().max()) <= 1e-5
     assert float((y[sample].double() - torch.softmax(x[sample].double(), dim=1)).abs().max()) <= 1e-7
     # loss and gradient from one pass over the logits: the same loss to the reduction bar, the same
-    # gradient bit for bit (both keep a row in registers and use the exact exponential)
+    # gradient to 5e-7 (rows this long use the hardware exponential, as the backward pass from forward
+    # statistics does)
     loss1, status1, d1pass = G.ce_index_fused(x, idxf)
     assert status1 == 0 and abs(float(loss1) - want) <= 1e-5 * want
-    assert torch.equal(d1pass, d)
+    assert float((d1pass - d).abs().max()) <= 5e-7
+    assert float(d1pass.double().sum(1).abs().max()) <= 1e-4
+    assert float((d1pass[sample].double() - sm).abs().max()) <= 1e-6
     del d, y, d1pass
     # linearity of the gradient in the upstream scalar
     half = G.fill(1, 0.5)

@@ -286,7 +286,8 @@ def test_cross_entropy_backward_from_forward_statistics(oracle, shape):
 def test_cross_entropy_loss_and_gradient_in_one_pass(oracle, shape):
     """ctamd_cross_entropy_index_fused_f32: the loss of the forward entry point and the gradient the
     backward entry point gives for an upstream gradient of 1 - bit for bit against the recomputing
-    backward (same exponential, same sums), to the reduction bar against the oracle."""
+    backward for rows under 2048 columns (same exponential, same sums), to the reduction bar against
+    the oracle everywhere."""
     print("case ce fused", shape, flush=True)
     rows, cols = shape
     x = oracle.normal(shape, 92, 0, 2)
@@ -299,7 +300,10 @@ def test_cross_entropy_loss_and_gradient_in_one_pass(oracle, shape):
     oh[np.arange(rows), idx.astype(int)] = 1
     assert np.abs(G.host(grad) - oracle.ce_bwd_onehot(x, oh, F(1.0))).max() <= 1e-6
     one = G.dev(np.array([1.0]))
-    bits_equal(G.host(grad), G.host(G.ce_bwd(dx, didx, one, True)), "fused gradient vs the backward entry point")
+    if cols < 2048:
+        bits_equal(G.host(grad), G.host(G.ce_bwd(dx, didx, one, True)), "fused gradient vs the backward entry point")
+    else:   # long rows use the hardware exponential, as the forward / backward-from-statistics pair does
+        assert np.abs(G.host(grad) - G.host(G.ce_bwd(dx, didx, one, True))).max() <= 5e-7
     assert np.all(np.abs(G.host(grad).astype(np.float64).sum(1)) <= 1e-5)
     # a bad index: status and a NaN loss as the forward entry point; the row's gradient is its softmax
     if cols > 1:
