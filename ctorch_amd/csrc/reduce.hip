@@ -140,7 +140,7 @@ int reduce(const char* name, const float* a, const float* b, float* out, int32_t
 // ----------------------------------------------------------------------------- column sum
 // A block owns a strip of 256 * CU vectors of columns (CU = 4: up to 4096 columns, 16 KiB per row;
 // CU = 1 when that would leave the chip short of blocks) and a chunk of rows, and walks its rows in
-// order, two rows in flight per thread.  Each block writes one partial row per strip; stage 2 adds
+// order, two (CU = 4) or four (CU = 1) rows in flight per thread.  Each block writes one partial row per strip; stage 2 adds
 // the (at most 256) partial rows in double, four lanes per column with eight loads in flight each -
 // a serial walk over the partial rows by one thread per column cost more than stage 1 itself.
 template <bool VEC, int CU>
@@ -151,9 +151,10 @@ __global__ __launch_bounds__(kThreads) void colsum_stage1(const float* __restric
     const size_t r0 = size_t(blockIdx.y) * rows_per_block;
     size_t r1 = r0 + rows_per_block;
     if (r1 > rows) r1 = rows;
-    float acc[2][CU][4];
+    constexpr int P = CU == 1 ? 4 : 2;       // rows in flight per thread (P * CU loads)
+    float acc[P][CU][4];
 #pragma unroll
-    for (int p = 0; p < 2; ++p)
+    for (int p = 0; p < P; ++p)
 #pragma unroll
         for (int u = 0; u < CU; ++u)
 #pragma unroll
@@ -166,10 +167,10 @@ __global__ __launch_bounds__(kThreads) void colsum_stage1(const float* __restric
         live[u] = col[u] < cols;
     }
     size_t r = r0;
-    for (; r + 1 < r1; r += 2) {
-        v4f x[2][CU];
+    for (; r + (P - 1) < r1; r += P) {
+        v4f x[P][CU];
 #pragma unroll
-        for (int p = 0; p < 2; ++p)
+        for (int p = 0; p < P; ++p)
 #pragma unroll
             for (int u = 0; u < CU; ++u)
                 if (live[u]) {
@@ -178,7 +179,7 @@ __global__ __launch_bounds__(kThreads) void colsum_stage1(const float* __restric
                     else x[p][u][0] = *src;
                 }
 #pragma unroll
-        for (int p = 0; p < 2; ++p)
+        for (int p = 0; p < P; ++p)
 #pragma unroll
             for (int u = 0; u < CU; ++u)
                 if (live[u]) {
@@ -186,7 +187,7 @@ __global__ __launch_bounds__(kThreads) void colsum_stage1(const float* __restric
                     for (int e = 0; e < W; ++e) acc[p][u][e] += x[p][u][e];
                 }
     }
-    if (r < r1) {
+    for (; r < r1; ++r) {
 #pragma unroll
         for (int u = 0; u < CU; ++u)
             if (live[u]) {
@@ -204,7 +205,12 @@ __global__ __launch_bounds__(kThreads) void colsum_stage1(const float* __restric
     for (int u = 0; u < CU; ++u)
         if (live[u]) {
 #pragma unroll
-            for (int e = 0; e < W; ++e) partials[size_t(blockIdx.y) * cols + col[u] + e] = acc[0][u][e] + acc[1][u][e];
+            for (int e = 0; e < W; ++e) {
+                float t = acc[0][u][e];
+#pragma unroll
+                for (int p = 1; p < P; ++p) t += acc[p][u][e];
+                partials[size_t(blockIdx.y) * cols + col[u] + e] = t;
+            }
         }
 }
 
@@ -363,8 +369,8 @@ int ctamd_colsum_f32(const float* g, float* out, size_t rows, size_t cols, void*
         account(4.0 * double(rows) * double(cols), double(rows) * double(cols));
         return launched(__func__);
     }
-    // at most 256 row chunks of at least 32 rows; wide strips unless that leaves the chip short of blocks
-    size_t chunks = (rows + 31) / 32;
+    // at most 256 row chunks of at least 16 rows; wide strips unless that leaves the chip short of blocks
+    size_t chunks = (rows + 15) / 16;
     if (chunks > 256) chunks = 256;
     if (chunks > kScratchFloats / cols) chunks = kScratchFloats / cols;
     if (chunks < 1) chunks = 1;
