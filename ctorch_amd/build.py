@@ -6,13 +6,16 @@ hipcc cross-compiles without a GPU.  Flags that matter for results:
                                does have are written out as explicit fma calls)
   -target-feature -packed-fp32-ops   no packed-fp32 VALU instructions
 """
+import json
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
+RESOURCES = os.path.join(os.path.dirname(os.path.abspath(__file__)), "kernel_resources.json")
 LIB = os.path.join(HERE, "libctorch_amd.so")
 SOURCES = ["runtime.hip", "elementwise.hip", "reduce.hip", "softmax_ce.hip", "matmul.hip", "dataset.hip", "expr.hip", "typed.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-fPIC",
@@ -44,14 +47,39 @@ def build(verbose=False, jobs=4):
 
     def one(pair):
         src, obj = pair
-        return _run([hipcc] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj])
+        return _run([hipcc] + FLAGS + ["-Rpass-analysis=kernel-resource-usage", "-c", os.path.join(CSRC, src), "-o", obj])
 
+    resources = {}
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        for out in ex.map(one, zip(SOURCES, objs)):
-            if verbose and out.strip():
-                print(out)
+        for src, out in zip(SOURCES, ex.map(one, zip(SOURCES, objs))):
+            rest = _kernel_resources(src, out, resources)
+            if verbose and rest.strip():
+                print(rest)
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
+    # what every kernel needs (registers, spills, LDS), next to the library: a spilled register costs a
+    # kernel its overlap of loads and arithmetic, so tests/test_build.py refuses a build that has one
+    with open(RESOURCES, "w") as f:
+        json.dump(resources, f, indent=0, sort_keys=True)
     return LIB
+
+
+def _kernel_resources(src, out, table):
+    """Moves the compiler's per-kernel resource remarks from `out` into `table`; returns the rest."""
+    rest, name = [], None
+    for line in out.splitlines():
+        m = re.search(r"remark: (?:\s*)(Function Name|VGPRs|VGPRs Spill|SGPRs Spill|LDS Size \[bytes/block\]|Occupancy \[waves/SIMD\]|"
+                      r"ScratchSize \[bytes/lane\]|AGPRs|SGPRs|Dynamic Stack|TotalSGPRs): (\S+)", line)
+        if not m:
+            if "-Rpass-analysis=kernel-resource-usage" not in line:
+                rest.append(line)
+            continue
+        key, val = m.group(1), m.group(2)
+        if key == "Function Name":
+            name = "%s:%s" % (src, val)
+            table[name] = {}
+        elif name and key in ("VGPRs", "VGPRs Spill", "LDS Size [bytes/block]", "Occupancy [waves/SIMD]", "ScratchSize [bytes/lane]"):
+            table[name][key] = int(val) if val.isdigit() else val
+    return "\n".join(rest)
 
 
 if __name__ == "__main__":

@@ -638,9 +638,17 @@ bool launch_resident(const Args& a, unsigned grid, hipStream_t s) {
     else if (groups <= 64 * 8) launch_cfg<MODE, 64, 8, W>(a, grid, s);
     else if (groups <= 256 * 2) launch_cfg<MODE, 256, 2, W>(a, grid, s);
     else if (groups <= 256 * 8) launch_cfg<MODE, 256, 8, W>(a, grid, s);
-    else if (groups <= 1024 * 2) launch_cfg<MODE, 1024, 2, W>(a, grid, s);
-    else if (groups <= 1024 * 8) launch_cfg<MODE, 1024, 8, W>(a, grid, s);
-    else return false;
+    else {
+        // rows of 2048 columns or more never reach these two modes (they go to the online forward
+        // kernel and to the long-row one-pass kernel): the 1024-thread shapes are not built for them
+        if constexpr (MODE == kCeIndex || MODE == kCeIndexBoth) {
+            return false;
+        } else {
+            if (groups <= 1024 * 2) launch_cfg<MODE, 1024, 2, W>(a, grid, s);
+            else if (groups <= 1024 * 8) launch_cfg<MODE, 1024, 8, W>(a, grid, s);
+            else return false;
+        }
+    }
     return true;
 }
 

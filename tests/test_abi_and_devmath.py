@@ -82,3 +82,18 @@ def test_division_through_a_double_reciprocal_is_ieee_division(tmp_path):
     print(out)
     f = out.strip().split()
     assert int(f[1]) == 64_000_000 and int(f[3]) == 0
+
+
+def test_no_kernel_spills_registers():
+    """The build records what every kernel needs (ctorch_amd/kernel_resources.json, written by
+    ctorch_amd.build).  A kernel that spills registers reloads them with waits that also wait for its
+    prefetched loads - the one-pass cross entropy lost a quarter of its speed to 25 spilled registers -
+    so a build with a spill or a per-lane scratch frame is refused."""
+    import json
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "ctorch_amd", "kernel_resources.json")
+    if not os.path.exists(path):
+        pytest.skip("the library was not built by ctorch_amd.build here")
+    table = json.load(open(path))
+    assert len(table) > 150
+    bad = {k: v for k, v in table.items() if v.get("VGPRs Spill", 0) or v.get("ScratchSize [bytes/lane]", 0)}
+    assert not bad, bad
