@@ -74,6 +74,8 @@ PROTOTYPES.update({
     "ctamd_fill_from_f32": [_P, _P, _Z, _P],
     "ctamd_accumulate_f32": [_P, _P, _Z, _P],
     "ctamd_mse_backward_f32": [_P, _P, _P, _P, _Z, _P],
+    "ctamd_mse_backward_acc_f32": [_P, _P, _P, _P, _P, _Z, _P],
+    "ctamd_mae_backward_acc_f32": [_P, _P, _P, _P, _P, _Z, _P],
     "ctamd_mae_backward_f32": [_P, _P, _P, _P, _Z, _P],
     "ctamd_softmax_backward_rows_f32": [_P, _P, _P, _Z, _Z, _P],
     "ctamd_softmax_backward_cols_f32": [_P, _P, _P, _Z, _Z, _P],

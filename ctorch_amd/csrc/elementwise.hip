@@ -479,6 +479,16 @@ int ctamd_mae_backward_f32(const float* p, const float* t, const float* g1, floa
     Ptrs<2> in{{p, t}};
     return launch_map<MaeBwdF>(__func__, in, dp, n, MaeBwdF{1.0 / double(float(n)), g1}, s);
 }
+int ctamd_mse_backward_acc_f32(const float* p, const float* t, const float* g1, const float* acc, float* dp, size_t n, void* s) {
+    if (n && !g1) return fail(CTAMD_EINVAL, "%s: null upstream gradient", __func__);
+    Ptrs<3> in{{p, t, acc}};
+    return launch_map<PlusF<MseBwdF>>(__func__, in, dp, n, PlusF<MseBwdF>{MseBwdF{1.0 / double(float(n)), g1}}, s);
+}
+int ctamd_mae_backward_acc_f32(const float* p, const float* t, const float* g1, const float* acc, float* dp, size_t n, void* s) {
+    if (n && !g1) return fail(CTAMD_EINVAL, "%s: null upstream gradient", __func__);
+    Ptrs<3> in{{p, t, acc}};
+    return launch_map<PlusF<MaeBwdF>>(__func__, in, dp, n, PlusF<MaeBwdF>{MaeBwdF{1.0 / double(float(n)), g1}}, s);
+}
 int ctamd_div_backward_b_rowbcast_f32(const float* a, const float* b, const float* g, float* db, size_t rows, size_t cols,
                                       void* s) {
     return launch_rowbcast<DivBwdBF>(__func__, a, b, db, rows, cols, s, g);

@@ -133,6 +133,14 @@ struct MaeBwdF { static constexpr int kIn = 2; static constexpr bool kTables = f
         float s = (d > 0.0f) ? 1.0f : ((d < 0.0f) ? -1.0f : 0.0f);
         float q = cta_div_rcp(s, rfn);           // sign / float(n)
         return 0.0f + q * *g; } };   // "0 +": the tape adds the term to a zero-filled buffer (-0 becomes +0)
+// inputs (F's inputs..., acc): acc + F(...) - a gradient term added to the gradient gathered so far in
+// the pass that forms it (the term is rounded before the addition, as the separate accumulate pass adds it)
+template <class F>
+struct PlusF { static constexpr int kIn = F::kIn + 1; static constexpr bool kTables = F::kTables;
+    F f;
+    __device__ float operator()(const float* x, const Tables& t) const {
+        float term = f(x, t);
+        return x[F::kIn] + term; } };
 // inputs (a, b, g): ((-a) * g) / (b * b)
 struct DivBwdBF { static constexpr int kIn = 3; static constexpr bool kTables = false;
     __device__ float operator()(const float* x, const Tables&) const {

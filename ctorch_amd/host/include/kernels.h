@@ -73,6 +73,8 @@ Tensor cos_backward(const Tensor& x, const Tensor& g);
 Tensor softmax_backward(const Tensor& y, const Tensor& g, int dim);
 Tensor mse_backward(const Tensor& p, const Tensor& t, const Tensor& g0d);
 Tensor mae_backward(const Tensor& p, const Tensor& t, const Tensor& g0d);
+// acc + the MSE (mae = false) or MAE gradient, in the pass that forms it
+Tensor loss_backward_plus(bool mae, const Tensor& p, const Tensor& t, const Tensor& g0d, const Tensor& acc);
 Tensor cross_entropy_backward(const Tensor& x, const Tensor& target, const Tensor& g0d);
 Tensor div_backward_b(const Tensor& a, const Tensor& b, const Tensor& g);
 // The stream every launch of this front-end goes to (as the C ABI's void*): the null stream unless a

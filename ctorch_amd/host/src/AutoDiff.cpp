@@ -369,6 +369,19 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
             size_t input_id = node->input_ids[pos];
             Node* in = find(input_id);
             if (!in || !in->requires_grad) continue;
+            // a second loss of the same predictions: its gradient is added to the one gathered so far
+            // in the pass that forms it (the same sum as term-then-accumulate, bit for bit)
+            if ((node->operation == op::MSE || node->operation == op::MAE) && pos == 0 && in->grad &&
+                node->input_ids.size() == 2 && node->input_ids[1] != input_id && in->grad->is_contiguous() &&
+                in->grad->sizes() == in->tensor->sizes() && in->tensor->device() == DeviceType::kAMD) {
+                Node* target = find(node->input_ids[1]);
+                if (target && target->tensor->sizes() == in->tensor->sizes()) {
+                    in->grad = std::make_unique<Tensor>(loss_backward_plus(node->operation == op::MAE, *in->tensor, *target->tensor,
+                                                                            node_grad, *in->grad));
+                    // the term carries its "0 +"; the sum holds no -0 unless the gathered part did
+                    continue;
+                }
+            }
             Tensor val = input_gradient(node, input_id, pos, node_grad);
             Tensor adj = adjust_grad_shape(val, in->tensor->sizes());
             const bool plus_zero = term_plus_zero_;

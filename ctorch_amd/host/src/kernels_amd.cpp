@@ -357,6 +357,17 @@ Tensor mae_backward(const Tensor& p, const Tensor& t, const Tensor& g) {
     run(ctamd_mae_backward_f32(p.fptr(), t.fptr(), g.fptr(), r.fptr(), p.numel(), current_stream()), "mae_backward");
     return r;
 }
+Tensor loss_backward_plus(bool mae, const Tensor& p, const Tensor& t, const Tensor& g, const Tensor& acc) {
+    check_device(p, "loss_backward");
+    check_device(acc, "loss_backward");
+    if (acc.numel() != p.numel() || t.numel() != p.numel())
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "loss_backward: sizes differ");
+    Tensor r = like(p);
+    run(mae ? ctamd_mae_backward_acc_f32(p.fptr(), t.fptr(), g.fptr(), acc.fptr(), r.fptr(), p.numel(), current_stream())
+            : ctamd_mse_backward_acc_f32(p.fptr(), t.fptr(), g.fptr(), acc.fptr(), r.fptr(), p.numel(), current_stream()),
+        "loss_backward");
+    return r;
+}
 namespace {
 // What the class-index CrossEntropy forward leaves for its backward: per-row (max, sum), or - when
 // loss and gradient were computed in one pass - the gradient for an upstream gradient of 1.  Keyed

@@ -311,6 +311,14 @@ int ctamd_softmax_backward_cols_f32(const float* y, const float* g, float* dx, s
  * include it as well. */
 int ctamd_mse_backward_f32(const float* p, const float* t, const float* g1, float* dp, size_t n, void* stream);
 int ctamd_mae_backward_f32(const float* p, const float* t, const float* g1, float* dp, size_t n, void* stream);
+/* The same two with the gradient gathered so far added in the same pass: dp[i] = acc[i] + term[i],
+ * the term rounded first - what ctamd_mse/mae_backward_f32 followed by ctamd_accumulate_f32 leaves
+ * (src/AutoDiff.cpp:1870-1907), in 16 instead of 24 bytes per element.  For a tensor that several
+ * losses are taken of. */
+int ctamd_mse_backward_acc_f32(const float* p, const float* t, const float* g1, const float* acc, float* dp, size_t n,
+                               void* stream);
+int ctamd_mae_backward_acc_f32(const float* p, const float* t, const float* g1, const float* acc, float* dp, size_t n,
+                               void* stream);
 /* dx = 0 + (softmax(x) - t) * g[0], gradient of the SUM-reduced loss.  src/AutoDiff.cpp:1546-1574.
  * The index form takes class indices (the reference throws there, :1569) and equals the one-hot
  * arithmetic with t = onehot(idx). */

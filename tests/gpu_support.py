@@ -166,6 +166,12 @@ def loss_bwd(name, p, t, g1):
     return dp
 
 
+def loss_bwd_acc(name, p, t, g1, acc):
+    dp = torch.empty_like(p)
+    call("ctamd_%s_backward_acc_f32" % name, ptr(p), ptr(t), ptr(g1), ptr(acc), ptr(dp), p.numel(), stream())
+    return dp
+
+
 def div_bwd_b_rowbcast(a, b, g):
     r = torch.empty_like(a)
     call("ctamd_div_backward_b_rowbcast_f32", ptr(a), ptr(b), ptr(g), ptr(r), a.shape[0], a.shape[1], stream())

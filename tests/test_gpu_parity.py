@@ -160,6 +160,11 @@ def test_elementwise_gradients(oracle):
     g1 = G.dev(np.array([0.37]))
     bits_equal(G.host(G.loss_bwd("mse", G.dev(p), G.dev(t), g1)), oracle.mse_bwd(p, t, F(0.37)), "mse bwd")
     bits_equal(G.host(G.loss_bwd("mae", G.dev(p), G.dev(t), g1)), oracle.mae_bwd(p, t, F(0.37)), "mae bwd")
+    # the term added to a gradient gathered so far in the same pass: gathered + term, the term rounded first
+    acc = oracle.normal((50001,), 20, 0, 1e-5)
+    acc[:50] = F(-0.0)
+    for name, want in (("mse", oracle.mse_bwd(p, t, F(0.37))), ("mae", oracle.mae_bwd(p, t, F(0.37)))):
+        bits_equal(G.host(G.loss_bwd_acc(name, G.dev(p), G.dev(t), g1, G.dev(acc))), (acc + want).astype(F), name + " bwd + gathered")
     b = (t + F(4.0) * np.sign(t) + F(0.5)).astype(F)
     bits_equal(G.host(G.div_bwd_b(G.dev(p), G.dev(b), G.dev(g[:50001]))), oracle.div_bwd_b(p, b, g[:50001]), "div bwd b")
     # row-vector divisor: the same arithmetic on the divisor repeated down the rows
