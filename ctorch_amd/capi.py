@@ -74,6 +74,11 @@ PROTOTYPES.update({
     "ctamd_fill_from_f32": [_P, _P, _Z, _P],
     "ctamd_accumulate_f32": [_P, _P, _Z, _P],
     "ctamd_mse_backward_f32": [_P, _P, _P, _P, _Z, _P],
+    "ctamd_relu_backward_acc_f32": [_P, _P, _P, _P, _Z, _P],
+    "ctamd_sigmoid_backward_acc_f32": [_P, _P, _P, _P, _Z, _P],
+    "ctamd_tanh_backward_acc_f32": [_P, _P, _P, _P, _Z, _P],
+    "ctamd_sin_backward_acc_f32": [_P, _P, _P, _P, _Z, _P],
+    "ctamd_cos_backward_acc_f32": [_P, _P, _P, _P, _Z, _P],
     "ctamd_mse_backward_acc_f32": [_P, _P, _P, _P, _P, _Z, _P],
     "ctamd_mae_backward_acc_f32": [_P, _P, _P, _P, _P, _Z, _P],
     "ctamd_mae_backward_f32": [_P, _P, _P, _P, _Z, _P],

@@ -479,6 +479,18 @@ int ctamd_mae_backward_f32(const float* p, const float* t, const float* g1, floa
     Ptrs<2> in{{p, t}};
     return launch_map<MaeBwdF>(__func__, in, dp, n, MaeBwdF{1.0 / double(float(n)), g1}, s);
 }
+// dx = acc + (the operator's gradient term), the term rounded first
+#define CTAMD_UNARY_BACKWARD_ACC(NAME, PF)                                                                              \
+    int NAME(const float* x, const float* g, const float* acc, float* dx, size_t n, void* s) {                         \
+        Ptrs<3> in{{x, g, acc}};                                                                                       \
+        return launch_map<PF>(__func__, in, dx, n, PF(), s);                                                           \
+    }
+CTAMD_UNARY_BACKWARD_ACC(ctamd_relu_backward_acc_f32, PlusF<ReluBwdF>)
+CTAMD_UNARY_BACKWARD_ACC(ctamd_sigmoid_backward_acc_f32, PlusF<SigmoidBwdF>)
+CTAMD_UNARY_BACKWARD_ACC(ctamd_tanh_backward_acc_f32, PlusF<TanhBwdF>)
+CTAMD_UNARY_BACKWARD_ACC(ctamd_sin_backward_acc_f32, PlusRareF<SinBwdF>)
+CTAMD_UNARY_BACKWARD_ACC(ctamd_cos_backward_acc_f32, PlusRareF<CosBwdF>)
+#undef CTAMD_UNARY_BACKWARD_ACC
 int ctamd_mse_backward_acc_f32(const float* p, const float* t, const float* g1, const float* acc, float* dp, size_t n, void* s) {
     if (n && !g1) return fail(CTAMD_EINVAL, "%s: null upstream gradient", __func__);
     Ptrs<3> in{{p, t, acc}};

@@ -141,6 +141,13 @@ struct PlusF { static constexpr int kIn = F::kIn + 1; static constexpr bool kTab
     __device__ float operator()(const float* x, const Tables& t) const {
         float term = f(x, t);
         return x[F::kIn] + term; } };
+// the same around a functor with a rare slow path (SinBwdF, CosBwdF)
+template <class F>
+struct PlusRareF : PlusF<F> { static constexpr bool kRare = true;
+    __device__ bool rare(const float* x) const { return this->f.rare(x); }
+    __device__ float slow(const float* x, const Tables& t) const {
+        float term = this->f.slow(x, t);
+        return x[F::kIn] + term; } };
 // inputs (a, b, g): ((-a) * g) / (b * b)
 struct DivBwdBF { static constexpr int kIn = 3; static constexpr bool kTables = false;
     __device__ float operator()(const float* x, const Tables&) const {

@@ -382,6 +382,15 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
                     continue;
                 }
             }
+            // likewise the gradient of a unary operator whose operand other operators use as well
+            if ((node->operation == op::ReLU || node->operation == op::Sigmoid || node->operation == op::Tanh ||
+                 node->operation == op::Sin || node->operation == op::Cos) && in->grad && in->grad->is_contiguous() &&
+                in->grad->sizes() == in->tensor->sizes() && node_grad.sizes() == in->tensor->sizes() &&
+                node_grad.is_contiguous() && in->tensor->device() == DeviceType::kAMD) {
+                in->grad = std::make_unique<Tensor>(unary_backward_plus(node->operation, *in->tensor, node_grad, *in->grad));
+                in->grad_plus_zero = false;          // g * 0 may be -0, and -0 + -0 is -0
+                continue;
+            }
             Tensor val = input_gradient(node, input_id, pos, node_grad);
             Tensor adj = adjust_grad_shape(val, in->tensor->sizes());
             const bool plus_zero = term_plus_zero_;

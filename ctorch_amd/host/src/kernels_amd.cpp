@@ -357,6 +357,20 @@ Tensor mae_backward(const Tensor& p, const Tensor& t, const Tensor& g) {
     run(ctamd_mae_backward_f32(p.fptr(), t.fptr(), g.fptr(), r.fptr(), p.numel(), current_stream()), "mae_backward");
     return r;
 }
+Tensor unary_backward_plus(op which, const Tensor& x, const Tensor& g, const Tensor& acc) {
+    check_device(x, "backward");
+    check_device(g, "backward");
+    check_device(acc, "backward");
+    if (g.numel() != x.numel() || acc.numel() != x.numel())
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "backward: sizes differ");
+    typedef int (*Fn)(const float*, const float*, const float*, float*, size_t, void*);
+    const Fn fn = which == op::ReLU ? ctamd_relu_backward_acc_f32 : which == op::Sigmoid ? ctamd_sigmoid_backward_acc_f32
+                : which == op::Tanh ? ctamd_tanh_backward_acc_f32 : which == op::Sin ? ctamd_sin_backward_acc_f32
+                                                                                      : ctamd_cos_backward_acc_f32;
+    Tensor r = like(x);
+    run(fn(x.fptr(), g.fptr(), acc.fptr(), r.fptr(), x.numel(), current_stream()), "backward");
+    return r;
+}
 Tensor loss_backward_plus(bool mae, const Tensor& p, const Tensor& t, const Tensor& g, const Tensor& acc) {
     check_device(p, "loss_backward");
     check_device(acc, "loss_backward");

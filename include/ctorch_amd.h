@@ -299,6 +299,15 @@ int ctamd_tanh_backward_f32(const float* x, const float* g, float* dx, size_t n,
 /* dx = cos(x) * g; dx = (-sin(x)) * g.  src/AutoDiff.cpp:1399-1407, :1408-1416. */
 int ctamd_sin_backward_f32(const float* x, const float* g, float* dx, size_t n, void* stream);
 int ctamd_cos_backward_f32(const float* x, const float* g, float* dx, size_t n, void* stream);
+/* The five gradients above with the gradient gathered so far added in the same pass:
+ * dx[i] = acc[i] + term[i], the term rounded first - what the entry point above followed by
+ * ctamd_accumulate_f32 leaves (src/AutoDiff.cpp:1870-1907), in 16 instead of 24 bytes per element.
+ * For an operand that other operators use as well. */
+int ctamd_relu_backward_acc_f32(const float* x, const float* g, const float* acc, float* dx, size_t n, void* stream);
+int ctamd_sigmoid_backward_acc_f32(const float* x, const float* g, const float* acc, float* dx, size_t n, void* stream);
+int ctamd_tanh_backward_acc_f32(const float* x, const float* g, const float* acc, float* dx, size_t n, void* stream);
+int ctamd_sin_backward_acc_f32(const float* x, const float* g, const float* acc, float* dx, size_t n, void* stream);
+int ctamd_cos_backward_acc_f32(const float* x, const float* g, const float* acc, float* dx, size_t n, void* stream);
 /* dx = y * (g - sum_j g*y) per row (dim 1) or per column (dim 0), y the stored softmax output.
  * src/AutoDiff.cpp:1462-1472, :1473-1484. */
 int ctamd_softmax_backward_rows_f32(const float* y, const float* g, float* dx, size_t rows, size_t cols,

@@ -166,6 +166,12 @@ def loss_bwd(name, p, t, g1):
     return dp
 
 
+def unary_bwd_acc(name, x, g, acc):
+    dx = torch.empty_like(x)
+    call("ctamd_%s_backward_acc_f32" % name, ptr(x), ptr(g), ptr(acc), ptr(dx), x.numel(), stream())
+    return dx
+
+
 def loss_bwd_acc(name, p, t, g1, acc):
     dp = torch.empty_like(p)
     call("ctamd_%s_backward_acc_f32" % name, ptr(p), ptr(t), ptr(g1), ptr(acc), ptr(dp), p.numel(), stream())

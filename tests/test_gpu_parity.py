@@ -154,6 +154,17 @@ def test_elementwise_gradients(oracle):
     bits_equal(G.host(G.unary_bwd("relu", dx, dg)), oracle.relu_bwd(x, g), "relu bwd")
     for name, code in [("sigmoid", SIGMOID), ("tanh", TANH), ("sin", SIN), ("cos", COS)]:
         ulp_close(G.host(G.unary_bwd(name, dx, dg)), oracle.unary_bwd(code, x, g), 2, name + " bwd")
+    # the same gradients added to a gradient gathered so far: bit for bit the separate kernel, then "+"
+    gathered = np.concatenate([oracle.normal((50001,), 21, 0, 1), SPECIAL[:32]])
+    gathered[:64] = F(-0.0)
+    dacc = G.dev(gathered)
+    with np.errstate(invalid="ignore", over="ignore"):
+        for name in ("relu", "sigmoid", "tanh", "sin", "cos"):
+            sep = G.host(G.unary_bwd(name, dx, dg))
+            got = G.host(G.unary_bwd_acc(name, dx, dg, dacc))
+            want = (gathered + sep).astype(F)
+            both_nan = np.isnan(got) & np.isnan(want)
+            assert np.array_equal(np.where(both_nan, 0, got.view(np.uint32)), np.where(both_nan, 0, want.view(np.uint32))), name
     p = oracle.normal((50001,), 18, 0, 2)
     t = oracle.normal((50001,), 19, 0, 2)
     t[:100] = p[:100]           # exact ties: sign(0) = 0
