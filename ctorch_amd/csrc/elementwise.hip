@@ -479,6 +479,11 @@ int ctamd_mae_backward_f32(const float* p, const float* t, const float* g1, floa
     Ptrs<2> in{{p, t}};
     return launch_map<MaeBwdF>(__func__, in, dp, n, MaeBwdF{1.0 / double(float(n)), g1}, s);
 }
+// out = acc + a * b, the product rounded first (the gradient term of Mul joining a gathered gradient)
+int ctamd_mul_acc_f32(const float* a, const float* b, const float* acc, float* out, size_t n, void* s) {
+    Ptrs<3> in{{a, b, acc}};
+    return launch_map<PlusF<MulF>>(__func__, in, out, n, PlusF<MulF>(), s);
+}
 // dx = acc + (the operator's gradient term), the term rounded first
 #define CTAMD_UNARY_BACKWARD_ACC(NAME, PF)                                                                              \
     int NAME(const float* x, const float* g, const float* acc, float* dx, size_t n, void* s) {                         \

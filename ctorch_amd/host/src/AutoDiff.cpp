@@ -391,6 +391,26 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
                 in->grad_plus_zero = false;          // g * 0 may be -0, and -0 + -0 is -0
                 continue;
             }
+            // and Neg, the second operand of Sub (gathered + (-g) is gathered - g, bit for bit) and
+            // Mul of two full tensors (gathered + other * g)
+            const bool joinable = in->grad && in->grad->is_contiguous() && in->grad->sizes() == in->tensor->sizes() &&
+                                  node_grad.sizes() == in->tensor->sizes() && node_grad.is_contiguous() &&
+                                  in->tensor->device() == DeviceType::kAMD;
+            if (joinable && (node->operation == op::Neg ||
+                             (node->operation == op::Sub && node->input_ids.size() == 2 && input_id != node->input_ids[0]))) {
+                in->grad = std::make_unique<Tensor>(Sub_AMD_kernel(*in->grad, node_grad));
+                in->grad_plus_zero = false;
+                continue;
+            }
+            if (joinable && node->operation == op::Mul && node->input_ids.size() == 2 && node->input_ids[0] != node->input_ids[1]) {
+                Node* o = find(input_id == node->input_ids[0] ? node->input_ids[1] : node->input_ids[0]);
+                if (o && o->tensor->device() == DeviceType::kAMD && o->tensor->sizes() == in->tensor->sizes() &&
+                    o->tensor->is_contiguous()) {
+                    in->grad = std::make_unique<Tensor>(mul_plus(*o->tensor, node_grad, *in->grad));
+                    in->grad_plus_zero = false;
+                    continue;
+                }
+            }
             Tensor val = input_gradient(node, input_id, pos, node_grad);
             Tensor adj = adjust_grad_shape(val, in->tensor->sizes());
             const bool plus_zero = term_plus_zero_;

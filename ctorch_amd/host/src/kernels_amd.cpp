@@ -371,6 +371,16 @@ Tensor unary_backward_plus(op which, const Tensor& x, const Tensor& g, const Ten
     run(fn(x.fptr(), g.fptr(), acc.fptr(), r.fptr(), x.numel(), current_stream()), "backward");
     return r;
 }
+Tensor mul_plus(const Tensor& a, const Tensor& b, const Tensor& acc) {
+    check_device(a, "backward");
+    check_device(b, "backward");
+    check_device(acc, "backward");
+    if (a.numel() != b.numel() || acc.numel() != a.numel())
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "backward: sizes differ");
+    Tensor r = like(acc);
+    run(ctamd_mul_acc_f32(a.fptr(), b.fptr(), acc.fptr(), r.fptr(), a.numel(), current_stream()), "backward");
+    return r;
+}
 Tensor loss_backward_plus(bool mae, const Tensor& p, const Tensor& t, const Tensor& g, const Tensor& acc) {
     check_device(p, "loss_backward");
     check_device(acc, "loss_backward");

@@ -308,6 +308,9 @@ int ctamd_sigmoid_backward_acc_f32(const float* x, const float* g, const float* 
 int ctamd_tanh_backward_acc_f32(const float* x, const float* g, const float* acc, float* dx, size_t n, void* stream);
 int ctamd_sin_backward_acc_f32(const float* x, const float* g, const float* acc, float* dx, size_t n, void* stream);
 int ctamd_cos_backward_acc_f32(const float* x, const float* g, const float* acc, float* dx, size_t n, void* stream);
+/* out[i] = acc[i] + a[i] * b[i], the product rounded first: the Mul gradient term other * g
+ * (src/AutoDiff.cpp:1234-1258) joining a gathered gradient (:1870-1907) in one pass. */
+int ctamd_mul_acc_f32(const float* a, const float* b, const float* acc, float* out, size_t n, void* stream);
 /* dx = y * (g - sum_j g*y) per row (dim 1) or per column (dim 0), y the stored softmax output.
  * src/AutoDiff.cpp:1462-1472, :1473-1484. */
 int ctamd_softmax_backward_rows_f32(const float* y, const float* g, float* dx, size_t rows, size_t cols,

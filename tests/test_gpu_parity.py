@@ -165,6 +165,11 @@ def test_elementwise_gradients(oracle):
             want = (gathered + sep).astype(F)
             both_nan = np.isnan(got) & np.isnan(want)
             assert np.array_equal(np.where(both_nan, 0, got.view(np.uint32)), np.where(both_nan, 0, want.view(np.uint32))), name
+        out = torch.empty_like(dx)
+        G.call("ctamd_mul_acc_f32", G.ptr(dx), G.ptr(dg), G.ptr(dacc), G.ptr(out), dx.numel(), G.stream())
+        want = (gathered + (x * g).astype(F)).astype(F)
+        both_nan = np.isnan(G.host(out)) & np.isnan(want)
+        assert np.array_equal(np.where(both_nan, 0, G.host(out).view(np.uint32)), np.where(both_nan, 0, want.view(np.uint32))), "mul + gathered"
     p = oracle.normal((50001,), 18, 0, 2)
     t = oracle.normal((50001,), 19, 0, 2)
     t[:100] = p[:100]           # exact ties: sign(0) = 0
