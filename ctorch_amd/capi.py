@@ -80,6 +80,8 @@ PROTOTYPES.update({
     "ctamd_sin_backward_acc_f32": [_P, _P, _P, _P, _Z, _P],
     "ctamd_cos_backward_acc_f32": [_P, _P, _P, _P, _Z, _P],
     "ctamd_mul_acc_f32": [_P, _P, _P, _P, _Z, _P],
+    "ctamd_div_acc_f32": [_P, _P, _P, _P, _Z, _P],
+    "ctamd_div_rowbcast_acc_f32": [_P, _P, _P, _P, _Z, _Z, _P],
     "ctamd_mse_backward_acc_f32": [_P, _P, _P, _P, _P, _Z, _P],
     "ctamd_mae_backward_acc_f32": [_P, _P, _P, _P, _P, _Z, _P],
     "ctamd_mae_backward_f32": [_P, _P, _P, _P, _Z, _P],

@@ -484,6 +484,15 @@ int ctamd_mul_acc_f32(const float* a, const float* b, const float* acc, float* o
     Ptrs<3> in{{a, b, acc}};
     return launch_map<PlusF<MulF>>(__func__, in, out, n, PlusF<MulF>(), s);
 }
+// out = acc + a / b, the quotient rounded first (Div's gradient term g / b joining a gathered
+// gradient); b of a's shape, or a row vector under a [rows, cols]
+int ctamd_div_acc_f32(const float* a, const float* b, const float* acc, float* out, size_t n, void* s) {
+    Ptrs<3> in{{a, b, acc}};
+    return launch_map<PlusF<DivF>>(__func__, in, out, n, PlusF<DivF>(), s);
+}
+int ctamd_div_rowbcast_acc_f32(const float* a, const float* b, const float* acc, float* out, size_t rows, size_t cols, void* s) {
+    return launch_rowbcast<PlusF<DivF>>(__func__, a, b, out, rows, cols, s, acc);
+}
 // dx = acc + (the operator's gradient term), the term rounded first
 #define CTAMD_UNARY_BACKWARD_ACC(NAME, PF)                                                                              \
     int NAME(const float* x, const float* g, const float* acc, float* dx, size_t n, void* s) {                         \

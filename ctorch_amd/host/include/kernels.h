@@ -75,6 +75,8 @@ Tensor mse_backward(const Tensor& p, const Tensor& t, const Tensor& g0d);
 Tensor mae_backward(const Tensor& p, const Tensor& t, const Tensor& g0d);
 // acc + the gradient of ReLU / Sigmoid / Tanh / Sin / Cos at x, in the pass that forms it
 Tensor unary_backward_plus(op which, const Tensor& x, const Tensor& g, const Tensor& acc);
+// acc + g / b (the quotient rounded first), one pass; b of g's shape or a row vector under it
+Tensor div_plus(const Tensor& g, const Tensor& b, const Tensor& acc);
 // acc + a * b (the product rounded first), one pass
 Tensor mul_plus(const Tensor& a, const Tensor& b, const Tensor& acc);
 // acc + the MSE (mae = false) or MAE gradient, in the pass that forms it

@@ -411,6 +411,21 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
                     continue;
                 }
             }
+            // and the first operand of Div by a full tensor or a row vector (gathered + g / b), after the
+            // zero-divisor check the Div branch makes
+            if (joinable && node->operation == op::Div && node->input_ids.size() == 2 && input_id == node->input_ids[0] &&
+                node->input_ids[0] != node->input_ids[1]) {
+                Node* bn = find(node->input_ids[1]);
+                if (bn && bn->tensor->device() == DeviceType::kAMD && bn->tensor->is_contiguous() &&
+                    (bn->tensor->sizes() == in->tensor->sizes() || is_row_vector_of(*bn->tensor, *in->tensor))) {
+                    if (check_div_zero_ && any_abs_lt_eps(*bn->tensor))
+                        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::TENSOR_STATE,
+                                                     "division by zero in the gradient of Div");
+                    in->grad = std::make_unique<Tensor>(div_plus(node_grad, *bn->tensor, *in->grad));
+                    in->grad_plus_zero = false;
+                    continue;
+                }
+            }
             Tensor val = input_gradient(node, input_id, pos, node_grad);
             Tensor adj = adjust_grad_shape(val, in->tensor->sizes());
             const bool plus_zero = term_plus_zero_;

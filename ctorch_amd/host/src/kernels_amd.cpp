@@ -381,6 +381,19 @@ Tensor mul_plus(const Tensor& a, const Tensor& b, const Tensor& acc) {
     run(ctamd_mul_acc_f32(a.fptr(), b.fptr(), acc.fptr(), r.fptr(), a.numel(), current_stream()), "backward");
     return r;
 }
+Tensor div_plus(const Tensor& g, const Tensor& b, const Tensor& acc) {
+    check_device(g, "backward");
+    check_device(b, "backward");
+    check_device(acc, "backward");
+    if (acc.numel() != g.numel())
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "backward: sizes differ");
+    Tensor r = like(acc);
+    if (b.numel() == g.numel())
+        run(ctamd_div_acc_f32(g.fptr(), b.fptr(), acc.fptr(), r.fptr(), g.numel(), current_stream()), "backward");
+    else
+        run(ctamd_div_rowbcast_acc_f32(g.fptr(), b.fptr(), acc.fptr(), r.fptr(), g.sizes()[0], g.sizes()[1], current_stream()), "backward");
+    return r;
+}
 Tensor loss_backward_plus(bool mae, const Tensor& p, const Tensor& t, const Tensor& g, const Tensor& acc) {
     check_device(p, "loss_backward");
     check_device(acc, "loss_backward");

@@ -311,6 +311,12 @@ int ctamd_cos_backward_acc_f32(const float* x, const float* g, const float* acc,
 /* out[i] = acc[i] + a[i] * b[i], the product rounded first: the Mul gradient term other * g
  * (src/AutoDiff.cpp:1234-1258) joining a gathered gradient (:1870-1907) in one pass. */
 int ctamd_mul_acc_f32(const float* a, const float* b, const float* acc, float* out, size_t n, void* stream);
+/* out[i] = acc[i] + a[i] / b[i], the quotient rounded first: Div's gradient term for its first
+ * operand, g / b (src/AutoDiff.cpp:1285), joining a gathered gradient; b of a's shape, or (rowbcast) a
+ * row vector [cols] under a [rows, cols]. */
+int ctamd_div_acc_f32(const float* a, const float* b, const float* acc, float* out, size_t n, void* stream);
+int ctamd_div_rowbcast_acc_f32(const float* a, const float* b, const float* acc, float* out, size_t rows, size_t cols,
+                               void* stream);
 /* dx = y * (g - sum_j g*y) per row (dim 1) or per column (dim 0), y the stored softmax output.
  * src/AutoDiff.cpp:1462-1472, :1473-1484. */
 int ctamd_softmax_backward_rows_f32(const float* y, const float* g, float* dx, size_t rows, size_t cols,

@@ -170,6 +170,17 @@ def test_elementwise_gradients(oracle):
         want = (gathered + (x * g).astype(F)).astype(F)
         both_nan = np.isnan(G.host(out)) & np.isnan(want)
         assert np.array_equal(np.where(both_nan, 0, G.host(out).view(np.uint32)), np.where(both_nan, 0, want.view(np.uint32))), "mul + gathered"
+        G.call("ctamd_div_acc_f32", G.ptr(dx), G.ptr(dg), G.ptr(dacc), G.ptr(out), dx.numel(), G.stream())
+        want = (gathered + (x / g).astype(F)).astype(F)
+        both_nan = np.isnan(G.host(out)) & np.isnan(want)
+        assert np.array_equal(np.where(both_nan, 0, G.host(out).view(np.uint32)), np.where(both_nan, 0, want.view(np.uint32))), "div + gathered"
+    for rows, cols in ((37, 53), (129, 1024)):
+        a2, acc2 = oracle.normal((rows, cols), 83, 0, 2), oracle.normal((rows, cols), 84)
+        rv = oracle.uniform((cols,), 85, 0.5, 2)
+        out2 = torch.empty(rows, cols, device=G.DEV)
+        da2, drv, dacc2 = G.dev(a2), G.dev(rv), G.dev(acc2)        # held: a pointer does not keep a tensor alive
+        G.call("ctamd_div_rowbcast_acc_f32", G.ptr(da2), G.ptr(drv), G.ptr(dacc2), G.ptr(out2), rows, cols, G.stream())
+        bits_equal(G.host(out2), (acc2 + (a2 / rv).astype(F)).astype(F), "row-vector div + gathered")
     p = oracle.normal((50001,), 18, 0, 2)
     t = oracle.normal((50001,), 19, 0, 2)
     t[:100] = p[:100]           # exact ties: sign(0) = 0
