@@ -65,8 +65,11 @@ def build(verbose=False, jobs=4):
 
 def _kernel_resources(src, out, table):
     """Moves the compiler's per-kernel resource remarks from `out` into `table`; returns the rest."""
-    rest, name = [], None
+    rest, name, after_remark = [], None, False
     for line in out.splitlines():
+        if after_remark and re.match(r"\s+(\d+ )?\|", line):      # the source excerpt under a remark
+            continue
+        after_remark = "[-Rpass-analysis=kernel-resource-usage]" in line
         m = re.search(r"remark: (?:\s*)(Function Name|VGPRs|VGPRs Spill|SGPRs Spill|LDS Size \[bytes/block\]|Occupancy \[waves/SIMD\]|"
                       r"ScratchSize \[bytes/lane\]|AGPRs|SGPRs|Dynamic Stack|TotalSGPRs): (\S+)", line)
         if not m:
