@@ -214,6 +214,7 @@ void accumulate(Tensor& grad, const Tensor& val) {
     if (grad.numel() != val.numel())
         Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "accumulate: gradient sizes differ");
     run(ctamd_accumulate_f32(grad.fptr(), val.fptr(), grad.numel(), current_stream()), "accumulate");
+    grad.forget_known_value();      // written in place: whatever the host knew of it is gone
 }
 // grad = 0 + val in one pass: what the reference's "zero-filled gradient, then grad[i] += val[i]"
 // (src/AutoDiff.cpp:1870-1907) leaves after the first contribution, bit for bit (-0 becomes +0).
