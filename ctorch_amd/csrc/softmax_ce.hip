@@ -408,6 +408,106 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
 // Streaming variant for rows that do not fit a block's registers: pass 1 keeps an online
 // (max, sum) pair per thread - sum is rescaled by exp(old_max - new_max) whenever the max grows -
 // pass 2 re-reads the row.  The rescaled sum differs from sum(exp(x - max)) by rounding only.
+// The same for softmax and its gradient with 128-bit accesses (rows of a multiple of four columns,
+// 16-byte aligned): four vectors in flight per thread, the row sum of the first sweep from the
+// hardware exp2 (only the sum is formed from it, ~1e-7 relative; the output sweep uses the bit-exact
+// exponential and the exact quotient), plain loads so that the second sweep finds the row in the
+// memory-side cache (one block per CU keeps 256 rows in flight), results written past the caches.
+template <int MODE>
+__global__ __launch_bounds__(1024) void row_stream_vec_kernel(Args a) {
+    constexpr int THREADS = 1024, U = 4;
+    static_assert(MODE == kSoftmax || MODE == kSoftmaxBwd, "only the two modes that write a row-shaped result");
+    __shared__ uint64_t s_exp2[32];
+    __shared__ float s_f[2][THREADS / 64 + 1];
+    stage_exp_table(s_exp2);
+    const unsigned n4 = unsigned(a.cols >> 2);
+    for (size_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
+        const v4f* __restrict__ xr = reinterpret_cast<const v4f*>(a.x + row * a.cols);
+        v4f* __restrict__ outr = reinterpret_cast<v4f*>(a.out + row * a.cols);
+        if (MODE == kSoftmaxBwd) {
+            const v4f* __restrict__ gr = reinterpret_cast<const v4f*>(a.t + row * a.cols);
+            float d0 = 0.0f, d1 = 0.0f;
+            unsigned i = threadIdx.x;
+            for (; i + (U / 2 - 1) * THREADS < n4; i += (U / 2) * THREADS) {
+                v4f y[U / 2], g[U / 2];
+#pragma unroll
+                for (int u = 0; u < U / 2; ++u) { y[u] = xr[i + u * THREADS]; g[u] = gr[i + u * THREADS]; }
+#pragma unroll
+                for (int u = 0; u < U / 2; ++u) {
+                    d0 += g[u][0] * y[u][0] + g[u][1] * y[u][1];
+                    d1 += g[u][2] * y[u][2] + g[u][3] * y[u][3];
+                }
+            }
+            for (; i < n4; i += THREADS) {
+                const v4f y = xr[i], g = gr[i];
+                d0 += g[0] * y[0] + g[1] * y[1];
+                d1 += g[2] * y[2] + g[3] * y[3];
+            }
+            const float d = block_sum<THREADS>(d0 + d1, s_f[0]);
+            i = threadIdx.x;
+            for (; i + (U / 2 - 1) * THREADS < n4; i += (U / 2) * THREADS) {
+                v4f y[U / 2], g[U / 2];
+#pragma unroll
+                for (int u = 0; u < U / 2; ++u) { y[u] = xr[i + u * THREADS]; g[u] = gr[i + u * THREADS]; }
+#pragma unroll
+                for (int u = 0; u < U / 2; ++u) {
+                    v4f o;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o[e] = y[u][e] * (g[u][e] - d);
+                    __builtin_nontemporal_store(o, outr + i + u * THREADS);
+                }
+            }
+            for (; i < n4; i += THREADS) {
+                const v4f y = xr[i], g = gr[i];
+                v4f o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = y[e] * (g[e] - d);
+                __builtin_nontemporal_store(o, outr + i);
+            }
+            continue;
+        }
+        float m = kNegInf, s = 0.0f;
+        auto take = [&](const v4f& v) {
+            const float vm = __builtin_fmaxf(__builtin_fmaxf(v[0], v[1]), __builtin_fmaxf(v[2], v[3]));
+            if (vm > m) {
+                s *= __builtin_amdgcn_exp2f((m - vm) * 1.44269504088896340736f);      // exp2(-inf) = 0 at the first vector
+                m = vm;
+            }
+            const float b = (m == kNegInf) ? 0.0f : m;
+            s += (__builtin_amdgcn_exp2f((v[0] - b) * 1.44269504088896340736f) + __builtin_amdgcn_exp2f((v[1] - b) * 1.44269504088896340736f)) +
+                 (__builtin_amdgcn_exp2f((v[2] - b) * 1.44269504088896340736f) + __builtin_amdgcn_exp2f((v[3] - b) * 1.44269504088896340736f));
+        };
+        unsigned i = threadIdx.x;
+        for (; i + (U - 1) * THREADS < n4; i += U * THREADS) {
+            v4f v[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) v[u] = xr[i + u * THREADS];
+#pragma unroll
+            for (int u = 0; u < U; ++u) take(v[u]);
+        }
+        for (; i < n4; i += THREADS) take(xr[i]);
+        const float M = block_max<THREADS>(m, s_f[0]);
+        s = (m == kNegInf) ? 0.0f : s * __builtin_amdgcn_exp2f((m - M) * 1.44269504088896340736f);
+        const float S = block_sum<THREADS>(s, s_f[1]);
+        const double rcp = 1.0 / double(S);
+        auto give = [&](const v4f& v, unsigned at) {
+            v4f o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = cta_div_rcp(cta_expf_nonpos(v[e] - M, s_exp2), rcp);
+            __builtin_nontemporal_store(o, outr + at);
+        };
+        i = threadIdx.x;
+        for (; i + (U - 1) * THREADS < n4; i += U * THREADS) {
+            v4f v[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) v[u] = xr[i + u * THREADS];
+#pragma unroll
+            for (int u = 0; u < U; ++u) give(v[u], i + u * THREADS);
+        }
+        for (; i < n4; i += THREADS) give(xr[i], i);
+    }
+}
+
 template <int MODE>
 __global__ __launch_bounds__(1024) void row_stream_kernel(Args a) {
     constexpr int THREADS = 1024;
@@ -713,7 +813,10 @@ int run_rows(const char* name, Args a, float* loss_out, void* stream) {
         if constexpr (kBoth)
             return fail(CTAMD_ERANGE, "%s: a row does not fit a block's registers (32768 columns, 8192 without 128-bit accesses): "
                         "use the separate forward and backward entry points", name);
-        else
+        else if constexpr (MODE == kSoftmax || MODE == kSoftmaxBwd) {
+            if (vec) hipLaunchKernelGGL((row_stream_vec_kernel<MODE>), dim3(grid), dim3(1024), 0, s, a);
+            else hipLaunchKernelGGL((row_stream_kernel<MODE>), dim3(grid), dim3(1024), 0, s, a);
+        } else
             hipLaunchKernelGGL((row_stream_kernel<MODE>), dim3(grid), dim3(1024), 0, s, a);
     }
     int rc = launched(name);

@@ -173,6 +173,16 @@ def main():
     row("softmax backward rows", lambda: call("ctamd_softmax_backward_rows_f32", P(Y), P(X), P(Y), rows, cols, S), 12)
     del X, Y
     torch.cuda.empty_cache()
+    # rows beyond what a block keeps in registers (more than 32768 columns): two sweeps per row
+    rows, cols = 4096, 65536
+    X = torch.randn(rows, cols, device="cuda") * 2
+    Y = torch.empty_like(X)
+    G2 = torch.randn(rows, cols, device="cuda")
+    report("softmax rows [4096 x 65536] (8 B/elem)", timeit(lambda: call("ctamd_softmax_rows_f32", P(X), P(Y), rows, cols, S), 10), 8 * rows * cols)
+    report("softmax backward rows [4096 x 65536] (12 B/elem)",
+           timeit(lambda: call("ctamd_softmax_backward_rows_f32", P(Y), P(G2), P(X), rows, cols, S), 10), 12 * rows * cols)
+    del X, Y, G2
+    torch.cuda.empty_cache()
 
     # ---- fp32 MatMul, square, the three operand layouts
     if not args.skip_matmul:
