@@ -257,7 +257,10 @@ def test_softmax_and_cross_entropy_rows(oracle, shape):
     e64 = np.exp(x64 - x64.max(1, keepdims=True))
     y64 = e64 / e64.sum(1, keepdims=True)
     assert np.all(np.abs(y - y64) <= 1e-5 * y64 + 1e-45)
-    assert np.all(np.abs(y - want) <= 1e-5 * want + 1e-45)
+    # (beyond 65536 columns the reference's own sequential fp32 sum has drifted from the true sum by
+    # more than 1e-5: ~sqrt(cols) roundings of 2^-24 each; the fp64 arbiter above keeps the 1e-5 bar)
+    ref_tol = 1e-5 if cols <= 65536 else 4 * np.sqrt(cols) * 2.0 ** -24
+    assert np.all(np.abs(y - want) <= ref_tol * want + 1e-45)
     assert np.allclose(y.astype(np.float64).sum(1), 1, atol=1e-5)
     idx = oracle.ints((rows,), 25, cols)
     oh = np.zeros(shape, F)
