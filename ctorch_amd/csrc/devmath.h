@@ -65,12 +65,26 @@ CTA_FN double cta_u2d(uint64_t u) {
 }
 
 // a / b for a divisor shared by many elements: with rcp_b = 1.0 / (double)b computed once,
-// (float)((double)a * rcp_b) IS the correctly rounded fp32 quotient.  The exact quotient of two
-// 24-bit significands lies at least 2^-49 (relative) away from every midpoint between adjacent
-// floats and can never sit on one (that would need 2^25 to divide a 24-bit integer), while the
-// double product is within 2^-52 of it; zeros, infinities, NaN and subnormals come out as IEEE
-// division gives them.  tests/native/divcheck.c compares it with `a / b` on billions of pairs.
-CTA_FN float cta_div_rcp(float a, double rcp_b) { return (float)((double)a * rcp_b); }
+// the double product q = (double)a * rcp_b lies within 2^-52 (relative) of the exact quotient.
+// Normal results: the exact quotient of two 24-bit significands is at least 2^-49 (relative) away
+// from every midpoint between adjacent floats and can never sit on one (that would need 2^25 to
+// divide a 24-bit integer), so (float)q is the correctly rounded fp32 quotient.  Subnormal results
+// are rounded at a fixed position (multiples of 2^-149), where the exact quotient CAN be a midpoint
+// (a = 147 * 2^-149, b = 98) and q, a hair off it, would break the tie the wrong way.  There, in
+// units of 2^-150, a quotient that is not an integer is at least 2^-24 away from every integer while
+// q is at most 2^-28 away from the quotient: a q within 2^-26 of an integer is moved onto it, which
+// restores every exact quotient - the midpoints among them - and touches nothing else.  Zeros,
+// infinities and NaN come out as IEEE division gives them.  tests/native/divcheck.c compares it with
+// `a / b` on random pairs and on the midpoint family a = M * B * 2^-149, b = 2 * B.
+CTA_FN float cta_div_rcp(float a, double rcp_b) {
+    double q = (double)a * rcp_b;
+    if (__builtin_expect(__builtin_fabs(q) < 0x1p-126, 0)) {
+        double t = q * 0x1p150;
+        double m = __builtin_rint(t);
+        if (__builtin_fabs(t - m) < 0x1p-26) q = m * 0x1p-150;
+    }
+    return (float)q;
+}
 
 // tab[i] = bits(2^(i/32)) - (i << 47): adding k << 47 yields bits(2^(k/32)) for any integer k.
 CTA_TAB_SPACE uint64_t cta_exp2_tab[32] = {

@@ -1,7 +1,9 @@
 /* Host check of cta_div_rcp (ctorch_amd/csrc/devmath.h): division by a shared divisor through its
  * double-precision reciprocal against IEEE fp32 division, on random operand pairs that include
  * subnormal numerators and divisors, numerators <= 1 with divisors >= 1 (the softmax case) and the
- * full exponent range.  Usage: divcheck [PAIRS_PER_THREAD]; prints "tested N bad M". */
+ * full exponent range, then on the family whose exact quotient is a midpoint between two subnormal
+ * floats (a = M * B * 2^-149 with M odd, b = 2 * B: the quotient is (M / 2) * 2^-149), both signs.
+ * Usage: divcheck [PAIRS_PER_THREAD]; prints "tested N bad M" and "ties N bad M". */
 #include <stdio.h>
 #include <stdint.h>
 #include <string.h>
@@ -32,5 +34,18 @@ int main(int argc,char**argv){
     }
   }
   printf("tested %llu bad %llu\n",(unsigned long long)total,(unsigned long long)bad);
+  uint64_t tbad=0,ties=0;
+  #pragma omp parallel for reduction(+:tbad,ties) schedule(dynamic,8)
+  for(int B=1;B<1024;++B){
+    for(uint32_t M=1;(uint64_t)M*B<(1u<<24);M+=2){
+      float a=ldexpf((float)(M*(uint32_t)B),-149), b=(float)(2*B);
+      if(M&2){ a=-a; }
+      volatile double rb=1.0/(double)b;
+      float q1=cta_div_rcp(a,rb), q2=a/b;
+      ++ties;
+      if(f2u(q1)!=f2u(q2)){ ++tbad; if(tbad<5) printf("tie a=%a b=%a fast=%a ieee=%a\n",a,b,q1,q2);}
+    }
+  }
+  printf("ties %llu bad %llu\n",(unsigned long long)ties,(unsigned long long)tbad);
   return 0;
 }

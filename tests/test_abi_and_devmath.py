@@ -74,14 +74,16 @@ def test_device_math_matches_glibc_on_a_strided_sweep(tmp_path):
 
 def test_division_through_a_double_reciprocal_is_ieee_division(tmp_path):
     """cta_div_rcp (softmax normalisation, x / n in the loss gradients, tensor / scalar) against a / b
-    on 64 million random pairs incl. subnormals; the argument in devmath.h says it is exact."""
+    on 64 million random pairs incl. subnormals, and on the 63 million operand pairs whose exact quotient
+    is a midpoint between two subnormal floats (where the plain product would break the tie wrongly)."""
     exe = str(tmp_path / "divcheck")
     subprocess.check_call(["gcc", "-O2", "-fopenmp", "-ffp-contract=off", "-o", exe,
                            os.path.join(ROOT, "tests", "native", "divcheck.c"), "-lm"])
     out = subprocess.check_output([exe, "1000000"], text=True)
     print(out)
-    f = out.strip().split()
-    assert int(f[1]) == 64_000_000 and int(f[3]) == 0
+    rand, ties = [l.split() for l in out.strip().splitlines()[-2:]]
+    assert rand[0] == "tested" and int(rand[1]) == 64_000_000 and int(rand[3]) == 0
+    assert ties[0] == "ties" and int(ties[1]) > 60_000_000 and int(ties[3]) == 0
 
 
 def test_no_kernel_spills_registers():

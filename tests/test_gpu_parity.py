@@ -90,6 +90,23 @@ def test_scalar_forms_bit_exact(oracle):
     bits_equal(G.host(G.scalar("div", da, 3.0)), oracle.scalar(2, a, 3.0), "scalar div")
 
 
+def test_division_by_a_shared_divisor_on_subnormal_midpoints(oracle):
+    """a = M * B * 2^-149 (M odd), b = 2 * B: the exact quotient lies halfway between two subnormal
+    floats, where IEEE division rounds to even.  Tensor / float and tensor / one-element tensor go
+    through the divisor's double reciprocal and must break those ties the same way."""
+    print("case division ties", flush=True)
+    for B in (1, 3, 49, 98, 405, 1023):
+        M = np.arange(1, min(1 << 18, (1 << 24) // B), 2, dtype=np.int64)
+        a = np.ldexp((M * B).astype(np.float64), -149).astype(F)
+        a[1::2] *= F(-1.0)
+        b = F(2 * B)
+        want = a / b
+        assert want.view(np.uint32).tolist() == oracle.scalar(2, a, float(b)).view(np.uint32).tolist()
+        da = G.dev(a)
+        bits_equal(G.host(G.scalar("div", da, float(b))), want, f"tensor / float, B={B}")
+        bits_equal(G.host(G.bscalar("div", da, G.dev(np.array([b])))), want, f"tensor / 0-D tensor, B={B}")
+
+
 def test_neg_relu_fill_accumulate_bit_exact(oracle):
     print("case neg relu fill accumulate", flush=True)
     a = np.concatenate([oracle.normal((70001,), 8, 0, 3), SPECIAL])
