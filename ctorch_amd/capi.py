@@ -48,6 +48,7 @@ for _op in ("neg", "relu", "sin", "cos", "tanh", "sigmoid"):
 PROTOTYPES.update({
     "ctamd_sum_f32": [_P, _P, _Z, _P],
     "ctamd_dot_f32": [_P, _P, _P, _Z, _P],
+    "ctamd_dot_static_f32": [_P, _P, _P, _Z, _P],
     "ctamd_mse_f32": [_P, _P, _P, _Z, _P],
     "ctamd_mae_f32": [_P, _P, _P, _Z, _P],
     "ctamd_colsum_f32": [_P, _P, _Z, _Z, _P],

@@ -26,6 +26,9 @@ float* scratch();
 // place of a vector that would lie beyond the end of a row.
 const float* pad_neg_inf();
 const float* pad_zero();
+// Looks up (once per device) the current device's address of the static partials array that
+// ctamd_dot_static_f32 uses; defined in reduce.hip next to the array.
+int static_partials(double** out);
 // Compute units of the current device (256 on MI355X); 0 before ctamd_init().
 int compute_units();
 

@@ -3,7 +3,15 @@
 // independent fp32 accumulators per thread, a wave64 butterfly, an LDS stage across the waves of
 // a block, then one block folds the per-block partials (held as doubles in the device scratch)
 // in a fixed order, so results are deterministic for a given size.
+#include <mutex>
+
 #include "common.h"
+
+// Per-block partials of ctamd_dot_static_f32, the entry point for callers that cannot allocate:
+// 2048 doubles (16 KiB) that every GPU the library runs on holds until the process ends.  In host
+// code this name is only a handle for hipGetSymbolAddress; the device address it yields (one per
+// device) is what launches are given.
+static __device__ __align__(256) double scratch_static[2048];
 
 namespace ctamd {
 namespace {
@@ -14,6 +22,12 @@ constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / 64;
 constexpr int kUnroll = 4;
 constexpr unsigned kMaxBlocks = 2048;   // partials folded by one block: keep that fold short
+static_assert(sizeof(scratch_static) == kMaxBlocks * sizeof(double), "one partial per block of the largest grid");
+
+// Device address of scratch_static on each device, looked up once per device with that device current.
+constexpr int kStaticMaxDevices = 16;
+std::mutex g_static_mu;
+double* g_static_partials[kStaticMaxDevices] = {};
 
 __device__ __forceinline__ double wave_sum(double v) {
 #pragma unroll
@@ -112,12 +126,13 @@ __global__ __launch_bounds__(kThreads) void reduce_stage2(const double* __restri
     }
 }
 
+// `partials`: room for kMaxBlocks doubles in device memory (nullptr: the per-device scratch).
 template <class T>
 int reduce(const char* name, const float* a, const float* b, float* out, int32_t* flag, size_t n, int mode,
-           void* stream) {
+           void* stream, double* partials = nullptr) {
     if ((mode != 2 && !out) || (mode == 2 && !flag)) return fail(CTAMD_EINVAL, "%s: null output", name);
     if (n && (!a || (T::kIn == 2 && !b))) return fail(CTAMD_EINVAL, "%s: null input", name);
-    double* partials = reinterpret_cast<double*>(scratch());
+    if (!partials) partials = reinterpret_cast<double*>(scratch());
     if (!partials) return CTAMD_EINVAL;
     hipStream_t s = as_stream(stream);
     unsigned grid = 0;
@@ -312,11 +327,44 @@ __global__ __launch_bounds__(kThreads) void colsum_stage2(const float* __restric
 }
 
 }  // namespace
+
+// The current device's copy of scratch_static: each GPU holds the array at its own address, so the
+// lookup runs once per device with that device current (ctamd_init calls this; a first call of
+// ctamd_dot_static_f32 on a device that was never initialised does as well).  Allocates nothing.
+int static_partials(double** out) {
+    *out = nullptr;
+    int d = -1;
+    int rc = check_hip(hipGetDevice(&d), "hipGetDevice");
+    if (rc) return rc;
+    if (d < 0 || d >= kStaticMaxDevices) return fail(CTAMD_EINVAL, "device %d out of range", d);
+    std::lock_guard<std::mutex> lock(g_static_mu);
+    if (!g_static_partials[d]) {
+        void* p = nullptr;
+        rc = check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch_static)), "hipGetSymbolAddress(scratch_static)");
+        if (rc) return rc;
+        if (!p) return fail(CTAMD_EHIP, "hipGetSymbolAddress(scratch_static) returned no address");
+        g_static_partials[d] = static_cast<double*>(p);
+    }
+    *out = g_static_partials[d];
+    return CTAMD_OK;
+}
+
 }  // namespace ctamd
 
 using namespace ctamd;
 
 extern "C" {
+
+int ctamd_dot_static_f32(const float* a, const float* b, float* out, size_t n, void* s) {
+    if (n > CTAMD_DOT_STATIC_MAX_N)
+        return fail(CTAMD_ERANGE, "%s: %zu elements exceed the supported maximum of %zu", __func__, n,
+                    size_t(CTAMD_DOT_STATIC_MAX_N));
+    double* partials = nullptr;
+    int rc = static_partials(&partials);
+    if (rc) return rc;
+    // every partial the fold launch reads was written by this call's first launch: nothing to clear
+    return reduce<DotT>(__func__, a, b, out, nullptr, n, 0, s, partials);
+}
 
 int ctamd_sum_f32(const float* a, float* out, size_t n, void* s) { return reduce<SumT>(__func__, a, nullptr, out, nullptr, n, 0, s); }
 int ctamd_dot_f32(const float* a, const float* b, float* out, size_t n, void* s) { return reduce<DotT>(__func__, a, b, out, nullptr, n, 0, s); }

@@ -119,6 +119,12 @@ int ctamd_init(int device) {
         (void)hipFree(p);
         return rc;
     }
+    double* static_scratch = nullptr;
+    rc = static_partials(&static_scratch);      // this device's address of the static partials array
+    if (rc) {
+        (void)hipFree(p);
+        return rc;
+    }
     g_scratch[device] = static_cast<float*>(p);
     return CTAMD_OK;
 }

@@ -134,6 +134,18 @@ int ctamd_dot_f32(const float* a, const float* b, float* out, size_t n, void* st
 /* out[0] = sum (a-b)^2 / n and sum |a-b| / n.  MSE_BASIC_kernel.cpp:35-43, MAE_BASIC_kernel.cpp:35-43. */
 int ctamd_mse_f32(const float* a, const float* b, float* out, size_t n, void* stream);
 int ctamd_mae_f32(const float* a, const float* b, float* out, size_t n, void* stream);
+/* ctamd_dot_f32 for callers that cannot allocate device memory or depend on memory the library
+ * allocated: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * It has no counterpart in the reference.  The per-block partial sums live in a 16 KiB array that is
+ * part of the library's device image (one copy per GPU, held until the process ends) instead of the
+ * scratch buffer ctamd_init() allocates; the call allocates and frees nothing.  Same kernels, same
+ * grid and therefore the same bits as ctamd_dot_f32.  n above CTAMD_DOT_STATIC_MAX_N (the reference's
+ * kernel counts elements in an int, Dot_BASIC_kernel.cpp:31) is refused with CTAMD_ERANGE and nothing
+ * is launched.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two
+ * streams, two host threads) race; calls on one stream are ordered.  Nothing needs clearing between
+ * calls - the fold launch reads only the partials its own first launch wrote. */
+#define CTAMD_DOT_STATIC_MAX_N ((size_t)2147483647)
+int ctamd_dot_static_f32(const float* a, const float* b, float* out, size_t n, void* stream);
 /* out[j] = sum_i g[i,j], g [rows, cols]: the complete gradient of a row-broadcast operand
  * (the reference's check_and_adjust_grad_shape, src/AutoDiff.cpp:690-757, returns row 0 instead;
  * that behaviour is a ctamd_memcpy_d2d of the first row followed by ctamd_accumulate_f32). */
