@@ -89,7 +89,7 @@ def _cpu_baseline(np, support):
                       "4096^3 extrapolates to %.0f s" % (rows - 1, rows, dt, dt * M / rows)}
 
 
-HOST_LIB = os.path.join(ROOT, "ctorch_amd", "host", "libctorch_amd_host.so")
+HOST_LIB = os.path.join(ROOT, "ctorch_amd", "host", "tests", "harness", "libctorch_amd_harness.so")
 
 
 def _timed(fn):

@@ -92,8 +92,23 @@ PROTOTYPES.update({
     "ctamd_cross_entropy_backward_index_f32": [_P, _P, _P, _P, _Z, _Z, _P],
     "ctamd_div_backward_b_f32": [_P, _P, _P, _P, _Z, _P],
 })
-for _op in ("relu", "sigmoid", "tanh", "sin", "cos"):
+for _op in ("relu", "sigmoid", "tanh", "sin", "cos", "abs", "sqrt", "square", "tan"):
     PROTOTYPES["ctamd_%s_backward_f32" % _op] = [_P, _P, _P, _Z, _P]
+for _op in ("abs", "exp", "log", "sqrt", "square", "tan"):
+    PROTOTYPES["ctamd_%s_f32" % _op] = [_P, _P, _Z, _P]
+PROTOTYPES.update({
+    "ctamd_sub_scalar_f32": [_P, C.c_float, _P, _Z, _P],
+    "ctamd_leaky_relu_f32": [_P, C.c_float, _P, _Z, _P],
+    "ctamd_leaky_relu_backward_f32": [_P, _P, C.c_float, _P, _Z, _P],
+    "ctamd_reduce_dim_f32": [C.c_int, _P, _P, _P, _P, _Z, _Z, _Z, C.c_int, _P],
+    "ctamd_reduce_dim_backward_f32": [C.c_int, _P, _P, _P, _P, _P, _P, _Z, _Z, _Z, C.c_int, _P],
+    "ctamd_fold_mod_f32": [_P, _P, _Z, _Z, _P],
+    "ctamd_broadcast_reduce_f32": [_P, _P, _P, C.c_int, _P, _P],
+    "ctamd_log_softmax_rows_f32": [_P, _P, _Z, _Z, _P],
+    "ctamd_log_softmax_cols_f32": [_P, _P, _Z, _Z, _P],
+    "ctamd_log_softmax_backward_rows_f32": [_P, _P, _P, _Z, _Z, _P],
+    "ctamd_log_softmax_backward_cols_f32": [_P, _P, _P, _Z, _Z, _P],
+})
 
 _lib = None
 

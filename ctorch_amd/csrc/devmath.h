@@ -245,4 +245,79 @@ CTA_FN float cta_sincosf(float y, int want_cos, const uint32_t* inv_pio4) {
     return cta_sincos_finish(y, ay, want_cos, n, xr);
 }
 
+// logf: glibc's algorithm (the published ARM optimized-routines logf: x = 2^k * z with z in
+// [0x1.66p-1, 0x1.66p0), 16 subintervals with tabulated 1/c and log(c), a cubic in r = z/c - 1, all
+// in double) with the same constants.  cta_log_tab[2*i] = 1/c_i, [2*i+1] = log(c_i).  Returns
+// glibc 2.35's float for every input (checked over all 2^32 bit patterns by
+// tests/native/devmath_check.c): log(+-0) = -inf, log(x < 0) = NaN, log(inf) = inf, subnormals exact.
+CTA_TAB_SPACE double cta_log_tab[32] = {
+    0x1.661ec79f8f3bep+0, -0x1.57bf7808caadep-2, 0x1.571ed4aaf883dp+0, -0x1.2bef0a7c06ddbp-2,
+    0x1.49539f0f010bp+0,  -0x1.01eae7f513a67p-2, 0x1.3c995b0b80385p+0, -0x1.b31d8a68224e9p-3,
+    0x1.30d190c8864a5p+0, -0x1.6574f0ac07758p-3, 0x1.25e227b0b8eap+0,  -0x1.1aa2bc79c81p-3,
+    0x1.1bb4a4a1a343fp+0, -0x1.a4e76ce8c0e5ep-4, 0x1.12358f08ae5bap+0, -0x1.1973c5a611cccp-4,
+    0x1.0953f419900a7p+0, -0x1.252f438e10c1ep-5, 0x1p+0,               0x0p+0,
+    0x1.e608cfd9a47acp-1, 0x1.aa5aa5df25984p-5,  0x1.ca4b31f026aap-1,  0x1.c5e53aa362eb4p-4,
+    0x1.b2036576afce6p-1, 0x1.526e57720db08p-3,  0x1.9c2d163a1aa2dp-1, 0x1.bc2860d22477p-3,
+    0x1.886e6037841edp-1, 0x1.1058bc8a07ee1p-2,  0x1.767dcf5534862p-1, 0x1.4043057b6ee09p-2};
+// `tab`: where the caller keeps the 32 doubles (LDS on the device, the array above on the host).
+CTA_FN float cta_logf(float x, const double* tab) {
+    uint32_t ix = cta_f2u(x);
+    uint32_t special = 0;                      // 1: -inf, 2: x itself (+inf), 3: NaN
+    if (ix - 0x00800000u >= 0x7f800000u - 0x00800000u) {
+        if (ix * 2u == 0u) special = 1;
+        else if (ix == 0x7f800000u) special = 2;
+        else if ((ix & 0x80000000u) || ix * 2u >= 0xff000000u) special = 3;
+        else ix = cta_f2u(x * 0x1p23f) - (23u << 23);      // subnormal: normalise
+    }
+    uint32_t tmp = ix - 0x3f330000u;
+    uint32_t i = (tmp >> 19) & 15u;
+    int32_t k = (int32_t)tmp >> 23;
+    uint32_t iz = ix - (tmp & 0xff800000u);
+    double invc = tab[2 * i], logc = tab[2 * i + 1];
+    double z = (double)cta_u2f(iz);
+    double r = CTA_FMA(z, invc, -1.0);
+    double y0 = CTA_FMA((double)k, 0x1.62e42fefa39efp-1, logc);
+    double r2 = r * r;
+    double y = CTA_FMA(0x1.5575b0be00b6ap-2, r, -0x1.ffffef20a4123p-2);
+    y = CTA_FMA(-0x1.00ea348b88334p-2, r2, y);
+    y = CTA_FMA(y, r2, y0 + r);
+    float f = (float)y;
+    if (special == 1) f = -__builtin_huge_valf();
+    if (special == 2) f = x;
+    if (special == 3) f = x - x, f = (f != f) ? f : __builtin_nanf("");     // NaN (x - x is 0 for finite negatives)
+    return f;
+}
+
+// tanf as the quotient of the sine and cosine polynomials of one reduced argument, in double,
+// rounded once: within 1 ulp of the correctly rounded tangent and of glibc 2.35's tanf (an fdlibm
+// routine in float arithmetic that this does not restate) over all floats
+// (tests/native/devmath_check.c).  tan(+-0) = +-0, inf / NaN -> NaN.
+CTA_FN float cta_tan_finish(float y, uint32_t ay, int n, double xr) {
+    double x2 = xr * xr;
+    double c = cta_cos_poly(x2);
+    double sn = cta_sin_poly(xr, x2);
+    double t = (n & 1) ? -c / sn : sn / c;
+    float f = (float)t;
+    return (ay < 0x39000000u) ? y : f;             // |y| < 2^-13: tan(y) = y, keeps the sign of -0
+}
+// Straight-line path, correct for |y| < 120 (cta_sincos_is_rare(y) == 0).
+CTA_FN float cta_tanf_fast(float y) {
+    uint32_t ay = cta_f2u(y) & 0x7fffffffu;
+    double x = (double)y;
+    double r = x * 0x1.45F306DC9C883p+23;
+    int n = ((int32_t)r + 0x800000) >> 24;
+    double xr = CTA_FMA(-(double)n, 0x1.921FB54442D18p0, x);
+    return cta_tan_finish(y, ay, n, xr);
+}
+CTA_FN float cta_tanf(float y, const uint32_t* inv_pio4) {
+    if (!cta_sincos_is_rare(y)) return cta_tanf_fast(y);
+    uint32_t uy = cta_f2u(y);
+    uint32_t ay = uy & 0x7fffffffu;
+    if (ay >= 0x7f800000u) return y - y;
+    int n;
+    double xr = cta_reduce_large(uy, &n, inv_pio4);     // reduces |y|; tan is odd
+    if (uy >> 31) { xr = -xr; n = -n; }
+    return cta_tan_finish(y, ay, n, xr);
+}
+
 #endif  // CTORCH_AMD_DEVMATH_H

@@ -23,6 +23,11 @@ struct HasRare { static constexpr bool value = false; };
 template <class F>
 struct HasRare<F, decltype(void(F::kRare))> { static constexpr bool value = F::kRare; };
 
+template <class F, class = void>
+struct HasLogTable { static constexpr bool value = false; };
+template <class F>
+struct HasLogTable<F, decltype(void(F::kLogTable))> { static constexpr bool value = F::kLogTable; };
+
 // One element: the functor's fast path, repaired through slow() when the functor flags the input.
 template <class F, int NI>
 __device__ __forceinline__ float apply1(const F& f, const float* x, const Tables& tabs) {
@@ -105,8 +110,10 @@ template <class F, bool VEC, bool NT>
 __global__ __launch_bounds__(kThreads) void map_kernel(Ptrs<F::kIn> in, float* __restrict__ out, size_t n, F f_in) {
     __shared__ uint64_t s_exp2[F::kTables ? 32 : 1];
     __shared__ uint32_t s_pio4[F::kTables ? 24 : 1];
+    __shared__ double s_log[HasLogTable<F>::value ? 32 : 1];
     if (F::kTables) stage_tables(s_exp2, s_pio4);
-    const Tables tabs{s_exp2, s_pio4};
+    if (HasLogTable<F>::value) stage_log_table(s_log);
+    const Tables tabs{s_exp2, s_pio4, s_log};
     constexpr int NI = F::kIn;
     const auto f = bind(f_in);
     using B = decltype(bind(f_in));
@@ -170,7 +177,7 @@ template <class Op, bool VEC, class Index, bool NT>
 __global__ __launch_bounds__(kThreads) void rowbcast_kernel(const float* __restrict__ a, const float* __restrict__ b,
                                                             const float* __restrict__ g, float* __restrict__ r,
                                                             size_t total, Index cols) {
-    const Tables tabs{nullptr, nullptr};
+    const Tables tabs{nullptr, nullptr, nullptr};
     constexpr bool kThird = (Op::kIn == 3);
     if (VEC) {
         const size_t n4 = total >> 2;
@@ -407,6 +414,26 @@ int ctamd_sin_f32(const float* a, float* r, size_t n, void* s) { return unary<Si
 int ctamd_cos_f32(const float* a, float* r, size_t n, void* s) { return unary<CosF>(__func__, a, r, n, s); }
 int ctamd_tanh_f32(const float* a, float* r, size_t n, void* s) { return unary<TanhF>(__func__, a, r, n, s); }
 int ctamd_sigmoid_f32(const float* a, float* r, size_t n, void* s) { return unary<SigmoidF>(__func__, a, r, n, s); }
+
+int ctamd_sub_scalar_f32(const float* a, float v, float* r, size_t n, void* s) { return host_scalar<SubF>(__func__, a, v, r, n, s); }
+int ctamd_abs_f32(const float* a, float* r, size_t n, void* s) { return unary<AbsF>(__func__, a, r, n, s); }
+int ctamd_exp_f32(const float* a, float* r, size_t n, void* s) { return unary<ExpF>(__func__, a, r, n, s); }
+int ctamd_log_f32(const float* a, float* r, size_t n, void* s) { return unary<LogF>(__func__, a, r, n, s); }
+int ctamd_sqrt_f32(const float* a, float* r, size_t n, void* s) { return unary<SqrtF>(__func__, a, r, n, s); }
+int ctamd_square_f32(const float* a, float* r, size_t n, void* s) { return unary<SquareF>(__func__, a, r, n, s); }
+int ctamd_tan_f32(const float* a, float* r, size_t n, void* s) { return unary<TanF>(__func__, a, r, n, s); }
+int ctamd_leaky_relu_f32(const float* a, float slope, float* r, size_t n, void* s) {
+    Ptrs<1> in{{a}};
+    return launch_map<LeakyReluF>(__func__, in, r, n, LeakyReluF{slope}, s);
+}
+int ctamd_abs_backward_f32(const float* x, const float* g, float* dx, size_t n, void* s) { return binary<AbsBwdF>(__func__, x, g, dx, n, s); }
+int ctamd_sqrt_backward_f32(const float* y, const float* g, float* dx, size_t n, void* s) { return binary<SqrtBwdF>(__func__, y, g, dx, n, s); }
+int ctamd_square_backward_f32(const float* x, const float* g, float* dx, size_t n, void* s) { return binary<SquareBwdF>(__func__, x, g, dx, n, s); }
+int ctamd_tan_backward_f32(const float* y, const float* g, float* dx, size_t n, void* s) { return binary<TanBwdF>(__func__, y, g, dx, n, s); }
+int ctamd_leaky_relu_backward_f32(const float* x, const float* g, float slope, float* dx, size_t n, void* s) {
+    Ptrs<2> in{{x, g}};
+    return launch_map<LeakyReluBwdF>(__func__, in, dx, n, LeakyReluBwdF{slope}, s);
+}
 
 int ctamd_fill_f32(float* r, float v, size_t n, void* s) {
     Ptrs<0> in{};

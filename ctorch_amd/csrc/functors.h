@@ -20,6 +20,7 @@ constexpr int kUnroll = 4;
 struct Tables {
     const uint64_t* exp2;
     const uint32_t* inv_pio4;
+    const double* log;       // cta_log_tab, staged only for functors with kLogTable
 };
 
 template <int N>
@@ -92,6 +93,51 @@ struct TanhF { static constexpr int kIn = 1; static constexpr bool kTables = tru
     __device__ float operator()(const float* x, const Tables& t) const { return tanh_ref(x[0], t); } };
 struct SigmoidF { static constexpr int kIn = 1; static constexpr bool kTables = true;
     __device__ float operator()(const float* x, const Tables& t) const { return sigmoid_ref(x[0], t); } };
+
+// ---- the operators the reference declares without defining (include/Tensor.h:954-996, :1052); the
+// semantics are the C++ library calls their names stand for: std::fabs, std::exp, std::log,
+// std::sqrt, x * x, std::tan on floats, and leaky ReLU as x > 0 ? x : x * slope
+struct AbsF { static constexpr int kIn = 1; static constexpr bool kTables = false;
+    __device__ float operator()(const float* x, const Tables&) const { return __builtin_fabsf(x[0]); } };
+struct ExpF { static constexpr int kIn = 1; static constexpr bool kTables = true;
+    __device__ float operator()(const float* x, const Tables& t) const { return cta_expf_tab(x[0], t.exp2); } };
+struct LogF { static constexpr int kIn = 1; static constexpr bool kTables = false; static constexpr bool kLogTable = true;
+    __device__ float operator()(const float* x, const Tables& t) const { return cta_logf(x[0], t.log); } };
+struct SqrtF { static constexpr int kIn = 1; static constexpr bool kTables = false;
+    __device__ float operator()(const float* x, const Tables&) const { return __builtin_sqrtf(x[0]); } };   // IEEE, correctly rounded (the build keeps fp32 sqrt and divide correctly rounded)
+struct SquareF { static constexpr int kIn = 1; static constexpr bool kTables = false;
+    __device__ float operator()(const float* x, const Tables&) const { return x[0] * x[0]; } };
+struct TanF { static constexpr int kIn = 1; static constexpr bool kTables = true; static constexpr bool kRare = true;
+    __device__ float operator()(const float* x, const Tables&) const { return cta_tanf_fast(x[0]); }
+    __device__ bool rare(const float* x) const { return cta_sincos_is_rare(x[0]); }
+    __device__ float slow(const float* x, const Tables& t) const { return cta_tanf(x[0], t.inv_pio4); } };
+struct LeakyReluF { static constexpr int kIn = 1; static constexpr bool kTables = false;
+    float slope;
+    __device__ float operator()(const float* x, const Tables&) const { return (x[0] > 0.0f) ? x[0] : x[0] * slope; } };
+
+// ---- their gradients; inputs (x or y, g).  Exp's is y * g and Log's g / x: the Mul and Div kernels.
+struct AbsBwdF { static constexpr int kIn = 2; static constexpr bool kTables = false;     // sign(x) * g
+    __device__ float operator()(const float* x, const Tables&) const {
+        float s = (x[0] > 0.0f) ? 1.0f : ((x[0] < 0.0f) ? -1.0f : 0.0f);
+        return s * x[1]; } };
+struct SqrtBwdF { static constexpr int kIn = 2; static constexpr bool kTables = false;    // g / (y * 2)
+    __device__ float operator()(const float* x, const Tables&) const {
+        float d = x[0] * 2.0f;
+        return x[1] / d; } };
+struct SquareBwdF { static constexpr int kIn = 2; static constexpr bool kTables = false;  // (x * 2) * g
+    __device__ float operator()(const float* x, const Tables&) const {
+        float d = x[0] * 2.0f;
+        return d * x[1]; } };
+struct TanBwdF { static constexpr int kIn = 2; static constexpr bool kTables = false;     // (1 + y * y) * g
+    __device__ float operator()(const float* x, const Tables&) const {
+        float yy = x[0] * x[0];
+        float s = 1.0f + yy;
+        return s * x[1]; } };
+struct LeakyReluBwdF { static constexpr int kIn = 2; static constexpr bool kTables = false;   // g * (x > 0 ? 1 : slope)
+    float slope;
+    __device__ float operator()(const float* x, const Tables&) const {
+        float m = (x[0] > 0.0f) ? 1.0f : slope;
+        return x[1] * m; } };
 
 // ---- gradient arithmetic; inputs (x, g) unless noted
 struct ReluBwdF { static constexpr int kIn = 2; static constexpr bool kTables = false;
@@ -169,6 +215,10 @@ struct FillFromF { static constexpr int kIn = 0; static constexpr bool kTables =
     const float* v;
     __device__ float operator()(const float*, const Tables&) const { return *v; } };
 
+__device__ __forceinline__ void stage_log_table(double* tab) {
+    if (threadIdx.x < 32) tab[threadIdx.x] = cta_log_tab[threadIdx.x];
+    __syncthreads();
+}
 __device__ __forceinline__ void stage_tables(uint64_t* exp2, uint32_t* pio4) {
     if (threadIdx.x < 32) exp2[threadIdx.x] = cta_exp2_tab[threadIdx.x];
     if (threadIdx.x >= 32 && threadIdx.x < 56) pio4[threadIdx.x - 32] = cta_inv_pio4[threadIdx.x - 32];

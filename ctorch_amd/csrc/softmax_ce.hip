@@ -144,6 +144,15 @@ struct Row {
             }
         return s;
     }
+    // sum of exp(v - m) with the bit-exact exponential, v unchanged
+    __device__ __forceinline__ float sum_exp(float m, const uint64_t* exp2) const {
+        float s = 0.0f;
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k)
+#pragma unroll
+            for (int i = 0; i < W; ++i) s += cta_expf_nonpos(v[k][i] - m, exp2);
+        return s;
+    }
     // v <- exp(v - m) with the hardware exp2 (~1e-7 relative near the maximum, where it matters)
     __device__ __forceinline__ float exp_shifted_fast(float m) {
         float s0 = 0.0f, s1 = 0.0f;
@@ -191,7 +200,8 @@ struct Row {
     }
 };
 
-enum Mode { kSoftmax, kCeOnehot, kCeIndex, kCeBwdOnehot, kCeBwdIndex, kSoftmaxBwd, kCeIndexBoth, kCeIndexBothFast };
+enum Mode { kSoftmax, kCeOnehot, kCeIndex, kCeBwdOnehot, kCeBwdIndex, kSoftmaxBwd, kCeIndexBoth, kCeIndexBothFast,
+            kLogSoftmax, kLogSoftmaxFast, kLogSoftmaxBwd };
 
 struct Args {
     const float* x;      // logits / softmax output y (kSoftmaxBwd)
@@ -220,7 +230,8 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
     __shared__ double s_d[THREADS / 64 + 1];
     stage_exp_table(s_exp2);
     constexpr bool kBoth = (MODE == kCeIndexBoth || MODE == kCeIndexBothFast);
-    constexpr bool kPipelined = (MODE == kSoftmax || MODE == kCeIndex || MODE == kCeBwdIndex || kBoth);
+    constexpr bool kLogSm = (MODE == kLogSoftmax || MODE == kLogSoftmaxFast);
+    constexpr bool kPipelined = (MODE == kSoftmax || MODE == kCeIndex || MODE == kCeBwdIndex || kBoth || kLogSm);
     double block_loss = 0.0;
     bool block_bad = false;   // a class index out of range was met (thread 0's copy counts)
 
@@ -228,6 +239,21 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
     auto process = [&](Row<THREADS, ITEMS, W>& r, size_t row, float mloc) {
         const float m = block_max<THREADS>(mloc, s_f[0]);
         constexpr bool kLossOnly = (MODE == kCeOnehot || MODE == kCeIndex);
+        if (kLogSm) {
+            // y = (x - m) - log(sum exp(x - m)); rows of 2048 columns or more form the sum with the
+            // hardware exponential (~1e-7 relative, i.e. ~1e-7 absolute in its logarithm)
+            const float s = block_sum<THREADS>(MODE == kLogSoftmaxFast ? r.sum_exp_fast(m) : r.sum_exp(m, s_exp2), s_f[1]);
+            const float lg = cta_logf(s, cta_log_tab);
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k)
+#pragma unroll
+                for (int i = 0; i < W; ++i) {
+                    const float d = r.v[k][i] - m;
+                    r.v[k][i] = d - lg;
+                }
+            r.store(a.out + row * a.cols, unsigned(a.cols));
+            return;
+        }
         // loss kernels keep x in r and only need the row sum; the others turn r into exp(x - m)
         const float s = block_sum<THREADS>(kLossOnly ? r.sum_exp_fast(m) : MODE == kCeIndexBothFast ? r.exp_shifted_fast(m) : r.exp_shifted(m, s_exp2), s_f[1]);
         const double rcp_s = 1.0 / double(s);     // e / s below is the exact fp32 quotient (cta_div_rcp)
@@ -350,7 +376,28 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
 
     const size_t stride = gridDim.x;
     size_t row = blockIdx.x;
-    if (MODE == kSoftmaxBwd) {
+    if (MODE == kLogSoftmaxBwd) {
+        for (; row < a.rows; row += stride) {
+            // r = y = log_softmax(x), q = g: d = sum g, dx = g - exp(y) * d
+            Row<THREADS, ITEMS, W> r, q;
+            r.load(a.x + row * a.cols, unsigned(a.cols), a.pad_neg_inf);
+            q.load(a.t + row * a.cols, unsigned(a.cols), a.pad_zero);
+            float d = 0.0f;
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k)
+#pragma unroll
+                for (int i = 0; i < W; ++i) d += q.v[k][i];
+            d = block_sum<THREADS>(d, s_f[0]);
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k)
+#pragma unroll
+                for (int i = 0; i < W; ++i) {
+                    const float t = cta_expf_tab(r.v[k][i], s_exp2) * d;
+                    r.v[k][i] = q.v[k][i] - t;
+                }
+            r.store(a.out + row * a.cols, unsigned(a.cols));
+        }
+    } else if (MODE == kSoftmaxBwd) {
         for (; row < a.rows; row += stride) {
             // r = y, q = g: d = sum g*y, dx = y * (g - d)
             Row<THREADS, ITEMS, W> r, q;
@@ -416,7 +463,8 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
 template <int MODE>
 __global__ __launch_bounds__(1024) void row_stream_vec_kernel(Args a) {
     constexpr int THREADS = 1024, U = 4;
-    static_assert(MODE == kSoftmax || MODE == kSoftmaxBwd, "only the two modes that write a row-shaped result");
+    static_assert(MODE == kSoftmax || MODE == kSoftmaxBwd || MODE == kLogSoftmaxFast || MODE == kLogSoftmaxBwd,
+                  "only the modes that write a row-shaped result");
     __shared__ uint64_t s_exp2[32];
     __shared__ float s_f[2][THREADS / 64 + 1];
     stage_exp_table(s_exp2);
@@ -424,6 +472,40 @@ __global__ __launch_bounds__(1024) void row_stream_vec_kernel(Args a) {
     for (size_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
         const v4f* __restrict__ xr = reinterpret_cast<const v4f*>(a.x + row * a.cols);
         v4f* __restrict__ outr = reinterpret_cast<v4f*>(a.out + row * a.cols);
+        if (MODE == kLogSoftmaxBwd) {
+            // d = sum g (first sweep over g alone), dx = g - exp(y) * d
+            const v4f* __restrict__ gr = reinterpret_cast<const v4f*>(a.t + row * a.cols);
+            float d0 = 0.0f, d1 = 0.0f;
+            unsigned i = threadIdx.x;
+            for (; i + (U - 1) * THREADS < n4; i += U * THREADS) {
+                v4f g[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) g[u] = gr[i + u * THREADS];
+#pragma unroll
+                for (int u = 0; u < U; ++u) { d0 += g[u][0] + g[u][1]; d1 += g[u][2] + g[u][3]; }
+            }
+            for (; i < n4; i += THREADS) { const v4f g = gr[i]; d0 += g[0] + g[1]; d1 += g[2] + g[3]; }
+            const float d = block_sum<THREADS>(d0 + d1, s_f[0]);
+            auto give = [&](const v4f& y, const v4f& g, unsigned at) {
+                v4f o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float t = cta_expf_tab(y[e], s_exp2) * d;
+                    o[e] = g[e] - t;
+                }
+                __builtin_nontemporal_store(o, outr + at);
+            };
+            i = threadIdx.x;
+            for (; i + (U / 2 - 1) * THREADS < n4; i += (U / 2) * THREADS) {
+                v4f y[U / 2], g[U / 2];
+#pragma unroll
+                for (int u = 0; u < U / 2; ++u) { y[u] = xr[i + u * THREADS]; g[u] = gr[i + u * THREADS]; }
+#pragma unroll
+                for (int u = 0; u < U / 2; ++u) give(y[u], g[u], i + u * THREADS);
+            }
+            for (; i < n4; i += THREADS) give(xr[i], gr[i], i);
+            continue;
+        }
         if (MODE == kSoftmaxBwd) {
             const v4f* __restrict__ gr = reinterpret_cast<const v4f*>(a.t + row * a.cols);
             float d0 = 0.0f, d1 = 0.0f;
@@ -490,10 +572,18 @@ __global__ __launch_bounds__(1024) void row_stream_vec_kernel(Args a) {
         s = (m == kNegInf) ? 0.0f : s * __builtin_amdgcn_exp2f((m - M) * 1.44269504088896340736f);
         const float S = block_sum<THREADS>(s, s_f[1]);
         const double rcp = 1.0 / double(S);
+        const float lg = (MODE == kLogSoftmaxFast) ? cta_logf(S, cta_log_tab) : 0.0f;
         auto give = [&](const v4f& v, unsigned at) {
             v4f o;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = cta_div_rcp(cta_expf_nonpos(v[e] - M, s_exp2), rcp);
+            for (int e = 0; e < 4; ++e) {
+                if (MODE == kLogSoftmaxFast) {
+                    const float d = v[e] - M;
+                    o[e] = d - lg;
+                } else {
+                    o[e] = cta_div_rcp(cta_expf_nonpos(v[e] - M, s_exp2), rcp);
+                }
+            }
             __builtin_nontemporal_store(o, outr + at);
         };
         i = threadIdx.x;
@@ -527,6 +617,17 @@ __global__ __launch_bounds__(1024) void row_stream_kernel(Args a) {
             for (size_t j = threadIdx.x; j < a.cols; j += THREADS) a.out[row * a.cols + j] = xr[j] * (gr[j] - d);
             continue;
         }
+        if (MODE == kLogSoftmaxBwd) {
+            const float* gr = a.t + row * a.cols;
+            float d = 0.0f;
+            for (size_t j = threadIdx.x; j < a.cols; j += THREADS) d += gr[j];
+            d = block_sum<THREADS>(d, s_f[0]);
+            for (size_t j = threadIdx.x; j < a.cols; j += THREADS) {
+                const float t = cta_expf_tab(xr[j], s_exp2) * d;
+                a.out[row * a.cols + j] = gr[j] - t;
+            }
+            continue;
+        }
         float m = kNegInf, s = 0.0f;
         for (size_t j = threadIdx.x; j < a.cols; j += THREADS) {
             float v = xr[j];
@@ -542,6 +643,12 @@ __global__ __launch_bounds__(1024) void row_stream_kernel(Args a) {
         if (MODE == kSoftmax) {
             for (size_t j = threadIdx.x; j < a.cols; j += THREADS)
                 a.out[row * a.cols + j] = cta_div_rcp(cta_expf_tab(xr[j] - M, s_exp2), 1.0 / double(S));
+        } else if (MODE == kLogSoftmax || MODE == kLogSoftmaxFast) {
+            const float lg = cta_logf(S, cta_log_tab);
+            for (size_t j = threadIdx.x; j < a.cols; j += THREADS) {
+                const float d = xr[j] - M;
+                a.out[row * a.cols + j] = d - lg;
+            }
         } else if (MODE == kCeOnehot) {
             const float* tr = a.t + row * a.cols;
             double loss = 0.0;
@@ -747,10 +854,11 @@ bool launch_resident(const Args& a, unsigned grid, hipStream_t s) {
     else {
         // rows of 2048 columns or more never reach these two modes (they go to the online forward
         // kernel and to the long-row one-pass kernel): the 1024-thread shapes are not built for them
-        if constexpr (MODE == kCeIndex || MODE == kCeIndexBoth) {
+        if constexpr (MODE == kCeIndex || MODE == kCeIndexBoth || MODE == kLogSoftmax) {
             return false;
         } else {
             if (groups <= 1024 * 2) launch_cfg<MODE, 1024, 2, W>(a, grid, s);
+            else if constexpr (MODE == kLogSoftmaxBwd) return false;   // two resident rows and the exponential do not fit 128 registers
             else if (groups <= 1024 * 8) launch_cfg<MODE, 1024, 8, W>(a, grid, s);
             else return false;
         }
@@ -770,7 +878,8 @@ int run_rows(const char* name, Args a, float* loss_out, void* stream) {
         if (kLoss) return ctamd_fill_f32(loss_out, 0.0f, 1, stream);
         return CTAMD_OK;
     }
-    if (!a.x || (!a.t && MODE != kSoftmax)) return fail(CTAMD_EINVAL, "%s: null input", name);
+    constexpr bool kLogSm = (MODE == kLogSoftmax || MODE == kLogSoftmaxFast);
+    if (!a.x || (!a.t && MODE != kSoftmax && !kLogSm)) return fail(CTAMD_EINVAL, "%s: null input", name);
     if (kWrites && !a.out) return fail(CTAMD_EINVAL, "%s: null output", name);
     if ((MODE == kCeBwdOnehot || MODE == kCeBwdIndex) && !a.g1) return fail(CTAMD_EINVAL, "%s: null upstream gradient", name);
     if (a.rows > (size_t(1) << 62) / a.cols) return fail(CTAMD_ERANGE, "%s: rows*cols overflows", name);
@@ -782,7 +891,7 @@ int run_rows(const char* name, Args a, float* loss_out, void* stream) {
         // algorithmic bytes per element: logits in (+ one-hot target in) (+ result out); a class
         // index adds 4 bytes per row; one exp per element
         const double n = double(a.rows) * double(a.cols);
-        const double per = MODE == kSoftmax ? 8.0 : MODE == kCeIndex ? 4.0 : MODE == kCeOnehot ? 8.0
+        const double per = (MODE == kSoftmax || kLogSm) ? 8.0 : MODE == kCeIndex ? 4.0 : MODE == kCeOnehot ? 8.0
                          : (MODE == kCeBwdIndex || kBoth) ? 8.0 : 12.0;   // kCeBwdOnehot, kSoftmaxBwd: two inputs, one output
         const bool index = (MODE == kCeIndex || MODE == kCeBwdIndex || kBoth);
         account(per * n + (index ? 4.0 * double(a.rows) : 0.0), n);
@@ -796,7 +905,7 @@ int run_rows(const char* name, Args a, float* loss_out, void* stream) {
     if (kLoss && fill > 2048) fill = 2048;         // one partial per block: keep the fold of the partials short
     unsigned grid = a.rows < fill ? unsigned(a.rows) : unsigned(fill);
     bool vec = (a.cols % 4 == 0) && aligned16(a.x) &&
-               (MODE == kSoftmax || MODE == kCeIndex || MODE == kCeBwdIndex || kBoth || aligned16(a.t)) &&
+               (MODE == kSoftmax || kLogSm || MODE == kCeIndex || MODE == kCeBwdIndex || kBoth || aligned16(a.t)) &&
                (!kWrites || aligned16(a.out));
     if (MODE == kCeIndex && a.cols >= 2048) {
         size_t fill_online = size_t(compute_units() > 0 ? compute_units() : 256) * 8;
@@ -813,7 +922,7 @@ int run_rows(const char* name, Args a, float* loss_out, void* stream) {
         if constexpr (kBoth)
             return fail(CTAMD_ERANGE, "%s: a row does not fit a block's registers (32768 columns, 8192 without 128-bit accesses): "
                         "use the separate forward and backward entry points", name);
-        else if constexpr (MODE == kSoftmax || MODE == kSoftmaxBwd) {
+        else if constexpr (MODE == kSoftmax || MODE == kSoftmaxBwd || MODE == kLogSoftmaxFast || MODE == kLogSoftmaxBwd) {
             if (vec) hipLaunchKernelGGL((row_stream_vec_kernel<MODE>), dim3(grid), dim3(1024), 0, s, a);
             else hipLaunchKernelGGL((row_stream_kernel<MODE>), dim3(grid), dim3(1024), 0, s, a);
         } else
@@ -859,6 +968,40 @@ __global__ __launch_bounds__(256) void softmax_bwd_cols_kernel(const float* __re
 }
 
 
+// log_softmax along dim 0 and its gradient, one thread per column, rows in order (small matrices)
+__global__ __launch_bounds__(256) void log_softmax_cols_kernel(const float* __restrict__ x, float* __restrict__ y,
+                                                               size_t rows, size_t cols) {
+    __shared__ uint64_t s_exp2[32];
+    stage_exp_table(s_exp2);
+    size_t j = size_t(blockIdx.x) * 256 + threadIdx.x;
+    if (j >= cols) return;
+    float m = x[j];
+    for (size_t i = 1; i < rows; ++i) {
+        float v = x[i * cols + j];
+        if (v > m) m = v;
+    }
+    float s = 0.0f;
+    for (size_t i = 0; i < rows; ++i) s += cta_expf_tab(x[i * cols + j] - m, s_exp2);
+    const float lg = cta_logf(s, cta_log_tab);
+    for (size_t i = 0; i < rows; ++i) {
+        const float d = x[i * cols + j] - m;
+        y[i * cols + j] = d - lg;
+    }
+}
+__global__ __launch_bounds__(256) void log_softmax_bwd_cols_kernel(const float* __restrict__ y, const float* __restrict__ g,
+                                                                   float* __restrict__ dx, size_t rows, size_t cols) {
+    __shared__ uint64_t s_exp2[32];
+    stage_exp_table(s_exp2);
+    size_t j = size_t(blockIdx.x) * 256 + threadIdx.x;
+    if (j >= cols) return;
+    float d = 0.0f;
+    for (size_t i = 0; i < rows; ++i) d += g[i * cols + j];
+    for (size_t i = 0; i < rows; ++i) {
+        const float t = cta_expf_tab(y[i * cols + j], s_exp2) * d;
+        dx[i * cols + j] = g[i * cols + j] - t;
+    }
+}
+
 // Tall matrices (128 rows or more): the column statistics as chunked reductions over rows, like the
 // column sum - a block owns a strip of 256 * W columns and a chunk of rows and walks its rows in
 // order, two rows in flight; per-chunk partials are folded by a second launch.  Forward: per chunk
@@ -869,7 +1012,7 @@ __global__ __launch_bounds__(256) void softmax_bwd_cols_kernel(const float* __re
 // chunk, double across chunks) where the reference adds the rows one after the other: the same
 // values to ~1e-7 relative, against 18 ms for a [16384 x 4096] matrix when one thread walks a
 // whole column alone.
-enum ColMode { kColOnline, kColSoftmaxOut, kColDot, kColBwdOut };
+enum ColMode { kColOnline, kColSoftmaxOut, kColDot, kColBwdOut, kColSum, kColLogSoftmaxOut, kColLogBwdOut };
 
 template <int MODE, int W>
 __global__ __launch_bounds__(256) void col_walk_kernel(const float* __restrict__ x, const float* __restrict__ x2,
@@ -877,7 +1020,7 @@ __global__ __launch_bounds__(256) void col_walk_kernel(const float* __restrict__
                                                        float* __restrict__ out, size_t rows, size_t cols,
                                                        size_t rows_per_block) {
     __shared__ uint64_t s_exp2[32];
-    if (MODE == kColSoftmaxOut) stage_exp_table(s_exp2);
+    if (MODE == kColSoftmaxOut || MODE == kColLogBwdOut) stage_exp_table(s_exp2);
     const size_t col = (size_t(blockIdx.x) * 256 + threadIdx.x) * W;
     if (col >= cols) return;
     const size_t r0 = size_t(blockIdx.y) * rows_per_block;
@@ -890,14 +1033,17 @@ __global__ __launch_bounds__(256) void col_walk_kernel(const float* __restrict__
     for (int e = 0; e < W; ++e) {
         a0[e] = a1[e] = 0.0f;
         m0[e] = m1[e] = kNegInf;
-        q0[e] = (MODE == kColSoftmaxOut || MODE == kColBwdOut) ? p0[col + e] : 0.0f;
+        q0[e] = (MODE == kColSoftmaxOut || MODE == kColBwdOut || MODE == kColLogSoftmaxOut || MODE == kColLogBwdOut) ? p0[col + e] : 0.0f;
         rcp[e] = (MODE == kColSoftmaxOut) ? 1.0 / double(p1[col + e]) : 0.0;
     }
+    float lg[W];                        // kColLogSoftmaxOut: log of the column's sum
+#pragma unroll
+    for (int e = 0; e < W; ++e) lg[e] = (MODE == kColLogSoftmaxOut) ? cta_logf(p1[col + e], cta_log_tab) : 0.0f;
     auto load = [&](const float* __restrict__ base, size_t r, float (&v)[W]) {
         if (W == 4) {
             // the writing passes read their operands for the last time: streaming hint (on the reading
             // passes it costs the second pass its cache hits: 152 -> 162 us at [16384 x 4096])
-            constexpr bool kLast = (MODE == kColSoftmaxOut || MODE == kColBwdOut);
+            constexpr bool kLast = (MODE == kColSoftmaxOut || MODE == kColBwdOut || MODE == kColLogSoftmaxOut || MODE == kColLogBwdOut);
             v4f t = kLast ? __builtin_nontemporal_load(reinterpret_cast<const v4f*>(base + r * cols + col))
                           : *reinterpret_cast<const v4f*>(base + r * cols + col);
 #pragma unroll
@@ -932,11 +1078,18 @@ __global__ __launch_bounds__(256) void col_walk_kernel(const float* __restrict__
                 mx[e] = up ? v[e] : mx[e];
             } else if (MODE == kColSoftmaxOut) o[e] = cta_div_rcp(cta_expf_nonpos(v[e] - q0[e], s_exp2), rcp[e]);
             else if (MODE == kColDot) acc[e] = __fmaf_rn(w[e], v[e], acc[e]);
-            else o[e] = v[e] * (w[e] - q0[e]);
+            else if (MODE == kColSum) acc[e] += v[e];
+            else if (MODE == kColLogSoftmaxOut) {
+                const float d = v[e] - q0[e];
+                o[e] = d - lg[e];
+            } else if (MODE == kColLogBwdOut) {                  // v = y, w = g, q0 = column sum of g
+                const float t = cta_expf_tab(v[e], s_exp2) * q0[e];
+                o[e] = w[e] - t;
+            } else o[e] = v[e] * (w[e] - q0[e]);
         }
-        if (MODE == kColSoftmaxOut || MODE == kColBwdOut) store(r, o);
+        if (MODE == kColSoftmaxOut || MODE == kColBwdOut || MODE == kColLogSoftmaxOut || MODE == kColLogBwdOut) store(r, o);
     };
-    constexpr bool kTwo = (MODE == kColDot || MODE == kColBwdOut);     // x = y, x2 = g
+    constexpr bool kTwo = (MODE == kColDot || MODE == kColBwdOut || MODE == kColLogBwdOut);     // x = y, x2 = g
     size_t r = r0;
     constexpr int kRows = 4;                // rows whose loads are in flight before the first is used (8: no gain)
     for (; r + kRows <= r1; r += kRows) {
@@ -960,7 +1113,7 @@ __global__ __launch_bounds__(256) void col_walk_kernel(const float* __restrict__
         if ((r - r0) & 1) one_row(r, a1, m1, v0, w0);
         else one_row(r, a0, m0, v0, w0);
     }
-    if (MODE == kColDot) {
+    if (MODE == kColDot || MODE == kColSum) {
 #pragma unroll
         for (int e = 0; e < W; ++e) out[size_t(blockIdx.y) * cols + col + e] = a0[e] + a1[e];
     }
@@ -1132,6 +1285,48 @@ int ctamd_cross_entropy_backward_index_f32(const float* x, const float* idx, con
 int ctamd_softmax_backward_rows_f32(const float* y, const float* g, float* dx, size_t rows, size_t cols, void* stream) {
     Args a{y, g, nullptr, dx, nullptr, nullptr, nullptr, rows, cols, nullptr, nullptr};
     return run_rows<kSoftmaxBwd>(__func__, a, nullptr, stream);
+}
+
+int ctamd_log_softmax_rows_f32(const float* x, float* y, size_t rows, size_t cols, void* stream) {
+    Args a{x, nullptr, nullptr, y, nullptr, nullptr, nullptr, rows, cols, nullptr, nullptr};
+    if (cols >= 2048) return run_rows<kLogSoftmaxFast>(__func__, a, nullptr, stream);
+    return run_rows<kLogSoftmax>(__func__, a, nullptr, stream);
+}
+int ctamd_log_softmax_backward_rows_f32(const float* y, const float* g, float* dx, size_t rows, size_t cols, void* stream) {
+    Args a{y, g, nullptr, dx, nullptr, nullptr, nullptr, rows, cols, nullptr, nullptr};
+    return run_rows<kLogSoftmaxBwd>(__func__, a, nullptr, stream);
+}
+int ctamd_log_softmax_cols_f32(const float* x, float* y, size_t rows, size_t cols, void* stream) {
+    if (rows == 0 || cols == 0) return CTAMD_OK;
+    if (!x || !y) return fail(CTAMD_EINVAL, "%s: null pointer", __func__);
+    ColPlan p;
+    account(8.0 * double(rows) * double(cols), double(rows) * double(cols));
+    if (plan_cols(rows, cols, aligned16(x) && aligned16(y), p)) {
+        hipStream_t s = as_stream(stream);
+        const unsigned fold_blocks = unsigned((cols + kFoldCols - 1) / kFoldCols);
+        launch_col_walk<kColOnline>(p, x, nullptr, nullptr, nullptr, p.partials, rows, cols, s);
+        hipLaunchKernelGGL(col_fold_kernel<true>, dim3(fold_blocks), dim3(256), 0, s, p.partials, p.v0, p.v1, cols, unsigned(p.chunks));
+        launch_col_walk<kColLogSoftmaxOut>(p, x, nullptr, p.v0, p.v1, y, rows, cols, s);
+        return launched(__func__);
+    }
+    hipLaunchKernelGGL(log_softmax_cols_kernel, dim3((unsigned)((cols + 255) / 256)), dim3(256), 0, as_stream(stream), x, y, rows, cols);
+    return launched(__func__);
+}
+int ctamd_log_softmax_backward_cols_f32(const float* y, const float* g, float* dx, size_t rows, size_t cols, void* stream) {
+    if (rows == 0 || cols == 0) return CTAMD_OK;
+    if (!y || !g || !dx) return fail(CTAMD_EINVAL, "%s: null pointer", __func__);
+    ColPlan p;
+    account(12.0 * double(rows) * double(cols), 2.0 * double(rows) * double(cols));
+    if (plan_cols(rows, cols, aligned16(y) && aligned16(g) && aligned16(dx), p)) {
+        hipStream_t s = as_stream(stream);
+        launch_col_walk<kColSum>(p, g, nullptr, nullptr, nullptr, p.partials, rows, cols, s);
+        hipLaunchKernelGGL(col_fold_kernel<false>, dim3(unsigned((cols + kFoldCols - 1) / kFoldCols)), dim3(256), 0, s, p.partials, nullptr, p.v0,
+                           cols, unsigned(p.chunks));
+        launch_col_walk<kColLogBwdOut>(p, y, g, p.v0, nullptr, dx, rows, cols, s);
+        return launched(__func__);
+    }
+    hipLaunchKernelGGL(log_softmax_bwd_cols_kernel, dim3((unsigned)((cols + 255) / 256)), dim3(256), 0, as_stream(stream), y, g, dx, rows, cols);
+    return launched(__func__);
 }
 
 int ctamd_softmax_cols_f32(const float* x, float* y, size_t rows, size_t cols, void* stream) {

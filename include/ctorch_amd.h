@@ -126,6 +126,21 @@ int ctamd_cos_f32(const float* a, float* r, size_t n, void* stream);
 int ctamd_tanh_f32(const float* a, float* r, size_t n, void* stream);
 int ctamd_sigmoid_f32(const float* a, float* r, size_t n, void* stream);
 
+/* Operators that the reference declares on Tensor and never defines (include/Tensor.h:719 operator-
+ * (float), :954-972 abs / exp / log / sqrt, :978 square, :996 tan, :1052 leaky_relu; the kernel
+ * LReLU_BASIC_kernel is declared at src/kernels/kernels.h:201 and registered without a function at
+ * include/Ctorch_Scheduler.h:51-52).  With no reference arithmetic to follow, each is the C++ library
+ * call its name stands for, on floats: a - s; std::fabs; expf, logf (glibc 2.35's floats, bit for
+ * bit); IEEE sqrt; a * a; tanf (within 1 ulp of glibc's); x > 0 ? x : x * slope. */
+int ctamd_sub_scalar_f32(const float* a, float s, float* r, size_t n, void* stream);
+int ctamd_abs_f32(const float* a, float* r, size_t n, void* stream);
+int ctamd_exp_f32(const float* a, float* r, size_t n, void* stream);
+int ctamd_log_f32(const float* a, float* r, size_t n, void* stream);
+int ctamd_sqrt_f32(const float* a, float* r, size_t n, void* stream);
+int ctamd_square_f32(const float* a, float* r, size_t n, void* stream);
+int ctamd_tan_f32(const float* a, float* r, size_t n, void* stream);
+int ctamd_leaky_relu_f32(const float* a, float slope, float* r, size_t n, void* stream);
+
 /* ------------------------------------------------------------------------------- reductions */
 /* out[0] = sum of a.  Tensor::sum() src/Tensor.cpp:638-666. */
 int ctamd_sum_f32(const float* a, float* out, size_t n, void* stream);
@@ -146,6 +161,35 @@ int ctamd_mae_f32(const float* a, const float* b, float* out, size_t n, void* st
  * calls - the fold launch reads only the partials its own first launch wrote. */
 #define CTAMD_DOT_STATIC_MAX_N ((size_t)2147483647)
 int ctamd_dot_static_f32(const float* a, const float* b, float* out, size_t n, void* stream);
+/* sum / mean / max / min / var / std along one axis: x is read as [outer, len, inner] (row-major) and
+ * out[o, i] is the reduction of x[o, :, i].  outer = inner = 1 reduces a whole tensor, inner = 1 the
+ * rows of a matrix, outer = 1 its columns.  These are Tensor::sum(dim) / mean / max / min / var / std,
+ * which the reference declares and never defines (include/Tensor.h:824-948); the arithmetic fixed
+ * here: fp32 terms added in a tree (sum), float(sum) / float(len) (mean), the extreme value and, in
+ * index (may be NULL), the position of its FIRST occurrence along the axis (NaN wins only from position 0, as a loop
+ * `if (v > m) m = v` started at element 0 behaves), var = sum((x - mean)^2) / (len - ddof) formed in
+ * double, std its square root; mean_out (var / std only, may be NULL) receives the mean that the
+ * gradient needs.  len <= 2^31 - 1.  Uses the per-device scratch. */
+enum { CTAMD_RED_SUM = 0, CTAMD_RED_MEAN = 1, CTAMD_RED_MAX = 2, CTAMD_RED_MIN = 3, CTAMD_RED_VAR = 4, CTAMD_RED_STD = 5 };
+int ctamd_reduce_dim_f32(int kind, const float* x, float* out, int32_t* index, float* mean_out, size_t outer, size_t len,
+                         size_t inner, int ddof, void* stream);
+/* Their gradients, dx of x's shape from g of out's shape: sum g; mean g / float(len); max / min g at
+ * index[o, i] and +0 elsewhere; var ((x - mean) * 2 / float(len - ddof)) * g; std
+ * ((x - mean) / (float(len - ddof) * y)) * g, each step rounded to fp32 in that order.  x and mean are
+ * read by var / std only, y by std only, index by max / min only (others may be NULL). */
+int ctamd_reduce_dim_backward_f32(int kind, const float* x, const float* y, const int32_t* index, const float* mean,
+                                  const float* g, float* dx, size_t outer, size_t len, size_t inner, int ddof, void* stream);
+/* out[i] = g[i] + g[i + out_count] + g[i + 2 * out_count] + ... added in that order from 0: what the
+ * reference's check_and_adjust_grad_shape does with a gradient whose shape does not broadcast to the
+ * operand's (src/AutoDiff.cpp:968-1046). */
+int ctamd_fold_mod_f32(const float* g, float* out, size_t g_count, size_t out_count, void* stream);
+/* The gradient of an operand that was broadcast to the gradient's shape, for any shapes of up to 8
+ * dimensions: g_shape and t_shape (HOST arrays of `rank` extents, the operand's shape padded with
+ * leading 1s) agree per dimension, or the operand's extent is 1 (out sums g over that dimension, in
+ * double), or the gradient's is 1 (its value is repeated).  The mathematically complete form of
+ * check_and_adjust_grad_shape's broadcast branch (src/AutoDiff.cpp:690-890, which takes one slice
+ * instead of the sum); ctamd_colsum_f32 is its [rows, cols] -> [cols] case at memory speed. */
+int ctamd_broadcast_reduce_f32(const float* g, const size_t* g_shape, const size_t* t_shape, int rank, float* out, void* stream);
 /* out[j] = sum_i g[i,j], g [rows, cols]: the complete gradient of a row-broadcast operand
  * (the reference's check_and_adjust_grad_shape, src/AutoDiff.cpp:690-757, returns row 0 instead;
  * that behaviour is a ctamd_memcpy_d2d of the first row followed by ctamd_accumulate_f32). */
@@ -161,6 +205,16 @@ int ctamd_any_abs_lt_eps_f32(const float* b, int32_t* flag, size_t n, void* stre
  * normalisation is a true division as in the reference. */
 int ctamd_softmax_rows_f32(const float* x, float* y, size_t rows, size_t cols, void* stream);
 int ctamd_softmax_cols_f32(const float* x, float* y, size_t rows, size_t cols, void* stream);
+/* Tensor::log_softmax(dim), declared by the reference and never defined (include/Tensor.h:1072):
+ * y = (x - max) - log(sum_j exp(x_j - max)) per row (dim 1 / 1-D) or per column (dim 0), in the style
+ * of Tensor::softmax (src/Tensor.cpp:1713-1744): the maximum subtracted first, expf terms of glibc's
+ * bits summed in a tree, glibc's logf of the sum; rows of 2048 columns or more and matrices of 128
+ * rows or more (columns) form the sum from the hardware exponential (~1e-7 relative).  Gradient:
+ * dx = g - exp(y) * sum_j g_j. */
+int ctamd_log_softmax_rows_f32(const float* x, float* y, size_t rows, size_t cols, void* stream);
+int ctamd_log_softmax_cols_f32(const float* x, float* y, size_t rows, size_t cols, void* stream);
+int ctamd_log_softmax_backward_rows_f32(const float* y, const float* g, float* dx, size_t rows, size_t cols, void* stream);
+int ctamd_log_softmax_backward_cols_f32(const float* y, const float* g, float* dx, size_t rows, size_t cols, void* stream);
 /* out[0] = SUM over rows of -sum_j t[i,j] * log(max(softmax(x)[i,j], 1e-10)).
  * CrossEntropy_BASIC_kernel.cpp:41-66 (2-D one-hot or soft targets), :67-82 (1-D: rows = 1). */
 int ctamd_cross_entropy_onehot_f32(const float* x, const float* t, float* out, size_t rows, size_t cols,
@@ -356,6 +410,14 @@ int ctamd_cross_entropy_backward_onehot_f32(const float* x, const float* t, cons
                                             size_t rows, size_t cols, void* stream);
 int ctamd_cross_entropy_backward_index_f32(const float* x, const float* idx, const float* g1, float* dx,
                                            size_t rows, size_t cols, void* stream);
+/* Gradients of the operators above that the reference declares without defining: sign(x) * g (sign(0)
+ * = 0); g / (y * 2) with y = sqrt(x); (x * 2) * g; (1 + y * y) * g with y = tan(x); g * (x > 0 ? 1 :
+ * slope).  exp's is y * g and log's g / x: ctamd_mul_f32 and ctamd_div_f32. */
+int ctamd_abs_backward_f32(const float* x, const float* g, float* dx, size_t n, void* stream);
+int ctamd_sqrt_backward_f32(const float* y, const float* g, float* dx, size_t n, void* stream);
+int ctamd_square_backward_f32(const float* x, const float* g, float* dx, size_t n, void* stream);
+int ctamd_tan_backward_f32(const float* y, const float* g, float* dx, size_t n, void* stream);
+int ctamd_leaky_relu_backward_f32(const float* x, const float* g, float slope, float* dx, size_t n, void* stream);
 /* db = ((-a) * g) / (b * b).  src/AutoDiff.cpp:1314.  (da = g / b is ctamd_div_f32, :1285.) */
 int ctamd_div_backward_b_f32(const float* a, const float* b, const float* g, float* db, size_t n, void* stream);
 /* The same for a row-vector divisor b[cols] under a[rows, cols] (the broadcast Div of this backend):

@@ -34,6 +34,14 @@
  * The MNIST functions (co_u8_to_unit ... co_mnist_predict) are
  * pinned bit for bit against the reference's loader, demo functions and its own main()
  * (tests/test_oracle_vs_ref_mnist.py, tests/golden/mnist.npz).
+ * co_adjust_grad_shape (the reference's whole gradient shape adjustment) is pinned bit for bit
+ * against the reference through its public AutoDiff::backward(root, grad_output) on every shape pair
+ * for which the reference stays inside its buffers (tests/test_oracle_vs_ref.py).
+ * The methods the reference declares and never defines have no reference arithmetic to be in parity
+ * with; their oracle functions are PINNED BY MATHEMATICS only (tests/test_oracle_math.py: numpy in
+ * double, closed forms, brute force on tiny inputs, central differences for the gradients):
+ *   co_unary_ext, co_unary_ext_bwd, co_reduce_dim, co_reduce_dim_bwd, co_log_softmax,
+ *   co_log_softmax_bwd, co_broadcast_reduce.
  * Transcendentals call glibc libm (expf, logf, sinf, cosf) exactly as the reference does; their
  * values are whatever the installed glibc returns (2.35 in this image).
  */
@@ -946,6 +954,256 @@ int co_expr_run(const int* prog, const float* imm, int n, const float* const* in
         }
     }
     return 0;
+}
+
+/* ------------------------------------------- gradient shape adjustment, the whole function */
+
+/* src/AutoDiff.cpp:562-1049, check_and_adjust_grad_shape, every branch, for float tensors of up to
+ * 8 dimensions.  Returns 0, or -1 where the reference itself reads beyond the end of the gradient
+ * (its index arithmetic at :727-757 takes the flat result index as the last coordinate), or -2 for
+ * more than 8 dimensions.  gs / ts: shapes, gr / tr: ranks.
+ *   :565-567   equal shapes: the gradient itself
+ *   :579-627   0-D gradient: every element of the result is its value
+ *   :633-687   rank(g) < rank(target): the gradient is copied into a tensor of shape [1, .., 1, g's
+ *              dims] element i from element i % numel(g) (the two element counts are equal, so this
+ *              is a reshape), then the function calls itself
+ *   :690-890   "can broadcast" (every trailing pair of dims equal or one of them 1): result[i] =
+ *              0 + g[grad_index(i)]; the coordinate loop :727-732 runs from the LAST dimension with
+ *              the full flat index, so the last coordinate is i itself and all others are 0: the
+ *              gradient's element i (or element 0 when its last dimension is 1)
+ *   :892-966   "can reduce": result[i % numel] += g[i] (unreachable: its condition implies the
+ *              previous one; kept in the order of the source)
+ *   :968-1046  otherwise: result[i] = sum over j with j % numel(result) == i of g[j], from 0 */
+int co_adjust_grad_shape(const float* g, const long* gs, int gr, float* out, const long* ts, int tr) {
+    if (gr > 8 || tr > 8) return -2;
+    long gn = 1, tn = 1;
+    for (int i = 0; i < gr; ++i) gn *= gs[i];
+    for (int i = 0; i < tr; ++i) tn *= ts[i];
+    int same = gr == tr;
+    for (int i = 0; same && i < gr; ++i) same = gs[i] == ts[i];
+    if (same) {
+        memcpy(out, g, (size_t)gn * sizeof(float));
+        return 0;
+    }
+    if (gr == 0) {
+        for (long i = 0; i < tn; ++i) out[i] = g[0];
+        return 0;
+    }
+    if (gr < tr) {
+        long ns[8];
+        for (int i = 0; i < tr; ++i) ns[i] = 1;
+        for (int i = 0; i < gr; ++i) ns[tr - gr + i] = gs[i];
+        float* temp = (float*)malloc((size_t)(gn > 0 ? gn : 1) * sizeof(float));
+        for (long i = 0; i < gn; ++i) temp[i] = g[i % gn];
+        int rc = co_adjust_grad_shape(temp, ns, tr, out, ts, tr);
+        free(temp);
+        return rc;
+    }
+    int can_broadcast = 1;
+    for (int i = 1; i <= tr; ++i) {
+        long gd = gs[gr - i], td = ts[tr - i];
+        if (gd != td && gd != 1 && td != 1) { can_broadcast = 0; break; }
+    }
+    if (can_broadcast) {
+        long gstr[8], rstr[8];
+        for (int i = gr - 1, a = 1; i >= 0; --i) { gstr[i] = a; a *= gs[i]; }
+        for (int i = tr - 1, a = 1; i >= 0; --i) { rstr[i] = a; a *= ts[i]; }
+        for (long i = 0; i < tn; ++i) {
+            long ri[8] = {0}, gi[8] = {0};
+            long temp = i;
+            for (int j = tr - 1; j >= 0; --j) {
+                ri[j] = temp / rstr[j];
+                temp %= rstr[j];
+            }
+            for (int j = 1; j <= tr; ++j) gi[gr - j] = (gs[gr - j] == 1) ? 0 : ri[tr - j];
+            long at = 0;
+            for (int j = 0; j < gr; ++j) at += gi[j] * gstr[j];
+            if (at >= gn) return -1;
+            out[i] = 0.0f + g[at];
+        }
+        return 0;
+    }
+    int can_reduce = 1;
+    for (int i = 1; i <= (gr < tr ? gr : tr); ++i) {
+        long gd = gs[gr - i], td = ts[tr - i];
+        if (gd != td && td != 1) { can_reduce = 0; break; }
+    }
+    if (can_reduce) {
+        for (long i = 0; i < tn; ++i) out[i] = 0.0f;
+        for (long i = 0; i < gn; ++i) out[i % tn] += g[i];
+        return 0;
+    }
+    for (long i = 0; i < tn; ++i) {
+        float sum = 0.0f;
+        for (long j = i; j < gn; j += tn) sum += g[j];
+        out[i] = sum;
+    }
+    return 0;
+}
+
+/* Extension: the gradient of a broadcast operand as the mathematics has it.  The target shape is
+ * padded with leading 1s to the gradient's rank; per dimension the two extents are equal (kept), the
+ * target's is 1 (summed over) or the gradient's is 1 (repeated).  Sums in double, in index order.
+ * -1: the shapes do not broadcast. */
+int co_broadcast_reduce(const float* g, const long* gs, int gr, float* out, const long* ts, int tr) {
+    if (gr > 8 || tr > gr) return -1;
+    long tp[8], tn = 1;
+    for (int i = 0; i < gr; ++i) tp[i] = (i < gr - tr) ? 1 : ts[i - (gr - tr)];
+    for (int i = 0; i < gr; ++i) {
+        if (tp[i] != gs[i] && tp[i] != 1 && gs[i] != 1) return -1;
+        tn *= tp[i];
+    }
+    long gstr[8];
+    for (int i = gr - 1, a = 1; i >= 0; --i) { gstr[i] = a; a *= gs[i]; }
+    for (long o = 0; o < tn; ++o) {
+        long rem = o, base = 0, red = 1;
+        for (int d = gr - 1; d >= 0; --d) {
+            long c = rem % tp[d];
+            rem /= tp[d];
+            if (gs[d] == tp[d]) base += c * gstr[d];
+        }
+        for (int d = 0; d < gr; ++d) if (tp[d] == 1 && gs[d] > 1) red *= gs[d];
+        double sum = 0.0;
+        for (long r = 0; r < red; ++r) {
+            long q = r, at = base;
+            for (int d = gr - 1; d >= 0; --d)
+                if (tp[d] == 1 && gs[d] > 1) { at += (q % gs[d]) * gstr[d]; q /= gs[d]; }
+            sum += (double)g[at];
+        }
+        out[o] = (float)sum;
+    }
+    return 0;
+}
+
+/* ------------------- methods the reference declares on Tensor and never defines (extensions) */
+
+/* include/Tensor.h:719 operator-(float), :954-972 abs / exp / log / sqrt, :978 square, :996 tan,
+ * :1052 leaky_relu(negative_slope): no bodies exist in the reference, so each is the C++ library call
+ * that its name stands for, on floats.  op: 0 abs, 1 exp, 2 log, 3 sqrt, 4 square, 5 tan,
+ * 6 leaky_relu (p = slope), 7 a - p. */
+void co_unary_ext(int op, const float* a, float p, float* r, long n) {
+    for (long i = 0; i < n; ++i) {
+        float x = a[i];
+        switch (op) {
+            case 0: r[i] = fabsf(x); break;
+            case 1: r[i] = expf(x); break;
+            case 2: r[i] = logf(x); break;
+            case 3: r[i] = sqrtf(x); break;
+            case 4: r[i] = x * x; break;
+            case 5: r[i] = tanf(x); break;
+            case 6: r[i] = (x > 0.0f) ? x : x * p; break;
+            default: r[i] = x - p; break;
+        }
+    }
+}
+/* Their gradients, the factor evaluated in fp32 in the stated order and then multiplied by g:
+ * abs sign(x) * g; exp y * g; log g / x; sqrt g / (y * 2); square (x * 2) * g; tan (1 + y * y) * g;
+ * leaky_relu g * (x > 0 ? 1 : slope); a - p: g.  v = x for abs, log, square, leaky_relu and the
+ * result y for exp, sqrt, tan. */
+void co_unary_ext_bwd(int op, const float* v, const float* g, float p, float* dx, long n) {
+    for (long i = 0; i < n; ++i) {
+        float x = v[i], u = g[i];
+        switch (op) {
+            case 0: { float s = (x > 0.0f) ? 1.0f : ((x < 0.0f) ? -1.0f : 0.0f); dx[i] = s * u; break; }
+            case 1: dx[i] = x * u; break;
+            case 2: dx[i] = u / x; break;
+            case 3: { float d = x * 2.0f; dx[i] = u / d; break; }
+            case 4: { float d = x * 2.0f; dx[i] = d * u; break; }
+            case 5: { float yy = x * x; float s = 1.0f + yy; dx[i] = s * u; break; }
+            case 6: { float m = (x > 0.0f) ? 1.0f : p; dx[i] = u * m; break; }
+            default: dx[i] = u; break;
+        }
+    }
+}
+
+/* include/Tensor.h:824-948: sum / mean / max / min / std / var over a dimension, declared only.
+ * x is read as [outer, len, inner]; out[o, i] reduces x[o, :, i].  kind: 0 sum (fp32, in index
+ * order, as Tensor::sum() src/Tensor.cpp:644-647 adds), 1 mean (that sum / float(len)), 2 max and
+ * 3 min (m = element 0, then `if (v > m)` / `if (v < m)` in index order: the first occurrence wins
+ * and a NaN only stays when it comes first; index = its position), 4 var and 5 std (two passes in
+ * double: mean, then sum of squared deviations / (len - ddof)); mean_out (4, 5) the mean as a float. */
+void co_reduce_dim(int kind, const float* x, float* out, int* index, float* mean_out, long outer, long len, long inner, int ddof) {
+    for (long o = 0; o < outer; ++o)
+        for (long i = 0; i < inner; ++i) {
+            const float* p = x + o * len * inner + i;
+            long at = o * inner + i;
+            if (kind == 0 || kind == 1) {
+                float s = 0.0f;
+                for (long l = 0; l < len; ++l) s += p[l * inner];
+                out[at] = kind == 0 ? s : s / (float)len;
+            } else if (kind == 2 || kind == 3) {
+                float m = p[0];
+                int pos = 0;
+                for (long l = 1; l < len; ++l) {
+                    float v = p[l * inner];
+                    if (kind == 2 ? (v > m) : (v < m)) { m = v; pos = (int)l; }
+                }
+                out[at] = m;
+                if (index) index[at] = pos;
+            } else {
+                double mean = 0.0, m2 = 0.0;
+                for (long l = 0; l < len; ++l) mean += (double)p[l * inner];
+                mean /= (double)len;
+                for (long l = 0; l < len; ++l) { double d = (double)p[l * inner] - mean; m2 += d * d; }
+                double var = m2 / ((double)len - (double)ddof);
+                out[at] = kind == 4 ? (float)var : (float)sqrt(var);
+                if (mean_out) mean_out[at] = (float)mean;
+            }
+        }
+}
+/* Gradients of the six, every step rounded to fp32 in this order: sum g; mean g / float(len);
+ * max / min g at index and +0 elsewhere; var ((x - mean) * 2 / float(len - ddof)) * g;
+ * std ((x - mean) / (float(len - ddof) * y)) * g. */
+void co_reduce_dim_bwd(int kind, const float* x, const float* y, const int* index, const float* mean, const float* g, float* dx,
+                       long outer, long len, long inner, int ddof) {
+    for (long o = 0; o < outer; ++o)
+        for (long i = 0; i < inner; ++i) {
+            long at = o * inner + i;
+            float u = g[at];
+            float nf = (float)((double)len - (double)ddof);
+            for (long l = 0; l < len; ++l) {
+                long e = (o * len + l) * inner + i;
+                if (kind == 0) dx[e] = u;
+                else if (kind == 1) dx[e] = u / (float)len;
+                else if (kind == 2 || kind == 3) dx[e] = (l == index[at]) ? u : 0.0f;
+                else {
+                    float d = x[e] - mean[at];
+                    if (kind == 4) { float t = d * 2.0f; float q = t / nf; dx[e] = q * u; }
+                    else { float den = nf * y[at]; float q = d / den; dx[e] = q * u; }
+                }
+            }
+        }
+}
+
+/* include/Tensor.h:1072 log_softmax(dim), declared only.  In the style of Tensor::softmax
+ * (src/Tensor.cpp:1713-1744): m = max (first wins), s = sum of expf(x - m) in index order,
+ * y = (x - m) - logf(s).  dim 1: rows, dim 0: columns. */
+void co_log_softmax(const float* x, float* y, long rows, long cols, int dim) {
+    long runs = dim == 1 ? rows : cols, len = dim == 1 ? cols : rows;
+    long step = dim == 1 ? 1 : cols, jump = dim == 1 ? cols : 1;
+    for (long r = 0; r < runs; ++r) {
+        const float* p = x + r * jump;
+        float m = p[0];
+        for (long j = 1; j < len; ++j) if (p[j * step] > m) m = p[j * step];
+        float s = 0.0f;
+        for (long j = 0; j < len; ++j) s += expf(p[j * step] - m);
+        float lg = logf(s);
+        for (long j = 0; j < len; ++j) { float d = p[j * step] - m; y[r * jump + j * step] = d - lg; }
+    }
+}
+/* its gradient: d = sum of g in index order; dx = g - expf(y) * d */
+void co_log_softmax_bwd(const float* y, const float* g, float* dx, long rows, long cols, int dim) {
+    long runs = dim == 1 ? rows : cols, len = dim == 1 ? cols : rows;
+    long step = dim == 1 ? 1 : cols, jump = dim == 1 ? cols : 1;
+    for (long r = 0; r < runs; ++r) {
+        float d = 0.0f;
+        for (long j = 0; j < len; ++j) d += g[r * jump + j * step];
+        for (long j = 0; j < len; ++j) {
+            long e = r * jump + j * step;
+            float t = expf(y[e]) * d;
+            dx[e] = g[e] - t;
+        }
+    }
 }
 
 /* ------------------------------------------------------------------------- input generator */

@@ -55,6 +55,18 @@ void co_div_bwd_a(const float* g, const float* b, float* da, long n);
 void co_div_bwd_b(const float* a, const float* b, const float* g, float* db, long n);
 int co_any_abs_lt_eps(const float* b, long n);
 
+int co_adjust_grad_shape(const float* g, const long* gs, int gr, float* out, const long* ts, int tr);
+int co_broadcast_reduce(const float* g, const long* gs, int gr, float* out, const long* ts, int tr);
+
+/* methods the reference declares and never defines (pinned by mathematics) */
+void co_unary_ext(int op, const float* a, float p, float* r, long n);
+void co_unary_ext_bwd(int op, const float* v, const float* g, float p, float* dx, long n);
+void co_reduce_dim(int kind, const float* x, float* out, int* index, float* mean_out, long outer, long len, long inner, int ddof);
+void co_reduce_dim_bwd(int kind, const float* x, const float* y, const int* index, const float* mean, const float* g, float* dx,
+                       long outer, long len, long inner, int ddof);
+void co_log_softmax(const float* x, float* y, long rows, long cols, int dim);
+void co_log_softmax_bwd(const float* y, const float* g, float* dx, long rows, long cols, int dim);
+
 /* whole configurations, composed from the pieces above in the reference's op order */
 void co_chain(const float* a, const float* b, long n, float* s, float* ga, float* gb);
 void co_mlp_step(const float* x, long B, long I, const float* W1, const float* b1, long H,

@@ -201,6 +201,32 @@ long ref_matmul_t(const float* a, long ar, long ac, int ta, const float* b, long
     }
 }
 
+// check_and_adjust_grad_shape (src/AutoDiff.cpp:562-1049, private) through the public
+// AutoDiff::backward(root, grad_output), which stores check_and_adjust_grad_shape(grad_output,
+// root shape) as the root's gradient (:1124-1126).  The root is a leaf, so nothing else runs.
+// The caller must only pass shape pairs for which the reference stays inside the gradient's buffer.
+long ref_adjust_grad_shape(const float* g, const long* gd, int gn, const long* td, int tn, float* out) {
+    try {
+        AutoDiff ctx;
+        Tensor tg = make(g, gd, gn);
+        Tensor root;
+        {
+            AutoDiffContext::Guard guard(&ctx);
+            if (tn == 0) root = Tensor(0.0f);
+            else root = Tensor(ShapeTag{}, shape_of(td, tn), DType::kFloat, DeviceType::kCPU);
+            root.requires_grad(true);
+        }
+        {
+            AutoDiffContext::Guard none(nullptr);
+            ctx.backward(root, tg);
+        }
+        AutoDiffContext::Guard guard(&ctx);
+        return emit(grad(root), out);
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
 // d/dx of  sum( f(x) * w )  through the reference's tape: the upstream gradient of f is w.
 long ref_grad_unary(int code, const float* x, const long* xd, int xn, const float* w, float* dx) {
     try {

@@ -1,6 +1,7 @@
 /* Host check of ctorch_amd/csrc/devmath.h against the installed glibc: counts the floats for
  * which the device algorithms (compiled here for the CPU, unchanged) return different bits from
- * expf / sinf / cosf.  Usage: devmath_check STRIDE  (1 = every one of the 2^32 bit patterns).
+ * expf / sinf / cosf / logf, and the worst distance of the tangent from glibc's tanf (not the same
+ * algorithm: at most 1 ulp).  Usage: devmath_check STRIDE  (1 = every one of the 2^32 bit patterns).
  * Prints one line per function: name, inputs tested, mismatches, worst ulp distance
  * (expf_pair: exp(x) and exp(-x) from the shared reduction, against expf(x) and expf(-x)). */
 #include <math.h>
@@ -25,9 +26,9 @@ static int differs(float a, float b, int64_t* ulp) {
 int main(int argc, char** argv) {
     uint64_t stride = argc > 1 ? strtoull(argv[1], 0, 10) : 1;
     if (stride == 0) stride = 1;
-    uint64_t n = 0, bad[4] = {0, 0, 0, 0}, covered[4] = {0, 0, 0, 0};
-    int64_t worst[4] = {0, 0, 0, 0};
-#pragma omp parallel for reduction(+ : n, bad[:4], covered[:4]) reduction(max : worst[:4]) schedule(static)
+    uint64_t n = 0, bad[6] = {0, 0, 0, 0, 0, 0}, covered[6] = {0, 0, 0, 0, 0, 0};
+    int64_t worst[6] = {0, 0, 0, 0, 0, 0};
+#pragma omp parallel for reduction(+ : n, bad[:6], covered[:6]) reduction(max : worst[:6]) schedule(static)
     for (uint64_t u = 0; u < (1ULL << 32); u += stride) {
         float x = cta_u2f((uint32_t)u);
         int64_t d = 0;
@@ -58,9 +59,19 @@ int main(int argc, char** argv) {
             ++bad[2];
             if (d > worst[2]) worst[2] = d;
         }
+        ++covered[4];
+        if (differs(cta_logf(x, cta_log_tab), logf(x), &d)) {
+            ++bad[4];
+            if (d > worst[4]) worst[4] = d;
+        }
+        ++covered[5];
+        if (differs(cta_tanf(x, cta_inv_pio4), tanf(x), &d)) {
+            if (d > 1) ++bad[5];                   /* a different algorithm: 1 ulp apart is expected */
+            if (d > worst[5]) worst[5] = d;
+        }
     }
-    const char* names[4] = {"expf", "sinf", "cosf", "expf_pair"};
-    for (int k = 0; k < 4; ++k)
+    const char* names[6] = {"expf", "sinf", "cosf", "expf_pair", "logf", "tanf(>1ulp)"};
+    for (int k = 0; k < 6; ++k)
         printf("%s tested %llu mismatches %llu worst_ulp %lld\n", names[k], (unsigned long long)covered[k],
                (unsigned long long)bad[k], (long long)worst[k]);
     return 0;

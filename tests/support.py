@@ -275,6 +275,76 @@ class Oracle:
         self.lib.co_colsum_f64(fp(g), r.ctypes.data_as(DP), C.c_long(g.shape[0]), C.c_long(g.shape[1]))
         return r
 
+    # ---- gradient shape adjustment (the reference's whole function) and its mathematical twin
+    def adjust_grad_shape(self, g, target_shape):
+        """co_adjust_grad_shape; None where the reference would read beyond its gradient buffer."""
+        g = f32(g)
+        gs = (C.c_long * max(1, g.ndim))(*g.shape)
+        ts = (C.c_long * max(1, len(target_shape)))(*target_shape)
+        out = np.empty(target_shape, np.float32)
+        rc = self.lib.co_adjust_grad_shape(fp(g.reshape(-1)), gs, C.c_int(g.ndim), fp(out.reshape(-1)), ts, C.c_int(len(target_shape)))
+        assert rc in (0, -1), rc
+        return out if rc == 0 else None
+
+    def broadcast_reduce(self, g, target_shape):
+        g = f32(g)
+        gs = (C.c_long * max(1, g.ndim))(*g.shape)
+        ts = (C.c_long * max(1, len(target_shape)))(*target_shape)
+        out = np.empty(target_shape, np.float32)
+        rc = self.lib.co_broadcast_reduce(fp(g.reshape(-1)), gs, C.c_int(g.ndim), fp(out.reshape(-1)), ts, C.c_int(len(target_shape)))
+        return out if rc == 0 else None
+
+    # ---- methods the reference declares and never defines
+    UNARY_EXT = {"abs": 0, "exp": 1, "log": 2, "sqrt": 3, "square": 4, "tan": 5, "leaky_relu": 6, "sub_scalar": 7}
+
+    def unary_ext(self, name, a, p=0.0):
+        a = f32(a)
+        r = np.empty_like(a)
+        self.lib.co_unary_ext(C.c_int(self.UNARY_EXT[name]), fp(a), C.c_float(p), fp(r), C.c_long(a.size))
+        return r
+
+    def unary_ext_bwd(self, name, v, g, p=0.0):
+        v, g = f32(v), f32(g)
+        r = np.empty_like(v)
+        self.lib.co_unary_ext_bwd(C.c_int(self.UNARY_EXT[name]), fp(v), fp(g), C.c_float(p), fp(r), C.c_long(v.size))
+        return r
+
+    REDUCE = {"sum": 0, "mean": 1, "max": 2, "min": 3, "var": 4, "std": 5}
+
+    def reduce_dim(self, kind, x, outer, length, inner, ddof=1):
+        """-> (out [outer, inner], index int32 [outer, inner], mean [outer, inner])"""
+        x = f32(x)
+        assert x.size == outer * length * inner
+        out = np.empty((outer, inner), np.float32)
+        index = np.zeros((outer, inner), np.int32)
+        mean = np.zeros((outer, inner), np.float32)
+        self.lib.co_reduce_dim(C.c_int(self.REDUCE[kind]), fp(x.reshape(-1)), fp(out.reshape(-1)), index.ctypes.data_as(C.c_void_p),
+                               fp(mean.reshape(-1)), C.c_long(outer), C.c_long(length), C.c_long(inner), C.c_int(ddof))
+        return out, index, mean
+
+    def reduce_dim_bwd(self, kind, x, y, index, mean, g, outer, length, inner, ddof=1):
+        x, y, mean, g = f32(x), f32(y), f32(mean), f32(g)
+        index = np.ascontiguousarray(index, np.int32)
+        dx = np.empty(outer * length * inner, np.float32)
+        self.lib.co_reduce_dim_bwd(C.c_int(self.REDUCE[kind]), fp(x.reshape(-1)), fp(y.reshape(-1)), index.ctypes.data_as(C.c_void_p),
+                                   fp(mean.reshape(-1)), fp(g.reshape(-1)), fp(dx), C.c_long(outer), C.c_long(length), C.c_long(inner),
+                                   C.c_int(ddof))
+        return dx.reshape(x.shape)
+
+    def log_softmax(self, x, dim=1):
+        x = f32(x)
+        x2 = x.reshape(1, -1) if x.ndim == 1 else x
+        y = np.empty_like(x2)
+        self.lib.co_log_softmax(fp(x2), fp(y), C.c_long(x2.shape[0]), C.c_long(x2.shape[1]), C.c_int(1 if x.ndim == 1 else dim))
+        return y.reshape(x.shape)
+
+    def log_softmax_bwd(self, y, g, dim=1):
+        y, g = f32(y), f32(g)
+        y2 = y.reshape(1, -1) if y.ndim == 1 else y
+        r = np.empty_like(y2)
+        self.lib.co_log_softmax_bwd(fp(y2), fp(g), fp(r), C.c_long(y2.shape[0]), C.c_long(y2.shape[1]), C.c_int(1 if y.ndim == 1 else dim))
+        return r.reshape(y.shape)
+
     # ---- configurations
     def chain(self, a, b):
         a, b = f32(a), f32(b)
@@ -773,6 +843,17 @@ class Reference:
         rc = self.lib.ref_grad_loss(code, fp(p), pd, pn, fp(t), td, tn, C.c_float(scale), C.byref(loss), fp(dp))
         return rc, np.float32(loss.value), dp
 
+    def adjust_grad_shape(self, g, target_shape):
+        """The gradient a root of `target_shape` holds after backward(root, grad_output = g): the
+        reference's check_and_adjust_grad_shape (src/AutoDiff.cpp:562-1049) through its public door
+        (:1124-1126).  None when the call failed."""
+        g = f32(g)
+        out = np.empty(target_shape, np.float32)
+        gd, gn = _dims(g.shape)
+        td, tn = _dims(tuple(target_shape))
+        n = self.lib.ref_adjust_grad_shape(fp(g.reshape(-1)), gd, gn, td, tn, fp(out.reshape(-1)))
+        return out if n == out.size else None
+
     def chain(self, a, b):
         a, b = f32(a), f32(b)
         s = C.c_float(0)
@@ -880,12 +961,12 @@ class Reference:
         return int(self.lib.ref_mnist_main_in(directory.encode()))
 
 
-HOST_LIB = os.path.join(ROOT, "ctorch_amd", "host", "libctorch_amd_host.so")
+HOST_LIB = os.path.join(ROOT, "ctorch_amd", "host", "tests", "harness", "libctorch_amd_harness.so")
 
 
 class HostLayer(Reference):
     """This repository's C++ front-end (Tensor / Ctorch_Scheduler / AutoDiff over the HIP launch layer)
-    through ctorch_amd/host/src/capi_host.cpp.  Needs a GPU for every call."""
+    through the test doorway ctorch_amd/host/tests/harness/capi_host.cpp.  Needs a GPU for every call."""
 
     def __init__(self):
         Reference.__init__(self, HOST_LIB, "cth_")

@@ -207,3 +207,184 @@ def test_input_generator_is_stable(oracle):
     assert abs(z.mean()) < 0.01 and abs(z.std() - 1) < 0.01
     k = oracle.ints((100000,), 9, 10)
     assert k.min() == 0 and k.max() == 9 and abs(k.mean() - 4.5) < 0.05
+
+
+# --------------------------------------------------------------------------------------------
+# The methods the reference declares on Tensor and never defines (include/Tensor.h:719, 824-1072):
+# no reference run can pin their oracle functions, so the mathematics does - numpy in double,
+# closed forms, brute force on tiny inputs, and central differences for the gradients.  Each check is
+# chosen so that a plausible slip (wrong ddof, wrong sign, axis mix-up, last instead of first
+# extreme, dropped factor 2) fails it.
+
+def _numeric_gradient(f, x, eps=1e-6):
+    """Central differences of a scalar function of a float64 array."""
+    g = np.zeros_like(x)
+    flat, gf = x.reshape(-1), g.reshape(-1)
+    for i in range(flat.size):
+        keep = flat[i]
+        flat[i] = keep + eps
+        up = f(x)
+        flat[i] = keep - eps
+        down = f(x)
+        flat[i] = keep
+        gf[i] = (up - down) / (2 * eps)
+    return g
+
+
+def test_extension_unary_operators_against_double_precision(oracle):
+    x = np.concatenate([oracle.normal((4000,), 41, 0, 3), np.array([0.0, -0.0, 1.0, -1.0, 0.5, 88.0, -88.0, 1e-30, 3e38], F)])
+    pos = np.abs(x) + F(1e-3)
+    x64, pos64 = x.astype(np.float64), pos.astype(np.float64)
+    assert same_bits(oracle.unary_ext("abs", x), np.abs(x))
+    with np.errstate(over="ignore"):
+        assert same_bits(oracle.unary_ext("square", x), x * x)
+    assert same_bits(oracle.unary_ext("sqrt", pos), np.sqrt(pos))                 # IEEE: correctly rounded
+    assert same_bits(oracle.unary_ext("sub_scalar", x, 1.25), x - F(1.25))
+    lr = oracle.unary_ext("leaky_relu", x, 0.01)
+    assert same_bits(lr, np.where(x > 0, x, x * F(0.01)))
+    assert lr[np.where(x == -1.0)[0][0]] == F(-0.01)
+    with np.errstate(over="ignore"):
+        assert ulp_diff(oracle.unary_ext("exp", x), np.exp(x64).astype(F)).max() <= 1
+    assert ulp_diff(oracle.unary_ext("log", pos), np.log(pos64).astype(F)).max() <= 1
+    small = x[np.abs(x) < 50]
+    assert ulp_diff(oracle.unary_ext("tan", small), np.tan(small.astype(np.float64)).astype(F)).max() <= 1
+    # identities: exp(log(x)) = x, tan = sin / cos, sqrt(x)^2 = x
+    assert np.allclose(oracle.unary_ext("exp", oracle.unary_ext("log", pos)), pos, rtol=5e-6)
+    assert np.allclose(oracle.unary_ext("tan", small), oracle.sin(small) / oracle.cos(small), rtol=1e-5, atol=1e-6)
+    # special values of the library calls
+    assert np.isneginf(oracle.unary_ext("log", np.zeros(1, F))[0]) and np.isnan(oracle.unary_ext("log", np.array([-1.0], F))[0])
+    assert np.isnan(oracle.unary_ext("sqrt", np.array([-4.0], F))[0]) and oracle.unary_ext("sqrt", np.array([-0.0], F)).view(np.uint32)[0] == 0x80000000
+
+
+def test_extension_unary_gradients_against_central_differences(oracle):
+    x = oracle.uniform((24,), 43, 0.3, 1.4)        # positive, inside (0, pi/2): every operator is smooth there
+    x[::3] *= F(-1.0)
+    w = oracle.normal((24,), 44)
+    x64, w64 = x.astype(np.float64), w.astype(np.float64)
+    fns = {
+        "abs": (np.abs, x), "exp": (np.exp, x), "square": (np.square, x), "tan": (np.tan, x),
+        "log": (np.log, np.abs(x)), "sqrt": (np.sqrt, np.abs(x)),
+        "leaky_relu": (lambda t: np.where(t > 0, t, 0.2 * t), x), "sub_scalar": (lambda t: t - 0.5, x),
+    }
+    for name, (fn, at) in fns.items():
+        at64 = at.astype(np.float64)
+        want = _numeric_gradient(lambda t: float(np.sum(w64 * fn(t))), at64.copy())
+        v = at if name in ("abs", "log", "square", "leaky_relu", "sub_scalar") else oracle.unary_ext(name, at)
+        got = oracle.unary_ext_bwd(name, v, w, 0.2 if name == "leaky_relu" else 0.5)
+        assert np.allclose(got, want, rtol=2e-5, atol=2e-6), name
+    # sign conventions at zero: d|x|/dx = 0 there, and the leaky slope applies to x <= 0
+    z = np.array([0.0, -0.0], F)
+    assert np.all(oracle.unary_ext_bwd("abs", z, np.ones(2, F)) == 0)
+    assert np.all(oracle.unary_ext_bwd("leaky_relu", z, np.ones(2, F), 0.3) == F(0.3))
+
+
+def _as3(x, outer, length, inner):
+    return np.asarray(x, np.float64).reshape(outer, length, inner)
+
+
+def test_reductions_along_an_axis_against_numpy_in_double(oracle):
+    for (outer, length, inner), seed in [((1, 37, 1), 1), ((5, 9, 1), 2), ((1, 11, 6), 3), ((3, 7, 4), 4), ((2, 1, 3), 5)]:
+        x = oracle.normal((outer, length, inner), 60 + seed, 3.0, 2.0)
+        x3 = _as3(x, outer, length, inner)
+        for kind, fn in [("sum", np.sum), ("mean", np.mean), ("max", np.max), ("min", np.min)]:
+            out, index, _ = oracle.reduce_dim(kind, x, outer, length, inner)
+            assert np.allclose(out, fn(x3, axis=1), rtol=1e-6, atol=1e-6), (kind, outer, length, inner)
+            if kind in ("max", "min"):
+                assert same_bits(out, fn(x3, axis=1).astype(F))
+                want = np.argmax(x3, axis=1) if kind == "max" else np.argmin(x3, axis=1)
+                assert np.array_equal(index, want)
+        if length > 1:
+            for ddof in (0, 1):
+                out, _, mean = oracle.reduce_dim("var", x, outer, length, inner, ddof)
+                assert np.allclose(out, np.var(x3, axis=1, ddof=ddof), rtol=1e-6), (ddof, outer, length, inner)
+                assert np.allclose(mean, np.mean(x3, axis=1), rtol=1e-6)
+                out, _, _ = oracle.reduce_dim("std", x, outer, length, inner, ddof)
+                assert np.allclose(out, np.std(x3, axis=1, ddof=ddof), rtol=1e-6)
+
+
+def test_reductions_closed_forms_and_first_occurrence(oracle):
+    n = 101
+    x = np.arange(1, n + 1, dtype=F)
+    assert oracle.reduce_dim("sum", x, 1, n, 1)[0][0, 0] == n * (n + 1) / 2
+    assert oracle.reduce_dim("mean", x, 1, n, 1)[0][0, 0] == (n + 1) / 2
+    assert oracle.reduce_dim("var", x, 1, n, 1, 0)[0][0, 0] == F((n * n - 1) / 12)      # variance of 1..n
+    assert oracle.reduce_dim("var", x, 1, n, 1, 1)[0][0, 0] == F(n * (n + 1) / 12)      # with Bessel's correction
+    assert abs(oracle.reduce_dim("std", x + F(1e4), 1, n, 1, 0)[0][0, 0] - np.sqrt((n * n - 1) / 12)) < 1e-4   # shift invariant
+    assert oracle.reduce_dim("var", np.full(50, 7.25, F), 1, 50, 1)[0][0, 0] == 0
+    # ties: the first occurrence; NaN: only a leading one stays (a loop `if (v > m)` from element 0)
+    t = np.array([1, 5, 2, 5, -3, -3], F)
+    out, idx, _ = oracle.reduce_dim("max", t, 1, 6, 1)
+    assert out[0, 0] == 5 and idx[0, 0] == 1
+    out, idx, _ = oracle.reduce_dim("min", t, 1, 6, 1)
+    assert out[0, 0] == -3 and idx[0, 0] == 4
+    out, idx, _ = oracle.reduce_dim("max", np.array([1, np.nan, 3], F), 1, 3, 1)
+    assert out[0, 0] == 3 and idx[0, 0] == 2
+    out, idx, _ = oracle.reduce_dim("max", np.array([np.nan, 1, 3], F), 1, 3, 1)
+    assert np.isnan(out[0, 0]) and idx[0, 0] == 0
+    # columns of a matrix: axis 0 of [3, 2]
+    m = np.array([[1, 9], [4, 2], [4, 9]], F)
+    out, idx, _ = oracle.reduce_dim("max", m, 1, 3, 2)
+    assert out.tolist() == [[4, 9]] and idx.tolist() == [[1, 0]]
+
+
+def test_reduction_gradients_against_central_differences(oracle):
+    outer, length, inner = 2, 5, 3
+    x = oracle.normal((outer, length, inner), 71, 1.0, 2.0)
+    w = oracle.normal((outer, inner), 72)
+    w64 = w.astype(np.float64)
+    fns = {"sum": lambda t: t.sum(1), "mean": lambda t: t.mean(1), "max": lambda t: t.max(1), "min": lambda t: t.min(1),
+           "var": lambda t: t.var(1, ddof=1), "std": lambda t: t.std(1, ddof=1)}
+    for kind, fn in fns.items():
+        y, index, mean = oracle.reduce_dim(kind, x, outer, length, inner, 1)
+        got = oracle.reduce_dim_bwd(kind, x, y, index, mean, w, outer, length, inner, 1)
+        want = _numeric_gradient(lambda t: float(np.sum(w64 * fn(t))), x.astype(np.float64).copy())
+        assert np.allclose(got, want, rtol=3e-5, atol=3e-6), kind
+    # population variance (ddof 0) as well: the divisor is len - ddof
+    y, index, mean = oracle.reduce_dim("var", x, outer, length, inner, 0)
+    got = oracle.reduce_dim_bwd("var", x, y, index, mean, w, outer, length, inner, 0)
+    want = _numeric_gradient(lambda t: float(np.sum(w64 * t.var(1, ddof=0))), x.astype(np.float64).copy())
+    assert np.allclose(got, want, rtol=3e-5, atol=3e-6)
+
+
+def test_log_softmax_against_double_precision_and_its_identities(oracle):
+    for shape, seed in [((7, 13), 1), ((1, 50), 2), ((33, 4), 3)]:
+        x = oracle.normal(shape, 80 + seed, 0, 3)
+        x64 = x.astype(np.float64)
+        for dim in (0, 1):
+            y = oracle.log_softmax(x, dim)
+            sh = x64 - x64.max(axis=dim, keepdims=True)
+            want = sh - np.log(np.exp(sh).sum(axis=dim, keepdims=True))
+            assert np.allclose(y, want, rtol=2e-6, atol=2e-6)
+            assert np.allclose(np.exp(y.astype(np.float64)).sum(axis=dim), 1, atol=1e-5)       # exp(y) is a distribution
+            assert np.allclose(np.exp(y.astype(np.float64)), oracle.softmax(x, dim), rtol=1e-5, atol=1e-8)
+            # shift invariance along the axis
+            assert np.allclose(oracle.log_softmax(x + F(5), dim), y, atol=3e-6)
+    v = oracle.normal((9,), 90)
+    assert np.allclose(oracle.log_softmax(v), oracle.log_softmax(v.reshape(1, 9), 1).reshape(9))
+    x = oracle.normal((4, 6), 91)
+    w = oracle.normal((4, 6), 92)
+    w64 = w.astype(np.float64)
+    for dim in (0, 1):
+        def f(t):
+            sh = t - t.max(axis=dim, keepdims=True)
+            return float(np.sum(w64 * (sh - np.log(np.exp(sh).sum(axis=dim, keepdims=True)))))
+        got = oracle.log_softmax_bwd(oracle.log_softmax(x, dim), w, dim)
+        assert np.allclose(got, _numeric_gradient(f, x.astype(np.float64).copy()), rtol=3e-5, atol=3e-6), dim
+        assert np.allclose(got.sum(axis=dim), 0, atol=2e-6)        # gradients of a normalised quantity sum to zero... times sum(w)
+    
+
+def test_broadcast_reduce_is_the_sum_over_broadcast_dimensions(oracle):
+    cases = [((4, 5), (5,)), ((4, 5), (4, 1)), ((4, 5), (1,)), ((4, 5), ()), ((2, 3, 4), (3, 1)), ((2, 3, 4), (4,)),
+             ((2, 3, 4), (2, 1, 4)), ((1, 5), (3, 5)), ((5,), (2, 5)), ((3, 1), (3, 4)), ((2, 1, 4), (3, 4))]
+    for gshape, tshape in cases:
+        g = oracle.normal(gshape, 95, 0, 2)
+        if len(tshape) > g.ndim:                    # the caller reshapes a lower-rank gradient to [1, .., 1, dims] first
+            g = g.reshape((1,) * (len(tshape) - g.ndim) + g.shape)
+        got = oracle.broadcast_reduce(g, tshape)
+        assert got is not None, (gshape, tshape)
+        g64 = g.astype(np.float64)
+        pad = (1,) * (g.ndim - len(tshape)) + tuple(tshape)
+        axes = tuple(d for d in range(g.ndim) if pad[d] == 1 and g.shape[d] > 1)
+        want = np.broadcast_to(g64.sum(axis=axes, keepdims=True), pad).reshape(tshape)
+        assert np.allclose(got, want, rtol=1e-6, atol=1e-6), (gshape, tshape)
+    assert oracle.broadcast_reduce(oracle.normal((2, 6), 1), (3,)) is None

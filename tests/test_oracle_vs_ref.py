@@ -145,3 +145,37 @@ def test_tensors_that_are_not_fp32(oracle, ref):
             assert ref.typed_grad(x, dt, steps)[0] == -1, (dt, steps)
     rc, code, raw = ref.typed_grad(x, 0, [(1, 3.0), (0, 5.0)])
     assert rc == 6 and code == 0 and np.array_equal(raw.view(np.float32)[:6], np.full(6, 3.0, np.float32))
+
+
+# shape pairs (gradient, target) that keep the reference's index arithmetic inside the gradient's
+# buffer, one or more for every branch of check_and_adjust_grad_shape (src/AutoDiff.cpp:562-1049)
+ADJUST_CASES = [
+    ((2, 3), (2, 3)),        # :565-567  equal
+    ((), (2, 3)), ((), (5,)),                      # :579-627  0-D gradient
+    ((3,), (1, 3)), ((4,), (4, 1)), ((6,), (1, 1, 6)), ((2, 3), (1, 2, 3)),   # :633-687 rank(g) < rank(target)
+    ((1,), (2, 3)),          # :633-687 then the broadcast branch from a one-element gradient
+    ((2, 3), (3,)), ((4, 5), (5,)), ((2, 3, 4), (4,)), ((2, 3, 4), (3, 4)),   # :690-757 slice with leading index 0
+    ((2, 3), (1,)), ((2, 3), ()), ((3, 1), (3, 1)), ((5, 1), (1,)), ((4, 1), (2,)),   # one-element / last dim 1
+    ((2, 6), (3,)), ((6,), (2, 2)), ((3, 5), (2,)), ((7,), (3,)), ((2, 3), (4, 3)),   # :968-1046 modulo fold
+]
+
+
+@pytest.mark.parametrize("gshape, tshape", ADJUST_CASES)
+def test_gradient_shape_adjustment_every_branch(oracle, ref, gshape, tshape):
+    for seed in range(3):
+        g = oracle.normal(gshape if gshape else (1,), 900 + seed, 0, 2).reshape(gshape)
+        if seed == 1:
+            g.reshape(-1)[0] = -0.0                  # the broadcast branch adds to +0: -0 must come out +0
+        want = ref.adjust_grad_shape(g, tshape)
+        assert want is not None
+        got = oracle.adjust_grad_shape(g, tshape)
+        assert got is not None
+        eq(got, want, (gshape, tshape, seed))
+
+
+def test_gradient_shape_adjustment_flags_the_reads_beyond_the_buffer(oracle):
+    # [3] -> [2, 3] and [1, 3] -> [2, 3]: the reference indexes the gradient with the flat result
+    # index (0..5) and reads past its three elements; the restatement reports that instead
+    g = oracle.normal((3,), 1)
+    assert oracle.adjust_grad_shape(g, (2, 3)) is None
+    assert oracle.adjust_grad_shape(g.reshape(1, 3), (2, 3)) is None
