@@ -296,8 +296,19 @@ CTA_FN float cta_tan_finish(float y, uint32_t ay, int n, double xr) {
     double x2 = xr * xr;
     double c = cta_cos_poly(x2);
     double sn = cta_sin_poly(xr, x2);
-    double t = (n & 1) ? -c / sn : sn / c;
-    float f = (float)t;
+    // tan = sin / cos in even quadrants, -cos / sin in odd ones.  The quotient through a reciprocal
+    // refined once in double from a single-precision start (relative error ~1e-14, far below the
+    // polynomials' own): a double-precision division costs more than the rest of the function.
+    double num = (n & 1) ? -c : sn;
+    double den = (n & 1) ? sn : c;
+#if defined(__HIPCC__)
+    double r0 = (double)__builtin_amdgcn_rcpf((float)den);
+#else
+    double r0 = (double)(1.0f / (float)den);
+#endif
+    double e = CTA_FMA(-den, r0, 1.0);
+    double r1 = CTA_FMA(r0, e, r0);
+    float f = (float)(num * r1);
     return (ay < 0x39000000u) ? y : f;             // |y| < 2^-13: tan(y) = y, keeps the sign of -0
 }
 // Straight-line path, correct for |y| < 120 (cta_sincos_is_rare(y) == 0).

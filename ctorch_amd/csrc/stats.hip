@@ -269,9 +269,11 @@ __global__ __launch_bounds__(kThreads) void reduce_cols_kernel(const float* __re
     }
 }
 
-// Second launch: the `chunks` partials of each result merged in chunk order.  Contiguous axis
-// (inner == 1): a wave per result, lane t takes chunks t, t + 64, ...; strided axis: a thread per
-// result (neighbouring threads read neighbouring partials).
+// Second launch: the `chunks` partials of each result merged.  Contiguous axis (inner == 1): a wave
+// per result, lane t takes chunks t, t + 64, ...; strided axis: a block folds 32 neighbouring
+// results, its 8 groups of 32 lanes take every 8th chunk (neighbouring lanes read neighbouring
+// partials) and are merged through LDS in group order.
+constexpr int kFinishCols = 32, kFinishGroups = kThreads / kFinishCols;
 template <int KIND, bool WAVE>
 __global__ __launch_bounds__(kThreads) void reduce_finish_kernel(const Part* __restrict__ parts, const float* __restrict__ x,
                                                                  float* __restrict__ out, int32_t* __restrict__ index,
@@ -286,12 +288,30 @@ __global__ __launch_bounds__(kThreads) void reduce_finish_kernel(const Part* __r
         p = wave_merge<KIND>(p);
         if (lane == 0 && r < results) finish<KIND>(p, x[r * len], len, ddof, out, index, mean_out, r);
     } else {
-        const size_t r = size_t(blockIdx.x) * kThreads + threadIdx.x;
-        if (r >= results) return;
-        const size_t slab = r / inner, c = r % inner;
+        __shared__ Part s_part[kFinishGroups][kFinishCols];
+        const unsigned lane = threadIdx.x % kFinishCols, group = threadIdx.x / kFinishCols;
+        const size_t r = size_t(blockIdx.x) * kFinishCols + lane;
+        const bool live = r < results;
+        const size_t slab = live ? r / inner : 0, c = live ? r % inner : 0;
         Part p = empty_part<KIND>();
-        for (unsigned k = 0; k < chunks; ++k) p = merge<KIND>(p, parts[(slab * chunks + k) * inner + c]);
-        finish<KIND>(p, x[slab * len * inner + c], len, ddof, out, index, mean_out, r);
+        if (live) {
+            unsigned k = group;
+            for (; k + 3 * kFinishGroups < chunks; k += 4 * kFinishGroups) {
+                Part q[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) q[u] = parts[(slab * chunks + k + u * kFinishGroups) * inner + c];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) p = merge<KIND>(p, q[u]);
+            }
+            for (; k < chunks; k += kFinishGroups) p = merge<KIND>(p, parts[(slab * chunks + k) * inner + c]);
+        }
+        s_part[group][lane] = p;
+        __syncthreads();
+        if (group == 0 && live) {
+#pragma unroll
+            for (int g = 1; g < kFinishGroups; ++g) p = merge<KIND>(p, s_part[g][lane]);
+            finish<KIND>(p, x[slab * len * inner + c], len, ddof, out, index, mean_out, r);
+        }
     }
 }
 
@@ -542,7 +562,7 @@ int run_forward(const char* name, const float* x, float* out, int32_t* index, fl
     int rc = launched(name);
     if (rc || p.chunks == 1) return rc;
     const size_t results = outer * inner;
-    hipLaunchKernelGGL((reduce_finish_kernel<KIND, false>), dim3(unsigned((results + kThreads - 1) / kThreads)), dim3(kThreads), 0, s, parts,
+    hipLaunchKernelGGL((reduce_finish_kernel<KIND, false>), dim3(unsigned((results + kFinishCols - 1) / kFinishCols)), dim3(kThreads), 0, s, parts,
                        x, out, index, mean_out, results, len, inner, p.chunks, ddof);
     return launched(name);
 }

@@ -58,6 +58,14 @@ class AutoDiff {
     struct OpPayload {
         virtual ~OpPayload() = default;
     };
+    // a reduction along dimensions (op::Reduce): which one, the [outer, len, inner] reading of the
+    // operand, and what the forward pass kept for the gradient
+    struct ReducePayload : OpPayload {
+        int kind = 0, ddof = 1;
+        size_t outer = 1, len = 1, inner = 1;
+        Tensor index;    // max / min: position of the extreme element along the axis (int32)
+        Tensor mean;     // var / std
+    };
     struct Node {
         size_t tensor_id = 0;
         op operation = op::Add;
@@ -66,6 +74,7 @@ class AutoDiff {
         std::unique_ptr<Tensor> tensor;   // shares storage with the user's tensor
         std::unique_ptr<Tensor> grad;
         bool grad_plus_zero = false;           // grad holds no -0: "0 + grad" (what get_grad returns) is grad itself
+        bool grad_assigned = false;            // grad is a root's seed: assigned, not added to zeros (src/AutoDiff.cpp:1126), read as it is
         std::unique_ptr<Tensor> shared_term;   // backward only: a factor that several inputs' gradients use
         std::vector<Tensor> input_grads;       // backward only: gradients of all inputs, computed together
         std::shared_ptr<OpPayload> payload;
@@ -114,6 +123,7 @@ class AutoDiff {
     bool check_div_zero_ = true;
     bool term_plus_zero_ = false;   // backward: the term just computed holds no -0
     bool seed_plus_zero_ = false;   // backward: the seed gradient holds no -0
+    bool adjust_adds_to_zero_ = false;   // the last adjust_grad_shape took a branch in which the reference adds the gradient to zeros
 
     Node* find(size_t id);
     Tensor adjust_grad_shape(const Tensor& grad, const std::vector<size_t>& target_shape);

@@ -22,6 +22,10 @@ enum class op {
     Sum,
     Linear,   // not in the reference: matmul + bias row (+ ReLU) as one taped operator, Tensor::linear
     Fused,    // not in the reference: an elementwise expression evaluated in one pass, Expr::eval
+    // methods the reference declares on Tensor without defining them (include/Tensor.h:824-1072); they
+    // have no enumerator there because nothing tapes them
+    Abs, Exp, Log, Sqrt, Square, Tan, LogSoftmax,
+    Reduce,   // sum / mean / max / min / var / std along dimensions; which one is in the node's payload
 };
 
 enum class ErrorLevel { TRACE = 0, DEBUG = 1, INFO = 2, WARN = 3, ERROR = 4, FATAL = 5 };

@@ -40,7 +40,9 @@ class Ctorch_Scheduler {
         unary_kernel_map_[op::Tanh][DeviceType::kAMD] = Tanh_AMD_kernel;
         unary_kernel_map_[op::Sigmoid][DeviceType::kAMD] = Sigmoid_AMD_kernel;
         unary_kernel_map_[op::Softmax][DeviceType::kAMD] = Softmax_AMD_kernel;
-        unary_kernel_map_[op::LReLU];   // registered without a kernel, as in the reference (:52)
+        // the reference registers LReLU without a function (:51-52) and defines no LReLU kernel anywhere;
+        // here the column has one
+        unary_kernel_map_[op::LReLU][DeviceType::kAMD] = LReLU_AMD_kernel;
     }
     void ensureInit() {
         std::lock_guard<std::mutex> lock(mutex_);

@@ -67,6 +67,9 @@ class Tensor {
     static Tensor view_rows(const Tensor& t, size_t first, size_t count);
     // element `index` of a contiguous tensor as a 0-D VIEW (shares storage, new id)
     static Tensor view_element(const Tensor& t, size_t index);
+    // the elements of a contiguous tensor under another shape of the same element count, as a VIEW
+    // (shares storage, new id)
+    static Tensor view_shape(const Tensor& t, const std::vector<size_t>& shape);
     void set_known_value(float v) { _known_value = std::make_shared<const float>(v); }
     void forget_known_value() { _known_value.reset(); }
     const float* known_value() const { return _known_value.get(); }   // null when the host does not know it
@@ -163,6 +166,42 @@ class Tensor {
     std::vector<unsigned char> to_bytes() const;    // the elements' bytes on the host, any dtype (contiguous tensors)
     Tensor sum() const;
     Tensor softmax(int dim = -1) const;
+    // ---- declared by the reference (include/Tensor.h:719, :824-1072, :1117) and never defined there;
+    // defined here for kAMD float tensors, each taped with its gradient.  Semantics: the C++ library
+    // call the name stands for; reductions over `dims` (negative counts from the end; none = all)
+    // drop the reduced dimensions unless keepdim; max / min return values only and pass the gradient
+    // to the first extreme element; var / std divide by count - 1 (the sample statistics that the
+    // API this class imitates returns by default) - var_of / std_of take the correction explicitly;
+    // several dimensions must be adjacent for var / std.
+    Tensor operator-(float scalar) const;
+    Tensor abs() const;
+    Tensor exp() const;
+    Tensor log() const;
+    Tensor sqrt() const;
+    Tensor square() const;
+    Tensor tan() const;
+    Tensor leaky_relu(float negative_slope = 0.01f) const;
+    Tensor log_softmax(int dim = -1) const;
+    Tensor sum(const std::vector<int>& dims, bool keepdim = false) const;
+    Tensor sum(int dim, bool keepdim = false) const;
+    Tensor mean(const std::vector<int>& dims, bool keepdim = false) const;
+    Tensor mean(int dim, bool keepdim = false) const;
+    Tensor mean() const;
+    Tensor max(const std::vector<int>& dims, bool keepdim = false) const;
+    Tensor max(int dim, bool keepdim = false) const;
+    Tensor max() const;
+    Tensor min(const std::vector<int>& dims, bool keepdim = false) const;
+    Tensor min(int dim, bool keepdim = false) const;
+    Tensor min() const;
+    Tensor std(const std::vector<int>& dims, bool keepdim = false) const;
+    Tensor std(int dim, bool keepdim = false) const;
+    Tensor std() const;
+    Tensor var(const std::vector<int>& dims, bool keepdim = false) const;
+    Tensor var(int dim, bool keepdim = false) const;
+    Tensor var() const;
+    Tensor var_of(const std::vector<int>& dims, bool keepdim, int ddof) const;
+    Tensor std_of(const std::vector<int>& dims, bool keepdim, int ddof) const;
+    Tensor matmul_unified(const Tensor& other) const;    // the reference's "unified" product (:1117): matmul
 
     // ---- autograd
     void backward() const;

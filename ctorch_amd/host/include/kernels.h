@@ -30,6 +30,9 @@ Tensor Sin_AMD_kernel(const Tensor& a);
 Tensor Tanh_AMD_kernel(const Tensor& a);
 Tensor Sigmoid_AMD_kernel(const Tensor& a);
 Tensor Softmax_AMD_kernel(const Tensor& a);
+// leaky ReLU with the default slope of Tensor::leaky_relu (0.01): the kernel that the reference
+// declares (src/kernels/kernels.h:201) and registers without a function (Ctorch_Scheduler.h:51-52)
+Tensor LReLU_AMD_kernel(const Tensor& a);
 
 namespace ctorch_amd_host {
 // Device branches of the arithmetic that the reference runs inline on the host (not behind the
@@ -38,6 +41,27 @@ Tensor scalar_op(const Tensor& a, float s, op which);
 // a (cmp) b or, with b == nullptr, a (cmp) s: a bool tensor; cmp is a CTAMD_CMP_* code
 Tensor compare_op(int cmp, const Tensor& a, const Tensor* b, float s);                 // a + s, a * s, a / s
 Tensor sum_all(const Tensor& a);
+// the methods the reference declares without defining them; `which` is op::Abs, Exp, Log, Sqrt,
+// Square, Tan or LReLU (param = slope)
+Tensor unary_declared(op which, const Tensor& a, float param = 0.0f);
+// their gradients; v is the operand (Abs, Log, Square, LReLU) or the result (Exp, Sqrt, Tan)
+Tensor unary_declared_backward(op which, const Tensor& v, const Tensor& g, float param = 0.0f);
+// sum / mean / max / min / var / std (kind: CTAMD_RED_*) of `a` read as [outer, len, inner] over its
+// middle axis; the result has `result_shape`.  index (max / min) and mean (var / std) receive what
+// the gradient needs when they are not null.
+Tensor reduce_axis(int kind, const Tensor& a, size_t outer, size_t len, size_t inner, int ddof,
+                   const std::vector<size_t>& result_shape, Tensor* index, Tensor* mean);
+Tensor reduce_axis_backward(int kind, const Tensor& x, const Tensor& y, const Tensor& index, const Tensor& mean, const Tensor& g,
+                            size_t outer, size_t len, size_t inner, int ddof);
+Tensor log_softmax_dim(const Tensor& a, int dim);                       // dim already normalised
+Tensor log_softmax_backward(const Tensor& y, const Tensor& g, int dim);
+// gradient shape adjustment beyond the row-vector cases: the modulo fold of shapes that do not
+// broadcast, and the sum over / repetition along broadcast dimensions (shapes padded to one rank)
+Tensor fold_mod(const Tensor& g, const std::vector<size_t>& target_shape);
+Tensor broadcast_reduce(const Tensor& g, const std::vector<size_t>& g_shape, const std::vector<size_t>& t_shape,
+                        const std::vector<size_t>& result_shape);
+// the first `count` elements of g as a tensor of `shape` (a copy)
+Tensor leading_elements(const Tensor& g, const std::vector<size_t>& shape);
 // Class-index cross entropy under a tape whose logits need a gradient computes loss and gradient in
 // one pass over the logits and keeps the gradient for backward() (default on; off: a forward pass
 // that leaves row statistics, and a streaming backward pass).

@@ -5,12 +5,14 @@
 
 #include <cfloat>
 #include <cmath>
+#include <cstring>
 
 #include <algorithm>
 
 #include "Ctorch_Scheduler.h"
 #include "Expr.h"
 #include "kernels.h"
+#include "ctorch_amd.h"
 
 using namespace ctorch_amd_host;
 
@@ -63,6 +65,7 @@ void AutoDiff::zero_grad(Tensor& t) {
     if (n) {
         n->grad.reset();
         n->grad_plus_zero = false;
+        n->grad_assigned = false;
     }
 }
 
@@ -86,7 +89,7 @@ Tensor AutoDiff::get_grad(const Tensor* t) {
         // the pending "0 +" (one pass, once); a gradient known to hold no -0 needs none.  The
         // result shares the tape's bytes instead of copying them: the tape never writes through
         // shared bytes (a later contribution goes to a fresh tensor), callers must not either.
-        if (!n->grad_plus_zero) {
+        if (!n->grad_plus_zero && !n->grad_assigned) {
             n->grad = std::make_unique<Tensor>(zero_plus(*n->grad, n->grad->sizes()));
             n->grad_plus_zero = true;
         }
@@ -133,11 +136,28 @@ void AutoDiff::clear_graph() {
     pending_.clear();
 }
 
-// src/AutoDiff.cpp:562-1049 for the cases that occur on this path.
+// src/AutoDiff.cpp:562-1049, every branch.  In the reference's mode the results are the reference's
+// bit for bit (the oracle's co_adjust_grad_shape restates the function and is pinned against it);
+// by default the broadcast branch is the mathematics instead: the sum over the dimensions along
+// which the operand was broadcast (the reference takes the slice with leading index 0).
 Tensor AutoDiff::adjust_grad_shape(const Tensor& grad, const std::vector<size_t>& target) {
-    if (grad.sizes() == target) return Tensor::alias(grad);
+    // The equal / 0-D / reshape branches hand the gradient's values on as they are; the broadcast
+    // branch adds them to a zero-filled result (`result[i] += g[..]`, :755), which turns -0 into +0.
+    // The values returned here are the raw ones; the flag tells a caller that stores them as a
+    // root's gradient (which nothing is added to afterwards) that the "0 +" is still due.
+    adjust_adds_to_zero_ = false;
+    if (grad.sizes() == target) return Tensor::alias(grad);                           // :565-567
     if (grad.sizes().empty()) return filled_from(target, grad);                       // :579-627
-    if (grad.dim() == 2 && target.size() == 1 && grad.sizes()[1] == target[0]) {      // :690-757
+    if (grad.dim() < target.size()) {
+        // :633-687: the gradient copied into shape [1, .., 1, its dims] (element i from element
+        // i % numel, the same count: a reshape), then the function again
+        const size_t gr = grad.dim(), tr = target.size();
+        std::vector<size_t> padded(tr, 1);
+        for (size_t i = 0; i < gr; ++i) padded[tr - gr + i] = grad.sizes()[i];
+        return adjust_grad_shape(Tensor::view_shape(grad, padded), target);
+    }
+    adjust_adds_to_zero_ = true;
+    if (grad.dim() == 2 && target.size() == 1 && grad.sizes()[1] == target[0]) {      // :690-757, the bias of a layer
         if (broadcast_grad_ == BroadcastGrad::kColumnSum) {
             term_plus_zero_ = true;                  // a sum that starts from +0 is never -0
             return column_sum(grad);
@@ -156,8 +176,49 @@ Tensor AutoDiff::adjust_grad_shape(const Tensor& grad, const std::vector<size_t>
         device_copy_d2d(first.fptr(), grad.fptr(), sizeof(float));
         return first;
     }
-    Ctorch_Error::throwException(ErrorPlatform::kAutoDiff, ErrorType::DIMENSION,
-                                 "backward: gradient shape cannot be reduced to the operand's shape");
+    const size_t gr = grad.dim(), tr = target.size();
+    bool can_broadcast = true;                                                        // :690-704
+    for (size_t i = 1; i <= tr; ++i) {
+        const size_t gd = grad.sizes()[gr - i], td = target[tr - i];
+        if (gd != td && gd != 1 && td != 1) can_broadcast = false;
+    }
+    if (!can_broadcast) {
+        // :968-1046 (the "can reduce" branch before it, :892-966, cannot be reached: its condition
+        // implies the broadcast one): result[i] = g[i] + g[i + n] + ..., in that order from 0
+        term_plus_zero_ = false;
+        return fold_mod(grad, target);
+    }
+    size_t tn = 1;
+    for (size_t e : target) tn *= e;
+    if (broadcast_grad_ == BroadcastGrad::kReferenceRow0) {
+        // :706-757: the coordinate loop starts at the LAST dimension with the whole flat index, so
+        // result[i] = 0 + g[i] (g[0] when the gradient's last dimension is 1); beyond the gradient's
+        // end the reference reads whatever follows its buffer
+        if (grad.sizes().back() == 1) return filled_from(target, Tensor::view_element(grad, 0));
+        if (tn > grad.numel())
+            Ctorch_Error::throwException(ErrorPlatform::kAutoDiff, ErrorType::DIMENSION,
+                                         "backward: the reference reads beyond the end of this gradient when it adjusts its shape");
+        return leading_elements(grad, target);
+    }
+    std::vector<size_t> padded(gr, 1);
+    for (size_t i = 0; i < tr; ++i) padded[gr - tr + i] = target[i];
+    term_plus_zero_ = true;                          // sums (in double, from +0) and their copies
+    // leading dimensions summed away and the rest kept whole: a column sum of [rows, cols]
+    size_t lead = 0;
+    while (lead < gr && padded[lead] == 1) ++lead;
+    bool rest_kept = true;
+    for (size_t d = lead; d < gr; ++d) rest_kept = rest_kept && padded[d] == grad.sizes()[d];
+    if (rest_kept && lead > 0 && grad.is_contiguous()) {
+        size_t rows = 1;
+        for (size_t d = 0; d < lead; ++d) rows *= grad.sizes()[d];
+        if (rows == 1) {
+            term_plus_zero_ = false;                 // the values themselves, -0 included
+            return Tensor::view_shape(grad, target);
+        }
+        Tensor sums = column_sum(Tensor::view_shape(grad, {rows, tn}));
+        return Tensor::view_shape(sums, target);
+    }
+    return broadcast_reduce(grad, grad.sizes(), padded, target);
 }
 
 namespace {
@@ -294,6 +355,25 @@ Tensor AutoDiff::input_gradient(Node* node, size_t input_id, size_t input_pos, c
         case op::Sum:                                                   // :1850-1855
             term_plus_zero_ = upstream_plus_zero;
             return adjust_grad_shape(g, x.sizes());
+        // the methods the reference declares without defining them (include/Tensor.h:824-1072)
+        case op::Abs: return unary_declared_backward(op::Abs, x, g);
+        case op::Square: return unary_declared_backward(op::Square, x, g);
+        case op::Log: return unary_declared_backward(op::Log, x, g);
+        case op::Exp: return unary_declared_backward(op::Exp, *node->tensor, g);
+        case op::Sqrt: return unary_declared_backward(op::Sqrt, *node->tensor, g);
+        case op::Tan: return unary_declared_backward(op::Tan, *node->tensor, g);
+        case op::LReLU: {
+            float slope = 0.0f;
+            std::memcpy(&slope, &node->op_param_i, sizeof(slope));
+            return unary_declared_backward(op::LReLU, x, g, slope);
+        }
+        case op::LogSoftmax: return log_softmax_backward(*node->tensor, g, node->op_param_i);
+        case op::Reduce: {
+            auto* r = dynamic_cast<ReducePayload*>(node->payload.get());
+            if (!r)
+                Ctorch_Error::throwException(ErrorPlatform::kAutoDiff, ErrorType::TENSOR_STATE, "backward: reduction without its record");
+            return reduce_axis_backward(r->kind, x, *node->tensor, r->index, r->mean, g, r->outer, r->len, r->inner, r->ddof);
+        }
         case op::Dot: {                                                 // extension: g * other
             Node* o = other_node();
             Tensor r = Mul_AMD_kernel(Tensor::alias(*o->tensor), g);
@@ -339,6 +419,7 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
     if (grad_output.device() != root.device()) grad_output = grad_output.to(root.device());
     root_node->grad = std::make_unique<Tensor>(adjust_grad_shape(grad_output, root.sizes()));
     root_node->grad_plus_zero = seed_plus_zero_;
+    root_node->grad_assigned = !adjust_adds_to_zero_;     // a seed taken as it is stays as it is (:1126)
     seed_plus_zero_ = false;
 
     // reversed depth-first post-order, inputs visited in recorded order (:1058-1077, :1138-1153)
@@ -369,6 +450,7 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
             size_t input_id = node->input_ids[pos];
             Node* in = find(input_id);
             if (!in || !in->requires_grad) continue;
+            in->grad_assigned = false;               // whatever it holds is added to from here on
             // a second loss of the same predictions: its gradient is added to the one gathered so far
             // in the pass that forms it (the same sum as term-then-accumulate, bit for bit)
             if ((node->operation == op::MSE || node->operation == op::MAE) && pos == 0 && in->grad &&

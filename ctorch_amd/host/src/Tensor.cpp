@@ -5,6 +5,9 @@
 
 #include <cfloat>
 #include <cmath>
+#include <cstring>
+
+#include <algorithm>
 
 #include "Ctorch_Scheduler.h"
 #include "ctorch_amd.h"
@@ -270,6 +273,19 @@ Tensor Tensor::view_element(const Tensor& t, size_t index) {
     return r;
 }
 
+Tensor Tensor::view_shape(const Tensor& t, const std::vector<size_t>& shape) {
+    size_t n = 1;
+    for (size_t e : shape) n *= e;
+    if (!t.is_contiguous() || n != t.numel())
+        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DIMENSION, "view_shape: element counts differ or tensor not contiguous");
+    Tensor r(AliasTag{}, t);
+    r.tensor_id_ = global_tensor_id++;
+    r._requires_grad = false;
+    r._shape = shape;
+    r.computeStrides();
+    return r;
+}
+
 Tensor Tensor::contiguous() const {
     if (is_contiguous()) return Tensor(*this);
     std::vector<float> v = to_vector();
@@ -289,7 +305,8 @@ void check_pair(const Tensor& a, const Tensor& b) {
 }
 
 // defer_record + commit_record, as every operator method of the reference does
-void tape(Tensor& result, op o, std::initializer_list<const Tensor*> inputs, int param = 0) {
+void tape(Tensor& result, op o, std::initializer_list<const Tensor*> inputs, int param = 0,
+          std::shared_ptr<AutoDiff::OpPayload> payload = nullptr) {
     AutoDiff* ctx = AutoDiffContext::current();
     if (!ctx) return;
     std::vector<Tensor*> in;
@@ -298,7 +315,7 @@ void tape(Tensor& result, op o, std::initializer_list<const Tensor*> inputs, int
         in.push_back(const_cast<Tensor*>(t));
         rg = rg || t->requires_grad();
     }
-    ctx->defer_record(result.id(), o, in, param);
+    ctx->defer_record(result.id(), o, in, param, std::move(payload));
     result.set_requires_grad(rg);
     if (rg) ctx->commit_record(result);
 }
@@ -425,6 +442,136 @@ Tensor Tensor::softmax(int dim) const {
     tape(result, op::Softmax, {this}, dim);
     return result;
 }
+
+// ------------------------------------------- declared by the reference, defined only here
+namespace {
+void need_device(const Tensor& t, const char* what) {
+    if (t.device() != DeviceType::kAMD)
+        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::PLATFORM_API, std::string(what) + ": no kernel for this device");
+}
+Tensor declared_unary(const Tensor& a, op o, float param = 0.0f) {
+    need_device(a, "unary operator");
+    Tensor result = unary_declared(o, a, param);
+    int bits = 0;
+    std::memcpy(&bits, &param, sizeof(bits));
+    tape(result, o, {&a}, bits);
+    return result;
+}
+
+// dims -> sorted, unique, non-negative; none = every dimension
+std::vector<int> normalised_dims(const Tensor& t, const std::vector<int>& dims) {
+    const int rank = int(t.dim());
+    std::vector<int> out;
+    if (dims.empty()) {
+        for (int d = 0; d < rank; ++d) out.push_back(d);
+        return out;
+    }
+    for (int d : dims) {
+        if (d < 0) d += rank;
+        if (d < 0 || d >= rank)
+            Ctorch_Error::throwException(ErrorPlatform::kAMD, ErrorType::DIMENSION, "reduction: dim out of range");
+        out.push_back(d);
+    }
+    std::sort(out.begin(), out.end());
+    out.erase(std::unique(out.begin(), out.end()), out.end());
+    return out;
+}
+
+// dimensions d0..d1 (adjacent) of `t` reduced in one launch and one tape entry
+Tensor reduce_block(const Tensor& t, int kind, int d0, int d1, bool keepdim, int ddof) {
+    const std::vector<size_t>& sh = t.shape();
+    size_t outer = 1, len = 1, inner = 1;
+    std::vector<size_t> result_shape;
+    for (int d = 0; d < int(sh.size()); ++d) {
+        if (d < d0) outer *= sh[d];
+        else if (d <= d1) len *= sh[d];
+        else inner *= sh[d];
+        if (d < d0 || d > d1) result_shape.push_back(sh[d]);
+        else if (keepdim) result_shape.push_back(1);
+    }
+    const bool taped = AutoDiffContext::current() && t.requires_grad();
+    auto payload = std::make_shared<AutoDiff::ReducePayload>();
+    payload->kind = kind;
+    payload->ddof = ddof;
+    payload->outer = outer;
+    payload->len = len;
+    payload->inner = inner;
+    Tensor result = reduce_axis(kind, t, outer, len, inner, ddof, result_shape, taped ? &payload->index : nullptr,
+                                taped ? &payload->mean : nullptr);
+    tape(result, op::Reduce, {&t}, kind, payload);
+    return result;
+}
+
+Tensor reduce_dims(const Tensor& t, int kind, const std::vector<int>& dims, bool keepdim, int ddof) {
+    need_device(t, "reduction");
+    if (t.dtype() != DType::kFloat)
+        Ctorch_Error::throwException(ErrorPlatform::kAMD, ErrorType::DATATYPE, "reduction: only float32 tensors");
+    if (t.dim() == 0) return reduce_block(t, kind, 0, -1, keepdim, ddof);       // one element: len = 1
+    const std::vector<int> ds = normalised_dims(t, dims);
+    bool adjacent = true;
+    for (size_t i = 1; i < ds.size(); ++i) adjacent = adjacent && ds[i] == ds[i - 1] + 1;
+    if (adjacent) return reduce_block(t, kind, ds.front(), ds.back(), keepdim, ddof);
+    if (kind == CTAMD_RED_VAR || kind == CTAMD_RED_STD)
+        Ctorch_Error::throwException(ErrorPlatform::kAMD, ErrorType::DIMENSION, "var / std: the dimensions must be adjacent");
+    // separated dimensions: one after the other from the last, which leaves the earlier ones in place
+    Tensor r = reduce_block(t, kind, ds.back(), ds.back(), keepdim, ddof);
+    for (size_t i = ds.size() - 1; i-- > 0;) r = reduce_block(r, kind, ds[i], ds[i], keepdim, ddof);
+    return r;
+}
+}  // namespace
+
+Tensor Tensor::operator-(float scalar) const { return with_scalar(*this, scalar, op::Sub); }
+Tensor Tensor::abs() const { return declared_unary(*this, op::Abs); }
+Tensor Tensor::exp() const { return declared_unary(*this, op::Exp); }
+Tensor Tensor::log() const { return declared_unary(*this, op::Log); }
+Tensor Tensor::sqrt() const { return declared_unary(*this, op::Sqrt); }
+Tensor Tensor::square() const { return declared_unary(*this, op::Square); }
+Tensor Tensor::tan() const { return declared_unary(*this, op::Tan); }
+Tensor Tensor::leaky_relu(float negative_slope) const {
+    if (negative_slope == 0.01f) {
+        // the default slope is the registered kernel's (the reference's kernel signature has no room for a slope)
+        Tensor result = Ctorch_Scheduler::getInstance().dispatch(*this, op::LReLU);
+        int bits = 0;
+        std::memcpy(&bits, &negative_slope, sizeof(bits));
+        tape(result, op::LReLU, {this}, bits);
+        return result;
+    }
+    return declared_unary(*this, op::LReLU, negative_slope);
+}
+Tensor Tensor::log_softmax(int dim) const {
+    need_device(*this, "log_softmax");
+    if (_shape.empty())
+        Ctorch_Error::throwException(ErrorPlatform::kAMD, ErrorType::DIMENSION, "log_softmax: 0-D tensor");
+    int rank = int(_shape.size());
+    if (dim < 0) dim += rank;
+    if (dim < 0 || dim >= rank)
+        Ctorch_Error::throwException(ErrorPlatform::kAMD, ErrorType::DIMENSION, "log_softmax: dim out of range");
+    if (rank > 2)
+        Ctorch_Error::throwException(ErrorPlatform::kAMD, ErrorType::DIMENSION, "log_softmax: only 1-D / 2-D tensors");
+    Tensor result = log_softmax_dim(*this, dim);
+    tape(result, op::LogSoftmax, {this}, dim);
+    return result;
+}
+Tensor Tensor::sum(const std::vector<int>& dims, bool keepdim) const { return reduce_dims(*this, CTAMD_RED_SUM, dims, keepdim, 0); }
+Tensor Tensor::sum(int dim, bool keepdim) const { return reduce_dims(*this, CTAMD_RED_SUM, {dim}, keepdim, 0); }
+Tensor Tensor::mean(const std::vector<int>& dims, bool keepdim) const { return reduce_dims(*this, CTAMD_RED_MEAN, dims, keepdim, 0); }
+Tensor Tensor::mean(int dim, bool keepdim) const { return reduce_dims(*this, CTAMD_RED_MEAN, {dim}, keepdim, 0); }
+Tensor Tensor::mean() const { return reduce_dims(*this, CTAMD_RED_MEAN, {}, false, 0); }
+Tensor Tensor::max(const std::vector<int>& dims, bool keepdim) const { return reduce_dims(*this, CTAMD_RED_MAX, dims, keepdim, 0); }
+Tensor Tensor::max(int dim, bool keepdim) const { return reduce_dims(*this, CTAMD_RED_MAX, {dim}, keepdim, 0); }
+Tensor Tensor::max() const { return reduce_dims(*this, CTAMD_RED_MAX, {}, false, 0); }
+Tensor Tensor::min(const std::vector<int>& dims, bool keepdim) const { return reduce_dims(*this, CTAMD_RED_MIN, dims, keepdim, 0); }
+Tensor Tensor::min(int dim, bool keepdim) const { return reduce_dims(*this, CTAMD_RED_MIN, {dim}, keepdim, 0); }
+Tensor Tensor::min() const { return reduce_dims(*this, CTAMD_RED_MIN, {}, false, 0); }
+Tensor Tensor::var_of(const std::vector<int>& dims, bool keepdim, int ddof) const { return reduce_dims(*this, CTAMD_RED_VAR, dims, keepdim, ddof); }
+Tensor Tensor::std_of(const std::vector<int>& dims, bool keepdim, int ddof) const { return reduce_dims(*this, CTAMD_RED_STD, dims, keepdim, ddof); }
+Tensor Tensor::var(const std::vector<int>& dims, bool keepdim) const { return var_of(dims, keepdim, 1); }
+Tensor Tensor::var(int dim, bool keepdim) const { return var_of({dim}, keepdim, 1); }
+Tensor Tensor::var() const { return var_of({}, false, 1); }
+Tensor Tensor::std(const std::vector<int>& dims, bool keepdim) const { return std_of(dims, keepdim, 1); }
+Tensor Tensor::std(int dim, bool keepdim) const { return std_of({dim}, keepdim, 1); }
+Tensor Tensor::std() const { return std_of({}, false, 1); }
+Tensor Tensor::matmul_unified(const Tensor& other) const { return matmul(other); }
 
 // --------------------------------------------------------------------------------- autograd
 void Tensor::backward() const {

@@ -134,7 +134,7 @@ Tensor cast_from_float(const Tensor& a, DType to) {
 Tensor scalar_op(const Tensor& a, float s, op which) {
     if (a.dtype() != DType::kFloat) {
         // the typed arms of src/Tensor.cpp:766-786, :870-890, :933-953; anything else is refused as there
-        if (a.dtype() != DType::kDouble && a.dtype() != DType::kInt && a.dtype() != DType::kLong)
+        if ((a.dtype() != DType::kDouble && a.dtype() != DType::kInt && a.dtype() != DType::kLong) || which == op::Sub)
             Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DATATYPE, "tensor (op) float: unsupported dtype");
         check_on_device(a, "tensor (op) float");
         Tensor r(ShapeTag{}, a.sizes(), a.dtype(), DeviceType::kAMD, false);
@@ -145,6 +145,7 @@ Tensor scalar_op(const Tensor& a, float s, op which) {
     check_device(a, "tensor (op) float");
     Tensor r = like(a);
     int rc = which == op::Add ? ctamd_add_scalar_f32(a.fptr(), s, r.fptr(), a.numel(), current_stream())
+           : which == op::Sub ? ctamd_sub_scalar_f32(a.fptr(), s, r.fptr(), a.numel(), current_stream())
            : which == op::Mul ? ctamd_mul_scalar_f32(a.fptr(), s, r.fptr(), a.numel(), current_stream())
                               : ctamd_div_scalar_f32(a.fptr(), s, r.fptr(), a.numel(), current_stream());
     run(rc, "tensor (op) float");
@@ -172,6 +173,114 @@ Tensor sum_all(const Tensor& a) {
     check_device(a, "sum");
     Tensor r = scalar0d();
     run(ctamd_sum_f32(a.fptr(), r.fptr(), a.numel(), current_stream()), "sum");
+    return r;
+}
+Tensor unary_declared(op which, const Tensor& a, float param) {
+    check_device(a, "unary operator");
+    if (!a.is_contiguous()) Ctorch_Error::throwException(kP, ErrorType::TENSOR_STATE, "unary operator: a contiguous tensor is needed");
+    Tensor r = like(a);
+    void* s = current_stream();
+    const size_t n = a.numel();
+    int rc = CTAMD_EINVAL;
+    switch (which) {
+        case op::Abs: rc = ctamd_abs_f32(a.fptr(), r.fptr(), n, s); break;
+        case op::Exp: rc = ctamd_exp_f32(a.fptr(), r.fptr(), n, s); break;
+        case op::Log: rc = ctamd_log_f32(a.fptr(), r.fptr(), n, s); break;
+        case op::Sqrt: rc = ctamd_sqrt_f32(a.fptr(), r.fptr(), n, s); break;
+        case op::Square: rc = ctamd_square_f32(a.fptr(), r.fptr(), n, s); break;
+        case op::Tan: rc = ctamd_tan_f32(a.fptr(), r.fptr(), n, s); break;
+        case op::LReLU: rc = ctamd_leaky_relu_f32(a.fptr(), param, r.fptr(), n, s); break;
+        default: Ctorch_Error::throwException(kP, ErrorType::UNKNOWN, "unary operator: not one of the declared methods");
+    }
+    run(rc, "unary operator");
+    return r;
+}
+Tensor unary_declared_backward(op which, const Tensor& v, const Tensor& g, float param) {
+    check_device(v, "unary gradient");
+    check_device(g, "unary gradient");
+    if (v.numel() != g.numel()) Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "unary gradient: sizes differ");
+    if (which == op::Exp) return Mul_AMD_kernel(v, g);            // y * g
+    if (which == op::Log) return Div_AMD_kernel(g, v);            // g / x
+    Tensor r = like(v);
+    void* s = current_stream();
+    const size_t n = v.numel();
+    int rc = CTAMD_EINVAL;
+    switch (which) {
+        case op::Abs: rc = ctamd_abs_backward_f32(v.fptr(), g.fptr(), r.fptr(), n, s); break;
+        case op::Sqrt: rc = ctamd_sqrt_backward_f32(v.fptr(), g.fptr(), r.fptr(), n, s); break;
+        case op::Square: rc = ctamd_square_backward_f32(v.fptr(), g.fptr(), r.fptr(), n, s); break;
+        case op::Tan: rc = ctamd_tan_backward_f32(v.fptr(), g.fptr(), r.fptr(), n, s); break;
+        case op::LReLU: rc = ctamd_leaky_relu_backward_f32(v.fptr(), g.fptr(), param, r.fptr(), n, s); break;
+        default: Ctorch_Error::throwException(kP, ErrorType::UNKNOWN, "unary gradient: not one of the declared methods");
+    }
+    run(rc, "unary gradient");
+    return r;
+}
+Tensor reduce_axis(int kind, const Tensor& a, size_t outer, size_t len, size_t inner, int ddof,
+                   const std::vector<size_t>& result_shape, Tensor* index, Tensor* mean) {
+    check_device(a, "reduction");
+    if (!a.is_contiguous()) Ctorch_Error::throwException(kP, ErrorType::TENSOR_STATE, "reduction: a contiguous tensor is needed");
+    if (len == 0) Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "reduction over an empty dimension");
+    Tensor r(ShapeTag{}, result_shape, DType::kFloat, DeviceType::kAMD, false);
+    const bool extreme = kind == CTAMD_RED_MAX || kind == CTAMD_RED_MIN, spread = kind == CTAMD_RED_VAR || kind == CTAMD_RED_STD;
+    if (index && extreme) *index = Tensor(ShapeTag{}, result_shape, DType::kInt, DeviceType::kAMD, false);
+    if (mean && spread) *mean = Tensor(ShapeTag{}, result_shape, DType::kFloat, DeviceType::kAMD, false);
+    run(ctamd_reduce_dim_f32(kind, a.fptr(), r.fptr(), (index && extreme) ? static_cast<int32_t*>(index->raw_ptr()) : nullptr,
+                             (mean && spread) ? mean->fptr() : nullptr, outer, len, inner, ddof, current_stream()),
+        "reduction");
+    return r;
+}
+Tensor reduce_axis_backward(int kind, const Tensor& x, const Tensor& y, const Tensor& index, const Tensor& mean, const Tensor& g,
+                            size_t outer, size_t len, size_t inner, int ddof) {
+    check_device(x, "reduction gradient");
+    check_device(g, "reduction gradient");
+    if (g.numel() != outer * inner || !g.is_contiguous())
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "reduction gradient: the upstream gradient does not have the result's size");
+    Tensor r = like(x);
+    run(ctamd_reduce_dim_backward_f32(kind, x.fptr(), y.is_cleared() ? nullptr : y.fptr(),
+                                      index.is_cleared() ? nullptr : static_cast<const int32_t*>(index.raw_ptr()),
+                                      mean.is_cleared() ? nullptr : mean.fptr(), g.fptr(), r.fptr(), outer, len, inner, ddof, current_stream()),
+        "reduction gradient");
+    return r;
+}
+Tensor log_softmax_dim(const Tensor& a, int dim) {
+    check_device(a, "log_softmax");
+    if (!a.is_contiguous()) Ctorch_Error::throwException(kP, ErrorType::TENSOR_STATE, "log_softmax: a contiguous tensor is needed");
+    Tensor r = like(a);
+    size_t rows, cols;
+    rows_cols(a, rows, cols);
+    if (a.dim() == 1 || dim == 1) run(ctamd_log_softmax_rows_f32(a.fptr(), r.fptr(), rows, cols, current_stream()), "log_softmax");
+    else run(ctamd_log_softmax_cols_f32(a.fptr(), r.fptr(), rows, cols, current_stream()), "log_softmax");
+    return r;
+}
+Tensor log_softmax_backward(const Tensor& y, const Tensor& g, int dim) {
+    check_device(y, "log_softmax_backward");
+    check_device(g, "log_softmax_backward");
+    Tensor r = like(y);
+    size_t rows, cols;
+    rows_cols(y, rows, cols);
+    if (y.dim() == 1 || dim == 1) run(ctamd_log_softmax_backward_rows_f32(y.fptr(), g.fptr(), r.fptr(), rows, cols, current_stream()), "log_softmax_backward");
+    else run(ctamd_log_softmax_backward_cols_f32(y.fptr(), g.fptr(), r.fptr(), rows, cols, current_stream()), "log_softmax_backward");
+    return r;
+}
+Tensor fold_mod(const Tensor& g, const std::vector<size_t>& target_shape) {
+    check_device(g, "fold_mod");
+    Tensor r(ShapeTag{}, target_shape, DType::kFloat, DeviceType::kAMD, false);
+    run(ctamd_fold_mod_f32(g.fptr(), r.fptr(), g.numel(), r.numel(), current_stream()), "fold_mod");
+    return r;
+}
+Tensor broadcast_reduce(const Tensor& g, const std::vector<size_t>& g_shape, const std::vector<size_t>& t_shape,
+                        const std::vector<size_t>& result_shape) {
+    check_device(g, "broadcast_reduce");
+    Tensor r(ShapeTag{}, result_shape, DType::kFloat, DeviceType::kAMD, false);
+    run(ctamd_broadcast_reduce_f32(g.fptr(), g_shape.data(), t_shape.data(), int(g_shape.size()), r.fptr(), current_stream()), "broadcast_reduce");
+    return r;
+}
+Tensor leading_elements(const Tensor& g, const std::vector<size_t>& shape) {
+    check_device(g, "leading_elements");
+    Tensor r(ShapeTag{}, shape, DType::kFloat, DeviceType::kAMD, false);
+    if (r.numel() > g.numel()) Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "leading_elements: the gradient is too short");
+    device_copy_d2d(r.fptr(), g.fptr(), r.numel() * sizeof(float));
     return r;
 }
 Tensor softmax_dim(const Tensor& a, int dim) {
@@ -586,6 +695,7 @@ Tensor Cos_AMD_kernel(const Tensor& a) { return map(ctamd_cos_f32, "Cos_AMD_kern
 Tensor Sin_AMD_kernel(const Tensor& a) { return map(ctamd_sin_f32, "Sin_AMD_kernel", a); }
 Tensor Tanh_AMD_kernel(const Tensor& a) { return map(ctamd_tanh_f32, "Tanh_AMD_kernel", a); }
 Tensor Sigmoid_AMD_kernel(const Tensor& a) { return map(ctamd_sigmoid_f32, "Sigmoid_AMD_kernel", a); }
+Tensor LReLU_AMD_kernel(const Tensor& a) { return unary_declared(op::LReLU, a, 0.01f); }
 // Softmax_BASIC_kernel.cpp:26-35, :95-98: float only, 1-D or 2-D (last dimension), throws otherwise
 Tensor Softmax_AMD_kernel(const Tensor& a) {
     check_device(a, "Softmax_AMD_kernel");

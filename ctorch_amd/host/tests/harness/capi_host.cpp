@@ -315,6 +315,184 @@ long cth_grad_binary(int code, const float* a, const long* ad, int an, const flo
     }
 }
 
+// ---- the methods the reference declares without defining them
+namespace {
+// 40 abs, 41 exp, 42 log, 43 sqrt, 44 square, 45 tan, 46 leaky_relu(p), 47 a - p,
+// 48 op::LReLU through Ctorch_Scheduler::dispatch (the registered kernel, slope 0.01)
+Tensor run_declared(int code, const Tensor& a, float p) {
+    switch (code) {
+        case 40: return a.abs();
+        case 41: return a.exp();
+        case 42: return a.log();
+        case 43: return a.sqrt();
+        case 44: return a.square();
+        case 45: return a.tan();
+        case 46: return a.leaky_relu(p);
+        case 47: return a - p;
+        case 48: return Ctorch_Scheduler::getInstance().dispatch(a, op::LReLU);
+    }
+    throw std::runtime_error("bad declared-unary code");
+}
+// kind 0 sum, 1 mean, 2 max, 3 min, 4 var, 5 std; no dims and no keepdim: the method without arguments
+// (sum() is the reference's own full sum); one dim: the (int, bool) overload; ddof < 0: the method's default
+Tensor run_reduce(int kind, const Tensor& a, const int* dims, int n_dims, bool keepdim, int ddof) {
+    std::vector<int> ds(dims, dims + n_dims);
+    if (kind == 4 && ddof >= 0) return a.var_of(ds, keepdim, ddof);
+    if (kind == 5 && ddof >= 0) return a.std_of(ds, keepdim, ddof);
+    if (n_dims == 0 && !keepdim) {
+        switch (kind) {
+            case 0: return a.sum();
+            case 1: return a.mean();
+            case 2: return a.max();
+            case 3: return a.min();
+            case 4: return a.var();
+            case 5: return a.std();
+        }
+    }
+    if (n_dims == 1) {
+        switch (kind) {
+            case 0: return a.sum(ds[0], keepdim);
+            case 1: return a.mean(ds[0], keepdim);
+            case 2: return a.max(ds[0], keepdim);
+            case 3: return a.min(ds[0], keepdim);
+            case 4: return a.var(ds[0], keepdim);
+            case 5: return a.std(ds[0], keepdim);
+        }
+    }
+    switch (kind) {
+        case 0: return a.sum(ds, keepdim);
+        case 1: return a.mean(ds, keepdim);
+        case 2: return a.max(ds, keepdim);
+        case 3: return a.min(ds, keepdim);
+        case 4: return a.var(ds, keepdim);
+        case 5: return a.std(ds, keepdim);
+    }
+    throw std::runtime_error("bad reduction kind");
+}
+}  // namespace
+
+long cth_declared_unary(int code, const float* a, const long* ad, int an, float p, float* out) {
+    try {
+        Tensor ta = make(a, ad, an);
+        return emit(run_declared(code, ta, p), out);
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+// d/dx of sum( f(x) * w )
+long cth_grad_declared_unary(int code, const float* x, const long* xd, int xn, float p, const float* w, float* dx) {
+    try {
+        AutoDiff ctx;
+        configure(ctx);
+        AutoDiffContext::Guard guard(&ctx);
+        Tensor tx = make(x, xd, xn), tw = make(w, xd, xn);
+        tx.requires_grad(true);
+        Tensor y = run_declared(code, tx, p);
+        if (code == 48) return -3;              // the bare dispatch is not taped
+        Tensor z = y * tw;
+        Tensor s = z.sum();
+        backward(s);
+        return emit(grad(tx), dx);
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+// out_dims / out_rank: the result's shape
+long cth_reduce(int kind, const float* a, const long* ad, int an, const int* dims, int n_dims, int keepdim, int ddof,
+                float* out, long* out_dims, int* out_rank) {
+    try {
+        Tensor ta = make(a, ad, an);
+        Tensor r = run_reduce(kind, ta, dims, n_dims, keepdim != 0, ddof);
+        *out_rank = int(r.dim());
+        for (size_t i = 0; i < r.dim(); ++i) out_dims[i] = long(r.sizes()[i]);
+        return emit(r, out);
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+// d/dx of sum( reduce(x) * w ), w of the result's shape
+long cth_grad_reduce(int kind, const float* x, const long* xd, int xn, const int* dims, int n_dims, int keepdim, int ddof,
+                     const float* w, float* dx) {
+    try {
+        AutoDiff ctx;
+        configure(ctx);
+        AutoDiffContext::Guard guard(&ctx);
+        Tensor tx = make(x, xd, xn);
+        tx.requires_grad(true);
+        Tensor y = run_reduce(kind, tx, dims, n_dims, keepdim != 0, ddof);
+        std::vector<long> yd(y.sizes().begin(), y.sizes().end());
+        Tensor tw = make(w, yd.data(), int(yd.size()));
+        Tensor z = y * tw;
+        Tensor s = z.sum();
+        backward(s);
+        return emit(grad(tx), dx);
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+long cth_log_softmax(const float* a, const long* ad, int an, int dim, float* out) {
+    try {
+        return emit(make(a, ad, an).log_softmax(dim), out);
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+long cth_grad_log_softmax(const float* x, const long* xd, int xn, int dim, const float* w, float* dx) {
+    try {
+        AutoDiff ctx;
+        configure(ctx);
+        AutoDiffContext::Guard guard(&ctx);
+        Tensor tx = make(x, xd, xn), tw = make(w, xd, xn);
+        tx.requires_grad(true);
+        Tensor y = tx.log_softmax(dim);
+        Tensor z = y * tw;
+        Tensor s = z.sum();
+        backward(s);
+        return emit(grad(tx), dx);
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+// The gradient a root of shape td ends up with after backward(root, grad_output = g): the tape's
+// gradient shape adjustment (the reference's check_and_adjust_grad_shape, src/AutoDiff.cpp:562-1049),
+// in the mode cth_set_reference_row0 selected.  The root is a leaf, so nothing else runs.
+long cth_adjust_grad_shape(const float* g, const long* gd, int gn, const long* td, int tn, float* out) {
+    try {
+        AutoDiff ctx;
+        configure(ctx);
+        AutoDiffContext::Guard guard(&ctx);
+        Tensor tg = make(g, gd, gn);
+        Tensor root(ShapeTag{}, shape_of(td, tn), DType::kFloat, DeviceType::kAMD);
+        root.requires_grad(true);
+        ctx.make_leaf(root, true);
+        ctx.backward(root, tg);
+        return emit(grad(root), out);
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+// d/da, d/db of dot(a, b) * scale: the closed form g * b, g * a that this tape adds (the reference
+// has no gradient for Dot, src/AutoDiff.cpp:1856-1862)
+long cth_grad_dot(const float* a, const float* b, long n, float scale, float* value, float* da, float* db) {
+    try {
+        AutoDiff ctx;
+        configure(ctx);
+        AutoDiffContext::Guard guard(&ctx);
+        long d[1] = {n};
+        Tensor ta = make(a, d, 1), tb = make(b, d, 1);
+        ta.requires_grad(true);
+        tb.requires_grad(true);
+        Tensor y = ta.dot(tb);
+        value[0] = y.item<float>();
+        Tensor root = y * scale;
+        backward(root);
+        long r1 = emit(grad(ta), da), r2 = emit(grad(tb), db);
+        return (r1 < 0 || r2 < 0) ? -2 : r1 + r2;
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
 // d/dpred of  loss(pred, target) * scale   (loss in MSE / MAE / CE); the upstream gradient of the
 // loss node is then the 0-D value `scale`.
 long cth_grad_loss(int code, const float* p, const long* pd, int pn, const float* t, const long* td,

@@ -1,6 +1,6 @@
 """Per-kernel timings of the launch layer through the C ABI on one MI355X.
 
-    python -m ctorch_amd.kernel_bench [--json] [--skip-matmul] [--only-expr]
+    python -m ctorch_amd.kernel_bench [--json] [--skip-matmul] [--only-expr] [--only-declared]
 
 Every operator is launched on operands resident in HBM (torch only provides the memory and the
 stream), timed with events over back-to-back launches after a warm-up, and reported as time,
@@ -23,6 +23,8 @@ def main():
     ap.add_argument("--json", action="store_true", help="one JSON object instead of a table")
     ap.add_argument("--skip-matmul", action="store_true")
     ap.add_argument("--only-expr", action="store_true", help="only the fused-expression programs (for counter runs)")
+    ap.add_argument("--only-declared", action="store_true",
+                    help="only the operators the reference declares without defining: abs .. leaky_relu, reductions along an axis, log_softmax")
     args = ap.parse_args()
 
     import torch
@@ -79,7 +81,7 @@ def main():
     def ew(name, fn, bytes_per_elem):
         report("%s, n=2^26 (%d B/elem)" % (name, bytes_per_elem), timeit(rotating(fn), 20), bytes_per_elem * n)
 
-    plain = not args.only_expr
+    plain = not args.only_expr and not args.only_declared
     for op in ("add", "sub", "mul", "div") if plain else ():
         ew(op, lambda k, op=op: call("ctamd_%s_f32" % op, P(A[k]), P(B[k]), P(R[k]), n, S), 12)
     for op in ("neg", "relu", "sin", "cos", "tanh", "sigmoid") if plain else ():
@@ -96,6 +98,45 @@ def main():
         ew("dot", lambda k: call("ctamd_dot_f32", P(A[k]), P(B[k]), P(out), n, S), 8)
         ew("mse", lambda k: call("ctamd_mse_f32", P(A[k]), P(B[k]), P(out), n, S), 8)
         ew("mae", lambda k: call("ctamd_mae_f32", P(A[k]), P(B[k]), P(out), n, S), 8)
+    # the operators the reference declares without defining: unary maps and their gradients ...
+    if not args.only_expr:
+        for op in ("abs", "exp", "log", "sqrt", "square", "tan"):
+            src = B if op in ("log", "sqrt") else A
+            ew(op, lambda k, op=op, src=src: call("ctamd_%s_f32" % op, P(src[k]), P(R[k]), n, S), 8)
+        ew("leaky_relu", lambda k: call("ctamd_leaky_relu_f32", P(A[k]), C.c_float(0.01), P(R[k]), n, S), 8)
+        ew("tensor - scalar", lambda k: call("ctamd_sub_scalar_f32", P(A[k]), C.c_float(5.0), P(R[k]), n, S), 8)
+        for op in ("abs", "sqrt", "square", "tan"):
+            ew(op + " backward", lambda k, op=op: call("ctamd_%s_backward_f32" % op, P(B[k]), P(A[k]), P(R[k]), n, S), 12)
+        ew("leaky_relu backward", lambda k: call("ctamd_leaky_relu_backward_f32", P(A[k]), P(B[k]), C.c_float(0.01), P(R[k]), n, S), 12)
+        # ... reductions along an axis: a whole tensor, the rows and the columns of [16384 x 4096]
+        small = torch.empty(16384, device="cuda")
+        small_i = torch.empty(16384, dtype=torch.int32, device="cuda")
+        small_m = torch.empty(16384, device="cuda")
+        for kind, code in (("sum", 0), ("mean", 1), ("max", 2), ("min", 3), ("var", 4), ("std", 5)):
+            for what, (o, l, i) in (("all", (1, n, 1)), ("rows of [16384 x 4096]", (16384, 4096, 1)), ("columns of [16384 x 4096]", (1, 16384, 4096))):
+                if kind in ("mean", "min", "std") and what != "all":
+                    continue
+                ew("%s, %s" % (kind, what), lambda k, code=code, o=o, l=l, i=i: call("ctamd_reduce_dim_f32", code, P(A[k]), P(small), P(small_i),
+                                                                                       P(small_m), o, l, i, 1, S), 4)
+        for kind, code, per in (("sum", 0, 4), ("max", 2, 4), ("var", 4, 8)):
+            for what, (o, l, i) in (("rows of [16384 x 4096]", (16384, 4096, 1)), ("columns of [16384 x 4096]", (1, 16384, 4096))):
+                ew("%s backward, %s" % (kind, what), lambda k, code=code, o=o, l=l, i=i: call(
+                    "ctamd_reduce_dim_backward_f32", code, P(A[k]), P(small), P(small_i), P(small_m), P(small), P(R[k]), o, l, i, 1, S), per)
+        ew("log_softmax columns [16384 x 4096]", lambda k: call("ctamd_log_softmax_cols_f32", P(A[k]), P(R[k]), 16384, 4096, S), 8)
+        ew("log_softmax rows [16384 x 4096]", lambda k: call("ctamd_log_softmax_rows_f32", P(A[k]), P(R[k]), 16384, 4096, S), 8)
+        ew("log_softmax backward rows [16384 x 4096]", lambda k: call("ctamd_log_softmax_backward_rows_f32", P(A[k]), P(B[k]), P(R[k]), 16384, 4096, S), 12)
+    if args.only_declared:
+        del A, B, R
+        torch.cuda.empty_cache()
+        rows, cols = 8192, 32000
+        X = torch.randn(rows, cols, device="cuda") * 2
+        Y = torch.empty_like(X)
+        report("log_softmax rows [8192 x 32000] (8 B/elem)", timeit(lambda: call("ctamd_log_softmax_rows_f32", P(X), P(Y), rows, cols, S), 10), 8 * rows * cols)
+        report("log_softmax backward rows [8192 x 32000] (12 B/elem)",
+               timeit(lambda: call("ctamd_log_softmax_backward_rows_f32", P(Y), P(X), P(Y), rows, cols, S), 10), 12 * rows * cols)
+        if args.json:
+            print(json.dumps({"device": torch.cuda.get_device_name(0), "results": results}))
+        return 0
     # fused expressions: a cheap chain (bound by the memory stream) ...
     class Insn(C.Structure):
         _fields_ = [("op", C.c_uint8), ("dst", C.c_uint8), ("a", C.c_uint8), ("b", C.c_uint8), ("imm", C.c_float)]

@@ -278,11 +278,12 @@ class Oracle:
     # ---- gradient shape adjustment (the reference's whole function) and its mathematical twin
     def adjust_grad_shape(self, g, target_shape):
         """co_adjust_grad_shape; None where the reference would read beyond its gradient buffer."""
-        g = f32(g)
-        gs = (C.c_long * max(1, g.ndim))(*g.shape)
+        gshape = np.shape(g)                      # (a 0-D array would come out of f32() as [1])
+        g = f32(g).reshape(-1)
+        gs = (C.c_long * max(1, len(gshape)))(*gshape)
         ts = (C.c_long * max(1, len(target_shape)))(*target_shape)
         out = np.empty(target_shape, np.float32)
-        rc = self.lib.co_adjust_grad_shape(fp(g.reshape(-1)), gs, C.c_int(g.ndim), fp(out.reshape(-1)), ts, C.c_int(len(target_shape)))
+        rc = self.lib.co_adjust_grad_shape(fp(g), gs, C.c_int(len(gshape)), fp(out.reshape(-1)), ts, C.c_int(len(target_shape)))
         assert rc in (0, -1), rc
         return out if rc == 0 else None
 
@@ -847,11 +848,12 @@ class Reference:
         """The gradient a root of `target_shape` holds after backward(root, grad_output = g): the
         reference's check_and_adjust_grad_shape (src/AutoDiff.cpp:562-1049) through its public door
         (:1124-1126).  None when the call failed."""
-        g = f32(g)
+        gshape = np.shape(g)                      # (a 0-D array would come out of f32() as [1])
+        g = f32(g).reshape(-1)
         out = np.empty(target_shape, np.float32)
-        gd, gn = _dims(g.shape)
+        gd, gn = _dims(gshape)
         td, tn = _dims(tuple(target_shape))
-        n = self.lib.ref_adjust_grad_shape(fp(g.reshape(-1)), gd, gn, td, tn, fp(out.reshape(-1)))
+        n = self.lib.ref_adjust_grad_shape(fp(g), gd, gn, td, tn, fp(out.reshape(-1)))
         return out if n == out.size else None
 
     def chain(self, a, b):
@@ -968,8 +970,76 @@ class HostLayer(Reference):
     """This repository's C++ front-end (Tensor / Ctorch_Scheduler / AutoDiff over the HIP launch layer)
     through the test doorway ctorch_amd/host/tests/harness/capi_host.cpp.  Needs a GPU for every call."""
 
+    DECLARED = {"abs": 40, "exp": 41, "log": 42, "sqrt": 43, "square": 44, "tan": 45, "leaky_relu": 46, "sub_scalar": 47,
+                "lrelu_dispatch": 48}
+    REDUCE = {"sum": 0, "mean": 1, "max": 2, "min": 3, "var": 4, "std": 5}
+
     def __init__(self):
         Reference.__init__(self, HOST_LIB, "cth_")
+        for n in ("declared_unary", "grad_declared_unary", "reduce", "grad_reduce", "log_softmax", "grad_log_softmax",
+                  "adjust_grad_shape", "grad_dot"):
+            getattr(self.cdll, "cth_" + n).restype = C.c_long
+
+    # ---- the methods the reference declares without defining them
+    def declared_unary(self, name, a, p=0.0):
+        a = f32(a)
+        ad, an = _dims(a.shape)
+        out = np.empty_like(a)
+        rc = self.cdll.cth_declared_unary(self.DECLARED[name], fp(a), ad, an, C.c_float(p), fp(out))
+        return out if rc == a.size else None
+
+    def grad_declared_unary(self, name, x, w, p=0.0):
+        x, w = f32(x), f32(w)
+        xd, xn = _dims(x.shape)
+        dx = np.empty_like(x)
+        rc = self.cdll.cth_grad_declared_unary(self.DECLARED[name], fp(x), xd, xn, C.c_float(p), fp(w), fp(dx))
+        return dx if rc == x.size else None
+
+    def reduce(self, kind, a, dims=(), keepdim=False, ddof=-1):
+        """-> the result with its shape, or None when the call threw"""
+        ashape = np.shape(a)                      # (a 0-D array would come out of f32() as [1])
+        a = f32(a).reshape(-1)
+        ad, an = _dims(ashape)
+        ds = (C.c_int * max(1, len(dims)))(*dims)
+        out = np.empty(max(1, a.size), np.float32)
+        od = (C.c_long * 8)()
+        orank = C.c_int(0)
+        rc = self.cdll.cth_reduce(self.REDUCE[kind], fp(a), ad, an, ds, len(dims), int(keepdim), ddof, fp(out), od, C.byref(orank))
+        if rc < 0:
+            return None
+        shape = tuple(od[i] for i in range(orank.value))
+        return out[:rc].reshape(shape)
+
+    def grad_reduce(self, kind, x, w, dims=(), keepdim=False, ddof=-1):
+        xshape = np.shape(x)
+        x, w = f32(x).reshape(-1), f32(w).reshape(-1)
+        xd, xn = _dims(xshape)
+        ds = (C.c_int * max(1, len(dims)))(*dims)
+        dx = np.empty_like(x)
+        rc = self.cdll.cth_grad_reduce(self.REDUCE[kind], fp(x), xd, xn, ds, len(dims), int(keepdim), ddof, fp(w), fp(dx))
+        return dx.reshape(xshape) if rc == x.size else None
+
+    def log_softmax(self, a, dim):
+        a = f32(a)
+        ad, an = _dims(a.shape)
+        out = np.empty_like(a)
+        rc = self.cdll.cth_log_softmax(fp(a), ad, an, dim, fp(out))
+        return out if rc == a.size else None
+
+    def grad_log_softmax(self, x, dim, w):
+        x, w = f32(x), f32(w)
+        xd, xn = _dims(x.shape)
+        dx = np.empty_like(x)
+        rc = self.cdll.cth_grad_log_softmax(fp(x), xd, xn, dim, fp(w), fp(dx))
+        return dx if rc == x.size else None
+
+    def grad_dot(self, a, b, scale):
+        a, b = f32(a), f32(b)
+        da, db = np.empty_like(a), np.empty_like(b)
+        value = C.c_float(0)
+        rc = self.cdll.cth_grad_dot(fp(a), fp(b), C.c_long(a.size), C.c_float(scale), C.byref(value), fp(da), fp(db))
+        assert rc == 2 * a.size, rc
+        return np.float32(value.value), da, db
 
     def set_reference_row0(self, on):
         self.cdll.cth_set_reference_row0(int(on))
