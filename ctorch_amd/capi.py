@@ -22,6 +22,8 @@ PROTOTYPES = {
     "ctamd_memcpy_d2h": [_P, _P, _Z, _P],
     "ctamd_memcpy_d2d": [_P, _P, _Z, _P],
     "ctamd_sync": [_P],
+    "ctamd_set_math_mode": [C.c_int],
+    "ctamd_math_mode": [],
     "ctamd_stream_create": [C.POINTER(_P)],
     "ctamd_stream_destroy": [_P],
     "ctamd_graph_begin": [_P],

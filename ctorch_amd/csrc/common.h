@@ -29,6 +29,10 @@ const float* pad_zero();
 // Looks up (once per device) the current device's address of the static partials array that
 // ctamd_dot_static_f32 uses; defined in reduce.hip next to the array.
 int static_partials(double** out);
+// Whether softmax, the cross-entropy gradients and fused expressions evaluate their transcendentals in
+// single precision (<= 2 ulp, the default) or with the double-precision routines that return glibc's
+// floats bit for bit; set by ctamd_set_math_mode().
+bool fast_math();
 // Compute units of the current device (256 on MI355X); 0 before ctamd_init().
 int compute_units();
 

@@ -331,4 +331,34 @@ CTA_FN float cta_tanf(float y, const uint32_t* inv_pio4) {
     return cta_tan_finish(y, ay, n, xr);
 }
 
+#if defined(__HIPCC__)
+// ----------------------------------------------------------------------------------------------
+// Single-precision exponential for the kernels whose time the double-precision one above would set
+// (row softmax, the cross-entropy gradients, fused expressions): exp(d) = 2^z * exp(d - z ln 2) with
+// z = d * log2(e) rounded to float and 2^z from the hardware instruction (accurate to 1 ulp).  What
+// the rounded z misses of d is recovered by two fused multiply-adds against ln 2 split in two floats
+// (t = d - z ln 2, |t| < 1e-5, known to ~1e-12) and put back as the first-order factor 1 + t (the
+// next term is below 1e-10).  Results stay within 2 ulp of expf (measured: 1).  NaN stays NaN,
+// arguments below -150 give the hardware's 2^-216 = 0, results that would be subnormal are flushed
+// to zero by the instruction.
+__device__ __forceinline__ static float cta_exp_hw_nonpos(float d) {
+    const float dc = (d < -150.0f) ? -150.0f : d;              // also keeps -inf out of inf - inf below
+    const float z = dc * 0x1.715476p+0f;
+    const float e = __builtin_amdgcn_exp2f(z);
+    float t = __fmaf_rn(z, -0x1.62e4p-1f, dc);                  // ln 2 = 0x1.62e4p-1 + 0x1.7f7d1cp-20 (the first exact in 16 bits)
+    t = __fmaf_rn(z, -0x1.7f7d1cp-20f, t);
+    return __fmaf_rn(e, t, e);
+}
+// The same for any argument: overflow gives +inf (the factor must not meet an infinite e: inf * 0).
+__device__ __forceinline__ static float cta_exp_hw(float d) {
+    const float dc = (d < -150.0f) ? -150.0f : ((d > 90.0f) ? 90.0f : d);
+    const float z = dc * 0x1.715476p+0f;
+    const float e = __builtin_amdgcn_exp2f(z);
+    float t = __fmaf_rn(z, -0x1.62e4p-1f, dc);
+    t = __fmaf_rn(z, -0x1.7f7d1cp-20f, t);
+    const float r = __fmaf_rn(e, t, e);
+    return (e == __builtin_huge_valf()) ? e : r;
+}
+#endif
+
 #endif  // CTORCH_AMD_DEVMATH_H

@@ -3,6 +3,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
 #include <mutex>
 
 #include "common.h"
@@ -21,6 +22,7 @@ int g_cus[kMaxDevices] = {};
 std::mutex g_count_mu;
 double g_bytes = 0.0, g_flops = 0.0, g_ideal_s = 0.0;
 uint64_t g_launches = 0;
+std::atomic<int> g_math_mode{CTAMD_MATH_FAST};
 constexpr double kHbmBytesPerS = 8.0e12;        // MI355X HBM3E
 constexpr double kMfmaF32FlopPerS = 157.3e12;   // MI355X dense fp32 matrix
 }  // namespace
@@ -72,6 +74,8 @@ float* scratch() {
     }
     return g_scratch[d];
 }
+
+bool fast_math() { return g_math_mode.load(std::memory_order_relaxed) == CTAMD_MATH_FAST; }
 
 int compute_units() {
     int d = current_device();
@@ -130,6 +134,12 @@ int ctamd_init(int device) {
 }
 
 const char* ctamd_last_error(void) { return g_err; }
+int ctamd_set_math_mode(int mode) {
+    if (mode != CTAMD_MATH_FAST && mode != CTAMD_MATH_EXACT) return fail(CTAMD_EINVAL, "%s: unknown mode %d", __func__, mode);
+    g_math_mode.store(mode, std::memory_order_relaxed);
+    return CTAMD_OK;
+}
+int ctamd_math_mode(void) { return g_math_mode.load(std::memory_order_relaxed); }
 void ctamd_counters_reset(void) {
     std::lock_guard<std::mutex> lock(g_count_mu);
     g_bytes = g_flops = g_ideal_s = 0.0;

@@ -153,14 +153,15 @@ struct Row {
             for (int i = 0; i < W; ++i) s += cta_expf_nonpos(v[k][i] - m, exp2);
         return s;
     }
-    // v <- exp(v - m) with the hardware exp2 (~1e-7 relative near the maximum, where it matters)
+    // v <- exp(v - m) in single precision, within 2 ulp of expf (the hardware exp2 with the lost
+    // part of its argument put back)
     __device__ __forceinline__ float exp_shifted_fast(float m) {
         float s0 = 0.0f, s1 = 0.0f;
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k)
 #pragma unroll
             for (int i = 0; i < W; ++i) {
-                v[k][i] = __builtin_amdgcn_exp2f((v[k][i] - m) * 1.44269504088896340736f);
+                v[k][i] = cta_exp_hw_nonpos(v[k][i] - m);
                 if ((k * W + i) & 1) s1 += v[k][i]; else s0 += v[k][i];
             }
         return s0 + s1;
@@ -200,8 +201,19 @@ struct Row {
     }
 };
 
+// The ...Fast variants of the modes that write exp(x - max) / sum (or a function of it) evaluate the
+// exponential in single precision (<= 2 ulp) and multiply by 1 / sum; the plain ones return glibc's
+// expf bit for bit and the exactly rounded quotient.  kLogSoftmaxFast only forms its row SUM with the
+// hardware exponential (its output needs no exponential).
 enum Mode { kSoftmax, kCeOnehot, kCeIndex, kCeBwdOnehot, kCeBwdIndex, kSoftmaxBwd, kCeIndexBoth, kCeIndexBothFast,
-            kLogSoftmax, kLogSoftmaxFast, kLogSoftmaxBwd };
+            kLogSoftmax, kLogSoftmaxFast, kLogSoftmaxBwd, kSoftmaxFast, kCeBwdOnehotFast, kCeBwdIndexFast, kLogSoftmaxBwdFast };
+constexpr bool fast_out(int mode) {
+    return mode == kSoftmaxFast || mode == kCeBwdOnehotFast || mode == kCeBwdIndexFast || mode == kCeIndexBothFast || mode == kLogSoftmaxBwdFast;
+}
+constexpr int base_mode(int mode) {
+    return mode == kSoftmaxFast ? kSoftmax : mode == kCeBwdOnehotFast ? kCeBwdOnehot : mode == kCeBwdIndexFast ? kCeBwdIndex
+         : mode == kCeIndexBothFast ? kCeIndexBoth : mode == kLogSoftmaxBwdFast ? kLogSoftmaxBwd : mode;
+}
 
 struct Args {
     const float* x;      // logits / softmax output y (kSoftmaxBwd)
@@ -223,13 +235,15 @@ struct Args {
 // row is processed, so HBM latency hides behind the exp / divide work of the row in hand: with
 // 1024-thread blocks only one block fits a CU, and without this the CU would alternate between
 // waiting for memory and computing.
-template <int MODE, int THREADS, int ITEMS, int W>
+template <int MODE_, int THREADS, int ITEMS, int W>
 __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
+    constexpr int MODE = base_mode(MODE_);          // what the kernel does
+    constexpr bool kFastOut = fast_out(MODE_);      // how it evaluates exp(x - max) / sum
     __shared__ uint64_t s_exp2[32];
     __shared__ float s_f[2][THREADS / 64 + 1];
     __shared__ double s_d[THREADS / 64 + 1];
     stage_exp_table(s_exp2);
-    constexpr bool kBoth = (MODE == kCeIndexBoth || MODE == kCeIndexBothFast);
+    constexpr bool kBoth = (MODE == kCeIndexBoth);
     constexpr bool kLogSm = (MODE == kLogSoftmax || MODE == kLogSoftmaxFast);
     constexpr bool kPipelined = (MODE == kSoftmax || MODE == kCeIndex || MODE == kCeBwdIndex || kBoth || kLogSm);
     double block_loss = 0.0;
@@ -255,13 +269,14 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
             return;
         }
         // loss kernels keep x in r and only need the row sum; the others turn r into exp(x - m)
-        const float s = block_sum<THREADS>(kLossOnly ? r.sum_exp_fast(m) : MODE == kCeIndexBothFast ? r.exp_shifted_fast(m) : r.exp_shifted(m, s_exp2), s_f[1]);
+        const float s = block_sum<THREADS>(kLossOnly ? r.sum_exp_fast(m) : kFastOut ? r.exp_shifted_fast(m) : r.exp_shifted(m, s_exp2), s_f[1]);
         const double rcp_s = 1.0 / double(s);     // e / s below is the exact fp32 quotient (cta_div_rcp)
+        const float rcp_sf = 1.0f / s;            // fast output: e * (1 / s)
         if (MODE == kSoftmax) {
 #pragma unroll
             for (int k = 0; k < ITEMS; ++k)
 #pragma unroll
-                for (int i = 0; i < W; ++i) r.v[k][i] = cta_div_rcp(r.v[k][i], rcp_s);
+                for (int i = 0; i < W; ++i) r.v[k][i] = kFastOut ? r.v[k][i] * rcp_sf : cta_div_rcp(r.v[k][i], rcp_s);
             r.store(a.out + row * a.cols, unsigned(a.cols));
         } else if (MODE == kCeOnehot) {
             // -sum_j t_j * log(max(e_j / s, 1e-10)); terms with t_j == 0 contribute exactly 0
@@ -321,13 +336,11 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
             // it with each element's constant position keeps 32 column indices out of the registers
             const int q = (ok ? c / W : -1) - int(threadIdx.x);
             const int slot = (q >= 0 && q % THREADS == 0) ? (q / THREADS) * W + c % W : -1;
-            float ec = 0.0f;
-#pragma unroll
-            for (int k = 0; k < ITEMS; ++k)
-#pragma unroll
-                for (int i = 0; i < W; ++i) ec = (slot == k * W + i) ? r.v[k][i] : ec;
-            ec = block_sum<THREADS>(ec, s_f[0]);
-            const float rcp_sf = 1.0f / s;
+            // exp(x_c - m) once more from the logit itself, by every thread (row and c are uniform:
+            // one broadcast read of a line the row's loads have just brought in) - the same value as
+            // the row's own element, with no search through the registers and no exchange
+            const float xc = ok ? a.x[row * a.cols + size_t(c)] : 0.0f;
+            const float ec = kFastOut ? cta_exp_hw_nonpos(xc - m) : cta_expf_nonpos(xc - m, s_exp2);
             if (!ok) {
                 block_bad = true;
                 block_loss += double(__builtin_nanf(""));
@@ -336,13 +349,15 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
                 p = (p < 1e-10f) ? 1e-10f : p;
                 block_loss -= double(float(log(double(p))));
             }
+            // the class column's gradient 0 + (e_c / s - 1); every other element 0 + (e / s - 0) = e / s
+            const float smc = kFastOut ? ec * rcp_sf : cta_div_rcp(ec, rcp_s);
+            const float dc = 0.0f + (smc - 1.0f);
 #pragma unroll
             for (int k = 0; k < ITEMS; ++k)
 #pragma unroll
                 for (int i = 0; i < W; ++i) {
-                    float sm = MODE == kCeIndexBothFast ? r.v[k][i] * rcp_sf : cta_div_rcp(r.v[k][i], rcp_s);
-                    float d = sm - ((slot == k * W + i) ? 1.0f : 0.0f);
-                    r.v[k][i] = 0.0f + d;
+                    const float sm = kFastOut ? r.v[k][i] * rcp_sf : cta_div_rcp(r.v[k][i], rcp_s);
+                    r.v[k][i] = (slot == k * W + i) ? dc : sm;
                 }
             r.store(a.out + row * a.cols, unsigned(a.cols));
         } else {   // kCeBwdOnehot / kCeBwdIndex: dx = 0 + (e / s - t) * g (the tape adds it to a zero-filled buffer)
@@ -354,7 +369,7 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
                     r.group(a.t + row * a.cols, unsigned(a.cols), k, 0.0f, tq);
 #pragma unroll
                     for (int i = 0; i < W; ++i) {
-                        float sm = cta_div_rcp(r.v[k][i], rcp_s);
+                        float sm = kFastOut ? r.v[k][i] * rcp_sf : cta_div_rcp(r.v[k][i], rcp_s);
                         float d = sm - tq[i];
                         r.v[k][i] = 0.0f + d * g;
                     }
@@ -365,7 +380,7 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
                 for (int k = 0; k < ITEMS; ++k)
 #pragma unroll
                     for (int i = 0; i < W; ++i) {
-                        float sm = cta_div_rcp(r.v[k][i], rcp_s);
+                        float sm = kFastOut ? r.v[k][i] * rcp_sf : cta_div_rcp(r.v[k][i], rcp_s);
                         float d = sm - ((r.index(k, i) == unsigned(c)) ? 1.0f : 0.0f);
                         r.v[k][i] = 0.0f + d * g;
                     }
@@ -392,7 +407,7 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
             for (int k = 0; k < ITEMS; ++k)
 #pragma unroll
                 for (int i = 0; i < W; ++i) {
-                    const float t = cta_expf_tab(r.v[k][i], s_exp2) * d;
+                    const float t = (kFastOut ? cta_exp_hw(r.v[k][i]) : cta_expf_tab(r.v[k][i], s_exp2)) * d;
                     r.v[k][i] = q.v[k][i] - t;
                 }
             r.store(a.out + row * a.cols, unsigned(a.cols));
@@ -460,9 +475,11 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
 // hardware exp2 (only the sum is formed from it, ~1e-7 relative; the output sweep uses the bit-exact
 // exponential and the exact quotient), plain loads so that the second sweep finds the row in the
 // memory-side cache (one block per CU keeps 256 rows in flight), results written past the caches.
-template <int MODE>
+template <int MODE_>
 __global__ __launch_bounds__(1024) void row_stream_vec_kernel(Args a) {
     constexpr int THREADS = 1024, U = 4;
+    constexpr int MODE = base_mode(MODE_);
+    constexpr bool kFastOut = fast_out(MODE_);
     static_assert(MODE == kSoftmax || MODE == kSoftmaxBwd || MODE == kLogSoftmaxFast || MODE == kLogSoftmaxBwd,
                   "only the modes that write a row-shaped result");
     __shared__ uint64_t s_exp2[32];
@@ -490,7 +507,7 @@ __global__ __launch_bounds__(1024) void row_stream_vec_kernel(Args a) {
                 v4f o;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const float t = cta_expf_tab(y[e], s_exp2) * d;
+                    const float t = (kFastOut ? cta_exp_hw(y[e]) : cta_expf_tab(y[e], s_exp2)) * d;
                     o[e] = g[e] - t;
                 }
                 __builtin_nontemporal_store(o, outr + at);
@@ -572,6 +589,7 @@ __global__ __launch_bounds__(1024) void row_stream_vec_kernel(Args a) {
         s = (m == kNegInf) ? 0.0f : s * __builtin_amdgcn_exp2f((m - M) * 1.44269504088896340736f);
         const float S = block_sum<THREADS>(s, s_f[1]);
         const double rcp = 1.0 / double(S);
+        const float rcp_f = 1.0f / S;
         const float lg = (MODE == kLogSoftmaxFast) ? cta_logf(S, cta_log_tab) : 0.0f;
         auto give = [&](const v4f& v, unsigned at) {
             v4f o;
@@ -580,6 +598,8 @@ __global__ __launch_bounds__(1024) void row_stream_vec_kernel(Args a) {
                 if (MODE == kLogSoftmaxFast) {
                     const float d = v[e] - M;
                     o[e] = d - lg;
+                } else if (kFastOut) {
+                    o[e] = cta_exp_hw_nonpos(v[e] - M) * rcp_f;
                 } else {
                     o[e] = cta_div_rcp(cta_expf_nonpos(v[e] - M, s_exp2), rcp);
                 }
@@ -598,9 +618,10 @@ __global__ __launch_bounds__(1024) void row_stream_vec_kernel(Args a) {
     }
 }
 
-template <int MODE>
+template <int MODE_>
 __global__ __launch_bounds__(1024) void row_stream_kernel(Args a) {
     constexpr int THREADS = 1024;
+    constexpr int MODE = base_mode(MODE_);          // this path (ragged or unaligned long rows) keeps the exact routines
     __shared__ uint64_t s_exp2[32];
     __shared__ float s_f[2][THREADS / 64 + 1];
     __shared__ double s_d[THREADS / 64 + 1];
@@ -788,7 +809,7 @@ __global__ __launch_bounds__(256) void ce_bwd_stats_kernel(Args a) {
         const float rcp_sf = float(rcp_s);
         const unsigned c = unsigned(int(a.t[row]));
         auto one = [&](float v, unsigned j) {
-            float sm = FAST ? __builtin_amdgcn_exp2f((v - M) * kLog2e) * rcp_sf
+            float sm = FAST ? cta_exp_hw_nonpos(v - M) * rcp_sf
                             : cta_div_rcp(cta_expf_nonpos(v - M, s_exp2), rcp_s);
             return 0.0f + (sm - ((j == c) ? 1.0f : 0.0f)) * g;
         };
@@ -854,11 +875,13 @@ bool launch_resident(const Args& a, unsigned grid, hipStream_t s) {
     else {
         // rows of 2048 columns or more never reach these two modes (they go to the online forward
         // kernel and to the long-row one-pass kernel): the 1024-thread shapes are not built for them
+        // (nor reach them in the exact forms below when the library runs in its fast mode, and vice versa -
+        // but both are built: the mode is a run-time switch)
         if constexpr (MODE == kCeIndex || MODE == kCeIndexBoth || MODE == kLogSoftmax) {
             return false;
         } else {
             if (groups <= 1024 * 2) launch_cfg<MODE, 1024, 2, W>(a, grid, s);
-            else if constexpr (MODE == kLogSoftmaxBwd) return false;   // two resident rows and the exponential do not fit 128 registers
+            else if constexpr (MODE == kLogSoftmaxBwd) return false;   // two resident rows and the double-precision exponential do not fit 128 registers
             else if (groups <= 1024 * 8) launch_cfg<MODE, 1024, 8, W>(a, grid, s);
             else return false;
         }
@@ -866,9 +889,10 @@ bool launch_resident(const Args& a, unsigned grid, hipStream_t s) {
     return true;
 }
 
-template <int MODE>
+template <int MODE_>
 int run_rows(const char* name, Args a, float* loss_out, void* stream) {
-    constexpr bool kBoth = (MODE == kCeIndexBoth || MODE == kCeIndexBothFast);
+    constexpr int MODE = base_mode(MODE_);
+    constexpr bool kBoth = (MODE == kCeIndexBoth);
     constexpr bool kLoss = (MODE == kCeOnehot || MODE == kCeIndex || kBoth);
     constexpr bool kIndexLoss = (MODE == kCeIndex || kBoth);
     constexpr bool kWrites = !kLoss || kBoth;                          // a [rows, cols] result
@@ -917,13 +941,13 @@ int run_rows(const char* name, Args a, float* loss_out, void* stream) {
         hipLaunchKernelGGL(loss_stage2, dim3(1), dim3(256), 0, s, a.partials, grid, loss_out, MODE == kCeIndex ? a.status : nullptr);
         return launched(name);
     }
-    bool done = vec ? launch_resident<MODE, 4>(a, grid, s) : launch_resident<MODE, 1>(a, grid, s);
+    bool done = vec ? launch_resident<MODE_, 4>(a, grid, s) : launch_resident<MODE_, 1>(a, grid, s);
     if (!done) {
         if constexpr (kBoth)
             return fail(CTAMD_ERANGE, "%s: a row does not fit a block's registers (32768 columns, 8192 without 128-bit accesses): "
                         "use the separate forward and backward entry points", name);
         else if constexpr (MODE == kSoftmax || MODE == kSoftmaxBwd || MODE == kLogSoftmaxFast || MODE == kLogSoftmaxBwd) {
-            if (vec) hipLaunchKernelGGL((row_stream_vec_kernel<MODE>), dim3(grid), dim3(1024), 0, s, a);
+            if (vec) hipLaunchKernelGGL((row_stream_vec_kernel<MODE_>), dim3(grid), dim3(1024), 0, s, a);
             else hipLaunchKernelGGL((row_stream_kernel<MODE>), dim3(grid), dim3(1024), 0, s, a);
         } else
             hipLaunchKernelGGL((row_stream_kernel<MODE>), dim3(grid), dim3(1024), 0, s, a);
@@ -1014,13 +1038,13 @@ __global__ __launch_bounds__(256) void log_softmax_bwd_cols_kernel(const float* 
 // whole column alone.
 enum ColMode { kColOnline, kColSoftmaxOut, kColDot, kColBwdOut, kColSum, kColLogSoftmaxOut, kColLogBwdOut };
 
-template <int MODE, int W>
+template <int MODE, int W, bool FAST>
 __global__ __launch_bounds__(256) void col_walk_kernel(const float* __restrict__ x, const float* __restrict__ x2,
                                                        const float* __restrict__ p0, const float* __restrict__ p1,
                                                        float* __restrict__ out, size_t rows, size_t cols,
                                                        size_t rows_per_block) {
     __shared__ uint64_t s_exp2[32];
-    if (MODE == kColSoftmaxOut || MODE == kColLogBwdOut) stage_exp_table(s_exp2);
+    if ((MODE == kColSoftmaxOut || MODE == kColLogBwdOut) && !FAST) stage_exp_table(s_exp2);
     const size_t col = (size_t(blockIdx.x) * 256 + threadIdx.x) * W;
     if (col >= cols) return;
     const size_t r0 = size_t(blockIdx.y) * rows_per_block;
@@ -1036,6 +1060,9 @@ __global__ __launch_bounds__(256) void col_walk_kernel(const float* __restrict__
         q0[e] = (MODE == kColSoftmaxOut || MODE == kColBwdOut || MODE == kColLogSoftmaxOut || MODE == kColLogBwdOut) ? p0[col + e] : 0.0f;
         rcp[e] = (MODE == kColSoftmaxOut) ? 1.0 / double(p1[col + e]) : 0.0;
     }
+    float rcp_f[W];                     // FAST: e * (1 / sum)
+#pragma unroll
+    for (int e = 0; e < W; ++e) rcp_f[e] = (MODE == kColSoftmaxOut && FAST) ? 1.0f / p1[col + e] : 0.0f;
     float lg[W];                        // kColLogSoftmaxOut: log of the column's sum
 #pragma unroll
     for (int e = 0; e < W; ++e) lg[e] = (MODE == kColLogSoftmaxOut) ? cta_logf(p1[col + e], cta_log_tab) : 0.0f;
@@ -1076,14 +1103,16 @@ __global__ __launch_bounds__(256) void col_walk_kernel(const float* __restrict__
                 ex = v[e] == kNegInf ? 0.0f : ex;
                 acc[e] = up ? __fmaf_rn(acc[e], ex, 1.0f) : acc[e] + ex;
                 mx[e] = up ? v[e] : mx[e];
-            } else if (MODE == kColSoftmaxOut) o[e] = cta_div_rcp(cta_expf_nonpos(v[e] - q0[e], s_exp2), rcp[e]);
+            } else if (MODE == kColSoftmaxOut) {
+                o[e] = FAST ? cta_exp_hw_nonpos(v[e] - q0[e]) * rcp_f[e] : cta_div_rcp(cta_expf_nonpos(v[e] - q0[e], s_exp2), rcp[e]);
+            }
             else if (MODE == kColDot) acc[e] = __fmaf_rn(w[e], v[e], acc[e]);
             else if (MODE == kColSum) acc[e] += v[e];
             else if (MODE == kColLogSoftmaxOut) {
                 const float d = v[e] - q0[e];
                 o[e] = d - lg[e];
             } else if (MODE == kColLogBwdOut) {                  // v = y, w = g, q0 = column sum of g
-                const float t = cta_expf_tab(v[e], s_exp2) * q0[e];
+                const float t = (FAST ? cta_exp_hw(v[e]) : cta_expf_tab(v[e], s_exp2)) * q0[e];
                 o[e] = w[e] - t;
             } else o[e] = v[e] * (w[e] - q0[e]);
         }
@@ -1217,11 +1246,11 @@ bool plan_cols(size_t rows, size_t cols, bool aligned, ColPlan& p) {
     return true;
 }
 
-template <int MODE>
+template <int MODE, bool FAST = false>
 void launch_col_walk(const ColPlan& p, const float* x, const float* x2, const float* p0, const float* p1, float* out, size_t rows,
                      size_t cols, hipStream_t s) {
-    if (p.vec) hipLaunchKernelGGL((col_walk_kernel<MODE, 4>), p.grid, dim3(256), 0, s, x, x2, p0, p1, out, rows, cols, p.rows_per_block);
-    else hipLaunchKernelGGL((col_walk_kernel<MODE, 1>), p.grid, dim3(256), 0, s, x, x2, p0, p1, out, rows, cols, p.rows_per_block);
+    if (p.vec) hipLaunchKernelGGL((col_walk_kernel<MODE, 4, FAST>), p.grid, dim3(256), 0, s, x, x2, p0, p1, out, rows, cols, p.rows_per_block);
+    else hipLaunchKernelGGL((col_walk_kernel<MODE, 1, FAST>), p.grid, dim3(256), 0, s, x, x2, p0, p1, out, rows, cols, p.rows_per_block);
 }
 
 }  // namespace
@@ -1233,6 +1262,7 @@ extern "C" {
 
 int ctamd_softmax_rows_f32(const float* x, float* y, size_t rows, size_t cols, void* stream) {
     Args a{x, nullptr, nullptr, y, nullptr, nullptr, nullptr, rows, cols, nullptr, nullptr};
+    if (fast_math()) return run_rows<kSoftmaxFast>(__func__, a, nullptr, stream);
     return run_rows<kSoftmax>(__func__, a, nullptr, stream);
 }
 int ctamd_cross_entropy_onehot_f32(const float* x, const float* t, float* out, size_t rows, size_t cols, void* stream) {
@@ -1253,7 +1283,7 @@ int ctamd_cross_entropy_backward_index_stats_f32(const float* x, const float* id
     const size_t fill = size_t(compute_units() > 0 ? compute_units() : 256) * 8;
     const unsigned grid = rows < fill ? unsigned(rows) : unsigned(fill);
     const bool vec = (cols % 4 == 0) && aligned16(x) && aligned16(dx);
-    if (vec && cols >= 2048) hipLaunchKernelGGL((ce_bwd_stats_kernel<true, true>), dim3(grid), dim3(256), 0, as_stream(stream), a);
+    if (vec && (cols >= 2048 || fast_math())) hipLaunchKernelGGL((ce_bwd_stats_kernel<true, true>), dim3(grid), dim3(256), 0, as_stream(stream), a);
     else if (vec) hipLaunchKernelGGL((ce_bwd_stats_kernel<true, false>), dim3(grid), dim3(256), 0, as_stream(stream), a);
     else hipLaunchKernelGGL((ce_bwd_stats_kernel<false, false>), dim3(grid), dim3(256), 0, as_stream(stream), a);
     account(8.0 * double(rows) * double(cols) + 12.0 * double(rows), double(rows) * double(cols));
@@ -1269,17 +1299,19 @@ int ctamd_cross_entropy_index_fused_f32(const float* x, const float* idx, float*
     Args a{x, idx, nullptr, dx, nullptr, status, nullptr, rows, cols, nullptr, nullptr};
     // long rows use the hardware exponential throughout, as the forward / backward-from-statistics
     // pair does (<= 2e-7 from the exact form)
-    if (cols >= 2048) return run_rows<kCeIndexBothFast>(__func__, a, out, stream);
+    if (cols >= 2048 || fast_math()) return run_rows<kCeIndexBothFast>(__func__, a, out, stream);
     return run_rows<kCeIndexBoth>(__func__, a, out, stream);
 }
 int ctamd_cross_entropy_backward_onehot_f32(const float* x, const float* t, const float* g1, float* dx, size_t rows,
                                             size_t cols, void* stream) {
     Args a{x, t, g1, dx, nullptr, nullptr, nullptr, rows, cols, nullptr, nullptr};
+    if (fast_math()) return run_rows<kCeBwdOnehotFast>(__func__, a, nullptr, stream);
     return run_rows<kCeBwdOnehot>(__func__, a, nullptr, stream);
 }
 int ctamd_cross_entropy_backward_index_f32(const float* x, const float* idx, const float* g1, float* dx, size_t rows,
                                            size_t cols, void* stream) {
     Args a{x, idx, g1, dx, nullptr, nullptr, nullptr, rows, cols, nullptr, nullptr};
+    if (fast_math()) return run_rows<kCeBwdIndexFast>(__func__, a, nullptr, stream);
     return run_rows<kCeBwdIndex>(__func__, a, nullptr, stream);
 }
 int ctamd_softmax_backward_rows_f32(const float* y, const float* g, float* dx, size_t rows, size_t cols, void* stream) {
@@ -1294,6 +1326,7 @@ int ctamd_log_softmax_rows_f32(const float* x, float* y, size_t rows, size_t col
 }
 int ctamd_log_softmax_backward_rows_f32(const float* y, const float* g, float* dx, size_t rows, size_t cols, void* stream) {
     Args a{y, g, nullptr, dx, nullptr, nullptr, nullptr, rows, cols, nullptr, nullptr};
+    if (fast_math()) return run_rows<kLogSoftmaxBwdFast>(__func__, a, nullptr, stream);
     return run_rows<kLogSoftmaxBwd>(__func__, a, nullptr, stream);
 }
 int ctamd_log_softmax_cols_f32(const float* x, float* y, size_t rows, size_t cols, void* stream) {
@@ -1322,7 +1355,8 @@ int ctamd_log_softmax_backward_cols_f32(const float* y, const float* g, float* d
         launch_col_walk<kColSum>(p, g, nullptr, nullptr, nullptr, p.partials, rows, cols, s);
         hipLaunchKernelGGL(col_fold_kernel<false>, dim3(unsigned((cols + kFoldCols - 1) / kFoldCols)), dim3(256), 0, s, p.partials, nullptr, p.v0,
                            cols, unsigned(p.chunks));
-        launch_col_walk<kColLogBwdOut>(p, y, g, p.v0, nullptr, dx, rows, cols, s);
+        if (fast_math()) launch_col_walk<kColLogBwdOut, true>(p, y, g, p.v0, nullptr, dx, rows, cols, s);
+        else launch_col_walk<kColLogBwdOut>(p, y, g, p.v0, nullptr, dx, rows, cols, s);
         return launched(__func__);
     }
     hipLaunchKernelGGL(log_softmax_bwd_cols_kernel, dim3((unsigned)((cols + 255) / 256)), dim3(256), 0, as_stream(stream), y, g, dx, rows, cols);
@@ -1338,7 +1372,8 @@ int ctamd_softmax_cols_f32(const float* x, float* y, size_t rows, size_t cols, v
         const unsigned fold_blocks = unsigned((cols + kFoldCols - 1) / kFoldCols);
         launch_col_walk<kColOnline>(p, x, nullptr, nullptr, nullptr, p.partials, rows, cols, s);
         hipLaunchKernelGGL(col_fold_kernel<true>, dim3(fold_blocks), dim3(256), 0, s, p.partials, p.v0, p.v1, cols, unsigned(p.chunks));
-        launch_col_walk<kColSoftmaxOut>(p, x, nullptr, p.v0, p.v1, y, rows, cols, s);
+        if (fast_math()) launch_col_walk<kColSoftmaxOut, true>(p, x, nullptr, p.v0, p.v1, y, rows, cols, s);
+        else launch_col_walk<kColSoftmaxOut>(p, x, nullptr, p.v0, p.v1, y, rows, cols, s);
         account(8.0 * double(rows) * double(cols), double(rows) * double(cols));
         return launched(__func__);
     }

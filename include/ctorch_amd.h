@@ -45,6 +45,19 @@ int ctamd_device_count(void);
 const char* ctamd_last_error(void);
 const char* ctamd_version(void);
 
+/* How softmax, log_softmax's gradient, the cross-entropy gradients and the fused expressions evaluate
+ * exp / sin / cos (process-wide; takes effect for later launches).  The reference calls glibc's expf,
+ * sinf, cosf (src/Tensor.cpp:1682,1722; src/AutoDiff.cpp:1558,1564; CrossEntropy_BASIC_kernel.cpp:56).
+ *   CTAMD_MATH_FAST  (default) single precision, within 2 ulp of those calls, and e * (1 / sum) for
+ *                    the softmax quotient: the kernels run at memory speed
+ *   CTAMD_MATH_EXACT the double-precision routines that return glibc 2.35's floats bit for bit and
+ *                    the exactly rounded quotient e / sum, as the reference computes it; 1.2 - 2x slower
+ * The one-operator kernels (ctamd_sin_f32, ctamd_exp_f32, ...) always return glibc's floats. */
+#define CTAMD_MATH_FAST 0
+#define CTAMD_MATH_EXACT 1
+int ctamd_set_math_mode(int mode);
+int ctamd_math_mode(void);
+
 /* Storage: device allocation and explicit transfers; replaces `new char[]` / memcpy in
  * Storage (include/Storage.h:77, :175-181). */
 int ctamd_malloc(void** ptr, size_t bytes);

@@ -279,3 +279,14 @@ def softmax_f64(x, dim):
     rows, cols = (1, x.numel()) if x.dim() == 1 else x.shape
     call("ctamd_softmax_f64", ptr(x), ptr(r), rows, cols, 1 if x.dim() == 1 else dim, stream())
     return r
+
+
+MATH_FAST, MATH_EXACT = 0, 1
+
+
+def set_math_mode(mode):
+    """CTAMD_MATH_FAST (0, the default) or CTAMD_MATH_EXACT (1) for later launches; returns the previous mode."""
+    l = lib()
+    prev = l.ctamd_math_mode()
+    capi.check(l.ctamd_set_math_mode(mode))
+    return prev
