@@ -245,7 +245,8 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
     stage_exp_table(s_exp2);
     constexpr bool kBoth = (MODE == kCeIndexBoth);
     constexpr bool kLogSm = (MODE == kLogSoftmax || MODE == kLogSoftmaxFast);
-    constexpr bool kPipelined = (MODE == kSoftmax || MODE == kCeIndex || MODE == kCeBwdIndex || kBoth || kLogSm);
+    // (a row of 16 groups per thread fills the registers by itself: no second copy to prefetch into)
+    constexpr bool kPipelined = (MODE == kSoftmax || MODE == kCeIndex || MODE == kCeBwdIndex || kBoth || kLogSm) && ITEMS <= 8;
     double block_loss = 0.0;
     bool block_bad = false;   // a class index out of range was met (thread 0's copy counts)
 
@@ -883,7 +884,11 @@ bool launch_resident(const Args& a, unsigned grid, hipStream_t s) {
             if (groups <= 1024 * 2) launch_cfg<MODE, 1024, 2, W>(a, grid, s);
             else if constexpr (MODE == kLogSoftmaxBwd) return false;   // two resident rows and the double-precision exponential do not fit 128 registers
             else if (groups <= 1024 * 8) launch_cfg<MODE, 1024, 8, W>(a, grid, s);
-            else return false;
+            else if constexpr (MODE == kSoftmaxFast && W == 4) {
+                // up to 65536 columns: the whole row in registers (64 per thread), one row at a time
+                if (groups <= 1024 * 16) launch_cfg<MODE, 1024, 16, W>(a, grid, s);
+                else return false;
+            } else return false;
         }
     }
     return true;
