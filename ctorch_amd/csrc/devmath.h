@@ -27,8 +27,10 @@
 #define CTA_FN __device__ __forceinline__ static
 #define CTA_TAB_SPACE __device__ static const
 #define CTA_FMA(a, b, c) __fma_rn((a), (b), (c))
+#define CTA_FMAF(a, b, c) __fmaf_rn((a), (b), (c))
 #else
 #define CTA_FMA(a, b, c) __builtin_fma((a), (b), (c))
+#define CTA_FMAF(a, b, c) __builtin_fmaf((a), (b), (c))
 #include <math.h>
 #include <string.h>
 #define CTA_FN static inline
@@ -331,6 +333,33 @@ CTA_FN float cta_tanf(float y, const uint32_t* inv_pio4) {
     return cta_tan_finish(y, ay, n, xr);
 }
 
+// ----------------------------------------------------------------------------------------------
+// Single-precision sine / cosine for |y| < 120 (cta_sincos_is_rare(y) == 0), for the kernels whose
+// time the double-precision routines above would set (fused expressions): the quadrant by one
+// multiplication, the argument reduced against pi/2 split in three floats whose first two have 16
+// significant bits (so their products with the quadrant number, below 2^8, are exact and the first
+// two steps lose nothing), then the classic degree-7 / degree-8 polynomials on [-pi/4, pi/4].  Only
+// IEEE single operations with explicit fused multiply-adds: the same bits on the host and on the
+// device.  Within 2 ulp of glibc's sinf / cosf for every |y| < 120
+// (tests/native/devmath_check.c, exhaustive); larger arguments take cta_sincosf.
+CTA_FN float cta_sincosf_f32(float y, int want_cos) {
+    const float nf = __builtin_rintf(y * 0x1.45f306p-1f);                  // 2 / pi
+    int n = (int)nf;
+    float r = CTA_FMAF(nf, -0x1.922p+0f, y);
+    r = CTA_FMAF(nf, 0x1.2aeep-18f, r);
+    r = CTA_FMAF(nf, 0x1.e974p-35f, r);
+    const float z = r * r;
+    float sp = CTA_FMAF(z, -1.9515295891e-4f, 8.3321608736e-3f);
+    sp = CTA_FMAF(sp, z, -1.6666654611e-1f);
+    const float sn = CTA_FMAF(r * z, sp, r);
+    float cp = CTA_FMAF(z, 2.443315711809948e-5f, -1.388731625493765e-3f);
+    cp = CTA_FMAF(cp, z, 4.166664568298827e-2f);
+    const float c = CTA_FMAF(z * z, cp, CTA_FMAF(z, -0.5f, 1.0f));
+    if (want_cos) n += 1;
+    const float res = (n & 1) ? c : sn;
+    return cta_u2f(cta_f2u(res) ^ ((uint32_t)(n & 2) << 30));
+}
+
 #if defined(__HIPCC__)
 // ----------------------------------------------------------------------------------------------
 // Single-precision exponential for the kernels whose time the double-precision one above would set
@@ -358,6 +387,44 @@ __device__ __forceinline__ static float cta_exp_hw(float d) {
     t = __fmaf_rn(z, -0x1.7f7d1cp-20f, t);
     const float r = __fmaf_rn(e, t, e);
     return (e == __builtin_huge_valf()) ? e : r;
+}
+// The same with the argument held to [-150, 88], so that the result is always finite (at most e^88 =
+// 1.65e38).  A NaN argument gives e^-150 = 0: callers that must return NaN for NaN select it themselves.
+__device__ __forceinline__ static float cta_exp_hw_bounded(float d) {
+    const float dc = __builtin_amdgcn_fmed3f(d, -150.0f, 88.0f);
+    const float z = dc * 0x1.715476p+0f;
+    const float e = __builtin_amdgcn_exp2f(z);
+    float t = __fmaf_rn(z, -0x1.62e4p-1f, dc);
+    t = __fmaf_rn(z, -0x1.7f7d1cp-20f, t);
+    return __fmaf_rn(e, t, e);
+}
+// 1 / s for finite s >= 1: the hardware reciprocal (1 ulp) and one Newton step, within 1 ulp of
+// the exactly rounded quotient.  Where 1 / s would be subnormal (s > 2^126) the result may be 0.
+__device__ __forceinline__ static float cta_rcp_refined(float s) {
+    const float r = __builtin_amdgcn_rcpf(s);
+    const float err = __fmaf_rn(-s, r, 1.0f);
+    return __fmaf_rn(err, r, r);
+}
+// Single-precision sigmoid by the reference's formula 1 / (1 + e^-x) on the exponential and the
+// reciprocal above.  Against the same formula on expf and an exact division (what the exact mode
+// returns): within 4 ulp - the sum 1 + e is rounded where its spacing is up to four times the
+// spacing of the quotient, so one ulp of the exponential is worth up to four of the result - and
+// below the smallest normal number (x < -87.3) possibly 0 where the exact mode has a subnormal.
+__device__ __forceinline__ static float cta_sigmoid_f32(float x) {
+    const float s = 1.0f + cta_exp_hw_bounded(-x);
+    const float r = cta_rcp_refined(s);
+    return (x != x) ? x : r;
+}
+// Single-precision tanh.  The reference computes (e^x - e^-x) / (e^x + e^-x); this computes the same
+// function as 1 - 2 / (e^2|x| + 1) with the sign of x (one exponential, one reciprocal): within 2 ulp
+// of tanh for |x| >= 1, within 1.2e-7 absolute below, where the reference's form loses its digits to
+// the same cancellation.  The reference's form is inf / inf = NaN once expf(|x|) overflows, that is
+// for |x| > 0x1.62e42ep+6: so is this, and NaN stays NaN.
+__device__ __forceinline__ static float cta_tanh_f32(float x) {
+    const float ax = __builtin_fabsf(x);
+    const float s = cta_exp_hw_bounded(ax + ax) + 1.0f;
+    const float v = __fmaf_rn(-2.0f, cta_rcp_refined(s), 1.0f);
+    return (ax <= 0x1.62e42ep+6f) ? __builtin_copysignf(v, x) : __builtin_nanf("");
 }
 #endif
 

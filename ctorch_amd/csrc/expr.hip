@@ -19,22 +19,41 @@
 #include "functors.h"
 
 #include <cfloat>
+#include <utility>
 
 namespace ctamd {
 namespace {
 
 constexpr int kExprThreads = 256;
-constexpr int kPerLane = 4;                   // elements per lane and pass
+constexpr int kMaxHalves = 2;                 // 128-bit words per lane and pass: one or two
 constexpr int kMaxInsns = CTAMD_EXPR_MAX_INSNS;
-constexpr int kMaxSlots = CTAMD_EXPR_MAX_SLOTS;
+constexpr int kMaxSlots = CTAMD_EXPR_MAX_SLOTS;          // slot numbers a program may name
+constexpr int kWordBytes = kExprThreads * 16;            // one value of a block in LDS, per 128-bit word of a lane
+constexpr int kLdsBudget = 155 << 10;                    // for values (160 KiB less the tables)
+constexpr int kMaxLive = kLdsBudget / kWordBytes;        // values that can be live in LDS at once, one word per lane
 constexpr int kMaxPorts = CTAMD_EXPR_MAX_PORTS;
 constexpr int kMaxDevices = 64;
 
+// What the kernel runs: the caller's program after value numbering.  Every instruction's result
+// stays in registers (the "carry") until the next result replaces it.  An instruction works in
+// place on the carry: its operand a is the carry, fetched from LDS first where the carry holds
+// something else (kAFetch); operand b is fetched from LDS (kBFetch) or is the carry too; the result
+// goes to LDS only if an instruction further on has to fetch it (kKeep).  Where only the second
+// operand of a - b, a / b or the ReLU gradient is in the carry, the operands change places and the
+// operator is one of the reversed ones below.  LDS places are handed out by liveness, so a program
+// may name many slots and still occupy few.
+enum : uint8_t { kAFetch = 1, kBFetch = 2, kKeep = 4 };
+enum : uint8_t { kRevSub = 32, kRevDiv = 33, kRevReluMul = 34 };   // b - a, b / a, a * (b > 0 ? 1 : 0)
 struct DevInsn {
-    uint8_t op, dst, a, b;
-    float imm;
-    double rcp;                               // DIVS: 1 / double(imm)
+    uint8_t op, flags;
+    uint16_t dst;                             // LDS place of the result (kKeep; in 128-bit words of a one-word-per-lane layout); stores: output port
+    uint16_t a, b;                            // LDS places of the operands; loads: a = input port
+    union {
+        float imm;
+        double rcp;                           // DIVS: 1 / double(imm)
+    };
 };
+static_assert(sizeof(DevInsn) == 16, "one 128-bit scalar load per instruction");
 
 struct ExprArgs {
     const float* in[kMaxPorts];
@@ -43,213 +62,279 @@ struct ExprArgs {
     size_t total;                             // elements of a full-shape value
     unsigned cols;                            // row length (row-vector loads)
     int n_insn;
-    int vec;                                  // 1: 128-bit accesses (all pointers aligned, total % 4 == 0, cols % 4 == 0)
     int has_row;                              // the program loads a row vector
     int n_lead;                               // the first n_lead instructions are loads (at most kLeadLoads)
     int n_tail;                               // VEC: the last n_tail instructions are stores (at most kTailStores)
-    DevInsn prog[kMaxInsns];
+    DevInsn prog[kMaxInsns + 1];              // one spare: the kernel fetches an instruction ahead
 };
 
-// One operator on the four elements of a lane; a, b are the operand values.  The operator is chosen
-// once (a scalar branch) and its four evaluations are independent instruction streams that the
-// compiler interleaves: the long dependent chains of the transcendental functors (fp64 inside
-// sinf / cosf) hide each other's latencies.
-template <class F>
-__device__ __forceinline__ void each(float (&o)[kPerLane], F f) {
+// One operator on the N elements of a lane, in place: c holds operand a on entry and the result on
+// return, b the second operand of the two-operand operators.  The operator is chosen once (a
+// scalar branch) and its N evaluations are independent instruction streams that the compiler
+// interleaves: the long dependent chains of the transcendental functors hide each other's latencies.
+template <int N, class F>
+__device__ __forceinline__ void each(float (&c)[N], F f) {
 #pragma unroll
-    for (int e = 0; e < kPerLane; ++e) o[e] = f(e);
+    for (int e = 0; e < N; ++e) c[e] = f(e);
 }
-__device__ __forceinline__ void apply(const DevInsn& q, const float (&a)[kPerLane], const float (&b)[kPerLane],
-                                      float (&o)[kPerLane], const Tables& t) {
+// FASTM: the transcendental operators in single precision (sin / cos within 2 ulp of sinf / cosf for
+// |x| < 120, the double-precision routines beyond; sigmoid within 4 ulp of the reference's formula on
+// expf; tanh within 2 ulp of tanh for |x| >= 1 and 1.2e-7 absolute below); otherwise the routines
+// that return glibc's floats.
+template <bool FASTM, int N>
+__device__ __forceinline__ void apply(const DevInsn& q, float (&c)[N], const float (&b)[N], const Tables& t) {
     switch (q.op) {
-        case CTAMD_EX_ADD: each(o, [&](int e) { return a[e] + b[e]; }); break;
-        case CTAMD_EX_SUB: each(o, [&](int e) { return a[e] - b[e]; }); break;
-        case CTAMD_EX_MUL: each(o, [&](int e) { return a[e] * b[e]; }); break;
-        case CTAMD_EX_DIV: each(o, [&](int e) { return a[e] / b[e]; }); break;
-        case CTAMD_EX_NEG: each(o, [&](int e) { return -a[e]; }); break;
-        case CTAMD_EX_RELU: each(o, [&](int e) { return (0.0f < a[e]) ? a[e] : 0.0f; }); break;
-        case CTAMD_EX_SIGMOID: each(o, [&](int e) { return sigmoid_ref(a[e], t); }); break;
-        case CTAMD_EX_TANH: each(o, [&](int e) { return tanh_ref(a[e], t); }); break;
+        case CTAMD_EX_ADD: each(c, [&](int e) { return c[e] + b[e]; }); break;
+        case CTAMD_EX_SUB: each(c, [&](int e) { return c[e] - b[e]; }); break;
+        case kRevSub: each(c, [&](int e) { return b[e] - c[e]; }); break;
+        case CTAMD_EX_MUL: each(c, [&](int e) { return c[e] * b[e]; }); break;
+        case CTAMD_EX_DIV: each(c, [&](int e) { return c[e] / b[e]; }); break;
+        case kRevDiv: each(c, [&](int e) { return b[e] / c[e]; }); break;
+        case CTAMD_EX_NEG: each(c, [&](int e) { return -c[e]; }); break;
+        case CTAMD_EX_RELU: each(c, [&](int e) { return (0.0f < c[e]) ? c[e] : 0.0f; }); break;
+        case CTAMD_EX_SIGMOID:
+            if (FASTM) each(c, [&](int e) { return cta_sigmoid_f32(c[e]); });
+            else each(c, [&](int e) { return sigmoid_ref(c[e], t); });
+            break;
+        case CTAMD_EX_TANH:
+            if (FASTM) each(c, [&](int e) { return cta_tanh_f32(c[e]); });
+            else each(c, [&](int e) { return tanh_ref(c[e], t); });
+            break;
         case CTAMD_EX_SIN:
         case CTAMD_EX_COS: {
             const int want_cos = (q.op == CTAMD_EX_COS);
             bool rare = false;
+            float x[N];
 #pragma unroll
-            for (int e = 0; e < kPerLane; ++e) {
-                o[e] = cta_sincosf_fast(a[e], want_cos);
-                rare = rare || cta_sincos_is_rare(a[e]);
+            for (int e = 0; e < N; ++e) {
+                x[e] = c[e];
+                c[e] = FASTM ? cta_sincosf_f32(x[e], want_cos) : cta_sincosf_fast(x[e], want_cos);
+                rare = rare || !(__builtin_fabsf(x[e]) < 120.0f);      // |x| >= 120, inf, NaN
             }
             if (__builtin_expect(rare, 0)) {
-                for (int e = 0; e < kPerLane; ++e)
-                    if (cta_sincos_is_rare(a[e])) o[e] = cta_sincosf(a[e], want_cos, t.inv_pio4);
+                for (int e = 0; e < N; ++e)
+                    if (cta_sincos_is_rare(x[e])) c[e] = cta_sincosf(x[e], want_cos, t.inv_pio4);
             }
             break;
         }
-        case CTAMD_EX_ADDS: each(o, [&](int e) { return a[e] + q.imm; }); break;
-        case CTAMD_EX_MULS: each(o, [&](int e) { return a[e] * q.imm; }); break;
-        case CTAMD_EX_DIVS: each(o, [&](int e) { return cta_div_rcp(a[e], q.rcp); }); break;
-        case CTAMD_EX_RSUBS: each(o, [&](int e) { return q.imm - a[e]; }); break;
-        case CTAMD_EX_RELUMUL: each(o, [&](int e) { return b[e] * ((a[e] > 0.0f) ? 1.0f : 0.0f); }); break;
-        default: each(o, [&](int e) { return a[e]; }); break;
+        case CTAMD_EX_ADDS: each(c, [&](int e) { return c[e] + q.imm; }); break;
+        case CTAMD_EX_MULS: each(c, [&](int e) { return c[e] * q.imm; }); break;
+        case CTAMD_EX_DIVS: each(c, [&](int e) { return cta_div_rcp(c[e], q.rcp); }); break;
+        case CTAMD_EX_RSUBS: each(c, [&](int e) { return q.imm - c[e]; }); break;
+        case CTAMD_EX_RELUMUL: each(c, [&](int e) { return b[e] * ((c[e] > 0.0f) ? 1.0f : 0.0f); }); break;
+        case kRevReluMul: each(c, [&](int e) { return c[e] * ((b[e] > 0.0f) ? 1.0f : 0.0f); }); break;
+        default: break;
     }
 }
 
 constexpr int kLeadLoads = 3;   // loads at the head of a program that run one pass ahead
 constexpr int kTailStores = 2;  // stores at the end of a program that are issued one pass late (VEC only)
 
-// Where a lane's four elements of one pass live.  VEC: four consecutive elements, one 128-bit
-// access (all pointers 16-byte aligned, total and cols multiples of four, fewer than 2^32
-// vectors): vector index v, and for row vectors the vector index within the row, stepped from
-// pass to pass without a division.  Otherwise: elements 256 apart, 32-bit accesses, any shape.
-template <bool VEC>
-struct Place {
-    size_t first;        // VEC: vector index; else: element index of element 0
-    unsigned col;        // VEC: vector index within the row; else unused
+template <int H>
+struct Vals {
+    v4f h[H];
 };
 
-template <bool VEC>
-__device__ __forceinline__ v4f load_elements(const ExprArgs& g, const DevInsn& q, const Place<VEC>& at) {
+// Where a lane's 4 H elements of one pass live.  VEC: H 128-bit words 256 words apart (all
+// pointers 16-byte aligned, total and cols multiples of four, fewer than 2^32 words): word index
+// of the first, and for row vectors the word indices within the row, stepped from pass to pass
+// without a division.  Otherwise: elements 256 apart, 32-bit accesses, any shape.
+template <bool VEC, int H>
+struct Place {
+    size_t first;            // VEC: word index of word 0; else: element index of element 0
+    unsigned col[H];         // VEC: word index within the row of each word; else unused
+};
+
+template <bool VEC, int H>
+__device__ __forceinline__ Vals<H> load_elements(const ExprArgs& g, const DevInsn& q, const Place<VEC, H>& at) {
     const float* __restrict__ src = g.in[q.a];
     const bool row = (q.op == CTAMD_EX_LOAD_ROW);
-    v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+    Vals<H> v;
+#pragma unroll
+    for (int h = 0; h < H; ++h) v.h[h] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
     if (VEC) {
         // a full tensor is touched once (streaming hint); a row vector is re-read by every row and stays cached
-        if (at.first < g.total / 4)
-            v = row ? reinterpret_cast<const v4f*>(src)[at.col] : __builtin_nontemporal_load(reinterpret_cast<const v4f*>(src) + at.first);
+#pragma unroll
+        for (int h = 0; h < H; ++h) {
+            const size_t w = at.first + size_t(h) * kExprThreads;
+            if (w < g.total / 4)
+                v.h[h] = row ? reinterpret_cast<const v4f*>(src)[at.col[h]] : __builtin_nontemporal_load(reinterpret_cast<const v4f*>(src) + w);
+        }
     } else {
 #pragma unroll
-        for (int e = 0; e < kPerLane; ++e) {
+        for (int e = 0; e < 4 * H; ++e) {
             size_t i = at.first + size_t(e) * kExprThreads;
-            if (i < g.total) v[e] = src[row ? i % g.cols : i];
+            if (i < g.total) v.h[e / 4][e % 4] = src[row ? i % g.cols : i];
         }
     }
     return v;
 }
 
-template <bool VEC>
-__global__ __launch_bounds__(kExprThreads) void expr_kernel(ExprArgs g) {
-    extern __shared__ v4f slots[];            // [slots used][kExprThreads]: the four elements of a lane are one word
+template <bool VEC, bool FASTM, int H>
+__global__ __launch_bounds__(kExprThreads, FASTM ? 4 : 3) void expr_kernel(ExprArgs g) {
+    constexpr int N = 4 * H;                  // elements per lane and pass
+    extern __shared__ v4f slots[];            // [places used][H][kExprThreads] 128-bit words
     __shared__ uint64_t s_exp2[32];
     __shared__ uint32_t s_pio4[24];
     stage_tables(s_exp2, s_pio4);
     const Tables tabs{s_exp2, s_pio4};
     const unsigned tid = threadIdx.x;
-    const size_t per_pass = size_t(kExprThreads) * kPerLane;
+    v4f* const lane = slots + tid;
+    // a place is given in 128-bit words of a one-word-per-lane layout; H words per lane scale it
+    auto get = [&](unsigned place) {
+        Vals<H> v;
+#pragma unroll
+        for (int h = 0; h < H; ++h) v.h[h] = lane[place * H + unsigned(h) * kExprThreads];
+        return v;
+    };
+    auto put = [&](unsigned place, const Vals<H>& v) {
+#pragma unroll
+        for (int h = 0; h < H; ++h) lane[place * H + unsigned(h) * kExprThreads] = v.h[h];
+    };
+    const size_t per_pass = size_t(kExprThreads) * N;
+    const size_t words_per_pass = size_t(kExprThreads) * H;
     const size_t passes = (g.total + per_pass - 1) / per_pass;
 
-    Place<VEC> next;                           // of the pass whose head loads are issued next
-    next.first = VEC ? size_t(blockIdx.x) * kExprThreads + tid : size_t(blockIdx.x) * per_pass + tid;
+    Place<VEC, H> next;                        // of the pass whose head loads are issued next
+    next.first = VEC ? size_t(blockIdx.x) * words_per_pass + tid : size_t(blockIdx.x) * per_pass + tid;
     const unsigned cols4 = g.cols / 4;
-    next.col = (VEC && g.has_row) ? unsigned(next.first % cols4) : 0u;
-    const unsigned col_step = (VEC && g.has_row) ? unsigned((size_t(gridDim.x) * kExprThreads) % cols4) : 0u;
-    auto advance = [&](Place<VEC>& p) {
-        p.first += VEC ? size_t(gridDim.x) * kExprThreads : size_t(gridDim.x) * per_pass;
-        if (VEC) {
-            p.col += col_step;
-            if (p.col >= cols4) p.col -= cols4;
+    const bool rows_used = VEC && g.has_row;
+    const unsigned half_step = rows_used ? unsigned(kExprThreads % cols4) : 0u;
+    const unsigned col_step = rows_used ? unsigned((size_t(gridDim.x) * words_per_pass) % cols4) : 0u;
+    next.col[0] = rows_used ? unsigned(next.first % cols4) : 0u;
+#pragma unroll
+    for (int h = 1; h < H; ++h) {
+        next.col[h] = next.col[h - 1] + half_step;
+        if (rows_used && next.col[h] >= cols4) next.col[h] -= cols4;
+    }
+    auto advance = [&](Place<VEC, H>& p) {
+        p.first += VEC ? size_t(gridDim.x) * words_per_pass : size_t(gridDim.x) * per_pass;
+        if (rows_used) {
+#pragma unroll
+            for (int h = 0; h < H; ++h) {
+                p.col[h] += col_step;
+                if (p.col[h] >= cols4) p.col[h] -= cols4;
+            }
         }
     };
     // The loads at the head of the program run one pass ahead, in registers: all of them go out
     // together, and they are in flight while the previous pass is being computed.
-    v4f pre[kLeadLoads];
+    Vals<H> pre[kLeadLoads];
     auto issue_lead = [&]() {
 #pragma unroll
         for (int k = 0; k < kLeadLoads; ++k)
-            if (k < g.n_lead) pre[k] = load_elements<VEC>(g, g.prog[k], next);
+            if (k < g.n_lead) pre[k] = load_elements<VEC, H>(g, g.prog[k], next);
     };
     // The stores at the end of the program go out one pass late, just before the next loads: the
     // memory counter of this hardware counts loads and stores in one order, so waiting for a
     // pass's loads would otherwise also wait for the stores of the pass before.
-    v4f post[kTailStores];
+    Vals<H> post[kTailStores];
     size_t post_at = 0;
-    bool post_full = false;
+    bool post_full[H] = {};
     auto issue_tail = [&]() {
-        if (VEC && post_full) {
+        if (VEC) {
 #pragma unroll
             for (int k = 0; k < kTailStores; ++k)
-                if (k < g.n_tail)
-                    __builtin_nontemporal_store(post[k], reinterpret_cast<v4f*>(g.out[g.prog[g.n_insn - g.n_tail + k].dst]) + post_at);
+                if (k < g.n_tail) {
+                    v4f* __restrict__ dst = reinterpret_cast<v4f*>(g.out[g.prog[g.n_insn - g.n_tail + k].dst]) + post_at;
+#pragma unroll
+                    for (int h = 0; h < H; ++h)
+                        if (post_full[h]) __builtin_nontemporal_store(post[k].h[h], dst + h * kExprThreads);
+                }
         }
     };
+    auto zero_plus = [](Vals<H>& v) {
+#pragma unroll
+        for (int h = 0; h < H; ++h)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v.h[h][e] = 0.0f + v.h[h][e];
+    };
     const int n_body = g.n_insn - (VEC ? g.n_tail : 0);
+    Vals<H> carry;                             // the latest result
+#pragma unroll
+    for (int h = 0; h < H; ++h) carry.h[h] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
     if (blockIdx.x < passes) issue_lead();
     for (size_t pass = blockIdx.x; pass < passes; pass += gridDim.x) {
-        const Place<VEC> at = next;
+        const Place<VEC, H> at = next;
         // one wait for this pass's loads on every path (vmcnt(0); 0x0F70 leaves the other counters
         // alone): with the waits only inside the conditional copies below, the compiler would
         // have to assume loads still in flight later on and wait again after the stores
         __builtin_amdgcn_s_waitcnt(0x0F70);
 #pragma unroll
         for (int k = 0; k < kLeadLoads; ++k)
-            if (k < g.n_lead) slots[unsigned(g.prog[k].dst) * kExprThreads + tid] = pre[k];
+            if (k < g.n_lead) put(g.prog[k].dst, pre[k]);
         advance(next);
         issue_tail();
         if (pass + gridDim.x < passes) issue_lead();
-        const bool inside = VEC ? (at.first < g.total / 4) : true;
+        bool inside[H];
+#pragma unroll
+        for (int h = 0; h < H; ++h) inside[h] = VEC ? (at.first + size_t(h) * kExprThreads < g.total / 4) : true;
+        DevInsn fetched = g.prog[g.n_lead];    // instructions are fetched one ahead of their execution (the array has a spare entry)
         for (int pc = g.n_lead; pc < n_body; ++pc) {
-            const DevInsn q = g.prog[pc];
-            v4f* __restrict__ d = slots + unsigned(q.dst) * kExprThreads + tid;
-            const v4f* __restrict__ pa = slots + unsigned(q.a) * kExprThreads + tid;
-            const v4f* __restrict__ pb = slots + unsigned(q.b) * kExprThreads + tid;
+            const DevInsn q = fetched;
+            fetched = g.prog[pc + 1];
             if (q.op == CTAMD_EX_LOAD_FULL || q.op == CTAMD_EX_LOAD_ROW) {
-                *d = load_elements<VEC>(g, q, at);
+                carry = load_elements<VEC, H>(g, q, at);
             } else if (q.op == CTAMD_EX_STORE || q.op == CTAMD_EX_STORE_ZP) {
                 float* __restrict__ dst = g.out[q.dst];
-                v4f v = *pa;
-                if (q.op == CTAMD_EX_STORE_ZP) {
-#pragma unroll
-                    for (int e = 0; e < kPerLane; ++e) v[e] = 0.0f + v[e];
-                }
+                Vals<H> v = carry;
+                if (q.flags & kAFetch) v = get(q.a);
+                if (q.op == CTAMD_EX_STORE_ZP) zero_plus(v);
                 if (VEC) {
-                    if (inside) __builtin_nontemporal_store(v, reinterpret_cast<v4f*>(dst) + at.first);
+#pragma unroll
+                    for (int h = 0; h < H; ++h)
+                        if (inside[h]) __builtin_nontemporal_store(v.h[h], reinterpret_cast<v4f*>(dst) + at.first + h * kExprThreads);
                 } else {
 #pragma unroll
-                    for (int e = 0; e < kPerLane; ++e) {
+                    for (int e = 0; e < N; ++e) {
                         size_t i = at.first + size_t(e) * kExprThreads;
-                        if (i < g.total) dst[i] = v[e];
+                        if (i < g.total) dst[i] = v.h[e / 4][e % 4];
                     }
                 }
+                continue;
             } else if (q.op == CTAMD_EX_DIVCHK) {
                 // the tape refuses to differentiate a division whose divisor has an element with
                 // |b| < FLT_EPSILON (the reference: src/AutoDiff.cpp:1267-1284); reported through status
                 bool bad = false;
-                const v4f v = *pa;
+                Vals<H> v = carry;
+                if (q.flags & kAFetch) v = get(q.a);
 #pragma unroll
-                for (int e = 0; e < kPerLane; ++e) {
-                    const bool live = VEC ? inside : (at.first + size_t(e) * kExprThreads < g.total);
-                    if (live) bad = bad || (fabsf(v[e]) < FLT_EPSILON);
+                for (int e = 0; e < N; ++e) {
+                    const bool live = VEC ? inside[e / 4] : (at.first + size_t(e) * kExprThreads < g.total);
+                    if (live) bad = bad || (fabsf(v.h[e / 4][e % 4]) < FLT_EPSILON);
                 }
                 if (bad) atomicOr(g.status, 1);
+                continue;
             } else {
                 // lanes past the end compute on the zeros their loads gave them and store nothing
-                const v4f va = *pa, vb = *pb;
-                float a[kPerLane], b[kPerLane], o[kPerLane];
+                if (q.flags & kAFetch) carry = get(q.a);
+                float c[N], b[N];
 #pragma unroll
-                for (int e = 0; e < kPerLane; ++e) {
-                    a[e] = va[e];
-                    b[e] = vb[e];
+                for (int e = 0; e < N; ++e) c[e] = b[e] = carry.h[e / 4][e % 4];   // b = the same value: x * x and the like
+                if (q.flags & kBFetch) {
+                    const Vals<H> vb = get(q.b);
+#pragma unroll
+                    for (int e = 0; e < N; ++e) b[e] = vb.h[e / 4][e % 4];
                 }
-                apply(q, a, b, o, tabs);
-                v4f vo;
+                apply<FASTM, N>(q, c, b, tabs);
 #pragma unroll
-                for (int e = 0; e < kPerLane; ++e) vo[e] = o[e];
-                *d = vo;
+                for (int e = 0; e < N; ++e) carry.h[e / 4][e % 4] = c[e];
             }
+            if (q.flags & kKeep) put(q.dst, carry);
         }
         if (VEC) {
 #pragma unroll
             for (int k = 0; k < kTailStores; ++k)
                 if (k < g.n_tail) {
                     const DevInsn q = g.prog[n_body + k];
-                    v4f v = slots[unsigned(q.a) * kExprThreads + tid];
-                    if (q.op == CTAMD_EX_STORE_ZP) {
-#pragma unroll
-                        for (int e = 0; e < kPerLane; ++e) v[e] = 0.0f + v[e];
-                    }
+                    Vals<H> v = carry;
+                    if (q.flags & kAFetch) v = get(q.a);
+                    if (q.op == CTAMD_EX_STORE_ZP) zero_plus(v);
                     post[k] = v;
                 }
             post_at = at.first;
-            post_full = inside;
+#pragma unroll
+            for (int h = 0; h < H; ++h) post_full[h] = inside[h];
         }
     }
     issue_tail();
@@ -288,14 +373,15 @@ extern "C" int ctamd_expr_run_f32(const ctamd_expr_insn* prog, int n_insn, const
     // every slot must be written before it is read, every port must exist: a bad program must not
     // become a bad access on the device
     bool written[kMaxSlots] = {};
-    int slots_used = 0;
     bool needs_status = false;
     double bytes = 0;
     for (int pc = 0; pc < n_insn; ++pc) {
         const ctamd_expr_insn& q = prog[pc];
         DevInsn& d = g.prog[pc];
-        d.op = q.op; d.dst = q.dst; d.a = q.a; d.b = q.b; d.imm = q.imm;
-        d.rcp = (q.op == CTAMD_EX_DIVS) ? 1.0 / double(q.imm) : 0.0;
+        d.op = q.op; d.flags = 0; d.dst = q.dst; d.a = q.a; d.b = q.b;
+        d.rcp = 0.0;
+        if (q.op == CTAMD_EX_DIVS) d.rcp = 1.0 / double(q.imm);
+        else d.imm = q.imm;
         auto slot_ok = [&](int s) { return s < kMaxSlots && written[s]; };
         switch (q.op) {
             case CTAMD_EX_LOAD_FULL:
@@ -332,7 +418,6 @@ extern "C" int ctamd_expr_run_f32(const ctamd_expr_insn* prog, int n_insn, const
         }
         if (q.op != CTAMD_EX_STORE && q.op != CTAMD_EX_STORE_ZP && q.op != CTAMD_EX_DIVCHK) {
             written[q.dst] = true;
-            if (q.dst + 1 > slots_used) slots_used = q.dst + 1;
         }
     }
     if (needs_status && !status) return fail(CTAMD_EINVAL, "%s: the program checks divisors but status is null", __func__);
@@ -340,7 +425,6 @@ extern "C" int ctamd_expr_run_f32(const ctamd_expr_insn* prog, int n_insn, const
     g.total = total;
     g.cols = unsigned(cols);
     g.n_insn = n_insn;
-    g.vec = vec ? 1 : 0;
     g.has_row = 0;
     for (int pc = 0; pc < n_insn; ++pc) g.has_row |= (prog[pc].op == CTAMD_EX_LOAD_ROW);
     g.n_lead = 0;
@@ -351,35 +435,111 @@ extern "C" int ctamd_expr_run_f32(const ctamd_expr_insn* prog, int n_insn, const
     while (g.n_tail < kTailStores && g.n_lead + g.n_tail < n_insn &&
            (prog[n_insn - 1 - g.n_tail].op == CTAMD_EX_STORE || prog[n_insn - 1 - g.n_tail].op == CTAMD_EX_STORE_ZP))
         ++g.n_tail;
-    if (slots_used < 1) slots_used = 1;
 
-    const size_t lds = size_t(slots_used) * kPerLane * kExprThreads * sizeof(float);
+    // Value numbering.  The kernel keeps the latest result in registers; an operand produced by
+    // the instruction that wrote those registers last is taken from there, every other operand
+    // is fetched from LDS, so only results with such a reader are kept.  The loads at the head run
+    // a pass ahead and are always kept.
+    auto is_load = [](int op) { return op == CTAMD_EX_LOAD_FULL || op == CTAMD_EX_LOAD_ROW; };
+    auto is_sink = [](int op) { return op == CTAMD_EX_STORE || op == CTAMD_EX_STORE_ZP || op == CTAMD_EX_DIVCHK; };
+    auto is_binary = [](int op) { return (op >= CTAMD_EX_ADD && op <= CTAMD_EX_DIV) || op == CTAMD_EX_RELUMUL; };
+    int producer[kMaxSlots];
+    for (int& v : producer) v = -1;
+    int from_a[kMaxInsns], from_b[kMaxInsns], last_fetch[kMaxInsns];
+    bool kept[kMaxInsns];
+    int in_carry = -1;
+    for (int pc = 0; pc < n_insn; ++pc) {
+        const ctamd_expr_insn& q = prog[pc];
+        DevInsn& d = g.prog[pc];
+        from_a[pc] = from_b[pc] = last_fetch[pc] = -1;
+        kept[pc] = pc < g.n_lead;
+        if (!is_load(q.op)) from_a[pc] = producer[q.a];
+        if (is_binary(q.op)) {
+            from_b[pc] = producer[q.b];
+            if (from_a[pc] != in_carry && from_b[pc] == in_carry) {   // only b is in the carry: change places
+                std::swap(from_a[pc], from_b[pc]);
+                if (q.op == CTAMD_EX_SUB) d.op = kRevSub;
+                if (q.op == CTAMD_EX_DIV) d.op = kRevDiv;
+                if (q.op == CTAMD_EX_RELUMUL) d.op = kRevReluMul;
+            }
+        }
+        auto fetch = [&](int from, uint8_t flag) {
+            if (from < 0 || from == in_carry) return;
+            d.flags |= flag;
+            kept[from] = true;
+            last_fetch[from] = pc;
+        };
+        fetch(from_a[pc], kAFetch);
+        fetch(from_b[pc], kBFetch);
+        if (!is_sink(q.op)) {
+            producer[q.dst] = pc;
+            if (pc >= g.n_lead) in_carry = pc;
+        }
+    }
+    // LDS places by liveness: a place is free again after the last instruction that fetches it (the
+    // result of that very instruction may take it: a lane reads its words before it writes them)
+    int place[kMaxInsns];
+    bool busy[kMaxLive] = {};
+    int places_used = 0;
+    for (int pc = 0; pc < n_insn; ++pc) {
+        DevInsn& d = g.prog[pc];
+        const int op = prog[pc].op;
+        if (d.flags & kAFetch) d.a = uint16_t(place[from_a[pc]] * kExprThreads);
+        if (d.flags & kBFetch) d.b = uint16_t(place[from_b[pc]] * kExprThreads);
+        if ((d.flags & kAFetch) && last_fetch[from_a[pc]] == pc) busy[place[from_a[pc]]] = false;
+        if ((d.flags & kBFetch) && last_fetch[from_b[pc]] == pc) busy[place[from_b[pc]]] = false;
+        if (!is_sink(op) && kept[pc]) {
+            int p = 0;
+            while (p < kMaxLive && busy[p]) ++p;
+            if (p == kMaxLive) return fail(CTAMD_ERANGE, "%s: more than %d values are live at instruction %d", __func__, kMaxLive, pc);
+            busy[p] = true;
+            place[pc] = p;
+            if (p + 1 > places_used) places_used = p + 1;
+            d.flags |= kKeep;
+            d.dst = uint16_t(p * kExprThreads);
+        }
+        if (pc == g.n_lead - 1)                 // head loads nobody fetches: written at the start of a pass, free after
+            for (int k = 0; k < g.n_lead; ++k)
+                if (last_fetch[k] < 0) busy[place[k]] = false;
+    }
+    if (places_used < 1) places_used = 1;
+    g.prog[n_insn] = g.prog[n_insn - 1];        // the spare entry: fetched, never run
+    // Two 128-bit words per lane and pass halve the interpretation per element and double what a
+    // wave has in flight; with many values live only one word per lane fits in LDS.
+    const int words = (places_used * 2 > kMaxLive) ? 1 : 2;
+
+    const size_t lds = size_t(places_used) * kWordBytes * words;
+    using Kernel = void (*)(ExprArgs);
+    static const Kernel kernels[2][2][kMaxHalves] = {
+        {{expr_kernel<false, false, 1>, expr_kernel<false, false, 2>}, {expr_kernel<false, true, 1>, expr_kernel<false, true, 2>}},
+        {{expr_kernel<true, false, 1>, expr_kernel<true, false, 2>}, {expr_kernel<true, true, 1>, expr_kernel<true, true, 2>}}};
+    const bool fastm = fast_math();
+    const Kernel kernel = kernels[vec ? 1 : 0][fastm ? 1 : 0][words - 1];
     // more than the default 64 KiB of LDS per block has to be asked for, once per device
     static int lds_raised[kMaxDevices] = {};
     int dev = 0;
     if (lds > (size_t(60) << 10)) {
         if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(CTAMD_EHIP, "%s: no current device", __func__);
         if (!lds_raised[dev]) {
-            const int most = int(size_t(kMaxSlots) * kPerLane * kExprThreads * sizeof(float));
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(expr_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, most);
-            if (e == hipSuccess)
-                e = hipFuncSetAttribute(reinterpret_cast<const void*>(expr_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, most);
-            if (e != hipSuccess) return fail(CTAMD_EHIP, "%s: %d value slots need %zu bytes of LDS: %s", __func__, slots_used, lds,
+            hipError_t e = hipSuccess;
+            for (int i = 0; i < 2 * 2 * kMaxHalves; ++i)
+                if (e == hipSuccess)
+                    e = hipFuncSetAttribute(reinterpret_cast<const void*>((&kernels[0][0][0])[i]), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBudget);
+            if (e != hipSuccess) return fail(CTAMD_EHIP, "%s: %d live values need %zu bytes of LDS: %s", __func__, places_used, lds,
                                              hipGetErrorString(e));
             lds_raised[dev] = 1;
         }
     }
-    const size_t per_pass = size_t(kExprThreads) * kPerLane;
+    const size_t per_pass = size_t(kExprThreads) * 4 * words;
     const size_t passes = (total + per_pass - 1) / per_pass;
-    // as many blocks as stay resident (registers and LDS decide; asked once per slot count): more
-    // would only queue behind them and break the one-pass-ahead loads, fewer leave CUs idle
+    // as many blocks as stay resident (registers and LDS decide; asked once per kernel and LDS
+    // size): more would only queue behind them and break the one-pass-ahead loads, fewer leave CUs idle
     const int cus = compute_units() > 0 ? compute_units() : 256;
-    static int resident[2][kMaxSlots + 1] = {};
-    int& per_cu_cached = resident[vec ? 1 : 0][slots_used];
+    static int resident[2][2][kMaxHalves][kMaxLive + 1] = {};
+    int& per_cu_cached = resident[vec ? 1 : 0][fastm ? 1 : 0][words - 1][places_used];
     if (per_cu_cached == 0) {
         int nb = 0;
-        hipError_t e = vec ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, expr_kernel<true>, kExprThreads, lds)
-                           : hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, expr_kernel<false>, kExprThreads, lds);
+        hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, reinterpret_cast<const void*>(kernel), kExprThreads, lds);
         if (e != hipSuccess || nb < 1) nb = 1;
         per_cu_cached = nb;
     }
@@ -387,7 +547,6 @@ extern "C" int ctamd_expr_run_f32(const ctamd_expr_insn* prog, int n_insn, const
     size_t blocks = size_t(cus) * per_cu;
     if (blocks > passes) blocks = passes;
     account(bytes, 0.0);
-    if (vec) hipLaunchKernelGGL(expr_kernel<true>, dim3(unsigned(blocks)), dim3(kExprThreads), lds, as_stream(stream), g);
-    else hipLaunchKernelGGL(expr_kernel<false>, dim3(unsigned(blocks)), dim3(kExprThreads), lds, as_stream(stream), g);
+    hipLaunchKernelGGL(kernel, dim3(unsigned(blocks)), dim3(kExprThreads), lds, as_stream(stream), g);
     return launched(__func__);
 }

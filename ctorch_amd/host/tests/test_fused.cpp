@@ -9,6 +9,7 @@
 #include "Ctorch_Error.h"
 #include "Expr.h"
 #include "check.h"
+#include "ctorch_amd.h"
 
 static bool same_bits(const Tensor& a, const Tensor& b) {
     std::vector<float> x = a.to_vector(), y = b.to_vector();
@@ -83,6 +84,28 @@ static void expression_chain() {
     }
 }
 
+// In the library's default mode the fused program evaluates sigmoid / tanh / sin / cos in single
+// precision (a few ulp from the operator-by-operator kernels, which return glibc's floats in both
+// modes): values and gradients agree to rounding, not to the bit.
+static void expression_chain_single_precision() {
+    const int before = ctamd_set_math_mode(CTAMD_MATH_FAST);
+    Tensor X = device_tensor({6, 8}, ramp(48, 2.0f, 0.2f));
+    Tensor T = device_tensor({6, 8}, ramp(48, 1.0f, 0.9f));
+    std::vector<float> rv = ramp(8, 0.5f, 0.4f);
+    for (float& v : rv) v = std::fabs(v) + 0.5f;
+    Tensor r = device_tensor({8}, rv);
+    auto plain = run([&] { return (X / r).sigmoid() - X.tanh() * X.sin() + (-X).cos() * T + 0.25f; }, {&X, &r, &T}, BroadcastGrad::kColumnSum);
+    auto fused = run([&] {
+        Expr x(X), t(T);
+        return (sigmoid(x / Expr(r)) - tanh(x) * sin(x) + cos(-x) * t + 0.25f).eval();
+    }, {&X, &r, &T}, BroadcastGrad::kColumnSum);
+    CHECK(all_close(fused[0], plain[0].to_vector(), 1e-6f), "fused chain, single-precision mode: value");
+    CHECK(all_close(fused[1], plain[1].to_vector(), 2e-6f) && all_close(fused[3], plain[3].to_vector(), 1e-6f),
+          "fused chain, single-precision mode: gradients of the full operands");
+    CHECK(all_close(fused[2], plain[2].to_vector(), 1e-5f), "fused chain, single-precision mode: row-vector gradient");
+    ctamd_set_math_mode(before);
+}
+
 static void same_operand_twice() {
     // x - x and x / x: the reference's tape counts both visits as the first operand (2g and 2g/x)
     Tensor X = device_tensor({4, 4}, ramp(16, 1.0f, 0.3f));
@@ -145,8 +168,10 @@ static void host_and_errors() {
 
 int main() {
     Ctorch_Error::setPrintLevel(PrintLevel::MINIUM);
+    ctamd_set_math_mode(CTAMD_MATH_EXACT);   // the bit-for-bit comparisons below hold in this mode
     linear_layer();
     expression_chain();
+    expression_chain_single_precision();
     same_operand_twice();
     one_dimensional_and_small();
     host_and_errors();

@@ -33,3 +33,13 @@ def golden():
     def load(name):
         return np.load(os.path.join(GOLDEN_DIR, name + ".npz"), allow_pickle=False)
     return load
+
+
+@pytest.fixture
+def exact_math():
+    """The library's exact mode (glibc's floats bit for bit, exactly rounded quotients) for one test;
+    the default single-precision mode is restored afterwards."""
+    import gpu_support as G
+    prev = G.set_math_mode(G.MATH_EXACT)
+    yield
+    G.set_math_mode(prev)

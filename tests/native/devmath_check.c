@@ -1,7 +1,8 @@
 /* Host check of ctorch_amd/csrc/devmath.h against the installed glibc: counts the floats for
  * which the device algorithms (compiled here for the CPU, unchanged) return different bits from
  * expf / sinf / cosf / logf, and the worst distance of the tangent from glibc's tanf (not the same
- * algorithm: at most 1 ulp).  Usage: devmath_check STRIDE  (1 = every one of the 2^32 bit patterns).
+ * algorithm: at most 1 ulp) and of the single-precision sine / cosine pair from sinf / cosf (at most 2
+ * ulp, |x| < 120).  Usage: devmath_check STRIDE  (1 = every one of the 2^32 bit patterns).
  * Prints one line per function: name, inputs tested, mismatches, worst ulp distance
  * (expf_pair: exp(x) and exp(-x) from the shared reduction, against expf(x) and expf(-x)). */
 #include <math.h>
@@ -26,9 +27,9 @@ static int differs(float a, float b, int64_t* ulp) {
 int main(int argc, char** argv) {
     uint64_t stride = argc > 1 ? strtoull(argv[1], 0, 10) : 1;
     if (stride == 0) stride = 1;
-    uint64_t n = 0, bad[6] = {0, 0, 0, 0, 0, 0}, covered[6] = {0, 0, 0, 0, 0, 0};
-    int64_t worst[6] = {0, 0, 0, 0, 0, 0};
-#pragma omp parallel for reduction(+ : n, bad[:6], covered[:6]) reduction(max : worst[:6]) schedule(static)
+    uint64_t n = 0, bad[8] = {0, 0, 0, 0, 0, 0, 0, 0}, covered[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    int64_t worst[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma omp parallel for reduction(+ : n, bad[:8], covered[:8]) reduction(max : worst[:8]) schedule(static)
     for (uint64_t u = 0; u < (1ULL << 32); u += stride) {
         float x = cta_u2f((uint32_t)u);
         int64_t d = 0;
@@ -69,9 +70,21 @@ int main(int argc, char** argv) {
             if (d > 1) ++bad[5];                   /* a different algorithm: 1 ulp apart is expected */
             if (d > worst[5]) worst[5] = d;
         }
+        if (!cta_sincos_is_rare(x)) {               /* the single-precision pair: |x| < 120, at most 2 ulp */
+            ++covered[6];
+            if (differs(cta_sincosf_f32(x, 0), sinf(x), &d)) {
+                if (d > 2) ++bad[6];
+                if (d > worst[6]) worst[6] = d;
+            }
+            ++covered[7];
+            if (differs(cta_sincosf_f32(x, 1), cosf(x), &d)) {
+                if (d > 2) ++bad[7];
+                if (d > worst[7]) worst[7] = d;
+            }
+        }
     }
-    const char* names[6] = {"expf", "sinf", "cosf", "expf_pair", "logf", "tanf(>1ulp)"};
-    for (int k = 0; k < 6; ++k)
+    const char* names[8] = {"expf", "sinf", "cosf", "expf_pair", "logf", "tanf(>1ulp)", "sinf_f32(>2ulp)", "cosf_f32(>2ulp)"};
+    for (int k = 0; k < 8; ++k)
         printf("%s tested %llu mismatches %llu worst_ulp %lld\n", names[k], (unsigned long long)covered[k],
                (unsigned long long)bad[k], (long long)worst[k]);
     return 0;

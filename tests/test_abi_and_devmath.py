@@ -63,8 +63,9 @@ def test_missing_library_fails_loudly(tmp_path, monkeypatch):
 
 
 def test_device_math_matches_glibc_on_a_strided_sweep(tmp_path):
-    """Every 251st float (17 million inputs, all exponents): expf, sinf, cosf of
-    ctorch_amd/csrc/devmath.h against the installed glibc.  Run with stride 1 for all 2^32."""
+    """Every 251st float (17 million inputs, all exponents): expf, sinf, cosf, logf of
+    ctorch_amd/csrc/devmath.h against the installed glibc (no mismatch), tanf within 1 ulp, the
+    single-precision sine / cosine within 2 ulp.  Run with stride 1 for all 2^32."""
     exe = str(tmp_path / "devmath_check")
     subprocess.check_call(["gcc", "-O2", "-fopenmp", "-ffp-contract=off", "-mfma", "-o", exe,
                            os.path.join(ROOT, "tests", "native", "devmath_check.c"), "-lm"])
@@ -72,7 +73,8 @@ def test_device_math_matches_glibc_on_a_strided_sweep(tmp_path):
     print(out)
     for line in out.strip().splitlines():
         f = line.split()
-        assert int(f[2]) > 17_000_000 and int(f[4]) == 0, line
+        # (the single-precision sine / cosine pair is defined for |x| < 120 only: about half of all floats)
+        assert int(f[2]) > (8_000_000 if "_f32" in f[0] else 17_000_000) and int(f[4]) == 0, line
 
 
 def test_division_through_a_double_reciprocal_is_ieee_division(tmp_path):

@@ -11,6 +11,18 @@ pytestmark = pytest.mark.gpu
 F = np.float32
 
 
+@pytest.fixture(autouse=True)
+def _exact_unless_asked(request):
+    """The bit-for-bit comparisons below hold in the library's exact mode; tests named *fast_mode* run in
+    the default single-precision one."""
+    if "fast_mode" in request.node.name:
+        yield
+        return
+    prev = G.set_math_mode(G.MATH_EXACT)
+    yield
+    G.set_math_mode(prev)
+
+
 def same_bits_or_both_nan(a, b):
     """Bit equality, except that where both are NaN any NaN will do (x86 and the GPU give the
     invalid-operation NaN opposite signs)."""
@@ -102,3 +114,51 @@ def test_malformed_programs_are_refused(oracle):
     G.expr_run([(E["LOAD_FULL"], 0, 0, 0, 0.0)] * 161, [x], 1, 4, 8, expect=-5)   # too long
     outs, _ = G.expr_run([], [x], 1, 4, 8)                                        # empty: nothing happens
     assert not G.host(outs[0]).any()
+
+
+def test_fast_mode_transcendentals_within_2_ulp_of_the_oracle(oracle):
+    """The default mode evaluates the transcendental operators in single precision: sin / cos within
+    2 ulp of the oracle's glibc calls over a sweep of the argument range (histograms printed); sigmoid,
+    the reference's formula on an exponential within 1 ulp and a reciprocal within 1 ulp, within 4 ulp
+    of the oracle's; tanh - the reference's (e^x - e^-x) / (e^x + e^-x) loses its digits near zero, as
+    does the 1 - 2 / (e^2|x| + 1) used here - within 2 ulp for |x| >= 1 and 2.5e-7 absolute below."""
+    print("case expr fast mode ulp", flush=True)
+    assert G.lib().ctamd_math_mode() == G.MATH_FAST
+    E = EX
+    from support import ulp_diff
+    u = np.arange(0, 1 << 32, 4099, dtype=np.uint64).astype(np.uint32).view(F)
+    x = u[np.isfinite(u)]
+    x = np.concatenate([x[np.abs(x) < 200.0], oracle.uniform((200000,), 7, -120, 120), oracle.normal((200000,), 8, 0, 2)])
+    x = x[: (x.size // 1024) * 1024].reshape(-1, 1024)
+    prog = [(E["LOAD_FULL"], 0, 0, 0, 0.0)]
+    for k, op in enumerate(("SIN", "COS", "SIGMOID", "TANH")):
+        prog += [(E[op], 1, 0, 0, 0.0), (E["STORE"], k, 1, 0, 0.0)]
+    got, _ = G.expr_run(prog, [G.dev(x)], 4, x.shape[0], x.shape[1])
+    want, _ = oracle.expr_run(prog, [x], 4, x.shape[0], x.shape[1])
+    for k, name in enumerate(("sin", "cos", "sigmoid", "tanh")):
+        g, w = G.host(got[k]).reshape(-1), want[k].reshape(-1)
+        ok = np.isfinite(w) & (np.abs(w) >= F(2.0 ** -126))
+        if name == "tanh":
+            big = ok & (np.abs(x.reshape(-1)) >= 1.0)
+            d = ulp_diff(g[big], w[big])
+            small = np.isfinite(w) & ~big
+            print(f"  tanh: |x| >= 1 ulp histogram { {int(v): int((d == v).sum()) for v in np.unique(d)} }; below: max abs error {np.abs(g[small] - w[small]).max():.2e}")
+            assert d.max() <= 2 and np.abs(g[small] - w[small]).max() <= 2.5e-7
+        else:
+            d = ulp_diff(g[ok], w[ok])
+            print(f"  {name}: ulp histogram { {int(v): int((d == v).sum()) for v in np.unique(d)} }")
+            # 1 / (1 + e): the sum is rounded where floats are up to four times as far apart as at
+            # the quotient, so one ulp of the exponential can move the result by four
+            assert d.max() <= (4 if name == "sigmoid" else 2), name
+        assert np.array_equal(np.isnan(g), np.isnan(w)), name
+
+
+@pytest.mark.parametrize("rows,cols", [(64, 256), (33, 100)])
+def test_fast_mode_config5_expression_against_the_oracle(oracle, rows, cols):
+    print("case expr config5 fast mode", rows, cols, flush=True)
+    X = oracle.uniform((rows, cols), 501, -2, 2)
+    r = oracle.uniform((cols,), 502, 0.5, 2)
+    (Y,), _ = G.expr_run(config5_program(), [G.dev(X), G.dev(r)], 1, rows, cols)
+    (cpu,), _ = oracle.expr_run(config5_program(), [X, r], 1, rows, cols)
+    # three terms of size <= 1 each, every one within 2 ulp (2.5e-7 absolute for the tanh factor)
+    assert np.abs(G.host(Y) - cpu).max() <= 8e-7

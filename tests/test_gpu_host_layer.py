@@ -279,7 +279,7 @@ def test_tape_programs_against_the_reference_vectors(oracle, host, golden):
             assert np.abs(got - want).max() <= 2e-5 * (1 + np.abs(want).max()), seed
 
 
-def test_fused_expressions_against_the_reference_vectors(oracle, host, golden):
+def test_fused_expressions_against_the_reference_vectors(oracle, host, golden, exact_math):
     """The same random programs with every chain of elementwise operators built as ONE fused
     expression (one launch forward, one launch for all gradients): in the reference's gradient mode
     the result and every gradient must still have the reference's bits; in the default mode the
@@ -379,7 +379,7 @@ def test_tensors_that_are_not_fp32(oracle, host, golden):
     assert host.typed(x, 2, [(2, 0.5)])[0] == -1
 
 
-def test_fused_expression_in_a_recorded_step(oracle, host):
+def test_fused_expression_in_a_recorded_step(oracle, host, exact_math):
     """A fused expression, its losses and its backward recorded into a HIP graph: the first replay
     reproduces the eager step bit for bit, a replay after the staged input was overwritten equals
     the eager step on the new input."""
@@ -402,7 +402,7 @@ def test_fused_expression_in_a_recorded_step(oracle, host):
     assert not same_bits(y1, y2)
 
 
-def test_fused_against_unfused_on_more_programs(oracle, host):
+def test_fused_against_unfused_on_more_programs(oracle, host, exact_math):
     """A hundred further random programs (longer, more inputs, shapes with rows that are not a
     multiple of four elements, so the 32-bit access path runs too, and a tensor large enough for
     several passes per block): the fused expression against the operator-by-operator tape on the
