@@ -3,17 +3,19 @@
 // once, every output written once, intermediates never leave the chip.  The front-end compiles
 // both an expression's forward values and its tape gradients into such programs, so a chain like
 // Y = sigmoid(X / r) - tanh(X) * sin(X) + cos(-X) is one launch forward and one launch backward
-// instead of nine and about fifteen, with the bits of the operator-by-operator evaluation.
+// instead of nine and about fifteen, with the bits of the operator-by-operator evaluation in the
+// exact math mode (a few ulp from them in the single-precision one).
 //
 // The kernel is an interpreter: the program sits in the kernel arguments (uniform, read through
-// the scalar unit), so every instruction is a scalar branch to one functor's code, applied to the
-// four elements each lane owns.  Values live in LDS "slots": the four elements of lane t in slot s
-// are the 128-bit word slots[s * 256 + t] - one LDS instruction per operand, consecutive lanes on
-// consecutive words, no conflicts.  An instruction costs two 128-bit LDS reads and one write next
-// to its arithmetic and about twenty scalar / address instructions of interpretation; for the
-// transcendental operators that is noise, a chain of cheap operators pays it in full and still
-// moves its bytes once instead of once per operator.  (Registers cannot hold the slots: the slot
-// number is data.)
+// the scalar unit, one instruction ahead of its execution), so every instruction is a scalar branch
+// to one functor's code, applied to the eight elements each lane owns (two 128-bit words; four
+// where a program has too many values live for LDS).  The latest result stays in registers and the
+// next instruction takes it from there; only a value that a later instruction needs goes to an LDS
+// place - word t of place p belongs to lane t, consecutive lanes on consecutive words, no
+// conflicts - and places are reused as values die.  A chain of cheap operators still pays about
+// thirty scalar instructions of interpretation per operator, shared by eight elements; for the
+// transcendental operators that is noise, and their arithmetic - not memory - bounds the kernel.
+// (Registers cannot hold the places: the place number is data.)
 #include "common.h"
 #include "devmath.h"
 #include "functors.h"

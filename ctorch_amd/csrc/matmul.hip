@@ -13,10 +13,12 @@
 // global -> register -> LDS staging is double buffered so the loads of tile t+1 are in flight while
 // tile t is multiplied, with one barrier per k tile.  Blocks are renumbered so that each XCD (blocks are
 // dealt round-robin to the 8 XCDs) works on a compact band of C and re-uses its operand tiles
-// from its own L2.  Skinny outputs with a long K (the weight gradients of a small layer) are
-// split along K over blockIdx.z; partial products go to the device scratch and are folded in a
-// fixed order, so results stay deterministic.
+// from its own L2.  The tiles of the last, partly filled round of blocks - all tiles of a skinny
+// output with a long K (the weight gradients of a small layer) - are cut along K into parts, one
+// block each, so that they fill the chip; the parts go to the device scratch and a second launch
+// adds them in a fixed order, so results stay deterministic.
 #include "common.h"
+
 
 namespace ctamd {
 namespace {
@@ -135,13 +137,19 @@ __device__ __forceinline__ void fetch(const float* __restrict__ lds, int stride,
 struct GemmArgs {
     const float* a; int64_t lda;
     const float* b; int64_t ldb;
-    float* c; int64_t ldc;          // C, or the partial buffer when split along K
+    float* c; int64_t ldc;          // C
     int m, n, k;
-    int k_per_split;                // multiple of BK
-    int64_t split_stride;           // elements between partial buffers (0 when not split)
     int tiles_m, tiles_n;
+    // Tiles [0, whole_tiles) are computed by one block each over all of K.  The remaining tiles - the
+    // last, partly filled round of blocks - are cut along K into `splits` parts of k_per_split, one
+    // block each: block whole_tiles + (t - whole_tiles) * splits + z computes part z of tile t.
+    int whole_tiles;
+    int splits;
+    int k_per_split;                // multiple of BK
+    float* partial;                 // [split tiles][splits][BM][BN]
+    int c_vec;                      // rows of C are 16-byte aligned
     const float* bias;              // optional row vector [n] added to every row of C (null: none)
-    int relu;                       // then max(0, .) when set; both only when not split along K
+    int relu;                       // then max(0, .) when set
 };
 
 // Output epilogue of a product that is not split along K: bias add, then ReLU as `v > 0 ? v : +0`
@@ -166,13 +174,17 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
     // XCD-aware renumbering: hardware block b runs on XCD b % 8; give each XCD a contiguous run of
     // tiles, and inside the run walk C in column-major bands of 8 tile rows so that co-resident
     // blocks share A row bands and B column bands in that XCD's L2.
-    const int tiles = g.tiles_m * g.tiles_n;
-    int bid = blockIdx.x;
-    {
-        int per = tiles / kXcds, rem = tiles % kXcds;
+    int bid = blockIdx.x, part = 0;
+    const bool split = bid >= g.whole_tiles;
+    if (!split) {
+        int per = g.whole_tiles / kXcds, rem = g.whole_tiles % kXcds;
         int xcd = bid % kXcds, local = bid / kXcds;
         // XCDs with index < rem own per+1 tiles
         bid = xcd * per + (xcd < rem ? xcd : rem) + local;
+    } else {
+        const int r = bid - g.whole_tiles;
+        bid = g.whole_tiles + r / g.splits;
+        part = r % g.splits;
     }
     constexpr int BAND = 8;
     int band = bid / (BAND * g.tiles_n);
@@ -182,10 +194,9 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
     const int tile_n = in_band / band_rows;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
-    const int k_begin = blockIdx.z * g.k_per_split;
-    int k_end = k_begin + g.k_per_split;
+    const int k_begin = split ? part * g.k_per_split : 0;
+    int k_end = split ? k_begin + g.k_per_split : g.k;
     if (k_end > g.k) k_end = g.k;
-    float* __restrict__ cout = g.c + int64_t(blockIdx.z) * g.split_stride;
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm = (wave / C::WAVES_N) * C::WM, wn = (wave % C::WAVES_N) * C::WN;
@@ -348,49 +359,78 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
     }
 
     // accumulator register r of lane l holds C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 tile
+    if (!split) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int col = n0 + wn + j * 32 + l32;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int row = m0 + wm + i * 32 + 8 * (r / 4) + 4 * half + (r % 4);
+                    if (row < g.m && col < g.n) g.c[int64_t(row) * g.ldc + col] = epilogue(acc[i][j][r], g.bias, col, g.relu);
+                }
+            }
+        return;
+    }
+    // A part of a split tile: the partial product goes to this part's [BM][BN] buffer (whole, the
+    // rows and columns past the edge of C are zeros); fold_parts adds the parts up.
+    const int split_tile = bid - g.whole_tiles;
+    float* __restrict__ mine = g.partial + (size_t(split_tile) * g.splits + part) * (BM * BN);
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            const int col = n0 + wn + j * 32 + l32;
+            const int col = wn + j * 32 + l32;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int row = m0 + wm + i * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-                if (row < g.m && col < g.n) cout[int64_t(row) * g.ldc + col] = epilogue(acc[i][j][r], g.bias, col, g.relu);
+                const int row = wm + i * 32 + 8 * (r / 4) + 4 * half + (r % 4);
+                mine[row * BN + col] = acc[i][j][r];
             }
         }
 }
 
-// Folds the K-split partial products: c[i] = sum_z partial[z][i], in order of z.
-// Then the optional bias add and ReLU of the fused product (n = row length of C).
-template <bool VEC>
-__global__ __launch_bounds__(kThreads) void splitk_fold(const float* __restrict__ partial, float* __restrict__ c,
-                                                        size_t mn, int splits, const float* __restrict__ bias, int n,
-                                                        int relu) {
-    size_t i = size_t(blockIdx.x) * kThreads + threadIdx.x;
-    if (VEC) {
-        if (i >= mn / 4) return;
-        const v4f* __restrict__ p = reinterpret_cast<const v4f*>(partial);
-        const size_t stride = mn / 4;
-        v4f t = p[i];
+// Adds the parts of the split tiles in their order and writes C (bias and ReLU of the fused
+// product included): blockIdx.x is the split tile, blockIdx.y one of its slices of kFoldSlice elements.
+constexpr int kFoldSlice = kThreads * 4 * 2;
+template <int BM, int BN>
+__global__ __launch_bounds__(kThreads) void fold_parts(GemmArgs g) {
+    static_assert(BM * BN % kFoldSlice == 0, "a tile is a whole number of slices");
+    const int split_tile = blockIdx.x;
+    const int bid = g.whole_tiles + split_tile;
+    constexpr int BAND = 8;
+    const int band = bid / (BAND * g.tiles_n);
+    const int band_rows = g.tiles_m - band * BAND < BAND ? g.tiles_m - band * BAND : BAND;
+    const int in_band = bid - band * BAND * g.tiles_n;
+    const int m0 = (band * BAND + in_band % band_rows) * BM, n0 = (in_band / band_rows) * BN;
+    const float* __restrict__ parts = g.partial + size_t(split_tile) * g.splits * (BM * BN);
+    const int first = blockIdx.y * (kFoldSlice / 4);
+    for (int idx = first + threadIdx.x; idx < first + kFoldSlice / 4; idx += kThreads) {
+        const int row = idx / (BN / 4), col = (idx % (BN / 4)) * 4;
+        const int grow = m0 + row, gcol = n0 + col;
+        if (grow >= g.m || gcol >= g.n) continue;
+        v4f t = *reinterpret_cast<const v4f*>(parts + row * BN + col);
         int z = 1;
-        for (; z + 3 < splits; z += 4) {       // four loads in flight, added in order of z
-            v4f a = p[size_t(z) * stride + i], b = p[size_t(z + 1) * stride + i];
-            v4f d = p[size_t(z + 2) * stride + i], e = p[size_t(z + 3) * stride + i];
-            t = ((t + a) + b) + d;
-            t = t + e;
+        for (; z + 3 < g.splits; z += 4) {     // four loads in flight, added in order of z
+            const v4f p0 = *reinterpret_cast<const v4f*>(parts + size_t(z) * (BM * BN) + row * BN + col);
+            const v4f p1 = *reinterpret_cast<const v4f*>(parts + size_t(z + 1) * (BM * BN) + row * BN + col);
+            const v4f p2 = *reinterpret_cast<const v4f*>(parts + size_t(z + 2) * (BM * BN) + row * BN + col);
+            const v4f p3 = *reinterpret_cast<const v4f*>(parts + size_t(z + 3) * (BM * BN) + row * BN + col);
+            t = ((t + p0) + p1) + p2;
+            t = t + p3;
         }
-        for (; z < splits; ++z) t = t + p[size_t(z) * stride + i];
-        if (bias || relu) {
+        for (; z < g.splits; ++z) t = t + *reinterpret_cast<const v4f*>(parts + size_t(z) * (BM * BN) + row * BN + col);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) t[e] = epilogue(t[e], bias, int((i * 4 + e) % size_t(n)), relu);
+        for (int e = 0; e < 4; ++e)
+            if (gcol + e < g.n) t[e] = epilogue(t[e], g.bias, gcol + e, g.relu);
+        float* __restrict__ dst = g.c + int64_t(grow) * g.ldc + gcol;
+        if (g.c_vec && gcol + 4 <= g.n) {
+            *reinterpret_cast<v4f*>(dst) = t;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (gcol + e < g.n) dst[e] = t[e];
         }
-        reinterpret_cast<v4f*>(c)[i] = t;
-    } else {
-        if (i >= mn) return;
-        float t = partial[i];
-        for (int z = 1; z < splits; ++z) t += partial[size_t(z) * mn + i];
-        c[i] = epilogue(t, bias, int(i % size_t(n)), relu);
     }
 }
 
@@ -408,35 +448,35 @@ __global__ __launch_bounds__(kThreads) void gemm_strided(const float* __restrict
     c[idx] = epilogue(s, bias, j, relu);
 }
 
-// Three tile shapes; the host picks the largest one that still gives every CU a tile.
+// Four tile shapes; the host picks one, and a cut of the last round of tiles along K, by a model of
+// the time each plan takes (matmul_impl).
 //   Big   256 x 256 x 16, 8 waves of 128 x 64 (128 accumulator registers, two waves per SIMD): the
-//         fewest LDS and global bytes per flop; 4096^3 in 0.95-0.98 ms (140-145 TFLOP/s).
-//   Wide  256 x 128 x 16, 4 waves of 128 x 64, two blocks per CU: 1-5% behind Big per flop, but its
-//         tiles are half as large - 6144^3 (576 Big tiles on 256 CUs: three rounds, the last a
-//         quarter full) in 3.59 ms (129 TFLOP/s) against 4.30 ms with Big tiles.
-//   Small 128 x 128 x 16, 4 waves of 64 x 64: 2048^3 in 0.135 ms (127 TFLOP/s).
-//   Tiny  64 x 64 x 16, 4 waves of 32 x 32, up to 8 blocks per CU: 1024^3 in 27 us (78 TFLOP/s) and
-//         the skinny products of a small layer ([8192 x 784] . [784 x 256] in 32 us); with a K split
-//         when even these tiles are fewer than the CUs ([784 x 8192] . [8192 x 256] in 50 us).
+//         fewest LDS and global bytes per flop; 4096^3 in 0.95 ms (145 TFLOP/s), 8192^3 at 146.
+//   Wide  256 x 128 x 16, 4 waves of 128 x 64, two blocks per CU: 1-5% behind Big per flop.
+//   Small 128 x 128 x 16, 4 waves of 64 x 64, two blocks per CU: 7% behind Big per flop; with the 64
+//         tiles that 3072^3 leaves after one round cut in four along K, 0.43 ms (134 TFLOP/s)
+//         against 0.55 ms uncut.
+//   Tiny  64 x 64 x 16, 4 waves of 32 x 32, up to 4 blocks per CU: 1024^3 in 28 us (76 TFLOP/s) and
+//         the skinny products of a small layer ([8192 x 784] . [784 x 256] in 32 us), cut along K
+//         when the tiles are fewer than the CUs ([784 x 8192] . [8192 x 256] in 43 us).
 using BigTile = Cfg<256, 256, 16, 128, 64>;
 using SmallTile = Cfg<128, 128, 16, 64, 64>;
 using TinyTile = Cfg<64, 64, 16, 32, 32>;
 using WideTile = Cfg<256, 128, 16, 128, 64>;
 
 template <class Tile, bool A_KC, bool B_KC>
-int launch_gemm(GemmArgs g, bool vec, int splits, hipStream_t s) {
-    dim3 grid(unsigned(g.tiles_m * g.tiles_n), 1, unsigned(splits));
-    if (vec) hipLaunchKernelGGL((gemm_kernel<Tile, A_KC, B_KC, true>), grid, dim3(Tile::THREADS), 0, s, g);
-    else hipLaunchKernelGGL((gemm_kernel<Tile, A_KC, B_KC, false>), grid, dim3(Tile::THREADS), 0, s, g);
+int launch_gemm(GemmArgs g, bool vec, int blocks, hipStream_t s) {
+    if (vec) hipLaunchKernelGGL((gemm_kernel<Tile, A_KC, B_KC, true>), dim3(unsigned(blocks)), dim3(Tile::THREADS), 0, s, g);
+    else hipLaunchKernelGGL((gemm_kernel<Tile, A_KC, B_KC, false>), dim3(unsigned(blocks)), dim3(Tile::THREADS), 0, s, g);
     return launched("ctamd_matmul_f32");
 }
 
 template <class Tile>
-int launch_layout(GemmArgs g, bool a_kc, bool b_kc, bool vec, int splits, hipStream_t s) {
-    if (a_kc && b_kc) return launch_gemm<Tile, true, true>(g, vec, splits, s);
-    if (a_kc) return launch_gemm<Tile, true, false>(g, vec, splits, s);
-    if (b_kc) return launch_gemm<Tile, false, true>(g, vec, splits, s);
-    return launch_gemm<Tile, false, false>(g, vec, splits, s);
+int launch_layout(GemmArgs g, bool a_kc, bool b_kc, bool vec, int blocks, hipStream_t s) {
+    if (a_kc && b_kc) return launch_gemm<Tile, true, true>(g, vec, blocks, s);
+    if (a_kc) return launch_gemm<Tile, true, false>(g, vec, blocks, s);
+    if (b_kc) return launch_gemm<Tile, false, true>(g, vec, blocks, s);
+    return launch_gemm<Tile, false, false>(g, vec, blocks, s);
 }
 
 }  // namespace
@@ -477,71 +517,94 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
     }
     const bool A_KC = a_kc, B_KC = !b_xc;
     const int cus = compute_units() > 0 ? compute_units() : 256;
-    auto tiles_of = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
-    // Big, Wide or Small by the time the slowest CU needs: rounds of tiles per CU x the tile's share
-    // of a Big tile x what the shape loses per flop (measured at 4096^3); Tiny when even the Small
-    // shape cannot give every CU a tile
-    auto rounds = [&](int64_t tiles) { return double((tiles + cus - 1) / cus); };
-    int shape = 0;
-    if (tiles_of(SmallTile::BM, SmallTile::BN) >= cus) {
-        const double big = rounds(tiles_of(BigTile::BM, BigTile::BN));
-        const double wide = rounds(tiles_of(WideTile::BM, WideTile::BN)) * 0.5 * 1.04;
-        const double small = rounds(tiles_of(SmallTile::BM, SmallTile::BN)) * 0.25 * 1.07;
-        shape = (big <= wide && big <= small) ? 2 : (wide <= small ? 3 : 1);
-    }
-    const int BM = shape == 3 ? WideTile::BM : shape == 2 ? BigTile::BM : shape == 1 ? SmallTile::BM : TinyTile::BM;
-    const int BN = shape == 3 ? WideTile::BN : shape == 2 ? BigTile::BN : shape == 1 ? SmallTile::BN : TinyTile::BN;
     constexpr int BK = 16;
     static_assert(BigTile::BK == BK && WideTile::BK == BK && SmallTile::BK == BK && TinyTile::BK == BK, "all tile shapes step K alike");
+    // The plan: a tile shape, and into how many parts along K the tiles of the last, partly filled
+    // round of blocks are cut (a round: `together` resident blocks on each CU), by a model of the
+    // time in seconds, fitted to measurements on this chip (1024^3 ... 7168^3 and the skinny
+    // products of a small layer):
+    //   a full round       together * per_flop * BM * BN * t    t = 2 k flops at one CU's peak rate
+    //   the last round     c blocks on the busiest CU, each 1 / parts of a tile: one block alone runs
+    //                      at `alone` (one wave per SIMD leaves the matrix pipe idle between k tiles),
+    //                      `together` of them at together * per_flop, in between in proportion; plus
+    //                      the memory latencies a block waits out before its first and after its last k tile
+    //   adding the parts   a launch and the parts' bytes written and read once
+    // parts fill the free places of the round with at least 8 k tiles each (4 when K allows no more).
+    struct Shape { int bm, bn, together; double per_flop, alone; };
+    static const Shape shapes[4] = {{TinyTile::BM, TinyTile::BN, 4, 1.30, 1.70}, {SmallTile::BM, SmallTile::BN, 2, 1.07, 1.34},
+                                    {BigTile::BM, BigTile::BN, 1, 1.00, 1.00}, {WideTile::BM, WideTile::BN, 2, 1.04, 1.32}};
+    const double t_elem = 2.0 * double(k) / (157.3e12 * 0.92 / cus);
+    int shape = 0, splits = 1, whole_tiles = 0;
+    double best = -1.0;
+    for (int sh = 0; sh < 4; ++sh) {
+        const Shape& q = shapes[sh];
+        const int64_t tiles = ((m + q.bm - 1) / q.bm) * ((n + q.bn - 1) / q.bn);
+        const int64_t places = int64_t(cus) * q.together;
+        const int64_t rounds = tiles / places, left = tiles % places;
+        const double area = double(q.bm) * q.bn;
+        int most = 1;
+        if (left > 0) {
+            int64_t want = places / left;
+            const int64_t by_scratch = int64_t(kScratchFloats) / (left * q.bm * q.bn);
+            if (want > by_scratch) want = by_scratch;
+            for (int min_ktiles = 8; min_ktiles >= 4 && most == 1; min_ktiles /= 2) {
+                const int64_t by_k = k / (min_ktiles * BK);
+                const int64_t p = want < by_k ? want : by_k;
+                if (p >= 2) most = int(p);
+            }
+        }
+        for (int parts : {1, most / 2, most}) {
+            if (parts < 1 || (parts == 1 && most > 1 && left == 0)) continue;
+            double cost = double(rounds) * q.together * q.per_flop * area * t_elem;
+            if (left > 0) {
+                const int64_t c = (left * parts + cus - 1) / cus;
+                const double busy = q.together == 1 ? q.alone
+                                                    : q.alone + double(c - 1) * (q.together * q.per_flop - q.alone) / (q.together - 1);
+                cost += busy * area * t_elem / parts + (rounds == 0 ? 3e-6 : 1e-6);
+                if (parts > 1) cost += 6e-6 + double(left) * parts * area * 8.0 / 4e12;
+            }
+            if (best < 0.0 || cost < best) {
+                best = cost; shape = sh; splits = parts; whole_tiles = int(parts > 1 ? tiles - left : tiles);
+            }
+        }
+    }
+    const int BM = shapes[shape].bm, BN = shapes[shape].bn;
     GemmArgs g;
     g.a = a; g.lda = A_KC ? as0 : as1;
     g.b = b; g.ldb = B_KC ? bs1 : bs0;
+    g.c = c; g.ldc = n;
     g.m = int(m); g.n = int(n); g.k = int(k);
     g.tiles_m = int((m + BM - 1) / BM);
     g.tiles_n = int((n + BN - 1) / BN);
+    g.bias = bias; g.relu = relu;
+    g.c_vec = (aligned16(c) && n % 4 == 0) ? 1 : 0;
     const bool vec = aligned16(a) && aligned16(b) && (g.lda % 4 == 0) && (g.ldb % 4 == 0);
-
-    // split along K when the output has too few tiles to fill the chip and K is long
-    int splits = 1;
-    const int64_t tiles = int64_t(g.tiles_m) * g.tiles_n;
-    float* partial = nullptr;
-    if (tiles < cus && k >= 16 * BK) {
-        // enough blocks for four per CU (they are co-resident), with at least 8 k tiles per block - or 4
-        // when K is so short that 8 would leave the product unsplit: a block walks its k tiles one
-        // memory latency after the other (16 tiles of [256 x 256] . [256 x 10]: 15 us unsplit, 8.5 us in
-        // four parts), while many short parts would only lengthen the fold
-        const int64_t want = (4 * cus + tiles - 1) / tiles;
-        const int64_t max_by_scratch = int64_t(kScratchFloats) / (m * n);
-        for (int min_ktiles = 8; min_ktiles >= 4 && splits == 1; min_ktiles /= 2) {
-            const int64_t max_by_k = k / (min_ktiles * BK);
-            int64_t parts = want < max_by_k ? want : max_by_k;
-            if (parts > max_by_scratch) parts = max_by_scratch;
-            if (parts >= 4) splits = int(parts);    // a two- or three-way split does not pay for its fold launch
-        }
-        if (splits > 1) {
-            partial = scratch();
-            if (!partial) return CTAMD_EINVAL;
-        }
+    const int tiles = g.tiles_m * g.tiles_n;
+    g.whole_tiles = whole_tiles;
+    g.splits = splits;
+    g.partial = nullptr;
+    g.k_per_split = int(k);
+    if (splits > 1) {
+        int kps = int((k + splits - 1) / splits);
+        kps = (kps + BK - 1) / BK * BK;
+        g.splits = splits = int((k + kps - 1) / kps);
+        g.k_per_split = kps;
+        g.partial = scratch();
+        if (!g.partial) return CTAMD_EINVAL;
+        if (size_t(tiles - whole_tiles) * size_t(splits) * size_t(BM) * size_t(BN) > kScratchFloats)
+            return fail(CTAMD_ERANGE, "%s: the parts of %d split tiles do not fit the device scratch", name, tiles - whole_tiles);
     }
-    int kps = int((k + splits - 1) / splits);
-    kps = (kps + BK - 1) / BK * BK;
-    splits = int((k + kps - 1) / kps);
-    g.k_per_split = kps;
-    if (splits > 1) { g.c = partial; g.ldc = n; g.split_stride = m * n; g.bias = nullptr; g.relu = 0; }
-    else { g.c = c; g.ldc = n; g.split_stride = 0; g.bias = bias; g.relu = relu; }
-
-    int rc = shape == 3 ? launch_layout<WideTile>(g, A_KC, B_KC, vec, splits, s)
-           : shape == 2 ? launch_layout<BigTile>(g, A_KC, B_KC, vec, splits, s)
-           : shape == 1 ? launch_layout<SmallTile>(g, A_KC, B_KC, vec, splits, s)
-                        : launch_layout<TinyTile>(g, A_KC, B_KC, vec, splits, s);
+    const int blocks = whole_tiles + (tiles - whole_tiles) * splits;
+    int rc = shape == 3 ? launch_layout<WideTile>(g, A_KC, B_KC, vec, blocks, s)
+           : shape == 2 ? launch_layout<BigTile>(g, A_KC, B_KC, vec, blocks, s)
+           : shape == 1 ? launch_layout<SmallTile>(g, A_KC, B_KC, vec, blocks, s)
+                        : launch_layout<TinyTile>(g, A_KC, B_KC, vec, blocks, s);
     if (rc || splits == 1) return rc;
-    size_t mn = size_t(m) * size_t(n);
-    if (mn % 4 == 0 && aligned16(c))
-        hipLaunchKernelGGL(splitk_fold<true>, dim3(unsigned((mn / 4 + kThreads - 1) / kThreads)), dim3(kThreads), 0, s,
-                           partial, c, mn, splits, bias, int(n), relu);
-    else
-        hipLaunchKernelGGL(splitk_fold<false>, dim3(unsigned((mn + kThreads - 1) / kThreads)), dim3(kThreads), 0, s,
-                           partial, c, mn, splits, bias, int(n), relu);
+    const dim3 fold_grid(unsigned(tiles - whole_tiles), unsigned(BM * BN / kFoldSlice));
+    if (shape == 3) hipLaunchKernelGGL((fold_parts<WideTile::BM, WideTile::BN>), fold_grid, dim3(kThreads), 0, s, g);
+    else if (shape == 2) hipLaunchKernelGGL((fold_parts<BigTile::BM, BigTile::BN>), fold_grid, dim3(kThreads), 0, s, g);
+    else if (shape == 1) hipLaunchKernelGGL((fold_parts<SmallTile::BM, SmallTile::BN>), fold_grid, dim3(kThreads), 0, s, g);
+    else hipLaunchKernelGGL((fold_parts<TinyTile::BM, TinyTile::BN>), fold_grid, dim3(kThreads), 0, s, g);
     return launched(name);
 }
 
