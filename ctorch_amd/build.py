@@ -57,7 +57,7 @@ def build(verbose=False, jobs=4):
                 print(rest)
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
     # what every kernel needs (registers, spills, LDS), next to the library: a spilled register costs a
-    # kernel its overlap of loads and arithmetic, so tests/test_build.py refuses a build that has one
+    # kernel its overlap of loads and arithmetic, so tests/test_abi_and_devmath.py refuses a build that has one
     with open(RESOURCES, "w") as f:
         json.dump(resources, f, indent=0, sort_keys=True)
     return LIB

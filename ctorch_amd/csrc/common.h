@@ -22,6 +22,12 @@ int launched(const char* kernel);
 // ctamd_init() and never freed.  Returns nullptr (and records an error) before ctamd_init().
 constexpr size_t kScratchFloats = size_t(1) << 24;   // 64 MiB
 float* scratch();
+// The same for work about to be launched on `stream`, which becomes the scratch's user.  The null
+// stream and blocking streams order themselves with each other; any other change of user is
+// accepted only when the previous user has nothing pending (and is not recording a graph):
+// otherwise nullptr, with the error text set - two streams would write the one buffer at once.
+float* scratch(void* stream);
+int scratch_claim(void* stream);
 // Four floats of -inf / of 0 in device memory (set up by ctamd_init): what row kernels read in
 // place of a vector that would lie beyond the end of a row.
 const float* pad_neg_inf();

@@ -589,7 +589,7 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
         kps = (kps + BK - 1) / BK * BK;
         g.splits = splits = int((k + kps - 1) / kps);
         g.k_per_split = kps;
-        g.partial = scratch();
+        g.partial = scratch(stream);
         if (!g.partial) return CTAMD_EINVAL;
         if (size_t(tiles - whole_tiles) * size_t(splits) * size_t(BM) * size_t(BN) > kScratchFloats)
             return fail(CTAMD_ERANGE, "%s: the parts of %d split tiles do not fit the device scratch", name, tiles - whole_tiles);

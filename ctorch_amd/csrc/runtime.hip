@@ -66,6 +66,48 @@ const float* pad_zero() {
     return s ? s + kScratchFloats + 4 : nullptr;
 }
 
+namespace {
+bool g_scratch_used[kMaxDevices] = {};
+void* g_scratch_user[kMaxDevices] = {};   // the stream whose work used the scratch last
+void* g_recording = nullptr;              // the stream a graph is being recorded on, if any
+
+bool blocking(void* stream) {             // orders itself with the null stream
+    if (!stream || stream == g_recording) return true;   // recordings are made on streams of ctamd_stream_create
+    unsigned flags = 0;
+    if (hipStreamGetFlags(as_stream(stream), &flags) != hipSuccess) return false;
+    return !(flags & hipStreamNonBlocking);
+}
+}  // namespace
+
+int scratch_claim(void* stream) {
+    int d = current_device();
+    if (d < 0 || d >= kMaxDevices) return fail(CTAMD_EINVAL, "no current device");
+    std::lock_guard<std::mutex> lock(g_mu);
+    void* user = g_scratch_user[d];
+    if (g_scratch_used[d] && user != stream) {
+        const bool ordered = (!user && blocking(stream)) || (!stream && blocking(user));
+        if (!ordered) {
+            if (user == g_recording && user)
+                return fail(CTAMD_EINVAL, "the device scratch belongs to the graph being recorded on another stream");
+            const hipError_t pending = hipStreamQuery(as_stream(user));
+            (void)hipGetLastError();
+            if (pending == hipErrorNotReady)
+                return fail(CTAMD_EINVAL,
+                            "two streams would use the one device scratch at once (reductions, losses, column softmax, split "
+                            "matrix products): wait for the first stream before issuing such work on a second");
+        }
+    }
+    g_scratch_used[d] = true;
+    g_scratch_user[d] = stream;
+    return CTAMD_OK;
+}
+
+float* scratch(void* stream) {
+    float* s = scratch();
+    if (!s || scratch_claim(stream) != CTAMD_OK) return nullptr;
+    return s;
+}
+
 float* scratch() {
     int d = current_device();
     if (d < 0 || d >= kMaxDevices || g_scratch[d] == nullptr) {
@@ -163,18 +205,32 @@ int ctamd_stream_create(void** stream) {
 }
 int ctamd_stream_destroy(void* stream) {
     if (!stream) return CTAMD_OK;
+    {
+        std::lock_guard<std::mutex> lock(g_mu);
+        for (int d = 0; d < kMaxDevices; ++d)
+            if (g_scratch_user[d] == stream) { g_scratch_user[d] = nullptr; g_scratch_used[d] = false; }   // destroying waits for its work
+    }
     return check_hip(hipStreamDestroy(as_stream(stream)), "hipStreamDestroy");
 }
 int ctamd_graph_begin(void* stream) {
     if (!stream) return fail(CTAMD_EINVAL, "%s: the null stream cannot record", __func__);
     // relaxed: host-side calls that are not stream work (an allocation by a pool that ran dry)
     // stay legal while recording
-    return check_hip(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeRelaxed), "hipStreamBeginCapture");
+    int rc = check_hip(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeRelaxed), "hipStreamBeginCapture");
+    if (!rc) {
+        std::lock_guard<std::mutex> lock(g_mu);
+        g_recording = stream;
+    }
+    return rc;
 }
 int ctamd_graph_end(void* stream, void** graph_out) {
     if (!stream || !graph_out) return fail(CTAMD_EINVAL, "%s: null argument", __func__);
     *graph_out = nullptr;
     hipGraph_t g = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_mu);
+        if (g_recording == stream) g_recording = nullptr;
+    }
     int rc = check_hip(hipStreamEndCapture(as_stream(stream), &g), "hipStreamEndCapture");
     if (rc) return rc;
     hipGraphExec_t exec = nullptr;
@@ -186,6 +242,7 @@ int ctamd_graph_end(void* stream, void** graph_out) {
 }
 int ctamd_graph_launch(void* graph, void* stream) {
     if (!graph) return fail(CTAMD_EINVAL, "%s: null graph", __func__);
+    if (scratch_claim(stream) != CTAMD_OK) return CTAMD_EINVAL;   // recorded reductions use the device scratch at replay
     return check_hip(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), as_stream(stream)), "hipGraphLaunch");
 }
 int ctamd_graph_destroy(void* graph) {

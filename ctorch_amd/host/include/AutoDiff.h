@@ -129,4 +129,7 @@ class AutoDiff {
     Tensor adjust_grad_shape(const Tensor& grad, const std::vector<size_t>& target_shape);
     Tensor input_gradient(Node* node, size_t input_id, size_t input_pos, const Tensor& node_grad);
 };
+// Makes this thread's device seed of backward(root) (a 0-D 1.0) now, if it does not exist yet.
+void prepare_backward_seed();
+
 #endif

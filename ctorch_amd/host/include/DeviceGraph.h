@@ -29,7 +29,8 @@ class DeviceGraph {
     DeviceGraph& operator=(const DeviceGraph&) = delete;
 
     void record(const std::function<void()>& body);
-    void replay();             // asynchronous; ordered after everything issued before it
+    void replay();             // asynchronous; ordered after everything issued before it: all graphs replay on one
+                               // stream, which the launches outside recordings (null stream) wait for and which waits for them
     void wait();               // until the replays issued so far have finished
     bool recorded() const { return graph_ != nullptr; }
 

@@ -49,11 +49,20 @@ class Storage {
             Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DATATYPE, "Storage data type mismatch");
         }
     }
+    // Returns a device block to the pool; it also carries what the host knows of a one-element
+    // block's value, so that every tensor sharing the block sees one state (std::get_deleter).
+    struct DeviceBlock {
+        size_t bytes;
+        bool known = false;
+        float value = 0.0f;
+        void operator()(char* q) const { ctorch_amd_host::device_release(q, bytes); }
+    };
+    DeviceBlock* block() const { return _data ? std::get_deleter<DeviceBlock>(_data) : nullptr; }
     static std::shared_ptr<char[]> allocate(size_t bytes, DeviceType device) {
         if (bytes == 0) return nullptr;
         if (device == DeviceType::kAMD) {
             char* p = static_cast<char*>(ctorch_amd_host::device_acquire(bytes));
-            return std::shared_ptr<char[]>(p, [bytes](char* q) { ctorch_amd_host::device_release(q, bytes); });
+            return std::shared_ptr<char[]>(p, DeviceBlock{bytes});
         }
         return std::shared_ptr<char[]>(new char[bytes], std::default_delete<char[]>());
     }
@@ -99,6 +108,21 @@ class Storage {
     // true while another Storage object (a view, an alias) refers to the same bytes
     bool shared() const { return _data.use_count() > 1; }
 
+    // The value of a one-element device storage when the host knows it without reading the device
+    // (it chose it, or a kernel's result came back with another read).  One state per block: an
+    // in-place writer that forgets it does so for every tensor that shares the block.
+    const float* known_value() const {
+        const DeviceBlock* b = block();
+        return (b && b->known) ? &b->value : nullptr;
+    }
+    void set_known_value(float v) {
+        DeviceBlock* b = block();
+        if (b && _size == 1) { b->known = true; b->value = v; }
+    }
+    void forget_known_value() {
+        if (DeviceBlock* b = block()) b->known = false;
+    }
+
     size_t size() const { return _size; }
     DType dtype() const { return _dtype; }
     DeviceType device() const { return _device; }
@@ -109,6 +133,7 @@ class Storage {
         if (_size > 0 && _data) {
             if (_device == DeviceType::kAMD) ctorch_amd_host::device_copy_d2d(s._data.get(), _data.get(), nbytes());
             else std::memcpy(s._data.get(), _data.get(), nbytes());
+            if (const float* v = known_value()) s.set_known_value(*v);
         }
         return s;
     }

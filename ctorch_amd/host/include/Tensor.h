@@ -35,9 +35,6 @@ class Tensor {
     DeviceType _device = DeviceType::kCPU;
     DType _dtype = DType::kFloat;
     Storage _storage;
-    // value of a one-element device tensor when the host already holds it (read back together with
-    // something else): item() then needs no transfer.  Dropped by the in-place writers.
-    std::shared_ptr<const float> _known_value;
 
     static std::atomic<size_t> global_tensor_id;
     void computeStrides();
@@ -70,9 +67,11 @@ class Tensor {
     // the elements of a contiguous tensor under another shape of the same element count, as a VIEW
     // (shares storage, new id)
     static Tensor view_shape(const Tensor& t, const std::vector<size_t>& shape);
-    void set_known_value(float v) { _known_value = std::make_shared<const float>(v); }
-    void forget_known_value() { _known_value.reset(); }
-    const float* known_value() const { return _known_value.get(); }   // null when the host does not know it
+    // value of a one-element device tensor when the host already holds it (it chose it, or it came back
+    // with another read): item() then needs no transfer.  Kept with the storage, dropped by the in-place writers.
+    void set_known_value(float v) { if (numel() == 1) _storage.set_known_value(v); }
+    void forget_known_value() { _storage.forget_known_value(); }       // for every tensor that shares the storage
+    const float* known_value() const { return numel() == 1 ? _storage.known_value() : nullptr; }   // null when the host does not know it
     // a tensor on `device` filled from host memory
     static Tensor from_host(const float* data, const std::vector<size_t>& shape, DeviceType device);
 

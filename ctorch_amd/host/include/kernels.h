@@ -66,6 +66,8 @@ Tensor leading_elements(const Tensor& g, const std::vector<size_t>& shape);
 // one pass over the logits and keeps the gradient for backward() (default on; off: a forward pass
 // that leaves row statistics, and a streaming backward pass).
 void set_ce_one_pass(bool on);
+void set_ce_kept_bytes(size_t cap);   // most bytes of one-pass CrossEntropy gradients kept for a backward() (default 4 GiB)
+size_t ce_kept_bytes();
 bool ce_one_pass();
 // tensors that are not fp32 (the typed arms of src/Tensor.cpp:197-243, :390-448)
 void fill_typed(void* device_ptr, DType dtype, double v, size_t n);    // zero() / ones() of any dtype, device memory

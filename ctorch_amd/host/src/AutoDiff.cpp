@@ -385,16 +385,23 @@ Tensor AutoDiff::input_gradient(Node* node, size_t input_id, size_t input_pos, c
     }
 }
 
+// The seed 1.0 on the device is made once per thread and shared (the tape never writes through a
+// shared gradient: accumulation goes to a fresh tensor then).
+static Tensor& device_seed() {
+    thread_local Tensor device_one;
+    if (device_one.is_cleared()) device_one = Tensor(1.0f, DeviceType::kAMD);
+    return device_one;
+}
+// Called before a recording starts: a seed made inside one would be a recorded launch into memory
+// reserved for that graph, and a backward() outside the graph would read it before any replay.
+void prepare_backward_seed() { (void)device_seed(); }
+
 // src/AutoDiff.cpp:548-553
 void AutoDiff::backward(Tensor& root) {
     AutoDiffContext::Guard guard(nullptr);
-    // the seed 1.0 on the device is made once per thread and shared (the tape never writes through
-    // a shared gradient: accumulation goes to a fresh tensor then)
-    thread_local Tensor device_one;
     if (root.device() == DeviceType::kAMD) {
-        if (device_one.is_cleared()) device_one = Tensor(1.0f, DeviceType::kAMD);
         seed_plus_zero_ = true;
-        backward(root, Tensor::alias(device_one));
+        backward(root, Tensor::alias(device_seed()));
         return;
     }
     Tensor grad_output(1.0f, root.device());

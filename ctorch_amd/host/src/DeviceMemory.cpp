@@ -3,8 +3,10 @@
 // kernel returns a new Tensor: src/kernels/CPU-BASIC/Add_BASIC_kernel.cpp:44); without a pool each
 // op would pay a hipMalloc and - worse - a hipFree, which synchronises the device.  Buckets are
 // 2^k * {1, 1.25, 1.5, 1.75}, at most 25 % over the request; freed blocks are kept until
-// device_trim().  All work is issued on the default stream, so a block handed out again is only
-// touched after every kernel that used it before.
+// device_trim().  Launches outside a graph recording go to the null stream, and graph replays go to
+// one blocking stream that the null stream orders itself with, so a block handed out again is only
+// touched after every kernel that used it before; what a recording allocates stays reserved for
+// its graph (BlockReservation) and is never handed to anyone else while the graph lives.
 #include <cstdio>
 #include <mutex>
 #include <unordered_map>
@@ -153,6 +155,7 @@ void device_release(void* p, size_t bytes) {
 }
 
 void device_trim() {
+    no_host_wait("device_trim");          // throws while a graph is being recorded: before anything is taken off the lists
     std::vector<void*> all;
     {
         std::lock_guard<std::mutex> lock(pool().mu);
@@ -163,7 +166,6 @@ void device_trim() {
         pool().cached_bytes = 0;
     }
     if (all.empty()) return;
-    no_host_wait("device_trim");
     ctamd_sync(nullptr);
     for (void* p : all) ctamd_free(p);
 }

@@ -55,7 +55,7 @@ Tensor::Tensor(ShapeTag, const std::vector<size_t>& shape, DType dtype, DeviceTy
 Tensor::Tensor(const Tensor& other)
     : tensor_id_(global_tensor_id++), _requires_grad(other._requires_grad), _shape(other._shape),
       _strides(other._strides), _storage_offset(other._storage_offset), _device(other._device),
-      _dtype(other._dtype), _storage(other._storage.clone()), _known_value(other._known_value) {}
+      _dtype(other._dtype), _storage(other._storage.clone()) {}
 
 Tensor& Tensor::operator=(const Tensor& other) {
     if (this != &other) {
@@ -67,7 +67,6 @@ Tensor& Tensor::operator=(const Tensor& other) {
         _device = other._device;
         _dtype = other._dtype;
         _storage = other._storage.clone();
-        _known_value = other._known_value;
     }
     return *this;
 }
@@ -75,7 +74,7 @@ Tensor& Tensor::operator=(const Tensor& other) {
 Tensor::Tensor(Tensor&& other) noexcept
     : tensor_id_(other.tensor_id_), _requires_grad(other._requires_grad), _shape(std::move(other._shape)),
       _strides(std::move(other._strides)), _storage_offset(other._storage_offset), _device(other._device),
-      _dtype(other._dtype), _storage(std::move(other._storage)), _known_value(std::move(other._known_value)) {
+      _dtype(other._dtype), _storage(std::move(other._storage)) {
     other.tensor_id_ = 0;
 }
 
@@ -89,7 +88,6 @@ Tensor& Tensor::operator=(Tensor&& other) noexcept {
         _device = other._device;
         _dtype = other._dtype;
         _storage = std::move(other._storage);
-        _known_value = std::move(other._known_value);
         other.tensor_id_ = 0;
     }
     return *this;
@@ -98,7 +96,7 @@ Tensor& Tensor::operator=(Tensor&& other) noexcept {
 Tensor::Tensor(AliasTag, const Tensor& other)
     : tensor_id_(other.tensor_id_), _requires_grad(other._requires_grad), _shape(other._shape),
       _strides(other._strides), _storage_offset(other._storage_offset), _device(other._device),
-      _dtype(other._dtype), _storage(other._storage), _known_value(other._known_value) {}
+      _dtype(other._dtype), _storage(other._storage) {}
 
 Tensor Tensor::from_host(const float* data, const std::vector<size_t>& shape, DeviceType device) {
     Tensor t(ShapeTag{}, shape, DType::kFloat, device, false);
@@ -138,7 +136,7 @@ float Tensor::item<float>() const {
     if (_dtype != DType::kFloat)
         Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DATATYPE, "item<float>(): dtype is not float");
     if (_device == DeviceType::kAMD) {
-        if (_known_value) return *_known_value;
+        if (const float* v = known_value()) return *v;
         float v;
         device_copy_d2h(&v, fptr(), sizeof(float));
         return v;
@@ -182,7 +180,7 @@ Tensor Tensor::to(DeviceType device) const {
 }
 
 void Tensor::fill(float v) {
-    _known_value.reset();
+    forget_known_value();
     if (_storage.empty()) return;
     if (_dtype != DType::kFloat)
         Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::DATATYPE, "fill(): only float tensors");

@@ -118,6 +118,12 @@ bool g_ce_one_pass = true;
 
 // ------------------------------------------------------------------ helpers for Tensor / tape
 void set_ce_one_pass(bool on) { g_ce_one_pass = on; }
+// Kept one-pass CrossEntropy gradients are as large as their logits and wait for a backward() that
+// may never come (a forward pass under a tape that is then dropped): together they hold at most
+// this many bytes, the oldest give way first, and logits larger than the cap get no such gradient.
+size_t g_ce_kept_cap = size_t(4) << 30;
+void set_ce_kept_bytes(size_t cap) { g_ce_kept_cap = cap; }
+size_t ce_kept_bytes() { return g_ce_kept_cap; }
 bool ce_one_pass() { return g_ce_one_pass; }
 
 void fill_typed(void* device_ptr, DType dtype, double v, size_t n) {
@@ -384,6 +390,7 @@ void sgd_step(Tensor& param, const Tensor& grad, float lr) {
     check_device(grad, "sgd_step");
     if (param.numel() != grad.numel() || !param.is_contiguous())
         Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "sgd_step: parameter and gradient differ in size");
+    param.forget_known_value();     // written in place
     run(ctamd_sgd_step_f32(param.fptr(), grad.fptr(), lr, param.numel(), current_stream()), "sgd_step");
 }
 void sgd_step_all(const std::vector<Tensor*>& params, const std::vector<Tensor>& grads, float lr) {
@@ -398,6 +405,7 @@ void sgd_step_all(const std::vector<Tensor*>& params, const std::vector<Tensor>&
         check_device(grads[i], "sgd_step_all");
         if (params[i]->numel() != grads[i].numel() || !params[i]->is_contiguous() || !grads[i].is_contiguous())
             Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "sgd_step_all: parameter and gradient differ in size");
+        params[i]->forget_known_value();                     // written in place
         p.push_back(params[i]->fptr());
         g.push_back(grads[i].fptr());
         n.push_back(params[i]->numel());
@@ -530,11 +538,21 @@ thread_local CeStats t_ce_stats[kCeStatsSlots];
 thread_local int t_ce_next = 0;
 void remember_ce(const Tensor& logits, const Tensor& target, Tensor stats, Tensor grad) {
     CeStats& slot = t_ce_stats[t_ce_next];
+    const int mine = t_ce_next;
     t_ce_next = (t_ce_next + 1) % kCeStatsSlots;
     slot.logits_id = logits.id();
     slot.target_id = target.id();
     slot.stats = std::move(stats);
     slot.grad = std::move(grad);
+    size_t held = 0;
+    for (const CeStats& c : t_ce_stats)
+        if (!c.grad.is_cleared()) held += c.grad.numel() * sizeof(float);
+    for (int age = 1; age < kCeStatsSlots && held > g_ce_kept_cap; ++age) {      // mine + 1 is the oldest
+        CeStats& old = t_ce_stats[(mine + age) % kCeStatsSlots];
+        if (old.grad.is_cleared()) continue;
+        held -= old.grad.numel() * sizeof(float);
+        old = CeStats();                                                       // its backward recomputes from the logits
+    }
 }
 CeStats* recall_ce(const Tensor& logits, const Tensor& target) {
     for (CeStats& c : t_ce_stats)
@@ -662,7 +680,8 @@ Tensor CrossEntropy_AMD_kernel(const Tensor& a, const Tensor& b) {
         // returns an empty Tensor), so it fetches the loss in the same transfer and item() is free
         Tensor pair(ShapeTag{}, {2}, DType::kFloat, DeviceType::kAMD, false);
         Tensor r = Tensor::view_element(pair, 0);
-        if (g_ce_one_pass && AutoDiffContext::current() && a.requires_grad() && ce_row_fits(a)) {
+        if (g_ce_one_pass && AutoDiffContext::current() && a.requires_grad() && ce_row_fits(a) &&
+            a.numel() * sizeof(float) <= g_ce_kept_cap) {
             Tensor grad = like(a);
             run(ctamd_cross_entropy_index_fused_f32(a.fptr(), b.fptr(), r.fptr(), reinterpret_cast<int32_t*>(pair.fptr() + 1),
                                                     grad.fptr(), a.sizes()[0], a.sizes()[1], current_stream()),

@@ -14,7 +14,9 @@
 #include "mnist_demo.h"
 
 #include <chrono>
+#include <cmath>
 #include <cstring>
+#include <thread>
 #include <vector>
 
 namespace {
@@ -725,8 +727,8 @@ long cth_time_chain(const float* a, const float* b, long n, int warm, int reps, 
         ta.requires_grad(true);
         tb.requires_grad(true);
         Tensor s = (g_fused_expr ? (Expr(ta) * Expr(tb) + 5.0f).relu().eval() : (ta * tb + 5.0f).relu()).sum();
+        s.backward();                      // enqueued before the read below waits for the device
         sink = s.item<float>();
-        s.backward();
         Tensor ga = grad(ta), gb = grad(tb);
     }, warm, reps, out);
 }
@@ -743,8 +745,8 @@ long cth_time_matmul(const float* A, const float* B, long M, int warm, int reps,
         tA.requires_grad(true);
         tB.requires_grad(true);
         Tensor L = tA.matmul(tB).sum();
+        backward(L);                       // enqueued before the read below waits for the device
         sink = L.item<float>();
-        backward(L);
         Tensor ga = grad(tA), gb = grad(tB);
     }, warm, reps, out);
 }
@@ -772,8 +774,8 @@ long cth_time_mlp(const float* x, long B, long I, const float* W1, const float* 
         tb2.requires_grad(true);
         Tensor h = g_fused_layers ? tx.linear(tW1, tb1, true) : (tx.matmul(tW1) + tb1).relu();
         Tensor loss = (g_fused_layers ? h.linear(tW2, tb2, false) : h.matmul(tW2) + tb2).cross_entropy(ty);
+        backward(loss);                    // enqueued before the read below waits for the device
         sink = loss.item<float>();
-        backward(loss);
         Tensor g1 = grad(tW1), g2 = grad(tb1), g3 = grad(tW2), g4 = grad(tb2);
     }, warm, reps, out);
 }
@@ -867,6 +869,131 @@ long cth_expr_graph(const float* X1, const float* X2, const float* R, const floa
     }
 }
 
+// Recorded steps under stress.  out[0..3]: sums from two graphs replayed alternately, with no host
+// wait between them and new input contents before each pair, and the same sums computed eagerly
+// on the last input; out[4]: item() of a one-element parameter after an in-place SGD step (2 - 1 *
+// 0.5); out[5]: gradient of sum(x * x) at x[0] from a backward() issued eagerly on a thread whose
+// first backward() was inside a recording; out[6]: 1 if a DeviceGraph whose first recording
+// failed records and replays a second body.  Returns 0, or a negative code for an exception.
+long cth_graph_hardening(const float* X, const float* X2, long n, float* out) {
+    try {
+        long d[1] = {n};
+        Tensor tx = make(X, d, 1), tx2 = make(X2, d, 1), staged = make(X, d, 1);
+        Tensor ty, sa, sb, sc;
+        auto body_a = [&] { ty = staged * 2.0f; sa = ty.sum(); };
+        auto body_b = [&] { Tensor tz = ty + 1.0f; sb = tz.sum(); sc = (tz * tz).sum(); };
+        body_a();
+        body_b();                                  // eagerly once: a warm pool, ty exists
+        DeviceGraph ga, gb;
+        ga.record(body_a);
+        gb.record(body_b);
+        for (int it = 0; it < 6; ++it) {
+            ctorch_amd_host::copy_into(staged, (it % 2) ? tx2 : tx);
+            ga.replay();
+            gb.replay();                           // reads what ga wrote; both use the device scratch
+        }
+        out[0] = sa.item<float>();
+        out[1] = sb.item<float>();
+        Tensor ey = tx2 * 2.0f, ez = ey + 1.0f;
+        out[2] = ey.sum().item<float>();
+        out[3] = ez.sum().item<float>();
+        if (sc.item<float>() != (ez * ez).sum().item<float>()) return -3;
+
+        Tensor p(2.0f, DeviceType::kAMD), g(0.5f, DeviceType::kAMD);
+        if (p.item<float>() != 2.0f) return -4;
+        ctorch_amd_host::sgd_step(p, g, 1.0f);
+        out[4] = p.item<float>();
+
+        float first_grad = -1.0f;
+        long thread_rc = 0;
+        std::thread worker([&] {
+            try {
+                AutoDiff ctx;
+                configure(ctx);
+                AutoDiffContext::Guard guard(&ctx);
+                Tensor w = make(X, d, 1), gw;
+                auto step = [&] {
+                    w.requires_grad(true);
+                    Tensor L = (w * w).sum();
+                    backward(L);
+                    gw = grad(w);
+                };
+                DeviceGraph rec;
+                rec.record(step);                  // this thread's first backward(): inside a recording
+                ctx.clear_graph();
+                step();                            // eagerly, before any replay
+                std::vector<float> host(static_cast<size_t>(n));
+                if (emit(gw, host.data()) < 0) { thread_rc = -5; return; }
+                first_grad = host[0];
+            } catch (const std::exception&) {
+                thread_rc = -6;
+            }
+        });
+        worker.join();
+        if (thread_rc) return thread_rc;
+        out[5] = first_grad;
+
+        DeviceGraph again;
+        bool threw = false;
+        try {
+            again.record([&] { Tensor t = staged * 3.0f; (void)t.sum().item<float>(); });   // a host wait: refused while recording
+        } catch (const std::exception&) {
+            threw = true;
+        }
+        Tensor kept;
+        again.record([&] { kept = staged * 3.0f; });
+        again.replay();
+        again.wait();
+        std::vector<float> host(static_cast<size_t>(n));
+        if (emit(kept, host.data()) < 0) return -7;
+        out[6] = (threw && again.recorded() && host[0] == X2[0] * 3.0f) ? 1.0f : 0.0f;   // staged holds X2 after the loop
+        return 0;
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
+// CrossEntropy (class index) of two logits matrices forward, then both backward, three times: with
+// the default cap on kept one-pass gradients, with a cap that holds only one of them (the older
+// gives way and its backward recomputes), and with a cap below either (no one-pass gradient at all).
+// Returns 0 when the first two agree bit for bit on both gradients and the third - which works from
+// the forward pass's row statistics - to 2e-7; writes the first into g1 / g2.
+long cth_ce_kept_cap(const float* x1, const float* x2, const float* labels, long rows, long cols, float* g1, float* g2) {
+    try {
+        long d[2] = {rows, cols}, yi[1] = {rows};
+        Tensor ty = make(labels, yi, 1);
+        const size_t before = ctorch_amd_host::ce_kept_bytes();
+        const size_t one = size_t(rows) * size_t(cols) * sizeof(float);
+        const size_t caps[3] = {before, one + one / 2, one / 2};
+        std::vector<float> a(size_t(rows * cols)), b(size_t(rows * cols));
+        long rc = 0;
+        for (int k = 0; k < 3 && rc == 0; ++k) {
+            ctorch_amd_host::set_ce_kept_bytes(caps[k]);
+            Tensor t1 = make(x1, d, 2), t2 = make(x2, d, 2);
+            AutoDiff ctx;
+            configure(ctx);
+            AutoDiffContext::Guard guard(&ctx);
+            t1.requires_grad(true);
+            t2.requires_grad(true);
+            Tensor l1 = t1.cross_entropy(ty), l2 = t2.cross_entropy(ty);
+            Tensor L = l1 + l2;
+            backward(L);
+            float* o1 = k == 0 ? g1 : a.data();
+            float* o2 = k == 0 ? g2 : b.data();
+            if (emit(grad(t1), o1) < 0 || emit(grad(t2), o2) < 0) rc = -2;
+            else if (k == 1 && (std::memcmp(o1, g1, a.size() * sizeof(float)) != 0 || std::memcmp(o2, g2, b.size() * sizeof(float)) != 0)) rc = -11;
+            else if (k == 2) {                  // from the forward pass's row statistics: the same values to rounding
+                for (size_t i = 0; i < a.size(); ++i)
+                    if (!(std::fabs(o1[i] - g1[i]) <= 2e-7f) || !(std::fabs(o2[i] - g2[i]) <= 2e-7f)) rc = -12;
+            }
+        }
+        ctorch_amd_host::set_ce_kept_bytes(before);
+        return rc;
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
 // loss_sum = CE(logits, class index), backward: dlogits = softmax - onehot.
 long cth_time_softmax_ce(const float* logits, const float* labels, long rows, long cols, int warm, int reps,
                          double* out) {
@@ -879,8 +1006,8 @@ long cth_time_softmax_ce(const float* logits, const float* labels, long rows, lo
         AutoDiffContext::Guard guard(&ctx);
         tx.requires_grad(true);
         Tensor loss = tx.cross_entropy(ty);
+        backward(loss);                    // enqueued before the read below waits for the device
         sink = loss.item<float>() / float(rows);
-        backward(loss);
         Tensor g = grad(tx);
     }, warm, reps, out);
 }
@@ -899,8 +1026,8 @@ long cth_time_expr(const float* X, const float* R, const float* T, long rows, lo
         Tensor Y = g_fused_expr ? (sigmoid(Expr(tX) / Expr(tR)) - tanh(Expr(tX)) * sin(Expr(tX)) + cos(-Expr(tX))).eval()
                                 : (tX / tR).sigmoid() - tX.tanh() * tX.sin() + (-tX).cos();
         Tensor L = Y.mse_loss(tT) + Y.mae_loss(tT);
+        backward(L);                       // enqueued before the read below waits for the device
         sink = L.item<float>();
-        backward(L);
         Tensor gX = grad(tX), gR = grad(tR);
     }, warm, reps, out);
 }

@@ -38,8 +38,10 @@ def golden():
 @pytest.fixture
 def exact_math():
     """The library's exact mode (glibc's floats bit for bit, exactly rounded quotients) for one test;
-    the default single-precision mode is restored afterwards."""
-    import gpu_support as G
-    prev = G.set_math_mode(G.MATH_EXACT)
+    the default single-precision mode is restored afterwards.  (Through ctypes alone: a test of the
+    C++ front-end must not start torch's own HIP runtime after the library's.)"""
+    from ctorch_amd import capi
+    lib = capi.load()
+    prev = lib.ctamd_set_math_mode(1)
     yield
-    G.set_math_mode(prev)
+    lib.ctamd_set_math_mode(prev)

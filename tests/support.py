@@ -1073,6 +1073,26 @@ class HostLayer(Reference):
         rc = self.cdll.cth_expr_graph(fp(X1), fp(X2), fp(r), fp(T), C.c_long(rows), C.c_long(cols), *[fp(o) for o in outs])
         return (rc, *outs)
 
+    def graph_hardening(self, X, X2):
+        """Two graphs replayed alternately without host waits, a parameter read after an in-place SGD
+        step, a thread's first backward() inside a recording, a DeviceGraph re-recorded after a failed
+        recording.  Returns (rc, out[7])."""
+        X, X2 = f32(X), f32(X2)
+        out = np.zeros(7, dtype=np.float32)
+        self.cdll.cth_graph_hardening.restype = C.c_long
+        rc = self.cdll.cth_graph_hardening(fp(X), fp(X2), C.c_long(X.size), fp(out))
+        return rc, out
+
+    def ce_kept_cap(self, x1, x2, labels):
+        """CrossEntropy gradients of two logits matrices under three caps on kept one-pass gradients.
+        Returns (rc, g1, g2); rc == 0: the runs agree (see cth_ce_kept_cap)."""
+        x1, x2, labels = f32(x1), f32(x2), f32(labels)
+        rows, cols = x1.shape
+        g1, g2 = np.empty_like(x1), np.empty_like(x2)
+        self.cdll.cth_ce_kept_cap.restype = C.c_long
+        rc = self.cdll.cth_ce_kept_cap(fp(x1), fp(x2), fp(labels), C.c_long(rows), C.c_long(cols), fp(g1), fp(g2))
+        return rc, g1, g2
+
     def set_fused_expr(self, on):
         """chain, expr, program and their timed versions evaluate their elementwise part as one fused
         expression (Expr::eval): one launch forward, one backward."""

@@ -431,3 +431,40 @@ def test_fused_against_unfused_on_more_programs(oracle, host, exact_math):
     finally:
         host.set_fused_expr(False)
         host.set_reference_row0(False)
+
+
+def test_recorded_steps_stay_ordered_and_keep_no_stale_state(oracle, host):
+    """Graphs replay on one stream: two graphs that share the device scratch and a tensor, replayed
+    alternately with new inputs and no host wait, give the eager sums of the last input.  item() of a
+    one-element parameter after an in-place SGD step reads the device.  A thread whose first
+    backward() happens inside a recording still seeds an eager backward() with 1.  A DeviceGraph
+    whose recording failed can record again."""
+    print("case graph hardening", flush=True)
+    X = oracle.uniform((1 << 20,), 611, -1, 1)
+    X2 = oracle.uniform((1 << 20,), 612, -1, 1)
+    rc, out = host.graph_hardening(X, X2)
+    assert rc == 0
+    assert out[0] == out[2] and out[1] == out[3]
+    assert out[4] == np.float32(1.5)
+    assert out[5] == np.float32(0.0) + (X[0] + X[0])      # d(sum x*x)/dx = x + x by the product rule, added to the tape's zero
+    assert out[6] == 1.0
+
+
+def test_kept_cross_entropy_gradients_are_capped(oracle, host, exact_math):
+    """The gradient that the one-pass CrossEntropy keeps for backward() is bounded in bytes: when the
+    cap holds only one of two, the older is dropped and recomputed from its logits; below the size
+    of one, none is kept and backward() works from the forward pass's row statistics.  The first two
+    agree bit for bit, the third to 2e-7, and all are the oracle's gradient to a few ulp."""
+    print("case ce kept cap", flush=True)
+    rows, cols = 96, 1000
+    x1 = oracle.normal((rows, cols), 621, 0, 2)
+    x2 = oracle.normal((rows, cols), 622, 0, 2)
+    lab = oracle.ints((rows,), 623, cols)
+    rc, g1, g2 = host.ce_kept_cap(x1, x2, lab)
+    assert rc == 0, rc
+    for x, g in ((x1, g1), (x2, g2)):
+        want = oracle.ce_bwd_index(x, lab, 1.0)
+        # the row's sum of exponentials is added in another order than the oracle's: a few ulp of each element
+        rel = np.abs(g - want) / np.maximum(np.abs(want), 1e-30)
+        print(f"  largest element-relative difference from the oracle {rel.max():.2e}")
+        assert rel.max() <= 5e-6      # the oracle adds 1000 exponentials in order, in single precision
