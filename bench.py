@@ -37,10 +37,30 @@ M = 4096
 DOT_N = 1 << 26
 EW_N = 1 << 26
 
-# HBM bytes per forward-GEMM launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, scaled
-# by the same counters on the 768 MiB elementwise add of the same run); see
-# profiles/gemm_f32_4096_hbm_traffic.txt (384 MiB fetched + 64 MiB written; 192 MiB algorithmic).
-GEMM_TRAFFIC_BYTES = 470203664
+# HBM bytes per forward-GEMM launch come from a committed summary of two rocprofv3 --pmc runs
+# (FETCH_SIZE, WRITE_SIZE, each scaled by the same counter on the elementwise add of the same run):
+# profiles/gemm_f32_4096_hbm_traffic.json, next to its .txt with the commands and the raw figures.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "gemm_f32_4096_hbm_traffic.json")
+
+
+def gemm_traffic():
+    """(bytes per launch, where the figure comes from) - (None, reason) when the summary is missing."""
+    try:
+        with open(TRAFFIC_PROFILE) as f:
+            p = json.load(f)
+        return int(p["forward_gemm"]["hbm_bytes_per_launch"]), {
+            "file": os.path.relpath(TRAFFIC_PROFILE, ROOT), "measured": p.get("date"), "head": p.get("head")}
+    except (OSError, KeyError, ValueError) as e:
+        return None, {"file": os.path.relpath(TRAFFIC_PROFILE, ROOT), "error": str(e)}
+
+
+# Seeds of the synthetic inputs (ctorch_amd/rng.py), one per tensor, as the configurations name them.
+SEEDS = {"config1": {"a": 101, "b": 102},
+         "config2": {"A": 201, "B": 202, "dot_u": 211, "dot_v": 212},
+         "config3": {"x": 301, "labels": 302, "W1": 311, "b1": 312, "W2": 313, "b2": 314},
+         "config4": {"logits": 401, "labels": 402},
+         "config5": {"X": 501, "r": 502, "T": 503},
+         "elementwise": {"a": 601, "b": 602}}
 
 
 def cpu_baseline(seconds_hint=15.0):
@@ -64,10 +84,10 @@ def cpu_baseline(seconds_hint=15.0):
 
 
 def _cpu_baseline(np, support):
-    rng = np.random.default_rng(202)
+    from ctorch_amd import rng
     rows = 160
-    A = rng.standard_normal((rows, M), dtype=np.float32)
-    B = rng.standard_normal((M, M), dtype=np.float32)
+    A = rng.normal((rows, M), SEEDS["config2"]["A"])      # the first rows of the benchmark's A
+    B = rng.normal((M, M), SEEDS["config2"]["B"])
     kind = "port"
     fn = None
     if support.ref_available():
@@ -106,12 +126,10 @@ def config_report(with_cpu):
         raise RuntimeError("%s is missing: run `make -C ctorch_amd/host`" % HOST_LIB)
     host = C.CDLL(HOST_LIB)
     host.cth_quiet()
-    FP, L, I, D5 = C.POINTER(C.c_float), C.c_long, C.c_int, C.c_double * 5
+    from ctorch_amd import rng
+    FP, L, I, D5 = C.POINTER(C.c_float), C.c_long, C.c_int, C.c_double * 6
     fp = lambda a: a.ctypes.data_as(FP)
     f32 = lambda a: np.ascontiguousarray(a, dtype=np.float32)
-    rng = np.random.default_rng(7)
-    uni = lambda shape, lo, hi: f32(rng.random(shape, dtype=np.float32) * (hi - lo) + lo)
-    nrm = lambda shape, sd=1.0: f32(rng.standard_normal(shape, dtype=np.float32) * sd)
 
     ref = None
     if with_cpu:
@@ -131,8 +149,8 @@ def config_report(with_cpu):
     def add(name, rc, out, cpu_ms=None, cpu_note=None, launch_bound=False):
         if rc < 0:
             raise RuntimeError("config step failed: " + name)
-        ms, nbytes, flops, ideal_s, launches = list(out)
-        e = {"name": name, "gpu_ms": round(ms, 4), "launches": int(round(launches)),
+        ms, nbytes, flops, ideal_s, launches, median_ms = list(out)
+        e = {"name": name, "gpu_ms": round(ms, 4), "gpu_ms_median": round(median_ms, 4), "launches": int(round(launches)),
              "algorithmic_GB": round(nbytes / 1e9, 4), "GFLOP": round(flops / 1e9, 3),
              "GB/s": round(nbytes / ms / 1e6, 1), "TFLOP/s": round(flops / ms / 1e9, 2),
              "roofline_frac": round(ideal_s * 1e3 / ms, 4)}
@@ -146,7 +164,7 @@ def config_report(with_cpu):
 
     # config 1: elementwise chain, n = 2^20
     n = 1 << 20
-    a, b = uni(n, -1, 1), uni(n, -1, 1)
+    a, b = rng.uniform(n, SEEDS["config1"]["a"], -1, 1), rng.uniform(n, SEEDS["config1"]["b"], -1, 1)
     out = D5()
     rc = host.cth_time_chain(fp(a), fp(b), L(n), I(5), I(50), out)
     cpu = _timed(lambda: ref.chain(a, b)) if with_cpu else None
@@ -161,7 +179,7 @@ def config_report(with_cpu):
     # config 2: MatMul forward + backward at 1024, 2048, 4096; Dot 2^26
     slab_ms = {}
     for Mm in (1024, 2048, 4096):
-        A, B = nrm((Mm, Mm)), nrm((Mm, Mm))
+        A, B = rng.normal((Mm, Mm), SEEDS["config2"]["A"]), rng.normal((Mm, Mm), SEEDS["config2"]["B"])
         out = D5()
         rc = host.cth_time_matmul(fp(A), fp(B), L(Mm), I(3), I(10), out)
         cpu, note = None, None
@@ -172,7 +190,7 @@ def config_report(with_cpu):
             note = "forward rows 0..%d (%.2f s), x%d for all rows, x3 for the two backward products" % (r - 1, t / 1e3, Mm // r)
         add("config 2: MatMul %d^3 forward + backward (dC = ones)" % Mm, rc, out, cpu, note)
         del A, B
-    u, v = uni(1 << 26, -1, 1), uni(1 << 26, -1, 1)
+    u, v = rng.uniform(1 << 26, SEEDS["config2"]["dot_u"], -1, 1), rng.uniform(1 << 26, SEEDS["config2"]["dot_v"], -1, 1)
     out = D5()
     rc = host.cth_time_dot(fp(u), fp(v), L(1 << 26), I(3), I(20), out)
     cpu, note = None, None
@@ -184,12 +202,13 @@ def config_report(with_cpu):
     del u, v
 
     # config 3: MLP 784-256-10 train step, batch 256 and 8192
-    W1, b1 = uni((784, 256), -1 / 28.0, 1 / 28.0), uni(256, -1 / 28.0, 1 / 28.0)
-    W2, b2 = uni((256, 10), -1 / 16.0, 1 / 16.0), uni(10, -1 / 16.0, 1 / 16.0)
+    s3 = SEEDS["config3"]
+    W1, b1 = rng.uniform((784, 256), s3["W1"], -1 / 28.0, 1 / 28.0), rng.uniform(256, s3["b1"], -1 / 28.0, 1 / 28.0)
+    W2, b2 = rng.uniform((256, 10), s3["W2"], -1 / 16.0, 1 / 16.0), rng.uniform(10, s3["b2"], -1 / 16.0, 1 / 16.0)
     cpu256 = None
     for Bn in (256, 8192):
-        x = f32(rng.integers(0, 256, (Bn, 784)) / 255.0)
-        lab = f32(rng.integers(0, 10, Bn))
+        x = f32(rng.ints((Bn, 784), s3["x"], 256) / np.float32(255.0))
+        lab = rng.ints(Bn, s3["labels"], 10)
         out = D5()
         rc = host.cth_time_mlp(fp(x), L(Bn), L(784), fp(W1), fp(b1), L(256), fp(W2), fp(b2), L(10), fp(lab), I(5),
                                I(30), out)
@@ -222,8 +241,8 @@ def config_report(with_cpu):
 
     # config 4: row softmax + cross entropy, [8192 x 32000]
     R4, C4 = 8192, 32000
-    logits = nrm((R4, C4), 2.0)
-    lab = f32(rng.integers(0, C4, R4))
+    logits = rng.normal((R4, C4), SEEDS["config4"]["logits"], 0.0, 2.0)
+    lab = rng.ints(R4, SEEDS["config4"]["labels"], C4)
     out = D5()
     rc = host.cth_time_softmax_ce(fp(logits), fp(lab), L(R4), L(C4), I(2), I(10), out)
     cpu, note = None, None
@@ -240,7 +259,8 @@ def config_report(with_cpu):
 
     # config 5: broadcast expression + MSE + MAE, one backward
     R5 = 4096
-    X, rv, T = uni((R5, R5), -2, 2), uni(R5, 0.5, 2), nrm((R5, R5))
+    s5 = SEEDS["config5"]
+    X, rv, T = rng.uniform((R5, R5), s5["X"], -2, 2), rng.uniform(R5, s5["r"], 0.5, 2), rng.normal((R5, R5), s5["T"])
     out = D5()
     rc = host.cth_time_expr(fp(X), fp(rv), fp(T), L(R5), L(R5), I(3), I(10), out)
     cpu, note = None, None
@@ -258,7 +278,7 @@ def config_report(with_cpu):
     host.cth_set_fused_expr(0)
     add("config 5: Y=sigmoid(X/r)-tanh(X)*sin(X)+cos(-X), MSE+MAE, backward; X [4096 x 4096], fused expression", rc, out, cpu,
         note)
-    return {"cores": 1, "cpu_kind": cpu_kind if with_cpu else None, "steps": rows}
+    return {"cores": 1, "cpu_kind": cpu_kind if with_cpu else None, "seeds": SEEDS, "steps": rows}
 
 
 def main():
@@ -285,14 +305,13 @@ def main():
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     P = lambda t: C.c_void_p(t.data_ptr())
 
-    g = torch.Generator(device=dev)
-    g.manual_seed(201)
-    A = torch.randn(M, M, device=dev, generator=g)
-    B = torch.randn(M, M, device=dev, generator=g)
+    from ctorch_amd import rng
+    up = lambda a: torch.from_numpy(a).to(dev)
+    s2 = SEEDS["config2"]
+    A, B = up(rng.normal((M, M), s2["A"])), up(rng.normal((M, M), s2["B"]))
     dC = torch.ones(M, M, device=dev)
     Cm, dA, dB = (torch.empty(M, M, device=dev) for _ in range(3))
-    u = torch.rand(DOT_N, device=dev, generator=g) * 2 - 1
-    v = torch.rand(DOT_N, device=dev, generator=g) * 2 - 1
+    u, v = up(rng.uniform(DOT_N, s2["dot_u"], -1, 1)), up(rng.uniform(DOT_N, s2["dot_v"], -1, 1))
     d = torch.empty(1, device=dev)
 
     def gemm(a, as0, as1, b, bs0, bs1, c):
@@ -300,9 +319,11 @@ def main():
 
     fwd_events = []
 
+    step_events = []
+
     def step(timed):
         if timed:
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0, e1, e2 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
             e0.record()
         gemm(A, M, 1, B, M, 1, Cm)            # C = A . B
         if timed:
@@ -311,6 +332,9 @@ def main():
         gemm(dC, M, 1, B, 1, M, dA)           # dA = dC . B^T  (B as a [n,k] -> [k,n] view)
         gemm(A, 1, M, dC, M, 1, dB)           # dB = A^T . dC
         capi.check(lib.ctamd_dot_f32(P(u), P(v), P(d), DOT_N, stream))
+        if timed:
+            e2.record()
+            step_events.append((e0, e2))
 
     for _ in range(args.warmup):
         step(False)
@@ -323,7 +347,11 @@ def main():
     ms_per_step = dt / args.steps * 1e3
     flop_per_step = 3 * 2.0 * M ** 3 + 2.0 * DOT_N
     value = flop_per_step / (ms_per_step * 1e-3) / 1e12
-    gemm_ms = sum(a.elapsed_time(b) for a, b in fwd_events) / len(fwd_events)
+    gemm_each = sorted(a.elapsed_time(b) for a, b in fwd_events)
+    gemm_ms = sum(gemm_each) / len(gemm_each)
+    gemm_ms_median = gemm_each[len(gemm_each) // 2]
+    step_each = sorted(a.elapsed_time(b) for a, b in step_events)
+    step_ms_median = step_each[len(step_each) // 2]
     achieved = 2.0 * M ** 3 / (gemm_ms * 1e-3) / 1e12
 
     # sanity of what was timed: C against an fp64 recomputation of a few rows
@@ -333,8 +361,9 @@ def main():
     assert bool(((Cm[rows].double() - ref).abs() <= bound).all()), "forward GEMM failed its fp64 check"
 
     # elementwise leg of the metric: a + b, 256 MiB per operand, four rotating buffer sets
-    sets = [tuple(torch.randn(EW_N, device=dev) for _ in range(2)) + (torch.empty(EW_N, device=dev),)
-            for _ in range(4)]
+    se = SEEDS["elementwise"]
+    sets = [(up(rng.normal(EW_N, se["a"] + 10 * i)), up(rng.normal(EW_N, se["b"] + 10 * i)), torch.empty(EW_N, device=dev))
+            for i in range(4)]
     def ew(i):
         a, b, r = sets[i % 4]
         capi.check(lib.ctamd_add_f32(P(a), P(b), P(r), EW_N, stream))
@@ -352,19 +381,22 @@ def main():
     ew_gbs = 12.0 * EW_N / ew_s / 1e9
     del sets
 
+    traffic, traffic_source = gemm_traffic()
     out = {
         "metric": "elementwise HBM GB/s + fp32 MatMul TFLOP/s (% of MI355X roofline), 1 GPU",
         "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(ms_per_step, 4), "ms_per_step_median": round(step_ms_median, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[1]: fp32 MatMul 4096^3 forward + backward (dA = dC.B^T, dB = A^T.dC, "
                                "dC = ones) + Dot of two 2^26-element vectors; N(0,1) / uniform[-1,1] inputs "
-                               "generated on the device", "M": M, "N": M, "K": M, "dot_n": DOT_N},
+                               "from the counter-based generator (ctorch_amd/rng.py)", "M": M, "N": M, "K": M,
+                   "dot_n": DOT_N, "seeds": SEEDS["config2"]},
         "roofline": {"bound": "mfma", "kernel": "gemm_kernel<Cfg<256,256,16,128,64>, A K-contiguous, "
                                                 "B N-contiguous> (forward C = A.B)",
                      "achieved": round(achieved, 2), "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / MFMA_FP32_PEAK_TFLOPS, 4), "traffic": GEMM_TRAFFIC_BYTES,
-                     "launch_ms": round(gemm_ms, 4)},
+                     "frac": round(achieved / MFMA_FP32_PEAK_TFLOPS, 4), "traffic": traffic,
+                     "traffic_source": traffic_source, "launch_ms": round(gemm_ms, 4),
+                     "launch_ms_median": round(gemm_ms_median, 4)},
         "elementwise": {"op": "a + b (ctamd_add_f32), 2^26 elements, 12 B/elem", "achieved": round(ew_gbs, 1),
                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ew_gbs / HBM_PEAK_GBS, 4)},
     }

@@ -13,6 +13,7 @@
 #include "DeviceGraph.h"
 #include "mnist_demo.h"
 
+#include <algorithm>
 #include <chrono>
 #include <cmath>
 #include <cstring>
@@ -690,16 +691,33 @@ long cth_program(const float* inputs, const int* kinds, int n_in, const int* ops
 // launches.
 }  // extern "C"
 namespace {
+double median_of(std::vector<double> v) {
+    if (v.empty()) return 0.0;
+    std::sort(v.begin(), v.end());
+    const size_t h = v.size() / 2;
+    return v.size() % 2 ? v[h] : 0.5 * (v[h - 1] + v[h]);
+}
 template <class Step>
 long time_steps(Step step, int warm, int reps, double* out) {
     try {
         for (int i = 0; i < warm; ++i) step();
         ctamd_sync(nullptr);
         ctamd_counters_reset();
+        // every step ends with a read that waits for the device (Dot's result, a loss), so the host
+        // clock around one step times that step: out[5] is the median of the steps
+        std::vector<double> each;
+        each.reserve(size_t(reps));
         auto t0 = std::chrono::steady_clock::now();
-        for (int i = 0; i < reps; ++i) step();
+        auto prev = t0;
+        for (int i = 0; i < reps; ++i) {
+            step();
+            auto now = std::chrono::steady_clock::now();
+            each.push_back(std::chrono::duration<double, std::milli>(now - prev).count());
+            prev = now;
+        }
         ctamd_sync(nullptr);
         auto t1 = std::chrono::steady_clock::now();
+        out[5] = median_of(each);
         double bytes = 0, flops = 0, ideal = 0;
         uint64_t launches = 0;
         ctamd_counters_read(&bytes, &flops, &ideal, &launches);
@@ -812,9 +830,18 @@ long cth_time_mlp_graph(const float* x, long B, long I, const float* W1, const f
         ctamd_counters_read(&bytes, &flops, &ideal, &launches);
         float sink = 0;
         for (int i = 0; i < warm; ++i) { step.replay(); sink += loss.item<float>(); }
+        std::vector<double> each;
         auto t0 = std::chrono::steady_clock::now();
-        for (int i = 0; i < reps; ++i) { step.replay(); sink += loss.item<float>(); }
+        auto prev = t0;
+        for (int i = 0; i < reps; ++i) {
+            step.replay();
+            sink += loss.item<float>();
+            auto now = std::chrono::steady_clock::now();
+            each.push_back(std::chrono::duration<double, std::milli>(now - prev).count());
+            prev = now;
+        }
         auto t1 = std::chrono::steady_clock::now();
+        out[5] = median_of(each);
         out[0] = std::chrono::duration<double, std::milli>(t1 - t0).count() / reps;
         out[1] = bytes;
         out[2] = flops;

@@ -36,10 +36,8 @@ def test_config1_elementwise_chain_2e20(oracle, host):
 @pytest.mark.parametrize("M", [1024, 2048, 4096])
 def test_config2_matmul_forward_backward(oracle, M):
     print("case config 2 M", M, flush=True)
-    g = torch.Generator(device=G.DEV)
-    g.manual_seed(201 + M)
-    A = torch.randn(M, M, device=G.DEV, generator=g)
-    B = torch.randn(M, M, device=G.DEV, generator=g)
+    A = G.dev(oracle.normal((M, M), 201))       # the configuration's seeds: 201 / 202 (203 for the linearity check)
+    B = G.dev(oracle.normal((M, M), 202))
     C = G.matmul(A, B)
     rows = torch.tensor([0, 1, M // 3, M - 1], device=G.DEV)
     ref = A[rows].double() @ B.double()
@@ -63,7 +61,7 @@ def test_config2_matmul_forward_backward(oracle, M):
     assert bool(((dA.double() - rs[None, :]).abs() <= 1e-5 * B.abs().double().sum(1)[None, :]).all())
     assert bool(((dB.double() - cs[:, None]).abs() <= 1e-5 * A.abs().double().sum(0)[:, None]).all())
     # linearity: A.(B + B2) = A.B + A.B2 up to rounding
-    B2 = torch.randn(M, M, device=G.DEV, generator=g)
+    B2 = G.dev(oracle.normal((M, M), 203))
     lhs = G.matmul(A, B + B2)
     rhs = C + G.matmul(A, B2)
     scale = A.abs().double() @ (B.abs() + B2.abs()).double()[:, :8]
@@ -73,10 +71,8 @@ def test_config2_matmul_forward_backward(oracle, M):
 def test_config2_dot_2e26(oracle):
     print("case config 2 dot", flush=True)
     n = 1 << 26
-    g = torch.Generator(device=G.DEV)
-    g.manual_seed(211)
-    a = torch.rand(n, device=G.DEV, generator=g) * 2 - 1
-    b = torch.rand(n, device=G.DEV, generator=g) * 2 - 1
+    a = G.dev(oracle.uniform((n,), 211, -1, 1))
+    b = G.dev(oracle.uniform((n,), 212, -1, 1))
     got = float(G.reduce2("dot", a, b).item())
     want = float(torch.dot(a.double(), b.double()).item())
     assert abs(got - want) <= 1e-5 * float((a.double() * b.double()).abs().sum().item())
@@ -124,14 +120,12 @@ def test_config3_mlp_train_step(oracle, host, B):
         assert np.abs(a - w).max() <= 1e-5 * max(1.0, np.abs(w).max()) * (B / 256) ** 0.5, n
 
 
-def test_config4_softmax_cross_entropy_8192x32000():
+def test_config4_softmax_cross_entropy_8192x32000(oracle):
     print("case config 4", flush=True)
     rows, cols = 8192, 32000
-    g = torch.Generator(device=G.DEV)
-    g.manual_seed(401)
-    x = torch.randn(rows, cols, device=G.DEV, generator=g) * 2
-    idx = torch.randint(0, cols, (rows,), device=G.DEV, generator=g)
-    idxf = idx.float()
+    x = G.dev(oracle.normal((rows, cols), 401, 0.0, 2.0))     # the configuration's seeds: 401 / 402
+    idxf = G.dev(oracle.ints((rows,), 402, cols))
+    idx = idxf.long()
     loss, status = G.ce_index(x, idxf)
     assert status == 0
     lse = torch.logsumexp(x.double(), dim=1)
