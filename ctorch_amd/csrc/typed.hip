@@ -6,6 +6,7 @@
 #include <limits.h>
 
 #include "common.h"
+#include "devmath.h"
 
 namespace ctamd {
 namespace {
@@ -150,6 +151,12 @@ unsigned typed_grid(size_t n) {
 
 // ------------------------------------------------------------------------------ double softmax
 
+// The exponential is glibc's exp bit for bit (cta_exp64); its 2 KiB table of 2^(k/128) sits in LDS.
+__device__ __forceinline__ void stage_exp64_table(uint64_t* tab) {
+    for (unsigned i = threadIdx.x; i < 256; i += blockDim.x) tab[i] = cta_exp64_tab[i];
+    __syncthreads();
+}
+
 __device__ __forceinline__ double block_reduce(double v, bool is_max, double* s_part) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
@@ -171,6 +178,8 @@ __device__ __forceinline__ double block_reduce(double v, bool is_max, double* s_
 __global__ __launch_bounds__(256) void softmax_rows_f64_kernel(const double* __restrict__ x, double* __restrict__ y, size_t rows,
                                                                size_t cols) {
     __shared__ double s_part[4];
+    __shared__ uint64_t s_tab[256];
+    stage_exp64_table(s_tab);
     for (size_t row = blockIdx.x; row < rows; row += gridDim.x) {
         const double* xr = x + row * cols;
         double* yr = y + row * cols;
@@ -178,49 +187,190 @@ __global__ __launch_bounds__(256) void softmax_rows_f64_kernel(const double* __r
         for (size_t j = threadIdx.x; j < cols; j += blockDim.x) m = xr[j] > m ? xr[j] : m;
         m = block_reduce(m, true, s_part);
         double sum = 0.0;
-        for (size_t j = threadIdx.x; j < cols; j += blockDim.x) sum += exp(xr[j] - m);
+        for (size_t j = threadIdx.x; j < cols; j += blockDim.x) sum += cta_exp64(xr[j] - m, s_tab);
         sum = block_reduce(sum, false, s_part);
-        for (size_t j = threadIdx.x; j < cols; j += blockDim.x) yr[j] = exp(xr[j] - m) / sum;
+        for (size_t j = threadIdx.x; j < cols; j += blockDim.x) yr[j] = cta_exp64(xr[j] - m, s_tab) / sum;
     }
 }
 
-// A block owns 32 neighbouring columns; its 8 groups of 32 lanes take every 8th row (a group reads
-// 256 contiguous bytes per row) and are combined through LDS in group order: column maximum, sum of
-// exp(x - max), y = exp(x - max) / sum.  (One thread walking a whole column, the reference's
-// order src/Tensor.cpp:1766-1781, took 11.9 ms on [8192 x 8192].)
-constexpr int kColsPerBlock = 32, kRowGroups = 8;
-__global__ __launch_bounds__(256) void softmax_cols_f64_kernel(const double* __restrict__ x, double* __restrict__ y, size_t rows,
-                                                               size_t cols) {
-    __shared__ double s_red[kRowGroups][kColsPerBlock];
-    const unsigned lane = threadIdx.x % kColsPerBlock, group = threadIdx.x / kColsPerBlock;
-    const size_t j = size_t(blockIdx.x) * kColsPerBlock + lane;
-    const bool live = j < cols;
-    double m = -__builtin_huge_val();
-    if (live) {
-#pragma unroll 4
-        for (size_t i = group; i < rows; i += kRowGroups) {
-            const double v = x[i * cols + j];
-            m = v > m ? v : m;
+// The same with the row in registers: every element is read once, its exponential computed once
+// and kept (as the reference keeps it: src/Tensor.cpp:1686-1696), then divided by the row's sum.
+// PAIRS 128-bit words (two doubles) per thread, 256 threads: rows of up to 512 * PAIRS columns;
+// cols even and both pointers 16-byte aligned.
+typedef double v2d __attribute__((ext_vector_type(2)));
+template <int PAIRS>
+__global__ __launch_bounds__(256) void softmax_rows_f64_resident_kernel(const double* __restrict__ x, double* __restrict__ y, size_t rows,
+                                                                        size_t cols) {
+    __shared__ double s_part[4];
+    __shared__ uint64_t s_tab[256];
+    stage_exp64_table(s_tab);
+    const size_t pairs = cols / 2;
+    for (size_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        const v2d* xr = reinterpret_cast<const v2d*>(x + row * cols);
+        v2d* yr = reinterpret_cast<v2d*>(y + row * cols);
+        v2d v[PAIRS];
+        double m = -__builtin_huge_val();
+#pragma unroll
+        for (int k = 0; k < PAIRS; ++k) {
+            const size_t j = size_t(k) * 256 + threadIdx.x;
+            v[k] = v2d{-__builtin_huge_val(), -__builtin_huge_val()};
+            if (j < pairs) v[k] = __builtin_nontemporal_load(xr + j);
+        }
+#pragma unroll
+        for (int k = 0; k < PAIRS; ++k) {
+            m = v[k][0] > m ? v[k][0] : m;
+            m = v[k][1] > m ? v[k][1] : m;
+        }
+        m = block_reduce(m, true, s_part);
+        double sum = 0.0;
+#pragma unroll
+        for (int k = 0; k < PAIRS; ++k) {
+            const size_t j = size_t(k) * 256 + threadIdx.x;
+            if (j < pairs) {
+                v[k][0] = cta_exp64(v[k][0] - m, s_tab);
+                v[k][1] = cta_exp64(v[k][1] - m, s_tab);
+                sum += v[k][0];
+                sum += v[k][1];
+            }
+        }
+        sum = block_reduce(sum, false, s_part);
+#pragma unroll
+        for (int k = 0; k < PAIRS; ++k) {
+            const size_t j = size_t(k) * 256 + threadIdx.x;
+            if (j < pairs) __builtin_nontemporal_store(v2d{v[k][0] / sum, v[k][1] / sum}, yr + j);
         }
     }
-    s_red[group][lane] = m;
-    __syncthreads();
+}
+
+// Column softmax in two launches over chunks of rows.  A block owns 32 neighbouring columns of one
+// chunk; its 8 groups of 32 lanes take every 8th row of the chunk (a group reads 256 contiguous
+// bytes per row).  First launch: a running (maximum, sum of exp(x - maximum)) pair per thread with
+// ONE exponential per element - of the element's distance below the maximum, or of the old
+// maximum's distance below the element when the maximum moves - combined over the groups in group
+// order and left per (chunk, column) in `pairs`.  Second launch: every block brings the chunks' pairs
+// of its columns to the column maximum in chunk order (a few exponentials per column), then writes
+// y = exp(x - max) / sum.  Two exponentials and 24 bytes per element, against three sweeps of the
+// whole matrix by 256 blocks before.  (One thread walking a whole column, the reference's order
+// src/Tensor.cpp:1766-1781, took 11.9 ms on [8192 x 8192].)
+constexpr int kLanesPerRow = 32, kRowGroups = 8;
+struct MaxSum {
+    double m, s;
+};
+__device__ __forceinline__ MaxSum join(MaxSum a, MaxSum b, const uint64_t* tab) {       // a's rows come before b's
+    const double m = b.m > a.m ? b.m : a.m;
+    MaxSum r;
+    r.m = m;
+    r.s = (a.s == 0.0 ? 0.0 : a.s * cta_exp64(a.m - m, tab)) + (b.s == 0.0 ? 0.0 : b.s * cta_exp64(b.m - m, tab));
+    return r;
+}
+// W columns per lane: 2 with 128-bit accesses (cols even, pointers 16-byte aligned), else 1.
+template <int W>
+__global__ __launch_bounds__(256) void softmax_cols_f64_scan_kernel(const double* __restrict__ x, MaxSum* __restrict__ pairs, size_t rows,
+                                                                    size_t cols, size_t rows_per_chunk, size_t col0, size_t col_end) {
+    __shared__ MaxSum s_red[kRowGroups][kLanesPerRow * W];
+    __shared__ uint64_t s_tab[256];
+    stage_exp64_table(s_tab);
+    const unsigned lane = threadIdx.x % kLanesPerRow, group = threadIdx.x / kLanesPerRow;
+    const size_t j = col0 + (size_t(blockIdx.x) * kLanesPerRow + lane) * W;
+    const size_t first = size_t(blockIdx.y) * rows_per_chunk;
+    size_t last = first + rows_per_chunk;
+    if (last > rows) last = rows;
+    MaxSum t[W];
 #pragma unroll
-    for (int g = 0; g < kRowGroups; ++g) m = s_red[g][lane] > m ? s_red[g][lane] : m;
-    __syncthreads();
-    double sum = 0.0;
-    if (live) {
+    for (int w = 0; w < W; ++w) t[w] = MaxSum{-__builtin_huge_val(), 0.0};
+    if (j < col_end) {
 #pragma unroll 4
-        for (size_t i = group; i < rows; i += kRowGroups) sum += exp(x[i * cols + j] - m);
+        for (size_t i = first + group; i < last; i += kRowGroups) {
+            double v[W];
+            if (W == 2) {
+                const v2d p = *reinterpret_cast<const v2d*>(x + i * cols + j);
+                v[0] = p[0];
+                v[W - 1] = p[1];
+            } else {
+                v[0] = x[i * cols + j];
+            }
+#pragma unroll
+            for (int w = 0; w < W; ++w) {
+                const bool up = v[w] > t[w].m;
+                const double e = cta_exp64(up ? t[w].m - v[w] : v[w] - t[w].m, s_tab);   // t.m = -inf at the start: exp(-inf) = 0
+                t[w].s = up ? t[w].s * e + 1.0 : t[w].s + e;
+                t[w].m = up ? v[w] : t[w].m;
+            }
+        }
     }
-    s_red[group][lane] = sum;
-    __syncthreads();
-    double total = 0.0;
 #pragma unroll
-    for (int g = 0; g < kRowGroups; ++g) total += s_red[g][lane];
-    if (live) {
+    for (int w = 0; w < W; ++w) s_red[group][lane * W + w] = t[w];
+    __syncthreads();
+    if (group == 0 && j < col_end) {
+#pragma unroll
+        for (int w = 0; w < W; ++w) {
+            MaxSum r = s_red[0][lane * W + w];
+#pragma unroll
+            for (int g = 1; g < kRowGroups; ++g) r = join(r, s_red[g][lane * W + w], s_tab);
+            pairs[size_t(blockIdx.y) * cols + j + w] = r;
+        }
+    }
+}
+template <int W>
+__global__ __launch_bounds__(256) void softmax_cols_f64_write_kernel(const double* __restrict__ x, const MaxSum* __restrict__ pairs,
+                                                                     double* __restrict__ y, size_t rows, size_t cols,
+                                                                     size_t rows_per_chunk, unsigned chunks, size_t col0, size_t col_end) {
+    __shared__ MaxSum s_total[kLanesPerRow * W];
+    __shared__ uint64_t s_tab[256];
+    stage_exp64_table(s_tab);
+    const unsigned lane = threadIdx.x % kLanesPerRow, group = threadIdx.x / kLanesPerRow;
+    const size_t j = col0 + (size_t(blockIdx.x) * kLanesPerRow + lane) * W;
+    // The chunks' pairs of this block's columns, brought to the column maximum: first the maximum
+    // over the chunks (no exponential), then the sums scaled to it - independent exponentials, added
+    // in chunk order.  The block's 256 threads share the work: thread t takes column t % (32 W) and
+    // every (256 / (32 W))-th chunk; the parts are added in part order.
+    {
+        constexpr int kCols = kLanesPerRow * W, kParts = 256 / kCols;
+        __shared__ double s_m[kParts][kCols], s_s[kParts][kCols];
+        const unsigned c_in = threadIdx.x % kCols, part = threadIdx.x / kCols;
+        const size_t col = col0 + size_t(blockIdx.x) * kCols + c_in;
+        double m = -__builtin_huge_val();
+        if (col < col_end)
+            for (unsigned c = part; c < chunks; c += kParts) {
+                const double v = pairs[size_t(c) * cols + col].m;
+                m = v > m ? v : m;
+            }
+        s_m[part][c_in] = m;
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < kParts; ++q) m = s_m[q][c_in] > m ? s_m[q][c_in] : m;
+        double sum = 0.0;
+        if (col < col_end)
+            for (unsigned c = part; c < chunks; c += kParts) {
+                const MaxSum p = pairs[size_t(c) * cols + col];
+                sum += p.s == 0.0 ? 0.0 : p.s * cta_exp64(p.m - m, s_tab);
+            }
+        s_s[part][c_in] = sum;
+        __syncthreads();
+        if (part == 0) {
+            double total = 0.0;
+#pragma unroll
+            for (int q = 0; q < kParts; ++q) total += s_s[q][c_in];
+            s_total[c_in] = MaxSum{m, total};
+        }
+    }
+    __syncthreads();
+    if (j >= col_end) return;
+    MaxSum total[W];
+#pragma unroll
+    for (int w = 0; w < W; ++w) total[w] = s_total[lane * W + w];
+    const size_t first = size_t(blockIdx.y) * rows_per_chunk;
+    size_t last = first + rows_per_chunk;
+    if (last > rows) last = rows;
 #pragma unroll 4
-        for (size_t i = group; i < rows; i += kRowGroups) y[i * cols + j] = exp(x[i * cols + j] - m) / total;
+    for (size_t i = first + group; i < last; i += kRowGroups) {
+        if (W == 2) {
+            const v2d p = *reinterpret_cast<const v2d*>(x + i * cols + j);
+            const v2d q{cta_exp64(p[0] - total[0].m, s_tab) / total[0].s, cta_exp64(p[1] - total[W - 1].m, s_tab) / total[W - 1].s};
+            __builtin_nontemporal_store(q, reinterpret_cast<v2d*>(y + i * cols + j));
+        } else {
+            y[i * cols + j] = cta_exp64(x[i * cols + j] - total[0].m, s_tab) / total[0].s;
+        }
     }
 }
 
@@ -355,11 +505,46 @@ int ctamd_softmax_f64(const double* x, double* y, size_t rows, size_t cols, int 
     hipStream_t s = as_stream(stream);
     if (dim == 1) {
         const unsigned blocks = stream_grid(rows, 1, 8);
-        hipLaunchKernelGGL(softmax_rows_f64_kernel, dim3(blocks), dim3(cols <= 64 ? 64 : 256), 0, s, x, y, rows, cols);
+        const bool pairs_ok = cols % 2 == 0 && aligned16(x) && aligned16(y);
+        if (pairs_ok && cols > 64 && cols <= 512) hipLaunchKernelGGL(softmax_rows_f64_resident_kernel<1>, dim3(blocks), dim3(256), 0, s, x, y, rows, cols);
+        else if (pairs_ok && cols > 64 && cols <= 1024) hipLaunchKernelGGL(softmax_rows_f64_resident_kernel<2>, dim3(blocks), dim3(256), 0, s, x, y, rows, cols);
+        else if (pairs_ok && cols > 64 && cols <= 2048) hipLaunchKernelGGL(softmax_rows_f64_resident_kernel<4>, dim3(blocks), dim3(256), 0, s, x, y, rows, cols);
+        else if (pairs_ok && cols > 64 && cols <= 4096) hipLaunchKernelGGL(softmax_rows_f64_resident_kernel<8>, dim3(blocks), dim3(256), 0, s, x, y, rows, cols);
+        else if (pairs_ok && cols > 64 && cols <= 8192) hipLaunchKernelGGL(softmax_rows_f64_resident_kernel<16>, dim3(blocks), dim3(256), 0, s, x, y, rows, cols);
+        else hipLaunchKernelGGL(softmax_rows_f64_kernel, dim3(blocks), dim3(cols <= 64 ? 64 : 256), 0, s, x, y, rows, cols);
     } else {
-        const size_t blocks = (cols + kColsPerBlock - 1) / kColsPerBlock;
-        if (blocks > 0x7fffffffu) return fail(CTAMD_ERANGE, "%s: too many columns", __func__);
-        hipLaunchKernelGGL(softmax_cols_f64_kernel, dim3(unsigned(blocks)), dim3(256), 0, s, x, y, rows, cols);
+        const bool wide = cols % 2 == 0 && aligned16(x) && aligned16(y);
+        const size_t per_block = size_t(kLanesPerRow) * (wide ? 2 : 1);
+        // (Column panels of 64 - 128 MiB, scanned and written in turn so that the writing launch would find
+        // its panel in the memory-side cache, were measured: 445 us against 345 us for the whole matrix
+        // at once on [8192 x 8192] - a panel's launches are too small to fill the chip.)
+        const size_t panel_cols = cols;
+        const size_t cus = compute_units() > 0 ? size_t(compute_units()) : 256;
+        MaxSum* pairs = reinterpret_cast<MaxSum*>(scratch(stream));
+        if (!pairs) return CTAMD_EINVAL;
+        for (size_t col0 = 0; col0 < cols; col0 += panel_cols) {
+            const size_t col_end = col0 + panel_cols < cols ? col0 + panel_cols : cols;
+            const size_t strips = (col_end - col0 + per_block - 1) / per_block;
+            if (strips > 0x7fffffffu) return fail(CTAMD_ERANGE, "%s: too many columns", __func__);
+            // chunks of rows so that the grid fills the chip (about eight blocks per CU), of at least 64
+            // rows each, as many as the scratch holds pairs for
+            size_t chunks = (8 * cus + strips - 1) / strips;
+            if (chunks > (rows + 63) / 64) chunks = (rows + 63) / 64;
+            const size_t room = kScratchFloats * sizeof(float) / sizeof(MaxSum) / cols;
+            if (chunks > room) chunks = room;
+            if (chunks > 65535) chunks = 65535;
+            if (chunks < 1) return fail(CTAMD_ERANGE, "%s: more than %zu columns", __func__, kScratchFloats * sizeof(float) / sizeof(MaxSum));
+            const size_t rows_per_chunk = (rows + chunks - 1) / chunks;
+            chunks = (rows + rows_per_chunk - 1) / rows_per_chunk;
+            const dim3 grid{unsigned(strips), unsigned(chunks), 1u};
+            if (wide) {
+                hipLaunchKernelGGL(softmax_cols_f64_scan_kernel<2>, grid, dim3(256), 0, s, x, pairs, rows, cols, rows_per_chunk, col0, col_end);
+                hipLaunchKernelGGL(softmax_cols_f64_write_kernel<2>, grid, dim3(256), 0, s, x, pairs, y, rows, cols, rows_per_chunk, unsigned(chunks), col0, col_end);
+            } else {
+                hipLaunchKernelGGL(softmax_cols_f64_scan_kernel<1>, grid, dim3(256), 0, s, x, pairs, rows, cols, rows_per_chunk, col0, col_end);
+                hipLaunchKernelGGL(softmax_cols_f64_write_kernel<1>, grid, dim3(256), 0, s, x, pairs, y, rows, cols, rows_per_chunk, unsigned(chunks), col0, col_end);
+            }
+        }
     }
     account(double(rows) * double(cols) * 16.0, 0.0);
     return launched(__func__);

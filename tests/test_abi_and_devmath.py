@@ -77,6 +77,19 @@ def test_device_math_matches_glibc_on_a_strided_sweep(tmp_path):
         assert int(f[2]) > (8_000_000 if "_f32" in f[0] else 17_000_000) and int(f[4]) == 0, line
 
 
+def test_double_exponential_is_glibcs(tmp_path):
+    """cta_exp64 (the exponential of the double softmax kernels) against the installed glibc's exp on 16
+    million random arguments: the whole range, around zero, the overflow threshold, the subnormal
+    results, special values.  No mismatch."""
+    exe = str(tmp_path / "exp64_check")
+    subprocess.check_call(["gcc", "-O2", "-fopenmp", "-ffp-contract=off", "-mfma", "-o", exe,
+                           os.path.join(ROOT, "tests", "native", "exp64_check.c"), "-lm"])
+    out = subprocess.check_output([exe, "2000000"], text=True)
+    print(out)
+    f = out.split()
+    assert f[0] == "tested" and int(f[1]) > 16_000_000 and int(f[3]) == 0, out
+
+
 def test_division_through_a_double_reciprocal_is_ieee_division(tmp_path):
     """cta_div_rcp (softmax normalisation, x / n in the loss gradients, tensor / scalar) against a / b
     on 64 million random pairs incl. subnormals, and on the 63 million operand pairs whose exact quotient

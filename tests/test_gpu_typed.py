@@ -1,7 +1,8 @@
 """Tensors that are not fp32 (double, int32, int64, bool) through the C ABI: conversion from fp32,
 fill, tensor (+ * /) float and the gradient accumulation byte for byte against the CPU oracle and the
-reference's golden vectors.  The double softmax (its exponential is the device library's, not glibc's; its sums are trees of
-sequential partial sums): within 4 + sqrt(len) units in the last place of an extended-
+reference's golden vectors.  The double softmax (its exponential is glibc's bit for bit - cta_exp64, checked on the
+host in tests/native/exp64_check.c; its sums are trees of sequential partial sums, and the column form
+scales chunk sums to the column maximum): within 4 + sqrt(len) units in the last place of an extended-
 precision arbiter and within 4 + 2 sqrt(len) of the reference, a sequential sum of len terms carrying
 about sqrt(len) roundings; through its invariants at a large size."""
 import ctypes as C
@@ -121,7 +122,12 @@ def test_refusals():
 
 
 @pytest.mark.parametrize("shape,dim", [((1, 1), 1), ((3, 7), 0), ((3, 7), 1), ((300, 64), 1), ((64, 300), 0), ((17, 5000), 1),
-                                        ((2000, 33), 0), ((4096,), 0)])
+                                        ((2000, 33), 0), ((4096,), 0),
+                                        # every register-resident row shape, the streaming one past it, odd lengths
+                                        ((9, 66), 1), ((8, 400), 1), ((8, 1000), 1), ((5, 2000), 1), ((4, 4000), 1), ((3, 8192), 1),
+                                        ((2, 8194), 1), ((3, 1001), 1),
+                                        # column chunks: several chunks, two columns per lane and one
+                                        ((1000, 64), 0), ((8192, 130), 0), ((8192, 131), 0), ((100000, 2), 0)])
 def test_double_softmax(oracle, shape, dim):
     print("case softmax f64", shape, dim, flush=True)
     rng = np.random.default_rng(shape[0] * 7 + dim)
