@@ -228,8 +228,17 @@ def config_report(with_cpu):
         out = D5()
         rc = host.cth_time_mlp(fp(x), L(Bn), L(784), fp(W1), fp(b1), L(256), fp(W2), fp(b2), L(10), fp(lab), I(5),
                                I(30), out)
-        host.cth_set_fused_layers(0)
         add("config 3: MLP 784-256-10 train step, batch %d, fused layers" % Bn, rc, out, cpu, note, launch_bound=(Bn == 256))
+        # the same with the class-index range check deferred to the loss read (a bad label then gives a
+        # NaN loss instead of an empty tensor): no host wait between the forward and backward passes
+        host.cth_set_ce_deferred_label_check(1)
+        out = D5()
+        rc = host.cth_time_mlp(fp(x), L(Bn), L(784), fp(W1), fp(b1), L(256), fp(W2), fp(b2), L(10), fp(lab), I(5),
+                               I(30), out)
+        host.cth_set_ce_deferred_label_check(0)
+        host.cth_set_fused_layers(0)
+        add("config 3: MLP 784-256-10 train step, batch %d, fused layers, label check deferred to the loss read" % Bn, rc, out,
+            cpu, note, launch_bound=(Bn == 256))
         # the same step (one-hot targets) recorded into a HIP graph once and replayed
         oh = np.zeros((Bn, 10), np.float32)
         oh[np.arange(Bn), lab.astype(int)] = 1

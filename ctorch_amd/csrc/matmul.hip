@@ -392,7 +392,7 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
 
 // Adds the parts of the split tiles in their order and writes C (bias and ReLU of the fused
 // product included): blockIdx.x is the split tile, blockIdx.y one of its slices of kFoldSlice elements.
-constexpr int kFoldSlice = kThreads * 4 * 2;
+constexpr int kFoldSlice = kThreads * 4;       // one 128-bit word per thread: a tile cut in many parts has few tiles, and the grid is tiles x slices
 template <int BM, int BN>
 __global__ __launch_bounds__(kThreads) void fold_parts(GemmArgs g) {
     static_assert(BM * BN % kFoldSlice == 0, "a tile is a whole number of slices");
@@ -409,17 +409,18 @@ __global__ __launch_bounds__(kThreads) void fold_parts(GemmArgs g) {
         const int row = idx / (BN / 4), col = (idx % (BN / 4)) * 4;
         const int grow = m0 + row, gcol = n0 + col;
         if (grow >= g.m || gcol >= g.n) continue;
-        v4f t = *reinterpret_cast<const v4f*>(parts + row * BN + col);
+        const v4f* __restrict__ src = reinterpret_cast<const v4f*>(parts + row * BN + col);
+        constexpr size_t kStep = size_t(BM) * BN / 4;      // 128-bit words between parts
+        v4f t = src[0];
         int z = 1;
-        for (; z + 3 < g.splits; z += 4) {     // four loads in flight, added in order of z
-            const v4f p0 = *reinterpret_cast<const v4f*>(parts + size_t(z) * (BM * BN) + row * BN + col);
-            const v4f p1 = *reinterpret_cast<const v4f*>(parts + size_t(z + 1) * (BM * BN) + row * BN + col);
-            const v4f p2 = *reinterpret_cast<const v4f*>(parts + size_t(z + 2) * (BM * BN) + row * BN + col);
-            const v4f p3 = *reinterpret_cast<const v4f*>(parts + size_t(z + 3) * (BM * BN) + row * BN + col);
-            t = ((t + p0) + p1) + p2;
-            t = t + p3;
+        for (; z + 7 < g.splits; z += 8) {     // eight loads in flight, added in order of z
+            v4f p[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) p[q] = src[size_t(z + q) * kStep];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) t = t + p[q];
         }
-        for (; z < g.splits; ++z) t = t + *reinterpret_cast<const v4f*>(parts + size_t(z) * (BM * BN) + row * BN + col);
+        for (; z < g.splits; ++z) t = t + src[size_t(z) * kStep];
 #pragma unroll
         for (int e = 0; e < 4; ++e)
             if (gcol + e < g.n) t[e] = epilogue(t[e], g.bias, gcol + e, g.relu);

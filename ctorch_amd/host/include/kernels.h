@@ -66,6 +66,12 @@ Tensor leading_elements(const Tensor& g, const std::vector<size_t>& shape);
 // one pass over the logits and keeps the gradient for backward() (default on; off: a forward pass
 // that leaves row statistics, and a streaming backward pass).
 void set_ce_one_pass(bool on);
+// The reference range-checks class indices before it computes and returns an empty Tensor for a bad
+// one (CrossEntropy_BASIC_kernel.cpp:96-100); on the device that answer costs a wait for the kernel in
+// the middle of a training step.  With the deferred check the loss comes back at once and is NaN for a
+// bad index (what a recorded step does anyway).  Off by default.
+void set_ce_deferred_label_check(bool on);
+bool ce_deferred_label_check();
 void set_ce_kept_bytes(size_t cap);   // most bytes of one-pass CrossEntropy gradients kept for a backward() (default 4 GiB)
 size_t ce_kept_bytes();
 bool ce_one_pass();

@@ -118,6 +118,9 @@ bool g_ce_one_pass = true;
 
 // ------------------------------------------------------------------ helpers for Tensor / tape
 void set_ce_one_pass(bool on) { g_ce_one_pass = on; }
+bool g_ce_deferred_check = false;
+void set_ce_deferred_label_check(bool on) { g_ce_deferred_check = on; }
+bool ce_deferred_label_check() { return g_ce_deferred_check; }
 // Kept one-pass CrossEntropy gradients are as large as their logits and wait for a backward() that
 // may never come (a forward pass under a tape that is then dropped): together they hold at most
 // this many bytes, the oldest give way first, and logits larger than the cap get no such gradient.
@@ -694,7 +697,10 @@ Tensor CrossEntropy_AMD_kernel(const Tensor& a, const Tensor& b) {
                 "CrossEntropy_AMD_kernel");
             remember_ce(a, b, std::move(stats), Tensor());
         }
-        if (recording()) return r;              // a recorded step cannot wait: a bad index shows as a NaN loss
+        // a recorded step cannot wait, and a caller may choose not to (set_ce_deferred_label_check): a
+        // bad index then shows as a NaN loss when the loss is read, and the step keeps the GPU busy
+        // between its forward and backward passes instead of idling it for the flag's round trip
+        if (recording() || g_ce_deferred_check) return r;
         struct { float loss; int32_t bad; } got = {0.0f, 0};
         device_copy_d2h(&got, pair.fptr(), sizeof(got));
         if (got.bad) {

@@ -106,6 +106,7 @@ void cth_quiet() { Ctorch_Error::setPrintLevel(PrintLevel::MINIUM); }
 static int g_row0 = 0;
 static int g_fused_layers = 0;
 static int g_fused_expr = 0;
+extern "C" void cth_set_ce_deferred_label_check(int on) { ctorch_amd_host::set_ce_deferred_label_check(on != 0); }
 // the elementwise parts of cth_chain, cth_expr, cth_program and their timed versions are built as
 // one fused expression (Expr::eval: one launch forward, one backward) when set
 void cth_set_fused_expr(int on) { g_fused_expr = on; }
