@@ -507,8 +507,10 @@ extern "C" int ctamd_expr_run_f32(const ctamd_expr_insn* prog, int n_insn, const
     if (places_used < 1) places_used = 1;
     g.prog[n_insn] = g.prog[n_insn - 1];        // the spare entry: fetched, never run
     // Two 128-bit words per lane and pass halve the interpretation per element and double what a
-    // wave has in flight; with many values live only one word per lane fits in LDS.
-    const int words = (places_used * 2 > kMaxLive) ? 1 : 2;
+    // wave has in flight; with seven or more values live, LDS would hold fewer than three such
+    // blocks per CU, and one word per lane - twice the blocks - is faster (config-5 gradient program,
+    // 8 values live: 227 against 246 us).
+    const int words = (kLdsBudget / (places_used * kWordBytes * 2) >= 3) ? 2 : 1;
 
     const size_t lds = size_t(places_used) * kWordBytes * words;
     using Kernel = void (*)(ExprArgs);

@@ -72,6 +72,12 @@ void set_ce_one_pass(bool on);
 // bad index (what a recorded step does anyway).  Off by default.
 void set_ce_deferred_label_check(bool on);
 bool ce_deferred_label_check();
+// A condition that a kernel reports through four bytes on the device and that has to become an
+// exception: registered while a backward pass queues its launches, read when the pass has queued
+// them all (AutoDiff::backward calls run_deferred_checks before it returns).
+void defer_status_check(const Tensor& status, const std::string& message);
+void run_deferred_checks();
+void drop_deferred_checks();
 void set_ce_kept_bytes(size_t cap);   // most bytes of one-pass CrossEntropy gradients kept for a backward() (default 4 GiB)
 size_t ce_kept_bytes();
 bool ce_one_pass();

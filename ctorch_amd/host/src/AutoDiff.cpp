@@ -424,6 +424,7 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
     if (root.dtype() != DType::kFloat || grad_output.dtype() != DType::kFloat)
         Ctorch_Error::throwException(ErrorPlatform::kAutoDiff, ErrorType::DATATYPE, "backward: only float tensors have gradients");
     if (grad_output.device() != root.device()) grad_output = grad_output.to(root.device());
+    ctorch_amd_host::drop_deferred_checks();     // of a pass that ended in an exception
     root_node->grad = std::make_unique<Tensor>(adjust_grad_shape(grad_output, root.sizes()));
     root_node->grad_plus_zero = seed_plus_zero_;
     root_node->grad_assigned = !adjust_adds_to_zero_;     // a seed taken as it is stays as it is (:1126)
@@ -543,4 +544,8 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
         node->shared_term.reset();
         node->input_grads.clear();
     }
+    // checks whose answer a kernel left on the device (a zero divisor seen by a fused gradient
+    // program): read now, with every launch of this pass already queued, instead of idling the GPU in
+    // the middle of the pass
+    ctorch_amd_host::run_deferred_checks();
 }

@@ -358,13 +358,7 @@ struct Program : FusedPayload {
         int rc = ctamd_expr_run_f32(b.code.data(), int(b.code.size()), in.data(), int(in.size()), out.data(), int(out.size()),
                                     status_ptr, rows, cols, current_stream());
         if (rc) Ctorch_Error::throwException(kP, ErrorType::KERNEL_LAUNCH, std::string("backward (fused expression): ") + ctamd_last_error());
-        if (checks) {
-            int32_t v = 0;
-            ctorch_amd_host::device_copy_d2h(&v, status.fptr(), sizeof(v));
-            if (v)
-                Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::TENSOR_STATE,
-                                             "division by zero in the gradient of Div");
-        }
+        if (checks) ctorch_amd_host::defer_status_check(status, "division by zero in the gradient of Div");
         return grads;
     }
 };

@@ -118,6 +118,24 @@ bool g_ce_one_pass = true;
 
 // ------------------------------------------------------------------ helpers for Tensor / tape
 void set_ce_one_pass(bool on) { g_ce_one_pass = on; }
+namespace {
+struct DeferredCheck {
+    Tensor status;          // four bytes on the device: nonzero = the condition was met
+    std::string message;
+};
+thread_local std::vector<DeferredCheck> t_deferred;
+}  // namespace
+void defer_status_check(const Tensor& status, const std::string& message) { t_deferred.push_back({Tensor::alias(status), message}); }
+void drop_deferred_checks() { t_deferred.clear(); }
+void run_deferred_checks() {
+    std::vector<DeferredCheck> pending;
+    pending.swap(t_deferred);
+    for (const DeferredCheck& c : pending) {
+        int32_t v = 0;
+        device_copy_d2h(&v, c.status.fptr(), sizeof(v));
+        if (v) Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::TENSOR_STATE, c.message);
+    }
+}
 bool g_ce_deferred_check = false;
 void set_ce_deferred_label_check(bool on) { g_ce_deferred_check = on; }
 bool ce_deferred_label_check() { return g_ce_deferred_check; }
