@@ -19,21 +19,24 @@ int g_cus[kMaxDevices] = {};
 
 // Work counters (per process): what the operators launched since the last reset had to move and
 // compute, and the time that work takes at the published peaks.
-std::mutex g_count_mu;
-double g_bytes = 0.0, g_flops = 0.0, g_ideal_s = 0.0;
-uint64_t g_launches = 0;
+// (lock-free: every launcher adds to them on its way to the launch)
+std::atomic<double> g_bytes{0.0}, g_flops{0.0}, g_ideal_s{0.0};
+std::atomic<uint64_t> g_launches{0};
+inline void add_to(std::atomic<double>& a, double v) {
+    double seen = a.load(std::memory_order_relaxed);
+    while (!a.compare_exchange_weak(seen, seen + v, std::memory_order_relaxed)) {}
+}
 std::atomic<int> g_math_mode{CTAMD_MATH_FAST};
 constexpr double kHbmBytesPerS = 8.0e12;        // MI355X HBM3E
 constexpr double kMfmaF32FlopPerS = 157.3e12;   // MI355X dense fp32 matrix
 }  // namespace
 
 void account(double bytes, double flops) {
-    std::lock_guard<std::mutex> lock(g_count_mu);
-    g_bytes += bytes;
-    g_flops += flops;
+    add_to(g_bytes, bytes);
+    add_to(g_flops, flops);
     const double tb = bytes / kHbmBytesPerS, tf = flops / kMfmaF32FlopPerS;
-    g_ideal_s += tb > tf ? tb : tf;
-    ++g_launches;
+    add_to(g_ideal_s, tb > tf ? tb : tf);
+    g_launches.fetch_add(1, std::memory_order_relaxed);
 }
 
 int fail(int code, const char* fmt, ...) {
@@ -183,16 +186,16 @@ int ctamd_set_math_mode(int mode) {
 }
 int ctamd_math_mode(void) { return g_math_mode.load(std::memory_order_relaxed); }
 void ctamd_counters_reset(void) {
-    std::lock_guard<std::mutex> lock(g_count_mu);
-    g_bytes = g_flops = g_ideal_s = 0.0;
-    g_launches = 0;
+    g_bytes.store(0.0);
+    g_flops.store(0.0);
+    g_ideal_s.store(0.0);
+    g_launches.store(0);
 }
 void ctamd_counters_read(double* bytes, double* flops, double* roofline_seconds, uint64_t* launches) {
-    std::lock_guard<std::mutex> lock(g_count_mu);
-    if (bytes) *bytes = g_bytes;
-    if (flops) *flops = g_flops;
-    if (roofline_seconds) *roofline_seconds = g_ideal_s;
-    if (launches) *launches = g_launches;
+    if (bytes) *bytes = g_bytes.load();
+    if (flops) *flops = g_flops.load();
+    if (roofline_seconds) *roofline_seconds = g_ideal_s.load();
+    if (launches) *launches = g_launches.load();
 }
 
 // ---- streams and recorded launch sequences (HIP graphs)

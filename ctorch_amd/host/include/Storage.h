@@ -55,6 +55,7 @@ class Storage {
         size_t bytes;
         bool known = false;
         float value = 0.0f;
+        bool frozen = false;    // handed out as a gradient that shares the tape's bytes: read-only while shared
         void operator()(char* q) const { ctorch_amd_host::device_release(q, bytes); }
     };
     DeviceBlock* block() const { return _data ? std::get_deleter<DeviceBlock>(_data) : nullptr; }
@@ -121,6 +122,18 @@ class Storage {
     }
     void forget_known_value() {
         if (DeviceBlock* b = block()) b->known = false;
+    }
+    // A gradient read from the tape shares the tape's bytes.  While more than one tensor holds the
+    // block it must not be written in place; the front-end's in-place writers ask here first.
+    void freeze() {
+        if (DeviceBlock* b = block()) b->frozen = true;
+    }
+    bool writable() {
+        DeviceBlock* b = block();
+        if (!b || !b->frozen) return true;
+        if (_data.use_count() > 1) return false;
+        b->frozen = false;      // the last holder may do what it likes
+        return true;
     }
 
     size_t size() const { return _size; }

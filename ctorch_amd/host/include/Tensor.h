@@ -71,6 +71,8 @@ class Tensor {
     // with another read): item() then needs no transfer.  Kept with the storage, dropped by the in-place writers.
     void set_known_value(float v) { if (numel() == 1) _storage.set_known_value(v); }
     void forget_known_value() { _storage.forget_known_value(); }       // for every tensor that shares the storage
+    // throws when this tensor shares a gradient's bytes with the tape (AutoDiff::get_grad): such bytes are read-only
+    void require_writable(const char* what);
     const float* known_value() const { return numel() == 1 ? _storage.known_value() : nullptr; }   // null when the host does not know it
     // a tensor on `device` filled from host memory
     static Tensor from_host(const float* data, const std::vector<size_t>& shape, DeviceType device);

@@ -180,6 +180,7 @@ Tensor Tensor::to(DeviceType device) const {
 }
 
 void Tensor::fill(float v) {
+    require_writable("fill");
     forget_known_value();
     if (_storage.empty()) return;
     if (_dtype != DType::kFloat)
@@ -245,7 +246,15 @@ Tensor Tensor::share(const Tensor& t) {
     Tensor r(AliasTag{}, t);
     r.tensor_id_ = global_tensor_id++;
     r._requires_grad = false;
+    r._storage.freeze();
     return r;
+}
+
+void Tensor::require_writable(const char* what) {
+    if (!_storage.writable())
+        Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::TENSOR_STATE,
+                                     std::string(what) + ": this tensor shares a gradient's bytes with the tape (grad() does not copy); "
+                                     "copy it before writing to it in place");
 }
 
 Tensor Tensor::view_rows(const Tensor& t, size_t first, size_t count) {

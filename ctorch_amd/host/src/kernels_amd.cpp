@@ -397,6 +397,7 @@ void copy_into(Tensor& dst, const Tensor& src) {
     check_device(src, "copy_into");
     if (dst.numel() != src.numel() || !dst.is_contiguous() || !src.is_contiguous())
         Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "copy_into: sizes differ or a tensor is not contiguous");
+    dst.require_writable("copy_into");
     dst.forget_known_value();
     device_copy_d2d(dst.fptr(), src.fptr(), dst.numel() * sizeof(float));
 }
@@ -411,6 +412,7 @@ void sgd_step(Tensor& param, const Tensor& grad, float lr) {
     check_device(grad, "sgd_step");
     if (param.numel() != grad.numel() || !param.is_contiguous())
         Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "sgd_step: parameter and gradient differ in size");
+    param.require_writable("sgd_step");
     param.forget_known_value();     // written in place
     run(ctamd_sgd_step_f32(param.fptr(), grad.fptr(), lr, param.numel(), current_stream()), "sgd_step");
 }
@@ -426,6 +428,7 @@ void sgd_step_all(const std::vector<Tensor*>& params, const std::vector<Tensor>&
         check_device(grads[i], "sgd_step_all");
         if (params[i]->numel() != grads[i].numel() || !params[i]->is_contiguous() || !grads[i].is_contiguous())
             Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "sgd_step_all: parameter and gradient differ in size");
+        params[i]->require_writable("sgd_step_all");
         params[i]->forget_known_value();                     // written in place
         p.push_back(params[i]->fptr());
         g.push_back(grads[i].fptr());

@@ -1022,6 +1022,37 @@ long cth_ce_kept_cap(const float* x1, const float* x2, const float* labels, long
     }
 }
 
+// A gradient read from the tape shares the tape's bytes and is read-only while it does: fill, copy_into
+// and an SGD step into it throw; once the tape has let go of it the last holder may write.
+// Returns 0 when all of that holds.
+long cth_shared_grad_is_readonly(const float* a, long n) {
+    try {
+        long d[1] = {n};
+        Tensor ta = make(a, d, 1), other = make(a, d, 1);
+        Tensor g;
+        int threw = 0;
+        {
+            AutoDiff ctx;
+            configure(ctx);
+            AutoDiffContext::Guard guard(&ctx);
+            ta.requires_grad(true);
+            Tensor L = (ta * ta).sum();
+            backward(L);
+            g = grad(ta);
+            try { g.fill(1.0f); } catch (const std::exception&) { ++threw; }
+            try { ctorch_amd_host::copy_into(g, other); } catch (const std::exception&) { ++threw; }
+            try { ctorch_amd_host::sgd_step(g, other, 0.1f); } catch (const std::exception&) { ++threw; }
+        }
+        if (threw != 3) return -2;
+        g.fill(1.0f);                              // the tape is gone: g is the only holder
+        std::vector<float> host(static_cast<size_t>(n));
+        if (emit(g, host.data()) < 0 || host[0] != 1.0f) return -3;
+        return 0;
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
 // loss_sum = CE(logits, class index), backward: dlogits = softmax - onehot.
 long cth_time_softmax_ce(const float* logits, const float* labels, long rows, long cols, int warm, int reps,
                          double* out) {

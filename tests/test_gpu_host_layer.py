@@ -468,3 +468,13 @@ def test_kept_cross_entropy_gradients_are_capped(oracle, host, exact_math):
         rel = np.abs(g - want) / np.maximum(np.abs(want), 1e-30)
         print(f"  largest element-relative difference from the oracle {rel.max():.2e}")
         assert rel.max() <= 5e-6      # the oracle adds 1000 exponentials in order, in single precision
+
+
+def test_a_gradient_read_from_the_tape_is_read_only_while_shared(oracle, host):
+    """grad() hands out the tape's bytes instead of a copy (the reference copies): writing them in place
+    through the front-end (fill, copy_into, sgd_step) throws while the tape still holds them."""
+    print("case shared gradient read-only", flush=True)
+    x = oracle.uniform((4096,), 631, -1, 1)
+    import ctypes as C
+    host.cdll.cth_shared_grad_is_readonly.restype = C.c_long
+    assert host.cdll.cth_shared_grad_is_readonly(x.ctypes.data_as(C.POINTER(C.c_float)), C.c_long(x.size)) == 0
