@@ -10,8 +10,15 @@
  *    row-major, contiguous unless strides are passed.  Counts are in elements.
  *  - Launchers never allocate, free or synchronise: they enqueue on `stream` (a hipStream_t passed
  *    as void*, NULL = the default stream) and return.  Results are ready after ctamd_sync(stream).
- *  - Reductions use a per-device scratch buffer that ctamd_init() allocates once; calls that use
- *    it must not overlap on different streams of one device.
+ *  - Reductions, losses, column softmax / sums and matrix products whose tiles are cut along K use
+ *    a per-device scratch buffer that ctamd_init() allocates once.  It serves one stream at a time:
+ *    the null stream and blocking streams order themselves with each other and may alternate; any
+ *    other stream is accepted only when the stream that used the scratch before has nothing
+ *    pending, else the call returns CTAMD_EINVAL and launches nothing.
+ *  - Math mode (ctamd_set_math_mode): CTAMD_MATH_FAST, the default, evaluates the exponentials of
+ *    softmax / log-softmax / cross entropy and the sigmoid, tanh, sin, cos of fused expressions in
+ *    single precision within 2 ulp (sigmoid 4); CTAMD_MATH_EXACT returns the bits of the reference's
+ *    libm loops.  The one-operator kernels return glibc's floats in both modes.
  *  - Return value: 0 on success, a negative CTAMD_E* code otherwise; ctamd_last_error() gives
  *    the text.  No C++ exception crosses this boundary.  The C++ shim above maps codes to the
  *    reference's two error conventions (Ctorch_Error::log / throwException,
