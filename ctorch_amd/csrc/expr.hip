@@ -83,6 +83,22 @@ __device__ __forceinline__ void each(float (&c)[N], F f) {
 // |x| < 120, the double-precision routines beyond; sigmoid within 4 ulp of the reference's formula on
 // expf; tanh within 2 ulp of tanh for |x| >= 1 and 1.2e-7 absolute below); otherwise the routines
 // that return glibc's floats.
+template <bool FASTM, int WANT_COS, int N>
+__device__ __forceinline__ void sin_or_cos(float (&c)[N], const Tables& t) {
+    bool rare = false;
+    float x[N];
+#pragma unroll
+    for (int e = 0; e < N; ++e) {
+        x[e] = c[e];
+        c[e] = FASTM ? cta_sincosf_f32(x[e], WANT_COS) : cta_sincosf_fast(x[e], WANT_COS);
+        rare = rare || !(__builtin_fabsf(x[e]) < 120.0f);      // |x| >= 120, inf, NaN
+    }
+    if (__builtin_expect(rare, 0)) {
+        for (int e = 0; e < N; ++e)
+            if (cta_sincos_is_rare(x[e])) c[e] = cta_sincosf(x[e], WANT_COS, t.inv_pio4);
+    }
+}
+
 template <bool FASTM, int N>
 __device__ __forceinline__ void apply(const DevInsn& q, float (&c)[N], const float (&b)[N], const Tables& t) {
     switch (q.op) {
@@ -102,23 +118,8 @@ __device__ __forceinline__ void apply(const DevInsn& q, float (&c)[N], const flo
             if (FASTM) each(c, [&](int e) { return cta_tanh_f32(c[e]); });
             else each(c, [&](int e) { return tanh_ref(c[e], t); });
             break;
-        case CTAMD_EX_SIN:
-        case CTAMD_EX_COS: {
-            const int want_cos = (q.op == CTAMD_EX_COS);
-            bool rare = false;
-            float x[N];
-#pragma unroll
-            for (int e = 0; e < N; ++e) {
-                x[e] = c[e];
-                c[e] = FASTM ? cta_sincosf_f32(x[e], want_cos) : cta_sincosf_fast(x[e], want_cos);
-                rare = rare || !(__builtin_fabsf(x[e]) < 120.0f);      // |x| >= 120, inf, NaN
-            }
-            if (__builtin_expect(rare, 0)) {
-                for (int e = 0; e < N; ++e)
-                    if (cta_sincos_is_rare(x[e])) c[e] = cta_sincosf(x[e], want_cos, t.inv_pio4);
-            }
-            break;
-        }
+        case CTAMD_EX_SIN: sin_or_cos<FASTM, 0>(c, t); break;       // two cases: the compiler then knows which of the two it builds
+        case CTAMD_EX_COS: sin_or_cos<FASTM, 1>(c, t); break;
         case CTAMD_EX_ADDS: each(c, [&](int e) { return c[e] + q.imm; }); break;
         case CTAMD_EX_MULS: each(c, [&](int e) { return c[e] * q.imm; }); break;
         case CTAMD_EX_DIVS: each(c, [&](int e) { return cta_div_rcp(c[e], q.rcp); }); break;
