@@ -57,7 +57,17 @@ struct DevInsn {
 };
 static_assert(sizeof(DevInsn) == 16, "one 128-bit scalar load per instruction");
 
-struct ExprArgs {
+// An instruction as the kernel holds it: fetched with ONE 128-bit load through the scalar unit and
+// taken apart with scalar bit operations.  (Read field by field, the 8- and 16-bit members came
+// through the vector memory path: every fetch then waited on the vector memory counter, which also
+// counts the loads issued a pass ahead.)
+struct Insn {
+    uint32_t op, flags, dst, a, b;
+    float imm;
+    double rcp;
+};
+
+struct alignas(16) ExprArgs {
     const float* in[kMaxPorts];
     float* out[kMaxPorts];
     int32_t* status;
@@ -67,8 +77,22 @@ struct ExprArgs {
     int has_row;                              // the program loads a row vector
     int n_lead;                               // the first n_lead instructions are loads (at most kLeadLoads)
     int n_tail;                               // VEC: the last n_tail instructions are stores (at most kTailStores)
-    DevInsn prog[kMaxInsns + 1];              // one spare: the kernel fetches an instruction ahead
+    alignas(16) DevInsn prog[kMaxInsns + 1];  // one spare: the kernel fetches an instruction ahead
 };
+
+__device__ __forceinline__ Insn fetch_insn(const ExprArgs& g, int pc) {
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    const u4 w = *reinterpret_cast<const u4*>(&g.prog[pc]);
+    Insn q;
+    q.op = w[0] & 0xffu;
+    q.flags = (w[0] >> 8) & 0xffu;
+    q.dst = w[0] >> 16;
+    q.a = w[1] & 0xffffu;
+    q.b = w[1] >> 16;
+    q.imm = __uint_as_float(w[2]);
+    q.rcp = __hiloint2double(int(w[3]), int(w[2]));
+    return q;
+}
 
 // One operator on the N elements of a lane, in place: c holds operand a on entry and the result on
 // return, b the second operand of the two-operand operators.  The operator is chosen once (a
@@ -100,7 +124,7 @@ __device__ __forceinline__ void sin_or_cos(float (&c)[N], const Tables& t) {
 }
 
 template <bool FASTM, int N>
-__device__ __forceinline__ void apply(const DevInsn& q, float (&c)[N], const float (&b)[N], const Tables& t) {
+__device__ __forceinline__ void apply(const Insn& q, float (&c)[N], const float (&b)[N], const Tables& t) {
     switch (q.op) {
         case CTAMD_EX_ADD: each(c, [&](int e) { return c[e] + b[e]; }); break;
         case CTAMD_EX_SUB: each(c, [&](int e) { return c[e] - b[e]; }); break;
@@ -149,7 +173,7 @@ struct Place {
 };
 
 template <bool VEC, int H>
-__device__ __forceinline__ Vals<H> load_elements(const ExprArgs& g, const DevInsn& q, const Place<VEC, H>& at) {
+__device__ __forceinline__ Vals<H> load_elements(const ExprArgs& g, const Insn& q, const Place<VEC, H>& at) {
     const float* __restrict__ src = g.in[q.a];
     const bool row = (q.op == CTAMD_EX_LOAD_ROW);
     Vals<H> v;
@@ -226,7 +250,7 @@ __global__ __launch_bounds__(kExprThreads, FASTM ? 4 : 3) void expr_kernel(ExprA
     auto issue_lead = [&]() {
 #pragma unroll
         for (int k = 0; k < kLeadLoads; ++k)
-            if (k < g.n_lead) pre[k] = load_elements<VEC, H>(g, g.prog[k], next);
+            if (k < g.n_lead) pre[k] = load_elements<VEC, H>(g, fetch_insn(g, k), next);
     };
     // The stores at the end of the program go out one pass late, just before the next loads: the
     // memory counter of this hardware counts loads and stores in one order, so waiting for a
@@ -239,7 +263,7 @@ __global__ __launch_bounds__(kExprThreads, FASTM ? 4 : 3) void expr_kernel(ExprA
 #pragma unroll
             for (int k = 0; k < kTailStores; ++k)
                 if (k < g.n_tail) {
-                    v4f* __restrict__ dst = reinterpret_cast<v4f*>(g.out[g.prog[g.n_insn - g.n_tail + k].dst]) + post_at;
+                    v4f* __restrict__ dst = reinterpret_cast<v4f*>(g.out[fetch_insn(g, g.n_insn - g.n_tail + k).dst]) + post_at;
 #pragma unroll
                     for (int h = 0; h < H; ++h)
                         if (post_full[h]) __builtin_nontemporal_store(post[k].h[h], dst + h * kExprThreads);
@@ -265,17 +289,17 @@ __global__ __launch_bounds__(kExprThreads, FASTM ? 4 : 3) void expr_kernel(ExprA
         __builtin_amdgcn_s_waitcnt(0x0F70);
 #pragma unroll
         for (int k = 0; k < kLeadLoads; ++k)
-            if (k < g.n_lead) put(g.prog[k].dst, pre[k]);
+            if (k < g.n_lead) put(fetch_insn(g, k).dst, pre[k]);
         advance(next);
         issue_tail();
         if (pass + gridDim.x < passes) issue_lead();
         bool inside[H];
 #pragma unroll
         for (int h = 0; h < H; ++h) inside[h] = VEC ? (at.first + size_t(h) * kExprThreads < g.total / 4) : true;
-        DevInsn fetched = g.prog[g.n_lead];    // instructions are fetched one ahead of their execution (the array has a spare entry)
+        Insn fetched = fetch_insn(g, g.n_lead);    // instructions are fetched one ahead of their execution (the array has a spare entry)
         for (int pc = g.n_lead; pc < n_body; ++pc) {
-            const DevInsn q = fetched;
-            fetched = g.prog[pc + 1];
+            const Insn q = fetched;
+            fetched = fetch_insn(g, pc + 1);
             if (q.op == CTAMD_EX_LOAD_FULL || q.op == CTAMD_EX_LOAD_ROW) {
                 carry = load_elements<VEC, H>(g, q, at);
             } else if (q.op == CTAMD_EX_STORE || q.op == CTAMD_EX_STORE_ZP) {
@@ -329,7 +353,7 @@ __global__ __launch_bounds__(kExprThreads, FASTM ? 4 : 3) void expr_kernel(ExprA
 #pragma unroll
             for (int k = 0; k < kTailStores; ++k)
                 if (k < g.n_tail) {
-                    const DevInsn q = g.prog[n_body + k];
+                    const Insn q = fetch_insn(g, n_body + k);
                     Vals<H> v = carry;
                     if (q.flags & kAFetch) v = get(q.a);
                     if (q.op == CTAMD_EX_STORE_ZP) zero_plus(v);
