@@ -17,6 +17,11 @@
 // output with a long K (the weight gradients of a small layer) - are cut along K into parts, one
 // block each, so that they fill the chip; the parts go to the device scratch and a second launch
 // adds them in a fixed order, so results stay deterministic.
+//
+// Two families of products do not go through those tiles (matmul_impl picks): a product of at most
+// one 32 x 32 tile per CU with a short K (gemm_micro: the waves of a block share out K and feed the
+// MFMAs from global memory directly), and a product with at most 16 output columns
+// (gemm_narrow_rows / gemm_narrow_cols: fp32 FMAs on the vector units, A streamed once).
 #include "common.h"
 
 
@@ -435,6 +440,361 @@ __global__ __launch_bounds__(kThreads) void fold_parts(GemmArgs g) {
     }
 }
 
+// ---- Small products: at most one 32 x 32 tile of C per CU.  The big tiles put such a product on a
+// handful of CUs, where it runs at those CUs' MFMA rate, or cut K over blocks and pay a second
+// launch to add the parts.  Here a block owns one 32 x 32 tile and its 16 waves share out K in
+// runs of 32-wide spans: every wave feeds its MFMA operands straight from global memory - lane l
+// holds row / column l % 32 at the 16 consecutive k of its half of the span (the sum over k is
+// order-free, so both operands simply use the same labelling; an operand contiguous in k is read
+// 64 bytes per lane) - with one span being multiplied while the next is on its way, and the 16
+// accumulator tiles are added in order through LDS.
+constexpr int kMicroWaves = 16;
+constexpr int kMicroSpan = 32;
+constexpr int kMicroMaxK = 512;
+struct MicroArgs {
+    const float* a; int64_t lda;       // lda, ldb: as in GemmArgs
+    const float* b; int64_t ldb;
+    float* c;
+    int m, n, k, tiles_m;
+    int spans_per_wave;
+    const float* bias; int relu;
+};
+// f[i] = operand element (x, k0 + i), i < 16; zeros past k or when x is outside the matrix
+template <bool KC, bool VEC>
+__device__ __forceinline__ void micro_fetch(const float* __restrict__ p, int64_t ld, int x, bool x_ok, int k0, int k, float (&f)[16]) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) f[i] = 0.0f;
+    if (!x_ok) return;
+    if (KC) {
+        const float* __restrict__ src = p + int64_t(x) * ld + k0;
+        if (VEC && k0 + 16 <= k) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const v4f v = reinterpret_cast<const v4f*>(src)[q];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) f[4 * q + e] = v[e];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                if (k0 + i < k) f[i] = src[i];
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            if (k0 + i < k) f[i] = p[int64_t(k0 + i) * ld + x];
+    }
+}
+template <bool A_KC, bool B_KC, bool VEC>
+__global__ __launch_bounds__(kMicroWaves * 64) void gemm_micro(MicroArgs g) {
+    __shared__ float s_red[kMicroWaves * 16 * 64];
+    const int lane = threadIdx.x & 63, l32 = lane & 31, half = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(int(threadIdx.x) >> 6);
+    const int m0 = (blockIdx.x % g.tiles_m) * 32, n0 = (blockIdx.x / g.tiles_m) * 32;
+    const int row = m0 + l32, col = n0 + l32;
+    const bool row_ok = row < g.m, col_ok = col < g.n;
+    v16f acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+    // this wave's spans: [first, last), wave-uniform
+    const int spans = (g.k + kMicroSpan - 1) / kMicroSpan;
+    const int first = wave * g.spans_per_wave;
+    const int last = first + g.spans_per_wave < spans ? first + g.spans_per_wave : spans;
+    float fa[2][16], fb[2][16];
+    auto request = [&](int span, int buf) {
+        const int k0 = span * kMicroSpan + 16 * half;
+        micro_fetch<A_KC, VEC>(g.a, g.lda, row, row_ok, k0, g.k, fa[buf]);
+        micro_fetch<B_KC, VEC>(g.b, g.ldb, col, col_ok, k0, g.k, fb[buf]);
+    };
+    auto multiply = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[buf][i], fb[buf][i], acc, 0, 0, 0);
+    };
+    if (first < last) request(first, 0);
+    for (int sp = first; sp < last; sp += 2) {
+        if (sp + 1 < last) request(sp + 1, 1);
+        multiply(0);
+        if (sp + 1 < last) {
+            if (sp + 2 < last) request(sp + 2, 0);
+            multiply(1);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s_red[(wave * 16 + r) * 64 + lane] = acc[r];
+    __syncthreads();
+    // value t = r * 64 + l is accumulator register r of lane l: C[8 (r / 4) + 4 (l / 32) + r % 4][l % 32]
+    const int t = threadIdx.x, r = t >> 6, l = t & 63;
+    float total = s_red[t];
+#pragma unroll
+    for (int w = 1; w < kMicroWaves; ++w) total = total + s_red[w * 1024 + t];
+    const int crow = m0 + 8 * (r / 4) + 4 * (l / 32) + r % 4, ccol = n0 + (l & 31);
+    if (crow < g.m && ccol < g.n) g.c[int64_t(crow) * g.n + ccol] = epilogue(total, g.bias, ccol, g.relu);
+}
+
+template <bool A_KC, bool B_KC>
+void launch_micro(const MicroArgs& g, bool vec, dim3 grid, dim3 block, hipStream_t s) {
+    if (vec) hipLaunchKernelGGL((gemm_micro<A_KC, B_KC, true>), grid, block, 0, s, g);
+    else hipLaunchKernelGGL((gemm_micro<A_KC, B_KC, false>), grid, block, 0, s, g);
+}
+
+// ---- Products with a narrow output, n <= 16: the logits of a classifier, [B x H] . [H x 10], and
+// the gradient of its weights, [H x B] . [B x 10].  A 64 x 64 MFMA tile would compute 54 of its 64
+// columns for nothing, and with rows of 10 floats B takes the element-wise edge path; these kernels
+// stream A once on the vector units instead.  fp32 fused multiply-adds and sums in a fixed order:
+// results are deterministic and the same for every row of the output.
+constexpr int kNarrowN = 16;
+constexpr int kNarrowRows = 4;                 // rows of A a wave works on at a time
+constexpr int kNarrowLdsBytes = 64 << 10;
+
+// Sums `P` values per lane over the 64 lanes of a wave in P + log2(64 / P) exchanges instead of
+// 6 P: each step halves the values a lane still carries (the upper lanes of the pair keep the upper
+// half).  Afterwards lane l holds the total of value l / (64 / P) in v[0].
+template <int CNT, int OFF, int P>
+__device__ __forceinline__ void wave_sums_step(float (&v)[P], int lane) {
+    if constexpr (CNT > 1) {
+        const bool upper = (lane & OFF) != 0;
+#pragma unroll
+        for (int j = 0; j < CNT / 2; ++j) {
+            const float send = upper ? v[j] : v[j + CNT / 2];
+            const float keep = upper ? v[j + CNT / 2] : v[j];
+            v[j] = keep + __shfl_xor(send, OFF, 64);
+        }
+        wave_sums_step<CNT / 2, OFF / 2, P>(v, lane);
+    } else if constexpr (OFF >= 1) {
+        v[0] = v[0] + __shfl_xor(v[0], OFF, 64);
+        wave_sums_step<1, OFF / 2, P>(v, lane);
+    }
+}
+template <int P>
+__device__ __forceinline__ void wave_sums(float (&v)[P], int lane) {
+    static_assert(P >= 1 && P <= 64 && (P & (P - 1)) == 0, "a power of two");
+    wave_sums_step<P, 32, P>(v, lane);
+}
+constexpr int pow2_at_least(int v) { return v <= 1 ? 1 : 2 * pow2_at_least((v + 1) / 2); }
+
+// A K-contiguous (row-major [m, k]), B in rows of n.  B is staged transposed into LDS as [n][kp]
+// (kp: k rounded up to the 256-wide slab, zeros behind k).  A wave takes kNarrowRows rows at a time:
+// lane l holds A[row][k0 + 4l .. 4l + 3] of a slab and the 4 x n values of B those k meet, and the
+// rows' n partial sums go round the wave.  VEC: rows of A are 16-byte aligned.  ONE_SLAB: k <= 256,
+// B stays in registers for all rows and the next rows of A are requested while these are multiplied.
+template <int N, bool VEC, bool ONE_SLAB>
+__global__ __launch_bounds__(kThreads) void gemm_narrow_rows(const float* __restrict__ a, int64_t lda, const float* __restrict__ b,
+                                                             int64_t ldb, float* __restrict__ c, int m, int k, int kp,
+                                                             int turns, const float* __restrict__ bias, int relu) {
+    extern __shared__ __attribute__((aligned(16))) float s_bt[];        // [N][kp]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    constexpr int R = kNarrowRows;
+    // the block's waves take consecutive groups of R rows, `turns` groups each, a block's rows in one run
+    const int first = (blockIdx.x * (kThreads / 64) * turns + wave) * R;
+    const int stride = (kThreads / 64) * R;
+    auto load_rows = [&](int row0, int k0, v4f (&av)[R]) {
+        const int kk = k0 + 4 * lane;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (row0 + r < m) {
+                const float* src = a + int64_t(row0 + r) * lda + kk;
+                if (VEC && kk + 4 <= k) v = *reinterpret_cast<const v4f*>(src);
+                else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (kk + e < k) v[e] = src[e];
+                }
+            }
+            av[r] = v;
+        }
+    };
+    v4f av[R];
+    if (ONE_SLAB) load_rows(first, 0, av);                     // on its way while B is staged
+    for (int e = threadIdx.x; e < kp * N; e += kThreads) {
+        const int l = e / N, q = e % N;
+        s_bt[q * kp + l] = l < k ? b[int64_t(l) * ldb + q] : 0.0f;
+    }
+    __syncthreads();
+    v4f bw[N];
+    if (ONE_SLAB) {
+#pragma unroll
+        for (int q = 0; q < N; ++q) bw[q] = *reinterpret_cast<const v4f*>(s_bt + q * kp + 4 * lane);
+    }
+    constexpr int P = pow2_at_least(R * N);
+    for (int t = 0; t < turns; ++t) {
+        const int row0 = first + t * stride;
+        if (row0 >= m) break;                                  // wave-uniform
+        float acc[P];
+#pragma unroll
+        for (int v = 0; v < P; ++v) acc[v] = 0.0f;
+        if (ONE_SLAB) {
+            v4f next[R];
+            if (t + 1 < turns) load_rows(row0 + stride, 0, next);
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int q = 0; q < N; ++q)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[r * N + q] = __fmaf_rn(av[r][e], bw[q][e], acc[r * N + q]);
+            if (t + 1 < turns) {
+#pragma unroll
+                for (int r = 0; r < R; ++r) av[r] = next[r];
+            }
+        } else {
+            for (int k0 = 0; k0 < k; k0 += 256) {
+                load_rows(row0, k0, av);
+#pragma unroll
+                for (int q = 0; q < N; ++q) {
+                    const v4f w = *reinterpret_cast<const v4f*>(s_bt + q * kp + k0 + 4 * lane);
+#pragma unroll
+                    for (int r = 0; r < R; ++r)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[r * N + q] = __fmaf_rn(av[r][e], w[e], acc[r * N + q]);
+                }
+            }
+        }
+        wave_sums<P>(acc, lane);
+        constexpr int kLanesPerValue = 64 / P;
+        const int v = lane / kLanesPerValue;
+        if (lane % kLanesPerValue == 0 && v < R * N && row0 + v / N < m)
+            c[int64_t(row0 + v / N) * N + v % N] = epilogue(acc[0], bias, v % N, relu);
+    }
+}
+
+// A X-contiguous (the transposed view of a row-major [k, m]), B in rows of n.  A block of 16 waves
+// owns 64 rows i of the output and a run of k; wave w takes l = w, w + 16, ... of the run, lane j
+// reads A[l][i0 + j] (a wave reads 256 contiguous bytes, eight l in flight and the next eight
+// requested) and multiplies it with B's row l, which all lanes read from LDS at one address.  The
+// 16 waves' sums are added in order through the same LDS.  With the k range cut in several runs
+// (gridDim.y) the results go to `out` as [run][m * n] and gemm_narrow_fold adds the runs.
+constexpr int kNarrowWaves = 16;
+template <int N>
+__global__ __launch_bounds__(kNarrowWaves * 64) void gemm_narrow_cols(const float* __restrict__ a, int64_t lda,
+                                                                      const float* __restrict__ b, int64_t ldb,
+                                                                      float* __restrict__ out, int m, int k, int k_per_run,
+                                                                      const float* __restrict__ bias, int relu) {
+    constexpr int kChunk = kNarrowWaves * 64;                  // rows of B resident at a time
+    __shared__ float s_mem[kChunk * N];                        // B's rows [kChunk][N]; at the end the sums [wave][N][64]
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(int(threadIdx.x) >> 6);
+    const int i = blockIdx.x * 64 + lane;
+    const int k_begin = blockIdx.y * k_per_run;
+    const int k_end = k_begin + k_per_run < k ? k_begin + k_per_run : k;
+    constexpr int kAhead = 8, kStep = kNarrowWaves * kAhead;
+    float acc[N];
+#pragma unroll
+    for (int q = 0; q < N; ++q) acc[q] = 0.0f;
+    const bool mine = i < m;
+    for (int c0 = k_begin; c0 < k_end; c0 += kChunk) {
+        const int len = k_end - c0 < kChunk ? k_end - c0 : kChunk;
+        const float* __restrict__ a0 = a + int64_t(c0) * lda + i;
+        auto request = [&](int l0, float (&av)[kAhead]) {
+#pragma unroll
+            for (int u = 0; u < kAhead; ++u) {
+                const int l = l0 + u * kNarrowWaves;
+                av[u] = (mine && l < len) ? a0[int64_t(l) * lda] : 0.0f;
+            }
+        };
+        float av[kAhead];
+        request(wave, av);                                     // on its way while B's rows are staged
+        if (c0 != k_begin) __syncthreads();
+        for (int e = threadIdx.x; e < len * N; e += kNarrowWaves * 64) s_mem[e] = b[int64_t(c0 + e / N) * ldb + e % N];
+        __syncthreads();
+        for (int l0 = wave; l0 < len; l0 += kStep) {
+            float next[kAhead];
+            if (l0 + kStep < len) request(l0 + kStep, next);
+#pragma unroll
+            for (int u = 0; u < kAhead; ++u) {
+                const int l = l0 + u * kNarrowWaves;
+                if (l < len) {                                 // wave-uniform
+#pragma unroll
+                    for (int q = 0; q < N; ++q) acc[q] = __fmaf_rn(av[u], s_mem[l * N + q], acc[q]);
+                }
+            }
+            if (l0 + kStep < len) {
+#pragma unroll
+                for (int u = 0; u < kAhead; ++u) av[u] = next[u];
+            }
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < N; ++q) s_mem[(wave * N + q) * 64 + lane] = acc[q];
+    __syncthreads();
+    const int t = threadIdx.x;
+    if (t >= 64 * N) return;
+    const int j = t / N, q = t % N;
+    if (blockIdx.x * 64 + j >= m) return;
+    float total = s_mem[q * 64 + j];
+#pragma unroll
+    for (int w = 1; w < kNarrowWaves; ++w) total = total + s_mem[(w * N + q) * 64 + j];
+    const size_t e = size_t(blockIdx.x) * 64 * N + t;          // = (i0 + j) * N + q
+    if (gridDim.y > 1) out[size_t(blockIdx.y) * size_t(m) * N + e] = total;
+    else out[e] = epilogue(total, bias, q, relu);
+}
+// 16 lanes per output element: lane j adds runs j, j + 16, ... in order, then the 16 go round.
+template <int N>
+__global__ __launch_bounds__(kThreads) void gemm_narrow_fold(const float* __restrict__ partial, float* __restrict__ c, int m, int runs,
+                                                             const float* __restrict__ bias, int relu) {
+    const size_t mn = size_t(m) * N;
+    const size_t e = (size_t(blockIdx.x) * kThreads + threadIdx.x) / 16;
+    const int j = threadIdx.x % 16;
+    float t = 0.0f;
+    if (e < mn) {
+        for (int z = j; z < runs; z += 16 * 4) {
+            float p[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) p[u] = z + 16 * u < runs ? partial[size_t(z + 16 * u) * mn + e] : 0.0f;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) t = t + p[u];
+        }
+    }
+#pragma unroll
+    for (int off = 8; off >= 1; off /= 2) t = t + __shfl_xor(t, off, 64);
+    if (e < mn && j == 0) c[e] = epilogue(t, bias, int(e % N), relu);
+}
+
+template <int N>
+int launch_narrow(const char* name, bool rows_form, const float* a, int64_t lda, const float* b, int64_t ldb, const float* bias, int relu,
+                  float* c, int m, int k, void* stream) {
+    hipStream_t s = as_stream(stream);
+    const int cus = compute_units() > 0 ? compute_units() : 256;
+    if (rows_form) {
+        const int kp = (k + 255) / 256 * 256;
+        const int groups = (m + kNarrowRows - 1) / kNarrowRows;          // of kNarrowRows rows, one wave each
+        const int waves = cus * (kThreads / 64);
+        const int turns = (groups + waves - 1) / waves;
+        const int blocks = (groups + turns * (kThreads / 64) - 1) / (turns * (kThreads / 64));
+        const size_t lds = size_t(N) * kp * sizeof(float);
+        const bool vec = aligned16(a) && lda % 4 == 0;
+        auto kernel = k <= 256 ? (vec ? gemm_narrow_rows<N, true, true> : gemm_narrow_rows<N, false, true>)
+                               : (vec ? gemm_narrow_rows<N, true, false> : gemm_narrow_rows<N, false, false>);
+        hipLaunchKernelGGL(kernel, dim3(unsigned(blocks)), dim3(kThreads), lds, s, a, lda, b, ldb, c, m, k, kp, turns, bias, relu);
+        return launched(name);
+    }
+    const int strips = (m + 63) / 64;
+    // one run while a wave's share of k is short (a second launch costs more than it saves);
+    // otherwise about one block per CU, and no run shorter than 128
+    int runs = 1;
+    if (k > 512) {
+        runs = (cus + strips - 1) / strips;
+        if (runs > k / 128) runs = k / 128;
+        const size_t by_scratch = kScratchFloats / (size_t(m) * N);
+        if (size_t(runs) > by_scratch) runs = int(by_scratch);
+        if (runs < 1) runs = 1;
+    }
+    const int k_per_run = (k + runs - 1) / runs;
+    runs = (k + k_per_run - 1) / k_per_run;
+    float* partial = nullptr;
+    if (runs > 1) {
+        partial = scratch(stream);
+        if (!partial) return CTAMD_EINVAL;
+    }
+    hipLaunchKernelGGL(gemm_narrow_cols<N>, dim3(unsigned(strips), unsigned(runs)), dim3(kNarrowWaves * 64), 0, s, a, lda, b, ldb,
+                       runs > 1 ? partial : c, m, k, k_per_run, bias, relu);
+    int rc = launched(name);
+    if (rc || runs == 1) return rc;
+    hipLaunchKernelGGL(gemm_narrow_fold<N>, dim3(unsigned((size_t(m) * N * 16 + kThreads - 1) / kThreads)), dim3(kThreads), 0, s,
+                       partial, c, m, runs, bias, relu);
+    return launched(name);
+}
+
 // Operands with no unit stride: one thread per output element.  Correct for any strides; only
 // the reference's own transposes of transposes could produce such views.
 __global__ __launch_bounds__(kThreads) void gemm_strided(const float* __restrict__ a, int64_t as0, int64_t as1,
@@ -518,6 +878,45 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
     }
     const bool A_KC = a_kc, B_KC = !b_xc;
     const int cus = compute_units() > 0 ? compute_units() : 256;
+    {
+        // one tile per CU at most, and a K a CU can stream by itself: a CU draws some tens of GB/s, and a
+        // 32 x 32 tile needs 256 bytes per k - beyond a few hundred k the tiled plan's cut of K over
+        // many CUs (and its second launch) is the faster way
+        const int64_t tiles32 = ((m + 31) / 32) * ((n + 31) / 32);
+        const bool use = tiles32 <= cus && k <= kMicroMaxK;
+        if (use) {
+            MicroArgs g;
+            g.a = a; g.lda = A_KC ? as0 : as1;
+            g.b = b; g.ldb = B_KC ? bs1 : bs0;
+            g.c = c; g.m = int(m); g.n = int(n); g.k = int(k);
+            g.tiles_m = int((m + 31) / 32);
+            const int spans = int((k + kMicroSpan - 1) / kMicroSpan);
+            g.spans_per_wave = (spans + kMicroWaves - 1) / kMicroWaves;
+            g.bias = bias; g.relu = relu;
+            const bool vec = (!A_KC || (aligned16(a) && g.lda % 4 == 0)) && (!B_KC || (aligned16(b) && g.ldb % 4 == 0));
+            const dim3 grid{unsigned(tiles32)}, block{unsigned(kMicroWaves * 64)};
+            if (A_KC && B_KC) launch_micro<true, true>(g, vec, grid, block, s);
+            else if (A_KC) launch_micro<true, false>(g, vec, grid, block, s);
+            else if (B_KC) launch_micro<false, true>(g, vec, grid, block, s);
+            else launch_micro<false, false>(g, vec, grid, block, s);
+            return launched(name);
+        }
+    }
+    // a narrow output from a B in rows of n: the streaming kernels
+    if (n <= kNarrowN && bs1 == 1 && m < (int64_t(1) << 27)) {
+        const bool rows_form = (as1 == 1 || k == 1) && size_t(n) * size_t((k + 255) / 256 * 256) * sizeof(float) <= size_t(kNarrowLdsBytes);
+        const bool cols_form = as0 == 1 && as1 != 1;
+        if (rows_form || cols_form) {
+            const int64_t lda = rows_form ? as0 : as1;
+            switch (n) {
+#define CTAMD_NARROW(N_) case N_: return launch_narrow<N_>(name, rows_form, a, lda, b, bs0, bias, relu, c, int(m), int(k), stream);
+                CTAMD_NARROW(1) CTAMD_NARROW(2) CTAMD_NARROW(3) CTAMD_NARROW(4) CTAMD_NARROW(5) CTAMD_NARROW(6) CTAMD_NARROW(7) CTAMD_NARROW(8)
+                CTAMD_NARROW(9) CTAMD_NARROW(10) CTAMD_NARROW(11) CTAMD_NARROW(12) CTAMD_NARROW(13) CTAMD_NARROW(14) CTAMD_NARROW(15) CTAMD_NARROW(16)
+#undef CTAMD_NARROW
+                default: break;
+            }
+        }
+    }
     constexpr int BK = 16;
     static_assert(BigTile::BK == BK && WideTile::BK == BK && SmallTile::BK == BK && TinyTile::BK == BK, "all tile shapes step K alike");
     // The plan: a tile shape, and into how many parts along K the tiles of the last, partly filled
@@ -595,6 +994,8 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
         if (size_t(tiles - whole_tiles) * size_t(splits) * size_t(BM) * size_t(BN) > kScratchFloats)
             return fail(CTAMD_ERANGE, "%s: the parts of %d split tiles do not fit the device scratch", name, tiles - whole_tiles);
     }
+    // a tile outside [0, whole_tiles) writes its parts to g.partial: there is none unless the plan cut K
+    if (splits == 1 && whole_tiles != tiles) return fail(CTAMD_EINVAL, "%s: plan leaves %d tiles without a part buffer", name, tiles - whole_tiles);
     const int blocks = whole_tiles + (tiles - whole_tiles) * splits;
     int rc = shape == 3 ? launch_layout<WideTile>(g, A_KC, B_KC, vec, blocks, s)
            : shape == 2 ? launch_layout<BigTile>(g, A_KC, B_KC, vec, blocks, s)

@@ -473,7 +473,15 @@ MM_SHAPES = [(1, 1, 1), (5, 3, 9), (33, 29, 47), (128, 128, 16), (130, 257, 70),
              (784, 256, 300), (256, 10, 8192), (17, 1, 33), (1, 40, 33), (200, 200, 1), (384, 512, 1024),
              # ragged edges and a K that is no multiple of the k tile, for the 128 x 128, the 256 x 256 and
              # the 256 x 128 tile shapes (the launcher picks by rounds of tiles per CU)
-             (2049, 2050, 33), (4100, 4101, 70), (4090, 4093, 40), (4090, 2047, 40)]
+             (2049, 2050, 33), (4100, 4101, 70), (4090, 4093, 40), (4090, 2047, 40),
+             # an output of at most 16 columns: the streaming kernels, in rows (A row-major) and in
+             # columns (A a transposed view) with and without a cut K, ragged m and k
+             (8192, 10, 256), (8190, 16, 252), (1000, 1, 512), (70, 3, 8), (5000, 7, 52), (300, 16, 1000),
+             (777, 13, 3001), (66000, 2, 12),
+             # at most one 32 x 32 tile per CU and K <= 512: the small-product kernel (those above with
+             # small extents take it too); the same extents with a longer K stay on the 64 x 64 tiles
+             (256, 256, 256), (784, 256, 256), (100, 70, 300), (512, 512, 512), (31, 33, 512),
+             (130, 257, 600), (70, 33, 1000), (100, 70, 513)]
 
 
 @pytest.mark.parametrize("m,n,k", MM_SHAPES)
@@ -495,7 +503,8 @@ def test_matmul_all_layouts_normwise(oracle, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(256, 128, 784), (128, 10, 64), (70, 33, 129), (8192, 256, 784), (96, 12, 4096),
-                                   (2100, 2050, 40), (4090, 4093, 24), (4090, 2047, 24), (5, 7, 0)])
+                                   (2100, 2050, 40), (4090, 4093, 24), (4090, 2047, 24), (5, 7, 0),
+                                   (8192, 10, 256), (256, 10, 8192), (777, 13, 3001), (256, 256, 256), (100, 70, 300)])
 def test_fused_layer_equals_the_three_launches(oracle, m, n, k):
     """matmul + bias row + ReLU in one launch against the same three operators launched in sequence,
     bit for bit, over all tile shapes, the K-split fold ((96, 12, 4096)) and ragged edges; and against
@@ -506,7 +515,8 @@ def test_fused_layer_equals_the_three_launches(oracle, m, n, k):
     bias = oracle.normal((n,), 63)
     dA, dB, db = G.dev(A), G.dev(B), G.dev(bias)
     dBt = G.dev(np.ascontiguousarray(B.T))
-    for a, b in ((dA, dB), (dA, dBt.t())):
+    dAt = G.dev(np.ascontiguousarray(A.T))
+    for a, b in ((dA, dB), (dA, dBt.t()), (dAt.t(), dB)):
         plain = G.matmul(a, b)
         biased = G.rowbcast("add", plain, db)
         assert same_bits(G.host(G.matmul_bias(a, b, None, False)), G.host(plain))
@@ -529,6 +539,10 @@ def test_matmul_exact_on_small_integers_and_unaligned_views(oracle):
     # row-sliced views: unit inner stride, leading dimension larger than the extent
     Abig, Bbig = G.dev(np.pad(A, ((0, 0), (0, 5)))), G.dev(np.pad(B, ((0, 0), (0, 3))))
     assert np.array_equal(G.host(G.matmul(Abig[:, :203], Bbig[:, :77])), want)
+    # a narrow output from row-sliced views (leading dimensions 208 and 80), A in rows and in columns
+    assert np.array_equal(G.host(G.matmul(Abig[:, :203], Bbig[:, :9])), want[:, :9])
+    Atbig = G.dev(np.pad(np.ascontiguousarray(A.T), ((0, 0), (0, 6))))
+    assert np.array_equal(G.host(G.matmul(Atbig[:, :150].t(), Bbig[:, :9])), want[:, :9])
     # no unit stride at all: generic kernel
     A2, B2 = G.dev(np.repeat(A, 2, axis=1)), G.dev(np.repeat(B, 2, axis=1))
     At2 = G.dev(np.repeat(np.ascontiguousarray(A.T), 2, axis=1))
