@@ -845,9 +845,19 @@ __global__ __launch_bounds__(256) void loss_stage2(const double* __restrict__ pa
                                                    float* __restrict__ out, int32_t* __restrict__ status) {
     __shared__ double s_d[256 / 64 + 1];
     double t = 0.0, bad = 0.0;
-    for (unsigned i = threadIdx.x; i < count; i += 256) t += partials[i];
-    if (status)
-        for (unsigned i = threadIdx.x; i < count; i += 256) bad += partials[count + i];
+    // eight loads (sixteen with the flags) in flight, added in the order of i
+    for (unsigned i0 = threadIdx.x; i0 < count; i0 += 256 * 8) {
+        double p[8], f[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const unsigned i = i0 + 256u * u;
+            p[u] = i < count ? partials[i] : 0.0;
+            f[u] = (status && i < count) ? partials[count + i] : 0.0;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (i0 + 256u * u < count) { t += p[u]; bad += f[u]; }
+    }
     t = block_sum<256>(t, s_d);
     if (status) {
         __syncthreads();
