@@ -155,6 +155,7 @@ struct GemmArgs {
     int c_vec;                      // rows of C are 16-byte aligned
     const float* bias;              // optional row vector [n] added to every row of C (null: none)
     int relu;                       // then max(0, .) when set
+    const float* mask;              // optional [m, n] row-major: C is multiplied by [mask > 0] last (null: none)
 };
 
 // Output epilogue of a product that is not split along K: bias add, then ReLU as `v > 0 ? v : +0`
@@ -164,6 +165,11 @@ __device__ __forceinline__ float epilogue(float v, const float* __restrict__ bia
     if (bias) v = v + bias[col];
     if (relu) v = v > 0.0f ? v : 0.0f;
     return v;
+}
+// The gradient of a ReLU applied to a product that has just been formed: v * [y > 0] with the 0 / 1
+// factor the separate kernel multiplies by (a zero keeps v's sign, NaN and infinities give NaN).
+__device__ __forceinline__ float masked(float v, const float* __restrict__ mask, int64_t at) {
+    return mask ? v * (mask[at] > 0.0f ? 1.0f : 0.0f) : v;
 }
 
 template <class C, bool A_KC, bool B_KC, bool VEC>
@@ -373,7 +379,8 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int row = m0 + wm + i * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-                    if (row < g.m && col < g.n) g.c[int64_t(row) * g.ldc + col] = epilogue(acc[i][j][r], g.bias, col, g.relu);
+                    if (row < g.m && col < g.n)
+                        g.c[int64_t(row) * g.ldc + col] = masked(epilogue(acc[i][j][r], g.bias, col, g.relu), g.mask, int64_t(row) * g.ldc + col);
                 }
             }
         return;
@@ -428,7 +435,7 @@ __global__ __launch_bounds__(kThreads) void fold_parts(GemmArgs g) {
         for (; z < g.splits; ++z) t = t + src[size_t(z) * kStep];
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-            if (gcol + e < g.n) t[e] = epilogue(t[e], g.bias, gcol + e, g.relu);
+            if (gcol + e < g.n) t[e] = masked(epilogue(t[e], g.bias, gcol + e, g.relu), g.mask, int64_t(grow) * g.ldc + gcol + e);
         float* __restrict__ dst = g.c + int64_t(grow) * g.ldc + gcol;
         if (g.c_vec && gcol + 4 <= g.n) {
             *reinterpret_cast<v4f*>(dst) = t;
@@ -458,6 +465,7 @@ struct MicroArgs {
     int m, n, k, tiles_m;
     int spans_per_wave;
     const float* bias; int relu;
+    const float* mask;                 // as in GemmArgs
 };
 // f[i] = operand element (x, k0 + i), i < 16; zeros past k or when x is outside the matrix
 template <bool KC, bool VEC>
@@ -528,7 +536,8 @@ __global__ __launch_bounds__(kMicroWaves * 64) void gemm_micro(MicroArgs g) {
 #pragma unroll
     for (int w = 1; w < kMicroWaves; ++w) total = total + s_red[w * 1024 + t];
     const int crow = m0 + 8 * (r / 4) + 4 * (l / 32) + r % 4, ccol = n0 + (l & 31);
-    if (crow < g.m && ccol < g.n) g.c[int64_t(crow) * g.n + ccol] = epilogue(total, g.bias, ccol, g.relu);
+    if (crow < g.m && ccol < g.n)
+        g.c[int64_t(crow) * g.n + ccol] = masked(epilogue(total, g.bias, ccol, g.relu), g.mask, int64_t(crow) * g.n + ccol);
 }
 
 template <bool A_KC, bool B_KC>
@@ -850,7 +859,7 @@ namespace {
 // C = A.B, optionally followed by "+ bias row" and ReLU in the same launch (in the fold launch when
 // the product is split along K).
 int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,
-                const float* bias, int relu, float* c, int64_t m, int64_t n, int64_t k, void* stream) {
+                const float* bias, int relu, const float* mask, float* c, int64_t m, int64_t n, int64_t k, void* stream) {
     if (m < 0 || n < 0 || k < 0) return fail(CTAMD_EINVAL, "%s: negative extent", name);
     if (m == 0 || n == 0) return CTAMD_OK;
     if (!c) return fail(CTAMD_EINVAL, "%s: null output", name);
@@ -860,6 +869,7 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
         int rc = ctamd_fill_f32(c, 0.0f, size_t(m) * size_t(n), stream);
         if (!rc && bias) rc = ctamd_add_rowbcast_f32(c, bias, c, size_t(m), size_t(n), stream);
         if (!rc && relu) rc = ctamd_relu_f32(c, c, size_t(m) * size_t(n), stream);
+        if (!rc && mask) rc = ctamd_relu_backward_f32(mask, c, c, size_t(m) * size_t(n), stream);
         return rc;
     }
     if (!a || !b) return fail(CTAMD_EINVAL, "%s: null input", name);
@@ -874,7 +884,9 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
     if (!(a_kc || a_xc) || !(b_kc || b_xc)) {
         hipLaunchKernelGGL(gemm_strided, dim3(unsigned((size_t(m) * n + kThreads - 1) / kThreads)), dim3(kThreads), 0, s,
                            a, as0, as1, b, bs0, bs1, c, int(m), int(n), int(k), bias, relu);
-        return launched(name);
+        int rc = launched(name);
+        if (!rc && mask) rc = ctamd_relu_backward_f32(mask, c, c, size_t(m) * size_t(n), stream);   // in place, as its own launch
+        return rc;
     }
     const bool A_KC = a_kc, B_KC = !b_xc;
     const int cus = compute_units() > 0 ? compute_units() : 256;
@@ -892,7 +904,7 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
             g.tiles_m = int((m + 31) / 32);
             const int spans = int((k + kMicroSpan - 1) / kMicroSpan);
             g.spans_per_wave = (spans + kMicroWaves - 1) / kMicroWaves;
-            g.bias = bias; g.relu = relu;
+            g.bias = bias; g.relu = relu; g.mask = mask;
             const bool vec = (!A_KC || (aligned16(a) && g.lda % 4 == 0)) && (!B_KC || (aligned16(b) && g.ldb % 4 == 0));
             const dim3 grid{unsigned(tiles32)}, block{unsigned(kMicroWaves * 64)};
             if (A_KC && B_KC) launch_micro<true, true>(g, vec, grid, block, s);
@@ -908,13 +920,16 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
         const bool cols_form = as0 == 1 && as1 != 1;
         if (rows_form || cols_form) {
             const int64_t lda = rows_form ? as0 : as1;
+            int rc = CTAMD_OK;
             switch (n) {
-#define CTAMD_NARROW(N_) case N_: return launch_narrow<N_>(name, rows_form, a, lda, b, bs0, bias, relu, c, int(m), int(k), stream);
+#define CTAMD_NARROW(N_) case N_: rc = launch_narrow<N_>(name, rows_form, a, lda, b, bs0, bias, relu, c, int(m), int(k), stream); break;
                 CTAMD_NARROW(1) CTAMD_NARROW(2) CTAMD_NARROW(3) CTAMD_NARROW(4) CTAMD_NARROW(5) CTAMD_NARROW(6) CTAMD_NARROW(7) CTAMD_NARROW(8)
                 CTAMD_NARROW(9) CTAMD_NARROW(10) CTAMD_NARROW(11) CTAMD_NARROW(12) CTAMD_NARROW(13) CTAMD_NARROW(14) CTAMD_NARROW(15) CTAMD_NARROW(16)
 #undef CTAMD_NARROW
                 default: break;
             }
+            if (!rc && mask) rc = ctamd_relu_backward_f32(mask, c, c, size_t(m) * size_t(n), stream);   // in place, as its own launch
+            return rc;
         }
     }
     constexpr int BK = 16;
@@ -976,7 +991,7 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
     g.m = int(m); g.n = int(n); g.k = int(k);
     g.tiles_m = int((m + BM - 1) / BM);
     g.tiles_n = int((n + BN - 1) / BN);
-    g.bias = bias; g.relu = relu;
+    g.bias = bias; g.relu = relu; g.mask = mask;
     g.c_vec = (aligned16(c) && n % 4 == 0) ? 1 : 0;
     const bool vec = aligned16(a) && aligned16(b) && (g.lda % 4 == 0) && (g.ldb % 4 == 0);
     const int tiles = g.tiles_m * g.tiles_n;
@@ -1014,11 +1029,17 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
 
 extern "C" int ctamd_matmul_f32(const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,
                                 float* c, int64_t m, int64_t n, int64_t k, void* stream) {
-    return matmul_impl(__func__, a, as0, as1, b, bs0, bs1, nullptr, 0, c, m, n, k, stream);
+    return matmul_impl(__func__, a, as0, as1, b, bs0, bs1, nullptr, 0, nullptr, c, m, n, k, stream);
 }
 
 extern "C" int ctamd_matmul_bias_f32(const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,
                                      const float* bias, int relu, float* c, int64_t m, int64_t n, int64_t k,
                                      void* stream) {
-    return matmul_impl(__func__, a, as0, as1, b, bs0, bs1, bias, relu ? 1 : 0, c, m, n, k, stream);
+    return matmul_impl(__func__, a, as0, as1, b, bs0, bs1, bias, relu ? 1 : 0, nullptr, c, m, n, k, stream);
+}
+
+extern "C" int ctamd_matmul_relu_mask_f32(const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,
+                                          const float* y, float* c, int64_t m, int64_t n, int64_t k, void* stream) {
+    if (m > 0 && n > 0 && !y) return fail(CTAMD_EINVAL, "%s: null activation", __func__);
+    return matmul_impl(__func__, a, as0, as1, b, bs0, bs1, nullptr, 0, y, c, m, n, k, stream);
 }

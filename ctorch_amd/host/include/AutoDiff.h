@@ -75,6 +75,11 @@ class AutoDiff {
         std::unique_ptr<Tensor> grad;
         bool grad_plus_zero = false;           // grad holds no -0: "0 + grad" (what get_grad returns) is grad itself
         bool grad_assigned = false;            // grad is a root's seed: assigned, not added to zeros (src/AutoDiff.cpp:1126), read as it is
+        // Set on a ReLU layer (op::Linear with its ReLU) whose output has one consumer, a product: that
+        // consumer's backward formed `grad` already multiplied by [y > 0], i.e. `grad` is the gradient at
+        // the pre-activation and the layer's own mask launch is skipped.  get_grad() forms the
+        // gradient of the output itself from the consumer when somebody asks for it.
+        Node* grad_premasked_by = nullptr;
         std::unique_ptr<Tensor> shared_term;   // backward only: a factor that several inputs' gradients use
         std::vector<Tensor> input_grads;       // backward only: gradients of all inputs, computed together
         std::shared_ptr<OpPayload> payload;
@@ -106,6 +111,10 @@ class AutoDiff {
     // AutoDiff.cpp:1267-1284).  On the device that is one more pass over b and a host wait; it can
     // be switched off.
     void set_check_div_zero(bool on) { check_div_zero_ = on; }
+    // The ReLU mask of a layer in the launch of the product that forms the layer's output gradient
+    // (on by default; the gradients are the same bits either way).
+    void set_fuse_relu_mask(bool on) { fuse_relu_mask_ = on; }
+    bool fuse_relu_mask() const { return fuse_relu_mask_; }
 
    private:
     struct Pending {
@@ -121,6 +130,7 @@ class AutoDiff {
     BroadcastGrad broadcast_grad_ = BroadcastGrad::kColumnSum;
     LeafValues leaf_values_ = LeafValues::kLive;
     bool check_div_zero_ = true;
+    bool fuse_relu_mask_ = true;
     bool term_plus_zero_ = false;   // backward: the term just computed holds no -0
     bool seed_plus_zero_ = false;   // backward: the seed gradient holds no -0
     bool adjust_adds_to_zero_ = false;   // the last adjust_grad_shape took a branch in which the reference adds the gradient to zeros
@@ -128,6 +138,7 @@ class AutoDiff {
     Node* find(size_t id);
     Tensor adjust_grad_shape(const Tensor& grad, const std::vector<size_t>& target_shape);
     Tensor input_gradient(Node* node, size_t input_id, size_t input_pos, const Tensor& node_grad);
+    const Tensor& linear_pre_activation_grad(Node* node, const Tensor& node_grad);
 };
 // Makes this thread's device seed of backward(root) (a 0-D 1.0) now, if it does not exist yet.
 void prepare_backward_seed();

@@ -18,6 +18,9 @@ Tensor Div_AMD_kernel(const Tensor& a, const Tensor& b);
 Tensor MatMul_AMD_kernel(const Tensor& a, const Tensor& b);
 // x.matmul(w) + bias (row vector), then ReLU when asked, in one launch; equals the separate kernels bit for bit
 Tensor Linear_AMD_kernel(const Tensor& x, const Tensor& w, const Tensor& bias, bool relu);
+// (a . b) * [y > 0] in the product's launch: what MatMul's backward branch followed by the ReLU branch
+// of the layer that produced y compute (src/AutoDiff.cpp:1692-1704, :1320-1371)
+Tensor MatMulReluMask_AMD_kernel(const Tensor& a, const Tensor& b, const Tensor& y);
 Tensor Dot_AMD_kernel(const Tensor& a, const Tensor& b);
 Tensor MSE_AMD_kernel(const Tensor& a, const Tensor& b);
 Tensor MAE_AMD_kernel(const Tensor& a, const Tensor& b);

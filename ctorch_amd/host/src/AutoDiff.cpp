@@ -66,6 +66,7 @@ void AutoDiff::zero_grad(Tensor& t) {
         n->grad.reset();
         n->grad_plus_zero = false;
         n->grad_assigned = false;
+        n->grad_premasked_by = nullptr;
     }
 }
 
@@ -76,7 +77,7 @@ Tensor AutoDiff::stored_grad(const Tensor& t) {
     if (t.id() == 0) return Tensor();
     std::lock_guard<std::mutex> lock(records_mutex);
     Node* n = find(t.id());
-    if (n && n->requires_grad && n->grad && n->grad->sizes() == t.sizes()) return Tensor::alias(*n->grad);
+    if (n && n->requires_grad && n->grad && n->grad->sizes() == t.sizes() && !n->grad_premasked_by) return Tensor::alias(*n->grad);
     return Tensor();
 }
 
@@ -85,6 +86,16 @@ Tensor AutoDiff::get_grad(const Tensor* t) {
     if (!t || t->id() == 0) return Tensor();
     std::lock_guard<std::mutex> lock(records_mutex);
     Node* n = find(t->id());
+    if (n && n->requires_grad && n->grad && n->grad_premasked_by) {
+        // the tape holds this layer's gradient at the pre-activation; the gradient of the output is
+        // the consumer's product without the mask, formed now
+        Node* by = n->grad_premasked_by;
+        if (!by->grad) return Tensor(ShapeTag{}, t->shape(), t->dtype(), t->device());
+        AutoDiffContext::Guard guard(nullptr);          // nothing below is taped
+        Tensor whole = input_gradient(by, n->tensor_id, 0, *by->grad);
+        by->shared_term.reset();
+        return whole;                                   // sums of products from +0: no "0 +" pending
+    }
     if (n && n->requires_grad && n->grad) {
         // the pending "0 +" (one pass, once); a gradient known to hold no -0 needs none.  The
         // result shares the tape's bytes instead of copying them: the tape never writes through
@@ -319,11 +330,7 @@ Tensor AutoDiff::input_gradient(Node* node, size_t input_id, size_t input_pos, c
             return MatMul_AMD_kernel(Tensor::view_t(other), g);                 // A^T . g
         }
         case op::Linear: {                                              // the three branches above in one
-            // gradient at the pre-activation: g * [y > 0], which is the reference's g * [z > 0]
-            // (:1320-1371) since y = max(0, z); computed once for the three inputs
-            if (node->op_param_i && !node->shared_term)
-                node->shared_term = std::make_unique<Tensor>(relu_backward(*node->tensor, g));
-            const Tensor& gz = node->op_param_i ? *node->shared_term : g;
+            const Tensor& gz = linear_pre_activation_grad(node, g);
             if (input_pos == 2) {                                       // bias: Add's branch, shaped by the caller
                 term_plus_zero_ = node->op_param_i ? false : upstream_plus_zero;   // g * 0 may be -0
                 return Tensor::alias(gz);
@@ -385,6 +392,15 @@ Tensor AutoDiff::input_gradient(Node* node, size_t input_id, size_t input_pos, c
     }
 }
 
+// The gradient at a layer's pre-activation: g * [y > 0], which is the reference's g * [z > 0]
+// (:1320-1371) since y = max(0, z); computed once for the three inputs - or g itself when the layer
+// has no ReLU, or when the product that formed g applied the mask already.
+const Tensor& AutoDiff::linear_pre_activation_grad(Node* node, const Tensor& g) {
+    if (!node->op_param_i || node->grad_premasked_by) return g;
+    if (!node->shared_term) node->shared_term = std::make_unique<Tensor>(relu_backward(*node->tensor, g));
+    return *node->shared_term;
+}
+
 // The seed 1.0 on the device is made once per thread and shared (the tape never writes through a
 // shared gradient: accumulation goes to a fresh tensor then).
 static Tensor& device_seed() {
@@ -425,6 +441,20 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
         Ctorch_Error::throwException(ErrorPlatform::kAutoDiff, ErrorType::DATATYPE, "backward: only float tensors have gradients");
     if (grad_output.device() != root.device()) grad_output = grad_output.to(root.device());
     ctorch_amd_host::drop_deferred_checks();     // of a pass that ended in an exception
+    // A gradient that an earlier pass left at a layer's pre-activation is brought back to the
+    // gradient of the layer's output before anything is added to it (a pass over a tape that was
+    // not cleared adds to what the nodes hold, as the reference's does).
+    for (auto& entry : id_to_node) {
+        Node* n = entry.second.get();
+        if (!n->grad_premasked_by) continue;
+        Node* by = n->grad_premasked_by;
+        n->grad_premasked_by = nullptr;
+        if (n->grad && by->grad) {
+            n->grad = std::make_unique<Tensor>(input_gradient(by, n->tensor_id, 0, *by->grad));
+            n->grad_plus_zero = true;
+            by->shared_term.reset();
+        }
+    }
     root_node->grad = std::make_unique<Tensor>(adjust_grad_shape(grad_output, root.sizes()));
     root_node->grad_plus_zero = seed_plus_zero_;
     root_node->grad_assigned = !adjust_adds_to_zero_;     // a seed taken as it is stays as it is (:1126)
@@ -450,6 +480,11 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
         }
         std::reverse(order.begin(), order.end());
     }
+
+    // how many operator inputs of this pass read each tensor
+    std::unordered_map<size_t, int> consumers;
+    for (Node* n : order)
+        for (size_t id : n->input_ids) ++consumers[id];
 
     for (Node* node : order) {
         if (!node->requires_grad || !node->grad || node->is_leaf) continue;
@@ -513,6 +548,25 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
                                                      "division by zero in the gradient of Div");
                     in->grad = std::make_unique<Tensor>(div_plus(node_grad, *bn->tensor, *in->grad));
                     in->grad_plus_zero = false;
+                    continue;
+                }
+            }
+            // The output of a ReLU layer read by this product alone: its gradient g . W^T is wanted only
+            // times the layer's mask, so the mask rides in the product's launch (one launch instead of
+            // two, the same bits: the 0 / 1 factor multiplies the same fp32 product).
+            if (fuse_relu_mask_ && pos == 0 && !in->grad && in != root_node && !in->is_leaf &&
+                (node->operation == op::Linear || node->operation == op::MatMul) && node->input_ids.size() >= 2 &&
+                node->input_ids[1] != input_id && in->operation == op::Linear && in->op_param_i != 0 &&
+                consumers[input_id] == 1 && node_grad.dim() == 2 && in->tensor->dim() == 2 &&
+                in->tensor->device() == DeviceType::kAMD && in->tensor->is_contiguous() && in->tensor->dtype() == DType::kFloat) {
+                Node* wn = find(node->input_ids[1]);
+                const Tensor& gz = node->operation == op::Linear ? linear_pre_activation_grad(node, node_grad) : node_grad;
+                if (wn && wn->tensor->dim() == 2 && wn->tensor->device() == DeviceType::kAMD && gz.device() == DeviceType::kAMD &&
+                    gz.sizes()[0] == in->tensor->sizes()[0] && gz.sizes()[1] == wn->tensor->sizes()[1] &&
+                    wn->tensor->sizes()[0] == in->tensor->sizes()[1]) {
+                    in->grad = std::make_unique<Tensor>(MatMulReluMask_AMD_kernel(gz, Tensor::view_t(*wn->tensor), *in->tensor));
+                    in->grad_plus_zero = false;          // g * 0 may be -0
+                    in->grad_premasked_by = node;
                     continue;
                 }
             }

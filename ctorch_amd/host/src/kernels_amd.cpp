@@ -659,6 +659,21 @@ Tensor MatMul_AMD_kernel(const Tensor& a, const Tensor& b) {
         "MatMul_AMD_kernel");
     return r;
 }
+Tensor MatMulReluMask_AMD_kernel(const Tensor& a, const Tensor& b, const Tensor& y) {
+    check_device(a, "MatMulReluMask_AMD_kernel");
+    check_device(b, "MatMulReluMask_AMD_kernel");
+    check_device(y, "MatMulReluMask_AMD_kernel");
+    if (a.shape().size() != 2 || b.shape().size() != 2 || a.shape()[1] != b.shape()[0])
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "MatMulReluMask_AMD_kernel: not a product of two matrices");
+    size_t m = a.shape()[0], k = a.shape()[1], n = b.shape()[1];
+    if (y.shape() != std::vector<size_t>{m, n} || !y.is_contiguous())
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "MatMulReluMask_AMD_kernel: the activation is not a contiguous [m, n]");
+    Tensor r(ShapeTag{}, {m, n}, DType::kFloat, DeviceType::kAMD, false);
+    run(ctamd_matmul_relu_mask_f32(a.fptr(), int64_t(a.strides()[0]), int64_t(a.strides()[1]), b.fptr(), int64_t(b.strides()[0]),
+                                   int64_t(b.strides()[1]), y.fptr(), r.fptr(), int64_t(m), int64_t(n), int64_t(k), current_stream()),
+        "MatMulReluMask_AMD_kernel");
+    return r;
+}
 Tensor Linear_AMD_kernel(const Tensor& x, const Tensor& w, const Tensor& bias, bool relu) {
     check_device(x, "Linear_AMD_kernel");
     check_device(w, "Linear_AMD_kernel");

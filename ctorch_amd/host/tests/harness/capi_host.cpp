@@ -125,8 +125,13 @@ void cth_last_expr_stats(int* out) {
 void cth_set_reference_row0(int on) { g_row0 = on; }
 // the MLP entry points below build each layer with Tensor::linear (one fused operator) when set
 void cth_set_fused_layers(int on) { g_fused_layers = on; }
+// the ReLU mask of a fused layer in the product that forms the layer's output gradient (default) or
+// as a launch of its own
+static int g_fuse_relu_mask = 1;
+void cth_set_fuse_relu_mask(int on) { g_fuse_relu_mask = on; }
 static void configure(AutoDiff& ctx) {
     ctx.set_broadcast_grad(g_row0 ? BroadcastGrad::kReferenceRow0 : BroadcastGrad::kColumnSum);
+    ctx.set_fuse_relu_mask(g_fuse_relu_mask != 0);
 }
 
 long cth_binary(int code, const float* a, const long* ad, int an, const float* b, const long* bd,
@@ -1047,6 +1052,55 @@ long cth_shared_grad_is_readonly(const float* a, long n) {
         g.fill(1.0f);                              // the tape is gone: g is the only holder
         std::vector<float> host(static_cast<size_t>(n));
         if (emit(g, host.data()) < 0 || host[0] != 1.0f) return -3;
+        return 0;
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
+// A three-layer network of fused layers, trained gradients and the gradients of the two hidden
+// activations, with the ReLU mask riding in the products of backward and without, after one
+// backward pass and after two passes over the same tape: 0 when every gradient agrees bit for bit,
+// else 1 + the index of the first that differs (+ 100 for the two-pass run).  out[0]: kernels
+// launched by one backward with the mask in the products, out[1]: without.
+long cth_relu_mask_fusion(const float* x, long B, long I, const float* W1, const float* b1, long H1, const float* W2,
+                          const float* b2, long H2, const float* W3, const float* b3, long C, const float* labels,
+                          double* out) {
+    try {
+        auto run = [&](bool fuse, int passes, double* launches) {
+            std::vector<std::vector<float>> grads;
+            AutoDiff ctx;
+            configure(ctx);
+            ctx.set_fuse_relu_mask(fuse);        // this check sets it itself
+            AutoDiffContext::Guard guard(&ctx);
+            long xd[2] = {B, I}, w1d[2] = {I, H1}, b1d[1] = {H1}, w2d[2] = {H1, H2}, b2d[1] = {H2}, w3d[2] = {H2, C},
+                 b3d[1] = {C}, yi[1] = {B};
+            Tensor tx = make(x, xd, 2), tW1 = make(W1, w1d, 2), tb1 = make(b1, b1d, 1), tW2 = make(W2, w2d, 2),
+                   tb2 = make(b2, b2d, 1), tW3 = make(W3, w3d, 2), tb3 = make(b3, b3d, 1), ty = make(labels, yi, 1);
+            for (Tensor* t : {&tW1, &tb1, &tW2, &tb2, &tW3, &tb3}) t->requires_grad(true);
+            Tensor h1 = tx.linear(tW1, tb1, true);
+            Tensor h2 = h1.linear(tW2, tb2, true);
+            Tensor logits = h2.linear(tW3, tb3, false);
+            Tensor loss = logits.cross_entropy(ty);
+            for (int p = 0; p < passes; ++p) {
+                double bytes = 0.0, flops = 0.0, ideal = 0.0;
+                uint64_t before = 0, after = 0;
+                ctamd_counters_read(&bytes, &flops, &ideal, &before);
+                backward(loss);
+                ctamd_counters_read(&bytes, &flops, &ideal, &after);
+                if (launches) *launches = double(after - before);
+            }
+            for (Tensor* t : {&tW1, &tb1, &tW2, &tb2, &tW3, &tb3, &h1, &h2}) grads.push_back(grad(*t).to_vector());
+            return grads;
+        };
+        for (int passes = 1; passes <= 2; ++passes) {
+            auto with = run(true, passes, passes == 1 ? out : nullptr);
+            auto without = run(false, passes, passes == 1 ? out + 1 : nullptr);
+            for (size_t i = 0; i < with.size(); ++i)
+                if (with[i].size() != without[i].size() ||
+                    std::memcmp(with[i].data(), without[i].data(), with[i].size() * sizeof(float)) != 0)
+                    return long(1 + i) + (passes == 2 ? 100 : 0);
+        }
         return 0;
     } catch (const std::exception&) {
         return -1;

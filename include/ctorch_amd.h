@@ -272,8 +272,10 @@ int ctamd_cross_entropy_index_fused_f32(const float* x, const float* idx, float*
  * are in elements and may describe a transposed view.  MatMul_BASIC_kernel.cpp:42-54.  The
  * reference's backward calls the same kernel with t() views: dA = g.matmul(B.t()),
  * dB = A.t().matmul(g) (src/AutoDiff.cpp:1692-1704, :1808-1810).  fp32 MFMA with fp32
- * accumulation; every operand layout with a unit stride in one dimension takes the MFMA path,
- * anything else a generic strided kernel. */
+ * accumulation; every operand layout with a unit stride in one dimension takes the MFMA path
+ * (products with at most 16 output columns that are too large for one launch of small MFMA
+ * tiles: fp32 FMAs on the vector units, in a fixed order), anything else a generic strided
+ * kernel.  Results are deterministic: the same call gives the same bits. */
 int ctamd_matmul_f32(const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,
                      float* c, int64_t m, int64_t n, int64_t k, void* stream);
 
@@ -284,6 +286,15 @@ int ctamd_matmul_f32(const float* a, int64_t as0, int64_t as1, const float* b, i
  * ctamd_matmul_f32, ctamd_add_rowbcast_f32, ctamd_relu_f32 in sequence bit for bit. */
 int ctamd_matmul_bias_f32(const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,
                           const float* bias, int relu, float* c, int64_t m, int64_t n, int64_t k, void* stream);
+
+/* The gradient that reaches a ReLU layer's pre-activation, formed by the product that computes it:
+ * C = (A.B) * [y > 0], y the [m, n] row-major output of that ReLU.  The reference computes the
+ * product in the MatMul branch of backward (g.matmul(B.t()), src/AutoDiff.cpp:1692-1704) and the
+ * mask in the ReLU branch of the layer below (grad * [x > 0], :1320-1371; y > 0 exactly where
+ * x > 0); here the factor 0 / 1 multiplies the accumulator as it is stored.  Equal to
+ * ctamd_matmul_f32 followed by ctamd_relu_backward_f32(y, C, C) bit for bit. */
+int ctamd_matmul_relu_mask_f32(const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,
+                               const float* y, float* c, int64_t m, int64_t n, int64_t k, void* stream);
 
 /* -------------------------------------------------------------------------- comparisons */
 /* out[i] = (a[i] cmp b[i]) or (a[i] cmp s) as one byte, 0 or 1 - the reference's bool tensors.

@@ -218,6 +218,17 @@ def matmul_bias(a, b, bias, relu):
     return c
 
 
+def matmul_relu_mask(a, b, y):
+    """(a.b) * [y > 0]: the gradient at a ReLU layer's pre-activation, in the product's launch."""
+    m, k = a.shape
+    k2, n = b.shape
+    assert k == k2 and tuple(y.shape) == (m, n) and y.is_contiguous()
+    c = torch.empty((m, n), device=DEV)
+    call("ctamd_matmul_relu_mask_f32", ptr(a), a.stride(0), a.stride(1), ptr(b), b.stride(0), b.stride(1), ptr(y), ptr(c),
+         m, n, k, stream())
+    return c
+
+
 def matmul(a, b):
     """a, b: 2-D device tensors, possibly transposed views (strides are passed through)."""
     m, k = a.shape

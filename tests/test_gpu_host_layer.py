@@ -478,3 +478,30 @@ def test_a_gradient_read_from_the_tape_is_read_only_while_shared(oracle, host):
     import ctypes as C
     host.cdll.cth_shared_grad_is_readonly.restype = C.c_long
     assert host.cdll.cth_shared_grad_is_readonly(x.ctypes.data_as(C.POINTER(C.c_float)), C.c_long(x.size)) == 0
+
+
+@pytest.mark.parametrize("batch", [8, 300, 4096])
+def test_relu_mask_rides_in_the_products_of_backward(oracle, host, batch):
+    """The gradient of a ReLU layer's output, when one product alone reads that output, is formed
+    already multiplied by the layer's mask (one launch fewer per hidden layer).  A three-layer
+    network: the six parameter gradients and the gradients of both hidden activations (which the
+    tape then has to form on request) equal the ones of the separate mask launch bit for bit, after
+    one backward pass and after two passes over the same tape; and backward launches fewer kernels."""
+    print("case relu mask in the product", batch, flush=True)
+    import ctypes as C
+    I, H1, H2, Cn = 200, 96, 72, 10
+    x = oracle.uniform((batch, I), 641, 0, 1)
+    W1, b1 = oracle.uniform((I, H1), 642, -0.1, 0.1), oracle.uniform((H1,), 643, -0.1, 0.1)
+    W2, b2 = oracle.uniform((H1, H2), 644, -0.15, 0.15), oracle.uniform((H2,), 645, -0.1, 0.1)
+    W3, b3 = oracle.uniform((H2, Cn), 646, -0.2, 0.2), oracle.uniform((Cn,), 647, -0.1, 0.1)
+    labels = oracle.ints((batch,), 648, Cn)
+    FP = C.POINTER(C.c_float)
+    fp = lambda a: a.ctypes.data_as(FP)
+    L = C.c_long
+    out = (C.c_double * 2)()
+    host.cdll.cth_relu_mask_fusion.restype = C.c_long
+    rc = host.cdll.cth_relu_mask_fusion(fp(x), L(batch), L(I), fp(W1), fp(b1), L(H1), fp(W2), fp(b2), L(H2), fp(W3), fp(b3),
+                                        L(Cn), fp(labels), out)
+    assert rc == 0, rc
+    print(f"  kernels launched by backward: {int(out[0])} with the mask in the products, {int(out[1])} without")
+    assert out[0] == out[1] - 2

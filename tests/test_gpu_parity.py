@@ -605,3 +605,31 @@ def test_comparisons_bit_exact(oracle, n):
             G.call("ctamd_compare_scalar_f32", cmp, G.ptr(da), C.c_float(s), G.ptr(out), n, G.stream())
             assert np.array_equal(out.cpu().numpy(), oracle.compare(cmp, a, None, s)), (cmp, s)
     assert G.lib().ctamd_compare_f32(9, G.ptr(da), G.ptr(db), G.ptr(out), n, G.stream()) == -1
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 256, 10), (8192, 256, 10), (100, 70, 300), (300, 200, 1000), (2100, 2050, 40),
+                                   (4090, 2047, 24), (96, 12, 4096), (64, 10, 256), (5, 7, 0)])
+def test_product_times_relu_mask_equals_the_two_launches(oracle, m, n, k):
+    """(a.b) * [y > 0] in the product's launch against the product followed by the ReLU gradient
+    kernel, bit for bit: the small-product kernel, the tiles with and without a cut K, ragged edges,
+    the narrow and strided forms (which launch the mask by itself), an empty sum; rows of y that
+    are zero, negative, NaN and infinite, and products that are."""
+    print("case product times mask", m, n, k, flush=True)
+    A = oracle.normal((m, k), 71)
+    B = oracle.normal((k, n), 72)
+    y = np.maximum(oracle.normal((m, n), 73), 0).astype(F)
+    if m * n >= 16:
+        y.flat[1], y.flat[2], y.flat[3], y.flat[5] = -0.0, np.nan, np.inf, -1.0
+    if k:
+        A[0, 0] = np.inf                 # products of row 0 are +-inf or NaN: times 0 they are NaN, as the separate launch gives
+    dA, dB, dy = G.dev(A), G.dev(B), G.dev(y)
+    dAt, dBt = G.dev(np.ascontiguousarray(A.T)), G.dev(np.ascontiguousarray(B.T))
+    views = [(dA, dB), (dA, dBt.t()), (dAt.t(), dB)]
+    if k:
+        A2 = G.dev(np.repeat(A, 2, axis=1))
+        views.append((A2[:, ::2], dB))       # no unit stride: the generic kernel
+    for a, b in views:
+        plain = G.matmul(a, b)
+        want = G.host(G.unary_bwd("relu", dy, plain))
+        got = G.host(G.matmul_relu_mask(a, b, dy))
+        assert same_bits(got, want)
