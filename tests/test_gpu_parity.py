@@ -477,7 +477,7 @@ MM_SHAPES = [(1, 1, 1), (5, 3, 9), (33, 29, 47), (128, 128, 16), (130, 257, 70),
              # an output of at most 16 columns: the streaming kernels, in rows (A row-major) and in
              # columns (A a transposed view) with and without a cut K, ragged m and k
              (8192, 10, 256), (8190, 16, 252), (1000, 1, 512), (70, 3, 8), (5000, 7, 52), (300, 16, 1000),
-             (777, 13, 3001), (66000, 2, 12),
+             (777, 13, 3001), (66000, 2, 12), (20000, 10, 256), (9000, 5, 700),
              # at most one 32 x 32 tile per CU and K <= 512: the small-product kernel (those above with
              # small extents take it too); the same extents with a longer K stay on the 64 x 64 tiles
              (256, 256, 256), (784, 256, 256), (100, 70, 300), (512, 512, 512), (31, 33, 512),
