@@ -1177,47 +1177,19 @@ __global__ __launch_bounds__(256) void col_walk_kernel(const float* __restrict__
     }
 }
 
-// The `chunks` partial rows of a column folded in double: their sum (PAIRS = false), or the
-// (max, sum) pairs of the online softmax brought to the column maximum (PAIRS = true: maxima in the
-// first `chunks` rows of partials, sums in the next; out_max[c], out[c]).  A block folds 32 columns;
-// its 8 groups of 32 lanes take every 8th chunk and are added in group order.
+// The `chunks` partial rows of a column folded in double.  A block folds 32 columns; its 8 groups
+// of 32 lanes take every 8th chunk and are added in group order.
 constexpr int kFoldCols = 32, kFoldGroups = 8;
-template <bool PAIRS>
-__global__ __launch_bounds__(256) void col_fold_kernel(const float* __restrict__ partials, float* __restrict__ out_max,
-                                                       float* __restrict__ out, size_t cols, unsigned chunks) {
-    __shared__ uint64_t s_exp2[32];
-    __shared__ float s_m[kFoldGroups][kFoldCols];
+__global__ __launch_bounds__(256) void col_fold_kernel(const float* __restrict__ partials, float* __restrict__ out, size_t cols,
+                                                       unsigned chunks) {
     __shared__ double s_t[kFoldGroups][kFoldCols];
-    if (PAIRS) stage_exp_table(s_exp2);
     const unsigned lane = threadIdx.x % kFoldCols, group = threadIdx.x / kFoldCols;
     const size_t c = size_t(blockIdx.x) * kFoldCols + lane;
     const bool live = c < cols;
-    float m = kNegInf;
-    if (PAIRS) {
-        if (live) {
-#pragma unroll 4
-            for (unsigned k = group; k < chunks; k += kFoldGroups) {
-                const float v = partials[size_t(k) * cols + c];
-                m = v > m ? v : m;
-            }
-        }
-        s_m[group][lane] = m;
-        __syncthreads();
-#pragma unroll
-        for (int g = 0; g < kFoldGroups; ++g) m = s_m[g][lane] > m ? s_m[g][lane] : m;
-    }
     double t = 0.0;
     if (live) {
 #pragma unroll 4
-        for (unsigned k = group; k < chunks; k += kFoldGroups) {
-            if (PAIRS) {
-                const float mk = partials[size_t(k) * cols + c];
-                const float sk = partials[(size_t(chunks) + k) * cols + c];
-                if (mk != kNegInf) t += double(sk) * double(cta_expf_nonpos(mk - m, s_exp2));
-            } else {
-                t += double(partials[size_t(k) * cols + c]);
-            }
-        }
+        for (unsigned k = group; k < chunks; k += kFoldGroups) t += double(partials[size_t(k) * cols + c]);
     }
     s_t[group][lane] = t;
     __syncthreads();
@@ -1225,7 +1197,64 @@ __global__ __launch_bounds__(256) void col_fold_kernel(const float* __restrict__
         double sum = 0.0;
 #pragma unroll
         for (int g = 0; g < kFoldGroups; ++g) sum += s_t[g][lane];
-        if (PAIRS) out_max[c] = m;
+        out[c] = float(sum);
+    }
+}
+
+// The (max, sum) pairs of the online column pass (maxima in the first `chunks` rows of partials,
+// sums in the next) brought to the column maximum, out_max[c], and added in double, out[c].  A CU
+// draws only some tens of GB/s by itself, so the fold is spread over as many blocks as the columns
+// allow: a block folds 16 columns, its 64 groups of 16 lanes take every 64th chunk (four loads in
+// flight each), and the groups' maxima and sums are combined through LDS in group order.  (32
+// columns x 8 groups on 128 blocks, or 64 columns x 16 groups on 64 blocks, took 18.5 us for the
+// 8 MiB of partials of a [16384 x 4096] matrix, an eighth of the whole softmax.)
+constexpr int kPairCols = 16, kPairGroups = 64, kPairAhead = 4;
+__global__ __launch_bounds__(kPairCols * kPairGroups) void col_fold_pairs_kernel(const float* __restrict__ partials,
+                                                                                 float* __restrict__ out_max, float* __restrict__ out,
+                                                                                 size_t cols, unsigned chunks) {
+    __shared__ uint64_t s_exp2[32];
+    __shared__ float s_m[kPairGroups][kPairCols];
+    __shared__ double s_t[kPairGroups][kPairCols];
+    stage_exp_table(s_exp2);
+    const unsigned lane = threadIdx.x % kPairCols, group = threadIdx.x / kPairCols;
+    const size_t c = size_t(blockIdx.x) * kPairCols + lane;
+    const bool live = c < cols;
+    float m = kNegInf;
+    for (unsigned k0 = group; k0 < chunks; k0 += kPairGroups * kPairAhead) {
+        float mk[kPairAhead];
+#pragma unroll
+        for (int i = 0; i < kPairAhead; ++i) {
+            const unsigned k = k0 + unsigned(i) * kPairGroups;
+            mk[i] = (live && k < chunks) ? partials[size_t(k) * cols + c] : kNegInf;
+        }
+#pragma unroll
+        for (int i = 0; i < kPairAhead; ++i) m = mk[i] > m ? mk[i] : m;
+    }
+    s_m[group][lane] = m;
+    __syncthreads();
+#pragma unroll
+    for (int g = 0; g < kPairGroups; ++g) m = s_m[g][lane] > m ? s_m[g][lane] : m;
+    double t = 0.0;
+    for (unsigned k0 = group; k0 < chunks; k0 += kPairGroups * kPairAhead) {
+        float mk[kPairAhead], sk[kPairAhead];
+#pragma unroll
+        for (int i = 0; i < kPairAhead; ++i) {
+            const unsigned k = k0 + unsigned(i) * kPairGroups;
+            const bool in = live && k < chunks;
+            mk[i] = in ? partials[size_t(k) * cols + c] : kNegInf;
+            sk[i] = in ? partials[(size_t(chunks) + k) * cols + c] : 0.0f;
+        }
+#pragma unroll
+        for (int i = 0; i < kPairAhead; ++i)
+            if (mk[i] != kNegInf) t += double(sk[i]) * double(cta_expf_nonpos(mk[i] - m, s_exp2));
+    }
+    s_t[group][lane] = t;
+    __syncthreads();
+    if (group == 0 && live) {
+        double sum = 0.0;
+#pragma unroll
+        for (int g = 0; g < kPairGroups; ++g) sum += s_t[g][lane];
+        out_max[c] = m;
         out[c] = float(sum);
     }
 }
@@ -1353,9 +1382,8 @@ int ctamd_log_softmax_cols_f32(const float* x, float* y, size_t rows, size_t col
     account(8.0 * double(rows) * double(cols), double(rows) * double(cols));
     if (plan_cols(rows, cols, aligned16(x) && aligned16(y), p, stream)) {
         hipStream_t s = as_stream(stream);
-        const unsigned fold_blocks = unsigned((cols + kFoldCols - 1) / kFoldCols);
         launch_col_walk<kColOnline>(p, x, nullptr, nullptr, nullptr, p.partials, rows, cols, s);
-        hipLaunchKernelGGL(col_fold_kernel<true>, dim3(fold_blocks), dim3(256), 0, s, p.partials, p.v0, p.v1, cols, unsigned(p.chunks));
+        hipLaunchKernelGGL(col_fold_pairs_kernel, dim3(unsigned((cols + kPairCols - 1) / kPairCols)), dim3(kPairCols * kPairGroups), 0, s, p.partials, p.v0, p.v1, cols, unsigned(p.chunks));
         launch_col_walk<kColLogSoftmaxOut>(p, x, nullptr, p.v0, p.v1, y, rows, cols, s);
         return launched(__func__);
     }
@@ -1371,7 +1399,7 @@ int ctamd_log_softmax_backward_cols_f32(const float* y, const float* g, float* d
     if (plan_cols(rows, cols, aligned16(y) && aligned16(g) && aligned16(dx), p, stream)) {
         hipStream_t s = as_stream(stream);
         launch_col_walk<kColSum>(p, g, nullptr, nullptr, nullptr, p.partials, rows, cols, s);
-        hipLaunchKernelGGL(col_fold_kernel<false>, dim3(unsigned((cols + kFoldCols - 1) / kFoldCols)), dim3(256), 0, s, p.partials, nullptr, p.v0,
+        hipLaunchKernelGGL(col_fold_kernel, dim3(unsigned((cols + kFoldCols - 1) / kFoldCols)), dim3(256), 0, s, p.partials, p.v0,
                            cols, unsigned(p.chunks));
         if (fast_math()) launch_col_walk<kColLogBwdOut, true>(p, y, g, p.v0, nullptr, dx, rows, cols, s);
         else launch_col_walk<kColLogBwdOut>(p, y, g, p.v0, nullptr, dx, rows, cols, s);
@@ -1388,9 +1416,8 @@ int ctamd_softmax_cols_f32(const float* x, float* y, size_t rows, size_t cols, v
     ColPlan p;
     if (plan_cols(rows, cols, aligned16(x) && aligned16(y), p, stream)) {
         hipStream_t s = as_stream(stream);
-        const unsigned fold_blocks = unsigned((cols + kFoldCols - 1) / kFoldCols);
         launch_col_walk<kColOnline>(p, x, nullptr, nullptr, nullptr, p.partials, rows, cols, s);
-        hipLaunchKernelGGL(col_fold_kernel<true>, dim3(fold_blocks), dim3(256), 0, s, p.partials, p.v0, p.v1, cols, unsigned(p.chunks));
+        hipLaunchKernelGGL(col_fold_pairs_kernel, dim3(unsigned((cols + kPairCols - 1) / kPairCols)), dim3(kPairCols * kPairGroups), 0, s, p.partials, p.v0, p.v1, cols, unsigned(p.chunks));
         if (fast_math()) launch_col_walk<kColSoftmaxOut, true>(p, x, nullptr, p.v0, p.v1, y, rows, cols, s);
         else launch_col_walk<kColSoftmaxOut>(p, x, nullptr, p.v0, p.v1, y, rows, cols, s);
         account(8.0 * double(rows) * double(cols), double(rows) * double(cols));
@@ -1409,7 +1436,7 @@ int ctamd_softmax_backward_cols_f32(const float* y, const float* g, float* dx, s
     if (plan_cols(rows, cols, aligned16(y) && aligned16(g) && aligned16(dx), p, stream)) {
         hipStream_t s = as_stream(stream);
         launch_col_walk<kColDot>(p, y, g, nullptr, nullptr, p.partials, rows, cols, s);
-        hipLaunchKernelGGL(col_fold_kernel<false>, dim3(unsigned((cols + kFoldCols - 1) / kFoldCols)), dim3(256), 0, s, p.partials, nullptr, p.v0,
+        hipLaunchKernelGGL(col_fold_kernel, dim3(unsigned((cols + kFoldCols - 1) / kFoldCols)), dim3(256), 0, s, p.partials, p.v0,
                            cols, unsigned(p.chunks));
         launch_col_walk<kColBwdOut>(p, y, g, p.v0, nullptr, dx, rows, cols, s);
         account(12.0 * double(rows) * double(cols), 2.0 * double(rows) * double(cols));

@@ -242,17 +242,20 @@ __global__ __launch_bounds__(256) void softmax_rows_f64_resident_kernel(const do
     }
 }
 
-// Column softmax in two launches over chunks of rows.  A block owns 32 neighbouring columns of one
-// chunk; its 8 groups of 32 lanes take every 8th row of the chunk (a group reads 256 contiguous
-// bytes per row).  First launch: a running (maximum, sum of exp(x - maximum)) pair per thread with
-// ONE exponential per element - of the element's distance below the maximum, or of the old
-// maximum's distance below the element when the maximum moves - combined over the groups in group
-// order and left per (chunk, column) in `pairs`.  Second launch: every block brings the chunks' pairs
-// of its columns to the column maximum in chunk order (a few exponentials per column), then writes
-// y = exp(x - max) / sum.  Two exponentials and 24 bytes per element, against three sweeps of the
-// whole matrix by 256 blocks before.  (One thread walking a whole column, the reference's order
-// src/Tensor.cpp:1766-1781, took 11.9 ms on [8192 x 8192].)
-constexpr int kLanesPerRow = 32, kRowGroups = 8;
+// Column softmax in three launches over chunks of rows, the layout of the fp32 column kernels: a
+// block owns a strip of 256 * W neighbouring columns of one chunk (a row of the strip is 4 KiB of
+// contiguous memory with two columns per thread) and every thread walks the chunk's rows in order,
+// four rows' loads in flight.  First launch: a running (maximum, sum of exp(x - maximum)) pair per
+// thread with ONE exponential per element - of the element's distance below the maximum, or of
+// the old maximum's distance below the element when the maximum moves - kept apart for the even
+// and odd rows of the chunk (two short dependency chains instead of one) and left per (chunk,
+// column) in `pairs`.  Second launch: the chunks' pairs of a column brought to the column maximum
+// and added in chunk-group order.  Third launch: y = exp(x - max) / sum, the quotient as a product
+// with the column's reciprocal and one correction step (e r + fma(-(e r), sum, e) r: the correctly
+// rounded quotient but for results in the subnormal range, where it is within one of their units).
+// Two exponentials and 24 bytes per element.  (One thread walking a whole column, the reference's
+// order src/Tensor.cpp:1766-1781, took 11.9 ms on [8192 x 8192]; blocks of 32 columns x 8 row
+// groups, which read 512 bytes of a row at a time, and a true division per element: 345 us.)
 struct MaxSum {
     double m, s;
 };
@@ -263,114 +266,142 @@ __device__ __forceinline__ MaxSum join(MaxSum a, MaxSum b, const uint64_t* tab) 
     r.s = (a.s == 0.0 ? 0.0 : a.s * cta_exp64(a.m - m, tab)) + (b.s == 0.0 ? 0.0 : b.s * cta_exp64(b.m - m, tab));
     return r;
 }
-// W columns per lane: 2 with 128-bit accesses (cols even, pointers 16-byte aligned), else 1.
+constexpr int kColRows = 4;             // rows whose loads are in flight
+// W columns per thread: 2 with 128-bit accesses (cols even, pointers 16-byte aligned), else 1.
 template <int W>
-__global__ __launch_bounds__(256) void softmax_cols_f64_scan_kernel(const double* __restrict__ x, MaxSum* __restrict__ pairs, size_t rows,
-                                                                    size_t cols, size_t rows_per_chunk, size_t col0, size_t col_end) {
-    __shared__ MaxSum s_red[kRowGroups][kLanesPerRow * W];
-    __shared__ uint64_t s_tab[256];
-    stage_exp64_table(s_tab);
-    const unsigned lane = threadIdx.x % kLanesPerRow, group = threadIdx.x / kLanesPerRow;
-    const size_t j = col0 + (size_t(blockIdx.x) * kLanesPerRow + lane) * W;
-    const size_t first = size_t(blockIdx.y) * rows_per_chunk;
-    size_t last = first + rows_per_chunk;
-    if (last > rows) last = rows;
-    MaxSum t[W];
-#pragma unroll
-    for (int w = 0; w < W; ++w) t[w] = MaxSum{-__builtin_huge_val(), 0.0};
-    if (j < col_end) {
-#pragma unroll 4
-        for (size_t i = first + group; i < last; i += kRowGroups) {
-            double v[W];
-            if (W == 2) {
-                const v2d p = *reinterpret_cast<const v2d*>(x + i * cols + j);
-                v[0] = p[0];
-                v[W - 1] = p[1];
-            } else {
-                v[0] = x[i * cols + j];
-            }
-#pragma unroll
-            for (int w = 0; w < W; ++w) {
-                const bool up = v[w] > t[w].m;
-                const double e = cta_exp64(up ? t[w].m - v[w] : v[w] - t[w].m, s_tab);   // t.m = -inf at the start: exp(-inf) = 0
-                t[w].s = up ? t[w].s * e + 1.0 : t[w].s + e;
-                t[w].m = up ? v[w] : t[w].m;
-            }
-        }
-    }
-#pragma unroll
-    for (int w = 0; w < W; ++w) s_red[group][lane * W + w] = t[w];
-    __syncthreads();
-    if (group == 0 && j < col_end) {
-#pragma unroll
-        for (int w = 0; w < W; ++w) {
-            MaxSum r = s_red[0][lane * W + w];
-#pragma unroll
-            for (int g = 1; g < kRowGroups; ++g) r = join(r, s_red[g][lane * W + w], s_tab);
-            pairs[size_t(blockIdx.y) * cols + j + w] = r;
-        }
+__device__ __forceinline__ void load_cols(const double* __restrict__ p, double (&v)[W]) {
+    if (W == 2) {
+        const v2d t = *reinterpret_cast<const v2d*>(p);
+        v[0] = t[0];
+        v[W - 1] = t[1];
+    } else {
+        v[0] = p[0];
     }
 }
 template <int W>
-__global__ __launch_bounds__(256) void softmax_cols_f64_write_kernel(const double* __restrict__ x, const MaxSum* __restrict__ pairs,
-                                                                     double* __restrict__ y, size_t rows, size_t cols,
-                                                                     size_t rows_per_chunk, unsigned chunks, size_t col0, size_t col_end) {
-    __shared__ MaxSum s_total[kLanesPerRow * W];
+__global__ __launch_bounds__(256) void softmax_cols_f64_scan_kernel(const double* __restrict__ x, MaxSum* __restrict__ pairs, size_t rows,
+                                                                    size_t cols, size_t rows_per_chunk) {
     __shared__ uint64_t s_tab[256];
     stage_exp64_table(s_tab);
-    const unsigned lane = threadIdx.x % kLanesPerRow, group = threadIdx.x / kLanesPerRow;
-    const size_t j = col0 + (size_t(blockIdx.x) * kLanesPerRow + lane) * W;
-    // The chunks' pairs of this block's columns, brought to the column maximum: first the maximum
-    // over the chunks (no exponential), then the sums scaled to it - independent exponentials, added
-    // in chunk order.  The block's 256 threads share the work: thread t takes column t % (32 W) and
-    // every (256 / (32 W))-th chunk; the parts are added in part order.
-    {
-        constexpr int kCols = kLanesPerRow * W, kParts = 256 / kCols;
-        __shared__ double s_m[kParts][kCols], s_s[kParts][kCols];
-        const unsigned c_in = threadIdx.x % kCols, part = threadIdx.x / kCols;
-        const size_t col = col0 + size_t(blockIdx.x) * kCols + c_in;
-        double m = -__builtin_huge_val();
-        if (col < col_end)
-            for (unsigned c = part; c < chunks; c += kParts) {
-                const double v = pairs[size_t(c) * cols + col].m;
-                m = v > m ? v : m;
-            }
-        s_m[part][c_in] = m;
-        __syncthreads();
-#pragma unroll
-        for (int q = 0; q < kParts; ++q) m = s_m[q][c_in] > m ? s_m[q][c_in] : m;
-        double sum = 0.0;
-        if (col < col_end)
-            for (unsigned c = part; c < chunks; c += kParts) {
-                const MaxSum p = pairs[size_t(c) * cols + col];
-                sum += p.s == 0.0 ? 0.0 : p.s * cta_exp64(p.m - m, s_tab);
-            }
-        s_s[part][c_in] = sum;
-        __syncthreads();
-        if (part == 0) {
-            double total = 0.0;
-#pragma unroll
-            for (int q = 0; q < kParts; ++q) total += s_s[q][c_in];
-            s_total[c_in] = MaxSum{m, total};
-        }
-    }
-    __syncthreads();
-    if (j >= col_end) return;
-    MaxSum total[W];
-#pragma unroll
-    for (int w = 0; w < W; ++w) total[w] = s_total[lane * W + w];
+    const size_t j = (size_t(blockIdx.x) * 256 + threadIdx.x) * W;
+    if (j >= cols) return;
     const size_t first = size_t(blockIdx.y) * rows_per_chunk;
     size_t last = first + rows_per_chunk;
     if (last > rows) last = rows;
-#pragma unroll 4
-    for (size_t i = first + group; i < last; i += kRowGroups) {
-        if (W == 2) {
-            const v2d p = *reinterpret_cast<const v2d*>(x + i * cols + j);
-            const v2d q{cta_exp64(p[0] - total[0].m, s_tab) / total[0].s, cta_exp64(p[1] - total[W - 1].m, s_tab) / total[W - 1].s};
-            __builtin_nontemporal_store(q, reinterpret_cast<v2d*>(y + i * cols + j));
-        } else {
-            y[i * cols + j] = cta_exp64(x[i * cols + j] - total[0].m, s_tab) / total[0].s;
+    MaxSum t[2][W];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int w = 0; w < W; ++w) t[h][w] = MaxSum{-__builtin_huge_val(), 0.0};
+    auto one_row = [&](int h, const double (&v)[W]) {
+#pragma unroll
+        for (int w = 0; w < W; ++w) {
+            MaxSum& q = t[h][w];
+            const bool up = v[w] > q.m;
+            const double e = cta_exp64(up ? q.m - v[w] : v[w] - q.m, s_tab);      // q.m = -inf at the start: exp(-inf) = 0
+            q.s = up ? q.s * e + 1.0 : q.s + e;
+            q.m = up ? v[w] : q.m;
         }
+    };
+    const double* __restrict__ p = x + first * cols + j;
+    size_t i = first;
+    for (; i + kColRows <= last; i += kColRows, p += kColRows * cols) {
+        double v[kColRows][W];
+#pragma unroll
+        for (int r = 0; r < kColRows; ++r) load_cols<W>(p + size_t(r) * cols, v[r]);
+#pragma unroll
+        for (int r = 0; r < kColRows; ++r) one_row(r & 1, v[r]);
+    }
+    for (; i < last; ++i, p += cols) {
+        double v[W];
+        load_cols<W>(p, v);
+        if ((i - first) & 1) one_row(1, v);              // constant indices keep the accumulators in registers
+        else one_row(0, v);
+    }
+#pragma unroll
+    for (int w = 0; w < W; ++w) pairs[size_t(blockIdx.y) * cols + j + w] = join(t[0][w], t[1][w], s_tab);
+}
+// A block folds 16 columns; its 64 groups of 16 lanes take every 64th chunk, and the groups are
+// combined through LDS in group order (every CU takes part: a CU alone draws little bandwidth).
+constexpr int kFoldCols64 = 16, kFoldGroups64 = 64;
+__global__ __launch_bounds__(kFoldCols64 * kFoldGroups64) void softmax_cols_f64_fold_kernel(const MaxSum* __restrict__ pairs,
+                                                                                          MaxSum* __restrict__ totals, size_t cols,
+                                                                                          unsigned chunks) {
+    __shared__ uint64_t s_tab[256];
+    __shared__ double s_m[kFoldGroups64][kFoldCols64], s_s[kFoldGroups64][kFoldCols64];
+    stage_exp64_table(s_tab);
+    const unsigned lane = threadIdx.x % kFoldCols64, group = threadIdx.x / kFoldCols64;
+    const size_t c = size_t(blockIdx.x) * kFoldCols64 + lane;
+    const bool live = c < cols;
+    double m = -__builtin_huge_val();
+    if (live)
+        for (unsigned k = group; k < chunks; k += kFoldGroups64) {
+            const double v = pairs[size_t(k) * cols + c].m;
+            m = v > m ? v : m;
+        }
+    s_m[group][lane] = m;
+    __syncthreads();
+#pragma unroll 8
+    for (int g = 0; g < kFoldGroups64; ++g) m = s_m[g][lane] > m ? s_m[g][lane] : m;
+    double sum = 0.0;
+    if (live)
+        for (unsigned k = group; k < chunks; k += kFoldGroups64) {
+            const MaxSum q = pairs[size_t(k) * cols + c];
+            sum += q.s == 0.0 ? 0.0 : q.s * cta_exp64(q.m - m, s_tab);
+        }
+    s_s[group][lane] = sum;
+    __syncthreads();
+    if (group == 0 && live) {
+        double total = 0.0;
+#pragma unroll 8
+        for (int g = 0; g < kFoldGroups64; ++g) total += s_s[g][lane];
+        totals[c] = MaxSum{m, total};
+    }
+}
+template <int W>
+__global__ __launch_bounds__(256) void softmax_cols_f64_write_kernel(const double* __restrict__ x, const MaxSum* __restrict__ totals,
+                                                                     double* __restrict__ y, size_t rows, size_t cols,
+                                                                     size_t rows_per_chunk) {
+    __shared__ uint64_t s_tab[256];
+    stage_exp64_table(s_tab);
+    const size_t j = (size_t(blockIdx.x) * 256 + threadIdx.x) * W;
+    if (j >= cols) return;
+    double m[W], sum[W], inv[W];
+#pragma unroll
+    for (int w = 0; w < W; ++w) {
+        const MaxSum q = totals[j + w];
+        m[w] = q.m;
+        sum[w] = q.s;
+        inv[w] = 1.0 / q.s;
+    }
+    const size_t first = size_t(blockIdx.y) * rows_per_chunk;
+    size_t last = first + rows_per_chunk;
+    if (last > rows) last = rows;
+    auto one_row = [&](const double (&v)[W], double* __restrict__ dst) {
+        double o[W];
+#pragma unroll
+        for (int w = 0; w < W; ++w) {
+            const double e = cta_exp64(v[w] - m[w], s_tab);
+            const double q0 = e * inv[w];
+            o[w] = __builtin_fma(__builtin_fma(-q0, sum[w], e), inv[w], q0);
+        }
+        if (W == 2) __builtin_nontemporal_store(v2d{o[0], o[W - 1]}, reinterpret_cast<v2d*>(dst));
+        else dst[0] = o[0];
+    };
+    const double* __restrict__ p = x + first * cols + j;
+    double* __restrict__ d = y + first * cols + j;
+    size_t i = first;
+    for (; i + kColRows <= last; i += kColRows, p += kColRows * cols, d += kColRows * cols) {
+        double v[kColRows][W];
+#pragma unroll
+        for (int r = 0; r < kColRows; ++r) load_cols<W>(p + size_t(r) * cols, v[r]);
+#pragma unroll
+        for (int r = 0; r < kColRows; ++r) one_row(v[r], d + size_t(r) * cols);
+    }
+    for (; i < last; ++i, p += cols, d += cols) {
+        double v[W];
+        load_cols<W>(p, v);
+        one_row(v, d);
     }
 }
 
@@ -514,37 +545,33 @@ int ctamd_softmax_f64(const double* x, double* y, size_t rows, size_t cols, int 
         else hipLaunchKernelGGL(softmax_rows_f64_kernel, dim3(blocks), dim3(cols <= 64 ? 64 : 256), 0, s, x, y, rows, cols);
     } else {
         const bool wide = cols % 2 == 0 && aligned16(x) && aligned16(y);
-        const size_t per_block = size_t(kLanesPerRow) * (wide ? 2 : 1);
+        const size_t per_block = size_t(256) * (wide ? 2 : 1);
         // (Column panels of 64 - 128 MiB, scanned and written in turn so that the writing launch would find
         // its panel in the memory-side cache, were measured: 445 us against 345 us for the whole matrix
         // at once on [8192 x 8192] - a panel's launches are too small to fill the chip.)
-        const size_t panel_cols = cols;
-        const size_t cus = compute_units() > 0 ? size_t(compute_units()) : 256;
+        const size_t strips = (cols + per_block - 1) / per_block;
+        if (strips > 0x7fffffffu) return fail(CTAMD_ERANGE, "%s: too many columns", __func__);
         MaxSum* pairs = reinterpret_cast<MaxSum*>(scratch(stream));
         if (!pairs) return CTAMD_EINVAL;
-        for (size_t col0 = 0; col0 < cols; col0 += panel_cols) {
-            const size_t col_end = col0 + panel_cols < cols ? col0 + panel_cols : cols;
-            const size_t strips = (col_end - col0 + per_block - 1) / per_block;
-            if (strips > 0x7fffffffu) return fail(CTAMD_ERANGE, "%s: too many columns", __func__);
-            // chunks of rows so that the grid fills the chip (about eight blocks per CU), of at least 64
-            // rows each, as many as the scratch holds pairs for
-            size_t chunks = (8 * cus + strips - 1) / strips;
-            if (chunks > (rows + 63) / 64) chunks = (rows + 63) / 64;
-            const size_t room = kScratchFloats * sizeof(float) / sizeof(MaxSum) / cols;
-            if (chunks > room) chunks = room;
-            if (chunks > 65535) chunks = 65535;
-            if (chunks < 1) return fail(CTAMD_ERANGE, "%s: more than %zu columns", __func__, kScratchFloats * sizeof(float) / sizeof(MaxSum));
-            const size_t rows_per_chunk = (rows + chunks - 1) / chunks;
-            chunks = (rows + rows_per_chunk - 1) / rows_per_chunk;
-            const dim3 grid{unsigned(strips), unsigned(chunks), 1u};
-            if (wide) {
-                hipLaunchKernelGGL(softmax_cols_f64_scan_kernel<2>, grid, dim3(256), 0, s, x, pairs, rows, cols, rows_per_chunk, col0, col_end);
-                hipLaunchKernelGGL(softmax_cols_f64_write_kernel<2>, grid, dim3(256), 0, s, x, pairs, y, rows, cols, rows_per_chunk, unsigned(chunks), col0, col_end);
-            } else {
-                hipLaunchKernelGGL(softmax_cols_f64_scan_kernel<1>, grid, dim3(256), 0, s, x, pairs, rows, cols, rows_per_chunk, col0, col_end);
-                hipLaunchKernelGGL(softmax_cols_f64_write_kernel<1>, grid, dim3(256), 0, s, x, pairs, y, rows, cols, rows_per_chunk, unsigned(chunks), col0, col_end);
-            }
-        }
+        // chunks of at least 32 rows, at most 256 of them (half as many ran the two sweeps 15% slower: they
+        // are bound by the exponential's arithmetic and want the blocks), as many as the scratch holds
+        // pairs for beside the columns' totals
+        const size_t slots = kScratchFloats * sizeof(float) / sizeof(MaxSum);
+        if (cols > slots / 2) return fail(CTAMD_ERANGE, "%s: more than %zu columns", __func__, slots / 2);
+        size_t chunks = (rows + 31) / 32;
+        if (chunks > 256) chunks = 256;
+        const size_t room = (slots - cols) / cols;
+        if (chunks > room) chunks = room;
+        const size_t rows_per_chunk = (rows + chunks - 1) / chunks;
+        chunks = (rows + rows_per_chunk - 1) / rows_per_chunk;
+        MaxSum* totals = pairs + chunks * cols;
+        const dim3 grid{unsigned(strips), unsigned(chunks), 1u};
+        const dim3 fold_grid{unsigned((cols + kFoldCols64 - 1) / kFoldCols64), 1u, 1u};
+        if (wide) hipLaunchKernelGGL(softmax_cols_f64_scan_kernel<2>, grid, dim3(256), 0, s, x, pairs, rows, cols, rows_per_chunk);
+        else hipLaunchKernelGGL(softmax_cols_f64_scan_kernel<1>, grid, dim3(256), 0, s, x, pairs, rows, cols, rows_per_chunk);
+        hipLaunchKernelGGL(softmax_cols_f64_fold_kernel, fold_grid, dim3(kFoldCols64 * kFoldGroups64), 0, s, pairs, totals, cols, unsigned(chunks));
+        if (wide) hipLaunchKernelGGL(softmax_cols_f64_write_kernel<2>, grid, dim3(256), 0, s, x, totals, y, rows, cols, rows_per_chunk);
+        else hipLaunchKernelGGL(softmax_cols_f64_write_kernel<1>, grid, dim3(256), 0, s, x, totals, y, rows, cols, rows_per_chunk);
     }
     account(double(rows) * double(cols) * 16.0, 0.0);
     return launched(__func__);
