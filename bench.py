@@ -242,11 +242,15 @@ def config_report(with_cpu):
         # the same step (one-hot targets) recorded into a HIP graph once and replayed
         oh = np.zeros((Bn, 10), np.float32)
         oh[np.arange(Bn), lab.astype(int)] = 1
-        out = D5()
-        rc = host.cth_time_mlp_graph(fp(x), L(Bn), L(784), fp(W1), fp(b1), L(256), fp(W2), fp(b2), L(10), fp(oh), I(5),
-                                     I(30), out)
-        add("config 3: MLP 784-256-10 train step, batch %d, replayed from a recorded HIP graph" % Bn, rc, out, cpu, note)
-        rows[-1]["launches_recorded"] = rows[-1].pop("launches")
+        for fused in (0, 1):
+            host.cth_set_fused_layers(fused)
+            out = D5()
+            rc = host.cth_time_mlp_graph(fp(x), L(Bn), L(784), fp(W1), fp(b1), L(256), fp(W2), fp(b2), L(10), fp(oh), I(5),
+                                         I(30), out)
+            host.cth_set_fused_layers(0)
+            add("config 3: MLP 784-256-10 train step, batch %d, %sreplayed from a recorded HIP graph"
+                % (Bn, "fused layers, " if fused else ""), rc, out, cpu, note)
+            rows[-1]["launches_recorded"] = rows[-1].pop("launches")
 
     # config 4: row softmax + cross entropy, [8192 x 32000]
     R4, C4 = 8192, 32000
