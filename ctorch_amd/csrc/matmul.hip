@@ -37,9 +37,14 @@ constexpr int kXcds = 8;
 constexpr int kMinWavesPerSimd = 2;   // register budget of both tile shapes: 256 VGPRs per lane
 
 
-template <int BM_, int BN_, int BK_, int WM_, int WN_>
+template <int BM_, int BN_, int BK_, int WM_, int WN_, bool EARLY_ = false>
 struct Cfg {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
+    // EARLY: the staged tile goes to LDS, and the next tile is requested from global memory, at the
+    // top of a k tile instead of around its barrier.  The request then has a whole k tile to arrive;
+    // where a k tile is a handful of MFMAs (the 64 x 64 and 128 x 128 block tiles: 8 and 32 per wave)
+    // the later place left it half of that, less than the latency of the L2.
+    static constexpr bool EARLY = EARLY_;
     static constexpr int TM = WM / 32, TN = WN / 32;       // MFMA tiles per wave
     static constexpr int WAVES_N = BN / WN;
     static constexpr int THREADS = (BM / WM) * (BN / WN) * 64;
@@ -290,43 +295,64 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
         for (int t = 0; t + 1 < ktiles; ++t) {
             const int cur = t & 1;
             __builtin_amdgcn_sched_barrier(0);
+            if (C::EARLY) {
+                // buffer cur ^ 1 is free since the last barrier; its first readers wait behind the next
+                sa.store(s_a[cur ^ 1], A_STRIDE);
+                sb.store(s_b[cur ^ 1], B_STRIDE);
+                const bool more = t + 3 < ktiles;
+                sa.load_fast(more ? a_step : 0);
+                sb.load_fast(more ? b_step : 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
             lds_wait();
             fetch_chunk(cur, 1, 1);
             mfmas(0);
-            sa.store(s_a[cur ^ 1], A_STRIDE);
-            sb.store(s_b[cur ^ 1], B_STRIDE);
+            if (!C::EARLY) {
+                sa.store(s_a[cur ^ 1], A_STRIDE);
+                sb.store(s_b[cur ^ 1], B_STRIDE);
+            }
 #pragma unroll
             for (int q = 0; q < kReadSlots; ++q) {
                 __builtin_amdgcn_sched_group_barrier(kMaskMfma, 1, 0);
                 __builtin_amdgcn_sched_group_barrier(kMaskDsRead, 1, 0);
             }
-            if (kMfmaPerChunk - kReadSlots - kStores > 0)
-                __builtin_amdgcn_sched_group_barrier(kMaskMfma, kMfmaPerChunk - kReadSlots - kStores, 0);
+            if (C::EARLY) {
+                if (kMfmaPerChunk - kReadSlots > 0) __builtin_amdgcn_sched_group_barrier(kMaskMfma, kMfmaPerChunk - kReadSlots, 0);
+            } else {
+                if (kMfmaPerChunk - kReadSlots - kStores > 0)
+                    __builtin_amdgcn_sched_group_barrier(kMaskMfma, kMfmaPerChunk - kReadSlots - kStores, 0);
 #pragma unroll
-            for (int q = 0; q < kStores; ++q) {
-                __builtin_amdgcn_sched_group_barrier(kMaskMfma, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(kMaskDsWrite, 1, 0);
+                for (int q = 0; q < kStores; ++q) {
+                    __builtin_amdgcn_sched_group_barrier(kMaskMfma, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(kMaskDsWrite, 1, 0);
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
             __syncthreads();
             __builtin_amdgcn_sched_barrier(0);
             fetch_chunk(cur ^ 1, 0, 0);
-            const bool more = t + 3 < ktiles;
-            sa.load_fast(more ? a_step : 0);
-            sb.load_fast(more ? b_step : 0);
+            if (!C::EARLY) {
+                const bool more = t + 3 < ktiles;
+                sa.load_fast(more ? a_step : 0);
+                sb.load_fast(more ? b_step : 0);
+            }
             mfmas(1);
 #pragma unroll
             for (int q = 0; q < kReadSlots; ++q) {
                 __builtin_amdgcn_sched_group_barrier(kMaskMfma, 1, 1);
                 __builtin_amdgcn_sched_group_barrier(kMaskDsRead, 1, 1);
             }
+            if (C::EARLY) {
+                if (kMfmaPerChunk - kReadSlots > 0) __builtin_amdgcn_sched_group_barrier(kMaskMfma, kMfmaPerChunk - kReadSlots, 1);
+            } else {
 #pragma unroll
-            for (int q = 0; q < kStores; ++q) {
-                __builtin_amdgcn_sched_group_barrier(kMaskMfma, 1, 1);
-                __builtin_amdgcn_sched_group_barrier(kMaskVmemRead, 1, 1);
+                for (int q = 0; q < kStores; ++q) {
+                    __builtin_amdgcn_sched_group_barrier(kMaskMfma, 1, 1);
+                    __builtin_amdgcn_sched_group_barrier(kMaskVmemRead, 1, 1);
+                }
+                if (kMfmaPerChunk - kReadSlots - kStores > 0)
+                    __builtin_amdgcn_sched_group_barrier(kMaskMfma, kMfmaPerChunk - kReadSlots - kStores, 1);
             }
-            if (kMfmaPerChunk - kReadSlots - kStores > 0)
-                __builtin_amdgcn_sched_group_barrier(kMaskMfma, kMfmaPerChunk - kReadSlots - kStores, 1);
             __builtin_amdgcn_sched_barrier(0);
         }
     } else {
@@ -833,6 +859,10 @@ using BigTile = Cfg<256, 256, 16, 128, 64>;
 using SmallTile = Cfg<128, 128, 16, 64, 64>;
 using TinyTile = Cfg<64, 64, 16, 32, 32>;
 using WideTile = Cfg<256, 128, 16, 128, 64>;
+// the 64 x 64 tile for a launch of at most one block per CU: no other block hides the wait for the next
+// tile ([1024 x 1024, K = 2048]: 67 -> 45 us; with several blocks per CU it is 1-2% slower, as is the
+// 128 x 128 tile either way)
+using TinyEarlyTile = Cfg<64, 64, 16, 32, 32, true>;
 
 template <class Tile, bool A_KC, bool B_KC>
 int launch_gemm(GemmArgs g, bool vec, int blocks, hipStream_t s) {
@@ -1012,7 +1042,8 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
     // a tile outside [0, whole_tiles) writes its parts to g.partial: there is none unless the plan cut K
     if (splits == 1 && whole_tiles != tiles) return fail(CTAMD_EINVAL, "%s: plan leaves %d tiles without a part buffer", name, tiles - whole_tiles);
     const int blocks = whole_tiles + (tiles - whole_tiles) * splits;
-    int rc = shape == 3 ? launch_layout<WideTile>(g, A_KC, B_KC, vec, blocks, s)
+    int rc = (shape == 0 && blocks <= cus) ? launch_layout<TinyEarlyTile>(g, A_KC, B_KC, vec, blocks, s)
+           : shape == 3 ? launch_layout<WideTile>(g, A_KC, B_KC, vec, blocks, s)
            : shape == 2 ? launch_layout<BigTile>(g, A_KC, B_KC, vec, blocks, s)
            : shape == 1 ? launch_layout<SmallTile>(g, A_KC, B_KC, vec, blocks, s)
                         : launch_layout<TinyTile>(g, A_KC, B_KC, vec, blocks, s);
