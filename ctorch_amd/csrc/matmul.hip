@@ -755,7 +755,7 @@ __global__ __launch_bounds__(kNarrowWaves * 64) void gemm_narrow_cols(const floa
     const int t = threadIdx.x;
     if (t >= 64 * N) return;
     const int j = t / N, q = t % N;
-    if (blockIdx.x * 64 + j >= m) return;
+    if (int(blockIdx.x) * 64 + j >= m) return;
     float total = s_mem[q * 64 + j];
 #pragma unroll
     for (int w = 1; w < kNarrowWaves; ++w) total = total + s_mem[(w * N + q) * 64 + j];

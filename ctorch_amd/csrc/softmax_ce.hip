@@ -1100,6 +1100,8 @@ __global__ __launch_bounds__(256) void col_walk_kernel(const float* __restrict__
             v4f t;
 #pragma unroll
             for (int e = 0; e < W; ++e) t[e] = v[e];
+            // always with the streaming hint: the pass that writes re-reads x, and what the memory-side cache
+            // still holds of x from the pass before must not be pushed out by the result (139 against 161 us)
             __builtin_nontemporal_store(t, reinterpret_cast<v4f*>(out + r * cols + col));
         } else {
             out[r * cols + col] = v[0];
