@@ -13,7 +13,7 @@ import pytest
 import torch
 
 import gpu_support as G
-from support import (ADD, COS, DIV, MUL, NEG, RELU, SIGMOID, SIN, SUB, TANH, f32, same_bits, ulp_diff)
+from support import (ADD, COS, DIV, EX, MUL, NEG, RELU, SIGMOID, SIN, SUB, TANH, f32, same_bits, ulp_diff)
 
 pytestmark = pytest.mark.gpu
 
@@ -53,6 +53,31 @@ def test_binary_same_shape_bit_exact(oracle, n):
     da, db = G.dev(a), G.dev(b)
     for name, code in BIN:
         bits_equal(G.host(G.binary(name, da, db)), oracle.binary(code, a, b), name)
+
+
+@pytest.mark.parametrize("n", [(6 << 20) + 8, (1 << 24) - 4, (1 << 24) + 4])
+def test_large_streams_take_every_access_hint_variant_bit_exact(oracle, n):
+    """Above 64 MiB of operands + result the loads carry the streaming hint, and above 64 MiB of
+    result the stores do too: one size per variant of the plain kernels, the row-broadcast kernel
+    and the fused-expression kernel (whose first result is the one that may go unhinted)."""
+    print("case access hints n", n, flush=True)
+    a = oracle.normal((n,), 11, 0, 3)
+    b = oracle.normal((n,), 12, 0, 3)
+    da, db = G.dev(a), G.dev(b)
+    bits_equal(G.host(G.binary("add", da, db)), oracle.binary(dict(BIN)["add"], a, b), "add")
+    bits_equal(G.host(G.unary("relu", da)), np.where(a > 0, a, np.float32(0)).astype(np.float32), "relu")
+    cols = 4
+    r = oracle.uniform((cols,), 13, 0.5, 2)
+    got = G.host(G.rowbcast("mul", da.view(n // cols, cols), G.dev(r)))
+    bits_equal(got.reshape(-1), (a.reshape(-1, cols) * r).astype(np.float32).reshape(-1), "row-broadcast mul")
+    E = EX
+    prog = [(E["LOAD_FULL"], 0, 0, 0, 0.0), (E["LOAD_FULL"], 1, 1, 0, 0.0), (E["MUL"], 2, 0, 1, 0.0), (E["ADDS"], 3, 2, 0, 5.0),
+            (E["RELU"], 4, 3, 0, 0.0), (E["STORE"], 0, 4, 0, 0.0), (E["STORE"], 1, 2, 0, 0.0)]
+    (y, p), _ = G.expr_run(prog, [da.view(n // cols, cols), db.view(n // cols, cols)], 2, n // cols, cols)
+    ab = (a * b).astype(np.float32)
+    t = (ab + np.float32(5.0)).astype(np.float32)
+    bits_equal(G.host(y).reshape(-1), np.where(t > 0, t, np.float32(0)).astype(np.float32), "fused relu(a*b+5)")
+    bits_equal(G.host(p).reshape(-1), ab, "fused a*b (second result)")
 
 
 def test_binary_unaligned_views_bit_exact(oracle):
