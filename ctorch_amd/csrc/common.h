@@ -62,23 +62,18 @@ inline unsigned stream_grid(size_t work_items, size_t per_block, int blocks_per_
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // A result of at most this many bytes - a quarter of the 256 MiB memory-side cache - is stored
-// without the streaming hint: what reads it next finds it in that cache, and a buffer that is
-// overwritten before it was evicted never costs HBM a write (the 28 launches of a forward and
-// backward pass over 64 MiB tensors: 851 -> 822 us).  Measured at 256 MiB per tensor, one input:
-// a chain in which every launch reads the result of the one before runs 78 us per launch with
-// hinted loads and plain stores against 85 us with the hint on both sides, but launches over
-// unrelated buffers lose (89 against 87 us; a kernel that re-reads its input, like the column
+// without the streaming hint by the elementwise kernels: what reads it next finds it in that cache,
+// and a buffer that is overwritten before it was evicted never costs HBM a write (the 28 launches of
+// a forward and backward pass over 64 MiB tensors: 851 -> 822 us).  Measured at 256 MiB per tensor,
+// one input: a chain in which every launch reads the result of the one before runs 78 us per launch
+// with hinted loads and plain stores against 85 us with the hint on both sides, but launches over
+// unrelated buffers lose (88 against 84 us; a kernel that re-reads its input, like the column
 // softmax, 161 against 139 us: the result pushes the input out), and at 1 GiB per tensor the hint
 // on both sides wins too (352 against 365 us).  Hence the bound well below the cache size.
+// The choice has to be a template argument of the kernel: a hinted and a plain store on the two
+// sides of a branch are folded by the compiler into ONE plain store.
 constexpr size_t kResidentBytes = size_t(64) << 20;
 inline bool result_streams(size_t bytes) { return bytes > kResidentBytes; }
-#if defined(__HIPCC__)
-template <class V>
-__device__ __forceinline__ void store_result(V* dst, V v, bool streams) {   // `streams` is uniform
-    if (streams) __builtin_nontemporal_store(v, dst);
-    else *dst = v;
-}
-#endif
 
 }  // namespace ctamd
 

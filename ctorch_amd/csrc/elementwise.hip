@@ -40,33 +40,35 @@ __device__ __forceinline__ float apply1(const F& f, const float* x, const Tables
     }
 }
 
-// 128-bit accesses.  Loads of large tensors carry the non-temporal hint: the operands are touched
-// once, and keeping them out of the caches' replacement order measured fastest on MI355X (6.2 TB/s
-// for a + b at 256 MiB per operand, against 5.5 TB/s with plain accesses and 4.7 TB/s for a
-// grid-stride loop whose four accesses per thread lie far apart).  The result carries the hint
-// only when it is too large to be worth keeping in the memory-side cache for its reader
-// (result_streams()).  With two or more streams of 256 MiB left unhinted that cache thrashes and
-// the time is that of no hints at all.  Small tensors (a chain of ops on a few MiB) use plain
-// accesses throughout, so that the next kernel finds its operands in L2.
-template <bool NT>
+// 128-bit accesses with the non-temporal hint: these streams touch every byte once, and keeping
+// them out of the caches' replacement order measured fastest on MI355X (6.2 TB/s for a + b at
+// 256 MiB per operand, against 5.5 TB/s with plain accesses and 4.7 TB/s for a grid-stride loop
+// whose four accesses per thread lie far apart).
+// Small tensors (a chain of ops on a few MiB) keep plain accesses so that the next kernel finds
+// its operands in L2 / Infinity Cache.  NT, chosen by the launcher from the bytes touched: 0 plain
+// accesses, 1 hinted loads and a plain store (the result is small enough to be kept in the
+// memory-side cache for its reader: result_streams()), 2 the hint on both sides.
+template <int NT>
 __device__ __forceinline__ v4f ld_stream(const float* p, size_t i4) {
-    if (NT) return __builtin_nontemporal_load(reinterpret_cast<const v4f*>(p) + i4);
+    if (NT >= 1) return __builtin_nontemporal_load(reinterpret_cast<const v4f*>(p) + i4);
     return reinterpret_cast<const v4f*>(p)[i4];
 }
-// out_streams: the result is too large to be kept for its reader (a uniform branch)
-template <bool NT>
-__device__ __forceinline__ void st_stream(float* p, size_t i4, v4f v, bool out_streams) {
-    if (NT && out_streams) __builtin_nontemporal_store(v, reinterpret_cast<v4f*>(p) + i4);
+template <int NT>
+__device__ __forceinline__ void st_stream(float* p, size_t i4, v4f v) {
+    if (NT == 2) __builtin_nontemporal_store(v, reinterpret_cast<v4f*>(p) + i4);
     else reinterpret_cast<v4f*>(p)[i4] = v;
 }
-// operands + result above this many bytes: loads carry the hint
+// operands + result above this many bytes cannot stay cache resident (256 MiB Infinity Cache)
 constexpr size_t kStreamBytes = size_t(64) << 20;
+inline int hint_level(size_t all_bytes, size_t result_bytes) {
+    return all_bytes >= kStreamBytes ? (result_streams(result_bytes) ? 2 : 1) : 0;
+}
 
 // The work of one thread of a vector block: its kUnroll vectors per operand, all loaded before the
 // first use.  CHECK guards each vector against the end of the tensor (last block only).
-template <class F, bool NT, bool CHECK>
+template <class F, int NT, bool CHECK>
 __device__ __forceinline__ void map_block(const Ptrs<F::kIn>& in, float* __restrict__ out, size_t n4, size_t base,
-                                          const F& f, const Tables& tabs, bool out_streams) {
+                                          const F& f, const Tables& tabs) {
     constexpr int NI = F::kIn;
     v4f v[NI > 0 ? NI : 1][kUnroll];
 #pragma unroll
@@ -100,7 +102,7 @@ __device__ __forceinline__ void map_block(const Ptrs<F::kIn>& in, float* __restr
                     }
                 }
             }
-            st_stream<NT>(out, i, o, out_streams);
+            st_stream<NT>(out, i, o);
         }
     }
 }
@@ -109,8 +111,8 @@ __device__ __forceinline__ void map_block(const Ptrs<F::kIn>& in, float* __restr
 // vectors starting at b*kThreads*kUnroll (no loop: the grid covers the tensor), thread t takes
 // vectors t, t+256, t+512, t+768 of that run, all loads issued before the first use.  The last
 // n % 4 elements are handled by block 0.  VEC = false: scalar grid-stride (unaligned views).
-template <class F, bool VEC, bool NT>
-__global__ __launch_bounds__(kThreads) void map_kernel(Ptrs<F::kIn> in, float* __restrict__ out, size_t n, F f_in, bool out_streams) {
+template <class F, bool VEC, int NT>
+__global__ __launch_bounds__(kThreads) void map_kernel(Ptrs<F::kIn> in, float* __restrict__ out, size_t n, F f_in) {
     __shared__ uint64_t s_exp2[F::kTables ? 32 : 1];
     __shared__ uint32_t s_pio4[F::kTables ? 24 : 1];
     __shared__ double s_log[HasLogTable<F>::value ? 32 : 1];
@@ -124,9 +126,9 @@ __global__ __launch_bounds__(kThreads) void map_kernel(Ptrs<F::kIn> in, float* _
         const size_t n4 = n >> 2;
         const size_t block_base = size_t(blockIdx.x) * (kThreads * kUnroll);
         if (block_base + size_t(kThreads) * kUnroll <= n4)
-            map_block<B, NT, false>(in, out, n4, block_base + threadIdx.x, f, tabs, out_streams);   // interior block: no bounds checks
+            map_block<B, NT, false>(in, out, n4, block_base + threadIdx.x, f, tabs);   // interior block: no bounds checks
         else
-            map_block<B, NT, true>(in, out, n4, block_base + threadIdx.x, f, tabs, out_streams);
+            map_block<B, NT, true>(in, out, n4, block_base + threadIdx.x, f, tabs);
         if (blockIdx.x == 0) {
             size_t i = (n4 << 2) + threadIdx.x;
             if (i < n) {
@@ -161,14 +163,16 @@ int launch_map(const char* name, Ptrs<F::kIn> in, float* out, size_t n, F f, voi
         size_t blocks = (n / 4 + size_t(kThreads) * kUnroll - 1) / (size_t(kThreads) * kUnroll);
         if (blocks < 1) blocks = 1;
         if (blocks > 0x7fffffffu) return fail(CTAMD_ERANGE, "%s: more than 2^43 elements", name);
-        const bool out_streams = result_streams(n * sizeof(float));
-        if (n * sizeof(float) * (F::kIn + 1) >= kStreamBytes)
-            hipLaunchKernelGGL((map_kernel<F, true, true>), dim3(unsigned(blocks)), dim3(kThreads), 0, as_stream(stream), in, out, n, f, out_streams);
+        const int hint = hint_level(n * sizeof(float) * (F::kIn + 1), n * sizeof(float));
+        if (hint == 2)
+            hipLaunchKernelGGL((map_kernel<F, true, 2>), dim3(unsigned(blocks)), dim3(kThreads), 0, as_stream(stream), in, out, n, f);
+        else if (hint == 1)
+            hipLaunchKernelGGL((map_kernel<F, true, 1>), dim3(unsigned(blocks)), dim3(kThreads), 0, as_stream(stream), in, out, n, f);
         else
-            hipLaunchKernelGGL((map_kernel<F, true, false>), dim3(unsigned(blocks)), dim3(kThreads), 0, as_stream(stream), in, out, n, f, false);
+            hipLaunchKernelGGL((map_kernel<F, true, 0>), dim3(unsigned(blocks)), dim3(kThreads), 0, as_stream(stream), in, out, n, f);
     } else {
         unsigned grid = stream_grid(n, size_t(kThreads) * kUnroll);
-        hipLaunchKernelGGL((map_kernel<F, false, false>), dim3(grid), dim3(kThreads), 0, as_stream(stream), in, out, n, f, false);
+        hipLaunchKernelGGL((map_kernel<F, false, 0>), dim3(grid), dim3(kThreads), 0, as_stream(stream), in, out, n, f);
     }
     account(double(F::kIn + 1) * 4.0 * double(n), 0.0);
     return launched(name);
@@ -177,10 +181,10 @@ int launch_map(const char* name, Ptrs<F::kIn> in, float* out, size_t n, F f, voi
 // r[i,j] = a[i,j] (op) b[j].  VEC: cols % 4 == 0 and aligned pointers - every 128-bit vector of a
 // meets one aligned vector of b (served from cache: b is cols*4 bytes, read rows times).
 // r[i, j] = Op(a[i, j], b[j]) or, for an Op with kIn == 3, Op(a[i, j], b[j], g[i, j]).
-template <class Op, bool VEC, class Index, bool NT>
+template <class Op, bool VEC, class Index, int NT>
 __global__ __launch_bounds__(kThreads) void rowbcast_kernel(const float* __restrict__ a, const float* __restrict__ b,
                                                             const float* __restrict__ g, float* __restrict__ r,
-                                                            size_t total, Index cols, bool out_streams) {
+                                                            size_t total, Index cols) {
     const Tables tabs{nullptr, nullptr, nullptr};
     constexpr bool kThird = (Op::kIn == 3);
     if (VEC) {
@@ -207,7 +211,7 @@ __global__ __launch_bounds__(kThreads) void rowbcast_kernel(const float* __restr
                     float x[3] = {va[u][e], vb[u][e], kThird ? vg[u][e] : 0.0f};
                     o[e] = Op()(x, tabs);
                 }
-                st_stream<NT>(r, i, o, out_streams);
+                st_stream<NT>(r, i, o);
             }
         }
     } else {
@@ -233,18 +237,19 @@ int launch_rowbcast(const char* name, const float* a, const float* b, float* r, 
     if (blocks > 0x7fffffffu) return fail(CTAMD_ERANGE, "%s: more than 2^43 elements", name);
     unsigned grid = vec ? unsigned(blocks) : stream_grid(total, size_t(kThreads) * kUnroll);
     hipStream_t s = as_stream(stream);
-    const bool nt = total * sizeof(float) * 2 >= kStreamBytes;
-    const bool out_streams = result_streams(total * sizeof(float));
-    if (vec && small && nt)
-        hipLaunchKernelGGL((rowbcast_kernel<Op, true, uint32_t, true>), dim3(grid), dim3(kThreads), 0, s, a, b, g, r, total, uint32_t(cols), out_streams);
+    const int hint = hint_level(total * sizeof(float) * 2, total * sizeof(float));
+    if (vec && small && hint == 2)
+        hipLaunchKernelGGL((rowbcast_kernel<Op, true, uint32_t, 2>), dim3(grid), dim3(kThreads), 0, s, a, b, g, r, total, uint32_t(cols));
+    else if (vec && small && hint == 1)
+        hipLaunchKernelGGL((rowbcast_kernel<Op, true, uint32_t, 1>), dim3(grid), dim3(kThreads), 0, s, a, b, g, r, total, uint32_t(cols));
     else if (vec && small)
-        hipLaunchKernelGGL((rowbcast_kernel<Op, true, uint32_t, false>), dim3(grid), dim3(kThreads), 0, s, a, b, g, r, total, uint32_t(cols), out_streams);
+        hipLaunchKernelGGL((rowbcast_kernel<Op, true, uint32_t, 0>), dim3(grid), dim3(kThreads), 0, s, a, b, g, r, total, uint32_t(cols));
     else if (vec)
-        hipLaunchKernelGGL((rowbcast_kernel<Op, true, uint64_t, true>), dim3(grid), dim3(kThreads), 0, s, a, b, g, r, total, uint64_t(cols), out_streams);
+        hipLaunchKernelGGL((rowbcast_kernel<Op, true, uint64_t, 2>), dim3(grid), dim3(kThreads), 0, s, a, b, g, r, total, uint64_t(cols));
     else if (small)
-        hipLaunchKernelGGL((rowbcast_kernel<Op, false, uint32_t, false>), dim3(grid), dim3(kThreads), 0, s, a, b, g, r, total, uint32_t(cols), out_streams);
+        hipLaunchKernelGGL((rowbcast_kernel<Op, false, uint32_t, 0>), dim3(grid), dim3(kThreads), 0, s, a, b, g, r, total, uint32_t(cols));
     else
-        hipLaunchKernelGGL((rowbcast_kernel<Op, false, uint64_t, false>), dim3(grid), dim3(kThreads), 0, s, a, b, g, r, total, uint64_t(cols), out_streams);
+        hipLaunchKernelGGL((rowbcast_kernel<Op, false, uint64_t, 0>), dim3(grid), dim3(kThreads), 0, s, a, b, g, r, total, uint64_t(cols));
     account((Op::kIn == 3 ? 12.0 : 8.0) * double(total) + 4.0 * double(cols), 0.0);
     return launched(name);
 }

@@ -79,7 +79,6 @@ struct alignas(16) ExprArgs {
     int has_row;                              // the program loads a row vector
     int n_lead;                               // the first n_lead instructions are loads (at most kLeadLoads)
     int n_tail;                               // VEC: the last n_tail instructions are stores (at most kTailStores)
-    int keep_first;                           // the first of those stores goes without the streaming hint
     alignas(16) DevInsn prog[kMaxInsns + 1];  // one spare: the kernel fetches an instruction ahead
 };
 
@@ -196,11 +195,11 @@ __device__ __forceinline__ Vals<H> load_elements(const ExprArgs& g, const Insn& 
     if (VEC) {
         // One load with the streaming hint for both kinds of operand.  Written as a hinted load of
         // a full tensor and a plain one of a row vector, the compiler folds the two into ONE plain
-        // load of a selected address, and the operands lose their hint: relaunched over the same two
-        // inputs of 256 MiB each, a + b then takes 148 instead of 126 us, because the unhinted streams
-        // turn the memory-side cache over.  Kept apart as two loads under a branch they cost more
-        // than that gains (the nine-operator program: 236 against 223 us).  A row vector is small
-        // enough to be found in L2 again whatever its hint says.
+        // load of a selected address, and the operands lose their hint: with two inputs of 256 MiB
+        // each, a + b then takes 148 instead of 139 us and relu(a * b + 5) 139 instead of 130 us.
+        // Kept apart as two loads under a branch they cost more than that gains (the nine-operator
+        // program: 236 against 223 us).  A row vector is small enough to be found in L2 again
+        // whatever its hint says.
 #pragma unroll
         for (int h = 0; h < H; ++h) {
             const size_t w = at.first + size_t(h) * kExprThreads;
@@ -286,10 +285,7 @@ __global__ __launch_bounds__(kExprThreads, FASTM ? 4 : 3) void expr_kernel(ExprA
                     v4f* __restrict__ dst = reinterpret_cast<v4f*>(g.out[fetch_insn<WHOLE>(g, g.n_insn - g.n_tail + k).dst]) + post_at;
 #pragma unroll
                     for (int h = 0; h < H; ++h)
-                        if (post_full[h]) {
-                            if (k == 0 && g.keep_first) dst[h * kExprThreads] = post[k].h[h];
-                            else __builtin_nontemporal_store(post[k].h[h], dst + h * kExprThreads);
-                        }
+                        if (post_full[h]) __builtin_nontemporal_store(post[k].h[h], dst + h * kExprThreads);
                 }
         }
     };
@@ -481,9 +477,6 @@ extern "C" int ctamd_expr_run_f32(const ctamd_expr_insn* prog, int n_insn, const
     while (g.n_lead < n_insn && g.n_lead < kLeadLoads &&
            (prog[g.n_lead].op == CTAMD_EX_LOAD_FULL || prog[g.n_lead].op == CTAMD_EX_LOAD_ROW))
         ++g.n_lead;
-    // One result stays in the memory-side cache for whatever reads it next, if it is small enough
-    // for that; every other stream carries the hint (two unhinted large streams thrash the cache).
-    g.keep_first = result_streams(total * sizeof(float)) ? 0 : 1;
     g.n_tail = 0;
     while (g.n_tail < kTailStores && g.n_lead + g.n_tail < n_insn &&
            (prog[n_insn - 1 - g.n_tail].op == CTAMD_EX_STORE || prog[n_insn - 1 - g.n_tail].op == CTAMD_EX_STORE_ZP))

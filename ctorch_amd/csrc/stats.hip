@@ -362,8 +362,7 @@ template <int KIND, bool VEC, int GROUP>
 __global__ __launch_bounds__(kThreads) void reduce_rows_backward_kernel(const float* __restrict__ x, const float* __restrict__ y,
                                                                         const int32_t* __restrict__ index, const float* __restrict__ mean,
                                                                         const float* __restrict__ g, float* __restrict__ dx, size_t rows,
-                                                                        size_t cols, size_t chunk_len, unsigned chunks, int ddof,
-                                                                        bool out_streams) {
+                                                                        size_t cols, size_t chunk_len, unsigned chunks, int ddof) {
     constexpr int kGroups = kThreads / GROUP;
     const unsigned lane = threadIdx.x % GROUP;
     const size_t work = size_t(blockIdx.x) * kGroups + threadIdx.x / GROUP;
@@ -389,7 +388,7 @@ __global__ __launch_bounds__(kThreads) void reduce_rows_backward_kernel(const fl
                 v4f o;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) o[e] = grad_one<KIND>(u, reads_x<KIND>() ? v[k][e] : 0.0f, unsigned((i + size_t(k) * GROUP) * 4 + e));
-                store_result(reinterpret_cast<v4f*>(dr) + i + size_t(k) * GROUP, o, out_streams);
+                __builtin_nontemporal_store(o, reinterpret_cast<v4f*>(dr) + i + size_t(k) * GROUP);
             }
         }
         for (; i < v1; i += GROUP) {
@@ -408,8 +407,7 @@ template <int KIND, int W>
 __global__ __launch_bounds__(kThreads) void reduce_cols_backward_kernel(const float* __restrict__ x, const float* __restrict__ y,
                                                                         const int32_t* __restrict__ index, const float* __restrict__ mean,
                                                                         const float* __restrict__ g, float* __restrict__ dx, size_t len,
-                                                                        size_t inner, size_t rows_per_chunk, unsigned tx_count, int ddof,
-                                                                        bool out_streams) {
+                                                                        size_t inner, size_t rows_per_chunk, unsigned tx_count, int ddof) {
     const unsigned tx = threadIdx.x % tx_count, ty = threadIdx.x / tx_count, ty_count = kThreads / tx_count;
     const size_t col = (size_t(blockIdx.x) * tx_count + tx) * W;
     if (col >= inner) return;
@@ -427,7 +425,7 @@ __global__ __launch_bounds__(kThreads) void reduce_cols_backward_kernel(const fl
         float* dst = dx + slab_at + r * inner + col;
         if (W == 4) {
             v4f t = {o[0], o[1 % W], o[2 % W], o[3 % W]};
-            store_result(reinterpret_cast<v4f*>(dst), t, out_streams);
+            __builtin_nontemporal_store(t, reinterpret_cast<v4f*>(dst));
         } else {
             dst[0] = o[0];
         }
@@ -572,12 +570,11 @@ int run_forward(const char* name, const float* x, float* out, int32_t* index, fl
 template <int KIND>
 int run_backward(const char* name, const float* x, const float* y, const int32_t* index, const float* mean, const float* g, float* dx,
                  size_t outer, size_t len, size_t inner, int ddof, hipStream_t s) {
-    const bool out_streams = result_streams(outer * len * inner * sizeof(float));
     if (inner == 1) {
         RowPlan p;
         if (!plan_rows(reads_x<KIND>() ? x : dx, dx, outer, len, p)) return fail(CTAMD_ERANGE, "%s: too many runs", name);
 #define CTAMD_ROWS(V, G) hipLaunchKernelGGL((reduce_rows_backward_kernel<KIND, V, G>), dim3(p.grid), dim3(kThreads), 0, s, x, y, index, mean, \
-                                            g, dx, outer, len, p.chunk_len, p.chunks, ddof, out_streams)
+                                            g, dx, outer, len, p.chunk_len, p.chunks, ddof)
         if (p.vec && p.group == 64) CTAMD_ROWS(true, 64);
         else if (p.vec) CTAMD_ROWS(true, 256);
         else if (p.group == 64) CTAMD_ROWS(false, 64);
@@ -589,10 +586,10 @@ int run_backward(const char* name, const float* x, const float* y, const int32_t
     if (!plan_cols(reads_x<KIND>() ? x : dx, dx, outer, len, inner, p)) return fail(CTAMD_ERANGE, "%s: shape exceeds the launch grid", name);
     if (p.vec)
         hipLaunchKernelGGL((reduce_cols_backward_kernel<KIND, 4>), p.grid, dim3(kThreads), 0, s, x, y, index, mean, g, dx, len, inner,
-                           p.rows_per_chunk, p.tx_count, ddof, out_streams);
+                           p.rows_per_chunk, p.tx_count, ddof);
     else
         hipLaunchKernelGGL((reduce_cols_backward_kernel<KIND, 1>), p.grid, dim3(kThreads), 0, s, x, y, index, mean, g, dx, len, inner,
-                           p.rows_per_chunk, p.tx_count, ddof, out_streams);
+                           p.rows_per_chunk, p.tx_count, ddof);
     return launched(name);
 }
 

@@ -71,7 +71,6 @@ __device__ __forceinline__ void stream_out(T* __restrict__ out, size_t n, LoadF 
     constexpr int L = Vec<T>::kLanes;
     const size_t nv = n / L;
     const size_t per_block = size_t(kThreads) * kUnroll;
-    const bool streams = n * sizeof(T) > kResidentBytes;
     for (size_t base = size_t(blockIdx.x) * per_block; base < nv; base += size_t(gridDim.x) * per_block) {
         V r[kUnroll];
 #pragma unroll
@@ -82,7 +81,7 @@ __device__ __forceinline__ void stream_out(T* __restrict__ out, size_t n, LoadF 
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             const size_t i = base + size_t(u) * kThreads + threadIdx.x;
-            if (i < nv) store_result(reinterpret_cast<V*>(out) + i, r[u], streams);
+            if (i < nv) __builtin_nontemporal_store(r[u], reinterpret_cast<V*>(out) + i);
         }
     }
     const size_t t = size_t(blockIdx.x) * kThreads + threadIdx.x;
@@ -206,7 +205,6 @@ __global__ __launch_bounds__(256) void softmax_rows_f64_resident_kernel(const do
     __shared__ uint64_t s_tab[256];
     stage_exp64_table(s_tab);
     const size_t pairs = cols / 2;
-    const bool streams = rows * cols * sizeof(double) > kResidentBytes;
     for (size_t row = blockIdx.x; row < rows; row += gridDim.x) {
         const v2d* xr = reinterpret_cast<const v2d*>(x + row * cols);
         v2d* yr = reinterpret_cast<v2d*>(y + row * cols);
@@ -239,7 +237,7 @@ __global__ __launch_bounds__(256) void softmax_rows_f64_resident_kernel(const do
 #pragma unroll
         for (int k = 0; k < PAIRS; ++k) {
             const size_t j = size_t(k) * 256 + threadIdx.x;
-            if (j < pairs) store_result(yr + j, v2d{v[k][0] / sum, v[k][1] / sum}, streams);
+            if (j < pairs) __builtin_nontemporal_store(v2d{v[k][0] / sum, v[k][1] / sum}, yr + j);
         }
     }
 }
@@ -368,7 +366,6 @@ __global__ __launch_bounds__(256) void softmax_cols_f64_write_kernel(const doubl
     stage_exp64_table(s_tab);
     const size_t j = (size_t(blockIdx.x) * 256 + threadIdx.x) * W;
     if (j >= cols) return;
-    const bool streams = rows * cols * sizeof(double) > kResidentBytes;
     double m[W], sum[W], inv[W];
 #pragma unroll
     for (int w = 0; w < W; ++w) {
@@ -388,7 +385,7 @@ __global__ __launch_bounds__(256) void softmax_cols_f64_write_kernel(const doubl
             const double q0 = e * inv[w];
             o[w] = __builtin_fma(__builtin_fma(-q0, sum[w], e), inv[w], q0);
         }
-        if (W == 2) store_result(reinterpret_cast<v2d*>(dst), v2d{o[0], o[W - 1]}, streams);
+        if (W == 2) __builtin_nontemporal_store(v2d{o[0], o[W - 1]}, reinterpret_cast<v2d*>(dst));
         else dst[0] = o[0];
     };
     const double* __restrict__ p = x + first * cols + j;

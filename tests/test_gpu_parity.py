@@ -58,8 +58,8 @@ def test_binary_same_shape_bit_exact(oracle, n):
 @pytest.mark.parametrize("n", [(6 << 20) + 8, (1 << 24) - 4, (1 << 24) + 4])
 def test_large_streams_take_every_access_hint_variant_bit_exact(oracle, n):
     """Above 64 MiB of operands + result the loads carry the streaming hint, and above 64 MiB of
-    result the stores do too: one size per variant of the plain kernels, the row-broadcast kernel
-    and the fused-expression kernel (whose first result is the one that may go unhinted)."""
+    result the stores do too: one size per variant of the plain kernels and the row-broadcast
+    kernel, and the fused-expression kernel on the same sizes (two results)."""
     print("case access hints n", n, flush=True)
     a = oracle.normal((n,), 11, 0, 3)
     b = oracle.normal((n,), 12, 0, 3)
