@@ -39,7 +39,8 @@ constexpr int kMaxDevices = 64;
 // What the kernel runs: the caller's program after value numbering.  Every instruction's result
 // stays in registers (the "carry") until the next result replaces it.  An instruction works in
 // place on the carry: its operand a is the carry, fetched from LDS first where the carry holds
-// something else (kAFetch); operand b is fetched from LDS (kBFetch) or is the carry too; the result
+// something else (kAFetch); operand b is always fetched from LDS (kBFetch: for x * x the value is kept
+// and fetched back); the result
 // goes to LDS only if an instruction further on has to fetch it (kKeep).  Where only the second
 // operand of a - b, a / b or the ReLU gradient is in the carry, the operands change places and the
 // operator is one of the reversed ones below.  LDS places are handed out by liveness, so a program
@@ -136,15 +137,21 @@ __device__ __forceinline__ void sin_or_cos(float (&c)[N], const Tables& t) {
     }
 }
 
-template <bool FASTM, int N>
-__device__ __forceinline__ void apply(const Insn& q, float (&c)[N], const float (&b)[N], const Tables& t) {
+// The second operand of a two-operand operator always comes from LDS, fetched (through `second`)
+// inside the operator's own case: fetched ahead of the switch - or defaulted to the carry for
+// x * x - it is a second live copy of eight registers at every operator, also the one-operand
+// ones, and keeps the compiler from computing the result in the carry's own registers (a dozen
+// register moves per operator on the nine-operator program).
+template <bool FASTM, int N, class Second>
+__device__ __forceinline__ void apply(const Insn& q, float (&c)[N], Second second, const Tables& t) {
+    float b[N];
     switch (q.op) {
-        case CTAMD_EX_ADD: each(c, [&](int e) { return c[e] + b[e]; }); break;
-        case CTAMD_EX_SUB: each(c, [&](int e) { return c[e] - b[e]; }); break;
-        case kRevSub: each(c, [&](int e) { return b[e] - c[e]; }); break;
-        case CTAMD_EX_MUL: each(c, [&](int e) { return c[e] * b[e]; }); break;
-        case CTAMD_EX_DIV: each(c, [&](int e) { return c[e] / b[e]; }); break;
-        case kRevDiv: each(c, [&](int e) { return b[e] / c[e]; }); break;
+        case CTAMD_EX_ADD: second(b); each(c, [&](int e) { return c[e] + b[e]; }); break;
+        case CTAMD_EX_SUB: second(b); each(c, [&](int e) { return c[e] - b[e]; }); break;
+        case kRevSub: second(b); each(c, [&](int e) { return b[e] - c[e]; }); break;
+        case CTAMD_EX_MUL: second(b); each(c, [&](int e) { return c[e] * b[e]; }); break;
+        case CTAMD_EX_DIV: second(b); each(c, [&](int e) { return c[e] / b[e]; }); break;
+        case kRevDiv: second(b); each(c, [&](int e) { return b[e] / c[e]; }); break;
         case CTAMD_EX_NEG: each(c, [&](int e) { return -c[e]; }); break;
         case CTAMD_EX_RELU: each(c, [&](int e) { return (0.0f < c[e]) ? c[e] : 0.0f; }); break;
         case CTAMD_EX_SIGMOID:
@@ -161,8 +168,8 @@ __device__ __forceinline__ void apply(const Insn& q, float (&c)[N], const float 
         case CTAMD_EX_MULS: each(c, [&](int e) { return c[e] * q.imm; }); break;
         case CTAMD_EX_DIVS: each(c, [&](int e) { return cta_div_rcp(c[e], q.rcp); }); break;
         case CTAMD_EX_RSUBS: each(c, [&](int e) { return q.imm - c[e]; }); break;
-        case CTAMD_EX_RELUMUL: each(c, [&](int e) { return b[e] * ((c[e] > 0.0f) ? 1.0f : 0.0f); }); break;
-        case kRevReluMul: each(c, [&](int e) { return c[e] * ((b[e] > 0.0f) ? 1.0f : 0.0f); }); break;
+        case CTAMD_EX_RELUMUL: second(b); each(c, [&](int e) { return b[e] * ((c[e] > 0.0f) ? 1.0f : 0.0f); }); break;
+        case kRevReluMul: second(b); each(c, [&](int e) { return c[e] * ((b[e] > 0.0f) ? 1.0f : 0.0f); }); break;
         default: break;
     }
 }
@@ -354,15 +361,14 @@ __global__ __launch_bounds__(kExprThreads, FASTM ? 4 : 3) void expr_kernel(ExprA
             } else {
                 // lanes past the end compute on the zeros their loads gave them and store nothing
                 if (q.flags & kAFetch) carry = get(q.a);
-                float c[N], b[N];
+                float c[N];
 #pragma unroll
-                for (int e = 0; e < N; ++e) c[e] = b[e] = carry.h[e / 4][e % 4];   // b = the same value: x * x and the like
-                if (q.flags & kBFetch) {
+                for (int e = 0; e < N; ++e) c[e] = carry.h[e / 4][e % 4];
+                apply<FASTM, N>(q, c, [&](float (&b)[N]) {
                     const Vals<H> vb = get(q.b);
 #pragma unroll
                     for (int e = 0; e < N; ++e) b[e] = vb.h[e / 4][e % 4];
-                }
-                apply<FASTM, N>(q, c, b, tabs);
+                }, tabs);
 #pragma unroll
                 for (int e = 0; e < N; ++e) carry.h[e / 4][e % 4] = c[e];
             }
@@ -510,7 +516,7 @@ extern "C" int ctamd_expr_run_f32(const ctamd_expr_insn* prog, int n_insn, const
             }
         }
         auto fetch = [&](int from, uint8_t flag) {
-            if (from < 0 || from == in_carry) return;
+            if (from < 0 || (from == in_carry && flag == kAFetch)) return;   // a second operand never comes from the carry (x * x: kept and fetched)
             d.flags |= flag;
             kept[from] = true;
             last_fetch[from] = pc;
