@@ -1,6 +1,6 @@
 """Per-kernel timings of the launch layer through the C ABI on one MI355X.
 
-    python -m ctorch_amd.kernel_bench [--json] [--skip-matmul] [--only-expr] [--only-declared]
+    python -m ctorch_amd.kernel_bench [--json] [--skip-matmul] [--only-expr] [--only-declared] [--only-mlp]
 
 Every operator is launched on operands resident in HBM (torch only provides the memory and the
 stream), timed with events over back-to-back launches after a warm-up, and reported as time,
@@ -26,6 +26,8 @@ def main():
     ap.add_argument("--only-expr", action="store_true", help="only the fused-expression programs (for counter runs)")
     ap.add_argument("--only-declared", action="store_true",
                     help="only the operators the reference declares without defining: abs .. leaky_relu, reductions along an axis, log_softmax")
+    ap.add_argument("--only-mlp", action="store_true",
+                    help="only the launches of one 784-256-10 training step at batch 256 and 8192 (the small-product kernels)")
     args = ap.parse_args()
 
     import torch
@@ -63,6 +65,44 @@ def main():
             rate = ("%8.1f GB/s %5.1f%% of 8 TB/s" % (e["GB/s"], 100 * e["frac_of_hbm_peak"]) if nbytes is not None else
                     "%8.2f TFLOP/s %5.1f%% of 157.3" % (e["TFLOP/s"], 100 * e["frac_of_mfma_peak"]))
             print("%-44s %9.1f us  %s" % (name, e["us"], rate), flush=True)
+
+    # ---- the launches of one training step of the 784-256-10 perceptron, each on its own: the fused
+    # layers forward, the class-index cross entropy with its gradient, the product with the ReLU mask,
+    # the weight-gradient products and the bias-gradient column sums.  (Operands of a few MiB: they
+    # stay cached from launch to launch, as they do inside a step.)
+    def mlp_rows(batch):
+        I, H, Cn = 784, 256, 10
+        x = torch.rand(batch, I, device="cuda")
+        W1, b1 = torch.randn(I, H, device="cuda") * 0.03, torch.zeros(H, device="cuda")
+        W2, b2 = torch.randn(H, Cn, device="cuda") * 0.06, torch.zeros(Cn, device="cuda")
+        h, z = torch.empty(batch, H, device="cuda"), torch.empty(batch, Cn, device="cuda")
+        dz, dh = torch.randn(batch, Cn, device="cuda"), torch.empty(batch, H, device="cuda")
+        gW1, gW2 = torch.empty(I, H, device="cuda"), torch.empty(H, Cn, device="cuda")
+        gb1, gb2 = torch.empty(H, device="cuda"), torch.empty(Cn, device="cuda")
+        labels = torch.randint(0, Cn, (batch,), device="cuda").float()
+        loss, status = torch.empty(1, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda")
+        mm = lambda a, b, c, m, n, k: call("ctamd_matmul_f32", P(a), a.stride(0), a.stride(1), P(b), b.stride(0), b.stride(1), P(c), m, n, k, S)
+        tag = "MLP step, batch %d: " % batch
+        def row(name, fn, flops=None, nbytes=None):
+            report(tag + name, timeit(fn, 50, warm=10), nbytes=nbytes, flops=flops)
+        row("h = relu(x.W1 + b1) [%d x 784].[784 x 256]" % batch,
+            lambda: call("ctamd_matmul_bias_f32", P(x), I, 1, P(W1), H, 1, P(b1), 1, P(h), batch, H, I, S), flops=2.0 * batch * H * I)
+        row("z = h.W2 + b2 [%d x 256].[256 x 10]" % batch,
+            lambda: call("ctamd_matmul_bias_f32", P(h), H, 1, P(W2), Cn, 1, P(b2), 0, P(z), batch, Cn, H, S), flops=2.0 * batch * Cn * H)
+        row("cross entropy (class index), loss + gradient [%d x 10]" % batch,
+            lambda: call("ctamd_cross_entropy_index_fused_f32", P(z), P(labels), P(loss), P(status), P(dz), batch, Cn, S), nbytes=8.0 * batch * Cn)
+        row("dh = (dz.W2^T) * [h > 0] [%d x 10].[10 x 256]" % batch,
+            lambda: call("ctamd_matmul_relu_mask_f32", P(dz), Cn, 1, P(W2), 1, Cn, P(h), P(dh), batch, H, Cn, S), flops=2.0 * batch * H * Cn)
+        row("gW2 = h^T.dz [256 x %d].[%d x 10]" % (batch, batch), lambda: mm(h.t(), dz, gW2, H, Cn, batch), flops=2.0 * batch * H * Cn)
+        row("gb2 = column sums of dz [%d x 10]" % batch, lambda: call("ctamd_colsum_f32", P(dz), P(gb2), batch, Cn, S), nbytes=4.0 * batch * Cn)
+        row("gW1 = x^T.dh [784 x %d].[%d x 256]" % (batch, batch), lambda: mm(x.t(), dh, gW1, I, H, batch), flops=2.0 * batch * H * I)
+        row("gb1 = column sums of dh [%d x 256]" % batch, lambda: call("ctamd_colsum_f32", P(dh), P(gb1), batch, H, S), nbytes=4.0 * batch * H)
+    if args.only_mlp:
+        for batch in (256, 8192):
+            mlp_rows(batch)
+        if args.json:
+            print(json.dumps({"device": torch.cuda.get_device_name(0), "results": results}))
+        return 0
 
     # ---- elementwise, scalar, fill, reductions: 2^26 elements (256 MiB per tensor), four buffer sets
     n, sets = 1 << 26, 4
