@@ -74,6 +74,7 @@ PROTOTYPES.update({
     "ctamd_expr_run_f32": [_P, C.c_int, _P, C.c_int, _P, C.c_int, _P, _Z, _Z, _P],
     "ctamd_matmul_bias_f32": [_P, _I64, _I64, _P, _I64, _I64, _P, C.c_int, _P, _I64, _I64, _I64, _P],
     "ctamd_matmul_relu_mask_f32": [_P, _I64, _I64, _P, _I64, _I64, _P, _P, _I64, _I64, _I64, _P],
+    "ctamd_matmul_colsum_f32": [_P, _I64, _I64, _P, _I64, _I64, _P, _P, _I64, _I64, _I64, _P],
     "ctamd_fill_f32": [_P, C.c_float, _Z, _P],
     "ctamd_fill_from_f32": [_P, _P, _Z, _P],
     "ctamd_accumulate_f32": [_P, _P, _Z, _P],

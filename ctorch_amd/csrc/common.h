@@ -45,7 +45,8 @@ int compute_units();
 // Adds one operator launch to the per-process work counters read by ctamd_counters_read():
 // `bytes` and `flops` are the operator's algorithmic traffic and arithmetic (what it must move and
 // compute, not what the kernels happen to do).
-void account(double bytes, double flops);
+// same_launch: work that rides in a launch already counted (the count of launches stays).
+void account(double bytes, double flops, bool same_launch = false);
 
 inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 

@@ -22,6 +22,7 @@
 // one 32 x 32 tile per CU with a short K (gemm_micro: the waves of a block share out K and feed the
 // MFMAs from global memory directly), and a product with at most 16 output columns
 // (gemm_narrow_rows / gemm_narrow_cols: fp32 FMAs on the vector units, A streamed once).
+#include "colsum_small.h"
 #include "common.h"
 
 
@@ -492,6 +493,11 @@ struct MicroArgs {
     int spans_per_wave;
     const float* bias; int relu;
     const float* mask;                 // as in GemmArgs
+    // the column sums of a small contiguous matrix, carried along as the blocks after the `tiles` of
+    // the product (sum_out null: none): the bias gradient of a layer beside its weight gradient
+    int tiles;
+    const float* sum_src; float* sum_out;
+    size_t sum_cols; unsigned sum_rows;
 };
 // f[i] = operand element (x, k0 + i), i < 16; zeros past k or when x is outside the matrix
 template <bool KC, bool VEC>
@@ -522,6 +528,12 @@ __device__ __forceinline__ void micro_fetch(const float* __restrict__ p, int64_t
 template <bool A_KC, bool B_KC, bool VEC>
 __global__ __launch_bounds__(kMicroWaves * 64) void gemm_micro(MicroArgs g) {
     __shared__ float s_red[kMicroWaves * 16 * 64];
+    if (blockIdx.x >= unsigned(g.tiles)) {         // block-uniform: one of the column-sum blocks
+        static_assert(sizeof(s_red) >= kColsumThreads * sizeof(double), "the column sums borrow the product's LDS");
+        colsum_fold_body<kSmallLanes>(g.sum_src, g.sum_out, g.sum_cols, g.sum_rows, blockIdx.x - unsigned(g.tiles), threadIdx.x,
+                                      reinterpret_cast<double*>(s_red));
+        return;
+    }
     const int lane = threadIdx.x & 63, l32 = lane & 31, half = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(int(threadIdx.x) >> 6);
     const int m0 = (blockIdx.x % g.tiles_m) * 32, n0 = (blockIdx.x / g.tiles_m) * 32;
@@ -888,8 +900,11 @@ namespace {
 
 // C = A.B, optionally followed by "+ bias row" and ReLU in the same launch (in the fold launch when
 // the product is split along K).
+// sums / sums_done (or null): the column sums of a contiguous b are wanted as well; *sums_done says
+// whether the product's launch carried them (only the small-product kernel can).
 int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,
-                const float* bias, int relu, const float* mask, float* c, int64_t m, int64_t n, int64_t k, void* stream) {
+                const float* bias, int relu, const float* mask, float* c, int64_t m, int64_t n, int64_t k, void* stream,
+                float* sums = nullptr, bool* sums_done = nullptr) {
     if (m < 0 || n < 0 || k < 0) return fail(CTAMD_EINVAL, "%s: negative extent", name);
     if (m == 0 || n == 0) return CTAMD_OK;
     if (!c) return fail(CTAMD_EINVAL, "%s: null output", name);
@@ -935,8 +950,17 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
             const int spans = int((k + kMicroSpan - 1) / kMicroSpan);
             g.spans_per_wave = (spans + kMicroWaves - 1) / kMicroWaves;
             g.bias = bias; g.relu = relu; g.mask = mask;
+            g.tiles = int(tiles32);
+            g.sum_src = nullptr; g.sum_out = nullptr; g.sum_cols = 0; g.sum_rows = 0;
+            unsigned sum_blocks = 0;
+            if (sums && sums_done && colsum_is_small(size_t(k), size_t(n))) {
+                g.sum_src = b; g.sum_out = sums; g.sum_cols = size_t(n); g.sum_rows = unsigned(k);
+                sum_blocks = colsum_small_blocks(size_t(n));
+                *sums_done = true;
+                account(4.0 * double(k) * double(n), double(k) * double(n), true);
+            }
             const bool vec = (!A_KC || (aligned16(a) && g.lda % 4 == 0)) && (!B_KC || (aligned16(b) && g.ldb % 4 == 0));
-            const dim3 grid{unsigned(tiles32)}, block{unsigned(kMicroWaves * 64)};
+            const dim3 grid{unsigned(tiles32) + sum_blocks}, block{unsigned(kMicroWaves * 64)};
             if (A_KC && B_KC) launch_micro<true, true>(g, vec, grid, block, s);
             else if (A_KC) launch_micro<true, false>(g, vec, grid, block, s);
             else if (B_KC) launch_micro<false, true>(g, vec, grid, block, s);
@@ -1067,6 +1091,19 @@ extern "C" int ctamd_matmul_bias_f32(const float* a, int64_t as0, int64_t as1, c
                                      const float* bias, int relu, float* c, int64_t m, int64_t n, int64_t k,
                                      void* stream) {
     return matmul_impl(__func__, a, as0, as1, b, bs0, bs1, bias, relu ? 1 : 0, nullptr, c, m, n, k, stream);
+}
+
+extern "C" int ctamd_matmul_colsum_f32(const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,
+                                       float* c, float* sums, int64_t m, int64_t n, int64_t k, void* stream) {
+    if (m < 0 || n < 0 || k < 0) return fail(CTAMD_EINVAL, "%s: negative extent", __func__);
+    if (n > 0 && !sums) return fail(CTAMD_EINVAL, "%s: null sums", __func__);
+    if ((n > 1 && bs1 != 1) || (k > 1 && bs0 != n))
+        return fail(CTAMD_EINVAL, "%s: the column sums need b in contiguous rows (strides %lld, %lld)", __func__, (long long)bs0,
+                    (long long)bs1);
+    bool done = false;
+    int rc = matmul_impl(__func__, a, as0, as1, b, bs0, bs1, nullptr, 0, nullptr, c, m, n, k, stream, sums, &done);
+    if (rc || done || n == 0) return rc;
+    return ctamd_colsum_f32(b, sums, size_t(k), size_t(n), stream);
 }
 
 extern "C" int ctamd_matmul_relu_mask_f32(const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,

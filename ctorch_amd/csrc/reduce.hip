@@ -5,6 +5,7 @@
 // in a fixed order, so results are deterministic for a given size.
 #include <mutex>
 
+#include "colsum_small.h"
 #include "common.h"
 
 // Per-block partials of ctamd_dot_static_f32, the entry point for callers that cannot allocate:
@@ -292,38 +293,15 @@ __global__ __launch_bounds__(kThreads) void colsum_narrow_stage1(const float* __
 }
 
 constexpr int kFoldLanes = 4;    // lanes per column in stage 2
-constexpr int kSmallLanes = 16;  // lanes per column when a small matrix is summed in one launch
+static_assert(kColsumThreads == kThreads, "the shared body assumes this file's block size");
 // out[c] = sum over the `chunks` rows of partials[., c], in double, LANES lanes per column.  Stage 2
-// of the two-stage sum (LANES = 4), and the whole column sum of a small matrix (LANES = 16, a
-// bias gradient of a few hundred rows: one launch instead of two).
+// of the two-stage sum (LANES = 4), and the whole column sum of a small matrix (LANES = kSmallLanes,
+// a bias gradient of a few hundred rows: one launch instead of two).
 template <int LANES>
 __global__ __launch_bounds__(kThreads) void colsum_stage2(const float* __restrict__ partials, float* __restrict__ out,
                                                           size_t cols, unsigned chunks) {
-    constexpr int kFoldLanes = LANES;
-    constexpr int TX = kThreads / kFoldLanes;
-    const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
-    const size_t c = size_t(blockIdx.x) * TX + tx;
-    double acc = 0.0;
-    if (c < cols) {
-        unsigned k = ty;
-        for (; k + 7 * kFoldLanes < chunks; k += 8 * kFoldLanes) {
-            float v[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = partials[size_t(k + u * kFoldLanes) * cols + c];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) acc += double(v[u]);
-        }
-        for (; k < chunks; k += kFoldLanes) acc += double(partials[size_t(k) * cols + c]);
-    }
-    __shared__ double s_acc[kFoldLanes][TX];
-    s_acc[ty][tx] = acc;
-    __syncthreads();
-    if (ty == 0 && c < cols) {
-        double t = 0.0;
-#pragma unroll
-        for (int y = 0; y < kFoldLanes; ++y) t += s_acc[y][tx];
-        out[c] = float(t);
-    }
+    __shared__ double s_acc[kThreads];
+    colsum_fold_body<LANES>(partials, out, cols, chunks, blockIdx.x, threadIdx.x, s_acc);
 }
 
 }  // namespace
@@ -381,9 +359,8 @@ int ctamd_colsum_f32(const float* g, float* out, size_t rows, size_t cols, void*
     if (!g) return fail(CTAMD_EINVAL, "%s: null input", __func__);
     if (rows > (size_t(1) << 62) / cols) return fail(CTAMD_ERANGE, "%s: rows*cols overflows", __func__);
     hipStream_t s = as_stream(stream);
-    if (rows <= 1024 && rows * cols <= (size_t(1) << 19)) {       // small: one launch, rows added in order
-        constexpr size_t kCols = kThreads / kSmallLanes;
-        hipLaunchKernelGGL(colsum_stage2<kSmallLanes>, dim3((unsigned)((cols + kCols - 1) / kCols)), dim3(kThreads), 0, s, g, out,
+    if (colsum_is_small(rows, cols)) {                            // one launch, rows added in order
+        hipLaunchKernelGGL(colsum_stage2<kSmallLanes>, dim3(colsum_small_blocks(cols)), dim3(kThreads), 0, s, g, out,
                            cols, (unsigned)rows);
         account(4.0 * double(rows) * double(cols), double(rows) * double(cols));
         return launched(__func__);

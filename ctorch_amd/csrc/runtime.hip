@@ -31,12 +31,12 @@ constexpr double kHbmBytesPerS = 8.0e12;        // MI355X HBM3E
 constexpr double kMfmaF32FlopPerS = 157.3e12;   // MI355X dense fp32 matrix
 }  // namespace
 
-void account(double bytes, double flops) {
+void account(double bytes, double flops, bool same_launch) {
     add_to(g_bytes, bytes);
     add_to(g_flops, flops);
     const double tb = bytes / kHbmBytesPerS, tf = flops / kMfmaF32FlopPerS;
     add_to(g_ideal_s, tb > tf ? tb : tf);
-    g_launches.fetch_add(1, std::memory_order_relaxed);
+    if (!same_launch) g_launches.fetch_add(1, std::memory_order_relaxed);
 }
 
 int fail(int code, const char* fmt, ...) {

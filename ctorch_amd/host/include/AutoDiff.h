@@ -115,6 +115,11 @@ class AutoDiff {
     // (on by default; the gradients are the same bits either way).
     void set_fuse_relu_mask(bool on) { fuse_relu_mask_ = on; }
     bool fuse_relu_mask() const { return fuse_relu_mask_; }
+    // The bias gradient of a fused layer (the column sums of the layer's output gradient) computed
+    // with the weight gradient, for a small layer in the same launch (on by default; the gradients
+    // are the same bits either way).
+    void set_bias_grad_with_weight_grad(bool on) { bias_grad_with_weight_grad_ = on; }
+    bool bias_grad_with_weight_grad() const { return bias_grad_with_weight_grad_; }
 
    private:
     struct Pending {
@@ -131,6 +136,7 @@ class AutoDiff {
     LeafValues leaf_values_ = LeafValues::kLive;
     bool check_div_zero_ = true;
     bool fuse_relu_mask_ = true;
+    bool bias_grad_with_weight_grad_ = true;
     bool term_plus_zero_ = false;   // backward: the term just computed holds no -0
     bool seed_plus_zero_ = false;   // backward: the seed gradient holds no -0
     bool adjust_adds_to_zero_ = false;   // the last adjust_grad_shape took a branch in which the reference adds the gradient to zeros

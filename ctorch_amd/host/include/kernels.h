@@ -21,6 +21,10 @@ Tensor Linear_AMD_kernel(const Tensor& x, const Tensor& w, const Tensor& bias, b
 // (a . b) * [y > 0] in the product's launch: what MatMul's backward branch followed by the ReLU branch
 // of the layer that produced y compute (src/AutoDiff.cpp:1692-1704, :1320-1371)
 Tensor MatMulReluMask_AMD_kernel(const Tensor& a, const Tensor& b, const Tensor& y);
+// a . b, and into `sums` (a new 1-D tensor) the column sums of the contiguous b, with the bits of
+// MatMul_AMD_kernel and of the column sum: a layer's weight gradient x^T . dz and its bias gradient
+// from one call, in one launch when the layer is small (src/AutoDiff.cpp:1692-1704, :690-757)
+Tensor MatMulColSum_AMD_kernel(const Tensor& a, const Tensor& b, Tensor& sums);
 Tensor Dot_AMD_kernel(const Tensor& a, const Tensor& b);
 Tensor MSE_AMD_kernel(const Tensor& a, const Tensor& b);
 Tensor MAE_AMD_kernel(const Tensor& a, const Tensor& b);

@@ -332,12 +332,33 @@ Tensor AutoDiff::input_gradient(Node* node, size_t input_id, size_t input_pos, c
         case op::Linear: {                                              // the three branches above in one
             const Tensor& gz = linear_pre_activation_grad(node, g);
             if (input_pos == 2) {                                       // bias: Add's branch, shaped by the caller
+                if (node->input_grads.size() == 3 && !node->input_grads[2].is_cleared()) {
+                    term_plus_zero_ = true;                             // the column sums that came with the weight gradient
+                    return Tensor::alias(node->input_grads[2]);
+                }
                 term_plus_zero_ = node->op_param_i ? false : upstream_plus_zero;   // g * 0 may be -0
                 return Tensor::alias(gz);
             }
             term_plus_zero_ = true;
             const Tensor& other = *find(node->input_ids[input_pos == 0 ? 1 : 0])->tensor;
             if (input_pos == 0) return MatMul_AMD_kernel(gz, Tensor::view_t(other));   // gz . W^T
+            // When the bias wants its gradient too - the column sums of gz, which the caller would ask
+            // for when the bias's turn comes - they are computed with the weight gradient: the same
+            // two results bit for bit, and for a small layer one launch instead of two.
+            if (bias_grad_with_weight_grad_ && broadcast_grad_ == BroadcastGrad::kColumnSum && node->input_ids.size() == 3 && gz.dim() == 2 &&
+                gz.is_contiguous() &&
+                gz.device() == DeviceType::kAMD && gz.dtype() == DType::kFloat && node->input_ids[2] != node->input_ids[1] &&
+                node->input_ids[2] != node->input_ids[0]) {
+                Node* bias = find(node->input_ids[2]);
+                if (bias && bias->requires_grad && bias->tensor->dim() == 1 && bias->tensor->sizes()[0] == gz.sizes()[1]) {
+                    Tensor sums;
+                    Tensor gw = MatMulColSum_AMD_kernel(Tensor::view_t(other), gz, sums);
+                    node->input_grads.clear();
+                    node->input_grads.resize(3);
+                    node->input_grads[2] = std::move(sums);
+                    return gw;
+                }
+            }
             return MatMul_AMD_kernel(Tensor::view_t(other), gz);                        // x^T . gz
         }
         case op::Fused: {                                               // every operator branch above, in one launch

@@ -674,6 +674,21 @@ Tensor MatMulReluMask_AMD_kernel(const Tensor& a, const Tensor& b, const Tensor&
         "MatMulReluMask_AMD_kernel");
     return r;
 }
+Tensor MatMulColSum_AMD_kernel(const Tensor& a, const Tensor& b, Tensor& sums) {
+    check_device(a, "MatMulColSum_AMD_kernel");
+    check_device(b, "MatMulColSum_AMD_kernel");
+    if (a.shape().size() != 2 || b.shape().size() != 2 || a.shape()[1] != b.shape()[0])
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "MatMulColSum_AMD_kernel: not a product of two matrices");
+    if (!b.is_contiguous())
+        Ctorch_Error::throwException(kP, ErrorType::DIMENSION, "MatMulColSum_AMD_kernel: the second operand is not contiguous");
+    size_t m = a.shape()[0], k = a.shape()[1], n = b.shape()[1];
+    Tensor r(ShapeTag{}, {m, n}, DType::kFloat, DeviceType::kAMD, false);
+    sums = Tensor(ShapeTag{}, {n}, DType::kFloat, DeviceType::kAMD, false);
+    run(ctamd_matmul_colsum_f32(a.fptr(), int64_t(a.strides()[0]), int64_t(a.strides()[1]), b.fptr(), int64_t(b.strides()[0]),
+                                int64_t(b.strides()[1]), r.fptr(), sums.fptr(), int64_t(m), int64_t(n), int64_t(k), current_stream()),
+        "MatMulColSum_AMD_kernel");
+    return r;
+}
 Tensor Linear_AMD_kernel(const Tensor& x, const Tensor& w, const Tensor& bias, bool relu) {
     check_device(x, "Linear_AMD_kernel");
     check_device(w, "Linear_AMD_kernel");

@@ -129,9 +129,13 @@ void cth_set_fused_layers(int on) { g_fused_layers = on; }
 // as a launch of its own
 static int g_fuse_relu_mask = 1;
 void cth_set_fuse_relu_mask(int on) { g_fuse_relu_mask = on; }
+// the bias gradient of a fused layer with its weight gradient (default) or as launches of its own
+static int g_bias_with_weight = 1;
+void cth_set_bias_grad_with_weight_grad(int on) { g_bias_with_weight = on; }
 static void configure(AutoDiff& ctx) {
     ctx.set_broadcast_grad(g_row0 ? BroadcastGrad::kReferenceRow0 : BroadcastGrad::kColumnSum);
     ctx.set_fuse_relu_mask(g_fuse_relu_mask != 0);
+    ctx.set_bias_grad_with_weight_grad(g_bias_with_weight != 0);
 }
 
 long cth_binary(int code, const float* a, const long* ad, int an, const float* b, const long* bd,

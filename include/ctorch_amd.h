@@ -287,6 +287,17 @@ int ctamd_matmul_f32(const float* a, int64_t as0, int64_t as1, const float* b, i
 int ctamd_matmul_bias_f32(const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,
                           const float* bias, int relu, float* c, int64_t m, int64_t n, int64_t k, void* stream);
 
+/* c = a . b as ctamd_matmul_f32 computes it, and sums[j] = sum over k of b[k, j] as
+ * ctamd_colsum_f32(b, sums, k, n) computes it - the same bits as the two calls: the weight gradient
+ * x^T . dz of a layer and its bias gradient, the column sums of dz (the tape's MatMul branch,
+ * src/AutoDiff.cpp:1692-1704, and the reduction of a broadcast operand's gradient, :690-757).  b must
+ * lie in contiguous rows (CTAMD_EINVAL otherwise, nothing launched).  When the product is small enough
+ * for the one-launch small-product kernel (at most 256 tiles of 32 x 32, k <= 512), the sums are
+ * computed by extra blocks of that launch: one kernel on the chain of dependent launches instead of
+ * two.  Every other shape runs the two operators one after the other. */
+int ctamd_matmul_colsum_f32(const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,
+                            float* c, float* sums, int64_t m, int64_t n, int64_t k, void* stream);
+
 /* The gradient that reaches a ReLU layer's pre-activation, formed by the product that computes it:
  * C = (A.B) * [y > 0], y the [m, n] row-major output of that ReLU.  The reference computes the
  * product in the MatMul branch of backward (g.matmul(B.t()), src/AutoDiff.cpp:1692-1704) and the

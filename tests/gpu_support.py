@@ -229,6 +229,18 @@ def matmul_relu_mask(a, b, y):
     return c
 
 
+def matmul_colsum(a, b):
+    """a.b and the column sums of b (the weight and bias gradients of a layer) from one call."""
+    m, k = a.shape
+    k2, n = b.shape
+    assert k == k2
+    c = torch.full((m, n), float("nan"), device=DEV)
+    sums = torch.full((n,), float("nan"), device=DEV)
+    call("ctamd_matmul_colsum_f32", ptr(a), a.stride(0), a.stride(1), ptr(b), b.stride(0), b.stride(1), ptr(c), ptr(sums), m, n, k,
+         stream())
+    return c, sums
+
+
 def matmul(a, b):
     """a, b: 2-D device tensors, possibly transposed views (strides are passed through)."""
     m, k = a.shape

@@ -1102,6 +1102,20 @@ class HostLayer(Reference):
         """mlp_step builds each layer with Tensor::linear (matmul + bias + ReLU as one operator)."""
         self.cdll.cth_set_fused_layers(int(on))
 
+    def set_bias_grad_with_weight_grad(self, on):
+        """The bias gradient of a fused layer with its weight gradient (the default) or on its own."""
+        self.cdll.cth_set_bias_grad_with_weight_grad(int(on))
+
+    def time_mlp(self, x, W1, b1, W2, b2, labels, warm=2, steps=3):
+        """One class-index training step timed by the harness: (ms per step, operator launches per step)."""
+        x, W1, b1, W2, b2, labels = map(f32, (x, W1, b1, W2, b2, labels))
+        out = (C.c_double * 6)()
+        L = C.c_long
+        rc = self.cdll.cth_time_mlp(fp(x), L(x.shape[0]), L(x.shape[1]), fp(W1), fp(b1), L(W1.shape[1]), fp(W2), fp(b2),
+                                    L(W2.shape[1]), fp(labels), C.c_int(warm), C.c_int(steps), out)
+        assert rc == steps, rc
+        return out[0], int(out[4])
+
     def mlp_step(self, x, W1, b1, W2, b2, target, target_is_index=False):
         return Reference.mlp_step(self, x, W1, b1, W2, b2, target, C.c_int(int(target_is_index)))
 

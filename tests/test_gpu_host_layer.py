@@ -480,6 +480,36 @@ def test_a_gradient_read_from_the_tape_is_read_only_while_shared(oracle, host):
     assert host.cdll.cth_shared_grad_is_readonly(x.ctypes.data_as(C.POINTER(C.c_float)), C.c_long(x.size)) == 0
 
 
+@pytest.mark.parametrize("batch", [8, 256, 512, 513, 4096])
+def test_bias_gradient_comes_with_the_weight_gradient(oracle, host, batch):
+    """A fused layer whose bias wants its gradient gets it from the call that forms the weight
+    gradient (column sums of the layer's output gradient beside x^T . dz).  The gradients are the
+    bits of the separate launches at every batch size; up to 512 rows (the longest K the one-launch
+    small-product kernel takes) the column sums ride in the product's own launch, and a step then
+    counts two operator launches fewer."""
+    print("case bias gradient with the weight gradient", batch, flush=True)
+    I, H, Cn = 784, 256, 10
+    x = oracle.uniform((batch, I), 651, 0, 1)
+    W1, b1 = oracle.uniform((I, H), 652, -0.05, 0.05), oracle.uniform((H,), 653, -0.05, 0.05)
+    W2, b2 = oracle.uniform((H, Cn), 654, -0.1, 0.1), oracle.uniform((Cn,), 655, -0.1, 0.1)
+    labels = oracle.ints((batch,), 656, Cn)
+    host.set_fused_layers(True)
+    try:
+        host.set_bias_grad_with_weight_grad(False)
+        apart = host.mlp_step(x, W1, b1, W2, b2, labels, True)
+        _, launches_apart = host.time_mlp(x, W1, b1, W2, b2, labels)
+        host.set_bias_grad_with_weight_grad(True)
+        together = host.mlp_step(x, W1, b1, W2, b2, labels, True)
+        _, launches_together = host.time_mlp(x, W1, b1, W2, b2, labels)
+    finally:
+        host.set_bias_grad_with_weight_grad(True)
+        host.set_fused_layers(False)
+    for name, a, b in zip(["loss", "logits", "gW1", "gb1", "gW2", "gb2"], together, apart):
+        assert same_bits(a, b), name
+    print(f"  operator launches per step: {launches_together} together, {launches_apart} apart")
+    assert launches_together == launches_apart - (2 if batch <= 512 else 0)
+
+
 @pytest.mark.parametrize("batch", [8, 300, 4096])
 def test_relu_mask_rides_in_the_products_of_backward(oracle, host, batch):
     """The gradient of a ReLU layer's output, when one product alone reads that output, is formed

@@ -632,6 +632,31 @@ def test_comparisons_bit_exact(oracle, n):
     assert G.lib().ctamd_compare_f32(9, G.ptr(da), G.ptr(db), G.ptr(out), n, G.stream()) == -1
 
 
+@pytest.mark.parametrize("m,n,k", [(256, 10, 256), (784, 256, 256), (256, 10, 8192), (784, 16, 1024), (70, 1, 129), (33, 3, 1), (1, 1, 1),
+                                   (31, 33, 512), (100, 70, 513), (512, 512, 64), (300, 7, 3000), (784, 256, 8192)])
+def test_product_with_the_column_sums_of_its_second_operand(oracle, m, n, k):
+    """The weight gradient x^T . dz and the bias gradient (column sums of dz) from one call: the
+    bits of ctamd_matmul_f32 and of ctamd_colsum_f32, whether the sums ride in the product's launch
+    (a product of at most 256 tiles of 32 x 32 with K <= 512) or follow it as launches of their own."""
+    print("case matmul + column sums", m, n, k, flush=True)
+    X = oracle.normal((k, m), 61)
+    dZ = oracle.normal((k, n), 62)
+    dX, dZd = G.dev(X), G.dev(dZ)
+    for name, a in (("x^T as a view", dX.t()), ("x^T materialised", G.dev(np.ascontiguousarray(X.T)))):
+        c, sums = G.matmul_colsum(a, dZd)
+        assert same_bits(G.host(c), G.host(G.matmul(a, dZd))), name
+        assert same_bits(G.host(sums), G.host(G.colsum(dZd))), name
+    l = G.lib()
+    # a second operand that is not in contiguous rows: refused before anything is launched
+    if n > 1 and k > 1:
+        wide = G.dev(oracle.normal((k, n + 3), 63))
+        c = torch.empty((m, n), device=G.DEV)
+        sums = torch.empty((n,), device=G.DEV)
+        a = G.dev(np.ascontiguousarray(X.T))
+        assert l.ctamd_matmul_colsum_f32(G.ptr(a), k, 1, G.ptr(wide), n + 3, 1, G.ptr(c), G.ptr(sums), m, n, k, G.stream()) == -1
+        assert l.ctamd_matmul_colsum_f32(G.ptr(a), k, 1, G.ptr(wide), 1, k, G.ptr(c), G.ptr(sums), m, n, k, G.stream()) == -1
+
+
 @pytest.mark.parametrize("m,n,k", [(256, 256, 10), (8192, 256, 10), (100, 70, 300), (300, 200, 1000), (2100, 2050, 40),
                                    (4090, 2047, 24), (96, 12, 4096), (64, 10, 256), (5, 7, 0)])
 def test_product_times_relu_mask_equals_the_two_launches(oracle, m, n, k):
