@@ -97,6 +97,11 @@ def main():
         row("gb2 = column sums of dz [%d x 10]" % batch, lambda: call("ctamd_colsum_f32", P(dz), P(gb2), batch, Cn, S), nbytes=4.0 * batch * Cn)
         row("gW1 = x^T.dh [784 x %d].[%d x 256]" % (batch, batch), lambda: mm(x.t(), dh, gW1, I, H, batch), flops=2.0 * batch * H * I)
         row("gb1 = column sums of dh [%d x 256]" % batch, lambda: call("ctamd_colsum_f32", P(dh), P(gb1), batch, H, S), nbytes=4.0 * batch * H)
+        # what the tape calls for a layer whose bias wants its gradient: both in one call (one launch while batch <= 512)
+        mmcs = lambda a, b, c, sums, m, n, k: call("ctamd_matmul_colsum_f32", P(a), a.stride(0), a.stride(1), P(b), b.stride(0), b.stride(1),
+                                                   P(c), P(sums), m, n, k, S)
+        row("gW2 and gb2 in one call", lambda: mmcs(h.t(), dz, gW2, gb2, H, Cn, batch), flops=2.0 * batch * H * Cn)
+        row("gW1 and gb1 in one call", lambda: mmcs(x.t(), dh, gW1, gb1, I, H, batch), flops=2.0 * batch * H * I)
     if args.only_mlp:
         for batch in (256, 8192):
             mlp_rows(batch)
