@@ -17,7 +17,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 RESOURCES = os.path.join(os.path.dirname(os.path.abspath(__file__)), "kernel_resources.json")
 LIB = os.path.join(HERE, "libctorch_amd.so")
-SOURCES = ["runtime.hip", "elementwise.hip", "reduce.hip", "softmax_ce.hip", "matmul.hip", "dataset.hip", "expr.hip", "typed.hip", "stats.hip"]
+SOURCES = ["runtime.hip", "elementwise.hip", "reduce.hip", "softmax_ce.hip", "matmul.hip", "dataset.hip", "expr.hip", "expr_jit.hip", "typed.hip", "stats.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function"]
 
@@ -44,10 +44,11 @@ def build(verbose=False, jobs=4):
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
     objs = [os.path.join(objdir, s.replace(".hip", ".o")) for s in SOURCES]
+    _write_jit_text(os.path.join(objdir, "jit_text.inc"))
 
     def one(pair):
         src, obj = pair
-        return _run([hipcc] + FLAGS + ["-Rpass-analysis=kernel-resource-usage", "-c", os.path.join(CSRC, src), "-o", obj])
+        return _run([hipcc] + FLAGS + ["-Rpass-analysis=kernel-resource-usage", "-I", objdir, "-c", os.path.join(CSRC, src), "-o", obj])
 
     resources = {}
     with ThreadPoolExecutor(max_workers=jobs) as ex:
@@ -55,12 +56,27 @@ def build(verbose=False, jobs=4):
             rest = _kernel_resources(src, out, resources)
             if verbose and rest.strip():
                 print(rest)
-    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs + ["-lhiprtc"])
     # what every kernel needs (registers, spills, LDS), next to the library: a spilled register costs a
     # kernel its overlap of loads and arithmetic, so tests/test_abi_and_devmath.py refuses a build that has one
     with open(RESOURCES, "w") as f:
         json.dump(resources, f, indent=0, sort_keys=True)
     return LIB
+
+
+def _write_jit_text(path):
+    """devmath.h and expr_ops.h as one C++ string literal (their #include lines removed): the text that
+    expr_jit.hip hands to the run-time compiler in front of every kernel it generates."""
+    text = ""
+    for name in ("devmath.h", "expr_ops.h"):
+        for line in open(os.path.join(CSRC, name)):
+            if not line.lstrip().startswith("#include"):
+                text += line
+    chunks = [text[i:i + 8000] for i in range(0, len(text), 8000)]      # below the compilers' limit on one literal
+    with open(path, "w") as f:
+        for c in chunks:
+            assert ')jit"' not in c
+            f.write('R"jit(' + c + ')jit"\n')
 
 
 def _kernel_resources(src, out, table):

@@ -72,6 +72,9 @@ PROTOTYPES.update({
     "ctamd_accumulate_typed": [_P, _P, C.c_int, _Z, _P],
     "ctamd_softmax_f64": [_P, _P, _Z, _Z, C.c_int, _P],
     "ctamd_expr_run_f32": [_P, C.c_int, _P, C.c_int, _P, C.c_int, _P, _Z, _Z, _P],
+    "ctamd_set_expr_jit": [C.c_int],
+    "ctamd_expr_jit": [],
+    "ctamd_expr_jit_compile": [_P, C.c_int, C.c_int, C.c_int, _P, _Z, _P],
     "ctamd_matmul_bias_f32": [_P, _I64, _I64, _P, _I64, _I64, _P, C.c_int, _P, _I64, _I64, _I64, _P],
     "ctamd_matmul_relu_mask_f32": [_P, _I64, _I64, _P, _I64, _I64, _P, _P, _I64, _I64, _I64, _P],
     "ctamd_matmul_colsum_f32": [_P, _I64, _I64, _P, _I64, _I64, _P, _P, _I64, _I64, _I64, _P],
@@ -139,6 +142,8 @@ def load():
     lib.ctamd_counters_reset.restype = None
     lib.ctamd_counters_read.argtypes = [C.POINTER(C.c_double)] * 3 + [C.POINTER(C.c_uint64)]
     lib.ctamd_counters_read.restype = None
+    lib.ctamd_expr_jit_stats.argtypes = [C.POINTER(C.c_uint64)] * 4
+    lib.ctamd_expr_jit_stats.restype = None
     lib.ctamd_last_error.restype = C.c_char_p
     lib.ctamd_version.restype = C.c_char_p
     _lib = lib

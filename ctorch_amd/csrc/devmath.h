@@ -507,43 +507,39 @@ __device__ __forceinline__ static float cta_exp_hw(float d) {
     const float r = __fmaf_rn(e, t, e);
     return (e == __builtin_huge_valf()) ? e : r;
 }
-// The same with the argument held to [-150, 88], so that the result is always finite (at most e^88 =
-// 1.65e38).  A NaN argument gives e^-150 = 0: callers that must return NaN for NaN select it themselves.
-__device__ __forceinline__ static float cta_exp_hw_bounded(float d) {
-    const float dc = __builtin_amdgcn_fmed3f(d, -150.0f, 88.0f);
-    const float z = dc * 0x1.715476p+0f;
-    const float e = __builtin_amdgcn_exp2f(z);
-    float t = __fmaf_rn(z, -0x1.62e4p-1f, dc);
-    t = __fmaf_rn(z, -0x1.7f7d1cp-20f, t);
-    return __fmaf_rn(e, t, e);
-}
-// 1 / s for finite s >= 1: the hardware reciprocal (1 ulp) and one Newton step, within 1 ulp of
-// the exactly rounded quotient.  Where 1 / s would be subnormal (s > 2^126) the result may be 0.
+// 1 / s for finite 1 <= s <= 2^126: the hardware reciprocal (1 ulp) and two Newton steps on the exact
+// residual.  Checked on the host over every significand and every starting value within 1 ulp
+// (tests/native/rcpcheck.c): the correctly rounded quotient, except for a significand of all ones,
+// where it is the float below (1 ulp off; 1 / s sits 2^-48 above a midpoint there).
 __device__ __forceinline__ static float cta_rcp_refined(float s) {
-    const float r = __builtin_amdgcn_rcpf(s);
-    const float err = __fmaf_rn(-s, r, 1.0f);
-    return __fmaf_rn(err, r, r);
+    float r = __builtin_amdgcn_rcpf(s);
+    r = __fmaf_rn(__fmaf_rn(-s, r, 1.0f), r, r);
+    return __fmaf_rn(__fmaf_rn(-s, r, 1.0f), r, r);
 }
-// Single-precision sigmoid by the reference's formula 1 / (1 + e^-x) on the exponential and the
-// reciprocal above.  Against the same formula on expf and an exact division (what the exact mode
-// returns): within 4 ulp - the sum 1 + e is rounded where its spacing is up to four times the
-// spacing of the quotient, so one ulp of the exponential is worth up to four of the result - and
-// below the smallest normal number (x < -87.3) possibly 0 where the exact mode has a subnormal.
+// Arguments for which cta_sigmoid_f32 below is not valid, or not within its bound: NaN, x > 128 (the
+// scaled argument overflows), and x < -16.625, where e^-x reaches 2^24: in [2^24, 2^25) the sum 1 + e is
+// a tie for every e, two exponentials one ulp apart can round to sums TWO ulps apart, and the
+// quotient moves by up to four of its ulps (seen on the device: x in [-16.93, -16.64]).  Beyond that
+// binade the bound would hold again, but such sigmoids are below 6e-8; they all take the
+// double-precision routine.
+__device__ __forceinline__ static int cta_sigmoid_is_rare(float x) { return !(x >= -16.625f && x <= 128.0f); }
+// Single-precision sigmoid by the reference's formula 1 / (1 + e^-x) for -16.625 <= x <= 128: the
+// exponential above (within 1 ulp of expf), the same rounded sum, and the reciprocal above.  Against the same
+// formula on expf and an exact division (what the exact mode returns): within 2 ulp.  Why: one ulp of
+// the exponential moves the rounded sum s = 1 + e by at most one of its own ulps (ulp(e) <= ulp(s),
+// rounding is monotonic, and for e < 2^24 at most one of two neighbouring sums is a tie).  With
+// s = m 2^k, 1 <= m < 2, neighbouring sums give quotients 2^-23 / m^2
+// (relative to 2^-k) apart while floats at 1 / s are 2^-24 apart: less than two ulps, so the two
+// correctly rounded quotients differ by at most 2.  Where the reciprocal above is the float below
+// the correct one (m all ones), the neighbours of s are 2^(k+1), whose quotient is that very float,
+// and s - ulp, whose quotient rounds to the float above it: 0 and 1 ulp.
 __device__ __forceinline__ static float cta_sigmoid_f32(float x) {
-    const float s = 1.0f + cta_exp_hw_bounded(-x);
-    const float r = cta_rcp_refined(s);
-    return (x != x) ? x : r;
-}
-// Single-precision tanh.  The reference computes (e^x - e^-x) / (e^x + e^-x); this computes the same
-// function as 1 - 2 / (e^2|x| + 1) with the sign of x (one exponential, one reciprocal): within 2 ulp
-// of tanh for |x| >= 1, within 1.2e-7 absolute below, where the reference's form loses its digits to
-// the same cancellation.  The reference's form is inf / inf = NaN once expf(|x|) overflows, that is
-// for |x| > 0x1.62e42ep+6: so is this, and NaN stays NaN.
-__device__ __forceinline__ static float cta_tanh_f32(float x) {
-    const float ax = __builtin_fabsf(x);
-    const float s = cta_exp_hw_bounded(ax + ax) + 1.0f;
-    const float v = __fmaf_rn(-2.0f, cta_rcp_refined(s), 1.0f);
-    return (ax <= 0x1.62e42ep+6f) ? __builtin_copysignf(v, x) : __builtin_nanf("");
+    const float z = x * -0x1.715476p+0f;
+    const float e = __builtin_amdgcn_exp2f(z);
+    float t = __fmaf_rn(z, -0x1.62e4p-1f, -x);
+    t = __fmaf_rn(z, -0x1.7f7d1cp-20f, t);
+    const float s = 1.0f + __fmaf_rn(e, t, e);
+    return cta_rcp_refined(s);
 }
 #endif
 

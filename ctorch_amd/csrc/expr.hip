@@ -19,6 +19,7 @@
 #include "common.h"
 #include "devmath.h"
 #include "functors.h"
+#include "expr_jit.h"
 
 #include <cfloat>
 #include <utility>
@@ -108,35 +109,6 @@ __device__ __forceinline__ Insn fetch_insn(const ExprArgs& g, int pc) {
     return q;
 }
 
-// One operator on the N elements of a lane, in place: c holds operand a on entry and the result on
-// return, b the second operand of the two-operand operators.  The operator is chosen once (a
-// scalar branch) and its N evaluations are independent instruction streams that the compiler
-// interleaves: the long dependent chains of the transcendental functors hide each other's latencies.
-template <int N, class F>
-__device__ __forceinline__ void each(float (&c)[N], F f) {
-#pragma unroll
-    for (int e = 0; e < N; ++e) c[e] = f(e);
-}
-// FASTM: the transcendental operators in single precision (sin / cos within 2 ulp of sinf / cosf for
-// |x| < 120, the double-precision routines beyond; sigmoid within 4 ulp of the reference's formula on
-// expf; tanh within 2 ulp of tanh for |x| >= 1 and 1.2e-7 absolute below); otherwise the routines
-// that return glibc's floats.
-template <bool FASTM, int WANT_COS, int N>
-__device__ __forceinline__ void sin_or_cos(float (&c)[N], const Tables& t) {
-    bool rare = false;
-    float x[N];
-#pragma unroll
-    for (int e = 0; e < N; ++e) {
-        x[e] = c[e];
-        c[e] = FASTM ? cta_sincosf_f32(x[e], WANT_COS) : cta_sincosf_fast(x[e], WANT_COS);
-        rare = rare || !(__builtin_fabsf(x[e]) < 120.0f);      // |x| >= 120, inf, NaN
-    }
-    if (__builtin_expect(rare, 0)) {
-        for (int e = 0; e < N; ++e)
-            if (cta_sincos_is_rare(x[e])) c[e] = cta_sincosf(x[e], WANT_COS, t.inv_pio4);
-    }
-}
-
 // The second operand of a two-operand operator always comes from LDS, fetched (through `second`)
 // inside the operator's own case: fetched ahead of the switch - or defaulted to the carry for
 // x * x - it is a second live copy of eight registers at every operator, also the one-operand
@@ -155,13 +127,13 @@ __device__ __forceinline__ void apply(const Insn& q, float (&c)[N], Second secon
         case CTAMD_EX_NEG: each(c, [&](int e) { return -c[e]; }); break;
         case CTAMD_EX_RELU: each(c, [&](int e) { return (0.0f < c[e]) ? c[e] : 0.0f; }); break;
         case CTAMD_EX_SIGMOID:
-            if (FASTM) each(c, [&](int e) { return cta_sigmoid_f32(c[e]); });
+            if (FASTM) sigmoid_fast(c, t);
             else each(c, [&](int e) { return sigmoid_ref(c[e], t); });
             break;
-        case CTAMD_EX_TANH:
-            if (FASTM) each(c, [&](int e) { return cta_tanh_f32(c[e]); });
-            else each(c, [&](int e) { return tanh_ref(c[e], t); });
-            break;
+        // tanh is the reference's (e^x - e^-x) / (e^x + e^-x) on glibc's own floats in both modes: near
+        // zero that quotient follows the rounding errors of the two exponentials, so nothing short
+        // of their exact bits stays within 2 ulp of it
+        case CTAMD_EX_TANH: each(c, [&](int e) { return tanh_ref(c[e], t); }); break;
         case CTAMD_EX_SIN: sin_or_cos<FASTM, 0>(c, t); break;       // two cases: the compiler then knows which of the two it builds
         case CTAMD_EX_COS: sin_or_cos<FASTM, 1>(c, t); break;
         case CTAMD_EX_ADDS: each(c, [&](int e) { return c[e] + q.imm; }); break;
@@ -473,6 +445,14 @@ extern "C" int ctamd_expr_run_f32(const ctamd_expr_insn* prog, int n_insn, const
         }
     }
     if (needs_status && !status) return fail(CTAMD_EINVAL, "%s: the program checks divisors but status is null", __func__);
+    // a program that has been launched often enough runs as a kernel compiled for it
+    {
+        const int rc = jit_try_launch(prog, n_insn, inputs, n_inputs, outputs, n_outputs, status, rows, cols, vec, fast_math(), stream);
+        if (rc != kJitDeclined) {
+            if (rc == CTAMD_OK) account(bytes, 0.0);
+            return rc;
+        }
+    }
     g.status = status;
     g.total = total;
     g.cols = unsigned(cols);

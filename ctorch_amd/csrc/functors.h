@@ -11,17 +11,10 @@
 namespace ctamd {
 namespace {
 
-typedef float v4f __attribute__((ext_vector_type(4)));
-
 constexpr int kThreads = 256;
 constexpr int kUnroll = 4;
 
-// Lookup tables of devmath.h staged in LDS once per block (random per-lane indices).
-struct Tables {
-    const uint64_t* exp2;
-    const uint32_t* inv_pio4;
-    const double* log;       // cta_log_tab, staged only for functors with kLogTable
-};
+#include "expr_ops.h"
 
 template <int N>
 struct Ptrs {
@@ -81,14 +74,6 @@ struct CosF { static constexpr int kIn = 1; static constexpr bool kTables = true
     __device__ bool rare(const float* x) const { return cta_sincos_is_rare(x[0]); }
     __device__ float slow(const float* x, const Tables& t) const { return cta_sincosf(x[0], 1, t.inv_pio4); } };
 
-__device__ __forceinline__ float tanh_ref(float x, const Tables& t) {
-    float ep, en;
-    cta_expf_pair(x, t.exp2, &ep, &en);
-    return (ep - en) / (ep + en);
-}
-__device__ __forceinline__ float sigmoid_ref(float x, const Tables& t) {
-    return 1.0f / (1.0f + cta_expf_tab(-x, t.exp2));
-}
 struct TanhF { static constexpr int kIn = 1; static constexpr bool kTables = true;
     __device__ float operator()(const float* x, const Tables& t) const { return tanh_ref(x[0], t); } };
 struct SigmoidF { static constexpr int kIn = 1; static constexpr bool kTables = true;
@@ -219,12 +204,6 @@ __device__ __forceinline__ void stage_log_table(double* tab) {
     if (threadIdx.x < 32) tab[threadIdx.x] = cta_log_tab[threadIdx.x];
     __syncthreads();
 }
-__device__ __forceinline__ void stage_tables(uint64_t* exp2, uint32_t* pio4) {
-    if (threadIdx.x < 32) exp2[threadIdx.x] = cta_exp2_tab[threadIdx.x];
-    if (threadIdx.x >= 32 && threadIdx.x < 56) pio4[threadIdx.x - 32] = cta_inv_pio4[threadIdx.x - 32];
-    __syncthreads();
-}
-
 }  // namespace
 }  // namespace ctamd
 

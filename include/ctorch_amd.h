@@ -16,9 +16,10 @@
  *    other stream is accepted only when the stream that used the scratch before has nothing
  *    pending, else the call returns CTAMD_EINVAL and launches nothing.
  *  - Math mode (ctamd_set_math_mode): CTAMD_MATH_FAST, the default, evaluates the exponentials of
- *    softmax / log-softmax / cross entropy and the sigmoid, tanh, sin, cos of fused expressions in
- *    single precision within 2 ulp (sigmoid 4); CTAMD_MATH_EXACT returns the bits of the reference's
- *    libm loops.  The one-operator kernels return glibc's floats in both modes.
+ *    softmax / log-softmax / cross entropy and the sigmoid, sin, cos of fused expressions in single
+ *    precision within 2 ulp of the reference's libm loops (a fused tanh keeps the reference's bits:
+ *    its quotient of exponentials amplifies any other rounding); CTAMD_MATH_EXACT returns the bits of
+ *    those loops everywhere.  The one-operator kernels return glibc's floats in both modes.
  *  - Return value: 0 on success, a negative CTAMD_E* code otherwise; ctamd_last_error() gives
  *    the text.  No C++ exception crosses this boundary.  The C++ shim above maps codes to the
  *    reference's two error conventions (Ctorch_Error::log / throwException,
@@ -388,6 +389,25 @@ typedef struct ctamd_expr_insn {
  * reads after the store. */
 int ctamd_expr_run_f32(const ctamd_expr_insn* prog, int n_insn, const float* const* inputs, int n_inputs,
                        float* const* outputs, int n_outputs, int32_t* status, size_t rows, size_t cols, void* stream);
+/* A program that ctamd_expr_run_f32 has been handed `threshold` times is written out as a
+ * straight-line HIP kernel, compiled for the device at run time (hiprtc; 20 - 200 ms, once per program
+ * and math mode) and launched from then on in place of the interpreter: the same per-element
+ * arithmetic from the same source text, so the same bits, without the interpreter's decoding and
+ * with divisions by row vectors turned into multiplications by reciprocals formed once per thread.
+ * threshold 0 switches compilation off, 1 compiles at first sight; default 2.  Operands that are not
+ * 16-byte aligned, rows that are not a multiple of four, programs with row vectors over rows of fewer
+ * than 512 elements, and launches that are being recorded into a graph before the program was
+ * compiled, stay with the interpreter; so does a program whose compilation fails.  No counterpart in
+ * the reference. */
+int ctamd_set_expr_jit(int threshold);
+int ctamd_expr_jit(void);
+/* Programs compiled / that failed to compile, launches of compiled kernels / of the interpreter. */
+void ctamd_expr_jit_stats(uint64_t* compiled, uint64_t* failed, uint64_t* compiled_launches, uint64_t* interpreted_launches);
+/* Generates and compiles the kernel for `prog` in the current math mode without launching anything
+ * (works without a GPU): columns = 1 for the access pattern of programs with row vectors, words = 128-bit
+ * words per lane (1, 2 or 4).  text (may be null) receives up to cap bytes of the generated source,
+ * code_bytes (may be null) the size of the code object. */
+int ctamd_expr_jit_compile(const ctamd_expr_insn* prog, int n_insn, int columns, int words, char* text, size_t cap, size_t* code_bytes);
 
 /* ----------------------------------------------------------------- backward arithmetic */
 /* r[i] = v.  A 0-D gradient expanded to a shape: src/AutoDiff.cpp:579-592; also Tensor::zero()

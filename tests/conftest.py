@@ -42,6 +42,7 @@ def exact_math():
     C++ front-end must not start torch's own HIP runtime after the library's.)"""
     from ctorch_amd import capi
     lib = capi.load()
-    prev = lib.ctamd_set_math_mode(1)
+    prev = lib.ctamd_math_mode()
+    assert lib.ctamd_set_math_mode(1) == 0
     yield
-    lib.ctamd_set_math_mode(prev)
+    assert lib.ctamd_set_math_mode(prev) == 0

@@ -304,6 +304,22 @@ def softmax_f64(x, dim):
     return r
 
 
+def set_expr_jit(threshold):
+    """After how many launches a fused-expression program is compiled at run time (0: never, 1: at
+    first sight); returns the previous setting."""
+    l = lib()
+    prev = l.ctamd_expr_jit()
+    capi.check(l.ctamd_set_expr_jit(threshold))
+    return prev
+
+
+def expr_jit_stats():
+    """(programs compiled, compilations failed, launches of compiled kernels, launches of the interpreter)."""
+    v = [C.c_uint64(0) for _ in range(4)]
+    lib().ctamd_expr_jit_stats(*[C.byref(x) for x in v])
+    return tuple(int(x.value) for x in v)
+
+
 MATH_FAST, MATH_EXACT = 0, 1
 
 

@@ -27,7 +27,7 @@ def test_library_exports_every_declared_entry_point():
     for n in names:
         assert hasattr(lib, n), n
     untyped = {"ctamd_device_count", "ctamd_last_error", "ctamd_version", "ctamd_counters_reset",
-               "ctamd_counters_read"}
+               "ctamd_counters_read", "ctamd_expr_jit_stats"}
     assert set(names) - untyped == set(capi.PROTOTYPES), set(names) ^ set(capi.PROTOTYPES)
     assert b"gfx950" in lib.ctamd_version()
 
@@ -102,6 +102,57 @@ def test_division_through_a_double_reciprocal_is_ieee_division(tmp_path):
     rand, ties = [l.split() for l in out.strip().splitlines()[-2:]]
     assert rand[0] == "tested" and int(rand[1]) == 64_000_000 and int(rand[3]) == 0
     assert ties[0] == "ties" and int(ties[1]) > 60_000_000 and int(ties[3]) == 0
+
+
+def test_refined_reciprocal_is_correctly_rounded(tmp_path):
+    """cta_rcp_refined (the quotient of the single-precision sigmoid): from any starting value within
+    1 ulp, two Newton steps give the correctly rounded 1 / s for every significand except all ones,
+    where the result is the float below - the case the sigmoid's 2-ulp argument treats separately."""
+    exe = str(tmp_path / "rcpcheck")
+    subprocess.check_call(["gcc", "-O2", "-ffp-contract=off", "-mfma", "-o", exe,
+                           os.path.join(ROOT, "tests", "native", "rcpcheck.c"), "-lm"])
+    f = subprocess.check_output([exe], text=True).split()
+    assert f[0] == "tested" and int(f[1]) == 3 << 23 and int(f[3]) == 0 and int(f[5]) <= 3, f
+
+
+def test_fused_expression_kernels_generate_and_compile_without_a_gpu():
+    """The run-time compiler path of fused expressions, up to the code object: the kernel text
+    generated for the config-5 expression (column-owning pattern, the row vector's reciprocals hoisted)
+    and for random programs (both patterns, both math modes) compiles for gfx950."""
+    import ctypes as C
+    from ctorch_amd import capi
+    from support import EX, random_slot_program
+    lib = capi.load()
+
+    class Insn(C.Structure):
+        _fields_ = [("op", C.c_uint8), ("dst", C.c_uint8), ("a", C.c_uint8), ("b", C.c_uint8), ("imm", C.c_float)]
+
+    def compile_(prog, columns, words):
+        arr = (Insn * len(prog))(*[Insn(*q) for q in prog])
+        text = C.create_string_buffer(1 << 20)
+        size = C.c_size_t(0)
+        rc = lib.ctamd_expr_jit_compile(arr, len(prog), columns, words, text, len(text), C.byref(size))
+        assert rc == 0, lib.ctamd_last_error().decode()[:4000]
+        assert size.value > 1000
+        return text.value.decode()
+
+    E = EX
+    c5 = [(E["LOAD_FULL"], 0, 0, 0, 0.0), (E["LOAD_ROW"], 1, 1, 0, 0.0), (E["DIV"], 2, 0, 1, 0.0), (E["SIGMOID"], 2, 2, 0, 0.0),
+          (E["TANH"], 3, 0, 0, 0.0), (E["SIN"], 4, 0, 0, 0.0), (E["MUL"], 3, 3, 4, 0.0), (E["SUB"], 2, 2, 3, 0.0),
+          (E["NEG"], 3, 0, 0, 0.0), (E["COS"], 3, 3, 0, 0.0), (E["ADD"], 2, 2, 3, 0.0), (E["STORE"], 0, 2, 0, 0.0)]
+    prev = lib.ctamd_math_mode()
+    try:
+        for mode in (0, 1):
+            assert lib.ctamd_set_math_mode(mode) == 0
+            text = compile_(c5, 1, 1)
+            assert "1.0 / (double)v1[e]" in text and "cta_div_rcp(v0[e], q1[e])" in text      # the divisor's reciprocal, once per thread
+            assert ("sigmoid_fast(v3, tabs)" in text) == (mode == 0)
+            compile_(random_slot_program(5, n_full=2, n_row=2, n_ops=24, n_out=3), 1, 2)
+            compile_(random_slot_program(6, n_full=3, n_row=0, n_ops=18, n_out=2), 0, 4)
+    finally:
+        lib.ctamd_set_math_mode(prev)
+    bad = (Insn * 1)(Insn(E["ADD"], 0, 1, 2, 0.0))
+    assert lib.ctamd_expr_jit_compile(bad, 1, 0, 2, None, 0, None) == -1
 
 
 def test_no_kernel_spills_registers():
