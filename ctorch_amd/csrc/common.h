@@ -22,12 +22,47 @@ int launched(const char* kernel);
 // ctamd_init() and never freed.  Returns nullptr (and records an error) before ctamd_init().
 constexpr size_t kScratchFloats = size_t(1) << 24;   // 64 MiB
 float* scratch();
-// The same for work about to be launched on `stream`, which becomes the scratch's user.  The null
-// stream and blocking streams order themselves with each other; any other change of user is
-// accepted only when the previous user has nothing pending (and is not recording a graph):
-// otherwise nullptr, with the error text set - two streams would write the one buffer at once.
-float* scratch(void* stream);
+// The scratch for work about to be launched on `stream`.  One buffer serves every stream of a device, so
+// its users are put in order: a stream other than the previous user first waits (on the device,
+// hipStreamWaitEvent) for the point the previous user had reached when it finished its own
+// scratch-using launches.  That point is an event owned by the library, recorded by release() on the
+// stream the caller has just passed in - a stream handle kept from an earlier call is never touched
+// again, it may have been destroyed by its owner since.  The null stream needs no event per use (one
+// is recorded on it when another stream takes over; blocking streams order themselves with it
+// anyway).  A stream that is recording a graph waits for nothing and records nothing: its launches
+// run at replay, and replays claim the scratch through ctamd_graph_launch.
+// Use: `ScratchUse use(stream); float* p = use.ptr(); if (!p) return CTAMD_EINVAL; ...launches...`;
+// the destructor releases after the last launch of the scope.
 int scratch_claim(void* stream);
+void scratch_release(void* stream);
+class ScratchUse {
+  public:
+    explicit ScratchUse(void* stream, bool wanted = true) : stream_(stream), held_(false), ptr_(nullptr) {
+        if (wanted) acquire();
+    }
+    ~ScratchUse() {
+        if (held_) scratch_release(stream_);
+    }
+    ScratchUse(const ScratchUse&) = delete;
+    ScratchUse& operator=(const ScratchUse&) = delete;
+    // claims now (for scopes that learn late whether they need the scratch); nullptr on failure
+    float* acquire() {
+        if (!held_) {
+            float* s = scratch();
+            if (s && scratch_claim(stream_) == CTAMD_OK) {
+                held_ = true;
+                ptr_ = s;
+            }
+        }
+        return ptr_;
+    }
+    float* ptr() const { return ptr_; }
+
+  private:
+    void* stream_;
+    bool held_;
+    float* ptr_;
+};
 // Four floats of -inf / of 0 in device memory (set up by ctamd_init): what row kernels read in
 // place of a vector that would lie beyond the end of a row.
 const float* pad_neg_inf();

@@ -828,11 +828,9 @@ int launch_narrow(const char* name, bool rows_form, const float* a, int64_t lda,
     }
     const int k_per_run = (k + runs - 1) / runs;
     runs = (k + k_per_run - 1) / k_per_run;
-    float* partial = nullptr;
-    if (runs > 1) {
-        partial = scratch(stream);
-        if (!partial) return CTAMD_EINVAL;
-    }
+    ScratchUse use(stream, runs > 1);
+    float* partial = use.ptr();
+    if (runs > 1 && !partial) return CTAMD_EINVAL;
     hipLaunchKernelGGL(gemm_narrow_cols<N>, dim3(unsigned(strips), unsigned(runs)), dim3(kNarrowWaves * 64), 0, s, a, lda, b, ldb,
                        runs > 1 ? partial : c, m, k, k_per_run, bias, relu);
     int rc = launched(name);
@@ -1053,12 +1051,13 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
     g.splits = splits;
     g.partial = nullptr;
     g.k_per_split = int(k);
+    ScratchUse use(stream, splits > 1);
     if (splits > 1) {
         int kps = int((k + splits - 1) / splits);
         kps = (kps + BK - 1) / BK * BK;
         g.splits = splits = int((k + kps - 1) / kps);
         g.k_per_split = kps;
-        g.partial = scratch(stream);
+        g.partial = use.ptr();
         if (!g.partial) return CTAMD_EINVAL;
         if (size_t(tiles - whole_tiles) * size_t(splits) * size_t(BM) * size_t(BN) > kScratchFloats)
             return fail(CTAMD_ERANGE, "%s: the parts of %d split tiles do not fit the device scratch", name, tiles - whole_tiles);

@@ -133,7 +133,8 @@ int reduce(const char* name, const float* a, const float* b, float* out, int32_t
            void* stream, double* partials = nullptr) {
     if ((mode != 2 && !out) || (mode == 2 && !flag)) return fail(CTAMD_EINVAL, "%s: null output", name);
     if (n && (!a || (T::kIn == 2 && !b))) return fail(CTAMD_EINVAL, "%s: null input", name);
-    if (!partials) partials = reinterpret_cast<double*>(scratch(stream));
+    ScratchUse use(stream, partials == nullptr);
+    if (!partials) partials = reinterpret_cast<double*>(use.ptr());
     if (!partials) return CTAMD_EINVAL;
     hipStream_t s = as_stream(stream);
     unsigned grid = 0;
@@ -365,7 +366,8 @@ int ctamd_colsum_f32(const float* g, float* out, size_t rows, size_t cols, void*
         account(4.0 * double(rows) * double(cols), double(rows) * double(cols));
         return launched(__func__);
     }
-    float* partials = scratch(stream);
+    ScratchUse use(stream);
+    float* partials = use.ptr();
     if (!partials) return CTAMD_EINVAL;
     if (cols > kScratchFloats) return fail(CTAMD_ERANGE, "%s: more than %zu columns", __func__, kScratchFloats);
     bool vec = (cols % 4 == 0) && aligned16(g);

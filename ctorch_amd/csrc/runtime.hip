@@ -71,14 +71,38 @@ const float* pad_zero() {
 
 namespace {
 bool g_scratch_used[kMaxDevices] = {};
-void* g_scratch_user[kMaxDevices] = {};   // the stream whose work used the scratch last
-void* g_recording = nullptr;              // the stream a graph is being recorded on, if any
+void* g_scratch_user[kMaxDevices] = {};      // the stream whose work used the scratch last (compared, never used)
+bool g_user_blocking[kMaxDevices] = {};      // whether that stream orders itself with the null stream
+bool g_event_recorded[kMaxDevices] = {};     // g_scratch_event marks the end of that stream's scratch-using work
+hipEvent_t g_scratch_event[kMaxDevices] = {};
+void* g_recording = nullptr;                 // the stream a graph is being recorded on, if any
 
-bool blocking(void* stream) {             // orders itself with the null stream
+bool blocking(void* stream) {                // orders itself with the null stream
     if (!stream || stream == g_recording) return true;   // recordings are made on streams of ctamd_stream_create
     unsigned flags = 0;
-    if (hipStreamGetFlags(as_stream(stream), &flags) != hipSuccess) return false;
+    if (hipStreamGetFlags(as_stream(stream), &flags) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
     return !(flags & hipStreamNonBlocking);
+}
+bool capturing(void* stream) {
+    if (!stream) return false;
+    if (stream == g_recording) return true;
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(as_stream(stream), &st) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return st != hipStreamCaptureStatusNone;
+}
+int scratch_event(int d, hipEvent_t* ev) {
+    if (!g_scratch_event[d]) {
+        int rc = check_hip(hipEventCreateWithFlags(&g_scratch_event[d], hipEventDisableTiming), "hipEventCreate(scratch)");
+        if (rc) return rc;
+    }
+    *ev = g_scratch_event[d];
+    return CTAMD_OK;
 }
 }  // namespace
 
@@ -88,27 +112,46 @@ int scratch_claim(void* stream) {
     std::lock_guard<std::mutex> lock(g_mu);
     void* user = g_scratch_user[d];
     if (g_scratch_used[d] && user != stream) {
-        const bool ordered = (!user && blocking(stream)) || (!stream && blocking(user));
-        if (!ordered) {
-            if (user == g_recording && user)
-                return fail(CTAMD_EINVAL, "the device scratch belongs to the graph being recorded on another stream");
-            const hipError_t pending = hipStreamQuery(as_stream(user));
-            (void)hipGetLastError();
-            if (pending == hipErrorNotReady)
-                return fail(CTAMD_EINVAL,
-                            "two streams would use the one device scratch at once (reductions, losses, column softmax, split "
-                            "matrix products): wait for the first stream before issuing such work on a second");
+        if (user == g_recording && user)
+            return fail(CTAMD_EINVAL, "the device scratch belongs to the graph being recorded on another stream");
+        if (!capturing(stream)) {            // a recording runs nothing now; its replays claim the scratch themselves
+            hipEvent_t ev = nullptr;
+            if (!user) {
+                // the null stream was the user: blocking streams follow it by themselves, any other waits
+                // for an event recorded on it now (the null stream's handle cannot go stale)
+                if (!blocking(stream)) {
+                    int rc = scratch_event(d, &ev);
+                    if (!rc) rc = check_hip(hipEventRecord(ev, nullptr), "hipEventRecord(scratch)");
+                    if (!rc) rc = check_hip(hipStreamWaitEvent(as_stream(stream), ev, 0), "hipStreamWaitEvent(scratch)");
+                    if (rc) return rc;
+                }
+            } else if (g_event_recorded[d] && !(stream == nullptr && g_user_blocking[d])) {
+                int rc = scratch_event(d, &ev);
+                if (!rc) rc = check_hip(hipStreamWaitEvent(as_stream(stream), ev, 0), "hipStreamWaitEvent(scratch)");
+                if (rc) return rc;
+            }
         }
     }
     g_scratch_used[d] = true;
-    g_scratch_user[d] = stream;
+    if (user != stream) {
+        g_scratch_user[d] = stream;
+        g_user_blocking[d] = blocking(stream);
+        g_event_recorded[d] = false;
+    }
     return CTAMD_OK;
 }
 
-float* scratch(void* stream) {
-    float* s = scratch();
-    if (!s || scratch_claim(stream) != CTAMD_OK) return nullptr;
-    return s;
+void scratch_release(void* stream) {
+    int d = current_device();
+    if (d < 0 || d >= kMaxDevices) return;
+    std::lock_guard<std::mutex> lock(g_mu);
+    if (g_scratch_user[d] != stream) return;          // another thread's stream took over in between
+    g_event_recorded[d] = false;
+    if (!stream || capturing(stream)) return;
+    hipEvent_t ev = nullptr;
+    if (scratch_event(d, &ev) != CTAMD_OK) return;
+    if (hipEventRecord(ev, as_stream(stream)) == hipSuccess) g_event_recorded[d] = true;
+    else (void)hipGetLastError();
 }
 
 float* scratch() {
@@ -245,7 +288,8 @@ int ctamd_graph_end(void* stream, void** graph_out) {
 }
 int ctamd_graph_launch(void* graph, void* stream) {
     if (!graph) return fail(CTAMD_EINVAL, "%s: null graph", __func__);
-    if (scratch_claim(stream) != CTAMD_OK) return CTAMD_EINVAL;   // recorded reductions use the device scratch at replay
+    ScratchUse use(stream);                      // recorded reductions use the device scratch at replay
+    if (!use.ptr()) return CTAMD_EINVAL;
     return check_hip(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), as_stream(stream)), "hipGraphLaunch");
 }
 int ctamd_graph_destroy(void* graph) {

@@ -935,7 +935,8 @@ int run_rows(const char* name, Args a, float* loss_out, void* stream) {
         const bool index = (MODE == kCeIndex || MODE == kCeBwdIndex || kBoth);
         account(per * n + (index ? 4.0 * double(a.rows) : 0.0), n);
     }
-    if (kLoss) a.partials = reinterpret_cast<double*>(scratch(stream));
+    ScratchUse use(stream, kLoss);
+    if (kLoss) a.partials = reinterpret_cast<double*>(use.ptr());
     if (kLoss && !a.partials) return CTAMD_EINVAL;
     // rows are dealt to a chip-filling number of blocks (each walks several rows, prefetching the next)
     const size_t groups = (a.cols + 3) / 4;
@@ -1272,7 +1273,7 @@ struct ColPlan {
 // false: the matrix is small (the sequential kernels serve it) or does not fit the scratch layout
 bool plan_cols(size_t rows, size_t cols, bool aligned, ColPlan& p, void* stream) {
     if (rows < 128) return false;
-    float* sc = scratch(stream);
+    float* sc = scratch();                 // claimed for `stream` by the caller (a ScratchUse in its scope)
     if (!sc) return false;
     size_t chunks = (rows + 31) / 32;
     if (chunks > 256) chunks = 256;
@@ -1379,7 +1380,8 @@ int ctamd_log_softmax_backward_rows_f32(const float* y, const float* g, float* d
 int ctamd_log_softmax_cols_f32(const float* x, float* y, size_t rows, size_t cols, void* stream) {
     if (rows == 0 || cols == 0) return CTAMD_OK;
     if (!x || !y) return fail(CTAMD_EINVAL, "%s: null pointer", __func__);
-    if (rows >= 128 && scratch_claim(stream) != CTAMD_OK) return CTAMD_EINVAL;
+    ScratchUse use(stream, rows >= 128);
+    if (rows >= 128 && !use.ptr()) return CTAMD_EINVAL;
     ColPlan p;
     account(8.0 * double(rows) * double(cols), double(rows) * double(cols));
     if (plan_cols(rows, cols, aligned16(x) && aligned16(y), p, stream)) {
@@ -1395,7 +1397,8 @@ int ctamd_log_softmax_cols_f32(const float* x, float* y, size_t rows, size_t col
 int ctamd_log_softmax_backward_cols_f32(const float* y, const float* g, float* dx, size_t rows, size_t cols, void* stream) {
     if (rows == 0 || cols == 0) return CTAMD_OK;
     if (!y || !g || !dx) return fail(CTAMD_EINVAL, "%s: null pointer", __func__);
-    if (rows >= 128 && scratch_claim(stream) != CTAMD_OK) return CTAMD_EINVAL;
+    ScratchUse use(stream, rows >= 128);
+    if (rows >= 128 && !use.ptr()) return CTAMD_EINVAL;
     ColPlan p;
     account(12.0 * double(rows) * double(cols), 2.0 * double(rows) * double(cols));
     if (plan_cols(rows, cols, aligned16(y) && aligned16(g) && aligned16(dx), p, stream)) {
@@ -1414,7 +1417,8 @@ int ctamd_log_softmax_backward_cols_f32(const float* y, const float* g, float* d
 int ctamd_softmax_cols_f32(const float* x, float* y, size_t rows, size_t cols, void* stream) {
     if (rows == 0 || cols == 0) return CTAMD_OK;
     if (!x || !y) return fail(CTAMD_EINVAL, "%s: null pointer", __func__);
-    if (rows >= 128 && scratch_claim(stream) != CTAMD_OK) return CTAMD_EINVAL;
+    ScratchUse use(stream, rows >= 128);
+    if (rows >= 128 && !use.ptr()) return CTAMD_EINVAL;
     ColPlan p;
     if (plan_cols(rows, cols, aligned16(x) && aligned16(y), p, stream)) {
         hipStream_t s = as_stream(stream);
@@ -1433,7 +1437,8 @@ int ctamd_softmax_cols_f32(const float* x, float* y, size_t rows, size_t cols, v
 int ctamd_softmax_backward_cols_f32(const float* y, const float* g, float* dx, size_t rows, size_t cols, void* stream) {
     if (rows == 0 || cols == 0) return CTAMD_OK;
     if (!y || !g || !dx) return fail(CTAMD_EINVAL, "%s: null pointer", __func__);
-    if (rows >= 128 && scratch_claim(stream) != CTAMD_OK) return CTAMD_EINVAL;
+    ScratchUse use(stream, rows >= 128);
+    if (rows >= 128 && !use.ptr()) return CTAMD_EINVAL;
     ColPlan p;
     if (plan_cols(rows, cols, aligned16(y) && aligned16(g) && aligned16(dx), p, stream)) {
         hipStream_t s = as_stream(stream);

@@ -525,7 +525,8 @@ bool plan_cols(const float* x, const void* other, size_t outer, size_t len, size
 template <int KIND>
 int run_forward(const char* name, const float* x, float* out, int32_t* index, float* mean_out, size_t outer, size_t len,
                 size_t inner, int ddof, hipStream_t s) {
-    Part* parts = reinterpret_cast<Part*>(scratch(static_cast<void*>(s)));
+    ScratchUse use(static_cast<void*>(s));
+    Part* parts = reinterpret_cast<Part*>(use.ptr());
     if (!parts) return CTAMD_EINVAL;
     constexpr size_t kSlots = kScratchFloats * sizeof(float) / sizeof(Part);
     if (inner == 1) {

@@ -551,7 +551,8 @@ int ctamd_softmax_f64(const double* x, double* y, size_t rows, size_t cols, int 
         // at once on [8192 x 8192] - a panel's launches are too small to fill the chip.)
         const size_t strips = (cols + per_block - 1) / per_block;
         if (strips > 0x7fffffffu) return fail(CTAMD_ERANGE, "%s: too many columns", __func__);
-        MaxSum* pairs = reinterpret_cast<MaxSum*>(scratch(stream));
+        ScratchUse use(stream);
+        MaxSum* pairs = reinterpret_cast<MaxSum*>(use.ptr());
         if (!pairs) return CTAMD_EINVAL;
         // chunks of at least 32 rows, at most 256 of them (half as many ran the two sweeps 15% slower: they
         // are bound by the exponential's arithmetic and want the blocks), as many as the scratch holds

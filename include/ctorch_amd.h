@@ -11,10 +11,13 @@
  *  - Launchers never allocate, free or synchronise: they enqueue on `stream` (a hipStream_t passed
  *    as void*, NULL = the default stream) and return.  Results are ready after ctamd_sync(stream).
  *  - Reductions, losses, column softmax / sums and matrix products whose tiles are cut along K use
- *    a per-device scratch buffer that ctamd_init() allocates once.  It serves one stream at a time:
- *    the null stream and blocking streams order themselves with each other and may alternate; any
- *    other stream is accepted only when the stream that used the scratch before has nothing
- *    pending, else the call returns CTAMD_EINVAL and launches nothing.
+ *    a per-device scratch buffer that ctamd_init() allocates once.  All streams of a device share
+ *    it, and the library puts them in order: a call on another stream than the previous such call
+ *    makes its stream wait (on the device) for the previous stream's scratch-using work, through an
+ *    event the library records after that work.  So such calls run one after another across streams,
+ *    never at once.  While a graph is being recorded the scratch belongs to the recording (other
+ *    streams get CTAMD_EINVAL); replays take their turn through ctamd_graph_launch.  Work recorded
+ *    into a graph by other means than ctamd_graph_begin / _end is not tracked at replay.
  *  - Math mode (ctamd_set_math_mode): CTAMD_MATH_FAST, the default, evaluates the exponentials of
  *    softmax / log-softmax / cross entropy and the sigmoid, sin, cos of fused expressions in single
  *    precision within 2 ulp of the reference's libm loops (a fused tanh keeps the reference's bits:
