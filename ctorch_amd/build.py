@@ -17,7 +17,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 RESOURCES = os.path.join(os.path.dirname(os.path.abspath(__file__)), "kernel_resources.json")
 LIB = os.path.join(HERE, "libctorch_amd.so")
-SOURCES = ["runtime.hip", "elementwise.hip", "reduce.hip", "softmax_ce.hip", "matmul.hip", "dataset.hip", "expr.hip", "expr_jit.hip", "typed.hip", "stats.hip"]
+SOURCES = ["runtime.hip", "elementwise.hip", "reduce.hip", "softmax_ce.hip", "matmul.hip", "dataset.hip", "expr.hip", "expr_jit.hip", "typed.hip", "stats.hip", "head.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function"]
 

@@ -72,6 +72,8 @@ PROTOTYPES.update({
     "ctamd_accumulate_typed": [_P, _P, C.c_int, _Z, _P],
     "ctamd_softmax_f64": [_P, _P, _Z, _Z, C.c_int, _P],
     "ctamd_expr_run_f32": [_P, C.c_int, _P, C.c_int, _P, C.c_int, _P, _Z, _Z, _P],
+    "ctamd_linear_ce_head_fits": [_Z, _Z],
+    "ctamd_linear_ce_head_f32": [_P, _P, _P, _P, _P, _P, _P, _P, _P, C.c_int, _P, _P, _Z, _Z, _Z, _P],
     "ctamd_set_expr_jit": [C.c_int],
     "ctamd_expr_jit": [],
     "ctamd_expr_jit_compile": [_P, C.c_int, C.c_int, C.c_int, _P, _Z, _P],

@@ -271,6 +271,23 @@ int ctamd_cross_entropy_backward_index_stats_f32(const float* x, const float* id
 int ctamd_cross_entropy_index_fused_f32(const float* x, const float* idx, float* out, int32_t* status, float* dx,
                                         size_t rows, size_t cols, void* stream);
 
+/* The classifier head of a small network - the last layer, its cross entropy and every gradient that
+ * flows out of them - in one pass over the hidden activations h [batch, hidden]:
+ *   z = h . w + bias (mnist/mnist.cpp:41), out[0] / status[0] as ctamd_cross_entropy_index_f32 (the SUM
+ *   over rows of -log(max(softmax(z)[label], 1e-10)), CrossEntropy_BASIC_kernel.cpp:88-120),
+ *   dz = softmax(z) - onehot(label) (src/AutoDiff.cpp:1517-1601 for an upstream gradient of 1),
+ *   dh = dz . w^T (src/AutoDiff.cpp:1684-1704), times [h > 0] when mask_by_h is set (the ReLU branch
+ *   :1320-1371 of the layer that produced h), gw = h^T . dz (:1766-1810), gb = the column sums of dz.
+ * z and dh may be null.  2 to 16 classes, hidden a multiple of four up to 256 (ctamd_linear_ce_head_fits
+ * tells), h and dh 16-byte aligned; CTAMD_ERANGE otherwise with nothing launched.  fp32 fused
+ * multiply-adds in a fixed order (deterministic), so products differ from ctamd_matmul_f32's in the last
+ * bits: equal to the five separate launches within the MatMul bound.  Uses the per-device scratch.
+ * The reference runs the five steps as separate kernels and tape branches. */
+int ctamd_linear_ce_head_fits(size_t hidden, size_t classes);
+int ctamd_linear_ce_head_f32(const float* h, const float* w, const float* bias, const float* labels, float* out, int32_t* status,
+                             float* z, float* dz, float* dh, int mask_by_h, float* gw, float* gb, size_t batch, size_t hidden,
+                             size_t classes, void* stream);
+
 /* -------------------------------------------------------------------------------- matmul */
 /* C[i,j] = sum_l A[i*as0 + l*as1] * B[l*bs0 + j*bs1]; C is [m, n] row-major contiguous; strides
  * are in elements and may describe a transposed view.  MatMul_BASIC_kernel.cpp:42-54.  The

@@ -252,6 +252,23 @@ def matmul(a, b):
     return c
 
 
+def linear_ce_head(h, w, bias, labels, mask_by_h, want_z=True, want_dh=True, expect=0):
+    """The classifier head in one pass: returns (loss, status, z, dz, dh, gw, gb) as device tensors / ints."""
+    B, H = h.shape
+    N = w.shape[1]
+    pair = torch.zeros(2, device=DEV)
+    status = torch.full((1,), -7, dtype=torch.int32, device=DEV)
+    z = torch.zeros((B, N), device=DEV) if want_z else None
+    dz = torch.zeros((B, N), device=DEV)
+    dh = torch.zeros((B, H), device=DEV) if want_dh else None
+    gw = torch.zeros((H, N), device=DEV)
+    gb = torch.zeros(N, device=DEV)
+    rc = lib().ctamd_linear_ce_head_f32(ptr(h), ptr(w), ptr(bias), ptr(labels), ptr(pair), ptr(status), ptr(z), ptr(dz), ptr(dh),
+                                        int(mask_by_h), ptr(gw), ptr(gb), B, H, N, stream())
+    assert rc == expect, (rc, lib().ctamd_last_error().decode())
+    return pair[:1], int(status.item()), z, dz, dh, gw, gb
+
+
 class ExprInsn(C.Structure):
     _fields_ = [("op", C.c_uint8), ("dst", C.c_uint8), ("a", C.c_uint8), ("b", C.c_uint8), ("imm", C.c_float)]
 
