@@ -236,9 +236,21 @@ def config_report(with_cpu):
         rc = host.cth_time_mlp(fp(x), L(Bn), L(784), fp(W1), fp(b1), L(256), fp(W2), fp(b2), L(10), fp(lab), I(5),
                                I(30), out)
         host.cth_set_ce_deferred_label_check(0)
-        host.cth_set_fused_layers(0)
         add("config 3: MLP 784-256-10 train step, batch %d, fused layers, label check deferred to the loss read" % Bn, rc, out,
             cpu, note, launch_bound=(Bn == 256))
+        # the last layer, its cross entropy and the gradients that leave them in one pass over the hidden
+        # activations (Tensor::linear_cross_entropy): equal within the MatMul bound, three launches fewer
+        host.cth_set_fused_head(1)
+        for deferred in (0, 1):
+            host.cth_set_ce_deferred_label_check(deferred)
+            out = D5()
+            rc = host.cth_time_mlp(fp(x), L(Bn), L(784), fp(W1), fp(b1), L(256), fp(W2), fp(b2), L(10), fp(lab), I(5),
+                                   I(30), out)
+            add("config 3: MLP 784-256-10 train step, batch %d, fused layers, one-pass head%s"
+                % (Bn, ", label check deferred to the loss read" if deferred else ""), rc, out, cpu, note, launch_bound=(Bn == 256))
+        host.cth_set_ce_deferred_label_check(0)
+        host.cth_set_fused_head(0)
+        host.cth_set_fused_layers(0)
         # the same step (one-hot targets) recorded into a HIP graph once and replayed
         oh = np.zeros((Bn, 10), np.float32)
         oh[np.arange(Bn), lab.astype(int)] = 1

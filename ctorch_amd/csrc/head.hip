@@ -14,7 +14,7 @@
 // meet (W stays in registers for all rows); the 4 x N partial logits go round the wave with the
 // halving exchange of the narrow products (lane r * N + c ends up with z[r][c]); the N lanes of a row
 // form its softmax by lane reads; dz comes back to every lane through scalar lane reads and meets h
-// and W in registers once more for dh and for the wave's share of gW.  The shares of the block's four
+// and W in registers once more for dh and for the wave's share of gW.  The shares of the block's eight
 // waves are added in wave order through LDS; every block leaves gW, gb, its loss (a double) and a
 // bad-label flag in the device scratch, and a second launch adds the blocks in block order
 // (deterministic; 16 lanes per element).
@@ -26,7 +26,7 @@ namespace {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-constexpr int kHeadThreads = 256;
+constexpr int kHeadThreads = 512;          // eight waves: two per SIMD, whose exchanges and lane reads hide each other's latency
 constexpr int kHeadWaves = kHeadThreads / 64;
 constexpr int kHeadRows = 4;              // rows a wave works on at a time
 constexpr int kHeadMaxBlocks = 256;       // partial results kept per launch
@@ -252,33 +252,65 @@ __global__ __launch_bounds__(kHeadThreads) void head_kernel(HeadArgs a) {
     }
 }
 
-// Adds the blocks' shares in block order: 16 lanes per element of [gW | gb], lane j of an element
-// adds blocks j, j + 16, ... in order and the 16 partial sums are added in a fixed tree.  The first
+// Adds the blocks' shares in block order.  A block of 256 threads owns 16 neighbouring elements of
+// [gW | gb]: thread (slice s, element e) adds blocks s, s + 16, s + 32, ... in that order, sixteen
+// loads in flight at a time, and the sixteen slices are added in slice order through LDS.  The first
 // thread of the launch adds the blocks' losses and flags.
-__global__ __launch_bounds__(kHeadThreads) void head_fold_kernel(const float* __restrict__ part, int blocks, int per_block, int gw_elems,
+constexpr int kFoldThreads = 256;
+__global__ __launch_bounds__(kFoldThreads) void head_fold_kernel(const float* __restrict__ part, int blocks, int per_block, int gw_elems,
                                                                   float* __restrict__ gw, float* __restrict__ gb, float* __restrict__ loss,
                                                                   int32_t* __restrict__ status) {
-    const int gid = blockIdx.x * kHeadThreads + threadIdx.x;
-    const int elem = gid / 16, j = gid % 16;
+    __shared__ float s_t[16][17];
+    const int e = threadIdx.x % 16, s = threadIdx.x / 16;
+    const int elem = blockIdx.x * 16 + e;
     float t = 0.0f;
     if (elem < per_block) {
-        for (int b = j; b < blocks; b += 16) t = t + part[size_t(b) * per_block + elem];
-    }
-    for (int off = 8; off >= 1; off /= 2) t = t + __shfl_xor(t, off, 64);
-    if (elem < per_block && j == 0) {
-        if (elem < gw_elems) gw[elem] = t;
-        else gb[elem - gw_elems] = t;
-    }
-    if (gid == 0) {
-        const double* tail = reinterpret_cast<const double*>(part + size_t(blocks) * per_block + (size_t(per_block) * blocks) % 2);
-        double l = 0.0;
-        bool bad = false;
-        for (int b = 0; b < blocks; ++b) {
-            l += tail[2 * b];
-            bad = bad || tail[2 * b + 1] != 0.0;
+        for (int base = 0; base < blocks; base += 256) {
+            float v[16];
+#pragma unroll
+            for (int q = 0; q < 16; ++q) {
+                const int b = base + s + 16 * q;
+                v[q] = b < blocks ? part[size_t(b) * per_block + elem] : 0.0f;
+            }
+#pragma unroll
+            for (int q = 0; q < 16; ++q) t = t + v[q];
         }
-        loss[0] = float(l);
-        if (status) status[0] = bad ? 1 : 0;
+    }
+    s_t[s][e] = t;
+    __syncthreads();
+    if (s == 0 && elem < per_block) {
+        float sum = s_t[0][e];
+#pragma unroll
+        for (int q = 1; q < 16; ++q) sum = sum + s_t[q][e];
+        if (elem < gw_elems) gw[elem] = sum;
+        else gb[elem - gw_elems] = sum;
+    }
+    // the blocks' losses and flags: the last wave of the first block, lane l adds blocks l, l + 64, ...
+    // in order (at most kHeadMaxBlocks / 64 loads each, all in flight), then the lanes in a fixed tree
+    if (blockIdx.x == 0 && threadIdx.x >= kFoldThreads - 64) {
+        const int lane = threadIdx.x & 63;
+        const double* tail = reinterpret_cast<const double*>(part + size_t(blocks) * per_block + (size_t(per_block) * blocks) % 2);
+        double v[kHeadMaxBlocks / 64], f[kHeadMaxBlocks / 64];
+#pragma unroll
+        for (int q = 0; q < kHeadMaxBlocks / 64; ++q) {
+            const int b = lane + 64 * q;
+            v[q] = b < blocks ? tail[2 * b] : 0.0;
+            f[q] = b < blocks ? tail[2 * b + 1] : 0.0;
+        }
+        double l = 0.0, bad = 0.0;
+#pragma unroll
+        for (int q = 0; q < kHeadMaxBlocks / 64; ++q) {
+            l += v[q];
+            bad += f[q];
+        }
+        for (int off = 32; off > 0; off >>= 1) {
+            l += __shfl_xor(l, off, 64);
+            bad += __shfl_xor(bad, off, 64);
+        }
+        if (lane == 0) {
+            loss[0] = float(l);
+            if (status) status[0] = bad != 0.0 ? 1 : 0;
+        }
     }
 }
 
@@ -342,9 +374,8 @@ extern "C" int ctamd_linear_ce_head_f32(const float* h, const float* w, const fl
     }
     if (rc) return rc;
     const int per_block = int(head_part_floats(H, N));
-    const int fold_threads = per_block * 16;
-    hipLaunchKernelGGL(head_fold_kernel, dim3(unsigned((fold_threads + kHeadThreads - 1) / kHeadThreads)), dim3(kHeadThreads), 0, s, part, blocks,
-                       per_block, H * N, gw, gb, loss, status);
+    hipLaunchKernelGGL(head_fold_kernel, dim3(unsigned((per_block + 15) / 16)), dim3(kFoldThreads), 0, s, part, blocks, per_block, H * N, gw, gb,
+                       loss, status);
     // what the five launches this replaces must move and compute: h read, dh written, the small
     // operands; three products of 2 B H N flop
     account(4.0 * (double(B) * H * (dh ? 2.0 : 1.0) + 2.0 * double(H) * N + 3.0 * double(B) * N), 6.0 * double(B) * double(H) * double(N));

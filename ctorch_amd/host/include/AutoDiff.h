@@ -66,6 +66,12 @@ class AutoDiff {
         Tensor index;    // max / min: position of the extreme element along the axis (int32)
         Tensor mean;     // var / std
     };
+    // what Tensor::linear_cross_entropy formed in its one pass (op::LinearCE): the gradient of the logits
+    // for an upstream gradient of 1, and from it the gradients of the three inputs
+    struct LinearCEPayload : OpPayload {
+        Tensor labels, dz, dh, gw, gb;
+        bool dh_masked = false;   // dh is already multiplied by [h > 0]: the gradient at the pre-activation of the ReLU layer that produced h
+    };
     struct Node {
         size_t tensor_id = 0;
         op operation = op::Add;
@@ -103,6 +109,8 @@ class AutoDiff {
     void backward(Tensor& root, Tensor grad_output);
     void clear_graph();
     size_t node_count();
+    // whether t is on the tape as the output of a fused layer with its ReLU (Tensor::linear(.., true))
+    bool is_relu_layer_output(const Tensor& t);
 
     void set_broadcast_grad(BroadcastGrad m) { broadcast_grad_ = m; }
     BroadcastGrad broadcast_grad() const { return broadcast_grad_; }

@@ -22,6 +22,7 @@ enum class op {
     Sum,
     Linear,   // not in the reference: matmul + bias row (+ ReLU) as one taped operator, Tensor::linear
     Fused,    // not in the reference: an elementwise expression evaluated in one pass, Expr::eval
+    LinearCE, // not in the reference: the last layer and its class-index cross entropy, Tensor::linear_cross_entropy
     // methods the reference declares on Tensor without defining them (include/Tensor.h:824-1072); they
     // have no enumerator there because nothing tapes them
     Abs, Exp, Log, Sqrt, Square, Tan, LogSoftmax,

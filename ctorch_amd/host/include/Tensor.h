@@ -138,6 +138,17 @@ class Tensor {
     // device, with the values and gradients of the three-operator form bit for bit.  On the host it
     // is the three operators.
     Tensor linear(const Tensor& weight, const Tensor& bias, bool relu = false) const;
+    // Not in the reference: `x.linear(weight, bias).cross_entropy(labels)` with class-index labels
+    // (mnist/mnist.cpp:41 and :67-73; CrossEntropy_BASIC_kernel.cpp:88-120) as ONE operator.  For a head
+    // of at most 16 classes over at most 256 hidden units the device forms the logits, the loss and -
+    // under a tape - the gradients of x, weight and bias in one pass over x; backward() hands them
+    // out when the loss is its root (any other upstream gradient rescales the kept gradient of the
+    // logits and takes the usual products).  Values agree with the two-operator form within the
+    // MatMul bound (the products are added in another order).  It is one node of the tape: a tape that
+    // is walked twice without being cleared adds one contribution per pass to x, weight and bias,
+    // where the two-operator form's logits node would accumulate too.  Any other shape, a host tensor or
+    // one-hot targets: the two operators.  logits (optional) receives x.linear(weight, bias).
+    Tensor linear_cross_entropy(const Tensor& weight, const Tensor& bias, const Tensor& labels, Tensor* logits = nullptr) const;
     Tensor dot(const Tensor& other) const;
     Tensor relu() const;
     Tensor sigmoid() const;

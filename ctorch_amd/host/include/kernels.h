@@ -127,6 +127,13 @@ Tensor mul_plus(const Tensor& a, const Tensor& b, const Tensor& acc);
 // acc + the MSE (mae = false) or MAE gradient, in the pass that forms it
 Tensor loss_backward_plus(bool mae, const Tensor& p, const Tensor& t, const Tensor& g0d, const Tensor& acc);
 Tensor cross_entropy_backward(const Tensor& x, const Tensor& target, const Tensor& g0d);
+// The classifier head in one pass (ctamd_linear_ce_head_f32); whether the shapes fit it, and the call:
+// returns the loss (an empty Tensor for a class index out of range, as CrossEntropy_AMD_kernel), fills
+// the gradient of the logits for an upstream gradient of 1, of the weights and of the bias, the
+// logits when wanted, and dh (times [h > 0] when mask_by_h) when wanted.
+bool linear_ce_head_fits(const Tensor& h, const Tensor& w, const Tensor& bias, const Tensor& labels);
+Tensor linear_ce_head(const Tensor& h, const Tensor& w, const Tensor& bias, const Tensor& labels, bool mask_by_h, Tensor* logits,
+                      Tensor& dz, Tensor* dh, Tensor& gw, Tensor& gb);
 Tensor div_backward_b(const Tensor& a, const Tensor& b, const Tensor& g);
 // The stream every launch of this front-end goes to (as the C ABI's void*): the null stream unless a
 // DeviceGraph is recording or has installed its own.  While a graph records, anything that would

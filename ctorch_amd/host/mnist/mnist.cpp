@@ -2,7 +2,7 @@
 // printed results, data set and parameters resident in HBM.
 //
 //   mnist.bin [--data DIR] [--epochs N] [--batch N] [--lr X] [--hidden1 N] [--hidden2 N]
-//             [--reference-tape | --graph] [--fused]
+//             [--reference-tape | --graph] [--fused | --fused-head]
 //
 // --graph records one training step into a HIP graph at the first batch and replays it for every
 // batch: one launch per step instead of about fifty.
@@ -34,6 +34,7 @@ int main(int argc, char** argv) {
         else if (a == "--reference-tape") opt.reference_tape = true;
         else if (a == "--graph") opt.use_graph = true;
         else if (a == "--fused") opt.fused_layers = true;
+        else if (a == "--fused-head") opt.fused_layers = opt.fused_head = true;
         else {
             std::fprintf(stderr, "unknown option %s\n", a.c_str());
             return 2;

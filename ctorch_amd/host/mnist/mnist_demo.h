@@ -26,6 +26,8 @@ struct MnistDemoOptions {
     bool use_graph = false;
     // each layer as one fused operator (Tensor::linear) and the optimiser update as one launch
     bool fused_layers = false;
+    // with fused_layers: the last layer and its loss as the one-pass head (Tensor::linear_cross_entropy)
+    bool fused_head = false;
 };
 
 struct MnistDemoResult {
@@ -48,6 +50,7 @@ inline MnistDemoResult run_mnist_demo(const MnistDemoOptions& opt) {
     res.pixels = train_images.shape()[1];
     NeuralNetwork model(int(res.pixels), opt.hidden1, opt.hidden2, 10, opt.learning_rate);
     model.fused_layers = opt.fused_layers;
+    model.fused_head = opt.fused_head;
     res.num_batches = int(res.train_images) / opt.batch_size;
 
     AutoDiff autodiff;

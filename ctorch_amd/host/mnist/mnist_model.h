@@ -43,6 +43,10 @@ class NeuralNetwork {
 
     // true: each layer is one fused operator (Tensor::linear); same values and gradients, fewer launches
     bool fused_layers = false;
+    // with fused_layers: the last layer, its cross entropy (on the class indices themselves, no one-hot
+    // matrix) and the gradients that leave them in one pass (Tensor::linear_cross_entropy); values
+    // within the MatMul bound of the other forms
+    bool fused_head = false;
 
     Tensor forward(const Tensor& x) {
         if (fused_layers) return x.linear(W1, b1, true).linear(W2, b2, true).linear(W3, b3, false);
@@ -65,9 +69,14 @@ class NeuralNetwork {
         for (Tensor* p : params) p->requires_grad(true);
         if (ctx)
             for (Tensor* p : params) ctx->zero_grad(*p);
-        Tensor logits = forward(x);
-        Tensor y_one_hot = ctorch_amd_host::onehot(y, logits.sizes()[1]);
-        Tensor loss = logits.cross_entropy(y_one_hot);
+        Tensor loss;
+        if (fused_layers && fused_head) {
+            loss = x.linear(W1, b1, true).linear(W2, b2, true).linear_cross_entropy(W3, b3, y);
+        } else {
+            Tensor logits = forward(x);
+            Tensor y_one_hot = ctorch_amd_host::onehot(y, logits.sizes()[1]);
+            loss = logits.cross_entropy(y_one_hot);
+        }
         backward(loss);
         update_parameters();
         return loss;

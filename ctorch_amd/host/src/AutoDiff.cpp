@@ -21,6 +21,13 @@ AutoDiff::Node* AutoDiff::find(size_t id) {
     return (it == id_to_node.end() || !it->second) ? nullptr : it->second.get();
 }
 
+bool AutoDiff::is_relu_layer_output(const Tensor& t) {
+    if (t.id() == 0) return false;
+    std::lock_guard<std::mutex> lock(records_mutex);
+    Node* n = find(t.id());
+    return n && !n->is_leaf && n->operation == op::Linear && n->op_param_i != 0;
+}
+
 size_t AutoDiff::node_count() {
     std::lock_guard<std::mutex> lock(records_mutex);
     return id_to_node.size();
@@ -361,6 +368,27 @@ Tensor AutoDiff::input_gradient(Node* node, size_t input_id, size_t input_pos, c
             }
             return MatMul_AMD_kernel(Tensor::view_t(other), gz);                        // x^T . gz
         }
+        case op::LinearCE: {                                            // Linear's and CE's branches on what the forward pass kept
+            auto* kept = dynamic_cast<LinearCEPayload*>(node->payload.get());
+            if (!kept)
+                Ctorch_Error::throwException(ErrorPlatform::kAutoDiff, ErrorType::TENSOR_STATE, "backward: classifier head without its record");
+            // the kept gradients are those for an upstream gradient of 1 (a loss that is the root)
+            const bool unit = g.known_value() && *g.known_value() == 1.0f;
+            if (!unit && !node->shared_term) node->shared_term = std::make_unique<Tensor>(Mul_AMD_kernel(kept->dz, g));
+            const Tensor& gz = unit ? kept->dz : *node->shared_term;
+            term_plus_zero_ = true;                                     // sums of products from +0, and "0 +" terms
+            if (input_pos == 0) {
+                if (unit && !kept->dh.is_cleared() && !kept->dh_masked) return Tensor::alias(kept->dh);
+                return MatMul_AMD_kernel(gz, Tensor::view_t(*find(node->input_ids[1])->tensor));   // gz . W^T
+            }
+            if (input_pos == 1) {
+                if (unit) return Tensor::alias(kept->gw);
+                return MatMul_AMD_kernel(Tensor::view_t(*find(node->input_ids[0])->tensor), gz);   // h^T . gz
+            }
+            if (unit && broadcast_grad_ == BroadcastGrad::kColumnSum) return Tensor::alias(kept->gb);
+            term_plus_zero_ = false;
+            return Tensor::alias(gz);                                   // shaped by the caller (column sums, or row 0)
+        }
         case op::Fused: {                                               // every operator branch above, in one launch
             if (node->input_grads.empty()) {
                 auto* program = dynamic_cast<FusedPayload*>(node->payload.get());
@@ -587,6 +615,18 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
                     wn->tensor->sizes()[0] == in->tensor->sizes()[1]) {
                     in->grad = std::make_unique<Tensor>(MatMulReluMask_AMD_kernel(gz, Tensor::view_t(*wn->tensor), *in->tensor));
                     in->grad_plus_zero = false;          // g * 0 may be -0
+                    in->grad_premasked_by = node;
+                    continue;
+                }
+            }
+            // The same for a classifier head whose one pass already formed that masked gradient.
+            if (fuse_relu_mask_ && pos == 0 && node->operation == op::LinearCE && !in->grad && in != root_node && !in->is_leaf &&
+                in->operation == op::Linear && in->op_param_i != 0 && consumers[input_id] == 1 && node_grad.known_value() &&
+                *node_grad.known_value() == 1.0f) {
+                auto* kept = dynamic_cast<LinearCEPayload*>(node->payload.get());
+                if (kept && kept->dh_masked && !kept->dh.is_cleared()) {
+                    in->grad = std::make_unique<Tensor>(Tensor::alias(kept->dh));
+                    in->grad_plus_zero = false;
                     in->grad_premasked_by = node;
                     continue;
                 }

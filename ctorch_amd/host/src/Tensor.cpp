@@ -357,6 +357,25 @@ Tensor Tensor::linear(const Tensor& weight, const Tensor& bias, bool relu) const
     tape(result, op::Linear, {this, &weight, &bias}, relu ? 1 : 0);
     return result;
 }
+Tensor Tensor::linear_cross_entropy(const Tensor& weight, const Tensor& bias, const Tensor& labels, Tensor* logits) const {
+    if (!ctorch_amd_host::linear_ce_head_fits(*this, weight, bias, labels)) {
+        Tensor z = linear(weight, bias, false);
+        if (logits) *logits = Tensor::alias(z);
+        return z.cross_entropy(labels);
+    }
+    AutoDiff* ctx = AutoDiffContext::current();
+    const bool taped = ctx && (requires_grad() || weight.requires_grad() || bias.requires_grad());
+    auto kept = std::make_shared<AutoDiff::LinearCEPayload>();
+    kept->labels = Tensor::alias(labels);
+    // under a tape the gradient of x is formed too, at the pre-activation when x comes out of a ReLU layer
+    const bool want_dh = taped && requires_grad();
+    kept->dh_masked = want_dh && ctx->is_relu_layer_output(*this);
+    Tensor result = ctorch_amd_host::linear_ce_head(*this, weight, bias, labels, kept->dh_masked, logits, kept->dz, want_dh ? &kept->dh : nullptr,
+                                                    kept->gw, kept->gb);
+    if (result.is_cleared()) return result;                       // a class index out of range: logged, empty, as cross_entropy
+    if (taped) tape(result, op::LinearCE, {this, &weight, &bias}, 0, kept);
+    return result;
+}
 namespace {
 Tensor compare_with(int cmp, const Tensor& a, const Tensor* b, float s) {
     if (a.device() != DeviceType::kAMD)

@@ -622,6 +622,38 @@ Tensor cross_entropy_backward(const Tensor& x, const Tensor& target, const Tenso
         run(ctamd_cross_entropy_backward_index_f32(x.fptr(), target.fptr(), g.fptr(), r.fptr(), rows, cols, current_stream()), "cross_entropy_backward");
     return r;
 }
+bool linear_ce_head_fits(const Tensor& h, const Tensor& w, const Tensor& bias, const Tensor& labels) {
+    auto dev_float = [](const Tensor& t) { return t.device() == DeviceType::kAMD && t.dtype() == DType::kFloat && t.is_contiguous(); };
+    if (!dev_float(h) || !dev_float(w) || !dev_float(bias) || !dev_float(labels)) return false;
+    if (h.dim() != 2 || w.dim() != 2 || bias.dim() != 1 || labels.dim() != 1) return false;
+    if (w.sizes()[0] != h.sizes()[1] || bias.sizes()[0] != w.sizes()[1] || labels.sizes()[0] != h.sizes()[0] || h.sizes()[0] == 0) return false;
+    if ((reinterpret_cast<uintptr_t>(h.fptr()) & 15u) != 0) return false;
+    return ctamd_linear_ce_head_fits(h.sizes()[1], w.sizes()[1]) != 0;
+}
+Tensor linear_ce_head(const Tensor& h, const Tensor& w, const Tensor& bias, const Tensor& labels, bool mask_by_h, Tensor* logits,
+                      Tensor& dz, Tensor* dh, Tensor& gw, Tensor& gb) {
+    const size_t B = h.sizes()[0], H = h.sizes()[1], N = w.sizes()[1];
+    Tensor pair(ShapeTag{}, {2}, DType::kFloat, DeviceType::kAMD, false);      // loss and bad-label flag side by side: one transfer
+    Tensor loss = Tensor::view_element(pair, 0);
+    if (logits) *logits = Tensor(ShapeTag{}, {B, N}, DType::kFloat, DeviceType::kAMD, false);
+    dz = Tensor(ShapeTag{}, {B, N}, DType::kFloat, DeviceType::kAMD, false);
+    if (dh) *dh = Tensor(ShapeTag{}, {B, H}, DType::kFloat, DeviceType::kAMD, false);
+    gw = Tensor(ShapeTag{}, {H, N}, DType::kFloat, DeviceType::kAMD, false);
+    gb = Tensor(ShapeTag{}, {N}, DType::kFloat, DeviceType::kAMD, false);
+    run(ctamd_linear_ce_head_f32(h.fptr(), w.fptr(), bias.fptr(), labels.fptr(), loss.fptr(), reinterpret_cast<int32_t*>(pair.fptr() + 1),
+                                 logits ? logits->fptr() : nullptr, dz.fptr(), dh ? dh->fptr() : nullptr, mask_by_h ? 1 : 0, gw.fptr(),
+                                 gb.fptr(), B, H, N, current_stream()),
+        "linear_cross_entropy");
+    if (recording() || g_ce_deferred_check) return loss;     // as CrossEntropy_AMD_kernel: a bad index then shows as a NaN loss
+    struct { float loss; int32_t bad; } got = {0.0f, 0};
+    device_copy_d2h(&got, pair.fptr(), sizeof(got));
+    if (got.bad) {
+        Ctorch_Error::log(ErrorLevel::ERROR, kP, ErrorType::TENSOR_STATE, "linear_cross_entropy: class index out of range");
+        return Tensor();
+    }
+    loss.set_known_value(got.loss);
+    return loss;
+}
 Tensor div_backward_b(const Tensor& a, const Tensor& b, const Tensor& g) {
     check_device(a, "div_backward");
     Tensor r = like(a);

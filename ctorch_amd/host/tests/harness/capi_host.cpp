@@ -105,6 +105,7 @@ void cth_quiet() { Ctorch_Error::setPrintLevel(PrintLevel::MINIUM); }
 // Applies to the contexts the entry points below create.
 static int g_row0 = 0;
 static int g_fused_layers = 0;
+static int g_fused_head = 0;
 static int g_fused_expr = 0;
 extern "C" void cth_set_ce_deferred_label_check(int on) { ctorch_amd_host::set_ce_deferred_label_check(on != 0); }
 // the elementwise parts of cth_chain, cth_expr, cth_program and their timed versions are built as
@@ -125,6 +126,8 @@ void cth_last_expr_stats(int* out) {
 void cth_set_reference_row0(int on) { g_row0 = on; }
 // the MLP entry points below build each layer with Tensor::linear (one fused operator) when set
 void cth_set_fused_layers(int on) { g_fused_layers = on; }
+// with fused layers: the last layer and its class-index cross entropy as one operator (Tensor::linear_cross_entropy)
+void cth_set_fused_head(int on) { g_fused_head = on; }
 // the ReLU mask of a fused layer in the product that forms the layer's output gradient (default) or
 // as a launch of its own
 static int g_fuse_relu_mask = 1;
@@ -572,8 +575,13 @@ long cth_mlp_step(const float* x, long B, long I, const float* W1, const float* 
         tW2.requires_grad(true);
         tb2.requires_grad(true);
         Tensor h = g_fused_layers ? tx.linear(tW1, tb1, true) : (tx.matmul(tW1) + tb1).relu();
-        Tensor logits = g_fused_layers ? h.linear(tW2, tb2, false) : h.matmul(tW2) + tb2;
-        Tensor loss = logits.cross_entropy(ty);
+        Tensor logits, loss;
+        if (g_fused_layers && g_fused_head && target_is_index) {
+            loss = h.linear_cross_entropy(tW2, tb2, ty, &logits);
+        } else {
+            logits = g_fused_layers ? h.linear(tW2, tb2, false) : h.matmul(tW2) + tb2;
+            loss = logits.cross_entropy(ty);
+        }
         loss_out[0] = loss.item<float>();
         emit(logits, logits_out);
         backward(loss);
@@ -801,7 +809,8 @@ long cth_time_mlp(const float* x, long B, long I, const float* W1, const float* 
         tW2.requires_grad(true);
         tb2.requires_grad(true);
         Tensor h = g_fused_layers ? tx.linear(tW1, tb1, true) : (tx.matmul(tW1) + tb1).relu();
-        Tensor loss = (g_fused_layers ? h.linear(tW2, tb2, false) : h.matmul(tW2) + tb2).cross_entropy(ty);
+        Tensor loss = (g_fused_layers && g_fused_head) ? h.linear_cross_entropy(tW2, tb2, ty)
+                                                        : (g_fused_layers ? h.linear(tW2, tb2, false) : h.matmul(tW2) + tb2).cross_entropy(ty);
         backward(loss);                    // enqueued before the read below waits for the device
         sink = loss.item<float>();
         Tensor g1 = grad(tW1), g2 = grad(tb1), g3 = grad(tW2), g4 = grad(tb2);
@@ -1111,6 +1120,91 @@ long cth_relu_mask_fusion(const float* x, long B, long I, const float* W1, const
     }
 }
 
+// The same three-layer network with its last layer and cross entropy as one operator
+// (Tensor::linear_cross_entropy) against the two-operator form: loss, logits, the six parameter
+// gradients and the gradients of the two hidden activations, for the loss as the root of backward
+// (the gradients the one pass kept), for `loss * scale` as the root (the kept gradient of the logits
+// rescaled, the usual products); then two passes over one tape with the head (see below).  0 when
+// everything agrees within tol * max(1, largest magnitude), else 1 + the index of the first result
+// that does not (+ 100 scaled root, + 200 two passes); out[0]: the worst ratio seen, out[1] / out[2]: operator launches of one
+// step with / without the one-pass head.
+long cth_head_fusion(const float* x, long B, long I, const float* W1, const float* b1, long H1, const float* W2,
+                     const float* b2, long H2, const float* W3, const float* b3, long C, const float* labels, double tol,
+                     float scale, double* out) {
+    try {
+        prepare_backward_seed();              // made once per thread by a launch that is not part of a step
+        auto run = [&](bool head, int variant, double* launches) {
+            std::vector<std::vector<float>> results;
+            AutoDiff ctx;
+            configure(ctx);
+            AutoDiffContext::Guard guard(&ctx);
+            long xd[2] = {B, I}, w1d[2] = {I, H1}, b1d[1] = {H1}, w2d[2] = {H1, H2}, b2d[1] = {H2}, w3d[2] = {H2, C},
+                 b3d[1] = {C}, yi[1] = {B};
+            Tensor tx = make(x, xd, 2), tW1 = make(W1, w1d, 2), tb1 = make(b1, b1d, 1), tW2 = make(W2, w2d, 2),
+                   tb2 = make(b2, b2d, 1), tW3 = make(W3, w3d, 2), tb3 = make(b3, b3d, 1), ty = make(labels, yi, 1);
+            for (Tensor* t : {&tW1, &tb1, &tW2, &tb2, &tW3, &tb3}) t->requires_grad(true);
+            double bytes = 0.0, flops = 0.0, ideal = 0.0;
+            uint64_t before = 0, after = 0;
+            ctamd_counters_read(&bytes, &flops, &ideal, &before);
+            Tensor h1 = tx.linear(tW1, tb1, true);
+            Tensor h2 = h1.linear(tW2, tb2, true);
+            Tensor logits, loss;
+            if (head) {
+                loss = h2.linear_cross_entropy(tW3, tb3, ty, &logits);
+            } else {
+                logits = h2.linear(tW3, tb3, false);
+                loss = logits.cross_entropy(ty);
+            }
+            Tensor root = variant == 1 ? loss * scale : Tensor::alias(loss);
+            if (variant == 1) root = loss * scale;
+            for (int p = 0; p < (variant == 2 ? 2 : 1); ++p) backward(variant == 1 ? root : loss);
+            ctamd_counters_read(&bytes, &flops, &ideal, &after);
+            if (launches) *launches = double(after - before);
+            results.push_back({loss.item<float>()});
+            results.push_back(logits.to_vector());
+            for (Tensor* t : {&tW1, &tb1, &tW2, &tb2, &tW3, &tb3, &h1, &h2}) results.push_back(grad(*t).to_vector());
+            return results;
+        };
+        double worst = 0.0;
+        for (int variant = 0; variant < 2; ++variant) {
+            auto with = run(true, variant, variant == 0 ? out + 1 : nullptr);
+            auto without = run(false, variant, variant == 0 ? out + 2 : nullptr);
+            for (size_t i = 0; i < with.size(); ++i) {
+                if (with[i].size() != without[i].size()) return long(1 + i) + 100 * variant;
+                double big = 1.0, diff = 0.0;
+                for (size_t k = 0; k < with[i].size(); ++k) {
+                    big = std::max(big, double(std::fabs(without[i][k])));
+                    const double d = std::fabs(double(with[i][k]) - double(without[i][k]));
+                    diff = (d == d) ? std::max(diff, d) : 1e30;
+                }
+                worst = std::max(worst, diff / big);
+                if (diff > tol * big) {
+                    out[0] = worst;
+                    return long(1 + i) + 100 * variant;
+                }
+            }
+        }
+        // Two passes over one tape.  The head is ONE node: each pass adds one contribution to its
+        // inputs, so the gradients of the last layer and of h2 are exactly twice those of one pass.  (The
+        // two-operator form has a logits node in between whose gradient accumulates as well - the
+        // reference's tape never clears a node's gradient - and hands on 1 + 2 contributions.)
+        {
+            auto once = run(true, 0, nullptr);
+            auto twice = run(true, 2, nullptr);
+            for (size_t i : {size_t(6), size_t(7), size_t(9)})
+                for (size_t k = 0; k < once[i].size(); ++k)
+                    if (twice[i][k] != once[i][k] + once[i][k]) {
+                        out[0] = worst;
+                        return long(1 + i) + 200;
+                    }
+        }
+        out[0] = worst;
+        return 0;
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
 // loss_sum = CE(logits, class index), backward: dlogits = softmax - onehot.
 long cth_time_softmax_ce(const float* logits, const float* labels, long rows, long cols, int warm, int reps,
                          double* out) {
@@ -1180,7 +1274,7 @@ float cth_mnist_accuracy(const float* pred, const float* labels, long rows) {
 // sums and a tape cleared after every step; 2: as 0 with the step recorded into a DeviceGraph at
 // the first batch and replayed for every batch (with unrelated eager work between the replays).
 // Adding 4 to the mode makes each layer one fused operator and the optimiser update one launch
-// (same values).  Parameters are written back; losses_out[s] = loss of step s.  ms_out (may be null) = milliseconds for all the steps.
+// (same values); adding 8 as well, the last layer and its loss are the one-pass head.  Parameters are written back; losses_out[s] = loss of step s.  ms_out (may be null) = milliseconds for all the steps.
 long cth_mnist_train(const float* images, const float* labels, long n_images, long I, long H1, long H2, long C,
                      float* W1, float* b1, float* W2, float* b2, float* W3, float* b3, long batch, long steps,
                      float lr, int mode_bits, float* losses_out, double* ms_out) {
@@ -1191,6 +1285,7 @@ long cth_mnist_train(const float* images, const float* labels, long n_images, lo
         Tensor all_images = make(images, id, 2), all_labels = make(labels, ld, 1);
         NeuralNetwork model(W1, b1, W2, b2, W3, b3, size_t(I), size_t(H1), size_t(H2), size_t(C), lr);
         model.fused_layers = fused;
+        model.fused_head = (mode_bits & 8) != 0;
         const long num_batches = n_images / batch;
         AutoDiff autodiff;
         if (reference_tape == 1) {

@@ -100,6 +100,11 @@ def main():
         # what the tape calls for a layer whose bias wants its gradient: both in one call (one launch while batch <= 512)
         mmcs = lambda a, b, c, sums, m, n, k: call("ctamd_matmul_colsum_f32", P(a), a.stride(0), a.stride(1), P(b), b.stride(0), b.stride(1),
                                                    P(c), P(sums), m, n, k, S)
+        # the last layer, its cross entropy and the three gradients that leave them, in one pass over h
+        pair = torch.zeros(2, device="cuda")
+        row("z, loss, dz, dh, gW2, gb2 in one pass over h (the classifier head)",
+            lambda: call("ctamd_linear_ce_head_f32", P(h), P(W2), P(b2), P(labels), P(pair), P(status), P(z), P(dz), P(dh), 1, P(gW2), P(gb2),
+                         batch, H, Cn, S), flops=6.0 * batch * H * Cn)
         row("gW2 and gb2 in one call", lambda: mmcs(h.t(), dz, gW2, gb2, H, Cn, batch), flops=2.0 * batch * H * Cn)
         row("gW1 and gb1 in one call", lambda: mmcs(x.t(), dh, gW1, gb1, I, H, batch), flops=2.0 * batch * H * I)
     if args.only_mlp:

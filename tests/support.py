@@ -1102,6 +1102,21 @@ class HostLayer(Reference):
         """mlp_step builds each layer with Tensor::linear (matmul + bias + ReLU as one operator)."""
         self.cdll.cth_set_fused_layers(int(on))
 
+    def set_fused_head(self, on):
+        """With fused layers: the last layer and its class-index cross entropy as one operator
+        (Tensor::linear_cross_entropy) in mlp_step and time_mlp."""
+        self.cdll.cth_set_fused_head(int(on))
+
+    def head_fusion(self, x, W1, b1, W2, b2, W3, b3, labels, tol, scale=3.0):
+        """cth_head_fusion: (rc, worst ratio, launches with the one-pass head, without)."""
+        x, W1, b1, W2, b2, W3, b3, labels = map(f32, (x, W1, b1, W2, b2, W3, b3, labels))
+        out = (C.c_double * 3)(0, 0, 0)
+        self.cdll.cth_head_fusion.restype = C.c_long
+        rc = self.cdll.cth_head_fusion(fp(x), C.c_long(x.shape[0]), C.c_long(x.shape[1]), fp(W1), fp(b1), C.c_long(W1.shape[1]), fp(W2),
+                                       fp(b2), C.c_long(W2.shape[1]), fp(W3), fp(b3), C.c_long(W3.shape[1]), fp(labels),
+                                       C.c_double(tol), C.c_float(scale), out)
+        return rc, out[0], out[1], out[2]
+
     def set_bias_grad_with_weight_grad(self, on):
         """The bias gradient of a fused layer with its weight gradient (the default) or on its own."""
         self.cdll.cth_set_bias_grad_with_weight_grad(int(on))

@@ -535,3 +535,47 @@ def test_relu_mask_rides_in_the_products_of_backward(oracle, host, batch):
     assert rc == 0, rc
     print(f"  kernels launched by backward: {int(out[0])} with the mask in the products, {int(out[1])} without")
     assert out[0] == out[1] - 2
+
+
+@pytest.mark.parametrize("batch", [8, 300, 4096])
+def test_the_one_pass_head_against_the_two_operator_form(oracle, host, batch):
+    """Tensor::linear_cross_entropy (logits, loss and the gradients of the last layer formed in one
+    pass over the hidden activations) against x.linear(W, b).cross_entropy(labels) in a three-layer
+    network: loss, logits, the six parameter gradients and the gradients of both hidden activations
+    (the second of which the one pass leaves at the ReLU layer's pre-activation, so the tape forms it on
+    request) within the MatMul bound - the head adds its products in another order - for the loss as
+    root and for a scaled root (the kept gradient of the logits rescaled); two passes over one tape give
+    the head's inputs exactly twice one pass's gradients; and a step is three operator launches shorter."""
+    print("case one-pass head", batch, flush=True)
+    I, H1, H2, Cn = 200, 96, 72, 10
+    x = oracle.uniform((batch, I), 741, 0, 1)
+    W1, b1 = oracle.uniform((I, H1), 742, -0.1, 0.1), oracle.uniform((H1,), 743, -0.1, 0.1)
+    W2, b2 = oracle.uniform((H1, H2), 744, -0.15, 0.15), oracle.uniform((H2,), 745, -0.1, 0.1)
+    W3, b3 = oracle.uniform((H2, Cn), 746, -0.2, 0.2), oracle.uniform((Cn,), 747, -0.1, 0.1)
+    labels = oracle.ints((batch,), 748, Cn)
+    rc, worst, with_head, without = host.head_fusion(x, W1, b1, W2, b2, W3, b3, labels, 2e-5)
+    print(f"  worst difference / largest magnitude {worst:.2e}; operator launches of a step: {int(with_head)} with the head, {int(without)} without")
+    assert rc == 0, (rc, worst)
+    assert with_head <= without - 3
+
+
+def test_mlp_step_with_the_one_pass_head_against_the_oracle(oracle, host, golden):
+    """configs[2]'s step with fused layers and the one-pass head: loss, logits and the four gradients
+    against the CPU oracle at the bar of the other forms of the step."""
+    print("case mlp step one-pass head", flush=True)
+    g = golden("configs")
+    lab = g["mlp_lab"]
+    oh = np.zeros((lab.size, 10), F)
+    oh[np.arange(lab.size), lab.astype(int)] = 1
+    args = (g["mlp_x"], g["mlp_W1"], g["mlp_b1"], g["mlp_W2"], g["mlp_b2"])
+    names = ["loss", "logits", "gW1", "gb1", "gW2", "gb2"]
+    want = oracle.mlp_step(*args, oh, False)
+    host.set_fused_layers(True)
+    host.set_fused_head(True)
+    try:
+        got = host.mlp_step(*args, lab, True)
+    finally:
+        host.set_fused_head(False)
+        host.set_fused_layers(False)
+    for n, a, b in zip(names, got, want):
+        assert np.abs(a - b).max() <= 1e-4 * max(1.0, np.abs(b).max()), n

@@ -206,3 +206,21 @@ def test_demo_with_a_recorded_step(host, tmp_path):
     rc2, l2, a2, _ = host.mnist_demo(str(tmp_path), epochs=3, lr=1e-3, reference_tape=2)
     assert rc1 == rc2 == 12
     assert same_bits(l1, l2) and same_bits(a1, a2)
+
+
+@pytest.mark.parametrize("tag", ["s", "m"])
+def test_training_with_the_one_pass_head(host, golden, tag):
+    """The training loop with the last layer and its loss as the one-pass head (class indices instead of
+    the one-hot matrix, products added in another order): losses and trained parameters agree with the
+    operator-by-operator run to the reduction bar compounded over the steps, eagerly and as a recorded
+    step."""
+    print("case training with the one-pass head", tag, flush=True)
+    g = golden("mnist")
+    batch, steps = (int(v) for v in g[tag + "_cfg"])
+    params = [g["%s_p%d" % (tag, k)] for k in range(6)]
+    plain_l, plain_p = host.mnist_train(g[tag + "_x"], g[tag + "_y"], params, batch, steps, 0.01, reference_tape=0)
+    for mode in (0, 2):
+        head_l, head_p = host.mnist_train(g[tag + "_x"], g[tag + "_y"], params, batch, steps, 0.01, reference_tape=mode + 12)
+        assert np.abs(head_l - plain_l).max() <= 1e-4 * np.abs(plain_l).max(), mode
+        for a, b in zip(head_p, plain_p):
+            assert np.abs(a - b).max() <= 1e-4 * max(1.0, np.abs(b).max()), mode
