@@ -10,7 +10,7 @@
 // A product with ten output columns cannot use the matrix cores (a 32 x 32 tile would be two thirds
 // idle); everything here is fp32 fused multiply-adds on the vector units, h read once, dh written once.
 //
-// A wave takes four rows at a time.  Lane l holds h[row][4l .. 4l+3] and the four rows of W those k
+// A wave takes four rows at a time (two when there are more than 13 classes).  Lane l holds h[row][4l .. 4l+3] and the four rows of W those k
 // meet (W stays in registers for all rows); the 4 x N partial logits go round the wave with the
 // halving exchange of the narrow products (lane r * N + c ends up with z[r][c]); the N lanes of a row
 // form its softmax by lane reads; dz comes back to every lane through scalar lane reads and meets h
@@ -26,9 +26,11 @@ namespace {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-constexpr int kHeadThreads = 512;          // eight waves: two per SIMD, whose exchanges and lane reads hide each other's latency
-constexpr int kHeadWaves = kHeadThreads / 64;
-constexpr int kHeadRows = 4;              // rows a wave works on at a time
+// waves per block: eight (two per SIMD, whose exchanges and lane reads hide each other's latency) while
+// the kernel fits 256 registers per lane at that occupancy, four for the widest heads
+constexpr int head_waves(int n) { return n <= 13 ? 8 : 4; }
+// rows a wave works on at a time (their partial logits share one exchange): four, two for the widest heads
+constexpr int head_rows(int n) { return n <= 13 ? 4 : 2; }
 constexpr int kHeadMaxBlocks = 256;       // partial results kept per launch
 constexpr int kHeadMaxH = 256;
 
@@ -42,7 +44,7 @@ struct HeadArgs {
     float* dh;               // [B, H] (may be null)
     float* part;             // scratch: per block [H * N] + [N] floats, then per block {double loss, double bad}
     int B, H;
-    int turns;               // groups of four rows per wave
+    int turns;               // groups of rows per wave
     int mask;                // dh is multiplied by (h > 0 ? 1 : 0)
     int fast;                // single-precision exponential and e * (1 / s), as the row kernels' default mode
 };
@@ -69,8 +71,10 @@ __device__ __forceinline__ void wave_sums_step_(float (&v)[P], int lane) {
 __host__ __device__ inline size_t head_part_floats(int H, int N) { return size_t(H) * N + N; }
 
 template <int N>
-__global__ __launch_bounds__(kHeadThreads) void head_kernel(HeadArgs a) {
-    constexpr int R = kHeadRows;
+__global__ __launch_bounds__(head_waves(N) * 64) void head_kernel(HeadArgs a) {
+    constexpr int kHeadWaves = head_waves(N);
+    constexpr int kHeadThreads = kHeadWaves * 64;
+    constexpr int R = head_rows(N);
     constexpr int P = pow2_at_least_(R * N);
     constexpr int kLanesPerValue = 64 / P;
     __shared__ __attribute__((aligned(16))) float s_wt[N][kHeadMaxH];     // W transposed, zeros behind H
@@ -171,7 +175,7 @@ __global__ __launch_bounds__(kHeadThreads) void head_kernel(HeadArgs a) {
             a.dz[size_t(row_mine) * N + c_mine] = dz_mine;
         }
         gb_mine += dz_mine;
-        // dz of the four rows to every lane (scalar lane reads), then dh and the share of gW
+        // dz of the rows to every lane (scalar lane reads), then dh and the share of gW
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             float d[N];
@@ -316,7 +320,7 @@ __global__ __launch_bounds__(kFoldThreads) void head_fold_kernel(const float* __
 
 template <int N>
 int launch_head(const HeadArgs& a, int blocks, hipStream_t s) {
-    hipLaunchKernelGGL(head_kernel<N>, dim3(unsigned(blocks)), dim3(kHeadThreads), 0, s, a);
+    hipLaunchKernelGGL(head_kernel<N>, dim3(unsigned(blocks)), dim3(head_waves(N) * 64), 0, s, a);
     return launched("ctamd_linear_ce_head_f32");
 }
 
@@ -341,13 +345,15 @@ extern "C" int ctamd_linear_ce_head_f32(const float* h, const float* w, const fl
     float* part = use.ptr();
     if (!part) return CTAMD_EINVAL;
     const int B = int(batch), H = int(hidden), N = int(classes);
-    const int groups = (B + kHeadRows - 1) / kHeadRows;                 // groups of four rows
+    const int rows_at_a_time = head_rows(N);
+    const int groups = (B + rows_at_a_time - 1) / rows_at_a_time;       // groups of rows a wave takes together
+    const int waves = head_waves(N);
     const int cus = compute_units() > 0 ? compute_units() : 256;
-    int blocks = (groups + kHeadWaves - 1) / kHeadWaves;
+    int blocks = (groups + waves - 1) / waves;
     const int cap = cus < kHeadMaxBlocks ? cus : kHeadMaxBlocks;
     if (blocks > cap) blocks = cap;
-    const int turns = (groups + blocks * kHeadWaves - 1) / (blocks * kHeadWaves);
-    blocks = (groups + turns * kHeadWaves - 1) / (turns * kHeadWaves);
+    const int turns = (groups + blocks * waves - 1) / (blocks * waves);
+    blocks = (groups + turns * waves - 1) / (turns * waves);
     if ((head_part_floats(H, N) + 4) * size_t(blocks) + 2 > kScratchFloats) return fail(CTAMD_ERANGE, "%s: does not fit the device scratch", __func__);
     HeadArgs a;
     a.h = h; a.w = w; a.bias = bias; a.labels = labels; a.z = z; a.dz = dz; a.dh = dh; a.part = part;
