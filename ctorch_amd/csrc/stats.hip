@@ -496,6 +496,7 @@ struct ColPlan {
     bool vec;
     dim3 grid;
 };
+constexpr size_t kMaxGridZ = 65535;
 bool plan_cols(const float* x, const void* other, size_t outer, size_t len, size_t inner, ColPlan& p) {
     const size_t target = size_t(compute_units() > 0 ? compute_units() : 256) * 4;
     p.vec = inner % 4 == 0 && aligned16(x) && (!other || aligned16(other));
@@ -517,10 +518,13 @@ bool plan_cols(const float* x, const void* other, size_t outer, size_t len, size
     p.rows_per_chunk = (len + chunks - 1) / chunks;
     chunks = (len + p.rows_per_chunk - 1) / p.rows_per_chunk;
     p.chunks = unsigned(chunks);
-    if (strips > 0x7fffffffu || chunks > 65535 || outer > 65535) return false;
-    p.grid = dim3(unsigned(strips), unsigned(chunks), unsigned(outer));
+    if (strips > 0x7fffffffu || chunks > 65535) return false;
+    // the grid's third dimension holds at most kMaxGridZ slabs: a launch per run of that many (p.grid.z is the first run's)
+    p.grid = dim3(unsigned(strips), unsigned(chunks), unsigned(outer < kMaxGridZ ? outer : kMaxGridZ));
     return true;
 }
+template <class T>
+T* at_offset(T* p, size_t n) { return p ? p + n : nullptr; }
 
 template <int KIND>
 int run_forward(const char* name, const float* x, float* out, int32_t* index, float* mean_out, size_t outer, size_t len,
@@ -554,12 +558,17 @@ int run_forward(const char* name, const float* x, float* out, int32_t* index, fl
         p.rows_per_chunk = len;
         p.grid.y = 1;
     }
-    if (p.vec)
-        hipLaunchKernelGGL((reduce_cols_kernel<KIND, 4>), p.grid, dim3(kThreads), 0, s, x, parts, out, index, mean_out, len, inner,
-                           p.rows_per_chunk, p.chunks, p.tx_count, ddof);
-    else
-        hipLaunchKernelGGL((reduce_cols_kernel<KIND, 1>), p.grid, dim3(kThreads), 0, s, x, parts, out, index, mean_out, len, inner,
-                           p.rows_per_chunk, p.chunks, p.tx_count, ddof);
+    for (size_t o0 = 0; o0 < outer; o0 += kMaxGridZ) {
+        p.grid.z = unsigned(outer - o0 < kMaxGridZ ? outer - o0 : kMaxGridZ);
+        const float* xs = x + o0 * len * inner;
+        Part* ps = parts + o0 * p.chunks * inner;
+        if (p.vec)
+            hipLaunchKernelGGL((reduce_cols_kernel<KIND, 4>), p.grid, dim3(kThreads), 0, s, xs, ps, at_offset(out, o0 * inner),
+                               at_offset(index, o0 * inner), at_offset(mean_out, o0 * inner), len, inner, p.rows_per_chunk, p.chunks, p.tx_count, ddof);
+        else
+            hipLaunchKernelGGL((reduce_cols_kernel<KIND, 1>), p.grid, dim3(kThreads), 0, s, xs, ps, at_offset(out, o0 * inner),
+                               at_offset(index, o0 * inner), at_offset(mean_out, o0 * inner), len, inner, p.rows_per_chunk, p.chunks, p.tx_count, ddof);
+    }
     int rc = launched(name);
     if (rc || p.chunks == 1) return rc;
     const size_t results = outer * inner;
@@ -585,12 +594,17 @@ int run_backward(const char* name, const float* x, const float* y, const int32_t
     }
     ColPlan p;
     if (!plan_cols(reads_x<KIND>() ? x : dx, dx, outer, len, inner, p)) return fail(CTAMD_ERANGE, "%s: shape exceeds the launch grid", name);
-    if (p.vec)
-        hipLaunchKernelGGL((reduce_cols_backward_kernel<KIND, 4>), p.grid, dim3(kThreads), 0, s, x, y, index, mean, g, dx, len, inner,
-                           p.rows_per_chunk, p.tx_count, ddof);
-    else
-        hipLaunchKernelGGL((reduce_cols_backward_kernel<KIND, 1>), p.grid, dim3(kThreads), 0, s, x, y, index, mean, g, dx, len, inner,
-                           p.rows_per_chunk, p.tx_count, ddof);
+    for (size_t o0 = 0; o0 < outer; o0 += kMaxGridZ) {
+        p.grid.z = unsigned(outer - o0 < kMaxGridZ ? outer - o0 : kMaxGridZ);
+        if (p.vec)
+            hipLaunchKernelGGL((reduce_cols_backward_kernel<KIND, 4>), p.grid, dim3(kThreads), 0, s, at_offset(x, o0 * len * inner),
+                               at_offset(y, o0 * inner), at_offset(index, o0 * inner), at_offset(mean, o0 * inner), at_offset(g, o0 * inner),
+                               dx + o0 * len * inner, len, inner, p.rows_per_chunk, p.tx_count, ddof);
+        else
+            hipLaunchKernelGGL((reduce_cols_backward_kernel<KIND, 1>), p.grid, dim3(kThreads), 0, s, at_offset(x, o0 * len * inner),
+                               at_offset(y, o0 * inner), at_offset(index, o0 * inner), at_offset(mean, o0 * inner), at_offset(g, o0 * inner),
+                               dx + o0 * len * inner, len, inner, p.rows_per_chunk, p.tx_count, ddof);
+    }
     return launched(name);
 }
 

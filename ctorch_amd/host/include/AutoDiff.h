@@ -86,6 +86,7 @@ class AutoDiff {
         // the pre-activation and the layer's own mask launch is skipped.  get_grad() forms the
         // gradient of the output itself from the consumer when somebody asks for it.
         Node* grad_premasked_by = nullptr;
+        std::unique_ptr<Tensor> unmasked_grad;  // with grad_premasked_by: the gradient of the output, once somebody asked for it
         std::unique_ptr<Tensor> shared_term;   // backward only: a factor that several inputs' gradients use
         std::vector<Tensor> input_grads;       // backward only: gradients of all inputs, computed together
         std::shared_ptr<OpPayload> payload;
@@ -139,6 +140,7 @@ class AutoDiff {
     std::mutex records_mutex;
     std::unordered_map<size_t, std::unique_ptr<Node>> id_to_node;
     std::unordered_map<size_t, Pending> pending_;
+    std::unordered_set<Node*> premasked_;    // nodes whose grad_premasked_by is set (what the next backward() has to bring back)
     bool retain_graph_ = false;
     BroadcastGrad broadcast_grad_ = BroadcastGrad::kColumnSum;
     LeafValues leaf_values_ = LeafValues::kLive;

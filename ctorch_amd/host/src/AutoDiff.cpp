@@ -74,6 +74,23 @@ void AutoDiff::zero_grad(Tensor& t) {
         n->grad_plus_zero = false;
         n->grad_assigned = false;
         n->grad_premasked_by = nullptr;
+        n->unmasked_grad.reset();
+        // A layer below whose gradient this node's backward left at the pre-activation: the gradient of
+        // that layer's output could only be formed from the gradient just dropped, so it goes as well
+        // (what is left would otherwise be read as the output's gradient by a later pass).
+        for (auto it = premasked_.begin(); it != premasked_.end();) {
+            Node* below = *it;
+            if (below->grad_premasked_by == n) {
+                below->grad.reset();
+                below->grad_plus_zero = false;
+                below->grad_premasked_by = nullptr;
+                below->unmasked_grad.reset();
+                it = premasked_.erase(it);
+            } else {
+                ++it;
+            }
+        }
+        premasked_.erase(n);
     }
 }
 
@@ -98,10 +115,12 @@ Tensor AutoDiff::get_grad(const Tensor* t) {
         // the consumer's product without the mask, formed now
         Node* by = n->grad_premasked_by;
         if (!by->grad) return Tensor(ShapeTag{}, t->shape(), t->dtype(), t->device());
-        AutoDiffContext::Guard guard(nullptr);          // nothing below is taped
-        Tensor whole = input_gradient(by, n->tensor_id, 0, *by->grad);
-        by->shared_term.reset();
-        return whole;                                   // sums of products from +0: no "0 +" pending
+        if (!n->unmasked_grad) {                        // one product, kept for the next reader
+            AutoDiffContext::Guard guard(nullptr);      // nothing below is taped
+            n->unmasked_grad = std::make_unique<Tensor>(input_gradient(by, n->tensor_id, 0, *by->grad));
+            by->shared_term.reset();
+        }
+        return Tensor::share(*n->unmasked_grad);        // sums of products from +0: no "0 +" pending
     }
     if (n && n->requires_grad && n->grad) {
         // the pending "0 +" (one pass, once); a gradient known to hold no -0 needs none.  The
@@ -150,6 +169,7 @@ void AutoDiff::commit_record(Tensor& output) {
 
 void AutoDiff::clear_graph() {
     std::lock_guard<std::mutex> lock(records_mutex);
+    premasked_.clear();
     id_to_node.clear();
     pending_.clear();
 }
@@ -493,17 +513,22 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
     // A gradient that an earlier pass left at a layer's pre-activation is brought back to the
     // gradient of the layer's output before anything is added to it (a pass over a tape that was
     // not cleared adds to what the nodes hold, as the reference's does).
-    for (auto& entry : id_to_node) {
-        Node* n = entry.second.get();
-        if (!n->grad_premasked_by) continue;
+    for (Node* n : premasked_) {
         Node* by = n->grad_premasked_by;
+        if (!by) continue;
         n->grad_premasked_by = nullptr;
         if (n->grad && by->grad) {
-            n->grad = std::make_unique<Tensor>(input_gradient(by, n->tensor_id, 0, *by->grad));
+            n->grad = n->unmasked_grad ? std::move(n->unmasked_grad)
+                                       : std::make_unique<Tensor>(input_gradient(by, n->tensor_id, 0, *by->grad));
             n->grad_plus_zero = true;
             by->shared_term.reset();
+        } else {
+            n->grad.reset();                     // its source is gone: nothing to bring back
+            n->grad_plus_zero = false;
         }
+        n->unmasked_grad.reset();
     }
+    premasked_.clear();
     root_node->grad = std::make_unique<Tensor>(adjust_grad_shape(grad_output, root.sizes()));
     root_node->grad_plus_zero = seed_plus_zero_;
     root_node->grad_assigned = !adjust_adds_to_zero_;     // a seed taken as it is stays as it is (:1126)
@@ -616,6 +641,7 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
                     in->grad = std::make_unique<Tensor>(MatMulReluMask_AMD_kernel(gz, Tensor::view_t(*wn->tensor), *in->tensor));
                     in->grad_plus_zero = false;          // g * 0 may be -0
                     in->grad_premasked_by = node;
+                    premasked_.insert(in);
                     continue;
                 }
             }
@@ -628,6 +654,7 @@ void AutoDiff::backward(Tensor& root, Tensor grad_output) {
                     in->grad = std::make_unique<Tensor>(Tensor::alias(kept->dh));
                     in->grad_plus_zero = false;
                     in->grad_premasked_by = node;
+                    premasked_.insert(in);
                     continue;
                 }
             }

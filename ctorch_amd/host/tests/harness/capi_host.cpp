@@ -1120,6 +1120,58 @@ long cth_relu_mask_fusion(const float* x, long B, long I, const float* W1, const
     }
 }
 
+// A hidden ReLU layer whose gradient the tape holds at the pre-activation (the mask rode in the
+// consumer's product): reading the gradient of the layer's output forms it once (the second read
+// launches nothing and returns the same bits); clearing the consumer's gradient takes the hidden
+// layer's with it (it reads as zeros, as any cleared gradient); a further backward pass over the tape
+// then gives the gradients of a first pass again.  0, or the number of the first check that failed.
+long cth_premasked_grad_reads(const float* x, long B, long I, const float* W1, const float* b1, long H, const float* W2,
+                              const float* b2, long C, const float* labels) {
+    try {
+        prepare_backward_seed();
+        AutoDiff ctx;
+        configure(ctx);
+        AutoDiffContext::Guard guard(&ctx);
+        long xd[2] = {B, I}, w1d[2] = {I, H}, b1d[1] = {H}, w2d[2] = {H, C}, b2d[1] = {C}, yi[1] = {B};
+        Tensor tx = make(x, xd, 2), tW1 = make(W1, w1d, 2), tb1 = make(b1, b1d, 1), tW2 = make(W2, w2d, 2), tb2 = make(b2, b2d, 1),
+               ty = make(labels, yi, 1);
+        for (Tensor* t : {&tW1, &tb1, &tW2, &tb2}) t->requires_grad(true);
+        Tensor h = tx.linear(tW1, tb1, true);
+        Tensor logits = h.linear(tW2, tb2, false);
+        Tensor loss = logits.cross_entropy(ty);
+        backward(loss);
+        auto launches = [] {
+            double a = 0, b = 0, c = 0;
+            uint64_t n = 0;
+            ctamd_counters_read(&a, &b, &c, &n);
+            return n;
+        };
+        const std::vector<float> gw1 = grad(tW1).to_vector();
+        const uint64_t n0 = launches();
+        const std::vector<float> first = grad(h).to_vector();
+        const uint64_t n1 = launches();
+        const std::vector<float> second = grad(h).to_vector();
+        const uint64_t n2 = launches();
+        if (n1 == n0) return 1;                                   // the first read has to form the product
+        if (n2 != n1) return 2;                                   // the second must not
+        if (first != second) return 3;
+        bool any = false;
+        for (float v : first) any = any || v != 0.0f;
+        if (!any) return 4;
+        ctx.zero_grad(logits);
+        for (float v : grad(h).to_vector())
+            if (v != 0.0f) return 5;                              // its source is gone
+        for (Tensor* t : {&tW1, &tb1, &tW2, &tb2}) ctx.zero_grad(*t);
+        ctx.zero_grad(loss);
+        backward(loss);                                           // over the same tape: as a first pass
+        if (grad(tW1).to_vector() != gw1) return 6;
+        if (grad(h).to_vector() != first) return 7;
+        return 0;
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
 // The same three-layer network with its last layer and cross entropy as one operator
 // (Tensor::linear_cross_entropy) against the two-operator form: loss, logits, the six parameter
 // gradients and the gradients of the two hidden activations, for the loss as the root of backward

@@ -178,9 +178,8 @@ int ctamd_mae_f32(const float* a, const float* b, float* out, size_t n, void* st
  * It has no counterpart in the reference.  The per-block partial sums live in a 16 KiB array that is
  * part of the library's device image (one copy per GPU, held until the process ends) instead of the
  * scratch buffer ctamd_init() allocates; the call allocates and frees nothing.  Same kernels, same
- * grid and therefore the same bits as ctamd_dot_f32.  n above CTAMD_DOT_STATIC_MAX_N (the reference's
- * kernel counts elements in an int, Dot_BASIC_kernel.cpp:31) is refused with CTAMD_ERANGE and nothing
- * is launched.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two
+ * grid and therefore the same bits as ctamd_dot_f32.  n above CTAMD_DOT_STATIC_MAX_N (2^31 - 1,
+ * this entry point's stated maximum) is refused with CTAMD_ERANGE and nothing is launched.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two
  * streams, two host threads) race; calls on one stream are ordered.  Nothing needs clearing between
  * calls - the fold launch reads only the partials its own first launch wrote. */
 #define CTAMD_DOT_STATIC_MAX_N ((size_t)2147483647)

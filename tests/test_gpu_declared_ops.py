@@ -122,7 +122,8 @@ def reduce_dim_bwd(kind, x, y, index, mean, g, outer, length, inner, ddof=1):
 
 
 SHAPES = [(1, 1, 1), (1, 37, 1), (1, 4099, 1), (1, (1 << 20) + 5, 1), (7, 33, 1), (300, 1000, 1), (5, 8192, 1), (2048, 64, 1),
-          (1, 9, 6), (1, 700, 10), (1, 4096, 256), (1, 130, 4100), (3, 17, 5), (2, 300, 64), (1, 1, 9), (4, 1, 1)]
+          (1, 9, 6), (1, 700, 10), (1, 4096, 256), (1, 130, 4100), (3, 17, 5), (2, 300, 64), (1, 1, 9), (4, 1, 1),
+          (70000, 6, 8), (66000, 7, 3)]          # more slabs than a launch grid's third dimension holds
 
 
 @pytest.mark.parametrize("shape", SHAPES)
@@ -157,7 +158,8 @@ def test_reductions_along_an_axis(oracle, shape):
                 assert np.all(np.abs(gm - x64.mean(axis=1)) <= 1e-6 * np.abs(x64).mean(axis=1) + 1e-30)
 
 
-@pytest.mark.parametrize("shape", [(1, 37, 1), (7, 33, 1), (3, 5000, 1), (1, 9, 6), (1, 700, 10), (1, 130, 4100), (3, 17, 5), (2, 300, 64), (1, 70001, 1)])
+@pytest.mark.parametrize("shape", [(1, 37, 1), (7, 33, 1), (3, 5000, 1), (1, 9, 6), (1, 700, 10), (1, 130, 4100), (3, 17, 5), (2, 300, 64), (1, 70001, 1),
+                                   (70000, 6, 8)])
 def test_reduction_gradients_bit_exact(oracle, shape):
     outer, length, inner = shape
     print("case reduce_dim backward", shape, flush=True)

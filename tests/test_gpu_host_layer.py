@@ -579,3 +579,22 @@ def test_mlp_step_with_the_one_pass_head_against_the_oracle(oracle, host, golden
         host.set_fused_layers(False)
     for n, a, b in zip(names, got, want):
         assert np.abs(a - b).max() <= 1e-4 * max(1.0, np.abs(b).max()), n
+
+
+def test_reading_a_gradient_the_tape_holds_at_a_pre_activation(oracle, host):
+    """The gradient of a hidden ReLU layer's output, which the tape keeps multiplied by the layer's mask:
+    formed once on the first read, gone with the consumer's gradient when that is cleared, and back
+    with the next pass over the tape."""
+    print("case premasked gradient reads", flush=True)
+    import ctypes as C
+    B, I, H, Cn = 64, 40, 32, 10
+    x = oracle.uniform((B, I), 841, 0, 1)
+    W1, b1 = oracle.uniform((I, H), 842, -0.3, 0.3), oracle.uniform((H,), 843, -0.1, 0.1)
+    W2, b2 = oracle.uniform((H, Cn), 844, -0.3, 0.3), oracle.uniform((Cn,), 845, -0.1, 0.1)
+    labels = oracle.ints((B,), 846, Cn)
+    FP = C.POINTER(C.c_float)
+    fp = lambda a: np.ascontiguousarray(a, dtype=np.float32).ctypes.data_as(FP)
+    L = C.c_long
+    host.cdll.cth_premasked_grad_reads.restype = C.c_long
+    rc = host.cdll.cth_premasked_grad_reads(fp(x), L(B), L(I), fp(W1), fp(b1), L(H), fp(W2), fp(b2), L(Cn), fp(labels))
+    assert rc == 0, rc

@@ -17,18 +17,34 @@ def _dot(G, name, a, b):
     return G.host(out).copy()
 
 
+def _free_device_bytes(lib):
+    """hipMemGetInfo of the HIP runtime the library itself is bound to (its symbols are reachable
+    through the library's handle): what any allocation by the call, torch's or hipMalloc's, would lower."""
+    fn = lib.hipMemGetInfo
+    fn.argtypes, fn.restype = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)], C.c_int
+    free, total = C.c_size_t(0), C.c_size_t(0)
+    assert fn(C.byref(free), C.byref(total)) == 0
+    return free.value
+
+
 def test_static_dot_equals_dot_on_two_calls_in_a_row():
     import gpu_support as G
     import torch
     from support import Oracle
     o = Oracle()
-    G.lib()
+    lib = G.lib()
     sizes = [(1 << 22) + 3, 4099]            # 1025 blocks with a ragged tail, then a 2-block input
     for k, n in enumerate(sizes):
         a_h, b_h = o.uniform((n,), 211 + 10 * k, -1, 1), o.uniform((n,), 212 + 10 * k, -1, 1)
         a, b = G.dev(a_h), G.dev(b_h)
-        before = torch.cuda.memory_allocated()
-        got = _dot(G, "ctamd_dot_static_f32", a, b)
+        out = torch.full((1,), float("nan"), device=G.DEV)
+        torch.cuda.synchronize()
+        before, before_torch = _free_device_bytes(lib), torch.cuda.memory_reserved()
+        G.call("ctamd_dot_static_f32", G.ptr(a), G.ptr(b), G.ptr(out), a.numel(), G.stream())
+        torch.cuda.synchronize()
+        # the call took no device memory: neither from the driver nor from torch's pool
+        assert _free_device_bytes(lib) == before and torch.cuda.memory_reserved() == before_torch
+        got = G.host(out).copy()
         want = _dot(G, "ctamd_dot_f32", a, b)
         assert got.view(np.uint32)[0] == want.view(np.uint32)[0], (n, got, want)
         # and both within the reduction bar of an fp64 dot product
@@ -37,7 +53,6 @@ def test_static_dot_equals_dot_on_two_calls_in_a_row():
         assert abs(float(got[0]) - exact) <= 1e-5 * scale
         # the oracle's sequential fp32 dot product is inside the same bar
         assert abs(float(o.dot(a_h, b_h)) - float(got[0])) <= 2e-5 * scale
-        assert torch.cuda.memory_allocated() >= before    # (outputs only; the call itself takes no memory)
 
 
 def test_static_dot_edges_and_limit():
