@@ -619,6 +619,152 @@ __global__ __launch_bounds__(1024) void row_stream_vec_kernel(Args a) {
     }
 }
 
+// Rows of more than 32768 and at most 65536 columns (128-bit accesses): the two sweeps of the kernel
+// above with the operand that both sweeps need kept on the chip between them - sixteen 128-bit words
+// per thread, eight in registers and eight in LDS (128 KiB per block; one block of 1024 threads per CU)
+// - so that it is read from memory once:
+//   softmax, log-softmax        x kept:  8 B/elem moved instead of 12
+//   softmax gradient            y kept: 16 instead of 20 (g, which the first sweep needs for the row's
+//                                       dot product and the second for the result, is read twice)
+//   log-softmax gradient        g kept: 12 instead of 16
+// The arithmetic, and so every bit of the results, is the kernel's above.
+constexpr int kKeepRegs = 8, kKeepLds = 8;
+constexpr unsigned kKeepVectors = (kKeepRegs + kKeepLds) * 1024;
+template <int MODE_>
+__global__ __launch_bounds__(1024) void row_keep_kernel(Args a) {
+    constexpr int THREADS = 1024;
+    constexpr int MODE = base_mode(MODE_);
+    constexpr bool kFastOut = fast_out(MODE_);
+    static_assert(MODE == kSoftmax || MODE == kSoftmaxBwd || MODE == kLogSoftmaxFast || MODE == kLogSoftmaxBwd,
+                  "only the modes that write a row-shaped result");
+    static_assert(kKeepRegs % 2 == 0 && kKeepLds % 2 == 0, "words are taken two at a time");
+    extern __shared__ v4f s_keep[];                 // [kKeepLds][THREADS]
+    __shared__ uint64_t s_exp2[32];
+    __shared__ float s_f[2][THREADS / 64 + 1];
+    stage_exp_table(s_exp2);
+    const unsigned n4 = unsigned(a.cols >> 2);      // at most kKeepVectors
+    const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    v4f* const mine = s_keep + threadIdx.x;
+    for (size_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
+        const v4f* __restrict__ xr = reinterpret_cast<const v4f*>(a.x + row * a.cols);
+        const v4f* __restrict__ gr = reinterpret_cast<const v4f*>(a.t + row * a.cols);
+        v4f* __restrict__ outr = reinterpret_cast<v4f*>(a.out + row * a.cols);
+        v4f keep[kKeepRegs];
+        // A sweep visits the row's words two at a time: first the words kept in registers (unrolled:
+        // their register numbers must be constants), then - in a loop - the words kept in LDS.
+        // `first(i0, i1, ok0, ok1, slot0, slot1)` is handed two word indices, whether they lie inside the
+        // row, and where the kept copies live.
+        auto sweep = [&](auto&& visit) {
+#pragma unroll
+            for (int u = 0; u < kKeepRegs; u += 2) {
+                const unsigned i0 = threadIdx.x + unsigned(u) * THREADS, i1 = i0 + THREADS;
+                visit(i0, i1, i0 < n4, i1 < n4, keep[u], keep[u + 1]);
+                __builtin_amdgcn_sched_barrier(0);          // the next pair's loads stay behind this pair's work
+            }
+#pragma unroll 1
+            for (int u = 0; u < kKeepLds; u += 2) {
+                const unsigned i0 = threadIdx.x + unsigned(kKeepRegs + u) * THREADS, i1 = i0 + THREADS;
+                if (i0 >= n4) break;
+                visit(i0, i1, true, i1 < n4, mine[u * THREADS], mine[(u + 1) * THREADS]);
+            }
+        };
+        if (MODE == kSoftmaxBwd) {
+            // d = sum g * y with y left on the chip; then dx = y * (g - d) from the kept y and g read again
+            float d0 = 0.0f, d1 = 0.0f;
+            sweep([&](unsigned i0, unsigned i1, bool ok0, bool ok1, v4f& k0, v4f& k1) {
+                const v4f y0 = ok0 ? xr[i0] : zero, y1 = ok1 ? xr[i1] : zero;
+                const v4f g0 = ok0 ? gr[i0] : zero, g1 = ok1 ? gr[i1] : zero;
+                d0 += g0[0] * y0[0] + g0[1] * y0[1];
+                d1 += g0[2] * y0[2] + g0[3] * y0[3];
+                d0 += g1[0] * y1[0] + g1[1] * y1[1];
+                d1 += g1[2] * y1[2] + g1[3] * y1[3];
+                k0 = y0;
+                k1 = y1;
+            });
+            const float d = block_sum<THREADS>(d0 + d1, s_f[0]);
+            sweep([&](unsigned i0, unsigned i1, bool ok0, bool ok1, v4f& k0, v4f& k1) {
+                const v4f g0 = ok0 ? __builtin_nontemporal_load(gr + i0) : zero, g1 = ok1 ? __builtin_nontemporal_load(gr + i1) : zero;
+                v4f o0, o1;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    o0[e] = k0[e] * (g0[e] - d);
+                    o1[e] = k1[e] * (g1[e] - d);
+                }
+                if (ok0) __builtin_nontemporal_store(o0, outr + i0);
+                if (ok1) __builtin_nontemporal_store(o1, outr + i1);
+            });
+            continue;
+        }
+        if (MODE == kLogSoftmaxBwd) {
+            // d = sum g with g left on the chip; then dx = g - exp(y) * d from the kept g and y read once
+            float d0 = 0.0f, d1 = 0.0f;
+            sweep([&](unsigned i0, unsigned i1, bool ok0, bool ok1, v4f& k0, v4f& k1) {
+                k0 = ok0 ? __builtin_nontemporal_load(gr + i0) : zero;
+                k1 = ok1 ? __builtin_nontemporal_load(gr + i1) : zero;
+                d0 += (k0[0] + k0[1]) + (k1[0] + k1[1]);
+                d1 += (k0[2] + k0[3]) + (k1[2] + k1[3]);
+            });
+            const float d = block_sum<THREADS>(d0 + d1, s_f[0]);
+            sweep([&](unsigned i0, unsigned i1, bool ok0, bool ok1, v4f& k0, v4f& k1) {
+                const v4f y0 = ok0 ? __builtin_nontemporal_load(xr + i0) : zero, y1 = ok1 ? __builtin_nontemporal_load(xr + i1) : zero;
+                v4f o0, o1;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    o0[e] = k0[e] - (kFastOut ? cta_exp_hw(y0[e]) : cta_expf_tab(y0[e], s_exp2)) * d;
+                    o1[e] = k1[e] - (kFastOut ? cta_exp_hw(y1[e]) : cta_expf_tab(y1[e], s_exp2)) * d;
+                }
+                if (ok0) __builtin_nontemporal_store(o0, outr + i0);
+                if (ok1) __builtin_nontemporal_store(o1, outr + i1);
+            });
+            continue;
+        }
+        // softmax / log-softmax: the online (max, sum) pair of the kernel above over the words as they
+        // arrive, x left on the chip; then the result from the kept x
+        float m = kNegInf, s = 0.0f;
+        auto take = [&](const v4f& v) {
+            const float vm = __builtin_fmaxf(__builtin_fmaxf(v[0], v[1]), __builtin_fmaxf(v[2], v[3]));
+            if (vm > m) {
+                s *= __builtin_amdgcn_exp2f((m - vm) * 1.44269504088896340736f);
+                m = vm;
+            }
+            const float b = (m == kNegInf) ? 0.0f : m;
+            s += (__builtin_amdgcn_exp2f((v[0] - b) * 1.44269504088896340736f) + __builtin_amdgcn_exp2f((v[1] - b) * 1.44269504088896340736f)) +
+                 (__builtin_amdgcn_exp2f((v[2] - b) * 1.44269504088896340736f) + __builtin_amdgcn_exp2f((v[3] - b) * 1.44269504088896340736f));
+        };
+        sweep([&](unsigned i0, unsigned i1, bool ok0, bool ok1, v4f& k0, v4f& k1) {
+            k0 = ok0 ? __builtin_nontemporal_load(xr + i0) : zero;
+            k1 = ok1 ? __builtin_nontemporal_load(xr + i1) : zero;
+            if (ok0) take(k0);
+            if (ok1) take(k1);
+        });
+        const float M = block_max<THREADS>(m, s_f[0]);
+        s = (m == kNegInf) ? 0.0f : s * __builtin_amdgcn_exp2f((m - M) * 1.44269504088896340736f);
+        const float S = block_sum<THREADS>(s, s_f[1]);
+        const double rcp = 1.0 / double(S);
+        const float rcp_f = 1.0f / S;
+        const float lg = (MODE == kLogSoftmaxFast) ? cta_logf(S, cta_log_tab) : 0.0f;
+        auto result = [&](const v4f& v) {
+            v4f o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (MODE == kLogSoftmaxFast) {
+                    const float d = v[e] - M;
+                    o[e] = d - lg;
+                } else if (kFastOut) {
+                    o[e] = cta_exp_hw_nonpos(v[e] - M) * rcp_f;
+                } else {
+                    o[e] = cta_div_rcp(cta_expf_nonpos(v[e] - M, s_exp2), rcp);
+                }
+            }
+            return o;
+        };
+        sweep([&](unsigned i0, unsigned i1, bool ok0, bool ok1, v4f& k0, v4f& k1) {
+            if (ok0) __builtin_nontemporal_store(result(k0), outr + i0);
+            if (ok1) __builtin_nontemporal_store(result(k1), outr + i1);
+        });
+    }
+}
+
 template <int MODE_>
 __global__ __launch_bounds__(1024) void row_stream_kernel(Args a) {
     constexpr int THREADS = 1024;
@@ -964,7 +1110,21 @@ int run_rows(const char* name, Args a, float* loss_out, void* stream) {
             return fail(CTAMD_ERANGE, "%s: a row does not fit a block's registers (32768 columns, 8192 without 128-bit accesses): "
                         "use the separate forward and backward entry points", name);
         else if constexpr (MODE == kSoftmax || MODE == kSoftmaxBwd || MODE == kLogSoftmaxFast || MODE == kLogSoftmaxBwd) {
-            if (vec) hipLaunchKernelGGL((row_stream_vec_kernel<MODE_>), dim3(grid), dim3(1024), 0, s, a);
+            if (vec && (a.cols >> 2) <= kKeepVectors) {
+                // the kept operand takes 128 KiB of LDS: more than a kernel gets without asking, once per device
+                constexpr size_t kKeepBytes = size_t(kKeepLds) * 1024 * sizeof(v4f);
+                static bool raised[64] = {};
+                int dev = 0;
+                if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail(CTAMD_EHIP, "%s: no current device", name);
+                if (!raised[dev]) {
+                    if (hipFuncSetAttribute(reinterpret_cast<const void*>(row_keep_kernel<MODE_>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                            int(kKeepBytes)) != hipSuccess)
+                        return fail(CTAMD_EHIP, "%s: the device does not give a block %zu bytes of LDS", name, kKeepBytes);
+                    raised[dev] = true;
+                }
+                const unsigned cus = unsigned(compute_units() > 0 ? compute_units() : 256);
+                hipLaunchKernelGGL((row_keep_kernel<MODE_>), dim3(grid < cus ? grid : cus), dim3(1024), kKeepBytes, s, a);
+            } else if (vec) hipLaunchKernelGGL((row_stream_vec_kernel<MODE_>), dim3(grid), dim3(1024), 0, s, a);
             else hipLaunchKernelGGL((row_stream_kernel<MODE>), dim3(grid), dim3(1024), 0, s, a);
         } else
             hipLaunchKernelGGL((row_stream_kernel<MODE>), dim3(grid), dim3(1024), 0, s, a);

@@ -69,6 +69,27 @@ class Ctorch_Scheduler {
         return a.device();
     }
 
+    // The kernel registered for (operator, device).  The reference calls whatever its lookup left in the
+    // pointer, a null pointer included (include/Ctorch_Scheduler.h:128, :165); here a missing entry or a
+    // device that is not there throws.
+    template <class Table>
+    typename Table::mapped_type::mapped_type find_kernel(Table& table, op which, DeviceType where) {
+        ensureInit();
+        typename Table::mapped_type::mapped_type found = nullptr;
+        {
+            std::lock_guard<std::mutex> lock(mutex_);
+            auto row = table.find(which);
+            if (row != table.end() && isDeviceAvailable(where)) {
+                auto cell = row->second.find(where);
+                if (cell != row->second.end()) found = cell->second;
+            }
+        }
+        if (found == nullptr)
+            Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::PLATFORM_API,
+                                         "Ctorch_Scheduler: no kernel available for this op on this device");
+        return found;
+    }
+
     Tensor dispatch(const Tensor& a, const Tensor& b, op op_type) {
         if (a.dtype() != b.dtype())
             Ctorch_Error::log(ErrorLevel::ERROR, ErrorPlatform::kGENERAL, ErrorType::DATATYPE,
@@ -77,39 +98,13 @@ class Ctorch_Scheduler {
             op_type != op::CE && op_type != op::MatMul && a.sizes() != b.sizes())
             Ctorch_Error::log(ErrorLevel::ERROR, ErrorPlatform::kGENERAL, ErrorType::DIMENSION,
                               "Ctorch_Scheduler: tensor shapes differ");
-        ensureInit();
-        DeviceType target_dev = getTargetDevice(a, b);
-        BinaryKernelFunc target_kernel = nullptr;
-        {
-            std::lock_guard<std::mutex> lock(mutex_);
-            auto op_it = binary_kernel_map_.find(op_type);
-            if (op_it != binary_kernel_map_.end()) {
-                auto dev_it = op_it->second.find(target_dev);
-                if (dev_it != op_it->second.end() && isDeviceAvailable(target_dev)) target_kernel = dev_it->second;
-            }
-        }
-        if (target_kernel == nullptr)
-            Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::PLATFORM_API,
-                                         "Ctorch_Scheduler: no kernel available for this op on this device");
-        return target_kernel(a, b);
+        BinaryKernelFunc run = find_kernel(binary_kernel_map_, op_type, getTargetDevice(a, b));
+        return run(a, b);
     }
 
     Tensor dispatch(const Tensor& a, op op_type) {
-        ensureInit();
-        DeviceType target_dev = a.device();
-        UnaryKernelFunc target_kernel = nullptr;
-        {
-            std::lock_guard<std::mutex> lock(mutex_);
-            auto op_it = unary_kernel_map_.find(op_type);
-            if (op_it != unary_kernel_map_.end()) {
-                auto dev_it = op_it->second.find(target_dev);
-                if (dev_it != op_it->second.end() && isDeviceAvailable(target_dev)) target_kernel = dev_it->second;
-            }
-        }
-        if (target_kernel == nullptr)
-            Ctorch_Error::throwException(ErrorPlatform::kGENERAL, ErrorType::PLATFORM_API,
-                                         "Ctorch_Scheduler: no kernel available for this op on this device");
-        return target_kernel(a);
+        UnaryKernelFunc run = find_kernel(unary_kernel_map_, op_type, a.device());
+        return run(a);
     }
 
     // Registration point for further device columns (and for tests that register a stand-in).

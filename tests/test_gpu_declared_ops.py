@@ -221,7 +221,7 @@ def log_softmax_bwd(y, g, dim):
 
 
 @pytest.mark.parametrize("shape", [(1, 1), (3, 7), (33, 47), (64, 130), (5, 1000), (256, 10), (7, 2048), (3, 4099), (9, 32000), (2, 40000),
-                                   (2, 70001), (300, 64), (1000, 260)])
+                                   (2, 70001), (300, 64), (1000, 260), (3, 65536), (2, 49156)])
 def test_log_softmax_and_its_gradient(oracle, shape):
     print("case log_softmax", shape, flush=True)
     x = oracle.normal(shape, 41, 0, 2.5)

@@ -282,7 +282,8 @@ def test_column_sum(oracle, shape):
 
 
 SOFTMAX_SHAPES = [(1, 1), (3, 7), (19, 301), (64, 10), (5, 1000), (7, 1024), (4, 2052), (3, 8192), (2, 8200),
-                  (2, 32000), (2, 32768), (2, 33000), (3, 40001), (2, 131076)]
+                  (2, 32000), (2, 32768), (2, 33000), (3, 40001), (2, 131076),
+                  (3, 65536), (2, 49156), (2, 65540)]      # rows kept on the chip between the two sweeps: full, partly, one word too long
 
 
 @pytest.mark.parametrize("shape", SOFTMAX_SHAPES)
