@@ -169,12 +169,14 @@ def config_report(with_cpu):
     rc = host.cth_time_chain(fp(a), fp(b), L(n), I(5), I(50), out)
     cpu = _timed(lambda: ref.chain(a, b)) if with_cpu else None
     add("config 1: c=a*b+5, relu, sum, backward; n=2^20", rc, out, cpu, "whole step", launch_bound=True)
-    # the elementwise chain as one fused expression (one launch forward, one backward); same bits
+    # the elementwise chain as one fused expression (one launch forward, one backward); no
+    # transcendental operator in it, so the same bits in either math mode
     host.cth_set_fused_expr(1)
     out = D5()
     rc = host.cth_time_chain(fp(a), fp(b), L(n), I(5), I(50), out)
     host.cth_set_fused_expr(0)
     add("config 1: c=a*b+5, relu, sum, backward; n=2^20, fused expression", rc, out, cpu, "whole step", launch_bound=True)
+    rows[-1]["math_mode"] = "default (CTAMD_MATH_FAST); this program has no transcendental operator: bit-equal to the unfused step"
 
     # config 2: MatMul forward + backward at 1024, 2048, 4096; Dot 2^26
     slab_ms = {}
@@ -184,10 +186,14 @@ def config_report(with_cpu):
         rc = host.cth_time_matmul(fp(A), fp(B), L(Mm), I(3), I(10), out)
         cpu, note = None, None
         if with_cpu:
-            r = {1024: 64, 2048: 32, 4096: 16}[Mm]
+            # 1024^3 is timed in full; the larger products on a slab of rows, extrapolated (the loop
+            # runs row by row, so its time is linear in the rows); the two backward products run the
+            # same loop on transposed views and are counted at the forward product's time
+            r = {1024: 1024, 2048: 256, 4096: 16}[Mm]
             t = _timed(lambda: ref.matmul_t(A[:r], 0, B, 0) if cpu_kind == "reference" else ref.matmul(A[:r], B))
             cpu = t * (Mm / r) * 3
-            note = "forward rows 0..%d (%.2f s), x%d for all rows, x3 for the two backward products" % (r - 1, t / 1e3, Mm // r)
+            note = ("forward product in full (%.2f s), x3 for the two backward products" % (t / 1e3) if r == Mm else
+                    "forward rows 0..%d (%.2f s), x%d for all rows, x3 for the two backward products" % (r - 1, t / 1e3, Mm // r))
         add("config 2: MatMul %d^3 forward + backward (dC = ones)" % Mm, rc, out, cpu, note)
         del A, B
     u, v = rng.uniform(1 << 26, SEEDS["config2"]["dot_u"], -1, 1), rng.uniform(1 << 26, SEEDS["config2"]["dot_v"], -1, 1)
@@ -296,13 +302,27 @@ def config_report(with_cpu):
         t = _timed(lambda: ref.expr(Xs, Rs, Ts))
         cpu, note = t * (R5 / r), "rows 0..%d with the row vector materialised (%.2f s), x%d" % (r - 1, t / 1e3, R5 // r)
     add("config 5: Y=sigmoid(X/r)-tanh(X)*sin(X)+cos(-X), MSE+MAE, backward; X [4096 x 4096]", rc, out, cpu, note)
-    # Y as one fused expression: one pass forward, one pass for dX and dr; same Y and dX bits
+    # Y as one fused expression: one pass forward, one pass for dX and dr, in the library's default math
+    # mode: sigmoid, sin and cos in single precision within 2 ulp of the reference's libm loops, tanh with
+    # the reference's bits (CTAMD_MATH_EXACT gives the unfused step's Y and dX bit for bit)
     host.cth_set_fused_expr(1)
     out = D5()
     rc = host.cth_time_expr(fp(X), fp(rv), fp(T), L(R5), L(R5), I(3), I(10), out)
     host.cth_set_fused_expr(0)
     add("config 5: Y=sigmoid(X/r)-tanh(X)*sin(X)+cos(-X), MSE+MAE, backward; X [4096 x 4096], fused expression", rc, out, cpu,
         note)
+    rows[-1]["math_mode"] = "default (CTAMD_MATH_FAST): sigmoid / sin / cos <= 2 ulp of the reference's formulas, tanh bit-equal"
+    # and in the exact mode, where every element of Y and dX has the bits of the operator-by-operator step
+    capi_lib = C.CDLL(os.path.join(ROOT, "ctorch_amd", "libctorch_amd.so"))
+    capi_lib.ctamd_set_math_mode(1)
+    host.cth_set_fused_expr(1)
+    out = D5()
+    rc = host.cth_time_expr(fp(X), fp(rv), fp(T), L(R5), L(R5), I(3), I(10), out)
+    host.cth_set_fused_expr(0)
+    capi_lib.ctamd_set_math_mode(0)
+    add("config 5: Y=sigmoid(X/r)-tanh(X)*sin(X)+cos(-X), MSE+MAE, backward; X [4096 x 4096], fused expression, exact math mode",
+        rc, out, cpu, note)
+    rows[-1]["math_mode"] = "CTAMD_MATH_EXACT: bit-equal to the unfused step"
     return {"cores": 1, "cpu_kind": cpu_kind if with_cpu else None, "seeds": SEEDS, "steps": rows}
 
 

@@ -217,6 +217,13 @@ def main():
                  (SIN, 4, 0, 0, 0.0), (MUL, 3, 3, 4, 0.0), (SUB, 2, 2, 3, 0.0), (NEG, 3, 0, 0, 0.0), (COS, 3, 3, 0, 0.0),
                  (ADD, 2, 2, 3, 0.0), (STORE, 0, 2, 0, 0.0))
     ew("fused sigmoid(X/r) - tanh(X)*sin(X) + cos(-X) [16384 x 4096]", lambda k: run_expr(c5, [A[k], B[0]], [R[k]], 16384, 4096), 8)
+    # the rows above ran as kernels compiled for their programs (from the second launch on); the same
+    # programs through the interpreter, for comparison
+    jit = lib.ctamd_expr_jit()
+    call("ctamd_set_expr_jit", 0)
+    ew("interpreted relu(a * b + 5)", lambda k: run_expr(chain, [A[k], B[k]], [R[k]], 16384, 4096), 12)
+    ew("interpreted sigmoid(X/r) - tanh(X)*sin(X) + cos(-X) [16384 x 4096]", lambda k: run_expr(c5, [A[k], B[0]], [R[k]], 16384, 4096), 8)
+    call("ctamd_set_expr_jit", jit)
     if args.only_expr:
         if args.json:
             print(json.dumps({"device": torch.cuda.get_device_name(0), "results": results}))
