@@ -38,9 +38,13 @@ constexpr int kXcds = 8;
 constexpr int kMinWavesPerSimd = 2;   // register budget of both tile shapes: 256 VGPRs per lane
 
 
-template <int BM_, int BN_, int BK_, int WM_, int WN_, bool EARLY_ = false>
+template <int BM_, int BN_, int BK_, int WM_, int WN_, bool EARLY_ = false, int KG_ = 1>
 struct Cfg {
-    static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
+    // KG: wave groups per block.  Each group computes the whole BM x BN tile over its own KSLICE-wide
+    // slice of every k tile (the block stages KG slices at a time), and the groups' accumulators are
+    // added in group order through LDS at the end: more waves per SIMD on a tile too small to give
+    // each its own piece of C, without a second launch to add the parts.
+    static constexpr int BM = BM_, BN = BN_, KSLICE = BK_, KG = KG_, BK = BK_ * KG_, WM = WM_, WN = WN_;
     // EARLY: the staged tile goes to LDS, and the next tile is requested from global memory, at the
     // top of a k tile instead of around its barrier.  The request then has a whole k tile to arrive;
     // where a k tile is a handful of MFMAs (the 64 x 64 and 128 x 128 block tiles: 8 and 32 per wave)
@@ -48,9 +52,10 @@ struct Cfg {
     static constexpr bool EARLY = EARLY_;
     static constexpr int TM = WM / 32, TN = WN / 32;       // MFMA tiles per wave
     static constexpr int WAVES_N = BN / WN;
-    static constexpr int THREADS = (BM / WM) * (BN / WN) * 64;
-    static_assert(THREADS == 256 || THREADS == 512, "4 or 8 waves per block");
-    static_assert(BK % 8 == 0, "k tile is a multiple of the 8-wide chunk");
+    static constexpr int WAVES_MN = (BM / WM) * (BN / WN);
+    static constexpr int THREADS = WAVES_MN * KG * 64;
+    static_assert(THREADS == 256 || THREADS == 512 || THREADS == 1024, "4, 8 or 16 waves per block");
+    static_assert(KSLICE % 8 == 0, "a group's k slice is a multiple of the 8-wide chunk");
     static constexpr int KPAD = BK + 4;                    // K-contiguous row stride (floats)
     static constexpr int XPAD_M = BM + 8, XPAD_N = BN + 8; // X-contiguous row strides
 };
@@ -90,7 +95,6 @@ struct Stage {
             r[q] = *reinterpret_cast<const v4f*>(base + size_t(q) * piece_step + off);
         base += step_bytes;
     }
-
     // x0: first row/col of the tile in the X dimension, k0: first k; dimX, K: extents; ld: leading
     // dimension (elements) of the contiguous direction's rows.  VEC: 16-byte aligned rows.
     template <bool VEC>
@@ -187,6 +191,8 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
     constexpr int B_FLOATS = tile_floats<C, B_KC, false>();
     __shared__ __attribute__((aligned(16))) float s_a[2][A_FLOATS];
     __shared__ __attribute__((aligned(16))) float s_b[2][B_FLOATS];
+    constexpr int KG = C::KG;
+    __shared__ __attribute__((aligned(16))) float s_sum[KG > 1 ? (KG - 1) * BM * BN : 4];   // the other groups' accumulators
 
     // XCD-aware renumbering: hardware block b runs on XCD b % 8; give each XCD a contiguous run of
     // tiles, and inside the run walk C in column-major bands of 8 tile rows so that co-resident
@@ -215,7 +221,7 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
     int k_end = split ? k_begin + g.k_per_split : g.k;
     if (k_end > g.k) k_end = g.k;
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) % C::WAVES_MN, group = (threadIdx.x >> 6) / C::WAVES_MN;
     const int wm = (wave / C::WAVES_N) * C::WM, wn = (wave % C::WAVES_N) * C::WN;
     const int l32 = lane & 31, half = lane >> 5;
 
@@ -243,13 +249,13 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
     // s_waitcnt lgkmcnt(0) as an instruction the compiler's wait-count bookkeeping sees (it cannot
     // look inside inline asm): vmcnt and expcnt fields at their maxima, lgkmcnt 0.
     auto lds_wait = [] { __builtin_amdgcn_s_waitcnt(0xC07F); };
-    constexpr int NCH = BK / 8;
+    constexpr int NCH = C::KSLICE / 8;
     static_assert(NCH == 2, "the pipeline below alternates two fragment buffers over two chunks");
     float fa[2][TM][4], fb[2][TN][4];
     auto fetch_chunk = [&](int buf, int ch, int which) {
         const float* __restrict__ la = s_a[buf];
         const float* __restrict__ lb = s_b[buf];
-        const int kb = ch * 8 + half * 4;
+        const int kb = group * C::KSLICE + ch * 8 + half * 4;
 #pragma unroll
         for (int i = 0; i < TM; ++i) fetch<A_KC>(la, A_STRIDE, wm + i * 32 + l32, kb, fa[which][i]);
 #pragma unroll
@@ -396,6 +402,30 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
         mfmas(1);
     }
 
+    if (KG > 1) {
+        // group 0 adds the other groups' accumulators to its own in group order; lane-contiguous
+        // words, so neither side meets a bank conflict
+        float* __restrict__ mine = s_sum + (size_t(group > 0 ? group - 1 : 0) * C::WAVES_MN + wave) * (TM * TN * 16 * 64) + lane;
+        if (group > 0) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) mine[((i * TN + j) * 16 + r) * 64] = acc[i][j][r];
+        }
+        __syncthreads();
+        if (group > 0) return;
+#pragma unroll
+        for (int z = 1; z < KG; ++z)
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        acc[i][j][r] += mine[(size_t(z - 1) * C::WAVES_MN * TM * TN * 16 + (i * TN + j) * 16 + r) * 64];
+    }
     // accumulator register r of lane l holds C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 tile
     if (!split) {
 #pragma unroll
@@ -873,6 +903,9 @@ using WideTile = Cfg<256, 128, 16, 128, 64>;
 // tile ([1024 x 1024, K = 2048]: 67 -> 45 us; with several blocks per CU it is 1-2% slower, as is the
 // 128 x 128 tile either way)
 using TinyEarlyTile = Cfg<64, 64, 16, 32, 32, true>;
+using TinyK2Tile = Cfg<64, 64, 16, 32, 32, true, 2>;
+using TinyK4Tile = Cfg<64, 64, 16, 32, 32, true, 4>;
+using SmallK2Tile = Cfg<128, 128, 16, 64, 64, false, 2>;
 
 template <class Tile, bool A_KC, bool B_KC>
 int launch_gemm(GemmArgs g, bool vec, int blocks, hipStream_t s) {
@@ -985,7 +1018,7 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
         }
     }
     constexpr int BK = 16;
-    static_assert(BigTile::BK == BK && WideTile::BK == BK && SmallTile::BK == BK && TinyTile::BK == BK, "all tile shapes step K alike");
+    static_assert(BigTile::BK == 16 && WideTile::BK == 16 && SmallTile::BK == 16 && TinyTile::BK == 16, "all tile shapes step K alike");
     // The plan: a tile shape, and into how many parts along K the tiles of the last, partly filled
     // round of blocks are cut (a round: `together` resident blocks on each CU), by a model of the
     // time in seconds, fitted to measurements on this chip (1024^3 ... 7168^3 and the skinny
@@ -997,11 +1030,22 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
     //                      the memory latencies a block waits out before its first and after its last k tile
     //   adding the parts   a launch and the parts' bytes written and read once
     // parts fill the free places of the round with at least 8 k tiles each (4 when K allows no more).
+    // A launch of at most one block per CU on the 64 x 64 or 128 x 128 tiles runs on their kernels with
+    // 4 (2) wave groups per block when each block has a long enough run of K in whole k tiles of all
+    // groups: measured 1024^3 26 -> 24 us, [1024 x 1024, K = 4096] 88 -> 76 us, 2048^3 138 -> 134 us
+    // (and 153 us on four 64 x 64 tiles per CU, which the old figure for a lone 128 x 128 block preferred).
+    auto wave_groups = [&](int sh, int64_t blocks, int parts) -> int {
+        if (blocks > cus || sh > 1) return 1;
+        const int64_t run = (k + parts - 1) / parts;
+        if (sh == 0) return run >= 512 && k % 64 == 0 ? 4 : run >= 512 && k % 32 == 0 ? 2 : 1;
+        return run >= 1024 && k % 32 == 0 ? 2 : 1;
+    };
+    static const double alone_grouped[2][5] = {{0, 0, 1.40, 0, 1.32}, {0, 0, 1.09, 0, 0}};   // [shape][groups]
     struct Shape { int bm, bn, together; double per_flop, alone; };
     static const Shape shapes[4] = {{TinyTile::BM, TinyTile::BN, 4, 1.30, 1.70}, {SmallTile::BM, SmallTile::BN, 2, 1.07, 1.34},
                                     {BigTile::BM, BigTile::BN, 1, 1.00, 1.00}, {WideTile::BM, WideTile::BN, 2, 1.04, 1.32}};
     const double t_elem = 2.0 * double(k) / (157.3e12 * 0.92 / cus);
-    int shape = 0, splits = 1, whole_tiles = 0;
+    int shape = 0, splits = 1, whole_tiles = 0, groups = 1;
     double best = -1.0;
     for (int sh = 0; sh < 4; ++sh) {
         const Shape& q = shapes[sh];
@@ -1020,18 +1064,23 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
                 if (p >= 2) most = int(p);
             }
         }
-        for (int parts : {1, most / 2, most}) {
+        // also: as many parts as keep the launch at one block per CU
+        const int fit = rounds == 0 && left > 0 && cus / left < most ? int(cus / left) : 0;
+        for (int parts : {1, fit, most / 2, most}) {
             if (parts < 1 || (parts == 1 && most > 1 && left == 0)) continue;
             double cost = double(rounds) * q.together * q.per_flop * area * t_elem;
+            int kg = 1;
             if (left > 0) {
                 const int64_t c = (left * parts + cus - 1) / cus;
-                const double busy = q.together == 1 ? q.alone
-                                                    : q.alone + double(c - 1) * (q.together * q.per_flop - q.alone) / (q.together - 1);
+                kg = rounds == 0 ? wave_groups(sh, left * parts, parts) : 1;
+                const double alone = kg > 1 ? alone_grouped[sh][kg] : q.alone;
+                const double busy = q.together == 1 ? alone
+                                                    : alone + double(c - 1) * (q.together * q.per_flop - alone) / (q.together - 1);
                 cost += busy * area * t_elem / parts + (rounds == 0 ? 3e-6 : 1e-6);
                 if (parts > 1) cost += 6e-6 + double(left) * parts * area * 8.0 / 4e12;
             }
             if (best < 0.0 || cost < best) {
-                best = cost; shape = sh; splits = parts; whole_tiles = int(parts > 1 ? tiles - left : tiles);
+                best = cost; shape = sh; splits = parts; whole_tiles = int(parts > 1 ? tiles - left : tiles); groups = kg;
             }
         }
     }
@@ -1054,7 +1103,7 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
     ScratchUse use(stream, splits > 1);
     if (splits > 1) {
         int kps = int((k + splits - 1) / splits);
-        kps = (kps + BK - 1) / BK * BK;
+        kps = (kps + BK * groups - 1) / (BK * groups) * (BK * groups);
         g.splits = splits = int((k + kps - 1) / kps);
         g.k_per_split = kps;
         g.partial = use.ptr();
@@ -1065,7 +1114,10 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
     // a tile outside [0, whole_tiles) writes its parts to g.partial: there is none unless the plan cut K
     if (splits == 1 && whole_tiles != tiles) return fail(CTAMD_EINVAL, "%s: plan leaves %d tiles without a part buffer", name, tiles - whole_tiles);
     const int blocks = whole_tiles + (tiles - whole_tiles) * splits;
-    int rc = (shape == 0 && blocks <= cus) ? launch_layout<TinyEarlyTile>(g, A_KC, B_KC, vec, blocks, s)
+    int rc = groups == 4 ? launch_layout<TinyK4Tile>(g, A_KC, B_KC, vec, blocks, s)
+           : groups == 2 && shape == 0 ? launch_layout<TinyK2Tile>(g, A_KC, B_KC, vec, blocks, s)
+           : groups == 2 ? launch_layout<SmallK2Tile>(g, A_KC, B_KC, vec, blocks, s)
+           : (shape == 0 && blocks <= cus) ? launch_layout<TinyEarlyTile>(g, A_KC, B_KC, vec, blocks, s)
            : shape == 3 ? launch_layout<WideTile>(g, A_KC, B_KC, vec, blocks, s)
            : shape == 2 ? launch_layout<BigTile>(g, A_KC, B_KC, vec, blocks, s)
            : shape == 1 ? launch_layout<SmallTile>(g, A_KC, B_KC, vec, blocks, s)
