@@ -236,10 +236,15 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
     Stage<BM, BK, A_KC, C::THREADS> sa;
     Stage<BN, BK, B_KC, C::THREADS> sb;
     const int ktiles = (k_end - k_begin + BK - 1) / BK;
-    // interior: the whole BM x BN tile and every k tile lie inside the operands and rows are
-    // 16-byte aligned - true for all blocks of a 4096^3 product, false only on ragged edges
-    const bool interior = VEC && m0 + BM <= g.m && n0 + BN <= g.n && (k_end - k_begin) % BK == 0 &&
+    const int whole_ktiles = (k_end - k_begin) / BK;
+    // interior: the whole BM x BN tile lies inside C and rows are 16-byte aligned - true for all blocks
+    // of a 4096^3 product, false only on ragged edges.  The pipelined loop then runs while the k tile it
+    // requests (two ahead) is a whole one; a K that ends inside a k tile leaves the last iterations to
+    // the bounds-checked loop below, which takes over the same state (tile t in LDS, tile t+1 in the
+    // staging registers, chunk 0 of tile t fetched).
+    const bool interior = VEC && m0 + BM <= g.m && n0 + BN <= g.n && (whole_ktiles == ktiles || whole_ktiles >= 2) &&
                           g.lda < (int64_t(1) << 21) && g.ldb < (int64_t(1) << 21);   // tile extent < 2^32 bytes
+    const int fast_iters = !interior ? 0 : whole_ktiles == ktiles ? ktiles - 1 : whole_ktiles - 2;
     const int64_t a_step = (A_KC ? BK : int64_t(BK) * g.lda) * 4;   // bytes per k tile
     const int64_t b_step = (B_KC ? BK : int64_t(BK) * g.ldb) * 4;
     if (interior) {
@@ -289,6 +294,11 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
     // is a wait in front of an MFMA for data requested just before it.  Interior blocks pin the
     // interleaving with scheduling groups; the two waves of a SIMD run in phase (one barrier per
     // tile), so housekeeping outside the bursts would idle the pipe for both.
+    auto stage_tile = [&](int kt) {
+        sa.template load<VEC>(g.a, g.lda, m0, k_begin + kt * BK, g.m, k_end);
+        sb.template load<VEC>(g.b, g.ldb, n0, k_begin + kt * BK, g.n, k_end);
+    };
+    int t = 0;
     if (interior) {
         sa.load_fast(a_step);
         sb.load_fast(b_step);
@@ -299,7 +309,7 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
         // (in bounds, never stored), which keeps the loop body free of branches
         if (ktiles > 1) { sa.load_fast(ktiles > 2 ? a_step : 0); sb.load_fast(ktiles > 2 ? b_step : 0); }
         fetch_chunk(0, 0, 0);
-        for (int t = 0; t + 1 < ktiles; ++t) {
+        for (; t < fast_iters; ++t) {
             const int cur = t & 1;
             __builtin_amdgcn_sched_barrier(0);
             if (C::EARLY) {
@@ -363,17 +373,15 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
             __builtin_amdgcn_sched_barrier(0);
         }
     } else {
-        auto stage_tile = [&](int t) {
-            sa.template load<VEC>(g.a, g.lda, m0, k_begin + t * BK, g.m, k_end);
-            sb.template load<VEC>(g.b, g.ldb, n0, k_begin + t * BK, g.n, k_end);
-        };
         stage_tile(0);
         sa.store(s_a[0], A_STRIDE);
         sb.store(s_b[0], B_STRIDE);
         __syncthreads();
         if (ktiles > 1) stage_tile(1);
         fetch_chunk(0, 0, 0);
-        for (int t = 0; t + 1 < ktiles; ++t) {
+    }
+    {
+        for (; t + 1 < ktiles; ++t) {
             const int cur = t & 1;
             lds_wait();
             fetch_chunk(cur, 1, 1);
@@ -903,7 +911,6 @@ using WideTile = Cfg<256, 128, 16, 128, 64>;
 // tile ([1024 x 1024, K = 2048]: 67 -> 45 us; with several blocks per CU it is 1-2% slower, as is the
 // 128 x 128 tile either way)
 using TinyEarlyTile = Cfg<64, 64, 16, 32, 32, true>;
-using TinyK2Tile = Cfg<64, 64, 16, 32, 32, true, 2>;
 using TinyK4Tile = Cfg<64, 64, 16, 32, 32, true, 4>;
 using SmallK2Tile = Cfg<128, 128, 16, 64, 64, false, 2>;
 
@@ -1031,16 +1038,15 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
     //   adding the parts   a launch and the parts' bytes written and read once
     // parts fill the free places of the round with at least 8 k tiles each (4 when K allows no more).
     // A launch of at most one block per CU on the 64 x 64 or 128 x 128 tiles runs on their kernels with
-    // 4 (2) wave groups per block when each block has a long enough run of K in whole k tiles of all
-    // groups: measured 1024^3 26 -> 24 us, [1024 x 1024, K = 4096] 88 -> 76 us, 2048^3 138 -> 134 us
+    // 4 (2) wave groups per block when each block has a long enough run of K: measured 1024^3 26 -> 24 us, [1024 x 1024, K = 4096] 88 -> 76 us, 2048^3 138 -> 134 us
     // (and 153 us on four 64 x 64 tiles per CU, which the old figure for a lone 128 x 128 block preferred).
     auto wave_groups = [&](int sh, int64_t blocks, int parts) -> int {
         if (blocks > cus || sh > 1) return 1;
         const int64_t run = (k + parts - 1) / parts;
-        if (sh == 0) return run >= 512 && k % 64 == 0 ? 4 : run >= 512 && k % 32 == 0 ? 2 : 1;
-        return run >= 1024 && k % 32 == 0 ? 2 : 1;
+        if (sh == 0) return run >= 512 ? 4 : 1;
+        return run >= 1024 ? 2 : 1;
     };
-    static const double alone_grouped[2][5] = {{0, 0, 1.40, 0, 1.32}, {0, 0, 1.09, 0, 0}};   // [shape][groups]
+    static const double alone_grouped[2][5] = {{0, 0, 0, 0, 1.32}, {0, 0, 1.09, 0, 0}};   // [shape][groups]
     struct Shape { int bm, bn, together; double per_flop, alone; };
     static const Shape shapes[4] = {{TinyTile::BM, TinyTile::BN, 4, 1.30, 1.70}, {SmallTile::BM, SmallTile::BN, 2, 1.07, 1.34},
                                     {BigTile::BM, BigTile::BN, 1, 1.00, 1.00}, {WideTile::BM, WideTile::BN, 2, 1.04, 1.32}};
@@ -1115,7 +1121,6 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
     if (splits == 1 && whole_tiles != tiles) return fail(CTAMD_EINVAL, "%s: plan leaves %d tiles without a part buffer", name, tiles - whole_tiles);
     const int blocks = whole_tiles + (tiles - whole_tiles) * splits;
     int rc = groups == 4 ? launch_layout<TinyK4Tile>(g, A_KC, B_KC, vec, blocks, s)
-           : groups == 2 && shape == 0 ? launch_layout<TinyK2Tile>(g, A_KC, B_KC, vec, blocks, s)
            : groups == 2 ? launch_layout<SmallK2Tile>(g, A_KC, B_KC, vec, blocks, s)
            : (shape == 0 && blocks <= cus) ? launch_layout<TinyEarlyTile>(g, A_KC, B_KC, vec, blocks, s)
            : shape == 3 ? launch_layout<WideTile>(g, A_KC, B_KC, vec, blocks, s)

@@ -510,7 +510,10 @@ MM_SHAPES = [(1, 1, 1), (5, 3, 9), (33, 29, 47), (128, 128, 16), (130, 257, 70),
              (130, 257, 600), (70, 33, 1000), (100, 70, 513),
              # at most one block per CU with a long K: the 64 x 64 tile's kernels with four and two wave
              # groups per block and the 128 x 128 tile's with two, ragged edges, and with K cut over blocks
-             (1000, 1010, 1024), (1024, 1000, 544), (2040, 2048, 1056), (512, 500, 4096), (1024, 1024, 1024)]
+             (1000, 1010, 1024), (1024, 1000, 544), (2040, 2048, 1056), (512, 500, 4096), (1024, 1024, 1024),
+             # aligned rows and a K that ends inside a k tile: the pipelined loop hands its last tiles to
+             # the bounds-checked one (one and four wave groups, K cut over blocks, the 256 x 256 tile)
+             (1024, 1024, 1000), (256, 128, 40), (300, 200, 4100), (2048, 2048, 1052), (4096, 2048, 100), (512, 512, 36)]
 
 
 @pytest.mark.parametrize("m,n,k", MM_SHAPES)
@@ -534,7 +537,8 @@ def test_matmul_all_layouts_normwise(oracle, m, n, k):
 @pytest.mark.parametrize("m,n,k", [(256, 128, 784), (128, 10, 64), (70, 33, 129), (8192, 256, 784), (96, 12, 4096),
                                    (2100, 2050, 40), (4090, 4093, 24), (4090, 2047, 24), (5, 7, 0),
                                    (8192, 10, 256), (256, 10, 8192), (777, 13, 3001), (256, 256, 256), (100, 70, 300),
-                                   (1000, 1010, 1024), (1024, 1000, 544), (2040, 2048, 1056), (512, 500, 4096)])
+                                   (1000, 1010, 1024), (1024, 1000, 544), (2040, 2048, 1056), (512, 500, 4096),
+                                   (1024, 1024, 1000), (300, 200, 4100), (4096, 2048, 100)])
 def test_fused_layer_equals_the_three_launches(oracle, m, n, k):
     """matmul + bias row + ReLU in one launch against the same three operators launched in sequence,
     bit for bit, over all tile shapes (the last four: wave groups inside a block), the K-split fold
