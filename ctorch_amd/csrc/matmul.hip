@@ -166,6 +166,13 @@ struct GemmArgs {
     const float* bias;              // optional row vector [n] added to every row of C (null: none)
     int relu;                       // then max(0, .) when set
     const float* mask;              // optional [m, n] row-major: C is multiplied by [mask > 0] last (null: none)
+    // The column sums of b ([k, n] in contiguous rows) riding along (sum_out null: not wanted): blocks
+    // [product_blocks, product_blocks + sum.chunks) of the product's launch run stage 1 of the narrow
+    // column sum into sum_partials, and the last blocks of the launch that adds the parts run stage 2.
+    float* sum_out;
+    float* sum_partials;
+    ColsumNarrowPlan sum;
+    int product_blocks;
 };
 
 // Output epilogue of a product that is not split along K: bias add, then ReLU as `v > 0 ? v : +0`
@@ -182,7 +189,7 @@ __device__ __forceinline__ float masked(float v, const float* __restrict__ mask,
     return mask ? v * (mask[at] > 0.0f ? 1.0f : 0.0f) : v;
 }
 
-template <class C, bool A_KC, bool B_KC, bool VEC>
+template <class C, bool A_KC, bool B_KC, bool VEC, bool SUMS = false>
 __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(GemmArgs g) {
     constexpr int BM = C::BM, BN = C::BN, BK = C::BK, TM = C::TM, TN = C::TN;
     constexpr int A_STRIDE = A_KC ? C::KPAD : C::XPAD_M;
@@ -194,6 +201,12 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
     constexpr int KG = C::KG;
     __shared__ __attribute__((aligned(16))) float s_sum[KG > 1 ? (KG - 1) * BM * BN : 4];   // the other groups' accumulators
 
+    if (SUMS && int(blockIdx.x) >= g.product_blocks) {
+        static_assert(!SUMS || (2 * A_FLOATS >= kColsumThreads * 4 && !B_KC && VEC), "stage 1 borrows the A tiles' LDS; b in aligned contiguous rows");
+        colsum_narrow_body<true>(g.b, g.sum_partials, size_t(g.k), size_t(g.n), g.sum.lanes, g.sum.groups, g.sum.rows_per_block,
+                                 blockIdx.x - unsigned(g.product_blocks), threadIdx.x, &s_a[0][0]);
+        return;
+    }
     // XCD-aware renumbering: hardware block b runs on XCD b % 8; give each XCD a contiguous run of
     // tiles, and inside the run walk C in column-major bands of 8 tile rows so that co-resident
     // blocks share A row bands and B column bands in that XCD's L2.
@@ -473,6 +486,13 @@ constexpr int kFoldSlice = kThreads * 4;       // one 128-bit word per thread: a
 template <int BM, int BN>
 __global__ __launch_bounds__(kThreads) void fold_parts(GemmArgs g) {
     static_assert(BM * BN % kFoldSlice == 0, "a tile is a whole number of slices");
+    __shared__ double s_acc[kColsumThreads];
+    if (blockIdx.x >= unsigned(g.tiles_m * g.tiles_n - g.whole_tiles)) {       // past the split tiles: stage 2 of b's column sums
+        if (blockIdx.y == 0)
+            colsum_fold_body<kFoldLanes>(g.sum_partials, g.sum_out, size_t(g.n), g.sum.chunks,
+                                         blockIdx.x - unsigned(g.tiles_m * g.tiles_n - g.whole_tiles), threadIdx.x, s_acc);
+        return;
+    }
     const int split_tile = blockIdx.x;
     const int bid = g.whole_tiles + split_tile;
     constexpr int BAND = 8;
@@ -921,6 +941,14 @@ int launch_gemm(GemmArgs g, bool vec, int blocks, hipStream_t s) {
     return launched("ctamd_matmul_f32");
 }
 
+// the product with stage 1 of b's column sums as extra blocks (b in contiguous aligned rows)
+template <class Tile>
+int launch_with_sums(GemmArgs g, bool a_kc, int blocks, hipStream_t s) {
+    if (a_kc) hipLaunchKernelGGL((gemm_kernel<Tile, true, false, true, true>), dim3(unsigned(blocks)), dim3(Tile::THREADS), 0, s, g);
+    else hipLaunchKernelGGL((gemm_kernel<Tile, false, false, true, true>), dim3(unsigned(blocks)), dim3(Tile::THREADS), 0, s, g);
+    return launched("ctamd_matmul_colsum_f32");
+}
+
 template <class Tile>
 int launch_layout(GemmArgs g, bool a_kc, bool b_kc, bool vec, int blocks, hipStream_t s) {
     if (a_kc && b_kc) return launch_gemm<Tile, true, true>(g, vec, blocks, s);
@@ -1099,6 +1127,7 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
     g.tiles_m = int((m + BM - 1) / BM);
     g.tiles_n = int((n + BN - 1) / BN);
     g.bias = bias; g.relu = relu; g.mask = mask;
+    g.sum_out = nullptr; g.sum_partials = nullptr; g.sum = ColsumNarrowPlan{0, 0, 0, 0}; g.product_blocks = 0;
     g.c_vec = (aligned16(c) && n % 4 == 0) ? 1 : 0;
     const bool vec = aligned16(a) && aligned16(b) && (g.lda % 4 == 0) && (g.ldb % 4 == 0);
     const int tiles = g.tiles_m * g.tiles_n;
@@ -1120,6 +1149,25 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
     // a tile outside [0, whole_tiles) writes its parts to g.partial: there is none unless the plan cut K
     if (splits == 1 && whole_tiles != tiles) return fail(CTAMD_EINVAL, "%s: plan leaves %d tiles without a part buffer", name, tiles - whole_tiles);
     const int blocks = whole_tiles + (tiles - whole_tiles) * splits;
+    // b's column sums ride along when the product is cut along K on the 64 x 64 tile (the weight gradient
+    // of a layer a few hundred wide at a large batch): stage 1 as extra blocks of the product's launch,
+    // stage 2 as extra blocks of the launch that adds the parts - two launches fewer, the same bits
+    if (sums && sums_done && splits > 1 && shape == 0 && groups == 1 && vec && !B_KC && bs0 == n &&
+        colsum_narrow_plan(size_t(k), size_t(n), true, &g.sum) &&
+        size_t(tiles - whole_tiles) * size_t(splits) * size_t(BM) * size_t(BN) + size_t(g.sum.chunks) * size_t(n) <= kScratchFloats) {
+        g.sum_out = sums;
+        g.sum_partials = g.partial + size_t(tiles - whole_tiles) * size_t(splits) * size_t(BM) * size_t(BN);
+        g.product_blocks = blocks;
+        *sums_done = true;
+        account(4.0 * double(k) * double(n), double(k) * double(n), true);
+        const int all = blocks + int(g.sum.chunks);
+        int rc = blocks <= cus ? launch_with_sums<TinyEarlyTile>(g, A_KC, all, s) : launch_with_sums<TinyTile>(g, A_KC, all, s);
+        if (rc) return rc;
+        constexpr unsigned kFoldCols = kColsumThreads / kFoldLanes;
+        const dim3 fold_grid(unsigned(tiles - whole_tiles) + (unsigned(n) + kFoldCols - 1) / kFoldCols, unsigned(BM * BN / kFoldSlice));
+        hipLaunchKernelGGL((fold_parts<TinyTile::BM, TinyTile::BN>), fold_grid, dim3(kThreads), 0, s, g);
+        return launched(name);
+    }
     int rc = groups == 4 ? launch_layout<TinyK4Tile>(g, A_KC, B_KC, vec, blocks, s)
            : groups == 2 ? launch_layout<SmallK2Tile>(g, A_KC, B_KC, vec, blocks, s)
            : (shape == 0 && blocks <= cus) ? launch_layout<TinyEarlyTile>(g, A_KC, B_KC, vec, blocks, s)

@@ -240,60 +240,10 @@ template <bool VEC>
 __global__ __launch_bounds__(kThreads) void colsum_narrow_stage1(const float* __restrict__ g, float* __restrict__ partials,
                                                                  size_t rows, size_t cols, unsigned lanes, unsigned groups,
                                                                  size_t rows_per_block) {
-    constexpr int W = VEC ? 4 : 1;
-    __shared__ float s_part[kThreads][W];
-    const unsigned lane = threadIdx.x % lanes, group = threadIdx.x / lanes;
-    const size_t r0 = size_t(blockIdx.x) * rows_per_block;
-    size_t r1 = r0 + rows_per_block;
-    if (r1 > rows) r1 = rows;
-    float acc[4][W];
-#pragma unroll
-    for (int p = 0; p < 4; ++p)
-#pragma unroll
-        for (int e = 0; e < W; ++e) acc[p][e] = 0.0f;
-    if (group < groups) {
-        const float* col = g + size_t(lane) * W;
-        size_t r = r0 + group;
-        for (; r + 3 * size_t(groups) < r1; r += 4 * size_t(groups)) {
-            float x[4][W];
-#pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                const float* src = col + (r + size_t(p) * groups) * cols;
-                if (VEC) {
-                    v4f t = *reinterpret_cast<const v4f*>(src);
-#pragma unroll
-                    for (int e = 0; e < W; ++e) x[p][e] = t[e];
-                } else {
-                    x[p][0] = *src;
-                }
-            }
-#pragma unroll
-            for (int p = 0; p < 4; ++p)
-#pragma unroll
-                for (int e = 0; e < W; ++e) acc[p][e] += x[p][e];
-        }
-        for (; r < r1; r += groups) {
-            const float* src = col + r * cols;
-#pragma unroll
-            for (int e = 0; e < W; ++e) acc[0][e] += src[e];
-        }
-    }
-#pragma unroll
-    for (int e = 0; e < W; ++e) s_part[threadIdx.x][e] = (acc[0][e] + acc[1][e]) + (acc[2][e] + acc[3][e]);
-    __syncthreads();
-    if (group == 0) {
-        float t[W];
-#pragma unroll
-        for (int e = 0; e < W; ++e) t[e] = s_part[lane][e];
-        for (unsigned k = 1; k < groups; ++k)
-#pragma unroll
-            for (int e = 0; e < W; ++e) t[e] += s_part[k * lanes + lane][e];
-#pragma unroll
-        for (int e = 0; e < W; ++e) partials[size_t(blockIdx.x) * cols + size_t(lane) * W + e] = t[e];
-    }
+    __shared__ float s_part[kThreads * (VEC ? 4 : 1)];
+    colsum_narrow_body<VEC>(g, partials, rows, cols, lanes, groups, rows_per_block, blockIdx.x, threadIdx.x, s_part);
 }
 
-constexpr int kFoldLanes = 4;    // lanes per column in stage 2
 static_assert(kColsumThreads == kThreads, "the shared body assumes this file's block size");
 // out[c] = sum over the `chunks` rows of partials[., c], in double, LANES lanes per column.  Stage 2
 // of the two-stage sum (LANES = 4), and the whole column sum of a small matrix (LANES = kSmallLanes,
@@ -373,15 +323,9 @@ int ctamd_colsum_f32(const float* g, float* out, size_t rows, size_t cols, void*
     bool vec = (cols % 4 == 0) && aligned16(g);
     const size_t w = vec ? 4 : 1;
     const size_t cus = size_t(compute_units() > 0 ? compute_units() : 256);
-    const size_t lanes = cols / w;                                 // vectors per row
-    if (lanes <= 128) {
-        const size_t groups = kThreads / lanes;
-        size_t rows_per_block = groups * 8;                         // eight rows per thread, four in flight
-        size_t chunks = (rows + rows_per_block - 1) / rows_per_block;
-        if (chunks > 256) {
-            rows_per_block = (rows + 255) / 256;
-            chunks = (rows + rows_per_block - 1) / rows_per_block;
-        }
+    ColsumNarrowPlan narrow;
+    if (colsum_narrow_plan(rows, cols, vec, &narrow)) {
+        const size_t lanes = narrow.lanes, groups = narrow.groups, rows_per_block = narrow.rows_per_block, chunks = narrow.chunks;
         if (vec)
             hipLaunchKernelGGL((colsum_narrow_stage1<true>), dim3((unsigned)chunks), dim3(kThreads), 0, s, g, partials, rows, cols,
                                (unsigned)lanes, (unsigned)groups, rows_per_block);
