@@ -229,31 +229,27 @@ def config_report(with_cpu):
             else:
                 cpu, note = cpu256 * 32, "batch-256 step x32 (every operator is linear in the batch)"
         add("config 3: MLP 784-256-10 train step, batch %d" % Bn, rc, out, cpu, note, launch_bound=(Bn == 256))
-        # each layer (matmul + bias row + ReLU) as one fused operator: same values, fewer launches
-        host.cth_set_fused_layers(1)
-        out = D5()
-        rc = host.cth_time_mlp(fp(x), L(Bn), L(784), fp(W1), fp(b1), L(256), fp(W2), fp(b2), L(10), fp(lab), I(5),
-                               I(30), out)
-        add("config 3: MLP 784-256-10 train step, batch %d, fused layers" % Bn, rc, out, cpu, note, launch_bound=(Bn == 256))
-        # the same with the class-index range check deferred to the loss read (a bad label then gives a
-        # NaN loss instead of an empty tensor): no host wait between the forward and backward passes
-        host.cth_set_ce_deferred_label_check(1)
-        out = D5()
-        rc = host.cth_time_mlp(fp(x), L(Bn), L(784), fp(W1), fp(b1), L(256), fp(W2), fp(b2), L(10), fp(lab), I(5),
-                               I(30), out)
-        host.cth_set_ce_deferred_label_check(0)
-        add("config 3: MLP 784-256-10 train step, batch %d, fused layers, label check deferred to the loss read" % Bn, rc, out,
-            cpu, note, launch_bound=(Bn == 256))
+        # each layer (matmul + bias row + ReLU) as one fused operator: same values, fewer launches; then
         # the last layer, its cross entropy and the gradients that leave them in one pass over the hidden
-        # activations (Tensor::linear_cross_entropy): equal within the MatMul bound, three launches fewer
-        host.cth_set_fused_head(1)
-        for deferred in (0, 1):
-            host.cth_set_ce_deferred_label_check(deferred)
-            out = D5()
-            rc = host.cth_time_mlp(fp(x), L(Bn), L(784), fp(W1), fp(b1), L(256), fp(W2), fp(b2), L(10), fp(lab), I(5),
-                                   I(30), out)
-            add("config 3: MLP 784-256-10 train step, batch %d, fused layers, one-pass head%s"
-                % (Bn, ", label check deferred to the loss read" if deferred else ""), rc, out, cpu, note, launch_bound=(Bn == 256))
+        # activations (Tensor::linear_cross_entropy): equal within the MatMul bound, three launches fewer.
+        # Each in three forms of the class-index range check: indices uploaded from the host (the upload
+        # looked at them: the step waits for nothing, a bad one is refused before anything runs); indices
+        # a device computation produced (the loss kernel's flag is read back between the passes); and
+        # those with the check deferred to the loss read (a bad index then gives a NaN loss instead of an
+        # empty tensor)
+        host.cth_set_fused_layers(1)
+        for head in (0, 1):
+            host.cth_set_fused_head(head)
+            for unseen, deferred, what in ((0, 0, ""), (1, 0, ", class indices from the device (range flag read back mid-step)"),
+                                           (1, 1, ", class indices from the device, range check deferred to the loss read")):
+                host.cth_set_inputs_unseen(unseen)
+                host.cth_set_ce_deferred_label_check(deferred)
+                out = D5()
+                rc = host.cth_time_mlp(fp(x), L(Bn), L(784), fp(W1), fp(b1), L(256), fp(W2), fp(b2), L(10), fp(lab), I(5),
+                                       I(30), out)
+                add("config 3: MLP 784-256-10 train step, batch %d, fused layers%s%s" % (Bn, ", one-pass head" if head else "", what),
+                    rc, out, cpu, note, launch_bound=(Bn == 256))
+        host.cth_set_inputs_unseen(0)
         host.cth_set_ce_deferred_label_check(0)
         host.cth_set_fused_head(0)
         host.cth_set_fused_layers(0)

@@ -85,6 +85,12 @@ void account(double bytes, double flops, bool same_launch = false);
 
 inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 
+// A class index kept as a float, read the way the reference reads it (a conversion to int that truncates
+// toward zero).  NaN: the reference's host turns it into the most negative int, which no class count
+// admits; the conversion instruction here would make it 0, a valid class - so it is mapped out of range.
+// Infinities and magnitudes beyond int saturate on this side and are out of range on both.
+__device__ __forceinline__ int class_index(float t) { return t == t ? int(t) : -1; }
+
 // Grid for a streaming kernel: enough 256-thread blocks to cover `work_items` (each block
 // iteration handles `per_block` items), capped at `waves_per_cu`-deep occupancy of the chip so
 // that grid-stride loops amortise launch cost on large tensors.

@@ -50,7 +50,7 @@ __global__ __launch_bounds__(kThreads) void onehot_kernel(const float* __restric
     const size_t stride = size_t(gridDim.x) * kThreads;
     for (size_t idx = size_t(blockIdx.x) * kThreads + threadIdx.x; idx < rows * classes; idx += stride) {
         const size_t i = idx / classes, j = idx - i * classes;
-        out[idx] = (int64_t(j) == int64_t(int(labels[i]))) ? 1.0f : 0.0f;
+        out[idx] = (int64_t(j) == int64_t(class_index(labels[i]))) ? 1.0f : 0.0f;
     }
 }
 
@@ -78,7 +78,7 @@ __global__ __launch_bounds__(kThreads) void count_correct_kernel(const float* __
                 best = int(j);
             }
         }
-        hit = (best == int(labels[i])) ? 1 : 0;
+        hit = (best == class_index(labels[i])) ? 1 : 0;
     }
     const int wave_hits = __popcll(__ballot(hit));
     if ((threadIdx.x & 63) == 0 && wave_hits) atomicAdd(&s_hits, wave_hits);

@@ -157,7 +157,7 @@ __global__ __launch_bounds__(head_waves(N) * 64) void head_kernel(HeadArgs a) {
 #pragma unroll
         for (int c = 0; c < N; ++c) s = s + __shfl(e_mine, (r_mine * N + c) * kLanesPerValue, 64);
         const float sm = a.fast ? e_mine * (1.0f / s) : cta_div_rcp(e_mine, 1.0 / double(s));
-        const int label = live ? int(a.labels[row_mine]) : 0;
+        const int label = live ? class_index(a.labels[row_mine]) : 0;
         const bool label_ok = label >= 0 && label < N;
         const bool is_class = live && label_ok && label == c_mine;
         const float dz_mine = live ? 0.0f + (sm - (is_class ? 1.0f : 0.0f)) : 0.0f;

@@ -299,7 +299,7 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
             loss = block_sum<THREADS>(loss, s_d);
             block_loss += loss;
         } else if (MODE == kCeIndex) {
-            const int c = int(a.t[row]);
+            const int c = class_index(a.t[row]);
             if (threadIdx.x == 0 && a.stats) {
                 a.stats[2 * row] = m;
                 a.stats[2 * row + 1] = s;
@@ -331,7 +331,7 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
             // the gradient is the one for an upstream gradient of 1 (d * 1.0f is d)
             // (the class index is read here, not earlier: a wait for it right after the next row's
             // loads were issued would wait for those as well)
-            const int c = int(a.t[row]);
+            const int c = class_index(a.t[row]);
             const bool ok = c >= 0 && c < int(a.cols);
             // which of this thread's elements is column c, as one number (k * W + i, or -1): comparing
             // it with each element's constant position keeps 32 column indices out of the registers
@@ -376,7 +376,7 @@ __global__ __launch_bounds__(THREADS) void row_kernel(Args a) {
                     }
                 }
             } else {
-                const int c = int(a.t[row]);
+                const int c = class_index(a.t[row]);
 #pragma unroll
                 for (int k = 0; k < ITEMS; ++k)
 #pragma unroll
@@ -830,7 +830,7 @@ __global__ __launch_bounds__(1024) void row_stream_kernel(Args a) {
             }
             block_loss += block_sum<THREADS>(loss, s_d);
         } else if (MODE == kCeIndex) {
-            const int c = int(a.t[row]);
+            const int c = class_index(a.t[row]);
             if (threadIdx.x == 0 && a.stats) {
                 a.stats[2 * row] = M;
                 a.stats[2 * row + 1] = S;
@@ -845,7 +845,7 @@ __global__ __launch_bounds__(1024) void row_stream_kernel(Args a) {
             }
         } else {
             const float g = a.g1[0];
-            const int c = (MODE == kCeBwdIndex) ? int(a.t[row]) : -1;
+            const int c = (MODE == kCeBwdIndex) ? class_index(a.t[row]) : -1;
             for (size_t j = threadIdx.x; j < a.cols; j += THREADS) {
                 float sm = cta_expf_tab(xr[j] - M, s_exp2) / S;
                 float tj = (MODE == kCeBwdOnehot) ? a.t[row * a.cols + j] : ((j == size_t(c) && c >= 0) ? 1.0f : 0.0f);
@@ -915,7 +915,7 @@ __global__ __launch_bounds__(256) void ce_index_online_kernel(Args a) {
         const float M = block_max<THREADS>(m, s_f[0]);
         s = (m == kNegInf) ? 0.0f : s * __builtin_amdgcn_exp2f((m - M) * kLog2e);
         const float S = block_sum<THREADS>(s, s_f[1]);
-        const int c = int(a.t[row]);
+        const int c = class_index(a.t[row]);
         if (threadIdx.x == 0 && a.stats) {
             a.stats[2 * row] = M;
             a.stats[2 * row + 1] = S;
@@ -954,7 +954,7 @@ __global__ __launch_bounds__(256) void ce_bwd_stats_kernel(Args a) {
         const float M = a.stats[2 * row];
         const double rcp_s = 1.0 / double(a.stats[2 * row + 1]);
         const float rcp_sf = float(rcp_s);
-        const unsigned c = unsigned(int(a.t[row]));
+        const unsigned c = unsigned(class_index(a.t[row]));
         auto one = [&](float v, unsigned j) {
             float sm = FAST ? cta_exp_hw_nonpos(v - M) * rcp_sf
                             : cta_div_rcp(cta_expf_nonpos(v - M, s_exp2), rcp_s);

@@ -6,6 +6,7 @@
 // device storage throws instead of handing a host pointer to HBM.
 #ifndef CTORCH_AMD_HOST_STORAGE_H
 #define CTORCH_AMD_HOST_STORAGE_H
+#include <cmath>
 #include <cstring>
 #include <memory>
 #include <type_traits>
@@ -56,6 +57,11 @@ class Storage {
         bool known = false;
         float value = 0.0f;
         bool frozen = false;    // handed out as a gradient that shares the tape's bytes: read-only while shared
+        // what the host saw when it uploaded the block's floats, read as class indices (converted to int
+        // the way the reference converts them): the least and the greatest, or seen_bad for one that no
+        // class count admits (NaN, an infinity, beyond int)
+        bool seen = false, seen_bad = false;
+        int lo = 0, hi = 0;
         void operator()(char* q) const { ctorch_amd_host::device_release(q, bytes); }
     };
     DeviceBlock* block() const { return _data ? std::get_deleter<DeviceBlock>(_data) : nullptr; }
@@ -76,8 +82,12 @@ class Storage {
     template <typename T>
     Storage(const T* data, size_t size, DType dtype, DeviceType device = DeviceType::kCPU) : Storage(size, dtype, device) {
         if (size > 0 && _data.get()) {
-            if (device == DeviceType::kAMD) ctorch_amd_host::device_copy_h2d(_data.get(), data, size * dtypeSize(dtype));
-            else std::memcpy(_data.get(), data, size * dtypeSize(dtype));
+            if (device == DeviceType::kAMD) {
+                ctorch_amd_host::device_copy_h2d(_data.get(), data, size * dtypeSize(dtype));
+                if (dtype == DType::kFloat && sizeof(T) == sizeof(float)) note_uploaded_floats(reinterpret_cast<const float*>(data), size);
+            } else {
+                std::memcpy(_data.get(), data, size * dtypeSize(dtype));
+            }
         }
     }
 
@@ -121,7 +131,35 @@ class Storage {
         if (b && _size == 1) { b->known = true; b->value = v; }
     }
     void forget_known_value() {
-        if (DeviceBlock* b = block()) b->known = false;
+        if (DeviceBlock* b = block()) { b->known = false; b->seen = false; }
+    }
+    // Class indices uploaded from the host: the upload looked at them (a short vector of floats), so a
+    // loss over them need not wait for the device to say whether they are in range.  1: every element,
+    // converted to int as the reference converts it, lies in [0, classes); 0: some element does not;
+    // -1: the host does not know (the block was computed on the device, written in place since, or is long).
+    int class_indices_below(size_t classes) const {
+        const DeviceBlock* b = block();
+        if (!b || !b->seen) return -1;
+        if (b->seen_bad) return 0;
+        return (b->lo >= 0 && size_t(b->hi) < classes) ? 1 : 0;
+    }
+    static constexpr size_t kLooksAtUploadsUpTo = size_t(1) << 16;
+    void note_uploaded_floats(const float* host, size_t n) {
+        DeviceBlock* b = block();
+        if (!b || n == 0 || n > kLooksAtUploadsUpTo) return;
+        bool bad = false;
+        int lo = 0, hi = 0;
+        for (size_t i = 0; i < n; ++i) {
+            const float v = host[i];
+            if (!(std::fabs(v) < 2147483648.0f)) { bad = true; break; }     // NaN too
+            const int c = static_cast<int>(v);
+            if (i == 0 || c < lo) lo = c;
+            if (i == 0 || c > hi) hi = c;
+        }
+        b->seen = true;
+        b->seen_bad = bad;
+        b->lo = lo;
+        b->hi = hi;
     }
     // A gradient read from the tape shares the tape's bytes.  While more than one tensor holds the
     // block it must not be written in place; the front-end's in-place writers ask here first.
@@ -158,8 +196,12 @@ class Storage {
             Ctorch_Error::throwException(DeviceTypeToErrorPlatform(device), ErrorType::DEVICE_COMPAT, "Storage::to: unsupported device");
         Storage s(_size, _dtype, device);
         if (_size > 0 && _data) {
-            if (device == DeviceType::kAMD) ctorch_amd_host::device_copy_h2d(s._data.get(), _data.get(), nbytes());
-            else ctorch_amd_host::device_copy_d2h(s._data.get(), _data.get(), nbytes());
+            if (device == DeviceType::kAMD) {
+                ctorch_amd_host::device_copy_h2d(s._data.get(), _data.get(), nbytes());
+                if (_dtype == DType::kFloat) s.note_uploaded_floats(reinterpret_cast<const float*>(_data.get()), _size);
+            } else {
+                ctorch_amd_host::device_copy_d2h(s._data.get(), _data.get(), nbytes());
+            }
         }
         return s;
     }

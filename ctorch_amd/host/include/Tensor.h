@@ -74,6 +74,9 @@ class Tensor {
     // throws when this tensor shares a gradient's bytes with the tape (AutoDiff::get_grad): such bytes are read-only
     void require_writable(const char* what);
     const float* known_value() const { return numel() == 1 ? _storage.known_value() : nullptr; }   // null when the host does not know it
+    // 1 / 0: the host saw these floats when it uploaded them and, read as class indices, every one lies /
+    // some do not lie in [0, classes); -1: it does not know (Storage::class_indices_below)
+    int class_indices_below(size_t classes) const { return _storage.class_indices_below(classes); }
     // a tensor on `device` filled from host memory
     static Tensor from_host(const float* data, const std::vector<size_t>& shape, DeviceType device);
 

@@ -101,8 +101,12 @@ Tensor::Tensor(AliasTag, const Tensor& other)
 Tensor Tensor::from_host(const float* data, const std::vector<size_t>& shape, DeviceType device) {
     Tensor t(ShapeTag{}, shape, DType::kFloat, device, false);
     if (t.numel()) {
-        if (device == DeviceType::kAMD) device_copy_h2d(t.fptr(), data, t.numel() * sizeof(float));
-        else std::memcpy(t.data<float>(), data, t.numel() * sizeof(float));
+        if (device == DeviceType::kAMD) {
+            device_copy_h2d(t.fptr(), data, t.numel() * sizeof(float));
+            t._storage.note_uploaded_floats(data, t.numel());
+        } else {
+            std::memcpy(t.data<float>(), data, t.numel() * sizeof(float));
+        }
     }
     return t;
 }

@@ -633,6 +633,11 @@ bool linear_ce_head_fits(const Tensor& h, const Tensor& w, const Tensor& bias, c
 Tensor linear_ce_head(const Tensor& h, const Tensor& w, const Tensor& bias, const Tensor& labels, bool mask_by_h, Tensor* logits,
                       Tensor& dz, Tensor* dh, Tensor& gw, Tensor& gb) {
     const size_t B = h.sizes()[0], H = h.sizes()[1], N = w.sizes()[1];
+    const int labels_ok = labels.class_indices_below(N);       // what the host saw when it uploaded them, if it did
+    if (labels_ok == 0 && !recording() && !g_ce_deferred_check) {
+        Ctorch_Error::log(ErrorLevel::ERROR, kP, ErrorType::TENSOR_STATE, "linear_cross_entropy: class index out of range");
+        return Tensor();
+    }
     Tensor pair(ShapeTag{}, {2}, DType::kFloat, DeviceType::kAMD, false);      // loss and bad-label flag side by side: one transfer
     Tensor loss = Tensor::view_element(pair, 0);
     if (logits) *logits = Tensor(ShapeTag{}, {B, N}, DType::kFloat, DeviceType::kAMD, false);
@@ -645,6 +650,7 @@ Tensor linear_ce_head(const Tensor& h, const Tensor& w, const Tensor& bias, cons
                                  gb.fptr(), B, H, N, current_stream()),
         "linear_cross_entropy");
     if (recording() || g_ce_deferred_check) return loss;     // as CrossEntropy_AMD_kernel: a bad index then shows as a NaN loss
+    if (labels_ok == 1) return loss;                          // nothing to wait for: the indices are known to be in range
     struct { float loss; int32_t bad; } got = {0.0f, 0};
     device_copy_d2h(&got, pair.fptr(), sizeof(got));
     if (got.bad) {
@@ -762,7 +768,15 @@ Tensor CrossEntropy_AMD_kernel(const Tensor& a, const Tensor& b) {
         return r;
     }
     if (b.dim() == 1 && a.dim() == 2 && b.sizes()[0] == a.sizes()[0]) {
-        // loss and bad-index flag side by side: the host has to wait for the flag anyway (a bad index
+        // class indices that came from the host were looked at when they were uploaded: a bad one is
+        // refused here, before anything is computed (as the reference does), and good ones leave the
+        // host nothing to wait for
+        const int labels_ok = b.class_indices_below(a.sizes()[1]);
+        if (labels_ok == 0 && !recording() && !g_ce_deferred_check) {
+            Ctorch_Error::log(ErrorLevel::ERROR, kP, ErrorType::TENSOR_STATE, "CrossEntropy_AMD_kernel: class index out of range");
+            return Tensor();
+        }
+        // loss and bad-index flag side by side: otherwise the host has to wait for the flag (a bad index
         // returns an empty Tensor), so it fetches the loss in the same transfer and item() is free
         Tensor pair(ShapeTag{}, {2}, DType::kFloat, DeviceType::kAMD, false);
         Tensor r = Tensor::view_element(pair, 0);
@@ -783,7 +797,7 @@ Tensor CrossEntropy_AMD_kernel(const Tensor& a, const Tensor& b) {
         // a recorded step cannot wait, and a caller may choose not to (set_ce_deferred_label_check): a
         // bad index then shows as a NaN loss when the loss is read, and the step keeps the GPU busy
         // between its forward and backward passes instead of idling it for the flag's round trip
-        if (recording() || g_ce_deferred_check) return r;
+        if (recording() || g_ce_deferred_check || labels_ok == 1) return r;
         struct { float loss; int32_t bad; } got = {0.0f, 0};
         device_copy_d2h(&got, pair.fptr(), sizeof(got));
         if (got.bad) {

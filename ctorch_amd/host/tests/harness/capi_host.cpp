@@ -28,8 +28,13 @@ std::vector<size_t> shape_of(const long* dims, int nd) {
     return s;
 }
 
+// set: inputs arrive as if a device computation had produced them - the front-end keeps nothing of what
+// the upload saw (whether a short vector holds class indices in range), so range checks run on the device
+bool g_inputs_unseen = false;
 Tensor make(const float* src, const long* dims, int nd) {
-    return Tensor::from_host(src, shape_of(dims, nd), DeviceType::kAMD);
+    Tensor t = Tensor::from_host(src, shape_of(dims, nd), DeviceType::kAMD);
+    if (g_inputs_unseen) t.forget_known_value();
+    return t;
 }
 
 long emit(const Tensor& t, float* dst) {
@@ -114,6 +119,7 @@ void cth_set_fused_expr(int on) { g_fused_expr = on; }
 // class-index cross entropy under a tape: loss and gradient in one pass over the logits (default), or
 // a forward pass that leaves row statistics and a streaming backward pass
 void cth_set_ce_one_pass(int on) { ctorch_amd_host::set_ce_one_pass(on != 0); }
+void cth_set_inputs_unseen(int on) { g_inputs_unseen = on != 0; }
 // sizes of the programs the last Expr::eval() compiled: out[0..3] = forward instructions, forward
 // slots, backward instructions, backward slots (zeros: evaluated operator by operator)
 void cth_last_expr_stats(int* out) {

@@ -1047,6 +1047,11 @@ class HostLayer(Reference):
     def set_ce_one_pass(self, on):
         self.cdll.cth_set_ce_one_pass(int(on))
 
+    def set_inputs_unseen(self, on):
+        """Inputs then reach the front-end as if the device had computed them: what the upload saw of
+        them (class indices in range or not) is forgotten, and range checks run on the device."""
+        self.cdll.cth_set_inputs_unseen(int(on))
+
     def compare(self, cmp, a, b=None, s=0.0):
         """The Tensor comparison operators on the device; returns the bool tensor as uint8, or the
         negative return code."""

@@ -91,6 +91,9 @@ def test_head_edges(oracle):
     lab[7] = 10.0                                                # out of range: status 1, NaN loss, the other rows as usual
     loss, status, z, dz, dh, gw, gb = G.linear_ce_head(G.dev(h), G.dev(w), G.dev(b), G.dev(lab), 0)
     assert status == 1 and np.isnan(float(loss.item()))
+    for wrong in (np.nan, np.inf, -1.0, 3e9):                    # read as the reference reads an index: none of these is a class
+        lab[7] = wrong
+        assert G.linear_ce_head(G.dev(h), G.dev(w), G.dev(b), G.dev(lab), 0)[1] == 1, wrong
     lab[7] = 3.0
     loss, status, z2, dz2, _, _, _ = G.linear_ce_head(G.dev(h), G.dev(w), G.dev(b), G.dev(lab), 0, want_dh=False)
     assert status == 0 and np.isfinite(float(loss.item()))

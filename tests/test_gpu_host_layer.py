@@ -80,6 +80,31 @@ def test_cross_entropy_target_forms_and_errors(oracle, host):
     bad[3] = 31
     assert host.binary(CE, x, bad, ())[0] == -2          # empty Tensor, as the reference
     assert host.binary(CE, x, idx[:5], ())[0] == -2      # incompatible shapes: empty Tensor
+    # class indices the host never saw (a device computation's result): the range check runs on the device
+    host.set_inputs_unseen(True)
+    try:
+        rc, out = host.binary(CE, x, idx, ())
+        assert rc == 1 and abs(out - want) <= 1e-5 * want
+        assert host.binary(CE, x, bad, ())[0] == -2
+        for wrong in (-1.0, 31.5, np.nan, np.inf, -np.inf, 3e9):
+            bad[3] = wrong
+            assert host.binary(CE, x, bad, ())[0] == -2
+    finally:
+        host.set_inputs_unseen(False)
+    for wrong in (-1.0, 31.5, np.nan, np.inf, -np.inf, 3e9):            # and those the upload looked at
+        bad[3] = wrong
+        assert host.binary(CE, x, bad, ())[0] == -2
+    # an index is read by truncation, as the reference reads it: 2.9 is class 2, -0.9 class 0
+    frac = idx.copy()
+    frac[3], frac[4] = 2.9, -0.9
+    whole = idx.copy()
+    whole[3], whole[4] = 2.0, 0.0
+    for unseen in (False, True):
+        host.set_inputs_unseen(unseen)
+        try:
+            assert host.binary(CE, x, frac, ()) == host.binary(CE, x, whole, ())
+        finally:
+            host.set_inputs_unseen(False)
     # backward: one-hot as the reference; class indices are accepted too (the reference throws)
     wantd = oracle.accumulate0(oracle.ce_bwd_onehot(x, oh, F(0.37)))
     for t in (oh, idx):
@@ -579,6 +604,48 @@ def test_mlp_step_with_the_one_pass_head_against_the_oracle(oracle, host, golden
         host.set_fused_layers(False)
     for n, a, b in zip(names, got, want):
         assert np.abs(a - b).max() <= 1e-4 * max(1.0, np.abs(b).max()), n
+
+
+def test_class_indices_seen_at_upload_or_checked_on_the_device(oracle, host, golden):
+    """A step's class indices come from the host (the upload looked at them: nothing to wait for, a bad
+    one refused before anything is computed) or from the device (the loss kernel's flag is read): the
+    same results bit for bit, the same refusal, with the one-pass head and without."""
+    print("case class indices seen / unseen", flush=True)
+    import ctypes as C
+    g = golden("configs")
+    args = (g["mlp_x"], g["mlp_W1"], g["mlp_b1"], g["mlp_W2"], g["mlp_b2"])
+    lab = g["mlp_lab"]
+    bad = lab.copy()
+    bad[5] = 10.0
+
+    def refused(labels):
+        x, W1, b1, W2, b2, t = (np.ascontiguousarray(a, dtype=np.float32) for a in args + (labels,))
+        FP = C.POINTER(C.c_float)
+        fp = lambda a: a.ctypes.data_as(FP)
+        L = C.c_long
+        outs = [np.empty(n, np.float32) for n in (1, x.shape[0] * 10, W1.size, b1.size, W2.size, b2.size)]
+        host.cdll.cth_mlp_step.restype = C.c_long
+        rc = host.cdll.cth_mlp_step(fp(x), L(x.shape[0]), L(x.shape[1]), fp(W1), fp(b1), L(W1.shape[1]), fp(W2), fp(b2), L(10), fp(t),
+                                    *(fp(o) for o in outs), C.c_int(1))
+        return rc < 0
+
+    host.set_fused_layers(True)
+    try:
+        for head in (False, True):
+            host.set_fused_head(head)
+            seen = host.mlp_step(*args, lab, True)
+            assert refused(bad)
+            host.set_inputs_unseen(True)
+            try:
+                unseen = host.mlp_step(*args, lab, True)
+                assert refused(bad)
+            finally:
+                host.set_inputs_unseen(False)
+            for a, b in zip(seen, unseen):
+                assert same_bits(np.asarray(a), np.asarray(b)), head
+    finally:
+        host.set_fused_head(False)
+        host.set_fused_layers(False)
 
 
 def test_reading_a_gradient_the_tape_holds_at_a_pre_activation(oracle, host):

@@ -413,6 +413,17 @@ def test_cross_entropy_edge_cases(oracle):
     assert status == 1 and np.isnan(G.host(loss)[0]) and oracle.ce_index(x, bad) is None
     bad[3] = -1
     assert G.ce_index(G.dev(x), G.dev(bad))[1] == 1
+    # an index is a float read by truncation: NaN, the infinities and magnitudes beyond int are out of
+    # range (the reference's conversion yields the most negative int for them); 30.9 is class 30, -0.9 class 0
+    for wrong in (np.nan, np.inf, -np.inf, 3e9, -3e9, 31.2):
+        bad[3] = wrong
+        assert G.ce_index(G.dev(x), G.dev(bad))[1] == 1 and oracle.ce_index(x, bad) is None, wrong
+        assert G.ce_index_fused(G.dev(x), G.dev(bad))[1] == 1, wrong
+    frac, whole = idx.copy(), idx.copy()
+    frac[3], frac[4], whole[3], whole[4] = 30.9, -0.9, 30.0, 0.0
+    a, b = G.ce_index(G.dev(x), G.dev(frac)), G.ce_index(G.dev(x), G.dev(whole))
+    assert a[1] == 0 and b[1] == 0 and same_bits(G.host(a[0]), G.host(b[0]))
+    assert abs(G.host(a[0])[0] - oracle.ce_index(x, frac)) <= 1e-5 * abs(oracle.ce_index(x, frac))
     # the 1e-10 clamp
     hx = x.copy()
     hx[:, 0] += 60.0
