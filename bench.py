@@ -183,7 +183,10 @@ def config_report(with_cpu):
     for Mm in (1024, 2048, 4096):
         A, B = rng.normal((Mm, Mm), SEEDS["config2"]["A"]), rng.normal((Mm, Mm), SEEDS["config2"]["B"])
         out = D5()
-        rc = host.cth_time_matmul(fp(A), fp(B), L(Mm), I(3), I(10), out)
+        # (some tens of milliseconds of untimed steps first: the chip reaches its clocks only under
+        # sustained matrix work, and a step at 1024 is a tenth of a millisecond)
+        warm, reps = {1024: 300, 2048: 80, 4096: 10}[Mm], {1024: 50, 2048: 20, 4096: 10}[Mm]
+        rc = host.cth_time_matmul(fp(A), fp(B), L(Mm), I(warm), I(reps), out)
         cpu, note = None, None
         if with_cpu:
             # 1024^3 is timed in full; the larger products on a slab of rows, extrapolated (the loop

@@ -1,6 +1,6 @@
 """Per-kernel timings of the launch layer through the C ABI on one MI355X.
 
-    python -m ctorch_amd.kernel_bench [--json] [--skip-matmul] [--only-expr] [--only-declared] [--only-mlp]
+    python -m ctorch_amd.kernel_bench [--json] [--skip-matmul] [--only-matmul] [--only-expr] [--only-declared] [--only-mlp]
 
 Every operator is launched on operands resident in HBM (torch only provides the memory and the
 stream), timed with events over back-to-back launches after a warm-up, and reported as time,
@@ -14,6 +14,7 @@ import argparse
 import ctypes as C
 import json
 import sys
+import time
 
 HBM_PEAK = 8.0e12
 MFMA_F32_PEAK = 157.3e12
@@ -26,6 +27,7 @@ def main():
     ap.add_argument("--only-expr", action="store_true", help="only the fused-expression programs (for counter runs)")
     ap.add_argument("--only-declared", action="store_true",
                     help="only the operators the reference declares without defining: abs .. leaky_relu, reductions along an axis, log_softmax")
+    ap.add_argument("--only-matmul", action="store_true", help="only the fp32 MatMul rows")
     ap.add_argument("--only-mlp", action="store_true",
                     help="only the launches of one 784-256-10 training step at batch 256 and 8192 (the small-product kernels)")
     args = ap.parse_args()
@@ -65,6 +67,37 @@ def main():
             rate = ("%8.1f GB/s %5.1f%% of 8 TB/s" % (e["GB/s"], 100 * e["frac_of_hbm_peak"]) if nbytes is not None else
                     "%8.2f TFLOP/s %5.1f%% of 157.3" % (e["TFLOP/s"], 100 * e["frac_of_mfma_peak"]))
             print("%-44s %9.1f us  %s" % (name, e["us"], rate), flush=True)
+
+    # ---- fp32 MatMul, square, the three operand layouts
+    # (the chip takes some tens of milliseconds of matrix work to reach its clocks: [2048]^3 measured right
+    # after start reads 10% slower than the same launch a little later, so every row first launches for
+    # 40 ms untimed)
+    def warm_up(fn, seconds=0.04):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(10):
+                fn()
+            torch.cuda.synchronize()
+
+    def matmul_rows():
+        for M in (1024, 2048, 4096, 8192):
+            a, b = torch.randn(M, M, device="cuda"), torch.randn(M, M, device="cuda")
+            c = torch.empty(M, M, device="cuda")
+            for name, (x, y) in (("A.B", (a, b)), ("A.B^T", (a, b.t())), ("A^T.B", (a.t(), b))):
+                fn = lambda x=x, y=y: call("ctamd_matmul_f32", P(x), x.stride(0), x.stride(1), P(y), y.stride(0), y.stride(1),
+                                           P(c), M, M, M, S)
+                warm_up(fn)
+                report("matmul %s %d^3" % (name, M), timeit(fn, 20 if M < 8192 else 4, warm=2), flops=2.0 * M ** 3)
+            del a, b, c
+        # not square: a long K over one 64 x 64 tile per CU, and a K that ends inside a k tile
+        for (m, n, k) in ((1024, 1024, 4096), (4096, 4096, 4088)):
+            a, b, c = torch.randn(m, k, device="cuda"), torch.randn(k, n, device="cuda"), torch.empty(m, n, device="cuda")
+            fn = lambda: call("ctamd_matmul_f32", P(a), k, 1, P(b), n, 1, P(c), m, n, k, S)
+            warm_up(fn)
+            report("matmul A.B [%d x %d, K = %d]" % (m, n, k), timeit(fn, 20, warm=2), flops=2.0 * m * n * k)
+            del a, b, c
 
     # ---- the launches of one training step of the 784-256-10 perceptron, each on its own: the fused
     # layers forward, the class-index cross entropy with its gradient, the product with the ReLU mask,
@@ -107,6 +140,11 @@ def main():
                          batch, H, Cn, S), flops=6.0 * batch * H * Cn)
         row("gW2 and gb2 in one call", lambda: mmcs(h.t(), dz, gW2, gb2, H, Cn, batch), flops=2.0 * batch * H * Cn)
         row("gW1 and gb1 in one call", lambda: mmcs(x.t(), dh, gW1, gb1, I, H, batch), flops=2.0 * batch * H * I)
+    if args.only_matmul:
+        matmul_rows()
+        if args.json:
+            print(json.dumps({"device": torch.cuda.get_device_name(0), "results": results}))
+        return 0
     if args.only_mlp:
         for batch in (256, 8192):
             mlp_rows(batch)
@@ -289,17 +327,8 @@ def main():
     del X, Y, G2
     torch.cuda.empty_cache()
 
-    # ---- fp32 MatMul, square, the three operand layouts
     if not args.skip_matmul:
-        for M in (1024, 2048, 4096, 8192):
-            a, b = torch.randn(M, M, device="cuda"), torch.randn(M, M, device="cuda")
-            c = torch.empty(M, M, device="cuda")
-            for name, (x, y) in (("A.B", (a, b)), ("A.B^T", (a, b.t())), ("A^T.B", (a.t(), b))):
-                fn = lambda x=x, y=y: call("ctamd_matmul_f32", P(x), x.stride(0), x.stride(1), P(y), y.stride(0), y.stride(1),
-                                           P(c), M, M, M, S)
-                report("matmul %s %d^3" % (name, M), timeit(fn, 20 if M < 8192 else 4, warm=8 if M < 8192 else 2),
-                       flops=2.0 * M ** 3)
-            del a, b, c
+        matmul_rows()
     if args.json:
         print(json.dumps({"device": torch.cuda.get_device_name(0), "results": results}))
     return 0
