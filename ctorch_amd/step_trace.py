@@ -6,8 +6,8 @@ Meant to be run under `rocprofv3 --kernel-trace`: the trace then shows which ker
 launches, in order, with their start times and durations (the dependent-launch gaps included).
 Prints the front-end's own figure per step (host clock around a step that ends with reading the
 loss) and its count of operator launches.  The steps are the ones bench.py reports: the
-784-256-10 perceptron at batch 256 and 8192 with fused layers and the one-pass classifier head (label
-check deferred to the loss read), and the broadcast expression of configuration 5 as one fused
+784-256-10 perceptron at batch 256 and 8192 with fused layers and the one-pass classifier head (class
+indices uploaded from the host: the step reads no flag back), and the broadcast expression of configuration 5 as one fused
 expression, inputs from the configurations' seeds.
 """
 import ctypes as C
@@ -32,7 +32,6 @@ def main():
     W2, b2 = rng.uniform((256, 10), 313, -1 / 16.0, 1 / 16.0), rng.uniform(10, 314, -1 / 16.0, 1 / 16.0)
     host.cth_set_fused_layers(1)
     host.cth_set_fused_head(1)
-    host.cth_set_ce_deferred_label_check(1)
     for batch in (256, 8192):
         x = f32(rng.ints((batch, 784), 301, 256) / np.float32(255.0))
         lab = rng.ints(batch, 302, 10)
@@ -42,7 +41,6 @@ def main():
         print("MLP 784-256-10 step, batch %d, fused layers, one-pass head: %.1f us per step, %d operator launches" % (batch, out[0] * 1e3, round(out[4])), flush=True)
     host.cth_set_fused_layers(0)
     host.cth_set_fused_head(0)
-    host.cth_set_ce_deferred_label_check(0)
     n = 4096
     X, rv, T = rng.uniform((n, n), 501, -2, 2), rng.uniform(n, 502, 0.5, 2), rng.normal((n, n), 503)
     host.cth_set_fused_expr(1)
