@@ -314,7 +314,11 @@ int ctamd_matmul_bias_f32(const float* a, int64_t as0, int64_t as1, const float*
  * lie in contiguous rows (CTAMD_EINVAL otherwise, nothing launched).  When the product is small enough
  * for the one-launch small-product kernel (at most 256 tiles of 32 x 32, k <= 512), the sums are
  * computed by extra blocks of that launch: one kernel on the chain of dependent launches instead of
- * two.  Every other shape runs the two operators one after the other. */
+ * two.  When the product is cut along K on the 64 x 64 tiles (a long k over a few hundred columns: the
+ * weight gradient of a small layer at a large batch) and b has at most 512 columns in 16-byte aligned
+ * rows, the first stage of the column sum runs as extra blocks of the product's launch and the second as
+ * extra blocks of the launch that adds the parts: two launches instead of four.  Every other shape runs
+ * the two operators one after the other. */
 int ctamd_matmul_colsum_f32(const float* a, int64_t as0, int64_t as1, const float* b, int64_t bs0, int64_t bs1,
                             float* c, float* sums, int64_t m, int64_t n, int64_t k, void* stream);
 
