@@ -654,20 +654,30 @@ def test_comparisons_bit_exact(oracle, n):
 
 
 @pytest.mark.parametrize("m,n,k", [(256, 10, 256), (784, 256, 256), (256, 10, 8192), (784, 16, 1024), (70, 1, 129), (33, 3, 1), (1, 1, 1),
-                                   (31, 33, 512), (100, 70, 513), (512, 512, 64), (300, 7, 3000), (784, 256, 8192)])
+                                   (31, 33, 512), (100, 70, 513), (512, 512, 64), (300, 7, 3000), (784, 256, 8192),
+                                   (520, 128, 5000), (200, 512, 3000), (130, 516, 3000), (64, 64, 100000)])
 def test_product_with_the_column_sums_of_its_second_operand(oracle, m, n, k):
     """The weight gradient x^T . dz and the bias gradient (column sums of dz) from one call: the
     bits of ctamd_matmul_f32 and of ctamd_colsum_f32, whether the sums ride in the product's launch
-    (a product of at most 256 tiles of 32 x 32 with K <= 512) or follow it as launches of their own."""
+    (a product of at most 256 tiles of 32 x 32 with K <= 512), in the two launches of a product cut
+    along K on the 64 x 64 tiles (the last five shapes; 516 columns are one vector too many for that
+    and K = 5000 ends inside a k tile) or follow it as launches of their own."""
     print("case matmul + column sums", m, n, k, flush=True)
     X = oracle.normal((k, m), 61)
     dZ = oracle.normal((k, n), 62)
     dX, dZd = G.dev(X), G.dev(dZ)
+    l = G.lib()
     for name, a in (("x^T as a view", dX.t()), ("x^T materialised", G.dev(np.ascontiguousarray(X.T)))):
+        l.ctamd_counters_reset()
         c, sums = G.matmul_colsum(a, dZd)
+        by, fl, ideal, launches = C.c_double(), C.c_double(), C.c_double(), C.c_uint64()
+        l.ctamd_counters_read(C.byref(by), C.byref(fl), C.byref(ideal), C.byref(launches))
+        # one operator when the sums ride along, two when the column sum follows as its own
+        small = -(-m // 32) * -(-n // 32) <= 256 and k <= 512            # the one-launch small-product kernel
+        rides = small or (m, n, k) in ((784, 256, 8192), (520, 128, 5000), (200, 512, 3000), (64, 64, 100000))
+        assert launches.value == (1 if rides else 2), (name, launches.value)
         assert same_bits(G.host(c), G.host(G.matmul(a, dZd))), name
         assert same_bits(G.host(sums), G.host(G.colsum(dZd))), name
-    l = G.lib()
     # a second operand that is not in contiguous rows: refused before anything is launched
     if n > 1 and k > 1:
         wide = G.dev(oracle.normal((k, n + 3), 63))
