@@ -40,6 +40,10 @@ struct MnistDemoResult {
 
 inline MnistDemoResult run_mnist_demo(const MnistDemoOptions& opt) {
     MnistDemoResult res;
+    // The device first: bringing the GPU runtime up draws from the C library's rand(), and the weights
+    // below must be the ones the reference draws after srand(seed) (mnist/mnist.cpp:24-29, :225) - without
+    // this the first demo of a process trained from other weights than every later one.
+    ctorch_amd_host::init_device();
     srand(opt.seed);
     MNISTLoader loader(opt.dir);
     Tensor train_images, train_labels, test_images, test_labels;

@@ -208,6 +208,25 @@ def test_demo_with_a_recorded_step(host, tmp_path):
     assert same_bits(l1, l2) and same_bits(a1, a2)
 
 
+def test_demo_as_the_first_device_work_of_a_process(host, tmp_path):
+    """The demo seeds the C library's generator and draws its weights from it, as the reference does; bringing
+    the GPU runtime up draws from the same generator, so the device is initialised before the seed is set.
+    A fresh process whose first device work is the demo trains to the same losses as this one."""
+    print("case demo in a fresh process", flush=True)
+    import subprocess
+    import sys
+    write_mnist_dir(str(tmp_path))
+    rc, want, acc, _ = host.mnist_demo(str(tmp_path), epochs=2, lr=1e-3, reference_tape=0)
+    assert rc == 8
+    code = ("import sys; sys.path.insert(0, %r); from support import HostLayer; h = HostLayer(); h.cdll.cth_quiet(); "
+            "rc, l, a, _ = h.mnist_demo(%r, epochs=2, lr=1e-3, reference_tape=0); print('LOSSES', rc, ' '.join(float(v).hex() for v in l))"
+            % (os.path.dirname(os.path.abspath(__file__)), str(tmp_path)))
+    p = subprocess.run([sys.executable, "-c", code], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=110)
+    line = [ln for ln in p.stdout.splitlines() if ln.startswith("LOSSES")]
+    assert p.returncode == 0 and line, p.stdout[-2000:]
+    assert line[0].split()[1] == "8" and line[0].split()[2:] == [float(v).hex() for v in want], (line[0], want)
+
+
 @pytest.mark.parametrize("tag", ["s", "m"])
 def test_training_with_the_one_pass_head(host, golden, tag):
     """The training loop with the last layer and its loss as the one-pass head (class indices instead of
