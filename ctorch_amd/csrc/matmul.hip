@@ -189,7 +189,96 @@ __device__ __forceinline__ float masked(float v, const float* __restrict__ mask,
     return mask ? v * (mask[at] > 0.0f ? 1.0f : 0.0f) : v;
 }
 
-template <class C, bool A_KC, bool B_KC, bool VEC, bool SUMS = false>
+// One k tile of the pipelined loop and of the bounds-checked loop, as text: both start from tile t in LDS,
+// tile t+1 in the staging registers and chunk 0 of tile t fetched, and leave the same for t+1.  (Text, not a
+// lambda: the loop of the whole-K products must compile exactly as if the hand-over below did not exist.)
+// In the pipelined tile with EARLY the buffer cur ^ 1 is free since the last barrier and its first readers
+// wait behind the next, so the staged tile goes to LDS and the next is requested at the top.
+#define CTAMD_PIPELINED_TILE(t) \
+    {   \
+            const int cur = t & 1; \
+            __builtin_amdgcn_sched_barrier(0); \
+            if (C::EARLY) { \
+                sa.store(s_a[cur ^ 1], A_STRIDE); \
+                sb.store(s_b[cur ^ 1], B_STRIDE); \
+                const bool more = t + 3 < ktiles; \
+                sa.load_fast(more ? a_step : 0); \
+                sb.load_fast(more ? b_step : 0); \
+                __builtin_amdgcn_sched_barrier(0); \
+            } \
+            lds_wait(); \
+            fetch_chunk(cur, 1, 1); \
+            mfmas(0); \
+            if (!C::EARLY) { \
+                sa.store(s_a[cur ^ 1], A_STRIDE); \
+                sb.store(s_b[cur ^ 1], B_STRIDE); \
+            } \
+    _Pragma("unroll") \
+            for (int q = 0; q < kReadSlots; ++q) { \
+                __builtin_amdgcn_sched_group_barrier(kMaskMfma, 1, 0); \
+                __builtin_amdgcn_sched_group_barrier(kMaskDsRead, 1, 0); \
+            } \
+            if (C::EARLY) { \
+                if (kMfmaPerChunk - kReadSlots > 0) __builtin_amdgcn_sched_group_barrier(kMaskMfma, kMfmaPerChunk - kReadSlots, 0); \
+            } else { \
+                if (kMfmaPerChunk - kReadSlots - kStores > 0) \
+                    __builtin_amdgcn_sched_group_barrier(kMaskMfma, kMfmaPerChunk - kReadSlots - kStores, 0); \
+    _Pragma("unroll") \
+                for (int q = 0; q < kStores; ++q) { \
+                    __builtin_amdgcn_sched_group_barrier(kMaskMfma, 1, 0); \
+                    __builtin_amdgcn_sched_group_barrier(kMaskDsWrite, 1, 0); \
+                } \
+            } \
+            __builtin_amdgcn_sched_barrier(0); \
+            __syncthreads(); \
+            __builtin_amdgcn_sched_barrier(0); \
+            fetch_chunk(cur ^ 1, 0, 0); \
+            if (!C::EARLY) { \
+                const bool more = t + 3 < ktiles; \
+                sa.load_fast(more ? a_step : 0); \
+                sb.load_fast(more ? b_step : 0); \
+            } \
+            mfmas(1); \
+    _Pragma("unroll") \
+            for (int q = 0; q < kReadSlots; ++q) { \
+                __builtin_amdgcn_sched_group_barrier(kMaskMfma, 1, 1); \
+                __builtin_amdgcn_sched_group_barrier(kMaskDsRead, 1, 1); \
+            } \
+            if (C::EARLY) { \
+                if (kMfmaPerChunk - kReadSlots > 0) __builtin_amdgcn_sched_group_barrier(kMaskMfma, kMfmaPerChunk - kReadSlots, 1); \
+            } else { \
+    _Pragma("unroll") \
+                for (int q = 0; q < kStores; ++q) { \
+                    __builtin_amdgcn_sched_group_barrier(kMaskMfma, 1, 1); \
+                    __builtin_amdgcn_sched_group_barrier(kMaskVmemRead, 1, 1); \
+                } \
+                if (kMfmaPerChunk - kReadSlots - kStores > 0) \
+                    __builtin_amdgcn_sched_group_barrier(kMaskMfma, kMfmaPerChunk - kReadSlots - kStores, 1); \
+            } \
+            __builtin_amdgcn_sched_barrier(0); \
+    }
+#define CTAMD_CHECKED_TILE(t) \
+    {   \
+            const int cur = t & 1; \
+            lds_wait(); \
+            fetch_chunk(cur, 1, 1); \
+            __builtin_amdgcn_sched_barrier(0); \
+            mfmas(0); \
+            __builtin_amdgcn_sched_barrier(0); \
+            sa.store(s_a[cur ^ 1], A_STRIDE); \
+            sb.store(s_b[cur ^ 1], B_STRIDE); \
+            __syncthreads(); \
+            fetch_chunk(cur ^ 1, 0, 0); \
+            if (t + 2 < ktiles) stage_tile(t + 2); \
+            __builtin_amdgcn_sched_barrier(0); \
+            mfmas(1); \
+            __builtin_amdgcn_sched_barrier(0); \
+    }
+// RAGGED: the launch's K is no whole number of k tiles (and rows are aligned): blocks inside C keep the
+// pipelined loop for their whole k tiles and finish on the bounds-checked one.  A kernel of its own
+// because the hand-over, merely by being there, cost the loop of the whole-K products 0.9% (registers
+// and address arithmetic around the same 64 MFMAs: 4096^3 955 -> 962 us).
+template <class C, bool A_KC, bool B_KC, bool VEC, bool SUMS = false, bool RAGGED = false>
 __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(GemmArgs g) {
     constexpr int BM = C::BM, BN = C::BN, BK = C::BK, TM = C::TM, TN = C::TN;
     constexpr int A_STRIDE = A_KC ? C::KPAD : C::XPAD_M;
@@ -249,15 +338,11 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
     Stage<BM, BK, A_KC, C::THREADS> sa;
     Stage<BN, BK, B_KC, C::THREADS> sb;
     const int ktiles = (k_end - k_begin + BK - 1) / BK;
-    const int whole_ktiles = (k_end - k_begin) / BK;
-    // interior: the whole BM x BN tile lies inside C and rows are 16-byte aligned - true for all blocks
-    // of a 4096^3 product, false only on ragged edges.  The pipelined loop then runs while the k tile it
-    // requests (two ahead) is a whole one; a K that ends inside a k tile leaves the last iterations to
-    // the bounds-checked loop below, which takes over the same state (tile t in LDS, tile t+1 in the
-    // staging registers, chunk 0 of tile t fetched).
-    const bool interior = VEC && m0 + BM <= g.m && n0 + BN <= g.n && (whole_ktiles == ktiles || whole_ktiles >= 2) &&
+    // interior: the whole BM x BN tile lies inside C, rows are 16-byte aligned and K is a whole number of k
+    // tiles (RAGGED: at least two whole ones) - true for all blocks of a 4096^3 product, false only on ragged edges
+    const bool interior = VEC && m0 + BM <= g.m && n0 + BN <= g.n &&
+                          (RAGGED ? ((k_end - k_begin) % BK == 0 || (k_end - k_begin) / BK >= 2) : (k_end - k_begin) % BK == 0) &&
                           g.lda < (int64_t(1) << 21) && g.ldb < (int64_t(1) << 21);   // tile extent < 2^32 bytes
-    const int fast_iters = !interior ? 0 : whole_ktiles == ktiles ? ktiles - 1 : whole_ktiles - 2;
     const int64_t a_step = (A_KC ? BK : int64_t(BK) * g.lda) * 4;   // bytes per k tile
     const int64_t b_step = (B_KC ? BK : int64_t(BK) * g.ldb) * 4;
     if (interior) {
@@ -307,109 +392,58 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
     // is a wait in front of an MFMA for data requested just before it.  Interior blocks pin the
     // interleaving with scheduling groups; the two waves of a SIMD run in phase (one barrier per
     // tile), so housekeeping outside the bursts would idle the pipe for both.
-    auto stage_tile = [&](int kt) {
-        sa.template load<VEC>(g.a, g.lda, m0, k_begin + kt * BK, g.m, k_end);
-        sb.template load<VEC>(g.b, g.ldb, n0, k_begin + kt * BK, g.n, k_end);
-    };
-    int t = 0;
-    if (interior) {
-        sa.load_fast(a_step);
-        sb.load_fast(b_step);
-        sa.store(s_a[0], A_STRIDE);
-        sb.store(s_b[0], B_STRIDE);
-        __syncthreads();
-        // the loop always requests tile t+2; past the end the request repeats the last tile
-        // (in bounds, never stored), which keeps the loop body free of branches
-        if (ktiles > 1) { sa.load_fast(ktiles > 2 ? a_step : 0); sb.load_fast(ktiles > 2 ? b_step : 0); }
-        fetch_chunk(0, 0, 0);
-        for (; t < fast_iters; ++t) {
-            const int cur = t & 1;
-            __builtin_amdgcn_sched_barrier(0);
-            if (C::EARLY) {
-                // buffer cur ^ 1 is free since the last barrier; its first readers wait behind the next
-                sa.store(s_a[cur ^ 1], A_STRIDE);
-                sb.store(s_b[cur ^ 1], B_STRIDE);
-                const bool more = t + 3 < ktiles;
-                sa.load_fast(more ? a_step : 0);
-                sb.load_fast(more ? b_step : 0);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            lds_wait();
-            fetch_chunk(cur, 1, 1);
-            mfmas(0);
-            if (!C::EARLY) {
-                sa.store(s_a[cur ^ 1], A_STRIDE);
-                sb.store(s_b[cur ^ 1], B_STRIDE);
-            }
-#pragma unroll
-            for (int q = 0; q < kReadSlots; ++q) {
-                __builtin_amdgcn_sched_group_barrier(kMaskMfma, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(kMaskDsRead, 1, 0);
-            }
-            if (C::EARLY) {
-                if (kMfmaPerChunk - kReadSlots > 0) __builtin_amdgcn_sched_group_barrier(kMaskMfma, kMfmaPerChunk - kReadSlots, 0);
-            } else {
-                if (kMfmaPerChunk - kReadSlots - kStores > 0)
-                    __builtin_amdgcn_sched_group_barrier(kMaskMfma, kMfmaPerChunk - kReadSlots - kStores, 0);
-#pragma unroll
-                for (int q = 0; q < kStores; ++q) {
-                    __builtin_amdgcn_sched_group_barrier(kMaskMfma, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(kMaskDsWrite, 1, 0);
-                }
-            }
-            __builtin_amdgcn_sched_barrier(0);
+    const int64_t span_k = k_end - k_begin;
+    if constexpr (!RAGGED) {
+        if (interior) {
+            sa.load_fast(a_step);
+            sb.load_fast(b_step);
+            sa.store(s_a[0], A_STRIDE);
+            sb.store(s_b[0], B_STRIDE);
             __syncthreads();
-            __builtin_amdgcn_sched_barrier(0);
-            fetch_chunk(cur ^ 1, 0, 0);
-            if (!C::EARLY) {
-                const bool more = t + 3 < ktiles;
-                sa.load_fast(more ? a_step : 0);
-                sb.load_fast(more ? b_step : 0);
-            }
-            mfmas(1);
-#pragma unroll
-            for (int q = 0; q < kReadSlots; ++q) {
-                __builtin_amdgcn_sched_group_barrier(kMaskMfma, 1, 1);
-                __builtin_amdgcn_sched_group_barrier(kMaskDsRead, 1, 1);
-            }
-            if (C::EARLY) {
-                if (kMfmaPerChunk - kReadSlots > 0) __builtin_amdgcn_sched_group_barrier(kMaskMfma, kMfmaPerChunk - kReadSlots, 1);
-            } else {
-#pragma unroll
-                for (int q = 0; q < kStores; ++q) {
-                    __builtin_amdgcn_sched_group_barrier(kMaskMfma, 1, 1);
-                    __builtin_amdgcn_sched_group_barrier(kMaskVmemRead, 1, 1);
-                }
-                if (kMfmaPerChunk - kReadSlots - kStores > 0)
-                    __builtin_amdgcn_sched_group_barrier(kMaskMfma, kMfmaPerChunk - kReadSlots - kStores, 1);
-            }
-            __builtin_amdgcn_sched_barrier(0);
+            // the loop always requests tile t+2; past the end the request repeats the last tile
+            // (in bounds, never stored), which keeps the loop body free of branches
+            if (ktiles > 1) { sa.load_fast(ktiles > 2 ? a_step : 0); sb.load_fast(ktiles > 2 ? b_step : 0); }
+            fetch_chunk(0, 0, 0);
+            for (int t = 0; t + 1 < ktiles; ++t) CTAMD_PIPELINED_TILE(t)
+        } else {
+            auto stage_tile = [&](int kt) {
+                sa.template load<VEC>(g.a, g.lda, m0, k_begin + kt * BK, g.m, k_end);
+                sb.template load<VEC>(g.b, g.ldb, n0, k_begin + kt * BK, g.n, k_end);
+            };
+            stage_tile(0);
+            sa.store(s_a[0], A_STRIDE);
+            sb.store(s_b[0], B_STRIDE);
+            __syncthreads();
+            if (ktiles > 1) stage_tile(1);
+            fetch_chunk(0, 0, 0);
+            for (int t = 0; t + 1 < ktiles; ++t) CTAMD_CHECKED_TILE(t)
         }
     } else {
-        stage_tile(0);
-        sa.store(s_a[0], A_STRIDE);
-        sb.store(s_b[0], B_STRIDE);
-        __syncthreads();
-        if (ktiles > 1) stage_tile(1);
-        fetch_chunk(0, 0, 0);
-    }
-    {
-        for (; t + 1 < ktiles; ++t) {
-            const int cur = t & 1;
-            lds_wait();
-            fetch_chunk(cur, 1, 1);
-            __builtin_amdgcn_sched_barrier(0);
-            mfmas(0);
-            __builtin_amdgcn_sched_barrier(0);
-            sa.store(s_a[cur ^ 1], A_STRIDE);
-            sb.store(s_b[cur ^ 1], B_STRIDE);
+        auto stage_tile = [&](int kt) {
+            sa.template load<VEC>(g.a, g.lda, m0, k_begin + kt * BK, g.m, k_end);
+            sb.template load<VEC>(g.b, g.ldb, n0, k_begin + kt * BK, g.n, k_end);
+        };
+        int t = 0;
+        if (interior) {
+            sa.load_fast(a_step);
+            sb.load_fast(b_step);
+            sa.store(s_a[0], A_STRIDE);
+            sb.store(s_b[0], B_STRIDE);
             __syncthreads();
-            fetch_chunk(cur ^ 1, 0, 0);
-            if (t + 2 < ktiles) stage_tile(t + 2);
-            __builtin_amdgcn_sched_barrier(0);
-            mfmas(1);
-            __builtin_amdgcn_sched_barrier(0);
+            if (ktiles > 1) { sa.load_fast(ktiles > 2 ? a_step : 0); sb.load_fast(ktiles > 2 ? b_step : 0); }
+            fetch_chunk(0, 0, 0);
+            // the pipelined loop while the tile it requests, two ahead, is a whole one
+            const int fast_iters = span_k % BK == 0 ? ktiles - 1 : int(span_k / BK) - 2;
+            for (; t < fast_iters; ++t) CTAMD_PIPELINED_TILE(t)
+        } else {
+            stage_tile(0);
+            sa.store(s_a[0], A_STRIDE);
+            sb.store(s_b[0], B_STRIDE);
+            __syncthreads();
+            if (ktiles > 1) stage_tile(1);
+            fetch_chunk(0, 0, 0);
         }
+        for (; t + 1 < ktiles; ++t) CTAMD_CHECKED_TILE(t)
     }
     // last k tile: nothing left to stage
     {
@@ -479,6 +513,9 @@ __global__ __launch_bounds__(C::THREADS, kMinWavesPerSimd) void gemm_kernel(Gemm
             }
         }
 }
+
+#undef CTAMD_PIPELINED_TILE
+#undef CTAMD_CHECKED_TILE
 
 // Adds the parts of the split tiles in their order and writes C (bias and ReLU of the fused
 // product included): blockIdx.x is the split tile, blockIdx.y one of its slices of kFoldSlice elements.
@@ -932,11 +969,21 @@ using WideTile = Cfg<256, 128, 16, 128, 64>;
 // 128 x 128 tile either way)
 using TinyEarlyTile = Cfg<64, 64, 16, 32, 32, true>;
 using TinyK4Tile = Cfg<64, 64, 16, 32, 32, true, 4>;
-using SmallK2Tile = Cfg<128, 128, 16, 64, 64, false, 2>;
+// the 128 x 128 tile for a launch of at most one block per CU: eight waves of 64 x 32 (2048^3: 129 / 133 us
+// for A.B / A^T.B against 138 / 141 on the four-wave block and 131.5 / 135 on that block with two wave
+// groups; [2048 x 2048, K = 256] 22.9 against 25.7 us), and for two K-contiguous operands with a long K
+// sixteen: the same eight in two wave groups (A.B^T 2048^3 130.0 against 133.4 us)
+using Small8Tile = Cfg<128, 128, 16, 64, 32, true>;
+using Small16Tile = Cfg<128, 128, 16, 64, 32, false, 2>;
+// the 256 x 256 tile as sixteen waves of 64 x 64, four per SIMD, for A.B^T and A^T.B: 4096^3 939 / 966 us
+// against 956 / 976 on the eight-wave block, 8192^3 7.42 / 7.63 against 7.55 / 7.69 ms (A.B loses 4% on it)
+using Big16Tile = Cfg<256, 256, 16, 64, 64, true>;
 
 template <class Tile, bool A_KC, bool B_KC>
 int launch_gemm(GemmArgs g, bool vec, int blocks, hipStream_t s) {
-    if (vec) hipLaunchKernelGGL((gemm_kernel<Tile, A_KC, B_KC, true>), dim3(unsigned(blocks)), dim3(Tile::THREADS), 0, s, g);
+    const bool ragged = g.k % Tile::BK != 0;        // parts of a cut K are whole k tiles each, but for the last
+    if (vec && ragged) hipLaunchKernelGGL((gemm_kernel<Tile, A_KC, B_KC, true, false, true>), dim3(unsigned(blocks)), dim3(Tile::THREADS), 0, s, g);
+    else if (vec) hipLaunchKernelGGL((gemm_kernel<Tile, A_KC, B_KC, true>), dim3(unsigned(blocks)), dim3(Tile::THREADS), 0, s, g);
     else hipLaunchKernelGGL((gemm_kernel<Tile, A_KC, B_KC, false>), dim3(unsigned(blocks)), dim3(Tile::THREADS), 0, s, g);
     return launched("ctamd_matmul_f32");
 }
@@ -1065,16 +1112,17 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
     //                      the memory latencies a block waits out before its first and after its last k tile
     //   adding the parts   a launch and the parts' bytes written and read once
     // parts fill the free places of the round with at least 8 k tiles each (4 when K allows no more).
-    // A launch of at most one block per CU on the 64 x 64 or 128 x 128 tiles runs on their kernels with
-    // 4 (2) wave groups per block when each block has a long enough run of K: measured 1024^3 26 -> 24 us, [1024 x 1024, K = 4096] 88 -> 76 us, 2048^3 138 -> 134 us
-    // (and 153 us on four 64 x 64 tiles per CU, which the old figure for a lone 128 x 128 block preferred).
+    // A launch of at most one block per CU runs on kernels made for that: the 64 x 64 tile with four wave
+    // groups per block when each block has a long enough run of K (1024^3 26 -> 24 us, [1024 x 1024,
+    // K = 4096] 88 -> 76 us), the 128 x 128 tile as eight waves of 64 x 32, in two wave groups for two
+    // K-contiguous operands with a long K (2048^3 138 - 141 -> 129 - 133 us; 153 us on four 64 x 64 tiles
+    // per CU, which the old figure for a lone 128 x 128 block preferred).
     auto wave_groups = [&](int sh, int64_t blocks, int parts) -> int {
         if (blocks > cus || sh > 1) return 1;
         const int64_t run = (k + parts - 1) / parts;
         if (sh == 0) return run >= 512 ? 4 : 1;
-        return run >= 1024 ? 2 : 1;
+        return (A_KC && B_KC && run >= 1024) ? 2 : 1;
     };
-    static const double alone_grouped[2][5] = {{0, 0, 0, 0, 1.32}, {0, 0, 1.09, 0, 0}};   // [shape][groups]
     struct Shape { int bm, bn, together; double per_flop, alone; };
     static const Shape shapes[4] = {{TinyTile::BM, TinyTile::BN, 4, 1.30, 1.70}, {SmallTile::BM, SmallTile::BN, 2, 1.07, 1.34},
                                     {BigTile::BM, BigTile::BN, 1, 1.00, 1.00}, {WideTile::BM, WideTile::BN, 2, 1.04, 1.32}};
@@ -1107,7 +1155,10 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
             if (left > 0) {
                 const int64_t c = (left * parts + cus - 1) / cus;
                 kg = rounds == 0 ? wave_groups(sh, left * parts, parts) : 1;
-                const double alone = kg > 1 ? alone_grouped[sh][kg] : q.alone;
+                const bool one_per_cu = rounds == 0 && left * parts <= cus;
+                // (fitted at [2048 x 2048]: 8.7 us + 60 us per 1024 of K for the uncut eight-wave block; a cut
+                // one keeps the four-wave block's figure, which its measured times are nearer to)
+                const double alone = sh == 0 ? (kg == 4 ? 1.32 : q.alone) : (sh == 1 && one_per_cu && parts == 1) ? 1.08 : q.alone;
                 const double busy = q.together == 1 ? alone
                                                     : alone + double(c - 1) * (q.together * q.per_flop - alone) / (q.together - 1);
                 cost += busy * area * t_elem / parts + (rounds == 0 ? 3e-6 : 1e-6);
@@ -1169,7 +1220,10 @@ int matmul_impl(const char* name, const float* a, int64_t as0, int64_t as1, cons
         return launched(name);
     }
     int rc = groups == 4 ? launch_layout<TinyK4Tile>(g, A_KC, B_KC, vec, blocks, s)
-           : groups == 2 ? launch_layout<SmallK2Tile>(g, A_KC, B_KC, vec, blocks, s)
+           : groups == 2 ? launch_gemm<Small16Tile, true, true>(g, vec, blocks, s)
+           : (shape == 1 && blocks <= cus) ? launch_layout<Small8Tile>(g, A_KC, B_KC, vec, blocks, s)
+           : (shape == 2 && A_KC && B_KC) ? launch_gemm<Big16Tile, true, true>(g, vec, blocks, s)
+           : (shape == 2 && !A_KC && !B_KC) ? launch_gemm<Big16Tile, false, false>(g, vec, blocks, s)
            : (shape == 0 && blocks <= cus) ? launch_layout<TinyEarlyTile>(g, A_KC, B_KC, vec, blocks, s)
            : shape == 3 ? launch_layout<WideTile>(g, A_KC, B_KC, vec, blocks, s)
            : shape == 2 ? launch_layout<BigTile>(g, A_KC, B_KC, vec, blocks, s)
