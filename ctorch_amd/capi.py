@@ -20,6 +20,7 @@ PROTOTYPES = {
     "ctamd_free": [_P],
     "ctamd_memcpy_h2d": [_P, _P, _Z, _P],
     "ctamd_memcpy_d2h": [_P, _P, _Z, _P],
+    "ctamd_read_small": [_P, _P, _Z, _P],
     "ctamd_memcpy_d2d": [_P, _P, _Z, _P],
     "ctamd_sync": [_P],
     "ctamd_set_math_mode": [C.c_int],

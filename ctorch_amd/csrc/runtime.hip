@@ -328,4 +328,20 @@ int ctamd_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream) {
 }
 int ctamd_sync(void* stream) { return check_hip(hipStreamSynchronize(as_stream(stream)), "hipStreamSynchronize"); }
 
+int ctamd_read_small(void* dst_host, const void* src, size_t bytes, void* stream) {
+    if (bytes == 0) return CTAMD_OK;
+    if (!dst_host || !src) return fail(CTAMD_EINVAL, "ctamd_read_small: null pointer");
+    if (bytes > CTAMD_READ_SMALL_MAX) return fail(CTAMD_ERANGE, "ctamd_read_small: %zu bytes, at most %d", bytes, CTAMD_READ_SMALL_MAX);
+    // one page-locked landing buffer per host thread, allocated on the thread's first read and kept
+    thread_local void* landing = nullptr;
+    if (!landing) {
+        int rc = check_hip(hipHostMalloc(&landing, CTAMD_READ_SMALL_MAX, hipHostMallocDefault), "hipHostMalloc(landing buffer)");
+        if (rc) { landing = nullptr; return rc; }
+    }
+    int rc = check_hip(hipMemcpyAsync(landing, src, bytes, hipMemcpyDeviceToHost, as_stream(stream)), "ctamd_read_small");
+    if (!rc) rc = check_hip(hipStreamSynchronize(as_stream(stream)), "ctamd_read_small: hipStreamSynchronize");
+    if (!rc) memcpy(dst_host, landing, bytes);
+    return rc;
+}
+
 }  // extern "C"

@@ -77,6 +77,13 @@ int ctamd_memcpy_h2d(void* dst, const void* src_host, size_t bytes, void* stream
 int ctamd_memcpy_d2h(void* dst_host, const void* src, size_t bytes, void* stream);
 int ctamd_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream);
 int ctamd_sync(void* stream);
+/* Tensor::item<T>() (include/Tensor.h:642-660) and the other reads of a few bytes that a training loop
+ * makes every step (a loss, a Dot, a status word): `bytes` <= CTAMD_READ_SMALL_MAX from device memory into
+ * host memory once the work queued on `stream` is done.  The copy goes into a page-locked buffer the
+ * library keeps per host thread, so it is queued behind that work at once and the host waits a single
+ * time; a copy into pageable memory makes the host wait for the stream, copy, and wait again. */
+#define CTAMD_READ_SMALL_MAX 256
+int ctamd_read_small(void* dst_host, const void* src, size_t bytes, void* stream);
 
 /* Streams and recorded launch sequences, with no counterpart in the reference (which is
  * synchronous): a caller whose step is a fixed sequence of small launches (a training step at a

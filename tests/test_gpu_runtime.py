@@ -75,3 +75,43 @@ def test_a_destroyed_foreign_stream_is_never_touched_again(oracle):
         assert (G.host(out)[:3] == want).all()
     finally:
         L.ctamd_stream_destroy(s2)
+
+
+def test_small_reads_land_behind_the_queued_work(oracle):
+    """ctamd_read_small: a few bytes read after the work queued on a stream, through the page-locked buffer
+    the library keeps per host thread - the value of the kernel launched just before, from several host
+    threads, and the refusals."""
+    print("case small reads", flush=True)
+    import threading
+    L = G.lib()
+    a = G.dev(oracle.uniform((1 << 20,), 73, -1, 1))
+    b = G.dev(oracle.uniform((1 << 20,), 74, -1, 1))
+    out = torch.zeros(4, device=G.DEV)
+    want = np.float32(np.dot(G.host(a).astype(np.float64), G.host(b).astype(np.float64)))
+    got = (C.c_float * 4)()
+    for _ in range(5):
+        out.zero_()
+        G.call("ctamd_dot_f32", G.ptr(a), G.ptr(b), G.ptr(out), 1 << 20, G.stream())
+        assert L.ctamd_read_small(got, G.ptr(out), 16, G.stream()) == 0
+        assert abs(got[0] - want) <= 1e-6 * abs(want) + 1e-6 and got[1] == 0.0
+    raw = torch.arange(64, dtype=torch.float32, device=G.DEV)
+    wide = (C.c_float * 64)()
+    assert L.ctamd_read_small(wide, G.ptr(raw), 256, G.stream()) == 0 and list(wide) == [float(i) for i in range(64)]
+    assert L.ctamd_read_small(wide, G.ptr(raw), 0, G.stream()) == 0
+    assert L.ctamd_read_small(wide, G.ptr(torch.zeros(128, device=G.DEV)), 260, G.stream()) == -5
+    assert L.ctamd_read_small(None, G.ptr(raw), 4, G.stream()) == -1 and L.ctamd_read_small(wide, None, 4, G.stream()) == -1
+    torch.cuda.synchronize()
+    # every host thread has a landing buffer of its own
+    results = {}
+
+    def worker(i):
+        mine = (C.c_float * 1)()
+        ok = all(L.ctamd_read_small(mine, C.c_void_p(raw.data_ptr() + 4 * i), 4, G.stream()) == 0 and mine[0] == float(i) for _ in range(50))
+        results[i] = ok
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(1, 5)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert results == {1: True, 2: True, 3: True, 4: True}
