@@ -254,6 +254,19 @@ def config_report(with_cpu):
                     rc, out, cpu, note, launch_bound=(Bn == 256))
         host.cth_set_inputs_unseen(0)
         host.cth_set_ce_deferred_label_check(0)
+        # the same steps queued back to back, the loss not read until all of them are issued (a loop that adds
+        # its losses up on the device, as the MNIST demo here does): the host runs ahead, the device never waits
+        # for it, and a step costs the larger of the host's time to issue it and the device's time to run it
+        host.cth_set_no_loss_read(1)
+        for fused, head, what in ((0, 0, ""), (1, 1, ", fused layers, one-pass head")):
+            host.cth_set_fused_layers(fused)
+            host.cth_set_fused_head(head)
+            out = D5()
+            rc = host.cth_time_mlp(fp(x), L(Bn), L(784), fp(W1), fp(b1), L(256), fp(W2), fp(b2), L(10), fp(lab), I(20),
+                                   I(200), out)
+            add("config 3: MLP 784-256-10 train step, batch %d%s, steps queued back to back (no loss read per step)" % (Bn, what),
+                rc, out, cpu, note, launch_bound=(Bn == 256))
+        host.cth_set_no_loss_read(0)
         host.cth_set_fused_head(0)
         host.cth_set_fused_layers(0)
         # the same step (one-hot targets) recorded into a HIP graph once and replayed

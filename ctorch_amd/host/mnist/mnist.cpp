@@ -2,7 +2,7 @@
 // printed results, data set and parameters resident in HBM.
 //
 //   mnist.bin [--data DIR] [--epochs N] [--batch N] [--lr X] [--hidden1 N] [--hidden2 N]
-//             [--reference-tape | --graph] [--fused | --fused-head]
+//             [--reference-tape | --graph] [--fused | --fused-head] [--loss-each-step]
 //
 // --graph records one training step into a HIP graph at the first batch and replays it for every
 // batch: one launch per step instead of about fifty.
@@ -35,6 +35,7 @@ int main(int argc, char** argv) {
         else if (a == "--graph") opt.use_graph = true;
         else if (a == "--fused") opt.fused_layers = true;
         else if (a == "--fused-head") opt.fused_layers = opt.fused_head = true;
+        else if (a == "--loss-each-step") opt.loss_on_device = false;
         else {
             std::fprintf(stderr, "unknown option %s\n", a.c_str());
             return 2;

@@ -28,6 +28,12 @@ struct MnistDemoOptions {
     bool fused_layers = false;
     // with fused_layers: the last layer and its loss as the one-pass head (Tensor::linear_cross_entropy)
     bool fused_head = false;
+    // true (the default): the batch losses of an epoch are added up on the device, in the order and
+    // precision the reference adds them on the host (fp32, batch after batch), and read once per epoch -
+    // no step makes the host wait, so the host runs ahead and the device never idles between steps.
+    // false: every step reads its loss, as the reference's loop does for its progress line
+    // (mnist/mnist.cpp:253-260).
+    bool loss_on_device = true;
 };
 
 struct MnistDemoResult {
@@ -75,6 +81,8 @@ inline MnistDemoResult run_mnist_demo(const MnistDemoOptions& opt) {
     auto t0 = std::chrono::steady_clock::now();
     for (int epoch = 0; epoch < opt.epochs; ++epoch) {
         float epoch_loss = 0.0f;
+        Tensor epoch_sum;                   // with loss_on_device: epoch_loss as a device scalar
+        if (opt.loss_on_device && !opt.use_graph) epoch_sum = ctorch_amd_host::filled({}, 0.0f, DeviceType::kAMD);
         for (int batch = 0; batch < res.num_batches; ++batch) {
             Tensor batch_images, batch_labels;
             get_batch(train_images, train_labels, opt.batch_size, batch, batch_images, batch_labels);
@@ -89,9 +97,15 @@ inline MnistDemoResult run_mnist_demo(const MnistDemoOptions& opt) {
                 epoch_loss += staged_loss.item<float>();
                 continue;
             }
-            epoch_loss += model.train_step(batch_images, batch_labels);
+            if (opt.loss_on_device) {
+                Tensor loss = model.train_step_on_device(batch_images, batch_labels);
+                ctorch_amd_host::accumulate(epoch_sum, loss);       // epoch_sum = epoch_sum + loss, the same fp32 addition
+            } else {
+                epoch_loss += model.train_step(batch_images, batch_labels);
+            }
             if (!opt.reference_tape) autodiff.clear_graph();
         }
+        if (opt.loss_on_device && !opt.use_graph && res.num_batches > 0) epoch_loss = epoch_sum.item<float>();
         epoch_loss /= static_cast<float>(res.num_batches);
         res.epoch_loss.push_back(epoch_loss);
     }

@@ -1425,6 +1425,7 @@ long cth_mnist_demo(const char* dir, int epochs, int batch, float lr, int hidden
         const int reference_tape = mode_bits & 3;
         opt.fused_layers = (mode_bits & 4) != 0;
         opt.fused_head = (mode_bits & 8) != 0;
+        opt.loss_on_device = (mode_bits & 16) == 0;       // 16: every step reads its loss
         opt.reference_tape = reference_tape == 1;
         opt.use_graph = reference_tape == 2;          // 2: live leaves and the step replayed from a recorded graph
         MnistDemoResult r = run_mnist_demo(opt);

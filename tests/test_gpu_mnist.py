@@ -208,6 +208,20 @@ def test_demo_with_a_recorded_step(host, tmp_path):
     assert same_bits(l1, l2) and same_bits(a1, a2)
 
 
+def test_demo_adds_its_epoch_loss_on_the_device(host, tmp_path):
+    """The demo adds the batch losses of an epoch on the device (the reference's fp32 additions in the
+    reference's order) and reads the sum once per epoch; with every step reading its loss instead (mode
+    bit 16) the epoch losses and accuracies are the same bits - operator by operator, with fused layers
+    and with the one-pass head."""
+    print("case demo epoch loss on the device", flush=True)
+    write_mnist_dir(str(tmp_path))
+    for mode in (0, 4, 12):
+        rc1, l1, a1, _ = host.mnist_demo(str(tmp_path), epochs=3, lr=1e-3, reference_tape=mode)
+        rc2, l2, a2, _ = host.mnist_demo(str(tmp_path), epochs=3, lr=1e-3, reference_tape=mode + 16)
+        assert rc1 == rc2 == 12, mode
+        assert same_bits(l1, l2) and same_bits(a1, a2), mode
+
+
 def test_demo_as_the_first_device_work_of_a_process(host, tmp_path):
     """The demo seeds the C library's generator and draws its weights from it, as the reference does; bringing
     the GPU runtime up draws from the same generator, so the device is initialised before the seed is set.
