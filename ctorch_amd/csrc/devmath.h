@@ -335,29 +335,38 @@ CTA_FN float cta_tanf(float y, const uint32_t* inv_pio4) {
 
 // ----------------------------------------------------------------------------------------------
 // Single-precision sine / cosine for |y| < 120 (cta_sincos_is_rare(y) == 0), for the kernels whose
-// time the double-precision routines above would set (fused expressions).  y = j pi + r with j the
-// nearest integer (sine) or the nearest integer plus a half (cosine) and |r| <= pi/2 (1 + 1e-5):
-// sin y = (-1)^k sin r, cos y = (-1)^(k+1) sin r.  pi is split in three floats whose first two have 17
-// significant bits, so the first step of the reduction is exact and the second loses half an ulp
-// of r at most; sin r is one odd polynomial of degree 9 (fitted on [0, 1.0001 pi/2] to 6e-9
-// relative).  Only IEEE single operations with explicit fused multiply-adds: the same bits on the
-// host and on the device.  Against glibc's sinf / cosf over every |y| < 120
-// (tests/native/devmath_check.c, exhaustive): at most 2 ulp; sine 98.6 % equal, cosine 94.8 %.
-// Larger arguments take cta_sincosf.
+// time the double-precision routines above would set (fused expressions).  y = k pi/2 + r with k the
+// nearest integer and |r| <= pi/4 (1 + 1e-4); sin r from an odd polynomial of degree 7, cos r from
+// an even one of degree 8 (fitted on that interval to 4e-9 and 6e-11 relative), and the quadrant
+// k mod 4 picks which of the two, and with which sign, is the sine and which the cosine.  pi/2 is
+// split in three floats whose first two have 17 significant bits, so the first step of the
+// reduction is exact (|k| < 2^7) and the second loses half an ulp of r at most.  Everything up to
+// the pick is the same for the sine and the cosine of one argument: a kernel that needs both (a
+// product's gradient, sin and cos of one tensor in one expression) pays the reduction and the two
+// polynomials once, since the compiler merges the equal computations.  Exactly odd / even in y.
+// Only IEEE single operations with explicit fused multiply-adds: the same bits on the host and on
+// the device.  Against glibc's sinf / cosf over every |y| < 120 (tests/native/devmath_check.c,
+// exhaustive): at most 2 ulp; sine 99.1 % equal, cosine 98.9 %, 2 ulp on fewer than 900 arguments
+// each.  Larger arguments take cta_sincosf.
 CTA_FN float cta_sincosf_f32(float y, int want_cos) {
-    const float q = want_cos ? CTA_FMAF(y, 0x1.45f306p-2f, -0.5f) : y * 0x1.45f306p-2f;    // y / pi (- 1/2)
-    const float k = __builtin_rintf(q);
-    const float j = want_cos ? k + 0.5f : k;
-    float r = CTA_FMAF(j, -0x1.921fp+1f, y);
-    r = CTA_FMAF(j, -0x1.6a88p-16f, r);
-    r = CTA_FMAF(j, -0x1.0b46p-33f, r);
+    const float k = __builtin_rintf(y * 0x1.45f306p-1f);          // y * 2 / pi
+    float r = CTA_FMAF(k, -0x1.921fp+0f, y);
+    r = CTA_FMAF(k, -0x1.6a88p-17f, r);
+    r = CTA_FMAF(k, -0x1.0b4612p-34f, r);
     const float s = r * r;
-    float p = CTA_FMAF(s, 0x1.5dbce8p-19f, -0x1.9f6feep-13f);
-    p = CTA_FMAF(p, s, 0x1.110ed4p-7f);
-    p = CTA_FMAF(p, s, -0x1.55554cp-3f);
-    const float v = CTA_FMAF(r * s, p, r);
-    const int32_t ki = (int32_t)k + (want_cos ? 1 : 0);
-    return cta_u2f(cta_f2u(v) ^ ((uint32_t)ki << 31));
+    float ps = CTA_FMAF(s, -0x1.994e02p-13f, 0x1.11075ep-7f);
+    ps = CTA_FMAF(ps, s, -0x1.555546p-3f);
+    const float sn = CTA_FMAF(r * s, ps, r);
+    float pc = CTA_FMAF(s, 0x1.99337cp-16f, -0x1.6c087cp-10f);
+    pc = CTA_FMAF(pc, s, 0x1.55553ep-5f);
+    pc = CTA_FMAF(pc, s, -0.5f);
+    const float cs = CTA_FMAF(pc, s, 1.0f);
+    const int32_t ki = (int32_t)k;
+    // quadrants 0..3: sine = sn, cs, -sn, -cs; cosine = cs, -sn, -cs, sn
+    const float v = ((ki & 1) != want_cos) ? cs : sn;
+    const uint32_t quadrant = (uint32_t)ki + (uint32_t)want_cos;
+    const float t = cta_u2f(cta_f2u(v) ^ ((quadrant << 30) & 0x80000000u));
+    return (!want_cos && y == 0.0f) ? y : t;                      // sin(-0) = -0 (the sums above turn it into +0)
 }
 
 // ---- exp for doubles: glibc's algorithm (sysdeps/ieee754/dbl-64/e_exp.c, the ARM optimized-routines

@@ -164,8 +164,24 @@ void emit_op(std::string& o, const ctamd_expr_insn* prog, const Ssa& s, int pc, 
             else loop("sigmoid_ref(" + a + "[e], tabs)");
             break;
         case CTAMD_EX_TANH: loop("tanh_ref(" + a + "[e], tabs)"); break;
-        case CTAMD_EX_SIN: in_place(std::string("sin_or_cos<") + (fastm ? "true" : "false") + ", 0>(" + d + ", tabs)"); break;
-        case CTAMD_EX_COS: in_place(std::string("sin_or_cos<") + (fastm ? "true" : "false") + ", 1>(" + d + ", tabs)"); break;
+        case CTAMD_EX_SIN:
+        case CTAMD_EX_COS: {
+            // The single-precision routines of the default mode are exactly odd / even, so the sine or cosine
+            // of a negated value is formed from the value itself: sin(x) and cos(-x) of one expression then
+            // share their argument reduction and both polynomials (the compiler merges the equal work).
+            // The bits are those of the operator applied to the negated value, which the interpreter forms.
+            int src = s.a[size_t(pc)];
+            bool flipped = false;
+            while (fastm && prog[src].op == CTAMD_EX_NEG) {
+                src = s.a[size_t(src)];
+                flipped = !flipped;
+            }
+            const bool sine = q.op == CTAMD_EX_SIN;
+            o += "    float " + d + "[N];\n    _Pragma(\"unroll\") for (int e = 0; e < N; ++e) " + d + "[e] = " + name(src) + "[e];\n    sin_or_cos<" +
+                 (fastm ? "true" : "false") + ", " + (sine ? "0" : "1") + ">(" + d + ", tabs);\n";
+            if (sine && flipped) o += "    _Pragma(\"unroll\") for (int e = 0; e < N; ++e) " + d + "[e] = -" + d + "[e];\n";
+            break;
+        }
         case CTAMD_EX_ADDS: loop(a + "[e] + " + f32_literal(q.imm)); break;
         case CTAMD_EX_MULS: loop(a + "[e] * " + f32_literal(q.imm)); break;
         case CTAMD_EX_DIVS: loop("cta_div_rcp(" + a + "[e], " + f64_literal(1.0 / double(q.imm)) + ")"); break;

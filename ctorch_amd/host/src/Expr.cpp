@@ -74,8 +74,20 @@ struct Code {
     };
     std::vector<I> code;
     std::map<std::tuple<int, int, int, uint32_t, int>, int> seen;
+    // cos(-v) = cos(v) and sin(-v) = -sin(v): exact for the single-precision routines of the default
+    // math mode, and what lets sin(v) and cos(-v) of one expression share their argument reduction.
+    // glibc's sinf / cosf round the quadrant of -v and v differently on the boundary between two
+    // quadrants, so programs for the exact mode keep the negation where the expression has it.
+    bool fold_signs = false;
 
     int emit(int op, int a, int b, float imm = 0.0f, int port = 0) {
+        if (fold_signs && (op == CTAMD_EX_COS || op == CTAMD_EX_SIN) && code[size_t(a)].op == CTAMD_EX_NEG) {
+            const int v = code[size_t(a)].a;
+            if (op == CTAMD_EX_COS) return emit(CTAMD_EX_COS, v, v);
+            const int s = emit(CTAMD_EX_SIN, v, v);
+            return emit(CTAMD_EX_NEG, s, s);
+        }
+        if (fold_signs && op == CTAMD_EX_NEG && code[size_t(a)].op == CTAMD_EX_NEG) return code[size_t(a)].a;
         uint32_t bits;
         std::memcpy(&bits, &imm, sizeof(bits));
         if (op == CTAMD_EX_ADD || op == CTAMD_EX_MUL) {       // commutative bit for bit: one canonical operand order
@@ -107,14 +119,21 @@ bool is_load(int op) { return op == CTAMD_EX_LOAD_FULL || op == CTAMD_EX_LOAD_RO
 // an operand that dies in the same instruction (operands are read before the result is written).
 // False when the program needs more than the launch layer's slots or instructions.
 bool lower(const Code& in, std::vector<ctamd_expr_insn>& out) {
-    // loads first: the kernel issues the loads at the head of a program together
+    // loads first: the kernel issues the loads at the head of a program together; values nobody
+    // reads (a negation that cos(-v) = cos(v) left behind) are dropped
     Code c;
     {
+        std::vector<bool> live(in.code.size(), false);
+        for (size_t i = in.code.size(); i-- > 0;) {
+            const Code::I& q = in.code[i];
+            if (!has_result(q.op)) live[i] = true;
+            if (live[i] && !is_load(q.op)) live[size_t(q.a)] = live[size_t(q.b)] = true;
+        }
         std::vector<int> renumber(in.code.size(), -1);
         for (int pass = 0; pass < 2; ++pass)
             for (size_t i = 0; i < in.code.size(); ++i) {
                 Code::I q = in.code[i];
-                if (is_load(q.op) != (pass == 0)) continue;
+                if (!live[i] || is_load(q.op) != (pass == 0)) continue;
                 if (!is_load(q.op)) {
                     q.a = renumber[size_t(q.a)];
                     q.b = renumber[size_t(q.b)];
@@ -183,7 +202,7 @@ struct Program : FusedPayload {
         std::vector<ctamd_expr_insn> code;
         std::vector<int> out_port;        // output k is the gradient of input out_port[k]
     };
-    std::map<std::pair<unsigned, bool>, Backward> backward_code;   // by (mask of wanted inputs, check_div_zero)
+    std::map<std::tuple<unsigned, bool, bool>, Backward> backward_code;   // by (mask of wanted inputs, check_div_zero, default math mode)
 
     int ports() const { return int(port_is_row.size()); }
 
@@ -205,6 +224,7 @@ struct Program : FusedPayload {
 
     bool compile_forward() {
         Code c;
+        c.fold_signs = ctamd_math_mode() == CTAMD_MATH_FAST;
         std::vector<int> done(vals.size(), -1);
         int root = need(c, done, int(vals.size()) - 1);
         c.effect(CTAMD_EX_STORE, root, 0);
@@ -214,9 +234,10 @@ struct Program : FusedPayload {
     // The tape's backward over the expression (src/AutoDiff.cpp:1138-1153 order, :1216-1416
     // formulas, :1870-1907 accumulation) written out as one program: upstream gradient g = input
     // `ports()`, one output per wanted input that the walk reaches.
-    void compile_backward(unsigned mask, bool check, Backward& out) const {
+    void compile_backward(unsigned mask, bool check, bool fast, Backward& out) const {
         const int n = int(vals.size());
         Code c;
+        c.fold_signs = fast;
         std::vector<int> done(size_t(n), -1), adj(size_t(n), -1);
         std::vector<bool> wants(size_t(n), false);
         std::set<int> checked;
@@ -324,11 +345,12 @@ struct Program : FusedPayload {
         unsigned mask = 0;
         for (size_t p = 0; p < wanted.size(); ++p)
             if (wanted[p]) mask |= 1u << p;
-        auto key = std::make_pair(mask, check_div_zero);
+        const bool fast = ctamd_math_mode() == CTAMD_MATH_FAST;
+        auto key = std::make_tuple(mask, check_div_zero, fast);
         auto it = backward_code.find(key);
         if (it == backward_code.end()) {
             Backward b;
-            compile_backward(mask, check_div_zero, b);
+            compile_backward(mask, check_div_zero, fast, b);
             it = backward_code.emplace(key, std::move(b)).first;
         }
         const Backward& b = it->second;
@@ -518,9 +540,10 @@ Tensor Expr::eval() const {
             if (lin.tensors[k].requires_grad()) mask |= 1u << k;
         if (mask) {
             Program::Backward b;
-            program->compile_backward(mask, true, b);
+            const bool fast = ctamd_math_mode() == CTAMD_MATH_FAST;
+            program->compile_backward(mask, true, fast, b);
             fusable = b.fits;
-            program->backward_code.emplace(std::make_pair(mask, true), std::move(b));
+            program->backward_code.emplace(std::make_tuple(mask, true, fast), std::move(b));
         }
     }
     t_stats = ProgramStats();

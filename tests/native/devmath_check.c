@@ -2,7 +2,7 @@
  * which the device algorithms (compiled here for the CPU, unchanged) return different bits from
  * expf / sinf / cosf / logf, and the worst distance of the tangent from glibc's tanf (not the same
  * algorithm: at most 1 ulp) and of the single-precision sine / cosine pair from sinf / cosf (at most 2
- * ulp, |x| < 120).  Usage: devmath_check STRIDE  (1 = every one of the 2^32 bit patterns).
+ * ulp, |x| < 120; also that the pair is exactly odd / even).  Usage: devmath_check STRIDE  (1 = every one of the 2^32 bit patterns).
  * Prints one line per function: name, inputs tested, mismatches, worst ulp distance
  * (expf_pair: exp(x) and exp(-x) from the shared reduction, against expf(x) and expf(-x)). */
 #include <math.h>
@@ -73,14 +73,17 @@ int main(int argc, char** argv) {
         if (!cta_sincos_is_rare(x)) {               /* the single-precision pair: |x| < 120, at most 2 ulp */
             ++covered[6];
             if (differs(cta_sincosf_f32(x, 0), sinf(x), &d)) {
-                if (d > 2) ++bad[6];
+                if (d > 2 || d == 0) ++bad[6];     /* d == 0: zeros of opposite sign */
                 if (d > worst[6]) worst[6] = d;
             }
             ++covered[7];
             if (differs(cta_sincosf_f32(x, 1), cosf(x), &d)) {
-                if (d > 2) ++bad[7];
+                if (d > 2 || d == 0) ++bad[7];
                 if (d > worst[7]) worst[7] = d;
             }
+            /* exactly odd / even: the fused-expression compiler forms sin(-x), cos(-x) from sin(x), cos(x) */
+            if (cta_f2u(cta_sincosf_f32(-x, 0)) != (cta_f2u(cta_sincosf_f32(x, 0)) ^ 0x80000000u)) ++bad[6];
+            if (cta_f2u(cta_sincosf_f32(-x, 1)) != cta_f2u(cta_sincosf_f32(x, 1))) ++bad[7];
         }
     }
     const char* names[8] = {"expf", "sinf", "cosf", "expf_pair", "logf", "tanf(>1ulp)", "sinf_f32(>2ulp)", "cosf_f32(>2ulp)"};
