@@ -1103,6 +1103,13 @@ class HostLayer(Reference):
         expression (Expr::eval): one launch forward, one backward."""
         self.cdll.cth_set_fused_expr(int(on))
 
+    def last_expr_stats(self):
+        """(forward instructions, forward slots, backward instructions, backward slots) of the programs the
+        last fused expression compiled; zeros when it was evaluated operator by operator."""
+        out = (C.c_int * 4)()
+        self.cdll.cth_last_expr_stats(out)
+        return tuple(out)
+
     def set_fused_layers(self, on):
         """mlp_step builds each layer with Tensor::linear (matmul + bias + ReLU as one operator)."""
         self.cdll.cth_set_fused_layers(int(on))

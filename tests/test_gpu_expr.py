@@ -150,6 +150,31 @@ def test_compiled_config5_expression_equals_the_interpreter(oracle, mode, rows, 
     assert same_bits(G.host(got[0]), G.host(want[0]))
 
 
+@pytest.mark.parametrize("mode", ["exact", "fast_mode"])
+def test_compiled_sine_and_cosine_of_negated_values_equal_the_interpreter(oracle, mode):
+    """sin(-x), cos(-x), sin(-(-x)) beside sin(x), cos(x): in the default mode the compiled kernel forms
+    them from x itself (the single-precision routines are exactly odd / even, special values included),
+    the interpreter applies the operators as written - the same bits; the exact mode keeps the
+    negations in both."""
+    print("case expr compiled negated sin / cos", mode, flush=True)
+    E = EX
+    prog = [(E["LOAD_FULL"], 0, 0, 0, 0.0), (E["NEG"], 1, 0, 0, 0.0), (E["NEG"], 2, 1, 0, 0.0),
+            (E["SIN"], 3, 1, 0, 0.0), (E["STORE"], 0, 3, 0, 0.0), (E["COS"], 3, 1, 0, 0.0), (E["STORE"], 1, 3, 0, 0.0),
+            (E["SIN"], 3, 2, 0, 0.0), (E["STORE"], 2, 3, 0, 0.0), (E["SIN"], 3, 0, 0, 0.0), (E["STORE"], 3, 3, 0, 0.0),
+            (E["COS"], 3, 0, 0, 0.0), (E["STORE"], 4, 3, 0, 0.0)]
+    x = oracle.uniform((64, 1024), 77, -130, 130)
+    x[0, :10] = [0.0, -0.0, np.inf, -np.inf, np.nan, 119.99999, 120.0, -120.0, 1e-45, -1e-45]
+    (got, _), (want, _) = _run_both_ways(prog, [G.dev(x)], 5, 64, 1024)
+    for k in range(5):
+        assert same_bits_or_both_nan(G.host(got[k]), G.host(want[k])), k
+    s_neg, c_neg, s_back, s, c = (G.host(v) for v in got)
+    fin = np.isfinite(s)
+    assert np.array_equal(s_back[fin].view(np.uint32), s[fin].view(np.uint32))
+    if mode == "fast_mode":
+        assert np.array_equal(s_neg[fin].view(np.uint32), (-s[fin]).view(np.uint32))
+        assert np.array_equal(c_neg[fin].view(np.uint32), c[fin].view(np.uint32))
+
+
 def test_a_program_is_compiled_at_the_second_launch(oracle):
     """The default: the first launch of a program is interpreted, the second compiles it; operands the
     compiled kernels do not take (rows that are not a multiple of four) stay with the interpreter."""

@@ -365,6 +365,37 @@ def test_fused_expressions_against_the_reference_vectors(oracle, host, golden, e
         host.set_reference_row0(False)
 
 
+def test_fused_expression_in_the_default_mode_drops_the_negations_under_sine_and_cosine(oracle, host, golden):
+    """Configuration 5 as one fused expression in the default math mode: the expression compiler forms
+    cos(-X) from X (and sin(-X) in the gradient program as -sin(X)), so both programs are shorter than
+    the exact mode's, which keeps the negations where glibc's quadrant rounding could tell -x from x;
+    value and gradients stay within the default mode's bound of the exact mode's."""
+    from ctorch_amd import capi
+    print("case host fused expression, default mode", flush=True)
+    lib = capi.load()
+    assert lib.ctamd_math_mode() == 0
+    c = golden("configs")
+    X, rv, T = c["expr_X"], c["expr_r"], c["expr_T"]
+    host.set_fused_expr(True)
+    try:
+        y, mse, mae, gX, gr = host.expr(X, rv, T)
+        fast = host.last_expr_stats()
+        assert lib.ctamd_set_math_mode(1) == 0
+        try:
+            ye, msee, maee, gXe, gre = host.expr(X, rv, T)
+            exact = host.last_expr_stats()
+        finally:
+            assert lib.ctamd_set_math_mode(0) == 0
+    finally:
+        host.set_fused_expr(False)
+    print("  program sizes (forward, slots, backward, slots): default", fast, "exact", exact)
+    assert fast[0] == exact[0] - 1 and 0 < fast[2] < exact[2]
+    assert np.abs(y - ye).max() <= 8e-7
+    assert abs(float(mse) - float(msee)) <= 1e-5 * float(msee) and abs(float(mae) - float(maee)) <= 1e-5 * float(maee)
+    assert np.abs(gX - gXe).max() <= 1e-5 * np.abs(gXe).max()
+    assert np.abs(gr - gre).max() <= 1e-5 * np.abs(gre).max()
+
+
 def test_comparison_operators(oracle, host):
     """Tensor (cmp) Tensor and Tensor (cmp) float through the front-end: DType::kBool results equal
     to the oracle's; tensors of different shapes throw (src/Tensor.cpp:1124-1126)."""
