@@ -16,10 +16,26 @@ struct Tables {
     const double* log;       // cta_log_tab, staged only for functors with kLogTable
 };
 
+// num / den for the tanh quotient below (den >= 2, |num| <= den): the steps of the division the compiler
+// writes for `/` - reciprocal, one Newton step on it, the quotient, two corrections on exact residuals -
+// without that sequence's operand scaling and fix-up instructions, which take as long as the
+// rest together and only matter for operands this quotient does not have.  den >= 2^100 (|x| > 69),
+// infinite (inf / inf = NaN for |x| > 88.72) or NaN takes the plain division.  The same bits as `/`:
+// every float through the tanh kernel against the quotient formed by the division kernel
+// (tests/test_gpu_parity.py, all 2^32 arguments).
+__device__ __forceinline__ float tanh_quotient(float num, float den) {
+    float y = __builtin_amdgcn_rcpf(den);
+    y = __fmaf_rn(__fmaf_rn(-den, y, 1.0f), y, y);
+    float q = num * y;
+    q = __fmaf_rn(__fmaf_rn(-den, q, num), y, q);
+    q = __fmaf_rn(__fmaf_rn(-den, q, num), y, q);
+    if (__builtin_expect(!(den < 0x1p100f), 0)) q = num / den;
+    return q;
+}
 __device__ __forceinline__ float tanh_ref(float x, const Tables& t) {
     float ep, en;
     cta_expf_pair(x, t.exp2, &ep, &en);
-    return (ep - en) / (ep + en);
+    return tanh_quotient(ep - en, ep + en);
 }
 __device__ __forceinline__ float sigmoid_ref(float x, const Tables& t) {
     return 1.0f / (1.0f + cta_expf_tab(-x, t.exp2));

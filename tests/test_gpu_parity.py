@@ -174,6 +174,35 @@ def test_transcendentals_bit_identical_over_a_sweep_of_all_floats(oracle):
         assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32)), name
 
 
+def test_tanh_over_every_float_against_its_formula_through_the_operator_kernels():
+    """All 2^32 bit patterns: the tanh kernel against (e^x - e^-x) / (e^x + e^-x) formed by the exp, neg,
+    sub, add and div kernels (the exponential's bits are glibc's - sweep above, native check - and the
+    others are single IEEE operations).  tanh forms its quotient without the scaling and fix-up steps of
+    the division the compiler writes: this is the check that those never mattered.  The gradient kernel
+    recomputes tanh by the same routine: checked through 1 - tanh^2 on every 64th chunk."""
+    import torch
+    print("case tanh, every float", flush=True)
+    chunk = 1 << 26
+    base = torch.arange(chunk, dtype=torch.int64, device=G.DEV)
+    ones = torch.ones(chunk, device=G.DEV)
+    for c in range((1 << 32) // chunk):
+        x = (base + c * chunk).to(torch.int32).view(torch.float32)
+        ep, en = G.unary("exp", x), G.unary("exp", G.unary("neg", x))
+        want = G.binary("div", G.binary("sub", ep, en), G.binary("add", ep, en))
+        got = G.unary("tanh", x)
+        nan = torch.isnan(want)
+        assert bool((torch.isnan(got) == nan).all()), c
+        assert bool((got.view(torch.int32)[~nan] == want.view(torch.int32)[~nan]).all()), c
+        if c % 16 == 0:
+            gb = G.unary_bwd("tanh", x, ones)
+            wb = (1.0 - want * want) * ones          # three single operations, as the gradient kernel's
+            ok = ~torch.isnan(wb)
+            assert bool((torch.isnan(gb) == ~ok).all()), c
+            assert bool((gb.view(torch.int32)[ok] == wb.view(torch.int32)[ok]).all()), c
+        if c % 16 == 15:
+            print("  chunk", c, flush=True)
+
+
 def test_transcendentals_against_golden_reference_vectors(golden):
     print("case transcendentals golden", flush=True)
     g = golden("elementwise")
