@@ -365,6 +365,35 @@ def test_fused_expressions_against_the_reference_vectors(oracle, host, golden, e
         host.set_reference_row0(False)
 
 
+def test_fused_programs_in_the_default_math_mode_against_the_mathematics(oracle, host):
+    """The random tape programs as fused expressions in the default math mode (single-precision sine /
+    cosine / sigmoid, negations under a sine or cosine folded away by the expression compiler): value
+    and every gradient against the fp64 interpreter, as the exact mode is held to."""
+    import importlib.util
+    import os
+    from ctorch_amd import capi
+    from support import program_fp64, program_inputs, random_program
+    spec = importlib.util.spec_from_file_location("make_golden", os.path.join(os.path.dirname(__file__), "golden",
+                                                                            "make_golden.py"))
+    mg = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mg)
+    assert capi.load().ctamd_math_mode() == 0
+    host.set_fused_expr(True)
+    try:
+        for seed in mg.PROGRAM_SEEDS:
+            print("case fused program, default mode", seed, flush=True)
+            rows, cols = mg.program_shape(seed)
+            kinds, ops = random_program(seed)
+            xs, w = program_inputs(oracle, seed, kinds, rows, cols)
+            rc, y, L, grads = host.program(xs, kinds, ops, w)
+            y64, L64, g64 = program_fp64(xs, kinds, ops, w, row0=False)
+            assert rc >= 0 and np.abs(y - y64).max() <= 1e-5 * (1 + np.abs(y64).max()), seed
+            for got, want in zip(grads, g64):
+                assert np.abs(got - want).max() <= 2e-5 * (1 + np.abs(want).max()), seed
+    finally:
+        host.set_fused_expr(False)
+
+
 def test_fused_expression_in_the_default_mode_drops_the_negations_under_sine_and_cosine(oracle, host, golden):
     """Configuration 5 as one fused expression in the default math mode: the expression compiler forms
     cos(-X) from X (and sin(-X) in the gradient program as -sin(X)), so both programs are shorter than
