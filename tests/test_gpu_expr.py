@@ -162,9 +162,12 @@ def test_compiled_sine_and_cosine_of_negated_values_equal_the_interpreter(oracle
             (E["SIN"], 3, 1, 0, 0.0), (E["STORE"], 0, 3, 0, 0.0), (E["COS"], 3, 1, 0, 0.0), (E["STORE"], 1, 3, 0, 0.0),
             (E["SIN"], 3, 2, 0, 0.0), (E["STORE"], 2, 3, 0, 0.0), (E["SIN"], 3, 0, 0, 0.0), (E["STORE"], 3, 3, 0, 0.0),
             (E["COS"], 3, 0, 0, 0.0), (E["STORE"], 4, 3, 0, 0.0)]
-    x = oracle.uniform((64, 1024), 77, -130, 130)
-    x[0, :10] = [0.0, -0.0, np.inf, -np.inf, np.nan, 119.99999, 120.0, -120.0, 1e-45, -1e-45]
-    (got, _), (want, _) = _run_both_ways(prog, [G.dev(x)], 5, 64, 1024)
+    # every 509th bit pattern (all exponents, both signs, infinities, NaNs) and a dense sample of the usual range
+    sweep = np.arange(0, 1 << 32, 509, dtype=np.uint64).astype(np.uint32).view(F)
+    x = np.concatenate([oracle.uniform((64 * 1024,), 77, -130, 130), sweep])
+    x[:10] = [0.0, -0.0, np.inf, -np.inf, np.nan, 119.99999, 120.0, -120.0, 1e-45, -1e-45]
+    x = x[: (x.size // 1024) * 1024].reshape(-1, 1024)
+    (got, _), (want, _) = _run_both_ways(prog, [G.dev(x)], 5, x.shape[0], 1024)
     for k in range(5):
         assert same_bits_or_both_nan(G.host(got[k]), G.host(want[k])), k
     s_neg, c_neg, s_back, s, c = (G.host(v) for v in got)
