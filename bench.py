@@ -144,6 +144,9 @@ def config_report(with_cpu):
         if ref is None:
             ref = support.Oracle()
 
+    # Every step below is timed after some 40 ms of untimed steps of the same kind: the chip's clock keeps
+    # moving for about 25 ms after a change of load (up after idling, down and part of the way back under
+    # heavy vector work), and a training loop runs in the state after that.
     rows = []
 
     def add(name, rc, out, cpu_ms=None, cpu_note=None, launch_bound=False):
@@ -166,14 +169,14 @@ def config_report(with_cpu):
     n = 1 << 20
     a, b = rng.uniform(n, SEEDS["config1"]["a"], -1, 1), rng.uniform(n, SEEDS["config1"]["b"], -1, 1)
     out = D5()
-    rc = host.cth_time_chain(fp(a), fp(b), L(n), I(5), I(50), out)
+    rc = host.cth_time_chain(fp(a), fp(b), L(n), I(300), I(50), out)
     cpu = _timed(lambda: ref.chain(a, b)) if with_cpu else None
     add("config 1: c=a*b+5, relu, sum, backward; n=2^20", rc, out, cpu, "whole step", launch_bound=True)
     # the elementwise chain as one fused expression (one launch forward, one backward); no
     # transcendental operator in it, so the same bits in either math mode
     host.cth_set_fused_expr(1)
     out = D5()
-    rc = host.cth_time_chain(fp(a), fp(b), L(n), I(5), I(50), out)
+    rc = host.cth_time_chain(fp(a), fp(b), L(n), I(300), I(50), out)
     host.cth_set_fused_expr(0)
     add("config 1: c=a*b+5, relu, sum, backward; n=2^20, fused expression", rc, out, cpu, "whole step", launch_bound=True)
     rows[-1]["math_mode"] = "default (CTAMD_MATH_FAST); this program has no transcendental operator: bit-equal to the unfused step"
@@ -201,7 +204,7 @@ def config_report(with_cpu):
         del A, B
     u, v = rng.uniform(1 << 26, SEEDS["config2"]["dot_u"], -1, 1), rng.uniform(1 << 26, SEEDS["config2"]["dot_v"], -1, 1)
     out = D5()
-    rc = host.cth_time_dot(fp(u), fp(v), L(1 << 26), I(3), I(20), out)
+    rc = host.cth_time_dot(fp(u), fp(v), L(1 << 26), I(200), I(20), out)
     cpu, note = None, None
     if with_cpu:
         m = 1 << 24
@@ -219,7 +222,7 @@ def config_report(with_cpu):
         x = f32(rng.ints((Bn, 784), s3["x"], 256) / np.float32(255.0))
         lab = rng.ints(Bn, s3["labels"], 10)
         out = D5()
-        rc = host.cth_time_mlp(fp(x), L(Bn), L(784), fp(W1), fp(b1), L(256), fp(W2), fp(b2), L(10), fp(lab), I(5),
+        rc = host.cth_time_mlp(fp(x), L(Bn), L(784), fp(W1), fp(b1), L(256), fp(W2), fp(b2), L(10), fp(lab), I(300),
                                I(30), out)
         cpu, note = None, None
         if with_cpu:
@@ -248,7 +251,7 @@ def config_report(with_cpu):
                 host.cth_set_inputs_unseen(unseen)
                 host.cth_set_ce_deferred_label_check(deferred)
                 out = D5()
-                rc = host.cth_time_mlp(fp(x), L(Bn), L(784), fp(W1), fp(b1), L(256), fp(W2), fp(b2), L(10), fp(lab), I(5),
+                rc = host.cth_time_mlp(fp(x), L(Bn), L(784), fp(W1), fp(b1), L(256), fp(W2), fp(b2), L(10), fp(lab), I(300),
                                        I(30), out)
                 add("config 3: MLP 784-256-10 train step, batch %d, fused layers%s%s" % (Bn, ", one-pass head" if head else "", what),
                     rc, out, cpu, note, launch_bound=(Bn == 256))
@@ -262,7 +265,7 @@ def config_report(with_cpu):
             host.cth_set_fused_layers(fused)
             host.cth_set_fused_head(head)
             out = D5()
-            rc = host.cth_time_mlp(fp(x), L(Bn), L(784), fp(W1), fp(b1), L(256), fp(W2), fp(b2), L(10), fp(lab), I(20),
+            rc = host.cth_time_mlp(fp(x), L(Bn), L(784), fp(W1), fp(b1), L(256), fp(W2), fp(b2), L(10), fp(lab), I(400),
                                    I(200), out)
             add("config 3: MLP 784-256-10 train step, batch %d%s, steps queued back to back (no loss read per step)" % (Bn, what),
                 rc, out, cpu, note, launch_bound=(Bn == 256))
@@ -275,7 +278,7 @@ def config_report(with_cpu):
         for fused in (0, 1):
             host.cth_set_fused_layers(fused)
             out = D5()
-            rc = host.cth_time_mlp_graph(fp(x), L(Bn), L(784), fp(W1), fp(b1), L(256), fp(W2), fp(b2), L(10), fp(oh), I(5),
+            rc = host.cth_time_mlp_graph(fp(x), L(Bn), L(784), fp(W1), fp(b1), L(256), fp(W2), fp(b2), L(10), fp(oh), I(300),
                                          I(30), out)
             host.cth_set_fused_layers(0)
             add("config 3: MLP 784-256-10 train step, batch %d, %sreplayed from a recorded HIP graph"
@@ -287,7 +290,7 @@ def config_report(with_cpu):
     logits = rng.normal((R4, C4), SEEDS["config4"]["logits"], 0.0, 2.0)
     lab = rng.ints(R4, SEEDS["config4"]["labels"], C4)
     out = D5()
-    rc = host.cth_time_softmax_ce(fp(logits), fp(lab), L(R4), L(C4), I(2), I(10), out)
+    rc = host.cth_time_softmax_ce(fp(logits), fp(lab), L(R4), L(C4), I(100), I(20), out)
     cpu, note = None, None
     if with_cpu:
         r = 512
@@ -305,7 +308,7 @@ def config_report(with_cpu):
     s5 = SEEDS["config5"]
     X, rv, T = rng.uniform((R5, R5), s5["X"], -2, 2), rng.uniform(R5, s5["r"], 0.5, 2), rng.normal((R5, R5), s5["T"])
     out = D5()
-    rc = host.cth_time_expr(fp(X), fp(rv), fp(T), L(R5), L(R5), I(3), I(10), out)
+    rc = host.cth_time_expr(fp(X), fp(rv), fp(T), L(R5), L(R5), I(60), I(20), out)
     cpu, note = None, None
     if with_cpu:
         r = 1024
@@ -319,7 +322,7 @@ def config_report(with_cpu):
     # the reference's bits (CTAMD_MATH_EXACT gives the unfused step's Y and dX bit for bit)
     host.cth_set_fused_expr(1)
     out = D5()
-    rc = host.cth_time_expr(fp(X), fp(rv), fp(T), L(R5), L(R5), I(3), I(10), out)
+    rc = host.cth_time_expr(fp(X), fp(rv), fp(T), L(R5), L(R5), I(150), I(20), out)
     host.cth_set_fused_expr(0)
     add("config 5: Y=sigmoid(X/r)-tanh(X)*sin(X)+cos(-X), MSE+MAE, backward; X [4096 x 4096], fused expression", rc, out, cpu,
         note)
@@ -329,7 +332,7 @@ def config_report(with_cpu):
     capi_lib.ctamd_set_math_mode(1)
     host.cth_set_fused_expr(1)
     out = D5()
-    rc = host.cth_time_expr(fp(X), fp(rv), fp(T), L(R5), L(R5), I(3), I(10), out)
+    rc = host.cth_time_expr(fp(X), fp(rv), fp(T), L(R5), L(R5), I(150), I(20), out)
     host.cth_set_fused_expr(0)
     capi_lib.ctamd_set_math_mode(0)
     add("config 5: Y=sigmoid(X/r)-tanh(X)*sin(X)+cos(-X), MSE+MAE, backward; X [4096 x 4096], fused expression, exact math mode",

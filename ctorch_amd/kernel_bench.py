@@ -44,10 +44,18 @@ def main():
     call = lambda name, *a: capi.check(getattr(lib, name)(*a))
     results = []
 
-    def timeit(fn, reps, warm=3):
+    # (the chip's clock keeps moving for about 25 ms after a change of load - up after idling, down and part of
+    # the way back under heavy vector work: a run of fused config-5 launches reads 190, 174, 162, 155, 155, ... us
+    # over successive 10 ms - so every row first keeps its launches coming for `settle` seconds)
+    def timeit(fn, reps, warm=3, settle=0.03):
         for _ in range(warm):
             fn()
         torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < settle:
+            for _ in range(5):
+                fn()
+            torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(reps):
