@@ -345,9 +345,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    # (15 steps = 45 ms: the chip's clock keeps moving for some 25 - 30 ms after the load starts; with 5 the
-    # first timed steps still ran 2 - 7 % slower than the rest)
-    ap.add_argument("--warmup", type=int, default=15)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-configs", action="store_true", help="skip the per-configuration report")
     args = ap.parse_args()
@@ -398,6 +396,16 @@ def main():
             e2.record()
             step_events.append((e0, e2))
 
+    # Before the W warm-up steps: untimed steps for 45 ms, whatever W is.  The chip reaches the clock it keeps
+    # under this load only after some 25 - 30 ms of it (the first forward products of a process take 1.12 ms,
+    # the steady ones 0.965), and a training loop runs in that state.  The count is reported as
+    # "clock_settle_steps".
+    settle_steps = 0
+    t_settle = time.perf_counter()
+    while time.perf_counter() - t_settle < 0.045:
+        step(False)
+        torch.cuda.synchronize()
+        settle_steps += 1
     for _ in range(args.warmup):
         step(False)
     torch.cuda.synchronize()
@@ -447,6 +455,7 @@ def main():
     out = {
         "metric": "elementwise HBM GB/s + fp32 MatMul TFLOP/s (% of MI355X roofline), 1 GPU",
         "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "clock_settle_steps": settle_steps,
         "ms_per_step": round(ms_per_step, 4), "ms_per_step_median": round(step_ms_median, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[1]: fp32 MatMul 4096^3 forward + backward (dA = dC.B^T, dB = A^T.dC, "
